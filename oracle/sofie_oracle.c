@@ -1,0 +1,538 @@
+/*
+ * sofie_oracle.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * A plain-C, single-threaded CPU restatement of the arithmetic that SOFIE's
+ * generated inference code performs for Gemm, Conv, Relu, MaxPool and Flatten,
+ * plus the quantized (int8 QLinear-style) and FP8 e4m3 operators that the HIP
+ * library adds.  It exists only so that tests, the smoke check and the CPU
+ * baseline leg of the benchmark have something to compare the GPU results with.
+ * Nothing in the shipped library links or calls it.
+ *
+ * Pinning status of each function (what independent evidence fixes its result):
+ *   or_sgemm, or_gemm_f32        pinned: Linear_16/32/64 known answers held by the
+ *                                reference's tests, numpy float64 closed form
+ *   or_im2col, or_conv2d_f32     pinned: ConvWith* known answers (ONNX spec examples),
+ *                                torch.nn.functional.conv2d on CPU, brute-force 7-loop
+ *   or_relu, or_maxpool2d        pinned: MaxPool2d known answer, torch CPU
+ *   or_broadcast_rows            pinned through the Linear_* answers (bias broadcast)
+ *   or_qgemm_s8, or_qconv2d_s8,
+ *   or_quantize_*, or_dequantize_*, or_gemm_fp8, or_e4m3_*, or_bf16_*
+ *                                the reference has no quantized operators at all
+ *                                ("parity unpinned" by the reference); pinned by
+ *                                mathematics instead: numpy int64 exact accumulators,
+ *                                exhaustive rounding-boundary checks, torch CPU
+ *                                float8_e4m3fn / bfloat16 casts, fp64 GEMM of the
+ *                                decoded operands.
+ *
+ * The fp32 FLOPs of the reference run inside an external Fortran BLAS that is not
+ * part of the reference tree (found by CMake find_package(BLAS), no pinned version).
+ * or_sgemm restates the textbook column-major SGEMM definition
+ *   C := alpha*op(A)*op(B) + beta*C
+ * with fp32 accumulation in increasing k, the loop order of the netlib reference BLAS.
+ *
+ * Build: gcc -O2 -ffp-contract=off -fPIC -shared (see Makefile). -ffp-contract=off
+ * keeps every multiply and add a separately rounded fp32 operation.
+ */
+#include <math.h>
+#include <stddef.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------- */
+/* Column-major SGEMM with Fortran calling convention semantics.             */
+/* Replaces: the external BLAS::sgemm_ declared by the generated code        */
+/* (src/SOFIE_core/src/RModel_Base.cxx:40-58).                               */
+/* ------------------------------------------------------------------------- */
+void or_sgemm(char transa, char transb, int m, int n, int k, float alpha,
+              const float *A, int lda, const float *B, int ldb, float beta,
+              float *C, int ldc)
+{
+    const int ta = (transa == 't' || transa == 'T');
+    const int tb = (transb == 't' || transb == 'T');
+    for (int j = 0; j < n; ++j) {
+        float *cj = C + (size_t)j * ldc;
+        if (beta == 0.0f) {
+            for (int i = 0; i < m; ++i) cj[i] = 0.0f;
+        } else if (beta != 1.0f) {
+            for (int i = 0; i < m; ++i) cj[i] = beta * cj[i];
+        }
+        if (!ta) {
+            /* C(:,j) += (alpha*B(l,j)) * A(:,l), l increasing */
+            for (int l = 0; l < k; ++l) {
+                const float b = tb ? B[(size_t)l * ldb + j] : B[(size_t)j * ldb + l];
+                const float t = alpha * b;
+                const float *al = A + (size_t)l * lda;
+                for (int i = 0; i < m; ++i) cj[i] += t * al[i];
+            }
+        } else {
+            /* C(i,j) += alpha * sum_l A(l,i)*B(l,j) */
+            for (int i = 0; i < m; ++i) {
+                const float *ai = A + (size_t)i * lda;
+                float t = 0.0f;
+                for (int l = 0; l < k; ++l) {
+                    const float b = tb ? B[(size_t)l * ldb + j] : B[(size_t)j * ldb + l];
+                    t += ai[l] * b;
+                }
+                cj[i] += alpha * t;
+            }
+        }
+    }
+}
+
+/* y := y + a*x. Replaces BLAS::saxpy_ (RModel_Base.cxx:40-58) for unit strides. */
+void or_saxpy(int n, float a, const float *x, float *y)
+{
+    for (int i = 0; i < n; ++i) y[i] += a * x[i];
+}
+
+/* ------------------------------------------------------------------------- */
+/* Bias broadcast used by Gemm: a rank-1 bias [N] (or any C whose trailing   */
+/* dims match) is materialised to the full [M,N] output shape once, in the   */
+/* Session constructor.                                                      */
+/* Follows ROperator_Gemm.hxx:271-290 and SOFIE_common.hxx:346-451 for the   */
+/* numpy-style case "prepend ones, repeat along leading dims".               */
+/* ------------------------------------------------------------------------- */
+void or_broadcast_rows(const float *c, int len_c, int rows, float *out)
+{
+    for (int r = 0; r < rows; ++r)
+        memcpy(out + (size_t)r * len_c, c, (size_t)len_c * sizeof(float));
+}
+
+/* ------------------------------------------------------------------------- */
+/* Gemm as emitted by ROperator_Gemm<float>::Generate                        */
+/* (ROperator_Gemm.hxx:292-390):                                             */
+/*   1. copy the pre-broadcast bias [M,N] into Y (:360-365)                  */
+/*   2. sgemm_(tB,tA,n,m,k,alpha,B,ldb,A,lda,beta,Y,n) -- the row-major      */
+/*      product through the column-major swap (:370-375)                     */
+/*   3. optional in-place ReLU (:377-381)                                    */
+/* bias_bcast may be NULL, in which case beta must be 0 (:343-349).          */
+/* Returns 0, or -1 for the "no bias but beta != 0" error of the reference.  */
+/* ------------------------------------------------------------------------- */
+int or_gemm_f32(int transA, int transB, int M, int N, int K, float alpha,
+                const float *A, const float *B, float beta,
+                const float *bias_bcast, float *Y, int relu)
+{
+    if (!bias_bcast && beta != 0.0f) return -1;
+    const int lda = transA ? M : K;
+    const int ldb = transB ? K : N;
+    if (bias_bcast) memcpy(Y, bias_bcast, (size_t)M * N * sizeof(float));
+    or_sgemm(transB ? 't' : 'n', transA ? 't' : 'n', N, M, K, alpha, B, ldb, A, lda,
+             beta, Y, N);
+    if (relu) {
+        const size_t len = (size_t)M * N;
+        for (size_t i = 0; i < len; ++i) Y[i] = (Y[i] > 0) ? Y[i] : 0;
+    }
+    return 0;
+}
+
+/* Out-of-place ReLU. Follows ROperator_Relu.hxx:54-66. */
+void or_relu_f32(const float *x, float *y, size_t len)
+{
+    for (size_t i = 0; i < len; ++i) y[i] = (x[i] > 0) ? x[i] : 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* im2col: one image [C,H,W] -> matrix [C*kh*kw, OH*OW], zero fill outside.  */
+/* Same result as UTILITY::Im2col (SOFIE_common.hxx:485-518); written as a   */
+/* gather over (row of the column matrix, output pixel).                     */
+/* ------------------------------------------------------------------------- */
+void or_im2col(const float *im, int C, int H, int W, int kh, int kw, int ph, int pw,
+               int sh, int sw, int dh, int dw, float *col)
+{
+    const int OH = (H + 2 * ph - (dh * (kh - 1) + 1)) / sh + 1;
+    const int OW = (W + 2 * pw - (dw * (kw - 1) + 1)) / sw + 1;
+    size_t o = 0;
+    for (int c = 0; c < C; ++c)
+        for (int r = 0; r < kh; ++r)
+            for (int s = 0; s < kw; ++s)
+                for (int oh = 0; oh < OH; ++oh) {
+                    const int ih = oh * sh - ph + r * dh;
+                    for (int ow = 0; ow < OW; ++ow) {
+                        const int iw = ow * sw - pw + s * dw;
+                        const int inside = (ih >= 0 && ih < H && iw >= 0 && iw < W);
+                        col[o++] = inside ? im[((size_t)c * H + ih) * W + iw] : 0.0f;
+                    }
+                }
+}
+
+/* ------------------------------------------------------------------------- */
+/* 2-D convolution as emitted by ROperator_Conv<float>::Generate             */
+/* (ROperator_Conv.hxx:302-522), NCHW, groups >= 1:                          */
+/*   - the kernel [OC, IC/g, kh, kw] is viewed as a matrix x_f [OC, k]       */
+/*     (:342-363; for dilation 1 this is a plain copy of W)                  */
+/*   - per image (and per group): im2col, then                               */
+/*     sgemm_('N','N', m=OH*OW, n=OC/g, k=IC/g*kh*kw, 1, xcol, m, x_f, k, 0, */
+/*     Y+off, m) (:447-451,:499-504), which writes NCHW directly             */
+/*   - per image: saxpy of the bias broadcast to [OC,OH,OW] (:509-518)       */
+/* Dilation > 1: the reference expands the kernel with zeros AND passes the  */
+/* dilation to Im2col again (:132-134,:342-363,:418-431), and its shape rule */
+/* (:173-199) disagrees with Im2col's own output size; no fixture or         */
+/* configuration uses it. Here dilation follows the ONNX definition (taps    */
+/* spaced by the dilation), which torch.nn.functional.conv2d pins.           */
+/* bias may be NULL. relu != 0 applies the separate Relu operator afterwards */
+/* (ROperator_Relu.hxx:54-66).                                               */
+/* ------------------------------------------------------------------------- */
+int or_conv2d_f32(const float *x, const float *w, const float *bias, float *y,
+                  int N, int C, int H, int W, int OC, int kh, int kw, int ph, int pw,
+                  int sh, int sw, int dh, int dw, int groups, int relu)
+{
+    if (groups < 1 || C % groups || OC % groups) return -1;
+    const int icg = C / groups, ocg = OC / groups;
+    const int OH = (H + 2 * ph - (dh * (kh - 1) + 1)) / sh + 1;
+    const int OW = (W + 2 * pw - (dw * (kw - 1) + 1)) / sw + 1;
+    if (OH <= 0 || OW <= 0) return -1;
+    const int m = OH * OW, k = icg * kh * kw;
+    float *col = (float *)malloc((size_t)k * m * sizeof(float));
+    if (!col) return -2;
+    for (int n = 0; n < N; ++n) {
+        for (int g = 0; g < groups; ++g) {
+            const float *xg = x + ((size_t)n * C + (size_t)g * icg) * H * W;
+            float *yg = y + ((size_t)n * OC + (size_t)g * ocg) * m;
+            or_im2col(xg, icg, H, W, kh, kw, ph, pw, sh, sw, dh, dw, col);
+            or_sgemm('n', 'n', m, ocg, k, 1.0f, col, m, w + (size_t)g * ocg * k, k, 0.0f,
+                     yg, m);
+        }
+        if (bias) {
+            float *yn = y + (size_t)n * OC * m;
+            for (int oc = 0; oc < OC; ++oc)
+                for (int p = 0; p < m; ++p) yn[(size_t)oc * m + p] += 1.0f * bias[oc];
+        }
+    }
+    if (relu) {
+        const size_t len = (size_t)N * OC * m;
+        for (size_t i = 0; i < len; ++i) y[i] = (y[i] > 0) ? y[i] : 0;
+    }
+    free(col);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* 2-D max pooling, NCHW, floor output size, -inf start value, pad cells     */
+/* skipped. Follows ROperator_Pool.hxx:371-416 (2-D branch) and the output   */
+/* size rule of :92-199. Pads are (top, left, bottom, right) = ONNX order    */
+/* pads[0], pads[1], pads[2], pads[3].                                        */
+/* ------------------------------------------------------------------------- */
+void or_maxpool2d_f32(const float *x, float *y, int NC, int H, int W, int kh, int kw,
+                      int pt, int pl, int pb, int pr, int sh, int sw)
+{
+    const int OH = (H + pt + pb - kh) / sh + 1;
+    const int OW = (W + pl + pr - kw) / sw + 1;
+    size_t o = 0;
+    for (int nc = 0; nc < NC; ++nc) {
+        const float *xi = x + (size_t)nc * H * W;
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow) {
+                float v = -INFINITY;
+                for (int r = 0; r < kh; ++r) {
+                    const int ih = oh * sh - pt + r;
+                    if (ih < 0 || ih >= H) continue;
+                    for (int s = 0; s < kw; ++s) {
+                        const int iw = ow * sw - pl + s;
+                        if (iw < 0 || iw >= W) continue;
+                        const float xv = xi[(size_t)ih * W + iw];
+                        if (xv > v) v = xv;
+                    }
+                }
+                y[o++] = v;
+            }
+    }
+}
+
+/* int8 variant of the same pooling (quantized activations keep their scale). */
+void or_maxpool2d_s8(const int8_t *x, int8_t *y, int NC, int H, int W, int kh, int kw,
+                     int pt, int pl, int pb, int pr, int sh, int sw)
+{
+    const int OH = (H + pt + pb - kh) / sh + 1;
+    const int OW = (W + pl + pr - kw) / sw + 1;
+    size_t o = 0;
+    for (int nc = 0; nc < NC; ++nc) {
+        const int8_t *xi = x + (size_t)nc * H * W;
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow) {
+                int v = -128;
+                for (int r = 0; r < kh; ++r) {
+                    const int ih = oh * sh - pt + r;
+                    if (ih < 0 || ih >= H) continue;
+                    for (int s = 0; s < kw; ++s) {
+                        const int iw = ow * sw - pl + s;
+                        if (iw < 0 || iw >= W) continue;
+                        const int xv = xi[(size_t)ih * W + iw];
+                        if (xv > v) v = xv;
+                    }
+                }
+                y[o++] = (int8_t)v;
+            }
+    }
+}
+
+/* ========================================================================= */
+/* Quantized operators. The reference has none; semantics are ONNX's         */
+/* QuantizeLinear / DequantizeLinear / QLinearMatMul / QLinearConv with one   */
+/* fixed requantisation formula:                                             */
+/*    r = rintf( (float)acc * scale )      (int32->fp32 RNE, one fp32 multiply,*/
+/*                                          round half to even)              */
+/*    q = clamp(r + zp, lo, 127),  lo = relu ? max(zp,-128) : -128           */
+/* ========================================================================= */
+
+static inline int8_t or_requant(int32_t acc, float scale, int zp, int relu)
+{
+    const float f = (float)acc;          /* RNE conversion */
+    const float p = f * scale;           /* one fp32 multiply */
+    float r = rintf(p);                  /* RNE in the default rounding mode */
+    if (r > 1024.0f) r = 1024.0f;        /* keep the int conversion in range */
+    if (r < -1024.0f) r = -1024.0f;
+    int q = (int)r + zp;
+    int lo = -128;
+    if (relu && zp > lo) lo = zp;
+    if (q < lo) q = lo;
+    if (q > 127) q = 127;
+    return (int8_t)q;
+}
+
+int8_t or_requant_one(int32_t acc, float scale, int zp, int relu)
+{
+    return or_requant(acc, scale, zp, relu);
+}
+
+/* QuantizeLinear: q = sat(rne(x / s) + zp), computed as rintf(x * (1/s)) is NOT
+ * used -- the division is performed in fp32 exactly as ONNX writes it. */
+void or_quantize_f32_s8(const float *x, int8_t *q, size_t len, float scale, int zp)
+{
+    for (size_t i = 0; i < len; ++i) {
+        float r = rintf(x[i] / scale);
+        if (r > 1024.0f) r = 1024.0f;
+        if (r < -1024.0f) r = -1024.0f;
+        int v = (int)r + zp;
+        if (v < -128) v = -128;
+        if (v > 127) v = 127;
+        q[i] = (int8_t)v;
+    }
+}
+
+/* DequantizeLinear: x = (q - zp) * s. */
+void or_dequantize_s8_f32(const int8_t *q, float *x, size_t len, float scale, int zp)
+{
+    for (size_t i = 0; i < len; ++i) x[i] = (float)((int)q[i] - zp) * scale;
+}
+
+/* Raw int32 accumulators of A[M,K] (row-major int8) times B (row-major [K,N], or
+ * [N,K] when transB), with zero-points removed: acc = sum (a-zpa)*(b-zpb). */
+void or_igemm_s8(int transB, int M, int N, int K, const int8_t *A, const int8_t *B,
+                 int zpa, int zpb, int32_t *acc)
+{
+    int32_t *row = (int32_t *)malloc((size_t)N * sizeof(int32_t));
+    for (int i = 0; i < M; ++i) {
+        memset(row, 0, (size_t)N * sizeof(int32_t));
+        if (!transB) {
+            for (int l = 0; l < K; ++l) {
+                const int32_t a = (int32_t)A[(size_t)i * K + l] - zpa;
+                const int8_t *bl = B + (size_t)l * N;
+                for (int j = 0; j < N; ++j) row[j] += a * ((int32_t)bl[j] - zpb);
+            }
+        } else {
+            const int8_t *ai = A + (size_t)i * K;
+            for (int j = 0; j < N; ++j) {
+                const int8_t *bj = B + (size_t)j * K;
+                int32_t s = 0;
+                for (int l = 0; l < K; ++l) s += ((int32_t)ai[l] - zpa) * ((int32_t)bj[l] - zpb);
+                row[j] = s;
+            }
+        }
+        memcpy(acc + (size_t)i * N, row, (size_t)N * sizeof(int32_t));
+    }
+    free(row);
+}
+
+/* QLinearMatMul-style GEMM: int32 accumulate, optional int32 bias per output
+ * column, per-output-column fp32 scale, requantise to int8. */
+void or_qgemm_s8(int transB, int M, int N, int K, const int8_t *A, const int8_t *B,
+                 int zpa, const float *scale, const int32_t *bias, int zpy, int relu,
+                 int8_t *Y)
+{
+    int32_t *acc = (int32_t *)malloc((size_t)M * N * sizeof(int32_t));
+    or_igemm_s8(transB, M, N, K, A, B, zpa, 0, acc);
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j) {
+            int32_t a = acc[(size_t)i * N + j];
+            if (bias) a += bias[j];
+            Y[(size_t)i * N + j] = or_requant(a, scale[j], zpy, relu);
+        }
+    free(acc);
+}
+
+/* Same product with the accumulator dequantised to fp32: y = (float)(acc+bias)*scale[n]
+ * (the logits layer of a quantized network). */
+void or_qgemm_s8_f32out(int transB, int M, int N, int K, const int8_t *A, const int8_t *B,
+                        int zpa, const float *scale, const int32_t *bias, int relu, float *Y)
+{
+    int32_t *acc = (int32_t *)malloc((size_t)M * N * sizeof(int32_t));
+    or_igemm_s8(transB, M, N, K, A, B, zpa, 0, acc);
+    for (int i = 0; i < M; ++i)
+        for (int j = 0; j < N; ++j) {
+            int32_t a = acc[(size_t)i * N + j];
+            if (bias) a += bias[j];
+            float v = (float)a * scale[j];
+            if (relu && !(v > 0)) v = 0;
+            Y[(size_t)i * N + j] = v;
+        }
+    free(acc);
+}
+
+/* Raw int32 accumulators of a quantized NCHW convolution: padding cells
+ * contribute (zpx - zpx) = 0, weights are symmetric (zero-point 0). */
+int or_iconv2d_s8(const int8_t *x, const int8_t *w, int32_t *acc, int N, int C, int H,
+                  int W, int OC, int kh, int kw, int ph, int pw, int sh, int sw,
+                  int groups, int zpx)
+{
+    if (groups < 1 || C % groups || OC % groups) return -1;
+    const int icg = C / groups, ocg = OC / groups;
+    const int OH = (H + 2 * ph - kh) / sh + 1;
+    const int OW = (W + 2 * pw - kw) / sw + 1;
+    if (OH <= 0 || OW <= 0) return -1;
+    for (int n = 0; n < N; ++n)
+        for (int oc = 0; oc < OC; ++oc) {
+            const int g = oc / ocg;
+            int32_t *out = acc + ((size_t)n * OC + oc) * OH * OW;
+            memset(out, 0, (size_t)OH * OW * sizeof(int32_t));
+            for (int ic = 0; ic < icg; ++ic) {
+                const int8_t *xi = x + ((size_t)n * C + (size_t)g * icg + ic) * H * W;
+                for (int r = 0; r < kh; ++r)
+                    for (int s = 0; s < kw; ++s) {
+                        const int32_t wv = w[(((size_t)oc * icg + ic) * kh + r) * kw + s];
+                        if (wv == 0) continue;
+                        for (int oh = 0; oh < OH; ++oh) {
+                            const int ih = oh * sh - ph + r;
+                            if (ih < 0 || ih >= H) continue;
+                            for (int ow = 0; ow < OW; ++ow) {
+                                const int iw = ow * sw - pw + s;
+                                if (iw < 0 || iw >= W) continue;
+                                out[(size_t)oh * OW + ow] +=
+                                    wv * ((int32_t)xi[(size_t)ih * W + iw] - zpx);
+                            }
+                        }
+                    }
+            }
+        }
+    return 0;
+}
+
+/* QLinearConv: accumulators above + int32 bias per output channel, per-output-channel
+ * scale, requantise, optional fused ReLU (clamp at zpy). NCHW in and out. */
+int or_qconv2d_s8(const int8_t *x, const int8_t *w, const int32_t *bias,
+                  const float *scale, int8_t *y, int N, int C, int H, int W, int OC,
+                  int kh, int kw, int ph, int pw, int sh, int sw, int groups, int zpx,
+                  int zpy, int relu)
+{
+    const int OH = (H + 2 * ph - kh) / sh + 1;
+    const int OW = (W + 2 * pw - kw) / sw + 1;
+    if (OH <= 0 || OW <= 0) return -1;
+    const size_t len = (size_t)N * OC * OH * OW;
+    int32_t *acc = (int32_t *)malloc(len * sizeof(int32_t));
+    if (!acc) return -2;
+    const int rc = or_iconv2d_s8(x, w, acc, N, C, H, W, OC, kh, kw, ph, pw, sh, sw, groups, zpx);
+    if (rc) { free(acc); return rc; }
+    const size_t plane = (size_t)OH * OW;
+    for (size_t i = 0; i < len; ++i) {
+        const int oc = (int)((i / plane) % (size_t)OC);
+        int32_t a = acc[i];
+        if (bias) a += bias[oc];
+        y[i] = or_requant(a, scale[oc], zpy, relu);
+    }
+    free(acc);
+    return 0;
+}
+
+/* ========================================================================= */
+/* FP8 e4m3 (OCP "e4m3fn": bias 7, no infinities, 0x7f/0xff = NaN, max 448)   */
+/* and bfloat16 helpers.                                                     */
+/* ========================================================================= */
+
+float or_e4m3_to_f32(uint8_t v)
+{
+    const int sign = v >> 7, e = (v >> 3) & 0xf, m = v & 7;
+    float r;
+    if (e == 0xf && m == 7) return NAN;
+    if (e == 0) r = ldexpf((float)m, -9);            /* subnormal: m * 2^-3 * 2^-6 */
+    else r = ldexpf(1.0f + (float)m / 8.0f, e - 7);
+    return sign ? -r : r;
+}
+
+/* fp32 -> e4m3 with round-to-nearest-even, saturating to +-448 (NaN stays NaN). */
+uint8_t or_f32_to_e4m3_sat(float x)
+{
+    if (x != x) return 0x7f;
+    const uint8_t s = signbit(x) ? 0x80 : 0;
+    float a = fabsf(x);
+    if (a >= 448.0f) return (uint8_t)(s | 0x7e);
+    if (a < ldexpf(1.0f, -10)) return s;             /* below half of min subnormal */
+    int e;
+    (void)frexpf(a, &e);                             /* a = f * 2^e, f in [0.5,1) */
+    int ex = e - 1;                                  /* a = 1.xxx * 2^ex */
+    if (ex < -6) ex = -6;                            /* subnormal range */
+    const float step = ldexpf(1.0f, ex - 3);         /* spacing of representable values */
+    const float q = rintf(a / step);                 /* exact: power-of-two division */
+    const float r = q * step;
+    if (r >= 448.0f) return (uint8_t)(s | 0x7e);
+    if (r < ldexpf(1.0f, -6)) return (uint8_t)(s | (int)(r / ldexpf(1.0f, -9)));
+    (void)frexpf(r, &e);
+    ex = e - 1;
+    const int mant = (int)((r / ldexpf(1.0f, ex) - 1.0f) * 8.0f);
+    return (uint8_t)(s | ((ex + 7) << 3) | mant);
+}
+
+/* fp32 -> bf16 bits, round to nearest even (NaN quieted). */
+uint16_t or_f32_to_bf16(float x)
+{
+    uint32_t u;
+    memcpy(&u, &x, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+
+float or_bf16_to_f32(uint16_t b)
+{
+    const uint32_t u = (uint32_t)b << 16;
+    float x;
+    memcpy(&x, &u, 4);
+    return x;
+}
+
+/* FP8 GEMM: A[M,K] e4m3 row-major; B row-major [K,N] (or [N,K] when transB);
+ *   t = (sum_k a*b accumulated in fp32, increasing k) * (sa*sb)  [+ bias[n]]
+ * written as bf16 (RNE) into Ybf16 and/or as fp32 into Yf32 (either may be NULL).
+ * acc64 != 0 accumulates in double instead: the "truth" that the stated FP8
+ * tolerance is measured against. */
+void or_gemm_fp8(int transB, int M, int N, int K, const uint8_t *A, const uint8_t *B,
+                 float sa, float sb, const float *bias, uint16_t *Ybf16, float *Yf32,
+                 int acc64)
+{
+    float lut[256];
+    for (int i = 0; i < 256; ++i) lut[i] = or_e4m3_to_f32((uint8_t)i);
+    const float s = sa * sb;
+    float *bt = (float *)malloc((size_t)K * sizeof(float));
+    for (int j = 0; j < N; ++j) {
+        for (int l = 0; l < K; ++l)
+            bt[l] = lut[transB ? B[(size_t)j * K + l] : B[(size_t)l * N + j]];
+        for (int i = 0; i < M; ++i) {
+            const uint8_t *ai = A + (size_t)i * K;
+            float t;
+            if (acc64) {
+                double d = 0.0;
+                for (int l = 0; l < K; ++l) d += (double)lut[ai[l]] * (double)bt[l];
+                d *= (double)s;
+                if (bias) d += (double)bias[j];
+                t = (float)d;
+            } else {
+                float f = 0.0f;
+                for (int l = 0; l < K; ++l) f += lut[ai[l]] * bt[l];
+                t = f * s;
+                if (bias) t = t + bias[j];
+            }
+            if (Yf32) Yf32[(size_t)i * N + j] = t;
+            if (Ybf16) Ybf16[(size_t)i * N + j] = or_f32_to_bf16(t);
+        }
+    }
+    free(bt);
+}

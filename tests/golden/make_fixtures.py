@@ -1,0 +1,72 @@
+"""Collect the known-answer fixtures that the reference's own tests hold for the
+Gemm / Conv / MaxPool path into tests/golden/.
+
+Run in the authoring container only (it reads /root/reference, which does not exist
+on the GPU box):   python tests/golden/make_fixtures.py
+
+What is written:
+  tests/golden/onnx/<name>.onnx      byte copies of the reference's binary test models
+                                     (data files: graph + weights)
+  tests/golden/expected.json         the expected output arrays of the reference's
+                                     <name>.ref.hxx headers (numbers only) together with
+                                     the input each test feeds (ones / iota / literal list,
+                                     from TestCustomModelsFromONNX.cxx:330-349,372-391,
+                                     693-712,860-967,1023-1052)
+"""
+import json
+import os
+import re
+import shutil
+
+REF = "/root/reference/src/SOFIE_core/test/input_models"
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+# name -> (input kind, input shape, array name inside the ref header)
+CASES = {
+    "Linear_16": ("ones", [16, 100], "all_ones"),
+    "Linear_32": ("ones", [32, 100], "all_ones"),
+    "Linear_64": ("ones", [64, 100], "all_ones"),
+    "ConvWithPadding": ("iota", [1, 1, 5, 5], "all_ones"),
+    "ConvWithoutPadding": ("iota", [1, 1, 5, 5], "all_ones"),
+    "ConvWithAutopadSameLower": ("iota", [1, 1, 5, 5], "all_ones"),
+    "ConvWithStridesPadding": ("iota", [1, 1, 7, 5], "all_ones"),
+    "ConvWithStridesNoPadding": ("iota", [1, 1, 7, 5], "all_ones"),
+    "ConvWithAsymmetricPadding": ("iota", [1, 1, 7, 5], "all_ones"),
+    "MaxPool2d": ("literal", [1, 1, 5, 10], "output"),
+}
+
+# Input of the reference's MaxPool2d test (TestCustomModelsFromONNX.cxx:1027-1038).
+MAXPOOL2D_INPUT = [
+    0.6266, 0.1656, 0.2753, -0.4558, -1.4592, 0.9285, -1.3410, 1.3223, -0.5936, -1.3648,
+    -0.2989, 0.5901, -0.8845, -0.0433, 0.8314, -1.7159, -0.5765, 0.8678, 1.0257, 0.7847,
+    -0.3421, -1.2364, -0.5805, 0.4421, 1.2184, 0.5043, 1.6823, -1.0483, -2.2798, -1.8927,
+    0.7716, 0.0405, 0.3121, -0.3011, -0.3266, -1.9660, 1.0837, 0.2317, 0.9084, -0.3285,
+    -0.9398, -0.2065, -0.9499, -0.9739, -0.1288, -0.1375, -1.2612, 0.8810, 0.8506, 0.4455,
+]
+
+
+def numbers_of(header_text, array):
+    m = re.search(r"float\s+%s\s*\[\s*\]\s*=\s*\{(.*?)\}" % re.escape(array), header_text, re.S)
+    body = re.sub(r"//[^\n]*", "", m.group(1))
+    return [float(t.rstrip("f")) for t in re.findall(r"[-+]?(?:\d+\.?\d*|\.\d+)(?:[eE][-+]?\d+)?f?", body)]
+
+
+def main():
+    os.makedirs(os.path.join(HERE, "onnx"), exist_ok=True)
+    expected = {}
+    for name, (kind, shape, arr) in CASES.items():
+        shutil.copyfile(os.path.join(REF, name + ".onnx"), os.path.join(HERE, "onnx", name + ".onnx"))
+        os.chmod(os.path.join(HERE, "onnx", name + ".onnx"), 0o644)
+        with open(os.path.join(REF, "references", name + ".ref.hxx")) as f:
+            vals = numbers_of(f.read(), arr)
+        entry = {"input_kind": kind, "input_shape": shape, "expected": vals}
+        if kind == "literal":
+            entry["input"] = MAXPOOL2D_INPUT
+        expected[name] = entry
+    with open(os.path.join(HERE, "expected.json"), "w") as f:
+        json.dump(expected, f, indent=0)
+    print({k: len(v["expected"]) for k, v in expected.items()})
+
+
+if __name__ == "__main__":
+    main()

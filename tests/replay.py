@@ -1,0 +1,86 @@
+"""Replay a decoded ONNX graph (Gemm / Relu / Conv / MaxPool / Flatten) through a backend.
+
+A backend is any object with the methods gemm_f32, relu_f32, conv2d_f32 and maxpool2d
+taking and returning numpy arrays: the CPU oracle module, or the HIP library wrapper.
+The attribute handling restates what the reference's operators do at Initialize time.
+"""
+import numpy as np
+
+
+def conv_pads_like_reference(attrs, kshape):
+    """Pads (h, w) that the reference's Conv finally passes to Im2col.
+
+    ROperator_Conv.hxx:136-158: absent pads with auto_pad NOTSET mean 1 on every side;
+    SAME_UPPER/SAME_LOWER start from k/2 and add one at the begin (UPPER) or end (LOWER)
+    for odd kernels; :387-401: asymmetric begin/end pads are averaged (integer division).
+    """
+    kh, kw = kshape
+    auto = attrs.get("auto_pad", "NOTSET")
+    pads = list(attrs.get("pads", []))
+    if auto == "NOTSET":
+        if not pads:
+            pads = [1, 1, 1, 1]
+    elif auto in ("SAME_UPPER", "SAME_LOWER"):
+        pads = [kh // 2, kw // 2, kh // 2, kw // 2]
+        if kh % 2 == 1:
+            pads[0 if auto == "SAME_UPPER" else 2] += 1
+        if kw % 2 == 1:
+            pads[1 if auto == "SAME_UPPER" else 3] += 1
+    elif auto == "VALID":
+        pads = [0, 0, 0, 0]
+    else:
+        raise RuntimeError("TMVA SOFIE Conv Op invalid fAutopad")
+    out_h_pad_total = pads[0] + pads[2]
+    out_w_pad_total = pads[1] + pads[3]
+    ph, pw = pads[0], pads[1]
+    if pads[0] != pads[2] or pads[1] != pads[3]:
+        ph = (pads[0] + pads[2]) // 2
+        pw = (pads[1] + pads[3]) // 2
+    return (ph, pw), (out_h_pad_total, out_w_pad_total)
+
+
+def run_graph(graph, feeds, backend):
+    """Evaluate the nodes in file order; returns the first graph output as numpy."""
+    env = dict(graph["initializers"])
+    env.update(feeds)
+    for node in graph["nodes"]:
+        op, a, ins = node["op_type"], node["attrs"], node["inputs"]
+        if op == "Gemm":
+            bias = env[ins[2]] if len(ins) > 2 else None
+            y = backend.gemm_f32(env[ins[0]], env[ins[1]], bias, alpha=a.get("alpha", 1.0),
+                                 beta=a.get("beta", 1.0) if bias is not None else 0.0,
+                                 transA=bool(a.get("transA", 0)), transB=bool(a.get("transB", 0)))
+        elif op == "Relu":
+            y = backend.relu_f32(env[ins[0]])
+        elif op == "Conv":
+            w = env[ins[1]]
+            (ph, pw), _ = conv_pads_like_reference(a, w.shape[2:])
+            bias = env[ins[2]] if len(ins) > 2 else None
+            y = backend.conv2d_f32(env[ins[0]], w, bias, pads=(ph, pw),
+                                   strides=tuple(a.get("strides", [1, 1])),
+                                   dilations=tuple(a.get("dilations", [1, 1])),
+                                   groups=a.get("group", 1))
+        elif op == "MaxPool":
+            y = backend.maxpool2d(env[ins[0]], tuple(a["kernel_shape"]),
+                                  tuple(a.get("strides", [1, 1])),
+                                  tuple(a.get("pads", [0, 0, 0, 0])))
+        elif op == "Flatten":
+            x = env[ins[0]]
+            y = np.ascontiguousarray(x).reshape(x.shape[0], -1)
+        else:
+            raise NotImplementedError(op)
+        env[node["outputs"][0]] = y
+    return env[graph["outputs"][0][0]]
+
+
+def fixture_input(entry):
+    shape = entry["input_shape"]
+    n = int(np.prod(shape))
+    kind = entry["input_kind"]
+    if kind == "ones":
+        x = np.ones(n, np.float32)
+    elif kind == "iota":
+        x = np.arange(n, dtype=np.float32)
+    else:
+        x = np.array(entry["input"], np.float32)
+    return x.reshape(shape)

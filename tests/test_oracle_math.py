@@ -1,0 +1,308 @@
+"""Pins the CPU oracle with facts that do not depend on its own formulas: float64 /
+int64 closed forms, torch CPU operators, brute force on tiny inputs, exact rational
+rounding, and library fp8 / bf16 casts. The reference has no quantized or FP8 operators,
+so for those these checks are the only pin ("parity unpinned" by the reference)."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import oracle
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ----------------------------------------------------------------------------- fp32 Gemm
+@pytest.mark.parametrize("transA,transB,alpha,beta,relu", [
+    (0, 0, 1.0, 1.0, False), (0, 1, 1.0, 1.0, True), (1, 0, 0.5, 2.0, False),
+    (1, 1, -1.25, 0.0, True), (0, 0, 1.0, 0.0, False)])
+def test_gemm_f32_closed_form(transA, transB, alpha, beta, relu):
+    r = rng(1)
+    M, N, K = 37, 29, 53
+    A = r.standard_normal((K, M) if transA else (M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if transB else (K, N)).astype(np.float32)
+    bias = r.standard_normal(N).astype(np.float32) if beta != 0.0 else None
+    y = oracle.gemm_f32(A, B, bias, alpha, beta, bool(transA), bool(transB), relu)
+    a = (A.T if transA else A).astype(np.float64)
+    b = (B.T if transB else B).astype(np.float64)
+    t = alpha * (a @ b) + (beta * bias.astype(np.float64) if bias is not None else 0.0)
+    if relu:
+        t = np.maximum(t, 0)
+    assert np.max(np.abs(y - t)) <= 1e-5 * np.max(np.abs(t))
+
+
+def test_gemm_without_bias_and_nonzero_beta_is_an_error():
+    A = np.ones((2, 2), np.float32)
+    with pytest.raises(RuntimeError):
+        oracle.gemm_f32(A, A, None, 1.0, 1.0)
+
+
+def test_gemm_full_shape_bias_is_taken_as_is():
+    r = rng(2)
+    A = r.standard_normal((5, 7)).astype(np.float32)
+    B = r.standard_normal((7, 3)).astype(np.float32)
+    Cfull = r.standard_normal((5, 3)).astype(np.float32)
+    y = oracle.gemm_f32(A, B, Cfull)
+    assert np.allclose(y, A.astype(np.float64) @ B + Cfull, rtol=1e-5, atol=1e-5)
+
+
+# ----------------------------------------------------------------------------- fp32 Conv
+def brute_conv(x, w, b, ph, pw, sh, sw, dh, dw, groups):
+    N, C, H, W = x.shape
+    OC, icg, kh, kw = w.shape
+    OH = (H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1
+    OW = (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1
+    y = np.zeros((N, OC, OH, OW), np.float64)
+    ocg = OC // groups
+    for n in range(N):
+        for oc in range(OC):
+            g = oc // ocg
+            for oh in range(OH):
+                for ow in range(OW):
+                    s = 0.0
+                    for ic in range(icg):
+                        for r in range(kh):
+                            for q in range(kw):
+                                ih, iw = oh * sh - ph + r * dh, ow * sw - pw + q * dw
+                                if 0 <= ih < H and 0 <= iw < W:
+                                    s += float(x[n, g * icg + ic, ih, iw]) * float(w[oc, ic, r, q])
+                    y[n, oc, oh, ow] = s + (float(b[oc]) if b is not None else 0.0)
+    return y
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(N=2, C=3, H=7, W=6, OC=4, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, bias=True),
+    dict(N=1, C=4, H=9, W=8, OC=6, k=(3, 2), p=(0, 1), s=(2, 1), d=(1, 1), g=2, bias=False),
+    dict(N=2, C=2, H=8, W=8, OC=2, k=(2, 2), p=(1, 1), s=(2, 2), d=(1, 1), g=1, bias=True),
+    dict(N=1, C=2, H=10, W=9, OC=3, k=(3, 3), p=(2, 2), s=(1, 1), d=(2, 2), g=1, bias=True),
+])
+def test_conv2d_f32_against_brute_force_and_torch(cfg):
+    r = rng(3)
+    x = r.standard_normal((cfg["N"], cfg["C"], cfg["H"], cfg["W"])).astype(np.float32)
+    w = r.standard_normal((cfg["OC"], cfg["C"] // cfg["g"]) + cfg["k"]).astype(np.float32)
+    b = r.standard_normal(cfg["OC"]).astype(np.float32) if cfg["bias"] else None
+    y = oracle.conv2d_f32(x, w, b, cfg["p"], cfg["s"], cfg["d"], cfg["g"])
+    t = brute_conv(x, w, b, *cfg["p"], *cfg["s"], *cfg["d"], cfg["g"])
+    assert y.shape == t.shape
+    assert np.max(np.abs(y - t)) <= 1e-5 * np.max(np.abs(t))
+    tt = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(),
+                  torch.from_numpy(b).double() if b is not None else None,
+                  stride=cfg["s"], padding=cfg["p"], dilation=cfg["d"], groups=cfg["g"]).numpy()
+    assert np.max(np.abs(y - tt)) <= 1e-5 * np.max(np.abs(tt))
+
+
+def test_conv_1x1_is_a_gemm_and_ones_kernel_is_a_box_sum():
+    r = rng(4)
+    x = r.integers(-5, 6, (2, 8, 5, 5)).astype(np.float32)
+    w = r.integers(-3, 4, (6, 8, 1, 1)).astype(np.float32)
+    y = oracle.conv2d_f32(x, w)
+    t = np.einsum("oc,nchw->nohw", w[:, :, 0, 0], x)
+    assert np.array_equal(y, t)
+    ones = np.ones((1, 8, 3, 3), np.float32)
+    yb = oracle.conv2d_f32(x, ones, pads=(1, 1))
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    tb = sum(xp[:, :, i:i + 5, j:j + 5] for i in range(3) for j in range(3)).sum(1, keepdims=True)
+    assert np.array_equal(yb, tb)
+
+
+def test_im2col_times_weights_equals_direct_conv():
+    r = rng(5)
+    x = r.integers(-4, 5, (3, 6, 7)).astype(np.float32)
+    w = r.integers(-2, 3, (5, 3, 3, 3)).astype(np.float32)
+    col = oracle.im2col(x, 3, 3, 1, 1, 1, 1)
+    y = (w.reshape(5, -1) @ col).reshape(1, 5, 6, 7)
+    assert np.array_equal(y, oracle.conv2d_f32(x[None], w, pads=(1, 1)))
+
+
+def test_relu_and_maxpool_against_torch():
+    r = rng(6)
+    x = r.standard_normal((2, 3, 9, 8)).astype(np.float32)
+    assert np.array_equal(oracle.relu_f32(x), np.maximum(x, 0))
+    for k, s, p in [((2, 2), (2, 2), (0, 0, 0, 0)), ((3, 2), (1, 1), (0, 0, 0, 0)),
+                    ((3, 3), (2, 2), (1, 1, 1, 1))]:
+        y = oracle.maxpool2d(x, k, s, p)
+        t = F.max_pool2d(torch.from_numpy(x), k, s, (p[0], p[1])).numpy()
+        assert np.array_equal(y, t)
+    q = r.integers(-128, 128, (2, 3, 8, 8)).astype(np.int8)
+    yq = oracle.maxpool2d(q, (2, 2), (2, 2))
+    tq = q.reshape(2, 3, 4, 2, 4, 2).max(axis=(3, 5))
+    assert np.array_equal(yq, tq)
+
+
+# ----------------------------------------------------------------------------- int8
+def exact_requant(acc, scale32, zp, relu):
+    """Independent statement: fp32(acc) and the fp32 product are obtained by exact
+    arithmetic followed by one correctly rounded conversion; half-even via Fraction."""
+    a32 = np.float32(acc)                                  # correctly rounded int->fp32
+    prod = np.float32(np.float64(a32) * np.float64(scale32))  # exact in fp64, one rounding
+    r = round(Fraction(float(prod)))                       # Python rounds halves to even
+    lo = max(zp, -128) if relu else -128
+    return int(min(127, max(lo, r + zp)))
+
+
+def test_requant_rounding_boundaries_exhaustive():
+    r = rng(7)
+    scales = [np.float32(0.5), np.float32(0.25), np.float32(1.0), np.float32(0.001953125),
+              np.float32(1e-3), np.float32(7.3e-3), np.float32(1.2e-4), np.float32(0.0123)]
+    for s in scales:
+        inv = int(round(1.0 / float(s)))
+        accs = set()
+        for q in range(-140, 141):                         # around every .5 boundary
+            c = int(round((q + 0.5) / float(s)))
+            accs.update(range(c - 3, c + 4))
+        accs.update([0, 1, -1, inv, -inv, 2 ** 24 + 1, -(2 ** 24) - 1, 2 ** 31 - 1, -(2 ** 31),
+                     16777217, 33554435])
+        accs.update(int(v) for v in r.integers(-2 ** 31, 2 ** 31, 200))
+        for acc in accs:
+            acc = max(-(2 ** 31), min(2 ** 31 - 1, acc))
+            for zp, relu in [(0, False), (-128, True), (3, True), (-5, False)]:
+                assert oracle.requant_one(acc, s, zp, relu) == exact_requant(acc, s, zp, relu), \
+                    (acc, s, zp, relu)
+
+
+def test_rne_examples():
+    assert [oracle.requant_one(a, 0.5) for a in (1, 3, 5, -1, -3, -5)] == [0, 2, 2, 0, -2, -2]
+    assert oracle.requant_one(10 ** 6, 1.0) == 127 and oracle.requant_one(-10 ** 6, 1.0) == -128
+    assert oracle.requant_one(-10, 1.0, zp=-128, relu=True) == -128
+
+
+@pytest.mark.parametrize("transB", [False, True])
+def test_igemm_and_qgemm_against_int64(transB):
+    r = rng(8)
+    M, N, K = 33, 47, 300
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    B = r.integers(-127, 128, (N, K) if transB else (K, N)).astype(np.int8)
+    acc = oracle.igemm_s8(A, B, transB)
+    b = B.T if transB else B
+    t = A.astype(np.int64) @ b.astype(np.int64)
+    assert np.array_equal(acc, t)
+    ti = torch._int_mm(torch.from_numpy(np.ascontiguousarray(np.pad(A, ((0, 31), (0, 4))))),
+                       torch.from_numpy(np.ascontiguousarray(np.pad(b, ((0, 4), (0, 1))))))
+    assert np.array_equal(ti.numpy()[:M, :N], t)
+    scale = r.uniform(2e-5, 2e-4, N).astype(np.float32)
+    bias = r.integers(-5000, 5000, N).astype(np.int32)
+    y = oracle.qgemm_s8(A, B, scale, bias, transB, zpy=-3, relu=True)
+    want = np.array([[exact_requant(int(t[i, j] + bias[j]), scale[j], -3, True)
+                      for j in range(N)] for i in range(M)], np.int8)
+    assert np.array_equal(y, want)
+    yf = oracle.qgemm_s8_f32out(A, B, scale, bias, transB)
+    wf = ((t + bias).astype(np.float32) * scale).astype(np.float32)
+    assert np.array_equal(yf, wf)
+
+
+def test_igemm_zero_points():
+    r = rng(9)
+    A = r.integers(-128, 128, (5, 40)).astype(np.int8)
+    B = r.integers(-128, 128, (40, 6)).astype(np.int8)
+    acc = oracle.igemm_s8(A, B, False, zpa=-128, zpb=7)
+    assert np.array_equal(acc, (A.astype(np.int64) + 128) @ (B.astype(np.int64) - 7))
+
+
+def test_quantize_dequantize():
+    r = rng(10)
+    x = r.uniform(0, 1, 1000).astype(np.float32)
+    s = np.float32(1 / 255)
+    q = oracle.quantize_f32_s8(x, s, -128)
+    want = np.clip(np.rint(x / s) - 128, -128, 127).astype(np.int8)
+    assert np.array_equal(q, want)
+    halves = (np.arange(-6, 7, dtype=np.float32) + np.float32(0.5))
+    assert np.array_equal(oracle.quantize_f32_s8(halves, 1.0, 0),
+                          np.array([round(Fraction(float(v))) for v in halves], np.int8))
+    assert np.array_equal(oracle.dequantize_s8_f32(q, s, -128),
+                          ((q.astype(np.int32) + 128).astype(np.float32) * s))
+
+
+def test_qconv_against_int64_convolution():
+    r = rng(11)
+    x = r.integers(-128, 128, (2, 6, 7, 6)).astype(np.int8)
+    w = r.integers(-127, 128, (8, 3, 3, 3)).astype(np.int8)
+    zpx = -128
+    acc = oracle.iconv2d_s8(x, w, (1, 1), (1, 1), groups=2, zpx=zpx)
+    xs = x.astype(np.float64) - zpx                       # padding then contributes 0
+    t = F.conv2d(torch.from_numpy(xs), torch.from_numpy(w.astype(np.float64)), None,
+                 stride=1, padding=1, groups=2).numpy()
+    assert np.array_equal(acc, t.astype(np.int64))
+    scale = r.uniform(1e-4, 1e-3, 8).astype(np.float32)
+    bias = r.integers(-3000, 3000, 8).astype(np.int32)
+    y = oracle.qconv2d_s8(x, w, scale, bias, (1, 1), (1, 1), 2, zpx, -128, True)
+    tt = t.astype(np.int64) + bias[None, :, None, None]
+    want = np.empty_like(y)
+    for idx in np.ndindex(*y.shape):
+        want[idx] = exact_requant(int(tt[idx]), scale[idx[1]], -128, True)
+    assert np.array_equal(y, want)
+
+
+def test_integer_valued_fp32_conv_pins_int8_accumulators():
+    """For integer data with |acc| < 2^24 the fp32 Conv path (pinned by the reference's
+    fixtures) is exact, so it fixes the int32 accumulators of the int8 path."""
+    r = rng(12)
+    x = r.integers(-15, 16, (2, 8, 9, 9)).astype(np.int8)
+    w = r.integers(-15, 16, (4, 8, 3, 3)).astype(np.int8)
+    acc = oracle.iconv2d_s8(x, w, (1, 1), (1, 1))
+    yf = oracle.conv2d_f32(x.astype(np.float32), w.astype(np.float32), None, (1, 1))
+    assert np.array_equal(acc, yf.astype(np.int32))
+    A = r.integers(-15, 16, (16, 1024)).astype(np.int8)
+    B = r.integers(-15, 16, (1024, 24)).astype(np.int8)
+    assert np.array_equal(oracle.igemm_s8(A, B),
+                          oracle.gemm_f32(A.astype(np.float32), B.astype(np.float32),
+                                          beta=0.0).astype(np.int32))
+
+
+# ----------------------------------------------------------------------------- fp8 / bf16
+def test_e4m3_table_against_torch_and_closed_form():
+    table = oracle.e4m3_table()
+    codes = torch.arange(256, dtype=torch.uint8)
+    tt = codes.view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.isnan(table), np.isnan(tt))
+    ok = ~np.isnan(tt)
+    assert np.array_equal(table[ok], tt[ok])
+    assert table[0x7e] == 448.0 and table[0x08] == 2.0 ** -6 and table[0x01] == 2.0 ** -9
+
+
+def test_e4m3_encode_against_torch_cast():
+    r = rng(13)
+    x = np.concatenate([r.standard_normal(4000).astype(np.float32) * 50,
+                        r.uniform(-1e-2, 1e-2, 2000).astype(np.float32),
+                        oracle.e4m3_table()[~np.isnan(oracle.e4m3_table())],
+                        np.array([0.0, -0.0, 448.0, -448.0, 1000.0, -1e9, 464.0, 463.9, 2 ** -10,
+                                  2 ** -10 * 1.01, 2 ** -9 * 1.5, 2 ** -9 * 2.5], np.float32)])
+    mine = oracle.e4m3_encode(x)
+    clamped = torch.from_numpy(np.clip(x, -448, 448))
+    theirs = clamped.to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    # -0.0 and +0.0 may differ in sign bit after underflow; compare decoded values
+    assert np.array_equal(oracle.e4m3_decode(mine), oracle.e4m3_decode(theirs))
+
+
+def test_bf16_round_to_nearest_even_against_torch():
+    r = rng(14)
+    x = np.concatenate([r.standard_normal(5000).astype(np.float32) * 100,
+                        np.array([1.0, 1.00390625, 1.01171875, -3.0e38, 1e-40, 0.0], np.float32)])
+    mine = oracle.bf16_encode(x)
+    theirs = torch.from_numpy(x).bfloat16().view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(mine, theirs)
+    assert np.array_equal(oracle.bf16_decode(mine),
+                          torch.from_numpy(x).bfloat16().float().numpy())
+
+
+@pytest.mark.parametrize("transB", [False, True])
+def test_gemm_fp8_against_float64(transB):
+    r = rng(15)
+    M, N, K = 24, 40, 512
+    a = r.standard_normal((M, K)).astype(np.float32)
+    b = r.standard_normal((N, K) if transB else (K, N)).astype(np.float32)
+    sa, sb = np.float32(np.abs(a).max() / 448), np.float32(np.abs(b).max() / 448)
+    A, B = oracle.e4m3_encode(a / sa), oracle.e4m3_encode(b / sb)
+    bias = r.standard_normal(N).astype(np.float32)
+    yb, yf = oracle.gemm_fp8(A, B, sa, sb, bias, transB)
+    da, db = oracle.e4m3_decode(A).astype(np.float64), oracle.e4m3_decode(B).astype(np.float64)
+    if transB:
+        db = db.T
+    truth = (da @ db) * (np.float64(sa) * np.float64(sb)) + bias
+    assert np.max(np.abs(yf - truth)) <= 2e-6 * np.max(np.abs(truth)) * np.sqrt(K)
+    assert np.array_equal(yb, oracle.bf16_encode(yf))
+    yb64, yf64 = oracle.gemm_fp8(A, B, sa, sb, bias, transB, acc64=True)
+    assert np.max(np.abs(yf64 - truth)) <= 1e-6 * np.max(np.abs(truth))
