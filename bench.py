@@ -1,0 +1,185 @@
+#!/usr/bin/env python3
+"""Benchmark of the SOFIE hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): standalone int8 GEMM with QLinearMatMul
+semantics, M=N=K=4096, A and B int8 uniform in [-127,127], per-output-channel fp32 scales
+uniform in [1e-3,1e-2], int32 accumulate, round-half-to-even requantise to int8. One "step"
+is one call of sofie_hip_qgemm_s8 on device-resident operands. Prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--extras]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA, 5.0 POP/s
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_FP32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def cpu_baseline_int8(A, B, scale, rows):
+    """The oracle (a scalar C port of the same arithmetic) on the first `rows` rows of A."""
+    from oracle import oracle
+    t0 = time.perf_counter()
+    y = oracle.qgemm_s8(A[:rows], B, scale)
+    dt = time.perf_counter() - t0
+    ops = 2.0 * rows * B.shape[0] * B.shape[1]
+    return y, {"value": ops / dt / 1e12, "unit": "TOPS", "cores": 1, "kind": "port",
+               "sample": "oracle/sofie_oracle.c or_qgemm_s8 on the first %d of %d rows of A against the full B "
+                         "(%.1f GOP, %.1f s, gcc -O2, 1 thread)" % (rows, A.shape[0], ops / 1e9, dt)}
+
+
+def time_launches(ctx, fn, steps, warmup):
+    """HIP events on the stream the kernels run on; returns average ms per launch."""
+    for _ in range(warmup):
+        fn()
+    ctx.sync()
+    ctx.timer_start()
+    for _ in range(steps):
+        fn()
+    return ctx.timer_stop() / steps
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-rows", type=int, default=1024)
+    ap.add_argument("--extras", action="store_true", help="also time the FP8 GEMM, fp32 GEMM and conv layers")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collective, no sharding "
+                 "code exists). Run with --gpus 1." % args.gpus)
+
+    import torch
+    from sofie_amd import lib as L
+    from sofie_amd import ops
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible (the HIP library has no CPU fallback)")
+    ctx = ops.default_context()
+
+    n = 4096
+    rng = np.random.default_rng(0)
+    A = rng.integers(-127, 128, (n, n)).astype(np.int8)
+    B = rng.integers(-127, 128, (n, n)).astype(np.int8)
+    scale = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
+    dA, dB, dS = ctx.dev(A), ctx.dev(B), ctx.dev(scale)
+    dY = ctx.empty((n, n), torch.int8)
+
+    def step():
+        ctx.check(ctx.lib.sofie_hip_qgemm_s8(ctx.h, 0, n, n, n, ctx.ptr(dA), n, ctx.ptr(dB), n, ctx.ptr(dS), None,
+                                             0, L.ACT_NONE, ctx.ptr(dY), n, L.OUT_S8))
+
+    # warm-up, then EXACTLY `steps` timed steps bracketed by device synchronisation
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    ops_per_step = 2.0 * n * n * n
+    tops = ops_per_step / (ms_per_step * 1e-3) / 1e12
+
+    # kernel duration from HIP events on the launch stream
+    kernel_ms = time_launches(ctx, step, args.steps, 2)
+    achieved = ops_per_step / (kernel_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "int8/FP8 GEMM TOPS & % MFMA peak; model inferences/sec at batch 4096",
+        "value": tops, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8", "data": "synthetic",
+        "config": {"workload": "int8 GEMM (QLinearMatMul) M=N=K=4096, A [M,K] and B [K,N] int8 U[-127,127], "
+                               "zero-point 0, per-column fp32 scale U[1e-3,1e-2], int32 accumulate, RNE requantise "
+                               "to int8, operands resident in HBM", "M": n, "N": n, "K": n, "seed": 0},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_INT8_TOPS, "traffic": None, "kernel": "k_gemm_bytes<MmaI8,...>",
+                     "kernel_ms": kernel_ms, "ops_per_launch": ops_per_step,
+                     "note": "unit counts int8 multiply-add as 2 ops (TOP/s)"},
+    }
+
+    # parity spot check inside the benchmark: the timed output against the oracle on a few rows
+    if not args.no_cpu:
+        y_ref, base = cpu_baseline_int8(A, B, scale, args.cpu_rows)
+        y_gpu = dY[:args.cpu_rows].cpu().numpy()
+        out["cpu_baseline"] = base
+        out["parity_rows_checked"] = int(args.cpu_rows)
+        out["parity_bit_exact"] = bool(np.array_equal(y_gpu, y_ref))
+    else:
+        out["cpu_baseline"] = None
+
+    if args.extras:
+        out["extras"] = extras(ctx, torch, L, ops, rng)
+    print(json.dumps(out))
+
+
+def extras(ctx, torch, L, ops, rng):
+    """Secondary figures of the other BASELINE.json configurations (not the headline value)."""
+    ex = {}
+    # pre-transposed weights: the layout a Session keeps B in when it is an initializer
+    n = 4096
+    A = ctx.dev(rng.integers(-127, 128, (n, n)).astype(np.int8))
+    Bt = ctx.dev(rng.integers(-127, 128, (n, n)).astype(np.int8))
+    S = ctx.dev(rng.uniform(1e-3, 1e-2, n).astype(np.float32))
+    Y = ctx.empty((n, n), torch.int8)
+    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_qgemm_s8(
+        ctx.h, 1, n, n, n, ctx.ptr(A), n, ctx.ptr(Bt), n, ctx.ptr(S), None, 0, 0, ctx.ptr(Y), n, L.OUT_S8)), 50, 5)
+    ex["int8_gemm_4096_transB"] = {"ms": ms, "tops": 2.0 * n ** 3 / ms / 1e9, "frac_peak": 2.0 * n ** 3 / ms / 1e9 / PEAK_INT8_TOPS}
+    # FP8 GEMM 8192 x 8192 x 4096, bf16 out, fused bias
+    M, N, K = 8192, 8192, 4096
+    A8 = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=ctx.device)
+    B8 = torch.randint(0, 120, (K, N), dtype=torch.uint8, device=ctx.device)
+    bias = torch.randn(N, device=ctx.device)
+    Y16 = ctx.empty((M, N), torch.bfloat16)
+    for tb, Bm in ((0, B8), (1, B8.t().contiguous())):
+        ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_gemm_fp8(
+            ctx.h, tb, M, N, K, ctx.ptr(A8), K, ctx.ptr(Bm), Bm.shape[1], 0.01, 0.01, ctx.ptr(bias), ctx.ptr(Y16), N,
+            L.OUT_BF16)), 20, 3)
+        fl = 2.0 * M * N * K
+        ex["fp8_gemm_8192x8192x4096_transB%d" % tb] = {"ms": ms, "tflops": fl / ms / 1e9,
+                                                       "frac_peak": fl / ms / 1e9 / PEAK_FP8_TFLOPS}
+    del A8, B8, Y16
+    # fp32 conv layer: batch 256, 64 -> 128 channels, 56x56, 3x3, pad 1, bias + ReLU
+    x = torch.rand(256, 64, 56, 56, device=ctx.device)
+    w = torch.randn(128, 64, 3, 3, device=ctx.device) * (2.0 / 576) ** 0.5
+    b = torch.randn(128, device=ctx.device) * 0.1
+    y = ctx.empty((256, 128, 56, 56), torch.float32)
+    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_conv2d_f32(
+        ctx.h, ctx.ptr(x), ctx.ptr(w), ctx.ptr(b), ctx.ptr(y), 256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)),
+        5, 1)
+    fl = 2.0 * 256 * 128 * 3136 * 576
+    ex["conv2d_f32_b256_64to128_56x56"] = {"ms": ms, "tflops": fl / ms / 1e9, "frac_peak": fl / ms / 1e9 / PEAK_FP32_TFLOPS}
+    # fp32 MLP batch 256: 64 -> 128 -> 64 -> 8 (three Gemm launches, ReLU fused)
+    X = torch.randn(256, 64, device=ctx.device)
+    Ws = [torch.randn(64, 128, device=ctx.device), torch.randn(128, 64, device=ctx.device),
+          torch.randn(64, 8, device=ctx.device)]
+    Bs = [torch.zeros(128, device=ctx.device), torch.zeros(64, device=ctx.device), torch.zeros(8, device=ctx.device)]
+    Hs = [ctx.empty((256, 128), torch.float32), ctx.empty((256, 64), torch.float32), ctx.empty((256, 8), torch.float32)]
+
+    def mlp():
+        cur = X
+        for i, (Wm, bm, h) in enumerate(zip(Ws, Bs, Hs)):
+            ctx.check(ctx.lib.sofie_hip_gemm_f32(ctx.h, 0, 0, 256, Wm.shape[1], Wm.shape[0], 1.0, ctx.ptr(cur),
+                                                 Wm.shape[0], ctx.ptr(Wm), Wm.shape[1], 1.0, ctx.ptr(bm), L.BIAS_ROW,
+                                                 ctx.ptr(h), Wm.shape[1], 1 if i < 2 else 0))
+            cur = h
+    ms = time_launches(ctx, mlp, 200, 10)
+    ex["mlp_f32_b256"] = {"us": ms * 1e3, "inferences_per_s": 256 / (ms * 1e-3), "gbs": 142112 / (ms * 1e-3) / 1e9}
+    return ex
+
+
+if __name__ == "__main__":
+    main()

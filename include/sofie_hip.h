@@ -1,0 +1,189 @@
+/*
+ * sofie_hip.h -- C ABI of the MI355X (gfx950) kernel library that SOFIE-generated
+ * inference code calls instead of a host BLAS.
+ *
+ * The generated code of the reference calls, per operator, the Fortran BLAS routines
+ * declared in its own header (src/SOFIE_core/src/RModel_Base.cxx:40-58: sgemm_, sgemv_,
+ * saxpy_, scopy_) plus the header templates SOFIE::UTILITY::Im2col and
+ * UnidirectionalBroadcast (src/SOFIE_core/inc/SOFIE/SOFIE_common.hxx:346-518) on host
+ * pointers. Each entry point below names the emitted call sequence it replaces.
+ *
+ * Conventions
+ *  - Every tensor pointer is a DEVICE pointer unless the name says host.
+ *  - All matrices are row-major with explicit leading dimensions in ELEMENTS; no
+ *    column-major swap trick is needed by the caller.
+ *  - Calls are asynchronous on the context's stream; sofie_hip_sync() waits.
+ *  - Return value: 0 on success, a negative SOFIE_HIP_E* code otherwise;
+ *    sofie_hip_last_error() gives the message. Generated code turns a non-zero
+ *    status into std::runtime_error, the reference's error convention
+ *    (ROperator_Gemm.hxx:76,143,295,347).
+ *  - The library keeps no global mutable state; one context per Session, one Session
+ *    per thread slot (the reference's threading contract, SOFIEHelpers.hxx:27-48).
+ */
+#ifndef SOFIE_HIP_H
+#define SOFIE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct sofie_hip_ctx sofie_hip_ctx;
+
+enum {
+   SOFIE_HIP_OK = 0,
+   SOFIE_HIP_EINVAL = -1,       /* bad argument (null pointer, negative size, bad enum) */
+   SOFIE_HIP_EHIP = -2,         /* a HIP runtime call failed */
+   SOFIE_HIP_ENOMEM = -3,       /* device allocation failed */
+   SOFIE_HIP_EUNSUPPORTED = -4  /* valid request that no kernel covers */
+};
+
+/* Fused activation of an epilogue. Only ReLU exists, as in the reference
+ * (ROperator_Gemm.hxx:377-381 acts on EActivationType::RELU only). */
+enum { SOFIE_ACT_NONE = 0, SOFIE_ACT_RELU = 1 };
+
+/* How the fp32 bias operand of sofie_hip_gemm_f32 is shaped. */
+enum {
+   SOFIE_BIAS_NONE = 0,
+   SOFIE_BIAS_ROW = 1,  /* [N]: one value per output column, same for every row */
+   SOFIE_BIAS_FULL = 2, /* [M,N] with leading dimension ldy: already broadcast */
+   SOFIE_BIAS_COL = 3   /* [M]: one value per output row */
+};
+
+/* Element type written by the quantized / FP8 GEMMs. */
+enum {
+   SOFIE_OUT_S8 = 0,   /* requantised int8 */
+   SOFIE_OUT_F32 = 1,  /* fp32 */
+   SOFIE_OUT_S32 = 2,  /* raw int32 accumulators (+bias) */
+   SOFIE_OUT_BF16 = 3  /* bfloat16, round to nearest even */
+};
+
+/* Memory layout of an int8 activation tensor. */
+enum { SOFIE_LAYOUT_NCHW = 0, SOFIE_LAYOUT_NHWC = 1 };
+
+/* ---------------------------------------------------------------- context, memory */
+
+/* Create a context on `device`. `stream` is a hipStream_t to launch on (borrowed), or
+ * NULL to create and own a new stream. Replaces nothing in the reference: its Session
+ * owns host vectors only (RModel.cxx:574-653). */
+int sofie_hip_create(sofie_hip_ctx **ctx, int device, void *stream);
+int sofie_hip_destroy(sofie_hip_ctx *ctx);
+/* Message of the last failed call on this context ("" if none). Never NULL. */
+const char *sofie_hip_last_error(const sofie_hip_ctx *ctx);
+/* ABI version of the library (bumped on incompatible change). */
+int sofie_hip_version(void);
+
+/* Device allocations owned by the caller (the generated Session): weights uploaded once
+ * in its constructor and the intermediate-tensor arena. Replace the std::vector<float>
+ * members and `new char[]` pool of the generated Session (RModel.cxx:574-604). */
+int sofie_hip_malloc(sofie_hip_ctx *ctx, void **dptr, size_t bytes);
+int sofie_hip_free(sofie_hip_ctx *ctx, void *dptr);
+int sofie_hip_upload(sofie_hip_ctx *ctx, void *dst_device, const void *src_host, size_t bytes);
+int sofie_hip_download(sofie_hip_ctx *ctx, void *dst_host, const void *src_device, size_t bytes);
+int sofie_hip_copy(sofie_hip_ctx *ctx, void *dst_device, const void *src_device, size_t bytes);
+int sofie_hip_memset(sofie_hip_ctx *ctx, void *dptr, int byte_value, size_t bytes);
+int sofie_hip_sync(sofie_hip_ctx *ctx);
+
+/* Event timing on the context's stream: start, enqueue work, stop (synchronises). */
+int sofie_hip_timer_start(sofie_hip_ctx *ctx);
+int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *elapsed_ms);
+
+/* ---------------------------------------------------------------- fp32 operators */
+
+/* Y[M,N] = alpha * op(A) * op(B) + beta * bias, then optional ReLU.
+ * op(A) is [M,K]: A is stored [M,K] (lda >= K) or, if transA, [K,M] (lda >= M).
+ * op(B) is [K,N]: B is stored [K,N] (ldb >= N) or, if transB, [N,K] (ldb >= K).
+ * bias == NULL requires beta == 0 (error otherwise, as ROperator_Gemm.hxx:343-349).
+ * Replaces the emitted sequence std::copy(bias_bcast -> Y); BLAS::sgemm_(...); ReLU loop
+ * of ROperator_Gemm<float>::Generate (ROperator_Gemm.hxx:360-381) and the bias
+ * materialisation of GenerateInitCode (:271-290): a rank-1 bias is broadcast inside
+ * the kernel epilogue instead of being stored M times. */
+int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, int M, int N, int K,
+                       float alpha, const float *A, int lda, const float *B, int ldb,
+                       float beta, const float *bias, int bias_kind, float *Y, int ldy,
+                       int act);
+
+/* NCHW 2-D convolution y = conv(x, w) + bias[oc], optional ReLU.
+ * x [N,C,H,W], w [OC, C/groups, KH, KW] (the ONNX layout, unpacked), bias [OC] or NULL,
+ * y [N,OC,OH,OW] with OH = (H + 2*pad_h - (dil_h*(KH-1)+1)) / stride_h + 1.
+ * Replaces, per image, the emitted weight re-layout loop, UTILITY::Im2col, BLAS::sgemm_
+ * and BLAS::saxpy_ of ROperator_Conv<float>::Generate (ROperator_Conv.hxx:342-518) and
+ * the following ROperator_Relu loop (ROperator_Relu.hxx:54-66) with one implicit-GEMM
+ * kernel over the whole batch; no im2col matrix is materialised. */
+int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
+                         const float *bias, float *y, int N, int C, int H, int W, int OC,
+                         int KH, int KW, int pad_h, int pad_w, int stride_h, int stride_w,
+                         int dil_h, int dil_w, int groups, int act);
+
+/* y[i] = x[i] > 0 ? x[i] : 0. Replaces the loop of ROperator_Relu.hxx:62-64. */
+int sofie_hip_relu_f32(sofie_hip_ctx *ctx, const float *x, float *y, size_t len);
+
+/* NCHW max pooling over NC = N*C planes; pads in ONNX order (top, left, bottom, right);
+ * floor output size; padding cells never win. Replaces the emitted loops of
+ * ROperator_Pool.hxx:371-416. */
+int sofie_hip_maxpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, int H,
+                            int W, int kh, int kw, int pad_t, int pad_l, int pad_b,
+                            int pad_r, int stride_h, int stride_w);
+
+/* ---------------------------------------------------------------- quantized operators
+ * The reference has no quantized operator (its parser rejects int8 initialisers,
+ * src/SOFIE_parsers/src/RModelParser_ONNX.cxx:560-591); these follow ONNX's
+ * QuantizeLinear / DequantizeLinear / QLinearMatMul / QLinearConv and are emitted through
+ * the same ROperator interface. Requantisation is one fixed formula everywhere:
+ *     r = rint_half_even( float(acc + bias) * scale[channel] )
+ *     q = clamp(r + zp_y, lo, 127),  lo = (act == RELU) ? max(zp_y, -128) : -128        */
+
+/* q = sat_s8(rint_half_even(x / scale) + zp). */
+int sofie_hip_quantize_f32_s8(sofie_hip_ctx *ctx, const float *x, int8_t *q, size_t len,
+                              float scale, int zp);
+/* x = (q - zp) * scale. */
+int sofie_hip_dequantize_s8_f32(sofie_hip_ctx *ctx, const int8_t *q, float *x, size_t len,
+                                float scale, int zp);
+
+/* int8 GEMM with int32 accumulation: acc[m,n] = sum_k A[m,k] * B[k,n] (+ bias[n]).
+ * A [M,K] row-major (lda); B [K,N] row-major (ldb) or, if transB, [N,K].
+ * scale [N] fp32 per output column (= s_a*s_b[n]/s_y), bias [N] int32 or NULL.
+ * A's zero-point is folded by the caller: bias[n] -= zp_a * sum_k B[k,n].
+ * out_kind: SOFIE_OUT_S8 (requantised, zp_y, act), SOFIE_OUT_F32 (float(acc)*scale[n],
+ * act), SOFIE_OUT_S32 (acc+bias; scale may be NULL). ldy in elements of the output type. */
+int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const int8_t *A,
+                       int lda, const int8_t *B, int ldb, const float *scale,
+                       const int32_t *bias, int zp_y, int act, void *Y, int ldy, int out_kind);
+
+/* int8 2-D convolution with int32 accumulation and fused requantisation.
+ * x, y: int8 activations in x_layout / y_layout; w [OC, C/groups, KH, KW] int8 (symmetric,
+ * zero-point 0) unpacked ONNX layout; bias [OC] int32 or NULL; scale [OC] fp32.
+ * Padding cells hold zp_x (so that they contribute zero once the caller has folded
+ * bias[oc] -= zp_x * sum(w[oc])). out_kind SOFIE_OUT_S8 or SOFIE_OUT_S32. */
+int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
+                         const int32_t *bias, const float *scale, void *y, int y_layout,
+                         int N, int C, int H, int W, int OC, int KH, int KW, int pad_h,
+                         int pad_w, int stride_h, int stride_w, int groups, int zp_x,
+                         int zp_y, int act, int out_kind);
+
+/* int8 max pooling, NCHW or NHWC. */
+int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N,
+                           int C, int H, int W, int kh, int kw, int pad_t, int pad_l,
+                           int pad_b, int pad_r, int stride_h, int stride_w);
+
+/* Layout change of an int8 activation tensor [N,C,H,W] <-> [N,H,W,C]. */
+int sofie_hip_relayout_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int N, int C, int H,
+                          int W, int from_layout, int to_layout);
+
+/* FP8 e4m3 (OCP e4m3fn) GEMM with fp32 accumulation:
+ *   t = (sum_k a*b) * (scale_a*scale_b) [+ bias[n]]  -> bf16 (RNE) or fp32.
+ * A [M,K] row-major; B [K,N] row-major or, if transB, [N,K]; bias [N] fp32 or NULL. */
+int sofie_hip_gemm_fp8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const uint8_t *A,
+                       int lda, const uint8_t *B, int ldb, float scale_a, float scale_b,
+                       const float *bias, void *Y, int ldy, int out_kind);
+
+/* fp32 -> e4m3 codes of x * inv_scale, RNE, saturating at +-448 (per-tensor scaling). */
+int sofie_hip_quantize_f32_e4m3(sofie_hip_ctx *ctx, const float *x, uint8_t *q, size_t len,
+                                float inv_scale);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SOFIE_HIP_H */

@@ -1,0 +1,73 @@
+// Internal helpers shared by the kernel translation units of libsofie_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "sofie_hip.h"
+
+struct sofie_hip_ctx {
+   int device = 0;
+   hipStream_t stream = nullptr;
+   bool owns_stream = false;
+   hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+   void *workspace = nullptr;   // scratch owned by the context (layout changes, B transposes)
+   size_t workspace_bytes = 0;
+   char err[512] = {0};
+};
+
+namespace sofie {
+
+int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...);
+// Grow-only scratch buffer of the context. Never shrinks; freed in sofie_hip_destroy.
+int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr);
+int check_launch(sofie_hip_ctx *ctx, const char *what);
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// Requantisation shared by every int8 epilogue:
+//   rint_half_even(float(acc) * scale) + zp, clamped to [lo, 127].
+// One int->fp32 conversion (RNE), one fp32 multiply, one round-to-nearest-even.
+__device__ __forceinline__ int requant(int acc, float scale, int zp, int lo)
+{
+   float r = rintf(__fmul_rn(__int2float_rn(acc), scale));
+   r = fminf(fmaxf(r, -1024.0f), 1024.0f);
+   int q = (int)r + zp;
+   return min(127, max(lo, q));
+}
+
+// fp32 -> bf16 bits, round to nearest even, NaN quieted.
+__device__ __forceinline__ unsigned f32_to_bf16(float x)
+{
+   unsigned u = __float_as_uint(x);
+   if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+   u += 0x7fffu + ((u >> 16) & 1u);
+   return u >> 16;
+}
+
+// Layout change of an int8 activation tensor (defined with the element-wise kernels).
+int relayout_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int N, int C, int H, int W, int from, int to);
+
+inline int cdiv(int a, int b) { return (a + b - 1) / b; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace sofie
+
+#define SOFIE_REQUIRE(ctx, cond, msg)                                             \
+   do {                                                                           \
+      if (!(cond)) return sofie::set_error((ctx), SOFIE_HIP_EINVAL, "%s: %s", __func__, (msg)); \
+   } while (0)
+
+#define SOFIE_HIP_CALL(ctx, expr)                                                 \
+   do {                                                                           \
+      hipError_t e_ = (expr);                                                     \
+      if (e_ != hipSuccess)                                                       \
+         return sofie::set_error((ctx), SOFIE_HIP_EHIP, "%s: %s failed: %s", __func__, #expr, \
+                                 hipGetErrorString(e_));                          \
+   } while (0)

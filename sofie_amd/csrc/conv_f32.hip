@@ -1,0 +1,235 @@
+// fp32 NCHW convolution as an implicit GEMM on the matrix cores (v_mfma_f32_32x32x2_f32).
+//
+// Per image and group:  Y[oc, pixel] = sum_k Wmat[oc, k] * xcol[k, pixel],  k = (ic, kh, kw),
+// which is the product the reference forms with Im2col + sgemm_, except that xcol is never
+// written anywhere: a workgroup stages the raw input patch (rows and columns its pixel tile
+// touches, halo included, zero filled outside the image) for a block of input channels in LDS
+// and every MFMA column operand is gathered from that patch at  base(pixel) + offset(k).
+// base() depends only on the lane's pixel and is computed once; offset() depends only on k and
+// lives in a small LDS table. The weight block of the K-chunk is staged k-major next to it.
+// Output rows of the MFMA tile are output channels, columns are pixels, so 32 lanes write 32
+// consecutive pixels of one channel plane: coalesced NCHW stores, bias and ReLU fused.
+// Roofline: MFMA fp32; per K-step of 2 each wavefront issues TI*TJ MFMAs (64 cycles each)
+// against TI+TJ+1 ds_read_b32.
+#include "common.h"
+
+using namespace sofie;
+
+namespace {
+
+struct ConvArgs {
+   const float *x, *w, *bias;
+   float *y;
+   int N, C, H, W, OC, KH, KW, ph, pw, sh, sw, dh, dw, groups;
+   int OH, OW, icg, ocg;
+   int ICB, KC;        // input channels per K-chunk, K-chunk length (even)
+   int PH, PW;         // staged patch extent
+   int rows_out;       // output rows a pixel tile can span
+   int relu;
+};
+
+template <int TI, int TJ>
+__global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
+{
+   constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
+   extern __shared__ __align__(16) unsigned char smem_raw[];
+   float *sW = reinterpret_cast<float *>(smem_raw);                  // [KC][LDW]
+   float *patch = sW + g.KC * LDW;                                   // [ICB][PH][PW]
+   int *koff = reinterpret_cast<int *>(patch + g.ICB * g.PH * g.PW); // [KC]
+
+   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int wm = wave >> 1, wn = wave & 1;
+   const int fr = lane & 31, fk = lane >> 5;
+
+   const int octiles = (g.ocg + BOC - 1) / BOC;
+   const int grp = blockIdx.y / octiles;
+   const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
+   const int n = blockIdx.z;
+   const int OHW = g.OH * g.OW;
+   const int p0 = blockIdx.x * BP;
+   const int oh0 = p0 / g.OW;
+   const int ih0 = oh0 * g.sh - g.ph, iw0 = -g.pw;
+   const int KHW = g.KH * g.KW;
+   const int Kfull = g.icg * KHW;
+
+   for (int k = tid; k < g.KC; k += 256) {
+      const int icl = k / KHW, t = k % KHW;
+      const int kh = t / g.KW, kw = t % g.KW;
+      koff[k] = (icl < g.ICB) ? (icl * g.PH + kh * g.dh) * g.PW + kw * g.dw : 0;
+   }
+
+   int base[TJ];
+#pragma unroll
+   for (int j = 0; j < TJ; ++j) {
+      const int p = p0 + wn * TJ * 32 + j * 32 + fr;
+      base[j] = (p < OHW) ? ((p / g.OW - oh0) * g.sh) * g.PW + (p % g.OW) * g.sw : 0;
+   }
+
+   v16f acc[TI][TJ];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+#pragma unroll
+         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+   const float *xg = g.x + ((size_t)n * g.C + (size_t)grp * g.icg) * g.H * g.W;
+   const float *wg = g.w + (size_t)grp * g.ocg * Kfull;
+   const int patch_len = g.ICB * g.PH * g.PW;
+
+   for (int ic0 = 0; ic0 < g.icg; ic0 += g.ICB) {
+      const int icn = (g.icg - ic0) < g.ICB ? (g.icg - ic0) : g.ICB;
+      const int kc = icn * KHW;
+      __syncthreads();   // previous chunk fully consumed (also orders the koff table on entry)
+      for (int e = tid; e < patch_len; e += 256) {
+         const int c = e % g.PW, r = (e / g.PW) % g.PH, icl = e / (g.PW * g.PH);
+         const int ih = ih0 + r, iw = iw0 + c;
+         float v = 0.0f;
+         if (icl < icn && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
+            v = xg[((size_t)(ic0 + icl) * g.H + ih) * g.W + iw];
+         patch[e] = v;
+      }
+      for (int e = tid; e < g.KC * BOC; e += 256) {
+         const int k = e % g.KC, ocl = e / g.KC;
+         float v = 0.0f;
+         if (k < kc && oc0 + ocl < g.ocg) v = wg[(size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k];
+         sW[k * LDW + ocl] = v;
+      }
+      __syncthreads();
+      const float *wrow = sW + wm * TI * 32 + fr;
+      for (int s = 0; s < g.KC / 2; ++s) {
+         const int kk = 2 * s + fk;
+         const int ko = koff[kk];
+         float fa[TI], fb[TJ];
+#pragma unroll
+         for (int i = 0; i < TI; ++i) fa[i] = wrow[kk * LDW + i * 32];
+#pragma unroll
+         for (int j = 0; j < TJ; ++j) fb[j] = patch[base[j] + ko];
+#pragma unroll
+         for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+   }
+
+   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * OHW;
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) {
+         const int p = p0 + wn * TJ * 32 + j * 32 + fr;
+         if (p >= OHW) continue;
+#pragma unroll
+         for (int r = 0; r < 16; ++r) {
+            const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
+            if (oc >= g.ocg) continue;
+            float v = acc[i][j][r];
+            if (g.bias) v = __fadd_rn(v, g.bias[grp * g.ocg + oc]);
+            if (g.relu) v = v > 0.0f ? v : 0.0f;
+            yn[(size_t)oc * OHW + p] = v;
+         }
+      }
+}
+
+// One thread per output element: any kernel size, used when the staged patch of the tiled
+// kernel would not fit LDS.
+__global__ void k_conv2d_f32_simple(ConvArgs g)
+{
+   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   const size_t total = (size_t)g.N * g.OC * g.OH * g.OW;
+   if (idx >= total) return;
+   size_t r = idx;
+   const int ow = (int)(r % g.OW); r /= g.OW;
+   const int oh = (int)(r % g.OH); r /= g.OH;
+   const int oc = (int)(r % g.OC);
+   const int n = (int)(r / g.OC);
+   const int grp = oc / g.ocg;
+   float acc = 0.0f;
+   for (int ic = 0; ic < g.icg; ++ic)
+      for (int kh = 0; kh < g.KH; ++kh) {
+         const int ih = oh * g.sh - g.ph + kh * g.dh;
+         if (ih < 0 || ih >= g.H) continue;
+         for (int kw = 0; kw < g.KW; ++kw) {
+            const int iw = ow * g.sw - g.pw + kw * g.dw;
+            if (iw < 0 || iw >= g.W) continue;
+            acc = __fadd_rn(acc, __fmul_rn(g.x[(((size_t)n * g.C + grp * g.icg + ic) * g.H + ih) * g.W + iw],
+                                           g.w[(((size_t)oc * g.icg + ic) * g.KH + kh) * g.KW + kw]));
+         }
+      }
+   if (g.bias) acc = __fadd_rn(acc, g.bias[oc]);
+   if (g.relu) acc = acc > 0.0f ? acc : 0.0f;
+   g.y[idx] = acc;
+}
+
+template <int TI, int TJ>
+int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
+{
+   constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
+   const int KHW = g.KH * g.KW;
+   const int OHW = g.OH * g.OW;
+   g.rows_out = (BP + g.OW - 2) / g.OW + 1;
+   if (g.rows_out > g.OH) g.rows_out = g.OH;
+   g.PH = (g.rows_out - 1) * g.sh + (g.KH - 1) * g.dh + 1;
+   g.PW = (g.OW - 1) * g.sw + (g.KW - 1) * g.dw + 1;
+   const size_t budget = 64 * 1024;
+   *done = false;
+   int icb = 96 / KHW;
+   if (icb < 1) icb = 1;
+   if (icb > g.icg) icb = g.icg;
+   size_t lds = 0;
+   for (; icb >= 1; --icb) {
+      const int kc = (icb * KHW + 1) & ~1;
+      lds = ((size_t)kc * LDW + (size_t)icb * g.PH * g.PW + kc) * 4;
+      if (lds <= budget) {
+         g.ICB = icb;
+         g.KC = kc;
+         break;
+      }
+   }
+   if (icb < 1) return SOFIE_HIP_OK;   // does not fit: caller uses the simple kernel
+   const int octiles = cdiv(g.ocg, BOC);
+   if ((size_t)g.groups * octiles > 65535 || g.N > 65535) return SOFIE_HIP_OK;
+   auto kern = k_conv2d_f32<TI, TJ>;
+   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+   hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, g);
+   *done = true;
+   return check_launch(ctx, "k_conv2d_f32");
+}
+
+}  // namespace
+
+extern "C" int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w, const float *bias, float *y,
+                                    int N, int C, int H, int W, int OC, int KH, int KW, int pad_h, int pad_w,
+                                    int stride_h, int stride_w, int dil_h, int dil_w, int groups, int act)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, N >= 0 && C > 0 && H > 0 && W > 0 && OC > 0 && KH > 0 && KW > 0, "non-positive dimension");
+   SOFIE_REQUIRE(ctx, pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0,
+                 "bad pads/strides/dilations");
+   SOFIE_REQUIRE(ctx, groups > 0 && C % groups == 0 && OC % groups == 0, "channels not divisible by groups");
+   SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
+   const int eh = dil_h * (KH - 1) + 1, ew = dil_w * (KW - 1) + 1;
+   SOFIE_REQUIRE(ctx, H + 2 * pad_h >= eh && W + 2 * pad_w >= ew, "kernel larger than padded input");
+   if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && w && y, "null operand");
+   ConvArgs g{};
+   g.x = x; g.w = w; g.bias = bias; g.y = y;
+   g.N = N; g.C = C; g.H = H; g.W = W; g.OC = OC; g.KH = KH; g.KW = KW;
+   g.ph = pad_h; g.pw = pad_w; g.sh = stride_h; g.sw = stride_w; g.dh = dil_h; g.dw = dil_w; g.groups = groups;
+   g.OH = (H + 2 * pad_h - eh) / stride_h + 1;
+   g.OW = (W + 2 * pad_w - ew) / stride_w + 1;
+   g.icg = C / groups;
+   g.ocg = OC / groups;
+   g.relu = act == SOFIE_ACT_RELU;
+   bool done = false;
+   int rc;
+   if (g.ocg > 64) rc = launch<2, 2>(ctx, g, &done);
+   else if (g.ocg > 32) rc = launch<1, 2>(ctx, g, &done);
+   else rc = launch<1, 2>(ctx, g, &done);
+   if (rc || done) return rc;
+   const size_t total = (size_t)N * OC * g.OH * g.OW;
+   hipLaunchKernelGGL(k_conv2d_f32_simple, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, g);
+   return check_launch(ctx, "k_conv2d_f32_simple");
+}

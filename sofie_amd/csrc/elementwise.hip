@@ -1,0 +1,269 @@
+// Memory-bound operators: ReLU, max pooling, quantize / dequantize, int8 layout changes.
+// All are grid-stride-free flat launches with 16-byte accesses where the shape allows;
+// their roofline is HBM bandwidth (bytes in + bytes out per element).
+#include "common.h"
+
+using namespace sofie;
+
+namespace {
+
+__global__ void k_relu_f32(const float *__restrict__ x, float *__restrict__ y, size_t len)
+{
+   const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+   if (i + 3 < len) {
+      const v4f v = *reinterpret_cast<const v4f *>(x + i);
+      v4f r;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) r[t] = v[t] > 0.0f ? v[t] : 0.0f;
+      *reinterpret_cast<v4f *>(y + i) = r;
+   } else {
+      for (size_t j = i; j < len; ++j) y[j] = x[j] > 0.0f ? x[j] : 0.0f;
+   }
+}
+
+__global__ void k_relu_f32_scalar(const float *__restrict__ x, float *__restrict__ y, size_t len)
+{
+   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   if (i < len) y[i] = x[i] > 0.0f ? x[i] : 0.0f;
+}
+
+template <typename T>
+__device__ __forceinline__ T lowest();
+template <>
+__device__ __forceinline__ float lowest<float>() { return -__builtin_inff(); }
+template <>
+__device__ __forceinline__ int8_t lowest<int8_t>() { return -128; }
+
+// One thread per output element. NHWC: channel is the fastest index.
+template <typename T, bool NHWC>
+__global__ void k_maxpool2d(const T *__restrict__ x, T *__restrict__ y, int N, int C, int H, int W, int OH, int OW,
+                            int kh, int kw, int pt, int pl, int sh, int sw)
+{
+   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   const size_t total = (size_t)N * C * OH * OW;
+   if (idx >= total) return;
+   int n, c, oh, ow;
+   size_t r = idx;
+   if (NHWC) {
+      c = (int)(r % C); r /= C;
+      ow = (int)(r % OW); r /= OW;
+      oh = (int)(r % OH); n = (int)(r / OH);
+   } else {
+      ow = (int)(r % OW); r /= OW;
+      oh = (int)(r % OH); r /= OH;
+      c = (int)(r % C); n = (int)(r / C);
+   }
+   T best = lowest<T>();
+   for (int i = 0; i < kh; ++i) {
+      const int ih = oh * sh - pt + i;
+      if (ih < 0 || ih >= H) continue;
+      for (int j = 0; j < kw; ++j) {
+         const int iw = ow * sw - pl + j;
+         if (iw < 0 || iw >= W) continue;
+         const size_t off = NHWC ? (((size_t)n * H + ih) * W + iw) * C + c : (((size_t)n * C + c) * H + ih) * W + iw;
+         const T v = x[off];
+         if (v > best) best = v;
+      }
+   }
+   y[idx] = best;
+}
+
+__global__ void k_quantize_f32_s8(const float *__restrict__ x, int8_t *__restrict__ q, size_t len, float scale, int zp)
+{
+   const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+   if (i >= len) return;
+   unsigned packed = 0;
+   const int cnt = (len - i) < 4 ? (int)(len - i) : 4;
+   for (int t = 0; t < cnt; ++t) {
+      float r = rintf(__fdiv_rn(x[i + t], scale));
+      r = fminf(fmaxf(r, -1024.0f), 1024.0f);
+      const int v = min(127, max(-128, (int)r + zp));
+      packed |= ((unsigned)v & 0xffu) << (8 * t);
+   }
+   if (cnt == 4 && (reinterpret_cast<uintptr_t>(q + i) & 3u) == 0) {
+      *reinterpret_cast<unsigned *>(q + i) = packed;
+   } else {
+      for (int t = 0; t < cnt; ++t) q[i + t] = (int8_t)(packed >> (8 * t));
+   }
+}
+
+__global__ void k_dequantize_s8_f32(const int8_t *__restrict__ q, float *__restrict__ x, size_t len, float scale, int zp)
+{
+   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   if (i < len) x[i] = __fmul_rn(__int2float_rn((int)q[i] - zp), scale);
+}
+
+// fp32 -> e4m3 (OCP), round to nearest even, saturating at +-448; NaN -> 0x7f.
+__device__ __forceinline__ unsigned f32_to_e4m3_sat(float x)
+{
+   const unsigned u = __float_as_uint(x);
+   const unsigned sign = (u >> 24) & 0x80u;
+   const unsigned a = u & 0x7fffffffu;
+   if (a > 0x7f800000u) return 0x7fu;
+   const float af = __uint_as_float(a);
+   if (af >= 448.0f) return sign | 0x7eu;
+   // Scale so that the e4m3 grid becomes the integer grid, round, scale back.
+   // Normal range (>= 2^-6): spacing 2^(e-3); subnormal: spacing 2^-9.
+   int e = (int)(a >> 23) - 127;
+   if (e < -6) e = -6;
+   const float step = __uint_as_float((unsigned)(e - 3 + 127) << 23);
+   const float q = rintf(__fdiv_rn(af, step));      // exact power-of-two division
+   const float r = __fmul_rn(q, step);
+   if (r >= 448.0f) return sign | 0x7eu;
+   if (r < 0.015625f) return sign | (unsigned)(int)__fmul_rn(r, 512.0f);   // multiples of 2^-9
+   const unsigned rb = __float_as_uint(r);
+   const unsigned re = (rb >> 23) - 127u + 7u;
+   return sign | (re << 3) | ((rb >> 20) & 7u);
+}
+
+__global__ void k_quantize_f32_e4m3(const float *__restrict__ x, uint8_t *__restrict__ q, size_t len, float inv_scale)
+{
+   const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   if (i < len) q[i] = (uint8_t)f32_to_e4m3_sat(__fmul_rn(x[i], inv_scale));
+}
+
+// [N,C,HW] <-> [N,HW,C] through a 64x64 LDS tile so both sides move contiguous bytes.
+__global__ void k_transpose_s8(const int8_t *__restrict__ x, int8_t *__restrict__ y, int R, int Ccols)
+{
+   // x is [batch][R][Ccols], y is [batch][Ccols][R]
+   __shared__ int8_t tile[64][65];
+   const size_t base = (size_t)blockIdx.z * R * Ccols;
+   const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+   for (int i = threadIdx.y; i < 64; i += blockDim.y) {
+      const int r = r0 + i, c = c0 + threadIdx.x;
+      if (r < R && c < Ccols) tile[i][threadIdx.x] = x[base + (size_t)r * Ccols + c];
+   }
+   __syncthreads();
+   for (int i = threadIdx.y; i < 64; i += blockDim.y) {
+      const int c = c0 + i, r = r0 + threadIdx.x;
+      if (r < R && c < Ccols) y[base + (size_t)c * R + r] = tile[threadIdx.x][i];
+   }
+}
+
+inline unsigned blocks_for(size_t n, unsigned per) { return (unsigned)((n + per - 1) / per); }
+
+}  // namespace
+
+namespace sofie {
+int relayout_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int N, int C, int H, int W, int from, int to)
+{
+   const size_t len = (size_t)N * C * H * W;
+   if (len == 0) return SOFIE_HIP_OK;
+   if (from == to) {
+      if (x != y) SOFIE_HIP_CALL(ctx, hipMemcpyAsync(y, x, len, hipMemcpyDeviceToDevice, ctx->stream));
+      return SOFIE_HIP_OK;
+   }
+   const int HW = H * W;
+   // NCHW -> NHWC: per image transpose [C][HW] -> [HW][C]; the reverse swaps the roles.
+   const int R = (from == SOFIE_LAYOUT_NCHW) ? C : HW;
+   const int Cc = (from == SOFIE_LAYOUT_NCHW) ? HW : C;
+   dim3 grid(cdiv(Cc, 64), cdiv(R, 64), N), block(64, 4);
+   hipLaunchKernelGGL(k_transpose_s8, grid, block, 0, ctx->stream, x, y, R, Cc);
+   return check_launch(ctx, "k_transpose_s8");
+}
+}  // namespace sofie
+
+extern "C" {
+
+int sofie_hip_relu_f32(sofie_hip_ctx *ctx, const float *x, float *y, size_t len)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (len == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && y, "null operand");
+   if (aligned16(x) && aligned16(y))
+      hipLaunchKernelGGL(k_relu_f32, dim3(blocks_for(len, 1024)), dim3(256), 0, ctx->stream, x, y, len);
+   else
+      hipLaunchKernelGGL(k_relu_f32_scalar, dim3(blocks_for(len, 256)), dim3(256), 0, ctx->stream, x, y, len);
+   return check_launch(ctx, "k_relu_f32");
+}
+
+static int pool_dims(sofie_hip_ctx *ctx, int H, int W, int kh, int kw, int pt, int pl, int pb, int pr, int sh,
+                     int sw, int *OH, int *OW)
+{
+   SOFIE_REQUIRE(ctx, H > 0 && W > 0 && kh > 0 && kw > 0 && sh > 0 && sw > 0, "non-positive dimension");
+   SOFIE_REQUIRE(ctx, pt >= 0 && pl >= 0 && pb >= 0 && pr >= 0, "negative padding");
+   SOFIE_REQUIRE(ctx, H + pt + pb >= kh && W + pl + pr >= kw, "kernel larger than padded input");
+   *OH = (H + pt + pb - kh) / sh + 1;
+   *OW = (W + pl + pr - kw) / sw + 1;
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_maxpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, int H, int W, int kh, int kw,
+                            int pt, int pl, int pb, int pr, int sh, int sw)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, NC >= 0, "negative dimension");
+   if (NC == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && y, "null operand");
+   int OH, OW;
+   if (int rc = pool_dims(ctx, H, W, kh, kw, pt, pl, pb, pr, sh, sw, &OH, &OW)) return rc;
+   const size_t total = (size_t)NC * OH * OW;
+   hipLaunchKernelGGL((k_maxpool2d<float, false>), dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y, 1,
+                      NC, H, W, OH, OW, kh, kw, pt, pl, sh, sw);
+   return check_launch(ctx, "k_maxpool2d");
+}
+
+int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N, int C, int H, int W,
+                           int kh, int kw, int pt, int pl, int pb, int pr, int sh, int sw)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, N >= 0 && C >= 0, "negative dimension");
+   SOFIE_REQUIRE(ctx, layout == SOFIE_LAYOUT_NCHW || layout == SOFIE_LAYOUT_NHWC, "unknown layout");
+   if (N == 0 || C == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && y, "null operand");
+   int OH, OW;
+   if (int rc = pool_dims(ctx, H, W, kh, kw, pt, pl, pb, pr, sh, sw, &OH, &OW)) return rc;
+   const size_t total = (size_t)N * C * OH * OW;
+   if (layout == SOFIE_LAYOUT_NHWC)
+      hipLaunchKernelGGL((k_maxpool2d<int8_t, true>), dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y,
+                         N, C, H, W, OH, OW, kh, kw, pt, pl, sh, sw);
+   else
+      hipLaunchKernelGGL((k_maxpool2d<int8_t, false>), dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y,
+                         N, C, H, W, OH, OW, kh, kw, pt, pl, sh, sw);
+   return check_launch(ctx, "k_maxpool2d");
+}
+
+int sofie_hip_quantize_f32_s8(sofie_hip_ctx *ctx, const float *x, int8_t *q, size_t len, float scale, int zp)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (len == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && q, "null operand");
+   SOFIE_REQUIRE(ctx, scale > 0.0f, "scale must be positive");
+   SOFIE_REQUIRE(ctx, zp >= -128 && zp <= 127, "zero-point out of int8 range");
+   hipLaunchKernelGGL(k_quantize_f32_s8, dim3(blocks_for(len, 1024)), dim3(256), 0, ctx->stream, x, q, len, scale, zp);
+   return check_launch(ctx, "k_quantize_f32_s8");
+}
+
+int sofie_hip_dequantize_s8_f32(sofie_hip_ctx *ctx, const int8_t *q, float *x, size_t len, float scale, int zp)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (len == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && q, "null operand");
+   SOFIE_REQUIRE(ctx, zp >= -128 && zp <= 127, "zero-point out of int8 range");
+   hipLaunchKernelGGL(k_dequantize_s8_f32, dim3(blocks_for(len, 256)), dim3(256), 0, ctx->stream, q, x, len, scale, zp);
+   return check_launch(ctx, "k_dequantize_s8_f32");
+}
+
+int sofie_hip_quantize_f32_e4m3(sofie_hip_ctx *ctx, const float *x, uint8_t *q, size_t len, float inv_scale)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (len == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && q, "null operand");
+   hipLaunchKernelGGL(k_quantize_f32_e4m3, dim3(blocks_for(len, 256)), dim3(256), 0, ctx->stream, x, q, len, inv_scale);
+   return check_launch(ctx, "k_quantize_f32_e4m3");
+}
+
+int sofie_hip_relayout_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int N, int C, int H, int W, int from,
+                          int to)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, N >= 0 && C >= 0 && H >= 0 && W >= 0, "negative dimension");
+   SOFIE_REQUIRE(ctx, (from == SOFIE_LAYOUT_NCHW || from == SOFIE_LAYOUT_NHWC) &&
+                         (to == SOFIE_LAYOUT_NCHW || to == SOFIE_LAYOUT_NHWC), "unknown layout");
+   if ((size_t)N * C * H * W == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && y, "null operand");
+   SOFIE_REQUIRE(ctx, N <= 65535, "batch too large for one launch");
+   return sofie::relayout_s8(ctx, x, y, N, C, H, W, from, to);
+}
+
+}  // extern "C"

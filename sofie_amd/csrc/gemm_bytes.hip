@@ -1,0 +1,559 @@
+// One-byte-element GEMMs on the gfx950 matrix cores: int8 x int8 -> int32 with fused
+// requantisation (QLinearMatMul semantics) and FP8 e4m3 x e4m3 -> fp32 -> bf16/fp32.
+//
+// Kernel shape (k_gemm_bytes): 256 threads = 4 wavefronts in a 2x2 arrangement, each
+// wavefront owning a (TI*32) x (TJ*32) block of the output built from 32x32 MFMA tiles
+// (v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x64_f8f6f4). Both operands are staged in LDS
+// as [row][K-bytes] with a 16-byte pad per row, which makes the 16-byte-per-lane operand
+// reads bank-conflict free; global -> register -> LDS staging is double buffered so the
+// loads of K-step t+1 are in flight while the MFMAs of step t issue. The MFMA row operand
+// is the B^T tile (output column n), the column operand the A tile (output row m), so a lane
+// holds four consecutive n for one m and the epilogue packs them into one 4*esize store; the
+// packed results go through a per-wavefront LDS staging block and leave as 16-byte row
+// segments. Workgroup ids are remapped so that each XCD (ids are dealt round-robin over the
+// 8 XCDs) owns a compact rectangle of output tiles and its L2 sees each operand panel once.
+#include "common.h"
+
+using namespace sofie;
+
+namespace {
+
+struct MmaI8 {
+   typedef v16i Acc;
+   typedef v4i Frag;
+   static constexpr int KB = 32;           // bytes of K consumed by one instruction
+   static constexpr int LANE_BYTES = 16;   // bytes of K one lane supplies per operand
+   static __device__ __forceinline__ Frag load(const unsigned char *p) { return *reinterpret_cast<const v4i *>(p); }
+   static __device__ __forceinline__ Acc mma(Frag a, Frag b, Acc c)
+   {
+      return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+   }
+};
+
+struct MmaF8 {
+   typedef v16f Acc;
+   typedef v8i Frag;
+   static constexpr int KB = 64;
+   static constexpr int LANE_BYTES = 32;
+   static __device__ __forceinline__ Frag load(const unsigned char *p)
+   {
+      const v4i lo = *reinterpret_cast<const v4i *>(p), hi = *reinterpret_cast<const v4i *>(p + 16);
+      Frag f = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      return f;
+   }
+   static __device__ __forceinline__ Acc mma(Frag a, Frag b, Acc c)
+   {
+      // cbsz = blgp = 0 selects e4m3 for both operands; zero scale operands = unscaled.
+      return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+   }
+};
+
+struct GemmArgs {
+   const uint8_t *A;
+   const uint8_t *B;
+   void *Y;
+   const float *scale;   // [N] (int8) or nullptr
+   const void *bias;     // int32 [N] (int8) / float [N] (fp8) or nullptr
+   int M, N, K, lda, ldb, ldy;
+   int zp, lo;           // int8 output zero-point and lower clamp
+   int relu;
+   float s;              // fp8: scale_a * scale_b
+   int tiles_m, tiles_n;
+   int vec_store;        // rows of Y may be written with 16-byte stores
+};
+
+template <int OUT> struct OutSize { static constexpr int value = 4; };
+template <> struct OutSize<SOFIE_OUT_S8> { static constexpr int value = 1; };
+template <> struct OutSize<SOFIE_OUT_BF16> { static constexpr int value = 2; };
+
+__device__ __forceinline__ float e4m3_to_f32(unsigned v)
+{
+   const unsigned e = (v >> 3) & 15u, m = v & 7u;
+   float r;
+   if (e == 15u && m == 7u) return __uint_as_float(0x7fc00000u);
+   if (e == 0u) r = (float)m * 0.001953125f;
+   else r = __uint_as_float(((e + 120u) << 23) | (m << 20));
+   return (v & 0x80u) ? -r : r;
+}
+
+// One output element of the epilogue from an int32 (int8 path) or fp32 (fp8 path) accumulator.
+// `bias_bits` holds the column's int32 bias (int8 path) or fp32 bias bits (fp8 path), 0 if none.
+template <bool IS_INT, int OUT>
+__device__ __forceinline__ unsigned epilogue_value(const GemmArgs &g, float sc, int bias_bits, int raw_i, float raw_f)
+{
+   if constexpr (IS_INT) {
+      const int a = raw_i + bias_bits;
+      if constexpr (OUT == SOFIE_OUT_S32) return (unsigned)a;
+      if constexpr (OUT == SOFIE_OUT_S8) return (unsigned)requant(a, sc, g.zp, g.lo) & 0xffu;
+      float v = __fmul_rn(__int2float_rn(a), sc);
+      if (g.relu && !(v > 0.0f)) v = 0.0f;
+      return __float_as_uint(v);
+   } else {
+      float t = __fmul_rn(raw_f, g.s);
+      if (g.bias) t = __fadd_rn(t, __int_as_float(bias_bits));
+      if constexpr (OUT == SOFIE_OUT_BF16) return f32_to_bf16(t);
+      return __float_as_uint(t);
+   }
+}
+
+template <class Mma, int BK, int NSETS, int TI, int TJ, int OUT, bool B_KN, bool FULL>
+__global__ void __launch_bounds__(256, (TI * TJ >= 16) ? 1 : 2) k_gemm_bytes(GemmArgs g)
+{
+   constexpr int BN = 2 * TI * 32, BM = 2 * TJ * 32;
+   constexpr int LDK = BK + 16;
+   constexpr int CPR = BK / 16;
+   constexpr int NSUB = BK / Mma::KB;
+   constexpr int ESZ = OutSize<OUT>::value;
+   constexpr bool IS_INT = __is_same(typename Mma::Acc, v16i);
+   extern __shared__ __align__(16) unsigned char smem[];
+   unsigned char *const sA = smem;                  // [2][BM][LDK]
+   unsigned char *const sB = smem + 2 * BM * LDK;   // [2][BN][LDK]
+
+   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int wm = wave >> 1, wn = wave & 1;
+
+   // --- workgroup id -> output tile, XCD aware -----------------------------------------
+   const int tiles = g.tiles_m * g.tiles_n;
+   int pid = blockIdx.x;
+   {
+      const int xcd = pid & 7, local = pid >> 3;
+      const int base = tiles >> 3, rem = tiles & 7;
+      pid = local + xcd * base + (xcd < rem ? xcd : rem);
+   }
+   int tm, tn;
+   {
+      constexpr int GM = 4;
+      const int width = GM * g.tiles_n;
+      const int group = pid / width;
+      const int first = group * GM;
+      const int gsize = (g.tiles_m - first) < GM ? (g.tiles_m - first) : GM;
+      tm = first + (pid % width) % gsize;
+      tn = (pid % width) / gsize;
+   }
+   const int m0 = tm * BM, n0 = tn * BN;
+
+   // --- global -> register staging -----------------------------------------------------
+   // A thread owns A_CH 16-byte chunks of the A tile and B_CH of the B tile per K-step.
+   // NSETS register sets are in flight: the chunk written to LDS during step t (tile t+1) is
+   // re-requested for tile t+1+NSETS right behind its LDS write, so every request has NSETS
+   // full K-steps to return.
+   constexpr int A_CH = BM * CPR / 256;
+   constexpr int B_UNITS = BN / 4 * CPR;                 // transposing loader: 16k x 4n units per tile
+   constexpr int B_UPT = (B_UNITS + 255) / 256;          // units per thread
+   constexpr int B_CH = B_KN ? B_UPT * 4 : BN * CPR / 256;
+   constexpr int B_PARTS = B_KN ? B_UPT : B_CH;          // independently movable pieces of B
+   struct Staged {
+      v4i a[A_CH];
+      v4i b[B_CH];
+   };
+   const v4i zero4 = {0, 0, 0, 0};
+
+   // Row/column part of each thread's addresses is fixed for the whole K loop. Out-of-range
+   // rows are clamped to a valid row and their data replaced by zero after the load, so the
+   // loads themselves are never predicated.
+   const unsigned char *pa[A_CH];
+   bool oka[A_CH];
+#pragma unroll
+   for (int i = 0; i < A_CH; ++i) {
+      const int c = i * 256 + tid;
+      const int gm = m0 + c / CPR;
+      oka[i] = FULL || gm < g.M;
+      pa[i] = g.A + (size_t)(oka[i] ? gm : g.M - 1) * g.lda + (c % CPR) * 16;
+   }
+   const unsigned char *pb[B_PARTS];
+   bool okb[B_PARTS];
+#pragma unroll
+   for (int i = 0; i < B_PARTS; ++i) {
+      if constexpr (!B_KN) {
+         const int c = i * 256 + tid;
+         const int gn = n0 + c / CPR;
+         okb[i] = FULL || gn < g.N;
+         pb[i] = g.B + (size_t)(okb[i] ? gn : g.N - 1) * g.ldb + (c % CPR) * 16;
+      } else {
+         const int u = i * 256 + tid;
+         const int kg = u % CPR, ng = u / CPR;
+         const int gn = n0 + ng * 4;
+         okb[i] = (B_UNITS % 256 == 0 || u < B_UNITS) && (FULL || gn < g.N);
+         pb[i] = g.B + (size_t)(kg * 16) * g.ldb + (okb[i] ? gn : 0);
+      }
+   }
+   const int kmax = g.K - 16;   // K is a multiple of 16 on this path
+
+   auto fetch_a = [&](Staged &G, int k0, int i) {
+      const int kc = ((i * 256 + tid) % CPR) * 16;
+      const bool kin = FULL || k0 + kc <= kmax;
+      const v4i v = *reinterpret_cast<const v4i *>(pa[i] + (kin ? k0 : kmax - kc));
+      G.a[i] = (oka[i] && kin) ? v : zero4;
+   };
+   auto fetch_b = [&](Staged &G, int k0, int i) {
+      const int kc = ((i * 256 + tid) % CPR) * 16;
+      const bool kin = FULL || k0 + kc <= kmax;
+      if constexpr (!B_KN) {
+         const v4i v = *reinterpret_cast<const v4i *>(pb[i] + (kin ? k0 : kmax - kc));
+         G.b[i] = (okb[i] && kin) ? v : zero4;
+      } else {
+         // B is [K,N]: a unit is 16 k-rows x 4 n-columns = 16 dwords, kept raw in registers and
+         // transposed into four K-contiguous 16-byte chunks when written to LDS.
+         const unsigned char *p = pb[i] + (size_t)(kin ? k0 : kmax - kc) * g.ldb;
+#pragma unroll
+         for (int q = 0; q < 4; ++q) {
+            v4i v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = *reinterpret_cast<const int *>(p + (size_t)(4 * q + e) * g.ldb);
+            G.b[i * 4 + q] = (okb[i] && kin) ? v : zero4;
+         }
+      }
+   };
+   auto stash_a = [&](const Staged &G, int stage, int i) {
+      const int c = i * 256 + tid;
+      *reinterpret_cast<v4i *>(sA + stage * BM * LDK + (c / CPR) * LDK + (c % CPR) * 16) = G.a[i];
+   };
+   auto stash_b = [&](const Staged &G, int stage, int i) {
+      unsigned char *b = sB + stage * BN * LDK;
+      if constexpr (!B_KN) {
+         const int c = i * 256 + tid;
+         *reinterpret_cast<v4i *>(b + (c / CPR) * LDK + (c % CPR) * 16) = G.b[i];
+      } else {
+         const int u = i * 256 + tid;
+         const bool live = B_UNITS % 256 == 0 || u < B_UNITS;
+         const int kg = u % CPR, ng = u / CPR;
+         unsigned o[4][4];   // o[column][k-quad]: 4x4 byte transposes with v_perm_b32
+#pragma unroll
+         for (int q = 0; q < 4; ++q) {
+            const v4i d = G.b[i * 4 + q];
+            const unsigned t0 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u);
+            const unsigned t1 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
+            const unsigned t2 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u);
+            const unsigned t3 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+            o[0][q] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+            o[1][q] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+            o[2][q] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+            o[3][q] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+         }
+         if (live) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+               const v4i v = {(int)o[j][0], (int)o[j][1], (int)o[j][2], (int)o[j][3]};
+               *reinterpret_cast<v4i *>(b + (ng * 4 + j) * LDK + kg * 16) = v;
+            }
+         }
+      }
+   };
+   // Pieces of a tile pair are numbered 0..A_CH+B_PARTS-1 and dealt round-robin to the MFMA
+   // groups of a K-step; group `grp` of `ngrp` moves the pieces p with p % ngrp == grp.
+   auto move_pieces = [&](Staged &G, int stage, int k_next, int grp, int ngrp, bool do_stash, bool do_fetch) {
+#pragma unroll
+      for (int p = 0; p < A_CH + B_PARTS; ++p) {
+         if (p % ngrp != grp) continue;
+         if (p < A_CH) {
+            if (do_stash) stash_a(G, stage, p);
+            if (do_fetch) fetch_a(G, k_next, p);
+         } else {
+            if (do_stash) stash_b(G, stage, p - A_CH);
+            if (do_fetch) fetch_b(G, k_next, p - A_CH);
+         }
+      }
+   };
+
+   typename Mma::Acc acc[TI][TJ];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+#pragma unroll
+         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+   const int frag_row = lane & 31;
+   const int frag_k = (lane >> 5) * Mma::LANE_BYTES;
+   const int a_off = (wm * TJ * 32 + frag_row) * LDK + frag_k;
+   const int b_off = (wn * TI * 32 + frag_row) * LDK + frag_k;
+   constexpr int TMAX = TI > TJ ? TI : TJ;
+   static_assert(NSUB >= 2 && NSUB % 2 == 0, "the software pipeline needs an even number of MFMA K-substeps per stage");
+
+   // Operand fragments: two register sets used alternately by consecutive MFMA K-substeps.
+   typename Mma::Frag fn[2][TI], fm[2][TJ];
+   auto read_pair = [&](int set, int stage, int sub, int i) {
+      if (i < TI) fn[set][i] = Mma::load(sB + stage * BN * LDK + b_off + i * 32 * LDK + sub * Mma::KB);
+      if (i < TJ) fm[set][i] = Mma::load(sA + stage * BM * LDK + a_off + i * 32 * LDK + sub * Mma::KB);
+   };
+   auto mma_row = [&](int set, int i) {
+      if (i < TI) {
+#pragma unroll
+         for (int j = 0; j < TJ; ++j) acc[i][j] = Mma::mma(fn[set][i], fm[set][j], acc[i][j]);
+      }
+   };
+
+   // One K-step on LDS stage `stage`. On entry fragment set 0 holds substep 0 of this stage.
+   //   substeps 0..NSUB-2: multiply while the next substep's fragments are read, and while
+   //                       register set G (tile of the next step) moves into the other stage
+   //                       and is re-requested for tile `k_next`;
+   //   barrier:            the other stage is complete and nobody reads this stage any more;
+   //   substep NSUB-1:     multiply while set 0 is refilled from the other stage.
+   // The instruction order is pinned with scheduling barriers so that every group of TJ MFMAs
+   // has memory instructions issued right behind it to overlap with.
+   auto kstep = [&](int stage, Staged &G, int k_next, bool more) {
+      constexpr int NGRP = (NSUB - 1) * TMAX;
+#pragma unroll
+      for (int sub = 0; sub < NSUB - 1; ++sub) {
+#pragma unroll
+         for (int i = 0; i < TMAX; ++i) {
+            read_pair((sub + 1) & 1, stage, sub + 1, i);
+            mma_row(sub & 1, i);
+            move_pieces(G, stage ^ 1, k_next, sub * TMAX + i, NGRP, more, true);
+            __builtin_amdgcn_sched_barrier(0);
+         }
+      }
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TMAX; ++i) {
+         if (more) read_pair(0, stage ^ 1, 0, i);
+         mma_row((NSUB - 1) & 1, i);
+         __builtin_amdgcn_sched_barrier(0);
+      }
+   };
+
+   const int nk = (g.K + BK - 1) / BK;
+   const int klast = nk > 0 ? (nk - 1) * BK : 0;
+   auto kclamp = [&](int t) { return t * BK < klast ? t * BK : klast; };
+   // Requests past the end of K re-read the last tile (never used): keeping every request
+   // unconditional keeps the number of loads in flight identical on every path.
+   Staged G[NSETS];
+   if (nk > 0) {
+      move_pieces(G[0], 0, 0, 0, 1, false, true);               // tile 0
+      move_pieces(G[0], 0, kclamp(NSETS), 0, 1, true, NSETS == 1);   // -> stage 0
+      if (NSETS == 2) {
+         move_pieces(G[1], 0, kclamp(1), 0, 1, false, true);   // tile 1
+         move_pieces(G[0], 0, kclamp(2), 0, 1, false, true);   // tile 2
+      }
+      __syncthreads();
+#pragma unroll
+      for (int i = 0; i < TMAX; ++i) read_pair(0, 0, 0, i);
+      __builtin_amdgcn_sched_barrier(0);
+   }
+   // step t multiplies stage t&1, moves tile t+1 (register set (t+1) % NSETS) into stage (t+1)&1
+   // and re-requests that set for tile t+1+NSETS
+   int kt = 0;
+   for (; kt + 2 <= nk; kt += 2) {
+      kstep(0, G[1 % NSETS], kclamp(kt + 1 + NSETS), true);
+      kstep(1, G[0], kclamp(kt + 2 + NSETS), kt + 2 < nk);
+   }
+   if (kt < nk) kstep(0, G[1 % NSETS], klast, false);
+   __syncthreads();
+
+   // --- epilogue: pack -> per-wavefront LDS staging -> 16-byte row segments -------------
+   constexpr int WN = TI * 32;                       // output columns of one wavefront
+   constexpr int SROW = WN * ESZ + 16;               // staging row stride in bytes
+   constexpr int CR = WN * ESZ / 16;                 // 16-byte chunks per staging row
+   unsigned char *stg = smem + wave * (32 * SROW);
+   float *s_scale = reinterpret_cast<float *>(smem + 4 * 32 * SROW);   // [BN] per-column scale
+   int *s_bias = reinterpret_cast<int *>(s_scale + BN);                // [BN] per-column bias bits
+   if (tid < BN) {
+      const int n = n0 + tid;
+      s_scale[tid] = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
+      s_bias[tid] = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
+   }
+   __syncthreads();
+   const int m_local = lane & 31;
+   const int nq = (lane >> 5) * 4;
+#pragma unroll
+   for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+      for (int i = 0; i < TI; ++i) {
+#pragma unroll
+         for (int q = 0; q < 4; ++q) {
+            const int nl = i * 32 + q * 8 + nq;
+            unsigned e[4];
+            const v4f sc = *reinterpret_cast<const v4f *>(s_scale + wn * WN + nl);
+            const v4i bi = *reinterpret_cast<const v4i *>(s_bias + wn * WN + nl);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+               if constexpr (IS_INT)
+                  e[t] = epilogue_value<true, OUT>(g, sc[t], bi[t], acc[i][j][q * 4 + t], 0.0f);
+               else
+                  e[t] = epilogue_value<false, OUT>(g, sc[t], bi[t], 0, acc[i][j][q * 4 + t]);
+            }
+            unsigned char *dst = stg + m_local * SROW + nl * ESZ;
+            if constexpr (ESZ == 1) {
+               *reinterpret_cast<unsigned *>(dst) = e[0] | (e[1] << 8) | (e[2] << 16) | (e[3] << 24);
+            } else if constexpr (ESZ == 2) {
+               v2i p = {(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16))};
+               *reinterpret_cast<v2i *>(dst) = p;
+            } else {
+               v4i p = {(int)e[0], (int)e[1], (int)e[2], (int)e[3]};
+               *reinterpret_cast<v4i *>(dst) = p;
+            }
+         }
+      }
+      __syncthreads();
+      constexpr int ITERS = 32 * CR / 64;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+         const int c = it * 64 + lane;
+         const int row = c / CR, cc = c % CR;
+         const int m = m0 + wm * (TJ * 32) + j * 32 + row;
+         const int nfirst = n0 + wn * WN + cc * (16 / ESZ);
+         if (m < g.M && nfirst < g.N) {
+            const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
+            unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
+            if (g.vec_store && nfirst + 16 / ESZ <= g.N) {
+               *reinterpret_cast<v4i *>(out) = v;
+            } else {
+               const unsigned char *src = stg + row * SROW + cc * 16;
+               const int cnt = (g.N - nfirst) < (16 / ESZ) ? (g.N - nfirst) : (16 / ESZ);
+               for (int b = 0; b < cnt * ESZ; ++b) out[b] = src[b];
+            }
+         }
+      }
+      __syncthreads();
+   }
+}
+
+// Any shape, any alignment: one thread per output element. Correctness path for operands
+// the tiled kernel cannot take (K not a multiple of 16, unaligned rows).
+template <bool IS_INT, int OUT>
+__global__ void k_gemm_bytes_simple(GemmArgs g, int transB)
+{
+   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   if (idx >= (size_t)g.M * g.N) return;
+   const int m = (int)(idx / g.N), n = (int)(idx % g.N);
+   const uint8_t *a = g.A + (size_t)m * g.lda;
+   constexpr int ESZ = OutSize<OUT>::value;
+   unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + n) * ESZ;
+   unsigned r;
+   if constexpr (IS_INT) {
+      int acc = 0;
+      for (int k = 0; k < g.K; ++k) {
+         const int b = (int)(int8_t)(transB ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n]);
+         acc += (int)(int8_t)a[k] * b;
+      }
+      r = epilogue_value<true, OUT>(g, g.scale ? g.scale[n] : 0.0f, g.bias ? static_cast<const int *>(g.bias)[n] : 0, acc, 0.0f);
+   } else {
+      float acc = 0.0f;
+      for (int k = 0; k < g.K; ++k) {
+         const unsigned b = transB ? g.B[(size_t)n * g.ldb + k] : g.B[(size_t)k * g.ldb + n];
+         acc = __fadd_rn(acc, __fmul_rn(e4m3_to_f32(a[k]), e4m3_to_f32(b)));
+      }
+      r = epilogue_value<false, OUT>(g, 0.0f, g.bias ? static_cast<const int *>(g.bias)[n] : 0, 0, acc);
+   }
+   if constexpr (ESZ == 1) *out = (unsigned char)r;
+   else if constexpr (ESZ == 2) *reinterpret_cast<unsigned short *>(out) = (unsigned short)r;
+   else *reinterpret_cast<unsigned *>(out) = r;
+}
+
+template <class Mma, int BK, int NSETS, int TI, int TJ, int OUT, bool B_KN, bool FULL>
+int launch_tiled_impl(sofie_hip_ctx *ctx, GemmArgs &g)
+{
+   constexpr int BN = 2 * TI * 32, BM = 2 * TJ * 32;
+   constexpr int LDK = BK + 16;
+   constexpr size_t stage_bytes = (size_t)2 * (BM + BN) * LDK;
+   constexpr size_t epi_bytes = (size_t)4 * 32 * (TI * 32 * OutSize<OUT>::value + 16) + (size_t)2 * BN * 4;
+   constexpr size_t lds = stage_bytes > epi_bytes ? stage_bytes : epi_bytes;
+   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
+   g.tiles_m = cdiv(g.M, BM);
+   g.tiles_n = cdiv(g.N, BN);
+   auto kern = k_gemm_bytes<Mma, BK, NSETS, TI, TJ, OUT, B_KN, FULL>;
+   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+   hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), lds, ctx->stream, g);
+   return check_launch(ctx, "k_gemm_bytes");
+}
+
+template <class Mma, int BK, int NSETS, int TI, int TJ, int OUT, bool B_KN>
+int launch_tiled(sofie_hip_ctx *ctx, GemmArgs &g)
+{
+   constexpr int BN = 2 * TI * 32, BM = 2 * TJ * 32;
+   if (g.M % BM == 0 && g.N % BN == 0 && g.K % BK == 0)
+      return launch_tiled_impl<Mma, BK, NSETS, TI, TJ, OUT, B_KN, true>(ctx, g);
+   return launch_tiled_impl<Mma, BK, NSETS, TI, TJ, OUT, B_KN, false>(ctx, g);
+}
+
+template <bool IS_INT, int OUT>
+int launch_simple(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
+{
+   const size_t total = (size_t)g.M * g.N;
+   hipLaunchKernelGGL((k_gemm_bytes_simple<IS_INT, OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
+                      ctx->stream, g, transB);
+   return check_launch(ctx, "k_gemm_bytes_simple");
+}
+
+template <class Mma, int OUT>
+int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
+{
+   constexpr bool IS_INT = __is_same(typename Mma::Acc, v16i);
+   constexpr int ESZ = OutSize<OUT>::value;
+   const bool a_ok = g.K % 16 == 0 && g.lda % 16 == 0 && aligned16(g.A);
+   const bool b_nk_ok = transB && g.ldb % 16 == 0 && aligned16(g.B);
+   const bool b_kn_ok = !transB && g.ldb % 4 == 0 && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.B) & 3u) == 0;
+   g.vec_store = ((size_t)g.ldy * ESZ) % 16 == 0 && aligned16(g.Y);
+   if (!a_ok || !(b_nk_ok || b_kn_ok)) return launch_simple<IS_INT, OUT>(ctx, g, transB);
+   const bool big = (size_t)g.M * g.N >= (size_t)256 * 256 * 128 && g.M >= 256 && g.N >= 256;
+   // 128 bytes of K per stage; int8 keeps two register sets in flight, fp8 (twice the
+   // fragment registers) one.
+   constexpr int BK = 128;
+   constexpr int NSETS = IS_INT ? 2 : 1;
+   if (transB) {
+      if (big) return launch_tiled<Mma, BK, NSETS, 4, 4, OUT, false>(ctx, g);
+      return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, false>(ctx, g);
+   }
+   if (big) return launch_tiled<Mma, BK, NSETS, 4, 4, OUT, true>(ctx, g);
+   return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, true>(ctx, g);
+}
+
+}  // namespace
+
+extern "C" {
+
+int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const int8_t *A, int lda,
+                       const int8_t *B, int ldb, const float *scale, const int32_t *bias, int zp_y,
+                       int act, void *Y, int ldy, int out_kind)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, M >= 0 && N >= 0 && K >= 0, "negative dimension");
+   if (M == 0 || N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, A && B && Y, "null operand");
+   SOFIE_REQUIRE(ctx, lda >= K && ldb >= (transB ? K : N) && ldy >= N, "leading dimension too small");
+   SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
+   SOFIE_REQUIRE(ctx, out_kind == SOFIE_OUT_S8 || out_kind == SOFIE_OUT_F32 || out_kind == SOFIE_OUT_S32,
+                 "output kind must be S8, F32 or S32");
+   SOFIE_REQUIRE(ctx, scale || out_kind == SOFIE_OUT_S32, "scale is required for S8/F32 output");
+   SOFIE_REQUIRE(ctx, zp_y >= -128 && zp_y <= 127, "zero-point out of int8 range");
+   GemmArgs g{};
+   g.A = reinterpret_cast<const uint8_t *>(A);
+   g.B = reinterpret_cast<const uint8_t *>(B);
+   g.Y = Y;
+   g.scale = scale;
+   g.bias = bias;
+   g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldy = ldy;
+   g.zp = zp_y;
+   g.relu = act == SOFIE_ACT_RELU;
+   g.lo = (g.relu && zp_y > -128) ? zp_y : -128;
+   g.s = 1.0f;
+   switch (out_kind) {
+   case SOFIE_OUT_S8: return dispatch<MmaI8, SOFIE_OUT_S8>(ctx, g, transB);
+   case SOFIE_OUT_F32: return dispatch<MmaI8, SOFIE_OUT_F32>(ctx, g, transB);
+   default: return dispatch<MmaI8, SOFIE_OUT_S32>(ctx, g, transB);
+   }
+}
+
+int sofie_hip_gemm_fp8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const uint8_t *A, int lda,
+                       const uint8_t *B, int ldb, float scale_a, float scale_b, const float *bias, void *Y,
+                       int ldy, int out_kind)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, M >= 0 && N >= 0 && K >= 0, "negative dimension");
+   if (M == 0 || N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, A && B && Y, "null operand");
+   SOFIE_REQUIRE(ctx, lda >= K && ldb >= (transB ? K : N) && ldy >= N, "leading dimension too small");
+   SOFIE_REQUIRE(ctx, out_kind == SOFIE_OUT_BF16 || out_kind == SOFIE_OUT_F32, "output kind must be BF16 or F32");
+   GemmArgs g{};
+   g.A = A; g.B = B; g.Y = Y;
+   g.scale = nullptr;
+   g.bias = bias;
+   g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldy = ldy;
+   g.s = scale_a * scale_b;
+   if (out_kind == SOFIE_OUT_BF16) return dispatch<MmaF8, SOFIE_OUT_BF16>(ctx, g, transB);
+   return dispatch<MmaF8, SOFIE_OUT_F32>(ctx, g, transB);
+}
+
+}  // extern "C"

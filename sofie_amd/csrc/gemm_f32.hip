@@ -1,0 +1,172 @@
+// fp32 GEMM on the matrix cores (v_mfma_f32_32x32x2_f32) with a fused
+// alpha / beta*bias / ReLU epilogue.
+//
+// 256 threads = 4 wavefronts (2x2), each owning TI x TJ tiles of 32x32. Operands are staged
+// in LDS k-major ([k][row]) so that the one-float-per-lane MFMA operand read is a conflict-free
+// ds_read_b32 for either storage order of A and B; the accumulator layout puts 32 consecutive
+// output columns in 32 consecutive lanes, so results are stored straight from registers as
+// 128-byte row segments. Loads are guarded scalar loads: no alignment or size restrictions.
+// Roofline: MFMA fp32 (256 flop/clk/CU); each K-step of 16 issues 8*TI*TJ MFMAs of 64 cycles
+// per wavefront against 16 scalar loads per thread.
+#include "common.h"
+
+using namespace sofie;
+
+namespace {
+
+struct GemmF32Args {
+   const float *A, *B, *bias;
+   float *Y;
+   int M, N, K, lda, ldb, ldy;
+   int transA, transB;
+   float alpha, beta;
+   int bias_kind, relu;
+};
+
+constexpr int BK = 16;
+
+// Stage a [rows x BK] block of a matrix into LDS as dst[k][row].
+// k_major_src: the source is stored [K][rows] (row index contiguous); else [rows][K].
+template <int ROWS, int LD>
+__device__ __forceinline__ void fetch(float (&reg)[ROWS * BK / 256], const float *src, int ld, bool k_major_src,
+                                      int row0, int k0, int nrows, int K, int tid)
+{
+#pragma unroll
+   for (int i = 0; i < ROWS * BK / 256; ++i) {
+      const int e = i * 256 + tid;
+      int r, k;
+      if (k_major_src) { k = e / ROWS; r = e % ROWS; }
+      else { r = e / BK; k = e % BK; }
+      const int gr = row0 + r, gk = k0 + k;
+      float v = 0.0f;
+      if (gr < nrows && gk < K) v = k_major_src ? src[(size_t)gk * ld + gr] : src[(size_t)gr * ld + gk];
+      reg[i] = v;
+   }
+}
+
+template <int ROWS, int LD>
+__device__ __forceinline__ void stash(const float (&reg)[ROWS * BK / 256], float *dst, bool k_major_src, int tid)
+{
+#pragma unroll
+   for (int i = 0; i < ROWS * BK / 256; ++i) {
+      const int e = i * 256 + tid;
+      int r, k;
+      if (k_major_src) { k = e / ROWS; r = e % ROWS; }
+      else { r = e / BK; k = e % BK; }
+      dst[k * LD + r] = reg[i];
+   }
+}
+
+template <int TI, int TJ>
+__global__ void __launch_bounds__(256) k_gemm_f32(GemmF32Args g)
+{
+   constexpr int BM = 2 * TI * 32, BN = 2 * TJ * 32;
+   constexpr int LDA = BM + 4, LDB = BN + 4;
+   __shared__ float sA[2][BK * LDA];
+   __shared__ float sB[2][BK * LDB];
+
+   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int wm = wave >> 1, wn = wave & 1;
+   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+
+   float ra[BM * BK / 256], rb[BN * BK / 256];
+   v16f acc[TI][TJ];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+#pragma unroll
+         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+   const bool a_kmajor = g.transA != 0;   // A stored [K][M]
+   const bool b_kmajor = g.transB == 0;   // B stored [K][N]
+   const int nk = (g.K + BK - 1) / BK;
+
+   fetch<BM, LDA>(ra, g.A, g.lda, a_kmajor, m0, 0, g.M, g.K, tid);
+   fetch<BN, LDB>(rb, g.B, g.ldb, b_kmajor, n0, 0, g.N, g.K, tid);
+   stash<BM, LDA>(ra, sA[0], a_kmajor, tid);
+   stash<BN, LDB>(rb, sB[0], b_kmajor, tid);
+   __syncthreads();
+
+   const int fr = lane & 31, fk = lane >> 5;
+   for (int kt = 0; kt < nk; ++kt) {
+      const int cur = kt & 1;
+      if (kt + 1 < nk) {
+         fetch<BM, LDA>(ra, g.A, g.lda, a_kmajor, m0, (kt + 1) * BK, g.M, g.K, tid);
+         fetch<BN, LDB>(rb, g.B, g.ldb, b_kmajor, n0, (kt + 1) * BK, g.N, g.K, tid);
+      }
+      const float *a = sA[cur] + fk * LDA + wm * TI * 32 + fr;
+      const float *b = sB[cur] + fk * LDB + wn * TJ * 32 + fr;
+#pragma unroll
+      for (int s = 0; s < BK / 2; ++s) {
+         float fa[TI], fb[TJ];
+#pragma unroll
+         for (int i = 0; i < TI; ++i) fa[i] = a[2 * s * LDA + i * 32];
+#pragma unroll
+         for (int j = 0; j < TJ; ++j) fb[j] = b[2 * s * LDB + j * 32];
+#pragma unroll
+         for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+      if (kt + 1 < nk) {
+         stash<BM, LDA>(ra, sA[cur ^ 1], a_kmajor, tid);
+         stash<BN, LDB>(rb, sB[cur ^ 1], b_kmajor, tid);
+      }
+      __syncthreads();
+   }
+
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) {
+         const int n = n0 + wn * TJ * 32 + j * 32 + fr;
+         if (n >= g.N) continue;
+         float brow = 0.0f;
+         if (g.bias_kind == SOFIE_BIAS_ROW) brow = __fmul_rn(g.beta, g.bias[n]);
+#pragma unroll
+         for (int r = 0; r < 16; ++r) {
+            const int m = m0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
+            if (m >= g.M) continue;
+            float v = __fmul_rn(g.alpha, acc[i][j][r]);
+            if (g.bias_kind == SOFIE_BIAS_ROW) v = __fadd_rn(v, brow);
+            else if (g.bias_kind == SOFIE_BIAS_FULL) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[(size_t)m * g.ldy + n]));
+            else if (g.bias_kind == SOFIE_BIAS_COL) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[m]));
+            if (g.relu) v = v > 0.0f ? v : 0.0f;
+            g.Y[(size_t)m * g.ldy + n] = v;
+         }
+      }
+}
+
+}  // namespace
+
+extern "C" int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, int M, int N, int K, float alpha,
+                                  const float *A, int lda, const float *B, int ldb, float beta, const float *bias,
+                                  int bias_kind, float *Y, int ldy, int act)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, M >= 0 && N >= 0 && K >= 0, "negative dimension");
+   if (M == 0 || N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, Y && (K == 0 || (A && B)), "null operand");
+   SOFIE_REQUIRE(ctx, lda >= (transA ? M : K) && ldb >= (transB ? K : N) && ldy >= N, "leading dimension too small");
+   SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
+   SOFIE_REQUIRE(ctx, bias_kind >= SOFIE_BIAS_NONE && bias_kind <= SOFIE_BIAS_COL, "unknown bias kind");
+   if (!bias || bias_kind == SOFIE_BIAS_NONE) {
+      // Same rule as the reference emitter: without a bias tensor beta must be zero.
+      if (beta != 0.0f)
+         return sofie::set_error(ctx, SOFIE_HIP_EINVAL,
+                                 "sofie_hip_gemm_f32: Bias tensor is not present but beta value in Gemm is not zero");
+      bias = nullptr;
+      bias_kind = SOFIE_BIAS_NONE;
+   }
+   GemmF32Args g{A, B, bias, Y, M, N, K, lda, ldb, ldy, transA != 0, transB != 0, alpha, beta, bias_kind,
+                 act == SOFIE_ACT_RELU};
+   const bool small = (size_t)cdiv(M, 128) * cdiv(N, 128) < 256;
+   if (small) {
+      hipLaunchKernelGGL((k_gemm_f32<1, 1>), dim3(cdiv(N, 64), cdiv(M, 64)), dim3(256), 0, ctx->stream, g);
+   } else {
+      hipLaunchKernelGGL((k_gemm_f32<2, 2>), dim3(cdiv(N, 128), cdiv(M, 128)), dim3(256), 0, ctx->stream, g);
+   }
+   return check_launch(ctx, "k_gemm_f32");
+}

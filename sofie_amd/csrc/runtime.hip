@@ -1,0 +1,176 @@
+// Context, memory and timing entry points of libsofie_hip.so.
+#include <stdarg.h>
+
+#include "common.h"
+
+namespace sofie {
+
+int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...)
+{
+   if (ctx) {
+      va_list ap;
+      va_start(ap, fmt);
+      vsnprintf(ctx->err, sizeof(ctx->err), fmt, ap);
+      va_end(ap);
+   }
+   return code;
+}
+
+int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr)
+{
+   if (bytes > ctx->workspace_bytes) {
+      // the old buffer may still be read by kernels in flight on the stream
+      if (ctx->workspace) {
+         SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
+         SOFIE_HIP_CALL(ctx, hipFree(ctx->workspace));
+         ctx->workspace = nullptr;
+         ctx->workspace_bytes = 0;
+      }
+      size_t want = bytes + (bytes >> 2);
+      if (hipMalloc(&ctx->workspace, want) != hipSuccess) {
+         (void)hipGetLastError();
+         return set_error(ctx, SOFIE_HIP_ENOMEM, "workspace of %zu bytes", want);
+      }
+      ctx->workspace_bytes = want;
+   }
+   *ptr = ctx->workspace;
+   return SOFIE_HIP_OK;
+}
+
+int check_launch(sofie_hip_ctx *ctx, const char *what)
+{
+   hipError_t e = hipGetLastError();
+   if (e != hipSuccess)
+      return set_error(ctx, SOFIE_HIP_EHIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+   return SOFIE_HIP_OK;
+}
+
+}  // namespace sofie
+
+extern "C" {
+
+int sofie_hip_version(void) { return 1; }
+
+int sofie_hip_create(sofie_hip_ctx **out, int device, void *stream)
+{
+   if (!out) return SOFIE_HIP_EINVAL;
+   *out = nullptr;
+   int count = 0;
+   if (hipGetDeviceCount(&count) != hipSuccess || device < 0 || device >= count) return SOFIE_HIP_EHIP;
+   if (hipSetDevice(device) != hipSuccess) return SOFIE_HIP_EHIP;
+   sofie_hip_ctx *ctx = new sofie_hip_ctx();
+   ctx->device = device;
+   if (stream) {
+      ctx->stream = static_cast<hipStream_t>(stream);
+   } else {
+      if (hipStreamCreate(&ctx->stream) != hipSuccess) { delete ctx; return SOFIE_HIP_EHIP; }
+      ctx->owns_stream = true;
+   }
+   if (hipEventCreate(&ctx->ev_start) != hipSuccess || hipEventCreate(&ctx->ev_stop) != hipSuccess) {
+      if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+      delete ctx;
+      return SOFIE_HIP_EHIP;
+   }
+   *out = ctx;
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_destroy(sofie_hip_ctx *ctx)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   (void)hipStreamSynchronize(ctx->stream);
+   if (ctx->workspace) (void)hipFree(ctx->workspace);
+   (void)hipEventDestroy(ctx->ev_start);
+   (void)hipEventDestroy(ctx->ev_stop);
+   if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+   delete ctx;
+   return SOFIE_HIP_OK;
+}
+
+const char *sofie_hip_last_error(const sofie_hip_ctx *ctx) { return ctx ? ctx->err : "null context"; }
+
+int sofie_hip_malloc(sofie_hip_ctx *ctx, void **dptr, size_t bytes)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, dptr != nullptr, "null result pointer");
+   *dptr = nullptr;
+   if (bytes == 0) return SOFIE_HIP_OK;
+   if (hipMalloc(dptr, bytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return sofie::set_error(ctx, SOFIE_HIP_ENOMEM, "sofie_hip_malloc: %zu bytes", bytes);
+   }
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_free(sofie_hip_ctx *ctx, void *dptr)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (!dptr) return SOFIE_HIP_OK;
+   SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
+   SOFIE_HIP_CALL(ctx, hipFree(dptr));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_upload(sofie_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (bytes == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, dst && src, "null pointer");
+   SOFIE_HIP_CALL(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
+   SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_download(sofie_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (bytes == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, dst && src, "null pointer");
+   SOFIE_HIP_CALL(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
+   SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_copy(sofie_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (bytes == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, dst && src, "null pointer");
+   SOFIE_HIP_CALL(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_memset(sofie_hip_ctx *ctx, void *dptr, int value, size_t bytes)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (bytes == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, dptr != nullptr, "null pointer");
+   SOFIE_HIP_CALL(ctx, hipMemsetAsync(dptr, value, bytes, ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_sync(sofie_hip_ctx *ctx)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_timer_start(sofie_hip_ctx *ctx)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_HIP_CALL(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *ms)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, ms != nullptr, "null result pointer");
+   SOFIE_HIP_CALL(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
+   SOFIE_HIP_CALL(ctx, hipEventSynchronize(ctx->ev_stop));
+   SOFIE_HIP_CALL(ctx, hipEventElapsedTime(ms, ctx->ev_start, ctx->ev_stop));
+   return SOFIE_HIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,292 @@
+"""Operator front end over the C ABI: numpy or torch arrays in, same kind out.
+
+torch is used only to own device memory and the stream; every computation is a call into
+libsofie_hip.so. The function names and argument meanings mirror what the reference's
+operators compute (ROperator_Gemm, ROperator_Conv, ROperator_Relu, ROperator_Pool) plus the
+quantized / FP8 operators this library adds.
+"""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import lib as L
+
+
+class SofieHipError(RuntimeError):
+    pass
+
+
+class Context:
+    """One sofie_hip_ctx bound to torch's current stream on `device`."""
+
+    def __init__(self, device=0):
+        if not torch.cuda.is_available():
+            raise SofieHipError("no GPU visible: the HIP library has no CPU fallback")
+        self.lib = L.load()
+        self.device = torch.device("cuda", device)
+        torch.cuda.set_device(self.device)
+        self.stream = torch.cuda.current_stream(self.device)
+        h = C.c_void_p()
+        rc = self.lib.sofie_hip_create(C.byref(h), device, C.c_void_p(self.stream.cuda_stream))
+        if rc:
+            raise SofieHipError("sofie_hip_create failed: %d" % rc)
+        self.h = h
+
+    def close(self):
+        if self.h:
+            self.lib.sofie_hip_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def check(self, rc):
+        if rc:
+            msg = self.lib.sofie_hip_last_error(self.h).decode()
+            raise SofieHipError("%s (status %d)" % (msg, rc))
+
+    def sync(self):
+        self.check(self.lib.sofie_hip_sync(self.h))
+
+    def timer_start(self):
+        self.check(self.lib.sofie_hip_timer_start(self.h))
+
+    def timer_stop(self):
+        ms = C.c_float()
+        self.check(self.lib.sofie_hip_timer_stop(self.h, C.byref(ms)))
+        return ms.value
+
+    # -- helpers ---------------------------------------------------------------------
+    def dev(self, a, dtype=None):
+        """numpy/torch -> contiguous device tensor (no copy if already there)."""
+        if a is None:
+            return None
+        if isinstance(a, np.ndarray):
+            a = torch.from_numpy(np.ascontiguousarray(a))
+        if dtype is not None and a.dtype != dtype:
+            a = a.to(dtype)
+        return a.to(self.device).contiguous()
+
+    @staticmethod
+    def ptr(t):
+        return C.c_void_p(t.data_ptr()) if t is not None else None
+
+    def empty(self, shape, dtype):
+        return torch.empty(shape, dtype=dtype, device=self.device)
+
+
+_default = None
+
+
+def default_context():
+    global _default
+    if _default is None:
+        _default = Context(0)
+    return _default
+
+
+def _ret(t, like):
+    return t.cpu().numpy() if isinstance(like, np.ndarray) else t
+
+
+# ------------------------------------------------------------------------------- fp32
+def gemm_f32(A, B, bias=None, alpha=1.0, beta=1.0, transA=False, transB=False, relu=False, ctx=None):
+    """Y = alpha*op(A)*op(B) + beta*bias [ReLU]; bias rank-1 [N] or full [M,N]."""
+    ctx = ctx or default_context()
+    a, b = ctx.dev(A, torch.float32), ctx.dev(B, torch.float32)
+    M, K = (a.shape[1], a.shape[0]) if transA else a.shape
+    N = b.shape[0] if transB else b.shape[1]
+    y = ctx.empty((M, N), torch.float32)
+    kind, bt = L.BIAS_NONE, None
+    if bias is not None:
+        bt = ctx.dev(bias, torch.float32)
+        if bt.numel() == N and bt.dim() <= 2 and bt.shape[-1] == N:
+            kind = L.BIAS_ROW
+        elif tuple(bt.shape) == (M, N):
+            kind = L.BIAS_FULL
+        else:
+            raise SofieHipError("bias shape %s cannot be broadcast to (%d, %d)" % (tuple(bt.shape), M, N))
+    ctx.check(ctx.lib.sofie_hip_gemm_f32(ctx.h, int(transA), int(transB), M, N, K, alpha, ctx.ptr(a), a.shape[1],
+                                         ctx.ptr(b), b.shape[1], beta, ctx.ptr(bt), kind, ctx.ptr(y), N,
+                                         L.ACT_RELU if relu else L.ACT_NONE))
+    return _ret(y, A)
+
+
+def relu_f32(x, ctx=None):
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.float32)
+    y = torch.empty_like(xd)
+    ctx.check(ctx.lib.sofie_hip_relu_f32(ctx.h, ctx.ptr(xd), ctx.ptr(y), xd.numel()))
+    return _ret(y, x)
+
+
+def conv_out_hw(H, W, kh, kw, ph, pw, sh, sw, dh=1, dw=1):
+    return ((H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1, (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1)
+
+
+def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), groups=1, relu=False, ctx=None):
+    ctx = ctx or default_context()
+    xd, wd, bd = ctx.dev(x, torch.float32), ctx.dev(w, torch.float32), ctx.dev(bias, torch.float32)
+    N, Cc, H, W = xd.shape
+    OC, _, kh, kw = wd.shape
+    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1], *dilations)
+    y = ctx.empty((N, OC, OH, OW), torch.float32)
+    ctx.check(ctx.lib.sofie_hip_conv2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, H, W,
+                                           OC, kh, kw, pads[0], pads[1], strides[0], strides[1], dilations[0],
+                                           dilations[1], groups, L.ACT_RELU if relu else L.ACT_NONE))
+    return _ret(y, x)
+
+
+def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0), layout=L.LAYOUT_NCHW, ctx=None):
+    """pads = (top, left, bottom, right). int8 tensors may be NHWC (layout flag); fp32 is NCHW."""
+    ctx = ctx or default_context()
+    xd = ctx.dev(x)
+    if layout == L.LAYOUT_NCHW:
+        N, Cc, H, W = xd.shape
+    else:
+        N, H, W, Cc = xd.shape
+    OH = (H + pads[0] + pads[2] - kernel[0]) // strides[0] + 1
+    OW = (W + pads[1] + pads[3] - kernel[1]) // strides[1] + 1
+    shape = (N, Cc, OH, OW) if layout == L.LAYOUT_NCHW else (N, OH, OW, Cc)
+    y = ctx.empty(shape, xd.dtype)
+    if xd.dtype == torch.float32:
+        ctx.check(ctx.lib.sofie_hip_maxpool2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(y), N * Cc, H, W, kernel[0],
+                                                  kernel[1], pads[0], pads[1], pads[2], pads[3], strides[0],
+                                                  strides[1]))
+    else:
+        ctx.check(ctx.lib.sofie_hip_maxpool2d_s8(ctx.h, ctx.ptr(xd), ctx.ptr(y), layout, N, Cc, H, W, kernel[0],
+                                                 kernel[1], pads[0], pads[1], pads[2], pads[3], strides[0],
+                                                 strides[1]))
+    return _ret(y, x)
+
+
+# ------------------------------------------------------------------------------- int8
+def quantize_f32_s8(x, scale, zp=0, ctx=None):
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.float32)
+    q = ctx.empty(xd.shape, torch.int8)
+    ctx.check(ctx.lib.sofie_hip_quantize_f32_s8(ctx.h, ctx.ptr(xd), ctx.ptr(q), xd.numel(), float(scale), int(zp)))
+    return _ret(q, x)
+
+
+def dequantize_s8_f32(q, scale, zp=0, ctx=None):
+    ctx = ctx or default_context()
+    qd = ctx.dev(q, torch.int8)
+    x = ctx.empty(qd.shape, torch.float32)
+    ctx.check(ctx.lib.sofie_hip_dequantize_s8_f32(ctx.h, ctx.ptr(qd), ctx.ptr(x), qd.numel(), float(scale), int(zp)))
+    return _ret(x, q)
+
+
+_OUT_DTYPE = {L.OUT_S8: torch.int8, L.OUT_F32: torch.float32, L.OUT_S32: torch.int32, L.OUT_BF16: torch.bfloat16}
+
+
+def fold_zero_point_gemm(B, bias, zpa, transB=False):
+    """bias[n] - zp_a * sum_k B[k,n]: lets the kernel accumulate raw A values (host side, once)."""
+    Bn = np.asarray(B.cpu() if isinstance(B, torch.Tensor) else B).astype(np.int64)
+    colsum = Bn.sum(axis=1 if transB else 0)
+    base = np.zeros(colsum.shape, np.int64) if bias is None else \
+        np.asarray(bias.cpu() if isinstance(bias, torch.Tensor) else bias).astype(np.int64)
+    return (base - int(zpa) * colsum).astype(np.int32)
+
+
+def qgemm_s8(A, B, scale, bias=None, transB=False, zpa=0, zpy=0, relu=False, out=L.OUT_S8, ctx=None):
+    """int8 GEMM, int32 accumulate, per-column scale; out: OUT_S8 / OUT_F32 / OUT_S32."""
+    ctx = ctx or default_context()
+    if zpa != 0:
+        bias = fold_zero_point_gemm(B, bias, zpa, transB)
+    a, b = ctx.dev(A, torch.int8), ctx.dev(B, torch.int8)
+    M, K = a.shape
+    N = b.shape[0] if transB else b.shape[1]
+    sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
+    y = ctx.empty((M, N), _OUT_DTYPE[out])
+    ctx.check(ctx.lib.sofie_hip_qgemm_s8(ctx.h, int(transB), M, N, K, ctx.ptr(a), a.shape[1], ctx.ptr(b),
+                                         b.shape[1], ctx.ptr(sd), ctx.ptr(bd), int(zpy),
+                                         L.ACT_RELU if relu else L.ACT_NONE, ctx.ptr(y), N, out))
+    return _ret(y, A)
+
+
+def qgemm_s8_f32out(A, B, scale, bias=None, transB=False, zpa=0, relu=False, ctx=None):
+    return qgemm_s8(A, B, scale, bias, transB, zpa, 0, relu, L.OUT_F32, ctx)
+
+
+def igemm_s8(A, B, transB=False, ctx=None):
+    return qgemm_s8(A, B, None, None, transB, out=L.OUT_S32, ctx=ctx)
+
+
+def fold_zero_point_conv(w, bias, zpx):
+    wn = np.asarray(w.cpu() if isinstance(w, torch.Tensor) else w).astype(np.int64)
+    wsum = wn.reshape(wn.shape[0], -1).sum(axis=1)
+    base = np.zeros(wsum.shape, np.int64) if bias is None else \
+        np.asarray(bias.cpu() if isinstance(bias, torch.Tensor) else bias).astype(np.int64)
+    return (base - int(zpx) * wsum).astype(np.int32)
+
+
+def qconv2d_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, zpy=0, relu=False,
+               x_layout=L.LAYOUT_NCHW, y_layout=L.LAYOUT_NCHW, out=L.OUT_S8, ctx=None):
+    """QLinearConv. x in x_layout, w [OC, C/g, KH, KW]; bias is the ONNX int32 bias (the input
+    zero-point is folded here, host side, as a Session constructor would do once)."""
+    ctx = ctx or default_context()
+    if zpx != 0:
+        bias = fold_zero_point_conv(w, bias, zpx)
+    xd, wd = ctx.dev(x, torch.int8), ctx.dev(w, torch.int8)
+    if x_layout == L.LAYOUT_NCHW:
+        N, Cc, H, W = xd.shape
+    else:
+        N, H, W, Cc = xd.shape
+    OC, _, kh, kw = wd.shape
+    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1])
+    shape = (N, OC, OH, OW) if y_layout == L.LAYOUT_NCHW else (N, OH, OW, OC)
+    y = ctx.empty(shape, _OUT_DTYPE[out])
+    sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
+    ctx.check(ctx.lib.sofie_hip_qconv2d_s8(ctx.h, ctx.ptr(xd), x_layout, ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(sd),
+                                           ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, pads[0], pads[1],
+                                           strides[0], strides[1], groups, int(zpx), int(zpy),
+                                           L.ACT_RELU if relu else L.ACT_NONE, out))
+    return _ret(y, x)
+
+
+def iconv2d_s8(x, w, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, ctx=None):
+    return qconv2d_s8(x, w, None, None, pads, strides, groups, zpx, out=L.OUT_S32, ctx=ctx)
+
+
+def relayout_s8(x, from_layout, to_layout, ctx=None):
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.int8)
+    if from_layout == L.LAYOUT_NCHW:
+        N, Cc, H, W = xd.shape
+    else:
+        N, H, W, Cc = xd.shape
+    shape = (N, Cc, H, W) if to_layout == L.LAYOUT_NCHW else (N, H, W, Cc)
+    y = ctx.empty(shape, torch.int8)
+    ctx.check(ctx.lib.sofie_hip_relayout_s8(ctx.h, ctx.ptr(xd), ctx.ptr(y), N, Cc, H, W, from_layout, to_layout))
+    return _ret(y, x)
+
+
+# ------------------------------------------------------------------------------- fp8
+def quantize_f32_e4m3(x, inv_scale, ctx=None):
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.float32)
+    q = ctx.empty(xd.shape, torch.uint8)
+    ctx.check(ctx.lib.sofie_hip_quantize_f32_e4m3(ctx.h, ctx.ptr(xd), ctx.ptr(q), xd.numel(), float(inv_scale)))
+    return _ret(q, x)
+
+
+def gemm_fp8(A, B, sa, sb, bias=None, transB=False, out=L.OUT_BF16, ctx=None):
+    """e4m3 codes (uint8) in; returns bf16 bit patterns as uint16 (numpy) / bfloat16 tensor, or fp32."""
+    ctx = ctx or default_context()
+    a, b = ctx.dev(A, torch.uint8), ctx.dev(B, torch.uint8)
+    M, K = a.shape
+    N = b.shape[0] if transB else b.shape[1]
+    bd = ctx.dev(bias, torch.float32)
+    y = ctx.empty((M, N), _OUT_DTYPE[out])
+    ctx.check(ctx.lib.sofie_hip_gemm_fp8(ctx.h, int(transB), M, N, K, ctx.ptr(a), a.shape[1], ctx.ptr(b),
+                                         b.shape[1], float(sa), float(sb), ctx.ptr(bd), ctx.ptr(y), N, out))
+    if isinstance(A, np.ndarray):
+        if out == L.OUT_BF16:
+            return y.view(torch.int16).cpu().numpy().view(np.uint16)
+        return y.cpu().numpy()
+    return y
