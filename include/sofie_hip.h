@@ -172,6 +172,14 @@ int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int l
 int sofie_hip_relayout_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int N, int C, int H,
                           int W, int from_layout, int to_layout);
 
+/* One-byte-element matrix transpose: src [rows, cols] (ld_src) -> dst [cols, rows] (ld_dst).
+ * Used once per weight tensor by a Session constructor to bring an ONNX [K,N] int8 / e4m3
+ * matrix into the K-contiguous [N,K] layout the GEMM kernels read fastest (then transB = 1);
+ * the reference re-lays weights out on every infer call instead (ROperator_Conv.hxx:342-363).
+ * rows % 16 == 0, cols % 4 == 0, ld_src % 4 == 0, ld_dst % 16 == 0. */
+int sofie_hip_transpose_bytes(sofie_hip_ctx *ctx, const void *src, void *dst, int rows, int cols,
+                              int ld_src, int ld_dst);
+
 /* FP8 e4m3 (OCP e4m3fn) GEMM with fp32 accumulation:
  *   t = (sum_k a*b) * (scale_a*scale_b) [+ bias[n]]  -> bf16 (RNE) or fp32.
  * A [M,K] row-major; B [K,N] row-major or, if transB, [N,K]; bias [N] fp32 or NULL. */

@@ -42,6 +42,17 @@ __device__ __forceinline__ int requant(int acc, float scale, int zp, int lo)
    return min(127, max(lo, q));
 }
 
+// The same requantisation, returned as the float (q + 128) in [0, 255] for epilogues that
+// pack with v_cvt_pk_u8_f32: rint(float(acc)*scale) + zp + 128, clamped below at lo + 128;
+// the clamp at 255 (q = 127) and at 0 (q = -128) is the saturation of the u8 conversion.
+// All quantities are integers well inside fp32's exact range after the first clamp.
+__device__ __forceinline__ float requant_biased(int acc, float scale, int zp, int lo)
+{
+   float r = rintf(__fmul_rn(__int2float_rn(acc), scale));
+   r = fminf(fmaxf(r, -1024.0f), 1024.0f);
+   return fmaxf(r + (float)(zp + 128), (float)(lo + 128));
+}
+
 // fp32 -> bf16 bits, round to nearest even, NaN quieted.
 __device__ __forceinline__ unsigned f32_to_bf16(float x)
 {

@@ -84,7 +84,7 @@ __device__ __forceinline__ unsigned epilogue_value(const GemmArgs &g, float sc, 
    if constexpr (IS_INT) {
       const int a = raw_i + bias_bits;
       if constexpr (OUT == SOFIE_OUT_S32) return (unsigned)a;
-      if constexpr (OUT == SOFIE_OUT_S8) return (unsigned)requant(a, sc, g.zp, g.lo) & 0xffu;
+      if constexpr (OUT == SOFIE_OUT_S8) return __float_as_uint(requant_biased(a, sc, g.zp, g.lo));
       float v = __fmul_rn(__int2float_rn(a), sc);
       if (g.relu && !(v > 0.0f)) v = 0.0f;
       return __float_as_uint(v);
@@ -94,6 +94,113 @@ __device__ __forceinline__ unsigned epilogue_value(const GemmArgs &g, float sc, 
       if constexpr (OUT == SOFIE_OUT_BF16) return f32_to_bf16(t);
       return __float_as_uint(t);
    }
+}
+
+// Epilogue shared by the tiled kernels. Each wavefront owns TI x TJ accumulator tiles
+// (rows = output columns n, columns = output rows m). Per pass j it converts TI tiles, packs
+// four consecutive n of one m into a 4*esize store into its private LDS staging block
+// [32 m][TI*32 n], then the wavefront writes the block out as 16-byte row segments.
+// smem is reused: all waves must have finished reading operand stages before the call.
+//   m_wave: first output row of this wavefront; n0: first output column of the workgroup;
+//   wn: index of the wavefront's column block; BN: columns of the workgroup tile.
+template <class Mma, int TI, int TJ, int OUT, int NWAVES>
+__device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ], unsigned char *smem,
+                                              int tid, int m_wave, int n0, int wn, int BN)
+{
+   constexpr int ESZ = OutSize<OUT>::value;
+   constexpr bool IS_INT = __is_same(typename Mma::Acc, v16i);
+   constexpr int WN = TI * 32;                       // output columns of one wavefront
+   constexpr int SROW = WN * ESZ + 16;               // staging row stride in bytes
+   constexpr int CR = WN * ESZ / 16;                 // 16-byte chunks per staging row
+   const int lane = tid & 63, wave = tid >> 6;
+   unsigned char *stg = smem + wave * (32 * SROW);
+   float *s_scale = reinterpret_cast<float *>(smem + NWAVES * 32 * SROW);   // [BN] per-column scale
+   int *s_bias = reinterpret_cast<int *>(s_scale + BN);                     // [BN] per-column bias bits
+   if (tid < BN) {
+      const int n = n0 + tid;
+      s_scale[tid] = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
+      s_bias[tid] = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
+   }
+   __syncthreads();
+   const int m_local = lane & 31;
+   const int nq = (lane >> 5) * 4;
+#pragma unroll
+   for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+      for (int i = 0; i < TI; ++i) {
+#pragma unroll
+         for (int q = 0; q < 4; ++q) {
+            const int nl = i * 32 + q * 8 + nq;
+            unsigned e[4];
+            const v4f sc = *reinterpret_cast<const v4f *>(s_scale + wn * WN + nl);
+            const v4i bi = *reinterpret_cast<const v4i *>(s_bias + wn * WN + nl);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+               if constexpr (IS_INT)
+                  e[t] = epilogue_value<true, OUT>(g, sc[t], bi[t], acc[i][j][q * 4 + t], 0.0f);
+               else
+                  e[t] = epilogue_value<false, OUT>(g, sc[t], bi[t], 0, acc[i][j][q * 4 + t]);
+            }
+            unsigned char *dst = stg + m_local * SROW + nl * ESZ;
+            if constexpr (ESZ == 1) {
+               // e[] hold q+128 as floats in [0,255]: convert-and-insert, then flip the sign bits
+               unsigned pk = 0;
+               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[0]), 0, pk);
+               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[1]), 1, pk);
+               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[2]), 2, pk);
+               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[3]), 3, pk);
+               *reinterpret_cast<unsigned *>(dst) = pk ^ 0x80808080u;
+            } else if constexpr (ESZ == 2) {
+               v2i p = {(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16))};
+               *reinterpret_cast<v2i *>(dst) = p;
+            } else {
+               v4i p = {(int)e[0], (int)e[1], (int)e[2], (int)e[3]};
+               *reinterpret_cast<v4i *>(dst) = p;
+            }
+         }
+      }
+      __syncthreads();
+      constexpr int ITERS = 32 * CR / 64;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+         const int c = it * 64 + lane;
+         const int row = c / CR, cc = c % CR;
+         const int m = m_wave + j * 32 + row;
+         const int nfirst = n0 + wn * WN + cc * (16 / ESZ);
+         if (m < g.M && nfirst < g.N) {
+            const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
+            unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
+            if (g.vec_store && nfirst + 16 / ESZ <= g.N) {
+               *reinterpret_cast<v4i *>(out) = v;
+            } else {
+               const unsigned char *src = stg + row * SROW + cc * 16;
+               const int cnt = (g.N - nfirst) < (16 / ESZ) ? (g.N - nfirst) : (16 / ESZ);
+               for (int b = 0; b < cnt * ESZ; ++b) out[b] = src[b];
+            }
+         }
+      }
+      __syncthreads();
+   }
+}
+
+// Workgroup id -> output tile. Ids are dealt round-robin over the 8 XCDs, each with its own
+// L2; the remap gives every XCD a contiguous run of ids and the grouped order turns that run
+// into a compact rectangle of tiles, so an XCD's L2 sees each operand panel once.
+__device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tiles_n, int &tm, int &tn)
+{
+   const int tiles = tiles_m * tiles_n;
+   {
+      const int xcd = pid & 7, local = pid >> 3;
+      const int base = tiles >> 3, rem = tiles & 7;
+      pid = local + xcd * base + (xcd < rem ? xcd : rem);
+   }
+   constexpr int GM = 4;
+   const int width = GM * tiles_n;
+   const int group = pid / width;
+   const int first = group * GM;
+   const int gsize = (tiles_m - first) < GM ? (tiles_m - first) : GM;
+   tm = first + (pid % width) % gsize;
+   tn = (pid % width) / gsize;
 }
 
 template <class Mma, int BK, int NSETS, int TI, int TJ, int OUT, bool B_KN, bool FULL>
@@ -112,24 +219,8 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16) ? 1 : 2) k_gemm_bytes(Gem
    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
    const int wm = wave >> 1, wn = wave & 1;
 
-   // --- workgroup id -> output tile, XCD aware -----------------------------------------
-   const int tiles = g.tiles_m * g.tiles_n;
-   int pid = blockIdx.x;
-   {
-      const int xcd = pid & 7, local = pid >> 3;
-      const int base = tiles >> 3, rem = tiles & 7;
-      pid = local + xcd * base + (xcd < rem ? xcd : rem);
-   }
    int tm, tn;
-   {
-      constexpr int GM = 4;
-      const int width = GM * g.tiles_n;
-      const int group = pid / width;
-      const int first = group * GM;
-      const int gsize = (g.tiles_m - first) < GM ? (g.tiles_m - first) : GM;
-      tm = first + (pid % width) % gsize;
-      tn = (pid % width) / gsize;
-   }
+   tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
 
    // --- global -> register staging -----------------------------------------------------
@@ -341,72 +432,235 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16) ? 1 : 2) k_gemm_bytes(Gem
    if (kt < nk) kstep(0, G[1 % NSETS], klast, false);
    __syncthreads();
 
-   // --- epilogue: pack -> per-wavefront LDS staging -> 16-byte row segments -------------
-   constexpr int WN = TI * 32;                       // output columns of one wavefront
-   constexpr int SROW = WN * ESZ + 16;               // staging row stride in bytes
-   constexpr int CR = WN * ESZ / 16;                 // 16-byte chunks per staging row
-   unsigned char *stg = smem + wave * (32 * SROW);
-   float *s_scale = reinterpret_cast<float *>(smem + 4 * 32 * SROW);   // [BN] per-column scale
-   int *s_bias = reinterpret_cast<int *>(s_scale + BN);                // [BN] per-column bias bits
-   if (tid < BN) {
-      const int n = n0 + tid;
-      s_scale[tid] = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
-      s_bias[tid] = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
+   tile_epilogue<Mma, TI, TJ, OUT, 4>(g, acc, smem, tid, m0 + wm * (TJ * 32), n0, wn, BN);
+}
+
+// ---------------------------------------------------------------------------------------
+// k_gemm_dma: both operands K-contiguous (A [M,K], B^T [N,K]).
+//
+// 512 threads = 8 wavefronts, two per SIMD, on a 256x256 output tile; a wavefront owns
+// 128 columns x 64 rows (4x2 MFMA tiles of 32x32). The operand tiles of a K-step (64 bytes
+// of K) travel HBM/L2 -> LDS with buffer_load_dwordx4 ... lds: no registers and no
+// ds_write are spent on staging, and NST LDS stages keep NST-1 K-steps of requests in
+// flight. A 1 KB load block holds 16 rows x 64 bytes; the 16-byte chunk c of row r sits in
+// slot c ^ ((r >> 2) & 3), which makes the 16-byte-per-lane MFMA operand reads of 16
+// consecutive rows hit 16 distinct bank groups without any padding (the DMA writes LDS
+// linearly, so the permutation is applied to the global address of each lane instead).
+// Out-of-range rows come back as zeros through the buffer descriptor's size check.
+// The LDS-DMA instructions are issued from inline assembly so that their completion is
+// waited for explicitly (s_waitcnt vmcnt) one stage at a time.
+#ifndef SOFIE_DMA_BK
+#define SOFIE_DMA_BK 128   // bytes of K per LDS stage of k_gemm_dma
+#define SOFIE_DMA_NST 2    // LDS stages
+#endif
+typedef int rsrc_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, unsigned bytes)
+{
+   // every component is wave-uniform; readfirstlane tells the compiler so (SGPR operands)
+   const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+   rsrc_t r = {__builtin_amdgcn_readfirstlane((int)(unsigned)a),
+               __builtin_amdgcn_readfirstlane((int)(unsigned)((a >> 32) & 0xffffu)),
+               __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+   return r;
+}
+
+// 16 bytes per lane from global (descriptor + per-lane offset + uniform offset) to
+// LDS address lds_base + lane*16.
+__device__ __forceinline__ void dma16(rsrc_t rs, unsigned lds_base, int voff, int soff)
+{
+   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                :
+                : "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "v"(voff), "s"(rs),
+                  "s"(__builtin_amdgcn_readfirstlane(soff))
+                : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+   // s_waitcnt with only the vector-memory counter constrained
+   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <class Mma, int BK, int NST, int OUT>
+__global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
+{
+   constexpr int BM = 256, BN = 256;
+   constexpr int TI = 4, TJ = 2;                      // wavefront tile: 128 n x 64 m
+   constexpr int STAGE = (BM + BN) * BK;              // A rows, then B^T rows
+   constexpr int DIST = NST - 1;                      // K-steps of requests in flight
+   constexpr int NSUB = BK / Mma::KB;
+   constexpr int CPR = BK / 16;                       // 16-byte chunks per row
+   constexpr int RPB = 1024 / BK;                     // rows per 1 KB load block
+   constexpr int SWS = BK == 64 ? 2 : 1;              // swizzle: chunk ^ ((row >> SWS) & (CPR-1))
+   static_assert(BK == 64 || BK == 128, "stage depth");
+   extern __shared__ __align__(16) unsigned char smem[];
+   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
+
+   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int wn = wave & 1, wm = wave >> 1;
+   int tm, tn;
+   tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+   const int m0 = tm * BM, n0 = tn * BN;
+
+   // --- loads: wavefronts 0-3 request the A tile, 4-7 the B^T tile -------------------------
+   constexpr int LPW = (BM + BN) / RPB / 8;           // load blocks per wavefront and stage
+   const bool uses_a = wave < 4;
+   const int ld = uses_a ? g.lda : g.ldb;
+   const int rows_total = uses_a ? g.M : g.N;
+   const int row0 = uses_a ? m0 : n0;
+   const int rows_left = (rows_total - row0) < 256 ? (rows_total - row0) : 256;
+   const unsigned char *tile_base = (uses_a ? g.A : g.B) + (size_t)row0 * ld;
+   const rsrc_t rs = make_rsrc(tile_base, (unsigned)((size_t)(rows_left - 1) * ld + g.K));
+   const int blk0 = wave * LPW;                        // first load block of this wavefront
+   const int lrow = lane / CPR;                        // row inside a block
+   // K-chunk this lane fetches in load block i: slot ^ swizzle(row); for BK = 128 the row
+   // bits that enter the swizzle include the parity of the block
+   int chunk[2], voff[2];
+#pragma unroll
+   for (int par = 0; par < 2; ++par) {
+      const int row_in_tile = par * RPB + lrow;        // low bits only matter
+      chunk[par] = (lane % CPR) ^ ((row_in_tile >> SWS) & (CPR - 1));
+      voff[par] = (((blk0 * RPB) & 255) + lrow) * ld + chunk[par] * 16;
    }
+   const bool ktail = (g.K % BK) != 0;
+   const int nk = (g.K + BK - 1) / BK;
+   auto request = [&](int t) {
+      // tile of K-step t -> stage t % NST; steps past the end repeat the last tile into a
+      // stage nobody reads any more, so the number of loads in flight never changes
+      const int tt = t < nk ? t : nk - 1;
+      const int k0 = tt * BK;
+      int vo[2] = {voff[0], voff[1]};
+      if (ktail) {
+#pragma unroll
+         for (int par = 0; par < 2; ++par)
+            if (k0 + chunk[par] * 16 >= g.K) vo[par] = 0x7ffffff0;   // beyond the descriptor: zeros
+      }
+      const unsigned dst = lds0 + (t % NST) * STAGE + blk0 * 1024;
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) dma16(rs, dst + i * 1024, vo[(BK == 128) ? (i & 1) : 0], i * RPB * ld + k0);
+   };
+   // --- MFMA operand addresses ---------------------------------------------------------
+   const int fr = lane & 31, half = lane >> 5;
+   const int sw = (fr >> SWS) & (CPR - 1);
+   // byte offset of this lane's first chunk inside a stage; later chunks differ by XOR
+   // The order in which K is consumed is free as long as both operands agree, so the lower
+   // and upper half of the wavefront always read chunks that differ in bit 1 (slot ^ 2):
+   // with the row swizzle this keeps the two halves of one ds_read_b128 off each other's banks.
+   const int first_chunk = half * 2;
+   const int n_off = BM * BK + (wn * 128 + fr) * BK + ((first_chunk ^ sw) * 16);
+   const int m_off = (wm * 64 + fr) * BK + ((first_chunk ^ sw) * 16);
+   auto load_frag = [&](const unsigned char *stage, int off, int sub) -> typename Mma::Frag {
+      if constexpr (Mma::LANE_BYTES == 16) {      // chunk = (sub/2)*4 + half*2 + sub%2
+         return *reinterpret_cast<const v4i *>(stage + (off ^ ((sub & 1) * 16) ^ ((sub >> 1) * 64)));
+      } else {                                    // chunks sub*4 + half*2 + {0,1}
+         const v4i lo = *reinterpret_cast<const v4i *>(stage + (off ^ (sub * 64)));
+         const v4i hi = *reinterpret_cast<const v4i *>(stage + (off ^ (sub * 64) ^ 16));
+         typename Mma::Frag f = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+         return f;
+      }
+   };
+
+   typename Mma::Acc acc[TI][TJ];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+#pragma unroll
+         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+   // --- ping-pong schedule -----------------------------------------------------------------
+   // The two wavefronts of a SIMD run half a K-step apart: while one multiplies (MFMAs only,
+   // operands already in registers) the other issues the LDS-DMA requests and reads its next
+   // operands from LDS; a workgroup barrier ends every phase. Group 1 gets its phase shift
+   // from one extra barrier at the start, group 0 pays it back after its last multiply.
+   const int group = wave >> 2;
+   auto barrier = [&]() {
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+   };
+   if (nk > 0) {
+#pragma unroll
+      for (int t = 0; t < DIST; ++t) request(t);
+      wait_vmcnt<LPW *(DIST - 1)>();     // this wavefront's part of stage 0 has landed
+   }
+   barrier();
+   if (group == 1) barrier();
+   for (int t = 0; t < nk; ++t) {
+      // load phase: requests for stage t+DIST (its buffer was last read one phase ago), then
+      // every operand fragment of stage t into registers
+      request(t + DIST);
+      const unsigned char *stage = smem + (t % NST) * STAGE;
+      typename Mma::Frag fn[NSUB][TI], fm[NSUB][TJ];
+#pragma unroll
+      for (int sub = 0; sub < NSUB; ++sub) {
+#pragma unroll
+         for (int i = 0; i < TI; ++i) fn[sub][i] = load_frag(stage, n_off + i * 32 * BK, sub);
+#pragma unroll
+         for (int j = 0; j < TJ; ++j) fm[sub][j] = load_frag(stage, m_off + j * 32 * BK, sub);
+      }
+      __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): fragments are in registers
+      // Stage t+1 is first read by group 0 right after the barrier that ends its multiply
+      // phase, which is the barrier that ends group 1's load phase: each group waits for its
+      // own part of stage t+1 just before that barrier.
+      if (group == 1) wait_vmcnt<LPW *(DIST - 1)>();
+      barrier();
+      // multiply phase
+#pragma unroll
+      for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+         for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) acc[i][j] = Mma::mma(fn[sub][i], fm[sub][j], acc[i][j]);
+      if (group == 0) wait_vmcnt<LPW *(DIST - 1)>();
+      if (group == 0 || t + 1 < nk) barrier();
+   }
+   wait_vmcnt<0>();                         // the trailing dummy requests still target LDS
    __syncthreads();
-   const int m_local = lane & 31;
-   const int nq = (lane >> 5) * 4;
+   tile_epilogue<Mma, TI, TJ, OUT, 8>(g, acc, smem, tid, m0 + wm * 64, n0, wn, BN);
+}
+
+// Byte-matrix transpose src [R, C] (ld_src) -> dst [C, R] (ld_dst), R % 16 == 0, C % 4 == 0.
+// A thread takes 16 rows x 4 columns (16 dwords), transposes them in registers with
+// v_perm_b32 and writes four 16-byte row segments; eight neighbouring lanes write 128
+// contiguous bytes of one output row. HBM-bound: R*C bytes in, R*C bytes out.
+__global__ void __launch_bounds__(256) k_transpose_bytes(const unsigned char *__restrict__ src, unsigned char *__restrict__ dst,
+                                                         int R, int C, int ld_src, int ld_dst)
+{
+   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+   const int rg = blockIdx.x * 8 + (lane & 7);                 // 16-row group
+   const int cg = (blockIdx.y * 4 + wave) * 8 + (lane >> 3);   // 4-column group
+   if (rg * 16 >= R || cg * 4 >= C) return;
+   const unsigned char *p = src + (size_t)rg * 16 * ld_src + cg * 4;
+   unsigned d[16];
 #pragma unroll
-   for (int j = 0; j < TJ; ++j) {
+   for (int r = 0; r < 16; ++r) d[r] = *reinterpret_cast<const unsigned *>(p + (size_t)r * ld_src);
+   unsigned o[4][4];
 #pragma unroll
-      for (int i = 0; i < TI; ++i) {
-#pragma unroll
-         for (int q = 0; q < 4; ++q) {
-            const int nl = i * 32 + q * 8 + nq;
-            unsigned e[4];
-            const v4f sc = *reinterpret_cast<const v4f *>(s_scale + wn * WN + nl);
-            const v4i bi = *reinterpret_cast<const v4i *>(s_bias + wn * WN + nl);
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-               if constexpr (IS_INT)
-                  e[t] = epilogue_value<true, OUT>(g, sc[t], bi[t], acc[i][j][q * 4 + t], 0.0f);
-               else
-                  e[t] = epilogue_value<false, OUT>(g, sc[t], bi[t], 0, acc[i][j][q * 4 + t]);
-            }
-            unsigned char *dst = stg + m_local * SROW + nl * ESZ;
-            if constexpr (ESZ == 1) {
-               *reinterpret_cast<unsigned *>(dst) = e[0] | (e[1] << 8) | (e[2] << 16) | (e[3] << 24);
-            } else if constexpr (ESZ == 2) {
-               v2i p = {(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16))};
-               *reinterpret_cast<v2i *>(dst) = p;
-            } else {
-               v4i p = {(int)e[0], (int)e[1], (int)e[2], (int)e[3]};
-               *reinterpret_cast<v4i *>(dst) = p;
-            }
-         }
-      }
-      __syncthreads();
-      constexpr int ITERS = 32 * CR / 64;
-#pragma unroll
-      for (int it = 0; it < ITERS; ++it) {
-         const int c = it * 64 + lane;
-         const int row = c / CR, cc = c % CR;
-         const int m = m0 + wm * (TJ * 32) + j * 32 + row;
-         const int nfirst = n0 + wn * WN + cc * (16 / ESZ);
-         if (m < g.M && nfirst < g.N) {
-            const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
-            unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
-            if (g.vec_store && nfirst + 16 / ESZ <= g.N) {
-               *reinterpret_cast<v4i *>(out) = v;
-            } else {
-               const unsigned char *src = stg + row * SROW + cc * 16;
-               const int cnt = (g.N - nfirst) < (16 / ESZ) ? (g.N - nfirst) : (16 / ESZ);
-               for (int b = 0; b < cnt * ESZ; ++b) out[b] = src[b];
-            }
-         }
-      }
-      __syncthreads();
+   for (int q = 0; q < 4; ++q) {
+      const unsigned t0 = __builtin_amdgcn_perm(d[4 * q + 1], d[4 * q + 0], 0x05010400u);
+      const unsigned t1 = __builtin_amdgcn_perm(d[4 * q + 1], d[4 * q + 0], 0x07030602u);
+      const unsigned t2 = __builtin_amdgcn_perm(d[4 * q + 3], d[4 * q + 2], 0x05010400u);
+      const unsigned t3 = __builtin_amdgcn_perm(d[4 * q + 3], d[4 * q + 2], 0x07030602u);
+      o[0][q] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+      o[1][q] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+      o[2][q] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+      o[3][q] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
    }
+#pragma unroll
+   for (int j = 0; j < 4; ++j) {
+      const v4i v = {(int)o[j][0], (int)o[j][1], (int)o[j][2], (int)o[j][3]};
+      *reinterpret_cast<v4i *>(dst + (size_t)(cg * 4 + j) * ld_dst + rg * 16) = v;
+   }
+}
+
+int transpose_bytes(sofie_hip_ctx *ctx, const unsigned char *src, unsigned char *dst, int R, int C, int ld_src, int ld_dst)
+{
+   hipLaunchKernelGGL(k_transpose_bytes, dim3(cdiv(R, 128), cdiv(C, 128)), dim3(256), 0, ctx->stream, src, dst, R, C,
+                      ld_src, ld_dst);
+   return check_launch(ctx, "k_transpose_bytes");
 }
 
 // Any shape, any alignment: one thread per output element. Correctness path for operands
@@ -436,7 +690,7 @@ __global__ void k_gemm_bytes_simple(GemmArgs g, int transB)
       }
       r = epilogue_value<false, OUT>(g, 0.0f, g.bias ? static_cast<const int *>(g.bias)[n] : 0, 0, acc);
    }
-   if constexpr (ESZ == 1) *out = (unsigned char)r;
+   if constexpr (ESZ == 1) *out = (unsigned char)((int)fminf(__uint_as_float(r), 255.0f) - 128);
    else if constexpr (ESZ == 2) *reinterpret_cast<unsigned short *>(out) = (unsigned short)r;
    else *reinterpret_cast<unsigned *>(out) = r;
 }
@@ -468,6 +722,22 @@ int launch_tiled(sofie_hip_ctx *ctx, GemmArgs &g)
    return launch_tiled_impl<Mma, BK, NSETS, TI, TJ, OUT, B_KN, false>(ctx, g);
 }
 
+template <class Mma, int BK, int NST, int OUT>
+int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
+{
+   constexpr size_t stage_bytes = (size_t)NST * 512 * BK;
+   constexpr size_t epi_bytes = (size_t)8 * 32 * (128 * OutSize<OUT>::value + 16) + (size_t)2 * 256 * 4;
+   constexpr size_t lds = stage_bytes > epi_bytes ? stage_bytes : epi_bytes;
+   static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
+   g.tiles_m = cdiv(g.M, 256);
+   g.tiles_n = cdiv(g.N, 256);
+   auto kern = k_gemm_dma<Mma, BK, NST, OUT>;
+   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+   hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(512), lds, ctx->stream, g);
+   return check_launch(ctx, "k_gemm_dma");
+}
+
 template <bool IS_INT, int OUT>
 int launch_simple(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
 {
@@ -493,8 +763,21 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
    constexpr int BK = 128;
    constexpr int NSETS = IS_INT ? 2 : 1;
    if (transB) {
+      // descriptor offsets are 32-bit: a 256-row panel plus K must stay below 2 GiB
+      const bool fits = (size_t)256 * g.lda + g.K < (1u << 31) && (size_t)256 * g.ldb + g.K < (1u << 31);
+      if (big && fits) return launch_dma<Mma, SOFIE_DMA_BK, SOFIE_DMA_NST, OUT>(ctx, g);
       if (big) return launch_tiled<Mma, BK, NSETS, 4, 4, OUT, false>(ctx, g);
       return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, false>(ctx, g);
+   }
+   if (big && g.K % 16 == 0 && (size_t)256 * g.lda + g.K < (1u << 31) && (size_t)257 * g.K < (1u << 31)) {
+      // B [K,N] -> B^T [N,K] in the context's scratch buffer, then the K-contiguous kernel.
+      // A caller that reuses B (weights) should transpose once and call with transB = 1.
+      void *bt = nullptr;
+      if (int rc = workspace(ctx, (size_t)g.N * g.K, &bt)) return rc;
+      if (int rc = transpose_bytes(ctx, g.B, static_cast<unsigned char *>(bt), g.K, g.N, g.ldb, g.K)) return rc;
+      g.B = static_cast<const uint8_t *>(bt);
+      g.ldb = g.K;
+      return launch_dma<Mma, SOFIE_DMA_BK, SOFIE_DMA_NST, OUT>(ctx, g);
    }
    if (big) return launch_tiled<Mma, BK, NSETS, 4, 4, OUT, true>(ctx, g);
    return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, true>(ctx, g);
@@ -534,6 +817,21 @@ int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, cons
    case SOFIE_OUT_F32: return dispatch<MmaI8, SOFIE_OUT_F32>(ctx, g, transB);
    default: return dispatch<MmaI8, SOFIE_OUT_S32>(ctx, g, transB);
    }
+}
+
+int sofie_hip_transpose_bytes(sofie_hip_ctx *ctx, const void *src, void *dst, int rows, int cols, int ld_src,
+                               int ld_dst)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, rows >= 0 && cols >= 0, "negative dimension");
+   if (rows == 0 || cols == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, src && dst && src != dst, "null or aliased operand");
+   SOFIE_REQUIRE(ctx, ld_src >= cols && ld_dst >= rows, "leading dimension too small");
+   SOFIE_REQUIRE(ctx, rows % 16 == 0 && cols % 4 == 0 && ld_src % 4 == 0 && ld_dst % 16 == 0 &&
+                         (reinterpret_cast<uintptr_t>(src) & 3u) == 0 && aligned16(dst),
+                 "needs rows % 16 == 0, cols % 4 == 0 and matching alignment");
+   return transpose_bytes(ctx, static_cast<const unsigned char *>(src), static_cast<unsigned char *>(dst), rows, cols,
+                          ld_src, ld_dst);
 }
 
 int sofie_hip_gemm_fp8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const uint8_t *A, int lda,
