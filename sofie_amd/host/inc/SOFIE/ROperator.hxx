@@ -1,0 +1,57 @@
+// Emitter interface: one ROperator per graph node. Same virtuals, call order and naming as
+// the reference's src/SOFIE_core/inc/SOFIE/ROperator.hxx:17-57; RModel calls
+// Initialize(model) once, then GenerateSessionMembersCode / GenerateInitCode while it writes
+// the Session, then Generate(opName) inside infer. The extra hooks at the bottom exist for
+// the device emission only (activation fusion, view outputs, constructor-time weight work).
+#ifndef SOFIE_ROPERATOR
+#define SOFIE_ROPERATOR
+
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "SOFIE/SOFIE_common.hxx"
+
+namespace SOFIE {
+
+class RModel;
+
+class ROperator {
+public:
+   virtual std::vector<std::string> GetBlasRoutines() { return {}; }
+   virtual std::vector<std::string> GetStdLibs() { return {}; }
+   virtual std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>>) = 0;
+   virtual std::vector<ETensorType> TypeInference(std::vector<ETensorType>) = 0;
+   virtual void Initialize(RModel &) = 0;
+   virtual std::string Generate(std::string OpName) = 0;   // expects a unique OpName per operator
+   virtual std::string GenerateInitCode() { return ""; }
+   virtual std::string GenerateDeclCode() { return ""; }
+   virtual std::string GenerateSessionMembersCode(std::string /*opName*/) { return ""; }
+   virtual std::string Header() { return ""; }
+   virtual ~ROperator() {}
+
+   // --- device-emission hooks ------------------------------------------------------------
+   // operator family name ("Gemm", "Conv", "Relu", ...), used by RModel's fusion pass
+   virtual std::string Kind() const { return ""; }
+   // try to absorb a following activation into this operator's epilogue
+   virtual bool FuseActivation(EActivationType) { return false; }
+   // the output is a view of this input tensor (no kernel, no memory): "" if not a view
+   virtual std::string ViewOf() const { return ""; }
+   // when fused away, the operator emits nothing and its output aliases its input
+   void SetFusedAway() { fFusedAway = true; }
+   bool IsFusedAway() const { return fFusedAway; }
+
+   const std::vector<std::string> &GetOpInputTensors() const { return fInputTensorNames; }
+   const std::vector<std::string> &GetOpOutputTensors() const { return fOutputTensorNames; }
+
+protected:
+   const std::string SP = "   ";   // indentation of generated code
+   bool fUseSession = false;
+   bool fIsOutputConstant = false;
+   bool fFusedAway = false;
+   std::vector<std::string> fInputTensorNames;    // every tensor the emitted code reads
+   std::vector<std::string> fOutputTensorNames;   // tensors the emitted code writes
+};
+
+}   // namespace SOFIE
+#endif

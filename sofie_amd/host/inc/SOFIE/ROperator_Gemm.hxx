@@ -1,0 +1,153 @@
+// Gemm / MatMul(+Add) / Gemm+ReLU emitter. Constructor signatures, attribute meaning, bias rules and
+// error messages follow the reference's ROperator_Gemm<T> (src/SOFIE_core/inc/SOFIE/
+// ROperator_Gemm.hxx:47-67,139-269,292-390); what is emitted is one call of sofie_hip_gemm_f32
+// with the bias broadcast and the activation fused in the kernel epilogue, instead of
+// std::copy(bias) + BLAS::sgemm_ + a scalar ReLU loop.
+#ifndef SOFIE_ROPERATOR_GEMM
+#define SOFIE_ROPERATOR_GEMM
+
+#include <iomanip>
+#include <limits>
+#include <sstream>
+
+#include "SOFIE/RModel.hxx"
+#include "SOFIE/ROperator.hxx"
+
+namespace SOFIE {
+
+inline std::string FloatLiteral(float v)
+{
+   std::stringstream s;
+   s << "static_cast<float>(" << std::setprecision(std::numeric_limits<float>::max_digits10) << v << ")";
+   return s.str();
+}
+
+template <typename T>
+class ROperator_Gemm final : public ROperator {
+private:
+   float fAttrAlpha = 1.0;
+   float fAttrBeta = 1.0;
+   int_t fAttrTransA = 0;
+   int_t fAttrTransB = 0;
+   std::string fNA, fNB, fNC = "", fNY;
+   EActivationType fActivation = EActivationType::UNDEFINED;
+   std::vector<size_t> fShapeA, fShapeB, fShapeC, fShapeY;
+   int fBiasKind = 0;   // SOFIE_BIAS_*
+
+public:
+   ROperator_Gemm() {}
+   ROperator_Gemm(float alpha, float beta, int_t transA, int_t transB, std::string nameA, std::string nameB,
+                  std::string nameY, EActivationType activation = EActivationType::UNDEFINED)
+      : fAttrAlpha(alpha), fAttrBeta(beta), fAttrTransA(transA), fAttrTransB(transB), fNA(UTILITY::Clean_name(nameA)),
+        fNB(UTILITY::Clean_name(nameB)), fNY(UTILITY::Clean_name(nameY)), fActivation(activation)
+   {
+      static_assert(std::is_same<T, float>::value, "TMVA::SOFIE - Unsupported type parsing a Gemm operator");
+      fInputTensorNames = {fNA, fNB};
+      fOutputTensorNames = {fNY};
+   }
+   ROperator_Gemm(float alpha, float beta, int_t transA, int_t transB, std::string nameA, std::string nameB,
+                  std::string nameC, std::string nameY, EActivationType activation = EActivationType::UNDEFINED)
+      : fAttrAlpha(alpha), fAttrBeta(beta), fAttrTransA(transA), fAttrTransB(transB), fNA(UTILITY::Clean_name(nameA)),
+        fNB(UTILITY::Clean_name(nameB)), fNC(UTILITY::Clean_name(nameC)), fNY(UTILITY::Clean_name(nameY)),
+        fActivation(activation)
+   {
+      static_assert(std::is_same<T, float>::value, "TMVA::SOFIE - Unsupported type parsing a Gemm operator");
+      fInputTensorNames = {fNA, fNB, fNC};
+      fOutputTensorNames = {fNY};
+   }
+
+   std::string Kind() const override { return "Gemm"; }
+   bool FuseActivation(EActivationType act) override
+   {
+      if (act != EActivationType::RELU || fActivation != EActivationType::UNDEFINED) return false;
+      fActivation = act;
+      return true;
+   }
+
+   std::vector<ETensorType> TypeInference(std::vector<ETensorType> input) override { return {input[0]}; }
+
+   std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>> input) override
+   {
+      if (input.size() > 3) throw std::runtime_error("TMVA SOFIE Gemm Op Shape Inference only need 2 or 3 input tensor");
+      for (auto &i : input)
+         if (i.size() < 2)
+            throw std::runtime_error("TMVA SOFIE Gemm Op Shape Inference only accept input tensor with >=2 dimensions");
+      if (input.size() == 3) return {input[2]};   // with three inputs the shape of Y is the shape of C
+      std::vector<size_t> a = input[0], b = input[1];
+      if (fAttrTransA) std::reverse(a.begin(), a.end());
+      if (fAttrTransB) std::reverse(b.begin(), b.end());
+      return {{a[0], b[1]}};
+   }
+
+   void Initialize(RModel &model) override
+   {
+      if (!model.CheckIfTensorAlreadyExist(fNA) || !model.CheckIfTensorAlreadyExist(fNB))
+         throw std::runtime_error("TMVA SOFIE Gemm Op Input Tensor " + fNA + " or " + fNB + " is not found in model");
+      if (fNC != "" && !model.CheckIfTensorAlreadyExist(fNC))
+         throw std::runtime_error("TMVA SOFIE Gemm Op Input Tensor" + fNC + " is not found in model");
+      fShapeA = model.GetTensorShape(fNA);
+      fShapeB = model.GetTensorShape(fNB);
+      // a rank-1 A gets a leading 1, a rank-1 B a trailing 1, removed again from Y (reference :158-177)
+      bool prependOne = false, appendOne = false;
+      if (fShapeA.size() == 1) { fShapeA.insert(fShapeA.begin(), 1); prependOne = true; }
+      if (fShapeB.size() == 1) { fShapeB.push_back(1); appendOne = true; }
+      if (fShapeA.size() != 2 || fShapeB.size() != 2)
+         throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + ": stacked (rank > 2) MatMul is not supported by the device emission");
+      std::vector<size_t> a = fShapeA, b = fShapeB;
+      if (fAttrTransA) std::reverse(a.begin(), a.end());
+      if (fAttrTransB) std::reverse(b.begin(), b.end());
+      if (a[1] != b[0])
+         throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + " has invalid shape" + ConvertShapeToString(fShapeA) + " x " +
+                                  ConvertShapeToString(fShapeB));
+      fShapeY = {a[0], b[1]};
+      if (model.GetTensorType(fNA) != ETensorType::FLOAT || model.GetTensorType(fNB) != ETensorType::FLOAT)
+         throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + ": only float tensors are supported");
+      if (fNC != "") {
+         fShapeC = model.GetTensorShape(fNC);
+         const size_t lenC = ConvertShapeToLength(fShapeC), M = fShapeY[0], N = fShapeY[1];
+         // unidirectional broadcast of C to [M,N] happens inside the kernel epilogue; the reference
+         // materialises the broadcast tensor in the Session constructor (:271-290)
+         if (lenC == M * N && (fShapeC.size() < 2 || fShapeC.back() == N)) fBiasKind = 2;      // full
+         else if (lenC == N && fShapeC.back() == N) fBiasKind = 1;                              // one row
+         else if (lenC == M && fShapeC.size() == 2 && fShapeC[1] == 1) fBiasKind = 3;           // one column
+         else if (lenC == 1 && model.IsInitializedTensor(fNC)) {
+            // scalar: expanded to one row at generation time
+            float v = static_cast<float *>(model.GetInitializedTensorData(fNC).get())[0];
+            std::shared_ptr<void> row(malloc(N * sizeof(float)), free);
+            std::fill_n(static_cast<float *>(row.get()), N, v);
+            model.UpdateInitializedTensor(fNC, ETensorType::FLOAT, {N}, row);
+            fShapeC = {N};
+            fBiasKind = 1;
+         } else
+            throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + " Bias tensor has not correct size " +
+                                     ConvertShapeToString(fShapeC) + " output shape " + ConvertShapeToString(fShapeY));
+      }
+      std::vector<size_t> shapeY = fShapeY;
+      if (prependOne) shapeY.erase(shapeY.begin());
+      if (appendOne) shapeY.pop_back();
+      model.AddIntermediateTensor(fNY, model.GetTensorType(fNA), shapeY);
+      model.AddNeededStdLib("algorithm");
+   }
+
+   std::string Generate(std::string opName) override
+   {
+      opName = "op_" + opName;
+      if (fShapeA.empty() || fShapeB.empty() || fShapeY.empty() || (fNC != "" && fShapeC.empty()))
+         throw std::runtime_error("TMVA SOFIE Gemm Op called to Generate without being initialized first");
+      if (fNC.empty() && fAttrBeta != 0)
+         throw std::runtime_error("TMVA SOFIE Gemm Op " + opName + " Bias tensor is not present but beta value in Gemm is not zero");
+      const size_t m = fShapeY[0], n = fShapeY[1];
+      const size_t k = fAttrTransA ? fShapeA[0] : fShapeA[1];
+      std::stringstream out;
+      out << "\n//--------- Gemm\n";
+      out << SP << "Check(sofie_hip_gemm_f32(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << m << ", "
+          << n << ", " << k << ", " << FloatLiteral(fAttrAlpha) << ", tensor_" << fNA << ", " << fShapeA[1] << ", tensor_" << fNB
+          << ", " << fShapeB[1] << ", " << FloatLiteral(fNC.empty() ? 0.0f : fAttrBeta) << ", "
+          << (fNC.empty() ? std::string("nullptr") : "tensor_" + fNC) << ", " << fBiasKind << ", tensor_" << fNY << ", " << n << ", "
+          << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << "), \"Gemm " << opName << "\");\n";
+      return out.str();
+   }
+};
+
+}   // namespace SOFIE
+#endif

@@ -1,0 +1,99 @@
+// Pooling emitter; interface of the reference's ROperator_Pool<T> (ROperator_Pool.hxx:17-90): a mode,
+// an attribute struct, input and output names. The device emission covers 2-D MaxPool (float NCHW and
+// int8 NCHW), with the reference's output-size rule (floor division, default pads 0, :92-199).
+#ifndef SOFIE_ROPERATOR_POOL
+#define SOFIE_ROPERATOR_POOL
+
+#include <sstream>
+
+#include "SOFIE/RModel.hxx"
+#include "SOFIE/ROperator.hxx"
+
+namespace SOFIE {
+
+struct RAttributes_Pool {
+   std::string auto_pad = "NOTSET";
+   int ceil_mode = 0;
+   int count_include_pad = 0;
+   int storage_order = 0;
+   std::vector<size_t> dilations;
+   std::vector<size_t> kernel_shape;
+   std::vector<size_t> pads;
+   std::vector<size_t> strides;
+};
+
+enum PoolOpMode { InvalidPool, MaxPool, AveragePool, GlobalAveragePool };
+
+template <typename T>
+class ROperator_Pool final : public ROperator {
+private:
+   PoolOpMode fPoolMode;
+   RAttributes_Pool fAttr;
+   std::string fNX, fNY;
+   std::vector<size_t> fShapeX, fShapeY;
+   ETensorType fType = ETensorType::UNDEFINED;
+
+public:
+   ROperator_Pool() {}
+   ROperator_Pool(PoolOpMode mode, RAttributes_Pool attr, std::string nameX, std::string nameY)
+      : fPoolMode(mode), fAttr(attr), fNX(UTILITY::Clean_name(nameX)), fNY(UTILITY::Clean_name(nameY))
+   {
+      fInputTensorNames = {fNX};
+      fOutputTensorNames = {fNY};
+   }
+   std::string Kind() const override { return "Pool"; }
+   std::string Name() { return fPoolMode == MaxPool ? "MaxPool" : fPoolMode == AveragePool ? "AveragePool" : "Invalid"; }
+   std::vector<ETensorType> TypeInference(std::vector<ETensorType> input) override { return input; }
+   std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>> input) override
+   {
+      if (input.size() != 1) throw std::runtime_error("TMVA SOFIE" + Name() + "Op Shape inference need 1 input tensor");
+      if (input[0].size() != 4)
+         throw std::runtime_error("TMVA SOFIE" + Name() + "Op : tensors with dimension " + std::to_string(input[0].size()) +
+                                  " are not yet supported");
+      if (fAttr.kernel_shape.empty()) fAttr.kernel_shape = {input[0][2], input[0][3]};
+      if (fAttr.auto_pad != "NOTSET")
+         throw std::runtime_error("TMVA SOFIE" + Name() + "Op : auto_pad is not supported by the device emission");
+      if (fAttr.pads.empty()) fAttr.pads = {0, 0, 0, 0};
+      fAttr.pads.resize(4, 0);
+      if (fAttr.strides.empty()) fAttr.strides = {1, 1};
+      for (auto d : fAttr.dilations)
+         if (d != 1) throw std::runtime_error("TMVA SOFIE" + Name() + "Op : dilations are not supported by the device emission");
+      const size_t oh = (input[0][2] + fAttr.pads[0] + fAttr.pads[2] - fAttr.kernel_shape[0]) / fAttr.strides[0] + 1;
+      const size_t ow = (input[0][3] + fAttr.pads[1] + fAttr.pads[3] - fAttr.kernel_shape[1]) / fAttr.strides[1] + 1;
+      return {{input[0][0], input[0][1], oh, ow}};
+   }
+   void Initialize(RModel &model) override
+   {
+      if (!model.CheckIfTensorAlreadyExist(fNX))
+         throw std::runtime_error("TMVA SOFIE Pool op Input Tensor " + fNX + " is not found in model");
+      if (fPoolMode != MaxPool)
+         throw std::runtime_error("TMVA SOFIE Pool op " + Name() + " is not supported by the device emission");
+      fShapeX = model.GetTensorShape(fNX);
+      fType = model.GetTensorType(fNX);
+      if (fType != ETensorType::FLOAT && fType != ETensorType::INT8)
+         throw std::runtime_error("TMVA SOFIE Encountered unsupported type parsing a Pool operator");
+      fShapeY = ShapeInference({fShapeX})[0];
+      model.AddIntermediateTensor(fNY, fType, fShapeY);
+   }
+   std::string Generate(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShapeX.empty() || fShapeY.empty())
+         throw std::runtime_error("TMVA SOFIE Pool Op called to Generate without being initialized first");
+      std::stringstream out;
+      out << "\n//----  operator " << Name() << "  " << OpName << "\n";
+      const auto &a = fAttr;
+      if (fType == ETensorType::FLOAT)
+         out << SP << "Check(sofie_hip_maxpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << fShapeX[0] * fShapeX[1]
+             << ", " << fShapeX[2] << ", " << fShapeX[3];
+      else
+         out << SP << "Check(sofie_hip_maxpool2d_s8(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", SOFIE_LAYOUT_NCHW, "
+             << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3];
+      out << ", " << a.kernel_shape[0] << ", " << a.kernel_shape[1] << ", " << a.pads[0] << ", " << a.pads[1] << ", " << a.pads[2]
+          << ", " << a.pads[3] << ", " << a.strides[0] << ", " << a.strides[1] << "), \"" << Name() << " " << OpName << "\");\n";
+      return out.str();
+   }
+};
+
+}   // namespace SOFIE
+#endif

@@ -1,0 +1,608 @@
+// RModel: tensor registries, operator list, memory plan and Session emission for the HIP path.
+// Structure of the generated Session follows the reference's emitter
+// (src/SOFIE_core/src/RModel.cxx:574-910): tensor members, intermediate pool with offsets,
+// constructor that reads the text weight file with name/length checks, infer() that runs every
+// operator's Generate() text and returns a std::vector copy of the output.
+#include "SOFIE/RModel.hxx"
+
+#include <cmath>
+#include <fstream>
+#include <iomanip>
+#include <iostream>
+#include <limits>
+
+namespace SOFIE {
+
+std::underlying_type_t<Options> operator|(Options opA, Options opB)
+{
+   return static_cast<std::underlying_type_t<Options>>(opA) | static_cast<std::underlying_type_t<Options>>(opB);
+}
+std::underlying_type_t<Options> operator|(std::underlying_type_t<Options> opA, Options opB)
+{
+   return opA | static_cast<std::underlying_type_t<Options>>(opB);
+}
+
+RModel::RModel(std::string name, std::string parsedtime) : fFileName(name), fParseTime(parsedtime)
+{
+   // model name = file name without directory and extension, as the reference derives it
+   fName = fFileName.substr(0, fFileName.rfind("."));
+   fName = UTILITY::Clean_name(fName.substr(fName.find_last_of("/\\") + 1));
+}
+
+const std::vector<size_t> &RModel::GetTensorShape(std::string name) const
+{
+   auto f = fReadyInputTensorInfos.find(name);
+   if (f != fReadyInputTensorInfos.end()) return f->second.shape;
+   auto f2 = fInitializedTensors.find(name);
+   if (f2 != fInitializedTensors.end()) return f2->second.shape();
+   auto f4 = fIntermediateTensorInfos.find(name);
+   if (f4 != fIntermediateTensorInfos.end()) return f4->second.shape;
+   throw std::runtime_error("TMVA SOFIE tensor [" + name + "] for which the shape is requested is not found");
+}
+
+std::vector<Dim> RModel::GetDynamicTensorShape(std::string name) const
+{
+   return ConvertShapeToDim(GetTensorShape(name));
+}
+
+const ETensorType &RModel::GetTensorType(std::string name) const
+{
+   auto f = fReadyInputTensorInfos.find(name);
+   if (f != fReadyInputTensorInfos.end()) return f->second.type;
+   auto f2 = fInitializedTensors.find(name);
+   if (f2 != fInitializedTensors.end()) return f2->second.type();
+   auto f4 = fIntermediateTensorInfos.find(name);
+   if (f4 != fIntermediateTensorInfos.end()) return f4->second.type;
+   throw std::runtime_error("TMVA SOFIE tensor [" + name + "] for which the type is requested is not found, model name: " +
+                            fName);
+}
+
+bool RModel::CheckIfTensorAlreadyExist(std::string tensor_name)
+{
+   return fReadyInputTensorInfos.count(tensor_name) || fInitializedTensors.count(tensor_name) ||
+          fIntermediateTensorInfos.count(tensor_name);
+}
+
+bool RModel::IsInitializedTensor(const std::string &name) const { return fInitializedTensors.count(name) != 0; }
+bool RModel::IsReadyInputTensor(const std::string &name) const { return fReadyInputTensorInfos.count(name) != 0; }
+
+void RModel::AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<Dim> shape)
+{
+   std::vector<size_t> s = ConvertShapeToInt(shape);
+   if (s.empty() && !shape.empty())
+      throw std::runtime_error("TMVA-SOFIE: parametric input shapes are not supported by the device emission (tensor " +
+                               input_name + ")");
+   AddInputTensorInfo(input_name, type, s);
+}
+
+void RModel::AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<size_t> shape)
+{
+   input_name = UTILITY::Clean_name(input_name);
+   if (CheckIfTensorAlreadyExist(input_name))
+      throw std::runtime_error("TMVA-SOFIE: input tensor with name " + input_name + " already exists \n");
+   fReadyInputTensorInfos[input_name] = TensorInfo{type, shape};
+}
+
+void RModel::AddInputTensorName(std::string input_name) { fInputTensorNames.emplace_back(UTILITY::Clean_name(input_name)); }
+
+void RModel::AddOperator(std::unique_ptr<ROperator> op, int order_execution)
+{
+   AddBlasRoutines(op->GetBlasRoutines());
+   for (auto &stdlib : op->GetStdLibs()) AddNeededStdLib(stdlib);
+   if (order_execution >= 0 && order_execution <= (int)fOperators.size())
+      fOperators.insert(fOperators.begin() + order_execution, std::move(op));
+   else
+      fOperators.push_back(std::move(op));
+}
+
+void RModel::AddInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape,
+                                  std::shared_ptr<void> data)
+{
+   tensor_name = UTILITY::Clean_name(tensor_name);
+   if (CheckIfTensorAlreadyExist(tensor_name))
+      throw std::runtime_error("TMVA-SOFIE: initialized tensor with name " + tensor_name + " already exists \n");
+   fInitializedTensors[tensor_name] = InitializedTensor{type, shape, data};
+}
+
+void RModel::UpdateInitializedTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape,
+                                     std::shared_ptr<void> data)
+{
+   tensor_name = UTILITY::Clean_name(tensor_name);
+   if (!fInitializedTensors.count(tensor_name))
+      throw std::runtime_error("TMVA-SOFIE: tensor " + tensor_name + " not found when trying to update it");
+   fInitializedTensors[tensor_name] = InitializedTensor{type, shape, data};
+}
+
+std::shared_ptr<void> RModel::GetInitializedTensorData(std::string tensor_name)
+{
+   auto f = fInitializedTensors.find(tensor_name);
+   if (f == fInitializedTensors.end())
+      throw std::runtime_error("TMVA-SOFIE: tensor " + tensor_name + " not found when trying to get its data");
+   return f->second.sharedptr();
+}
+
+void RModel::SetNotWritableInitializedTensor(const std::string &tensor_name)
+{
+   auto f = fInitializedTensors.find(tensor_name);
+   if (f == fInitializedTensors.end())
+      throw std::runtime_error("TMVA-SOFIE: initialized tensor " + tensor_name + " not found");
+   f->second.SetNotWritable();
+}
+
+void RModel::AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape)
+{
+   tensor_name = UTILITY::Clean_name(tensor_name);
+   if (CheckIfTensorAlreadyExist(tensor_name))
+      throw std::runtime_error("TMVA-SOFIE: intermediate tensor with name " + tensor_name + " already exists \n");
+   fIntermediateTensorInfos[tensor_name] = TensorInfo{type, shape};
+}
+
+void RModel::AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<Dim> dim_shape)
+{
+   AddIntermediateTensor(tensor_name, type, ConvertShapeToInt(dim_shape));
+}
+
+void RModel::AddOutputTensorNameList(std::vector<std::string> output_tensor_names)
+{
+   fOutputTensorNames.clear();
+   for (auto &n : output_tensor_names) fOutputTensorNames.emplace_back(UTILITY::Clean_name(n));
+}
+
+void RModel::AddBlasRoutines(std::vector<std::string> routines)
+{
+   for (auto &r : routines) fNeededBlasRoutines.insert(r);
+}
+
+void RModel::AddNeededStdLib(std::string libname)
+{
+   if (fAllowedStdLib.count(libname)) fNeededStdLib.insert(libname);
+}
+
+void RModel::Initialize(int /*batchSize*/, bool verbose)
+{
+   fVerbose = int(verbose);
+   if (fIsInitialized) return;
+   fIntermediateTensorInfos.clear();
+   // every declared input must have a shape, as in the reference (RModel.cxx:410-468)
+   for (auto &n : fInputTensorNames)
+      if (!fReadyInputTensorInfos.count(n))
+         throw std::runtime_error("TMVA-SOFIE: input tensor " + n + " has no shape information");
+   if (fInputTensorNames.empty())
+      for (auto &it : fReadyInputTensorInfos) fInputTensorNames.push_back(it.first);
+   for (auto &op : fOperators) op->Initialize(*this);
+   for (auto &n : fOutputTensorNames)
+      if (!CheckIfTensorAlreadyExist(n))
+         throw std::runtime_error("TMVA-SOFIE: output tensor " + n + " is not produced by any operator");
+   fIsInitialized = true;
+}
+
+// Conv / Gemm / QLinear* followed by a Relu that is the only consumer of their output:
+// the activation moves into the producer's epilogue and the Relu becomes a view.
+void RModel::FuseActivations()
+{
+   for (size_t i = 0; i + 1 < fOperators.size(); ++i) {
+      ROperator &prod = *fOperators[i];
+      ROperator &act = *fOperators[i + 1];
+      if (act.Kind() != "Relu" || prod.GetOpOutputTensors().empty()) continue;
+      const std::string &mid = prod.GetOpOutputTensors()[0];
+      if (act.GetOpInputTensors().empty() || act.GetOpInputTensors()[0] != mid) continue;
+      bool other_use = std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), mid) != fOutputTensorNames.end();
+      for (size_t j = 0; j < fOperators.size() && !other_use; ++j) {
+         if (j == i + 1) continue;
+         for (auto &in : fOperators[j]->GetOpInputTensors())
+            if (in == mid) other_use = true;
+      }
+      if (other_use) continue;
+      if (prod.FuseActivation(EActivationType::RELU)) act.SetFusedAway();
+   }
+}
+
+std::string RModel::RootOf(const std::string &name) const
+{
+   std::string r = name;
+   for (auto it = fViewOf.find(r); it != fViewOf.end(); it = fViewOf.find(r)) r = it->second;
+   return r;
+}
+
+// Lifetime of every intermediate = [index of its producer, index of its last consumer]; views
+// extend the lifetime of the tensor they alias. Slots are assigned first-fit in producer order
+// against all already-placed tensors whose lifetimes overlap (the reference's planner has the
+// same goal, RModel.cxx:304-394, but tracks last use from incomplete operator input lists).
+void RModel::PlanIntermediateMemory()
+{
+   fViewOf.clear();
+   fPlacement.clear();
+   for (auto &op : fOperators) {
+      std::string v = op->IsFusedAway() ? op->GetOpInputTensors()[0] : op->ViewOf();
+      if (!v.empty() && !op->GetOpOutputTensors().empty() && fIntermediateTensorInfos.count(v))
+         fViewOf[op->GetOpOutputTensors()[0]] = v;
+   }
+   const int nops = (int)fOperators.size();
+   std::vector<std::string> order;
+   for (int i = 0; i < nops; ++i) {
+      for (auto &out : fOperators[i]->GetOpOutputTensors()) {
+         if (!fIntermediateTensorInfos.count(out) || fViewOf.count(out) || fPlacement.count(out)) continue;
+         Placement p;
+         p.first = p.last = i;
+         auto &info = fIntermediateTensorInfos[out];
+         p.bytes = (ConvertShapeToLength(info.shape) * GetTypeSize(info.type) + 255) / 256 * 256;
+         fPlacement[out] = p;
+         order.push_back(out);
+      }
+   }
+   for (int i = 0; i < nops; ++i)
+      for (auto &in : fOperators[i]->GetOpInputTensors()) {
+         auto f = fPlacement.find(RootOf(in));
+         if (f != fPlacement.end() && i > f->second.last) f->second.last = i;
+      }
+   for (auto &n : fOutputTensorNames) {
+      auto f = fPlacement.find(RootOf(n));
+      if (f != fPlacement.end()) f->second.last = nops;
+   }
+   // intermediates registered by an operator but never listed as its output (none today) stay alive throughout
+   for (auto &it : fIntermediateTensorInfos)
+      if (!fPlacement.count(it.first) && !fViewOf.count(it.first)) {
+         Placement p;
+         p.first = 0;
+         p.last = nops;
+         p.bytes = (ConvertShapeToLength(it.second.shape) * GetTypeSize(it.second.type) + 255) / 256 * 256;
+         fPlacement[it.first] = p;
+         order.push_back(it.first);
+      }
+   fArenaBytes = 0;
+   std::vector<std::string> placed;
+   for (auto &name : order) {
+      Placement &p = fPlacement[name];
+      size_t off = 0;
+      bool moved = true;
+      while (moved) {
+         moved = false;
+         for (auto &other : placed) {
+            const Placement &q = fPlacement[other];
+            const bool time_overlap = p.first <= q.last && q.first <= p.last;
+            const bool space_overlap = off < q.offset + q.bytes && q.offset < off + p.bytes;
+            if (time_overlap && space_overlap) {
+               off = q.offset + q.bytes;
+               moved = true;
+            }
+         }
+      }
+      p.offset = off;
+      placed.push_back(name);
+      if (off + p.bytes > fArenaBytes) fArenaBytes = off + p.bytes;
+   }
+}
+
+void RModel::GenerateHeaderInfo(std::string &hgname)
+{
+   fGC += "//Code generated automatically by SOFIE (MI355X device emission) from file " + fFileName +
+          " at [" + fParseTime.substr(0, fParseTime.length() - 1) + "] \n";
+   hgname = fName;
+   std::transform(hgname.begin(), hgname.end(), hgname.begin(), [](unsigned char c) { return std::toupper(c); });
+   hgname = "SOFIE_" + hgname;
+   fGC += "\n#ifndef " + hgname + "\n";
+   fGC += "#define " + hgname + "\n\n";
+   for (auto &i : fNeededStdLib) fGC += "#include <" + i + ">\n";
+   for (auto &i : fCustomOpHeaders) fGC += "#include \"" + i + "\"\n";
+   fGC += "#include <cstdint>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n";
+   // the numerical library: a C ABI over device pointers instead of the reference's
+   // extern "C" BLAS prototypes (RModel_Base.cxx:40-58)
+   fGC += "#include \"sofie_hip.h\"\n";
+   fGC += "\nnamespace SOFIE_" + fName + "{\n";
+}
+
+std::string RModel::GenerateInferSignature(bool isdecl)
+{
+   std::string rGC;
+   int i_input = 0;
+   for (auto &name : fInputTensorNames) {
+      if (i_input++ > 0) rGC += ", ";
+      if (isdecl) rGC += ConvertTypeToString(GetTensorType(name)) + "* ";
+      rGC += "tensor_" + name;
+   }
+   return rGC;
+}
+
+void RModel::ReadInitializedTensorsFromFile(long /*pos*/)
+{
+   // Generated reader of the text weight file: "tensor_<name> <length>" then the values, with the
+   // reference's name and length checks (RModel.cxx:970-1018). Integer tensors use the same
+   // record layout (the reference silently skips every non-float tensor, :1150-1152).
+   bool any = false;
+   for (auto &i : fInitializedTensors) any |= i.second.IsWeightTensor();
+   if (!any) return;
+   fGC += "   std::ifstream f;\n";
+   fGC += "   f.open(filename);\n";
+   fGC += "   if (!f.is_open()) {\n";
+   fGC += "      throw std::runtime_error(\"tmva-sofie failed to open file \" + filename + \" for input weights\");\n";
+   fGC += "   }\n";
+   fGC += "   std::string tensor_name;\n";
+   fGC += "   size_t length;\n";
+   for (auto &i : fInitializedTensors) {
+      if (!i.second.IsWeightTensor()) continue;
+      const std::string tensor_name = "tensor_" + i.first;
+      const std::string slength = std::to_string(ConvertShapeToLength(i.second.shape()));
+      const std::string ctype = ConvertTypeToString(i.second.type());
+      const bool narrow = GetTypeSize(i.second.type()) == 1;   // read bytes through int, not char
+      fGC += "   f >> tensor_name >> length;\n";
+      fGC += "   if (tensor_name != \"" + tensor_name + "\" ) {\n";
+      fGC += "      std::string err_msg = \"TMVA-SOFIE failed to read the correct tensor name; expected name is " +
+             tensor_name + " , read \" + tensor_name;\n";
+      fGC += "      throw std::runtime_error(err_msg);\n";
+      fGC += "    }\n";
+      fGC += "   if (length != " + slength + ") {\n";
+      fGC += "      std::string err_msg = \"TMVA-SOFIE failed to read the correct tensor size; expected size is " + slength +
+             " , read \" + std::to_string(length) ;\n";
+      fGC += "      throw std::runtime_error(err_msg);\n";
+      fGC += "    }\n";
+      fGC += "   {\n";
+      fGC += "      std::vector<" + ctype + "> host(" + slength + ");\n";
+      if (narrow)
+         fGC += "      for (size_t i = 0; i < length; ++i) { int v; f >> v; host[i] = static_cast<" + ctype + ">(v); }\n";
+      else
+         fGC += "      for (size_t i = 0; i < length; ++i) f >> host[i];\n";
+      fGC += "      if (f.fail()) {\n";
+      fGC += "         throw std::runtime_error(\"TMVA-SOFIE failed to read the values for tensor " + tensor_name + "\");\n";
+      fGC += "      }\n";
+      fGC += "      Check(sofie_hip_upload(fCtx, " + tensor_name + ", host.data(), length * sizeof(" + ctype + ")), \"upload of " +
+             tensor_name + "\");\n";
+      fGC += "   }\n";
+   }
+   fGC += "   f.close();\n";
+}
+
+long RModel::WriteInitializedTensorsToFile(std::string filename)
+{
+   if (filename == "") filename = fName + ".dat";
+   std::ofstream f(filename);
+   if (!f.is_open()) throw std::runtime_error("tmva-sofie failed to open file " + filename + " for tensor weight data");
+   for (auto &i : fInitializedTensors) {
+      if (!i.second.IsWeightTensor()) continue;
+      const size_t length = ConvertShapeToLength(i.second.shape());
+      f << "tensor_" << i.first << " " << length << "\n";
+      for (size_t idx = 0; idx < length; idx++) {
+         switch (i.second.type()) {
+         case ETensorType::FLOAT: {
+            // same text as the reference: max_digits10, subnormals flushed to zero (RModel.cxx:1140-1147)
+            float value = i.second.data<float>()[idx];
+            if (value != 0. && std::abs(value) < std::numeric_limits<float>::min()) value = 0;
+            f << std::setprecision(std::numeric_limits<float>::max_digits10) << value;
+            break;
+         }
+         case ETensorType::INT8: f << (int)i.second.data<int8_t>()[idx]; break;
+         case ETensorType::UINT8:
+         case ETensorType::FLOAT8E4M3FN: f << (int)i.second.data<uint8_t>()[idx]; break;
+         case ETensorType::INT32: f << i.second.data<int32_t>()[idx]; break;
+         case ETensorType::INT64: f << i.second.data<int64_t>()[idx]; break;
+         default:
+            throw std::runtime_error("tmva-sofie tensor tensor_" + i.first + " with type " +
+                                     ConvertTypeToString(i.second.type()) + " cannot be written to a file");
+         }
+         f << ((idx < length - 1) ? " " : "\n");
+      }
+      if (length == 0) f << "\n";
+      if (f.fail()) throw std::runtime_error("tmva-sofie failed to write tensor data to file for tensor_" + i.first);
+   }
+   long pos = f.tellp();
+   f.close();
+   return pos;
+}
+
+void RModel::GenerateSessionCode()
+{
+   fGC += "struct Session {\n";
+   fGC += "sofie_hip_ctx* fCtx = nullptr;\n";
+   fGC += "static void Check(sofie_hip_ctx* ctx, int status, const char* what) {\n";
+   fGC += "   if (status != 0) throw std::runtime_error(std::string(\"TMVA SOFIE device error in \") + what + \": \" + "
+          "sofie_hip_last_error(ctx));\n";
+   fGC += "}\n";
+   fGC += "void Check(int status, const char* what) { Check(fCtx, status, what); }\n";
+   // weights: device pointers, uploaded once in the constructor
+   for (auto &i : fInitializedTensors) {
+      if (!i.second.IsWeightTensor()) continue;   // folded into other tensors at generation time
+      const std::string ctype = ConvertTypeToString(i.second.type());
+      fGC += ctype + " * tensor_" + i.first + " = nullptr;   // device, " +
+             std::to_string(ConvertShapeToLength(i.second.shape())) + " elements\n";
+   }
+   // inputs: device staging buffers for the host-pointer infer()
+   for (auto &n : fInputTensorNames)
+      fGC += ConvertTypeToString(GetTensorType(n)) + " * fInput_" + n + " = nullptr;   // device copy of the input\n";
+   // intermediates: one device arena, offsets from the memory plan
+   fGC += "char* fIntermediateMemoryPool = nullptr;   // device, " + std::to_string(fArenaBytes) + " bytes\n";
+   for (auto &it : fIntermediateTensorInfos)
+      fGC += ConvertTypeToString(it.second.type) + " * tensor_" + it.first + " = nullptr;\n";
+   for (size_t id = 0; id < fOperators.size(); id++) fGC += fOperators[id]->GenerateSessionMembersCode(std::to_string(id));
+   fGC += "\n";
+
+   // ---- constructor
+   fGC += "Session(std::string filename =\"" + (fUseWeightFile ? fName + ".dat" : std::string("")) + "\", int device = 0) {\n";
+   fGC += "   { int status = sofie_hip_create(&fCtx, device, nullptr);\n";
+   fGC += "     if (status != 0) throw std::runtime_error(\"TMVA SOFIE cannot create a device context\"); }\n";
+   fGC += "   try {\n";
+   for (auto &i : fInitializedTensors) {
+      if (!i.second.IsWeightTensor()) continue;
+      const size_t bytes = ConvertShapeToLength(i.second.shape()) * GetTypeSize(i.second.type());
+      fGC += "   Check(sofie_hip_malloc(fCtx, reinterpret_cast<void**>(&tensor_" + i.first + "), " + std::to_string(bytes) +
+             "), \"allocation of tensor_" + i.first + "\");\n";
+   }
+   for (auto &n : fInputTensorNames) {
+      const size_t bytes = ConvertShapeToLength(GetTensorShape(n)) * GetTypeSize(GetTensorType(n));
+      fGC += "   Check(sofie_hip_malloc(fCtx, reinterpret_cast<void**>(&fInput_" + n + "), " + std::to_string(bytes) +
+             "), \"allocation of the input buffer\");\n";
+   }
+   fGC += "   Check(sofie_hip_malloc(fCtx, reinterpret_cast<void**>(&fIntermediateMemoryPool), " +
+          std::to_string(fArenaBytes) + "), \"allocation of the intermediate pool\");\n";
+   for (auto &it : fIntermediateTensorInfos) {
+      if (fViewOf.count(it.first)) continue;
+      fGC += "   tensor_" + it.first + " = reinterpret_cast<" + ConvertTypeToString(it.second.type) +
+             "*>(fIntermediateMemoryPool + " + std::to_string(fPlacement[it.first].offset) + ");\n";
+   }
+   // views after their roots
+   for (auto &op : fOperators)
+      for (auto &out : op->GetOpOutputTensors()) {
+         auto v = fViewOf.find(out);
+         if (v == fViewOf.end()) continue;
+         fGC += "   tensor_" + out + " = reinterpret_cast<" + ConvertTypeToString(fIntermediateTensorInfos[out].type) +
+                "*>(tensor_" + v->second + ");\n";
+      }
+   if (fUseWeightFile) {
+      ReadInitializedTensorsFromFile(0);
+   } else {
+      for (auto &i : fInitializedTensors) {
+         if (!i.second.IsWeightTensor()) continue;
+         const std::string ctype = ConvertTypeToString(i.second.type());
+         const size_t length = ConvertShapeToLength(i.second.shape());
+         std::stringstream lit;
+         lit << "   { static const " << ctype << " host[" << (length ? length : 1) << "] = {";
+         for (size_t idx = 0; idx < length; ++idx) {
+            if (idx) lit << ", ";
+            switch (i.second.type()) {
+            case ETensorType::FLOAT:
+            {
+               std::stringstream one;
+               one << std::setprecision(std::numeric_limits<float>::max_digits10) << i.second.data<float>()[idx];
+               std::string text = one.str();
+               if (!std::isfinite(i.second.data<float>()[idx]))
+                  throw std::runtime_error("tmva-sofie tensor_" + i.first + " holds a non-finite value");
+               // a float literal needs a '.' or an exponent before its suffix
+               if (text.find_first_of(".e") == std::string::npos) text += ".";
+               lit << text << "f";
+               break;
+            }
+            case ETensorType::INT8: lit << (int)i.second.data<int8_t>()[idx]; break;
+            case ETensorType::UINT8:
+            case ETensorType::FLOAT8E4M3FN: lit << (int)i.second.data<uint8_t>()[idx]; break;
+            case ETensorType::INT32: lit << i.second.data<int32_t>()[idx]; break;
+            case ETensorType::INT64: lit << i.second.data<int64_t>()[idx]; break;
+            default: throw std::runtime_error("tmva-sofie tensor_" + i.first + " cannot be written as a literal");
+            }
+         }
+         lit << "};\n     Check(sofie_hip_upload(fCtx, tensor_" << i.first << ", host, " << length * GetTypeSize(i.second.type())
+             << "), \"upload of tensor_" << i.first << "\"); }\n";
+         fGC += lit.str();
+      }
+   }
+   for (size_t id = 0; id < fOperators.size(); id++) fGC += fOperators[id]->GenerateInitCode();
+   fGC += "   Check(sofie_hip_sync(fCtx), \"Session construction\");\n";
+   fGC += "   } catch (...) { Release(); throw; }\n";
+   fGC += "}\n\n";
+
+   // ---- destructor (the reference's Session leaks its pool; device memory must not)
+   fGC += "void Release() {\n";
+   fGC += "   if (!fCtx) return;\n";
+   for (auto &i : fInitializedTensors)
+      if (i.second.IsWeightTensor()) fGC += "   sofie_hip_free(fCtx, tensor_" + i.first + ");\n";
+   for (auto &n : fInputTensorNames) fGC += "   sofie_hip_free(fCtx, fInput_" + n + ");\n";
+   fGC += "   sofie_hip_free(fCtx, fIntermediateMemoryPool);\n";
+   fGC += "   sofie_hip_destroy(fCtx);\n";
+   fGC += "   fCtx = nullptr;\n";
+   fGC += "}\n";
+   fGC += "~Session() { Release(); }\n";
+   fGC += "Session(const Session&) = delete;\n";
+   fGC += "Session& operator=(const Session&) = delete;\n\n";
+
+   // ---- the operator sequence on device pointers
+   fGC += "// every argument is a device pointer; kernels are enqueued on the Session's stream\n";
+   fGC += "void run_device(";
+   {
+      int k = 0;
+      for (auto &n : fInputTensorNames) {
+         if (k++) fGC += ", ";
+         fGC += "const " + ConvertTypeToString(GetTensorType(n)) + "* tensor_" + n;
+      }
+   }
+   fGC += "){\n";
+   for (size_t id = 0; id < fOperators.size(); id++) {
+      if (fOperators[id]->IsFusedAway()) continue;
+      fGC += fOperators[id]->Generate(std::to_string(id));
+   }
+   fGC += "}\n\n";
+
+   if (fOutputTensorNames.size() != 1)
+      throw std::runtime_error("TMVA-SOFIE: the device emission supports exactly one output tensor");
+   const std::string out = fOutputTensorNames[0];
+   const std::string otype = ConvertTypeToString(GetTensorType(out));
+   const size_t olen = ConvertShapeToLength(GetTensorShape(out));
+
+   // ---- infer on host pointers: same signature and return convention as the reference
+   // (RModel.cxx:680-801): one upload, the kernel sequence, one download
+   fGC += "std::vector<" + otype + "> infer(" + GenerateInferSignature(true) + "){\n";
+   for (auto &n : fInputTensorNames) {
+      const size_t bytes = ConvertShapeToLength(GetTensorShape(n)) * GetTypeSize(GetTensorType(n));
+      fGC += "   Check(sofie_hip_upload(fCtx, fInput_" + n + ", tensor_" + n + ", " + std::to_string(bytes) + "), \"input upload\");\n";
+   }
+   fGC += "   run_device(";
+   {
+      int k = 0;
+      for (auto &n : fInputTensorNames) fGC += std::string(k++ ? ", " : "") + "fInput_" + n;
+   }
+   fGC += ");\n";
+   fGC += "   std::vector<" + otype + "> ret(" + std::to_string(olen) + ");\n";
+   fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", " + std::to_string(olen) + " * sizeof(" + otype +
+          ")), \"output download\");\n";
+   fGC += "   return ret;\n";
+   fGC += "}\n\n";
+
+   // ---- infer on device pointers: nothing crosses PCIe; returns the device address of the output
+   fGC += "const " + otype + "* infer_device(";
+   {
+      int k = 0;
+      for (auto &n : fInputTensorNames) {
+         if (k++) fGC += ", ";
+         fGC += "const " + ConvertTypeToString(GetTensorType(n)) + "* tensor_" + n;
+      }
+   }
+   fGC += "){\n   run_device(";
+   {
+      int k = 0;
+      for (auto &n : fInputTensorNames) fGC += std::string(k++ ? ", " : "") + "tensor_" + n;
+   }
+   fGC += ");\n   return tensor_" + out + ";\n}\n";
+   fGC += "void sync() { Check(sofie_hip_sync(fCtx), \"sync\"); }\n";
+   fGC += "};\n";
+}
+
+void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, long pos, bool verbose)
+{
+   fVerbose = verbose;
+   if (static_cast<std::underlying_type_t<Options>>(Options::kNoSession) & options)
+      throw std::runtime_error("TMVA-SOFIE: Options::kNoSession is not available: device weights and buffers need the Session as owner");
+   if (static_cast<std::underlying_type_t<Options>>(Options::kRootBinaryWeightFile) & options)
+      throw std::runtime_error("TMVA-SOFIE: ROOT binary weight files are not available in this build");
+   if (static_cast<std::underlying_type_t<Options>>(Options::kNoWeightFile) & options) {
+      fUseWeightFile = false;
+      fWeightFile = WeightFileType::None;
+   }
+   (void)pos;
+   Initialize(batchSize, verbose);
+   FuseActivations();
+   PlanIntermediateMemory();
+   fGC.clear();
+   std::string hgname;
+   GenerateHeaderInfo(hgname);
+   GenerateSessionCode();
+   fGC += ("} //SOFIE_" + fName + "\n");
+   fGC += "\n#endif  // " + hgname + "\n";
+}
+
+void RModel::PrintGenerated() { std::cout << fGC; }
+
+void RModel::OutputGenerated(std::string filename, bool append)
+{
+   if (filename == "") filename = fName + ".hxx";
+   std::ofstream f;
+   f.open(filename, append ? std::ios::app : std::ios::out);
+   if (!f.is_open()) throw std::runtime_error("tmva-sofie failed to open file for output generated inference code");
+   f << fGC;
+   f.close();
+   if (fUseWeightFile) {
+      // weight file next to the header, same stem (RModel.cxx:1290-1310)
+      size_t p = filename.find(".hxx");
+      std::string dat = filename;
+      if (p != std::string::npos) dat.replace(p, 4, ".dat");
+      else dat += ".dat";
+      WriteInitializedTensorsToFile(dat);
+   }
+}
+
+}   // namespace SOFIE

@@ -1,0 +1,42 @@
+"""Generate and compile (on the CPU, ahead of any GPU run) the Session code of every network the GPU tests
+and the benchmark execute: the reference's Gemm / Conv / MaxPool fixtures, the fp32 MLP, the CNN in fp32
+and the int8 CNN. Output: sofie_amd/generated/{<name>.hxx, <name>.dat, run_<name>}.
+
+    python tests/build_generated.py
+"""
+import os
+import sys
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+for p in (ROOT, os.path.join(ROOT, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+import models  # noqa: E402
+from oracle import oracle  # noqa: E402
+from sofie_amd import emit  # noqa: E402
+
+
+def all_specs(with_large=True):
+    specs = [models.fixture_spec(n)[0] for n in models.FIXTURES]
+    specs.append(models.mlp_spec()[0])
+    specs.append(models.cnn_f32_spec(8))
+    specs.append(models.qcnn_spec(oracle, 8))
+    if with_large:
+        specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
+    return specs
+
+
+def main():
+    emit.build_emitter()
+    for spec in all_specs():
+        hxx, dat, res = spec.generate()
+        exe = spec.compile_runner()
+        if spec.name == "qcnn_b4096":
+            os.remove(dat)      # same tensors as qcnn.dat: the runner is pointed at that file
+        print("%-28s %s" % (spec.name, res.stdout.strip().split(", ")[-1]))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,184 @@
+"""The networks the tests and the benchmark push through the C++ emitter, with seeded weights, and the
+CPU-oracle evaluation of each (test infrastructure)."""
+import os
+
+import numpy as np
+
+from sofie_amd import emit, onnx_wire
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+FIXTURES = ["Linear_16", "Linear_32", "Linear_64", "ConvWithPadding", "ConvWithoutPadding",
+            "ConvWithAutopadSameLower", "ConvWithStridesPadding", "ConvWithStridesNoPadding",
+            "ConvWithAsymmetricPadding", "MaxPool2d"]
+
+
+def fixture_spec(name):
+    graph = onnx_wire.load(os.path.join(GOLD, "onnx", name + ".onnx"))
+    return emit.spec_from_onnx(name, graph), graph
+
+
+# ------------------------------------------------------------------------------------------ fp32 MLP
+def mlp_weights(seed=0):
+    """Glorot-uniform weights, zero biases, N(0,1) input; draw order W1, W2, W3, x."""
+    r = np.random.default_rng(seed)
+    dims = [(64, 128), (128, 64), (64, 8)]
+    Ws = [r.uniform(-np.sqrt(6.0 / (a + b)), np.sqrt(6.0 / (a + b)), (a, b)).astype(np.float32) for a, b in dims]
+    Bs = [np.zeros(b, np.float32) for _, b in dims]
+    x = r.standard_normal((256, 64)).astype(np.float32)
+    return Ws, Bs, x
+
+
+def mlp_spec(name="mlp_c1", seed=0):
+    Ws, Bs, x = mlp_weights(seed)
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", x.shape)
+    for i, (W, B) in enumerate(zip(Ws, Bs)):
+        s.add_init("W%d" % i, W)
+        s.add_init("B%d" % i, B)
+    s.gemm("x", "W0", "B0", "h0", relu=True)
+    s.gemm("h0", "W1", "B1", "h1", relu=True)
+    s.gemm("h1", "W2", "B2", "y")
+    s.set_output("y")
+    return s, x
+
+
+def mlp_reference(oracle, seed=0):
+    Ws, Bs, x = mlp_weights(seed)
+    h = oracle.gemm_f32(x, Ws[0], Bs[0], relu=True)
+    h = oracle.gemm_f32(h, Ws[1], Bs[1], relu=True)
+    return oracle.gemm_f32(h, Ws[2], Bs[2])
+
+
+# ------------------------------------------------------------------------------------------ CNN (fp32 and int8)
+def cnn_float_params(seed=1):
+    r = np.random.default_rng(seed)
+
+    def kaiming(shape):
+        fan = int(np.prod(shape[1:]))
+        return (r.standard_normal(shape) * np.sqrt(2.0 / fan)).astype(np.float32)
+    p = {"w1": kaiming((32, 1, 3, 3)), "w2": kaiming((64, 32, 3, 3)), "w3": kaiming((128, 64, 3, 3)),
+         "fc1": kaiming((256, 12800)).T.copy(), "fc2": kaiming((5, 256)).T.copy()}
+    for k, n in (("b1", 32), ("b2", 64), ("b3", 128), ("bf1", 256), ("bf2", 5)):
+        p[k] = (r.standard_normal(n) * 0.05).astype(np.float32)
+    return p
+
+
+def cnn_input(batch, seed=2):
+    return np.random.default_rng(seed).uniform(0, 1, (batch, 1, 40, 40)).astype(np.float32)
+
+
+def cnn_f32_spec(batch, name="cnn_f32"):
+    p = cnn_float_params()
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", (batch, 1, 40, 40))
+    for k, v in p.items():
+        s.add_init(k, v)
+    s.conv("x", "w1", "b1", "c1", (3, 3), (1, 1, 1, 1), (1, 1)); s.relu("c1", "r1")
+    s.maxpool("r1", "p1", (2, 2), (0, 0, 0, 0), (2, 2))
+    s.conv("p1", "w2", "b2", "c2", (3, 3), (1, 1, 1, 1), (1, 1)); s.relu("c2", "r2")
+    s.maxpool("r2", "p2", (2, 2), (0, 0, 0, 0), (2, 2))
+    s.conv("p2", "w3", "b3", "c3", (3, 3), (1, 1, 1, 1), (1, 1)); s.relu("c3", "r3")
+    s.flatten("r3", "f")
+    s.gemm("f", "fc1", "bf1", "g1"); s.relu("g1", "rg1")
+    s.gemm("rg1", "fc2", "bf2", "y")
+    s.set_output("y")
+    return s
+
+
+def cnn_f32_stages(oracle, x):
+    """Float activations after every layer (also used to calibrate the int8 network)."""
+    p = cnn_float_params()
+    a1 = oracle.conv2d_f32(x, p["w1"], p["b1"], (1, 1), relu=True)
+    q1 = oracle.maxpool2d(a1, (2, 2), (2, 2))
+    a2 = oracle.conv2d_f32(q1, p["w2"], p["b2"], (1, 1), relu=True)
+    q2 = oracle.maxpool2d(a2, (2, 2), (2, 2))
+    a3 = oracle.conv2d_f32(q2, p["w3"], p["b3"], (1, 1), relu=True)
+    f = a3.reshape(a3.shape[0], -1)
+    g1 = oracle.gemm_f32(f, p["fc1"], p["bf1"], relu=True)
+    y = oracle.gemm_f32(g1, p["fc2"], p["bf2"])
+    return {"a1": a1, "a2": a2, "a3": a3, "g1": g1, "y": y}
+
+
+_QP = None
+
+
+def qcnn_params(oracle):
+    """Per-output-channel symmetric int8 weights, int32 biases, activation scales from a seeded
+    calibration batch (max / 255 with zero-point -128, i.e. the uint8 range of a post-ReLU tensor)."""
+    global _QP
+    if _QP is not None:
+        return _QP
+    p = cnn_float_params()
+    st = cnn_f32_stages(oracle, cnn_input(8, seed=3))
+    q = {"sx": np.float32(1.0 / 255.0)}
+    for k in ("a1", "a2", "a3", "g1"):
+        q["s_" + k] = np.float32(float(st[k].max()) / 255.0)
+
+    def qweights(w, axis_out):
+        flat = w.reshape(w.shape[0], -1) if axis_out == 0 else w.T.reshape(w.shape[1], -1)
+        sw = (np.abs(flat).max(axis=1) / 127.0).astype(np.float32)
+        shape = [-1] + [1] * (w.ndim - 1) if axis_out == 0 else [1, -1]
+        wq = np.clip(np.rint(w / sw.reshape(shape)), -127, 127).astype(np.int8)
+        return wq, sw
+    s_in = {"w1": q["sx"], "w2": q["s_a1"], "w3": q["s_a2"], "fc1": q["s_a3"], "fc2": q["s_g1"]}
+    bias = {"w1": "b1", "w2": "b2", "w3": "b3", "fc1": "bf1", "fc2": "bf2"}
+    for k in ("w1", "w2", "w3"):
+        q[k], q["s_" + k] = qweights(p[k], 0)
+    for k in ("fc1", "fc2"):
+        q[k], q["s_" + k] = qweights(p[k], 1)      # [K,N], scale per column
+    for k, b in bias.items():
+        q[b] = np.rint(p[b] / (s_in[k] * q["s_" + k])).astype(np.int32)
+    _QP = q
+    return q
+
+
+def qcnn_spec(oracle, batch, name="qcnn"):
+    q = qcnn_params(oracle)
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", (batch, 1, 40, 40))
+    s.add_scalar("sx", q["sx"], np.float32)
+    s.add_scalar("zp", -128, np.int8)
+    for k in ("a1", "a2", "a3", "g1"):
+        s.add_scalar("s_" + k, q["s_" + k], np.float32)
+    for k in ("w1", "w2", "w3", "fc1", "fc2"):
+        s.add_init(k, q[k])
+        s.add_init("s_" + k, q["s_" + k])
+    for b in ("b1", "b2", "b3", "bf1", "bf2"):
+        s.add_init(b, q[b])
+    s.quantize("x", "sx", "zp", "xq")
+    s.qlinear_conv("xq", "sx", "zp", "w1", "s_w1", None, "s_a1", "zp", "c1", "b1", (3, 3), (1, 1, 1, 1), (1, 1))
+    s.relu("c1", "r1")
+    s.maxpool("r1", "p1", (2, 2), (0, 0, 0, 0), (2, 2))
+    s.qlinear_conv("p1", "s_a1", "zp", "w2", "s_w2", None, "s_a2", "zp", "c2", "b2", (3, 3), (1, 1, 1, 1), (1, 1))
+    s.relu("c2", "r2")
+    s.maxpool("r2", "p2", (2, 2), (0, 0, 0, 0), (2, 2))
+    s.qlinear_conv("p2", "s_a2", "zp", "w3", "s_w3", None, "s_a3", "zp", "c3", "b3", (3, 3), (1, 1, 1, 1), (1, 1))
+    s.relu("c3", "r3")
+    s.flatten("r3", "f")
+    s.qlinear_matmul("f", "s_a3", "zp", "fc1", "s_fc1", None, "s_g1", "zp", "g1", "bf1")
+    s.relu("g1", "rg1")
+    s.qlinear_matmul("rg1", "s_g1", "zp", "fc2", "s_fc2", None, None, None, "y", "bf2")
+    s.set_output("y")
+    return s
+
+
+def qcnn_reference(oracle, x):
+    """The same network evaluated with the CPU oracle; per-channel scales are formed in fp32 in the
+    emitter's order, (s_in * s_w[n]) / s_out."""
+    q = qcnn_params(oracle)
+    f32 = np.float32
+    xq = oracle.quantize_f32_s8(x, q["sx"], -128)
+
+    def conv(xi, w, b, s_in, s_out):
+        scale = ((f32(s_in) * q["s_" + w]).astype(f32) / f32(s_out)).astype(f32)
+        return oracle.qconv2d_s8(xi, q[w], scale, q[b], (1, 1), (1, 1), 1, -128, -128, True)
+    c1 = oracle.maxpool2d(conv(xq, "w1", "b1", q["sx"], q["s_a1"]), (2, 2), (2, 2))
+    c2 = oracle.maxpool2d(conv(c1, "w2", "b2", q["s_a1"], q["s_a2"]), (2, 2), (2, 2))
+    c3 = conv(c2, "w3", "b3", q["s_a2"], q["s_a3"])
+    f = c3.reshape(c3.shape[0], -1)
+    s1 = ((f32(q["s_a3"]) * q["s_fc1"]).astype(f32) / f32(q["s_g1"])).astype(f32)
+    g1 = oracle.qgemm_s8(f, q["fc1"], s1, q["bf1"], False, zpa=-128, zpy=-128, relu=True)
+    s2 = (f32(q["s_g1"]) * q["s_fc2"]).astype(f32)
+    bias2 = (q["bf2"].astype(np.int64) + 128 * q["fc2"].astype(np.int64).sum(axis=0)).astype(np.int32)
+    acc = oracle.igemm_s8(g1, q["fc2"]).astype(np.int64) + bias2
+    return (acc.astype(np.int32).astype(f32) * s2).astype(f32)

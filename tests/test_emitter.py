@@ -1,0 +1,178 @@
+"""Host-side code generator (RModel / ROperator mirror): generation, fusion, memory plan, weight file
+format and error behaviour. No GPU needed: the generated Sessions are only compiled here."""
+import os
+import re
+import subprocess
+
+import numpy as np
+import pytest
+
+import models
+from oracle import oracle
+from sofie_amd import emit
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _emitter():
+    emit.build_emitter()
+
+
+def gen(spec, tmp_path, **kw):
+    return spec.generate(str(tmp_path), **kw)
+
+
+def test_weight_file_text_matches_the_reference_format(tmp_path):
+    """`tensor_<name> <count>` header line, one value line, max_digits10 significant digits: the text the
+    reference writes for B = [0.5, 0.5, -10, 0] and a 12-element W (RModel.cxx:1121-1158)."""
+    s = emit.ModelSpec("probe")
+    s.add_input("x", "FLOAT", (2, 3))
+    s.add_init("B", np.array([0.5, 0.5, -10, 0], np.float32))
+    s.add_init("W", np.array([1, 2, 3, -1, -2, -3, 0.5, 0.5, 0.5, 0, 0, 1], np.float32).reshape(4, 3))
+    s.gemm("x", "W", "B", "y", transB=1, relu=True)
+    s.set_output("y")
+    hxx, dat, _ = gen(s, tmp_path)
+    assert open(dat).read() == "tensor_B 4\n0.5 0.5 -10 0\ntensor_W 12\n1 2 3 -1 -2 -3 0.5 0.5 0.5 0 0 1\n"
+    code = open(hxx).read()
+    assert "namespace SOFIE_probe{" in code and "struct Session {" in code
+    assert 'Session(std::string filename ="probe.dat"' in code
+    assert "std::vector<float> infer(float* tensor_x)" in code
+    # Gemm with transB, rank-1 bias broadcast in the epilogue (kind 1), fused ReLU
+    assert re.search(r"sofie_hip_gemm_f32\(fCtx, 0, 1, 2, 4, 3, .*tensor_x, 3, tensor_W, 3, .*tensor_B, 1, tensor_y, 4, SOFIE_ACT_RELU\)", code)
+
+
+def test_subnormal_weights_are_flushed_and_digits_round_trip(tmp_path):
+    s = emit.ModelSpec("tiny")
+    s.add_input("x", "FLOAT", (1, 2))
+    w = np.array([[1e-42, 0.1], [np.float32(1) / 3, -2.5e-39]], np.float32)
+    s.add_init("W", w)
+    s.gemm("x", "W", None, "y", beta=0.0)
+    s.set_output("y")
+    _, dat, _ = gen(s, tmp_path)
+    vals = np.array(open(dat).read().split("\n")[1].split(), np.float64).astype(np.float32)
+    want = w.reshape(-1).copy()
+    want[np.abs(want) < np.finfo(np.float32).tiny] = 0
+    assert np.array_equal(vals, want)          # 9 significant digits reproduce every float32 exactly
+
+
+def test_relu_after_gemm_and_conv_is_fused_and_flatten_is_a_view(tmp_path):
+    spec = models.cnn_f32_spec(2, "cnn_small")
+    hxx, _, res = gen(spec, tmp_path)
+    code = open(hxx).read()
+    assert code.count("sofie_hip_conv2d_f32(") == 3 and code.count("SOFIE_ACT_RELU") == 4
+    assert "sofie_hip_relu_f32" not in code
+    assert "tensor_f = reinterpret_cast<float*>(tensor_r3);" in code
+    assert "tensor_r1 = reinterpret_cast<float*>(tensor_c1);" in code
+    # liveness-based reuse: the pool is smaller than the sum of all intermediates
+    sizes = {"c1": 2 * 32 * 40 * 40, "p1": 2 * 32 * 20 * 20, "c2": 2 * 64 * 20 * 20, "p2": 2 * 64 * 10 * 10,
+             "c3": 2 * 128 * 10 * 10, "g1": 2 * 256, "y": 2 * 5}
+    pool = int(re.search(r"intermediate pool (\d+) bytes", res.stdout).group(1))
+    assert pool < 4 * sum(sizes.values())
+    assert pool >= 4 * (sizes["c1"] + sizes["p1"])      # producer and consumer are live together
+
+
+def test_pool_offsets_never_overlap_while_both_tensors_are_live(tmp_path):
+    spec, _ = models.mlp_spec("mlp_plan")
+    hxx, _, _ = gen(spec, tmp_path)
+    code = open(hxx).read()
+    off = {m.group(1): int(m.group(2)) for m in re.finditer(r"tensor_(\w+) = reinterpret_cast<float\*>\(fIntermediateMemoryPool \+ (\d+)\)", code)}
+    size = {"h0": 256 * 128 * 4, "h1": 256 * 64 * 4, "y": 256 * 8 * 4}
+    assert set(off) == set(size)
+    for a, b in (("h0", "h1"), ("h1", "y")):            # producer/consumer pairs
+        assert off[a] + size[a] <= off[b] or off[b] + size[b] <= off[a]
+    assert all(v % 256 == 0 for v in off.values())
+
+
+def test_conv_default_pads_follow_the_reference(tmp_path):
+    """auto_pad NOTSET and no pads attribute means 1 on every side (ROperator_Conv.hxx:136-139);
+    SAME_LOWER with stride 2 on 5x5 gives the 3x3 output of the reference's fixture."""
+    s = emit.ModelSpec("pads")
+    s.add_input("x", "FLOAT", (1, 1, 5, 5))
+    s.add_init("W", np.ones((1, 1, 3, 3), np.float32))
+    s.conv("x", "W", None, "y", kernel=(3, 3))
+    s.set_output("y")
+    hxx, _, _ = gen(s, tmp_path)
+    assert re.search(r"sofie_hip_conv2d_f32\(fCtx, tensor_x, tensor_W, nullptr, tensor_y, 1, 1, 5, 5, 1, 3, 3, 1, 1, 1, 1, 1, 1, 1,", open(hxx).read())
+    spec, _ = models.fixture_spec("ConvWithAutopadSameLower")
+    hxx, _, res = gen(spec, tmp_path)
+    code = open(hxx).read()
+    assert "std::vector<float> ret(9);" in code
+    assert re.search(r"3, 3, 1, 1, 2, 2, 1, 1, 1, SOFIE_ACT_NONE", code)
+
+
+def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
+    spec = models.qcnn_spec(oracle, 2, "qcnn_small")
+    hxx, dat, _ = gen(spec, tmp_path)
+    code = open(hxx).read()
+    assert code.count("sofie_hip_qconv2d_s8(") == 3 and code.count("sofie_hip_qgemm_s8(") == 2
+    assert "int8_t * tensor_fc1_nk" in code and "tensor_fc1 =" not in code      # transposed once, original dropped
+    assert "SOFIE_OUT_F32" in code and "std::vector<float> infer(float* tensor_x)" in code
+    q = models.qcnn_params(oracle)
+    text = open(dat).read().split("\n")
+    rec = {text[i].split()[0]: text[i + 1] for i in range(0, len(text) - 1, 2)}
+    scale = np.array(rec["tensor_c1_qscale"].split(), np.float64).astype(np.float32)
+    want = ((np.float32(q["sx"]) * q["s_w1"]).astype(np.float32) / np.float32(q["s_a1"])).astype(np.float32)
+    assert np.array_equal(scale, want)
+    qb = np.array(rec["tensor_c1_qbias"].split(), np.int64)
+    assert np.array_equal(qb, q["b1"].astype(np.int64) + 128 * q["w1"].astype(np.int64).reshape(32, -1).sum(axis=1))
+    fc1 = np.array(rec["tensor_fc1_nk"].split(), np.int64).reshape(256, 12800)
+    assert np.array_equal(fc1, q["fc1"].T)
+
+
+def emit_error(spec, tmp_path):
+    _, _, res = spec.generate(str(tmp_path), check=False)
+    assert res.returncode != 0
+    return res.stderr
+
+
+def test_error_messages_follow_the_reference(tmp_path):
+    s = emit.ModelSpec("e1")
+    s.add_input("x", "FLOAT", (2, 3))
+    s.add_init("W", np.ones((3, 4), np.float32))
+    s.gemm("x", "W", None, "y", beta=1.0)
+    s.set_output("y")
+    assert "Bias tensor is not present but beta value in Gemm is not zero" in emit_error(s, tmp_path)
+
+    s = emit.ModelSpec("e2")
+    s.add_input("x", "FLOAT", (2, 3))
+    s.gemm("x", "nope", None, "y", beta=0.0)
+    s.set_output("y")
+    assert "TMVA SOFIE Gemm Op Input Tensor x or nope is not found in model" in emit_error(s, tmp_path)
+
+    s = emit.ModelSpec("e3")
+    s.add_input("x", "FLOAT", (1, 2, 5, 5))
+    s.add_init("W", np.ones((4, 2, 3, 3), np.float32))
+    s.add_init("B", np.ones(3, np.float32))
+    s.conv("x", "W", "B", "y", (3, 3), (1, 1, 1, 1))
+    s.set_output("y")
+    assert "TMVA SOFIE Conv op: Bias Tensor has wrong shape" in emit_error(s, tmp_path)
+
+    s = emit.ModelSpec("e4")
+    s.add_input("x", "FLOAT", (2, 3))
+    s.add_init("W", np.ones((5, 4), np.float32))
+    s.gemm("x", "W", None, "y", beta=0.0)
+    s.set_output("y")
+    assert "has invalid shape" in emit_error(s, tmp_path)
+
+
+def test_no_weight_file_option_embeds_literals(tmp_path):
+    s = emit.ModelSpec("lit")
+    s.add_input("x", "FLOAT", (1, 2))
+    s.add_init("W", np.array([[1.5, -2.0], [0.25, 3.0]], np.float32))
+    s.gemm("x", "W", None, "y", beta=0.0)
+    s.set_output("y")
+    hxx, dat, _ = gen(s, tmp_path, no_weight_file=True)
+    code = open(hxx).read()
+    assert "static const float host[4] = {1.5f, -2.f, 0.25f, 3.f};" in code
+    assert not os.path.exists(dat)
+    # the generated header compiles against the C ABI
+    exe = s.compile_runner(str(tmp_path))
+    assert os.path.exists(exe)
+
+
+def test_every_prebuilt_session_compiles():
+    """tests/build_generated.py output (made by build()): header, weights and runner of each network."""
+    import build_generated
+    for spec in build_generated.all_specs(with_large=True):
+        for ext in (".hxx",):
+            assert os.path.exists(os.path.join(emit.GEN_DIR, spec.name + ext)), spec.name
+        assert os.path.exists(os.path.join(emit.GEN_DIR, "run_" + spec.name)), spec.name

@@ -1,0 +1,87 @@
+"""Generated Sessions on the GPU: the code the C++ emitter wrote (prebuilt by tests/build_generated.py) is run
+as its own process, the way a user of the generated header runs it, and its output is compared with the
+reference's expected vectors and with the CPU oracle.
+
+Bars: fp32 networks 1e-5 relative (max |d| / max |ref|); int8 network logits identical, since they are an exact
+int32 accumulator times an fp32 scale."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import models
+import replay
+from oracle import oracle
+from sofie_amd import emit
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def run_session(name, x, tmp_path, out_dtype=np.float32, dat=None, iters=0):
+    exe = os.path.join(emit.GEN_DIR, "run_" + name)
+    if not os.path.exists(exe):
+        raise RuntimeError("%s is missing: run python tests/build_generated.py on the build machine" % exe)
+    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    np.ascontiguousarray(x).tofile(fin)
+    cmd = [exe, os.path.join(emit.GEN_DIR, (dat or name) + ".dat"), fin, fout] + ([str(iters)] if iters else [])
+    print("running", " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=110)
+    assert res.returncode == 0, res.stderr
+    y = np.fromfile(fout, out_dtype)
+    return (y, json.loads(res.stdout)) if iters else y
+
+
+def rel_err(a, b):
+    return float(np.max(np.abs(a.astype(np.float64) - b.astype(np.float64))) / max(float(np.max(np.abs(b))), 1e-30))
+
+
+@pytest.mark.parametrize("name", models.FIXTURES)
+def test_reference_fixture_through_generated_session(name, tmp_path):
+    entry = json.load(open(os.path.join(GOLD, "expected.json")))[name]
+    _, graph = models.fixture_spec(name)
+    x = replay.fixture_input(entry)
+    y = run_session(name, x, tmp_path)
+    want = np.array(entry["expected"], np.float32)
+    assert y.size == want.size
+    assert np.max(np.abs(y - want)) <= 1e-3             # the reference's own tolerance
+    yo = replay.run_graph(graph, {graph["inputs"][0][0]: x}, oracle)
+    assert rel_err(y, yo.reshape(-1)) <= 1e-5
+
+
+def test_mlp_session(tmp_path):
+    _, x = models.mlp_spec()
+    y = run_session("mlp_c1", x, tmp_path)
+    ref = models.mlp_reference(oracle)
+    assert rel_err(y, ref.reshape(-1)) <= 1e-5
+
+
+def test_cnn_f32_session(tmp_path):
+    x = models.cnn_input(8)
+    y = run_session("cnn_f32", x, tmp_path)
+    ref = models.cnn_f32_stages(oracle, x)["y"]
+    assert rel_err(y, ref.reshape(-1)) <= 1e-5
+
+
+def test_int8_cnn_session_is_bit_exact(tmp_path):
+    x = models.cnn_input(8)
+    y = run_session("qcnn", x, tmp_path)
+    ref = models.qcnn_reference(oracle, x)
+    assert np.array_equal(y, ref.reshape(-1))
+    # and it classifies like the float network it was quantized from
+    f = models.cnn_f32_stages(oracle, x)["y"]
+    assert np.array_equal(np.argmax(y.reshape(8, 5), 1), np.argmax(f, 1)) or rel_err(y, f.reshape(-1)) < 0.1
+
+
+def test_int8_cnn_batch_4096_matches_the_oracle_on_a_sample_and_is_batch_invariant(tmp_path):
+    """Full benchmark batch: every image is computed independently of its neighbours, so the first 8 rows
+    equal the batch-8 Session's output, and 16 images spread over the batch equal the oracle."""
+    x = models.cnn_input(4096)
+    y = run_session("qcnn_b4096", x, tmp_path, dat="qcnn").reshape(4096, 5)
+    pick = np.arange(0, 4096, 256)
+    ref = models.qcnn_reference(oracle, x[pick])
+    assert np.array_equal(y[pick], ref)
+    y8 = run_session("qcnn", x[:8], tmp_path).reshape(8, 5)
+    assert np.array_equal(y[:8], y8)

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-import onnx_wire
+from sofie_amd import onnx_wire
 import replay
 from oracle import oracle
 

@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-import onnx_wire
+from sofie_amd import onnx_wire
 import replay
 from oracle import oracle
 
