@@ -153,15 +153,20 @@ int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, cons
                        const int32_t *bias, int zp_y, int act, void *Y, int ldy, int out_kind);
 
 /* int8 2-D convolution with int32 accumulation and fused requantisation.
- * x, y: int8 activations in x_layout / y_layout; w [OC, C/groups, KH, KW] int8 (symmetric,
- * zero-point 0) unpacked ONNX layout; bias [OC] int32 or NULL; scale [OC] fp32.
+ * x, y: int8 activations in x_layout / y_layout. w int8 (symmetric, zero-point 0):
+ * w_layout SOFIE_LAYOUT_NCHW = ONNX [OC, C/groups, KH, KW], SOFIE_LAYOUT_NHWC =
+ * [OC, KH, KW, C/groups] (channels innermost, the order the matrix-core kernel reads).
+ * bias [OC] int32 or NULL; scale [OC] fp32.
  * Padding cells hold zp_x (so that they contribute zero once the caller has folded
- * bias[oc] -= zp_x * sum(w[oc])). out_kind SOFIE_OUT_S8 or SOFIE_OUT_S32. */
+ * bias[oc] -= zp_x * sum(w[oc])). out_kind SOFIE_OUT_S8 or SOFIE_OUT_S32.
+ * The matrix-core kernel takes groups = 1, C % 32 == 0, OC % 64 == 0 with every layout NHWC;
+ * NCHW operands of such a shape are converted through the context's scratch buffer on each
+ * call, every other shape runs a plain one-thread-per-output kernel. */
 int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
-                         const int32_t *bias, const float *scale, void *y, int y_layout,
-                         int N, int C, int H, int W, int OC, int KH, int KW, int pad_h,
-                         int pad_w, int stride_h, int stride_w, int groups, int zp_x,
-                         int zp_y, int act, int out_kind);
+                         int w_layout, const int32_t *bias, const float *scale, void *y,
+                         int y_layout, int N, int C, int H, int W, int OC, int KH, int KW,
+                         int pad_h, int pad_w, int stride_h, int stride_w, int groups,
+                         int zp_x, int zp_y, int act, int out_kind);
 
 /* int8 max pooling, NCHW or NHWC. */
 int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N,

@@ -9,6 +9,7 @@
 
 struct sofie_hip_ctx {
    int device = 0;
+   int num_cus = 256;           // compute units of the device (persistent kernels size their grid by it)
    hipStream_t stream = nullptr;
    bool owns_stream = false;
    hipEvent_t ev_start = nullptr, ev_stop = nullptr;

@@ -1,7 +1,29 @@
 // int8 convolution with int32 accumulation and fused requantisation (QLinearConv semantics).
 //
+// k_qconv_mfma: implicit GEMM on the matrix cores for NHWC activations, weights packed
+// [OC][KH][KW][C], groups = 1, C a multiple of 32 and OC a multiple of 64. The GEMM view is
+// Y[pixel, oc] = sum_k patch[pixel, k] * w[oc, k] with k = (kh, kw, c), so the NHWC output is
+// the row-major GEMM result and shares the GEMM epilogue (requantise, pack four channels per
+// lane, 16-byte row stores through an LDS staging block).
+//   * 512 threads = 8 wavefronts; each wavefront owns MB x NB accumulator tiles of 32 x 32
+//     (v_mfma_i32_32x32x32_i8); a workgroup covers TM = (8/WN)*MB*32 consecutive output pixels
+//     of the linear (n, oh, ow) order times WN*NB*32 output channels.
+//   * Workgroups are persistent: the workgroup's slice of the weights stays in LDS for its
+//     whole life ([oc][K + pad]), and it walks over pixel tiles with a stride of the grid.
+//   * The input of a pixel tile is a contiguous band of rows of the zero-point-padded images
+//     stacked on top of each other ("virtual rows": image n, padded row r -> n*HP + r). The
+//     band is copied once into LDS as [row][padded column][C + pad]; every (kh, kw) tap of
+//     every pixel then reads it from there, so HBM/L2 sees each input byte about once per
+//     tile instead of KH*KW times. Cells outside the image are written as zp_x.
+//   * The band of the NEXT tile is fetched into registers before the MFMA loop of the current
+//     one and written to LDS after its epilogue.
+// The 16-byte pads make the pixel stride and the weight row stride odd multiples of 16 bytes,
+// which keeps the 16-byte-per-lane operand reads of 32 consecutive pixels / channels off the
+// same LDS banks.
+//
 // k_qconv_simple: one thread per output element, any layout / group count / channel count.
 #include "common.h"
+#include "gemm_tile.h"
 
 using namespace sofie;
 
@@ -15,7 +37,7 @@ struct QConvArgs {
    int N, C, H, W, OC, KH, KW, ph, pw, sh, sw, groups;
    int OH, OW, icg, ocg;
    int zpx, zpy, lo, relu;
-   int x_nhwc, y_nhwc;
+   int x_nhwc, y_nhwc, w_ohwi;
 };
 
 template <int OUT>
@@ -48,7 +70,9 @@ __global__ void k_qconv_simple(QConvArgs g)
             if (inside)
                xv = g.x_nhwc ? g.x[(((size_t)n * g.H + ih) * g.W + iw) * g.C + c]
                              : g.x[(((size_t)n * g.C + c) * g.H + ih) * g.W + iw];
-            acc += xv * (int)g.w[(((size_t)oc * g.icg + ic) * g.KH + kh) * g.KW + kw];
+            const int wv = g.w_ohwi ? g.w[(((size_t)oc * g.KH + kh) * g.KW + kw) * g.icg + ic]
+                                    : g.w[(((size_t)oc * g.icg + ic) * g.KH + kh) * g.KW + kw];
+            acc += xv * wv;
          }
       }
    }
@@ -57,9 +81,319 @@ __global__ void k_qconv_simple(QConvArgs g)
    else static_cast<int8_t *>(g.y)[idx] = (int8_t)requant(acc, g.scale[oc], g.zpy, g.lo);
 }
 
+// ------------------------------------------------------------------------------ MFMA path
+// floor(x / d) for 0 <= x < 2^31 as a multiply-high and a shift (shift < 0: d == 1).
+struct FastDiv {
+   unsigned magic;
+   int shift;
+};
+
+FastDiv make_fastdiv(unsigned d)
+{
+   if (d <= 1) return {0u, -1};
+   int s = 0;
+   while ((1u << s) < d) ++s;
+   const unsigned long long num = 1ull << (31 + s);
+   return {(unsigned)((num + d - 1) / d), s - 1};
+}
+
+__device__ __forceinline__ int fdiv(int x, FastDiv f)
+{
+   return f.shift < 0 ? x : (int)(__umulhi((unsigned)x, f.magic) >> f.shift);
+}
+
+struct QConvTileArgs {
+   const int8_t *x;      // NHWC
+   const int8_t *w;      // [OC][KH][KW][C]
+   GemmArgs ep;          // Y, scale, bias, M = N*OH*OW, N = OC, ldy = OC, zp, lo, relu
+   int H, W, C, KH, KW, ph, pw, sh, sw, OH, OW, HP, WP;
+   int K, KS, CS;        // bytes of one weight row, its LDS stride, LDS stride of one pixel
+   int C16, C32;
+   int RL, RP;           // 16-byte chunks per band row; band rows fetched per pass
+   int ntiles;
+   unsigned fill;        // zp_x replicated into four bytes
+   FastDiv dOW, dOH, dHP, dRL, dC16;
+};
+
+template <int MB, int NB, int WN, int PF, int OUT>
+__global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
+{
+   constexpr int WM = 8 / WN;
+   constexpr int TM = WM * MB * 32;
+   constexpr int OCT = WN * NB * 32;
+   extern __shared__ __align__(16) unsigned char smem[];
+   unsigned char *const s_w = smem;                    // [OCT][KS]
+   unsigned char *const s_p = smem + OCT * a.KS;       // band [rows][WP][CS], later the epilogue staging
+
+   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int wn = wave % WN, wm = wave / WN;
+   const int half = lane >> 5, l32 = lane & 31;
+   const int nob = a.ep.N / OCT;
+   const int ob = blockIdx.x % nob;
+   const int wg = blockIdx.x / nob, nwg = gridDim.x / nob;
+   const int mtot = a.ep.M;
+
+   // ---- weights of this channel block: resident for the life of the workgroup
+   {
+      const int K16 = a.K >> 4;
+      const int8_t *wsrc = a.w + (size_t)ob * OCT * a.K;
+      for (int r = wave; r < OCT; r += 8)
+         for (int c = lane; c < K16; c += 64)
+            *reinterpret_cast<v4i *>(s_w + r * a.KS + c * 16) =
+               *reinterpret_cast<const v4i *>(wsrc + (size_t)r * a.K + c * 16);
+   }
+
+   // ---- band loader: thread -> (row of the pass, 16-byte chunk of the row)
+   const int rsub = fdiv(tid, a.dRL);
+   const int col = tid - rsub * a.RL;
+   const int wp = fdiv(col, a.dC16);
+   const int c16 = col - wp * a.C16;
+   const int iw = wp - a.pw;
+   const bool col_active = rsub < a.RP;
+   const bool col_inside = iw >= 0 && iw < a.W;
+   const int src_col = iw * a.C + c16 * 16;
+   const int lds_col = wp * a.CS + c16 * 16;
+   const int row_bytes = a.WP * a.CS;
+   const v4i fillv = {(int)a.fill, (int)a.fill, (int)a.fill, (int)a.fill};
+
+   struct Band { int vr_lo, rows; };
+   auto band_of = [&](int t) {
+      const int m0 = t * TM;
+      const int mlast = (m0 + TM < mtot ? m0 + TM : mtot) - 1;
+      const int R0 = fdiv(m0, a.dOW), R1 = fdiv(mlast, a.dOW);
+      const int n0 = fdiv(R0, a.dOH), n1 = fdiv(R1, a.dOH);
+      Band b;
+      b.vr_lo = n0 * a.HP + (R0 - n0 * a.OH) * a.sh;
+      b.rows = n1 * a.HP + (R1 - n1 * a.OH) * a.sh + a.KH - b.vr_lo;
+      return b;
+   };
+   v4i pre[PF];
+   auto fetch = [&](Band b) {
+#pragma unroll
+      for (int i = 0; i < PF; ++i) {
+         const int r = i * a.RP + rsub;
+         const int vr = b.vr_lo + r;
+         const int n = fdiv(vr, a.dHP);
+         const int ih = vr - n * a.HP - a.ph;
+         const bool inside = col_active && col_inside && r < b.rows && ih >= 0 && ih < a.H;
+         pre[i] = fillv;
+         if (inside)
+            pre[i] = *reinterpret_cast<const v4i *>(a.x + ((size_t)(n * a.H + ih) * a.W) * a.C + src_col);
+      }
+   };
+   auto stash = [&](Band b) {
+#pragma unroll
+      for (int i = 0; i < PF; ++i) {
+         const int r = i * a.RP + rsub;
+         if (col_active && r < b.rows) *reinterpret_cast<v4i *>(s_p + r * row_bytes + lds_col) = pre[i];
+      }
+   };
+
+   int t = wg;
+   Band cur = {0, 0};
+   if (t < a.ntiles) {
+      cur = band_of(t);
+      fetch(cur);
+   }
+   int b_off[NB];
+#pragma unroll
+   for (int i = 0; i < NB; ++i) b_off[i] = ((wn * NB + i) * 32 + l32) * a.KS + half * 16;
+   const int tap_step = a.CS - a.C32 * 32;              // from the end of one tap's channels to the next tap
+   const int row_step = (a.WP - a.KW) * a.CS;           // from the end of one kernel row to the next
+   const int nsteps = a.KH * a.KW * a.C32;
+
+   for (; t < a.ntiles; t += nwg) {
+      stash(cur);
+      __syncthreads();
+      const int m0 = t * TM;
+      const int vr_lo = cur.vr_lo;
+      const int tn = t + nwg;
+      if (tn < a.ntiles) {
+         cur = band_of(tn);
+         fetch(cur);
+      }
+
+      int a_off[MB];
+#pragma unroll
+      for (int j = 0; j < MB; ++j) {
+         int m = m0 + (wm * MB + j) * 32 + l32;
+         m = m < mtot ? m : mtot - 1;
+         const int R = fdiv(m, a.dOW);
+         const int ow = m - R * a.OW;
+         const int n = fdiv(R, a.dOH);
+         const int v = n * a.HP + (R - n * a.OH) * a.sh - vr_lo;
+         a_off[j] = (v * a.WP + ow * a.sw) * a.CS + half * 16;
+      }
+
+      v16i acc[NB][MB];
+#pragma unroll
+      for (int i = 0; i < NB; ++i)
+#pragma unroll
+         for (int j = 0; j < MB; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+      // K loop over (kh, kw, 32-channel block); fragments of step s+1 are read while the
+      // matrix instructions of step s issue
+      v4i fa[2][MB], fb[2][NB];
+      int ka = 0, kb = 0, c32 = 0, kw = 0;
+#pragma unroll
+      for (int j = 0; j < MB; ++j) fa[0][j] = *reinterpret_cast<const v4i *>(s_p + a_off[j]);
+#pragma unroll
+      for (int i = 0; i < NB; ++i) fb[0][i] = *reinterpret_cast<const v4i *>(s_w + b_off[i]);
+      for (int s = 0; s < nsteps; s += 2) {
+#pragma unroll
+         for (int u = 0; u < 2; ++u) {
+            // advance to the next step's offsets
+            ka += 32; kb += 32;
+            if (++c32 == a.C32) {
+               c32 = 0; ka += tap_step;
+               if (++kw == a.KW) { kw = 0; ka += row_step; }
+            }
+            const bool more = s + u + 1 < nsteps;
+            if (more) {
+#pragma unroll
+               for (int j = 0; j < MB; ++j) fa[u ^ 1][j] = *reinterpret_cast<const v4i *>(s_p + a_off[j] + ka);
+#pragma unroll
+               for (int i = 0; i < NB; ++i) fb[u ^ 1][i] = *reinterpret_cast<const v4i *>(s_w + b_off[i] + kb);
+            }
+            if (s + u < nsteps) {
+#pragma unroll
+               for (int i = 0; i < NB; ++i)
+#pragma unroll
+                  for (int j = 0; j < MB; ++j) acc[i][j] = MmaI8::mma(fb[u][i], fa[u][j], acc[i][j]);
+            }
+         }
+      }
+      __syncthreads();   // every wavefront is done with the band: its memory becomes the staging block
+      tile_epilogue<MmaI8, NB, MB, OUT, 8>(a.ep, acc, s_p, tid, m0 + wm * MB * 32, ob * OCT, wn, OCT);
+   }
+}
+
+size_t epilogue_bytes(int oct, int wn_cols, int esz) { return (size_t)8 * 32 * (wn_cols * esz + 16) + (size_t)2 * oct * 4; }
+
+// Launches the MFMA kernel if the problem fits it; *done tells whether it did.
+template <int OUT>
+int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
+{
+   *done = false;
+   constexpr int ESZ = OutSize<OUT>::value;
+   if (g.groups != 1 || g.C % 32 != 0 || g.OC % 64 != 0 || !g.x_nhwc || !g.y_nhwc || !g.w_ohwi) return SOFIE_HIP_OK;
+   if (!aligned16(g.x) || !aligned16(g.w) || !aligned16(g.y)) return SOFIE_HIP_OK;
+   const long long mtot = (long long)g.N * g.OH * g.OW;
+   const int HP = g.H + 2 * g.ph, WP = g.W + 2 * g.pw;
+   if (mtot >= (1ll << 31) - 1024 || (long long)g.N * HP >= (1ll << 31) - 4096) return SOFIE_HIP_OK;
+   if ((size_t)g.N * g.H * g.W * g.C >= ((size_t)1 << 40)) return SOFIE_HIP_OK;
+   const int WN = g.OC % 128 == 0 ? 2 : 1;
+   const int OCT = WN * 64;
+   const int TM = (8 / WN) * 64;
+   QConvTileArgs a{};
+   a.x = g.x; a.w = g.w;
+   a.ep.Y = g.y; a.ep.scale = g.scale; a.ep.bias = g.bias;
+   a.ep.M = (int)mtot; a.ep.N = g.OC; a.ep.ldy = g.OC;
+   a.ep.zp = g.zpy; a.ep.lo = g.lo; a.ep.relu = g.relu; a.ep.s = 1.0f;
+   a.ep.vec_store = 1;   // OC % 64 == 0 and y 16-byte aligned
+   a.H = g.H; a.W = g.W; a.C = g.C; a.KH = g.KH; a.KW = g.KW; a.ph = g.ph; a.pw = g.pw; a.sh = g.sh; a.sw = g.sw;
+   a.OH = g.OH; a.OW = g.OW; a.HP = HP; a.WP = WP;
+   a.K = g.KH * g.KW * g.C;
+   a.KS = ((a.K / 16) % 2 == 0) ? a.K + 16 : a.K;
+   a.CS = ((g.C / 16) % 2 == 0) ? g.C + 16 : g.C;
+   a.C16 = g.C / 16; a.C32 = g.C / 32;
+   a.RL = WP * a.C16;
+   if (a.RL > 512) return SOFIE_HIP_OK;
+   a.RP = 512 / a.RL;
+   a.ntiles = (int)((mtot + TM - 1) / TM);
+   a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
+   a.dOW = make_fastdiv(g.OW); a.dOH = make_fastdiv(g.OH); a.dHP = make_fastdiv(HP);
+   a.dRL = make_fastdiv(a.RL); a.dC16 = make_fastdiv(a.C16);
+   // most rows a band can have: the output rows a tile touches, the image boundaries it can cross
+   // (each adds the rows between the last window of one image and the first of the next) and KH - 1
+   const int out_rows = (TM - 1) / g.OW + 2;
+   int gap = HP - g.OH * g.sh;
+   if (gap < 0) gap = 0;
+   int crossings = (out_rows - 1) / g.OH + 1;
+   if (crossings > g.N - 1) crossings = g.N - 1;
+   const long long rows_max = (long long)(out_rows - 1) * g.sh + (long long)crossings * gap + g.KH;
+   const int passes = (int)((rows_max + a.RP - 1) / a.RP);
+   if (passes > 12) return SOFIE_HIP_OK;
+   const size_t band = (size_t)rows_max * WP * a.CS;
+   const size_t epi = epilogue_bytes(OCT, 64, ESZ);
+   const size_t lds = (size_t)OCT * a.KS + (band > epi ? band : epi);
+   if (lds > 160 * 1024) return SOFIE_HIP_OK;
+   if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
+
+   const int nob = g.OC / OCT;
+   int per = ctx->num_cus / nob;
+   if (per < 1) per = 1;
+   if (per > a.ntiles) per = a.ntiles;
+   const dim3 grid((unsigned)(per * nob)), block(512);
+#define SOFIE_QCONV_LAUNCH(WN_, PF_)                                                                          \
+   do {                                                                                                       \
+      auto kern = k_qconv_mfma<2, 2, WN_, PF_, OUT>;                                                          \
+      SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));         \
+      hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                             \
+   } while (0)
+   if (WN == 2) {
+      if (passes <= 4) SOFIE_QCONV_LAUNCH(2, 4);
+      else if (passes <= 8) SOFIE_QCONV_LAUNCH(2, 8);
+      else SOFIE_QCONV_LAUNCH(2, 12);
+   } else {
+      if (passes <= 4) SOFIE_QCONV_LAUNCH(1, 4);
+      else if (passes <= 8) SOFIE_QCONV_LAUNCH(1, 8);
+      else SOFIE_QCONV_LAUNCH(1, 12);
+   }
+#undef SOFIE_QCONV_LAUNCH
+   *done = true;
+   return check_launch(ctx, "k_qconv_mfma");
+}
+
+template <int OUT>
+int run(sofie_hip_ctx *ctx, QConvArgs g)
+{
+   constexpr int ESZ = OutSize<OUT>::value;
+   // MFMA path: activations NHWC, weights [OC][KH][KW][C]; other layouts are converted through the
+   // context's scratch buffer when the shape is one the MFMA kernel takes
+   const bool shape_ok = g.groups == 1 && g.C % 32 == 0 && g.OC % 64 == 0 && g.N <= 65535 && ESZ == 1;
+   if (shape_ok && (!g.x_nhwc || !g.y_nhwc || !g.w_ohwi)) {
+      const size_t xb = g.x_nhwc ? 0 : (size_t)g.N * g.C * g.H * g.W;
+      const size_t yb = g.y_nhwc ? 0 : (size_t)g.N * g.OC * g.OH * g.OW;
+      const size_t wb = g.w_ohwi ? 0 : (size_t)g.OC * g.C * g.KH * g.KW;
+      auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+      void *ws = nullptr;
+      if (int rc = workspace(ctx, up(xb) + up(yb) + up(wb), &ws)) return rc;
+      int8_t *xs = static_cast<int8_t *>(ws), *ys = xs + up(xb), *wsb = ys + up(yb);
+      QConvArgs h = g;
+      if (xb) {
+         if (int rc = relayout_s8(ctx, g.x, xs, g.N, g.C, g.H, g.W, SOFIE_LAYOUT_NCHW, SOFIE_LAYOUT_NHWC)) return rc;
+         h.x = xs; h.x_nhwc = 1;
+      }
+      if (wb) {
+         if (int rc = relayout_s8(ctx, g.w, wsb, g.OC, g.C, g.KH, g.KW, SOFIE_LAYOUT_NCHW, SOFIE_LAYOUT_NHWC)) return rc;
+         h.w = wsb; h.w_ohwi = 1;
+      }
+      if (yb) { h.y = ys; h.y_nhwc = 1; }
+      bool done = false;
+      if (int rc = launch_mfma<OUT>(ctx, h, &done)) return rc;
+      if (done) {
+         if (yb) return relayout_s8(ctx, ys, static_cast<int8_t *>(g.y), g.N, g.OC, g.OH, g.OW, SOFIE_LAYOUT_NHWC,
+                                    SOFIE_LAYOUT_NCHW);
+         return SOFIE_HIP_OK;
+      }
+   } else {
+      bool done = false;
+      if (int rc = launch_mfma<OUT>(ctx, g, &done)) return rc;
+      if (done) return SOFIE_HIP_OK;
+   }
+   const size_t total = (size_t)g.N * g.OC * g.OH * g.OW;
+   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+   hipLaunchKernelGGL(k_qconv_simple<OUT>, grid, block, 0, ctx->stream, g);
+   return check_launch(ctx, "k_qconv_simple");
+}
+
 }  // namespace
 
-extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
+extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w, int w_layout,
                                     const int32_t *bias, const float *scale, void *y, int y_layout, int N, int C,
                                     int H, int W, int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,
                                     int stride_w, int groups, int zp_x, int zp_y, int act, int out_kind)
@@ -70,7 +404,8 @@ extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_l
    SOFIE_REQUIRE(ctx, groups > 0 && C % groups == 0 && OC % groups == 0, "channels not divisible by groups");
    SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
    SOFIE_REQUIRE(ctx, (x_layout == SOFIE_LAYOUT_NCHW || x_layout == SOFIE_LAYOUT_NHWC) &&
-                         (y_layout == SOFIE_LAYOUT_NCHW || y_layout == SOFIE_LAYOUT_NHWC), "unknown layout");
+                         (y_layout == SOFIE_LAYOUT_NCHW || y_layout == SOFIE_LAYOUT_NHWC) &&
+                         (w_layout == SOFIE_LAYOUT_NCHW || w_layout == SOFIE_LAYOUT_NHWC), "unknown layout");
    SOFIE_REQUIRE(ctx, out_kind == SOFIE_OUT_S8 || out_kind == SOFIE_OUT_S32, "output kind must be S8 or S32");
    SOFIE_REQUIRE(ctx, zp_x >= -128 && zp_x <= 127 && zp_y >= -128 && zp_y <= 127, "zero-point out of int8 range");
    SOFIE_REQUIRE(ctx, H + 2 * pad_h >= KH && W + 2 * pad_w >= KW, "kernel larger than padded input");
@@ -88,11 +423,10 @@ extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_l
    g.zpx = zp_x; g.zpy = zp_y;
    g.relu = act == SOFIE_ACT_RELU;
    g.lo = (g.relu && zp_y > -128) ? zp_y : -128;
-   g.x_nhwc = x_layout == SOFIE_LAYOUT_NHWC;
-   g.y_nhwc = y_layout == SOFIE_LAYOUT_NHWC;
-   const size_t total = (size_t)N * OC * g.OH * g.OW;
-   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
-   if (out_kind == SOFIE_OUT_S32) hipLaunchKernelGGL(k_qconv_simple<SOFIE_OUT_S32>, grid, block, 0, ctx->stream, g);
-   else hipLaunchKernelGGL(k_qconv_simple<SOFIE_OUT_S8>, grid, block, 0, ctx->stream, g);
-   return check_launch(ctx, "k_qconv_simple");
+   // with one channel (one output channel) both activation layouts are the same bytes
+   g.x_nhwc = x_layout == SOFIE_LAYOUT_NHWC || C == 1;
+   g.y_nhwc = y_layout == SOFIE_LAYOUT_NHWC || OC == 1;
+   g.w_ohwi = w_layout == SOFIE_LAYOUT_NHWC || g.icg == 1 || KH * KW == 1;
+   if (out_kind == SOFIE_OUT_S32) return run<SOFIE_OUT_S32>(ctx, g);
+   return run<SOFIE_OUT_S8>(ctx, g);
 }

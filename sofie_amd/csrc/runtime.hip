@@ -60,6 +60,11 @@ int sofie_hip_create(sofie_hip_ctx **out, int device, void *stream)
    if (hipSetDevice(device) != hipSuccess) return SOFIE_HIP_EHIP;
    sofie_hip_ctx *ctx = new sofie_hip_ctx();
    ctx->device = device;
+   {
+      int cus = 0;
+      if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus > 0)
+         ctx->num_cus = cus;
+   }
    if (stream) {
       ctx->stream = static_cast<hipStream_t>(stream);
    } else {

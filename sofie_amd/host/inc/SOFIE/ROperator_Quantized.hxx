@@ -368,7 +368,7 @@ public:
       fGeom.SymmetricPads(ph, pw);
       std::stringstream out;
       out << "\n//----  operator QLinearConv op_" << OpName << "\n";
-      out << SP << "Check(sofie_hip_qconv2d_s8(fCtx, tensor_" << fNX << ", SOFIE_LAYOUT_NCHW, tensor_" << fNW << ", "
+      out << SP << "Check(sofie_hip_qconv2d_s8(fCtx, tensor_" << fNX << ", SOFIE_LAYOUT_NCHW, tensor_" << fNW << ", SOFIE_LAYOUT_NCHW, "
           << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", tensor_" << fNScale << ", tensor_" << fNY
           << ", SOFIE_LAYOUT_NCHW, " << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", "
           << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3] << ", " << ph << ", " << pw << ", " << fGeom.strides[0] << ", "

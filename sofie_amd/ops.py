@@ -132,7 +132,10 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
     ctx = ctx or default_context()
     xd, wd, bd = ctx.dev(x, torch.float32), ctx.dev(w, torch.float32), ctx.dev(bias, torch.float32)
     N, Cc, H, W = xd.shape
-    OC, _, kh, kw = wd.shape
+    if w_layout == L.LAYOUT_NCHW:
+        OC, _, kh, kw = wd.shape
+    else:
+        OC, kh, kw, _ = wd.shape
     OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1], *dilations)
     y = ctx.empty((N, OC, OH, OW), torch.float32)
     ctx.check(ctx.lib.sofie_hip_conv2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, H, W,
@@ -226,9 +229,10 @@ def fold_zero_point_conv(w, bias, zpx):
 
 
 def qconv2d_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, zpy=0, relu=False,
-               x_layout=L.LAYOUT_NCHW, y_layout=L.LAYOUT_NCHW, out=L.OUT_S8, ctx=None):
-    """QLinearConv. x in x_layout, w [OC, C/g, KH, KW]; bias is the ONNX int32 bias (the input
-    zero-point is folded here, host side, as a Session constructor would do once)."""
+               x_layout=L.LAYOUT_NCHW, y_layout=L.LAYOUT_NCHW, out=L.OUT_S8, ctx=None, w_layout=L.LAYOUT_NCHW):
+    """QLinearConv. x in x_layout, w [OC, C/g, KH, KW] (or [OC, KH, KW, C/g] with w_layout NHWC); bias is
+    the ONNX int32 bias (the input zero-point is folded here, host side, as a Session constructor would
+    do once)."""
     ctx = ctx or default_context()
     if zpx != 0:
         bias = fold_zero_point_conv(w, bias, zpx)
@@ -237,12 +241,15 @@ def qconv2d_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zp
         N, Cc, H, W = xd.shape
     else:
         N, H, W, Cc = xd.shape
-    OC, _, kh, kw = wd.shape
+    if w_layout == L.LAYOUT_NCHW:
+        OC, _, kh, kw = wd.shape
+    else:
+        OC, kh, kw, _ = wd.shape
     OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1])
     shape = (N, OC, OH, OW) if y_layout == L.LAYOUT_NCHW else (N, OH, OW, OC)
     y = ctx.empty(shape, _OUT_DTYPE[out])
     sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
-    ctx.check(ctx.lib.sofie_hip_qconv2d_s8(ctx.h, ctx.ptr(xd), x_layout, ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(sd),
+    ctx.check(ctx.lib.sofie_hip_qconv2d_s8(ctx.h, ctx.ptr(xd), x_layout, ctx.ptr(wd), w_layout, ctx.ptr(bd), ctx.ptr(sd),
                                            ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, pads[0], pads[1],
                                            strides[0], strides[1], groups, int(zpx), int(zpy),
                                            L.ACT_RELU if relu else L.ACT_NONE, out))

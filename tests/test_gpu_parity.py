@@ -277,6 +277,44 @@ def test_qconv2d_s8(ops, cfg):
     assert np.array_equal(y0, oracle.qconv2d_s8(x, w, scale, None, cfg["p"], cfg["s"], cfg["g"], 0, 7, False))
 
 
+@pytest.mark.parametrize("cfg", [
+    # the matrix-core kernel's shapes: bands that cross image boundaries, a partial last tile, strides,
+    # 1x1 / 5x5 / non-square kernels, no padding, wide padding, one image smaller than a tile
+    dict(N=3, C=32, H=20, W=20, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=7, C=64, H=10, W=10, OC=128, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=2, C=64, H=56, W=56, OC=128, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=5, C=32, H=9, W=13, OC=64, k=(3, 3), p=(0, 0), s=(1, 1)),
+    dict(N=4, C=64, H=15, W=17, OC=192, k=(3, 3), p=(1, 1), s=(2, 2)),
+    dict(N=9, C=96, H=6, W=5, OC=64, k=(1, 1), p=(0, 0), s=(1, 1)),
+    dict(N=2, C=32, H=12, W=12, OC=128, k=(5, 5), p=(2, 2), s=(1, 1)),
+    dict(N=3, C=32, H=11, W=8, OC=64, k=(3, 1), p=(1, 0), s=(2, 1)),
+    dict(N=1, C=32, H=4, W=4, OC=64, k=(3, 3), p=(2, 2), s=(1, 1)),
+    dict(N=300, C=32, H=3, W=3, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
+])
+def test_qconv2d_s8_matrix_core_path(ops, cfg):
+    """NHWC activations and [OC,KH,KW,C] weights straight into the MFMA kernel; NCHW operands of the same
+    shape reach it through the layout conversion. Both must equal the oracle bit for bit."""
+    from sofie_amd import lib as L
+    r = rng(500 + cfg["C"] + cfg["OC"] + cfg["H"])
+    x = r.integers(-128, 128, (cfg["N"], cfg["C"], cfg["H"], cfg["W"])).astype(np.int8)
+    w = r.integers(-127, 128, (cfg["OC"], cfg["C"]) + cfg["k"]).astype(np.int8)
+    K = cfg["C"] * cfg["k"][0] * cfg["k"][1]
+    scale = (r.uniform(20, 60, cfg["OC"]) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    bias = r.integers(-3000, 3000, cfg["OC"]).astype(np.int32)
+    xh = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    wh = np.ascontiguousarray(w.transpose(0, 2, 3, 1))
+    for zpx, zpy, relu in ((-128, -128, True), (3, 11, False)):
+        ref = oracle.qconv2d_s8(x, w, scale, bias, cfg["p"], cfg["s"], 1, zpx, zpy, relu)
+        yh = ops.qconv2d_s8(xh, wh, scale, bias, cfg["p"], cfg["s"], 1, zpx, zpy, relu, x_layout=L.LAYOUT_NHWC,
+                            y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+        assert np.array_equal(yh.transpose(0, 3, 1, 2), ref)
+        y = ops.qconv2d_s8(x, w, scale, bias, cfg["p"], cfg["s"], 1, zpx, zpy, relu)
+        assert np.array_equal(y, ref)
+    acc = ops.qconv2d_s8(xh, wh, None, None, cfg["p"], cfg["s"], 1, 5, x_layout=L.LAYOUT_NHWC, y_layout=L.LAYOUT_NHWC,
+                         w_layout=L.LAYOUT_NHWC, out=L.OUT_S32)
+    assert np.array_equal(acc.transpose(0, 3, 1, 2), oracle.iconv2d_s8(x, w, cfg["p"], cfg["s"], 1, 5))
+
+
 # --------------------------------------------------------------------------- fp8
 def fp8_operands(r, M, N, K, transB):
     a = r.standard_normal((M, K)).astype(np.float32)
