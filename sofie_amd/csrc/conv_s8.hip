@@ -122,8 +122,12 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    constexpr int TM = WM * MB * 32;
    constexpr int OCT = WN * NB * 32;
    extern __shared__ __align__(16) unsigned char smem[];
-   unsigned char *const s_w = smem;                    // [OCT][KS]
-   unsigned char *const s_p = smem + OCT * a.KS;       // band [rows][WP][CS], later the epilogue staging
+   constexpr int WB = EpilogueStaging<NB, OUT>::WAVE_BYTES;
+   unsigned char *const s_w = smem;                                        // [OCT][KS]
+   float *const s_scale = reinterpret_cast<float *>(smem + OCT * a.KS);    // [OCT]
+   int *const s_bias = reinterpret_cast<int *>(s_scale + OCT);             // [OCT]
+   unsigned char *const s_stg = reinterpret_cast<unsigned char *>(s_bias + OCT);   // [8][WB] epilogue staging
+   unsigned char *const s_p = s_stg + 8 * WB;                              // band [rows][WP][CS]
 
    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
    const int wn = wave % WN, wm = wave / WN;
@@ -142,6 +146,9 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
             *reinterpret_cast<v4i *>(s_w + r * a.KS + c * 16) =
                *reinterpret_cast<const v4i *>(wsrc + (size_t)r * a.K + c * 16);
    }
+
+   stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
+   const bool plain = OUT == SOFIE_OUT_S8 && a.ep.zp == -128 && a.ep.lo == -128;
 
    // ---- band loader: thread -> (row of the pass, 16-byte chunk of the row)
    const int rsub = fdiv(tid, a.dRL);
@@ -176,9 +183,11 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          const int n = fdiv(vr, a.dHP);
          const int ih = vr - n * a.HP - a.ph;
          const bool inside = col_active && col_inside && r < b.rows && ih >= 0 && ih < a.H;
-         pre[i] = fillv;
-         if (inside)
-            pre[i] = *reinterpret_cast<const v4i *>(a.x + ((size_t)(n * a.H + ih) * a.W) * a.C + src_col);
+         // the load is unconditional (clamped to the first pixel when the cell is outside) so that
+         // all of a pass's loads are in flight together; the value is selected afterwards
+         const size_t off = inside ? ((size_t)(n * a.H + ih) * a.W) * a.C + src_col : 0;
+         const v4i v = *reinterpret_cast<const v4i *>(a.x + off);
+         pre[i] = inside ? v : fillv;
       }
    };
    auto stash = [&](Band b) {
@@ -202,9 +211,18 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    const int row_step = (a.WP - a.KW) * a.CS;           // from the end of one kernel row to the next
    const int nsteps = a.KH * a.KW * a.C32;
 
+#ifdef ABL_TIMING
+   long long tm[6] = {0, 0, 0, 0, 0, 0};
+   long long t0 = clock64(), t1;
+#define TICK(i) do { t1 = clock64(); tm[i] += t1 - t0; t0 = t1; } while (0)
+#else
+#define TICK(i)
+#endif
    for (; t < a.ntiles; t += nwg) {
+      TICK(5);
       stash(cur);
       __syncthreads();
+      TICK(0);
       const int m0 = t * TM;
       const int vr_lo = cur.vr_lo;
       const int tn = t + nwg;
@@ -232,6 +250,7 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          for (int j = 0; j < MB; ++j)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+      TICK(1);
 
       // K loop over (kh, kw, 32-channel block); fragments of step s+1 are read while the
       // matrix instructions of step s issue
@@ -257,7 +276,12 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 #pragma unroll
                for (int i = 0; i < NB; ++i) fb[u ^ 1][i] = *reinterpret_cast<const v4i *>(s_w + b_off[i] + kb);
             }
-            if (s + u < nsteps) {
+#ifndef ABL_NO_MMA
+            if (s + u < nsteps)
+#else
+            if (s + u < nsteps && a.ph == 77)
+#endif
+            {
 #pragma unroll
                for (int i = 0; i < NB; ++i)
 #pragma unroll
@@ -265,12 +289,29 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
             }
          }
       }
+      TICK(2);
       __syncthreads();   // every wavefront is done with the band: its memory becomes the staging block
-      tile_epilogue<MmaI8, NB, MB, OUT, 8>(a.ep, acc, s_p, tid, m0 + wm * MB * 32, ob * OCT, wn, OCT);
+      TICK(3);
+#ifdef ABL_NO_EPI
+      if (acc[0][0][0] == 0x12345 || a.ph == 77)
+#endif
+      if (plain)
+         tile_epilogue_wave<MmaI8, NB, MB, OUT, true>(a.ep, acc, s_stg + wave * WB, s_scale + wn * NB * 32,
+                                                      s_bias + wn * NB * 32, lane, m0 + wm * MB * 32,
+                                                      ob * OCT + wn * NB * 32);
+      else
+         tile_epilogue_wave<MmaI8, NB, MB, OUT, false>(a.ep, acc, s_stg + wave * WB, s_scale + wn * NB * 32,
+                                                       s_bias + wn * NB * 32, lane, m0 + wm * MB * 32,
+                                                       ob * OCT + wn * NB * 32);
+      TICK(4);
    }
+#ifdef ABL_TIMING
+   if (blockIdx.x == 3 && (tid & 63) == 0) {
+      long long *d = (long long *)a.ep.A + (tid >> 6) * 8;
+      for (int i = 0; i < 6; ++i) d[i] = tm[i];
+   }
+#endif
 }
-
-size_t epilogue_bytes(int oct, int wn_cols, int esz) { return (size_t)8 * 32 * (wn_cols * esz + 16) + (size_t)2 * oct * 4; }
 
 // Launches the MFMA kernel if the problem fits it; *done tells whether it did.
 template <int OUT>
@@ -289,6 +330,11 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const int TM = (8 / WN) * 64;
    QConvTileArgs a{};
    a.x = g.x; a.w = g.w;
+#ifdef ABL_TIMING
+   static long long *dbg = nullptr;
+   if (!dbg) hipMalloc(&dbg, 512);
+   a.ep.A = (const uint8_t *)dbg;
+#endif
    a.ep.Y = g.y; a.ep.scale = g.scale; a.ep.bias = g.bias;
    a.ep.M = (int)mtot; a.ep.N = g.OC; a.ep.ldy = g.OC;
    a.ep.zp = g.zpy; a.ep.lo = g.lo; a.ep.relu = g.relu; a.ep.s = 1.0f;
@@ -317,8 +363,7 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const int passes = (int)((rows_max + a.RP - 1) / a.RP);
    if (passes > 12) return SOFIE_HIP_OK;
    const size_t band = (size_t)rows_max * WP * a.CS;
-   const size_t epi = epilogue_bytes(OCT, 64, ESZ);
-   const size_t lds = (size_t)OCT * a.KS + (band > epi ? band : epi);
+   const size_t lds = (size_t)OCT * a.KS + (size_t)OCT * 8 + (size_t)8 * EpilogueStaging<2, OUT>::WAVE_BYTES + band;
    if (lds > 160 * 1024) return SOFIE_HIP_OK;
    if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
 
@@ -344,6 +389,18 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
       else SOFIE_QCONV_LAUNCH(1, 12);
    }
 #undef SOFIE_QCONV_LAUNCH
+#ifdef ABL_TIMING
+   {
+      static int calls = 0;
+      if (++calls % 23 == 0) {
+         hipDeviceSynchronize();
+         long long h[64];
+         hipMemcpy(h, dbg, sizeof(h), hipMemcpyDeviceToHost);
+         for (int w = 0; w < 8; w += 7)
+            printf("wave %d: stash+bar %lld  fetch+aoff %lld  kloop %lld  bar %lld  epi %lld  looptop %lld\n", w, h[w*8+0], h[w*8+1], h[w*8+2], h[w*8+3], h[w*8+4], h[w*8+5]);
+      }
+   }
+#endif
    *done = true;
    return check_launch(ctx, "k_qconv_mfma");
 }

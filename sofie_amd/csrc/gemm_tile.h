@@ -87,41 +87,70 @@ __device__ __forceinline__ unsigned epilogue_value(const GemmArgs &g, float sc, 
 // Epilogue shared by the tiled kernels. Each wavefront owns TI x TJ accumulator tiles
 // (rows = output columns n, columns = output rows m). Per pass j it converts TI tiles, packs
 // four consecutive n of one m into a 4*esize store into its private LDS staging block
-// [32 m][TI*32 n], then the wavefront writes the block out as 16-byte row segments.
-// smem is reused: all waves must have finished reading operand stages before the call.
-//   m_wave: first output row of this wavefront; n0: first output column of the workgroup;
-//   wn: index of the wavefront's column block; BN: columns of the workgroup tile.
-template <class Mma, int TI, int TJ, int OUT, int NWAVES>
-__device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ], unsigned char *smem,
-                                              int tid, int m_wave, int n0, int wn, int BN)
+// [32 m][TI*32 n], then writes the block out as 16-byte row segments. The staging block is
+// private to the wavefront and LDS operations of one wavefront complete in order, so no
+// workgroup barrier is needed between the passes.
+//   stg: this wavefront's staging block, 32 * (TI*32*esize + 16) bytes;
+//   s_scale, s_bias: per-column scale and bias bits in LDS, already pointing at the
+//     wavefront's first column, filled and made visible by the caller;
+//   m_wave, n_wave: first output row and column of this wavefront.
+// PLAIN: int8 output with zero-point -128 and lower clamp -128 (the saturating byte
+// conversion does the clamping, two instructions per element fewer).
+template <int TI, int OUT> struct EpilogueStaging {
+   static constexpr int ESZ = OutSize<OUT>::value;
+   static constexpr int SROW = TI * 32 * ESZ + 16;   // staging row stride in bytes
+   static constexpr int WAVE_BYTES = 32 * SROW;
+};
+
+template <class Mma, int TI, int TJ, int OUT, bool PLAIN>
+__device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ],
+                                                   unsigned char *stg, const float *s_scale, const int *s_bias,
+                                                   int lane, int m_wave, int n_wave)
 {
    constexpr int ESZ = OutSize<OUT>::value;
    constexpr bool IS_INT = __is_same(typename Mma::Acc, v16i);
    constexpr int WN = TI * 32;                       // output columns of one wavefront
-   constexpr int SROW = WN * ESZ + 16;               // staging row stride in bytes
+   constexpr int SROW = EpilogueStaging<TI, OUT>::SROW;
    constexpr int CR = WN * ESZ / 16;                 // 16-byte chunks per staging row
-   const int lane = tid & 63, wave = tid >> 6;
-   unsigned char *stg = smem + wave * (32 * SROW);
-   float *s_scale = reinterpret_cast<float *>(smem + NWAVES * 32 * SROW);   // [BN] per-column scale
-   int *s_bias = reinterpret_cast<int *>(s_scale + BN);                     // [BN] per-column bias bits
-   if (tid < BN) {
-      const int n = n0 + tid;
-      s_scale[tid] = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
-      s_bias[tid] = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
-   }
-   __syncthreads();
+   constexpr int NG = TI * 4;                        // groups of four columns per lane and pass
    const int m_local = lane & 31;
    const int nq = (lane >> 5) * 4;
+   const float zpo = (float)(g.zp + 128), lof = (float)(g.lo + 128);
 #pragma unroll
    for (int j = 0; j < TJ; ++j) {
+      // scale and bias of group gi+1 are read while group gi is converted
+      v4f sc_next = *reinterpret_cast<const v4f *>(s_scale + nq);
+      v4i bi_next = *reinterpret_cast<const v4i *>(s_bias + nq);
 #pragma unroll
-      for (int i = 0; i < TI; ++i) {
+      for (int gi = 0; gi < NG; ++gi) {
+         const int i = gi >> 2, q = gi & 3;
+         const int nl = i * 32 + q * 8 + nq;
+         const v4f sc = sc_next;
+         const v4i bi = bi_next;
+         if (gi + 1 < NG) {
+            const int nn = ((gi + 1) >> 2) * 32 + ((gi + 1) & 3) * 8 + nq;
+            sc_next = *reinterpret_cast<const v4f *>(s_scale + nn);
+            bi_next = *reinterpret_cast<const v4i *>(s_bias + nn);
+         }
+         unsigned char *dst = stg + m_local * SROW + nl * ESZ;
+         if constexpr (IS_INT && ESZ == 1) {
+            // rint(float(acc) * scale) + zp + 128, clamped below at lo + 128; the byte conversion
+            // saturates at 0 and 255, i.e. at q = -128 and q = 127
+            unsigned pk = 0;
+            float e[4];
 #pragma unroll
-         for (int q = 0; q < 4; ++q) {
-            const int nl = i * 32 + q * 8 + nq;
+            for (int t = 0; t < 4; ++t) {
+               float r = rintf(__fmul_rn(__int2float_rn(acc[i][j][q * 4 + t] + bi[t]), sc[t]));
+               if constexpr (!PLAIN) r = fmaxf(__fadd_rn(r, zpo), lof);
+               e[t] = r;
+            }
+            pk = __builtin_amdgcn_cvt_pk_u8_f32(e[0], 0, pk);
+            pk = __builtin_amdgcn_cvt_pk_u8_f32(e[1], 1, pk);
+            pk = __builtin_amdgcn_cvt_pk_u8_f32(e[2], 2, pk);
+            pk = __builtin_amdgcn_cvt_pk_u8_f32(e[3], 3, pk);
+            *reinterpret_cast<unsigned *>(dst) = pk ^ 0x80808080u;
+         } else {
             unsigned e[4];
-            const v4f sc = *reinterpret_cast<const v4f *>(s_scale + wn * WN + nl);
-            const v4i bi = *reinterpret_cast<const v4i *>(s_bias + wn * WN + nl);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                if constexpr (IS_INT)
@@ -129,16 +158,7 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::A
                else
                   e[t] = epilogue_value<false, OUT>(g, sc[t], bi[t], 0, acc[i][j][q * 4 + t]);
             }
-            unsigned char *dst = stg + m_local * SROW + nl * ESZ;
-            if constexpr (ESZ == 1) {
-               // e[] hold q+128 as floats in [0,255]: convert-and-insert, then flip the sign bits
-               unsigned pk = 0;
-               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[0]), 0, pk);
-               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[1]), 1, pk);
-               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[2]), 2, pk);
-               pk = __builtin_amdgcn_cvt_pk_u8_f32(__uint_as_float(e[3]), 3, pk);
-               *reinterpret_cast<unsigned *>(dst) = pk ^ 0x80808080u;
-            } else if constexpr (ESZ == 2) {
+            if constexpr (ESZ == 2) {
                v2i p = {(int)(e[0] | (e[1] << 16)), (int)(e[2] | (e[3] << 16))};
                *reinterpret_cast<v2i *>(dst) = p;
             } else {
@@ -147,14 +167,14 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::A
             }
          }
       }
-      __syncthreads();
+      __builtin_amdgcn_wave_barrier();
       constexpr int ITERS = 32 * CR / 64;
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
          const int c = it * 64 + lane;
          const int row = c / CR, cc = c % CR;
          const int m = m_wave + j * 32 + row;
-         const int nfirst = n0 + wn * WN + cc * (16 / ESZ);
+         const int nfirst = n_wave + cc * (16 / ESZ);
          if (m < g.M && nfirst < g.N) {
             const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
             unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
@@ -167,8 +187,43 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::A
             }
          }
       }
-      __syncthreads();
+      __builtin_amdgcn_wave_barrier();
    }
+}
+
+// Per-column scale and bias bits of a workgroup's BN columns starting at n0 -> LDS.
+__device__ __forceinline__ void stage_column_params(const GemmArgs &g, float *s_scale, int *s_bias, int tid, int n0,
+                                                    int BN)
+{
+   if (tid < BN) {
+      const int n = n0 + tid;
+      s_scale[tid] = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
+      s_bias[tid] = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
+   }
+}
+
+// Whole-workgroup form: smem is reused ([NWAVES staging blocks][BN scales][BN biases]), so all
+// wavefronts must have finished reading operand stages before the call.
+//   m_wave: first output row of this wavefront; n0: first output column of the workgroup;
+//   wn: index of the wavefront's column block; BN: columns of the workgroup tile.
+template <class Mma, int TI, int TJ, int OUT, int NWAVES>
+__device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ], unsigned char *smem,
+                                              int tid, int m_wave, int n0, int wn, int BN)
+{
+   constexpr int WB = EpilogueStaging<TI, OUT>::WAVE_BYTES;
+   constexpr int WN = TI * 32;
+   const int lane = tid & 63, wave = tid >> 6;
+   float *s_scale = reinterpret_cast<float *>(smem + NWAVES * WB);
+   int *s_bias = reinterpret_cast<int *>(s_scale + BN);
+   stage_column_params(g, s_scale, s_bias, tid, n0, BN);
+   __syncthreads();
+   unsigned char *stg = smem + wave * WB;
+   if (OUT == SOFIE_OUT_S8 && g.zp == -128 && g.lo == -128)
+      tile_epilogue_wave<Mma, TI, TJ, OUT, true>(g, acc, stg, s_scale + wn * WN, s_bias + wn * WN, lane, m_wave,
+                                                 n0 + wn * WN);
+   else
+      tile_epilogue_wave<Mma, TI, TJ, OUT, false>(g, acc, stg, s_scale + wn * WN, s_bias + wn * WN, lane, m_wave,
+                                                  n0 + wn * WN);
 }
 
 }  // namespace sofie

@@ -132,10 +132,7 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
     ctx = ctx or default_context()
     xd, wd, bd = ctx.dev(x, torch.float32), ctx.dev(w, torch.float32), ctx.dev(bias, torch.float32)
     N, Cc, H, W = xd.shape
-    if w_layout == L.LAYOUT_NCHW:
-        OC, _, kh, kw = wd.shape
-    else:
-        OC, kh, kw, _ = wd.shape
+    OC, _, kh, kw = wd.shape
     OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1], *dilations)
     y = ctx.empty((N, OC, OH, OW), torch.float32)
     ctx.check(ctx.lib.sofie_hip_conv2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, H, W,
