@@ -175,7 +175,9 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
       return b;
    };
    v4i pre[PF];
+   unsigned pre_inside = 0;    // bit i: pre[i] holds image data (otherwise the cell is padding)
    auto fetch = [&](Band b) {
+      pre_inside = 0;
 #pragma unroll
       for (int i = 0; i < PF; ++i) {
          const int r = i * a.RP + rsub;
@@ -183,58 +185,39 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          const int n = fdiv(vr, a.dHP);
          const int ih = vr - n * a.HP - a.ph;
          const bool inside = col_active && col_inside && r < b.rows && ih >= 0 && ih < a.H;
-         // the load is unconditional (clamped to the first pixel when the cell is outside) so that
-         // all of a pass's loads are in flight together; the value is selected afterwards
+         // the load is unconditional (of the first pixel when the cell is outside) and its value is
+         // looked at only when it is written to LDS, so all loads of a band are in flight together
          const size_t off = inside ? ((size_t)(n * a.H + ih) * a.W) * a.C + src_col : 0;
-         const v4i v = *reinterpret_cast<const v4i *>(a.x + off);
-         pre[i] = inside ? v : fillv;
+         pre[i] = *reinterpret_cast<const v4i *>(a.x + off);
+         pre_inside |= inside ? (1u << i) : 0u;
       }
    };
    auto stash = [&](Band b) {
 #pragma unroll
       for (int i = 0; i < PF; ++i) {
          const int r = i * a.RP + rsub;
-         if (col_active && r < b.rows) *reinterpret_cast<v4i *>(s_p + r * row_bytes + lds_col) = pre[i];
+         if (col_active && r < b.rows)
+            *reinterpret_cast<v4i *>(s_p + r * row_bytes + lds_col) = ((pre_inside >> i) & 1u) ? pre[i] : fillv;
       }
    };
 
-   int t = wg;
-   Band cur = {0, 0};
-   if (t < a.ntiles) {
-      cur = band_of(t);
-      fetch(cur);
-   }
    int b_off[NB];
 #pragma unroll
    for (int i = 0; i < NB; ++i) b_off[i] = ((wn * NB + i) * 32 + l32) * a.KS + half * 16;
    const int tap_step = a.CS - a.C32 * 32;              // from the end of one tap's channels to the next tap
    const int row_step = (a.WP - a.KW) * a.CS;           // from the end of one kernel row to the next
    const int nsteps = a.KH * a.KW * a.C32;
+   const int nq = half * 4;
+   const float *const w_scale = s_scale + wn * NB * 32;
+   const int *const w_bias = s_bias + wn * NB * 32;
+   unsigned char *const w_stg = s_stg + wave * WB;
 
-#ifdef ABL_TIMING
-   long long tm[6] = {0, 0, 0, 0, 0, 0};
-   long long t0 = clock64(), t1;
-#define TICK(i) do { t1 = clock64(); tm[i] += t1 - t0; t0 = t1; } while (0)
-#else
-#define TICK(i)
-#endif
-   for (; t < a.ntiles; t += nwg) {
-      TICK(5);
-      stash(cur);
-      __syncthreads();
-      TICK(0);
-      const int m0 = t * TM;
-      const int vr_lo = cur.vr_lo;
-      const int tn = t + nwg;
-      if (tn < a.ntiles) {
-         cur = band_of(tn);
-         fetch(cur);
-      }
-
-      int a_off[MB];
+   // LDS offsets of the wavefront's pixels inside the band of tile tt
+   int a_off[MB];
+   auto pixel_offsets = [&](int tt, int vr_lo) {
 #pragma unroll
       for (int j = 0; j < MB; ++j) {
-         int m = m0 + (wm * MB + j) * 32 + l32;
+         int m = tt * TM + (wm * MB + j) * 32 + l32;
          m = m < mtot ? m : mtot - 1;
          const int R = fdiv(m, a.dOW);
          const int ow = m - R * a.OW;
@@ -242,75 +225,106 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          const int v = n * a.HP + (R - n * a.OH) * a.sh - vr_lo;
          a_off[j] = (v * a.WP + ow * a.sw) * a.CS + half * 16;
       }
+   };
 
-      v16i acc[NB][MB];
+   // K loop over (kh, kw, 32-channel block) of one tile into acc; the accumulators start at the
+   // bias. Fragments of step s+1 are read while the matrix instructions of step s issue.
+   auto kloop = [&](v16i (&acc)[NB][MB]) {
 #pragma unroll
       for (int i = 0; i < NB; ++i)
 #pragma unroll
-         for (int j = 0; j < MB; ++j)
+         for (int q = 0; q < 4; ++q) {
+            const v4i bi = *reinterpret_cast<const v4i *>(w_bias + i * 32 + q * 8 + nq);
 #pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
-      TICK(1);
-
-      // K loop over (kh, kw, 32-channel block); fragments of step s+1 are read while the
-      // matrix instructions of step s issue
+            for (int j = 0; j < MB; ++j)
+#pragma unroll
+               for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = bi[e];
+         }
       v4i fa[2][MB], fb[2][NB];
       int ka = 0, kb = 0, c32 = 0, kw = 0;
-#pragma unroll
-      for (int j = 0; j < MB; ++j) fa[0][j] = *reinterpret_cast<const v4i *>(s_p + a_off[j]);
-#pragma unroll
-      for (int i = 0; i < NB; ++i) fb[0][i] = *reinterpret_cast<const v4i *>(s_w + b_off[i]);
-      for (int s = 0; s < nsteps; s += 2) {
-#pragma unroll
-         for (int u = 0; u < 2; ++u) {
-            // advance to the next step's offsets
-            ka += 32; kb += 32;
-            if (++c32 == a.C32) {
-               c32 = 0; ka += tap_step;
-               if (++kw == a.KW) { kw = 0; ka += row_step; }
-            }
-            const bool more = s + u + 1 < nsteps;
-            if (more) {
-#pragma unroll
-               for (int j = 0; j < MB; ++j) fa[u ^ 1][j] = *reinterpret_cast<const v4i *>(s_p + a_off[j] + ka);
-#pragma unroll
-               for (int i = 0; i < NB; ++i) fb[u ^ 1][i] = *reinterpret_cast<const v4i *>(s_w + b_off[i] + kb);
-            }
-#ifndef ABL_NO_MMA
-            if (s + u < nsteps)
-#else
-            if (s + u < nsteps && a.ph == 77)
-#endif
-            {
-#pragma unroll
-               for (int i = 0; i < NB; ++i)
-#pragma unroll
-                  for (int j = 0; j < MB; ++j) acc[i][j] = MmaI8::mma(fb[u][i], fa[u][j], acc[i][j]);
-            }
+      auto advance = [&]() {
+         ka += 32; kb += 32;
+         if (++c32 == a.C32) {
+            c32 = 0; ka += tap_step;
+            if (++kw == a.KW) { kw = 0; ka += row_step; }
          }
+      };
+      auto load = [&](int buf, int oa, int ob_) {
+#pragma unroll
+         for (int j = 0; j < MB; ++j) fa[buf][j] = *reinterpret_cast<const v4i *>(s_p + a_off[j] + oa);
+#pragma unroll
+         for (int i = 0; i < NB; ++i) fb[buf][i] = *reinterpret_cast<const v4i *>(s_w + b_off[i] + ob_);
+      };
+      auto mma = [&](int buf) {
+#pragma unroll
+         for (int i = 0; i < NB; ++i)
+#pragma unroll
+            for (int j = 0; j < MB; ++j) acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], acc[i][j]);
+      };
+      // two steps per trip; every fragment load is unconditional (the one past the last step re-reads
+      // step 0) so that the waits in front of the matrix instructions count exactly
+      load(0, 0, 0);
+      int s = 0;
+      for (; s + 1 < nsteps; s += 2) {
+         advance();
+         load(1, ka, kb);
+         mma(0);
+         advance();
+         const bool more = s + 2 < nsteps;
+         load(0, more ? ka : 0, more ? kb : 0);
+         mma(1);
       }
-      TICK(2);
-      __syncthreads();   // every wavefront is done with the band: its memory becomes the staging block
-      TICK(3);
-#ifdef ABL_NO_EPI
-      if (acc[0][0][0] == 0x12345 || a.ph == 77)
-#endif
+      if (s < nsteps) mma(0);
+   };
+   v4f r_scale[NB * 4];    // the lane's scales, loaded once (after the first barrier)
+   auto epilogue = [&](v16i (&acc)[NB][MB], int tt) {
+      const int m_wave = tt * TM + wm * MB * 32, n_wave = ob * OCT + wn * NB * 32;
       if (plain)
-         tile_epilogue_wave<MmaI8, NB, MB, OUT, true>(a.ep, acc, s_stg + wave * WB, s_scale + wn * NB * 32,
-                                                      s_bias + wn * NB * 32, lane, m0 + wm * MB * 32,
-                                                      ob * OCT + wn * NB * 32);
+         tile_epilogue_wave<MmaI8, NB, MB, OUT, true, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
+                                                                   n_wave, &r_scale);
       else
-         tile_epilogue_wave<MmaI8, NB, MB, OUT, false>(a.ep, acc, s_stg + wave * WB, s_scale + wn * NB * 32,
-                                                       s_bias + wn * NB * 32, lane, m0 + wm * MB * 32,
-                                                       ob * OCT + wn * NB * 32);
-      TICK(4);
+         tile_epilogue_wave<MmaI8, NB, MB, OUT, false, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
+                                                                    n_wave, &r_scale);
+   };
+
+   // One tile per iteration. The two wavefronts that share a SIMD do their halves in opposite order:
+   // wavefronts 0-3 run the matrix loop of tile t and then its epilogue, wavefronts 4-7 first finish
+   // the epilogue of their previous tile and then run the matrix loop of tile t, so the conversion
+   // arithmetic of one wavefront overlaps the matrix instructions of the other.
+   const bool mma_first = wave < 4;
+   int t = wg, t_prev = -1;
+   Band cur = {0, 0};
+   if (t < a.ntiles) {
+      cur = band_of(t);
+      fetch(cur);
+      pixel_offsets(t, cur.vr_lo);
    }
-#ifdef ABL_TIMING
-   if (blockIdx.x == 3 && (tid & 63) == 0) {
-      long long *d = (long long *)a.ep.A + (tid >> 6) * 8;
-      for (int i = 0; i < 6; ++i) d[i] = tm[i];
+   __syncthreads();   // weights and column parameters are in LDS
+#pragma unroll
+   for (int gi = 0; gi < NB * 4; ++gi)
+      r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+   v16i acc[NB][MB];
+   while (t < a.ntiles) {
+      stash(cur);
+      __syncthreads();                       // the band of tile t is complete
+      const int tn = t + nwg;
+      const bool more = tn < a.ntiles;
+      if (more) cur = band_of(tn);
+      if (mma_first) {
+         if (more) fetch(cur);
+         kloop(acc);
+         epilogue(acc, t);
+      } else {
+         if (t_prev >= 0) epilogue(acc, t_prev);
+         if (more) fetch(cur);
+         kloop(acc);
+      }
+      if (more) pixel_offsets(tn, cur.vr_lo);
+      t_prev = t;
+      t = tn;
+      __syncthreads();                       // every wavefront is done reading the band
    }
-#endif
+   if (!mma_first && t_prev >= 0) epilogue(acc, t_prev);
 }
 
 // Launches the MFMA kernel if the problem fits it; *done tells whether it did.
@@ -330,11 +344,6 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const int TM = (8 / WN) * 64;
    QConvTileArgs a{};
    a.x = g.x; a.w = g.w;
-#ifdef ABL_TIMING
-   static long long *dbg = nullptr;
-   if (!dbg) hipMalloc(&dbg, 512);
-   a.ep.A = (const uint8_t *)dbg;
-#endif
    a.ep.Y = g.y; a.ep.scale = g.scale; a.ep.bias = g.bias;
    a.ep.M = (int)mtot; a.ep.N = g.OC; a.ep.ldy = g.OC;
    a.ep.zp = g.zpy; a.ep.lo = g.lo; a.ep.relu = g.relu; a.ep.s = 1.0f;
@@ -379,28 +388,20 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));         \
       hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                             \
    } while (0)
-   if (WN == 2) {
-      if (passes <= 4) SOFIE_QCONV_LAUNCH(2, 4);
-      else if (passes <= 8) SOFIE_QCONV_LAUNCH(2, 8);
-      else SOFIE_QCONV_LAUNCH(2, 12);
-   } else {
-      if (passes <= 4) SOFIE_QCONV_LAUNCH(1, 4);
-      else if (passes <= 8) SOFIE_QCONV_LAUNCH(1, 8);
-      else SOFIE_QCONV_LAUNCH(1, 12);
-   }
+#define SOFIE_QCONV_BY_PASSES(WN_)                                                                            \
+   do {                                                                                                       \
+      if constexpr (OUT != SOFIE_OUT_S8) SOFIE_QCONV_LAUNCH(WN_, 12); /* raw accumulators: not tuned */      \
+      else if (passes <= 3) SOFIE_QCONV_LAUNCH(WN_, 3);                                                       \
+      else if (passes <= 4) SOFIE_QCONV_LAUNCH(WN_, 4);                                                       \
+      else if (passes <= 5) SOFIE_QCONV_LAUNCH(WN_, 5);                                                       \
+      else if (passes <= 6) SOFIE_QCONV_LAUNCH(WN_, 6);                                                       \
+      else if (passes <= 8) SOFIE_QCONV_LAUNCH(WN_, 8);                                                       \
+      else SOFIE_QCONV_LAUNCH(WN_, 12);                                                                       \
+   } while (0)
+   if (WN == 2) SOFIE_QCONV_BY_PASSES(2);
+   else SOFIE_QCONV_BY_PASSES(1);
+#undef SOFIE_QCONV_BY_PASSES
 #undef SOFIE_QCONV_LAUNCH
-#ifdef ABL_TIMING
-   {
-      static int calls = 0;
-      if (++calls % 23 == 0) {
-         hipDeviceSynchronize();
-         long long h[64];
-         hipMemcpy(h, dbg, sizeof(h), hipMemcpyDeviceToHost);
-         for (int w = 0; w < 8; w += 7)
-            printf("wave %d: stash+bar %lld  fetch+aoff %lld  kloop %lld  bar %lld  epi %lld  looptop %lld\n", w, h[w*8+0], h[w*8+1], h[w*8+2], h[w*8+3], h[w*8+4], h[w*8+5]);
-      }
-   }
-#endif
    *done = true;
    return check_launch(ctx, "k_qconv_mfma");
 }

@@ -94,6 +94,7 @@ __device__ __forceinline__ unsigned epilogue_value(const GemmArgs &g, float sc, 
 //   s_scale, s_bias: per-column scale and bias bits in LDS, already pointing at the
 //     wavefront's first column, filled and made visible by the caller;
 //   m_wave, n_wave: first output row and column of this wavefront.
+// ADD_BIAS false: the accumulators already include the bias.
 // PLAIN: int8 output with zero-point -128 and lower clamp -128 (the saturating byte
 // conversion does the clamping, two instructions per element fewer).
 template <int TI, int OUT> struct EpilogueStaging {
@@ -102,10 +103,14 @@ template <int TI, int OUT> struct EpilogueStaging {
    static constexpr int WAVE_BYTES = 32 * SROW;
 };
 
-template <class Mma, int TI, int TJ, int OUT, bool PLAIN>
+// FULLN: every 16-byte row segment lies inside the matrix and rows may be written with 16-byte
+// stores (no column checks). reg_scale: if not null, the lane's TI*4 scale vectors held in
+// registers (group gi = i*4 + q covers columns i*32 + q*8 + (lane/32)*4 .. +3); s_scale is then unused.
+template <class Mma, int TI, int TJ, int OUT, bool PLAIN, bool ADD_BIAS = true, bool FULLN = false>
 __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ],
                                                    unsigned char *stg, const float *s_scale, const int *s_bias,
-                                                   int lane, int m_wave, int n_wave)
+                                                   int lane, int m_wave, int n_wave,
+                                                   const v4f (*reg_scale)[TI * 4] = nullptr)
 {
    constexpr int ESZ = OutSize<OUT>::value;
    constexpr bool IS_INT = __is_same(typename Mma::Acc, v16i);
@@ -119,18 +124,20 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
 #pragma unroll
    for (int j = 0; j < TJ; ++j) {
       // scale and bias of group gi+1 are read while group gi is converted
-      v4f sc_next = *reinterpret_cast<const v4f *>(s_scale + nq);
-      v4i bi_next = *reinterpret_cast<const v4i *>(s_bias + nq);
+      v4f sc_next = {0.0f, 0.0f, 0.0f, 0.0f};
+      v4i bi_next = {0, 0, 0, 0};
+      if (!reg_scale) sc_next = *reinterpret_cast<const v4f *>(s_scale + nq);
+      if (ADD_BIAS || !IS_INT) bi_next = *reinterpret_cast<const v4i *>(s_bias + nq);
 #pragma unroll
       for (int gi = 0; gi < NG; ++gi) {
          const int i = gi >> 2, q = gi & 3;
          const int nl = i * 32 + q * 8 + nq;
-         const v4f sc = sc_next;
+         const v4f sc = reg_scale ? (*reg_scale)[gi] : sc_next;
          const v4i bi = bi_next;
          if (gi + 1 < NG) {
             const int nn = ((gi + 1) >> 2) * 32 + ((gi + 1) & 3) * 8 + nq;
-            sc_next = *reinterpret_cast<const v4f *>(s_scale + nn);
-            bi_next = *reinterpret_cast<const v4i *>(s_bias + nn);
+            if (!reg_scale) sc_next = *reinterpret_cast<const v4f *>(s_scale + nn);
+            if (ADD_BIAS || !IS_INT) bi_next = *reinterpret_cast<const v4i *>(s_bias + nn);
          }
          unsigned char *dst = stg + m_local * SROW + nl * ESZ;
          if constexpr (IS_INT && ESZ == 1) {
@@ -140,7 +147,7 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
             float e[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-               float r = rintf(__fmul_rn(__int2float_rn(acc[i][j][q * 4 + t] + bi[t]), sc[t]));
+               float r = rintf(__fmul_rn(__int2float_rn(acc[i][j][q * 4 + t] + (ADD_BIAS ? bi[t] : 0)), sc[t]));
                if constexpr (!PLAIN) r = fmaxf(__fadd_rn(r, zpo), lof);
                e[t] = r;
             }
@@ -154,7 +161,7 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
                if constexpr (IS_INT)
-                  e[t] = epilogue_value<true, OUT>(g, sc[t], bi[t], acc[i][j][q * 4 + t], 0.0f);
+                  e[t] = epilogue_value<true, OUT>(g, sc[t], ADD_BIAS ? bi[t] : 0, acc[i][j][q * 4 + t], 0.0f);
                else
                   e[t] = epilogue_value<false, OUT>(g, sc[t], bi[t], 0, acc[i][j][q * 4 + t]);
             }
@@ -175,10 +182,10 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
          const int row = c / CR, cc = c % CR;
          const int m = m_wave + j * 32 + row;
          const int nfirst = n_wave + cc * (16 / ESZ);
-         if (m < g.M && nfirst < g.N) {
+         if (m < g.M && (FULLN || nfirst < g.N)) {
             const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
             unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
-            if (g.vec_store && nfirst + 16 / ESZ <= g.N) {
+            if (FULLN || (g.vec_store && nfirst + 16 / ESZ <= g.N)) {
                *reinterpret_cast<v4i *>(out) = v;
             } else {
                const unsigned char *src = stg + row * SROW + cc * 16;
