@@ -168,6 +168,21 @@ int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, cons
                          int pad_h, int pad_w, int stride_h, int stride_w, int groups,
                          int zp_x, int zp_y, int act, int out_kind);
 
+/* QLinearConv -> (ReLU) -> MaxPool in one call: y is the pooled int8 tensor
+ * [N, OC, PH, PW] (y_layout), PH = (OH - pool_kh) / pool_stride_h + 1, no pooling pads.
+ * Same operands and rules as sofie_hip_qconv2d_s8; the result equals that call followed by
+ * sofie_hip_maxpool2d_s8 bit for bit. One-input-channel 3x3 layers with 2x2/2 pooling run a
+ * single kernel that never writes the unpooled tensor; other shapes run the convolution
+ * into the context's scratch buffer and pool from there. Replaces the reference's Conv,
+ * Relu and MaxPool emissions (ROperator_Conv.hxx:302-522, ROperator_Relu.hxx:54-66,
+ * ROperator_Pool.hxx:371-416) for quantized tensors. */
+int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
+                              int w_layout, const int32_t *bias, const float *scale, int8_t *y,
+                              int y_layout, int N, int C, int H, int W, int OC, int KH, int KW,
+                              int pad_h, int pad_w, int stride_h, int stride_w, int groups,
+                              int zp_x, int zp_y, int act, int pool_kh, int pool_kw,
+                              int pool_stride_h, int pool_stride_w);
+
 /* int8 max pooling, NCHW or NHWC. */
 int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N,
                            int C, int H, int W, int kh, int kw, int pad_t, int pad_l,

@@ -23,22 +23,12 @@
 //
 // k_qconv_simple: one thread per output element, any layout / group count / channel count.
 #include "common.h"
+#include "conv_s8.h"
 #include "gemm_tile.h"
 
 using namespace sofie;
 
 namespace {
-
-struct QConvArgs {
-   const int8_t *x, *w;
-   const int32_t *bias;
-   const float *scale;
-   void *y;
-   int N, C, H, W, OC, KH, KW, ph, pw, sh, sw, groups;
-   int OH, OW, icg, ocg;
-   int zpx, zpy, lo, relu;
-   int x_nhwc, y_nhwc, w_ohwi;
-};
 
 template <int OUT>
 __global__ void k_qconv_simple(QConvArgs g)
@@ -406,21 +396,33 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    return check_launch(ctx, "k_qconv_mfma");
 }
 
+size_t up256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+// The MFMA kernel takes channels-last activations and [OC][KH][KW][C] weights; other layouts of a shape
+// it takes are converted through scratch memory of this many bytes.
+bool mfma_shape(const QConvArgs &g) { return g.groups == 1 && g.C % 32 == 0 && g.OC % 64 == 0 && g.N <= 65535; }
+size_t layout_scratch_bytes(const QConvArgs &g)
+{
+   if (!mfma_shape(g) || (g.x_nhwc && g.y_nhwc && g.w_ohwi)) return 0;
+   return up256(g.x_nhwc ? 0 : (size_t)g.N * g.C * g.H * g.W) + up256(g.y_nhwc ? 0 : (size_t)g.N * g.OC * g.OH * g.OW) +
+          up256(g.w_ohwi ? 0 : (size_t)g.OC * g.C * g.KH * g.KW);
+}
+
+// Convolution without pooling; scratch has layout_scratch_bytes(g) bytes.
 template <int OUT>
-int run(sofie_hip_ctx *ctx, QConvArgs g)
+int run_conv(sofie_hip_ctx *ctx, const QConvArgs &g, int8_t *scratch)
 {
    constexpr int ESZ = OutSize<OUT>::value;
-   // MFMA path: activations NHWC, weights [OC][KH][KW][C]; other layouts are converted through the
-   // context's scratch buffer when the shape is one the MFMA kernel takes
-   const bool shape_ok = g.groups == 1 && g.C % 32 == 0 && g.OC % 64 == 0 && g.N <= 65535 && ESZ == 1;
-   if (shape_ok && (!g.x_nhwc || !g.y_nhwc || !g.w_ohwi)) {
+   bool done = false;
+   if constexpr (OUT == SOFIE_OUT_S8) {
+      if (int rc = qconv_first_layer(ctx, g, &done)) return rc;
+      if (done) return SOFIE_HIP_OK;
+   }
+   if (ESZ == 1 && mfma_shape(g) && (!g.x_nhwc || !g.y_nhwc || !g.w_ohwi)) {
       const size_t xb = g.x_nhwc ? 0 : (size_t)g.N * g.C * g.H * g.W;
       const size_t yb = g.y_nhwc ? 0 : (size_t)g.N * g.OC * g.OH * g.OW;
       const size_t wb = g.w_ohwi ? 0 : (size_t)g.OC * g.C * g.KH * g.KW;
-      auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
-      void *ws = nullptr;
-      if (int rc = workspace(ctx, up(xb) + up(yb) + up(wb), &ws)) return rc;
-      int8_t *xs = static_cast<int8_t *>(ws), *ys = xs + up(xb), *wsb = ys + up(yb);
+      int8_t *xs = scratch, *ys = xs + up256(xb), *wsb = ys + up256(yb);
       QConvArgs h = g;
       if (xb) {
          if (int rc = relayout_s8(ctx, g.x, xs, g.N, g.C, g.H, g.W, SOFIE_LAYOUT_NCHW, SOFIE_LAYOUT_NHWC)) return rc;
@@ -431,7 +433,6 @@ int run(sofie_hip_ctx *ctx, QConvArgs g)
          h.w = wsb; h.w_ohwi = 1;
       }
       if (yb) { h.y = ys; h.y_nhwc = 1; }
-      bool done = false;
       if (int rc = launch_mfma<OUT>(ctx, h, &done)) return rc;
       if (done) {
          if (yb) return relayout_s8(ctx, ys, static_cast<int8_t *>(g.y), g.N, g.OC, g.OH, g.OW, SOFIE_LAYOUT_NHWC,
@@ -439,7 +440,6 @@ int run(sofie_hip_ctx *ctx, QConvArgs g)
          return SOFIE_HIP_OK;
       }
    } else {
-      bool done = false;
       if (int rc = launch_mfma<OUT>(ctx, g, &done)) return rc;
       if (done) return SOFIE_HIP_OK;
    }
@@ -449,14 +449,38 @@ int run(sofie_hip_ctx *ctx, QConvArgs g)
    return check_launch(ctx, "k_qconv_simple");
 }
 
-}  // namespace
-
-extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w, int w_layout,
-                                    const int32_t *bias, const float *scale, void *y, int y_layout, int N, int C,
-                                    int H, int W, int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,
-                                    int stride_w, int groups, int zp_x, int zp_y, int act, int out_kind)
+template <int OUT>
+int run(sofie_hip_ctx *ctx, const QConvArgs &g)
 {
-   if (!ctx) return SOFIE_HIP_EINVAL;
+   void *ws = nullptr;
+   if (g.pool_kh == 0) {
+      const size_t need = layout_scratch_bytes(g);
+      if (need)
+         if (int rc = workspace(ctx, need, &ws)) return rc;
+      return run_conv<OUT>(ctx, g, static_cast<int8_t *>(ws));
+   }
+   // fused kernels first; otherwise the convolution goes to scratch memory in the layout of y and the
+   // pooling kernel reads it from there
+   bool done = false;
+   if (int rc = qconv_first_layer(ctx, g, &done)) return rc;
+   if (done) return SOFIE_HIP_OK;
+   QConvArgs h = g;
+   h.pool_kh = h.pool_kw = h.pool_sh = h.pool_sw = 0;
+   h.PH = g.OH; h.PW = g.OW;
+   const size_t conv_bytes = up256((size_t)g.N * g.OC * g.OH * g.OW);
+   if (int rc = workspace(ctx, conv_bytes + layout_scratch_bytes(h), &ws)) return rc;
+   h.y = ws;
+   if (int rc = run_conv<OUT>(ctx, h, static_cast<int8_t *>(ws) + conv_bytes)) return rc;
+   return sofie_hip_maxpool2d_s8(ctx, static_cast<const int8_t *>(ws), static_cast<int8_t *>(g.y),
+                                 g.y_nhwc ? SOFIE_LAYOUT_NHWC : SOFIE_LAYOUT_NCHW, g.N, g.OC, g.OH, g.OW, g.pool_kh,
+                                 g.pool_kw, 0, 0, 0, 0, g.pool_sh, g.pool_sw);
+}
+
+int fill_args(sofie_hip_ctx *ctx, QConvArgs &g, const int8_t *x, int x_layout, const int8_t *w, int w_layout,
+              const int32_t *bias, const float *scale, void *y, int y_layout, int N, int C, int H, int W, int OC, int KH,
+              int KW, int pad_h, int pad_w, int stride_h, int stride_w, int groups, int zp_x, int zp_y, int act,
+              int out_kind)
+{
    SOFIE_REQUIRE(ctx, N >= 0 && C > 0 && H > 0 && W > 0 && OC > 0 && KH > 0 && KW > 0, "non-positive dimension");
    SOFIE_REQUIRE(ctx, pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0, "bad pads/strides");
    SOFIE_REQUIRE(ctx, groups > 0 && C % groups == 0 && OC % groups == 0, "channels not divisible by groups");
@@ -470,12 +494,12 @@ extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_l
    if (N == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, x && w && y, "null operand");
    SOFIE_REQUIRE(ctx, scale || out_kind == SOFIE_OUT_S32, "scale is required for S8 output");
-   QConvArgs g{};
    g.x = x; g.w = w; g.bias = bias; g.scale = scale; g.y = y;
    g.N = N; g.C = C; g.H = H; g.W = W; g.OC = OC; g.KH = KH; g.KW = KW;
    g.ph = pad_h; g.pw = pad_w; g.sh = stride_h; g.sw = stride_w; g.groups = groups;
    g.OH = (H + 2 * pad_h - KH) / stride_h + 1;
    g.OW = (W + 2 * pad_w - KW) / stride_w + 1;
+   g.PH = g.OH; g.PW = g.OW;
    g.icg = C / groups;
    g.ocg = OC / groups;
    g.zpx = zp_x; g.zpy = zp_y;
@@ -485,6 +509,42 @@ extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_l
    g.x_nhwc = x_layout == SOFIE_LAYOUT_NHWC || C == 1;
    g.y_nhwc = y_layout == SOFIE_LAYOUT_NHWC || OC == 1;
    g.w_ohwi = w_layout == SOFIE_LAYOUT_NHWC || g.icg == 1 || KH * KW == 1;
+   return SOFIE_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w, int w_layout,
+                                    const int32_t *bias, const float *scale, void *y, int y_layout, int N, int C,
+                                    int H, int W, int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,
+                                    int stride_w, int groups, int zp_x, int zp_y, int act, int out_kind)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   QConvArgs g{};
+   if (int rc = fill_args(ctx, g, x, x_layout, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW, pad_h, pad_w,
+                          stride_h, stride_w, groups, zp_x, zp_y, act, out_kind))
+      return rc;
+   if (N == 0) return SOFIE_HIP_OK;
    if (out_kind == SOFIE_OUT_S32) return run<SOFIE_OUT_S32>(ctx, g);
+   return run<SOFIE_OUT_S8>(ctx, g);
+}
+
+extern "C" int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
+                                         int w_layout, const int32_t *bias, const float *scale, int8_t *y, int y_layout,
+                                         int N, int C, int H, int W, int OC, int KH, int KW, int pad_h, int pad_w,
+                                         int stride_h, int stride_w, int groups, int zp_x, int zp_y, int act,
+                                         int pool_kh, int pool_kw, int pool_stride_h, int pool_stride_w)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   QConvArgs g{};
+   if (int rc = fill_args(ctx, g, x, x_layout, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW, pad_h, pad_w,
+                          stride_h, stride_w, groups, zp_x, zp_y, act, SOFIE_OUT_S8))
+      return rc;
+   SOFIE_REQUIRE(ctx, pool_kh > 0 && pool_kw > 0 && pool_stride_h > 0 && pool_stride_w > 0, "bad pooling window");
+   SOFIE_REQUIRE(ctx, pool_kh <= g.OH && pool_kw <= g.OW, "pooling window larger than the convolution output");
+   if (N == 0) return SOFIE_HIP_OK;
+   g.pool_kh = pool_kh; g.pool_kw = pool_kw; g.pool_sh = pool_stride_h; g.pool_sw = pool_stride_w;
+   g.PH = (g.OH - pool_kh) / pool_stride_h + 1;
+   g.PW = (g.OW - pool_kw) / pool_stride_w + 1;
    return run<SOFIE_OUT_S8>(ctx, g);
 }

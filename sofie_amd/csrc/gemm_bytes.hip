@@ -604,6 +604,10 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
       const bool fits = (size_t)256 * g.lda + g.K < (1u << 31) && (size_t)256 * g.ldb + g.K < (1u << 31);
       if (big && fits) return launch_dma<Mma, SOFIE_DMA_BK, SOFIE_DMA_NST, OUT>(ctx, g);
       if (big) return launch_tiled<Mma, BK, NSETS, 4, 4, OUT, false>(ctx, g);
+      // a long K with few 128 x 128 tiles (a wide fully connected layer on a small batch x width):
+      // 64 x 64 tiles put four times as many workgroups on the device
+      if (cdiv(g.M, 128) * cdiv(g.N, 128) * 2 <= ctx->num_cus && g.K >= 1024)
+         return launch_tiled<Mma, BK, NSETS, 1, 1, OUT, false>(ctx, g);
       return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, false>(ctx, g);
    }
    if (big && g.K % 16 == 0 && (size_t)256 * g.lda + g.K < (1u << 31) && (size_t)257 * g.K < (1u << 31)) {

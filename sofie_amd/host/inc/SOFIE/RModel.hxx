@@ -77,6 +77,18 @@ public:
                                 std::shared_ptr<void> data);
    std::shared_ptr<void> GetInitializedTensorData(std::string tensor_name);
    void SetNotWritableInitializedTensor(const std::string &tensor_name);
+   // Channels-last bookkeeping of int8 activations. The quantized operators keep 4-D activations as
+   // [N,H,W,C] in memory (the order the matrix-core convolution reads); the tensor's shape stays the
+   // logical [N,C,H,W]. A Flatten of such a tensor is recorded with the same (C,H,W) so that the next
+   // matrix product can permute its weight rows instead of moving the activations.
+   void MarkChannelsLast(const std::string &name, size_t C, size_t H, size_t W) { fChannelsLast[name] = {C, H, W}; }
+   bool IsChannelsLast(const std::string &name, std::vector<size_t> *chw = nullptr) const
+   {
+      auto it = fChannelsLast.find(name);
+      if (it == fChannelsLast.end()) return false;
+      if (chw) *chw = it->second;
+      return true;
+   }
    void AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<std::size_t> shape);
    void AddIntermediateTensor(std::string tensor_name, ETensorType type, std::vector<Dim> dim_shape);
    void AddOutputTensorNameList(std::vector<std::string> output_tensor_names);
@@ -133,6 +145,7 @@ private:
    const std::set<std::string> fAllowedStdLib = {"vector", "algorithm", "cmath", "memory", "span"};
 
    std::map<std::string, std::string> fViewOf;      // view tensor -> tensor it aliases
+   std::map<std::string, std::vector<size_t>> fChannelsLast;   // tensor stored channels-last -> (C,H,W)
    std::map<std::string, Placement> fPlacement;     // arena slot of every non-view intermediate
    size_t fArenaBytes = 0;
    const std::string SP = "   ";

@@ -32,6 +32,7 @@ private:
    std::string fNX, fNY;
    std::vector<size_t> fShapeX, fShapeY;
    ETensorType fType = ETensorType::UNDEFINED;
+   bool fChannelsLast = false;   // int8 input stored [N,H,W,C]
 
 public:
    ROperator_Pool() {}
@@ -74,6 +75,8 @@ public:
          throw std::runtime_error("TMVA SOFIE Encountered unsupported type parsing a Pool operator");
       fShapeY = ShapeInference({fShapeX})[0];
       model.AddIntermediateTensor(fNY, fType, fShapeY);
+      fChannelsLast = model.IsChannelsLast(fNX);
+      if (fChannelsLast) model.MarkChannelsLast(fNY, fShapeY[1], fShapeY[2], fShapeY[3]);
    }
    std::string Generate(std::string OpName) override
    {
@@ -87,7 +90,7 @@ public:
          out << SP << "Check(sofie_hip_maxpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << fShapeX[0] * fShapeX[1]
              << ", " << fShapeX[2] << ", " << fShapeX[3];
       else
-         out << SP << "Check(sofie_hip_maxpool2d_s8(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", SOFIE_LAYOUT_NCHW, "
+         out << SP << "Check(sofie_hip_maxpool2d_s8(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << (fChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << ", "
              << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3];
       out << ", " << a.kernel_shape[0] << ", " << a.kernel_shape[1] << ", " << a.pads[0] << ", " << a.pads[1] << ", " << a.pads[2]
           << ", " << a.pads[3] << ", " << a.strides[0] << ", " << a.strides[1] << "), \"" << Name() << " " << OpName << "\");\n";

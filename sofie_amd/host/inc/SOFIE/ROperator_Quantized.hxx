@@ -115,7 +115,7 @@ public:
 
 // x = (q - zero_point) * scale
 class ROperator_DequantizeLinear final : public ROperator {
-   std::string fNX, fNScale, fNZp, fNY;
+   std::string fNX, fNScale, fNZp, fNY, fNXNchw;
    std::vector<size_t> fShape;
    float fScale = 1;
    int fZp = 0;
@@ -141,12 +141,28 @@ public:
       fZp = QUTIL::ScalarZeroPoint(model, fNZp, "DequantizeLinear");
       QUTIL::MarkFolded(model, {fNScale, fNZp});
       model.AddIntermediateTensor(fNY, ETensorType::FLOAT, fShape);
+      std::vector<size_t> chw;
+      if (model.IsChannelsLast(fNX, &chw) && chw[0] > 1 && chw[1] * chw[2] > 1) {
+         if (fShape.size() != 4)
+            throw std::runtime_error("TMVA SOFIE DequantizeLinear Op: flattened channels-last tensor " + fNX + " cannot be dequantized");
+         // float consumers expect [N,C,H,W]: convert the int8 tensor first
+         fNXNchw = fNX + "_nchw";
+         model.AddIntermediateTensor(fNXNchw, ETensorType::INT8, fShape);
+         fOutputTensorNames.push_back(fNXNchw);
+      }
    }
    std::string Generate(std::string OpName) override
    {
       std::stringstream out;
       out << "\n//------ DequantizeLinear op_" << OpName << "\n";
-      out << SP << "Check(sofie_hip_dequantize_s8_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << ConvertShapeToLength(fShape)
+      std::string src = fNX;
+      if (!fNXNchw.empty()) {
+         out << SP << "Check(sofie_hip_relayout_s8(fCtx, tensor_" << fNX << ", tensor_" << fNXNchw << ", " << fShape[0] << ", " << fShape[1]
+             << ", " << fShape[2] << ", " << fShape[3] << ", SOFIE_LAYOUT_NHWC, SOFIE_LAYOUT_NCHW), \"DequantizeLinear op_" << OpName
+             << "\");\n";
+         src = fNXNchw;
+      }
+      out << SP << "Check(sofie_hip_dequantize_s8_f32(fCtx, tensor_" << src << ", tensor_" << fNY << ", " << ConvertShapeToLength(fShape)
           << ", " << FloatLiteral(fScale) << ", " << fZp << "), \"DequantizeLinear op_" << OpName << "\");\n";
       return out.str();
    }
@@ -220,16 +236,28 @@ public:
       const float sy = fFloatOut ? 1.0f : QUTIL::ScalarFloat(model, fNYScale, op);
       fZpY = fFloatOut ? 0 : QUTIL::ScalarZeroPoint(model, fNYZp, op);
       // weights: [N,K], K contiguous
+      // If A is the Flatten of a channels-last tensor its columns are in (h,w,c) order: the weight rows
+      // are permuted to that order here instead of moving the activations at run time.
+      std::vector<size_t> chw;
+      const bool permute = model.IsChannelsLast(fNA, &chw) && chw[0] > 1 && chw[1] * chw[2] > 1;
+      if (permute && chw[0] * chw[1] * chw[2] != fK)
+         throw std::runtime_error("TMVA SOFIE QLinearMatMul Op: channels-last input " + fNA + " does not match K");
       const int8_t *b = static_cast<int8_t *>(model.GetInitializedTensorData(fNB).get());
       std::vector<int8_t> bt(fN * fK);
       std::vector<int64_t> colsum(fN, 0);
-      for (size_t k = 0; k < fK; ++k)
+      for (size_t k = 0; k < fK; ++k) {
+         size_t kdst = k;
+         if (permute) {
+            const size_t hw = chw[1] * chw[2], c = k / hw, pos = k % hw;
+            kdst = pos * chw[0] + c;
+         }
          for (size_t n = 0; n < fN; ++n) {
             const int8_t v = fTransB ? b[n * fK + k] : b[k * fN + n];
-            bt[n * fK + k] = v;
+            bt[n * fK + kdst] = v;
             colsum[n] += v;
          }
-      fNBt = fNB + "_nk";
+      }
+      fNBt = fNB + (permute ? "_nk_cl" : "_nk");
       if (!model.CheckIfTensorAlreadyExist(fNBt)) model.AddInitializedTensor(fNBt, ETensorType::INT8, {fN, fK}, QUTIL::Share(bt));
       // per-column scale
       std::vector<float> scale(fN);
@@ -278,10 +306,10 @@ public:
 class ROperator_QLinearConv final : public ROperator {
    ConvGeometry fGeom;
    std::string fNX, fNXScale, fNXZp, fNW, fNWScale, fNWZp, fNYScale, fNYZp, fNBias, fNY;
-   std::string fNScale, fNQBias;
+   std::string fNScale, fNQBias, fNWPacked;
    std::vector<size_t> fShapeX, fShapeW, fShapeY;
    int fZpX = 0, fZpY = 0;
-   bool fHasBias = false;
+   bool fHasBias = false, fXChannelsLast = false;
    EActivationType fActivation = EActivationType::UNDEFINED;
 public:
    ROperator_QLinearConv(std::string autopad, std::vector<size_t> dilations, size_t group, std::vector<size_t> kernelShape,
@@ -357,7 +385,23 @@ public:
          model.AddInitializedTensor(fNQBias, ETensorType::INT32, {OC}, QUTIL::Share(qb));
       }
       QUTIL::MarkFolded(model, {fNXScale, fNXZp, fNWScale, fNWZp, fNYScale, fNYZp, fNBias});
-      fInputTensorNames = {fNX, fNW, fNScale};
+      // Layouts: the output is kept channels-last (what the matrix-core kernel writes and what the next
+      // quantized operator reads); the weights are repacked once, here, to [OC][KH][KW][C/group].
+      fXChannelsLast = model.IsChannelsLast(fNX);
+      model.MarkChannelsLast(fNY, fShapeY[1], fShapeY[2], fShapeY[3]);
+      {
+         const int8_t *w = static_cast<int8_t *>(model.GetInitializedTensorData(fNW).get());
+         const size_t icg = fShapeW[1], khw = fShapeW[2] * fShapeW[3];
+         std::vector<int8_t> packed(OC * per);
+         for (size_t oc = 0; oc < OC; ++oc)
+            for (size_t ic = 0; ic < icg; ++ic)
+               for (size_t t = 0; t < khw; ++t) packed[(oc * khw + t) * icg + ic] = w[(oc * icg + ic) * khw + t];
+         fNWPacked = fNW + "_ohwi";
+         if (!model.CheckIfTensorAlreadyExist(fNWPacked))
+            model.AddInitializedTensor(fNWPacked, ETensorType::INT8, {OC, fShapeW[2], fShapeW[3], icg}, QUTIL::Share(packed));
+         QUTIL::MarkFolded(model, {fNW});
+      }
+      fInputTensorNames = {fNX, fNWPacked, fNScale};
       if (fHasBias) fInputTensorNames.push_back(fNQBias);
       model.AddIntermediateTensor(fNY, ETensorType::INT8, fShapeY);
    }
@@ -368,9 +412,10 @@ public:
       fGeom.SymmetricPads(ph, pw);
       std::stringstream out;
       out << "\n//----  operator QLinearConv op_" << OpName << "\n";
-      out << SP << "Check(sofie_hip_qconv2d_s8(fCtx, tensor_" << fNX << ", SOFIE_LAYOUT_NCHW, tensor_" << fNW << ", SOFIE_LAYOUT_NCHW, "
+      out << SP << "Check(sofie_hip_qconv2d_s8(fCtx, tensor_" << fNX << ", " << (fXChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW")
+          << ", tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, "
           << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", tensor_" << fNScale << ", tensor_" << fNY
-          << ", SOFIE_LAYOUT_NCHW, " << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", "
+          << ", SOFIE_LAYOUT_NHWC, " << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", "
           << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3] << ", " << ph << ", " << pw << ", " << fGeom.strides[0] << ", "
           << fGeom.strides[1] << ", " << fGeom.group << ", " << fZpX << ", " << fZpY << ", "
           << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << ", SOFIE_OUT_S8), \"QLinearConv op_"

@@ -35,6 +35,8 @@ public:
       fShape = model.GetTensorShape(fNX);
       fType = model.GetTensorType(fNX);
       model.AddIntermediateTensor(fNY, fType, fShape);
+      std::vector<size_t> chw;   // element-wise: the output keeps the input's memory order
+      if (model.IsChannelsLast(fNX, &chw)) model.MarkChannelsLast(fNY, chw[0], chw[1], chw[2]);
    }
    std::string Generate(std::string OpName) override
    {

@@ -77,6 +77,14 @@ public:
          model.SetNotWritableInitializedTensor(fNShape);
       }
       model.AddIntermediateTensor(fNOutput, model.GetTensorType(fNData), fShapeOutput);
+      std::vector<size_t> chw;
+      if (model.IsChannelsLast(fNData, &chw) && chw[0] > 1 && chw[1] * chw[2] > 1) {
+         // the bytes stay in (h,w,c) order: only a flatten to [N, C*H*W] can be handed on, with the order recorded
+         if (fShapeOutput.size() == 2 && fShapeOutput[0] == fShapeInput[0] && fShapeOutput[1] == chw[0] * chw[1] * chw[2])
+            model.MarkChannelsLast(fNOutput, chw[0], chw[1], chw[2]);
+         else
+            throw std::runtime_error("TMVA Reshape Op: tensor " + fNData + " is stored channels-last and can only be flattened to [N, C*H*W]");
+      }
    }
    std::string Generate(std::string OpName) override
    {

@@ -173,6 +173,12 @@ void RModel::Initialize(int /*batchSize*/, bool verbose)
    for (auto &n : fOutputTensorNames)
       if (!CheckIfTensorAlreadyExist(n))
          throw std::runtime_error("TMVA-SOFIE: output tensor " + n + " is not produced by any operator");
+   for (auto &n : fOutputTensorNames) {
+      std::vector<size_t> chw;
+      if (IsChannelsLast(n, &chw) && chw[0] > 1 && chw[1] * chw[2] > 1)
+         throw std::runtime_error("TMVA-SOFIE: output tensor " + n + " is an int8 activation stored channels-last; "
+                                  "end the graph with DequantizeLinear or a matrix product");
+   }
    fIsInitialized = true;
 }
 

@@ -253,6 +253,34 @@ def qconv2d_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zp
     return _ret(y, x)
 
 
+def qconv2d_pool_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, zpy=0, relu=False,
+                    pool=(2, 2), pool_strides=(2, 2), x_layout=L.LAYOUT_NCHW, y_layout=L.LAYOUT_NCHW, ctx=None,
+                    w_layout=L.LAYOUT_NCHW):
+    """QLinearConv -> (ReLU) -> MaxPool(pool, pool_strides, no pads) in one library call."""
+    ctx = ctx or default_context()
+    if zpx != 0:
+        bias = fold_zero_point_conv(w, bias, zpx)
+    xd, wd = ctx.dev(x, torch.int8), ctx.dev(w, torch.int8)
+    if x_layout == L.LAYOUT_NCHW:
+        N, Cc, H, W = xd.shape
+    else:
+        N, H, W, Cc = xd.shape
+    if w_layout == L.LAYOUT_NCHW:
+        OC, _, kh, kw = wd.shape
+    else:
+        OC, kh, kw, _ = wd.shape
+    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1])
+    PH, PW = (OH - pool[0]) // pool_strides[0] + 1, (OW - pool[1]) // pool_strides[1] + 1
+    y = ctx.empty((N, OC, PH, PW) if y_layout == L.LAYOUT_NCHW else (N, PH, PW, OC), torch.int8)
+    sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
+    ctx.check(ctx.lib.sofie_hip_qconv2d_pool_s8(ctx.h, ctx.ptr(xd), x_layout, ctx.ptr(wd), w_layout, ctx.ptr(bd),
+                                                ctx.ptr(sd), ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, pads[0],
+                                                pads[1], strides[0], strides[1], groups, int(zpx), int(zpy),
+                                                L.ACT_RELU if relu else L.ACT_NONE, pool[0], pool[1], pool_strides[0],
+                                                pool_strides[1]))
+    return _ret(y, x)
+
+
 def iconv2d_s8(x, w, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, ctx=None):
     return qconv2d_s8(x, w, None, None, pads, strides, groups, zpx, out=L.OUT_S32, ctx=ctx)
 

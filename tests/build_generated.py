@@ -22,6 +22,7 @@ def all_specs(with_large=True):
     specs.append(models.mlp_spec()[0])
     specs.append(models.cnn_f32_spec(8))
     specs.append(models.qcnn_spec(oracle, 8))
+    specs.append(models.qdq_conv_spec())
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs

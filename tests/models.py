@@ -182,3 +182,41 @@ def qcnn_reference(oracle, x):
     bias2 = (q["bf2"].astype(np.int64) + 128 * q["fc2"].astype(np.int64).sum(axis=0)).astype(np.int32)
     acc = oracle.igemm_s8(g1, q["fc2"]).astype(np.int64) + bias2
     return (acc.astype(np.int32).astype(f32) * s2).astype(f32)
+
+
+# ------------------------------------------------------------------------------------------ QDQ conv layer
+def qdq_conv_params(seed=7):
+    """One quantized conv layer between QuantizeLinear and DequantizeLinear: float [2,32,9,7] in, float
+    [2,64,9,7] out. Exercises NCHW int8 input, channels-last output and the conversion back for float."""
+    r = np.random.default_rng(seed)
+    x = r.uniform(-1, 1, (2, 32, 9, 7)).astype(np.float32)
+    w = r.integers(-127, 128, (64, 32, 3, 3)).astype(np.int8)
+    sw = r.uniform(0.001, 0.003, 64).astype(np.float32)
+    b = r.integers(-500, 500, 64).astype(np.int32)
+    return {"x": x, "w": w, "sw": sw, "b": b, "sx": np.float32(1 / 127.0), "zx": 3, "sy": np.float32(0.05), "zy": -7}
+
+
+def qdq_conv_spec(name="qdq_conv"):
+    p = qdq_conv_params()
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", p["x"].shape)
+    s.add_scalar("sx", p["sx"], np.float32)
+    s.add_scalar("zx", p["zx"], np.int8)
+    s.add_scalar("sy", p["sy"], np.float32)
+    s.add_scalar("zy", p["zy"], np.int8)
+    s.add_init("w", p["w"])
+    s.add_init("sw", p["sw"])
+    s.add_init("b", p["b"])
+    s.quantize("x", "sx", "zx", "xq")
+    s.qlinear_conv("xq", "sx", "zx", "w", "sw", None, "sy", "zy", "c", "b", (3, 3), (1, 1, 1, 1), (1, 1))
+    s.dequantize("c", "sy", "zy", "y")
+    s.set_output("y")
+    return s
+
+
+def qdq_conv_reference(oracle):
+    p = qdq_conv_params()
+    xq = oracle.quantize_f32_s8(p["x"], p["sx"], p["zx"])
+    scale = ((p["sx"] * p["sw"]).astype(np.float32) / p["sy"]).astype(np.float32)
+    c = oracle.qconv2d_s8(xq, p["w"], scale, p["b"], (1, 1), (1, 1), 1, p["zx"], p["zy"], False)
+    return oracle.dequantize_s8_f32(c, p["sy"], p["zy"])

@@ -104,7 +104,10 @@ def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
     hxx, dat, _ = gen(spec, tmp_path)
     code = open(hxx).read()
     assert code.count("sofie_hip_qconv2d_s8(") == 3 and code.count("sofie_hip_qgemm_s8(") == 2
-    assert "int8_t * tensor_fc1_nk" in code and "tensor_fc1 =" not in code      # transposed once, original dropped
+    assert "int8_t * tensor_fc1_nk_cl" in code and "tensor_fc1 =" not in code   # transposed once, original dropped
+    assert "tensor_w2_ohwi, SOFIE_LAYOUT_NHWC" in code and "tensor_w2 =" not in code
+    # conv1 reads the one-channel quantized input as it is, everything after it is channels-last
+    assert code.count("SOFIE_LAYOUT_NCHW, tensor_w") == 1 and code.count("sofie_hip_maxpool2d_s8(fCtx, tensor_r1, tensor_p1, SOFIE_LAYOUT_NHWC") == 1
     assert "SOFIE_OUT_F32" in code and "std::vector<float> infer(float* tensor_x)" in code
     q = models.qcnn_params(oracle)
     text = open(dat).read().split("\n")
@@ -114,8 +117,12 @@ def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
     assert np.array_equal(scale, want)
     qb = np.array(rec["tensor_c1_qbias"].split(), np.int64)
     assert np.array_equal(qb, q["b1"].astype(np.int64) + 128 * q["w1"].astype(np.int64).reshape(32, -1).sum(axis=1))
-    fc1 = np.array(rec["tensor_fc1_nk"].split(), np.int64).reshape(256, 12800)
-    assert np.array_equal(fc1, q["fc1"].T)
+    # fc1 consumes the flattened channels-last conv3 output: rows reordered from (c,h,w) to (h,w,c)
+    fc1 = np.array(rec["tensor_fc1_nk_cl"].split(), np.int64).reshape(256, 12800)
+    want_fc1 = q["fc1"].T.reshape(256, 128, 100).transpose(0, 2, 1).reshape(256, 12800)
+    assert np.array_equal(fc1, want_fc1)
+    w2 = np.array(rec["tensor_w2_ohwi"].split(), np.int64).reshape(64, 3, 3, 32)
+    assert np.array_equal(w2, q["w2"].transpose(0, 2, 3, 1))
 
 
 def emit_error(spec, tmp_path):

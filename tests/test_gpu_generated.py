@@ -75,6 +75,15 @@ def test_int8_cnn_session_is_bit_exact(tmp_path):
     assert np.array_equal(np.argmax(y.reshape(8, 5), 1), np.argmax(f, 1)) or rel_err(y, f.reshape(-1)) < 0.1
 
 
+def test_quantize_conv_dequantize_session(tmp_path):
+    """NCHW int8 into the conv, channels-last out of it, converted back for the float consumer: the floats are
+    exact products of an int8 and the output scale, so they equal the oracle's bit for bit."""
+    p = models.qdq_conv_params()
+    y = run_session("qdq_conv", p["x"], tmp_path)
+    ref = models.qdq_conv_reference(oracle)
+    assert np.array_equal(y, ref.reshape(-1))
+
+
 def test_int8_cnn_batch_4096_matches_the_oracle_on_a_sample_and_is_batch_invariant(tmp_path):
     """Full benchmark batch: every image is computed independently of its neighbours, so the first 8 rows
     equal the batch-8 Session's output, and 16 images spread over the batch equal the oracle."""

@@ -315,6 +315,54 @@ def test_qconv2d_s8_matrix_core_path(ops, cfg):
     assert np.array_equal(acc.transpose(0, 3, 1, 2), oracle.iconv2d_s8(x, w, cfg["p"], cfg["s"], 1, 5))
 
 
+@pytest.mark.parametrize("cfg", [
+    dict(N=3, H=40, W=40, OC=32), dict(N=2, H=7, W=9, OC=8), dict(N=1, H=1, W=1, OC=4), dict(N=5, H=13, W=6, OC=20),
+    dict(N=2, H=64, W=50, OC=64),
+])
+def test_first_layer_kernel(ops, cfg):
+    """One input channel, 3x3, pad 1: the dot-product kernel, with both zero-point conventions, a ReLU clamp and
+    scales of both signs (the pooled variant picks max or min of the accumulators by the sign)."""
+    from sofie_amd import lib as L
+    r = rng(600 + cfg["H"] + cfg["OC"])
+    x = r.integers(-128, 128, (cfg["N"], 1, cfg["H"], cfg["W"])).astype(np.int8)
+    w = r.integers(-127, 128, (cfg["OC"], 1, 3, 3)).astype(np.int8)
+    scale = (r.uniform(20, 60, cfg["OC"]) / (73.3 * 73.3 * 3)).astype(np.float32)
+    scale[::3] *= -1
+    bias = r.integers(-3000, 3000, cfg["OC"]).astype(np.int32)
+    for zpx, zpy, relu in ((-128, -128, True), (5, -3, False)):
+        ref = oracle.qconv2d_s8(x, w, scale, bias, (1, 1), (1, 1), 1, zpx, zpy, relu)
+        y = ops.qconv2d_s8(x, w, scale, bias, (1, 1), (1, 1), 1, zpx, zpy, relu, y_layout=L.LAYOUT_NHWC)
+        assert np.array_equal(y.transpose(0, 3, 1, 2), ref)
+        if cfg["H"] >= 2 and cfg["W"] >= 2:
+            pooled = oracle.maxpool2d(ref, (2, 2), (2, 2))
+            yp = ops.qconv2d_pool_s8(x, w, scale, bias, (1, 1), (1, 1), 1, zpx, zpy, relu, y_layout=L.LAYOUT_NHWC)
+            assert np.array_equal(yp.transpose(0, 3, 1, 2), pooled)
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(N=2, C=32, H=20, W=20, OC=64, k=(3, 3), p=(1, 1), pool=(2, 2), ps=(2, 2)),
+    dict(N=2, C=6, H=9, W=8, OC=10, k=(3, 3), p=(0, 0), pool=(3, 2), ps=(2, 1)),
+    dict(N=1, C=64, H=11, W=11, OC=128, k=(3, 3), p=(1, 1), pool=(2, 2), ps=(2, 2)),
+])
+def test_conv_pool_entry_point(ops, cfg):
+    """The fused entry point on shapes without a fused kernel: convolution into scratch memory, then pooling,
+    in both layouts."""
+    from sofie_amd import lib as L
+    r = rng(700 + cfg["C"])
+    x = r.integers(-128, 128, (cfg["N"], cfg["C"], cfg["H"], cfg["W"])).astype(np.int8)
+    w = r.integers(-127, 128, (cfg["OC"], cfg["C"]) + cfg["k"]).astype(np.int8)
+    K = cfg["C"] * cfg["k"][0] * cfg["k"][1]
+    scale = (r.uniform(20, 60, cfg["OC"]) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    bias = r.integers(-3000, 3000, cfg["OC"]).astype(np.int32)
+    ref = oracle.maxpool2d(oracle.qconv2d_s8(x, w, scale, bias, cfg["p"], (1, 1), 1, -128, -128, True), cfg["pool"], cfg["ps"])
+    y = ops.qconv2d_pool_s8(x, w, scale, bias, cfg["p"], (1, 1), 1, -128, -128, True, cfg["pool"], cfg["ps"])
+    assert np.array_equal(y, ref)
+    xh = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    yh = ops.qconv2d_pool_s8(xh, w, scale, bias, cfg["p"], (1, 1), 1, -128, -128, True, cfg["pool"], cfg["ps"],
+                             x_layout=L.LAYOUT_NHWC, y_layout=L.LAYOUT_NHWC)
+    assert np.array_equal(yh.transpose(0, 3, 1, 2), ref)
+
+
 # --------------------------------------------------------------------------- fp8
 def fp8_operands(r, M, N, K, transB):
     a = r.standard_normal((M, K)).astype(np.float32)
