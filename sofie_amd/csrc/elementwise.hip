@@ -68,6 +68,47 @@ __global__ void k_maxpool2d(const T *__restrict__ x, T *__restrict__ y, int N, i
    y[idx] = best;
 }
 
+// Channels-last int8 max pooling, 16 channels (one 16-byte vector) of one output pixel per thread.
+// Signed bytes are compared as unsigned after flipping the sign bit, four at a time.
+__device__ __forceinline__ unsigned max_u8x4(unsigned a, unsigned b)
+{
+   unsigned r = 0;
+#pragma unroll
+   for (int i = 0; i < 4; ++i) {
+      const unsigned x = (a >> (8 * i)) & 0xffu, y = (b >> (8 * i)) & 0xffu;
+      r |= (x > y ? x : y) << (8 * i);
+   }
+   return r;
+}
+
+__global__ void k_maxpool2d_s8_nhwc16(const int8_t *__restrict__ x, int8_t *__restrict__ y, int N, int C16, int H, int W,
+                                      int OH, int OW, int kh, int kw, int pt, int pl, int sh, int sw)
+{
+   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   const size_t total = (size_t)N * OH * OW * C16;
+   if (idx >= total) return;
+   size_t r = idx;
+   const int c = (int)(r % C16); r /= C16;
+   const int ow = (int)(r % OW); r /= OW;
+   const int oh = (int)(r % OH);
+   const int n = (int)(r / OH);
+   v4i best = {0, 0, 0, 0};   // bytes with the sign bit flipped: 0 is the lowest value
+   for (int i = 0; i < kh; ++i) {
+      const int ih = oh * sh - pt + i;
+      if (ih < 0 || ih >= H) continue;
+      for (int j = 0; j < kw; ++j) {
+         const int iw = ow * sw - pl + j;
+         if (iw < 0 || iw >= W) continue;
+         const v4i v = *reinterpret_cast<const v4i *>(x + ((((size_t)n * H + ih) * W + iw) * C16 + c) * 16);
+#pragma unroll
+         for (int e = 0; e < 4; ++e) best[e] = (int)max_u8x4((unsigned)best[e], (unsigned)v[e] ^ 0x80808080u);
+      }
+   }
+#pragma unroll
+   for (int e = 0; e < 4; ++e) best[e] ^= (int)0x80808080u;
+   *reinterpret_cast<v4i *>(y + idx * 16) = best;
+}
+
 __global__ void k_quantize_f32_s8(const float *__restrict__ x, int8_t *__restrict__ q, size_t len, float scale, int zp)
 {
    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
@@ -214,6 +255,11 @@ int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int l
    int OH, OW;
    if (int rc = pool_dims(ctx, H, W, kh, kw, pt, pl, pb, pr, sh, sw, &OH, &OW)) return rc;
    const size_t total = (size_t)N * C * OH * OW;
+   if (layout == SOFIE_LAYOUT_NHWC && C % 16 == 0 && aligned16(x) && aligned16(y)) {
+      hipLaunchKernelGGL(k_maxpool2d_s8_nhwc16, dim3(blocks_for(total / 16, 256)), dim3(256), 0, ctx->stream, x, y, N, C / 16,
+                         H, W, OH, OW, kh, kw, pt, pl, sh, sw);
+      return check_launch(ctx, "k_maxpool2d_s8_nhwc16");
+   }
    if (layout == SOFIE_LAYOUT_NHWC)
       hipLaunchKernelGGL((k_maxpool2d<int8_t, true>), dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y,
                          N, C, H, W, OH, OW, kh, kw, pt, pl, sh, sw);

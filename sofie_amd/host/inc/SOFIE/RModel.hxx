@@ -125,6 +125,7 @@ private:
       int first = 0, last = 0;
    };
    void FuseActivations();
+   void FusePooling();
    void PlanIntermediateMemory();
    void GenerateHeaderInfo(std::string &hgname);
    void GenerateSessionCode();

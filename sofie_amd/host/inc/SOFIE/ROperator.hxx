@@ -40,6 +40,16 @@ public:
    // when fused away, the operator emits nothing and its output aliases its input
    void SetFusedAway() { fFusedAway = true; }
    bool IsFusedAway() const { return fFusedAway; }
+   // try to absorb a following max pooling (kernel, strides, no pads) whose output tensor becomes this
+   // operator's output; on success the operator no longer writes its original output tensor
+   virtual bool FusePooling(const std::vector<size_t> & /*kernel*/, const std::vector<size_t> & /*strides*/,
+                            const std::string & /*pooledName*/, const std::vector<size_t> & /*pooledShape*/)
+   {
+      return false;
+   }
+   // absorbed into another operator: emits nothing, and its output is written by the absorbing operator
+   void SetAbsorbed() { fAbsorbed = true; }
+   bool IsAbsorbed() const { return fAbsorbed; }
 
    const std::vector<std::string> &GetOpInputTensors() const { return fInputTensorNames; }
    const std::vector<std::string> &GetOpOutputTensors() const { return fOutputTensorNames; }
@@ -49,6 +59,7 @@ protected:
    bool fUseSession = false;
    bool fIsOutputConstant = false;
    bool fFusedAway = false;
+   bool fAbsorbed = false;
    std::vector<std::string> fInputTensorNames;    // every tensor the emitted code reads
    std::vector<std::string> fOutputTensorNames;   // tensors the emitted code writes
 };

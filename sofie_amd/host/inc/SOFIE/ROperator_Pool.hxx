@@ -43,6 +43,18 @@ public:
       fOutputTensorNames = {fNY};
    }
    std::string Kind() const override { return "Pool"; }
+   // what a producer needs to know to absorb this pooling (valid after Initialize)
+   bool IsPlainMaxPool() const
+   {
+      if (fPoolMode != MaxPool || fAttr.ceil_mode != 0) return false;
+      for (auto p : fAttr.pads)
+         if (p != 0) return false;
+      return fAttr.kernel_shape.size() == 2 && fAttr.strides.size() == 2;
+   }
+   const std::vector<size_t> &KernelShape() const { return fAttr.kernel_shape; }
+   const std::vector<size_t> &Strides() const { return fAttr.strides; }
+   const std::vector<size_t> &OutputShape() const { return fShapeY; }
+   ETensorType TensorType() const { return fType; }
    std::string Name() { return fPoolMode == MaxPool ? "MaxPool" : fPoolMode == AveragePool ? "AveragePool" : "Invalid"; }
    std::vector<ETensorType> TypeInference(std::vector<ETensorType> input) override { return input; }
    std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>> input) override

@@ -306,8 +306,8 @@ public:
 class ROperator_QLinearConv final : public ROperator {
    ConvGeometry fGeom;
    std::string fNX, fNXScale, fNXZp, fNW, fNWScale, fNWZp, fNYScale, fNYZp, fNBias, fNY;
-   std::string fNScale, fNQBias, fNWPacked;
-   std::vector<size_t> fShapeX, fShapeW, fShapeY;
+   std::string fNScale, fNQBias, fNWPacked, fNYPooled;
+   std::vector<size_t> fShapeX, fShapeW, fShapeY, fShapePooled, fPoolKernel, fPoolStrides;
    int fZpX = 0, fZpY = 0;
    bool fHasBias = false, fXChannelsLast = false;
    EActivationType fActivation = EActivationType::UNDEFINED;
@@ -330,6 +330,18 @@ public:
    {
       if (act != EActivationType::RELU || fActivation != EActivationType::UNDEFINED) return false;
       fActivation = act;
+      return true;
+   }
+   bool FusePooling(const std::vector<size_t> &kernel, const std::vector<size_t> &strides, const std::string &pooledName,
+                    const std::vector<size_t> &pooledShape) override
+   {
+      if (fShapeY.empty() || !fPoolKernel.empty() || kernel.size() != 2 || strides.size() != 2) return false;
+      if (kernel[0] > fShapeY[2] || kernel[1] > fShapeY[3]) return false;
+      fPoolKernel = kernel;
+      fPoolStrides = strides;
+      fNYPooled = pooledName;
+      fShapePooled = pooledShape;
+      fOutputTensorNames = {fNYPooled};
       return true;
    }
    std::vector<ETensorType> TypeInference(std::vector<ETensorType>) override { return {ETensorType::INT8}; }
@@ -411,15 +423,20 @@ public:
       size_t ph, pw;
       fGeom.SymmetricPads(ph, pw);
       std::stringstream out;
-      out << "\n//----  operator QLinearConv op_" << OpName << "\n";
-      out << SP << "Check(sofie_hip_qconv2d_s8(fCtx, tensor_" << fNX << ", " << (fXChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW")
-          << ", tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, "
-          << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", tensor_" << fNScale << ", tensor_" << fNY
-          << ", SOFIE_LAYOUT_NHWC, " << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", "
-          << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3] << ", " << ph << ", " << pw << ", " << fGeom.strides[0] << ", "
-          << fGeom.strides[1] << ", " << fGeom.group << ", " << fZpX << ", " << fZpY << ", "
-          << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << ", SOFIE_OUT_S8), \"QLinearConv op_"
-          << OpName << "\");\n";
+      const bool pooled = !fPoolKernel.empty();
+      out << "\n//----  operator QLinearConv" << (pooled ? " + MaxPool" : "") << " op_" << OpName << "\n";
+      out << SP << "Check(" << (pooled ? "sofie_hip_qconv2d_pool_s8" : "sofie_hip_qconv2d_s8") << "(fCtx, tensor_" << fNX << ", "
+          << (fXChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << ", tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, "
+          << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", tensor_" << fNScale << ", tensor_"
+          << (pooled ? fNYPooled : fNY) << ", SOFIE_LAYOUT_NHWC, " << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", "
+          << fShapeX[3] << ", " << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3] << ", " << ph << ", " << pw << ", "
+          << fGeom.strides[0] << ", " << fGeom.strides[1] << ", " << fGeom.group << ", " << fZpX << ", " << fZpY << ", "
+          << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE");
+      if (pooled)
+         out << ", " << fPoolKernel[0] << ", " << fPoolKernel[1] << ", " << fPoolStrides[0] << ", " << fPoolStrides[1];
+      else
+         out << ", SOFIE_OUT_S8";
+      out << "), \"QLinearConv op_" << OpName << "\");\n";
       return out.str();
    }
 };

@@ -4,6 +4,7 @@
 // constructor that reads the text weight file with name/length checks, infer() that runs every
 // operator's Generate() text and returns a std::vector copy of the output.
 #include "SOFIE/RModel.hxx"
+#include "SOFIE/ROperator_Pool.hxx"
 
 #include <cmath>
 #include <fstream>
@@ -203,6 +204,44 @@ void RModel::FuseActivations()
    }
 }
 
+// QLinearConv (with its fused Relu) followed by a pad-free int8 MaxPool that is the only consumer of the
+// activation: the pooling moves into the convolution call, which then writes the pooled tensor only.
+// The unpooled tensors disappear from the model, the Relu and the MaxPool emit nothing.
+void RModel::FusePooling()
+{
+   for (size_t i = 0; i + 1 < fOperators.size(); ++i) {
+      ROperator &conv = *fOperators[i];
+      if (conv.Kind() != "QLinearConv" || conv.GetOpOutputTensors().empty()) continue;
+      std::vector<std::string> chain = {conv.GetOpOutputTensors()[0]};   // tensors that stop existing
+      size_t j = i + 1;
+      if (fOperators[j]->Kind() == "Relu" && fOperators[j]->IsFusedAway() && fOperators[j]->GetOpInputTensors()[0] == chain[0]) {
+         chain.push_back(fOperators[j]->GetOpOutputTensors()[0]);
+         ++j;
+      }
+      if (j >= fOperators.size() || fOperators[j]->Kind() != "Pool") continue;
+      auto *pool = dynamic_cast<ROperator_Pool<float> *>(fOperators[j].get());
+      if (!pool || !pool->IsPlainMaxPool() || pool->TensorType() != ETensorType::INT8) continue;
+      if (pool->GetOpInputTensors()[0] != chain.back()) continue;
+      // nobody else may read the unpooled tensors
+      bool other_use = false;
+      for (auto &t : chain) {
+         if (std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), t) != fOutputTensorNames.end()) other_use = true;
+         for (size_t k = 0; k < fOperators.size() && !other_use; ++k) {
+            if (k == j || (k > i && k < j)) continue;
+            for (auto &in : fOperators[k]->GetOpInputTensors())
+               if (in == t) other_use = true;
+         }
+      }
+      if (other_use) continue;
+      if (!conv.FusePooling(pool->KernelShape(), pool->Strides(), pool->GetOpOutputTensors()[0], pool->OutputShape())) continue;
+      for (size_t k = i + 1; k <= j; ++k) fOperators[k]->SetAbsorbed();
+      for (auto &t : chain) {
+         fIntermediateTensorInfos.erase(t);
+         fChannelsLast.erase(t);
+      }
+   }
+}
+
 std::string RModel::RootOf(const std::string &name) const
 {
    std::string r = name;
@@ -219,6 +258,7 @@ void RModel::PlanIntermediateMemory()
    fViewOf.clear();
    fPlacement.clear();
    for (auto &op : fOperators) {
+      if (op->IsAbsorbed()) continue;
       std::string v = op->IsFusedAway() ? op->GetOpInputTensors()[0] : op->ViewOf();
       if (!v.empty() && !op->GetOpOutputTensors().empty() && fIntermediateTensorInfos.count(v))
          fViewOf[op->GetOpOutputTensors()[0]] = v;
@@ -519,7 +559,7 @@ void RModel::GenerateSessionCode()
    }
    fGC += "){\n";
    for (size_t id = 0; id < fOperators.size(); id++) {
-      if (fOperators[id]->IsFusedAway()) continue;
+      if (fOperators[id]->IsFusedAway() || fOperators[id]->IsAbsorbed()) continue;
       fGC += fOperators[id]->Generate(std::to_string(id));
    }
    fGC += "}\n\n";
@@ -582,6 +622,7 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    (void)pos;
    Initialize(batchSize, verbose);
    FuseActivations();
+   FusePooling();
    PlanIntermediateMemory();
    fGC.clear();
    std::string hgname;

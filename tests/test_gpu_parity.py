@@ -166,6 +166,12 @@ def test_quantize_dequantize(ops):
     assert np.array_equal(ops.maxpool2d(q8, (2, 2), (2, 2)), oracle.maxpool2d(q8, (2, 2), (2, 2)))
     pooled_nhwc = ops.maxpool2d(nhwc, (2, 2), (2, 2), layout=L.LAYOUT_NHWC)
     assert np.array_equal(pooled_nhwc.transpose(0, 3, 1, 2), oracle.maxpool2d(q8, (2, 2), (2, 2)))
+    # channel counts that take the 16-channels-per-thread kernel, with pads and an overlapping window
+    for shape, k, st, p in (((3, 32, 9, 11), (3, 3), (2, 2), (1, 1, 1, 1)), ((2, 48, 8, 8), (2, 2), (2, 2), (0, 0, 0, 0)),
+                            ((1, 16, 5, 7), (3, 2), (1, 2), (1, 0, 0, 1))):
+        q = r.integers(-128, 128, shape).astype(np.int8)
+        got = ops.maxpool2d(np.ascontiguousarray(q.transpose(0, 2, 3, 1)), k, st, p, layout=L.LAYOUT_NHWC)
+        assert np.array_equal(got.transpose(0, 3, 1, 2), oracle.maxpool2d(q, k, st, p))
 
 
 QGEMM_SHAPES = [
