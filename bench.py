@@ -23,6 +23,10 @@ PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA, 5.0 POP/s
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_FP32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes of one call of the headline entry point (B transpose + GEMM), from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE runs scaled by the same counters on a 64 MiB copy-like kernel (FETCH_SIZE x1.999, WRITE_SIZE x1.000):
+# (96.3 + 16.0) MiB for the GEMM kernel + (16.0 + 16.0) MiB for the transpose. Algorithmic bytes: 50.3 MB.
+TRAFFIC_BYTES_PER_CALL = 144.3 * 1024 * 1024
 
 
 def cpu_baseline_int8(A, B, scale, rows):
@@ -108,9 +112,10 @@ def main():
                                "zero-point 0, per-column fp32 scale U[1e-3,1e-2], int32 accumulate, RNE requantise "
                                "to int8, operands resident in HBM", "M": n, "N": n, "K": n, "seed": 0},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_INT8_TOPS, "traffic": None,
+                     "frac": achieved / PEAK_INT8_TOPS, "traffic": TRAFFIC_BYTES_PER_CALL,
                      "kernel": "k_transpose_bytes + k_gemm_dma<MmaI8,128,2,S8>",
                      "kernel_ms": kernel_ms, "ops_per_launch": ops_per_step,
+                     "traffic_unit": "bytes per launch (profiles/int8_gemm_4096_k_gemm_dma.md)",
                      "note": "unit counts an int8 multiply-add as 2 ops (TOP/s); kernel_ms is one call of the "
                              "entry point = B transpose + GEMM kernel"},
     }
@@ -125,6 +130,8 @@ def main():
     else:
         out["cpu_baseline"] = None
 
+    # second half of the metric: the int8 CNN Session at batch 4096 (its own process, runs in about a second)
+    out["model_inferences"] = cnn_session_rate()
     if args.extras:
         out["extras"] = extras(ctx, torch, L, ops, rng)
     print(json.dumps(out))
@@ -182,7 +189,46 @@ def extras(ctx, torch, L, ops, rng):
             cur = h
     ms = time_launches(ctx, mlp, 200, 10)
     ex["mlp_f32_b256"] = {"us": ms * 1e3, "inferences_per_s": 256 / (ms * 1e-3), "gbs": 142112 / (ms * 1e-3) / 1e9}
+    del x, w, b, y
+    # int8 conv layer of the same shape, channels-last, weights [OC][KH][KW][C], bias + ReLU + requantise fused
+    xq = torch.randint(-128, 128, (256, 56, 56, 64), dtype=torch.int8, device=ctx.device)
+    wq = torch.randint(-127, 128, (128, 3, 3, 64), dtype=torch.int8, device=ctx.device)
+    sq = torch.full((128,), 2.0e-4, device=ctx.device)
+    bq = torch.randint(-1000, 1000, (128,), dtype=torch.int32, device=ctx.device)
+    yq = ctx.empty((256, 56, 56, 128), torch.int8)
+    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_qconv2d_s8(
+        ctx.h, ctx.ptr(xq), L.LAYOUT_NHWC, ctx.ptr(wq), L.LAYOUT_NHWC, ctx.ptr(bq), ctx.ptr(sq), ctx.ptr(yq), L.LAYOUT_NHWC,
+        256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, -128, -128, L.ACT_RELU, L.OUT_S8)), 20, 3)
+    ex["conv2d_s8_b256_64to128_56x56"] = {"ms": ms, "tops": fl / ms / 1e9, "frac_peak": fl / ms / 1e9 / PEAK_INT8_TOPS,
+                                          "gbs": (xq.numel() + yq.numel() + wq.numel()) / ms / 1e6}
+    del xq, yq
     return ex
+
+
+def cnn_session_rate(iters=50):
+    """The generated Session of the int8 CNN at batch 4096 (1x40x40 input; conv 1->32, pool, conv 32->64, pool,
+    conv 64->128, fc 12800->256, fc 256->5), run by its prebuilt runner as a child process: device time of
+    infer_device() on a resident input, and wall time of infer() including the PCIe copies."""
+    import subprocess
+    import tempfile
+    gen = os.path.join(ROOT, "sofie_amd", "generated")
+    exe, dat = os.path.join(gen, "run_qcnn_b4096"), os.path.join(gen, "qcnn.dat")
+    if not (os.path.exists(exe) and os.path.exists(dat)):
+        return {"error": "generated Session missing: run build() first"}
+    with tempfile.TemporaryDirectory() as tmp:
+        xin, yout = os.path.join(tmp, "x.bin"), os.path.join(tmp, "y.bin")
+        np.random.default_rng(2).uniform(0, 1, (4096, 1, 40, 40)).astype(np.float32).tofile(xin)
+        res = subprocess.run([exe, dat, xin, yout, str(iters)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                             timeout=300)
+    if res.returncode != 0:
+        return {"error": res.stderr.strip()[-300:]}
+    t = json.loads(res.stdout.strip().splitlines()[-1])
+    ops_per_image = 36968960.0
+    return {"workload": "int8 CNN classifier, batch 4096, 1x40x40 input, generated Session (infer_device on a resident input)",
+            "device_ms": t["device_ms"], "inferences_per_s": 4096 / (t["device_ms"] * 1e-3),
+            "tops": 4096 * ops_per_image / t["device_ms"] / 1e9,
+            "frac_peak": 4096 * ops_per_image / t["device_ms"] / 1e9 / PEAK_INT8_TOPS,
+            "host_ms_with_pcie": t["host_ms"], "inferences_per_s_with_pcie": 4096 / (t["host_ms"] * 1e-3)}
 
 
 if __name__ == "__main__":
