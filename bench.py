@@ -60,6 +60,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=1024)
     ap.add_argument("--extras", action="store_true", help="also time the FP8 GEMM, fp32 GEMM and conv layers")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="launch a 64 MiB copy-like kernel and the headline call three times and exit (the target of the "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collective, no sharding "
@@ -85,6 +88,15 @@ def main():
         # scratch buffer on every call (a Session would do that once, see extras.int8_gemm_4096_transB).
         ctx.check(ctx.lib.sofie_hip_qgemm_s8(ctx.h, 0, n, n, n, ctx.ptr(dA), n, ctx.ptr(dB), n, ctx.ptr(dS), None,
                                              0, L.ACT_NONE, ctx.ptr(dY), n, L.OUT_S8))
+
+    if args.traffic_probe:
+        X = torch.randn(16 * 1024 * 1024, device=ctx.device)      # the ReLU kernel reads 64 MiB and writes 64 MiB
+        Z = torch.empty_like(X)
+        for _ in range(3):
+            ctx.check(ctx.lib.sofie_hip_relu_f32(ctx.h, ctx.ptr(X), ctx.ptr(Z), X.numel()))
+            step()
+        torch.cuda.synchronize()
+        return
 
     # warm-up, then EXACTLY `steps` timed steps bracketed by device synchronisation
     for _ in range(args.warmup):
