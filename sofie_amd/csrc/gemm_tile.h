@@ -95,8 +95,8 @@ __device__ __forceinline__ unsigned epilogue_value(const GemmArgs &g, float sc, 
 //     wavefront's first column, filled and made visible by the caller;
 //   m_wave, n_wave: first output row and column of this wavefront.
 // ADD_BIAS false: the accumulators already include the bias.
-// PLAIN: int8 output with zero-point -128 and lower clamp -128 (the saturating byte
-// conversion does the clamping, two instructions per element fewer).
+// PLAIN: int8 output with zero-point -128 and lower clamp -128: the byte conversion rounds half to
+// even and saturates, so it is the whole requantisation after the multiply.
 template <int TI, int OUT> struct EpilogueStaging {
    static constexpr int ESZ = OutSize<OUT>::value;
    static constexpr int SROW = TI * 32 * ESZ + 16;   // staging row stride in bytes
@@ -147,8 +147,9 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
             float e[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-               float r = rintf(__fmul_rn(__int2float_rn(acc[i][j][q * 4 + t] + (ADD_BIAS ? bi[t] : 0)), sc[t]));
-               if constexpr (!PLAIN) r = fmaxf(__fadd_rn(r, zpo), lof);
+               float r = __fmul_rn(__int2float_rn(acc[i][j][q * 4 + t] + (ADD_BIAS ? bi[t] : 0)), sc[t]);
+               // v_cvt_pk_u8_f32 itself rounds to nearest even: with nothing to add, the product goes in as it is
+               if constexpr (!PLAIN) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
                e[t] = r;
             }
             pk = __builtin_amdgcn_cvt_pk_u8_f32(e[0], 0, pk);

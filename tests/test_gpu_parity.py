@@ -252,6 +252,31 @@ def test_qgemm_s8_full_size_properties(ops):
     assert np.array_equal(acc_t, acc)
 
 
+def test_qgemm_rounding_ties_and_saturation(ops):
+    """Scale 0.5 (and 0.25, 1.5) makes every odd accumulator an exact tie; the byte-packing epilogues must round
+    them half to even like the oracle, for the zero-point -128 path (conversion instruction does the rounding)
+    and for a general zero-point, and saturate at both ends."""
+    M, N, K = 256, 256, 64
+    A = np.zeros((M, K), np.int8)
+    A[:, 0] = (np.arange(M) - 128).clip(-128, 127)
+    A[:, 1] = 1
+    B = np.zeros((K, N), np.int8)
+    B[0, :] = 1
+    B[1, :] = (np.arange(N) % 7) - 3                 # acc[m,n] = (m - 128) + (n % 7 - 3)
+    B[2:, :] = 5                                      # multiplied by zeros of A
+    for sval in (0.5, 0.25, 1.5, 2.5):
+        scale = np.full(N, sval, np.float32)
+        bias = (np.arange(N) % 3).astype(np.int32)
+        for zpy, relu in ((-128, False), (-128, True), (3, False), (-5, True)):
+            ref = oracle.qgemm_s8(A, B, scale, bias, False, zpy=zpy, relu=relu)
+            assert np.array_equal(ops.qgemm_s8(A, B, scale, bias, zpy=zpy, relu=relu), ref), (sval, zpy, relu)
+            Bt = np.ascontiguousarray(B.T)
+            assert np.array_equal(ops.qgemm_s8(A, Bt, scale, bias, transB=True, zpy=zpy, relu=relu), ref)
+    # the accumulators really contain ties
+    acc = oracle.igemm_s8(A, B)
+    assert np.any((acc % 2) != 0)
+
+
 @pytest.mark.parametrize("cfg", [
     dict(N=2, C=6, H=7, W=6, OC=8, k=(3, 3), p=(1, 1), s=(1, 1), g=2),
     dict(N=1, C=1, H=40, W=40, OC=32, k=(3, 3), p=(1, 1), s=(1, 1), g=1),
