@@ -105,11 +105,19 @@ struct QConvTileArgs {
    FastDiv dOW, dOH, dHP, dRL, dC16;
 };
 
-template <int MB, int NB, int WN, int PF, int OUT>
+// POOL: a 2x2 stride-2 max pooling is fused. A wavefront then owns 32 POOLED pixels; its MB = 4
+// accumulator tiles along m are the four positions of the pooling window, so the pooling is a
+// register-wise maximum over the four tiles (on the int32 accumulators: the requantisation is monotonic;
+// for a negative scale the minimum is taken) and only a quarter of the values is converted and stored.
+// In that mode the "pixels" the tiles, the epilogue and a.OH / a.OW / a.ep.M count are pooled pixels.
+template <int MB, int NB, int WN, int PF, int OUT, bool POOL>
 __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 {
+   static_assert(!POOL || MB == 4, "the four window positions are the four m tiles");
    constexpr int WM = 8 / WN;
-   constexpr int TM = WM * MB * 32;
+   constexpr int MBP = POOL ? 1 : MB;                 // m tiles of 32 (pooled) pixels per wavefront
+   constexpr int TM = WM * MBP * 32;                  // (pooled) pixels per workgroup tile
+   constexpr int RPP = POOL ? 2 : 1;                  // convolution rows per (pooled) row
    constexpr int OCT = WN * NB * 32;
    extern __shared__ __align__(16) unsigned char smem[];
    constexpr int WB = EpilogueStaging<NB, OUT>::WAVE_BYTES;
@@ -160,8 +168,8 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
       const int R0 = fdiv(m0, a.dOW), R1 = fdiv(mlast, a.dOW);
       const int n0 = fdiv(R0, a.dOH), n1 = fdiv(R1, a.dOH);
       Band b;
-      b.vr_lo = n0 * a.HP + (R0 - n0 * a.OH) * a.sh;
-      b.rows = n1 * a.HP + (R1 - n1 * a.OH) * a.sh + a.KH - b.vr_lo;
+      b.vr_lo = n0 * a.HP + (R0 - n0 * a.OH) * RPP * a.sh;
+      b.rows = n1 * a.HP + ((R1 - n1 * a.OH) * RPP + RPP - 1) * a.sh + a.KH - b.vr_lo;
       return b;
    };
    v4i pre[PF];
@@ -205,15 +213,27 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    // LDS offsets of the wavefront's pixels inside the band of tile tt
    int a_off[MB];
    auto pixel_offsets = [&](int tt, int vr_lo) {
-#pragma unroll
-      for (int j = 0; j < MB; ++j) {
-         int m = tt * TM + (wm * MB + j) * 32 + l32;
+      if constexpr (POOL) {
+         int m = tt * TM + wm * 32 + l32;
          m = m < mtot ? m : mtot - 1;
          const int R = fdiv(m, a.dOW);
-         const int ow = m - R * a.OW;
+         const int pw_ = m - R * a.OW;
          const int n = fdiv(R, a.dOH);
-         const int v = n * a.HP + (R - n * a.OH) * a.sh - vr_lo;
-         a_off[j] = (v * a.WP + ow * a.sw) * a.CS + half * 16;
+         const int v = n * a.HP + (R - n * a.OH) * 2 * a.sh - vr_lo;
+#pragma unroll
+         for (int j = 0; j < 4; ++j)
+            a_off[j] = ((v + (j >> 1) * a.sh) * a.WP + (2 * pw_ + (j & 1)) * a.sw) * a.CS + half * 16;
+      } else {
+#pragma unroll
+         for (int j = 0; j < MB; ++j) {
+            int m = tt * TM + (wm * MB + j) * 32 + l32;
+            m = m < mtot ? m : mtot - 1;
+            const int R = fdiv(m, a.dOW);
+            const int ow = m - R * a.OW;
+            const int n = fdiv(R, a.dOH);
+            const int v = n * a.HP + (R - n * a.OH) * a.sh - vr_lo;
+            a_off[j] = (v * a.WP + ow * a.sw) * a.CS + half * 16;
+         }
       }
    };
 
@@ -266,15 +286,40 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
       }
       if (s < nsteps) mma(0);
    };
-   v4f r_scale[NB * 4];    // the lane's scales, loaded once (after the first barrier)
+   // the lane's scales, loaded once (after the first barrier); the pooled variant needs the registers for
+   // its four accumulator tiles and reads the scales from LDS instead
+   v4f r_scale[POOL ? 1 : NB * 4];
    auto epilogue = [&](v16i (&acc)[NB][MB], int tt) {
-      const int m_wave = tt * TM + wm * MB * 32, n_wave = ob * OCT + wn * NB * 32;
-      if (plain)
-         tile_epilogue_wave<MmaI8, NB, MB, OUT, true, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
-                                                                   n_wave, &r_scale);
-      else
-         tile_epilogue_wave<MmaI8, NB, MB, OUT, false, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
-                                                                    n_wave, &r_scale);
+      const int m_wave = tt * TM + wm * MBP * 32, n_wave = ob * OCT + wn * NB * 32;
+      if constexpr (POOL) {
+         v16i pooled[NB][1];
+#pragma unroll
+         for (int i = 0; i < NB; ++i)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+               const v4f sc = *reinterpret_cast<const v4f *>(w_scale + i * 32 + q * 8 + nq);
+#pragma unroll
+               for (int t = 0; t < 4; ++t) {
+                  const int e = q * 4 + t;
+                  const int hi = max(max(acc[i][0][e], acc[i][1][e]), max(acc[i][2][e], acc[i][3][e]));
+                  const int lo = min(min(acc[i][0][e], acc[i][1][e]), min(acc[i][2][e], acc[i][3][e]));
+                  pooled[i][0][e] = sc[t] < 0.0f ? lo : hi;
+               }
+            }
+         if (plain)
+            tile_epilogue_wave<MmaI8, NB, 1, OUT, true, false, true>(a.ep, pooled, w_stg, w_scale, w_bias, lane, m_wave,
+                                                                     n_wave);
+         else
+            tile_epilogue_wave<MmaI8, NB, 1, OUT, false, false, true>(a.ep, pooled, w_stg, w_scale, w_bias, lane, m_wave,
+                                                                      n_wave);
+      } else {
+         if (plain)
+            tile_epilogue_wave<MmaI8, NB, MB, OUT, true, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
+                                                                      n_wave, &r_scale);
+         else
+            tile_epilogue_wave<MmaI8, NB, MB, OUT, false, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
+                                                                       n_wave, &r_scale);
+      }
    };
 
    // One tile per iteration. The two wavefronts that share a SIMD do their halves in opposite order:
@@ -290,9 +335,11 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
       pixel_offsets(t, cur.vr_lo);
    }
    __syncthreads();   // weights and column parameters are in LDS
+   if constexpr (!POOL) {
 #pragma unroll
-   for (int gi = 0; gi < NB * 4; ++gi)
-      r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+      for (int gi = 0; gi < NB * 4; ++gi)
+         r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+   }
    v16i acc[NB][MB];
    while (t < a.ntiles) {
       stash(cur);
@@ -317,21 +364,27 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    if (!mma_first && t_prev >= 0) epilogue(acc, t_prev);
 }
 
-// Launches the MFMA kernel if the problem fits it; *done tells whether it did.
+// Launches the MFMA kernel if the problem fits it; *done tells whether it did. With g.pool_kh != 0 only the
+// kernel with the fused 2x2 stride-2 pooling is considered.
 template <int OUT>
 int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
 {
    *done = false;
-   constexpr int ESZ = OutSize<OUT>::value;
+   const bool pool = g.pool_kh != 0;
    if (g.groups != 1 || g.C % 32 != 0 || g.OC % 64 != 0 || !g.x_nhwc || !g.y_nhwc || !g.w_ohwi) return SOFIE_HIP_OK;
    if (!aligned16(g.x) || !aligned16(g.w) || !aligned16(g.y)) return SOFIE_HIP_OK;
-   const long long mtot = (long long)g.N * g.OH * g.OW;
+   if (pool && !(OUT == SOFIE_OUT_S8 && g.pool_kh == 2 && g.pool_kw == 2 && g.pool_sh == 2 && g.pool_sw == 2)) return SOFIE_HIP_OK;
+   // rows and columns the tiles count: pooled pixels when the pooling is fused
+   const int TH = pool ? g.PH : g.OH, TW = pool ? g.PW : g.OW;
+   const int rpp = pool ? 2 : 1;                      // convolution rows per tile row
+   const long long mtot = (long long)g.N * TH * TW;
    const int HP = g.H + 2 * g.ph, WP = g.W + 2 * g.pw;
+   if (mtot <= 0) return SOFIE_HIP_OK;
    if (mtot >= (1ll << 31) - 1024 || (long long)g.N * HP >= (1ll << 31) - 4096) return SOFIE_HIP_OK;
    if ((size_t)g.N * g.H * g.W * g.C >= ((size_t)1 << 40)) return SOFIE_HIP_OK;
    const int WN = g.OC % 128 == 0 ? 2 : 1;
    const int OCT = WN * 64;
-   const int TM = (8 / WN) * 64;
+   const int TM = pool ? (8 / WN) * 32 : (8 / WN) * 64;
    QConvTileArgs a{};
    a.x = g.x; a.w = g.w;
    a.ep.Y = g.y; a.ep.scale = g.scale; a.ep.bias = g.bias;
@@ -339,7 +392,7 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.ep.zp = g.zpy; a.ep.lo = g.lo; a.ep.relu = g.relu; a.ep.s = 1.0f;
    a.ep.vec_store = 1;   // OC % 64 == 0 and y 16-byte aligned
    a.H = g.H; a.W = g.W; a.C = g.C; a.KH = g.KH; a.KW = g.KW; a.ph = g.ph; a.pw = g.pw; a.sh = g.sh; a.sw = g.sw;
-   a.OH = g.OH; a.OW = g.OW; a.HP = HP; a.WP = WP;
+   a.OH = TH; a.OW = TW; a.HP = HP; a.WP = WP;
    a.K = g.KH * g.KW * g.C;
    a.KS = ((a.K / 16) % 2 == 0) ? a.K + 16 : a.K;
    a.CS = ((g.C / 16) % 2 == 0) ? g.C + 16 : g.C;
@@ -349,16 +402,16 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.RP = 512 / a.RL;
    a.ntiles = (int)((mtot + TM - 1) / TM);
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
-   a.dOW = make_fastdiv(g.OW); a.dOH = make_fastdiv(g.OH); a.dHP = make_fastdiv(HP);
+   a.dOW = make_fastdiv(TW); a.dOH = make_fastdiv(TH); a.dHP = make_fastdiv(HP);
    a.dRL = make_fastdiv(a.RL); a.dC16 = make_fastdiv(a.C16);
-   // most rows a band can have: the output rows a tile touches, the image boundaries it can cross
+   // most rows a band can have: the convolution rows a tile touches, the image boundaries it can cross
    // (each adds the rows between the last window of one image and the first of the next) and KH - 1
-   const int out_rows = (TM - 1) / g.OW + 2;
-   int gap = HP - g.OH * g.sh;
+   const int tile_rows = (TM - 1) / TW + 2;
+   int gap = HP - TH * rpp * g.sh;
    if (gap < 0) gap = 0;
-   int crossings = (out_rows - 1) / g.OH + 1;
+   int crossings = (tile_rows - 1) / TH + 1;
    if (crossings > g.N - 1) crossings = g.N - 1;
-   const long long rows_max = (long long)(out_rows - 1) * g.sh + (long long)crossings * gap + g.KH;
+   const long long rows_max = (long long)(tile_rows * rpp - 1) * g.sh + (long long)crossings * gap + g.KH;
    const int passes = (int)((rows_max + a.RP - 1) / a.RP);
    if (passes > 12) return SOFIE_HIP_OK;
    const size_t band = (size_t)rows_max * WP * a.CS;
@@ -371,25 +424,30 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (per < 1) per = 1;
    if (per > a.ntiles) per = a.ntiles;
    const dim3 grid((unsigned)(per * nob)), block(512);
-#define SOFIE_QCONV_LAUNCH(WN_, PF_)                                                                          \
+#define SOFIE_QCONV_LAUNCH(MB_, WN_, PF_, POOL_)                                                              \
    do {                                                                                                       \
-      auto kern = k_qconv_mfma<2, 2, WN_, PF_, OUT>;                                                          \
+      auto kern = k_qconv_mfma<MB_, 2, WN_, PF_, OUT, POOL_>;                                                 \
       SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));         \
       hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                             \
    } while (0)
-#define SOFIE_QCONV_BY_PASSES(WN_)                                                                            \
+#define SOFIE_QCONV_BY_PASSES(MB_, WN_, POOL_)                                                                \
    do {                                                                                                       \
-      if constexpr (OUT != SOFIE_OUT_S8) SOFIE_QCONV_LAUNCH(WN_, 12); /* raw accumulators: not tuned */      \
-      else if (passes <= 3) SOFIE_QCONV_LAUNCH(WN_, 3);                                                       \
-      else if (passes <= 4) SOFIE_QCONV_LAUNCH(WN_, 4);                                                       \
-      else if (passes <= 5) SOFIE_QCONV_LAUNCH(WN_, 5);                                                       \
-      else if (passes <= 6) SOFIE_QCONV_LAUNCH(WN_, 6);                                                       \
-      else if (passes <= 8) SOFIE_QCONV_LAUNCH(WN_, 8);                                                       \
-      else SOFIE_QCONV_LAUNCH(WN_, 12);                                                                       \
+      if constexpr (OUT != SOFIE_OUT_S8) SOFIE_QCONV_LAUNCH(2, WN_, 12, false); /* raw accumulators: not tuned */ \
+      else if (passes <= 3) SOFIE_QCONV_LAUNCH(MB_, WN_, 3, POOL_);                                           \
+      else if (passes <= 4) SOFIE_QCONV_LAUNCH(MB_, WN_, 4, POOL_);                                           \
+      else if (passes <= 5) SOFIE_QCONV_LAUNCH(MB_, WN_, 5, POOL_);                                           \
+      else if (passes <= 6) SOFIE_QCONV_LAUNCH(MB_, WN_, 6, POOL_);                                           \
+      else if (passes <= 8) SOFIE_QCONV_LAUNCH(MB_, WN_, 8, POOL_);                                           \
+      else SOFIE_QCONV_LAUNCH(MB_, WN_, 12, POOL_);                                                           \
    } while (0)
-   if (WN == 2) SOFIE_QCONV_BY_PASSES(2);
-   else SOFIE_QCONV_BY_PASSES(1);
+   if (pool) {
+      if (WN == 2) SOFIE_QCONV_BY_PASSES(4, 2, true);
+      else SOFIE_QCONV_BY_PASSES(4, 1, true);
+   } else {
+      if (WN == 2) SOFIE_QCONV_BY_PASSES(2, 2, false);
+      else SOFIE_QCONV_BY_PASSES(2, 1, false);
+   }
 #undef SOFIE_QCONV_BY_PASSES
 #undef SOFIE_QCONV_LAUNCH
    *done = true;
@@ -463,6 +521,8 @@ int run(sofie_hip_ctx *ctx, const QConvArgs &g)
    // pooling kernel reads it from there
    bool done = false;
    if (int rc = qconv_first_layer(ctx, g, &done)) return rc;
+   if (done) return SOFIE_HIP_OK;
+   if (int rc = launch_mfma<OUT>(ctx, g, &done)) return rc;
    if (done) return SOFIE_HIP_OK;
    QConvArgs h = g;
    h.pool_kh = h.pool_kw = h.pool_sh = h.pool_sw = 0;

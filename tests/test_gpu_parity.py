@@ -394,6 +394,34 @@ def test_conv_pool_entry_point(ops, cfg):
     assert np.array_equal(yh.transpose(0, 3, 1, 2), ref)
 
 
+@pytest.mark.parametrize("cfg", [
+    dict(N=5, C=32, H=20, W=20, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),      # the CNN's second layer
+    dict(N=3, C=64, H=11, W=13, OC=128, k=(3, 3), p=(1, 1), s=(1, 1)),     # odd output size: last row / column dropped
+    dict(N=70, C=32, H=4, W=6, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),       # many small images per tile
+    dict(N=2, C=32, H=17, W=9, OC=192, k=(1, 1), p=(0, 0), s=(1, 1)),
+    dict(N=2, C=64, H=21, W=21, OC=64, k=(3, 3), p=(0, 0), s=(2, 2)),      # strided convolution before the pool
+    dict(N=1, C=32, H=2, W=2, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),        # a single pooled pixel
+])
+def test_conv_pool_fused_matrix_core_kernel(ops, cfg):
+    """Channels-last operands with a 2x2 stride-2 pooling: one kernel whose wavefronts pool on the accumulators.
+    Scales of both signs (maximum / minimum of the accumulators), both zero-point conventions."""
+    from sofie_amd import lib as L
+    r = rng(800 + cfg["C"] + cfg["H"])
+    x = r.integers(-128, 128, (cfg["N"], cfg["C"], cfg["H"], cfg["W"])).astype(np.int8)
+    w = r.integers(-127, 128, (cfg["OC"], cfg["C"]) + cfg["k"]).astype(np.int8)
+    K = cfg["C"] * cfg["k"][0] * cfg["k"][1]
+    scale = (r.uniform(20, 60, cfg["OC"]) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    scale[1::5] *= -1
+    bias = r.integers(-3000, 3000, cfg["OC"]).astype(np.int32)
+    xh = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    wh = np.ascontiguousarray(w.transpose(0, 2, 3, 1))
+    for zpx, zpy, relu in ((-128, -128, True), (7, -20, False), (0, 5, True)):
+        ref = oracle.maxpool2d(oracle.qconv2d_s8(x, w, scale, bias, cfg["p"], cfg["s"], 1, zpx, zpy, relu), (2, 2), (2, 2))
+        y = ops.qconv2d_pool_s8(xh, wh, scale, bias, cfg["p"], cfg["s"], 1, zpx, zpy, relu, x_layout=L.LAYOUT_NHWC,
+                                y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+        assert np.array_equal(y.transpose(0, 3, 1, 2), ref), (zpx, zpy, relu)
+
+
 # --------------------------------------------------------------------------- fp8
 def fp8_operands(r, M, N, K, transB):
     a = r.standard_normal((M, K)).astype(np.float32)
