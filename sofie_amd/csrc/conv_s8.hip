@@ -72,26 +72,6 @@ __global__ void k_qconv_simple(QConvArgs g)
 }
 
 // ------------------------------------------------------------------------------ MFMA path
-// floor(x / d) for 0 <= x < 2^31 as a multiply-high and a shift (shift < 0: d == 1).
-struct FastDiv {
-   unsigned magic;
-   int shift;
-};
-
-FastDiv make_fastdiv(unsigned d)
-{
-   if (d <= 1) return {0u, -1};
-   int s = 0;
-   while ((1u << s) < d) ++s;
-   const unsigned long long num = 1ull << (31 + s);
-   return {(unsigned)((num + d - 1) / d), s - 1};
-}
-
-__device__ __forceinline__ int fdiv(int x, FastDiv f)
-{
-   return f.shift < 0 ? x : (int)(__umulhi((unsigned)x, f.magic) >> f.shift);
-}
-
 struct QConvTileArgs {
    const int8_t *x;      // NHWC
    const int8_t *w;      // [OC][KH][KW][C]

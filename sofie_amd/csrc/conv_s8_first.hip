@@ -1,15 +1,17 @@
 // First layer of an int8 CNN: one input channel, 3x3 kernel, stride 1, padding 1, with the
 // requantisation, the ReLU clamp and (optionally) a 2x2 stride-2 max pooling fused.
 //
-// With K = 9 the layer is bound by its output bytes, not by arithmetic, so it runs on the vector
-// ALUs: one workgroup per image keeps the zero-point-padded image in LDS; a work item is one output
-// pixel (or one pooled pixel = 2x2 output pixels) times all output channels. A kernel row of three
-// taps plus a zero is one packed dword, so an output pixel costs three v_dot4_i32_i8 per channel on
-// the packed rows of its window (unaligned 4-byte windows are cut out of two aligned dwords with
-// v_alignbyte). Pooling is taken on the int32 accumulators: requantisation is monotonic in the
-// accumulator (non-decreasing for scale >= 0, non-increasing for scale < 0), so the maximum of the
-// requantised values is the requantised maximum (minimum for a negative scale), which equals
-// pooling after requantisation bit for bit and needs a quarter of the conversions.
+// With K = 9 the layer is bound by its output bytes, so the point is to spend few vector instructions
+// per output. A workgroup keeps four zero-point-padded images in LDS; a wavefront takes 32 (pooled)
+// pixels at a time and computes them with v_mfma_i32_32x32x16_i8, K = 16 laid out as the three
+// kernel rows of four bytes (three taps and a zero weight) plus four zero weights. With that order the
+// pixel operand of a lane is simply two 4-byte windows of consecutive image rows (lanes 0-31: rows
+// y, y+1; lanes 32-63: rows y+2, y+3), cut out of aligned dwords with v_alignbyte; no byte shuffling.
+// For the pooled variant the four window positions are four matrix instructions whose accumulators are
+// pooled register-wise (on the int32 values: requantisation is monotonic in the accumulator; if any
+// scale of the workgroup's channels is negative, the minimum is taken for those channels), so a quarter
+// of the values is converted. Two v_permlane32_swap turn the lane's four 4-channel groups into 16
+// consecutive channels and the result leaves as one 16-byte store per lane.
 #include "conv_s8.h"
 
 using namespace sofie;
@@ -22,90 +24,207 @@ struct FirstArgs {
    const int32_t *bias;   // [OC] or null
    const float *scale;    // [OC]
    int8_t *y;             // [N][PH][PW][OC]
-   int H, W, OC, PH, PW;
+   int N, H, W, OC, PH, PW;
    int zpx, zpy, lo;
-   int stride;            // LDS row stride of the padded image, a multiple of 4
+   int stride;            // LDS row stride of a padded image, a multiple of 4
+   int img_bytes;         // LDS bytes of one padded image
+   int ocb;               // blocks of 32 output channels (the last may be half used)
+   int rows;              // LDS rows of one padded image (H + 3)
+   int dword_fill;        // W % 4 == 0 and x 4-byte aligned: the images are filled a dword at a time
+   FastDiv drows, dper_image, dPW;
 };
 
-__device__ __forceinline__ int window4(const unsigned char *row, int col)
+constexpr int kImages = 4;   // images per workgroup
+
+__device__ __forceinline__ void windows(const unsigned char *row, int col, int &w0, int &w1)
 {
-   // bytes col .. col+3 of an LDS row whose base is 4-byte aligned
+   // bytes col..col+3 and col+1..col+4 of an LDS row whose base is 4-byte aligned (col even)
+   const int *p = reinterpret_cast<const int *>(row + (col & ~3));
+   const unsigned lo = (unsigned)p[0], hi = (unsigned)p[1];
+   w0 = (int)__builtin_amdgcn_alignbyte(hi, lo, (unsigned)(col & 3));
+   w1 = (int)__builtin_amdgcn_alignbyte(hi, lo, (unsigned)(col & 3) + 1u);
+}
+
+__device__ __forceinline__ int window(const unsigned char *row, int col)
+{
    const int *p = reinterpret_cast<const int *>(row + (col & ~3));
    return (int)__builtin_amdgcn_alignbyte((unsigned)p[1], (unsigned)p[0], (unsigned)(col & 3));
 }
 
+__device__ __forceinline__ long pack64(int lo, int hi)
+{
+   return (long)(((unsigned long long)(unsigned)hi << 32) | (unsigned long long)(unsigned)lo);
+}
+
 template <bool POOL>
-__global__ void __launch_bounds__(256) k_qconv_first(FirstArgs a)
+__global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
 {
    extern __shared__ __align__(16) unsigned char smem[];
-   v4i *const s_w = reinterpret_cast<v4i *>(smem);                         // [OC] {row0, row1, row2, bias}
-   float *const s_scale = reinterpret_cast<float *>(smem + a.OC * 16);     // [OC]
-   unsigned char *const s_img = smem + a.OC * 20;                          // [(H+2)][stride] (+8 bytes slack)
-   const int tid = threadIdx.x;
-   const int n = blockIdx.x;
+   const int OCP = a.ocb * 32;                                              // channels padded to blocks of 32
+   float *const s_scale = reinterpret_cast<float *>(smem);                  // [OCP]
+   int *const s_bias = reinterpret_cast<int *>(s_scale + OCP);              // [OCP]
+   long *const s_wfrag = reinterpret_cast<long *>(s_bias + OCP);            // [OCP][2] matrix operand of the weights
+   int *const s_flag = reinterpret_cast<int *>(s_wfrag + OCP * 2);          // [4] any negative scale
+   unsigned char *const s_img = reinterpret_cast<unsigned char *>(s_flag + 4);
+   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int half = lane >> 5, l32 = lane & 31;
+   const int n0 = blockIdx.x * kImages;
+   const int nimg = (a.N - n0) < kImages ? (a.N - n0) : kImages;
 
-   for (int oc = tid; oc < a.OC; oc += 256) {
+   if (tid == 0) s_flag[0] = 0;
+   __syncthreads();
+   for (int oc = tid; oc < OCP; oc += 256) {
+      const bool real = oc < a.OC;
       const int8_t *w = a.w + oc * 9;
-      v4i t;
+      unsigned r[3] = {0u, 0u, 0u};
+      if (real) {
 #pragma unroll
-      for (int r = 0; r < 3; ++r)
-         t[r] = (int)((unsigned)(unsigned char)w[r * 3] | ((unsigned)(unsigned char)w[r * 3 + 1] << 8) |
-                      ((unsigned)(unsigned char)w[r * 3 + 2] << 16));
-      t[3] = a.bias ? a.bias[oc] : 0;
-      s_w[oc] = t;
-      s_scale[oc] = a.scale[oc];
+         for (int k = 0; k < 3; ++k)
+            r[k] = (unsigned)(unsigned char)w[k * 3] | ((unsigned)(unsigned char)w[k * 3 + 1] << 8) |
+                   ((unsigned)(unsigned char)w[k * 3 + 2] << 16);
+      }
+      s_wfrag[oc * 2] = pack64((int)r[0], (int)r[1]);      // lanes 0-31: kernel rows 0 and 1
+      s_wfrag[oc * 2 + 1] = pack64((int)r[2], 0);          // lanes 32-63: kernel row 2 and four zero weights
+      const float sc = real ? a.scale[oc] : 0.0f;
+      s_scale[oc] = sc;
+      s_bias[oc] = (real && a.bias) ? a.bias[oc] : 0;
+      if (sc < 0.0f) s_flag[0] = 1;
    }
-   // padded image: border cells hold the input zero-point
-   {
-      const int8_t *img = a.x + (size_t)n * a.H * a.W;
-      const int cells = (a.H + 2) * a.stride + 8;
-      for (int i = tid; i < cells; i += 256) {
-         const int r = i / a.stride, c = i - r * a.stride;
+   // padded images: border cells hold the input zero-point; one spare row below each image is read (with
+   // zero weights) by the upper half of the wavefront
+   if (a.dword_fill) {
+      // LDS dword j of a row = padded columns 4j..4j+3 = image columns 4j-1..4j+2: the last byte of image
+      // dword j-1 and the first three of image dword j. 16 threads per row, 16 rows per pass.
+      const int SD = a.stride >> 2, WD = a.W >> 2;
+      const unsigned zp4 = 0x01010101u * (unsigned)(a.zpx & 0xff);
+      const int jj = tid & 15, rsub = tid >> 4;
+      const int total_rows = nimg * a.rows;
+      constexpr int UN = 6;   // rows per thread whose loads are in flight together
+      for (int j = jj; j < SD; j += 16) {
+         for (int base = 0; base < total_rows; base += 16 * UN) {
+            unsigned lo[UN], hi[UN];
+            bool has_lo[UN], has_hi[UN];
+            unsigned *dst[UN];
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+               const int row_id = base + u * 16 + rsub;
+               const int rid = row_id < total_rows ? row_id : total_rows - 1;
+               const int im = fdiv(rid, a.drows);
+               const int ih = rid - im * a.rows - 1;
+               const bool row_inside = row_id < total_rows && ih >= 0 && ih < a.H;
+               const unsigned *gsrc =
+                  reinterpret_cast<const unsigned *>(a.x + ((size_t)(n0 + im) * a.H + (row_inside ? ih : 0)) * a.W);
+               dst[u] = row_id < total_rows
+                           ? reinterpret_cast<unsigned *>(s_img + im * a.img_bytes + (rid - im * a.rows) * a.stride) + j
+                           : nullptr;
+               has_lo[u] = row_inside && j >= 1 && j - 1 < WD;
+               has_hi[u] = row_inside && j < WD;
+               lo[u] = gsrc[has_lo[u] ? j - 1 : 0];
+               hi[u] = gsrc[has_hi[u] ? j : 0];
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u)
+               if (dst[u]) *dst[u] = __builtin_amdgcn_alignbyte(has_hi[u] ? hi[u] : zp4, has_lo[u] ? lo[u] : zp4, 3u);
+         }
+      }
+   } else {
+      for (int i = tid; i < nimg * a.img_bytes; i += 256) {
+         const int im = i / a.img_bytes, o = i - im * a.img_bytes;
+         const int r = o / a.stride, c = o - r * a.stride;
          const int ih = r - 1, iw = c - 1;
          const bool inside = ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-         s_img[i] = inside ? (unsigned char)img[ih * a.W + iw] : (unsigned char)a.zpx;
+         s_img[i] = inside ? (unsigned char)a.x[((size_t)(n0 + im) * a.H + ih) * a.W + iw] : (unsigned char)a.zpx;
       }
    }
    __syncthreads();
+   const bool any_negative = s_flag[0] != 0;
 
    const float zpo = (float)(a.zpy + 128), lof = (float)(a.lo + 128);
-   const int items = a.PH * a.PW;
-   for (int it = tid; it < items; it += 256) {
-      const int py = it / a.PW, px = it - py * a.PW;
-      constexpr int NR = POOL ? 4 : 3, ND = POOL ? 2 : 1;
-      const int oy = POOL ? 2 * py : py, ox = POOL ? 2 * px : px;
-      int rows[NR][ND];
+   const bool plain = a.zpy == -128 && a.lo == -128;
+   const int per_image = a.PH * a.PW;
+   const int total = nimg * per_image;
+   const int groups = (total + 31) / 32;
+   constexpr int NP = POOL ? 4 : 1;               // matrix instructions (window positions) per group
+   // weight operand, bias and scales of a block of 32 channels: register e of a tile belongs to channel
+   // (e/4)*8 + half*4 + e%4. With one block they are loaded once.
+   long wfrag = 0;
+   v16i binit;
+   v16i zero16;
 #pragma unroll
-      for (int r = 0; r < NR; ++r) {
-         const unsigned char *row = s_img + (oy + r) * a.stride;
+   for (int e = 0; e < 16; ++e) zero16[e] = 0;
+   v4f sc[4];
+   auto load_params = [&](int ob) {
+      wfrag = s_wfrag[(ob * 32 + l32) * 2 + half];
 #pragma unroll
-         for (int d = 0; d < ND; ++d) rows[r][d] = window4(row, ox + d);
+      for (int gq = 0; gq < 4; ++gq) {
+         const v4i b = *reinterpret_cast<const v4i *>(s_bias + ob * 32 + gq * 8 + half * 4);
+         sc[gq] = *reinterpret_cast<const v4f *>(s_scale + ob * 32 + gq * 8 + half * 4);
+#pragma unroll
+         for (int t = 0; t < 4; ++t) binit[gq * 4 + t] = b[t];
       }
-      int8_t *out = a.y + ((size_t)(n * a.PH + py) * a.PW + px) * a.OC;
-      for (int oc0 = 0; oc0 < a.OC; oc0 += 4) {
-         unsigned pk = 0;
+   };
+   const bool single = a.ocb == 1;
+   load_params(0);
+   for (int g = wave; g < groups; g += 4) {
+      const int q = g * 32 + l32;
+      const int qq = q < total ? q : total - 1;
+      const int im = fdiv(qq, a.dper_image), rem = qq - im * per_image;
+      const int py = fdiv(rem, a.dPW), px = rem - py * a.PW;
+      const int row0 = (POOL ? 2 * py : py) + 2 * half, col = POOL ? 2 * px : px;
+      const unsigned char *base = s_img + im * a.img_bytes + row0 * a.stride;
+      long pix[NP];
+      if constexpr (POOL) {
+         int r[3][2];
 #pragma unroll
-         for (int e = 0; e < 4; ++e) {
-            const v4i wt = s_w[oc0 + e];
-            const float sc = s_scale[oc0 + e];
-            int hi = 0, lo = 0;
+         for (int k = 0; k < 3; ++k) windows(base + k * a.stride, col, r[k][0], r[k][1]);
 #pragma unroll
-            for (int dy = 0; dy < ND; ++dy)
+         for (int j = 0; j < 4; ++j) pix[j] = pack64(r[j >> 1][j & 1], r[(j >> 1) + 1][j & 1]);
+      } else {
+         pix[0] = pack64(window(base, col), window(base + a.stride, col));
+      }
+      int8_t *out = a.y + ((size_t)(n0 + im) * per_image + rem) * a.OC;
+      for (int ob = 0; ob < a.ocb; ++ob) {
+         if (!single) load_params(ob);
+         // one window position at a time keeps two accumulator tiles live (more wavefronts per SIMD)
+         v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(wfrag, pix[0], zero16, 0, 0, 0);
+         if constexpr (POOL) {
+            v16i lo = acc;
 #pragma unroll
-               for (int dx = 0; dx < ND; ++dx) {
-                  int acc = wt[3];
-                  acc = __builtin_amdgcn_sdot4(rows[dy][dx], wt[0], acc, false);
-                  acc = __builtin_amdgcn_sdot4(rows[dy + 1][dx], wt[1], acc, false);
-                  acc = __builtin_amdgcn_sdot4(rows[dy + 2][dx], wt[2], acc, false);
-                  if (dy == 0 && dx == 0) { hi = acc; lo = acc; }
-                  else { hi = max(hi, acc); lo = min(lo, acc); }
+            for (int j = 1; j < 4; ++j) {
+               const v16i c = __builtin_amdgcn_mfma_i32_32x32x16_i8(wfrag, pix[j], zero16, 0, 0, 0);
+#pragma unroll
+               for (int e = 0; e < 16; ++e) acc[e] = max(acc[e], c[e]);
+               if (any_negative) {
+#pragma unroll
+                  for (int e = 0; e < 16; ++e) lo[e] = min(lo[e], c[e]);
                }
-            const int sel = sc < 0.0f ? lo : hi;
-            float r = rintf(__fmul_rn(__int2float_rn(sel), sc));
-            r = fmaxf(__fadd_rn(r, zpo), lof);
-            pk = __builtin_amdgcn_cvt_pk_u8_f32(r, e, pk);
+            }
+            if (any_negative) {
+#pragma unroll
+               for (int e = 0; e < 16; ++e) acc[e] = sc[e >> 2][e & 3] < 0.0f ? lo[e] : acc[e];
+            }
          }
-         *reinterpret_cast<unsigned *>(out + oc0) = pk ^ 0x80808080u;
+         unsigned d[4];
+#pragma unroll
+         for (int gq = 0; gq < 4; ++gq) {
+            unsigned pk = 0;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+               // the bias is added after the pooling (max(a + b) = max(a) + b), so the matrix instructions
+               // start from a constant zero and need no copy of an initial tile
+               float r = __fmul_rn(__int2float_rn(acc[gq * 4 + t] + binit[gq * 4 + t]), sc[gq][t]);
+               if (!plain) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);   // the byte conversion rounds half to even itself
+               pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);
+            }
+            d[gq] = pk ^ 0x80808080u;
+         }
+         // lanes 0-31 hold channels {0-3, 8-11, 16-19, 24-27} of their pixel, lanes 32-63 {4-7, 12-15, 20-23, 28-31}:
+         // after the swaps the lower half has channels 0-15 and the upper half 16-31, in order
+         const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+         const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+         const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+         const int oc_first = ob * 32 + half * 16;
+         if (q < total && oc_first < a.OC) *reinterpret_cast<v4i *>(out + oc_first) = v;
       }
    }
 }
@@ -119,16 +238,24 @@ int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    *done = false;
    const bool pool = g.pool_kh != 0;
    if (g.C != 1 || g.groups != 1 || g.KH != 3 || g.KW != 3 || g.sh != 1 || g.sw != 1 || g.ph != 1 || g.pw != 1) return SOFIE_HIP_OK;
-   if (g.OC % 4 != 0 || !(g.y_nhwc) || (reinterpret_cast<uintptr_t>(g.y) & 3u) != 0) return SOFIE_HIP_OK;
+   if (g.OC % 16 != 0 || !g.y_nhwc || !aligned16(g.y)) return SOFIE_HIP_OK;
    if (pool && !(g.pool_kh == 2 && g.pool_kw == 2 && g.pool_sh == 2 && g.pool_sw == 2)) return SOFIE_HIP_OK;
+   if (g.PH <= 0 || g.PW <= 0) return SOFIE_HIP_OK;
    FirstArgs a{};
    a.x = g.x; a.w = g.w; a.bias = g.bias; a.scale = g.scale; a.y = static_cast<int8_t *>(g.y);
-   a.H = g.H; a.W = g.W; a.OC = g.OC; a.PH = g.PH; a.PW = g.PW;
+   a.N = g.N; a.H = g.H; a.W = g.W; a.OC = g.OC; a.PH = g.PH; a.PW = g.PW;
    a.zpx = g.zpx; a.zpy = g.zpy; a.lo = g.lo;
-   a.stride = (g.W + 2 + 3) / 4 * 4 + 4;
-   const size_t lds = (size_t)g.OC * 20 + (size_t)(g.H + 2) * a.stride + 8;
+   a.stride = (g.W + 2 + 3) / 4 * 4 + 8;          // a window may start at the last column and spans two dwords
+   a.img_bytes = (g.H + 3) * a.stride;
+   a.ocb = (g.OC + 31) / 32;
+   a.rows = g.H + 3;
+   a.dword_fill = g.W % 4 == 0 && (reinterpret_cast<uintptr_t>(g.x) & 3u) == 0;
+   a.drows = make_fastdiv((unsigned)a.rows);
+   a.dper_image = make_fastdiv((unsigned)(g.PH * g.PW));
+   a.dPW = make_fastdiv((unsigned)g.PW);
+   const size_t lds = (size_t)a.ocb * 32 * 24 + 16 + (size_t)kImages * a.img_bytes + 16;
    if (lds > 64 * 1024) return SOFIE_HIP_OK;
-   const dim3 grid((unsigned)g.N), block(256);
+   const dim3 grid((unsigned)((g.N + kImages - 1) / kImages)), block(256);
    if (pool) hipLaunchKernelGGL(k_qconv_first<true>, grid, block, lds, ctx->stream, a);
    else hipLaunchKernelGGL(k_qconv_first<false>, grid, block, lds, ctx->stream, a);
    *done = true;

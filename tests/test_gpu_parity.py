@@ -347,20 +347,24 @@ def test_qconv2d_s8_matrix_core_path(ops, cfg):
 
 
 @pytest.mark.parametrize("cfg", [
-    dict(N=3, H=40, W=40, OC=32), dict(N=2, H=7, W=9, OC=8), dict(N=1, H=1, W=1, OC=4), dict(N=5, H=13, W=6, OC=20),
-    dict(N=2, H=64, W=50, OC=64),
+    dict(N=3, H=40, W=40, OC=32), dict(N=6, H=7, W=9, OC=16), dict(N=1, H=1, W=1, OC=32), dict(N=5, H=13, W=6, OC=48),
+    dict(N=2, H=64, W=50, OC=64), dict(N=9, H=5, W=4, OC=8),
 ])
 def test_first_layer_kernel(ops, cfg):
-    """One input channel, 3x3, pad 1: the dot-product kernel, with both zero-point conventions, a ReLU clamp and
-    scales of both signs (the pooled variant picks max or min of the accumulators by the sign)."""
+    """One input channel, 3x3, pad 1: the K = 16 matrix-instruction kernel (OC a multiple of 16; OC = 8 takes the
+    plain kernel), with both zero-point conventions, a ReLU clamp, all-positive scales and scales of both signs
+    (the pooled variant then picks max or min of the accumulators by the sign), image counts that do not fill
+    the last workgroup."""
     from sofie_amd import lib as L
     r = rng(600 + cfg["H"] + cfg["OC"])
     x = r.integers(-128, 128, (cfg["N"], 1, cfg["H"], cfg["W"])).astype(np.int8)
     w = r.integers(-127, 128, (cfg["OC"], 1, 3, 3)).astype(np.int8)
     scale = (r.uniform(20, 60, cfg["OC"]) / (73.3 * 73.3 * 3)).astype(np.float32)
-    scale[::3] *= -1
     bias = r.integers(-3000, 3000, cfg["OC"]).astype(np.int32)
-    for zpx, zpy, relu in ((-128, -128, True), (5, -3, False)):
+    for zpx, zpy, relu, negate in ((-128, -128, True, False), (5, -3, False, True), (-128, -128, False, True)):
+        if negate:
+            scale = scale.copy()
+            scale[::3] *= -1
         ref = oracle.qconv2d_s8(x, w, scale, bias, (1, 1), (1, 1), 1, zpx, zpy, relu)
         y = ops.qconv2d_s8(x, w, scale, bias, (1, 1), (1, 1), 1, zpx, zpy, relu, y_layout=L.LAYOUT_NHWC)
         assert np.array_equal(y.transpose(0, 3, 1, 2), ref)
