@@ -532,6 +532,60 @@ __global__ void k_gemm_bytes_simple(GemmArgs g, int transB)
    else *reinterpret_cast<unsigned *>(out) = r;
 }
 
+// int8 product with at most 16 output columns (the last layer of a classifier): B^T [N,K] is tiny and
+// stays in cache, the work is streaming A. 16 lanes share a row of A, each takes every 16th 16-byte
+// chunk of K and multiplies it into all N columns with v_dot4_i32_i8; the 16 partial sums of a column
+// are added with four butterfly steps inside the 16-lane group. Four rows per wavefront.
+template <int OUT, int NMAX>
+__global__ void __launch_bounds__(256) k_qgemm_skinny(GemmArgs g)
+{
+   const int lane16 = threadIdx.x & 15;
+   const int row = (int)(((size_t)blockIdx.x * 256 + threadIdx.x) >> 4);
+   const int m = row < g.M ? row : g.M - 1;
+   const uint8_t *a = g.A + (size_t)m * g.lda;
+   int acc[NMAX];
+#pragma unroll
+   for (int n = 0; n < NMAX; ++n) acc[n] = 0;
+   const int chunks = g.K >> 4;
+   for (int c = lane16; c < chunks; c += 16) {
+      const v4i av = *reinterpret_cast<const v4i *>(a + c * 16);
+#pragma unroll
+      for (int n = 0; n < NMAX; ++n) {
+         if (n < g.N) {
+            const v4i bv = *reinterpret_cast<const v4i *>(g.B + (size_t)n * g.ldb + c * 16);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[n] = __builtin_amdgcn_sdot4(av[e], bv[e], acc[n], false);
+         }
+      }
+   }
+#pragma unroll
+   for (int n = 0; n < NMAX; ++n) {
+#pragma unroll
+      for (int d = 1; d < 16; d <<= 1) acc[n] += __shfl_xor(acc[n], d, 16);
+   }
+   if (row >= g.M) return;
+   constexpr int ESZ = OutSize<OUT>::value;
+#pragma unroll
+   for (int n = 0; n < NMAX; ++n) {
+      if (n == lane16 && n < g.N) {
+         const unsigned r = epilogue_value<true, OUT>(g, g.scale ? g.scale[n] : 0.0f,
+                                                      g.bias ? static_cast<const int *>(g.bias)[n] : 0, acc[n], 0.0f);
+         unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + n) * ESZ;
+         if constexpr (ESZ == 1) *out = (unsigned char)((int)fminf(__uint_as_float(r), 255.0f) - 128);
+         else *reinterpret_cast<unsigned *>(out) = r;
+      }
+   }
+}
+
+template <int OUT>
+int launch_skinny(sofie_hip_ctx *ctx, GemmArgs &g)
+{
+   const dim3 grid((unsigned)(((size_t)g.M * 16 + 255) / 256)), block(256);
+   if (g.N <= 8) hipLaunchKernelGGL((k_qgemm_skinny<OUT, 8>), grid, block, 0, ctx->stream, g);
+   else hipLaunchKernelGGL((k_qgemm_skinny<OUT, 16>), grid, block, 0, ctx->stream, g);
+   return check_launch(ctx, "k_qgemm_skinny");
+}
+
 template <class Mma, int BK, int NSETS, int TI, int TJ, int OUT, bool B_KN, bool FULL>
 int launch_tiled_impl(sofie_hip_ctx *ctx, GemmArgs &g)
 {
@@ -593,6 +647,10 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
    const bool b_nk_ok = transB && g.ldb % 16 == 0 && aligned16(g.B);
    const bool b_kn_ok = !transB && g.ldb % 4 == 0 && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.B) & 3u) == 0;
    g.vec_store = ((size_t)g.ldy * ESZ) % 16 == 0 && aligned16(g.Y);
+   if constexpr (IS_INT && OUT != SOFIE_OUT_BF16) {
+      if (transB && g.N <= 16 && a_ok && g.ldb % 16 == 0 && aligned16(g.B) && (size_t)g.M * 16 < ((size_t)1 << 40))
+         return launch_skinny<OUT>(ctx, g);
+   }
    if (!a_ok || !(b_nk_ok || b_kn_ok)) return launch_simple<IS_INT, OUT>(ctx, g, transB);
    const bool big = (size_t)g.M * g.N >= (size_t)256 * 256 * 128 && g.M >= 256 && g.N >= 256;
    // 128 bytes of K per stage; int8 keeps two register sets in flight, fp8 (twice the

@@ -182,7 +182,8 @@ QGEMM_SHAPES = [
     (512, 2048, 512, True), (512, 2048, 512, False),    # 256-tile kernel
     (777, 1028, 1040, True), (777, 1028, 1040, False),  # 256-tile kernel, ragged
     (33, 47, 50, True), (33, 47, 50, False),            # K % 16 != 0: simple kernel
-    (4096, 5, 256, True), (1, 16, 16, True),
+    (4096, 5, 256, True), (1, 16, 16, True),             # at most 16 columns: the dot-product kernel
+    (70, 13, 1040, True), (5, 1, 32, True), (300, 9, 48, True),
 ]
 
 
