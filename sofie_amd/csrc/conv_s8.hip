@@ -78,6 +78,7 @@ struct QConvTileArgs {
    GemmArgs ep;          // Y, scale, bias, M = N*OH*OW, N = OC, ldy = OC, zp, lo, relu
    int H, W, C, KH, KW, ph, pw, sh, sw, OH, OW, HP, WP;
    int K, KS, CS;        // bytes of one weight row, its LDS stride, LDS stride of one pixel
+   int RB;               // LDS stride of one band row
    int C16, C32;
    int RL, RP;           // 16-byte chunks per band row; band rows fetched per pass
    int ntiles;
@@ -105,7 +106,8 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    float *const s_scale = reinterpret_cast<float *>(smem + OCT * a.KS);    // [OCT]
    int *const s_bias = reinterpret_cast<int *>(s_scale + OCT);             // [OCT]
    unsigned char *const s_stg = reinterpret_cast<unsigned char *>(s_bias + OCT);   // [8][WB] epilogue staging
-   unsigned char *const s_p = s_stg + 8 * WB;                              // band [rows][WP][CS]
+   // the int8 epilogue needs no staging (it transposes with lane swaps)
+   unsigned char *const s_p = s_stg + (OUT == SOFIE_OUT_S8 ? 0 : 8 * WB);   // band [rows][WP][CS]
 
    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
    const int wn = wave % WN, wm = wave / WN;
@@ -138,7 +140,7 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    const bool col_inside = iw >= 0 && iw < a.W;
    const int src_col = iw * a.C + c16 * 16;
    const int lds_col = wp * a.CS + c16 * 16;
-   const int row_bytes = a.WP * a.CS;
+   const int row_bytes = a.RB;
    const v4i fillv = {(int)a.fill, (int)a.fill, (int)a.fill, (int)a.fill};
 
    struct Band { int vr_lo, rows; };
@@ -183,7 +185,7 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 #pragma unroll
    for (int i = 0; i < NB; ++i) b_off[i] = ((wn * NB + i) * 32 + l32) * a.KS + half * 16;
    const int tap_step = a.CS - a.C32 * 32;              // from the end of one tap's channels to the next tap
-   const int row_step = (a.WP - a.KW) * a.CS;           // from the end of one kernel row to the next
+   const int row_step = a.RB - a.KW * a.CS;             // from the end of one kernel row to the next
    const int nsteps = a.KH * a.KW * a.C32;
    const int nq = half * 4;
    const float *const w_scale = s_scale + wn * NB * 32;
@@ -202,7 +204,7 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          const int v = n * a.HP + (R - n * a.OH) * 2 * a.sh - vr_lo;
 #pragma unroll
          for (int j = 0; j < 4; ++j)
-            a_off[j] = ((v + (j >> 1) * a.sh) * a.WP + (2 * pw_ + (j & 1)) * a.sw) * a.CS + half * 16;
+            a_off[j] = (v + (j >> 1) * a.sh) * a.RB + (2 * pw_ + (j & 1)) * a.sw * a.CS + half * 16;
       } else {
 #pragma unroll
          for (int j = 0; j < MB; ++j) {
@@ -212,7 +214,7 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
             const int ow = m - R * a.OW;
             const int n = fdiv(R, a.dOH);
             const int v = n * a.HP + (R - n * a.OH) * a.sh - vr_lo;
-            a_off[j] = (v * a.WP + ow * a.sw) * a.CS + half * 16;
+            a_off[j] = v * a.RB + ow * a.sw * a.CS + half * 16;
          }
       }
    };
@@ -230,7 +232,7 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 #pragma unroll
                for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = bi[e];
          }
-      v4i fa[2][MB], fb[2][NB];
+      v4i fa[POOL ? 2 : 3][MB], fb[POOL ? 2 : 3][NB];
       int ka = 0, kb = 0, c32 = 0, kw = 0;
       auto advance = [&]() {
          ka += 32; kb += 32;
@@ -239,7 +241,10 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
             if (++kw == a.KW) { kw = 0; ka += row_step; }
          }
       };
-      auto load = [&](int buf, int oa, int ob_) {
+      auto load = [&](int buf, bool valid) {
+         // every fragment load is unconditional (one past the last step re-reads step 0), so that the
+         // waits in front of the matrix instructions count exactly
+         const int oa = valid ? ka : 0, ob_ = valid ? kb : 0;
 #pragma unroll
          for (int j = 0; j < MB; ++j) fa[buf][j] = *reinterpret_cast<const v4i *>(s_p + a_off[j] + oa);
 #pragma unroll
@@ -251,20 +256,39 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 #pragma unroll
             for (int j = 0; j < MB; ++j) acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], acc[i][j]);
       };
-      // two steps per trip; every fragment load is unconditional (the one past the last step re-reads
-      // step 0) so that the waits in front of the matrix instructions count exactly
-      load(0, 0, 0);
-      int s = 0;
-      for (; s + 1 < nsteps; s += 2) {
+      if constexpr (!POOL) {
+         // three fragment buffers: the reads of step s+2 are issued before the matrix instructions of step s
+         load(0, true);
          advance();
-         load(1, ka, kb);
-         mma(0);
-         advance();
-         const bool more = s + 2 < nsteps;
-         load(0, more ? ka : 0, more ? kb : 0);
-         mma(1);
+         load(1, nsteps > 1);
+         int s = 0;
+         for (; s + 2 < nsteps; s += 3) {
+            advance();
+            load(2, true);
+            mma(0);
+            advance();
+            load(0, s + 3 < nsteps);
+            mma(1);
+            advance();
+            load(1, s + 4 < nsteps);
+            mma(2);
+         }
+         if (s < nsteps) mma(0);
+         if (s + 1 < nsteps) mma(1);
+      } else {
+         // the pooled variant has twice the accumulators and keeps two fragment buffers
+         load(0, true);
+         int s = 0;
+         for (; s + 1 < nsteps; s += 2) {
+            advance();
+            load(1, true);
+            mma(0);
+            advance();
+            load(0, s + 2 < nsteps);
+            mma(1);
+         }
+         if (s < nsteps) mma(0);
       }
-      if (s < nsteps) mma(0);
    };
    // the lane's scales, loaded once (after the first barrier); the pooled variant needs the registers for
    // its four accumulator tiles and reads the scales from LDS instead
@@ -286,19 +310,16 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
                   pooled[i][0][e] = sc[t] < 0.0f ? lo : hi;
                }
             }
-         if (plain)
-            tile_epilogue_wave<MmaI8, NB, 1, OUT, true, false, true>(a.ep, pooled, w_stg, w_scale, w_bias, lane, m_wave,
-                                                                     n_wave);
-         else
-            tile_epilogue_wave<MmaI8, NB, 1, OUT, false, false, true>(a.ep, pooled, w_stg, w_scale, w_bias, lane, m_wave,
-                                                                      n_wave);
+         if constexpr (OUT == SOFIE_OUT_S8) {
+            if (plain) tile_epilogue_s8_direct<NB, 1, true, false>(a.ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+            else tile_epilogue_s8_direct<NB, 1, false, false>(a.ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+         }
+      } else if constexpr (OUT == SOFIE_OUT_S8) {
+         if (plain) tile_epilogue_s8_direct<NB, MB, true, false>(a.ep, acc, w_scale, w_bias, lane, m_wave, n_wave, &r_scale);
+         else tile_epilogue_s8_direct<NB, MB, false, false>(a.ep, acc, w_scale, w_bias, lane, m_wave, n_wave, &r_scale);
       } else {
-         if (plain)
-            tile_epilogue_wave<MmaI8, NB, MB, OUT, true, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
-                                                                      n_wave, &r_scale);
-         else
-            tile_epilogue_wave<MmaI8, NB, MB, OUT, false, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave,
-                                                                       n_wave, &r_scale);
+         tile_epilogue_wave<MmaI8, NB, MB, OUT, false, false, true>(a.ep, acc, w_stg, w_scale, w_bias, lane, m_wave, n_wave,
+                                                                    &r_scale);
       }
    };
 
@@ -394,8 +415,17 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const long long rows_max = (long long)(tile_rows * rpp - 1) * g.sh + (long long)crossings * gap + g.KH;
    const int passes = (int)((rows_max + a.RP - 1) / a.RP);
    if (passes > 12) return SOFIE_HIP_OK;
-   const size_t band = (size_t)rows_max * WP * a.CS;
-   const size_t lds = (size_t)OCT * a.KS + (size_t)OCT * 8 + (size_t)8 * EpilogueStaging<2, OUT>::WAVE_BYTES + band;
+   // Band row pitch. Consecutive output pixels sit sw*CS bytes apart; the pitch is padded so that the
+   // step from the last pixel of an output row to the first of the next is the same modulo the 256 bytes
+   // the LDS banks span. The 16 lanes that read together then keep hitting distinct banks across row ends.
+   a.RB = WP * a.CS;
+   if (g.sh == 1 && !pool) {
+      const int want = (int)(((long long)g.OW * g.sw * a.CS) % 256);
+      a.RB += ((want - a.RB % 256) % 256 + 256) % 256;
+   }
+   const size_t band = (size_t)rows_max * a.RB;
+   const size_t staging = OUT == SOFIE_OUT_S8 ? 0 : (size_t)8 * EpilogueStaging<2, OUT>::WAVE_BYTES;
+   const size_t lds = (size_t)OCT * a.KS + (size_t)OCT * 8 + staging + band;
    if (lds > 160 * 1024) return SOFIE_HIP_OK;
    if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
 

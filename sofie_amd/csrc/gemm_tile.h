@@ -199,6 +199,48 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
    }
 }
 
+// int8 epilogue without LDS staging, for tiles whose columns are all inside the matrix: a lane packs its
+// four 4-column groups of a 32 x 32 accumulator tile into four dwords; two v_permlane32_swap between the
+// halves of the wavefront turn them into 16 consecutive columns per lane (lanes 0-31: columns 0-15 of
+// the tile, lanes 32-63: columns 16-31), which leave as one 16-byte store. Rows need ldy % 16 == 0 and
+// a 16-byte aligned Y. reg_scale as in tile_epilogue_wave (may be null: scales are then read from s_scale).
+template <int TI, int TJ, bool PLAIN, bool ADD_BIAS>
+__device__ __forceinline__ void tile_epilogue_s8_direct(const GemmArgs &g, v16i (&acc)[TI][TJ], const float *s_scale,
+                                                        const int *s_bias, int lane, int m_wave, int n_wave,
+                                                        const v4f (*reg_scale)[TI * 4] = nullptr)
+{
+   const int l32 = lane & 31, half = lane >> 5;
+   const int nq = half * 4;
+   const float zpo = (float)(g.zp + 128), lof = (float)(g.lo + 128);
+#pragma unroll
+   for (int j = 0; j < TJ; ++j) {
+      const int m = m_wave + j * 32 + l32;
+      int8_t *row = static_cast<int8_t *>(g.Y) + (size_t)(m < g.M ? m : 0) * g.ldy + n_wave + half * 16;
+#pragma unroll
+      for (int i = 0; i < TI; ++i) {
+         unsigned d[4];
+#pragma unroll
+         for (int q = 0; q < 4; ++q) {
+            const v4f sc = reg_scale ? (*reg_scale)[i * 4 + q] : *reinterpret_cast<const v4f *>(s_scale + i * 32 + q * 8 + nq);
+            v4i bi = {0, 0, 0, 0};
+            if (ADD_BIAS) bi = *reinterpret_cast<const v4i *>(s_bias + i * 32 + q * 8 + nq);
+            unsigned pk = 0;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+               float r = __fmul_rn(__int2float_rn(acc[i][j][q * 4 + t] + bi[t]), sc[t]);
+               if constexpr (!PLAIN) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);   // the byte conversion rounds half to even
+               pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);
+            }
+            d[q] = pk ^ 0x80808080u;
+         }
+         const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+         const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+         const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+         if (m < g.M) *reinterpret_cast<v4i *>(row + i * 32) = v;
+      }
+   }
+}
+
 // Per-column scale and bias bits of a workgroup's BN columns starting at n0 -> LDS.
 __device__ __forceinline__ void stage_column_params(const GemmArgs &g, float *s_scale, int *s_bias, int tid, int n0,
                                                     int BN)
