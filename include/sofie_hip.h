@@ -183,6 +183,20 @@ int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout,
                               int zp_x, int zp_y, int act, int pool_kh, int pool_kw,
                               int pool_stride_h, int pool_stride_w);
 
+/* QuantizeLinear -> QLinearConv -> (ReLU) -> (MaxPool) in one call, for the first layer of a
+ * quantized network: x is the float tensor [N, C, H, W], quantized as in
+ * sofie_hip_quantize_f32_s8(x, x_scale, zp_x); everything else as in
+ * sofie_hip_qconv2d_pool_s8, pool_kh = pool_kw = 0 meaning no pooling. One-input-channel 3x3
+ * stride-1 pad-1 layers quantize while the image is copied on chip and never write the int8
+ * input; other shapes quantize into the context's scratch buffer first. Bit-identical to the
+ * separate calls. */
+int sofie_hip_quantize_qconv2d_s8(sofie_hip_ctx *ctx, const float *x, float x_scale, int zp_x,
+                                  const int8_t *w, int w_layout, const int32_t *bias,
+                                  const float *scale, int8_t *y, int y_layout, int N, int C, int H,
+                                  int W, int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,
+                                  int stride_w, int groups, int zp_y, int act, int pool_kh,
+                                  int pool_kw, int pool_stride_h, int pool_stride_w);
+
 /* int8 max pooling, NCHW or NHWC. */
 int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N,
                            int C, int H, int W, int kh, int kw, int pad_t, int pad_l,

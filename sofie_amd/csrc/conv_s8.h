@@ -6,6 +6,8 @@ namespace sofie {
 
 struct QConvArgs {
    const int8_t *x, *w;
+   const float *xf;          // if not null: the input is this float tensor, quantized with xscale / zpx on the fly
+   float xscale;
    const int32_t *bias;
    const float *scale;
    void *y;

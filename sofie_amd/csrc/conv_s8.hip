@@ -519,16 +519,20 @@ int run_conv(sofie_hip_ctx *ctx, const QConvArgs &g, int8_t *scratch)
    return check_launch(ctx, "k_qconv_simple");
 }
 
-template <int OUT>
-int run(sofie_hip_ctx *ctx, const QConvArgs &g)
+// Scratch bytes run() needs for g (beyond what the caller may have reserved in front of them).
+size_t run_scratch_bytes(const QConvArgs &g)
 {
-   void *ws = nullptr;
-   if (g.pool_kh == 0) {
-      const size_t need = layout_scratch_bytes(g);
-      if (need)
-         if (int rc = workspace(ctx, need, &ws)) return rc;
-      return run_conv<OUT>(ctx, g, static_cast<int8_t *>(ws));
-   }
+   if (g.pool_kh == 0) return layout_scratch_bytes(g);
+   QConvArgs h = g;
+   h.pool_kh = h.pool_kw = h.pool_sh = h.pool_sw = 0;
+   return up256((size_t)g.N * g.OC * g.OH * g.OW) + layout_scratch_bytes(h);
+}
+
+// scratch: run_scratch_bytes(g) bytes of device memory.
+template <int OUT>
+int run(sofie_hip_ctx *ctx, const QConvArgs &g, int8_t *scratch)
+{
+   if (g.pool_kh == 0) return run_conv<OUT>(ctx, g, scratch);
    // fused kernels first; otherwise the convolution goes to scratch memory in the layout of y and the
    // pooling kernel reads it from there
    bool done = false;
@@ -540,12 +544,21 @@ int run(sofie_hip_ctx *ctx, const QConvArgs &g)
    h.pool_kh = h.pool_kw = h.pool_sh = h.pool_sw = 0;
    h.PH = g.OH; h.PW = g.OW;
    const size_t conv_bytes = up256((size_t)g.N * g.OC * g.OH * g.OW);
-   if (int rc = workspace(ctx, conv_bytes + layout_scratch_bytes(h), &ws)) return rc;
-   h.y = ws;
-   if (int rc = run_conv<OUT>(ctx, h, static_cast<int8_t *>(ws) + conv_bytes)) return rc;
-   return sofie_hip_maxpool2d_s8(ctx, static_cast<const int8_t *>(ws), static_cast<int8_t *>(g.y),
+   h.y = scratch;
+   if (int rc = run_conv<OUT>(ctx, h, scratch + conv_bytes)) return rc;
+   return sofie_hip_maxpool2d_s8(ctx, scratch, static_cast<int8_t *>(g.y),
                                  g.y_nhwc ? SOFIE_LAYOUT_NHWC : SOFIE_LAYOUT_NCHW, g.N, g.OC, g.OH, g.OW, g.pool_kh,
                                  g.pool_kw, 0, 0, 0, 0, g.pool_sh, g.pool_sw);
+}
+
+template <int OUT>
+int run(sofie_hip_ctx *ctx, const QConvArgs &g)
+{
+   void *ws = nullptr;
+   const size_t need = run_scratch_bytes(g);
+   if (need)
+      if (int rc = workspace(ctx, need, &ws)) return rc;
+   return run<OUT>(ctx, g, static_cast<int8_t *>(ws));
 }
 
 int fill_args(sofie_hip_ctx *ctx, QConvArgs &g, const int8_t *x, int x_layout, const int8_t *w, int w_layout,
@@ -564,7 +577,7 @@ int fill_args(sofie_hip_ctx *ctx, QConvArgs &g, const int8_t *x, int x_layout, c
    SOFIE_REQUIRE(ctx, zp_x >= -128 && zp_x <= 127 && zp_y >= -128 && zp_y <= 127, "zero-point out of int8 range");
    SOFIE_REQUIRE(ctx, H + 2 * pad_h >= KH && W + 2 * pad_w >= KW, "kernel larger than padded input");
    if (N == 0) return SOFIE_HIP_OK;
-   SOFIE_REQUIRE(ctx, x && w && y, "null operand");
+   SOFIE_REQUIRE(ctx, w && y, "null operand");
    SOFIE_REQUIRE(ctx, scale || out_kind == SOFIE_OUT_S32, "scale is required for S8 output");
    g.x = x; g.w = w; g.bias = bias; g.scale = scale; g.y = y;
    g.N = N; g.C = C; g.H = H; g.W = W; g.OC = OC; g.KH = KH; g.KW = KW;
@@ -597,6 +610,7 @@ extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_l
                           stride_h, stride_w, groups, zp_x, zp_y, act, out_kind))
       return rc;
    if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x, "null operand");
    if (out_kind == SOFIE_OUT_S32) return run<SOFIE_OUT_S32>(ctx, g);
    return run<SOFIE_OUT_S8>(ctx, g);
 }
@@ -615,8 +629,47 @@ extern "C" int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, in
    SOFIE_REQUIRE(ctx, pool_kh > 0 && pool_kw > 0 && pool_stride_h > 0 && pool_stride_w > 0, "bad pooling window");
    SOFIE_REQUIRE(ctx, pool_kh <= g.OH && pool_kw <= g.OW, "pooling window larger than the convolution output");
    if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x, "null operand");
    g.pool_kh = pool_kh; g.pool_kw = pool_kw; g.pool_sh = pool_stride_h; g.pool_sw = pool_stride_w;
    g.PH = (g.OH - pool_kh) / pool_stride_h + 1;
    g.PW = (g.OW - pool_kw) / pool_stride_w + 1;
    return run<SOFIE_OUT_S8>(ctx, g);
+}
+
+extern "C" int sofie_hip_quantize_qconv2d_s8(sofie_hip_ctx *ctx, const float *x, float x_scale, int zp_x, const int8_t *w,
+                                             int w_layout, const int32_t *bias, const float *scale, int8_t *y,
+                                             int y_layout, int N, int C, int H, int W, int OC, int KH, int KW, int pad_h,
+                                             int pad_w, int stride_h, int stride_w, int groups, int zp_y, int act,
+                                             int pool_kh, int pool_kw, int pool_stride_h, int pool_stride_w)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, x_scale > 0.0f, "the input scale must be positive");
+   QConvArgs g{};
+   if (int rc = fill_args(ctx, g, nullptr, SOFIE_LAYOUT_NCHW, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW,
+                          pad_h, pad_w, stride_h, stride_w, groups, zp_x, zp_y, act, SOFIE_OUT_S8))
+      return rc;
+   if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x, "null operand");
+   const bool pool = pool_kh != 0 || pool_kw != 0;
+   if (pool) {
+      SOFIE_REQUIRE(ctx, pool_kh > 0 && pool_kw > 0 && pool_stride_h > 0 && pool_stride_w > 0, "bad pooling window");
+      SOFIE_REQUIRE(ctx, pool_kh <= g.OH && pool_kw <= g.OW, "pooling window larger than the convolution output");
+      g.pool_kh = pool_kh; g.pool_kw = pool_kw; g.pool_sh = pool_stride_h; g.pool_sw = pool_stride_w;
+      g.PH = (g.OH - pool_kh) / pool_stride_h + 1;
+      g.PW = (g.OW - pool_kw) / pool_stride_w + 1;
+   }
+   // the first-layer kernel quantizes while it copies the image into LDS
+   g.xf = x;
+   g.xscale = x_scale;
+   bool done = false;
+   if (int rc = qconv_first_layer(ctx, g, &done)) return rc;
+   if (done) return SOFIE_HIP_OK;
+   // otherwise: quantize into scratch memory, then the int8 path
+   g.xf = nullptr;
+   const size_t xbytes = up256((size_t)N * C * H * W);
+   void *ws = nullptr;
+   if (int rc = workspace(ctx, xbytes + run_scratch_bytes(g), &ws)) return rc;
+   if (int rc = sofie_hip_quantize_f32_s8(ctx, x, static_cast<int8_t *>(ws), (size_t)N * C * H * W, x_scale, zp_x)) return rc;
+   g.x = static_cast<const int8_t *>(ws);
+   return run<SOFIE_OUT_S8>(ctx, g, static_cast<int8_t *>(ws) + xbytes);
 }

@@ -20,6 +20,8 @@ namespace {
 
 struct FirstArgs {
    const int8_t *x;
+   const float *xf;       // float input to quantize on the fly (then x is unused), or null
+   float xscale;
    const int8_t *w;       // [OC][9]
    const int32_t *bias;   // [OC] or null
    const float *scale;    // [OC]
@@ -54,6 +56,14 @@ __device__ __forceinline__ int window(const unsigned char *row, int col)
 __device__ __forceinline__ long pack64(int lo, int hi)
 {
    return (long)(((unsigned long long)(unsigned)hi << 32) | (unsigned long long)(unsigned)lo);
+}
+
+// QuantizeLinear of one value: sat_s8(rint_half_even(x / scale) + zp), returned as a byte.
+__device__ __forceinline__ unsigned quantize_byte(float v, float scale, int zp)
+{
+   float r = rintf(__fdiv_rn(v, scale));
+   r = fminf(fmaxf(r, -1024.0f), 1024.0f);
+   return (unsigned)min(127, max(-128, (int)r + zp)) & 0xffu;
 }
 
 template <bool POOL>
@@ -103,6 +113,8 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
       for (int j = jj; j < SD; j += 16) {
          for (int base = 0; base < total_rows; base += 16 * UN) {
             unsigned lo[UN], hi[UN];
+            float flo[UN];
+            v4f fhi[UN];
             bool has_lo[UN], has_hi[UN];
             unsigned *dst[UN];
 #pragma unroll
@@ -119,8 +131,23 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
                            : nullptr;
                has_lo[u] = row_inside && j >= 1 && j - 1 < WD;
                has_hi[u] = row_inside && j < WD;
-               lo[u] = gsrc[has_lo[u] ? j - 1 : 0];
-               hi[u] = gsrc[has_hi[u] ? j : 0];
+               if (a.xf) {
+                  // image columns 4j-1 .. 4j+2 as floats, quantized here
+                  const float *fsrc = a.xf + ((size_t)(n0 + im) * a.H + (row_inside ? ih : 0)) * a.W;
+                  flo[u] = fsrc[has_lo[u] ? 4 * j - 1 : 0];
+                  fhi[u] = *reinterpret_cast<const v4f *>(fsrc + (has_hi[u] ? 4 * j : 0));
+               } else {
+                  lo[u] = gsrc[has_lo[u] ? j - 1 : 0];
+                  hi[u] = gsrc[has_hi[u] ? j : 0];
+               }
+            }
+            if (a.xf) {
+#pragma unroll
+               for (int u = 0; u < UN; ++u) {
+                  lo[u] = quantize_byte(flo[u], a.xscale, a.zpx) << 24;
+                  hi[u] = quantize_byte(fhi[u][0], a.xscale, a.zpx) | (quantize_byte(fhi[u][1], a.xscale, a.zpx) << 8) |
+                          (quantize_byte(fhi[u][2], a.xscale, a.zpx) << 16);
+               }
             }
 #pragma unroll
             for (int u = 0; u < UN; ++u)
@@ -133,7 +160,9 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
          const int r = o / a.stride, c = o - r * a.stride;
          const int ih = r - 1, iw = c - 1;
          const bool inside = ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
-         s_img[i] = inside ? (unsigned char)a.x[((size_t)(n0 + im) * a.H + ih) * a.W + iw] : (unsigned char)a.zpx;
+         const size_t src = ((size_t)(n0 + im) * a.H + (inside ? ih : 0)) * a.W + (inside ? iw : 0);
+         const unsigned char v = a.xf ? (unsigned char)quantize_byte(a.xf[src], a.xscale, a.zpx) : (unsigned char)a.x[src];
+         s_img[i] = inside ? v : (unsigned char)a.zpx;
       }
    }
    __syncthreads();
@@ -242,14 +271,14 @@ int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (pool && !(g.pool_kh == 2 && g.pool_kw == 2 && g.pool_sh == 2 && g.pool_sw == 2)) return SOFIE_HIP_OK;
    if (g.PH <= 0 || g.PW <= 0) return SOFIE_HIP_OK;
    FirstArgs a{};
-   a.x = g.x; a.w = g.w; a.bias = g.bias; a.scale = g.scale; a.y = static_cast<int8_t *>(g.y);
+   a.x = g.x; a.xf = g.xf; a.xscale = g.xscale; a.w = g.w; a.bias = g.bias; a.scale = g.scale; a.y = static_cast<int8_t *>(g.y);
    a.N = g.N; a.H = g.H; a.W = g.W; a.OC = g.OC; a.PH = g.PH; a.PW = g.PW;
    a.zpx = g.zpx; a.zpy = g.zpy; a.lo = g.lo;
    a.stride = (g.W + 2 + 3) / 4 * 4 + 8;          // a window may start at the last column and spans two dwords
    a.img_bytes = (g.H + 3) * a.stride;
    a.ocb = (g.OC + 31) / 32;
    a.rows = g.H + 3;
-   a.dword_fill = g.W % 4 == 0 && (reinterpret_cast<uintptr_t>(g.x) & 3u) == 0;
+   a.dword_fill = g.W % 4 == 0 && (g.xf ? aligned16(g.xf) : (reinterpret_cast<uintptr_t>(g.x) & 3u) == 0);
    a.drows = make_fastdiv((unsigned)a.rows);
    a.dper_image = make_fastdiv((unsigned)(g.PH * g.PW));
    a.dPW = make_fastdiv((unsigned)g.PW);

@@ -126,6 +126,7 @@ private:
    };
    void FuseActivations();
    void FusePooling();
+   void FuseInputQuantization();
    void PlanIntermediateMemory();
    void GenerateHeaderInfo(std::string &hgname);
    void GenerateSessionCode();

@@ -47,6 +47,9 @@ public:
    {
       return false;
    }
+   // try to absorb a preceding QuantizeLinear (float tensor xFloat quantized with scale / zeroPoint into this
+   // operator's int8 input): on success the operator reads the float tensor itself
+   virtual bool FuseInputQuantization(const std::string & /*xFloat*/, float /*scale*/, int /*zeroPoint*/) { return false; }
    // absorbed into another operator: emits nothing, and its output is written by the absorbing operator
    void SetAbsorbed() { fAbsorbed = true; }
    bool IsAbsorbed() const { return fAbsorbed; }

@@ -88,6 +88,10 @@ public:
       fOutputTensorNames = {fNY};
    }
    std::string Kind() const override { return "QuantizeLinear"; }
+   // what a consumer needs to absorb this operator (valid after Initialize)
+   const std::string &InputName() const { return fNX; }
+   float Scale() const { return fScale; }
+   int ZeroPoint() const { return fZp; }
    std::vector<ETensorType> TypeInference(std::vector<ETensorType>) override { return {ETensorType::INT8}; }
    std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>> input) override { return {input[0]}; }
    void Initialize(RModel &model) override
@@ -306,7 +310,8 @@ public:
 class ROperator_QLinearConv final : public ROperator {
    ConvGeometry fGeom;
    std::string fNX, fNXScale, fNXZp, fNW, fNWScale, fNWZp, fNYScale, fNYZp, fNBias, fNY;
-   std::string fNScale, fNQBias, fNWPacked, fNYPooled;
+   std::string fNScale, fNQBias, fNWPacked, fNYPooled, fNXFloat;
+   float fScaleX = 0;
    std::vector<size_t> fShapeX, fShapeW, fShapeY, fShapePooled, fPoolKernel, fPoolStrides;
    int fZpX = 0, fZpY = 0;
    bool fHasBias = false, fXChannelsLast = false;
@@ -330,6 +335,22 @@ public:
    {
       if (act != EActivationType::RELU || fActivation != EActivationType::UNDEFINED) return false;
       fActivation = act;
+      return true;
+   }
+   bool FuseInputQuantization(const std::string &xFloat, float scale, int zeroPoint) override
+   {
+      // the fused call exists for any shape, but only first layers (one input channel, 3x3, stride 1, pad 1,
+      // OC a multiple of 16) have a kernel that never writes the int8 input: fuse only those
+      if (fShapeX.empty() || !fNXFloat.empty() || fXChannelsLast) return false;
+      size_t ph, pw;
+      fGeom.SymmetricPads(ph, pw);
+      if (fShapeX[1] != 1 || fGeom.group != 1 || fShapeW[2] != 3 || fShapeW[3] != 3 || fGeom.strides[0] != 1 ||
+          fGeom.strides[1] != 1 || ph != 1 || pw != 1 || fShapeW[0] % 16 != 0)
+         return false;
+      if (zeroPoint != fZpX || scale != fScaleX) return false;   // must be the quantization this operator assumes
+      fNXFloat = xFloat;
+      for (auto &n : fInputTensorNames)
+         if (n == fNX) n = xFloat;
       return true;
    }
    bool FusePooling(const std::vector<size_t> &kernel, const std::vector<size_t> &strides, const std::string &pooledName,
@@ -367,6 +388,7 @@ public:
          throw std::runtime_error("TMVA SOFIE QLinearConv op: weight tensor " + fNW + " does not match the input channels and group");
       const size_t OC = fShapeW[0], per = fShapeW[1] * fShapeW[2] * fShapeW[3];
       const float sx = QUTIL::ScalarFloat(model, fNXScale, op);
+      fScaleX = sx;
       fZpX = QUTIL::ScalarZeroPoint(model, fNXZp, op);
       const std::vector<float> sw = QUTIL::ChannelScales(model, fNWScale, OC, op);
       QUTIL::CheckSymmetricWeights(model, fNWZp, op);
@@ -424,16 +446,25 @@ public:
       fGeom.SymmetricPads(ph, pw);
       std::stringstream out;
       const bool pooled = !fPoolKernel.empty();
-      out << "\n//----  operator QLinearConv" << (pooled ? " + MaxPool" : "") << " op_" << OpName << "\n";
-      out << SP << "Check(" << (pooled ? "sofie_hip_qconv2d_pool_s8" : "sofie_hip_qconv2d_s8") << "(fCtx, tensor_" << fNX << ", "
-          << (fXChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << ", tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, "
-          << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", tensor_" << fNScale << ", tensor_"
-          << (pooled ? fNYPooled : fNY) << ", SOFIE_LAYOUT_NHWC, " << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", "
-          << fShapeX[3] << ", " << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3] << ", " << ph << ", " << pw << ", "
-          << fGeom.strides[0] << ", " << fGeom.strides[1] << ", " << fGeom.group << ", " << fZpX << ", " << fZpY << ", "
-          << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE");
+      const bool fromFloat = !fNXFloat.empty();
+      out << "\n//----  operator " << (fromFloat ? "QuantizeLinear + " : "") << "QLinearConv" << (pooled ? " + MaxPool" : "") << " op_"
+          << OpName << "\n";
+      out << SP << "Check(";
+      if (fromFloat)
+         out << "sofie_hip_quantize_qconv2d_s8(fCtx, tensor_" << fNXFloat << ", " << FloatLiteral(fScaleX) << ", " << fZpX;
+      else
+         out << (pooled ? "sofie_hip_qconv2d_pool_s8" : "sofie_hip_qconv2d_s8") << "(fCtx, tensor_" << fNX << ", "
+             << (fXChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW");
+      out << ", tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, " << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr"))
+          << ", tensor_" << fNScale << ", tensor_" << (pooled ? fNYPooled : fNY) << ", SOFIE_LAYOUT_NHWC, " << fShapeX[0] << ", "
+          << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", " << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3]
+          << ", " << ph << ", " << pw << ", " << fGeom.strides[0] << ", " << fGeom.strides[1] << ", " << fGeom.group << ", ";
+      if (!fromFloat) out << fZpX << ", ";
+      out << fZpY << ", " << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE");
       if (pooled)
          out << ", " << fPoolKernel[0] << ", " << fPoolKernel[1] << ", " << fPoolStrides[0] << ", " << fPoolStrides[1];
+      else if (fromFloat)
+         out << ", 0, 0, 0, 0";
       else
          out << ", SOFIE_OUT_S8";
       out << "), \"QLinearConv op_" << OpName << "\");\n";

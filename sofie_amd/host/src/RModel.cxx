@@ -5,6 +5,7 @@
 // operator's Generate() text and returns a std::vector copy of the output.
 #include "SOFIE/RModel.hxx"
 #include "SOFIE/ROperator_Pool.hxx"
+#include "SOFIE/ROperator_Quantized.hxx"
 
 #include <cmath>
 #include <fstream>
@@ -239,6 +240,33 @@ void RModel::FusePooling()
          fIntermediateTensorInfos.erase(t);
          fChannelsLast.erase(t);
       }
+   }
+}
+
+// QuantizeLinear whose int8 output is read by exactly one QLinearConv that can quantize its input itself
+// (a first layer): the convolution reads the float tensor, the QuantizeLinear emits nothing and its output
+// tensor disappears.
+void RModel::FuseInputQuantization()
+{
+   for (size_t i = 0; i < fOperators.size(); ++i) {
+      auto *q = dynamic_cast<ROperator_QuantizeLinear *>(fOperators[i].get());
+      if (!q || q->IsAbsorbed() || q->GetOpOutputTensors().empty()) continue;
+      const std::string &mid = q->GetOpOutputTensors()[0];
+      if (std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), mid) != fOutputTensorNames.end()) continue;
+      int consumer = -1, uses = 0;
+      for (size_t j = 0; j < fOperators.size(); ++j) {
+         if (j == i || fOperators[j]->IsAbsorbed()) continue;
+         for (auto &in : fOperators[j]->GetOpInputTensors())
+            if (in == mid) {
+               ++uses;
+               consumer = (int)j;
+            }
+      }
+      if (uses != 1 || consumer < (int)i || fOperators[consumer]->Kind() != "QLinearConv") continue;
+      if (!fOperators[consumer]->FuseInputQuantization(q->InputName(), q->Scale(), q->ZeroPoint())) continue;
+      q->SetAbsorbed();
+      fIntermediateTensorInfos.erase(mid);
+      fChannelsLast.erase(mid);
    }
 }
 
@@ -623,6 +651,7 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    Initialize(batchSize, verbose);
    FuseActivations();
    FusePooling();
+   FuseInputQuantization();
    PlanIntermediateMemory();
    fGC.clear();
    std::string hgname;

@@ -41,6 +41,7 @@ SIGNATURES = {
     "sofie_hip_qgemm_s8": [_p, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i],
     "sofie_hip_qconv2d_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 16,
     "sofie_hip_qconv2d_pool_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 19,
+    "sofie_hip_quantize_qconv2d_s8": [_p, _p, C.c_float, _i, _p, _i, _p, _p, _p, _i] + [_i] * 18,
     "sofie_hip_maxpool2d_s8": [_p, _p, _p] + [_i] * 13,
     "sofie_hip_relayout_s8": [_p, _p, _p] + [_i] * 6,
     "sofie_hip_transpose_bytes": [_p, _p, _p, _i, _i, _i, _i],

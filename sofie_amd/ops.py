@@ -281,6 +281,32 @@ def qconv2d_pool_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=
     return _ret(y, x)
 
 
+def quantize_qconv2d_s8(x, x_scale, zpx, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zpy=0, relu=False,
+                        pool=None, pool_strides=(2, 2), y_layout=L.LAYOUT_NCHW, w_layout=L.LAYOUT_NCHW, ctx=None):
+    """QuantizeLinear(x float NCHW) -> QLinearConv -> (ReLU) -> (MaxPool) in one library call."""
+    ctx = ctx or default_context()
+    if zpx != 0:
+        bias = fold_zero_point_conv(w, bias, zpx)
+    xd, wd = ctx.dev(x, torch.float32), ctx.dev(w, torch.int8)
+    N, Cc, H, W = xd.shape
+    if w_layout == L.LAYOUT_NCHW:
+        OC, _, kh, kw = wd.shape
+    else:
+        OC, kh, kw, _ = wd.shape
+    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1])
+    if pool:
+        OH, OW = (OH - pool[0]) // pool_strides[0] + 1, (OW - pool[1]) // pool_strides[1] + 1
+    y = ctx.empty((N, OC, OH, OW) if y_layout == L.LAYOUT_NCHW else (N, OH, OW, OC), torch.int8)
+    sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
+    pk = pool or (0, 0)
+    ctx.check(ctx.lib.sofie_hip_quantize_qconv2d_s8(ctx.h, ctx.ptr(xd), float(x_scale), int(zpx), ctx.ptr(wd), w_layout,
+                                                    ctx.ptr(bd), ctx.ptr(sd), ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw,
+                                                    pads[0], pads[1], strides[0], strides[1], groups, int(zpy),
+                                                    L.ACT_RELU if relu else L.ACT_NONE, pk[0], pk[1],
+                                                    pool_strides[0] if pool else 0, pool_strides[1] if pool else 0))
+    return _ret(y, x)
+
+
 def iconv2d_s8(x, w, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, ctx=None):
     return qconv2d_s8(x, w, None, None, pads, strides, groups, zpx, out=L.OUT_S32, ctx=ctx)
 

@@ -104,14 +104,17 @@ def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
     hxx, dat, _ = gen(spec, tmp_path)
     code = open(hxx).read()
     # conv1 and conv2 absorb their MaxPool; the unpooled tensors no longer exist
-    assert code.count("sofie_hip_qconv2d_pool_s8(") == 2 and code.count("sofie_hip_qconv2d_s8(") == 1
+    assert code.count("sofie_hip_qconv2d_pool_s8(") == 1 and code.count("sofie_hip_qconv2d_s8(") == 1
+    assert code.count("sofie_hip_quantize_qconv2d_s8(") == 1
     assert "sofie_hip_maxpool2d_s8" not in code and "tensor_c1" not in code.replace("tensor_c1_q", "") and "tensor_r2" not in code
     assert code.count("sofie_hip_qgemm_s8(") == 2
     assert "int8_t * tensor_fc1_nk_cl" in code and "tensor_fc1 =" not in code   # transposed once, original dropped
     assert "tensor_w2_ohwi, SOFIE_LAYOUT_NHWC" in code and "tensor_w2 =" not in code
     # conv1 reads the one-channel quantized input as it is, everything after it is channels-last
-    assert code.count("SOFIE_LAYOUT_NCHW, tensor_w") == 1
-    assert "tensor_p1, SOFIE_LAYOUT_NHWC, 2, 1, 40, 40, 32, 3, 3, 1, 1, 1, 1, 1, -128, -128, SOFIE_ACT_RELU, 2, 2, 2, 2)" in code
+    # the first layer also absorbs the QuantizeLinear in front of it: it reads the float input
+    assert "sofie_hip_quantize_f32_s8" not in code and "tensor_xq" not in code
+    assert "sofie_hip_quantize_qconv2d_s8(fCtx, tensor_x, static_cast<float>(0.00392156886), -128, tensor_w1_ohwi" in code
+    assert "tensor_p1, SOFIE_LAYOUT_NHWC, 2, 1, 40, 40, 32, 3, 3, 1, 1, 1, 1, 1, -128, SOFIE_ACT_RELU, 2, 2, 2, 2)" in code
     assert "SOFIE_OUT_F32" in code and "std::vector<float> infer(float* tensor_x)" in code
     q = models.qcnn_params(oracle)
     text = open(dat).read().split("\n")

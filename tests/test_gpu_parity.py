@@ -376,6 +376,34 @@ def test_first_layer_kernel(ops, cfg):
 
 
 @pytest.mark.parametrize("cfg", [
+    dict(N=5, C=1, H=40, W=40, OC=32, k=(3, 3), p=(1, 1), pool=(2, 2)),    # first-layer kernel, dword fill
+    dict(N=3, C=1, H=9, W=7, OC=16, k=(3, 3), p=(1, 1), pool=None),        # first-layer kernel, byte fill
+    dict(N=2, C=1, H=12, W=12, OC=8, k=(3, 3), p=(1, 1), pool=(2, 2)),     # plain kernels through scratch memory
+    dict(N=2, C=32, H=8, W=8, OC=64, k=(3, 3), p=(1, 1), pool=None),       # multi-channel float input, MFMA conv
+])
+def test_quantize_conv_fused_entry_point(ops, cfg):
+    """QuantizeLinear -> QLinearConv -> ReLU -> (MaxPool) from a float tensor equals the separate oracle steps,
+    including values that saturate and exact .5 ties of x / scale."""
+    from sofie_amd import lib as L
+    r = rng(900 + cfg["H"] + cfg["OC"])
+    shape = (cfg["N"], cfg["C"], cfg["H"], cfg["W"])
+    x = r.uniform(-0.2, 1.2, shape).astype(np.float32)
+    x.reshape(-1)[::7] = (r.integers(-10, 300, x.reshape(-1)[::7].size) + 0.5) / 255.0
+    sx, zpx = np.float32(1 / 255.0), -128
+    w = r.integers(-127, 128, (cfg["OC"], cfg["C"]) + cfg["k"]).astype(np.int8)
+    K = cfg["C"] * 9
+    scale = (r.uniform(20, 60, cfg["OC"]) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    bias = r.integers(-3000, 3000, cfg["OC"]).astype(np.int32)
+    xq = oracle.quantize_f32_s8(x, sx, zpx)
+    ref = oracle.qconv2d_s8(xq, w, scale, bias, cfg["p"], (1, 1), 1, zpx, -128, True)
+    if cfg["pool"]:
+        ref = oracle.maxpool2d(ref, cfg["pool"], (2, 2))
+    y = ops.quantize_qconv2d_s8(x, sx, zpx, w, scale, bias, cfg["p"], (1, 1), 1, -128, True, cfg["pool"], (2, 2),
+                                y_layout=L.LAYOUT_NHWC)
+    assert np.array_equal(y.transpose(0, 3, 1, 2), ref)
+
+
+@pytest.mark.parametrize("cfg", [
     dict(N=2, C=32, H=20, W=20, OC=64, k=(3, 3), p=(1, 1), pool=(2, 2), ps=(2, 2)),
     dict(N=2, C=6, H=9, W=8, OC=10, k=(3, 3), p=(0, 0), pool=(3, 2), ps=(2, 1)),
     dict(N=1, C=64, H=11, W=11, OC=128, k=(3, 3), p=(1, 1), pool=(2, 2), ps=(2, 2)),
