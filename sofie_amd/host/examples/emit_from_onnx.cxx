@@ -1,0 +1,27 @@
+// ONNX file -> generated Session header and weight file, the flow of the reference's own tests
+// (src/SOFIE_core/test/EmitFromONNX.cxx.in: Parse, Generate, OutputGenerated).
+//   emit_from_onnx <model.onnx> <output directory> [--check]
+#include <iostream>
+
+#include "SOFIE/RModelParser_ONNX.hxx"
+
+int main(int argc, char **argv)
+{
+   if (argc < 3) {
+      std::cerr << "usage: emit_from_onnx <model.onnx> <output directory> [--check]\n";
+      return 2;
+   }
+   try {
+      SOFIE::RModelParser_ONNX parser;
+      if (argc > 3 && std::string(argv[3]) == "--check") return parser.CheckModel(argv[1], true) ? 0 : 1;
+      SOFIE::RModel model = parser.Parse(argv[1]);
+      model.Generate();
+      const std::string out = std::string(argv[2]) + "/" + model.GetName() + ".hxx";
+      model.OutputGenerated(out);
+      std::cout << "generated " << out << ", intermediate pool " << model.GetIntermediateMemorySize() << " bytes\n";
+   } catch (const std::exception &e) {
+      std::cerr << "emit_from_onnx: " << e.what() << "\n";
+      return 1;
+   }
+   return 0;
+}

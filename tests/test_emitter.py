@@ -183,6 +183,68 @@ def test_no_weight_file_option_embeds_literals(tmp_path):
     assert os.path.exists(exe)
 
 
+def _onnx_emit(path, outdir):
+    exe = os.path.join(emit.GEN_DIR, "emit_from_onnx")
+    return subprocess.run([exe, path, str(outdir)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+
+
+def _body(path):
+    return [line for line in open(path).read().split("\n") if not line.startswith("//Code generated")]
+
+
+@pytest.mark.parametrize("name", models.FIXTURES)
+def test_cpp_onnx_front_end_on_reference_fixtures(name, tmp_path):
+    """RModelParser_ONNX::Parse -> Generate on the reference's own .onnx files gives the same Session code and the
+    same weight file as the description-driven route the GPU tests run (so those results hold for it too)."""
+    res = _onnx_emit(os.path.join(models.GOLD, "onnx", name + ".onnx"), tmp_path)
+    assert res.returncode == 0, res.stderr
+    spec, _ = models.fixture_spec(name)
+    sub = tmp_path / "spec"
+    sub.mkdir()
+    hxx, dat, _ = spec.generate(str(sub))
+    assert _body(str(tmp_path / (name + ".hxx"))) == _body(hxx)
+    assert open(str(tmp_path / (name + ".dat"))).read() == open(dat).read()
+
+
+def test_cpp_onnx_front_end_quantized_graph_and_fusions(tmp_path):
+    """A hand-written ONNX file with int8 / int32 initializers (QuantizeLinear -> QLinearConv -> DequantizeLinear,
+    which the reference's parser rejects) and a MatMul -> Add -> Relu chain: same code as the description route,
+    MatMul + Add becomes one Gemm call."""
+    import onnx_write as ow
+    p = models.qdq_conv_params()
+    init = {"sx": np.array(p["sx"], np.float32), "zx": np.array(p["zx"], np.int8), "sy": np.array(p["sy"], np.float32),
+            "zy": np.array(p["zy"], np.int8), "w": p["w"], "sw": p["sw"], "b": p["b"]}
+    nodes = [ow.node("QuantizeLinear", ["x", "sx", "zx"], ["xq"]),
+             ow.node("QLinearConv", ["xq", "sx", "zx", "w", "sw", "", "sy", "zy", "b"], ["c"], kernel_shape=[3, 3],
+                     pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("DequantizeLinear", ["c", "sy", "zy"], ["y"])]
+    path = tmp_path / "qdq_conv.onnx"
+    path.write_bytes(ow.model(nodes, init, [("x", 1, p["x"].shape)], [("y", 1, (2, 64, 9, 7))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode == 0, res.stderr
+    sub = tmp_path / "spec"
+    sub.mkdir()
+    hxx, dat, _ = models.qdq_conv_spec().generate(str(sub))
+    assert _body(str(tmp_path / "qdq_conv.hxx")) == _body(hxx)
+    assert open(str(tmp_path / "qdq_conv.dat")).read() == open(dat).read()
+
+    r = np.random.default_rng(5)
+    init = {"W": r.standard_normal((6, 4)).astype(np.float32), "B": r.standard_normal(4).astype(np.float32)}
+    nodes = [ow.node("MatMul", ["x", "W"], ["m"]), ow.node("Add", ["m", "B"], ["a"]), ow.node("Relu", ["a"], ["y"])]
+    path = tmp_path / "mm_add.onnx"
+    path.write_bytes(ow.model(nodes, init, [("x", 1, (3, 6))], [("y", 1, (3, 4))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode == 0, res.stderr
+    code = open(str(tmp_path / "mm_add.hxx")).read()
+    assert code.count("sofie_hip_gemm_f32(") == 1 and "tensor_B, 1, tensor_a, 4, SOFIE_ACT_RELU" in code
+
+    # an operator outside the path is reported the way the reference words it
+    path = tmp_path / "bad.onnx"
+    path.write_bytes(ow.model([ow.node("Softmax", ["x"], ["y"])], {}, [("x", 1, (3, 6))], [("y", 1, (3, 6))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode != 0 and "Operator type Softmax is not yet supported" in res.stderr
+
+
 def test_every_prebuilt_session_compiles():
     """tests/build_generated.py output (made by build()): header, weights and runner of each network."""
     import build_generated
