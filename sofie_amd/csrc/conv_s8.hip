@@ -220,18 +220,23 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    };
 
    // K loop over (kh, kw, 32-channel block) of one tile into acc; the accumulators start at the
-   // bias. Fragments of step s+1 are read while the matrix instructions of step s issue.
+   // bias. Fragments of later steps are read while the matrix instructions of the current step issue.
+   // r_bias (unpooled variant): the bias as accumulator tiles, loaded once; it is the C operand of the first
+   // step's matrix instructions, which saves copying it into every accumulator of every tile.
+   v16i r_bias[POOL ? 1 : NB];
    auto kloop = [&](v16i (&acc)[NB][MB]) {
+      if constexpr (POOL) {
 #pragma unroll
-      for (int i = 0; i < NB; ++i)
+         for (int i = 0; i < NB; ++i)
 #pragma unroll
-         for (int q = 0; q < 4; ++q) {
-            const v4i bi = *reinterpret_cast<const v4i *>(w_bias + i * 32 + q * 8 + nq);
+            for (int q = 0; q < 4; ++q) {
+               const v4i bi = *reinterpret_cast<const v4i *>(w_bias + i * 32 + q * 8 + nq);
 #pragma unroll
-            for (int j = 0; j < MB; ++j)
+               for (int j = 0; j < MB; ++j)
 #pragma unroll
-               for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = bi[e];
-         }
+                  for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = bi[e];
+            }
+      }
       v4i fa[POOL ? 2 : 3][MB], fb[POOL ? 2 : 3][NB];
       int ka = 0, kb = 0, c32 = 0, kw = 0;
       auto advance = [&]() {
@@ -261,20 +266,29 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          load(0, true);
          advance();
          load(1, nsteps > 1);
-         int s = 0;
+         // step 0 starts the accumulators from the bias tiles
+         advance();
+         load(2, nsteps > 2);
+         if constexpr (!POOL) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+               for (int j = 0; j < MB; ++j) acc[i][j] = MmaI8::mma(fb[0][i], fa[0][j], r_bias[i]);
+         }
+         int s = 1;   // steps s and s+1 sit in buffers 1 and 2
          for (; s + 2 < nsteps; s += 3) {
             advance();
-            load(2, true);
-            mma(0);
-            advance();
-            load(0, s + 3 < nsteps);
+            load(0, true);
             mma(1);
             advance();
-            load(1, s + 4 < nsteps);
+            load(1, s + 3 < nsteps);
             mma(2);
+            advance();
+            load(2, s + 4 < nsteps);
+            mma(0);
          }
-         if (s < nsteps) mma(0);
-         if (s + 1 < nsteps) mma(1);
+         if (s < nsteps) mma(1);
+         if (s + 1 < nsteps) mma(2);
       } else {
          // the pooled variant has twice the accumulators and keeps two fragment buffers
          load(0, true);
@@ -340,8 +354,12 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    __syncthreads();   // weights and column parameters are in LDS
    if constexpr (!POOL) {
 #pragma unroll
-      for (int gi = 0; gi < NB * 4; ++gi)
+      for (int gi = 0; gi < NB * 4; ++gi) {
          r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+         const v4i bi = *reinterpret_cast<const v4i *>(w_bias + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+#pragma unroll
+         for (int e = 0; e < 4; ++e) r_bias[gi >> 2][(gi & 3) * 4 + e] = bi[e];
+      }
    }
    v16i acc[NB][MB];
    while (t < a.ntiles) {

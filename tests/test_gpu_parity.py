@@ -455,6 +455,42 @@ def test_conv_pool_fused_matrix_core_kernel(ops, cfg):
         assert np.array_equal(y.transpose(0, 3, 1, 2), ref), (zpx, zpy, relu)
 
 
+def test_error_codes_of_the_quantized_entry_points(ops):
+    """Bad arguments come back as SOFIE_HIP_EINVAL with a message and launch nothing; the context stays usable."""
+    from sofie_amd import lib as L
+    ctx = ops.default_context()
+    x = ctx.dev(np.zeros((1, 4, 4, 32), np.int8))
+    w = ctx.dev(np.zeros((64, 3, 3, 32), np.int8))
+    sc = ctx.dev(np.ones(64, np.float32))
+    y = ctx.empty((1, 4, 4, 64), torch.int8)
+    lib, h, p = ctx.lib, ctx.h, ctx.ptr
+
+    def conv(**kw):
+        a = dict(x=p(x), xl=L.LAYOUT_NHWC, w=p(w), wl=L.LAYOUT_NHWC, s=p(sc), y=p(y), groups=1, zpx=0, act=L.ACT_NONE,
+                 out=L.OUT_S8, ph=1)
+        a.update(kw)
+        return lib.sofie_hip_qconv2d_s8(h, a["x"], a["xl"], a["w"], a["wl"], None, a["s"], a["y"], L.LAYOUT_NHWC, 1, 32, 4, 4,
+                                        64, 3, 3, a["ph"], 1, 1, 1, a["groups"], a["zpx"], 0, a["act"], a["out"])
+    assert conv() == 0
+    for bad, text in ((dict(x=None), "null operand"), (dict(groups=3), "groups"), (dict(zpx=300), "zero-point"),
+                      (dict(act=7), "activation"), (dict(xl=5), "layout"), (dict(out=L.OUT_BF16), "output kind"),
+                      (dict(s=None), "scale is required"), (dict(ph=-1), "pads")):
+        assert conv(**bad) == L.EINVAL, bad
+        assert text in lib.sofie_hip_last_error(h).decode(), (bad, lib.sofie_hip_last_error(h))
+    assert lib.sofie_hip_qconv2d_pool_s8(h, p(x), 1, p(w), 1, None, p(sc), p(y), 1, 1, 32, 4, 4, 64, 3, 3, 1, 1, 1, 1, 1, 0, 0,
+                                         0, 9, 9, 1, 1) == L.EINVAL
+    assert "pooling window" in lib.sofie_hip_last_error(h).decode()
+    assert lib.sofie_hip_quantize_qconv2d_s8(h, p(ctx.dev(np.zeros((1, 32, 4, 4), np.float32))), -1.0, 0, p(w), 1, None, p(sc),
+                                             p(y), 1, 1, 32, 4, 4, 64, 3, 3, 1, 1, 1, 1, 1, 0, 0, 0, 0, 0, 0) == L.EINVAL
+    A = ctx.dev(np.zeros((16, 16), np.int8))
+    Y = ctx.empty((16, 16), torch.int8)
+    assert lib.sofie_hip_qgemm_s8(h, 1, 16, 16, 16, p(A), 8, p(A), 16, p(ctx.dev(np.ones(16, np.float32))), None, 0, 0, p(Y), 16,
+                                  L.OUT_S8) == L.EINVAL
+    assert "leading dimension" in lib.sofie_hip_last_error(h).decode()
+    assert conv() == 0      # still works
+    ctx.sync()
+
+
 # --------------------------------------------------------------------------- fp8
 def fp8_operands(r, M, N, K, transB):
     a = r.standard_normal((M, K)).astype(np.float32)
