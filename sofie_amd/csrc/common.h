@@ -66,6 +66,26 @@ __device__ __forceinline__ unsigned f32_to_bf16(float x)
 // Layout change of an int8 activation tensor (defined with the element-wise kernels).
 int relayout_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int N, int C, int H, int W, int from, int to);
 
+// floor(x / d) for 0 <= x < 2^31 as a multiply-high and a shift (shift < 0: d == 1).
+struct FastDiv {
+   unsigned magic;
+   int shift;
+};
+
+inline FastDiv make_fastdiv(unsigned d)
+{
+   if (d <= 1) return {0u, -1};
+   int s = 0;
+   while ((1u << s) < d) ++s;
+   const unsigned long long num = 1ull << (31 + s);
+   return {(unsigned)((num + d - 1) / d), s - 1};
+}
+
+__device__ __forceinline__ int fdiv(int x, FastDiv f)
+{
+   return f.shift < 0 ? x : (int)(__umulhi((unsigned)x, f.magic) >> f.shift);
+}
+
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -26,6 +26,7 @@ struct ConvArgs {
    int PH, PW;         // staged patch extent
    int rows_out;       // output rows a pixel tile can span
    int relu;
+   FastDiv dPW, dPH, dKC;   // divisions by the patch extents and the K-chunk length in the staging loops
 };
 
 template <int TI, int TJ>
@@ -82,7 +83,8 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       const int kc = icn * KHW;
       __syncthreads();   // previous chunk fully consumed (also orders the koff table on entry)
       for (int e = tid; e < patch_len; e += 256) {
-         const int c = e % g.PW, r = (e / g.PW) % g.PH, icl = e / (g.PW * g.PH);
+         const int t = fdiv(e, g.dPW), c = e - t * g.PW;
+         const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
          const int ih = ih0 + r, iw = iw0 + c;
          float v = 0.0f;
          if (icl < icn && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
@@ -90,7 +92,7 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
          patch[e] = v;
       }
       for (int e = tid; e < g.KC * BOC; e += 256) {
-         const int k = e % g.KC, ocl = e / g.KC;
+         const int ocl = fdiv(e, g.dKC), k = e - ocl * g.KC;
          float v = 0.0f;
          if (k < kc && oc0 + ocl < g.ocg) v = wg[(size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k];
          sW[k * LDW + ocl] = v;
@@ -188,6 +190,9 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
       }
    }
    if (icb < 1) return SOFIE_HIP_OK;   // does not fit: caller uses the simple kernel
+   g.dPW = make_fastdiv((unsigned)g.PW);
+   g.dPH = make_fastdiv((unsigned)g.PH);
+   g.dKC = make_fastdiv((unsigned)g.KC);
    const int octiles = cdiv(g.ocg, BOC);
    if ((size_t)g.groups * octiles > 65535 || g.N > 65535) return SOFIE_HIP_OK;
    auto kern = k_conv2d_f32<TI, TJ>;
