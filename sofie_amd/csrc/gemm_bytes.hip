@@ -320,9 +320,10 @@ __device__ __forceinline__ void wait_vmcnt()
    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <class Mma, int BK, int NST, int OUT>
+template <class Mma, int BK, int NST, int OUT, bool B_KN>
 __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
 {
+   static_assert(!B_KN || BK == 128, "the [K,N] operand path is laid out for 128-byte stages");
    constexpr int BM = 256, BN = 256;
    constexpr int TI = 4, TJ = 2;                      // wavefront tile: 128 n x 64 m
    constexpr int STAGE = (BM + BN) * BK;              // A rows, then B^T rows
@@ -344,12 +345,15 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    // --- loads: wavefronts 0-3 request the A tile, 4-7 the B^T tile -------------------------
    constexpr int LPW = (BM + BN) / RPB / 8;           // load blocks per wavefront and stage
    const bool uses_a = wave < 4;
+   const bool rows_are_k = B_KN && !uses_a;            // B [K,N]: a load block is 4 rows of k x 256 bytes of n
    const int ld = uses_a ? g.lda : g.ldb;
    const int rows_total = uses_a ? g.M : g.N;
    const int row0 = uses_a ? m0 : n0;
    const int rows_left = (rows_total - row0) < 256 ? (rows_total - row0) : 256;
-   const unsigned char *tile_base = (uses_a ? g.A : g.B) + (size_t)row0 * ld;
-   const rsrc_t rs = make_rsrc(tile_base, (unsigned)((size_t)(rows_left - 1) * ld + g.K));
+   const unsigned char *tile_base = rows_are_k ? g.B + n0 : (uses_a ? g.A : g.B) + (size_t)row0 * ld;
+   // rows of k past K lie beyond the descriptor and read as zeros
+   const rsrc_t rs = make_rsrc(tile_base, rows_are_k ? (unsigned)((size_t)(g.K - 1) * ld + (g.N - n0))
+                                                     : (unsigned)((size_t)(rows_left - 1) * ld + g.K));
    const int blk0 = wave * LPW;                        // first load block of this wavefront
    const int lrow = lane / CPR;                        // row inside a block
    // K-chunk this lane fetches in load block i: slot ^ swizzle(row); for BK = 128 the row
@@ -361,6 +365,17 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
       chunk[par] = (lane % CPR) ^ ((row_in_tile >> SWS) & (CPR - 1));
       voff[par] = (((blk0 * RPB) & 255) + lrow) * ld + chunk[par] * 16;
    }
+   if (rows_are_k) {
+      // [K,N] stage: row k holds 256 bytes of n as eight 32-byte pairs, pair p stored in slot p ^ (k & 7),
+      // so that the transposing LDS reads (eight rows of k, 32 bytes of n each) cover every bank once
+#pragma unroll
+      for (int par = 0; par < 2; ++par) {
+         const int krow = par * 4 + (lane >> 4);
+         const int slot = lane & 15;
+         chunk[par] = (((slot >> 1) ^ (krow & 7)) << 1) | (slot & 1);
+         voff[par] = (((blk0 - 4 * LPW) * 4) + (lane >> 4)) * ld + chunk[par] * 16;
+      }
+   }
    const bool ktail = (g.K % BK) != 0;
    const int nk = (g.K + BK - 1) / BK;
    auto request = [&](int t) {
@@ -369,14 +384,16 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
       const int tt = t < nk ? t : nk - 1;
       const int k0 = tt * BK;
       int vo[2] = {voff[0], voff[1]};
-      if (ktail) {
+      if (ktail && !rows_are_k) {
 #pragma unroll
          for (int par = 0; par < 2; ++par)
             if (k0 + chunk[par] * 16 >= g.K) vo[par] = 0x7ffffff0;   // beyond the descriptor: zeros
       }
       const unsigned dst = lds0 + (t % NST) * STAGE + blk0 * 1024;
+      const int row_step = rows_are_k ? 4 * ld : RPB * ld;
+      const int k_off = rows_are_k ? k0 * ld : k0;
 #pragma unroll
-      for (int i = 0; i < LPW; ++i) dma16(rs, dst + i * 1024, vo[(BK == 128) ? (i & 1) : 0], i * RPB * ld + k0);
+      for (int i = 0; i < LPW; ++i) dma16(rs, dst + i * 1024, vo[(BK == 128) ? (i & 1) : 0], i * row_step + k_off);
    };
    // --- MFMA operand addresses ---------------------------------------------------------
    const int fr = lane & 31, half = lane >> 5;
@@ -397,6 +414,28 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
          typename Mma::Frag f = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
          return f;
       }
+   };
+
+   // B [K,N]: ds_read_b64_tr_b8 hands a lane eight consecutive k of its column. Of a group of 16 lanes,
+   // lane s points at row (s >> 1), bytes (s & 1) * 8 .. + 7 of the group's 16 columns; lane t of the
+   // group then receives column t of those eight rows. A fragment is the same K slice the A operand reads.
+   const int ts = lane & 15;
+   const int kn_off = BM * BK + (ts >> 1) * 256 + ((((wn * 4) ^ (ts >> 1)) & 7) * 32) + ((lane >> 4) & 1) * 16 + (ts & 1) * 8;
+   auto load_frag_kn = [&](const unsigned char *stage, int i, int sub) -> typename Mma::Frag {
+      typedef int v2i_t __attribute__((ext_vector_type(2)));
+      constexpr int NR = Mma::LANE_BYTES / 8;
+      // first 16-byte chunk of K this half of the wavefront holds in sub-step `sub` (as in load_frag)
+      const int ck = Mma::LANE_BYTES == 16 ? (sub >> 1) * 4 + half * 2 + (sub & 1) : sub * 4 + half * 2;
+      const unsigned char *p = stage + ((kn_off + ck * 16 * 256) ^ (i * 32));
+      typename Mma::Frag f;
+#pragma unroll
+      for (int v = 0; v < NR; ++v) {
+         const v2i_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+            (v2i_t __attribute__((address_space(3))) *)(p + v * 8 * 256));
+         f[2 * v] = r[0];
+         f[2 * v + 1] = r[1];
+      }
+      return f;
    };
 
    typename Mma::Acc acc[TI][TJ];
@@ -434,7 +473,10 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
 #pragma unroll
       for (int sub = 0; sub < NSUB; ++sub) {
 #pragma unroll
-         for (int i = 0; i < TI; ++i) fn[sub][i] = load_frag(stage, n_off + i * 32 * BK, sub);
+         for (int i = 0; i < TI; ++i) {
+            if constexpr (B_KN) fn[sub][i] = load_frag_kn(stage, i, sub);
+            else fn[sub][i] = load_frag(stage, n_off + i * 32 * BK, sub);
+         }
 #pragma unroll
          for (int j = 0; j < TJ; ++j) fm[sub][j] = load_frag(stage, m_off + j * 32 * BK, sub);
       }
@@ -613,7 +655,7 @@ int launch_tiled(sofie_hip_ctx *ctx, GemmArgs &g)
    return launch_tiled_impl<Mma, BK, NSETS, TI, TJ, OUT, B_KN, false>(ctx, g);
 }
 
-template <class Mma, int BK, int NST, int OUT>
+template <class Mma, int BK, int NST, int OUT, bool B_KN = false>
 int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
 {
    constexpr size_t stage_bytes = (size_t)NST * 512 * BK;
@@ -622,7 +664,7 @@ int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
    static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
    g.tiles_m = cdiv(g.M, 256);
    g.tiles_n = cdiv(g.N, 256);
-   auto kern = k_gemm_dma<Mma, BK, NST, OUT>;
+   auto kern = k_gemm_dma<Mma, BK, NST, OUT, B_KN>;
    SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(512), lds, ctx->stream, g);
@@ -667,6 +709,11 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
       if (cdiv(g.M, 128) * cdiv(g.N, 128) * 2 <= ctx->num_cus && g.K >= 1024)
          return launch_tiled<Mma, BK, NSETS, 1, 1, OUT, false>(ctx, g);
       return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, false>(ctx, g);
+   }
+   if (big && g.ldb % 16 == 0 && aligned16(g.B) && (size_t)256 * g.lda + g.K < (1u << 31) &&
+       (size_t)(g.K + 128) * g.ldb < (1u << 31)) {
+      // B [K,N] as it lies: rows of k go to LDS and the transposing LDS read builds the operand
+      return launch_dma<Mma, SOFIE_DMA_BK, SOFIE_DMA_NST, OUT, true>(ctx, g);
    }
    if (big && g.K % 16 == 0 && (size_t)256 * g.lda + g.K < (1u << 31) && (size_t)257 * g.K < (1u << 31)) {
       // B [K,N] -> B^T [N,K] in the context's scratch buffer, then the K-contiguous kernel.

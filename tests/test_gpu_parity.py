@@ -253,6 +253,25 @@ def test_qgemm_s8_full_size_properties(ops):
     assert np.array_equal(acc_t, acc)
 
 
+@pytest.mark.parametrize("M,N,K", [(2100, 4112, 1040), (4096, 2048, 128), (2304, 4096, 16)])
+def test_qgemm_s8_large_b_as_k_by_n(ops, M, N, K):
+    """B [K,N] on the large-tile kernel (operand transposed by the LDS read): ragged M and N tiles,
+    a K tail, a single K step; sampled rows against the oracle and the transposed-B entry point."""
+    from sofie_amd import lib as L
+    r = rng(77 + M + N + K)
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    B = r.integers(-127, 128, (K, N)).astype(np.int8)
+    scale = (r.uniform(20.0, 60.0, N) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    bias = r.integers(-2000, 2000, N).astype(np.int32)
+    At, Bt = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    acc = ops.igemm_s8(At, Bt).cpu().numpy()
+    rows = np.concatenate([np.arange(0, 40), r.integers(0, M, 40), np.arange(M - 40, M)])
+    assert np.array_equal(acc[rows], oracle.igemm_s8(A[rows], B))
+    assert np.array_equal(acc, ops.igemm_s8(At, Bt.t().contiguous(), True).cpu().numpy())
+    y = ops.qgemm_s8(At, Bt, torch.from_numpy(scale).cuda(), torch.from_numpy(bias).cuda(), zpy=3, relu=True).cpu().numpy()
+    assert np.array_equal(y[rows], oracle.qgemm_s8(A[rows], B, scale, bias, zpy=3, relu=True))
+
+
 def test_qgemm_rounding_ties_and_saturation(ops):
     """Scale 0.5 (and 0.25, 1.5) makes every odd accumulator an exact tie; the byte-packing epilogues must round
     them half to even like the oracle, for the zero-point -128 path (conversion instruction does the rounding)
@@ -537,6 +556,19 @@ def test_gemm_fp8(ops, M, N, K, transB):
     assert np.all(np.abs(got - truth) <= 2.0 ** -8 * np.abs(truth) + slack)
     # the bf16 output is exactly the RNE rounding of the fp32 output of the same kernel
     assert np.array_equal(yb, oracle.bf16_encode(yf))
+
+
+def test_gemm_fp8_large_b_as_k_by_n(ops):
+    """B [K,N] on the large-tile FP8 kernel: small integers make every sum exact, so the result must
+    equal the integer product, ragged tiles and K tail included."""
+    from sofie_amd import lib as L
+    r = rng(16)
+    M, N, K = 2100, 4112, 1040
+    a = r.integers(-4, 5, (M, K)).astype(np.float32)
+    b = r.integers(-4, 5, (K, N)).astype(np.float32)
+    A, B = oracle.e4m3_encode(a), oracle.e4m3_encode(b)
+    y = ops.gemm_fp8(A, B, 1.0, 1.0, None, False, out=L.OUT_F32)
+    assert np.array_equal(y, a @ b)
 
 
 def test_gemm_fp8_exact_for_small_integers(ops):
