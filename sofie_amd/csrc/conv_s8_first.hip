@@ -2,16 +2,20 @@
 // requantisation, the ReLU clamp and (optionally) a 2x2 stride-2 max pooling fused.
 //
 // With K = 9 the layer is bound by its output bytes, so the point is to spend few vector instructions
-// per output. A workgroup keeps four zero-point-padded images in LDS; a wavefront takes 32 (pooled)
+// per output. A workgroup keeps a few zero-point-padded images in LDS; a wavefront takes 32 (pooled)
 // pixels at a time and computes them with v_mfma_i32_32x32x16_i8, K = 16 laid out as the three
-// kernel rows of four bytes (three taps and a zero weight) plus four zero weights. With that order the
+// kernel rows of four bytes (a zero weight and three taps) plus four zero weights. With that order the
 // pixel operand of a lane is simply two 4-byte windows of consecutive image rows (lanes 0-31: rows
 // y, y+1; lanes 32-63: rows y+2, y+3), cut out of aligned dwords with v_alignbyte; no byte shuffling.
+// An image row sits in LDS behind four bytes of padding, so image dword j is LDS dword j + 1 and the
+// staging is one aligned store per four pixels; the window of output column x starts at padded byte x + 2.
 // For the pooled variant the four window positions are four matrix instructions whose accumulators are
 // pooled register-wise (on the int32 values: requantisation is monotonic in the accumulator; if any
 // scale of the workgroup's channels is negative, the minimum is taken for those channels), so a quarter
 // of the values is converted. Two v_permlane32_swap turn the lane's four 4-channel groups into 16
 // consecutive channels and the result leaves as one 16-byte store per lane.
+#include <math.h>
+#include <type_traits>
 #include "conv_s8.h"
 
 using namespace sofie;
@@ -32,11 +36,13 @@ struct FirstArgs {
    int img_bytes;         // LDS bytes of one padded image
    int ocb;               // blocks of 32 output channels (the last may be half used)
    int rows;              // LDS rows of one padded image (H + 3)
-   int dword_fill;        // W % 4 == 0 and x 4-byte aligned: the images are filled a dword at a time
+   int images;            // images per workgroup
+   int dword_fill;        // W % 4 == 0 and x aligned: the images are filled a dword at a time
+   int fast_div;          // x / xscale as a reciprocal multiply and two fused corrections (see quantize4)
+   float xinv;            // 1 / xscale, correctly rounded
    FastDiv drows, dper_image, dPW;
 };
 
-constexpr int kImages = 4;   // images per workgroup
 
 __device__ __forceinline__ void windows(const unsigned char *row, int col, int &w0, int &w1)
 {
@@ -66,6 +72,30 @@ __device__ __forceinline__ unsigned quantize_byte(float v, float scale, int zp)
    return (unsigned)min(127, max(-128, (int)r + zp)) & 0xffu;
 }
 
+// Four values to four bytes, the same result as quantize_byte. With FAST the quotient is q0 = x * inv
+// corrected once, q = fma(fma(-q0, scale, x), inv, q0): for inv = RN(1 / scale) that is the correctly rounded
+// x / scale (the remainder is exact in the fused operation); the host takes this path only for
+// 2^-30 <= |scale| <= 2^30, and x is clamped to +-2^45 first (beyond it the result saturates either way), so
+// nothing overflows. zpo = zp + 128: the byte conversion saturates to [0, 255] and rounds an integer to itself.
+template <bool FAST>
+__device__ __forceinline__ unsigned quantize4(v4f v, float scale, float inv, int zp, float zpo)
+{
+   if constexpr (!FAST) {
+      return quantize_byte(v[0], scale, zp) | (quantize_byte(v[1], scale, zp) << 8) |
+             (quantize_byte(v[2], scale, zp) << 16) | (quantize_byte(v[3], scale, zp) << 24);
+   } else {
+      unsigned pk = 0;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+         const float x = __builtin_amdgcn_fmed3f(v[t], -0x1p45f, 0x1p45f);
+         const float q0 = __fmul_rn(x, inv);
+         const float q = __fmaf_rn(__fmaf_rn(-q0, scale, x), inv, q0);
+         pk = __builtin_amdgcn_cvt_pk_u8_f32(__fadd_rn(rintf(q), zpo), t, pk);
+      }
+      return pk ^ 0x80808080u;
+   }
+}
+
 template <bool POOL>
 __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
 {
@@ -78,8 +108,8 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
    unsigned char *const s_img = reinterpret_cast<unsigned char *>(s_flag + 4);
    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
    const int half = lane >> 5, l32 = lane & 31;
-   const int n0 = blockIdx.x * kImages;
-   const int nimg = (a.N - n0) < kImages ? (a.N - n0) : kImages;
+   const int n0 = blockIdx.x * a.images;
+   const int nimg = (a.N - n0) < a.images ? (a.N - n0) : a.images;
 
    if (tid == 0) s_flag[0] = 0;
    __syncthreads();
@@ -90,8 +120,8 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
       if (real) {
 #pragma unroll
          for (int k = 0; k < 3; ++k)
-            r[k] = (unsigned)(unsigned char)w[k * 3] | ((unsigned)(unsigned char)w[k * 3 + 1] << 8) |
-                   ((unsigned)(unsigned char)w[k * 3 + 2] << 16);
+            r[k] = ((unsigned)(unsigned char)w[k * 3] << 8) | ((unsigned)(unsigned char)w[k * 3 + 1] << 16) |
+                   ((unsigned)(unsigned char)w[k * 3 + 2] << 24);
       }
       s_wfrag[oc * 2] = pack64((int)r[0], (int)r[1]);      // lanes 0-31: kernel rows 0 and 1
       s_wfrag[oc * 2 + 1] = pack64((int)r[2], 0);          // lanes 32-63: kernel row 2 and four zero weights
@@ -100,65 +130,58 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
       s_bias[oc] = (real && a.bias) ? a.bias[oc] : 0;
       if (sc < 0.0f) s_flag[0] = 1;
    }
-   // padded images: border cells hold the input zero-point; one spare row below each image is read (with
-   // zero weights) by the upper half of the wavefront
+   // padded images: cells outside the image hold the input zero-point; one spare row below each image is
+   // read (with zero weights) by the upper half of the wavefront
    if (a.dword_fill) {
-      // LDS dword j of a row = padded columns 4j..4j+3 = image columns 4j-1..4j+2: the last byte of image
-      // dword j-1 and the first three of image dword j. 16 threads per row, 16 rows per pass.
+      // LDS dword j of a row = image columns 4j-4 .. 4j-1. 16 threads per row, 16 rows per pass.
       const int SD = a.stride >> 2, WD = a.W >> 2;
       const unsigned zp4 = 0x01010101u * (unsigned)(a.zpx & 0xff);
+      const float zpo = (float)(a.zpx + 128);
       const int jj = tid & 15, rsub = tid >> 4;
       const int total_rows = nimg * a.rows;
       constexpr int UN = 6;   // rows per thread whose loads are in flight together
       for (int j = jj; j < SD; j += 16) {
+         const bool col_inside = j >= 1 && j <= WD;
+         const int jsrc = col_inside ? j - 1 : 0;
          for (int base = 0; base < total_rows; base += 16 * UN) {
-            unsigned lo[UN], hi[UN];
-            float flo[UN];
-            v4f fhi[UN];
-            bool has_lo[UN], has_hi[UN];
+            unsigned q[UN];
+            v4f f[UN];
+            bool inside[UN];
             unsigned *dst[UN];
 #pragma unroll
             for (int u = 0; u < UN; ++u) {
                const int row_id = base + u * 16 + rsub;
                const int rid = row_id < total_rows ? row_id : total_rows - 1;
                const int im = fdiv(rid, a.drows);
-               const int ih = rid - im * a.rows - 1;
-               const bool row_inside = row_id < total_rows && ih >= 0 && ih < a.H;
-               const unsigned *gsrc =
-                  reinterpret_cast<const unsigned *>(a.x + ((size_t)(n0 + im) * a.H + (row_inside ? ih : 0)) * a.W);
-               dst[u] = row_id < total_rows
-                           ? reinterpret_cast<unsigned *>(s_img + im * a.img_bytes + (rid - im * a.rows) * a.stride) + j
-                           : nullptr;
-               has_lo[u] = row_inside && j >= 1 && j - 1 < WD;
-               has_hi[u] = row_inside && j < WD;
-               if (a.xf) {
-                  // image columns 4j-1 .. 4j+2 as floats, quantized here
-                  const float *fsrc = a.xf + ((size_t)(n0 + im) * a.H + (row_inside ? ih : 0)) * a.W;
-                  flo[u] = fsrc[has_lo[u] ? 4 * j - 1 : 0];
-                  fhi[u] = *reinterpret_cast<const v4f *>(fsrc + (has_hi[u] ? 4 * j : 0));
-               } else {
-                  lo[u] = gsrc[has_lo[u] ? j - 1 : 0];
-                  hi[u] = gsrc[has_hi[u] ? j : 0];
-               }
+               const int lr = rid - im * a.rows;
+               const int ih = lr - 1;
+               inside[u] = col_inside && row_id < total_rows && ih >= 0 && ih < a.H;
+               const size_t src = ((size_t)(n0 + im) * a.H + (inside[u] ? ih : 0)) * a.W;
+               dst[u] = row_id < total_rows ? reinterpret_cast<unsigned *>(s_img + im * a.img_bytes + lr * a.stride) + j
+                                            : nullptr;
+               // the loads are unconditional (of the row's first cells when the cell is outside)
+               if (a.xf) f[u] = *reinterpret_cast<const v4f *>(a.xf + src + 4 * jsrc);
+               else q[u] = reinterpret_cast<const unsigned *>(a.x + src)[jsrc];
             }
             if (a.xf) {
+               if (a.fast_div) {
 #pragma unroll
-               for (int u = 0; u < UN; ++u) {
-                  lo[u] = quantize_byte(flo[u], a.xscale, a.zpx) << 24;
-                  hi[u] = quantize_byte(fhi[u][0], a.xscale, a.zpx) | (quantize_byte(fhi[u][1], a.xscale, a.zpx) << 8) |
-                          (quantize_byte(fhi[u][2], a.xscale, a.zpx) << 16);
+                  for (int u = 0; u < UN; ++u) q[u] = quantize4<true>(f[u], a.xscale, a.xinv, a.zpx, zpo);
+               } else {
+#pragma unroll
+                  for (int u = 0; u < UN; ++u) q[u] = quantize4<false>(f[u], a.xscale, a.xinv, a.zpx, zpo);
                }
             }
 #pragma unroll
             for (int u = 0; u < UN; ++u)
-               if (dst[u]) *dst[u] = __builtin_amdgcn_alignbyte(has_hi[u] ? hi[u] : zp4, has_lo[u] ? lo[u] : zp4, 3u);
+               if (dst[u]) *dst[u] = inside[u] ? q[u] : zp4;
          }
       }
    } else {
       for (int i = tid; i < nimg * a.img_bytes; i += 256) {
          const int im = i / a.img_bytes, o = i - im * a.img_bytes;
          const int r = o / a.stride, c = o - r * a.stride;
-         const int ih = r - 1, iw = c - 1;
+         const int ih = r - 1, iw = c - 4;
          const bool inside = ih >= 0 && ih < a.H && iw >= 0 && iw < a.W;
          const size_t src = ((size_t)(n0 + im) * a.H + (inside ? ih : 0)) * a.W + (inside ? iw : 0);
          const unsigned char v = a.xf ? (unsigned char)quantize_byte(a.xf[src], a.xscale, a.zpx) : (unsigned char)a.x[src];
@@ -178,9 +201,6 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
    // (e/4)*8 + half*4 + e%4. With one block they are loaded once.
    long wfrag = 0;
    v16i binit;
-   v16i zero16;
-#pragma unroll
-   for (int e = 0; e < 16; ++e) zero16[e] = 0;
    v4f sc[4];
    auto load_params = [&](int ob) {
       wfrag = s_wfrag[(ob * 32 + l32) * 2 + half];
@@ -194,67 +214,82 @@ __global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
    };
    const bool single = a.ocb == 1;
    load_params(0);
-   for (int g = wave; g < groups; g += 4) {
-      const int q = g * 32 + l32;
-      const int qq = q < total ? q : total - 1;
-      const int im = fdiv(qq, a.dper_image), rem = qq - im * per_image;
-      const int py = fdiv(rem, a.dPW), px = rem - py * a.PW;
-      const int row0 = (POOL ? 2 * py : py) + 2 * half, col = POOL ? 2 * px : px;
-      const unsigned char *base = s_img + im * a.img_bytes + row0 * a.stride;
-      long pix[NP];
-      if constexpr (POOL) {
-         int r[3][2];
-#pragma unroll
-         for (int k = 0; k < 3; ++k) windows(base + k * a.stride, col, r[k][0], r[k][1]);
-#pragma unroll
-         for (int j = 0; j < 4; ++j) pix[j] = pack64(r[j >> 1][j & 1], r[(j >> 1) + 1][j & 1]);
-      } else {
-         pix[0] = pack64(window(base, col), window(base + a.stride, col));
-      }
-      int8_t *out = a.y + ((size_t)(n0 + im) * per_image + rem) * a.OC;
-      for (int ob = 0; ob < a.ocb; ++ob) {
-         if (!single) load_params(ob);
-         // one window position at a time keeps two accumulator tiles live (more wavefronts per SIMD)
-         v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(wfrag, pix[0], zero16, 0, 0, 0);
+   // The loop is instantiated for the four combinations of (plain requantisation, scales of both signs): both
+   // are uniform over the launch, and a run-time select inside the loop would cost more than the arithmetic.
+   auto process = [&](auto plain_c, auto negative_c) {
+      constexpr bool PLAIN = decltype(plain_c)::value;
+      constexpr bool NEGATIVE = decltype(negative_c)::value;
+      for (int g = wave; g < groups; g += 4) {
+         const int q = g * 32 + l32;
+         const int qq = q < total ? q : total - 1;
+         const int im = fdiv(qq, a.dper_image), rem = qq - im * per_image;
+         const int py = fdiv(rem, a.dPW), px = rem - py * a.PW;
+         const int row0 = (POOL ? 2 * py : py) + 2 * half, col = (POOL ? 2 * px : px) + 2;
+         const unsigned char *base = s_img + im * a.img_bytes + row0 * a.stride;
+         long pix[NP];
          if constexpr (POOL) {
-            v16i lo = acc;
+            int r[3][2];
 #pragma unroll
-            for (int j = 1; j < 4; ++j) {
-               const v16i c = __builtin_amdgcn_mfma_i32_32x32x16_i8(wfrag, pix[j], zero16, 0, 0, 0);
+            for (int k = 0; k < 3; ++k) windows(base + k * a.stride, col, r[k][0], r[k][1]);
 #pragma unroll
-               for (int e = 0; e < 16; ++e) acc[e] = max(acc[e], c[e]);
-               if (any_negative) {
+            for (int j = 0; j < 4; ++j) pix[j] = pack64(r[j >> 1][j & 1], r[(j >> 1) + 1][j & 1]);
+         } else {
+            pix[0] = pack64(window(base, col), window(base + a.stride, col));
+         }
+         int8_t *out = a.y + ((size_t)(n0 + im) * per_image + rem) * a.OC;
+         for (int ob = 0; ob < a.ocb; ++ob) {
+            if (!single) load_params(ob);
+            // one window position at a time keeps two accumulator tiles live (more wavefronts per SIMD); the
+            // bias tile is the C operand of every matrix instruction (max(a + b) = max(a) + b), which costs nothing
+            v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(wfrag, pix[0], binit, 0, 0, 0);
+            if constexpr (POOL) {
+               v16i lo;
+               if constexpr (NEGATIVE) lo = acc;
 #pragma unroll
-                  for (int e = 0; e < 16; ++e) lo[e] = min(lo[e], c[e]);
+               for (int j = 1; j < 4; ++j) {
+                  const v16i c = __builtin_amdgcn_mfma_i32_32x32x16_i8(wfrag, pix[j], binit, 0, 0, 0);
+#pragma unroll
+                  for (int e = 0; e < 16; ++e) acc[e] = max(acc[e], c[e]);
+                  if constexpr (NEGATIVE) {
+#pragma unroll
+                     for (int e = 0; e < 16; ++e) lo[e] = min(lo[e], c[e]);
+                  }
+               }
+               if constexpr (NEGATIVE) {
+#pragma unroll
+                  for (int e = 0; e < 16; ++e) acc[e] = sc[e >> 2][e & 3] < 0.0f ? lo[e] : acc[e];
                }
             }
-            if (any_negative) {
+            unsigned d[4];
 #pragma unroll
-               for (int e = 0; e < 16; ++e) acc[e] = sc[e >> 2][e & 3] < 0.0f ? lo[e] : acc[e];
+            for (int gq = 0; gq < 4; ++gq) {
+               unsigned pk = 0;
+#pragma unroll
+               for (int t = 0; t < 4; ++t) {
+                  float r = __fmul_rn(__int2float_rn(acc[gq * 4 + t]), sc[gq][t]);
+                  if constexpr (!PLAIN) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);   // the byte conversion rounds half to even itself
+                  pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);
+               }
+               d[gq] = pk ^ 0x80808080u;
             }
+            // lanes 0-31 hold channels {0-3, 8-11, 16-19, 24-27} of their pixel, lanes 32-63 {4-7, 12-15, 20-23, 28-31}:
+            // after the swaps the lower half has channels 0-15 and the upper half 16-31, in order
+            const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+            const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+            const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+            const int oc_first = ob * 32 + half * 16;
+            if (q < total && oc_first < a.OC) *reinterpret_cast<v4i *>(out + oc_first) = v;
          }
-         unsigned d[4];
-#pragma unroll
-         for (int gq = 0; gq < 4; ++gq) {
-            unsigned pk = 0;
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-               // the bias is added after the pooling (max(a + b) = max(a) + b), so the matrix instructions
-               // start from a constant zero and need no copy of an initial tile
-               float r = __fmul_rn(__int2float_rn(acc[gq * 4 + t] + binit[gq * 4 + t]), sc[gq][t]);
-               if (!plain) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);   // the byte conversion rounds half to even itself
-               pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);
-            }
-            d[gq] = pk ^ 0x80808080u;
-         }
-         // lanes 0-31 hold channels {0-3, 8-11, 16-19, 24-27} of their pixel, lanes 32-63 {4-7, 12-15, 20-23, 28-31}:
-         // after the swaps the lower half has channels 0-15 and the upper half 16-31, in order
-         const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
-         const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-         const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-         const int oc_first = ob * 32 + half * 16;
-         if (q < total && oc_first < a.OC) *reinterpret_cast<v4i *>(out + oc_first) = v;
       }
+   };
+   using yes = std::integral_constant<bool, true>;
+   using no = std::integral_constant<bool, false>;
+   if (plain) {
+      if (POOL && any_negative) process(yes{}, yes{});
+      else process(yes{}, no{});
+   } else {
+      if (POOL && any_negative) process(no{}, yes{});
+      else process(no{}, no{});
    }
 }
 
@@ -274,17 +309,36 @@ int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.x = g.x; a.xf = g.xf; a.xscale = g.xscale; a.w = g.w; a.bias = g.bias; a.scale = g.scale; a.y = static_cast<int8_t *>(g.y);
    a.N = g.N; a.H = g.H; a.W = g.W; a.OC = g.OC; a.PH = g.PH; a.PW = g.PW;
    a.zpx = g.zpx; a.zpy = g.zpy; a.lo = g.lo;
-   a.stride = (g.W + 2 + 3) / 4 * 4 + 8;          // a window may start at the last column and spans two dwords
+   a.stride = (((g.W + 2) >> 2) + 2) * 4;         // four bytes of left padding; a window spans two aligned dwords
    a.img_bytes = (g.H + 3) * a.stride;
    a.ocb = (g.OC + 31) / 32;
    a.rows = g.H + 3;
    a.dword_fill = g.W % 4 == 0 && (g.xf ? aligned16(g.xf) : (reinterpret_cast<uintptr_t>(g.x) & 3u) == 0);
+   {
+      const float as = fabsf(g.xscale);
+      a.fast_div = g.xf && as >= 0x1p-30f && as <= 0x1p30f;
+      a.xinv = a.fast_div ? 1.0f / g.xscale : 0.0f;
+   }
    a.drows = make_fastdiv((unsigned)a.rows);
    a.dper_image = make_fastdiv((unsigned)(g.PH * g.PW));
    a.dPW = make_fastdiv((unsigned)g.PW);
-   const size_t lds = (size_t)a.ocb * 32 * 24 + 16 + (size_t)kImages * a.img_bytes + 16;
-   if (lds > 64 * 1024) return SOFIE_HIP_OK;
-   const dim3 grid((unsigned)((g.N + kImages - 1) / kImages)), block(256);
+   // Images per workgroup: three workgroups share a CU, and the kernel is as slow as the busiest CU, so the
+   // count is the one that leaves the fewest image-times on a workgroup slot (rounds of workgroups x images each);
+   // of equal ones the larger (fewer parameter loads). At most 16 images and 48 KB of them.
+   const size_t fixed = (size_t)a.ocb * 32 * 24 + 16 + 16;
+   const int slots = 3 * (ctx->num_cus > 0 ? ctx->num_cus : 256);
+   int best = 0;
+   long best_cost = 0;
+   for (int k = 1; k <= 16; ++k) {
+      if (fixed + (size_t)k * a.img_bytes > 48 * 1024) break;
+      const long wgs = (g.N + k - 1) / k;
+      const long cost = ((wgs + slots - 1) / slots) * k;
+      if (best == 0 || cost <= best_cost) { best = k; best_cost = cost; }
+   }
+   if (best == 0) return SOFIE_HIP_OK;
+   a.images = best;
+   const size_t lds = fixed + (size_t)a.images * a.img_bytes;
+   const dim3 grid((unsigned)((g.N + a.images - 1) / a.images)), block(256);
    if (pool) hipLaunchKernelGGL(k_qconv_first<true>, grid, block, lds, ctx->stream, a);
    else hipLaunchKernelGGL(k_qconv_first<false>, grid, block, lds, ctx->stream, a);
    *done = true;

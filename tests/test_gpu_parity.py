@@ -422,6 +422,36 @@ def test_quantize_conv_fused_entry_point(ops, cfg):
     assert np.array_equal(y.transpose(0, 3, 1, 2), ref)
 
 
+@pytest.mark.parametrize("sx_bits,zpx", [(0x3c7fffff, -128), (0x3d17f4a8, 7), (0x2b000001, -128), (0x3b808081, 0),
+                                          (0x3c000000, -20)])
+def test_quantize_conv_fused_division_is_exact(ops, sx_bits, zpx):
+    """The first-layer kernel divides by the activation scale with a reciprocal and two fused corrections; the
+    result must equal the true float division for any scale (all-ones mantissa, a power of two, outside the range of
+    the short sequence), for exact ties, and for values far outside the int8 range."""
+    from sofie_amd import lib as L
+    r = rng(950 + zpx)
+    sx = np.array([sx_bits], np.uint32).view(np.float32)[0]
+    N, H, W, OC = 6, 16, 24, 32
+    x = (r.uniform(-140, 140, (N, 1, H, W)) * float(sx)).astype(np.float32)
+    flat = x.reshape(-1)
+    ties = ((r.integers(-200, 200, flat[::5].size) + 0.5) * float(sx)).astype(np.float32)
+    flat[::5] = ties
+    flat[1::5] = np.nextafter(ties, np.float32(0))[: flat[1::5].size]
+    flat[2::97] = np.float32(1e30)
+    flat[3::97] = np.float32(-1e30)
+    flat[4::97] = np.float32(1e-30)
+    w = r.integers(-127, 128, (OC, 1, 3, 3)).astype(np.int8)
+    scale = (r.uniform(20, 60, OC) / (73.3 * 73.3 * 3)).astype(np.float32)
+    bias = r.integers(-3000, 3000, OC).astype(np.int32)
+    xq = oracle.quantize_f32_s8(x, sx, zpx)
+    ref = oracle.maxpool2d(oracle.qconv2d_s8(xq, w, scale, bias, (1, 1), (1, 1), 1, zpx, -128, True), (2, 2), (2, 2))
+    y = ops.quantize_qconv2d_s8(x, sx, zpx, w, scale, bias, (1, 1), (1, 1), 1, -128, True, (2, 2), (2, 2),
+                                y_layout=L.LAYOUT_NHWC)
+    assert np.array_equal(y.transpose(0, 3, 1, 2), ref)
+    # and the quantizer on its own agrees with the oracle on the same input
+    assert np.array_equal(ops.quantize_f32_s8(x, sx, zpx), xq)
+
+
 @pytest.mark.parametrize("cfg", [
     dict(N=2, C=32, H=20, W=20, OC=64, k=(3, 3), p=(1, 1), pool=(2, 2), ps=(2, 2)),
     dict(N=2, C=6, H=9, W=8, OC=10, k=(3, 3), p=(0, 0), pool=(3, 2), ps=(2, 1)),
