@@ -2,10 +2,13 @@
 #include "SOFIE/RModelParser_ONNX.hxx"
 
 #include <algorithm>
+#include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <ctime>
 #include <fstream>
 #include <iostream>
+#include <map>
 #include <set>
 #include <sstream>
 #include <stdexcept>
@@ -341,6 +344,136 @@ const std::set<std::string> &Supported()
 
 std::string InputOr(const Node &n, size_t i) { return i < n.inputs.size() ? n.inputs[i] : std::string(); }
 
+
+// ---- QDQ pattern: DequantizeLinear -> Conv / MatMul / Gemm -> [Add] -> [Relu] -> QuantizeLinear ------------
+// A graph exported in the "QDQ" format keeps float operators between DequantizeLinear and QuantizeLinear nodes;
+// the integer operator it stands for is QLinearConv / QLinearMatMul on the quantized tensors (the reference's
+// parser rejects the int8 initializers such a graph holds, RModelParser_ONNX.cxx:560-591). The weight must be
+// an int8 initializer behind its own DequantizeLinear; the bias is an int32 initializer behind a
+// DequantizeLinear, or a float initializer that is quantized here with scale x_scale * w_scale[c].
+struct QdqPlan {
+   bool conv = false;
+   std::string xq, xScale, xZp, wq, wScale, wZp, yScale, yZp, bias, yq;
+   int64_t transB = 0;
+   bool relu = false;
+   std::vector<size_t> skip;       // nodes replaced by the fused operator (besides the anchor)
+   size_t dqx = 0;                 // the activation's DequantizeLinear (dropped when nothing else reads it)
+   std::vector<int32_t> quantizedBias;   // set when the bias was a float initializer
+};
+
+const Tensor *FindInit(const Graph &g, const std::string &name)
+{
+   for (auto &t : g.initializers)
+      if (t.name == name) return &t;
+   return nullptr;
+}
+
+std::vector<float> FloatsOf(const Tensor &t)
+{
+   size_t length = 1;
+   for (auto d : t.dims) length *= (size_t)d;
+   std::shared_ptr<void> data = TensorData(t, ETensorType::FLOAT, length);
+   const float *p = static_cast<const float *>(data.get());
+   return std::vector<float>(p, p + length);
+}
+
+bool PlanQdq(const Graph &g, size_t idx, const std::map<std::string, size_t> &producer, std::map<std::string, int> &uses,
+             QdqPlan &plan)
+{
+   const Node &n = g.nodes[idx];
+   const bool conv = n.opType == "Conv";
+   if (!conv && n.opType != "MatMul" && n.opType != "Gemm") return false;
+   if (n.inputs.size() < 2 || n.outputs.empty()) return false;
+   if (n.opType == "Gemm" && (n.Float("alpha", 1.0f) != 1.0f || n.Float("beta", 1.0f) != 1.0f || n.Int("transA", 0) != 0))
+      return false;
+   auto dq_of = [&](const std::string &tensor) -> const Node * {
+      auto it = producer.find(tensor);
+      if (it == producer.end()) return nullptr;
+      const Node &d = g.nodes[it->second];
+      return (d.opType == "DequantizeLinear" && d.inputs.size() >= 2) ? &d : nullptr;
+   };
+   const Node *dx = dq_of(n.inputs[0]);
+   const Node *dw = dq_of(n.inputs[1]);
+   if (!dx || !dw) return false;
+   const Tensor *w = FindInit(g, dw->inputs[0]);
+   if (!w || w->dataType != 3 /* INT8 */ || uses[dw->outputs[0]] != 1) return false;
+   if (FindInit(g, dx->inputs[0])) return false;               // a constant activation: nothing to gain
+   if (!FindInit(g, dx->inputs[1]) || !FindInit(g, dw->inputs[1])) return false;
+   {
+      // per-channel weight scales must run along the output channels
+      size_t nscale = 1;
+      for (auto d : FindInit(g, dw->inputs[1])->dims) nscale *= (size_t)d;
+      const int64_t want = conv ? 0 : ((n.opType == "Gemm" && n.Int("transB", 0)) ? 0 : 1);
+      if (nscale > 1 && dw->Int("axis", 1) != want) return false;
+   }
+   plan = QdqPlan();
+   plan.conv = conv;
+   plan.xq = dx->inputs[0];
+   plan.xScale = dx->inputs[1];
+   plan.xZp = InputOr(*dx, 2);
+   plan.wq = dw->inputs[0];
+   plan.wScale = dw->inputs[1];
+   plan.wZp = InputOr(*dw, 2);
+   plan.transB = n.opType == "Gemm" ? n.Int("transB", 0) : 0;
+   plan.dqx = producer.at(n.inputs[0]);
+   plan.skip.push_back(producer.at(n.inputs[1]));
+
+   // the tail: [Add bias] -> [Relu] -> QuantizeLinear, each the only reader of its input
+   std::string biasName = InputOr(n, 2);
+   std::string cur = n.outputs[0];
+   auto only_reader = [&](const std::string &tensor) -> size_t {
+      if (uses[tensor] != 1) return g.nodes.size();
+      for (size_t j = idx + 1; j < g.nodes.size(); ++j)
+         if (std::find(g.nodes[j].inputs.begin(), g.nodes[j].inputs.end(), tensor) != g.nodes[j].inputs.end()) return j;
+      return g.nodes.size();
+   };
+   size_t j = only_reader(cur);
+   if (n.opType == "MatMul" && j < g.nodes.size() && g.nodes[j].opType == "Add" && g.nodes[j].inputs.size() == 2) {
+      const Node &add = g.nodes[j];
+      biasName = add.inputs[0] == cur ? add.inputs[1] : add.inputs[0];
+      plan.skip.push_back(j);
+      cur = add.outputs[0];
+      j = only_reader(cur);
+   }
+   if (j < g.nodes.size() && g.nodes[j].opType == "Relu") {
+      plan.relu = true;
+      plan.skip.push_back(j);
+      cur = g.nodes[j].outputs[0];
+      j = only_reader(cur);
+   }
+   if (j >= g.nodes.size() || g.nodes[j].opType != "QuantizeLinear" || g.nodes[j].inputs.size() < 2) return false;
+   const Node &q = g.nodes[j];
+   if (!FindInit(g, q.inputs[1])) return false;
+   plan.skip.push_back(j);
+   plan.yScale = q.inputs[1];
+   plan.yZp = InputOr(q, 2);
+   plan.yq = q.outputs[0];
+
+   if (!biasName.empty()) {
+      if (const Node *db = dq_of(biasName)) {
+         const Tensor *b = FindInit(g, db->inputs[0]);
+         if (!b || b->dataType != 6 /* INT32 */ || uses[db->outputs[0]] != 1) return false;
+         plan.bias = db->inputs[0];
+         plan.skip.push_back(producer.at(biasName));
+      } else if (const Tensor *bf = FindInit(g, biasName)) {
+         if (bf->dataType != 1 /* FLOAT */) return false;
+         const std::vector<float> b = FloatsOf(*bf);
+         const std::vector<float> sx = FloatsOf(*FindInit(g, plan.xScale));
+         const std::vector<float> sw = FloatsOf(*FindInit(g, plan.wScale));
+         if (sx.size() != 1 || (sw.size() != 1 && sw.size() != b.size())) return false;
+         plan.quantizedBias.resize(b.size());
+         for (size_t c = 0; c < b.size(); ++c) {
+            const float sb = sx[0] * sw[sw.size() == 1 ? 0 : c];
+            plan.quantizedBias[c] = (int32_t)std::nearbyint((double)b[c] / (double)sb);
+         }
+         plan.bias = biasName + "_quantized";
+      } else {
+         return false;
+      }
+   }
+   return true;
+}
+
 }   // namespace
 
 bool RModelParser_ONNX::IsRegisteredOperator(const std::string &name) { return Supported().count(name) != 0; }
@@ -393,14 +526,6 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
       model.AddInputTensorName(in.name);
       if (verbose) std::cout << "input tensor " << in.name << " " << ConvertShapeToString(shape) << "\n";
    }
-   for (auto &t : g.initializers) {
-      const ETensorType type = TypeOfOnnx(t.dataType, t.name);
-      std::vector<size_t> shape;
-      for (auto d : t.dims) shape.push_back((size_t)d);
-      const size_t length = ConvertShapeToLength(shape);
-      model.AddInitializedTensor(t.name, type, shape, TensorData(t, type, length));
-   }
-
    // consumers of every tensor, for the single-consumer condition of the fusions
    std::map<std::string, int> uses;
    for (auto &n : g.nodes)
@@ -408,6 +533,50 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
    for (auto &o : g.outputs) uses[o.name]++;
 
    std::vector<bool> fused(g.nodes.size(), false);
+
+   // QDQ groups: the anchor (Conv / MatMul / Gemm) becomes the integer operator, the nodes around it vanish
+   std::map<std::string, size_t> producer;
+   for (size_t i = 0; i < g.nodes.size(); ++i)
+      for (auto &o : g.nodes[i].outputs) producer[o] = i;
+   std::map<size_t, QdqPlan> plans;
+   {
+      std::map<size_t, int> dqxReaders;
+      for (size_t i = 0; i < g.nodes.size(); ++i) {
+         QdqPlan plan;
+         if (!PlanQdq(g, i, producer, uses, plan)) continue;
+         bool clash = false;
+         for (size_t k : plan.skip) clash = clash || fused[k] || plans.count(k);
+         if (clash) continue;
+         for (size_t k : plan.skip) fused[k] = true;
+         dqxReaders[plan.dqx]++;
+         plans[i] = plan;
+      }
+      for (auto &d : dqxReaders)
+         if (uses[g.nodes[d.first].outputs[0]] == d.second) fused[d.first] = true;
+   }
+   // initializers: those some remaining node or fused operator still names
+   {
+      std::set<std::string> named;
+      for (size_t i = 0; i < g.nodes.size(); ++i) {
+         if (fused[i]) continue;
+         auto it = plans.find(i);
+         if (it == plans.end()) {
+            for (auto &in : g.nodes[i].inputs) named.insert(in);
+         } else {
+            const QdqPlan &q = it->second;
+            for (auto &nm : {q.xScale, q.xZp, q.wq, q.wScale, q.wZp, q.yScale, q.yZp, q.bias}) named.insert(nm);
+         }
+      }
+      for (auto &o : g.outputs) named.insert(o.name);
+      for (auto &t : g.initializers) {
+         if (!plans.empty() && !named.count(t.name)) continue;
+         const ETensorType type = TypeOfOnnx(t.dataType, t.name);
+         std::vector<size_t> shape;
+         for (auto d : t.dims) shape.push_back((size_t)d);
+         const size_t length = ConvertShapeToLength(shape);
+         model.AddInitializedTensor(t.name, type, shape, TensorData(t, type, length));
+      }
+   }
    int order = 0;
    for (size_t idx = 0; idx < g.nodes.size(); ++idx) {
       if (fused[idx]) continue;
@@ -419,7 +588,25 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
                                      std::find(next->inputs.begin(), next->inputs.end(), n.outputs[0]) != next->inputs.end();
       std::unique_ptr<ROperator> op;
       const std::string &t = n.opType;
-      if (t == "Gemm") {
+      auto planned = plans.find(idx);
+      if (planned != plans.end()) {
+         const QdqPlan &q = planned->second;
+         if (!q.quantizedBias.empty()) {
+            std::shared_ptr<void> data(malloc(q.quantizedBias.size() * sizeof(int32_t)), free);
+            std::memcpy(data.get(), q.quantizedBias.data(), q.quantizedBias.size() * sizeof(int32_t));
+            model.AddInitializedTensor(q.bias, ETensorType::INT32, {q.quantizedBias.size()}, data);
+         }
+         if (q.conv)
+            op.reset(new ROperator_QLinearConv(n.String("auto_pad", "NOTSET"), n.Sizes("dilations"), (size_t)n.Int("group", 1),
+                                               n.Sizes("kernel_shape"), n.Sizes("pads"), n.Sizes("strides"), q.xq, q.xScale,
+                                               q.xZp, q.wq, q.wScale, q.wZp, q.yScale, q.yZp, q.bias, q.yq));
+         else
+            op.reset(new ROperator_QLinearMatMul(q.xq, q.xScale, q.xZp, q.wq, q.wScale, q.wZp, q.yScale, q.yZp, q.yq, q.bias,
+                                                 q.transB));
+         if (q.relu && !op->FuseActivation(EActivationType::RELU))
+            throw std::runtime_error("TMVA::SOFIE - cannot fuse the Relu of the quantized group at node " + n.name);
+         if (verbose) std::cout << "\t\tQDQ group -> " << (q.conv ? "QLinearConv " : "QLinearMatMul ") << q.yq << "\n";
+      } else if (t == "Gemm") {
          // Gemm -> Relu with a single consumer: the activation becomes a constructor argument (ParseFuseGemmRelu.cxx)
          std::string out = n.outputs[0];
          EActivationType act = EActivationType::UNDEFINED;

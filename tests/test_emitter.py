@@ -245,6 +245,69 @@ def test_cpp_onnx_front_end_quantized_graph_and_fusions(tmp_path):
     assert res.returncode != 0 and "Operator type Softmax is not yet supported" in res.stderr
 
 
+def test_cpp_onnx_front_end_fuses_qdq_groups(tmp_path):
+    """The same layer written in the QDQ format (DequantizeLinear -> Conv -> QuantizeLinear around float operators,
+    int8 weights and int32 bias behind their own DequantizeLinear) parses into the code of the QLinearConv form;
+    a DequantizeLinear -> Gemm(transB) -> Relu -> QuantizeLinear group with a float bias becomes one int8 GEMM call
+    whose bias is quantized with x_scale * w_scale[n]."""
+    import onnx_write as ow
+    p = models.qdq_conv_params()
+    init = {"sx": np.array(p["sx"], np.float32), "zx": np.array(p["zx"], np.int8), "sy": np.array(p["sy"], np.float32),
+            "zy": np.array(p["zy"], np.int8), "w": p["w"], "sw": p["sw"], "b": p["b"],
+            "sb": (p["sx"] * p["sw"]).astype(np.float32), "zw": np.zeros(64, np.int8)}
+    nodes = [ow.node("QuantizeLinear", ["x", "sx", "zx"], ["xq"]),
+             ow.node("DequantizeLinear", ["xq", "sx", "zx"], ["xf"]),
+             ow.node("DequantizeLinear", ["w", "sw"], ["wf"], axis=0),
+             ow.node("DequantizeLinear", ["b", "sb"], ["bf"], axis=0),
+             ow.node("Conv", ["xf", "wf", "bf"], ["cf"], kernel_shape=[3, 3], pads=[1, 1, 1, 1], strides=[1, 1]),
+             ow.node("QuantizeLinear", ["cf", "sy", "zy"], ["c"]),
+             ow.node("DequantizeLinear", ["c", "sy", "zy"], ["y"])]
+    path = tmp_path / "qdq_conv.onnx"
+    path.write_bytes(ow.model(nodes, init, [("x", 1, p["x"].shape)], [("y", 1, (2, 64, 9, 7))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode == 0, res.stderr
+    sub = tmp_path / "spec"
+    sub.mkdir()
+    hxx, dat, _ = models.qdq_conv_spec().generate(str(sub))
+    assert _body(str(tmp_path / "qdq_conv.hxx")) == _body(hxx)
+    assert open(str(tmp_path / "qdq_conv.dat")).read() == open(dat).read()
+
+    r = np.random.default_rng(11)
+    M, K, N = 4, 32, 16
+    w = r.integers(-127, 128, (N, K)).astype(np.int8)
+    sw = r.uniform(0.01, 0.02, N).astype(np.float32)
+    sa = np.float32(0.05)
+    bf = r.uniform(-3, 3, N).astype(np.float32)
+    init = {"sa": np.array(sa, np.float32), "za": np.array(-5, np.int8), "w": w, "sw": sw, "bf": bf,
+            "sy": np.array(0.1, np.float32), "zy": np.array(-128, np.int8)}
+    nodes = [ow.node("DequantizeLinear", ["a", "sa", "za"], ["af"]),
+             ow.node("DequantizeLinear", ["w", "sw"], ["wf"], axis=0),
+             ow.node("Gemm", ["af", "wf", "bf"], ["g"], transB=1),
+             ow.node("Relu", ["g"], ["r"]),
+             ow.node("QuantizeLinear", ["r", "sy", "zy"], ["y"])]
+    path = tmp_path / "qdq_fc.onnx"
+    path.write_bytes(ow.model(nodes, init, [("a", 3, (M, K))], [("y", 3, (M, N))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode == 0, res.stderr
+    code = open(str(tmp_path / "qdq_fc.hxx")).read()
+    assert code.count("sofie_hip_qgemm_s8(") == 1 and "SOFIE_ACT_RELU" in code
+    assert "dequantize" not in code and "sofie_hip_gemm_f32" not in code
+    dat = open(str(tmp_path / "qdq_fc.dat")).read().split("\n")
+    # the folded bias: rne(bf / (sa * sw)) - za * sum_k w[n, k]
+    sb = (sa * sw).astype(np.float32)
+    want = np.rint(bf.astype(np.float64) / sb.astype(np.float64)).astype(np.int64) + 5 * w.astype(np.int64).sum(axis=1)
+    line = [i for i, l in enumerate(dat) if l.startswith("tensor_y_qbias ")][0]
+    got = np.array(dat[line + 1].split(), dtype=np.int64)
+    assert np.array_equal(got, want)
+
+    # a per-channel scale along the wrong axis is not a QDQ group: the float operators stay
+    nodes[1] = ow.node("DequantizeLinear", ["w", "sw"], ["wf"], axis=1)
+    path = tmp_path / "qdq_bad_axis.onnx"
+    path.write_bytes(ow.model(nodes, init, [("a", 3, (M, K))], [("y", 3, (M, N))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode != 0 or "sofie_hip_qgemm_s8(" not in open(str(tmp_path / "qdq_bad_axis.hxx")).read()
+
+
 def test_every_prebuilt_session_compiles():
     """tests/build_generated.py output (made by build()): header, weights and runner of each network."""
     import build_generated
