@@ -185,6 +185,18 @@ def extras(ctx, torch, L, ops, rng):
         5, 1)
     fl = 2.0 * 256 * 128 * 3136 * 576
     ex["conv2d_f32_b256_64to128_56x56"] = {"ms": ms, "tflops": fl / ms / 1e9, "frac_peak": fl / ms / 1e9 / PEAK_FP32_TFLOPS}
+    del x, w, y
+    # fp32 transposed conv (an upsampling layer): batch 64, 128 -> 64 channels, 28x28 -> 56x56, 4x4, stride 2, pad 1
+    x = torch.rand(64, 128, 28, 28, device=ctx.device)
+    w = torch.randn(128, 64, 4, 4, device=ctx.device) * 0.05
+    b = torch.randn(64, device=ctx.device) * 0.1
+    y = ctx.empty((64, 64, 56, 56), torch.float32)
+    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_conv_transpose2d_f32(
+        ctx.h, ctx.ptr(x), ctx.ptr(w), ctx.ptr(b), ctx.ptr(y), 64, 128, 28, 28, 64, 4, 4, 1, 1, 2, 2, 1, 1, 1, 56, 56, 0)),
+        5, 1)
+    fl = 2.0 * 64 * 128 * 64 * 16 * 784      # every input pixel meets every kernel tap once
+    ex["conv_transpose2d_f32_b64_128to64_28to56"] = {"ms": ms, "tflops": fl / ms / 1e9,
+                                                      "frac_peak": fl / ms / 1e9 / PEAK_FP32_TFLOPS}
     # fp32 MLP batch 256: 64 -> 128 -> 64 -> 8 (three Gemm launches, ReLU fused)
     X = torch.randn(256, 64, device=ctx.device)
     Ws = [torch.randn(64, 128, device=ctx.device), torch.randn(128, 64, device=ctx.device),

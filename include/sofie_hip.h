@@ -117,6 +117,21 @@ int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
                          int KH, int KW, int pad_h, int pad_w, int stride_h, int stride_w,
                          int dil_h, int dil_w, int groups, int act);
 
+/* NCHW 2-D transposed convolution (ONNX ConvTranspose), optional ReLU.
+ * x [N,C,H,W], w [C, OC/groups, KH, KW] (the ONNX layout), bias [OC] or NULL, y [N,OC,OH,OW]:
+ *   y[n,oc,oy,ox] = bias[oc] + sum over (ic,kh,kw) with oy + pad_h - kh*dil_h = stride_h*iy (same for x)
+ *                   of x[n,ic,iy,ix] * w[ic,oc',kh,kw].
+ * OH and OW are given by the caller: stride*(in-1) + dil*(K-1) + 1 + output_padding - pad_begin - pad_end
+ * (ROperator_ConvTranspose.icc:83-90); pad_h / pad_w are the begin pads. Replaces the emitted kernel
+ * re-layout, BLAS::sgemm_ into the column matrix, UTILITY::col2im and BLAS::saxpy_ of
+ * ROperator_ConvTranspose<float>::Generate (ROperator_ConvTranspose.icc:232-474) with the implicit-GEMM
+ * convolution kernel run over the zero-interleaved input with the kernel reversed; no column matrix exists. */
+int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
+                                   const float *bias, float *y, int N, int C, int H, int W,
+                                   int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,
+                                   int stride_w, int dil_h, int dil_w, int groups, int OH, int OW,
+                                   int act);
+
 /* y[i] = x[i] > 0 ? x[i] : 0. Replaces the loop of ROperator_Relu.hxx:62-64. */
 int sofie_hip_relu_f32(sofie_hip_ctx *ctx, const float *x, float *y, size_t len);
 

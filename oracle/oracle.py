@@ -59,6 +59,7 @@ _gemm_f32 = _sig("or_gemm_f32", C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.
 _relu = _sig("or_relu_f32", None, [_f32p, _f32p, C.c_size_t])
 _im2col = _sig("or_im2col", None, [_f32p] + [C.c_int] * 11 + [_f32p])
 _conv2d = _sig("or_conv2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 15)
+_convt = _sig("or_conv_transpose2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 17)
 _maxpool = _sig("or_maxpool2d_f32", None, [_f32p, _f32p] + [C.c_int] * 11)
 _maxpool_s8 = _sig("or_maxpool2d_s8", None, [_i8p, _i8p] + [C.c_int] * 11)
 _requant_one = _sig("or_requant_one", C.c_int8, [C.c_int32, C.c_float, C.c_int, C.c_int])
@@ -140,6 +141,25 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
                  strides[0], strides[1], dilations[0], dilations[1], groups, int(relu))
     if rc:
         raise RuntimeError("or_conv2d_f32 failed: %d" % rc)
+    return y
+
+
+def conv_transpose2d_f32(x, w, bias=None, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), groups=1,
+                         output_padding=(0, 0), relu=False):
+    """ONNX ConvTranspose (ROperator_ConvTranspose.icc:232-474): x [N,C,H,W], w [C, OC/groups, kh, kw],
+    pads = (top, left, bottom, right); begin pads position the result, end pads only shorten it."""
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    N, Cc, H, W = x.shape
+    _, ocg, kh, kw = w.shape
+    OC = ocg * groups
+    OH = strides[0] * (H - 1) + dilations[0] * (kh - 1) + 1 + output_padding[0] - pads[0] - pads[2]
+    OW = strides[1] * (W - 1) + dilations[1] * (kw - 1) + 1 + output_padding[1] - pads[1] - pads[3]
+    y = np.empty((N, OC, OH, OW), np.float32)
+    rc = _convt(x, w, _opt(bias, np.float32), y, N, Cc, H, W, OC, kh, kw, pads[0], pads[1], strides[0], strides[1],
+                dilations[0], dilations[1], groups, OH, OW, int(relu))
+    if rc:
+        raise RuntimeError("or_conv_transpose2d_f32 failed: %d" % rc)
     return y
 
 

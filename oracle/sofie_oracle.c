@@ -13,6 +13,8 @@
  *                                reference's tests, numpy float64 closed form
  *   or_im2col, or_conv2d_f32     pinned: ConvWith* known answers (ONNX spec examples),
  *                                torch.nn.functional.conv2d on CPU, brute-force 7-loop
+ *   or_conv_transpose2d_f32      pinned: ConvTranspose1d/2d/Bias2d/Bias2dBatched known
+ *                                answers, torch.nn.functional.conv_transpose2d on CPU
  *   or_relu, or_maxpool2d        pinned: MaxPool2d known answer, torch CPU
  *   or_broadcast_rows            pinned through the Linear_* answers (bias broadcast)
  *   or_qgemm_s8, or_qconv2d_s8,
@@ -203,6 +205,65 @@ int or_conv2d_f32(const float *x, const float *w, const float *bias, float *y,
         const size_t len = (size_t)N * OC * m;
         for (size_t i = 0; i < len; ++i) y[i] = (y[i] > 0) ? y[i] : 0;
     }
+    free(col);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* 2-D transposed convolution as emitted by ROperator_ConvTranspose<float>:: */
+/* Generate (ROperator_ConvTranspose.icc:232-474), NCHW, w [C, OC/g, kh, kw]:*/
+/*   - per image (and group): sgemm_('N','T', m=H*W, n=OC/g*kh*kw, k=C/g, 1, */
+/*     x, m, W, n, 0, xcol, m) (:364-372): xcol[(oc,r,s), pixel] =           */
+/*     sum_ic x[ic, pixel] * w[ic, oc, r, s], fp32 accumulation in ic order  */
+/*   - UTILITY::col2im (SOFIE_common.hxx:575-620): the output image starts   */
+/*     at zero and every xcol entry is added at output position              */
+/*     (ih*sh - ph + r*dh, iw*sw - pw + s*dw) when that lies inside, in the  */
+/*     order (oc, r, s, ih, iw)                                              */
+/*   - saxpy of the bias broadcast over [N,OC,OH,OW] (:463-471)              */
+/* OH, OW are the caller's (stride*(in-1) + dil*(k-1) + 1 + output_padding   */
+/* - pads, :83-90). Groups follow the ONNX definition (group g reads input   */
+/* channels [g*C/g, (g+1)*C/g) and its own slice of w); the reference's      */
+/* group branch multiplies every group with the first slice of w (:417-423,  */
+/* "probably need an offset"), which no fixture uses.                        */
+/* Pinned by: ConvTranspose1d / 2d / Bias2d / Bias2dBatched known answers of */
+/* the reference's tests, torch.nn.functional.conv_transpose2d on CPU.       */
+/* ------------------------------------------------------------------------- */
+int or_conv_transpose2d_f32(const float *x, const float *w, const float *bias, float *y,
+                            int N, int C, int H, int W, int OC, int kh, int kw, int ph, int pw,
+                            int sh, int sw, int dh, int dw, int groups, int OH, int OW, int relu)
+{
+    if (groups < 1 || C % groups || OC % groups || OH <= 0 || OW <= 0) return -1;
+    const int icg = C / groups, ocg = OC / groups;
+    const int m = H * W, n = ocg * kh * kw;
+    float *col = (float *)malloc((size_t)n * m * sizeof(float));
+    if (!col) return -2;
+    const size_t out_plane = (size_t)OH * OW;
+    for (size_t i = 0; i < (size_t)N * OC * out_plane; ++i) y[i] = 0.0f;
+    for (int b = 0; b < N; ++b) {
+        for (int g = 0; g < groups; ++g) {
+            const float *xg = x + ((size_t)b * C + (size_t)g * icg) * m;
+            const float *wg = w + (size_t)g * icg * n;
+            or_sgemm('n', 't', m, n, icg, 1.0f, xg, m, wg, n, 0.0f, col, m);
+            float *yg = y + ((size_t)b * OC + (size_t)g * ocg) * out_plane;
+            const float *c = col;
+            for (int oc = 0; oc < ocg; ++oc)
+                for (int r = 0; r < kh; ++r)
+                    for (int s = 0; s < kw; ++s)
+                        for (int ih = 0; ih < H; ++ih) {
+                            const int oh = ih * sh - ph + r * dh;
+                            for (int iw = 0; iw < W; ++iw, ++c) {
+                                const int ow = iw * sw - pw + s * dw;
+                                if (oh >= 0 && oh < OH && ow >= 0 && ow < OW)
+                                    yg[(size_t)oc * out_plane + (size_t)oh * OW + ow] += *c;
+                            }
+                        }
+        }
+    }
+    const size_t len = (size_t)N * OC * out_plane;
+    if (bias)
+        for (size_t i = 0; i < len; ++i) y[i] += 1.0f * bias[(i / out_plane) % OC];
+    if (relu)
+        for (size_t i = 0; i < len; ++i) y[i] = (y[i] > 0) ? y[i] : 0;
     free(col);
     return 0;
 }

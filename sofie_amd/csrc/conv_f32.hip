@@ -26,8 +26,22 @@ struct ConvArgs {
    int PH, PW;         // staged patch extent
    int rows_out;       // output rows a pixel tile can span
    int relu;
+   // Transposed convolution (uh, uw > 0): the same implicit GEMM over the input seen with uh-1 / uw-1 zeros
+   // between its rows / columns, unit output stride, and the weights w [C, OC/groups, KH, KW] read with both
+   // kernel axes reversed. ph / pw are then dil*(K-1) - pad of the transposed convolution (may be negative).
+   int transposed, uh, uw;
    FastDiv dPW, dPH, dKC;   // divisions by the patch extents and the K-chunk length in the staging loops
+   FastDiv dUH, dUW;
 };
+
+// Input row / column behind position `up` of the zero-interleaved input, or -1 where a zero sits.
+__device__ __forceinline__ int source_index(int up, int u, FastDiv d)
+{
+   if (up < 0) return -1;
+   if (u == 1) return up;
+   const int q = fdiv(up, d);
+   return q * u == up ? q : -1;
+}
 
 template <int TI, int TJ>
 __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
@@ -85,7 +99,11 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       for (int e = tid; e < patch_len; e += 256) {
          const int t = fdiv(e, g.dPW), c = e - t * g.PW;
          const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
-         const int ih = ih0 + r, iw = iw0 + c;
+         int ih = ih0 + r, iw = iw0 + c;
+         if (g.transposed) {
+            ih = source_index(ih, g.uh, g.dUH);
+            iw = source_index(iw, g.uw, g.dUW);
+         }
          float v = 0.0f;
          if (icl < icn && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
             v = xg[((size_t)(ic0 + icl) * g.H + ih) * g.W + iw];
@@ -94,7 +112,14 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       for (int e = tid; e < g.KC * BOC; e += 256) {
          const int ocl = fdiv(e, g.dKC), k = e - ocl * g.KC;
          float v = 0.0f;
-         if (k < kc && oc0 + ocl < g.ocg) v = wg[(size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k];
+         if (k < kc && oc0 + ocl < g.ocg) {
+            if (g.transposed) {
+               const int icl = k / KHW, t = k - icl * KHW;
+               v = g.w[(((size_t)grp * g.icg + ic0 + icl) * g.ocg + oc0 + ocl) * KHW + (KHW - 1 - t)];
+            } else {
+               v = wg[(size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k];
+            }
+         }
          sW[k * LDW + ocl] = v;
       }
       __syncthreads();
@@ -148,15 +173,20 @@ __global__ void k_conv2d_f32_simple(ConvArgs g)
    const int n = (int)(r / g.OC);
    const int grp = oc / g.ocg;
    float acc = 0.0f;
+   const int KHW = g.KH * g.KW;
    for (int ic = 0; ic < g.icg; ++ic)
       for (int kh = 0; kh < g.KH; ++kh) {
-         const int ih = oh * g.sh - g.ph + kh * g.dh;
+         int ih = oh * g.sh - g.ph + kh * g.dh;
+         if (g.transposed) ih = source_index(ih, g.uh, g.dUH);
          if (ih < 0 || ih >= g.H) continue;
          for (int kw = 0; kw < g.KW; ++kw) {
-            const int iw = ow * g.sw - g.pw + kw * g.dw;
+            int iw = ow * g.sw - g.pw + kw * g.dw;
+            if (g.transposed) iw = source_index(iw, g.uw, g.dUW);
             if (iw < 0 || iw >= g.W) continue;
-            acc = __fadd_rn(acc, __fmul_rn(g.x[(((size_t)n * g.C + grp * g.icg + ic) * g.H + ih) * g.W + iw],
-                                           g.w[(((size_t)oc * g.icg + ic) * g.KH + kh) * g.KW + kw]));
+            const float wv = g.transposed
+                                ? g.w[(((size_t)grp * g.icg + ic) * g.ocg + (oc - grp * g.ocg)) * KHW + (KHW - 1 - (kh * g.KW + kw))]
+                                : g.w[(((size_t)oc * g.icg + ic) * g.KH + kh) * g.KW + kw];
+            acc = __fadd_rn(acc, __fmul_rn(g.x[(((size_t)n * g.C + grp * g.icg + ic) * g.H + ih) * g.W + iw], wv));
          }
       }
    if (g.bias) acc = __fadd_rn(acc, g.bias[oc]);
@@ -205,6 +235,20 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    return check_launch(ctx, "k_conv2d_f32");
 }
 
+int run_conv(sofie_hip_ctx *ctx, ConvArgs &g)
+{
+   g.dUH = make_fastdiv((unsigned)(g.uh > 0 ? g.uh : 1));
+   g.dUW = make_fastdiv((unsigned)(g.uw > 0 ? g.uw : 1));
+   bool done = false;
+   int rc;
+   if (g.ocg > 64) rc = launch<2, 2>(ctx, g, &done);
+   else rc = launch<1, 2>(ctx, g, &done);
+   if (rc || done) return rc;
+   const size_t total = (size_t)g.N * g.OC * g.OH * g.OW;
+   hipLaunchKernelGGL(k_conv2d_f32_simple, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, g);
+   return check_launch(ctx, "k_conv2d_f32_simple");
+}
+
 }  // namespace
 
 extern "C" int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w, const float *bias, float *y,
@@ -230,13 +274,36 @@ extern "C" int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const fl
    g.icg = C / groups;
    g.ocg = OC / groups;
    g.relu = act == SOFIE_ACT_RELU;
-   bool done = false;
-   int rc;
-   if (g.ocg > 64) rc = launch<2, 2>(ctx, g, &done);
-   else if (g.ocg > 32) rc = launch<1, 2>(ctx, g, &done);
-   else rc = launch<1, 2>(ctx, g, &done);
-   if (rc || done) return rc;
-   const size_t total = (size_t)N * OC * g.OH * g.OW;
-   hipLaunchKernelGGL(k_conv2d_f32_simple, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, g);
-   return check_launch(ctx, "k_conv2d_f32_simple");
+   return run_conv(ctx, g);
+}
+
+extern "C" int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w, const float *bias,
+                                              float *y, int N, int C, int H, int W, int OC, int KH, int KW, int pad_h,
+                                              int pad_w, int stride_h, int stride_w, int dil_h, int dil_w, int groups,
+                                              int OH, int OW, int act)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, N >= 0 && C > 0 && H > 0 && W > 0 && OC > 0 && KH > 0 && KW > 0, "non-positive dimension");
+   SOFIE_REQUIRE(ctx, pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0,
+                 "bad pads/strides/dilations");
+   SOFIE_REQUIRE(ctx, groups > 0 && C % groups == 0 && OC % groups == 0, "channels not divisible by groups");
+   SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
+   // the output may be shorter than the full extent (end padding) or longer by less than a stride (output padding)
+   const long full_h = (long)stride_h * (H - 1) + (long)dil_h * (KH - 1) + 1 - pad_h;
+   const long full_w = (long)stride_w * (W - 1) + (long)dil_w * (KW - 1) + 1 - pad_w;
+   SOFIE_REQUIRE(ctx, OH > 0 && OW > 0 && OH < full_h + stride_h && OW < full_w + stride_w, "output size does not fit the geometry");
+   if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && w && y, "null operand");
+   ConvArgs g{};
+   g.x = x; g.w = w; g.bias = bias; g.y = y;
+   g.N = N; g.C = C; g.H = H; g.W = W; g.OC = OC; g.KH = KH; g.KW = KW;
+   g.ph = dil_h * (KH - 1) - pad_h;
+   g.pw = dil_w * (KW - 1) - pad_w;
+   g.sh = 1; g.sw = 1; g.dh = dil_h; g.dw = dil_w; g.groups = groups;
+   g.OH = OH; g.OW = OW;
+   g.icg = C / groups;
+   g.ocg = OC / groups;
+   g.relu = act == SOFIE_ACT_RELU;
+   g.transposed = 1; g.uh = stride_h; g.uw = stride_w;
+   return run_conv(ctx, g);
 }

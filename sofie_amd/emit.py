@@ -73,6 +73,12 @@ class ModelSpec:
         self.lines.append("op Conv %s %d %s %s %s %s %s %s %s %s" % (auto_pad, group, _lst(kernel), _lst(pads),
                                                                     _lst(strides), _lst(dilations), x, w, b or "-", y))
 
+    def conv_transpose(self, x, w, b, y, kernel=(), pads=(), strides=(), dilations=(), group=0, output_padding=(),
+                       output_shape=(), auto_pad="NOTSET"):
+        self.lines.append("op ConvTranspose %s %d %s %s %s %s %s %s %s %s %s %s" % (
+            auto_pad, group, _lst(kernel), _lst(pads), _lst(strides), _lst(dilations), _lst(output_padding),
+            _lst(output_shape), x, w, b or "-", y))
+
     def relu(self, x, y):
         self.lines.append("op Relu %s %s" % (x, y))
 
@@ -173,6 +179,10 @@ def spec_from_onnx(name, graph):
             spec.conv(ins[0], ins[1], ins[2] if len(ins) > 2 else None, out, a.get("kernel_shape", ()),
                       a.get("pads", ()), a.get("strides", ()), a.get("dilations", ()), a.get("group", 1),
                       a.get("auto_pad", "NOTSET"))
+        elif op == "ConvTranspose":
+            spec.conv_transpose(ins[0], ins[1], ins[2] if len(ins) > 2 else None, out, a.get("kernel_shape", ()),
+                                a.get("pads", ()), a.get("strides", ()), a.get("dilations", ()), a.get("group", 0),
+                                a.get("output_padding", ()), a.get("output_shape", ()), a.get("auto_pad", "NOTSET"))
         elif op == "MaxPool":
             spec.maxpool(ins[0], out, a["kernel_shape"], a.get("pads", (0, 0, 0, 0)), a.get("strides", (1, 1)))
         elif op == "Flatten":

@@ -12,6 +12,7 @@
 //   output NAME
 //   op Gemm ALPHA BETA TRANSA TRANSB A B C Y RELU
 //   op Conv AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. X W B Y
+//   op ConvTranspose AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. nop op.. nos os.. X W B Y
 //   op Relu X Y
 //   op MaxPool nk k.. np p.. ns s.. X Y
 //   op Flatten AXIS X Y
@@ -109,6 +110,13 @@ int main(int argc, char **argv)
                in >> x >> w >> b >> y;
                if (b == "-") r.reset(new ROperator_Conv<float>(autopad, d, group, k, p, s, x, w, y));
                else r.reset(new ROperator_Conv<float>(autopad, d, group, k, p, s, x, w, b, y));
+            } else if (op == "ConvTranspose") {
+               std::string autopad, x, w, b, y;
+               size_t group;
+               in >> autopad >> group;
+               auto k = List(in), p = List(in), s = List(in), d = List(in), op_ = List(in), os = List(in);
+               in >> x >> w >> b >> y;
+               r.reset(new ROperator_ConvTranspose<float>(autopad, d, group, k, op_, os, p, s, x, w, b == "-" ? std::string() : b, y));
             } else if (op == "Relu") {
                std::string x, y;
                in >> x >> y;

@@ -337,7 +337,7 @@ std::shared_ptr<void> TensorData(const Tensor &t, ETensorType type, size_t lengt
 
 const std::set<std::string> &Supported()
 {
-   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "Conv", "Relu", "MaxPool", "Flatten", "Reshape",
+   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "Conv", "ConvTranspose", "Relu", "MaxPool", "Flatten", "Reshape",
                                              "QuantizeLinear", "DequantizeLinear", "QLinearMatMul", "QLinearConv"};
    return ops;
 }
@@ -643,6 +643,14 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
             op.reset(new ROperator_Conv<float>(autopad, n.Sizes("dilations"), group, n.Sizes("kernel_shape"), n.Sizes("pads"),
                                                n.Sizes("strides"), n.inputs[0], n.inputs[1], n.inputs[2], n.outputs[0]));
          else throw std::runtime_error("TMVA::SOFIE - Conv node " + n.name + " needs 2 or 3 inputs");
+      } else if (t == "ConvTranspose") {
+         // attributes as read by ParseConvTranspose.cxx: group defaults to 0 (= 1 in the operator)
+         if (n.inputs.size() != 2 && n.inputs.size() != 3)
+            throw std::runtime_error("TMVA::SOFIE - ConvTranspose node " + n.name + " needs 2 or 3 inputs");
+         op.reset(new ROperator_ConvTranspose<float>(n.String("auto_pad", "NOTSET"), n.Sizes("dilations"), (size_t)n.Int("group", 0),
+                                                     n.Sizes("kernel_shape"), n.Sizes("output_padding"), n.Sizes("output_shape"),
+                                                     n.Sizes("pads"), n.Sizes("strides"), n.inputs[0], n.inputs[1], InputOr(n, 2),
+                                                     n.outputs[0]));
       } else if (t == "Relu") {
          op.reset(new ROperator_Relu<float>(n.inputs.at(0), n.outputs[0]));
       } else if (t == "MaxPool") {

@@ -141,6 +141,24 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
     return _ret(y, x)
 
 
+def conv_transpose2d_f32(x, w, bias=None, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), groups=1,
+                         output_padding=(0, 0), relu=False, ctx=None):
+    """ONNX ConvTranspose, NCHW; w [C, OC/groups, KH, KW]; pads = (top, left, bottom, right)."""
+    ctx = ctx or default_context()
+    xd, wd, bd = ctx.dev(x, torch.float32), ctx.dev(w, torch.float32), ctx.dev(bias, torch.float32)
+    N, Cc, H, W = xd.shape
+    _, ocg, kh, kw = wd.shape
+    OC = ocg * groups
+    OH = strides[0] * (H - 1) + dilations[0] * (kh - 1) + 1 + output_padding[0] - pads[0] - pads[2]
+    OW = strides[1] * (W - 1) + dilations[1] * (kw - 1) + 1 + output_padding[1] - pads[1] - pads[3]
+    y = ctx.empty((N, OC, OH, OW), torch.float32)
+    ctx.check(ctx.lib.sofie_hip_conv_transpose2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, H,
+                                                     W, OC, kh, kw, pads[0], pads[1], strides[0], strides[1],
+                                                     dilations[0], dilations[1], groups, OH, OW,
+                                                     L.ACT_RELU if relu else L.ACT_NONE))
+    return _ret(y, x)
+
+
 def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0), layout=L.LAYOUT_NCHW, ctx=None):
     """pads = (top, left, bottom, right). int8 tensors may be NHWC (layout flag); fp32 is NCHW."""
     ctx = ctx or default_context()

@@ -1,5 +1,5 @@
 """Collect the known-answer fixtures that the reference's own tests hold for the
-Gemm / Conv / MaxPool path into tests/golden/.
+Gemm / Conv / ConvTranspose / MaxPool path into tests/golden/.
 
 Run in the authoring container only (it reads /root/reference, which does not exist
 on the GPU box):   python tests/golden/make_fixtures.py
@@ -11,7 +11,7 @@ What is written:
                                      <name>.ref.hxx headers (numbers only) together with
                                      the input each test feeds (ones / iota / literal list,
                                      from TestCustomModelsFromONNX.cxx:330-349,372-391,
-                                     693-712,860-967,1023-1052)
+                                     693-712,860-967,1023-1052,2047-2152)
 """
 import json
 import os
@@ -33,6 +33,10 @@ CASES = {
     "ConvWithStridesNoPadding": ("iota", [1, 1, 7, 5], "all_ones"),
     "ConvWithAsymmetricPadding": ("iota", [1, 1, 7, 5], "all_ones"),
     "MaxPool2d": ("literal", [1, 1, 5, 10], "output"),
+    "ConvTranspose1d": ("iota", [1, 1, 3], "output"),
+    "ConvTranspose2d": ("iota", [1, 1, 3, 3], "output"),
+    "ConvTransposeBias2d": ("iota", [1, 1, 3, 3], "output"),
+    "ConvTransposeBias2dBatched": ("iota", [2, 1, 3, 3], "output"),
 }
 
 # Input of the reference's MaxPool2d test (TestCustomModelsFromONNX.cxx:1027-1038).

@@ -1,6 +1,6 @@
-"""Replay a decoded ONNX graph (Gemm / Relu / Conv / MaxPool / Flatten) through a backend.
+"""Replay a decoded ONNX graph (Gemm / Relu / Conv / ConvTranspose / MaxPool / Flatten) through a backend.
 
-A backend is any object with the methods gemm_f32, relu_f32, conv2d_f32 and maxpool2d
+A backend is any object with the methods gemm_f32, relu_f32, conv2d_f32, conv_transpose2d_f32 and maxpool2d
 taking and returning numpy arrays: the CPU oracle module, or the HIP library wrapper.
 The attribute handling restates what the reference's operators do at Initialize time.
 """
@@ -60,6 +60,33 @@ def run_graph(graph, feeds, backend):
                                    strides=tuple(a.get("strides", [1, 1])),
                                    dilations=tuple(a.get("dilations", [1, 1])),
                                    groups=a.get("group", 1))
+        elif op == "ConvTranspose":
+            # ROperator_ConvTranspose.icc:14-103: strides / dilations default to 1, pads and output_padding to 0;
+            # :318-346: begin/end pads that differ are averaged for the scatter while the output keeps the size
+            # the shape rule gave it. A 1-D operator runs as a 2-D one with a height of one.
+            x, w = env[ins[0]], env[ins[1]]
+            dim = x.ndim - 2
+            strides = list(a.get("strides", [1] * dim))
+            dil = list(a.get("dilations", [1] * dim))
+            pads = list(a.get("pads", [0] * (2 * dim)))
+            opad = list(a.get("output_padding", [0] * dim))
+            out = [strides[i] * (x.shape[2 + i] - 1) + dil[i] * (w.shape[2 + i] - 1) + 1 + opad[i] - pads[i] - pads[dim + i]
+                   for i in range(dim)]
+            begin = [pads[i] if pads[i] == pads[dim + i] else (pads[i] + pads[dim + i]) // 2 for i in range(dim)]
+            if dim == 1:
+                x, w = x[:, :, None, :], w[:, :, None, :]
+                strides, dil, begin, out = [1] + strides, [1] + dil, [0] + begin, [1] + out
+            # hand the backend pads whose end part reproduces the output size of the shape rule
+            full = [strides[i] * (x.shape[2 + i] - 1) + dil[i] * (w.shape[2 + i] - 1) + 1 for i in range(2)]
+            end = [full[i] - begin[i] - out[i] for i in range(2)]
+            extra = [max(0, -e) for e in end]
+            end = [max(0, e) for e in end]
+            bias = env[ins[2]] if len(ins) > 2 else None
+            y = backend.conv_transpose2d_f32(x, w, bias, pads=(begin[0], begin[1], end[0], end[1]), strides=tuple(strides),
+                                             dilations=tuple(dil), groups=max(1, a.get("group", 1)),
+                                             output_padding=tuple(extra))
+            if dim == 1:
+                y = y[:, :, 0, :]
         elif op == "MaxPool":
             y = backend.maxpool2d(env[ins[0]], tuple(a["kernel_shape"]),
                                   tuple(a.get("strides", [1, 1])),

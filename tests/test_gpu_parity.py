@@ -62,6 +62,49 @@ def test_reference_known_answers_through_hip(ops, name):
         assert np.array_equal(y, yo)
 
 
+# --------------------------------------------------------------------------- fp32 transposed convolution
+@pytest.mark.parametrize("cfg", [
+    dict(N=2, C=4, H=5, W=6, OC=6, k=(3, 3), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(0, 0)),
+    dict(N=1, C=6, H=4, W=4, OC=4, k=(2, 3), s=(3, 2), p=(0, 1, 0, 1), d=(2, 1), g=2, op=(1, 1)),
+    dict(N=2, C=3, H=7, W=5, OC=5, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(1, 0)),
+    dict(N=3, C=64, H=14, W=14, OC=96, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(0, 0)),   # 128-channel tile
+    dict(N=2, C=32, H=9, W=11, OC=32, k=(3, 3), s=(1, 1), p=(1, 1, 1, 1), d=(1, 1), g=4, op=(0, 0)),    # stride 1, groups
+    dict(N=1, C=8, H=6, W=6, OC=8, k=(3, 3), s=(2, 2), p=(2, 2, 2, 2), d=(1, 1), g=1, op=(1, 1)),       # pad = kernel - 1
+    dict(N=1, C=4, H=5, W=5, OC=4, k=(2, 2), s=(1, 1), p=(2, 2, 2, 2), d=(1, 1), g=1, op=(0, 0)),       # pad beyond the kernel
+    dict(N=1, C=2, H=3, W=40, OC=3, k=(1, 9), s=(1, 4), p=(0, 2, 0, 2), d=(1, 1), g=1, op=(0, 3)),
+    dict(N=1, C=2, H=2, W=2, OC=2, k=(31, 31), s=(1, 1), p=(0, 0, 0, 0), d=(1, 1), g=1, op=(0, 0)),     # large kernel
+])
+def test_conv_transpose2d_f32(ops, cfg):
+    """ConvTranspose through the implicit-GEMM kernel over the zero-interleaved input against the oracle's
+    GEMM + col2im restatement of the reference: strides, dilations, groups, begin/end pads (also larger than
+    the kernel reach), output padding, bias and ReLU. Tolerance 1e-5 relative (accumulation order differs)."""
+    r = rng(40 + cfg["C"] + cfg["H"])
+    x = r.standard_normal((cfg["N"], cfg["C"], cfg["H"], cfg["W"])).astype(np.float32)
+    w = (r.standard_normal((cfg["C"], cfg["OC"] // cfg["g"]) + cfg["k"]) * 0.2).astype(np.float32)
+    b = r.standard_normal(cfg["OC"]).astype(np.float32)
+    for bias, relu in ((b, False), (None, True)):
+        y = ops.conv_transpose2d_f32(x, w, bias, cfg["p"], cfg["s"], cfg["d"], cfg["g"], cfg["op"], relu)
+        ref = oracle.conv_transpose2d_f32(x, w, bias, cfg["p"], cfg["s"], cfg["d"], cfg["g"], cfg["op"], relu)
+        assert y.shape == ref.shape
+        assert rel_err(y, ref) <= FP32_TOL
+
+
+def test_conv_transpose2d_f32_is_the_adjoint_of_conv2d(ops):
+    """<conv(x, w), y> = <x, conv_transpose(y, w)> for matching geometry, at a size the oracle would take long for."""
+    r = rng(41)
+    N, C, H, W, OC = 4, 48, 28, 28, 64
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((OC, C, 4, 4)) * 0.1).astype(np.float32)
+    cy = ops.conv2d_f32(x, w, None, (1, 1), (2, 2))
+    y = r.standard_normal(cy.shape).astype(np.float32)
+    # conv weights [OC, C, kh, kw] are ConvTranspose weights for an input with OC channels and C outputs
+    ty = ops.conv_transpose2d_f32(y, w, None, (1, 1, 1, 1), (2, 2))
+    assert ty.shape == x.shape
+    lhs = float(np.sum(cy.astype(np.float64) * y))
+    rhs = float(np.sum(x.astype(np.float64) * ty))
+    assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), abs(rhs), 1.0) * 10
+
+
 # --------------------------------------------------------------------------- fp32 gemm
 @pytest.mark.parametrize("M,N,K,tA,tB,alpha,beta,relu", [
     (256, 128, 64, 0, 0, 1.0, 1.0, True),      # MLP layer 1 of the fp32 configuration
