@@ -132,6 +132,15 @@ int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x, const flo
                                    int stride_w, int dil_h, int dil_w, int groups, int OH, int OW,
                                    int act);
 
+/* Inference BatchNormalization on [N, C, plane] (plane = H*W, or 1 for a [N,C] tensor):
+ * y = (x - mean[c]) * scale[c] + bias[c], optional ReLU, where scale[c] already holds
+ * gamma[c] / sqrt(var[c] + epsilon) (the emitter folds it, as the reference's Initialize does,
+ * ROperator_BatchNormalization.hxx:163-167). Replaces the emitted BLAS::scopy_, BLAS::saxpy_(-mean), the
+ * multiply loop, BLAS::saxpy_(+bias) and the ReLU loop of ROperator_BatchNormalization<float>::Generate
+ * (:196-226), and the four [N,C,H,W]-sized broadcast tensors they read, with one pass over x. */
+int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, const float *x, const float *scale, const float *mean,
+                            const float *bias, float *y, int N, int C, int plane, int act);
+
 /* y[i] = x[i] > 0 ? x[i] : 0. Replaces the loop of ROperator_Relu.hxx:62-64. */
 int sofie_hip_relu_f32(sofie_hip_ctx *ctx, const float *x, float *y, size_t len);
 

@@ -60,6 +60,7 @@ _relu = _sig("or_relu_f32", None, [_f32p, _f32p, C.c_size_t])
 _im2col = _sig("or_im2col", None, [_f32p] + [C.c_int] * 11 + [_f32p])
 _conv2d = _sig("or_conv2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 15)
 _convt = _sig("or_conv_transpose2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 17)
+_bn = _sig("or_batchnorm_f32", None, [_f32p] * 5 + [C.c_float, _f32p] + [C.c_int] * 4)
 _maxpool = _sig("or_maxpool2d_f32", None, [_f32p, _f32p] + [C.c_int] * 11)
 _maxpool_s8 = _sig("or_maxpool2d_s8", None, [_i8p, _i8p] + [C.c_int] * 11)
 _requant_one = _sig("or_requant_one", C.c_int8, [C.c_int32, C.c_float, C.c_int, C.c_int])
@@ -160,6 +161,17 @@ def conv_transpose2d_f32(x, w, bias=None, pads=(0, 0, 0, 0), strides=(1, 1), dil
                 dilations[0], dilations[1], groups, OH, OW, int(relu))
     if rc:
         raise RuntimeError("or_conv_transpose2d_f32 failed: %d" % rc)
+    return y
+
+
+def batchnorm_f32(x, scale, bias, mean, var, epsilon=1e-5, relu=False):
+    """Inference BatchNormalization over axis 1 (ROperator_BatchNormalization.hxx:127-226)."""
+    x = np.ascontiguousarray(x, np.float32)
+    N, Cc = x.shape[0], x.shape[1]
+    plane = int(np.prod(x.shape[2:])) if x.ndim > 2 else 1
+    y = np.empty_like(x)
+    f = lambda a: np.ascontiguousarray(a, np.float32)
+    _bn(x.reshape(-1), f(scale), f(bias), f(mean), f(var), float(epsilon), y.reshape(-1), N, Cc, plane, int(relu))
     return y
 
 

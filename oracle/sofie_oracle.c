@@ -15,6 +15,8 @@
  *                                torch.nn.functional.conv2d on CPU, brute-force 7-loop
  *   or_conv_transpose2d_f32      pinned: ConvTranspose1d/2d/Bias2d/Bias2dBatched known
  *                                answers, torch.nn.functional.conv_transpose2d on CPU
+ *   or_batchnorm_f32             pinned: torch.nn.functional.batch_norm on CPU, float64
+ *                                closed form (the reference holds no fixture for it)
  *   or_relu, or_maxpool2d        pinned: MaxPool2d known answer, torch CPU
  *   or_broadcast_rows            pinned through the Linear_* answers (bias broadcast)
  *   or_qgemm_s8, or_qconv2d_s8,
@@ -266,6 +268,39 @@ int or_conv_transpose2d_f32(const float *x, const float *w, const float *bias, f
         for (size_t i = 0; i < len; ++i) y[i] = (y[i] > 0) ? y[i] : 0;
     free(col);
     return 0;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Inference BatchNormalization as ROperator_BatchNormalization<float> emits */
+/* it (ROperator_BatchNormalization.hxx:127-226), x [N, C, plane]:           */
+/*   Initialize: inv = 1. / sqrt(var[c] + epsilon) (fp32 sum, double root and*/
+/*   quotient, stored as fp32), scale'[c] = scale[c] * inv (fp32) (:163-167) */
+/*   Generate: Y = X (scopy_), Y += -1 * mean (saxpy_), Y *= scale' (loop),  */
+/*   Y += 1 * bias (saxpy_), optional ReLU loop (:196-226); every step is a  */
+/*   separately rounded fp32 operation.                                      */
+/* The reference's parser never reads the epsilon attribute (it always       */
+/* passes 1e-5, ParseBatchNormalization.cxx:20-31); epsilon is an argument   */
+/* here. Pinned by: torch.nn.functional.batch_norm on CPU, float64 closed    */
+/* form (no fixture of the reference covers this operator).                  */
+/* ------------------------------------------------------------------------- */
+void or_batchnorm_f32(const float *x, const float *scale, const float *bias, const float *mean,
+                      const float *var, float epsilon, float *y, int N, int C, int plane, int relu)
+{
+    for (int n = 0; n < N; ++n)
+        for (int c = 0; c < C; ++c) {
+            const float shifted = var[c] + epsilon;
+            const float inv = (float)(1. / sqrt((double)shifted));
+            const float s = scale[c] * inv;
+            const size_t off = ((size_t)n * C + c) * plane;
+            for (int i = 0; i < plane; ++i) {
+                float v = x[off + i];
+                v = v + (-1.0f) * mean[c];
+                v = v * s;
+                v = v + 1.0f * bias[c];
+                if (relu) v = (v > 0) ? v : 0;
+                y[off + i] = v;
+            }
+        }
 }
 
 /* ------------------------------------------------------------------------- */

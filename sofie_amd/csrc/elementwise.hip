@@ -27,6 +27,40 @@ __global__ void k_relu_f32_scalar(const float *__restrict__ x, float *__restrict
    if (i < len) y[i] = x[i] > 0.0f ? x[i] : 0.0f;
 }
 
+// Inference BatchNormalization over [N*C planes][plane] elements: y = (x - mean[c]) * scale[c] + bias[c], each
+// step rounded on its own as the reference's copy / axpy / multiply / axpy sequence does
+// (ROperator_BatchNormalization.hxx:196-226); scale already holds scale / sqrt(var + eps). One workgroup row
+// per plane (blockIdx.y), four elements per thread when the plane length allows it.
+template <bool VEC>
+__global__ void k_batchnorm_f32(const float *__restrict__ x, const float *__restrict__ scale, const float *__restrict__ mean,
+                                const float *__restrict__ bias, float *__restrict__ y, int C, int plane, int relu,
+                                int first_channel)
+{
+   const int pc = blockIdx.y;
+   const int c = (pc + first_channel) % C;
+   const float s = scale[c], m = mean[c], b = bias[c];
+   const float *xp = x + (size_t)pc * plane;
+   float *yp = y + (size_t)pc * plane;
+   if constexpr (VEC) {
+      for (int i = (blockIdx.x * blockDim.x + threadIdx.x) * 4; i < plane; i += gridDim.x * blockDim.x * 4) {
+         const v4f v = *reinterpret_cast<const v4f *>(xp + i);
+         v4f r;
+#pragma unroll
+         for (int t = 0; t < 4; ++t) {
+            r[t] = __fadd_rn(__fmul_rn(__fsub_rn(v[t], m), s), b);
+            if (relu) r[t] = r[t] > 0.0f ? r[t] : 0.0f;
+         }
+         *reinterpret_cast<v4f *>(yp + i) = r;
+      }
+   } else {
+      for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < plane; i += gridDim.x * blockDim.x) {
+         float r = __fadd_rn(__fmul_rn(__fsub_rn(xp[i], m), s), b);
+         if (relu) r = r > 0.0f ? r : 0.0f;
+         yp[i] = r;
+      }
+   }
+}
+
 template <typename T>
 __device__ __forceinline__ T lowest();
 template <>
@@ -216,6 +250,35 @@ int sofie_hip_relu_f32(sofie_hip_ctx *ctx, const float *x, float *y, size_t len)
    else
       hipLaunchKernelGGL(k_relu_f32_scalar, dim3(blocks_for(len, 256)), dim3(256), 0, ctx->stream, x, y, len);
    return check_launch(ctx, "k_relu_f32");
+}
+
+int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, const float *x, const float *scale, const float *mean, const float *bias,
+                            float *y, int N, int C, int plane, int act)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, N >= 0 && C > 0 && plane > 0, "non-positive dimension");
+   SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
+   if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && scale && mean && bias && y, "null operand");
+   const size_t planes = (size_t)N * C;
+   const bool vec = plane % 4 == 0 && aligned16(x) && aligned16(y);
+   const int per_block = vec ? 1024 : 256;
+   int bx = (plane + per_block - 1) / per_block;
+   if (bx > 64) bx = 64;
+   // planes ride in blockIdx.y (at most 65535 per launch)
+   for (size_t p0 = 0; p0 < planes; p0 += 65535) {
+      const unsigned np = (unsigned)((planes - p0) < 65535 ? (planes - p0) : 65535);
+      const float *xs = x + p0 * plane;
+      float *ys = y + p0 * plane;
+      const int c0 = (int)(p0 % (size_t)C);
+      if (vec)
+         hipLaunchKernelGGL(k_batchnorm_f32<true>, dim3(bx, np), dim3(256), 0, ctx->stream, xs, scale, mean, bias, ys, C, plane,
+                            act == SOFIE_ACT_RELU, c0);
+      else
+         hipLaunchKernelGGL(k_batchnorm_f32<false>, dim3(bx, np), dim3(256), 0, ctx->stream, xs, scale, mean, bias, ys, C, plane,
+                            act == SOFIE_ACT_RELU, c0);
+   }
+   return check_launch(ctx, "k_batchnorm_f32");
 }
 
 static int pool_dims(sofie_hip_ctx *ctx, int H, int W, int kh, int kw, int pt, int pl, int pb, int pr, int sh,

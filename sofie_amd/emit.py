@@ -79,6 +79,9 @@ class ModelSpec:
             auto_pad, group, _lst(kernel), _lst(pads), _lst(strides), _lst(dilations), _lst(output_padding),
             _lst(output_shape), x, w, b or "-", y))
 
+    def batchnorm(self, x, scale, b, mean, var, y, epsilon=1e-5):
+        self.lines.append("op BatchNormalization %r %s %s %s %s %s %s" % (float(epsilon), x, scale, b, mean, var, y))
+
     def relu(self, x, y):
         self.lines.append("op Relu %s %s" % (x, y))
 
@@ -183,6 +186,8 @@ def spec_from_onnx(name, graph):
             spec.conv_transpose(ins[0], ins[1], ins[2] if len(ins) > 2 else None, out, a.get("kernel_shape", ()),
                                 a.get("pads", ()), a.get("strides", ()), a.get("dilations", ()), a.get("group", 0),
                                 a.get("output_padding", ()), a.get("output_shape", ()), a.get("auto_pad", "NOTSET"))
+        elif op == "BatchNormalization":
+            spec.batchnorm(ins[0], ins[1], ins[2], ins[3], ins[4], out, a.get("epsilon", 1e-5))
         elif op == "MaxPool":
             spec.maxpool(ins[0], out, a["kernel_shape"], a.get("pads", (0, 0, 0, 0)), a.get("strides", (1, 1)))
         elif op == "Flatten":

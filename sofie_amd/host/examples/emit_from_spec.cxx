@@ -12,6 +12,7 @@
 //   output NAME
 //   op Gemm ALPHA BETA TRANSA TRANSB A B C Y RELU
 //   op Conv AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. X W B Y
+//   op BatchNormalization EPSILON X SCALE B MEAN VAR Y
 //   op ConvTranspose AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. nop op.. nos os.. X W B Y
 //   op Relu X Y
 //   op MaxPool nk k.. np p.. ns s.. X Y
@@ -117,6 +118,11 @@ int main(int argc, char **argv)
                auto k = List(in), p = List(in), s = List(in), d = List(in), op_ = List(in), os = List(in);
                in >> x >> w >> b >> y;
                r.reset(new ROperator_ConvTranspose<float>(autopad, d, group, k, op_, os, p, s, x, w, b == "-" ? std::string() : b, y));
+            } else if (op == "BatchNormalization") {
+               float eps;
+               std::string x, sc, b, m, v, y;
+               in >> eps >> x >> sc >> b >> m >> v >> y;
+               r.reset(new ROperator_BatchNormalization<float>(eps, 0.9f, 0, x, sc, b, m, v, y));
             } else if (op == "Relu") {
                std::string x, y;
                in >> x >> y;

@@ -1,4 +1,5 @@
 // Every operator emitter of this build (the reference's OperatorList.hxx lists all of its own).
+#include "SOFIE/ROperator_BatchNormalization.hxx"
 #include "SOFIE/ROperator_Conv.hxx"
 #include "SOFIE/ROperator_ConvTranspose.hxx"
 #include "SOFIE/ROperator_Gemm.hxx"

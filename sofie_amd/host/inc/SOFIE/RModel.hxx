@@ -124,6 +124,7 @@ private:
       size_t offset = 0, bytes = 0;
       int first = 0, last = 0;
    };
+   void FuseBatchNorm();
    void FuseActivations();
    void FusePooling();
    void FuseInputQuantization();

@@ -50,6 +50,14 @@ public:
    // try to absorb a preceding QuantizeLinear (float tensor xFloat quantized with scale / zeroPoint into this
    // operator's int8 input): on success the operator reads the float tensor itself
    virtual bool FuseInputQuantization(const std::string & /*xFloat*/, float /*scale*/, int /*zeroPoint*/) { return false; }
+   // try to absorb a following BatchNormalization y = (x - mean[c]) * scale[c] + bias[c] (one value per output
+   // channel, the variance already folded into scale) and, if relu is set, the ReLU behind it; on success the
+   // operator writes the tensor outName instead of its own output
+   virtual bool FuseBatchNorm(RModel & /*model*/, const std::vector<float> & /*scale*/, const std::vector<float> & /*mean*/,
+                              const std::vector<float> & /*bias*/, const std::string & /*outName*/, bool /*relu*/)
+   {
+      return false;
+   }
    // absorbed into another operator: emits nothing, and its output is written by the absorbing operator
    void SetAbsorbed() { fAbsorbed = true; }
    bool IsAbsorbed() const { return fAbsorbed; }

@@ -9,6 +9,7 @@
 #ifndef SOFIE_SOFIE_ROPERATOR_CONV
 #define SOFIE_SOFIE_ROPERATOR_CONV
 
+#include <cstdlib>
 #include <iostream>
 #include <sstream>
 
@@ -109,6 +110,39 @@ public:
       fActivation = act;
       return true;
    }
+   // Conv -> BatchNormalization: W'[oc] = W[oc] * scale[oc], b'[oc] = (b[oc] - mean[oc]) * scale[oc] + bias[oc],
+   // written as new initializers; the convolution then produces the normalised tensor directly.
+   bool FuseBatchNorm(RModel &model, const std::vector<float> &scale, const std::vector<float> &mean,
+                      const std::vector<float> &bias, const std::string &outName, bool relu) override
+   {
+      if (fShapeW.empty() || fActivation != EActivationType::UNDEFINED) return false;
+      if (!model.IsInitializedTensor(fNW) || (fNB != "" && !model.IsInitializedTensor(fNB))) return false;
+      const size_t oc = fShapeW[0];
+      if (scale.size() != oc || mean.size() != oc || bias.size() != oc) return false;
+      const size_t per = ConvertShapeToLength(fShapeW) / oc;
+      const float *w = static_cast<float *>(model.GetInitializedTensorData(fNW).get());
+      const float *b = fNB != "" ? static_cast<float *>(model.GetInitializedTensorData(fNB).get()) : nullptr;
+      std::shared_ptr<void> nw(malloc(oc * per * sizeof(float)), free), nb(malloc(oc * sizeof(float)), free);
+      float *pw = static_cast<float *>(nw.get()), *pb = static_cast<float *>(nb.get());
+      for (size_t c = 0; c < oc; ++c) {
+         for (size_t i = 0; i < per; ++i) pw[c * per + i] = w[c * per + i] * scale[c];
+         pb[c] = ((b ? b[c] : 0.0f) - mean[c]) * scale[c] + bias[c];
+      }
+      const std::string foldedW = outName + "_bnw", foldedB = outName + "_bnb";
+      model.AddInitializedTensor(foldedW, ETensorType::FLOAT, fShapeW, nw);
+      model.AddInitializedTensor(foldedB, ETensorType::FLOAT, {oc}, nb);
+      fNW = foldedW;
+      fNB = foldedB;
+      fShapeB = {oc};
+      fNY = outName;
+      fInputTensorNames = {fNX, fNW, fNB};
+      fOutputTensorNames = {fNY};
+      if (relu) fActivation = EActivationType::RELU;
+      return true;
+   }
+   const std::string &WeightName() const { return fNW; }
+   const std::string &BiasName() const { return fNB; }
+
    std::vector<ETensorType> TypeInference(std::vector<ETensorType> input) override { return {input[0]}; }
    std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>> input) override
    {

@@ -4,6 +4,8 @@
 // constructor that reads the text weight file with name/length checks, infer() that runs every
 // operator's Generate() text and returns a std::vector copy of the output.
 #include "SOFIE/RModel.hxx"
+#include "SOFIE/ROperator_BatchNormalization.hxx"
+#include "SOFIE/ROperator_Conv.hxx"
 #include "SOFIE/ROperator_Pool.hxx"
 #include "SOFIE/ROperator_Quantized.hxx"
 
@@ -184,16 +186,17 @@ void RModel::Initialize(int /*batchSize*/, bool verbose)
    fIsInitialized = true;
 }
 
-// Conv / Gemm / QLinear* followed by a Relu that is the only consumer of their output:
-// the activation moves into the producer's epilogue and the Relu becomes a view.
-void RModel::FuseActivations()
+// Float Conv followed by a BatchNormalization that is the only reader of its output: the normalisation is
+// folded into the convolution's weights and bias at generation time and the BatchNormalization emits nothing.
+// Runs before FuseActivations, so a Relu behind the pair is then fused into the convolution as usual.
+void RModel::FuseBatchNorm()
 {
    for (size_t i = 0; i + 1 < fOperators.size(); ++i) {
-      ROperator &prod = *fOperators[i];
-      ROperator &act = *fOperators[i + 1];
-      if (act.Kind() != "Relu" || prod.GetOpOutputTensors().empty()) continue;
-      const std::string &mid = prod.GetOpOutputTensors()[0];
-      if (act.GetOpInputTensors().empty() || act.GetOpInputTensors()[0] != mid) continue;
+      auto *conv = dynamic_cast<ROperator_Conv<float> *>(fOperators[i].get());
+      auto *bn = dynamic_cast<ROperator_BatchNormalization<float> *>(fOperators[i + 1].get());
+      if (!conv || !bn || conv->GetOpOutputTensors().empty()) continue;
+      const std::string mid = conv->GetOpOutputTensors()[0];
+      if (bn->GetOpInputTensors().empty() || bn->GetOpInputTensors()[0] != mid) continue;
       bool other_use = std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), mid) != fOutputTensorNames.end();
       for (size_t j = 0; j < fOperators.size() && !other_use; ++j) {
          if (j == i + 1) continue;
@@ -201,7 +204,50 @@ void RModel::FuseActivations()
             if (in == mid) other_use = true;
       }
       if (other_use) continue;
-      if (prod.FuseActivation(EActivationType::RELU)) act.SetFusedAway();
+      const std::string oldW = conv->WeightName(), oldB = conv->BiasName();
+      if (!conv->FuseBatchNorm(*this, bn->FoldedScale(), bn->Mean(), bn->Bias(), bn->GetOpOutputTensors()[0], bn->HasActivation()))
+         continue;
+      bn->SetAbsorbed();
+      fIntermediateTensorInfos.erase(mid);
+      // initializers nobody reads any more are neither written to the weight file nor uploaded
+      std::vector<std::string> orphans = bn->OwnInitializers();
+      orphans.push_back(oldW);
+      if (!oldB.empty()) orphans.push_back(oldB);
+      for (auto &name : orphans) {
+         bool used = false;
+         for (size_t j = 0; j < fOperators.size() && !used; ++j) {
+            if (j == i + 1) continue;
+            for (auto &in : fOperators[j]->GetOpInputTensors())
+               if (in == name) used = true;
+         }
+         if (!used && IsInitializedTensor(name)) SetNotWritableInitializedTensor(name);
+      }
+   }
+}
+
+// Conv / Gemm / QLinear* followed by a Relu that is the only consumer of their output:
+// the activation moves into the producer's epilogue and the Relu becomes a view.
+void RModel::FuseActivations()
+{
+   for (size_t j = 1; j < fOperators.size(); ++j) {
+      ROperator &act = *fOperators[j];
+      if (act.Kind() != "Relu" || act.GetOpInputTensors().empty()) continue;
+      const std::string &mid = act.GetOpInputTensors()[0];
+      // the operator that writes the activation's input (an absorbed operator writes nothing)
+      size_t i = j;
+      for (size_t k = 0; k < j; ++k) {
+         if (fOperators[k]->IsAbsorbed() || fOperators[k]->GetOpOutputTensors().empty()) continue;
+         if (fOperators[k]->GetOpOutputTensors()[0] == mid) i = k;
+      }
+      if (i == j) continue;
+      bool other_use = std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), mid) != fOutputTensorNames.end();
+      for (size_t k = 0; k < fOperators.size() && !other_use; ++k) {
+         if (k == j || fOperators[k]->IsAbsorbed()) continue;
+         for (auto &in : fOperators[k]->GetOpInputTensors())
+            if (in == mid) other_use = true;
+      }
+      if (other_use) continue;
+      if (fOperators[i]->FuseActivation(EActivationType::RELU)) act.SetFusedAway();
    }
 }
 
@@ -649,6 +695,7 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    }
    (void)pos;
    Initialize(batchSize, verbose);
+   FuseBatchNorm();
    FuseActivations();
    FusePooling();
    FuseInputQuantization();

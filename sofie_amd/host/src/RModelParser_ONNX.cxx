@@ -337,7 +337,7 @@ std::shared_ptr<void> TensorData(const Tensor &t, ETensorType type, size_t lengt
 
 const std::set<std::string> &Supported()
 {
-   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "Conv", "ConvTranspose", "Relu", "MaxPool", "Flatten", "Reshape",
+   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "BatchNormalization", "Conv", "ConvTranspose", "Relu", "MaxPool", "Flatten", "Reshape",
                                              "QuantizeLinear", "DequantizeLinear", "QLinearMatMul", "QLinearConv"};
    return ops;
 }
@@ -651,6 +651,14 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
                                                      n.Sizes("kernel_shape"), n.Sizes("output_padding"), n.Sizes("output_shape"),
                                                      n.Sizes("pads"), n.Sizes("strides"), n.inputs[0], n.inputs[1], InputOr(n, 2),
                                                      n.outputs[0]));
+      } else if (t == "BatchNormalization") {
+         // The reference's parser passes epsilon = 1e-5 whatever the node says (ParseBatchNormalization.cxx:20-31);
+         // the attribute is honoured here, so files written with the ONNX default give the same numbers.
+         if (n.inputs.size() != 5)
+            throw std::runtime_error("TMVA::SOFIE - BatchNormalization node " + n.name + " needs 5 inputs");
+         op.reset(new ROperator_BatchNormalization<float>(n.Float("epsilon", 1e-05f), n.Float("momentum", 0.9f),
+                                                          (size_t)n.Int("training_mode", 0), n.inputs[0], n.inputs[1], n.inputs[2],
+                                                          n.inputs[3], n.inputs[4], n.outputs[0]));
       } else if (t == "Relu") {
          op.reset(new ROperator_Relu<float>(n.inputs.at(0), n.outputs[0]));
       } else if (t == "MaxPool") {

@@ -35,6 +35,7 @@ SIGNATURES = {
     "sofie_hip_gemm_f32": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i, _p, _i, _i],
     "sofie_hip_conv2d_f32": [_p, _p, _p, _p, _p] + [_i] * 15,
     "sofie_hip_conv_transpose2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,
+    "sofie_hip_batchnorm_f32": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i],
     "sofie_hip_relu_f32": [_p, _p, _p, _z],
     "sofie_hip_maxpool2d_f32": [_p, _p, _p] + [_i] * 11,
     "sofie_hip_quantize_f32_s8": [_p, _p, _p, _z, _f, _i],

@@ -159,6 +159,22 @@ def conv_transpose2d_f32(x, w, bias=None, pads=(0, 0, 0, 0), strides=(1, 1), dil
     return _ret(y, x)
 
 
+def batchnorm_f32(x, scale, bias, mean, var, epsilon=1e-5, relu=False, ctx=None):
+    """Inference BatchNormalization over axis 1; the variance is folded into the scale on the host the way the
+    emitter does it: scale * float(1 / sqrt(double(var + epsilon)))."""
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.float32)
+    folded = (np.asarray(scale, np.float32) *
+              (1.0 / np.sqrt((np.asarray(var, np.float32) + np.float32(epsilon)).astype(np.float64))).astype(np.float32))
+    sd, md, bd = ctx.dev(folded.astype(np.float32), torch.float32), ctx.dev(mean, torch.float32), ctx.dev(bias, torch.float32)
+    N, Cc = xd.shape[0], xd.shape[1]
+    plane = int(np.prod(xd.shape[2:])) if xd.dim() > 2 else 1
+    y = ctx.empty(tuple(xd.shape), torch.float32)
+    ctx.check(ctx.lib.sofie_hip_batchnorm_f32(ctx.h, ctx.ptr(xd), ctx.ptr(sd), ctx.ptr(md), ctx.ptr(bd), ctx.ptr(y), N, Cc,
+                                              plane, L.ACT_RELU if relu else L.ACT_NONE))
+    return _ret(y, x)
+
+
 def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0), layout=L.LAYOUT_NCHW, ctx=None):
     """pads = (top, left, bottom, right). int8 tensors may be NHWC (layout flag); fp32 is NCHW."""
     ctx = ctx or default_context()

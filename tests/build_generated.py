@@ -23,6 +23,7 @@ def all_specs(with_large=True):
     specs.append(models.cnn_f32_spec(8))
     specs.append(models.qcnn_spec(oracle, 8))
     specs.append(models.qdq_conv_spec())
+    specs.append(models.convbn_spec())
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs

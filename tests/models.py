@@ -221,3 +221,46 @@ def qdq_conv_reference(oracle):
     scale = ((p["sx"] * p["sw"]).astype(np.float32) / p["sy"]).astype(np.float32)
     c = oracle.qconv2d_s8(xq, p["w"], scale, p["b"], (1, 1), (1, 1), 1, p["zx"], p["zy"], False)
     return oracle.dequantize_s8_f32(c, p["sy"], p["zy"])
+
+
+# ------------------------------------------------------------------------------------------ conv + batch norm
+def convbn_params(seed=21):
+    """Conv(3->16) -> BatchNormalization -> Relu -> MaxPool -> BatchNormalization -> ConvTranspose(16->4, stride 2) ->
+    Relu on [4,3,12,12]: the first normalisation folds into the convolution, the second one runs as its own
+    kernel (it follows a pooling), the transposed convolution takes the fused Relu."""
+    r = np.random.default_rng(seed)
+    p = {"x": r.standard_normal((4, 3, 12, 12)).astype(np.float32),
+         "w1": (r.standard_normal((16, 3, 3, 3)) * 0.3).astype(np.float32), "b1": r.standard_normal(16).astype(np.float32),
+         "wt": (r.standard_normal((16, 4, 4, 4)) * 0.2).astype(np.float32), "bt": r.standard_normal(4).astype(np.float32)}
+    for k in ("1", "2"):
+        p["g" + k] = r.uniform(0.5, 1.5, 16).astype(np.float32)
+        p["beta" + k] = r.standard_normal(16).astype(np.float32)
+        p["mean" + k] = r.standard_normal(16).astype(np.float32)
+        p["var" + k] = r.uniform(0.2, 2.0, 16).astype(np.float32)
+    return p
+
+
+def convbn_spec(name="convbn"):
+    p = convbn_params()
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", p["x"].shape)
+    for k in ("w1", "b1", "wt", "bt", "g1", "beta1", "mean1", "var1", "g2", "beta2", "mean2", "var2"):
+        s.add_init(k, p[k])
+    s.conv("x", "w1", "b1", "c1", (3, 3), (1, 1, 1, 1), (1, 1))
+    s.batchnorm("c1", "g1", "beta1", "mean1", "var1", "n1", 1e-5)
+    s.relu("n1", "r1")
+    s.maxpool("r1", "p1", (2, 2), (0, 0, 0, 0), (2, 2))
+    s.batchnorm("p1", "g2", "beta2", "mean2", "var2", "n2", 1e-3)
+    s.conv_transpose("n2", "wt", "bt", "t1", (), (1, 1, 1, 1), (2, 2))
+    s.relu("t1", "y")
+    s.set_output("y")
+    return s
+
+
+def convbn_reference(oracle):
+    p = convbn_params()
+    c1 = oracle.conv2d_f32(p["x"], p["w1"], p["b1"], (1, 1), (1, 1))
+    r1 = oracle.batchnorm_f32(c1, p["g1"], p["beta1"], p["mean1"], p["var1"], 1e-5, relu=True)
+    p1 = oracle.maxpool2d(r1, (2, 2), (2, 2))
+    n2 = oracle.batchnorm_f32(p1, p["g2"], p["beta2"], p["mean2"], p["var2"], 1e-3)
+    return oracle.conv_transpose2d_f32(n2, p["wt"], p["bt"], (1, 1, 1, 1), (2, 2), relu=True)

@@ -308,6 +308,31 @@ def test_cpp_onnx_front_end_fuses_qdq_groups(tmp_path):
     assert res.returncode != 0 or "sofie_hip_qgemm_s8(" not in open(str(tmp_path / "qdq_bad_axis.hxx")).read()
 
 
+def test_batchnorm_folds_into_conv_or_runs_alone(tmp_path):
+    """Conv -> BatchNormalization -> Relu becomes one convolution call whose weights and bias carry the
+    normalisation (W * s, (b - mean) * s + beta with s = gamma / sqrt(var + eps)); a BatchNormalization that does not
+    follow a convolution is one call of its own kernel with the folded per-channel scale; the tensors only the
+    absorbed operator read are not written to the weight file."""
+    spec = models.convbn_spec("convbn_t")
+    hxx, dat, _ = spec.generate(str(tmp_path))
+    code = open(hxx).read()
+    assert code.count("sofie_hip_conv2d_f32(") == 1 and code.count("sofie_hip_batchnorm_f32(") == 1
+    assert "tensor_n1_bnw, tensor_n1_bnb, tensor_n1, " in code and "SOFIE_ACT_RELU), \"Conv" in code
+    assert code.count("sofie_hip_conv_transpose2d_f32(") == 1 and code.count("sofie_hip_relu_f32(") == 0
+    lines = open(dat).read().split("\n")
+    names = [l.split()[0] for l in lines if l.startswith("tensor_")]
+    for gone in ("tensor_w1", "tensor_b1", "tensor_g1", "tensor_var1", "tensor_mean1", "tensor_beta1", "tensor_g2", "tensor_var2"):
+        assert gone not in names
+    for kept in ("tensor_n1_bnw", "tensor_n1_bnb", "tensor_n2_bnscale", "tensor_mean2", "tensor_beta2", "tensor_wt"):
+        assert kept in names
+    p = models.convbn_params()
+    s1 = p["g1"] * (1.0 / np.sqrt((p["var1"] + np.float32(1e-5)).astype(np.float64))).astype(np.float32)
+    got_w = np.array(lines[[i for i, l in enumerate(lines) if l.startswith("tensor_n1_bnw ")][0] + 1].split(), np.float32)
+    got_b = np.array(lines[[i for i, l in enumerate(lines) if l.startswith("tensor_n1_bnb ")][0] + 1].split(), np.float32)
+    assert np.array_equal(got_w, (p["w1"] * s1[:, None, None, None]).reshape(-1))
+    assert np.array_equal(got_b, (p["b1"] - p["mean1"]) * s1 + p["beta1"])
+
+
 def test_every_prebuilt_session_compiles():
     """tests/build_generated.py output (made by build()): header, weights and runner of each network."""
     import build_generated

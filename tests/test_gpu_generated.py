@@ -65,6 +65,17 @@ def test_cnn_f32_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
+def test_conv_batchnorm_convtranspose_session(tmp_path):
+    """Conv -> BatchNormalization -> Relu (folded into the convolution at generation time) -> MaxPool ->
+    BatchNormalization (its own kernel) -> ConvTranspose -> Relu against the unfused oracle steps; 1e-5 relative
+    (folding the scale into the weights rounds differently from scaling the sum)."""
+    p = models.convbn_params()
+    y = run_session("convbn", p["x"], tmp_path)
+    ref = models.convbn_reference(oracle)
+    assert y.size == ref.size
+    assert rel_err(y, ref.reshape(-1)) <= 1e-5
+
+
 def test_int8_cnn_session_is_bit_exact(tmp_path):
     x = models.cnn_input(8)
     y = run_session("qcnn", x, tmp_path)

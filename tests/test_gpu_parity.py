@@ -105,6 +105,21 @@ def test_conv_transpose2d_f32_is_the_adjoint_of_conv2d(ops):
     assert abs(lhs - rhs) <= 1e-5 * max(abs(lhs), abs(rhs), 1.0) * 10
 
 
+# --------------------------------------------------------------------------- batch normalisation
+@pytest.mark.parametrize("shape", [(3, 5, 7, 6), (4, 9), (2, 3, 10), (2, 64, 56, 56), (70000, 2), (1, 1, 1, 1)])
+def test_batchnorm_f32(ops, shape):
+    """Same rounding steps as the oracle's restatement of the reference (subtract, multiply by the folded scale, add):
+    identical bits, with and without the fused ReLU; vector and scalar planes, more planes than one launch holds."""
+    r = rng(60 + len(shape) + shape[1])
+    C = shape[1]
+    x = (r.standard_normal(shape) * 3).astype(np.float32)
+    g, b = r.uniform(0.5, 2, C).astype(np.float32), r.standard_normal(C).astype(np.float32)
+    m, v = r.standard_normal(C).astype(np.float32), r.uniform(0.1, 3, C).astype(np.float32)
+    for eps, relu in ((1e-5, False), (1e-3, True)):
+        y = ops.batchnorm_f32(x, g, b, m, v, eps, relu)
+        assert np.array_equal(y, oracle.batchnorm_f32(x, g, b, m, v, eps, relu))
+
+
 # --------------------------------------------------------------------------- fp32 gemm
 @pytest.mark.parametrize("M,N,K,tA,tB,alpha,beta,relu", [
     (256, 128, 64, 0, 0, 1.0, 1.0, True),      # MLP layer 1 of the fp32 configuration
