@@ -1,6 +1,8 @@
 // ONNX file -> generated Session header and weight file, the flow of the reference's own tests
 // (src/SOFIE_core/test/EmitFromONNX.cxx.in: Parse, Generate, OutputGenerated).
-//   emit_from_onnx <model.onnx> <output directory> [--check]
+//   emit_from_onnx <model.onnx> <output directory> [--check | --batch N]
+// --batch N gives a parametric batch dimension of the inputs ("bs", "batch_size", a -1) the value N, the way the
+// reference's users pass a batch size to RModel::Generate.
 #include <iostream>
 
 #include "SOFIE/RModelParser_ONNX.hxx"
@@ -8,14 +10,16 @@
 int main(int argc, char **argv)
 {
    if (argc < 3) {
-      std::cerr << "usage: emit_from_onnx <model.onnx> <output directory> [--check]\n";
+      std::cerr << "usage: emit_from_onnx <model.onnx> <output directory> [--check | --batch N]\n";
       return 2;
    }
    try {
       SOFIE::RModelParser_ONNX parser;
       if (argc > 3 && std::string(argv[3]) == "--check") return parser.CheckModel(argv[1], true) ? 0 : 1;
       SOFIE::RModel model = parser.Parse(argv[1]);
-      model.Generate();
+      int batch = -1;
+      if (argc > 4 && std::string(argv[3]) == "--batch") batch = std::stoi(argv[4]);
+      model.Generate(static_cast<std::underlying_type_t<SOFIE::Options>>(SOFIE::Options::kDefault), batch);
       const std::string out = std::string(argv[2]) + "/" + model.GetName() + ".hxx";
       model.OutputGenerated(out);
       std::cout << "generated " << out << ", intermediate pool " << model.GetIntermediateMemorySize() << " bytes\n";

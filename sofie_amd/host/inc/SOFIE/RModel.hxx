@@ -98,6 +98,7 @@ public:
    void AddNeededCustomHeader(std::string filename) { fCustomOpHeaders.insert(filename); }
 
    void Initialize(int batchSize = -1, bool verbose = false);
+   void Initialize(const std::map<std::string, size_t> &inputParams, bool verbose = false);
    void Generate(std::underlying_type_t<Options> options, int batchSize = -1, long pos = 0, bool verbose = false);
    void Generate(Options options = Options::kDefault, int batchSize = -1, int pos = 0, bool verbose = false)
    {
@@ -139,6 +140,8 @@ private:
    int fVerbose = 0;
 
    std::map<std::string, TensorInfo> fReadyInputTensorInfos;
+   struct ParametricInput { ETensorType type; std::vector<Dim> shape; };
+   std::map<std::string, ParametricInput> fInputTensorInfos;   // inputs whose shape still holds a parameter
    std::map<std::string, InitializedTensor> fInitializedTensors;
    std::map<std::string, TensorInfo> fIntermediateTensorInfos;
    std::vector<std::string> fOutputTensorNames, fInputTensorNames;

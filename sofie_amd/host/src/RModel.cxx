@@ -73,9 +73,15 @@ bool RModel::IsReadyInputTensor(const std::string &name) const { return fReadyIn
 void RModel::AddInputTensorInfo(std::string input_name, ETensorType type, std::vector<Dim> shape)
 {
    std::vector<size_t> s = ConvertShapeToInt(shape);
-   if (s.empty() && !shape.empty())
-      throw std::runtime_error("TMVA-SOFIE: parametric input shapes are not supported by the device emission (tensor " +
-                               input_name + ")");
+   if (s.empty() && !shape.empty()) {
+      // a parametric shape (a named batch dimension): kept until Initialize is told the value, as in the
+      // reference (RModel_Base / RModel.cxx:398-463)
+      input_name = UTILITY::Clean_name(input_name);
+      if (CheckIfTensorAlreadyExist(input_name))
+         throw std::runtime_error("TMVA-SOFIE: input tensor with name " + input_name + " already exists \n");
+      fInputTensorInfos[input_name] = ParametricInput{type, shape};
+      return;
+   }
    AddInputTensorInfo(input_name, type, s);
 }
 
@@ -162,10 +168,44 @@ void RModel::AddNeededStdLib(std::string libname)
    if (fAllowedStdLib.count(libname)) fNeededStdLib.insert(libname);
 }
 
-void RModel::Initialize(int /*batchSize*/, bool verbose)
+// batchSize > 0 gives the parameters "input_size", "batch_size" and "bs" that value (RModel.cxx:398-407).
+void RModel::Initialize(int batchSize, bool verbose)
+{
+   std::map<std::string, size_t> inputParams;
+   if (batchSize > 0) {
+      inputParams["input_size"] = batchSize;
+      inputParams["batch_size"] = batchSize;
+      inputParams["bs"] = batchSize;
+   }
+   Initialize(inputParams, verbose);
+}
+
+// Parametric input dimensions are replaced by the given values (a dimension named "<tensor>_size", which the
+// parser makes out of a -1, answers to "input_size"), RModel.cxx:408-463. The reference goes on to emit
+// shape-generic code for what is still parametric; the device emission sizes its buffers and launches at
+// generation time, so a parameter without a value is an error here.
+void RModel::Initialize(const std::map<std::string, size_t> &inputParams, bool verbose)
 {
    fVerbose = int(verbose);
    if (fIsInitialized) return;
+   auto parametric = fInputTensorInfos;
+   for (auto &input : parametric) {
+      for (auto &d : input.second.shape) {
+         if (!d.isParam) continue;
+         std::string pname = d.param;
+         if (pname == input.first + "_size") pname = "input_size";
+         auto itr = inputParams.find(pname);
+         if (itr != inputParams.end()) d = Dim{itr->second};
+      }
+      const std::vector<size_t> shape = ConvertShapeToInt(input.second.shape);
+      if (shape.empty())
+         throw std::runtime_error("TMVA-SOFIE: input tensor " + input.first + " has the parametric shape " +
+                                  ConvertDynamicShapeToString(input.second.shape) +
+                                  "; the device emission needs every dimension at generation time: pass the batch size "
+                                  "to Generate / Initialize");
+      fInputTensorInfos.erase(input.first);
+      AddInputTensorInfo(input.first, input.second.type, shape);
+   }
    fIntermediateTensorInfos.clear();
    // every declared input must have a shape, as in the reference (RModel.cxx:410-468)
    for (auto &n : fInputTensorNames)

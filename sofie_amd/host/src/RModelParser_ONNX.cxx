@@ -514,14 +514,21 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
    for (auto &in : g.inputs) {
       if (initNames.count(in.name)) continue;
       if (in.shape.empty()) throw std::runtime_error("TMVA::SOFIE - input tensor " + in.name + " has no shape");
+      // a dimension given by name (dim_param) or as -1 is a parameter; the -1 form gets the name "<input>_size"
+      // (RModelParser_ONNX.cxx:492-513). RModel::Initialize replaces parameters by the batch size it is given.
       bool dynamic = false;
       std::vector<size_t> shape;
-      for (auto &d : in.shape) {
+      std::vector<Dim> dims = in.shape;
+      for (auto &d : dims) {
+         if (!d.isParam && (int64_t)d.dim < 0) {
+            d.isParam = true;
+            d.param = UTILITY::Clean_name(in.name) + "_size";
+         }
          if (d.isParam) dynamic = true;
          shape.push_back(d.dim);
       }
       const ETensorType type = TypeOfOnnx(in.elemType, in.name);
-      if (dynamic) model.AddInputTensorInfo(in.name, type, in.shape);   // throws: parametric shapes are not emitted
+      if (dynamic) model.AddInputTensorInfo(in.name, type, dims);
       else model.AddInputTensorInfo(in.name, type, shape);
       model.AddInputTensorName(in.name);
       if (verbose) std::cout << "input tensor " << in.name << " " << ConvertShapeToString(shape) << "\n";

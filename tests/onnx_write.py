@@ -57,7 +57,8 @@ def node(op_type, inputs, outputs, name="", **attrs):
 
 
 def value_info(name, elem_type, shape):
-    dims = b"".join(_bytes(1, _int(1, d)) for d in shape)
+    # an int is a dim_value, a string a dim_param (a named, parametric dimension)
+    dims = b"".join(_bytes(1, _bytes(2, d.encode()) if isinstance(d, str) else _int(1, d)) for d in shape)
     tensor_type = _int(1, elem_type) + _bytes(2, dims)
     return _bytes(1, name.encode()) + _bytes(2, _bytes(1, tensor_type))
 

@@ -333,6 +333,26 @@ def test_batchnorm_folds_into_conv_or_runs_alone(tmp_path):
     assert np.array_equal(got_b, (p["b1"] - p["mean1"]) * s1 + p["beta1"])
 
 
+def test_parametric_batch_dimension_is_fixed_at_generation_time(tmp_path):
+    """An input whose first dimension is the parameter "bs" (or a -1) is given its value through the batch size
+    argument of Generate, as with the reference; without a value the device emission refuses, in words that say
+    what to do."""
+    import onnx_write as ow
+    r = np.random.default_rng(3)
+    init = {"W": r.standard_normal((6, 4)).astype(np.float32), "B": r.standard_normal(4).astype(np.float32)}
+    nodes = [ow.node("Gemm", ["x", "W", "B"], ["g"]), ow.node("Relu", ["g"], ["y"])]
+    for first in ("bs", -1):
+        path = tmp_path / "dyn.onnx"
+        path.write_bytes(ow.model(nodes, init, [("x", 1, (first, 6))], [("y", 1, (first, 4))]))
+        exe = os.path.join(emit.GEN_DIR, "emit_from_onnx")
+        res = subprocess.run([exe, str(path), str(tmp_path), "--batch", "7"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        assert res.returncode == 0, res.stderr
+        code = open(str(tmp_path / "dyn.hxx")).read()
+        assert "sofie_hip_gemm_f32(fCtx, 0, 0, 7, 4, 6," in code
+        res = _onnx_emit(str(path), tmp_path)
+        assert res.returncode != 0 and "parametric shape" in res.stderr and "pass the batch size" in res.stderr
+
+
 def test_every_prebuilt_session_compiles():
     """tests/build_generated.py output (made by build()): header, weights and runner of each network."""
     import build_generated
