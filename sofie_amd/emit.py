@@ -145,6 +145,19 @@ class ModelSpec:
         return exe
 
 
+def compile_example(source, model, exe_name, outdir=GEN_DIR):
+    """g++ one of host/examples/*.cxx against the generated header of `model` and libsofie_hip.so."""
+    exe = os.path.join(outdir, exe_name)
+    cmd = ["g++", "-std=c++17", "-O2", "-pthread", "-I" + os.path.join(ROOT, "include"), "-I" + outdir,
+           "-I" + os.path.join(_HERE, "host", "inc"), "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % model,
+           "-DSOFIE_MODEL_NS=SOFIE_%s" % model, os.path.join(_HERE, "host", "examples", source), "-o", exe,
+           "-L" + _HERE, "-lsofie_hip", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath," + _HERE]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode:
+        raise RuntimeError("compiling %s failed:\n%s" % (source, res.stdout))
+    return exe
+
+
 def clean(name):
     return "".join(c if (c.isalnum() or c == "_") else ("_" if c == "-" else "") for c in name)
 

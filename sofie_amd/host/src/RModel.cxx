@@ -551,7 +551,15 @@ long RModel::WriteInitializedTensorsToFile(std::string filename)
 void RModel::GenerateSessionCode()
 {
    fGC += "struct Session {\n";
-   fGC += "sofie_hip_ctx* fCtx = nullptr;\n";
+   fGC += "// the context handle empties its source when moved, so a moved-from Session releases nothing\n";
+   fGC += "struct CtxHandle {\n";
+   fGC += "   sofie_hip_ctx* p = nullptr;\n";
+   fGC += "   CtxHandle() = default;\n";
+   fGC += "   CtxHandle(CtxHandle&& o) noexcept : p(o.p) { o.p = nullptr; }\n";
+   fGC += "   CtxHandle& operator=(CtxHandle&&) = delete;\n";
+   fGC += "   operator sofie_hip_ctx*() const { return p; }\n";
+   fGC += "};\n";
+   fGC += "CtxHandle fCtx;\n";
    fGC += "static void Check(sofie_hip_ctx* ctx, int status, const char* what) {\n";
    fGC += "   if (status != 0) throw std::runtime_error(std::string(\"TMVA SOFIE device error in \") + what + \": \" + "
           "sofie_hip_last_error(ctx));\n";
@@ -576,7 +584,7 @@ void RModel::GenerateSessionCode()
 
    // ---- constructor
    fGC += "Session(std::string filename =\"" + (fUseWeightFile ? fName + ".dat" : std::string("")) + "\", int device = 0) {\n";
-   fGC += "   { int status = sofie_hip_create(&fCtx, device, nullptr);\n";
+   fGC += "   { int status = sofie_hip_create(&fCtx.p, device, nullptr);\n";
    fGC += "     if (status != 0) throw std::runtime_error(\"TMVA SOFIE cannot create a device context\"); }\n";
    fGC += "   try {\n";
    for (auto &i : fInitializedTensors) {
@@ -655,11 +663,12 @@ void RModel::GenerateSessionCode()
    for (auto &n : fInputTensorNames) fGC += "   sofie_hip_free(fCtx, fInput_" + n + ");\n";
    fGC += "   sofie_hip_free(fCtx, fIntermediateMemoryPool);\n";
    fGC += "   sofie_hip_destroy(fCtx);\n";
-   fGC += "   fCtx = nullptr;\n";
+   fGC += "   fCtx.p = nullptr;\n";
    fGC += "}\n";
    fGC += "~Session() { Release(); }\n";
    fGC += "Session(const Session&) = delete;\n";
-   fGC += "Session& operator=(const Session&) = delete;\n\n";
+   fGC += "Session& operator=(const Session&) = delete;\n";
+   fGC += "Session(Session&&) noexcept = default;   // containers of Sessions (SofieFunctor) need it\n\n";
 
    // ---- the operator sequence on device pointers
    fGC += "// every argument is a device pointer; kernels are enqueued on the Session's stream\n";

@@ -24,6 +24,7 @@ def all_specs(with_large=True):
     specs.append(models.qcnn_spec(oracle, 8))
     specs.append(models.qdq_conv_spec())
     specs.append(models.convbn_spec())
+    specs.append(models.functor_spec())
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs
@@ -34,6 +35,8 @@ def main():
     for spec in all_specs():
         hxx, dat, res = spec.generate()
         exe = spec.compile_runner()
+        if spec.name == "functor4":
+            emit.compile_example("run_functor.cxx", spec.name, "run_functor")
         if spec.name == "qcnn_b4096":
             os.remove(dat)      # same tensors as qcnn.dat: the runner is pointed at that file
         print("%-28s %s" % (spec.name, res.stdout.strip().split(", ")[-1]))

@@ -264,3 +264,29 @@ def convbn_reference(oracle):
     p1 = oracle.maxpool2d(r1, (2, 2), (2, 2))
     n2 = oracle.batchnorm_f32(p1, p["g2"], p["beta2"], p["mean2"], p["var2"], 1e-3)
     return oracle.conv_transpose2d_f32(n2, p["wt"], p["bt"], (1, 1, 1, 1), (2, 2), relu=True)
+
+
+# ------------------------------------------------------------------------------------------ four-value model for SofieFunctor
+def functor_params(seed=33):
+    r = np.random.default_rng(seed)
+    return {"W1": r.standard_normal((4, 8)).astype(np.float32), "B1": r.standard_normal(8).astype(np.float32),
+            "W2": r.standard_normal((8, 1)).astype(np.float32), "B2": r.standard_normal(1).astype(np.float32),
+            "rows": r.standard_normal((64, 4)).astype(np.float32)}
+
+
+def functor_spec(name="functor4"):
+    p = functor_params()
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", (1, 4))
+    for k in ("W1", "B1", "W2", "B2"):
+        s.add_init(k, p[k])
+    s.gemm("x", "W1", "B1", "h", relu=True)
+    s.gemm("h", "W2", "B2", "y")
+    s.set_output("y")
+    return s
+
+
+def functor_reference(oracle):
+    p = functor_params()
+    h = oracle.gemm_f32(p["rows"], p["W1"], p["B1"], relu=True)
+    return oracle.gemm_f32(h, p["W2"], p["B2"]).reshape(-1)

@@ -76,6 +76,25 @@ def test_conv_batchnorm_convtranspose_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
+def test_sofie_functor_slots_from_threads(tmp_path):
+    """SofieFunctor<4, Session> with three slots, each called from its own thread (one device context and stream
+    per Session): every row equals the oracle's two-layer network, and one slot gives the same numbers."""
+    p = models.functor_params()
+    ref = models.functor_reference(oracle)
+    fin = str(tmp_path / "rows.bin")
+    p["rows"].tofile(fin)
+    exe = os.path.join(emit.GEN_DIR, "run_functor")
+    outs = []
+    for slots in (3, 0):
+        fout = str(tmp_path / ("out%d.bin" % slots))
+        res = subprocess.run([exe, os.path.join(emit.GEN_DIR, "functor4.dat"), str(slots), fin, fout], stdout=subprocess.PIPE,
+                             stderr=subprocess.PIPE, text=True, timeout=110)
+        assert res.returncode == 0, res.stderr
+        outs.append(np.fromfile(fout, np.float64))
+    assert outs[0].size == ref.size and np.array_equal(outs[0], outs[1])
+    assert rel_err(outs[0], ref) <= 1e-5
+
+
 def test_int8_cnn_session_is_bit_exact(tmp_path):
     x = models.cnn_input(8)
     y = run_session("qcnn", x, tmp_path)
