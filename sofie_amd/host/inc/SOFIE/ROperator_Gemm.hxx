@@ -33,6 +33,9 @@ private:
    EActivationType fActivation = EActivationType::UNDEFINED;
    std::vector<size_t> fShapeA, fShapeB, fShapeC, fShapeY;
    int fBiasKind = 0;   // SOFIE_BIAS_*
+   size_t fStack = 1;                       // stacked products (numpy.matmul on rank > 2 operands)
+   std::vector<size_t> fStackA, fStackB;    // matrix index of A and B for every stacked product
+   std::vector<size_t> fLeadY;              // leading dimensions of Y
 
 public:
    ROperator_Gemm() {}
@@ -73,10 +76,25 @@ public:
          if (i.size() < 2)
             throw std::runtime_error("TMVA SOFIE Gemm Op Shape Inference only accept input tensor with >=2 dimensions");
       if (input.size() == 3) return {input[2]};   // with three inputs the shape of Y is the shape of C
-      std::vector<size_t> a = input[0], b = input[1];
+      // the last two dimensions multiply; leading dimensions of stacked operands broadcast against each other
+      // (reference :93-122, numpy.matmul)
+      const size_t ra = input[0].size(), rb = input[1].size();
+      std::vector<size_t> a(input[0].end() - 2, input[0].end()), b(input[1].end() - 2, input[1].end());
       if (fAttrTransA) std::reverse(a.begin(), a.end());
       if (fAttrTransB) std::reverse(b.begin(), b.end());
-      return {{a[0], b[1]}};
+      std::vector<size_t> y;
+      const size_t lead = std::max(ra, rb) - 2;
+      for (size_t i = 0; i < lead; ++i) {
+         const size_t da = i + ra >= lead + 2 ? input[0][i + ra - lead - 2] : 1;
+         const size_t db = i + rb >= lead + 2 ? input[1][i + rb - lead - 2] : 1;
+         if (da != db && da != 1 && db != 1)
+            throw std::runtime_error("TMVA SOFIE Gemm Op - invalid input shapes " + std::to_string(da) + " and " +
+                                     std::to_string(db));
+         y.push_back(da == 1 ? db : da);
+      }
+      y.push_back(a[0]);
+      y.push_back(b[1]);
+      return {y};
    }
 
    void Initialize(RModel &model) override
@@ -91,8 +109,38 @@ public:
       bool prependOne = false, appendOne = false;
       if (fShapeA.size() == 1) { fShapeA.insert(fShapeA.begin(), 1); prependOne = true; }
       if (fShapeB.size() == 1) { fShapeB.push_back(1); appendOne = true; }
-      if (fShapeA.size() != 2 || fShapeB.size() != 2)
-         throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + ": stacked (rank > 2) MatMul is not supported by the device emission");
+      // Stacked operands (rank > 2, numpy.matmul): the shorter shape gets leading ones (reference :180-187), the
+      // leading dimensions broadcast, and the emitted code runs one product per stacked matrix. The reference
+      // loops over the stack too (:353-387) but hands every iteration the first matrices of A and B; here each
+      // product reads its own.
+      std::vector<size_t> fullY = ShapeInference({fShapeA, fShapeB})[0];
+      {
+         const size_t rank = fullY.size();
+         std::vector<size_t> la(fShapeA), lb(fShapeB);
+         la.insert(la.begin(), rank - la.size(), 1);
+         lb.insert(lb.begin(), rank - lb.size(), 1);
+         fStack = 1;
+         fStackA.clear();
+         fStackB.clear();
+         // offsets (in matrices) of A and B for every stacked product, row-major over the leading dimensions
+         for (size_t i = 0; i + 2 < rank; ++i) fStack *= fullY[i];
+         for (size_t idx = 0; idx < fStack; ++idx) {
+            size_t rem = idx, oa = 0, ob = 0, sa = 1, sb = 1;
+            for (size_t i = rank - 2; i-- > 0;) {
+               const size_t pos = rem % fullY[i];
+               rem /= fullY[i];
+               if (la[i] != 1) oa += pos * sa;
+               if (lb[i] != 1) ob += pos * sb;
+               sa *= la[i];
+               sb *= lb[i];
+            }
+            fStackA.push_back(oa);
+            fStackB.push_back(ob);
+         }
+         fShapeA.assign(la.end() - 2, la.end());
+         fShapeB.assign(lb.end() - 2, lb.end());
+         fLeadY.assign(fullY.begin(), fullY.end() - 2);
+      }
       std::vector<size_t> a = fShapeA, b = fShapeB;
       if (fAttrTransA) std::reverse(a.begin(), a.end());
       if (fAttrTransB) std::reverse(b.begin(), b.end());
@@ -100,6 +148,8 @@ public:
          throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + " has invalid shape" + ConvertShapeToString(fShapeA) + " x " +
                                   ConvertShapeToString(fShapeB));
       fShapeY = {a[0], b[1]};
+      if (fStack > 1 && fNC != "")
+         throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + ": a bias on stacked operands is not supported by the device emission");
       if (model.GetTensorType(fNA) != ETensorType::FLOAT || model.GetTensorType(fNB) != ETensorType::FLOAT)
          throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + ": only float tensors are supported");
       if (fNC != "") {
@@ -122,8 +172,9 @@ public:
             throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + " Bias tensor has not correct size " +
                                      ConvertShapeToString(fShapeC) + " output shape " + ConvertShapeToString(fShapeY));
       }
-      std::vector<size_t> shapeY = fShapeY;
-      if (prependOne) shapeY.erase(shapeY.begin());
+      std::vector<size_t> shapeY = fLeadY;
+      shapeY.insert(shapeY.end(), fShapeY.begin(), fShapeY.end());
+      if (prependOne) shapeY.erase(shapeY.end() - 2);
       if (appendOne) shapeY.pop_back();
       model.AddIntermediateTensor(fNY, model.GetTensorType(fNA), shapeY);
       model.AddNeededStdLib("algorithm");
@@ -140,11 +191,29 @@ public:
       const size_t k = fAttrTransA ? fShapeA[0] : fShapeA[1];
       std::stringstream out;
       out << "\n//--------- Gemm\n";
-      out << SP << "Check(sofie_hip_gemm_f32(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << m << ", "
-          << n << ", " << k << ", " << FloatLiteral(fAttrAlpha) << ", tensor_" << fNA << ", " << fShapeA[1] << ", tensor_" << fNB
-          << ", " << fShapeB[1] << ", " << FloatLiteral(fNC.empty() ? 0.0f : fAttrBeta) << ", "
-          << (fNC.empty() ? std::string("nullptr") : "tensor_" + fNC) << ", " << fBiasKind << ", tensor_" << fNY << ", " << n << ", "
+      std::string offA, offB, offY, indent = SP;
+      if (fStack > 1) {
+         // one product per stacked matrix; the tables hold the matrix index of A and B (broadcast dimensions repeat)
+         const size_t lenA = fShapeA[0] * fShapeA[1], lenB = fShapeB[0] * fShapeB[1];
+         out << SP << "{\n";
+         out << SP << SP << "static const size_t " << opName << "_a[] = {";
+         for (size_t i = 0; i < fStack; ++i) out << (i ? ", " : "") << fStackA[i] * lenA;
+         out << "};\n";
+         out << SP << SP << "static const size_t " << opName << "_b[] = {";
+         for (size_t i = 0; i < fStack; ++i) out << (i ? ", " : "") << fStackB[i] * lenB;
+         out << "};\n";
+         out << SP << SP << "for (size_t i = 0; i < " << fStack << "; i++)\n";
+         offA = " + " + opName + "_a[i]";
+         offB = " + " + opName + "_b[i]";
+         offY = " + i * " + std::to_string(m * n);
+         indent = SP + SP + SP;
+      }
+      out << indent << "Check(sofie_hip_gemm_f32(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << m << ", "
+          << n << ", " << k << ", " << FloatLiteral(fAttrAlpha) << ", tensor_" << fNA << offA << ", " << fShapeA[1] << ", tensor_" << fNB
+          << offB << ", " << fShapeB[1] << ", " << FloatLiteral(fNC.empty() ? 0.0f : fAttrBeta) << ", "
+          << (fNC.empty() ? std::string("nullptr") : "tensor_" + fNC) << ", " << fBiasKind << ", tensor_" << fNY << offY << ", " << n << ", "
           << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << "), \"Gemm " << opName << "\");\n";
+      if (fStack > 1) out << SP << "}\n";
       return out.str();
    }
 };

@@ -25,6 +25,7 @@ def all_specs(with_large=True):
     specs.append(models.qdq_conv_spec())
     specs.append(models.convbn_spec())
     specs.append(models.functor_spec())
+    specs.append(models.stacked_spec())
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs

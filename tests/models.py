@@ -290,3 +290,29 @@ def functor_reference(oracle):
     p = functor_params()
     h = oracle.gemm_f32(p["rows"], p["W1"], p["B1"], relu=True)
     return oracle.gemm_f32(h, p["W2"], p["B2"]).reshape(-1)
+
+
+# ------------------------------------------------------------------------------------------ stacked MatMul
+def stacked_params(seed=44):
+    r = np.random.default_rng(seed)
+    return {"x": r.standard_normal((2, 1, 4, 5)).astype(np.float32), "B1": r.standard_normal((3, 5, 6)).astype(np.float32),
+            "B2": r.standard_normal((6, 2)).astype(np.float32)}
+
+
+def stacked_spec(name="stacked"):
+    """x [2,1,4,5] @ B1 [3,5,6] -> [2,3,4,6] (both operands broadcast over a leading dimension), then @ B2 [6,2]
+    -> [2,3,4,2] (a plain matrix against a stack)."""
+    p = stacked_params()
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", p["x"].shape)
+    s.add_init("B1", p["B1"])
+    s.add_init("B2", p["B2"])
+    s.gemm("x", "B1", None, "h", 1.0, 0.0)
+    s.gemm("h", "B2", None, "y", 1.0, 0.0)
+    s.set_output("y")
+    return s
+
+
+def stacked_reference():
+    p = stacked_params()
+    return np.matmul(np.matmul(p["x"].astype(np.float64), p["B1"].astype(np.float64)), p["B2"].astype(np.float64))

@@ -353,6 +353,24 @@ def test_parametric_batch_dimension_is_fixed_at_generation_time(tmp_path):
         assert res.returncode != 0 and "parametric shape" in res.stderr and "pass the batch size" in res.stderr
 
 
+def test_stacked_matmul_shapes_and_offsets(tmp_path):
+    """Leading dimensions broadcast as in numpy.matmul; the emitted loop indexes A and B per stacked product."""
+    hxx, _, _ = models.stacked_spec("stacked_t").generate(str(tmp_path))
+    code = open(hxx).read()
+    # x [2,1,4,5] @ B1 [3,5,6]: six products; A advances with the first dimension only, B with the second only
+    assert "_a[] = {0, 0, 0, 20, 20, 20};" in code and "_b[] = {0, 30, 60, 0, 30, 60};" in code
+    # h [2,3,4,6] @ B2 [6,2]: B is one matrix
+    assert "_a[] = {0, 24, 48, 72, 96, 120};" in code and "_b[] = {0, 0, 0, 0, 0, 0};" in code
+    assert code.count("sofie_hip_gemm_f32(") == 2
+    bad = emit.ModelSpec("bad_stack")
+    bad.add_input("x", "FLOAT", (2, 4, 5))
+    bad.add_init("B", np.zeros((3, 5, 6), np.float32))
+    bad.gemm("x", "B", None, "y", 1.0, 0.0)
+    bad.set_output("y")
+    with pytest.raises(RuntimeError, match="invalid input shapes 2 and 3"):
+        bad.generate(str(tmp_path))
+
+
 def test_every_prebuilt_session_compiles():
     """tests/build_generated.py output (made by build()): header, weights and runner of each network."""
     import build_generated

@@ -76,6 +76,16 @@ def test_conv_batchnorm_convtranspose_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
+def test_stacked_matmul_session(tmp_path):
+    """MatMul on stacked operands (numpy.matmul broadcasting of the leading dimensions): every product reads its
+    own matrices; against the float64 product, 1e-5 relative."""
+    p = models.stacked_params()
+    y = run_session("stacked", p["x"], tmp_path)
+    ref = models.stacked_reference()
+    assert y.size == ref.size
+    assert rel_err(y, ref.reshape(-1)) <= 1e-5
+
+
 def test_sofie_functor_slots_from_threads(tmp_path):
     """SofieFunctor<4, Session> with three slots, each called from its own thread (one device context and stream
     per Session): every row equals the oracle's two-layer network, and one slot gives the same numbers."""
