@@ -86,6 +86,19 @@ int sofie_hip_copy(sofie_hip_ctx *ctx, void *dst_device, const void *src_device,
 int sofie_hip_memset(sofie_hip_ctx *ctx, void *dptr, int byte_value, size_t bytes);
 int sofie_hip_sync(sofie_hip_ctx *ctx);
 
+/* HIP graph of a fixed call sequence. Between capture_begin and capture_end the calls made on the context are
+ * recorded instead of run; graph_launch replays them with one launch (a launch-bound chain of small kernels, such
+ * as a small MLP, then costs one submission instead of one per operator). The recorded calls keep their
+ * pointer arguments. Nothing may allocate while recording: run the sequence once eagerly first, so that the
+ * context's scratch buffer has its final size (a call that would grow it fails with a message saying so).
+ * Uploads, downloads, memset and sync are not to be called between begin and end. capture_end with a NULL result
+ * pointer abandons the recording. No counterpart in the reference (its generated code is a CPU call sequence). */
+typedef struct sofie_hip_graph sofie_hip_graph;
+int sofie_hip_capture_begin(sofie_hip_ctx *ctx);
+int sofie_hip_capture_end(sofie_hip_ctx *ctx, sofie_hip_graph **graph);
+int sofie_hip_graph_launch(sofie_hip_ctx *ctx, sofie_hip_graph *graph);
+int sofie_hip_graph_destroy(sofie_hip_ctx *ctx, sofie_hip_graph *graph);
+
 /* Event timing on the context's stream: start, enqueue work, stop (synchronises). */
 int sofie_hip_timer_start(sofie_hip_ctx *ctx);
 int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *elapsed_ms);

@@ -15,6 +15,7 @@ struct sofie_hip_ctx {
    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
    void *workspace = nullptr;   // scratch owned by the context (layout changes, B transposes)
    size_t workspace_bytes = 0;
+   bool capturing = false;      // between sofie_hip_capture_begin and _end: nothing may allocate or synchronise
    char err[512] = {0};
 };
 

@@ -19,6 +19,9 @@ int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...)
 int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr)
 {
    if (bytes > ctx->workspace_bytes) {
+      if (ctx->capturing)
+         return set_error(ctx, SOFIE_HIP_EINVAL, "the scratch buffer would grow to %zu bytes while a graph is captured: "
+                          "run the same calls once before capturing", bytes);
       // the old buffer may still be read by kernels in flight on the stream
       if (ctx->workspace) {
          SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
@@ -158,6 +161,67 @@ int sofie_hip_sync(sofie_hip_ctx *ctx)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
    SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+// ---- HIP graphs: a fixed sequence of calls recorded once and replayed with one launch -----------------------
+struct sofie_hip_graph {
+   hipGraph_t graph = nullptr;
+   hipGraphExec_t exec = nullptr;
+};
+
+int sofie_hip_capture_begin(sofie_hip_ctx *ctx)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "a capture is already open on this context");
+   SOFIE_HIP_CALL(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+   ctx->capturing = true;
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_capture_end(sofie_hip_ctx *ctx, sofie_hip_graph **out)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, ctx->capturing, "no capture is open on this context");
+   ctx->capturing = false;
+   hipGraph_t graph = nullptr;
+   SOFIE_HIP_CALL(ctx, hipStreamEndCapture(ctx->stream, &graph));
+   if (!out) {   // the caller gives the recording up (an error in between)
+      if (graph) (void)hipGraphDestroy(graph);
+      return SOFIE_HIP_OK;
+   }
+   *out = nullptr;
+   SOFIE_REQUIRE(ctx, graph != nullptr, "the capture recorded nothing");
+   hipGraphExec_t exec = nullptr;
+   if (hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0) != hipSuccess) {
+      (void)hipGetLastError();
+      (void)hipGraphDestroy(graph);
+      return sofie::set_error(ctx, SOFIE_HIP_EHIP, "hipGraphInstantiate failed");
+   }
+   sofie_hip_graph *g = new sofie_hip_graph();
+   g->graph = graph;
+   g->exec = exec;
+   *out = g;
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_graph_launch(sofie_hip_ctx *ctx, sofie_hip_graph *g)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, g && g->exec, "null graph");
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "a capture is open on this context");
+   SOFIE_HIP_CALL(ctx, hipGraphLaunch(g->exec, ctx->stream));
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_graph_destroy(sofie_hip_ctx *ctx, sofie_hip_graph *g)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (!g) return SOFIE_HIP_OK;
+   (void)hipStreamSynchronize(ctx->stream);
+   if (g->exec) (void)hipGraphExecDestroy(g->exec);
+   if (g->graph) (void)hipGraphDestroy(g->graph);
+   delete g;
    return SOFIE_HIP_OK;
 }
 

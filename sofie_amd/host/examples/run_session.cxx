@@ -3,6 +3,7 @@
 //   run_session <weights.dat> <input.bin> <output.bin> [timed iterations of infer_device]
 #include <chrono>
 #include <cstdio>
+#include <cstring>
 #include <fstream>
 #include <iostream>
 #include <vector>
@@ -38,7 +39,23 @@ int main(int argc, char **argv)
          auto t0 = std::chrono::steady_clock::now();
          for (int i = 0; i < iters; ++i) y = s.infer(x.data());
          const double host_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
-         std::printf("{\"device_ms\": %.6f, \"host_ms\": %.6f, \"iters\": %d}\n", ms / iters, host_ms / iters, iters);
+         // the same sequence replayed from a HIP graph: outputs must not change, timing of back-to-back replays
+         s.use_graph(true);
+         std::vector<SOFIE_OUT_T> yg = s.infer(x.data());
+         bool same = yg.size() == y.size();
+         for (int rep = 0; rep < 3 && same; ++rep) {
+            s.infer_device(s.SOFIE_INPUT_MEMBER);   // eager work and a synchronisation between replays
+            s.sync();
+            yg = s.infer(x.data());
+            for (size_t i = 0; i < y.size() && same; ++i) same = std::memcmp(&yg[i], &y[i], sizeof(SOFIE_OUT_T)) == 0;
+         }
+         s.sync();
+         float gms = 0;
+         sofie_hip_timer_start(s.fCtx);
+         for (int i = 0; i < iters; ++i) s.run_own_input();
+         sofie_hip_timer_stop(s.fCtx, &gms);
+         std::printf("{\"device_ms\": %.6f, \"host_ms\": %.6f, \"graph_ms\": %.6f, \"graph_matches\": %s, \"iters\": %d}\n", ms / iters,
+                     host_ms / iters, gms / iters, same ? "true" : "false", iters);
       }
    } catch (const std::exception &e) {
       std::cerr << "run_session: " << e.what() << "\n";

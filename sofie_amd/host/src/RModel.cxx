@@ -560,6 +560,8 @@ void RModel::GenerateSessionCode()
    fGC += "   operator sofie_hip_ctx*() const { return p; }\n";
    fGC += "};\n";
    fGC += "CtxHandle fCtx;\n";
+   fGC += "sofie_hip_graph* fGraph = nullptr;   // the operator sequence on the Session's own input buffer, recorded once\n";
+   fGC += "bool fUseGraph = false;\n";
    fGC += "static void Check(sofie_hip_ctx* ctx, int status, const char* what) {\n";
    fGC += "   if (status != 0) throw std::runtime_error(std::string(\"TMVA SOFIE device error in \") + what + \": \" + "
           "sofie_hip_last_error(ctx));\n";
@@ -658,6 +660,8 @@ void RModel::GenerateSessionCode()
    // ---- destructor (the reference's Session leaks its pool; device memory must not)
    fGC += "void Release() {\n";
    fGC += "   if (!fCtx) return;\n";
+   fGC += "   sofie_hip_graph_destroy(fCtx, fGraph);\n";
+   fGC += "   fGraph = nullptr;\n";
    for (auto &i : fInitializedTensors)
       if (i.second.IsWeightTensor()) fGC += "   sofie_hip_free(fCtx, tensor_" + i.first + ");\n";
    for (auto &n : fInputTensorNames) fGC += "   sofie_hip_free(fCtx, fInput_" + n + ");\n";
@@ -693,6 +697,27 @@ void RModel::GenerateSessionCode()
    const std::string otype = ConvertTypeToString(GetTensorType(out));
    const size_t olen = ConvertShapeToLength(GetTensorShape(out));
 
+   // ---- the sequence on the Session's own input buffer, optionally replayed from a HIP graph
+   {
+      std::string own;
+      int k = 0;
+      for (auto &n : fInputTensorNames) own += std::string(k++ ? ", " : "") + "fInput_" + n;
+      fGC += "// use_graph(true): infer() replays the operator sequence from a HIP graph recorded at the first call (one\n";
+      fGC += "// submission instead of one per operator; worth it for chains of small kernels). The first call runs the\n";
+      fGC += "// sequence once eagerly, so that nothing allocates while it is recorded.\n";
+      fGC += "void use_graph(bool on = true) { fUseGraph = on; }\n";
+      fGC += "void run_own_input() {\n";
+      fGC += "   if (!fUseGraph) { run_device(" + own + "); return; }\n";
+      fGC += "   if (!fGraph) {\n";
+      fGC += "      run_device(" + own + ");\n";
+      fGC += "      Check(sofie_hip_capture_begin(fCtx), \"graph capture\");\n";
+      fGC += "      try { run_device(" + own + "); } catch (...) { sofie_hip_capture_end(fCtx, nullptr); throw; }\n";
+      fGC += "      Check(sofie_hip_capture_end(fCtx, &fGraph), \"graph capture\");\n";
+      fGC += "   }\n";
+      fGC += "   Check(sofie_hip_graph_launch(fCtx, fGraph), \"graph launch\");\n";
+      fGC += "}\n\n";
+   }
+
    // ---- infer on host pointers: same signature and return convention as the reference
    // (RModel.cxx:680-801): one upload, the kernel sequence, one download
    fGC += "std::vector<" + otype + "> infer(" + GenerateInferSignature(true) + "){\n";
@@ -700,12 +725,7 @@ void RModel::GenerateSessionCode()
       const size_t bytes = ConvertShapeToLength(GetTensorShape(n)) * GetTypeSize(GetTensorType(n));
       fGC += "   Check(sofie_hip_upload(fCtx, fInput_" + n + ", tensor_" + n + ", " + std::to_string(bytes) + "), \"input upload\");\n";
    }
-   fGC += "   run_device(";
-   {
-      int k = 0;
-      for (auto &n : fInputTensorNames) fGC += std::string(k++ ? ", " : "") + "fInput_" + n;
-   }
-   fGC += ");\n";
+   fGC += "   run_own_input();\n";
    fGC += "   std::vector<" + otype + "> ret(" + std::to_string(olen) + ");\n";
    fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", " + std::to_string(olen) + " * sizeof(" + otype +
           ")), \"output download\");\n";

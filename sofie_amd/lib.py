@@ -35,6 +35,10 @@ SIGNATURES = {
     "sofie_hip_gemm_f32": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i, _p, _i, _i],
     "sofie_hip_conv2d_f32": [_p, _p, _p, _p, _p] + [_i] * 15,
     "sofie_hip_conv_transpose2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,
+    "sofie_hip_capture_begin": [_p],
+    "sofie_hip_capture_end": [_p, _p],
+    "sofie_hip_graph_launch": [_p, _p],
+    "sofie_hip_graph_destroy": [_p, _p],
     "sofie_hip_batchnorm_f32": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i],
     "sofie_hip_relu_f32": [_p, _p, _p, _z],
     "sofie_hip_maxpool2d_f32": [_p, _p, _p] + [_i] * 11,

@@ -76,6 +76,18 @@ def test_conv_batchnorm_convtranspose_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
+@pytest.mark.parametrize("name,make_input", [
+    ("mlp_c1", lambda: models.mlp_spec()[1]), ("cnn_f32", lambda: models.cnn_input(8)), ("qcnn", lambda: models.cnn_input(8)),
+    ("qdq_conv", lambda: models.qdq_conv_params()["x"]), ("convbn", lambda: models.convbn_params()["x"]),
+    ("stacked", lambda: models.stacked_params()["x"])])
+def test_graph_replay_matches_eager(name, make_input, tmp_path):
+    """Session::use_graph: the operator sequence recorded into a HIP graph at the first infer() and replayed afterwards
+    gives the same bytes as the eager sequence, on four replays with eager runs and synchronisations in between."""
+    _, timing = run_session(name, make_input(), tmp_path, iters=5)
+    assert timing["graph_matches"] is True
+    assert timing["graph_ms"] > 0
+
+
 def test_stacked_matmul_session(tmp_path):
     """MatMul on stacked operands (numpy.matmul broadcasting of the leading dimensions): every product reads its
     own matrices; against the float64 product, 1e-5 relative."""
