@@ -129,6 +129,7 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 
    stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
    const bool plain = OUT == SOFIE_OUT_S8 && a.ep.zp == -128 && a.ep.lo == -128;
+   bool any_negative = false;   // pooled variant: some scale of the workgroup's channels is negative (set below)
 
    // ---- band loader: thread -> (row of the pass, 16-byte chunk of the row)
    const int rsub = fdiv(tid, a.dRL);
@@ -225,18 +226,6 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    // step's matrix instructions, which saves copying it into every accumulator of every tile.
    v16i r_bias[POOL ? 1 : NB];
    auto kloop = [&](v16i (&acc)[NB][MB]) {
-      if constexpr (POOL) {
-#pragma unroll
-         for (int i = 0; i < NB; ++i)
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-               const v4i bi = *reinterpret_cast<const v4i *>(w_bias + i * 32 + q * 8 + nq);
-#pragma unroll
-               for (int j = 0; j < MB; ++j)
-#pragma unroll
-                  for (int e = 0; e < 4; ++e) acc[i][j][q * 4 + e] = bi[e];
-            }
-      }
       v4i fa[POOL ? 2 : 3][MB], fb[POOL ? 2 : 3][NB];
       int ka = 0, kb = 0, c32 = 0, kw = 0;
       auto advance = [&]() {
@@ -290,18 +279,31 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          if (s < nsteps) mma(1);
          if (s + 1 < nsteps) mma(2);
       } else {
-         // the pooled variant has twice the accumulators and keeps two fragment buffers
+         // the pooled variant has twice the accumulators and keeps two fragment buffers. Step 0 starts from a
+         // constant zero C operand (no accumulator is initialised); the bias is added to the pooled values, a
+         // quarter as many (max(a + b) = max(a) + b)
          load(0, true);
-         int s = 0;
+         advance();
+         load(1, nsteps > 1);
+         {
+            v16i zero;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) zero[e] = 0;
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+               for (int j = 0; j < MB; ++j) acc[i][j] = MmaI8::mma(fb[0][i], fa[0][j], zero);
+         }
+         int s = 1;   // step s sits in buffer 1
          for (; s + 1 < nsteps; s += 2) {
             advance();
-            load(1, true);
-            mma(0);
-            advance();
-            load(0, s + 2 < nsteps);
+            load(0, true);
             mma(1);
+            advance();
+            load(1, s + 2 < nsteps);
+            mma(0);
          }
-         if (s < nsteps) mma(0);
+         if (s < nsteps) mma(1);
       }
    };
    // the lane's scales, loaded once (after the first barrier); the pooled variant needs the registers for
@@ -311,22 +313,31 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
       const int m_wave = tt * TM + wm * MBP * 32, n_wave = ob * OCT + wn * NB * 32;
       if constexpr (POOL) {
          v16i pooled[NB][1];
+         if (!any_negative) {
 #pragma unroll
-         for (int i = 0; i < NB; ++i)
+            for (int i = 0; i < NB; ++i)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-               const v4f sc = *reinterpret_cast<const v4f *>(w_scale + i * 32 + q * 8 + nq);
+               for (int e = 0; e < 16; ++e)
+                  pooled[i][0][e] = max(max(acc[i][0][e], acc[i][1][e]), max(acc[i][2][e], acc[i][3][e]));
+         } else {
+            // a negative scale turns the order around: those channels take the minimum
 #pragma unroll
-               for (int t = 0; t < 4; ++t) {
-                  const int e = q * 4 + t;
-                  const int hi = max(max(acc[i][0][e], acc[i][1][e]), max(acc[i][2][e], acc[i][3][e]));
-                  const int lo = min(min(acc[i][0][e], acc[i][1][e]), min(acc[i][2][e], acc[i][3][e]));
-                  pooled[i][0][e] = sc[t] < 0.0f ? lo : hi;
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+               for (int q = 0; q < 4; ++q) {
+                  const v4f sc = *reinterpret_cast<const v4f *>(w_scale + i * 32 + q * 8 + nq);
+#pragma unroll
+                  for (int t = 0; t < 4; ++t) {
+                     const int e = q * 4 + t;
+                     const int hi = max(max(acc[i][0][e], acc[i][1][e]), max(acc[i][2][e], acc[i][3][e]));
+                     const int lo = min(min(acc[i][0][e], acc[i][1][e]), min(acc[i][2][e], acc[i][3][e]));
+                     pooled[i][0][e] = sc[t] < 0.0f ? lo : hi;
+                  }
                }
-            }
+         }
          if constexpr (OUT == SOFIE_OUT_S8) {
-            if (plain) tile_epilogue_s8_direct<NB, 1, true, false>(a.ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
-            else tile_epilogue_s8_direct<NB, 1, false, false>(a.ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+            if (plain) tile_epilogue_s8_direct<NB, 1, true, true>(a.ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+            else tile_epilogue_s8_direct<NB, 1, false, true>(a.ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
          }
       } else if constexpr (OUT == SOFIE_OUT_S8) {
          if (plain) tile_epilogue_s8_direct<NB, MB, true, false>(a.ep, acc, w_scale, w_bias, lane, m_wave, n_wave, &r_scale);
@@ -351,7 +362,14 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
       fetch(cur);
       pixel_offsets(t, cur.vr_lo);
    }
-   __syncthreads();   // weights and column parameters are in LDS
+   // weights and column parameters are in LDS; the pooled variant also learns whether any scale of the
+   // workgroup's channels is negative (uniform, so the common case pools with a maximum only)
+   __syncthreads();
+   if constexpr (POOL) {
+      int neg = 0;
+      for (int c = tid; c < OCT; c += 512) neg |= s_scale[c] < 0.0f;
+      any_negative = __syncthreads_or(neg) != 0;
+   }
    if constexpr (!POOL) {
 #pragma unroll
       for (int gi = 0; gi < NB * 4; ++gi) {
