@@ -111,7 +111,7 @@ class ModelSpec:
         self.lines.append("op GemmFP8 %s %s %s %s %s %s %d" % (a, a_scale, b, b_scale, bias or "-", y, transB))
 
     # ---- generation ------------------------------------------------------------------------
-    def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True):
+    def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False):
         """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess)."""
         os.makedirs(outdir, exist_ok=True)
         tdir = os.path.join(outdir, "tensors")
@@ -120,7 +120,8 @@ class ModelSpec:
             arr.tofile(os.path.join(tdir, fname))
         spec = os.path.join(outdir, self.name + ".spec")
         with open(spec, "w") as f:
-            f.write("\n".join(self.lines + ["generate" + (" noweightfile" if no_weight_file else "")]) + "\n")
+            flag = " noweightfile" if no_weight_file else (" binaryweightfile" if binary_weight_file else "")
+            f.write("\n".join(self.lines + ["generate" + flag]) + "\n")
         if not os.path.exists(EMIT):
             build_emitter()
         res = subprocess.run([EMIT, spec, tdir, outdir], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
@@ -128,7 +129,8 @@ class ModelSpec:
             raise RuntimeError("emitter failed: " + res.stderr)
         for fname in self.tensors:
             os.remove(os.path.join(tdir, fname))
-        return os.path.join(outdir, self.name + ".hxx"), os.path.join(outdir, self.name + ".dat"), res
+        return (os.path.join(outdir, self.name + ".hxx"),
+                os.path.join(outdir, self.name + (".bin" if binary_weight_file else ".dat")), res)
 
     def compile_runner(self, outdir=GEN_DIR):
         """g++ the generic runner against the generated header and libsofie_hip.so."""

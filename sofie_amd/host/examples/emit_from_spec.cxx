@@ -172,6 +172,7 @@ int main(int argc, char **argv)
             std::string flag;
             in >> flag;
             if (flag == "noweightfile") model->Generate(Options::kNoWeightFile);
+            else if (flag == "binaryweightfile") model->Generate(Options::kBinaryWeightFile);
             else model->Generate();
             model->OutputGenerated(odir + "/" + name + ".hxx");
             std::cout << "generated " << odir << "/" << name << ".hxx, intermediate pool " << model->GetIntermediateMemorySize()

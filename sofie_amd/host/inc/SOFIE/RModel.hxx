@@ -28,11 +28,12 @@ enum class Options {
    kRootBinaryWeightFile = 0x4,  // not available (no ROOT)
    kGNN = 0x8,
    kGNNComponent = 0x10,
+   kBinaryWeightFile = 0x20,     // typed binary records in <name>.bin instead of the text <name>.dat (not in the reference)
 };
 std::underlying_type_t<Options> operator|(Options opA, Options opB);
 std::underlying_type_t<Options> operator|(std::underlying_type_t<Options> opA, Options opB);
 
-enum class WeightFileType { None, RootBinary, Text };
+enum class WeightFileType { None, RootBinary, Text, Binary };
 
 class RModel {
 public:
@@ -110,6 +111,8 @@ public:
    std::string ReturnGenerated() { return fGC; }
    void OutputGenerated(std::string filename = "", bool append = false);
    long WriteInitializedTensorsToFile(std::string filename = "");
+   long WriteInitializedTensorsToBinaryFile(std::string filename = "");
+   std::string GenerateWeightReaderHelpers();
    void ReadInitializedTensorsFromFile(long pos);
 
    const std::vector<std::string> &GetInputTensorNames() const { return fInputTensorNames; }

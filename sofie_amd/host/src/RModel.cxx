@@ -10,6 +10,7 @@
 #include "SOFIE/ROperator_Quantized.hxx"
 
 #include <cmath>
+#include <cstring>
 #include <fstream>
 #include <iomanip>
 #include <iostream>
@@ -444,7 +445,7 @@ void RModel::GenerateHeaderInfo(std::string &hgname)
    fGC += "#define " + hgname + "\n\n";
    for (auto &i : fNeededStdLib) fGC += "#include <" + i + ">\n";
    for (auto &i : fCustomOpHeaders) fGC += "#include \"" + i + "\"\n";
-   fGC += "#include <cstdint>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n";
+   fGC += "#include <cstdint>\n#include <cstring>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n";
    // the numerical library: a C ABI over device pointers instead of the reference's
    // extern "C" BLAS prototypes (RModel_Base.cxx:40-58)
    fGC += "#include \"sofie_hip.h\"\n";
@@ -465,50 +466,131 @@ std::string RModel::GenerateInferSignature(bool isdecl)
 
 void RModel::ReadInitializedTensorsFromFile(long /*pos*/)
 {
-   // Generated reader of the text weight file: "tensor_<name> <length>" then the values, with the
-   // reference's name and length checks (RModel.cxx:970-1018). Integer tensors use the same
-   // record layout (the reference silently skips every non-float tensor, :1150-1152).
+   // Generated reader of the weight file. Text: "tensor_<name> <length>" then the values, with the
+   // reference's name and length checks (RModel.cxx:970-1018); integer tensors use the same record layout
+   // (the reference silently skips every non-float tensor, :1150-1152). Binary (the file starts with
+   // "SOFIEBIN"): the same records as name, type and length fields followed by the raw little-endian values.
+   // The format is recognised from the file, so a Session takes either.
    bool any = false;
    for (auto &i : fInitializedTensors) any |= i.second.IsWeightTensor();
    if (!any) return;
    fGC += "   std::ifstream f;\n";
-   fGC += "   f.open(filename);\n";
+   fGC += "   f.open(filename, std::ios::binary);\n";
    fGC += "   if (!f.is_open()) {\n";
    fGC += "      throw std::runtime_error(\"tmva-sofie failed to open file \" + filename + \" for input weights\");\n";
    fGC += "   }\n";
-   fGC += "   std::string tensor_name;\n";
-   fGC += "   size_t length;\n";
+   fGC += "   const bool binary = IsBinaryWeightFile(f);\n";
    for (auto &i : fInitializedTensors) {
       if (!i.second.IsWeightTensor()) continue;
       const std::string tensor_name = "tensor_" + i.first;
       const std::string slength = std::to_string(ConvertShapeToLength(i.second.shape()));
       const std::string ctype = ConvertTypeToString(i.second.type());
-      const bool narrow = GetTypeSize(i.second.type()) == 1;   // read bytes through int, not char
-      fGC += "   f >> tensor_name >> length;\n";
-      fGC += "   if (tensor_name != \"" + tensor_name + "\" ) {\n";
-      fGC += "      std::string err_msg = \"TMVA-SOFIE failed to read the correct tensor name; expected name is " +
-             tensor_name + " , read \" + tensor_name;\n";
-      fGC += "      throw std::runtime_error(err_msg);\n";
-      fGC += "    }\n";
-      fGC += "   if (length != " + slength + ") {\n";
-      fGC += "      std::string err_msg = \"TMVA-SOFIE failed to read the correct tensor size; expected size is " + slength +
-             " , read \" + std::to_string(length) ;\n";
-      fGC += "      throw std::runtime_error(err_msg);\n";
-      fGC += "    }\n";
       fGC += "   {\n";
       fGC += "      std::vector<" + ctype + "> host(" + slength + ");\n";
-      if (narrow)
-         fGC += "      for (size_t i = 0; i < length; ++i) { int v; f >> v; host[i] = static_cast<" + ctype + ">(v); }\n";
-      else
-         fGC += "      for (size_t i = 0; i < length; ++i) f >> host[i];\n";
-      fGC += "      if (f.fail()) {\n";
-      fGC += "         throw std::runtime_error(\"TMVA-SOFIE failed to read the values for tensor " + tensor_name + "\");\n";
-      fGC += "      }\n";
-      fGC += "      Check(sofie_hip_upload(fCtx, " + tensor_name + ", host.data(), length * sizeof(" + ctype + ")), \"upload of " +
+      fGC += "      ReadTensor(f, binary, \"" + tensor_name + "\", " + slength + ", host.data());\n";
+      fGC += "      Check(sofie_hip_upload(fCtx, " + tensor_name + ", host.data(), " + slength + " * sizeof(" + ctype + ")), \"upload of " +
              tensor_name + "\");\n";
       fGC += "   }\n";
    }
    fGC += "   f.close();\n";
+}
+
+// Helpers of the generated Session that read one record of the weight file in either format.
+std::string RModel::GenerateWeightReaderHelpers()
+{
+   std::string g;
+   g += "static bool IsBinaryWeightFile(std::ifstream& f) {\n";
+   g += "   char magic[8] = {0};\n";
+   g += "   f.read(magic, 8);\n";
+   g += "   if (f.gcount() == 8 && std::memcmp(magic, \"SOFIEBIN\", 8) == 0) {\n";
+   g += "      uint32_t header[2] = {0, 0};   // format version, number of records\n";
+   g += "      f.read(reinterpret_cast<char*>(header), sizeof(header));\n";
+   g += "      if (f.fail() || header[0] != 1) throw std::runtime_error(\"TMVA-SOFIE binary weight file has an unknown version\");\n";
+   g += "      return true;\n";
+   g += "   }\n";
+   g += "   f.clear();\n";
+   g += "   f.seekg(0);\n";
+   g += "   return false;\n";
+   g += "}\n";
+   g += "template <typename T>\n";
+   g += "static void ReadTensor(std::ifstream& f, bool binary, const std::string& expected, size_t expected_length, T* host) {\n";
+   g += "   std::string tensor_name;\n";
+   g += "   size_t length = 0;\n";
+   g += "   if (binary) {\n";
+   g += "      uint32_t name_length = 0, type = 0;\n";
+   g += "      uint64_t count = 0;\n";
+   g += "      f.read(reinterpret_cast<char*>(&name_length), 4);\n";
+   g += "      if (f.fail() || name_length > 4096) throw std::runtime_error(\"TMVA-SOFIE failed to read the record of tensor \" + expected);\n";
+   g += "      tensor_name.resize(name_length);\n";
+   g += "      f.read(&tensor_name[0], name_length);\n";
+   g += "      f.read(reinterpret_cast<char*>(&type), 4);\n";
+   g += "      f.read(reinterpret_cast<char*>(&count), 8);\n";
+   g += "      length = count;\n";
+   g += "   } else {\n";
+   g += "      f >> tensor_name >> length;\n";
+   g += "   }\n";
+   g += "   if (tensor_name != expected) {\n";
+   g += "      std::string err_msg = \"TMVA-SOFIE failed to read the correct tensor name; expected name is \" + expected + \" , read \" + tensor_name;\n";
+   g += "      throw std::runtime_error(err_msg);\n";
+   g += "   }\n";
+   g += "   if (length != expected_length) {\n";
+   g += "      std::string err_msg = \"TMVA-SOFIE failed to read the correct tensor size; expected size is \" + std::to_string(expected_length) + \" , read \" + std::to_string(length);\n";
+   g += "      throw std::runtime_error(err_msg);\n";
+   g += "   }\n";
+   g += "   if (binary) {\n";
+   g += "      f.read(reinterpret_cast<char*>(host), length * sizeof(T));\n";
+   g += "      const size_t pad = (8 - (length * sizeof(T)) % 8) % 8;   // records are padded to 8 bytes\n";
+   g += "      f.ignore(pad);\n";
+   g += "   } else if (sizeof(T) == 1) {\n";
+   g += "      for (size_t i = 0; i < length; ++i) { int v; f >> v; host[i] = static_cast<T>(v); }   // bytes are written as numbers\n";
+   g += "   } else {\n";
+   g += "      for (size_t i = 0; i < length; ++i) f >> host[i];\n";
+   g += "   }\n";
+   g += "   if (f.fail()) {\n";
+   g += "      throw std::runtime_error(\"TMVA-SOFIE failed to read the values for tensor \" + expected);\n";
+   g += "   }\n";
+   g += "}\n";
+   return g;
+}
+
+// Binary weight file: "SOFIEBIN", u32 version (1), u32 record count, then per tensor u32 name length, the name
+// ("tensor_<name>"), u32 element type (ETensorType), u64 element count, the raw values, zero padding to 8 bytes.
+// Same order, names and subnormal flush as the text file.
+long RModel::WriteInitializedTensorsToBinaryFile(std::string filename)
+{
+   if (filename == "") filename = fName + ".bin";
+   std::ofstream f(filename, std::ios::binary);
+   if (!f.is_open()) throw std::runtime_error("tmva-sofie failed to open file " + filename + " for tensor weight data");
+   uint32_t count = 0;
+   for (auto &i : fInitializedTensors) count += i.second.IsWeightTensor() ? 1 : 0;
+   const uint32_t header[2] = {1, count};
+   f.write("SOFIEBIN", 8);
+   f.write(reinterpret_cast<const char *>(header), sizeof(header));
+   for (auto &i : fInitializedTensors) {
+      if (!i.second.IsWeightTensor()) continue;
+      const std::string name = "tensor_" + i.first;
+      const uint32_t name_length = (uint32_t)name.size(), type = (uint32_t)i.second.type();
+      const uint64_t length = ConvertShapeToLength(i.second.shape());
+      const size_t bytes = length * GetTypeSize(i.second.type());
+      f.write(reinterpret_cast<const char *>(&name_length), 4);
+      f.write(name.data(), name_length);
+      f.write(reinterpret_cast<const char *>(&type), 4);
+      f.write(reinterpret_cast<const char *>(&length), 8);
+      if (i.second.type() == ETensorType::FLOAT) {
+         std::vector<float> v(i.second.data<float>(), i.second.data<float>() + length);
+         for (auto &x : v)
+            if (x != 0. && std::abs(x) < std::numeric_limits<float>::min()) x = 0;
+         f.write(reinterpret_cast<const char *>(v.data()), bytes);
+      } else {
+         f.write(reinterpret_cast<const char *>(i.second.data<char>()), bytes);
+      }
+      const char zeros[8] = {0};
+      f.write(zeros, (8 - bytes % 8) % 8);
+      if (f.fail()) throw std::runtime_error("tmva-sofie failed to write tensor data to file for " + name);
+   }
+   long pos = f.tellp();
+   f.close();
+   return pos;
 }
 
 long RModel::WriteInitializedTensorsToFile(std::string filename)
@@ -567,6 +649,11 @@ void RModel::GenerateSessionCode()
           "sofie_hip_last_error(ctx));\n";
    fGC += "}\n";
    fGC += "void Check(int status, const char* what) { Check(fCtx, status, what); }\n";
+   {
+      bool any = false;
+      for (auto &i : fInitializedTensors) any |= i.second.IsWeightTensor();
+      if (any && fUseWeightFile) fGC += GenerateWeightReaderHelpers();
+   }
    // weights: device pointers, uploaded once in the constructor
    for (auto &i : fInitializedTensors) {
       if (!i.second.IsWeightTensor()) continue;   // folded into other tensors at generation time
@@ -585,7 +672,9 @@ void RModel::GenerateSessionCode()
    fGC += "\n";
 
    // ---- constructor
-   fGC += "Session(std::string filename =\"" + (fUseWeightFile ? fName + ".dat" : std::string("")) + "\", int device = 0) {\n";
+   fGC += "Session(std::string filename =\"" +
+          (fUseWeightFile ? fName + (fWeightFile == WeightFileType::Binary ? ".bin" : ".dat") : std::string("")) +
+          "\", int device = 0) {\n";
    fGC += "   { int status = sofie_hip_create(&fCtx.p, device, nullptr);\n";
    fGC += "     if (status != 0) throw std::runtime_error(\"TMVA SOFIE cannot create a device context\"); }\n";
    fGC += "   try {\n";
@@ -761,6 +850,8 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    if (static_cast<std::underlying_type_t<Options>>(Options::kNoWeightFile) & options) {
       fUseWeightFile = false;
       fWeightFile = WeightFileType::None;
+   } else if (static_cast<std::underlying_type_t<Options>>(Options::kBinaryWeightFile) & options) {
+      fWeightFile = WeightFileType::Binary;
    }
    (void)pos;
    Initialize(batchSize, verbose);
@@ -791,9 +882,11 @@ void RModel::OutputGenerated(std::string filename, bool append)
       // weight file next to the header, same stem (RModel.cxx:1290-1310)
       size_t p = filename.find(".hxx");
       std::string dat = filename;
-      if (p != std::string::npos) dat.replace(p, 4, ".dat");
-      else dat += ".dat";
-      WriteInitializedTensorsToFile(dat);
+      const bool binary = fWeightFile == WeightFileType::Binary;
+      if (p != std::string::npos) dat.replace(p, 4, binary ? ".bin" : ".dat");
+      else dat += binary ? ".bin" : ".dat";
+      if (binary) WriteInitializedTensorsToBinaryFile(dat);
+      else WriteInitializedTensorsToFile(dat);
    }
 }
 

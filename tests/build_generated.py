@@ -36,6 +36,13 @@ def main():
     for spec in all_specs():
         hxx, dat, res = spec.generate()
         exe = spec.compile_runner()
+        if spec.name == "convbn":
+            # the same tensors as typed binary records: the compiled runner reads either file
+            import shutil
+            sub = os.path.join(emit.GEN_DIR, "binary")
+            _, binf, _ = models.convbn_spec().generate(sub, binary_weight_file=True)
+            shutil.copyfile(binf, os.path.join(emit.GEN_DIR, "convbn.bin"))
+            shutil.rmtree(sub)
         if spec.name == "functor4":
             emit.compile_example("run_functor.cxx", spec.name, "run_functor")
         if spec.name == "qcnn_b4096":

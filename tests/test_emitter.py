@@ -371,6 +371,46 @@ def test_stacked_matmul_shapes_and_offsets(tmp_path):
         bad.generate(str(tmp_path))
 
 
+def test_binary_weight_file_holds_the_same_tensors(tmp_path):
+    """Options::kBinaryWeightFile: the .bin file carries the records of the .dat file (same names, order, lengths and
+    values, typed and raw) and the generated constructor defaults to it; its reader takes either format."""
+    import struct
+    spec = models.qdq_conv_spec("qdq_bin")
+    hxx_b, binf, _ = spec.generate(str(tmp_path), binary_weight_file=True)
+    sub = tmp_path / "text"
+    sub.mkdir()
+    hxx_t, dat, _ = models.qdq_conv_spec("qdq_bin").generate(str(sub))
+    assert 'Session(std::string filename ="qdq_bin.bin"' in open(hxx_b).read()
+    assert 'Session(std::string filename ="qdq_bin.dat"' in open(hxx_t).read()
+    # apart from that default the two headers are the same code: the reader recognises the format from the file
+    strip = lambda path: [l for l in _body(path) if "Session(std::string filename" not in l]
+    assert strip(hxx_b) == strip(hxx_t)
+    raw = open(binf, "rb").read()
+    assert raw[:8] == b"SOFIEBIN" and struct.unpack_from("<II", raw, 8)[0] == 1
+    count = struct.unpack_from("<II", raw, 8)[1]
+    lines = open(dat).read().split("\n")
+    text = {}
+    for i in range(0, len(lines) - 1, 2):
+        name, length = lines[i].split()
+        text[name] = (int(length), lines[i + 1].split())
+    assert count == len(text)
+    off, np_types = 16, {1: np.float32, 3: np.int8, 6: np.int32, 2: np.uint8}
+    order = []
+    for _ in range(count):
+        (nlen,) = struct.unpack_from("<I", raw, off)
+        name = raw[off + 4:off + 4 + nlen].decode()
+        type_code, length = struct.unpack_from("<IQ", raw, off + 4 + nlen)
+        off += 4 + nlen + 12
+        dt = np.dtype(np_types[type_code])
+        vals = np.frombuffer(raw, dt, length, off)
+        off += length * dt.itemsize
+        off += (8 - (length * dt.itemsize) % 8) % 8
+        assert text[name][0] == length
+        assert np.array_equal(vals, np.array(text[name][1], dtype=np.float64).astype(dt))
+        order.append(name)
+    assert off == len(raw) and order == [l.split()[0] for l in lines[0:-1:2]]
+
+
 def test_every_prebuilt_session_compiles():
     """tests/build_generated.py output (made by build()): header, weights and runner of each network."""
     import build_generated

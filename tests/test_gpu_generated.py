@@ -117,6 +117,18 @@ def test_sofie_functor_slots_from_threads(tmp_path):
     assert rel_err(outs[0], ref) <= 1e-5
 
 
+def test_binary_weight_file_gives_the_same_session(tmp_path):
+    """The Session built from the binary weight file computes the same bytes as the one built from the text file."""
+    p = models.convbn_params()
+    y_text = run_session("convbn", p["x"], tmp_path)
+    exe = os.path.join(emit.GEN_DIR, "run_convbn")
+    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out_b.bin")
+    res = subprocess.run([exe, os.path.join(emit.GEN_DIR, "convbn.bin"), fin, fout], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                         text=True, timeout=110)
+    assert res.returncode == 0, res.stderr
+    assert np.array_equal(np.fromfile(fout, np.float32), y_text)
+
+
 def test_int8_cnn_session_is_bit_exact(tmp_path):
     x = models.cnn_input(8)
     y = run_session("qcnn", x, tmp_path)
