@@ -30,8 +30,14 @@ struct ConvArgs {
    // between its rows / columns, unit output stride, and the weights w [C, OC/groups, KH, KW] read with both
    // kernel axes reversed. ph / pw are then dil*(K-1) - pad of the transposed convolution (may be negative).
    int transposed, uh, uw;
+   // Tap (a, b) of this launch is element (th0 + a * ths, tw0 + b * tws) of the KH0 x KW0 kernel in memory, and output
+   // pixel (q, r) of this launch is pixel (oy0 + q * oys, ox0 + r * oxs) of the OH0 x OW0 output plane. A plain
+   // convolution has the identity for both; a transposed convolution with a stride runs one launch per output
+   // phase (oy mod stride, ox mod stride), each with the taps that reach that phase and no zeros in between.
+   int KH0, KW0, th0, ths, tw0, tws;
+   int OH0, OW0, oy0, oys, ox0, oxs;
    FastDiv dPW, dPH, dKC;   // divisions by the patch extents and the K-chunk length in the staging loops
-   FastDiv dUH, dUW;
+   FastDiv dUH, dUW, dOW;
 };
 
 // Input row / column behind position `up` of the zero-interleaved input, or -1 where a zero sits.
@@ -115,7 +121,9 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
          if (k < kc && oc0 + ocl < g.ocg) {
             if (g.transposed) {
                const int icl = k / KHW, t = k - icl * KHW;
-               v = g.w[(((size_t)grp * g.icg + ic0 + icl) * g.ocg + oc0 + ocl) * KHW + (KHW - 1 - t)];
+               const int ta = t / g.KW, tb = t - ta * g.KW;
+               v = g.w[((((size_t)grp * g.icg + ic0 + icl) * g.ocg + oc0 + ocl) * g.KH0 + g.th0 + ta * g.ths) * g.KW0 + g.tw0 +
+                       tb * g.tws];
             } else {
                v = wg[(size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k];
             }
@@ -140,13 +148,16 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       }
    }
 
-   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * OHW;
+   const size_t plane = (size_t)g.OH0 * g.OW0;
+   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane;
 #pragma unroll
    for (int i = 0; i < TI; ++i)
 #pragma unroll
       for (int j = 0; j < TJ; ++j) {
          const int p = p0 + wn * TJ * 32 + j * 32 + fr;
          if (p >= OHW) continue;
+         const int q = fdiv(p, g.dOW);
+         const size_t po = (size_t)(g.oy0 + q * g.oys) * g.OW0 + g.ox0 + (p - q * g.OW) * g.oxs;
 #pragma unroll
          for (int r = 0; r < 16; ++r) {
             const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
@@ -154,7 +165,7 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
             float v = acc[i][j][r];
             if (g.bias) v = __fadd_rn(v, g.bias[grp * g.ocg + oc]);
             if (g.relu) v = v > 0.0f ? v : 0.0f;
-            yn[(size_t)oc * OHW + p] = v;
+            yn[(size_t)oc * plane + po] = v;
          }
       }
 }
@@ -173,7 +184,6 @@ __global__ void k_conv2d_f32_simple(ConvArgs g)
    const int n = (int)(r / g.OC);
    const int grp = oc / g.ocg;
    float acc = 0.0f;
-   const int KHW = g.KH * g.KW;
    for (int ic = 0; ic < g.icg; ++ic)
       for (int kh = 0; kh < g.KH; ++kh) {
          int ih = oh * g.sh - g.ph + kh * g.dh;
@@ -184,14 +194,15 @@ __global__ void k_conv2d_f32_simple(ConvArgs g)
             if (g.transposed) iw = source_index(iw, g.uw, g.dUW);
             if (iw < 0 || iw >= g.W) continue;
             const float wv = g.transposed
-                                ? g.w[(((size_t)grp * g.icg + ic) * g.ocg + (oc - grp * g.ocg)) * KHW + (KHW - 1 - (kh * g.KW + kw))]
+                                ? g.w[((((size_t)grp * g.icg + ic) * g.ocg + (oc - grp * g.ocg)) * g.KH0 + g.th0 + kh * g.ths) * g.KW0 +
+                                      g.tw0 + kw * g.tws]
                                 : g.w[(((size_t)oc * g.icg + ic) * g.KH + kh) * g.KW + kw];
             acc = __fadd_rn(acc, __fmul_rn(g.x[(((size_t)n * g.C + grp * g.icg + ic) * g.H + ih) * g.W + iw], wv));
          }
       }
    if (g.bias) acc = __fadd_rn(acc, g.bias[oc]);
    if (g.relu) acc = acc > 0.0f ? acc : 0.0f;
-   g.y[idx] = acc;
+   g.y[(((size_t)n * g.OC + oc) * g.OH0 + g.oy0 + oh * g.oys) * g.OW0 + g.ox0 + ow * g.oxs] = acc;
 }
 
 template <int TI, int TJ>
@@ -237,8 +248,15 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
 
 int run_conv(sofie_hip_ctx *ctx, ConvArgs &g)
 {
+   if (g.KH0 == 0) {   // identity tap and output maps
+      g.KH0 = g.KH; g.KW0 = g.KW;
+      g.th0 = g.transposed ? g.KH - 1 : 0; g.ths = g.transposed ? -1 : 1;
+      g.tw0 = g.transposed ? g.KW - 1 : 0; g.tws = g.transposed ? -1 : 1;
+      g.OH0 = g.OH; g.OW0 = g.OW; g.oy0 = 0; g.oys = 1; g.ox0 = 0; g.oxs = 1;
+   }
    g.dUH = make_fastdiv((unsigned)(g.uh > 0 ? g.uh : 1));
    g.dUW = make_fastdiv((unsigned)(g.uw > 0 ? g.uw : 1));
+   g.dOW = make_fastdiv((unsigned)g.OW);
    bool done = false;
    int rc;
    if (g.ocg > 64) rc = launch<2, 2>(ctx, g, &done);
@@ -305,5 +323,37 @@ extern "C" int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x
    g.ocg = OC / groups;
    g.relu = act == SOFIE_ACT_RELU;
    g.transposed = 1; g.uh = stride_h; g.uw = stride_w;
-   return run_conv(ctx, g);
+   if (dil_h != 1 || dil_w != 1 || (stride_h == 1 && stride_w == 1)) return run_conv(ctx, g);
+   // One launch per output phase. Output row oy = ry + stride*q is reached by the reversed taps k0, k0 + stride, ...
+   // with (ry - p + k0) divisible by the stride (p = K-1-pad), and tap a reads input row q + a + (ry - p + k0)/stride:
+   // a unit-stride correlation over the input as it is, with a sub-kernel of about K/stride taps.
+   const int py = KH - 1 - pad_h, px = KW - 1 - pad_w;
+   for (int ry = 0; ry < stride_h; ++ry)
+      for (int rx = 0; rx < stride_w; ++rx) {
+         if (ry >= OH || rx >= OW) continue;
+         const int k0y = (((py - ry) % stride_h) + stride_h) % stride_h, k0x = (((px - rx) % stride_w) + stride_w) % stride_w;
+         ConvArgs p = g;
+         p.uh = 1; p.uw = 1;
+         p.KH0 = KH; p.KW0 = KW;
+         p.KH = k0y < KH ? (KH - 1 - k0y) / stride_h + 1 : 0;
+         p.KW = k0x < KW ? (KW - 1 - k0x) / stride_w + 1 : 0;
+         p.th0 = KH - 1 - k0y; p.ths = -stride_h;
+         p.tw0 = KW - 1 - k0x; p.tws = -stride_w;
+         p.ph = -((ry - py + k0y) / stride_h);
+         p.pw = -((rx - px + k0x) / stride_w);
+         p.OH0 = OH; p.OW0 = OW; p.oy0 = ry; p.oys = stride_h; p.ox0 = rx; p.oxs = stride_w;
+         p.OH = (OH - 1 - ry) / stride_h + 1;
+         p.OW = (OW - 1 - rx) / stride_w + 1;
+         if (p.KH == 0 || p.KW == 0) {
+            // no tap reaches this phase: the outputs are the bias; the plain kernel's loops run zero times
+            p.KH = 0; p.KW = 0;
+            p.dUH = make_fastdiv(1u); p.dUW = make_fastdiv(1u); p.dOW = make_fastdiv((unsigned)p.OW);
+            const size_t total = (size_t)N * OC * p.OH * p.OW;
+            hipLaunchKernelGGL(k_conv2d_f32_simple, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, p);
+            if (int rc = check_launch(ctx, "k_conv2d_f32_simple")) return rc;
+            continue;
+         }
+         if (int rc = run_conv(ctx, p)) return rc;
+      }
+   return SOFIE_HIP_OK;
 }
