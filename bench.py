@@ -223,6 +223,7 @@ def extras(ctx, torch, L, ops, rng):
     ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_qconv2d_s8(
         ctx.h, ctx.ptr(xq), L.LAYOUT_NHWC, ctx.ptr(wq), L.LAYOUT_NHWC, ctx.ptr(bq), ctx.ptr(sq), ctx.ptr(yq), L.LAYOUT_NHWC,
         256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, -128, -128, L.ACT_RELU, L.OUT_S8)), 20, 3)
+    fl = 2.0 * 256 * 128 * 3136 * 576
     ex["conv2d_s8_b256_64to128_56x56"] = {"ms": ms, "tops": fl / ms / 1e9, "frac_peak": fl / ms / 1e9 / PEAK_INT8_TOPS,
                                           "gbs": (xq.numel() + yq.numel() + wq.numel()) / ms / 1e6}
     del xq, yq
