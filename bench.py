@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the SOFIE hot path on one MI355X.
 
-Headline workload (BASELINE.json configs[1]): standalone int8 GEMM with QLinearMatMul
+Headline workload (the configuration the metric is quoted on): standalone int8 GEMM with QLinearMatMul
 semantics, M=N=K=4096, A and B int8 uniform in [-127,127], per-output-channel fp32 scales
 uniform in [1e-3,1e-2], int32 accumulate, round-half-to-even requantise to int8. One "step"
 is one call of sofie_hip_qgemm_s8 on device-resident operands. Prints ONE JSON line.
@@ -150,7 +150,7 @@ def main():
 
 
 def extras(ctx, torch, L, ops, rng):
-    """Secondary figures of the other BASELINE.json configurations (not the headline value)."""
+    """Secondary figures of the other benchmark configurations (not the headline value)."""
     ex = {}
     # pre-transposed weights: the layout a Session keeps B in when it is an initializer
     n = 4096
