@@ -689,6 +689,8 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
    const bool b_nk_ok = transB && g.ldb % 16 == 0 && aligned16(g.B);
    const bool b_kn_ok = !transB && g.ldb % 4 == 0 && g.N % 4 == 0 && (reinterpret_cast<uintptr_t>(g.B) & 3u) == 0;
    g.vec_store = ((size_t)g.ldy * ESZ) % 16 == 0 && aligned16(g.Y);
+   // K = 0 (an empty sum: the outputs are the epilogue of zero) takes the plain kernel, whose K loop runs zero times
+   if (g.K == 0) return launch_simple<IS_INT, OUT>(ctx, g, transB);
    if constexpr (IS_INT && OUT != SOFIE_OUT_BF16) {
       if (transB && g.N <= 16 && a_ok && g.ldb % 16 == 0 && aligned16(g.B) && (size_t)g.M * 16 < ((size_t)1 << 40))
          return launch_skinny<OUT>(ctx, g);

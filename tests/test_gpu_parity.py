@@ -562,6 +562,44 @@ def test_conv_pool_fused_matrix_core_kernel(ops, cfg):
         assert np.array_equal(y.transpose(0, 3, 1, 2), ref), (zpx, zpy, relu)
 
 
+def test_empty_and_degenerate_inputs(ops):
+    """Zero-sized problems return success without touching the output; K = 0 leaves the bias (the accumulators are an
+    empty sum); a 1x1 image, a single row and a single column go through the general kernels."""
+    from sofie_amd import lib as L
+    ctx = ops.default_context()
+    lib, h, p = ctx.lib, ctx.h, ctx.ptr
+    y = ctx.dev(np.full((4, 4), 7, np.int8))
+    A = ctx.dev(np.zeros((4, 16), np.int8))
+    sc = ctx.dev(np.ones(4, np.float32))
+    # M = 0 and N = 0: nothing is launched, y keeps its bytes; null operands are fine then
+    assert lib.sofie_hip_qgemm_s8(h, 1, 0, 4, 16, None, 16, None, 16, None, None, 0, 0, None, 4, L.OUT_S8) == 0
+    assert lib.sofie_hip_qgemm_s8(h, 1, 4, 0, 16, p(A), 16, p(A), 16, p(sc), None, 0, 0, p(y), 4, L.OUT_S8) == 0
+    assert lib.sofie_hip_gemm_f32(h, 0, 0, 0, 5, 3, 1.0, None, 3, None, 5, 0.0, None, 0, None, 5, 0) == 0
+    assert lib.sofie_hip_conv2d_f32(h, None, None, None, None, 0, 3, 5, 5, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0) == 0
+    assert lib.sofie_hip_conv_transpose2d_f32(h, None, None, None, None, 0, 3, 5, 5, 4, 3, 3, 0, 0, 1, 1, 1, 1, 1, 7, 7, 0) == 0
+    assert lib.sofie_hip_batchnorm_f32(h, None, None, None, None, None, 0, 3, 5, 0) == 0
+    assert lib.sofie_hip_relu_f32(h, None, None, 0) == 0
+    ctx.sync()
+    assert np.all(y.cpu().numpy() == 7)
+    # K = 0: int32 output equals the bias row
+    bias = np.array([5, -6, 7, 100000], np.int32)
+    acc = ctx.empty((3, 4), torch.int32)
+    assert lib.sofie_hip_qgemm_s8(h, 1, 3, 4, 0, p(A), 0, p(A), 0, None, p(ctx.dev(bias)), 0, 0, p(acc), 4, L.OUT_S32) == 0
+    ctx.sync()
+    assert np.array_equal(acc.cpu().numpy(), np.tile(bias, (3, 1)))
+    r = rng(99)
+    a1 = r.standard_normal((1, 7)).astype(np.float32)
+    b1 = r.standard_normal((7, 1)).astype(np.float32)
+    assert rel_err(ops.gemm_f32(a1, b1, beta=0.0), oracle.gemm_f32(a1, b1, beta=0.0)) <= FP32_TOL
+    x1 = r.standard_normal((1, 1, 1, 1)).astype(np.float32)
+    w1 = r.standard_normal((1, 1, 3, 3)).astype(np.float32)
+    assert rel_err(ops.conv2d_f32(x1, w1, None, (1, 1)), oracle.conv2d_f32(x1, w1, None, (1, 1))) <= FP32_TOL
+    q1 = r.integers(-128, 128, (1, 1, 1, 1)).astype(np.int8)
+    wq = r.integers(-127, 128, (1, 1, 1, 1)).astype(np.int8)
+    s1 = np.array([0.01], np.float32)
+    assert np.array_equal(ops.qconv2d_s8(q1, wq, s1, None, (0, 0)), oracle.qconv2d_s8(q1, wq, s1, None, (0, 0), (1, 1), 1, 0, 0, False))
+
+
 def test_error_codes_of_the_quantized_entry_points(ops):
     """Bad arguments come back as SOFIE_HIP_EINVAL with a message and launch nothing; the context stays usable."""
     from sofie_amd import lib as L
