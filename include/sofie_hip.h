@@ -155,6 +155,20 @@ int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x, const flo
 int sofie_hip_batchnorm_f32(sofie_hip_ctx *ctx, const float *x, const float *scale, const float *mean,
                             const float *bias, float *y, int N, int C, int plane, int act);
 
+/* Einstein summation of n_inputs fp32 operands that is not a matrix product:
+ *   y[o0, o1, ...] = sum over s0, s1, ... of x_0[...] * x_1[...] * ...
+ * The n_labels labels are numbered with the n_out output labels first, in the order of y's dimensions (y is
+ * dense row-major over them), then the summed labels, the first of them the outermost loop. extent[l] is the
+ * size of label l; stride[i * n_labels + l] is operand i's element stride along label l, 0 where the operand
+ * does not carry the label (a repeated label adds its strides up). Products and sums are rounded one by one in
+ * loop order, as in the nest of host loops that ROperator_Einsum<float>::Generate emits for the general case
+ * (ROperator_Einsum.hxx:236-278), which this call replaces. Equations that are (stacked) matrix products are
+ * emitted as sofie_hip_gemm_f32 calls instead, where the reference emits BLAS::sgemm_ (:280-336). */
+#define SOFIE_EINSUM_MAX_INPUTS 4
+#define SOFIE_EINSUM_MAX_LABELS 12
+int sofie_hip_einsum_f32(sofie_hip_ctx *ctx, int n_inputs, const float *const *inputs, int n_labels, int n_out,
+                         const int *extent, const long long *stride, float *y);
+
 /* y[i] = x[i] > 0 ? x[i] : 0. Replaces the loop of ROperator_Relu.hxx:62-64. */
 int sofie_hip_relu_f32(sofie_hip_ctx *ctx, const float *x, float *y, size_t len);
 

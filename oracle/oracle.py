@@ -60,6 +60,8 @@ _relu = _sig("or_relu_f32", None, [_f32p, _f32p, C.c_size_t])
 _im2col = _sig("or_im2col", None, [_f32p] + [C.c_int] * 11 + [_f32p])
 _conv2d = _sig("or_conv2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 15)
 _convt = _sig("or_conv_transpose2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 17)
+_einsum = _sig("or_einsum_f32", None, [C.c_int, C.POINTER(C.c_void_p), C.c_int, C.c_int, C.POINTER(C.c_int),
+                                     C.POINTER(C.c_longlong), _f32p])
 _bn = _sig("or_batchnorm_f32", None, [_f32p] * 5 + [C.c_float, _f32p] + [C.c_int] * 4)
 _maxpool = _sig("or_maxpool2d_f32", None, [_f32p, _f32p] + [C.c_int] * 11)
 _maxpool_s8 = _sig("or_maxpool2d_s8", None, [_i8p, _i8p] + [C.c_int] * 11)
@@ -172,6 +174,43 @@ def batchnorm_f32(x, scale, bias, mean, var, epsilon=1e-5, relu=False):
     y = np.empty_like(x)
     f = lambda a: np.ascontiguousarray(a, np.float32)
     _bn(x.reshape(-1), f(scale), f(bias), f(mean), f(var), float(epsilon), y.reshape(-1), N, Cc, plane, int(relu))
+    return y
+
+
+def einsum_plan(equation, shapes):
+    """Labels (output labels first, then the summed ones sorted by character, the order of the reference's
+    std::map, ROperator_Einsum.hxx:125-165), their extents, per-operand strides, the output shape."""
+    eq = equation.replace(" ", "")
+    lhs, out = eq.split("->")
+    ins = lhs.split(",")
+    assert len(ins) == len(shapes)
+    extent = {}
+    for labels, shape in zip(ins, shapes):
+        assert len(labels) == len(shape)
+        for l, d in zip(labels, shape):
+            assert extent.setdefault(l, d) == d
+    summed = "".join(sorted(l for l in extent if l not in out))
+    labels = out + summed
+    strides = []
+    for lab, shape in zip(ins, shapes):
+        st = [int(np.prod(shape[j + 1:], dtype=np.int64)) for j in range(len(shape))]
+        row = [0] * len(labels)
+        for j, l in enumerate(lab):
+            row[labels.index(l)] += st[j]
+        strides.append(row)
+    return labels, len(out), [extent[l] for l in labels], strides, [extent[l] for l in out]
+
+
+def einsum_f32(equation, operands):
+    """Einsum as the reference's emitted loop nest computes it (ROperator_Einsum.hxx:236-278)."""
+    xs = [np.ascontiguousarray(x, np.float32) for x in operands]
+    labels, n_out, extent, strides, oshape = einsum_plan(equation, [x.shape for x in xs])
+    y = np.empty(oshape, np.float32)
+    ptrs = (C.c_void_p * len(xs))(*[x.ctypes.data for x in xs])
+    ext = (C.c_int * max(1, len(labels)))(*extent)
+    flat = [v for row in strides for v in row]
+    st = (C.c_longlong * max(1, len(flat)))(*flat)
+    _einsum(len(xs), ptrs, len(labels), n_out, ext, st, y.reshape(-1))
     return y
 
 

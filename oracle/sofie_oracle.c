@@ -17,6 +17,8 @@
  *                                answers, torch.nn.functional.conv_transpose2d on CPU
  *   or_batchnorm_f32             pinned: torch.nn.functional.batch_norm on CPU, float64
  *                                closed form (the reference holds no fixture for it)
+ *   or_einsum_f32                pinned: Einsum_matmul / _dotprod / _3 / _4 known answers of
+ *                                the reference's tests, numpy.einsum in float64
  *   or_relu, or_maxpool2d        pinned: MaxPool2d known answer, torch CPU
  *   or_broadcast_rows            pinned through the Linear_* answers (bias broadcast)
  *   or_qgemm_s8, or_qconv2d_s8,
@@ -301,6 +303,45 @@ void or_batchnorm_f32(const float *x, const float *scale, const float *bias, con
                 y[off + i] = v;
             }
         }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Einstein summation, the loop nest ROperator_Einsum.hxx:236-278 emits: loops */
+/* over the output labels, the element set to zero, loops over the summed    */
+/* labels (first label outermost), "+=" of the product of the operands.      */
+/* Labels are numbered output labels first, then summed labels; extent[l] is */
+/* a label's size, stride[i*n_labels + l] operand i's element stride along   */
+/* it (0 if absent). The reference hands matrix-product equations to sgemm_  */
+/* (:280-336); with or_sgemm's increasing-k accumulation, alpha = 1 and      */
+/* beta = 0 that gives the same numbers as this nest, so one function covers */
+/* both. Pinned by: the four Einsum known answers, numpy.einsum in float64.  */
+/* ------------------------------------------------------------------------- */
+void or_einsum_f32(int n_inputs, const float *const *x, int n_labels, int n_out, const int *extent,
+                   const long long *stride, float *y)
+{
+    long long outputs = 1, terms = 1;
+    for (int l = 0; l < n_labels; ++l) {
+        if (l < n_out) outputs *= extent[l];
+        else terms *= extent[l];
+    }
+    int pos[32];
+    for (long long o = 0; o < outputs; ++o) {
+        long long rem = o;
+        for (int l = n_out - 1; l >= 0; --l) { pos[l] = (int)(rem % extent[l]); rem /= extent[l]; }
+        float sum = 0;
+        for (long long t = 0; t < terms; ++t) {
+            long long r2 = t;
+            for (int l = n_labels - 1; l >= n_out; --l) { pos[l] = (int)(r2 % extent[l]); r2 /= extent[l]; }
+            float prod = 1;
+            for (int i = 0; i < n_inputs; ++i) {
+                long long off = 0;
+                for (int l = 0; l < n_labels; ++l) off += pos[l] * stride[(size_t)i * n_labels + l];
+                prod = (i == 0) ? x[i][off] : prod * x[i][off];
+            }
+            sum += prod;
+        }
+        y[o] = sum;
+    }
 }
 
 /* ------------------------------------------------------------------------- */

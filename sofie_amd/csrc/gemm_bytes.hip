@@ -57,7 +57,20 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16) ? 1 : 2) k_gemm_bytes(Gem
    const int wm = wave >> 1, wn = wave & 1;
 
    int tm, tn;
-   tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+   int pid = blockIdx.x;
+   if constexpr (IS_INT && OUT == SOFIE_OUT_S32) {
+      if (g.splits > 1) {
+         const int tiles = g.tiles_m * g.tiles_n;
+         const int ks = pid / tiles;
+         pid -= ks * tiles;
+         const int k_begin = ks * g.kslice;
+         g.A += k_begin;
+         g.B += B_KN ? (size_t)k_begin * g.ldb : (size_t)k_begin;
+         g.K = (g.K - k_begin) < g.kslice ? (g.K - k_begin) : g.kslice;
+         g.Y = static_cast<unsigned char *>(g.Y) + (size_t)ks * g.ysplit;
+      }
+   }
+   tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
 
    // --- global -> register staging -----------------------------------------------------
@@ -628,6 +641,37 @@ int launch_skinny(sofie_hip_ctx *ctx, GemmArgs &g)
    return check_launch(ctx, "k_qgemm_skinny");
 }
 
+template <class Mma, int OUT> struct IS_SPLITTABLE {
+   static constexpr bool value = __is_same(typename Mma::Acc, v16i) && OUT == SOFIE_OUT_S32;
+};
+
+// Sum of the K slices' int32 partial tiles, then bias and the output conversion of the unsplit kernel.
+// One thread per four consecutive columns of one row; P is [splits][M][ldp], ldp a multiple of 4.
+template <int OUT>
+__global__ void __launch_bounds__(256) k_splitk_finish(GemmArgs g, const int *__restrict__ P, int splits, int ldp)
+{
+   const int quads = ldp >> 2;
+   const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+   if (t >= (size_t)g.M * quads) return;
+   const int m = (int)(t / quads), n = (int)(t % quads) * 4;
+   const size_t plane = (size_t)g.M * ldp;
+   v4i s = *reinterpret_cast<const v4i *>(P + (size_t)m * ldp + n);
+   for (int k = 1; k < splits; ++k) {
+      const v4i v = *reinterpret_cast<const v4i *>(P + k * plane + (size_t)m * ldp + n);
+      s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
+   }
+   constexpr int ESZ = OutSize<OUT>::value;
+   unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + n) * ESZ;
+#pragma unroll
+   for (int e = 0; e < 4; ++e) {
+      if (n + e >= g.N) break;
+      const unsigned r = epilogue_value<true, OUT>(g, g.scale ? g.scale[n + e] : 0.0f,
+                                                   g.bias ? static_cast<const int *>(g.bias)[n + e] : 0, s[e], 0.0f);
+      if constexpr (ESZ == 1) out[e] = (unsigned char)((int)fminf(__uint_as_float(r), 255.0f) - 128);
+      else reinterpret_cast<unsigned *>(out)[e] = r;
+   }
+}
+
 template <class Mma, int BK, int NSETS, int TI, int TJ, int OUT, bool B_KN, bool FULL>
 int launch_tiled_impl(sofie_hip_ctx *ctx, GemmArgs &g)
 {
@@ -642,7 +686,8 @@ int launch_tiled_impl(sofie_hip_ctx *ctx, GemmArgs &g)
    auto kern = k_gemm_bytes<Mma, BK, NSETS, TI, TJ, OUT, B_KN, FULL>;
    SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-   hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(256), lds, ctx->stream, g);
+   const int splits = (IS_SPLITTABLE<Mma, OUT>::value && g.splits > 1) ? g.splits : 1;
+   hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * splits), dim3(256), lds, ctx->stream, g);
    return check_launch(ctx, "k_gemm_bytes");
 }
 
@@ -669,6 +714,31 @@ int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(512), lds, ctx->stream, g);
    return check_launch(ctx, "k_gemm_dma");
+}
+
+// K cut into `splits` slices of `kslice` bytes (a multiple of BK): partial sums into the context's scratch
+// buffer, then k_splitk_finish writes Y.
+template <class Mma, int BK, int NSETS, int OUT>
+int launch_split_k(sofie_hip_ctx *ctx, GemmArgs &g, int splits, int kslice)
+{
+   const int ldp = cdiv(g.N, 4) * 4;
+   void *part = nullptr;
+   if (int rc = workspace(ctx, (size_t)splits * g.M * ldp * sizeof(int), &part)) return rc;
+   GemmArgs p = g;
+   p.Y = part;
+   p.ldy = ldp;
+   p.scale = nullptr;
+   p.bias = nullptr;
+   p.relu = 0;
+   p.vec_store = 1;
+   p.splits = splits;
+   p.kslice = kslice;
+   p.ysplit = (long long)g.M * ldp * sizeof(int);
+   if (int rc = launch_tiled<Mma, BK, NSETS, 2, 2, SOFIE_OUT_S32, false>(ctx, p)) return rc;
+   const size_t threads = (size_t)g.M * (ldp / 4);
+   hipLaunchKernelGGL((k_splitk_finish<OUT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, ctx->stream, g,
+                      static_cast<const int *>(part), splits, ldp);
+   return check_launch(ctx, "k_splitk_finish");
 }
 
 template <bool IS_INT, int OUT>
@@ -708,6 +778,21 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
       if (big) return launch_tiled<Mma, BK, NSETS, 4, 4, OUT, false>(ctx, g);
       // a long K with few 128 x 128 tiles (a wide fully connected layer on a small batch x width):
       // 64 x 64 tiles put four times as many workgroups on the device
+      if constexpr (IS_INT) {
+         // ... and a longer one is cut into slices of K: 128 x 128 tiles write int32 partial sums per slice
+         // (integer sums, so the result does not depend on the cut), a second kernel adds them and converts
+         const int tiles128 = cdiv(g.M, 128) * cdiv(g.N, 128);
+         // (measured: pays from K = 8192 on; below that the second pass over the partial sums costs more)
+         if (tiles128 * 2 <= ctx->num_cus && g.K >= 8192) {
+            int splits = ctx->num_cus / tiles128;
+            const int shortest = tiles128 * 8 <= ctx->num_cus ? 1024 : 2048;
+            if (splits > g.K / shortest) splits = g.K / shortest;
+            if (splits > 16) splits = 16;
+            const int kslice = cdiv(cdiv(g.K, splits), 128) * 128;
+            splits = cdiv(g.K, kslice);
+            if (splits > 1) return launch_split_k<Mma, BK, NSETS, OUT>(ctx, g, splits, kslice);
+         }
+      }
       if (cdiv(g.M, 128) * cdiv(g.N, 128) * 2 <= ctx->num_cus && g.K >= 1024)
          return launch_tiled<Mma, BK, NSETS, 1, 1, OUT, false>(ctx, g);
       return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, false>(ctx, g);

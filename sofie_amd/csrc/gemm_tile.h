@@ -48,6 +48,10 @@ struct GemmArgs {
    float s;              // fp8: scale_a * scale_b
    int tiles_m, tiles_n;
    int vec_store;        // rows of Y may be written with 16-byte stores
+   // split K (int32 partial sums only): workgroup b works on K slice b / (tiles_m * tiles_n) of `kslice`
+   // bytes and writes its tile into the slice's own copy of Y, `ysplit` bytes after the previous one
+   int splits, kslice;
+   long long ysplit;
 };
 
 template <int OUT> struct OutSize { static constexpr int value = 4; };

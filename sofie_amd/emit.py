@@ -40,14 +40,17 @@ class ModelSpec:
         self.name = name
         self.lines = ["model %s" % name]
         self.tensors = {}
-        self.input = None
+        self.input = None      # the first input (single-input runners)
+        self.inputs = []
         self.output = None
         self.out_type = "FLOAT"
 
     def add_input(self, name, dtype, shape):
         t = dtype if isinstance(dtype, str) else _TYPE[np.dtype(dtype)]
         self.lines.append("input %s %s %s" % (name, t, _lst(shape)))
-        self.input = (name, t, tuple(shape))
+        if self.input is None:
+            self.input = (name, t, tuple(shape))
+        self.inputs.append((name, t, tuple(shape)))
 
     def add_init(self, name, array, type_name=None):
         array = np.ascontiguousarray(array)
@@ -81,6 +84,9 @@ class ModelSpec:
 
     def batchnorm(self, x, scale, b, mean, var, y, epsilon=1e-5):
         self.lines.append("op BatchNormalization %r %s %s %s %s %s %s" % (float(epsilon), x, scale, b, mean, var, y))
+
+    def einsum(self, equation, xs, y):
+        self.lines.append("op Einsum %s %d %s %s" % (equation.replace(" ", ""), len(xs), " ".join(xs), y))
 
     def relu(self, x, y):
         self.lines.append("op Relu %s %s" % (x, y))
@@ -138,7 +144,7 @@ class ModelSpec:
         cmd = ["g++", "-std=c++17", "-O2", "-I" + os.path.join(ROOT, "include"), "-I" + outdir,
                "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % self.name, "-DSOFIE_MODEL_NS=SOFIE_%s" % self.name,
                "-DSOFIE_IN_T=%s" % _CTYPE[self.input[1]], "-DSOFIE_OUT_T=%s" % _CTYPE[self.out_type],
-               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0],
+               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs),
                os.path.join(_HERE, "host", "examples", "run_session.cxx"), "-o", exe,
                "-L" + _HERE, "-lsofie_hip", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath," + _HERE]
         res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -167,8 +173,8 @@ def clean(name):
 def spec_from_onnx(name, graph):
     """Gemm / Relu / Conv / MaxPool / Flatten graph (sofie_amd.onnx_wire.load) -> ModelSpec."""
     spec = ModelSpec(name)
-    iname, _, ishape = graph["inputs"][0]
-    spec.add_input(clean(iname), "FLOAT", ishape)
+    for iname, _, ishape in graph["inputs"]:
+        spec.add_input(clean(iname), "FLOAT", ishape)
     for k, v in graph["initializers"].items():
         spec.add_init(clean(k), v)
     nodes = graph["nodes"]
@@ -201,6 +207,9 @@ def spec_from_onnx(name, graph):
             spec.conv_transpose(ins[0], ins[1], ins[2] if len(ins) > 2 else None, out, a.get("kernel_shape", ()),
                                 a.get("pads", ()), a.get("strides", ()), a.get("dilations", ()), a.get("group", 0),
                                 a.get("output_padding", ()), a.get("output_shape", ()), a.get("auto_pad", "NOTSET"))
+        elif op == "Einsum":
+            eq = a["equation"]
+            spec.einsum(eq.decode() if isinstance(eq, bytes) else eq, ins, out)
         elif op == "BatchNormalization":
             spec.batchnorm(ins[0], ins[1], ins[2], ins[3], ins[4], out, a.get("epsilon", 1e-5))
         elif op == "MaxPool":

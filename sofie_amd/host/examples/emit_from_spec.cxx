@@ -14,6 +14,7 @@
 //   op Conv AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. X W B Y
 //   op BatchNormalization EPSILON X SCALE B MEAN VAR Y
 //   op ConvTranspose AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. nop op.. nos os.. X W B Y
+//   op Einsum EQUATION nx X.. Y                  (the equation without blanks)
 //   op Relu X Y
 //   op MaxPool nk k.. np p.. ns s.. X Y
 //   op Flatten AXIS X Y
@@ -123,6 +124,14 @@ int main(int argc, char **argv)
                std::string x, sc, b, m, v, y;
                in >> eps >> x >> sc >> b >> m >> v >> y;
                r.reset(new ROperator_BatchNormalization<float>(eps, 0.9f, 0, x, sc, b, m, v, y));
+            } else if (op == "Einsum") {
+               std::string eq, y;
+               size_t nx;
+               in >> eq >> nx;
+               std::vector<std::string> xs(nx);
+               for (auto &x : xs) in >> x;
+               in >> y;
+               r.reset(new ROperator_Einsum<float>(eq, xs, y));
             } else if (op == "Relu") {
                std::string x, y;
                in >> x >> y;

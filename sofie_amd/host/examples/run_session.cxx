@@ -1,14 +1,41 @@
-// Runs a generated Session: reads the input tensor from a raw file, calls infer(), writes the output.
-// Compile with -DSOFIE_MODEL_HEADER='"x.hxx"' -DSOFIE_MODEL_NS=SOFIE_x -DSOFIE_IN_T=float -DSOFIE_OUT_T=float -DSOFIE_INPUT_MEMBER=fInput_x.
+// Runs a generated Session: reads the input tensor(s) from raw files, calls infer(), writes the output.
+// Compile with -DSOFIE_MODEL_HEADER='"x.hxx"' -DSOFIE_MODEL_NS=SOFIE_x -DSOFIE_IN_T=float -DSOFIE_OUT_T=float -DSOFIE_INPUT_MEMBER=fInput_x
+// and, for a model with several inputs, -DSOFIE_NUM_INPUTS=n (then <input.bin> is a comma-separated list, one file per input
+// in the order of infer()'s arguments, and there is no timing).
 //   run_session <weights.dat> <input.bin> <output.bin> [timed iterations of infer_device]
 #include <chrono>
 #include <cstdio>
 #include <cstring>
 #include <fstream>
 #include <iostream>
+#include <string>
+#include <utility>
 #include <vector>
 
 #include SOFIE_MODEL_HEADER
+
+#ifndef SOFIE_NUM_INPUTS
+#define SOFIE_NUM_INPUTS 1
+#endif
+
+static std::vector<SOFIE_IN_T> ReadRaw(const std::string &path)
+{
+   std::ifstream fin(path, std::ios::binary | std::ios::ate);
+   if (!fin) throw std::runtime_error("cannot open input file " + path);
+   const size_t bytes = fin.tellg();
+   fin.seekg(0);
+   std::vector<SOFIE_IN_T> x(bytes / sizeof(SOFIE_IN_T));
+   fin.read(reinterpret_cast<char *>(x.data()), bytes);
+   return x;
+}
+
+#if SOFIE_NUM_INPUTS > 1
+template <size_t... I>
+static std::vector<SOFIE_OUT_T> InferAll(SOFIE_MODEL_NS::Session &s, std::vector<std::vector<SOFIE_IN_T>> &xs, std::index_sequence<I...>)
+{
+   return s.infer(xs[I].data()...);
+}
+#endif
 
 int main(int argc, char **argv)
 {
@@ -18,12 +45,21 @@ int main(int argc, char **argv)
    }
    try {
       SOFIE_MODEL_NS::Session s(argv[1]);
-      std::ifstream fin(argv[2], std::ios::binary | std::ios::ate);
-      if (!fin) throw std::runtime_error("cannot open input file");
-      const size_t bytes = fin.tellg();
-      fin.seekg(0);
-      std::vector<SOFIE_IN_T> x(bytes / sizeof(SOFIE_IN_T));
-      fin.read(reinterpret_cast<char *>(x.data()), bytes);
+#if SOFIE_NUM_INPUTS > 1
+      std::vector<std::vector<SOFIE_IN_T>> xs;
+      {
+         std::string list = argv[2];
+         size_t start = 0;
+         for (size_t comma; (comma = list.find(',', start)) != std::string::npos; start = comma + 1)
+            xs.push_back(ReadRaw(list.substr(start, comma - start)));
+         xs.push_back(ReadRaw(list.substr(start)));
+         if (xs.size() != SOFIE_NUM_INPUTS) throw std::runtime_error("the model takes " + std::to_string(SOFIE_NUM_INPUTS) + " input files");
+      }
+      std::vector<SOFIE_OUT_T> y = InferAll(s, xs, std::make_index_sequence<SOFIE_NUM_INPUTS>{});
+      std::ofstream fout(argv[3], std::ios::binary);
+      fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
+#else
+      std::vector<SOFIE_IN_T> x = ReadRaw(argv[2]);
       std::vector<SOFIE_OUT_T> y = s.infer(x.data());
       std::ofstream fout(argv[3], std::ios::binary);
       fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
@@ -57,6 +93,7 @@ int main(int argc, char **argv)
          std::printf("{\"device_ms\": %.6f, \"host_ms\": %.6f, \"graph_ms\": %.6f, \"graph_matches\": %s, \"iters\": %d}\n", ms / iters,
                      host_ms / iters, gms / iters, same ? "true" : "false", iters);
       }
+#endif
    } catch (const std::exception &e) {
       std::cerr << "run_session: " << e.what() << "\n";
       return 1;

@@ -95,6 +95,8 @@ namespace UTILITY {
 bool AreSameShape(const std::vector<size_t> &, const std::vector<size_t> &);
 // keeps [A-Za-z0-9_], turns '-' into '_' (reference: SOFIE_common.cxx:394-400)
 std::string Clean_name(std::string input_tensor_name);
+// row-major element strides of a dense tensor (reference: SOFIE_common.cxx:402-413)
+std::vector<size_t> ComputeStrideFromShape(const std::vector<size_t> &shape);
 }   // namespace UTILITY
 
 }   // namespace SOFIE

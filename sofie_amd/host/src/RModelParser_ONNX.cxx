@@ -337,7 +337,7 @@ std::shared_ptr<void> TensorData(const Tensor &t, ETensorType type, size_t lengt
 
 const std::set<std::string> &Supported()
 {
-   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "BatchNormalization", "Conv", "ConvTranspose", "Relu", "MaxPool", "Flatten", "Reshape",
+   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "BatchNormalization", "Conv", "ConvTranspose", "Einsum", "Relu", "MaxPool", "Flatten", "Reshape",
                                              "QuantizeLinear", "DequantizeLinear", "QLinearMatMul", "QLinearConv"};
    return ops;
 }
@@ -666,6 +666,12 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
          op.reset(new ROperator_BatchNormalization<float>(n.Float("epsilon", 1e-05f), n.Float("momentum", 0.9f),
                                                           (size_t)n.Int("training_mode", 0), n.inputs[0], n.inputs[1], n.inputs[2],
                                                           n.inputs[3], n.inputs[4], n.outputs[0]));
+      } else if (t == "Einsum") {
+         // as the reference's ParseEinsum.cxx:8-46: every operand known, the equation attribute present
+         const std::string equation = n.String("equation", "");
+         if (equation.empty())
+            throw std::runtime_error("TMVA::SOFIE ONNX Parser Einsum op has  no attribute defining the equation");
+         op.reset(new ROperator_Einsum<float>(equation, n.inputs, n.outputs[0]));
       } else if (t == "Relu") {
          op.reset(new ROperator_Relu<float>(n.inputs.at(0), n.outputs[0]));
       } else if (t == "MaxPool") {

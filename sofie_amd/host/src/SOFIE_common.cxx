@@ -115,4 +115,11 @@ std::string UTILITY::Clean_name(std::string s)
    return s;
 }
 
+std::vector<size_t> UTILITY::ComputeStrideFromShape(const std::vector<size_t> &shape)
+{
+   std::vector<size_t> strides(shape.size(), 1);
+   for (size_t i = shape.size(); i-- > 1;) strides[i - 1] = strides[i] * shape[i];
+   return strides;
+}
+
 }   // namespace SOFIE

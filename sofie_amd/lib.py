@@ -40,6 +40,7 @@ SIGNATURES = {
     "sofie_hip_graph_launch": [_p, _p],
     "sofie_hip_graph_destroy": [_p, _p],
     "sofie_hip_batchnorm_f32": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i],
+    "sofie_hip_einsum_f32": [_p, _i, C.POINTER(_p), _i, _i, C.POINTER(_i), C.POINTER(C.c_longlong), _p],
     "sofie_hip_relu_f32": [_p, _p, _p, _z],
     "sofie_hip_maxpool2d_f32": [_p, _p, _p] + [_i] * 11,
     "sofie_hip_quantize_f32_s8": [_p, _p, _p, _z, _f, _i],

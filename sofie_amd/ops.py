@@ -175,6 +175,79 @@ def batchnorm_f32(x, scale, bias, mean, var, epsilon=1e-5, relu=False, ctx=None)
     return _ret(y, x)
 
 
+def _matrix_product_type(ins, out, summed):
+    """The emitter's test (ROperator_Einsum::MatrixProductType): "nn" / "tn" / "nt" / "tt" or ""."""
+    if len(ins) != 2 or len(summed) != 1:
+        return ""
+    la, lb = ins
+    if len(la) < 2 or len(lb) < 2 or len(out) < 2 or len(set(la)) != len(la) or len(set(lb)) != len(lb):
+        return ""
+    s = summed[0]
+    pa, pb = la.find(s), lb.find(s)
+    if pa < len(la) - 2 or pb < len(lb) - 2:
+        return ""
+    ta, tb = pa == len(la) - 2, pb == len(lb) - 1
+    m = la[-1] if ta else la[-2]
+    n = lb[-2] if tb else lb[-1]
+    if m == n or out[-2] != m or out[-1] != n or m in lb or n in la:
+        return ""
+    if any(l not in out[:-2] for l in la[:-2] + lb[:-2]):
+        return ""
+    return ("t" if ta else "n") + ("t" if tb else "n")
+
+
+def einsum_f32(equation, operands, ctx=None):
+    """Einsum the way the emitted Session runs it: a (stacked) matrix product as one sofie_hip_gemm_f32 call per
+    stacked matrix, anything else as one sofie_hip_einsum_f32 call."""
+    ctx = ctx or default_context()
+    xs = [ctx.dev(x, torch.float32).contiguous() for x in operands]
+    eq = equation.replace(" ", "")
+    lhs, out = eq.split("->")
+    ins = lhs.split(",")
+    extent = {}
+    for labels, x in zip(ins, xs):
+        if len(labels) != x.dim():
+            raise SofieHipError("operand of rank %d with labels %s" % (x.dim(), labels))
+        for l, d in zip(labels, x.shape):
+            if extent.setdefault(l, int(d)) != int(d):
+                raise SofieHipError("label %s has two sizes" % l)
+    summed = "".join(sorted(l for l in extent if l not in out))
+    oshape = tuple(extent[l] for l in out)
+    y = ctx.empty(oshape if oshape else (1,), torch.float32)
+    kind = _matrix_product_type(ins, out, summed)
+    if kind:
+        a, b = xs
+        ta, tb = kind[0] == "t", kind[1] == "t"
+        M = a.shape[-1] if ta else a.shape[-2]
+        K = a.shape[-2] if ta else a.shape[-1]
+        N = b.shape[-2] if tb else b.shape[-1]
+        lead = out[:-2]
+        y3 = y.view(-1, M, N)
+        for idx in range(y3.shape[0]):
+            pos, rem = {}, idx
+            for l in reversed(lead):
+                pos[l] = rem % extent[l]
+                rem //= extent[l]
+            am = a[tuple(pos[l] for l in ins[0][:-2])]
+            bm = b[tuple(pos[l] for l in ins[1][:-2])]
+            ctx.check(ctx.lib.sofie_hip_gemm_f32(ctx.h, int(ta), int(tb), M, N, K, 1.0, ctx.ptr(am), a.shape[-1], ctx.ptr(bm),
+                                                 b.shape[-1], 0.0, None, L.BIAS_NONE, ctx.ptr(y3[idx]), N, L.ACT_NONE))
+    else:
+        labels = out + summed
+        strides = []
+        for lab, x in zip(ins, xs):
+            row = [0] * len(labels)
+            for j, l in enumerate(lab):
+                row[labels.index(l)] += int(x.stride(j))
+            strides += row
+        ptrs = (C.c_void_p * len(xs))(*[x.data_ptr() for x in xs])
+        ext = (C.c_int * max(1, len(labels)))(*[extent[l] for l in labels])
+        st = (C.c_longlong * max(1, len(strides)))(*strides)
+        ctx.check(ctx.lib.sofie_hip_einsum_f32(ctx.h, len(xs), ptrs, len(labels), len(out), ext, st, ctx.ptr(y)))
+    y = y.view(oshape)
+    return _ret(y, operands[0])
+
+
 def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0), layout=L.LAYOUT_NCHW, ctx=None):
     """pads = (top, left, bottom, right). int8 tensors may be NHWC (layout flag); fp32 is NCHW."""
     ctx = ctx or default_context()

@@ -11,7 +11,9 @@ What is written:
                                      <name>.ref.hxx headers (numbers only) together with
                                      the input each test feeds (ones / iota / literal list,
                                      from TestCustomModelsFromONNX.cxx:330-349,372-391,
-                                     693-712,860-967,1023-1052,2047-2152)
+                                     693-712,860-967,1023-1052,2047-2152); for the Einsum models
+                                     the literal inputs and outputs of the tests themselves
+                                     (TestCustomModelsFromONNX.cxx:3028-3103)
 """
 import json
 import os
@@ -49,6 +51,17 @@ MAXPOOL2D_INPUT = [
 ]
 
 
+# The reference's Einsum tests carry inputs and answers as literals (TestCustomModelsFromONNX.cxx:3028-3103).
+EINSUM_CASES = {
+    "Einsum_matmul": ([[1, 2, 3, 4], [5, 6, 7, 8]], [19, 22, 43, 50]),
+    "Einsum_dotprod": ([[1, 2, 3], [5, 6, 7]], [5 + 12 + 21]),
+    "Einsum_3": ([[1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12], [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12]],
+                 [66, 87, 108, 498, 555, 612]),
+    "Einsum_4": ([[1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12], [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17, 18]],
+                 [14, 32, 50, 32, 77, 122, 266, 338, 410, 365, 464, 563]),
+}
+
+
 def numbers_of(header_text, array):
     m = re.search(r"float\s+%s\s*\[\s*\]\s*=\s*\{(.*?)\}" % re.escape(array), header_text, re.S)
     body = re.sub(r"//[^\n]*", "", m.group(1))
@@ -67,6 +80,12 @@ def main():
         if kind == "literal":
             entry["input"] = MAXPOOL2D_INPUT
         expected[name] = entry
+    for name, (inputs, answer) in EINSUM_CASES.items():
+        shutil.copyfile(os.path.join(REF, name + ".onnx"), os.path.join(HERE, "onnx", name + ".onnx"))
+        os.chmod(os.path.join(HERE, "onnx", name + ".onnx"), 0o644)
+        # one literal list per graph input, in the order of the graph's inputs; shapes come from the model file
+        expected[name] = {"input_kind": "literals", "inputs": [[float(v) for v in x] for x in inputs],
+                          "expected": [float(v) for v in answer]}
     with open(os.path.join(HERE, "expected.json"), "w") as f:
         json.dump(expected, f, indent=0)
     print({k: len(v["expected"]) for k, v in expected.items()})

@@ -10,7 +10,7 @@ GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 FIXTURES = ["Linear_16", "Linear_32", "Linear_64", "ConvWithPadding", "ConvWithoutPadding",
             "ConvWithAutopadSameLower", "ConvWithStridesPadding", "ConvWithStridesNoPadding",
             "ConvWithAsymmetricPadding", "MaxPool2d", "ConvTranspose1d", "ConvTranspose2d", "ConvTransposeBias2d",
-            "ConvTransposeBias2dBatched"]
+            "ConvTransposeBias2dBatched", "Einsum_matmul", "Einsum_dotprod", "Einsum_3", "Einsum_4"]
 
 
 def fixture_spec(name):

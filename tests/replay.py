@@ -1,6 +1,6 @@
-"""Replay a decoded ONNX graph (Gemm / Relu / Conv / ConvTranspose / MaxPool / Flatten) through a backend.
+"""Replay a decoded ONNX graph (Gemm / Relu / Conv / ConvTranspose / Einsum / MaxPool / Flatten) through a backend.
 
-A backend is any object with the methods gemm_f32, relu_f32, conv2d_f32, conv_transpose2d_f32 and maxpool2d
+A backend is any object with the methods gemm_f32, relu_f32, conv2d_f32, conv_transpose2d_f32, einsum_f32 and maxpool2d
 taking and returning numpy arrays: the CPU oracle module, or the HIP library wrapper.
 The attribute handling restates what the reference's operators do at Initialize time.
 """
@@ -87,6 +87,9 @@ def run_graph(graph, feeds, backend):
                                              output_padding=tuple(extra))
             if dim == 1:
                 y = y[:, :, 0, :]
+        elif op == "Einsum":
+            eq = a["equation"]
+            y = backend.einsum_f32(eq.decode() if isinstance(eq, bytes) else eq, [env[i] for i in ins])
         elif op == "MaxPool":
             y = backend.maxpool2d(env[ins[0]], tuple(a["kernel_shape"]),
                                   tuple(a.get("strides", [1, 1])),
@@ -98,6 +101,14 @@ def run_graph(graph, feeds, backend):
             raise NotImplementedError(op)
         env[node["outputs"][0]] = y
     return env[graph["outputs"][0][0]]
+
+
+def fixture_feeds(entry, graph):
+    """{graph input name: array} for a fixture entry."""
+    if entry["input_kind"] == "literals":
+        return {name: np.array(vals, np.float32).reshape(shape)
+                for (name, _, shape), vals in zip(graph["inputs"], entry["inputs"])}
+    return {graph["inputs"][0][0]: fixture_input(entry)}
 
 
 def fixture_input(entry):

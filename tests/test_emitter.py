@@ -371,6 +371,56 @@ def test_stacked_matmul_shapes_and_offsets(tmp_path):
         bad.generate(str(tmp_path))
 
 
+def _einsum_spec(name, equation, shapes):
+    s = emit.ModelSpec(name)
+    xs = ["x%d" % i for i in range(len(shapes))]
+    for n, shape in zip(xs, shapes):
+        s.add_input(n, "FLOAT", shape)
+    s.einsum(equation, xs, "y")
+    s.set_output("y")
+    return s
+
+
+def test_einsum_matrix_products_become_gemm_calls_everything_else_one_kernel_call(tmp_path):
+    """The reference's four cases of a matrix product (ROperator_Einsum.hxx:181-197) map to transA / transB of
+    one Gemm call per stacked matrix; an equation whose free labels come out in another order, which the reference
+    would hand to sgemm_ all the same, takes the general kernel."""
+    def code(name, eq, shapes):
+        return open(_einsum_spec(name, eq, shapes).generate(str(tmp_path))[0]).read()
+    c = code("es_nn", "ik,kj->ij", [(4, 5), (5, 6)])
+    assert "sofie_hip_gemm_f32(fCtx, 0, 0, 4, 6, 5, 1.0f, tensor_x0, 5, tensor_x1, 6," in c
+    c = code("es_tn", "ki,kj->ij", [(5, 4), (5, 6)])
+    assert "sofie_hip_gemm_f32(fCtx, 1, 0, 4, 6, 5, 1.0f, tensor_x0, 4, tensor_x1, 6," in c
+    c = code("es_nt", "bik,bjk->bij", [(3, 4, 5), (3, 6, 5)])
+    assert "sofie_hip_gemm_f32(fCtx, 0, 1, 4, 6, 5," in c and "_a[] = {0, 20, 40};" in c and "_b[] = {0, 30, 60};" in c
+    c = code("es_tt", "ki,jk->ij", [(5, 4), (6, 5)])
+    assert "sofie_hip_gemm_f32(fCtx, 1, 1, 4, 6, 5, 1.0f, tensor_x0, 4, tensor_x1, 5," in c
+    # a stacked label that only one operand carries: the other operand's matrix repeats
+    c = code("es_bc", "abik,bkj->abij", [(2, 3, 4, 5), (3, 5, 6)])
+    assert "_a[] = {0, 20, 40, 60, 80, 100};" in c and "_b[] = {0, 30, 60, 0, 30, 60};" in c
+    # free labels swapped in the output: not a row-major product of these operands
+    c = code("es_sw", "ik,kj->ji", [(4, 5), (5, 6)])
+    assert "sofie_hip_gemm_f32" not in c
+    assert "_extent[] = {6, 4, 5};" in c and "_stride[] = {0, 5, 1, 1, 0, 6};" in c
+    assert "sofie_hip_einsum_f32(fCtx, 2, op_0_x, 3, 2, op_0_extent, op_0_stride, tensor_y)" in c
+    # two summed labels run in the order of their characters; a scalar result has no output label
+    c = code("es_2", "abc,abd->ad", [(2, 2, 3), (2, 2, 3)])
+    assert "_extent[] = {2, 3, 2, 3};" in c and "_stride[] = {6, 0, 3, 1, 6, 1, 3, 0};" in c
+    c = code("es_dot", "i,i->", [(7,), (7,)])
+    assert "sofie_hip_einsum_f32(fCtx, 2, op_0_x, 1, 0," in c and "std::vector<float> ret(1);" in c
+    # a repeated label walks the diagonal: its strides add up
+    c = code("es_diag", "ii->i", [(5, 5)])
+    assert "_stride[] = {6};" in c
+
+
+def test_einsum_errors(tmp_path):
+    assert "Error parsing the equation ik,kj" in emit_error(_einsum_spec("ee1", "ik,kj", [(2, 3), (3, 2)]), tmp_path)
+    assert "Error parsing the equation" in emit_error(_einsum_spec("ee2", "ik->i", [(2, 3), (3, 2)]), tmp_path)
+    assert "output label z is not present in inputs" in emit_error(_einsum_spec("ee3", "ik,kj->iz", [(2, 3), (3, 2)]), tmp_path)
+    assert "label k has two sizes, 3 and 4" in emit_error(_einsum_spec("ee4", "ik,kj->ij", [(2, 3), (4, 2)]), tmp_path)
+    assert "invalid label or shape" in emit_error(_einsum_spec("ee5", "ik,kj->ij", [(2, 3, 1), (3, 2)]), tmp_path)
+
+
 def test_binary_weight_file_holds_the_same_tensors(tmp_path):
     """Options::kBinaryWeightFile: the .bin file carries the records of the .dat file (same names, order, lengths and
     values, typed and raw) and the generated constructor defaults to it; its reader takes either format."""

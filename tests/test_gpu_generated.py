@@ -24,8 +24,16 @@ def run_session(name, x, tmp_path, out_dtype=np.float32, dat=None, iters=0):
     exe = os.path.join(emit.GEN_DIR, "run_" + name)
     if not os.path.exists(exe):
         raise RuntimeError("%s is missing: run python tests/build_generated.py on the build machine" % exe)
-    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
-    np.ascontiguousarray(x).tofile(fin)
+    fout = str(tmp_path / "out.bin")
+    if isinstance(x, (list, tuple)):
+        # one file per input of the model, in the order of infer()'s arguments
+        names = [str(tmp_path / ("in%d.bin" % i)) for i in range(len(x))]
+        for f, a in zip(names, x):
+            np.ascontiguousarray(a).tofile(f)
+        fin = ",".join(names)
+    else:
+        fin = str(tmp_path / "in.bin")
+        np.ascontiguousarray(x).tofile(fin)
     cmd = [exe, os.path.join(emit.GEN_DIR, (dat or name) + ".dat"), fin, fout] + ([str(iters)] if iters else [])
     print("running", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=110)
@@ -42,12 +50,13 @@ def rel_err(a, b):
 def test_reference_fixture_through_generated_session(name, tmp_path):
     entry = json.load(open(os.path.join(GOLD, "expected.json")))[name]
     _, graph = models.fixture_spec(name)
-    x = replay.fixture_input(entry)
-    y = run_session(name, x, tmp_path)
+    feeds = replay.fixture_feeds(entry, graph)
+    xs = [feeds[i[0]] for i in graph["inputs"]]
+    y = run_session(name, xs if len(xs) > 1 else xs[0], tmp_path)
     want = np.array(entry["expected"], np.float32)
     assert y.size == want.size
     assert np.max(np.abs(y - want)) <= 1e-3             # the reference's own tolerance
-    yo = replay.run_graph(graph, {graph["inputs"][0][0]: x}, oracle)
+    yo = replay.run_graph(graph, feeds, oracle)
     assert rel_err(y, yo.reshape(-1)) <= 1e-5
 
 

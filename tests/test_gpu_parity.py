@@ -51,14 +51,14 @@ FP32_TOL = 1e-5
 def test_reference_known_answers_through_hip(ops, name):
     entry = EXPECTED[name]
     graph = onnx_wire.load(os.path.join(GOLD, "onnx", name + ".onnx"))
-    x = replay.fixture_input(entry)
-    y = replay.run_graph(graph, {graph["inputs"][0][0]: x}, ops)
+    feeds = replay.fixture_feeds(entry, graph)
+    y = replay.run_graph(graph, feeds, ops)
     want = np.array(entry["expected"], np.float32)
     assert y.size == want.size
     assert np.max(np.abs(y.reshape(-1) - want)) <= 1e-3   # the reference's own tolerance
-    yo = replay.run_graph(graph, {graph["inputs"][0][0]: x}, oracle)
+    yo = replay.run_graph(graph, feeds, oracle)
     assert rel_err(y, yo) <= FP32_TOL
-    if name.startswith("Conv") or name.startswith("MaxPool"):
+    if name.startswith("Conv") or name.startswith("MaxPool") or name.startswith("Einsum"):
         assert np.array_equal(y, yo)
 
 
@@ -242,6 +242,8 @@ QGEMM_SHAPES = [
     (33, 47, 50, True), (33, 47, 50, False),            # K % 16 != 0: simple kernel
     (4096, 5, 256, True), (1, 16, 16, True),             # at most 16 columns: the dot-product kernel
     (70, 13, 1040, True), (5, 1, 32, True), (300, 9, 48, True),
+    (512, 256, 12800, True),                             # long K, few tiles: K cut into slices
+    (300, 130, 8464, True), (129, 40, 8208, True),       # ... with ragged tiles and a last slice that is shorter
 ]
 
 
@@ -707,3 +709,41 @@ def test_gemm_fp8_exact_for_small_integers(ops):
     A, B = oracle.e4m3_encode(a), oracle.e4m3_encode(b)
     y = ops.gemm_fp8(A, B, 1.0, 1.0, None, False, out=L.OUT_F32)
     assert np.array_equal(y, a @ b)
+
+
+# --------------------------------------------------------------------------- Einsum
+EINSUM_GENERAL = [
+    ("ik,kj->ji", [(40, 50), (50, 60)]), ("abc,abd->ad", [(7, 9, 33), (7, 9, 65)]), ("i,i->", [(1000,), (1000,)]),
+    ("ii->i", [(37, 37)]), ("ij->ji", [(130, 70)]), ("i,j->ij", [(300,), (129,)]), ("ab,bc,cd->ad", [(13, 14), (14, 15), (15, 12)]),
+    ("zy,y->z", [(500, 80), (80,)]), ("ijk->", [(5, 6, 7)]), ("abcd,efcd,ae,bf->ab", [(3, 4, 5, 6), (2, 3, 5, 6), (3, 2), (4, 3)]),
+]
+EINSUM_PRODUCTS = [
+    ("ik,kj->ij", [(70, 130), (130, 90)]), ("ki,kj->ij", [(50, 64), (50, 33)]), ("bik,bjk->bij", [(3, 40, 50), (3, 60, 50)]),
+    ("ki,jk->ij", [(48, 20), (36, 48)]), ("abik,bkj->abij", [(2, 3, 17, 20), (3, 20, 9)]),
+]
+
+
+@pytest.mark.parametrize("eq,shapes", EINSUM_GENERAL)
+def test_einsum_general_kernel_is_the_reference_loop_nest(ops, eq, shapes):
+    """Equations that are not matrix products: the kernel sums in the order of the reference's emitted loops with
+    separately rounded products and sums, so the result is the oracle's bit for bit."""
+    r = rng(sum(map(ord, eq)))
+    xs = [r.standard_normal(s).astype(np.float32) for s in shapes]
+    y = ops.einsum_f32(eq, xs)
+    ref = oracle.einsum_f32(eq, xs)
+    assert y.shape == ref.shape
+    assert np.array_equal(y, ref)
+
+
+@pytest.mark.parametrize("eq,shapes", EINSUM_PRODUCTS)
+def test_einsum_matrix_products_through_the_gemm_kernel(ops, eq, shapes):
+    """(Stacked) matrix products run on the Gemm kernel, whose sums associate differently: 1e-5 relative, and exact on
+    small integers."""
+    r = rng(sum(map(ord, eq)))
+    xs = [r.standard_normal(s).astype(np.float32) for s in shapes]
+    y = ops.einsum_f32(eq, xs)
+    ref = oracle.einsum_f32(eq, xs)
+    assert y.shape == ref.shape
+    assert rel_err(y, ref) <= FP32_TOL
+    xi = [r.integers(-4, 5, s).astype(np.float32) for s in shapes]
+    assert np.array_equal(ops.einsum_f32(eq, xi), oracle.einsum_f32(eq, xi))

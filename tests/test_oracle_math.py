@@ -306,3 +306,36 @@ def test_gemm_fp8_against_float64(transB):
     assert np.array_equal(yb, oracle.bf16_encode(yf))
     yb64, yf64 = oracle.gemm_fp8(A, B, sa, sb, bias, transB, acc64=True)
     assert np.max(np.abs(yf64 - truth)) <= 1e-6 * np.max(np.abs(truth))
+
+
+EINSUM_CASES = [
+    ("ik,kj->ij", [(4, 5), (5, 6)]), ("bik,bjk->bij", [(3, 4, 5), (3, 6, 5)]), ("ik,kj->ji", [(4, 5), (5, 6)]),
+    ("abc,abd->ad", [(2, 4, 3), (2, 4, 5)]), ("i,i->", [(9,), (9,)]), ("ii->i", [(6, 6)]), ("ij->ji", [(3, 7)]),
+    ("i,j->ij", [(4,), (3,)]), ("ab,bc,cd->ad", [(3, 4), (4, 5), (5, 2)]), ("abcd,abed->abce", [(2, 1, 2, 3), (2, 1, 3, 3)]),
+    ("zy,y->z", [(5, 8), (8,)]), ("ijk->", [(2, 3, 4)]),
+]
+
+
+@pytest.mark.parametrize("eq,shapes", EINSUM_CASES)
+def test_einsum_against_numpy_float64(eq, shapes):
+    """The oracle's loop nest against numpy.einsum on float64 copies (1e-6 relative), and exactly on small
+    integers, where the order of the sums cannot matter."""
+    r = np.random.default_rng(sum(map(ord, eq)))
+    xs = [r.standard_normal(s).astype(np.float32) for s in shapes]
+    y = oracle.einsum_f32(eq, xs)
+    truth = np.einsum(eq, *[x.astype(np.float64) for x in xs])
+    assert y.shape == truth.shape
+    assert np.max(np.abs(y - truth)) <= 1e-6 * max(1.0, float(np.max(np.abs(truth))))
+    xi = [r.integers(-4, 5, s).astype(np.float32) for s in shapes]
+    assert np.array_equal(oracle.einsum_f32(eq, xi), np.einsum(eq, *[x.astype(np.float64) for x in xi]).astype(np.float32))
+
+
+def test_einsum_sums_in_label_order():
+    """Summed labels run sorted by character, the first outermost (a std::map in the reference): with values that
+    cancel in one order only, the result tells the order."""
+    big = np.float32(2.0 ** 25)
+    x = np.array([[big, 1.0], [-big, 1.0]], np.float32)          # labels (a, b): terms in order (0,0) (0,1) (1,0) (1,1)
+    # ((big + 1) - big) + 1 = 1 in float32 (big + 1 rounds to big): a outermost, b inner
+    assert float(oracle.einsum_f32("ab->", [x])) == 1.0
+    # with the labels renamed so that the second axis sorts first, the loop order turns around: (big - big) + 1 + 1 = 2
+    assert float(oracle.einsum_f32("ba->", [x])) == 2.0
