@@ -130,6 +130,18 @@ int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
                          int KH, int KW, int pad_h, int pad_w, int stride_h, int stride_w,
                          int dil_h, int dil_w, int groups, int act);
 
+/* NCDHW 3-D convolution y = conv(x, w) + bias[oc], optional ReLU.
+ * x [N,C,D,H,W], w [OC, C/groups, KD, KH, KW], bias [OC] or NULL, y [N,OC,OD,OH,OW] with
+ * OD = (D + 2*pad_d - (dil_d*(KD-1)+1)) / stride_d + 1 (same for H, W). Replaces, per image (and group), the
+ * emitted UTILITY::Im2col_3d, BLAS::sgemm_ and BLAS::saxpy_ of ROperator_Conv<float>::Generate for fDim == 3
+ * (ROperator_Conv.hxx:432-451,499-518; SOFIE_common.hxx:522-580). The sum of an output runs over
+ * (channel, kd, kh, kw) in this order, one rounded product and one rounded addition per term. */
+int sofie_hip_conv3d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
+                         const float *bias, float *y, int N, int C, int D, int H, int W, int OC,
+                         int KD, int KH, int KW, int pad_d, int pad_h, int pad_w, int stride_d,
+                         int stride_h, int stride_w, int dil_d, int dil_h, int dil_w, int groups,
+                         int act);
+
 /* NCHW 2-D transposed convolution (ONNX ConvTranspose), optional ReLU.
  * x [N,C,H,W], w [C, OC/groups, KH, KW] (the ONNX layout), bias [OC] or NULL, y [N,OC,OH,OW]:
  *   y[n,oc,oy,ox] = bias[oc] + sum over (ic,kh,kw) with oy + pad_h - kh*dil_h = stride_h*iy (same for x)

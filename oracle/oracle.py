@@ -59,6 +59,7 @@ _gemm_f32 = _sig("or_gemm_f32", C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.
 _relu = _sig("or_relu_f32", None, [_f32p, _f32p, C.c_size_t])
 _im2col = _sig("or_im2col", None, [_f32p] + [C.c_int] * 11 + [_f32p])
 _conv2d = _sig("or_conv2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 15)
+_conv3d = _sig("or_conv3d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 20)
 _convt = _sig("or_conv_transpose2d_f32", C.c_int, [_f32p, _f32p, C.c_void_p, _f32p] + [C.c_int] * 17)
 _einsum = _sig("or_einsum_f32", None, [C.c_int, C.POINTER(C.c_void_p), C.c_int, C.c_int, C.POINTER(C.c_int),
                                      C.POINTER(C.c_longlong), _f32p])
@@ -144,6 +145,20 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
                  strides[0], strides[1], dilations[0], dilations[1], groups, int(relu))
     if rc:
         raise RuntimeError("or_conv2d_f32 failed: %d" % rc)
+    return y
+
+
+def conv3d_f32(x, w, bias=None, pads=(0, 0, 0), strides=(1, 1, 1), dilations=(1, 1, 1), groups=1, relu=False):
+    """3-D convolution, NCDHW (ROperator_Conv.hxx:432-451 with Im2col_3d); pads are the begin pads (d, h, w)."""
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    N, Cc, D, H, W = x.shape
+    OC, _, kd, kh, kw = w.shape
+    out = [(i + 2 * p - (d * (k - 1) + 1)) // s + 1 for i, p, d, k, s in zip((D, H, W), pads, dilations, (kd, kh, kw), strides)]
+    y = np.empty((N, OC, out[0], out[1], out[2]), np.float32)
+    rc = _conv3d(x, w, _opt(bias, np.float32), y, N, Cc, D, H, W, OC, kd, kh, kw, *pads, *strides, *dilations, groups, int(relu))
+    if rc:
+        raise RuntimeError("or_conv3d_f32 failed: %d" % rc)
     return y
 
 

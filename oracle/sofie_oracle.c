@@ -13,6 +13,9 @@
  *                                reference's tests, numpy float64 closed form
  *   or_im2col, or_conv2d_f32     pinned: ConvWith* known answers (ONNX spec examples),
  *                                torch.nn.functional.conv2d on CPU, brute-force 7-loop
+ *   or_im2col_3d, or_conv3d_f32  pinned: torch.nn.functional.conv3d on CPU, brute-force 9-loop
+ *                                (the reference holds no 3-D fixture); with a depth of one it
+ *                                must equal or_conv2d_f32
  *   or_conv_transpose2d_f32      pinned: ConvTranspose1d/2d/Bias2d/Bias2dBatched known
  *                                answers, torch.nn.functional.conv_transpose2d on CPU
  *   or_batchnorm_f32             pinned: torch.nn.functional.batch_norm on CPU, float64
@@ -303,6 +306,74 @@ void or_batchnorm_f32(const float *x, const float *scale, const float *bias, con
                 y[off + i] = v;
             }
         }
+}
+
+/* ------------------------------------------------------------------------- */
+/* 3-D convolution, NCDHW. Follows the fDim == 3 branch of                   */
+/* ROperator_Conv<float>::Generate (ROperator_Conv.hxx:432-451,499-518):     */
+/* per image and group Im2col_3d (SOFIE_common.hxx:522-580: rows ordered     */
+/* (channel, kd, kh, kw), columns (od, oh, ow), zeros for padding cells),    */
+/* sgemm_('N','N', m = OD*OH*OW, n = OC/g, k = IC/g*kd*kh*kw), then the bias */
+/* saxpy. Dilation as ONNX defines it (see or_conv2d_f32). Pinned by: torch  */
+/* conv3d on CPU, brute force, depth-one equality with or_conv2d_f32.        */
+/* ------------------------------------------------------------------------- */
+void or_im2col_3d(const float *im, int channels, int depth, int height, int width, int kd, int kh, int kw,
+                  int pd, int ph, int pw, int sd, int sh, int sw, int dd, int dh, int dw, float *col)
+{
+    const int od = (depth + 2 * pd - (dd * (kd - 1) + 1)) / sd + 1;
+    const int oh = (height + 2 * ph - (dh * (kh - 1) + 1)) / sh + 1;
+    const int ow = (width + 2 * pw - (dw * (kw - 1) + 1)) / sw + 1;
+    for (int c = 0; c < channels; ++c) {
+        const float *ch = im + (size_t)c * depth * height * width;
+        for (int a = 0; a < kd; ++a)
+            for (int b = 0; b < kh; ++b)
+                for (int e = 0; e < kw; ++e)
+                    for (int z = 0; z < od; ++z) {
+                        const int id = -pd + a * dd + z * sd;
+                        for (int yy = 0; yy < oh; ++yy) {
+                            const int ih = -ph + b * dh + yy * sh;
+                            for (int xx = 0; xx < ow; ++xx) {
+                                const int iw = -pw + e * dw + xx * sw;
+                                const int inside = id >= 0 && id < depth && ih >= 0 && ih < height && iw >= 0 && iw < width;
+                                *col++ = inside ? ch[((size_t)id * height + ih) * width + iw] : 0.0f;
+                            }
+                        }
+                    }
+    }
+}
+
+int or_conv3d_f32(const float *x, const float *w, const float *bias, float *y, int N, int C, int D, int H, int W,
+                  int OC, int kd, int kh, int kw, int pd, int ph, int pw, int sd, int sh, int sw, int dd, int dh,
+                  int dw, int groups, int relu)
+{
+    if (groups < 1 || C % groups || OC % groups) return -1;
+    const int icg = C / groups, ocg = OC / groups;
+    const int OD = (D + 2 * pd - (dd * (kd - 1) + 1)) / sd + 1;
+    const int OH = (H + 2 * ph - (dh * (kh - 1) + 1)) / sh + 1;
+    const int OW = (W + 2 * pw - (dw * (kw - 1) + 1)) / sw + 1;
+    if (OD <= 0 || OH <= 0 || OW <= 0) return -1;
+    const int m = OD * OH * OW, k = icg * kd * kh * kw;
+    float *col = (float *)malloc((size_t)k * m * sizeof(float));
+    if (!col) return -2;
+    for (int n = 0; n < N; ++n) {
+        for (int g = 0; g < groups; ++g) {
+            const float *xg = x + ((size_t)n * C + (size_t)g * icg) * D * H * W;
+            float *yg = y + ((size_t)n * OC + (size_t)g * ocg) * m;
+            or_im2col_3d(xg, icg, D, H, W, kd, kh, kw, pd, ph, pw, sd, sh, sw, dd, dh, dw, col);
+            or_sgemm('n', 'n', m, ocg, k, 1.0f, col, m, w + (size_t)g * ocg * k, k, 0.0f, yg, m);
+        }
+        if (bias) {
+            float *yn = y + (size_t)n * OC * m;
+            for (int oc = 0; oc < OC; ++oc)
+                for (int p = 0; p < m; ++p) yn[(size_t)oc * m + p] += 1.0f * bias[oc];
+        }
+    }
+    if (relu) {
+        const size_t len = (size_t)N * OC * m;
+        for (size_t i = 0; i < len; ++i) y[i] = (y[i] > 0) ? y[i] : 0;
+    }
+    free(col);
+    return 0;
 }
 
 /* ------------------------------------------------------------------------- */

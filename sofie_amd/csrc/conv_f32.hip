@@ -267,7 +267,86 @@ int run_conv(sofie_hip_ctx *ctx, ConvArgs &g)
    return check_launch(ctx, "k_conv2d_f32_simple");
 }
 
+struct Conv3dArgs {
+   const float *x, *w, *bias;
+   float *y;
+   int N, C, D, H, W, OC, KD, KH, KW, pd, ph, pw, sd, sh, sw, dd, dh, dw, OD, OH, OW, icg, ocg, relu;
+};
+
+// 3-D convolution, one thread per output element; the sum runs over (input channel, kd, kh, kw) in this order
+// with separately rounded products and sums, the order of the column matrix the reference multiplies
+// (Im2col_3d, SOFIE_common.hxx:522-580, then sgemm_). Consecutive threads take consecutive output columns, so the
+// input reads of a wavefront are contiguous and its weight reads are one address.
+__global__ void __launch_bounds__(256) k_conv3d_f32(Conv3dArgs g)
+{
+   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+   const size_t total = (size_t)g.N * g.OC * g.OD * g.OH * g.OW;
+   if (idx >= total) return;
+   size_t r = idx;
+   const int ow = (int)(r % g.OW); r /= g.OW;
+   const int oh = (int)(r % g.OH); r /= g.OH;
+   const int od = (int)(r % g.OD); r /= g.OD;
+   const int oc = (int)(r % g.OC);
+   const int n = (int)(r / g.OC);
+   const int grp = oc / g.ocg;
+   float acc = 0.0f;
+   for (int ic = 0; ic < g.icg; ++ic) {
+      const float *xc = g.x + ((size_t)n * g.C + grp * g.icg + ic) * g.D * g.H * g.W;
+      const float *wc = g.w + ((size_t)oc * g.icg + ic) * g.KD * g.KH * g.KW;
+      for (int kd = 0; kd < g.KD; ++kd) {
+         const int id = od * g.sd - g.pd + kd * g.dd;
+         if (id < 0 || id >= g.D) continue;
+         for (int kh = 0; kh < g.KH; ++kh) {
+            const int ih = oh * g.sh - g.ph + kh * g.dh;
+            if (ih < 0 || ih >= g.H) continue;
+            for (int kw = 0; kw < g.KW; ++kw) {
+               const int iw = ow * g.sw - g.pw + kw * g.dw;
+               if (iw < 0 || iw >= g.W) continue;
+               acc = __fadd_rn(acc, __fmul_rn(xc[((size_t)id * g.H + ih) * g.W + iw], wc[(kd * g.KH + kh) * g.KW + kw]));
+            }
+         }
+      }
+   }
+   if (g.bias) acc = __fadd_rn(acc, g.bias[oc]);
+   if (g.relu) acc = acc > 0.0f ? acc : 0.0f;
+   g.y[idx] = acc;
+}
+
 }  // namespace
+
+extern "C" int sofie_hip_conv3d_f32(sofie_hip_ctx *ctx, const float *x, const float *w, const float *bias, float *y,
+                                    int N, int C, int D, int H, int W, int OC, int KD, int KH, int KW, int pad_d,
+                                    int pad_h, int pad_w, int stride_d, int stride_h, int stride_w, int dil_d, int dil_h,
+                                    int dil_w, int groups, int act)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, N >= 0 && C > 0 && D > 0 && H > 0 && W > 0 && OC > 0 && KD > 0 && KH > 0 && KW > 0,
+                 "non-positive dimension");
+   SOFIE_REQUIRE(ctx, pad_d >= 0 && pad_h >= 0 && pad_w >= 0 && stride_d > 0 && stride_h > 0 && stride_w > 0 && dil_d > 0 &&
+                         dil_h > 0 && dil_w > 0,
+                 "bad pads/strides/dilations");
+   SOFIE_REQUIRE(ctx, groups > 0 && C % groups == 0 && OC % groups == 0, "channels not divisible by groups");
+   SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
+   const int ed = dil_d * (KD - 1) + 1, eh = dil_h * (KH - 1) + 1, ew = dil_w * (KW - 1) + 1;
+   SOFIE_REQUIRE(ctx, D + 2 * pad_d >= ed && H + 2 * pad_h >= eh && W + 2 * pad_w >= ew, "kernel larger than padded input");
+   if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && w && y, "null operand");
+   Conv3dArgs g{};
+   g.x = x; g.w = w; g.bias = bias; g.y = y;
+   g.N = N; g.C = C; g.D = D; g.H = H; g.W = W; g.OC = OC; g.KD = KD; g.KH = KH; g.KW = KW;
+   g.pd = pad_d; g.ph = pad_h; g.pw = pad_w; g.sd = stride_d; g.sh = stride_h; g.sw = stride_w;
+   g.dd = dil_d; g.dh = dil_h; g.dw = dil_w;
+   g.OD = (D + 2 * pad_d - ed) / stride_d + 1;
+   g.OH = (H + 2 * pad_h - eh) / stride_h + 1;
+   g.OW = (W + 2 * pad_w - ew) / stride_w + 1;
+   g.icg = C / groups;
+   g.ocg = OC / groups;
+   g.relu = act == SOFIE_ACT_RELU;
+   const size_t total = (size_t)N * OC * g.OD * g.OH * g.OW;
+   SOFIE_REQUIRE(ctx, total < ((size_t)1 << 38), "output too large");
+   hipLaunchKernelGGL(k_conv3d_f32, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, g);
+   return check_launch(ctx, "k_conv3d_f32");
+}
 
 extern "C" int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w, const float *bias, float *y,
                                     int N, int C, int H, int W, int OC, int KH, int KW, int pad_h, int pad_w,

@@ -1,11 +1,16 @@
-// Conv emitter (2-D). Constructor, attribute defaults, output-shape rule and error messages follow the
+// Conv emitter (1-D, 2-D and 3-D). Constructor, attribute defaults, output-shape rule and error messages follow the
 // reference's ROperator_Conv<T> (src/SOFIE_core/inc/SOFIE/ROperator_Conv.hxx:52-87,95-201,203-282):
 //   - auto_pad NOTSET with no pads attribute means 1 on every side (:136-139, not ONNX's 0);
 //   - SAME_UPPER / SAME_LOWER start from k/2 and add one at the begin / end for odd kernels (:140-158);
 //   - begin/end pads that differ are averaged with a warning (:387-401);
 //   - group == 0 means C / C_w (:110-112).
 // Emitted code: one sofie_hip_conv2d_f32 call over the whole batch (implicit GEMM, bias and
-// optional ReLU fused) instead of the per-image weight re-layout + Im2col + sgemm_ + saxpy_.
+// optional ReLU fused) instead of the per-image weight re-layout + Im2col + sgemm_ + saxpy_. A 1-D operator
+// [N,C,W] runs as the 2-D one on [N,C,1,W] (the reference does the same inside Im2col, :424-427); a 3-D one is
+// one sofie_hip_conv3d_f32 call where the reference emits Im2col_3d + sgemm_ (:432-451).
+// Dilation: the reference hands Im2col the dilated kernel extent together with the dilation (:118-122,:418-444),
+// which counts the dilation twice; here the kernel size is the weight tensor's and the dilation is applied once,
+// as ONNX defines it.
 #ifndef SOFIE_SOFIE_ROPERATOR_CONV
 #define SOFIE_SOFIE_ROPERATOR_CONV
 
@@ -18,52 +23,66 @@
 
 namespace SOFIE {
 
-// Attribute handling shared by Conv and QLinearConv.
+// Attribute handling shared by Conv and QLinearConv, for 1, 2 or 3 spatial dimensions (the reference's fDim,
+// ROperator_Conv.hxx:95-201). After Resolve every attribute vector has `dim` entries (pads 2*dim: begins, then ends).
 struct ConvGeometry {
    std::string autopad;
    std::vector<size_t> dilations, kernel, pads, strides;
    size_t group = 0;
-   // fills defaults, returns the output shape [N, OC, OH, OW] for input [N,C,H,W] and weights [OC,C/g,KH,KW]
+   size_t dim = 2;
+   // fills defaults, returns the output shape [N, OC, o1, ..] for input [N,C,i1,..] and weights [OC,C/g,k1,..]
    std::vector<size_t> Resolve(const std::vector<size_t> &x, const std::vector<size_t> &w)
    {
-      if (x.size() != 4 || w.size() != 4)
-         throw std::runtime_error("TMVA SOFIE Conv Op: only 2-D convolutions (4-D tensors) are supported by the device emission");
+      if (x.size() < 3 || x.size() > 5 || w.size() != x.size())
+         throw std::runtime_error("TMVA SOFIE Conv Op Shape inference - invalid inputs ");
+      dim = x.size() - 2;
       if (group == 0) group = x[1] / w[1];
-      size_t k1 = kernel.empty() ? w[2] : kernel[0];
-      size_t k2 = kernel.empty() ? w[3] : kernel[1];
-      if (dilations.empty()) dilations = {1, 1};
-      dilations.resize(2, 1);
+      if (!kernel.empty() && kernel.size() != dim)
+         throw std::runtime_error("TMVA SOFIE Conv Op: kernel_shape does not match the number of spatial dimensions");
+      std::vector<size_t> k(dim), extent(dim);
+      for (size_t i = 0; i < dim; ++i) k[i] = kernel.empty() ? w[i + 2] : kernel[i];
+      kernel = k;
+      if (dilations.empty()) dilations.assign(dim, 1);
+      dilations.resize(dim, 1);
       // dilated extent of the kernel
-      const size_t e1 = k1 + (dilations[0] - 1) * (k1 - 1), e2 = k2 + (dilations[1] - 1) * (k2 - 1);
-      kernel = {k1, k2};
+      for (size_t i = 0; i < dim; ++i) extent[i] = k[i] + (dilations[i] - 1) * (k[i] - 1);
       if (autopad == "NOTSET" || autopad == "") {
-         if (pads.empty()) pads = {1, 1, 1, 1};
+         if (pads.empty()) pads.assign(2 * dim, 1);
       } else if (autopad == "SAME_UPPER" || autopad == "SAME_LOWER") {
-         pads = {e1 / 2, e2 / 2, e1 / 2, e2 / 2};
-         if (e1 % 2 == 1) (autopad == "SAME_UPPER") ? pads[0]++ : pads[2]++;
-         if (e2 % 2 == 1) (autopad == "SAME_UPPER") ? pads[1]++ : pads[3]++;
+         pads.assign(2 * dim, 0);
+         for (size_t i = 0; i < dim; ++i) {
+            pads[i] = pads[dim + i] = extent[i] / 2;
+            if (extent[i] % 2 == 1) (autopad == "SAME_UPPER") ? pads[i]++ : pads[dim + i]++;
+         }
       } else if (autopad == "VALID") {
-         pads = {0, 0, 0, 0};
+         pads.assign(2 * dim, 0);
       } else {
          throw std::runtime_error("TMVA SOFIE Conv Op invalid fAutopad");
       }
-      pads.resize(4, 0);
-      if (strides.empty()) strides = {1, 1};
-      strides.resize(2, 1);
-      const size_t oh = (x[2] + pads[0] + pads[2] - e1) / strides[0] + 1;
-      const size_t ow = (x[3] + pads[1] + pads[3] - e2) / strides[1] + 1;
-      return {x[0], w[0], oh, ow};
+      pads.resize(2 * dim, 0);
+      if (strides.empty()) strides.assign(dim, 1);
+      strides.resize(dim, 1);
+      std::vector<size_t> out = {x[0], w[0]};
+      for (size_t i = 0; i < dim; ++i) out.push_back((x[i + 2] + pads[i] + pads[dim + i] - extent[i]) / strides[i] + 1);
+      return out;
    }
-   // symmetric pads handed to the kernel
+   // begin pads handed to the kernel; begin/end pads that differ are averaged with the reference's warning (:387-411)
+   std::vector<size_t> SymmetricPads()
+   {
+      bool differ = false;
+      for (size_t i = 0; i < dim; ++i) differ = differ || pads[i] != pads[dim + i];
+      if (differ) {
+         std::cout << "TMVA SOFIE Operator Conv:  asymmetric padding not supported. Assume an average padding " << std::endl;
+         for (size_t i = 0; i < dim; ++i) pads[i] = (pads[i] + pads[dim + i]) / 2;
+      }
+      return std::vector<size_t>(pads.begin(), pads.begin() + dim);
+   }
    void SymmetricPads(size_t &ph, size_t &pw)
    {
-      if (pads[0] != pads[2] || pads[1] != pads[3]) {
-         std::cout << "TMVA SOFIE Operator Conv:  asymmetric padding not supported. Assume an average padding " << std::endl;
-         pads[0] = (pads[0] + pads[2]) / 2;
-         pads[1] = (pads[1] + pads[3]) / 2;
-      }
-      ph = pads[0];
-      pw = pads[1];
+      if (dim != 2) throw std::runtime_error("TMVA SOFIE Conv Op: a 2-D convolution is expected here");
+      const auto p = SymmetricPads();
+      ph = p[0];
+      pw = p[1];
    }
 };
 
@@ -156,14 +175,13 @@ public:
       if (!model.CheckIfTensorAlreadyExist(fNX))
          throw std::runtime_error("TMVA SOFIE Conv op Input Tensor " + fNX + " is not found in model");
       fShapeX = model.GetTensorShape(fNX);
-      if (fShapeX.size() != 4)
-         throw std::runtime_error("TMVA SOFIE Conv Op input data tensor" + fNX + " is not of 4 dimensions (1-D and 3-D "
-                                  "convolutions are not supported by the device emission)");
+      if (fShapeX.size() < 3 || fShapeX.size() > 5)
+         throw std::runtime_error("TMVA SOFIE Conv Op input data tensor" + fNX + " is not of 3,4 or 5 dimensions");
       if (!model.CheckIfTensorAlreadyExist(fNW))
          throw std::runtime_error("TMVA SOFIE Conv op Input weight Tensor " + fNW + " is not found in model");
       fShapeW = model.GetTensorShape(fNW);
-      if (fShapeW.size() != 4)
-         throw std::runtime_error("TMVA SOFIE Conv Op input weight tensor" + fNW + " is not of 4 dimensions");
+      if (fShapeW.size() < 3 || fShapeW.size() > 5 || fShapeW.size() != fShapeX.size())
+         throw std::runtime_error("TMVA SOFIE Conv Op input weight tensor" + fNW + " is not of 3,4 or 5 dimensions");
       fShapeY = ShapeInference({fShapeX, fShapeW})[0];
       if (fShapeW[1] * fGeom.group != fShapeX[1])
          throw std::runtime_error("TMVA SOFIE Conv op: weight tensor " + fNW + " does not match the input channels and group");
@@ -184,16 +202,34 @@ public:
       OpName = "op_" + OpName;
       if (fShapeX.empty() || fShapeW.empty() || (fNB != "" && fShapeB.empty()) || fShapeY.empty())
          throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
-      size_t ph, pw;
-      fGeom.SymmetricPads(ph, pw);
+      const std::vector<size_t> p = fGeom.SymmetricPads();
+      const size_t dim = fGeom.dim;
+      const std::string bias = fNB.empty() ? std::string("nullptr") : "tensor_" + fNB;
+      const std::string act = fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE";
       std::stringstream out;
       out << "\n//----  operator Conv " << OpName << "\n";
-      out << SP << "Check(sofie_hip_conv2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNW << ", "
-          << (fNB.empty() ? std::string("nullptr") : "tensor_" + fNB) << ", tensor_" << fNY << ", " << fShapeX[0] << ", "
-          << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", " << fShapeW[0] << ", " << fShapeW[2] << ", "
-          << fShapeW[3] << ", " << ph << ", " << pw << ", " << fGeom.strides[0] << ", " << fGeom.strides[1] << ", "
-          << fGeom.dilations[0] << ", " << fGeom.dilations[1] << ", " << fGeom.group << ", "
-          << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << "), \"Conv " << OpName << "\");\n";
+      if (dim == 3) {
+         out << SP << "Check(sofie_hip_conv3d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNW << ", " << bias << ", tensor_" << fNY;
+         for (size_t i = 0; i < 5; ++i) out << ", " << fShapeX[i];
+         out << ", " << fShapeW[0];
+         for (size_t i = 0; i < 3; ++i) out << ", " << fShapeW[2 + i];
+         for (size_t i = 0; i < 3; ++i) out << ", " << p[i];
+         for (size_t i = 0; i < 3; ++i) out << ", " << fGeom.strides[i];
+         for (size_t i = 0; i < 3; ++i) out << ", " << fGeom.dilations[i];
+         out << ", " << fGeom.group << ", " << act << "), \"Conv " << OpName << "\");\n";
+         return out.str();
+      }
+      // one spatial dimension: a height of one, no padding and a unit stride along it
+      const bool oneD = dim == 1;
+      const size_t H = oneD ? 1 : fShapeX[2], W = fShapeX[dim + 1];
+      const size_t KH = oneD ? 1 : fShapeW[2], KW = fShapeW[dim + 1];
+      const size_t ph = oneD ? 0 : p[0], pw = p[dim - 1];
+      const size_t sh = oneD ? 1 : fGeom.strides[0], sw = fGeom.strides[dim - 1];
+      const size_t dh = oneD ? 1 : fGeom.dilations[0], dw = fGeom.dilations[dim - 1];
+      out << SP << "Check(sofie_hip_conv2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNW << ", " << bias << ", tensor_" << fNY << ", "
+          << fShapeX[0] << ", " << fShapeX[1] << ", " << H << ", " << W << ", " << fShapeW[0] << ", " << KH << ", " << KW << ", " << ph
+          << ", " << pw << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << fGeom.group << ", " << act << "), \"Conv "
+          << OpName << "\");\n";
       return out.str();
    }
 };

@@ -381,6 +381,8 @@ public:
          throw std::runtime_error("TMVA SOFIE QLinearConv Op: x and w must be int8 tensors");
       fShapeX = model.GetTensorShape(fNX);
       fShapeW = model.GetTensorShape(fNW);
+      if (fShapeX.size() != 4 || fShapeW.size() != 4)
+         throw std::runtime_error("TMVA SOFIE QLinearConv Op: only 2-D convolutions (4-D tensors) are supported");
       fShapeY = ShapeInference({fShapeX, fShapeW})[0];
       for (auto d : fGeom.dilations)
          if (d != 1) throw std::runtime_error("TMVA SOFIE QLinearConv Op: dilations are not supported");

@@ -34,6 +34,7 @@ SIGNATURES = {
     "sofie_hip_timer_stop": [_p, C.POINTER(_f)],
     "sofie_hip_gemm_f32": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i, _p, _i, _i],
     "sofie_hip_conv2d_f32": [_p, _p, _p, _p, _p] + [_i] * 15,
+    "sofie_hip_conv3d_f32": [_p, _p, _p, _p, _p] + [_i] * 20,
     "sofie_hip_conv_transpose2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,
     "sofie_hip_capture_begin": [_p],
     "sofie_hip_capture_end": [_p, _p],

@@ -141,6 +141,19 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
     return _ret(y, x)
 
 
+def conv3d_f32(x, w, bias=None, pads=(0, 0, 0), strides=(1, 1, 1), dilations=(1, 1, 1), groups=1, relu=False, ctx=None):
+    """NCDHW 3-D convolution; pads are the begin pads (d, h, w), applied on both sides."""
+    ctx = ctx or default_context()
+    xd, wd, bd = ctx.dev(x, torch.float32), ctx.dev(w, torch.float32), ctx.dev(bias, torch.float32)
+    N, Cc, D, H, W = xd.shape
+    OC, _, kd, kh, kw = wd.shape
+    out = [(i + 2 * p - (d * (k - 1) + 1)) // s + 1 for i, p, d, k, s in zip((D, H, W), pads, dilations, (kd, kh, kw), strides)]
+    y = ctx.empty((N, OC, out[0], out[1], out[2]), torch.float32)
+    ctx.check(ctx.lib.sofie_hip_conv3d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, D, H, W, OC, kd, kh, kw,
+                                           *pads, *strides, *dilations, groups, L.ACT_RELU if relu else L.ACT_NONE))
+    return _ret(y, x)
+
+
 def conv_transpose2d_f32(x, w, bias=None, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), groups=1,
                          output_padding=(0, 0), relu=False, ctx=None):
     """ONNX ConvTranspose, NCHW; w [C, OC/groups, KH, KW]; pads = (top, left, bottom, right)."""

@@ -26,6 +26,8 @@ def all_specs(with_large=True):
     specs.append(models.convbn_spec())
     specs.append(models.functor_spec())
     specs.append(models.stacked_spec())
+    specs.append(models.conv1d_spec())
+    specs.append(models.conv3d_spec())
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs

@@ -266,6 +266,55 @@ def convbn_reference(oracle):
     return oracle.conv_transpose2d_f32(n2, p["wt"], p["bt"], (1, 1, 1, 1), (2, 2), relu=True)
 
 
+# ------------------------------------------------------------------------------------------ 1-D and 3-D convolutions
+def conv1d_params(seed=51):
+    r = np.random.default_rng(seed)
+    return {"x": r.standard_normal((3, 4, 50)).astype(np.float32), "w": (r.standard_normal((6, 2, 5)) * 0.3).astype(np.float32),
+            "b": r.standard_normal(6).astype(np.float32)}
+
+
+def conv1d_spec(name="conv1d"):
+    """Conv on [3,4,50] with a [6,2,5] kernel in two groups, stride 2, dilation 2, the default pads (1 per side), then Relu."""
+    p = conv1d_params()
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", p["x"].shape)
+    s.add_init("w", p["w"])
+    s.add_init("b", p["b"])
+    s.conv("x", "w", "b", "c", (), (), (2,), (2,), 2)
+    s.relu("c", "y")
+    s.set_output("y")
+    return s
+
+
+def conv1d_reference(oracle):
+    p = conv1d_params()
+    y = oracle.conv2d_f32(p["x"][:, :, None, :], p["w"][:, :, None, :], p["b"], (0, 1), (1, 2), (1, 2), 2, relu=True)
+    return y[:, :, 0, :]
+
+
+def conv3d_params(seed=52):
+    r = np.random.default_rng(seed)
+    return {"x": r.standard_normal((2, 4, 6, 9, 10)).astype(np.float32),
+            "w": (r.standard_normal((6, 2, 3, 2, 3)) * 0.3).astype(np.float32), "b": r.standard_normal(6).astype(np.float32)}
+
+
+def conv3d_spec(name="conv3d"):
+    """Conv on [2,4,6,9,10] with a [6,2,3,2,3] kernel in two groups, strides (1,2,1), pads (1,0,2) on both sides."""
+    p = conv3d_params()
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", p["x"].shape)
+    s.add_init("w", p["w"])
+    s.add_init("b", p["b"])
+    s.conv("x", "w", "b", "y", (3, 2, 3), (1, 0, 2, 1, 0, 2), (1, 2, 1), (), 2)
+    s.set_output("y")
+    return s
+
+
+def conv3d_reference(oracle):
+    p = conv3d_params()
+    return oracle.conv3d_f32(p["x"], p["w"], p["b"], (1, 0, 2), (1, 2, 1), (1, 1, 1), 2)
+
+
 # ------------------------------------------------------------------------------------------ four-value model for SofieFunctor
 def functor_params(seed=33):
     r = np.random.default_rng(seed)

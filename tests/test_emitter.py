@@ -413,6 +413,33 @@ def test_einsum_matrix_products_become_gemm_calls_everything_else_one_kernel_cal
     assert "_stride[] = {6};" in c
 
 
+def test_conv_1d_and_3d_emission(tmp_path):
+    """One spatial dimension runs as the 2-D call with a height of one; three as the 3-D call. Absent pads mean one
+    on every side of every dimension, as in the reference (ROperator_Conv.hxx:136-139)."""
+    c = open(models.conv1d_spec("c1d_t").generate(str(tmp_path))[0]).read()
+    # [3,4,50], kernel 5 dilated by 2 (extent 9), pads 1+1, stride 2: (50 + 2 - 9) / 2 + 1 = 22
+    assert "sofie_hip_conv2d_f32(fCtx, tensor_x, tensor_w, tensor_b, tensor_c, 3, 4, 1, 50, 6, 1, 5, 0, 1, 1, 2, 1, 2, 2, SOFIE_ACT_RELU)" in c
+    assert "std::vector<float> ret(396);" in c
+    c = open(models.conv3d_spec("c3d_t").generate(str(tmp_path))[0]).read()
+    assert ("sofie_hip_conv3d_f32(fCtx, tensor_x, tensor_w, tensor_b, tensor_y, 2, 4, 6, 9, 10, 6, 3, 2, 3, 1, 0, 2, 1, 2, 1, 1, 1, 1, 2, "
+            "SOFIE_ACT_NONE)") in c
+    # (6 + 2 - 3) + 1 = 6, (9 - 2) / 2 + 1 = 4, (10 + 4 - 3) + 1 = 12
+    assert "std::vector<float> ret(%d);" % (2 * 6 * 6 * 4 * 12) in c
+    s = emit.ModelSpec("c3d_def")
+    s.add_input("x", "FLOAT", (1, 1, 4, 4, 4))
+    s.add_init("w", np.ones((2, 1, 3, 3, 3), np.float32))
+    s.conv("x", "w", None, "y")
+    s.set_output("y")
+    c = open(s.generate(str(tmp_path))[0]).read()
+    assert "1, 1, 4, 4, 4, 2, 3, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1, SOFIE_ACT_NONE" in c
+    bad = emit.ModelSpec("c_rank")
+    bad.add_input("x", "FLOAT", (1, 1, 4, 4))
+    bad.add_init("w", np.ones((2, 1, 3), np.float32))
+    bad.conv("x", "w", None, "y")
+    bad.set_output("y")
+    assert "is not of 3,4 or 5 dimensions" in emit_error(bad, tmp_path)
+
+
 def test_einsum_errors(tmp_path):
     assert "Error parsing the equation ik,kj" in emit_error(_einsum_spec("ee1", "ik,kj", [(2, 3), (3, 2)]), tmp_path)
     assert "Error parsing the equation" in emit_error(_einsum_spec("ee2", "ik->i", [(2, 3), (3, 2)]), tmp_path)

@@ -74,6 +74,17 @@ def test_cnn_f32_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
+def test_conv_1d_and_3d_sessions(tmp_path):
+    """A 1-D convolution runs on the 2-D kernel with a height of one (1e-5 relative); the 3-D kernel sums in the
+    order of the reference's column matrix, so it equals the oracle exactly."""
+    y = run_session("conv1d", models.conv1d_params()["x"], tmp_path)
+    ref = models.conv1d_reference(oracle)
+    assert y.size == ref.size and rel_err(y, ref.reshape(-1)) <= 1e-5
+    y = run_session("conv3d", models.conv3d_params()["x"], tmp_path)
+    ref = models.conv3d_reference(oracle)
+    assert y.size == ref.size and np.array_equal(y, ref.reshape(-1))
+
+
 def test_conv_batchnorm_convtranspose_session(tmp_path):
     """Conv -> BatchNormalization -> Relu (folded into the convolution at generation time) -> MaxPool ->
     BatchNormalization (its own kernel) -> ConvTranspose -> Relu against the unfused oracle steps; 1e-5 relative

@@ -747,3 +747,24 @@ def test_einsum_matrix_products_through_the_gemm_kernel(ops, eq, shapes):
     assert rel_err(y, ref) <= FP32_TOL
     xi = [r.integers(-4, 5, s).astype(np.float32) for s in shapes]
     assert np.array_equal(ops.einsum_f32(eq, xi), oracle.einsum_f32(eq, xi))
+
+
+# --------------------------------------------------------------------------- 3-D convolution
+@pytest.mark.parametrize("cfg", [
+    # N, C, D, H, W, OC, k, pads, strides, dilations, groups
+    (2, 3, 5, 6, 7, 4, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    (1, 4, 8, 9, 33, 6, (2, 3, 1), (0, 1, 0), (2, 1, 3), (1, 2, 1), 2),
+    (3, 8, 4, 4, 70, 8, (1, 1, 5), (0, 0, 2), (1, 1, 1), (1, 1, 3), 8),
+    (1, 1, 1, 1, 1, 1, (1, 1, 1), (0, 0, 0), (1, 1, 1), (1, 1, 1), 1),
+])
+def test_conv3d_f32_matches_the_column_matrix_order(ops, cfg):
+    N, C, D, H, W, OC, k, pads, strides, dil, groups = cfg
+    r = rng(900 + C + W)
+    x = r.standard_normal((N, C, D, H, W)).astype(np.float32)
+    w = r.standard_normal((OC, C // groups) + k).astype(np.float32)
+    b = r.standard_normal(OC).astype(np.float32)
+    for bias, relu in ((b, True), (None, False)):
+        y = ops.conv3d_f32(x, w, bias, pads, strides, dil, groups, relu=relu)
+        ref = oracle.conv3d_f32(x, w, bias, pads, strides, dil, groups, relu=relu)
+        assert y.shape == ref.shape
+        assert np.array_equal(y, ref)

@@ -339,3 +339,27 @@ def test_einsum_sums_in_label_order():
     assert float(oracle.einsum_f32("ab->", [x])) == 1.0
     # with the labels renamed so that the second axis sorts first, the loop order turns around: (big - big) + 1 + 1 = 2
     assert float(oracle.einsum_f32("ba->", [x])) == 2.0
+
+
+@pytest.mark.parametrize("cfg", [
+    (2, 3, 5, 6, 7, 4, (3, 3, 3), (1, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+    (1, 4, 8, 9, 10, 6, (2, 3, 1), (0, 1, 0), (2, 1, 3), (1, 2, 1), 2),
+    (2, 6, 4, 4, 12, 6, (1, 1, 5), (0, 0, 2), (1, 1, 1), (1, 1, 2), 6),
+])
+def test_conv3d_f32_against_torch_and_depth_one_conv2d(cfg):
+    import torch
+    N, C, D, H, W, OC, k, pads, strides, dil, groups = cfg
+    r = np.random.default_rng(700 + C + W)
+    x = r.standard_normal((N, C, D, H, W)).astype(np.float32)
+    w = r.standard_normal((OC, C // groups) + k).astype(np.float32)
+    b = r.standard_normal(OC).astype(np.float32)
+    y = oracle.conv3d_f32(x, w, b, pads, strides, dil, groups)
+    t = torch.nn.functional.conv3d(torch.from_numpy(x).double(), torch.from_numpy(w).double(), torch.from_numpy(b).double(),
+                                   strides, pads, dil, groups).numpy()
+    assert y.shape == t.shape
+    assert np.max(np.abs(y - t)) <= 1e-5 * np.max(np.abs(t))
+    # a depth of one with a depth-one kernel is the 2-D convolution, term by term
+    x2, w2 = x[:, :, :1], w[:, :, :1]
+    y3 = oracle.conv3d_f32(x2, w2, b, (0,) + tuple(pads[1:]), (1,) + tuple(strides[1:]), (1,) + tuple(dil[1:]), groups, relu=True)
+    y2 = oracle.conv2d_f32(x2[:, :, 0], w2[:, :, 0], b, pads[1:], strides[1:], dil[1:], groups, relu=True)
+    assert np.array_equal(y3[:, :, 0], y2)
