@@ -11,6 +11,8 @@
 // consecutive pixels of one channel plane: coalesced NCHW stores, bias and ReLU fused.
 // Roofline: MFMA fp32; per K-step of 2 each wavefront issues TI*TJ MFMAs (64 cycles each)
 // against TI+TJ+1 ds_read_b32.
+#include <type_traits>
+
 #include "common.h"
 
 using namespace sofie;
@@ -36,7 +38,8 @@ struct ConvArgs {
    // phase (oy mod stride, ox mod stride), each with the taps that reach that phase and no zeros in between.
    int KH0, KW0, th0, ths, tw0, tws;
    int OH0, OW0, oy0, oys, ox0, oxs;
-   FastDiv dPW, dPH, dKC;   // divisions by the patch extents and the K-chunk length in the staging loops
+   int wvec;           // weights are staged with 16-byte loads (see launch)
+   FastDiv dPW, dPH, dKC, dK4;   // divisions by the patch extents and the K-chunk length (/4) in the staging loops
    FastDiv dUH, dUW, dOW;
 };
 
@@ -49,7 +52,9 @@ __device__ __forceinline__ int source_index(int up, int u, FastDiv d)
    return q * u == up ? q : -1;
 }
 
-template <int TI, int TJ>
+// TR: the launch is (a phase of) a transposed convolution; the plain convolution is compiled without the tap and
+// output maps.
+template <int TI, int TJ, bool TR>
 __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
 {
    constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
@@ -102,33 +107,95 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       const int icn = (g.icg - ic0) < g.ICB ? (g.icg - ic0) : g.ICB;
       const int kc = icn * KHW;
       __syncthreads();   // previous chunk fully consumed (also orders the koff table on entry)
-      for (int e = tid; e < patch_len; e += 256) {
-         const int t = fdiv(e, g.dPW), c = e - t * g.PW;
-         const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
-         int ih = ih0 + r, iw = iw0 + c;
-         if (g.transposed) {
-            ih = source_index(ih, g.uh, g.dUH);
-            iw = source_index(iw, g.uw, g.dUW);
-         }
-         float v = 0.0f;
-         if (icl < icn && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W)
-            v = xg[((size_t)(ic0 + icl) * g.H + ih) * g.W + iw];
-         patch[e] = v;
-      }
-      for (int e = tid; e < g.KC * BOC; e += 256) {
-         const int ocl = fdiv(e, g.dKC), k = e - ocl * g.KC;
-         float v = 0.0f;
-         if (k < kc && oc0 + ocl < g.ocg) {
-            if (g.transposed) {
-               const int icl = k / KHW, t = k - icl * KHW;
-               const int ta = t / g.KW, tb = t - ta * g.KW;
-               v = g.w[((((size_t)grp * g.icg + ic0 + icl) * g.ocg + oc0 + ocl) * g.KH0 + g.th0 + ta * g.ths) * g.KW0 + g.tw0 +
-                       tb * g.tws];
-            } else {
-               v = wg[(size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k];
+      // Staging: every load of a batch is issued before the first value is used (the addresses of cells outside the
+      // image, channels past the block and columns past the group are clamped to element 0 and the value replaced
+      // by zero afterwards), so a batch costs one memory latency instead of one per element.
+      auto stage_patch = [&](auto batch) {
+         constexpr int UP = decltype(batch)::value;
+         for (int e0 = 0; e0 < patch_len; e0 += 256 * UP) {
+            float v[UP];
+            bool inside[UP];
+#pragma unroll
+            for (int u = 0; u < UP; ++u) {
+               const int e = e0 + u * 256 + tid;
+               const int t = fdiv(e, g.dPW), c = e - t * g.PW;
+               const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
+               int ih = ih0 + r, iw = iw0 + c;
+               if constexpr (TR) {
+                  ih = source_index(ih, g.uh, g.dUH);
+                  iw = source_index(iw, g.uw, g.dUW);
+               }
+               inside[u] = e < patch_len && icl < icn && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+               v[u] = xg[inside[u] ? ((size_t)(ic0 + icl) * g.H + ih) * g.W + iw : 0];
+            }
+#pragma unroll
+            for (int u = 0; u < UP; ++u) {
+               const int e = e0 + u * 256 + tid;
+               if (e < patch_len) patch[e] = inside[u] ? v[u] : 0.0f;
             }
          }
-         sW[k * LDW + ocl] = v;
+      };
+      // six loads per thread and batch: twelve (one batch for a 3x3 block of eight channels) costs a workgroup per CU
+      // in registers and measured 14 % slower
+      stage_patch(std::integral_constant<int, 6>{});
+      if (!TR && g.wvec) {
+         // four consecutive k of one output channel per 16-byte load (every block is full and 16-byte aligned)
+         const int K4 = g.KC >> 2, total4 = K4 * BOC;
+         auto stage_weights4 = [&](auto batch) {
+            constexpr int UW = decltype(batch)::value;
+            for (int e0 = 0; e0 < total4; e0 += 256 * UW) {
+               v4f v[UW];
+               int dst[UW];
+#pragma unroll
+               for (int u = 0; u < UW; ++u) {
+                  const int e = e0 + u * 256 + tid;
+                  const int ocl = fdiv(e, g.dK4), k4 = e - ocl * K4;
+                  const bool ok = e < total4 && oc0 + ocl < g.ocg;
+                  v[u] = *reinterpret_cast<const v4f *>(wg + (ok ? (size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + 4 * k4 : 0));
+                  if (!ok) v[u] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+                  dst[u] = e < total4 ? 4 * k4 * LDW + ocl : -1;
+               }
+#pragma unroll
+               for (int u = 0; u < UW; ++u) {
+                  if (dst[u] >= 0) {
+#pragma unroll
+                     for (int q = 0; q < 4; ++q) sW[dst[u] + q * LDW] = v[u][q];
+                  }
+               }
+            }
+         };
+         stage_weights4(std::integral_constant<int, 3>{});
+      } else {
+         constexpr int UW = 8;
+         const int total = g.KC * BOC;
+         for (int e0 = 0; e0 < total; e0 += 256 * UW) {
+            float v[UW];
+            bool ok[UW];
+#pragma unroll
+            for (int u = 0; u < UW; ++u) {
+               const int e = e0 + u * 256 + tid;
+               const int ocl = fdiv(e, g.dKC), k = e - ocl * g.KC;
+               ok[u] = e < total && k < kc && oc0 + ocl < g.ocg;
+               size_t off = 0;
+               if (ok[u]) {
+                  if constexpr (TR) {
+                     const int icl = k / KHW, t = k - icl * KHW;
+                     const int ta = t / g.KW, tb = t - ta * g.KW;
+                     off = ((((size_t)grp * g.icg + ic0 + icl) * g.ocg + oc0 + ocl) * g.KH0 + g.th0 + ta * g.ths) * g.KW0 + g.tw0 +
+                           tb * g.tws;
+                  } else {
+                     off = (size_t)grp * g.ocg * Kfull + (size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k;
+                  }
+               }
+               v[u] = g.w[off];
+            }
+#pragma unroll
+            for (int u = 0; u < UW; ++u) {
+               const int e = e0 + u * 256 + tid;
+               const int ocl = fdiv(e, g.dKC), k = e - ocl * g.KC;
+               if (e < total) sW[k * LDW + ocl] = ok[u] ? v[u] : 0.0f;
+            }
+         }
       }
       __syncthreads();
       const float *wrow = sW + wm * TI * 32 + fr;
@@ -148,7 +215,7 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       }
    }
 
-   const size_t plane = (size_t)g.OH0 * g.OW0;
+   const size_t plane = TR ? (size_t)g.OH0 * g.OW0 : (size_t)OHW;
    float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane;
 #pragma unroll
    for (int i = 0; i < TI; ++i)
@@ -156,8 +223,11 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       for (int j = 0; j < TJ; ++j) {
          const int p = p0 + wn * TJ * 32 + j * 32 + fr;
          if (p >= OHW) continue;
-         const int q = fdiv(p, g.dOW);
-         const size_t po = (size_t)(g.oy0 + q * g.oys) * g.OW0 + g.ox0 + (p - q * g.OW) * g.oxs;
+         size_t po = (size_t)p;
+         if constexpr (TR) {
+            const int q = fdiv(p, g.dOW);
+            po = (size_t)(g.oy0 + q * g.oys) * g.OW0 + g.ox0 + (p - q * g.OW) * g.oxs;
+         }
 #pragma unroll
          for (int r = 0; r < 16; ++r) {
             const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
@@ -236,9 +306,14 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    g.dPW = make_fastdiv((unsigned)g.PW);
    g.dPH = make_fastdiv((unsigned)g.PH);
    g.dKC = make_fastdiv((unsigned)g.KC);
+   g.dK4 = make_fastdiv((unsigned)(g.KC >= 4 ? g.KC / 4 : 1));
+   // 16-byte weight loads: every channel block full (no k past the block inside a load), blocks and rows of the
+   // [OC, K] matrix 16-byte aligned
+   g.wvec = !g.transposed && g.icg % g.ICB == 0 && g.KC == g.ICB * KHW && g.KC % 4 == 0 && (g.icg * KHW) % 4 == 0 &&
+            (reinterpret_cast<uintptr_t>(g.w) & 15u) == 0;
    const int octiles = cdiv(g.ocg, BOC);
    if ((size_t)g.groups * octiles > 65535 || g.N > 65535) return SOFIE_HIP_OK;
-   auto kern = k_conv2d_f32<TI, TJ>;
+   auto kern = g.transposed ? k_conv2d_f32<TI, TJ, true> : k_conv2d_f32<TI, TJ, false>;
    SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
    hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, g);
