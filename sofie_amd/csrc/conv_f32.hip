@@ -19,6 +19,10 @@ using namespace sofie;
 
 namespace {
 
+// Most values of a channel block that the threads of a workgroup carry in registers in k_conv2d_f32_pipe.
+#define SOFIE_CONV_PIPE_PATCH 1536
+#define SOFIE_CONV_PIPE_WEIGHTS 5120
+
 struct ConvArgs {
    const float *x, *w, *bias;
    float *y;
@@ -240,6 +244,156 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       }
 }
 
+// The same implicit GEMM with the staging of channel block c+1 under the matrix loop of block c: the loads of the
+// next block are issued into registers before the loop and written to the other LDS buffer after it, one barrier
+// per block. Blocks are small enough for a thread to carry its share: at most NP patch values and NW weights
+// (the launcher picks the channels per block accordingly and falls back to k_conv2d_f32 otherwise). Plain
+// convolutions only.
+template <int TI, int TJ>
+__global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs g)
+{
+   constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
+   constexpr int NP = SOFIE_CONV_PIPE_PATCH / 256, NW = SOFIE_CONV_PIPE_WEIGHTS / 256;
+   extern __shared__ __align__(16) unsigned char smem_raw[];
+   const int patch_len = g.ICB * g.PH * g.PW;
+   const int buf_len = g.KC * LDW + patch_len;                       // floats of one buffer: [KC][LDW] weights, patch
+   float *const bufs = reinterpret_cast<float *>(smem_raw);
+   int *const koff = reinterpret_cast<int *>(bufs + 2 * buf_len);    // [KC]
+
+   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int wm = wave >> 1, wn = wave & 1;
+   const int fr = lane & 31, fk = lane >> 5;
+   const int octiles = (g.ocg + BOC - 1) / BOC;
+   const int grp = blockIdx.y / octiles;
+   const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
+   const int n = blockIdx.z;
+   const int OHW = g.OH * g.OW;
+   const int p0 = blockIdx.x * BP;
+   const int oh0 = p0 / g.OW;
+   const int ih0 = oh0 * g.sh - g.ph, iw0 = -g.pw;
+   const int KHW = g.KH * g.KW;
+   const int Kfull = g.icg * KHW;
+
+   for (int k = tid; k < g.KC; k += 256) {
+      const int icl = k / KHW, t = k % KHW;
+      const int kh = t / g.KW, kw = t % g.KW;
+      koff[k] = (icl < g.ICB) ? (icl * g.PH + kh * g.dh) * g.PW + kw * g.dw : 0;
+   }
+   int base[TJ];
+#pragma unroll
+   for (int j = 0; j < TJ; ++j) {
+      const int p = p0 + wn * TJ * 32 + j * 32 + fr;
+      base[j] = (p < OHW) ? ((p / g.OW - oh0) * g.sh) * g.PW + (p % g.OW) * g.sw : 0;
+   }
+   v16f acc[TI][TJ];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+#pragma unroll
+         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+   const float *xg = g.x + ((size_t)n * g.C + (size_t)grp * g.icg) * g.H * g.W;
+   const float *wg = g.w + (size_t)grp * g.ocg * Kfull;
+   const int K4 = g.KC >> 2;
+
+   // a thread's share of one channel block, in registers between issue() and commit()
+   float pv[NP], wreg[NW];
+   unsigned pmask = 0, wmask = 0;
+   auto issue = [&](int ic0) {
+      const int icn = (g.icg - ic0) < g.ICB ? (g.icg - ic0) : g.ICB;
+      pmask = 0;
+      wmask = 0;
+#pragma unroll
+      for (int u = 0; u < NP; ++u) {
+         const int e = u * 256 + tid;
+         const int t = fdiv(e, g.dPW), c = e - t * g.PW;
+         const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
+         const int ih = ih0 + r, iw = iw0 + c;
+         const bool inside = e < patch_len && icl < icn && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+         // loads are unconditional (of element 0 where the cell is padding or past the block)
+         pv[u] = xg[inside ? ((size_t)(ic0 + icl) * g.H + ih) * g.W + iw : 0];
+         pmask |= inside ? (1u << u) : 0u;
+      }
+      // weights: four consecutive k of one output channel per 16-byte load (the launcher guarantees full,
+      // 16-byte aligned blocks)
+#pragma unroll
+      for (int u = 0; u < NW / 4; ++u) {
+         const int e = u * 256 + tid;
+         const int ocl = fdiv(e, g.dK4), k4 = e - ocl * K4;
+         const bool ok = e < K4 * BOC && oc0 + ocl < g.ocg;
+         const v4f v = *reinterpret_cast<const v4f *>(wg + (ok ? (size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + 4 * k4 : 0));
+#pragma unroll
+         for (int q = 0; q < 4; ++q) wreg[4 * u + q] = v[q];
+         wmask |= ok ? (1u << u) : 0u;
+      }
+   };
+   auto commit = [&](float *buf) {
+      float *const sW = buf, *const patch = buf + g.KC * LDW;
+#pragma unroll
+      for (int u = 0; u < NP; ++u) {
+         const int e = u * 256 + tid;
+         if (e < patch_len) patch[e] = ((pmask >> u) & 1u) ? pv[u] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < NW / 4; ++u) {
+         const int e = u * 256 + tid;
+         const int ocl = fdiv(e, g.dK4), k4 = e - ocl * K4;
+         if (e < K4 * BOC) {
+            const bool ok = (wmask >> u) & 1u;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) sW[(4 * k4 + q) * LDW + ocl] = ok ? wreg[4 * u + q] : 0.0f;
+         }
+      }
+   };
+
+   const int nblocks = (g.icg + g.ICB - 1) / g.ICB;
+   issue(0);
+   commit(bufs);
+   __syncthreads();   // block 0 and the koff table are in LDS
+   for (int c = 0; c < nblocks; ++c) {
+      const bool more = c + 1 < nblocks;
+      if (more) issue((c + 1) * g.ICB);
+      const float *const sW = bufs + (c & 1) * buf_len, *const patch = sW + g.KC * LDW;
+      const float *wrow = sW + wm * TI * 32 + fr;
+      for (int s = 0; s < g.KC / 2; ++s) {
+         const int kk = 2 * s + fk;
+         const int ko = koff[kk];
+         float fa[TI], fb[TJ];
+#pragma unroll
+         for (int i = 0; i < TI; ++i) fa[i] = wrow[kk * LDW + i * 32];
+#pragma unroll
+         for (int j = 0; j < TJ; ++j) fb[j] = patch[base[j] + ko];
+#pragma unroll
+         for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+      // the other buffer was last read in block c-1, before the barrier that ended it
+      if (more) commit(bufs + ((c + 1) & 1) * buf_len);
+      __syncthreads();
+   }
+
+   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * OHW;
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) {
+         const int p = p0 + wn * TJ * 32 + j * 32 + fr;
+         if (p >= OHW) continue;
+#pragma unroll
+         for (int r = 0; r < 16; ++r) {
+            const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
+            if (oc >= g.ocg) continue;
+            float v = acc[i][j][r];
+            if (g.bias) v = __fadd_rn(v, g.bias[grp * g.ocg + oc]);
+            if (g.relu) v = v > 0.0f ? v : 0.0f;
+            yn[(size_t)oc * OHW + p] = v;
+         }
+      }
+}
+
 // One thread per output element: any kernel size, used when the staged patch of the tiled
 // kernel would not fit LDS.
 __global__ void k_conv2d_f32_simple(ConvArgs g)
@@ -289,6 +443,35 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    // keep the matrix cores busy. Measured on 256x64x56x56 -> 128, 3x3: 2.66 ms at 64 KB, 1.99 ms at 52 KB.
    const size_t budget = 52 * 1024;
    *done = false;
+   const int octiles = cdiv(g.ocg, BOC);
+   if ((size_t)g.groups * octiles > 65535 || g.N > 65535) return SOFIE_HIP_OK;
+   if (!g.transposed) {
+      // staging under the matrix loop: the largest channel block whose two LDS buffers fit the budget and whose
+      // values fit the registers the kernel sets aside; at least nine K-steps of matrix work per block
+      for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
+         const int kc = (icb * KHW + 1) & ~1;
+         const size_t plen = (size_t)icb * g.PH * g.PW;
+         const size_t lds = (2 * ((size_t)kc * LDW + plen) + kc) * 4;
+         if (kc < 18) break;
+         if (lds > budget || (size_t)kc * BOC > SOFIE_CONV_PIPE_WEIGHTS || plen > SOFIE_CONV_PIPE_PATCH) continue;
+         g.ICB = icb;
+         g.KC = kc;
+         g.dPW = make_fastdiv((unsigned)g.PW);
+         g.dPH = make_fastdiv((unsigned)g.PH);
+         g.dKC = make_fastdiv((unsigned)g.KC);
+         g.dK4 = make_fastdiv((unsigned)(g.KC / 4));
+         // 16-byte weight loads only: every block full, blocks and rows of the [OC, K] matrix 16-byte aligned
+         g.wvec = g.icg % g.ICB == 0 && g.KC == g.ICB * KHW && g.KC % 4 == 0 && (g.icg * KHW) % 4 == 0 &&
+                  (reinterpret_cast<uintptr_t>(g.w) & 15u) == 0;
+         if (!g.wvec) continue;
+         auto kern = k_conv2d_f32_pipe<TI, TJ>;
+         SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+         hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, g);
+         *done = true;
+         return check_launch(ctx, "k_conv2d_f32_pipe");
+      }
+   }
    int icb = 96 / KHW;
    if (icb < 1) icb = 1;
    if (icb > g.icg) icb = g.icg;
@@ -311,8 +494,6 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    // [OC, K] matrix 16-byte aligned
    g.wvec = !g.transposed && g.icg % g.ICB == 0 && g.KC == g.ICB * KHW && g.KC % 4 == 0 && (g.icg * KHW) % 4 == 0 &&
             (reinterpret_cast<uintptr_t>(g.w) & 15u) == 0;
-   const int octiles = cdiv(g.ocg, BOC);
-   if ((size_t)g.groups * octiles > 65535 || g.N > 65535) return SOFIE_HIP_OK;
    auto kern = g.transposed ? k_conv2d_f32<TI, TJ, true> : k_conv2d_f32<TI, TJ, false>;
    SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
