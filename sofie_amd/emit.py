@@ -30,7 +30,7 @@ def build_emitter():
 
 def _lst(v):
     v = list(v)
-    return "%d %s" % (len(v), " ".join(str(int(x)) for x in v)) if v else "0"
+    return "%d %s" % (len(v), " ".join(str(x) if isinstance(x, str) else str(int(x)) for x in v)) if v else "0"
 
 
 class ModelSpec:
@@ -44,6 +44,8 @@ class ModelSpec:
         self.inputs = []
         self.output = None
         self.out_type = "FLOAT"
+        self.batch = None            # value of the inputs' shape parameters at generation time
+        self.runtime_batch = False   # ... as a capacity: the Session also takes infer(n, ...)
 
     def add_input(self, name, dtype, shape):
         t = dtype if isinstance(dtype, str) else _TYPE[np.dtype(dtype)]
@@ -117,8 +119,11 @@ class ModelSpec:
         self.lines.append("op GemmFP8 %s %s %s %s %s %s %d" % (a, a_scale, b, b_scale, bias or "-", y, transB))
 
     # ---- generation ------------------------------------------------------------------------
-    def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False):
-        """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess)."""
+    def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False, batch=None,
+                 runtime_batch=False):
+        """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess). `batch` gives the shape
+        parameters of the inputs (dimensions written as names) their value; with `runtime_batch` it is a capacity and
+        the generated Session also takes infer(n, ...) for any n up to it."""
         os.makedirs(outdir, exist_ok=True)
         tdir = os.path.join(outdir, "tensors")
         os.makedirs(tdir, exist_ok=True)
@@ -127,6 +132,11 @@ class ModelSpec:
         spec = os.path.join(outdir, self.name + ".spec")
         with open(spec, "w") as f:
             flag = " noweightfile" if no_weight_file else (" binaryweightfile" if binary_weight_file else "")
+            batch = self.batch if batch is None else batch
+            if batch is not None:
+                flag += " batch %d" % batch
+            if runtime_batch or self.runtime_batch:
+                flag += " runtimebatch"
             f.write("\n".join(self.lines + ["generate" + flag]) + "\n")
         if not os.path.exists(EMIT):
             build_emitter()
@@ -138,13 +148,15 @@ class ModelSpec:
         return (os.path.join(outdir, self.name + ".hxx"),
                 os.path.join(outdir, self.name + (".bin" if binary_weight_file else ".dat")), res)
 
-    def compile_runner(self, outdir=GEN_DIR):
-        """g++ the generic runner against the generated header and libsofie_hip.so."""
+    def compile_runner(self, outdir=GEN_DIR, runtime_batch=False):
+        """g++ the generic runner against the generated header and libsofie_hip.so. With runtime_batch the runner's
+        fourth argument is the batch it hands to infer(n, ...)."""
         exe = os.path.join(outdir, "run_" + self.name)
         cmd = ["g++", "-std=c++17", "-O2", "-I" + os.path.join(ROOT, "include"), "-I" + outdir,
                "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % self.name, "-DSOFIE_MODEL_NS=SOFIE_%s" % self.name,
                "-DSOFIE_IN_T=%s" % _CTYPE[self.input[1]], "-DSOFIE_OUT_T=%s" % _CTYPE[self.out_type],
-               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs),
+               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs)] + \
+              (["-DSOFIE_RUNTIME_BATCH"] if (runtime_batch or self.runtime_batch) else []) + [
                os.path.join(_HERE, "host", "examples", "run_session.cxx"), "-o", exe,
                "-L" + _HERE, "-lsofie_hip", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath," + _HERE]
         res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -7,7 +7,7 @@
 //
 // Statements (one per line, '-' stands for "absent"):
 //   model NAME
-//   input NAME TYPE RANK d0 d1 ...
+//   input NAME TYPE RANK d0 d1 ...                 a dimension that is not a number is a shape parameter (e.g. bs)
 //   init NAME TYPE RANK d0 d1 ... FILE           raw little-endian values
 //   output NAME
 //   op Gemm ALPHA BETA TRANSA TRANSB A B C Y RELU
@@ -22,7 +22,9 @@
 //   op QLinearMatMul A AS AZ B BS BZ YS YZ BIAS Y TRANSB
 //   op QLinearConv AUTOPAD GROUP nk k.. np p.. ns s.. X XS XZ W WS WZ YS YZ BIAS Y
 //   op GemmFP8 A AS B BS BIAS Y TRANSB
-//   generate [noweightfile]
+//   generate [noweightfile | binaryweightfile] [batch N] [runtimebatch]
+//                                                  batch N resolves the shape parameters; runtimebatch makes N a capacity
+#include <cctype>
 #include <fstream>
 #include <iostream>
 #include <sstream>
@@ -74,8 +76,18 @@ int main(int argc, char **argv)
             model.reset(new RModel(name + ".onnx", "generated from a model description \n"));
          } else if (kw == "input") {
             std::string n, t;
-            in >> n >> t;
-            model->AddInputTensorInfo(n, TypeOf(t), List(in));
+            size_t rank;
+            in >> n >> t >> rank;
+            std::vector<Dim> dims;
+            bool parametric = false;
+            for (size_t i = 0; i < rank; ++i) {
+               std::string tok;
+               in >> tok;
+               if (!tok.empty() && std::isdigit(static_cast<unsigned char>(tok[0]))) dims.push_back(Dim{(size_t)std::stoull(tok)});
+               else { dims.push_back(Dim{tok}); parametric = true; }
+            }
+            if (parametric) model->AddInputTensorInfo(n, TypeOf(t), dims);
+            else model->AddInputTensorInfo(n, TypeOf(t), ConvertShapeToInt(dims));
             model->AddInputTensorName(n);
          } else if (kw == "init") {
             std::string n, t, file;
@@ -178,11 +190,16 @@ int main(int argc, char **argv)
             if (!in) throw std::runtime_error("malformed statement: " + line);
             model->AddOperator(std::move(r), order++);
          } else if (kw == "generate") {
-            std::string flag;
-            in >> flag;
-            if (flag == "noweightfile") model->Generate(Options::kNoWeightFile);
-            else if (flag == "binaryweightfile") model->Generate(Options::kBinaryWeightFile);
-            else model->Generate();
+            std::underlying_type_t<Options> options = static_cast<std::underlying_type_t<Options>>(Options::kDefault);
+            int batch = -1;
+            for (std::string flag; in >> flag;) {
+               if (flag == "noweightfile") options = options | Options::kNoWeightFile;
+               else if (flag == "binaryweightfile") options = options | Options::kBinaryWeightFile;
+               else if (flag == "runtimebatch") options = options | Options::kRuntimeBatch;
+               else if (flag == "batch") in >> batch;
+               else throw std::runtime_error("unknown generate flag " + flag);
+            }
+            model->Generate(options, batch);
             model->OutputGenerated(odir + "/" + name + ".hxx");
             std::cout << "generated " << odir << "/" << name << ".hxx, intermediate pool " << model->GetIntermediateMemorySize()
                       << " bytes\n";

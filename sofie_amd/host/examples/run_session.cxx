@@ -2,7 +2,9 @@
 // Compile with -DSOFIE_MODEL_HEADER='"x.hxx"' -DSOFIE_MODEL_NS=SOFIE_x -DSOFIE_IN_T=float -DSOFIE_OUT_T=float -DSOFIE_INPUT_MEMBER=fInput_x
 // and, for a model with several inputs, -DSOFIE_NUM_INPUTS=n (then <input.bin> is a comma-separated list, one file per input
 // in the order of infer()'s arguments, and there is no timing).
-//   run_session <weights.dat> <input.bin> <output.bin> [timed iterations of infer_device]
+// With -DSOFIE_RUNTIME_BATCH (a Session generated with Options::kRuntimeBatch) the fourth argument is the batch: the
+// runner calls infer(batch, input) and writes that many rows.
+//   run_session <weights.dat> <input.bin> <output.bin> [timed iterations of infer_device | batch]
 #include <chrono>
 #include <cstdio>
 #include <cstring>
@@ -60,10 +62,17 @@ int main(int argc, char **argv)
       fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
 #else
       std::vector<SOFIE_IN_T> x = ReadRaw(argv[2]);
+#ifdef SOFIE_RUNTIME_BATCH
+      std::vector<SOFIE_OUT_T> y = argc > 4 ? s.infer((size_t)std::atoi(argv[4]), x.data()) : s.infer(x.data());
+      std::ofstream fout(argv[3], std::ios::binary);
+      fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
+      const int iters = 0;
+#else
       std::vector<SOFIE_OUT_T> y = s.infer(x.data());
       std::ofstream fout(argv[3], std::ios::binary);
       fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
       const int iters = argc > 4 ? std::atoi(argv[4]) : 0;
+#endif
       if (iters > 0) {
          // device-resident timing: the input stays in the Session's device buffer
          for (int i = 0; i < 3; ++i) s.infer_device(s.SOFIE_INPUT_MEMBER);

@@ -29,6 +29,7 @@ enum class Options {
    kGNN = 0x8,
    kGNNComponent = 0x10,
    kBinaryWeightFile = 0x20,     // typed binary records in <name>.bin instead of the text <name>.dat (not in the reference)
+   kRuntimeBatch = 0x40,         // the batch size given to Generate is a capacity: infer(n, ...) runs any n up to it
 };
 std::underlying_type_t<Options> operator|(Options opA, Options opB);
 std::underlying_type_t<Options> operator|(std::underlying_type_t<Options> opA, Options opB);
@@ -153,6 +154,10 @@ private:
    std::set<std::string> fNeededStdLib = {"vector"};
    const std::set<std::string> fAllowedStdLib = {"vector", "algorithm", "cmath", "memory", "span"};
 
+   // Options::kRuntimeBatch: tensors whose leading dimension is the batch parameter, and the value it was resolved with
+   bool fRuntimeBatch = false;
+   size_t fBatchCapacity = 0;
+   std::set<std::string> fBatchTensors;
    std::map<std::string, std::string> fViewOf;      // view tensor -> tensor it aliases
    std::map<std::string, std::vector<size_t>> fChannelsLast;   // tensor stored channels-last -> (C,H,W)
    std::map<std::string, Placement> fPlacement;     // arena slot of every non-view intermediate

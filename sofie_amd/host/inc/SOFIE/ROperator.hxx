@@ -7,6 +7,7 @@
 #define SOFIE_ROPERATOR
 
 #include <memory>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -58,6 +59,15 @@ public:
    {
       return false;
    }
+   // Run-time batch: the leading dimension of this operator's first input is the batch, which the generated
+   // Session keeps in the member named `expr` (at most `capacity`, the value the shapes were resolved with).
+   // Returns false if the operator cannot run on fewer rows than it was generated for.
+   virtual bool SetRuntimeBatch(const std::string &expr, size_t capacity)
+   {
+      fBatchExpr = expr;
+      fBatchCapacity = capacity;
+      return true;
+   }
    // absorbed into another operator: emits nothing, and its output is written by the absorbing operator
    void SetAbsorbed() { fAbsorbed = true; }
    bool IsAbsorbed() const { return fAbsorbed; }
@@ -67,6 +77,17 @@ public:
 
 protected:
    const std::string SP = "   ";   // indentation of generated code
+   std::string fBatchExpr;         // empty: every dimension is a constant of the generated code
+   size_t fBatchCapacity = 0;
+   // a count proportional to the batch (rows, images, elements of a batch-led tensor) as emitted text
+   std::string BatchCount(size_t value) const
+   {
+      if (fBatchExpr.empty() || fBatchCapacity == 0) return std::to_string(value);
+      if (value % fBatchCapacity != 0)
+         throw std::runtime_error("TMVA SOFIE run-time batch: a count of " + std::to_string(value) + " is not a multiple of the batch");
+      const size_t per = value / fBatchCapacity;
+      return per == 1 ? fBatchExpr : "(" + fBatchExpr + " * " + std::to_string(per) + ")";
+   }
    bool fUseSession = false;
    bool fIsOutputConstant = false;
    bool fFusedAway = false;

@@ -125,7 +125,7 @@ public:
       std::stringstream out;
       out << "\n\n//---- BatchNorm " << OpName << "\n";
       out << SP << "Check(sofie_hip_batchnorm_f32(fCtx, tensor_" << fNX << ", tensor_" << fNFolded << ", tensor_" << fNMean
-          << ", tensor_" << fNB << ", tensor_" << fNY << ", " << fShapeX[0] << ", " << fShapeX[1] << ", " << plane << ", "
+          << ", tensor_" << fNB << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << plane << ", "
           << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << "), \"BatchNorm " << OpName
           << "\");\n";
       return out.str();

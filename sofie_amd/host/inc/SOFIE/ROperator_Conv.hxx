@@ -210,7 +210,8 @@ public:
       out << "\n//----  operator Conv " << OpName << "\n";
       if (dim == 3) {
          out << SP << "Check(sofie_hip_conv3d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNW << ", " << bias << ", tensor_" << fNY;
-         for (size_t i = 0; i < 5; ++i) out << ", " << fShapeX[i];
+         out << ", " << BatchCount(fShapeX[0]);
+         for (size_t i = 1; i < 5; ++i) out << ", " << fShapeX[i];
          out << ", " << fShapeW[0];
          for (size_t i = 0; i < 3; ++i) out << ", " << fShapeW[2 + i];
          for (size_t i = 0; i < 3; ++i) out << ", " << p[i];
@@ -227,7 +228,7 @@ public:
       const size_t sh = oneD ? 1 : fGeom.strides[0], sw = fGeom.strides[dim - 1];
       const size_t dh = oneD ? 1 : fGeom.dilations[0], dw = fGeom.dilations[dim - 1];
       out << SP << "Check(sofie_hip_conv2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNW << ", " << bias << ", tensor_" << fNY << ", "
-          << fShapeX[0] << ", " << fShapeX[1] << ", " << H << ", " << W << ", " << fShapeW[0] << ", " << KH << ", " << KW << ", " << ph
+          << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << H << ", " << W << ", " << fShapeW[0] << ", " << KH << ", " << KW << ", " << ph
           << ", " << pw << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << fGeom.group << ", " << act << "), \"Conv "
           << OpName << "\");\n";
       return out.str();

@@ -147,7 +147,7 @@ public:
       std::stringstream out;
       out << "\n//----  operator ConvTranspose " << OpName << "\n";
       out << SP << "Check(sofie_hip_conv_transpose2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNW << ", "
-          << (fNB.empty() ? std::string("nullptr") : "tensor_" + fNB) << ", tensor_" << fNY << ", " << fShapeX[0] << ", "
+          << (fNB.empty() ? std::string("nullptr") : "tensor_" + fNB) << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0]) << ", "
           << fShapeX[1] << ", " << H << ", " << W << ", " << fShapeY[1] << ", " << KH << ", " << KW << ", " << ph << ", " << pw
           << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << fAttrGroup << ", " << OH << ", " << OW << ", "
           << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << "), \"ConvTranspose " << OpName

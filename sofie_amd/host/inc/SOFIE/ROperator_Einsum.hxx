@@ -74,6 +74,8 @@ public:
    }
 
    std::string Kind() const override { return "Einsum"; }
+   // no label is known to be the batch
+   bool SetRuntimeBatch(const std::string &, size_t) override { return false; }
    const std::string &GemmType() const { return fGemmType; }
 
    bool ParseEquation(const std::string &input_equation)

@@ -180,6 +180,13 @@ public:
       model.AddNeededStdLib("algorithm");
    }
 
+   // the rows of A are the batch: not with a transposed A, stacked operands or a bias of one value per row
+   bool SetRuntimeBatch(const std::string &expr, size_t capacity) override
+   {
+      if (fAttrTransA || fStack > 1 || fBiasKind == 3) return false;
+      return ROperator::SetRuntimeBatch(expr, capacity);
+   }
+
    std::string Generate(std::string opName) override
    {
       opName = "op_" + opName;
@@ -208,7 +215,7 @@ public:
          offY = " + i * " + std::to_string(m * n);
          indent = SP + SP + SP;
       }
-      out << indent << "Check(sofie_hip_gemm_f32(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << m << ", "
+      out << indent << "Check(sofie_hip_gemm_f32(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << BatchCount(m) << ", "
           << n << ", " << k << ", " << FloatLiteral(fAttrAlpha) << ", tensor_" << fNA << offA << ", " << fShapeA[1] << ", tensor_" << fNB
           << offB << ", " << fShapeB[1] << ", " << FloatLiteral(fNC.empty() ? 0.0f : fAttrBeta) << ", "
           << (fNC.empty() ? std::string("nullptr") : "tensor_" + fNC) << ", " << fBiasKind << ", tensor_" << fNY << offY << ", " << n << ", "

@@ -99,11 +99,11 @@ public:
       out << "\n//----  operator " << Name() << "  " << OpName << "\n";
       const auto &a = fAttr;
       if (fType == ETensorType::FLOAT)
-         out << SP << "Check(sofie_hip_maxpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << fShapeX[0] * fShapeX[1]
+         out << SP << "Check(sofie_hip_maxpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0] * fShapeX[1])
              << ", " << fShapeX[2] << ", " << fShapeX[3];
       else
          out << SP << "Check(sofie_hip_maxpool2d_s8(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << (fChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << ", "
-             << fShapeX[0] << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3];
+             << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3];
       out << ", " << a.kernel_shape[0] << ", " << a.kernel_shape[1] << ", " << a.pads[0] << ", " << a.pads[1] << ", " << a.pads[2]
           << ", " << a.pads[3] << ", " << a.strides[0] << ", " << a.strides[1] << "), \"" << Name() << " " << OpName << "\");\n";
       return out.str();

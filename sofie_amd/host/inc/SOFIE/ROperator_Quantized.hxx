@@ -111,7 +111,7 @@ public:
    {
       std::stringstream out;
       out << "\n//------ QuantizeLinear op_" << OpName << "\n";
-      out << SP << "Check(sofie_hip_quantize_f32_s8(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << ConvertShapeToLength(fShape)
+      out << SP << "Check(sofie_hip_quantize_f32_s8(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(ConvertShapeToLength(fShape))
           << ", " << FloatLiteral(fScale) << ", " << fZp << "), \"QuantizeLinear op_" << OpName << "\");\n";
       return out.str();
    }
@@ -161,12 +161,12 @@ public:
       out << "\n//------ DequantizeLinear op_" << OpName << "\n";
       std::string src = fNX;
       if (!fNXNchw.empty()) {
-         out << SP << "Check(sofie_hip_relayout_s8(fCtx, tensor_" << fNX << ", tensor_" << fNXNchw << ", " << fShape[0] << ", " << fShape[1]
+         out << SP << "Check(sofie_hip_relayout_s8(fCtx, tensor_" << fNX << ", tensor_" << fNXNchw << ", " << BatchCount(fShape[0]) << ", " << fShape[1]
              << ", " << fShape[2] << ", " << fShape[3] << ", SOFIE_LAYOUT_NHWC, SOFIE_LAYOUT_NCHW), \"DequantizeLinear op_" << OpName
              << "\");\n";
          src = fNXNchw;
       }
-      out << SP << "Check(sofie_hip_dequantize_s8_f32(fCtx, tensor_" << src << ", tensor_" << fNY << ", " << ConvertShapeToLength(fShape)
+      out << SP << "Check(sofie_hip_dequantize_s8_f32(fCtx, tensor_" << src << ", tensor_" << fNY << ", " << BatchCount(ConvertShapeToLength(fShape))
           << ", " << FloatLiteral(fScale) << ", " << fZp << "), \"DequantizeLinear op_" << OpName << "\");\n";
       return out.str();
    }
@@ -296,7 +296,7 @@ public:
       if (fShapeA.empty()) throw std::runtime_error("TMVA SOFIE QLinearMatMul Op called to Generate without being initialized first");
       std::stringstream out;
       out << "\n//--------- QLinearMatMul op_" << OpName << "\n";
-      out << SP << "Check(sofie_hip_qgemm_s8(fCtx, 1, " << fM << ", " << fN << ", " << fK << ", tensor_" << fNA << ", " << fK
+      out << SP << "Check(sofie_hip_qgemm_s8(fCtx, 1, " << BatchCount(fM) << ", " << fN << ", " << fK << ", tensor_" << fNA << ", " << fK
           << ", tensor_" << fNBt << ", " << fK << ", tensor_" << fNScale << ", "
           << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", " << fZpY << ", "
           << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << ", tensor_" << fNY << ", " << fN << ", "
@@ -458,7 +458,7 @@ public:
          out << (pooled ? "sofie_hip_qconv2d_pool_s8" : "sofie_hip_qconv2d_s8") << "(fCtx, tensor_" << fNX << ", "
              << (fXChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW");
       out << ", tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, " << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr"))
-          << ", tensor_" << fNScale << ", tensor_" << (pooled ? fNYPooled : fNY) << ", SOFIE_LAYOUT_NHWC, " << fShapeX[0] << ", "
+          << ", tensor_" << fNScale << ", tensor_" << (pooled ? fNYPooled : fNY) << ", SOFIE_LAYOUT_NHWC, " << BatchCount(fShapeX[0]) << ", "
           << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", " << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3]
           << ", " << ph << ", " << pw << ", " << fGeom.strides[0] << ", " << fGeom.strides[1] << ", " << fGeom.group << ", ";
       if (!fromFloat) out << fZpX << ", ";
@@ -531,7 +531,7 @@ public:
    {
       std::stringstream out;
       out << "\n//--------- GemmFP8 op_" << OpName << "\n";
-      out << SP << "Check(sofie_hip_gemm_fp8(fCtx, 1, " << fM << ", " << fN << ", " << fK << ", tensor_" << fNA << ", " << fK
+      out << SP << "Check(sofie_hip_gemm_fp8(fCtx, 1, " << BatchCount(fM) << ", " << fN << ", " << fK << ", tensor_" << fNA << ", " << fK
           << ", tensor_" << fNBt << ", " << fK << ", " << FloatLiteral(fSa) << ", " << FloatLiteral(fSb) << ", "
           << (fNBias.empty() ? std::string("nullptr") : "tensor_" + fNBias) << ", tensor_" << fNY << ", " << fN
           << ", SOFIE_OUT_BF16), \"GemmFP8 op_" << OpName << "\");\n";

@@ -46,7 +46,7 @@ public:
          throw std::runtime_error("TMVA SOFIE Relu Op " + OpName + ": a Relu on a quantized tensor must follow the operator it can fuse with");
       std::stringstream out;
       out << "\n//------ RELU\n";
-      out << SP << "Check(sofie_hip_relu_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << ConvertShapeToLength(fShape)
+      out << SP << "Check(sofie_hip_relu_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(ConvertShapeToLength(fShape))
           << "), \"Relu " << OpName << "\");\n";
       return out.str();
    }

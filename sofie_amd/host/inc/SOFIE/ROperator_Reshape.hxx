@@ -93,7 +93,7 @@ public:
       return "\n//------ " + std::string(fOpMode == Flatten ? "FLATTEN" : "RESHAPE") + " op_" + OpName + " (view of tensor_" + fNData +
              ")\n" + SP + "if (static_cast<const void*>(tensor_" + fNOutput + ") != static_cast<const void*>(tensor_" + fNData +
              ")) Check(sofie_hip_copy(fCtx, tensor_" + fNOutput + ", tensor_" + fNData + ", " +
-             std::to_string(ConvertShapeToLength(fShapeOutput)) + " * sizeof(*tensor_" + fNOutput + ")), \"Reshape\");\n";
+             BatchCount(ConvertShapeToLength(fShapeOutput)) + " * sizeof(*tensor_" + fNOutput + ")), \"Reshape\");\n";
    }
 };
 

@@ -191,6 +191,7 @@ void RModel::Initialize(const std::map<std::string, size_t> &inputParams, bool v
    if (fIsInitialized) return;
    auto parametric = fInputTensorInfos;
    for (auto &input : parametric) {
+      const bool batchLed = !input.second.shape.empty() && input.second.shape[0].isParam;
       for (auto &d : input.second.shape) {
          if (!d.isParam) continue;
          std::string pname = d.param;
@@ -206,7 +207,15 @@ void RModel::Initialize(const std::map<std::string, size_t> &inputParams, bool v
                                   "to Generate / Initialize");
       fInputTensorInfos.erase(input.first);
       AddInputTensorInfo(input.first, input.second.type, shape);
+      if (fRuntimeBatch && batchLed) {
+         if (fBatchCapacity != 0 && fBatchCapacity != shape[0])
+            throw std::runtime_error("TMVA-SOFIE: run-time batch: the inputs do not agree on the batch dimension");
+         fBatchCapacity = shape[0];
+         fBatchTensors.insert(UTILITY::Clean_name(input.first));
+      }
    }
+   if (fRuntimeBatch && fBatchTensors.empty())
+      throw std::runtime_error("TMVA-SOFIE: Options::kRuntimeBatch needs an input whose leading dimension is a parameter");
    fIntermediateTensorInfos.clear();
    // every declared input must have a shape, as in the reference (RModel.cxx:410-468)
    for (auto &n : fInputTensorNames)
@@ -214,7 +223,26 @@ void RModel::Initialize(const std::map<std::string, size_t> &inputParams, bool v
          throw std::runtime_error("TMVA-SOFIE: input tensor " + n + " has no shape information");
    if (fInputTensorNames.empty())
       for (auto &it : fReadyInputTensorInfos) fInputTensorNames.push_back(it.first);
-   for (auto &op : fOperators) op->Initialize(*this);
+   for (auto &op : fOperators) {
+      op->Initialize(*this);
+      if (!fRuntimeBatch) continue;
+      // The batch travels along the first input of an operator: its outputs are then batch-led too and the
+      // operator emits the Session's fBatch member where it would print the leading dimension.
+      const auto &ins = op->GetOpInputTensors();
+      for (size_t i = 1; i < ins.size(); ++i)
+         if (fBatchTensors.count(ins[i]))
+            throw std::runtime_error("TMVA-SOFIE: run-time batch: tensor " + ins[i] + " carries the batch but is not the first input of its " +
+                                     op->Kind() + " operator");
+      if (ins.empty() || !fBatchTensors.count(ins[0])) continue;
+      if (!op->SetRuntimeBatch("fBatch", fBatchCapacity))
+         throw std::runtime_error("TMVA-SOFIE: run-time batch: this " + op->Kind() + " operator cannot run on fewer rows than it is generated for");
+      for (auto &out : op->GetOpOutputTensors()) {
+         const auto shape = GetTensorShape(out);
+         if (shape.empty() || shape[0] != fBatchCapacity)
+            throw std::runtime_error("TMVA-SOFIE: run-time batch: tensor " + out + " loses the batch as its leading dimension");
+         fBatchTensors.insert(out);
+      }
+   }
    for (auto &n : fOutputTensorNames)
       if (!CheckIfTensorAlreadyExist(n))
          throw std::runtime_error("TMVA-SOFIE: output tensor " + n + " is not produced by any operator");
@@ -644,6 +672,9 @@ void RModel::GenerateSessionCode()
    fGC += "CtxHandle fCtx;\n";
    fGC += "sofie_hip_graph* fGraph = nullptr;   // the operator sequence on the Session's own input buffer, recorded once\n";
    fGC += "bool fUseGraph = false;\n";
+   if (fRuntimeBatch)
+      fGC += "size_t fBatch = " + std::to_string(fBatchCapacity) + ";   // rows of the batch the operators process, at most " +
+             std::to_string(fBatchCapacity) + " (the capacity every buffer is sized for)\n";
    fGC += "static void Check(sofie_hip_ctx* ctx, int status, const char* what) {\n";
    fGC += "   if (status != 0) throw std::runtime_error(std::string(\"TMVA SOFIE device error in \") + what + \": \" + "
           "sofie_hip_last_error(ctx));\n";
@@ -809,17 +840,47 @@ void RModel::GenerateSessionCode()
 
    // ---- infer on host pointers: same signature and return convention as the reference
    // (RModel.cxx:680-801): one upload, the kernel sequence, one download
-   fGC += "std::vector<" + otype + "> infer(" + GenerateInferSignature(true) + "){\n";
-   for (auto &n : fInputTensorNames) {
-      const size_t bytes = ConvertShapeToLength(GetTensorShape(n)) * GetTypeSize(GetTensorType(n));
-      fGC += "   Check(sofie_hip_upload(fCtx, fInput_" + n + ", tensor_" + n + ", " + std::to_string(bytes) + "), \"input upload\");\n";
+   const bool outBatch = fRuntimeBatch && fBatchTensors.count(out);
+   auto uploads = [&]() {
+      for (auto &n : fInputTensorNames) {
+         const size_t bytes = ConvertShapeToLength(GetTensorShape(n)) * GetTypeSize(GetTensorType(n));
+         const std::string count = (fRuntimeBatch && fBatchTensors.count(n)) ? "fBatch * " + std::to_string(bytes / fBatchCapacity)
+                                                                            : std::to_string(bytes);
+         fGC += "   Check(sofie_hip_upload(fCtx, fInput_" + n + ", tensor_" + n + ", " + count + "), \"input upload\");\n";
+      }
+   };
+   const std::string outCount = outBatch ? "fBatch * " + std::to_string(olen / fBatchCapacity) : std::to_string(olen);
+   if (fRuntimeBatch) {
+      fGC += "// the batch the next run processes: any value from 1 to the capacity of " + std::to_string(fBatchCapacity) + "\n";
+      fGC += "void set_batch(size_t batch) {\n";
+      fGC += "   if (batch == 0 || batch > " + std::to_string(fBatchCapacity) +
+             ") throw std::runtime_error(\"TMVA SOFIE: the batch must be between 1 and " + std::to_string(fBatchCapacity) +
+             ", the size this Session was generated for\");\n";
+      fGC += "   if (batch != fBatch && fGraph) { sofie_hip_graph_destroy(fCtx, fGraph); fGraph = nullptr; }   // recorded for another size\n";
+      fGC += "   fBatch = batch;\n";
+      fGC += "}\n";
+      fGC += "// infer on the first `batch` rows of the inputs; returns that many rows\n";
+      fGC += "std::vector<" + otype + "> infer(size_t batch, " + GenerateInferSignature(true) + "){\n";
+      fGC += "   set_batch(batch);\n";
+      uploads();
+      fGC += "   run_own_input();\n";
+      fGC += "   std::vector<" + otype + "> ret(" + outCount + ");\n";
+      fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", ret.size() * sizeof(" + otype + ")), \"output download\");\n";
+      fGC += "   return ret;\n";
+      fGC += "}\n";
+      fGC += "// the whole capacity, as a Session generated for a fixed batch\n";
+      fGC += "std::vector<" + otype + "> infer(" + GenerateInferSignature(true) + "){ return infer(" + std::to_string(fBatchCapacity) +
+             ", " + GenerateInferSignature(false) + "); }\n\n";
+   } else {
+      fGC += "std::vector<" + otype + "> infer(" + GenerateInferSignature(true) + "){\n";
+      uploads();
+      fGC += "   run_own_input();\n";
+      fGC += "   std::vector<" + otype + "> ret(" + std::to_string(olen) + ");\n";
+      fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", " + std::to_string(olen) + " * sizeof(" + otype +
+             ")), \"output download\");\n";
+      fGC += "   return ret;\n";
+      fGC += "}\n\n";
    }
-   fGC += "   run_own_input();\n";
-   fGC += "   std::vector<" + otype + "> ret(" + std::to_string(olen) + ");\n";
-   fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", " + std::to_string(olen) + " * sizeof(" + otype +
-          ")), \"output download\");\n";
-   fGC += "   return ret;\n";
-   fGC += "}\n\n";
 
    // ---- infer on device pointers: nothing crosses PCIe; returns the device address of the output
    fGC += "const " + otype + "* infer_device(";
@@ -854,6 +915,9 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
       fWeightFile = WeightFileType::Binary;
    }
    (void)pos;
+   fRuntimeBatch = (static_cast<std::underlying_type_t<Options>>(Options::kRuntimeBatch) & options) != 0;
+   if (fRuntimeBatch && batchSize <= 0)
+      throw std::runtime_error("TMVA-SOFIE: Options::kRuntimeBatch needs the largest batch as the batch size given to Generate");
    Initialize(batchSize, verbose);
    FuseBatchNorm();
    FuseActivations();

@@ -28,6 +28,8 @@ def all_specs(with_large=True):
     specs.append(models.stacked_spec())
     specs.append(models.conv1d_spec())
     specs.append(models.conv3d_spec())
+    specs.append(models.qcnn_rt_spec(oracle))
+    specs.append(models.cnn_f32_rt_spec())
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs
@@ -47,8 +49,8 @@ def main():
             shutil.rmtree(sub)
         if spec.name == "functor4":
             emit.compile_example("run_functor.cxx", spec.name, "run_functor")
-        if spec.name == "qcnn_b4096":
-            os.remove(dat)      # same tensors as qcnn.dat: the runner is pointed at that file
+        if spec.name in ("qcnn_b4096", "qcnn_rt", "cnn_f32_rt"):
+            os.remove(dat)      # same tensors as qcnn.dat / cnn_f32.dat: the runner is pointed at that file
         print("%-28s %s" % (spec.name, res.stdout.strip().split(", ")[-1]))
     return 0
 

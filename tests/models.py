@@ -163,6 +163,20 @@ def qcnn_spec(oracle, batch, name="qcnn"):
     return s
 
 
+def qcnn_rt_spec(oracle, name="qcnn_rt"):
+    """The int8 CNN with the batch as a shape parameter of the input ("bs"): generated with a capacity, run with any
+    batch up to it."""
+    s = qcnn_spec(oracle, "bs", name)
+    s.batch, s.runtime_batch = 8, True
+    return s
+
+
+def cnn_f32_rt_spec(name="cnn_f32_rt"):
+    s = cnn_f32_spec("bs", name)
+    s.batch, s.runtime_batch = 8, True
+    return s
+
+
 def qcnn_reference(oracle, x):
     """The same network evaluated with the CPU oracle; per-channel scales are formed in fp32 in the
     emitter's order, (s_in * s_w[n]) / s_out."""

@@ -413,6 +413,53 @@ def test_einsum_matrix_products_become_gemm_calls_everything_else_one_kernel_cal
     assert "_stride[] = {6};" in c
 
 
+def test_runtime_batch_session(tmp_path):
+    """Options::kRuntimeBatch: the batch given to Generate is a capacity (buffers and the arena are sized for it); every
+    operator prints the Session's fBatch member where it would print the leading dimension, and infer(n, ...) moves
+    n rows in and out."""
+    hxx, _, _ = models.cnn_f32_rt_spec("rt_t").generate(str(tmp_path))
+    c = open(hxx).read()
+    assert "size_t fBatch = 8;" in c
+    assert "sofie_hip_conv2d_f32(fCtx, tensor_x, tensor_w1, tensor_b1, tensor_c1, fBatch, 1, 40, 40, 32, 3, 3," in c
+    assert "sofie_hip_maxpool2d_f32(fCtx, tensor_r1, tensor_p1, (fBatch * 32), 40, 40," in c
+    assert "sofie_hip_gemm_f32(fCtx, 0, 0, fBatch, 256, 12800," in c
+    assert "std::vector<float> infer(size_t batch, float* tensor_x){" in c
+    assert "sofie_hip_upload(fCtx, fInput_x, tensor_x, fBatch * 6400)" in c and "std::vector<float> ret(fBatch * 5);" in c
+    assert "std::vector<float> infer(float* tensor_x){ return infer(8, tensor_x); }" in c
+    assert "the batch must be between 1 and 8" in c
+    # the arena is the one of the fixed batch of 8
+    fixed = open(models.cnn_f32_spec(8, "rt_f").generate(str(tmp_path))[0]).read()
+    pool = re.search(r"fIntermediateMemoryPool\), (\d+)\)", c).group(1)
+    assert pool == re.search(r"fIntermediateMemoryPool\), (\d+)\)", fixed).group(1)
+    assert "fBatch" not in fixed
+
+    # without a shape parameter there is no batch to vary; without a capacity there is nothing to size
+    s, _ = models.mlp_spec("rt_e1")
+    s.runtime_batch = True
+    s.batch = 4
+    assert "needs an input whose leading dimension is a parameter" in emit_error(s, tmp_path)
+    s = models.cnn_f32_spec("bs", "rt_e2")
+    s.runtime_batch = True
+    assert "needs the largest batch" in emit_error(s, tmp_path)
+    # an operator that cannot tell which of its dimensions is the batch refuses
+    s = emit.ModelSpec("rt_e3")
+    s.add_input("a", "FLOAT", ("bs", 4))
+    s.add_init("b", np.ones((4, 3), np.float32))
+    s.einsum("ik,kj->ij", ["a", "b"], "y")
+    s.set_output("y")
+    s.batch, s.runtime_batch = 6, True
+    assert "this Einsum operator cannot run on fewer rows" in emit_error(s, tmp_path)
+    # the same parameter resolved at generation time only: a plain Session for that batch
+    s = emit.ModelSpec("rt_fix")
+    s.add_input("a", "FLOAT", ("bs", 4))
+    s.add_init("b", np.ones((4, 3), np.float32))
+    s.gemm("a", "b", None, "y", 1.0, 0.0)
+    s.set_output("y")
+    s.batch = 6
+    c = open(s.generate(str(tmp_path))[0]).read()
+    assert "sofie_hip_gemm_f32(fCtx, 0, 0, 6, 3, 4," in c and "fBatch" not in c
+
+
 def test_conv_1d_and_3d_emission(tmp_path):
     """One spatial dimension runs as the 2-D call with a height of one; three as the 3-D call. Absent pads mean one
     on every side of every dimension, as in the reference (ROperator_Conv.hxx:136-139)."""

@@ -74,6 +74,38 @@ def test_cnn_f32_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
+def test_runtime_batch_sessions(tmp_path):
+    """Sessions generated with a batch capacity of 8 run 8, 3 and 1 images through infer(n, ...): the int8 network's
+    logits are those of the oracle on the same images bit for bit, the float network's within 1e-5."""
+    x = models.cnn_input(8)
+    for n in (8, 3, 1):
+        exe = os.path.join(emit.GEN_DIR, "run_qcnn_rt")
+        fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+        np.ascontiguousarray(x[:n]).tofile(fin)
+        cmd = [exe, os.path.join(emit.GEN_DIR, "qcnn.dat"), fin, fout, str(n)]   # the weight file of the fixed-batch Session
+        print("running", " ".join(cmd), flush=True)
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=110)
+        assert res.returncode == 0, res.stderr
+        y = np.fromfile(fout, np.float32)
+        ref = models.qcnn_reference(oracle, x[:n])
+        assert y.size == ref.size and np.array_equal(y, ref.reshape(-1))
+    n = 5
+    exe = os.path.join(emit.GEN_DIR, "run_cnn_f32_rt")
+    fin, fout = str(tmp_path / "inf.bin"), str(tmp_path / "outf.bin")
+    np.ascontiguousarray(x[:n]).tofile(fin)
+    res = subprocess.run([exe, os.path.join(emit.GEN_DIR, "cnn_f32.dat"), fin, fout, str(n)], stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=110)
+    assert res.returncode == 0, res.stderr
+    y = np.fromfile(fout, np.float32)
+    ref = models.cnn_f32_stages(oracle, x[:n])["y"]
+    assert y.size == ref.size and rel_err(y, ref.reshape(-1)) <= 1e-5
+    # a batch beyond the capacity is refused by the Session
+    np.ascontiguousarray(np.concatenate([x, x[:1]])).tofile(fin)
+    res = subprocess.run([exe, os.path.join(emit.GEN_DIR, "cnn_f32.dat"), fin, fout, "9"], stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=110)
+    assert res.returncode != 0 and "the batch must be between 1 and 8" in res.stderr
+
+
 def test_conv_1d_and_3d_sessions(tmp_path):
     """A 1-D convolution runs on the 2-D kernel with a height of one (1e-5 relative); the 3-D kernel sums in the
     order of the reference's column matrix, so it equals the oracle exactly."""
