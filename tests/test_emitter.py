@@ -351,6 +351,12 @@ def test_parametric_batch_dimension_is_fixed_at_generation_time(tmp_path):
         assert "sofie_hip_gemm_f32(fCtx, 0, 0, 7, 4, 6," in code
         res = _onnx_emit(str(path), tmp_path)
         assert res.returncode != 0 and "parametric shape" in res.stderr and "pass the batch size" in res.stderr
+        # the same file with the value as a capacity: the Gemm -> Relu pair prints the Session's batch member
+        res = subprocess.run([exe, str(path), str(tmp_path), "--batch", "7", "--runtime"], stdout=subprocess.PIPE,
+                             stderr=subprocess.PIPE, text=True)
+        assert res.returncode == 0, res.stderr
+        code = open(str(tmp_path / "dyn.hxx")).read()
+        assert "sofie_hip_gemm_f32(fCtx, 0, 0, fBatch, 4, 6," in code and "size_t fBatch = 7;" in code
 
 
 def test_stacked_matmul_shapes_and_offsets(tmp_path):
