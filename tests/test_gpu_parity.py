@@ -177,6 +177,11 @@ def test_gemm_f32_integer_data_is_exact(ops):
     dict(N=2, C=1, H=40, W=40, OC=32, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, bias=True, relu=True),
     dict(N=1, C=8, H=12, W=300, OC=16, k=(1, 1), p=(0, 0), s=(1, 1), d=(1, 1), g=1, bias=False, relu=False),
     dict(N=1, C=3, H=30, W=30, OC=5, k=(7, 7), p=(3, 3), s=(2, 2), d=(1, 1), g=1, bias=True, relu=False),
+    # channel blocks staged under the matrix loop (the kernel with two LDS buffers): two groups with 64-channel tiles
+    # and a stride; a dilation with a ragged second channel tile; a last pixel tile that is nearly empty
+    dict(N=2, C=16, H=9, W=19, OC=96, k=(3, 3), p=(1, 1), s=(2, 2), d=(1, 1), g=2, bias=True, relu=True),
+    dict(N=1, C=8, H=12, W=12, OC=130, k=(3, 3), p=(2, 2), s=(1, 1), d=(2, 2), g=1, bias=True, relu=False),
+    dict(N=3, C=12, H=13, W=10, OC=64, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, bias=False, relu=True),
 ])
 def test_conv2d_f32(ops, cfg):
     r = rng(200 + cfg["C"] + cfg["OC"])
