@@ -150,8 +150,8 @@ int sofie_hip_conv3d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
  * (ROperator_ConvTranspose.icc:83-90); pad_h / pad_w are the begin pads. Replaces the emitted kernel
  * re-layout, BLAS::sgemm_ into the column matrix, UTILITY::col2im and BLAS::saxpy_ of
  * ROperator_ConvTranspose<float>::Generate (ROperator_ConvTranspose.icc:232-474) with the implicit-GEMM
- * convolution kernel: one launch per output phase (oy mod stride, ox mod stride) with the reversed taps that
- * reach it, or, with a dilation, one launch over the zero-interleaved input; no column matrix exists. */
+ * convolution kernel: per output phase (oy mod stride, ox mod stride) the reversed taps that
+ * reach it (up to four phases share one launch), or, with a dilation, one launch over the zero-interleaved input; no column matrix exists. */
 int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
                                    const float *bias, float *y, int N, int C, int H, int W,
                                    int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,

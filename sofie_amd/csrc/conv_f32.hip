@@ -23,6 +23,13 @@ namespace {
 #define SOFIE_CONV_PIPE_PATCH 1536
 #define SOFIE_CONV_PIPE_WEIGHTS 5120
 
+// Geometry of one output phase of a strided transposed convolution when all phases run in one launch.
+struct PhaseArgs {
+   int KH, KW, th0, tw0, ph, pw, oy0, ox0, OH, OW, rows_out, PH, PW, ICB, KC;
+   FastDiv dPW, dPH, dKC, dOW;
+};
+#define SOFIE_CONV_MAX_PHASES 4
+
 struct ConvArgs {
    const float *x, *w, *bias;
    float *y;
@@ -45,6 +52,9 @@ struct ConvArgs {
    int wvec;           // weights are staged with 16-byte loads (see launch)
    FastDiv dPW, dPH, dKC, dK4;   // divisions by the patch extents and the K-chunk length (/4) in the staging loops
    FastDiv dUH, dUW, dOW;
+   // nphases > 1: blockIdx.z = image * nphases + phase, and the phase's geometry replaces the fields above
+   int nphases;
+   PhaseArgs phase[SOFIE_CONV_MAX_PHASES];
 };
 
 // Input row / column behind position `up` of the zero-interleaved input, or -1 where a zero sits.
@@ -62,10 +72,28 @@ template <int TI, int TJ, bool TR>
 __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
 {
    constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
+   // geometry of this workgroup's launch: the kernel's own, or that of its output phase when all phases of a strided
+   // transposed convolution run in one launch (picked with static indices so that it stays in scalar registers)
+   PhaseArgs q;
+   q.KH = g.KH; q.KW = g.KW; q.th0 = g.th0; q.tw0 = g.tw0; q.ph = g.ph; q.pw = g.pw; q.oy0 = g.oy0; q.ox0 = g.ox0;
+   q.OH = g.OH; q.OW = g.OW; q.rows_out = g.rows_out; q.PH = g.PH; q.PW = g.PW; q.ICB = g.ICB; q.KC = g.KC;
+   q.dPW = g.dPW; q.dPH = g.dPH; q.dKC = g.dKC; q.dOW = g.dOW;
+   int n = blockIdx.z;
+   if constexpr (TR) {
+      if (g.nphases > 1) {
+         const int pi = blockIdx.z % g.nphases;
+         n = blockIdx.z / g.nphases;
+         q = g.phase[0];
+#pragma unroll
+         for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
+            if (pi == i) q = g.phase[i];
+         if ((int)blockIdx.x * BP >= q.OH * q.OW) return;   // the grid is as wide as the phase with most pixel tiles
+      }
+   }
    extern __shared__ __align__(16) unsigned char smem_raw[];
    float *sW = reinterpret_cast<float *>(smem_raw);                  // [KC][LDW]
-   float *patch = sW + g.KC * LDW;                                   // [ICB][PH][PW]
-   int *koff = reinterpret_cast<int *>(patch + g.ICB * g.PH * g.PW); // [KC]
+   float *patch = sW + q.KC * LDW;                                   // [ICB][PH][PW]
+   int *koff = reinterpret_cast<int *>(patch + q.ICB * q.PH * q.PW); // [KC]
 
    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
    const int wm = wave >> 1, wn = wave & 1;
@@ -74,25 +102,24 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
    const int octiles = (g.ocg + BOC - 1) / BOC;
    const int grp = blockIdx.y / octiles;
    const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
-   const int n = blockIdx.z;
-   const int OHW = g.OH * g.OW;
+   const int OHW = q.OH * q.OW;
    const int p0 = blockIdx.x * BP;
-   const int oh0 = p0 / g.OW;
-   const int ih0 = oh0 * g.sh - g.ph, iw0 = -g.pw;
-   const int KHW = g.KH * g.KW;
+   const int oh0 = p0 / q.OW;
+   const int ih0 = oh0 * g.sh - q.ph, iw0 = -q.pw;
+   const int KHW = q.KH * q.KW;
    const int Kfull = g.icg * KHW;
 
-   for (int k = tid; k < g.KC; k += 256) {
+   for (int k = tid; k < q.KC; k += 256) {
       const int icl = k / KHW, t = k % KHW;
-      const int kh = t / g.KW, kw = t % g.KW;
-      koff[k] = (icl < g.ICB) ? (icl * g.PH + kh * g.dh) * g.PW + kw * g.dw : 0;
+      const int kh = t / q.KW, kw = t % q.KW;
+      koff[k] = (icl < q.ICB) ? (icl * q.PH + kh * g.dh) * q.PW + kw * g.dw : 0;
    }
 
    int base[TJ];
 #pragma unroll
    for (int j = 0; j < TJ; ++j) {
       const int p = p0 + wn * TJ * 32 + j * 32 + fr;
-      base[j] = (p < OHW) ? ((p / g.OW - oh0) * g.sh) * g.PW + (p % g.OW) * g.sw : 0;
+      base[j] = (p < OHW) ? ((p / q.OW - oh0) * g.sh) * q.PW + (p % q.OW) * g.sw : 0;
    }
 
    v16f acc[TI][TJ];
@@ -105,10 +132,10 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
 
    const float *xg = g.x + ((size_t)n * g.C + (size_t)grp * g.icg) * g.H * g.W;
    const float *wg = g.w + (size_t)grp * g.ocg * Kfull;
-   const int patch_len = g.ICB * g.PH * g.PW;
+   const int patch_len = q.ICB * q.PH * q.PW;
 
-   for (int ic0 = 0; ic0 < g.icg; ic0 += g.ICB) {
-      const int icn = (g.icg - ic0) < g.ICB ? (g.icg - ic0) : g.ICB;
+   for (int ic0 = 0; ic0 < g.icg; ic0 += q.ICB) {
+      const int icn = (g.icg - ic0) < q.ICB ? (g.icg - ic0) : q.ICB;
       const int kc = icn * KHW;
       __syncthreads();   // previous chunk fully consumed (also orders the koff table on entry)
       // Staging: every load of a batch is issued before the first value is used (the addresses of cells outside the
@@ -122,8 +149,8 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
 #pragma unroll
             for (int u = 0; u < UP; ++u) {
                const int e = e0 + u * 256 + tid;
-               const int t = fdiv(e, g.dPW), c = e - t * g.PW;
-               const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
+               const int t = fdiv(e, q.dPW), c = e - t * q.PW;
+               const int icl = fdiv(t, q.dPH), r = t - icl * q.PH;
                int ih = ih0 + r, iw = iw0 + c;
                if constexpr (TR) {
                   ih = source_index(ih, g.uh, g.dUH);
@@ -144,7 +171,7 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       stage_patch(std::integral_constant<int, 6>{});
       if (!TR && g.wvec) {
          // four consecutive k of one output channel per 16-byte load (every block is full and 16-byte aligned)
-         const int K4 = g.KC >> 2, total4 = K4 * BOC;
+         const int K4 = q.KC >> 2, total4 = K4 * BOC;
          auto stage_weights4 = [&](auto batch) {
             constexpr int UW = decltype(batch)::value;
             for (int e0 = 0; e0 < total4; e0 += 256 * UW) {
@@ -171,21 +198,21 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
          stage_weights4(std::integral_constant<int, 3>{});
       } else {
          constexpr int UW = 8;
-         const int total = g.KC * BOC;
+         const int total = q.KC * BOC;
          for (int e0 = 0; e0 < total; e0 += 256 * UW) {
             float v[UW];
             bool ok[UW];
 #pragma unroll
             for (int u = 0; u < UW; ++u) {
                const int e = e0 + u * 256 + tid;
-               const int ocl = fdiv(e, g.dKC), k = e - ocl * g.KC;
+               const int ocl = fdiv(e, q.dKC), k = e - ocl * q.KC;
                ok[u] = e < total && k < kc && oc0 + ocl < g.ocg;
                size_t off = 0;
                if (ok[u]) {
                   if constexpr (TR) {
                      const int icl = k / KHW, t = k - icl * KHW;
-                     const int ta = t / g.KW, tb = t - ta * g.KW;
-                     off = ((((size_t)grp * g.icg + ic0 + icl) * g.ocg + oc0 + ocl) * g.KH0 + g.th0 + ta * g.ths) * g.KW0 + g.tw0 +
+                     const int ta = t / q.KW, tb = t - ta * q.KW;
+                     off = ((((size_t)grp * g.icg + ic0 + icl) * g.ocg + oc0 + ocl) * g.KH0 + q.th0 + ta * g.ths) * g.KW0 + q.tw0 +
                            tb * g.tws;
                   } else {
                      off = (size_t)grp * g.ocg * Kfull + (size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + k;
@@ -196,14 +223,14 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
 #pragma unroll
             for (int u = 0; u < UW; ++u) {
                const int e = e0 + u * 256 + tid;
-               const int ocl = fdiv(e, g.dKC), k = e - ocl * g.KC;
+               const int ocl = fdiv(e, q.dKC), k = e - ocl * q.KC;
                if (e < total) sW[k * LDW + ocl] = ok[u] ? v[u] : 0.0f;
             }
          }
       }
       __syncthreads();
       const float *wrow = sW + wm * TI * 32 + fr;
-      for (int s = 0; s < g.KC / 2; ++s) {
+      for (int s = 0; s < q.KC / 2; ++s) {
          const int kk = 2 * s + fk;
          const int ko = koff[kk];
          float fa[TI], fb[TJ];
@@ -229,8 +256,8 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
          if (p >= OHW) continue;
          size_t po = (size_t)p;
          if constexpr (TR) {
-            const int q = fdiv(p, g.dOW);
-            po = (size_t)(g.oy0 + q * g.oys) * g.OW0 + g.ox0 + (p - q * g.OW) * g.oxs;
+            const int row = fdiv(p, q.dOW);
+            po = (size_t)(q.oy0 + row * g.oys) * g.OW0 + q.ox0 + (p - row * q.OW) * g.oxs;
          }
 #pragma unroll
          for (int r = 0; r < 16; ++r) {
@@ -502,6 +529,57 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    return check_launch(ctx, "k_conv2d_f32");
 }
 
+// All output phases of a strided transposed convolution in one launch of k_conv2d_f32<.., true>: every phase gets
+// the channel block and patch geometry a launch of its own would get; the grid is as wide as the phase with most
+// pixel tiles. *done stays false if a phase does not fit (the caller then launches the phases one by one).
+template <int TI, int TJ>
+int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
+{
+   constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
+   const size_t budget = 52 * 1024;
+   *done = false;
+   const int octiles = cdiv(g.ocg, BOC);
+   if ((size_t)g.groups * octiles > 65535 || (size_t)g.N * g.nphases > 65535) return SOFIE_HIP_OK;
+   size_t lds_max = 0;
+   int tiles_max = 0;
+   for (int i = 0; i < g.nphases; ++i) {
+      PhaseArgs &p = g.phase[i];
+      const int KHW = p.KH * p.KW;
+      p.rows_out = (BP + p.OW - 2) / p.OW + 1;
+      if (p.rows_out > p.OH) p.rows_out = p.OH;
+      p.PH = (p.rows_out - 1) + (p.KH - 1) + 1;      // unit stride and dilation inside a phase
+      p.PW = (p.OW - 1) + (p.KW - 1) + 1;
+      int icb = 96 / KHW;
+      if (icb < 1) icb = 1;
+      if (icb > g.icg) icb = g.icg;
+      size_t lds = 0;
+      for (; icb >= 1; --icb) {
+         const int kc = (icb * KHW + 1) & ~1;
+         lds = ((size_t)kc * LDW + (size_t)icb * p.PH * p.PW + kc) * 4;
+         if (lds <= budget) {
+            p.ICB = icb;
+            p.KC = kc;
+            break;
+         }
+      }
+      if (icb < 1) return SOFIE_HIP_OK;
+      p.dPW = make_fastdiv((unsigned)p.PW);
+      p.dPH = make_fastdiv((unsigned)p.PH);
+      p.dKC = make_fastdiv((unsigned)p.KC);
+      p.dOW = make_fastdiv((unsigned)p.OW);
+      if (lds > lds_max) lds_max = lds;
+      if (cdiv(p.OH * p.OW, BP) > tiles_max) tiles_max = cdiv(p.OH * p.OW, BP);
+   }
+   g.wvec = 0;
+   g.dK4 = make_fastdiv(1u);
+   auto kern = k_conv2d_f32<TI, TJ, true>;
+   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+   hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, g);
+   *done = true;
+   return check_launch(ctx, "k_conv2d_f32 (phases)");
+}
+
 int run_conv(sofie_hip_ctx *ctx, ConvArgs &g)
 {
    if (g.KH0 == 0) {   // identity tap and output maps
@@ -663,22 +741,52 @@ extern "C" int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x
    // with (ry - p + k0) divisible by the stride (p = K-1-pad), and tap a reads input row q + a + (ry - p + k0)/stride:
    // a unit-stride correlation over the input as it is, with a sub-kernel of about K/stride taps.
    const int py = KH - 1 - pad_h, px = KW - 1 - pad_w;
+   // the launch geometry of one phase: tap (a, b) of the phase is element (th0 + a*ths, tw0 + b*tws) of the kernel
+   auto phase_of = [&](int ry, int rx) {
+      const int k0y = (((py - ry) % stride_h) + stride_h) % stride_h, k0x = (((px - rx) % stride_w) + stride_w) % stride_w;
+      ConvArgs p = g;
+      p.uh = 1; p.uw = 1;
+      p.KH0 = KH; p.KW0 = KW;
+      p.KH = k0y < KH ? (KH - 1 - k0y) / stride_h + 1 : 0;
+      p.KW = k0x < KW ? (KW - 1 - k0x) / stride_w + 1 : 0;
+      p.th0 = KH - 1 - k0y; p.ths = -stride_h;
+      p.tw0 = KW - 1 - k0x; p.tws = -stride_w;
+      p.ph = -((ry - py + k0y) / stride_h);
+      p.pw = -((rx - px + k0x) / stride_w);
+      p.OH0 = OH; p.OW0 = OW; p.oy0 = ry; p.oys = stride_h; p.ox0 = rx; p.oxs = stride_w;
+      p.OH = (OH - 1 - ry) / stride_h + 1;
+      p.OW = (OW - 1 - rx) / stride_w + 1;
+      return p;
+   };
+   // All phases in one launch when there are at most SOFIE_CONV_MAX_PHASES of them and each has taps: a phase on its
+   // own fills a fraction of the device (a quarter of the output pixels), and the launches would run one after another.
+   {
+      ConvArgs all = g;
+      all.uh = 1; all.uw = 1;
+      all.KH0 = KH; all.KW0 = KW; all.ths = -stride_h; all.tws = -stride_w;
+      all.OH0 = OH; all.OW0 = OW; all.oys = stride_h; all.oxs = stride_w;
+      all.nphases = 0;
+      bool ok = stride_h * stride_w <= SOFIE_CONV_MAX_PHASES;
+      for (int ry = 0; ry < stride_h && ok; ++ry)
+         for (int rx = 0; rx < stride_w && ok; ++rx) {
+            if (ry >= OH || rx >= OW) { ok = false; break; }
+            const ConvArgs p = phase_of(ry, rx);
+            if (p.KH == 0 || p.KW == 0) { ok = false; break; }
+            PhaseArgs &q = all.phase[all.nphases++];
+            q.KH = p.KH; q.KW = p.KW; q.th0 = p.th0; q.tw0 = p.tw0; q.ph = p.ph; q.pw = p.pw;
+            q.oy0 = p.oy0; q.ox0 = p.ox0; q.OH = p.OH; q.OW = p.OW;
+         }
+      if (ok && all.nphases > 1) {
+         all.dUH = make_fastdiv(1u); all.dUW = make_fastdiv(1u); all.dOW = make_fastdiv(1u);
+         bool done = false;
+         const int rc = all.ocg > 64 ? launch_phases<2, 2>(ctx, all, &done) : launch_phases<1, 2>(ctx, all, &done);
+         if (rc || done) return rc;
+      }
+   }
    for (int ry = 0; ry < stride_h; ++ry)
       for (int rx = 0; rx < stride_w; ++rx) {
          if (ry >= OH || rx >= OW) continue;
-         const int k0y = (((py - ry) % stride_h) + stride_h) % stride_h, k0x = (((px - rx) % stride_w) + stride_w) % stride_w;
-         ConvArgs p = g;
-         p.uh = 1; p.uw = 1;
-         p.KH0 = KH; p.KW0 = KW;
-         p.KH = k0y < KH ? (KH - 1 - k0y) / stride_h + 1 : 0;
-         p.KW = k0x < KW ? (KW - 1 - k0x) / stride_w + 1 : 0;
-         p.th0 = KH - 1 - k0y; p.ths = -stride_h;
-         p.tw0 = KW - 1 - k0x; p.tws = -stride_w;
-         p.ph = -((ry - py + k0y) / stride_h);
-         p.pw = -((rx - px + k0x) / stride_w);
-         p.OH0 = OH; p.OW0 = OW; p.oy0 = ry; p.oys = stride_h; p.ox0 = rx; p.oxs = stride_w;
-         p.OH = (OH - 1 - ry) / stride_h + 1;
-         p.OW = (OW - 1 - rx) / stride_w + 1;
+         ConvArgs p = phase_of(ry, rx);
          if (p.KH == 0 || p.KW == 0) {
             // no tap reaches this phase: the outputs are the bias; the plain kernel's loops run zero times
             p.KH = 0; p.KW = 0;
