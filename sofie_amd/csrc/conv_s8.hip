@@ -91,7 +91,12 @@ struct QConvTileArgs {
 // register-wise maximum over the four tiles (on the int32 accumulators: the requantisation is monotonic;
 // for a negative scale the minimum is taken) and only a quarter of the values is converted and stored.
 // In that mode the "pixels" the tiles, the epilogue and a.OH / a.OW / a.ep.M count are pooled pixels.
-template <int MB, int NB, int WN, int PF, int OUT, bool POOL>
+//
+// KFIX: 0 for any kernel size and channel count (the K loop walks taps and channel blocks with run-time
+// counters); C/32 (1 or 2) for a 3x3 kernel on 32 or 64 channels. Then the K loop is unrolled over its
+// 9*KFIX steps: a fragment address is a per-tile register (pixel, kernel row) plus a constant that goes
+// into the offset field of the LDS read, and the loop holds matrix instructions and LDS reads only.
+template <int MB, int NB, int WN, int PF, int OUT, bool POOL, int KFIX>
 __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 {
    static_assert(!POOL || MB == 4, "the four window positions are the four m tiles");
@@ -227,6 +232,48 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    v16i r_bias[POOL ? 1 : NB];
    auto kloop = [&](v16i (&acc)[NB][MB]) {
       v4i fa[POOL ? 2 : 3][MB], fb[POOL ? 2 : 3][NB];
+      if constexpr (KFIX > 0) {
+         constexpr int NBUF = POOL ? 2 : 3;          // fragment buffers: the reads run NBUF - 1 steps ahead
+         constexpr int CSF = KFIX * 32 + 16;         // pixel stride of the band (a.CS) for 32 / 64 channels
+         constexpr int NS = 9 * KFIX;
+         const unsigned char *pa[3][MB], *pb[NB];
+#pragma unroll
+         for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int j = 0; j < MB; ++j) pa[kh][j] = s_p + (a_off[j] + kh * a.RB);
+#pragma unroll
+         for (int i = 0; i < NB; ++i) pb[i] = s_w + b_off[i];
+         v16i zero;
+#pragma unroll
+         for (int e = 0; e < 16; ++e) zero[e] = 0;
+#pragma unroll
+         for (int s = 0; s < NS + NBUF - 1; ++s) {
+            if (s < NS) {
+               const int kh = s / (3 * KFIX), kw = (s / KFIX) % 3, cb = s % KFIX;
+#pragma unroll
+               for (int j = 0; j < MB; ++j)
+                  fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[kh][j] + (kw * CSF + cb * 32));
+#pragma unroll
+               for (int i = 0; i < NB; ++i) fb[s % NBUF][i] = *reinterpret_cast<const v4i *>(pb[i] + s * 32);
+            }
+            if (s >= NBUF - 1) {
+               const int d = s - (NBUF - 1), buf = d % NBUF;
+#pragma unroll
+               for (int i = 0; i < NB; ++i)
+#pragma unroll
+                  for (int j = 0; j < MB; ++j) {
+                     if (d == 0) {
+                        // the first step starts from the bias tiles (from zero with the fused pooling)
+                        if constexpr (POOL) acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], zero);
+                        else acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], r_bias[i]);
+                     } else {
+                        acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], acc[i][j]);
+                     }
+                  }
+            }
+         }
+         return;
+      }
       int ka = 0, kb = 0, c32 = 0, kw = 0;
       auto advance = [&]() {
          ka += 32; kb += 32;
@@ -467,17 +514,26 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (lds > 160 * 1024) return SOFIE_HIP_OK;
    if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
 
+   // 3x3 kernels on 32 or 64 channels take the kernels whose K loop is unrolled with constant offsets
+   const int kfix = (g.KH == 3 && g.KW == 3 && (g.C == 32 || g.C == 64) && a.CS == g.C + 16) ? g.C / 32 : 0;
    const int nob = g.OC / OCT;
    int per = ctx->num_cus / nob;
    if (per < 1) per = 1;
    if (per > a.ntiles) per = a.ntiles;
    const dim3 grid((unsigned)(per * nob)), block(512);
-#define SOFIE_QCONV_LAUNCH(MB_, WN_, PF_, POOL_)                                                              \
+#define SOFIE_QCONV_LAUNCH_K(MB_, WN_, PF_, POOL_, KFIX_)                                                     \
    do {                                                                                                       \
-      auto kern = k_qconv_mfma<MB_, 2, WN_, PF_, OUT, POOL_>;                                                 \
+      auto kern = k_qconv_mfma<MB_, 2, WN_, PF_, OUT, POOL_, KFIX_>;                                          \
       SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));         \
       hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                             \
+   } while (0)
+#define SOFIE_QCONV_LAUNCH(MB_, WN_, PF_, POOL_)                                                              \
+   do {                                                                                                       \
+      if constexpr (OUT != SOFIE_OUT_S8) SOFIE_QCONV_LAUNCH_K(MB_, WN_, PF_, POOL_, 0);                       \
+      else if (kfix == 1) SOFIE_QCONV_LAUNCH_K(MB_, WN_, PF_, POOL_, 1);                                      \
+      else if (kfix == 2) SOFIE_QCONV_LAUNCH_K(MB_, WN_, PF_, POOL_, 2);                                      \
+      else SOFIE_QCONV_LAUNCH_K(MB_, WN_, PF_, POOL_, 0);                                                     \
    } while (0)
 #define SOFIE_QCONV_BY_PASSES(MB_, WN_, POOL_)                                                                \
    do {                                                                                                       \
@@ -498,6 +554,7 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    }
 #undef SOFIE_QCONV_BY_PASSES
 #undef SOFIE_QCONV_LAUNCH
+#undef SOFIE_QCONV_LAUNCH_K
    *done = true;
    return check_launch(ctx, "k_qconv_mfma");
 }
