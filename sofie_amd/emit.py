@@ -42,8 +42,9 @@ class ModelSpec:
         self.tensors = {}
         self.input = None      # the first input (single-input runners)
         self.inputs = []
-        self.output = None
+        self.output = None     # the first output
         self.out_type = "FLOAT"
+        self.outputs = []      # (name, type) of every output, in the order infer() returns them
         self.batch = None            # value of the inputs' shape parameters at generation time
         self.runtime_batch = False   # ... as a capacity: the Session also takes infer(n, ...)
 
@@ -66,8 +67,10 @@ class ModelSpec:
 
     def set_output(self, name, type_name="FLOAT"):
         self.lines.append("output %s" % name)
-        self.output = name
-        self.out_type = type_name
+        if self.output is None:
+            self.output = name
+            self.out_type = type_name
+        self.outputs.append((name, type_name))
 
     # ---- operators -------------------------------------------------------------------------
     def gemm(self, a, b, c, y, alpha=1.0, beta=1.0, transA=0, transB=0, relu=False):
@@ -155,7 +158,8 @@ class ModelSpec:
         cmd = ["g++", "-std=c++17", "-O2", "-I" + os.path.join(ROOT, "include"), "-I" + outdir,
                "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % self.name, "-DSOFIE_MODEL_NS=SOFIE_%s" % self.name,
                "-DSOFIE_IN_T=%s" % _CTYPE[self.input[1]], "-DSOFIE_OUT_T=%s" % _CTYPE[self.out_type],
-               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs)] + \
+               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs),
+               "-DSOFIE_NUM_OUTPUTS=%d" % max(1, len(self.outputs))] + \
               (["-DSOFIE_RUNTIME_BATCH"] if (runtime_batch or self.runtime_batch) else []) + [
                os.path.join(_HERE, "host", "examples", "run_session.cxx"), "-o", exe,
                "-L" + _HERE, "-lsofie_hip", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath," + _HERE]

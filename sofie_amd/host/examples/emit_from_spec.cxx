@@ -9,7 +9,7 @@
 //   model NAME
 //   input NAME TYPE RANK d0 d1 ...                 a dimension that is not a number is a shape parameter (e.g. bs)
 //   init NAME TYPE RANK d0 d1 ... FILE           raw little-endian values
-//   output NAME
+//   output NAME                                    once per output tensor, in the order infer() returns them
 //   op Gemm ALPHA BETA TRANSA TRANSB A B C Y RELU
 //   op Conv AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. X W B Y
 //   op BatchNormalization EPSILON X SCALE B MEAN VAR Y
@@ -66,6 +66,7 @@ int main(int argc, char **argv)
       const std::string tdir = argv[2], odir = argv[3];
       std::unique_ptr<RModel> model;
       std::string line, name;
+      std::vector<std::string> outputs;
       int order = 0;
       while (std::getline(spec, line)) {
          std::istringstream in(line);
@@ -103,7 +104,8 @@ int main(int argc, char **argv)
          } else if (kw == "output") {
             std::string n;
             in >> n;
-            model->AddOutputTensorNameList({n});
+            outputs.push_back(n);
+            model->AddOutputTensorNameList(outputs);   // every "output" statement extends the list
          } else if (kw == "op") {
             std::string op;
             in >> op;

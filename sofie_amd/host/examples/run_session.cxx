@@ -2,6 +2,8 @@
 // Compile with -DSOFIE_MODEL_HEADER='"x.hxx"' -DSOFIE_MODEL_NS=SOFIE_x -DSOFIE_IN_T=float -DSOFIE_OUT_T=float -DSOFIE_INPUT_MEMBER=fInput_x
 // and, for a model with several inputs, -DSOFIE_NUM_INPUTS=n (then <input.bin> is a comma-separated list, one file per input
 // in the order of infer()'s arguments, and there is no timing).
+// For a model with several outputs add -DSOFIE_NUM_OUTPUTS=n: <output.bin> is then a comma-separated list, one file per
+// output in the order of the model's output list (infer() returns a vector of vectors or a tuple of vectors), no timing.
 // With -DSOFIE_RUNTIME_BATCH (a Session generated with Options::kRuntimeBatch) the fourth argument is the batch: the
 // runner calls infer(batch, input) and writes that many rows.
 //   run_session <weights.dat> <input.bin> <output.bin> [timed iterations of infer_device | batch]
@@ -11,6 +13,7 @@
 #include <fstream>
 #include <iostream>
 #include <string>
+#include <tuple>
 #include <utility>
 #include <vector>
 
@@ -18,6 +21,48 @@
 
 #ifndef SOFIE_NUM_INPUTS
 #define SOFIE_NUM_INPUTS 1
+#endif
+#ifndef SOFIE_NUM_OUTPUTS
+#define SOFIE_NUM_OUTPUTS 1
+#endif
+
+static std::vector<std::string> SplitList(const std::string &list)
+{
+   std::vector<std::string> parts;
+   size_t start = 0;
+   for (size_t comma; (comma = list.find(',', start)) != std::string::npos; start = comma + 1) parts.push_back(list.substr(start, comma - start));
+   parts.push_back(list.substr(start));
+   return parts;
+}
+
+template <class T>
+static void WriteRaw(const std::string &path, const std::vector<T> &y)
+{
+   std::ofstream fout(path, std::ios::binary);
+   fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(T));
+   if (!fout) throw std::runtime_error("cannot write " + path);
+}
+
+#if SOFIE_NUM_OUTPUTS > 1
+// several outputs of one type: a vector of vectors
+template <class T>
+static void WriteOutputs(const std::vector<std::string> &paths, const std::vector<std::vector<T>> &ys)
+{
+   if (ys.size() != paths.size()) throw std::runtime_error("the model returns " + std::to_string(ys.size()) + " outputs");
+   for (size_t i = 0; i < ys.size(); ++i) WriteRaw(paths[i], ys[i]);
+}
+// outputs of different types: a tuple of vectors
+template <class... V, size_t... I>
+static void WriteTuple(const std::vector<std::string> &paths, const std::tuple<V...> &ys, std::index_sequence<I...>)
+{
+   (WriteRaw(paths[I], std::get<I>(ys)), ...);
+}
+template <class... V>
+static void WriteOutputs(const std::vector<std::string> &paths, const std::tuple<V...> &ys)
+{
+   if (sizeof...(V) != paths.size()) throw std::runtime_error("the model returns " + std::to_string(sizeof...(V)) + " outputs");
+   WriteTuple(paths, ys, std::index_sequence_for<V...>{});
+}
 #endif
 
 static std::vector<SOFIE_IN_T> ReadRaw(const std::string &path)
@@ -33,7 +78,7 @@ static std::vector<SOFIE_IN_T> ReadRaw(const std::string &path)
 
 #if SOFIE_NUM_INPUTS > 1
 template <size_t... I>
-static std::vector<SOFIE_OUT_T> InferAll(SOFIE_MODEL_NS::Session &s, std::vector<std::vector<SOFIE_IN_T>> &xs, std::index_sequence<I...>)
+static auto InferAll(SOFIE_MODEL_NS::Session &s, std::vector<std::vector<SOFIE_IN_T>> &xs, std::index_sequence<I...>)
 {
    return s.infer(xs[I].data()...);
 }
@@ -57,12 +102,21 @@ int main(int argc, char **argv)
          xs.push_back(ReadRaw(list.substr(start)));
          if (xs.size() != SOFIE_NUM_INPUTS) throw std::runtime_error("the model takes " + std::to_string(SOFIE_NUM_INPUTS) + " input files");
       }
-      std::vector<SOFIE_OUT_T> y = InferAll(s, xs, std::make_index_sequence<SOFIE_NUM_INPUTS>{});
-      std::ofstream fout(argv[3], std::ios::binary);
-      fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
+      auto y = InferAll(s, xs, std::make_index_sequence<SOFIE_NUM_INPUTS>{});
+#if SOFIE_NUM_OUTPUTS > 1
+      WriteOutputs(SplitList(argv[3]), y);
+#else
+      WriteRaw(argv[3], y);
+#endif
 #else
       std::vector<SOFIE_IN_T> x = ReadRaw(argv[2]);
-#ifdef SOFIE_RUNTIME_BATCH
+#if SOFIE_NUM_OUTPUTS > 1
+      WriteOutputs(SplitList(argv[3]), s.infer(x.data()));
+      // the device-pointer form returns the same tensors' device addresses, in the same order
+      auto dev = s.infer_device(s.SOFIE_INPUT_MEMBER);
+      s.sync();
+      static_assert(std::tuple_size<decltype(dev)>::value == SOFIE_NUM_OUTPUTS, "one device address per output");
+#elif defined(SOFIE_RUNTIME_BATCH)
       std::vector<SOFIE_OUT_T> y = argc > 4 ? s.infer((size_t)std::atoi(argv[4]), x.data()) : s.infer(x.data());
       std::ofstream fout(argv[3], std::ios::binary);
       fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
@@ -73,6 +127,7 @@ int main(int argc, char **argv)
       fout.write(reinterpret_cast<const char *>(y.data()), y.size() * sizeof(SOFIE_OUT_T));
       const int iters = argc > 4 ? std::atoi(argv[4]) : 0;
 #endif
+#if SOFIE_NUM_OUTPUTS == 1
       if (iters > 0) {
          // device-resident timing: the input stays in the Session's device buffer
          for (int i = 0; i < 3; ++i) s.infer_device(s.SOFIE_INPUT_MEMBER);
@@ -102,6 +157,7 @@ int main(int argc, char **argv)
          std::printf("{\"device_ms\": %.6f, \"host_ms\": %.6f, \"graph_ms\": %.6f, \"graph_matches\": %s, \"iters\": %d}\n", ms / iters,
                      host_ms / iters, gms / iters, same ? "true" : "false", iters);
       }
+#endif
 #endif
    } catch (const std::exception &e) {
       std::cerr << "run_session: " << e.what() << "\n";

@@ -473,7 +473,7 @@ void RModel::GenerateHeaderInfo(std::string &hgname)
    fGC += "#define " + hgname + "\n\n";
    for (auto &i : fNeededStdLib) fGC += "#include <" + i + ">\n";
    for (auto &i : fCustomOpHeaders) fGC += "#include \"" + i + "\"\n";
-   fGC += "#include <cstdint>\n#include <cstring>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n";
+   fGC += "#include <cstdint>\n#include <cstring>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n#include <tuple>\n#include <utility>\n";
    // the numerical library: a C ABI over device pointers instead of the reference's
    // extern "C" BLAS prototypes (RModel_Base.cxx:40-58)
    fGC += "#include \"sofie_hip.h\"\n";
@@ -811,11 +811,55 @@ void RModel::GenerateSessionCode()
    }
    fGC += "}\n\n";
 
-   if (fOutputTensorNames.size() != 1)
-      throw std::runtime_error("TMVA-SOFIE: the device emission supports exactly one output tensor");
+   // ---- return convention of infer(), as in the reference (RModel.cxx:744-801): one output is a std::vector of its
+   // type; several outputs of one type are a std::vector of std::vectors; outputs of different types are a
+   // std::tuple of std::vectors, all in the order of the output list
+   const size_t nout = fOutputTensorNames.size();
+   if (nout == 0) throw std::runtime_error("TMVA-SOFIE: output size=0 are not supported");
    const std::string out = fOutputTensorNames[0];
    const std::string otype = ConvertTypeToString(GetTensorType(out));
-   const size_t olen = ConvertShapeToLength(GetTensorShape(out));
+   bool sameOutputTypes = true;
+   for (auto &n : fOutputTensorNames) sameOutputTypes = sameOutputTypes && GetTensorType(n) == GetTensorType(out);
+   std::string inferReturnType = "std::vector<" + otype + ">";
+   std::string deviceReturnType = "const " + otype + "*";
+   if (nout > 1) {
+      if (sameOutputTypes) {
+         inferReturnType = "std::vector<std::vector<" + otype + ">>";
+      } else {
+         inferReturnType = "std::tuple<";
+         for (size_t i = 0; i < nout; ++i)
+            inferReturnType += std::string(i ? "," : "") + "std::vector<" + ConvertTypeToString(GetTensorType(fOutputTensorNames[i])) + ">";
+         inferReturnType += ">";
+      }
+      deviceReturnType = "std::tuple<";
+      for (size_t i = 0; i < nout; ++i)
+         deviceReturnType += std::string(i ? "," : "") + "const " + ConvertTypeToString(GetTensorType(fOutputTensorNames[i])) + "*";
+      deviceReturnType += ">";
+   }
+   // element count of output i as the generated code states it (rows of the current batch with a run-time batch)
+   auto outputCount = [&](const std::string &n) {
+      const size_t len = ConvertShapeToLength(GetTensorShape(n));
+      return (fRuntimeBatch && fBatchTensors.count(n)) ? "fBatch * " + std::to_string(len / fBatchCapacity) : std::to_string(len);
+   };
+   // the statements that download every output and return them
+   auto downloads = [&]() {
+      if (nout == 1) {
+         fGC += "   std::vector<" + otype + "> ret(" + outputCount(out) + ");\n";
+         fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", ret.size() * sizeof(" + otype + ")), \"output download\");\n";
+         fGC += "   return ret;\n";
+         return;
+      }
+      for (size_t i = 0; i < nout; ++i) {
+         const std::string &n = fOutputTensorNames[i];
+         const std::string t = ConvertTypeToString(GetTensorType(n));
+         const std::string v = "ret_" + std::to_string(i);
+         fGC += "   std::vector<" + t + "> " + v + "(" + outputCount(n) + ");\n";
+         fGC += "   Check(sofie_hip_download(fCtx, " + v + ".data(), tensor_" + n + ", " + v + ".size() * sizeof(" + t + ")), \"output download\");\n";
+      }
+      fGC += "   return " + inferReturnType + "{";
+      for (size_t i = 0; i < nout; ++i) fGC += std::string(i ? ", " : "") + "std::move(ret_" + std::to_string(i) + ")";
+      fGC += "};\n";
+   };
 
    // ---- the sequence on the Session's own input buffer, optionally replayed from a HIP graph
    {
@@ -840,7 +884,6 @@ void RModel::GenerateSessionCode()
 
    // ---- infer on host pointers: same signature and return convention as the reference
    // (RModel.cxx:680-801): one upload, the kernel sequence, one download
-   const bool outBatch = fRuntimeBatch && fBatchTensors.count(out);
    auto uploads = [&]() {
       for (auto &n : fInputTensorNames) {
          const size_t bytes = ConvertShapeToLength(GetTensorShape(n)) * GetTypeSize(GetTensorType(n));
@@ -849,7 +892,6 @@ void RModel::GenerateSessionCode()
          fGC += "   Check(sofie_hip_upload(fCtx, fInput_" + n + ", tensor_" + n + ", " + count + "), \"input upload\");\n";
       }
    };
-   const std::string outCount = outBatch ? "fBatch * " + std::to_string(olen / fBatchCapacity) : std::to_string(olen);
    if (fRuntimeBatch) {
       fGC += "// the batch the next run processes: any value from 1 to the capacity of " + std::to_string(fBatchCapacity) + "\n";
       fGC += "void set_batch(size_t batch) {\n";
@@ -860,30 +902,26 @@ void RModel::GenerateSessionCode()
       fGC += "   fBatch = batch;\n";
       fGC += "}\n";
       fGC += "// infer on the first `batch` rows of the inputs; returns that many rows\n";
-      fGC += "std::vector<" + otype + "> infer(size_t batch, " + GenerateInferSignature(true) + "){\n";
+      fGC += inferReturnType + " infer(size_t batch, " + GenerateInferSignature(true) + "){\n";
       fGC += "   set_batch(batch);\n";
       uploads();
       fGC += "   run_own_input();\n";
-      fGC += "   std::vector<" + otype + "> ret(" + outCount + ");\n";
-      fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", ret.size() * sizeof(" + otype + ")), \"output download\");\n";
-      fGC += "   return ret;\n";
+      downloads();
       fGC += "}\n";
       fGC += "// the whole capacity, as a Session generated for a fixed batch\n";
-      fGC += "std::vector<" + otype + "> infer(" + GenerateInferSignature(true) + "){ return infer(" + std::to_string(fBatchCapacity) +
+      fGC += inferReturnType + " infer(" + GenerateInferSignature(true) + "){ return infer(" + std::to_string(fBatchCapacity) +
              ", " + GenerateInferSignature(false) + "); }\n\n";
    } else {
-      fGC += "std::vector<" + otype + "> infer(" + GenerateInferSignature(true) + "){\n";
+      fGC += inferReturnType + " infer(" + GenerateInferSignature(true) + "){\n";
       uploads();
       fGC += "   run_own_input();\n";
-      fGC += "   std::vector<" + otype + "> ret(" + std::to_string(olen) + ");\n";
-      fGC += "   Check(sofie_hip_download(fCtx, ret.data(), tensor_" + out + ", " + std::to_string(olen) + " * sizeof(" + otype +
-             ")), \"output download\");\n";
-      fGC += "   return ret;\n";
+      downloads();
       fGC += "}\n\n";
    }
 
-   // ---- infer on device pointers: nothing crosses PCIe; returns the device address of the output
-   fGC += "const " + otype + "* infer_device(";
+   // ---- infer on device pointers: nothing crosses PCIe; returns the device address of the output (a tuple of the
+   // addresses, in the order of the output list, when there are several)
+   fGC += deviceReturnType + " infer_device(";
    {
       int k = 0;
       for (auto &n : fInputTensorNames) {
@@ -896,7 +934,15 @@ void RModel::GenerateSessionCode()
       int k = 0;
       for (auto &n : fInputTensorNames) fGC += std::string(k++ ? ", " : "") + "tensor_" + n;
    }
-   fGC += ");\n   return tensor_" + out + ";\n}\n";
+   fGC += ");\n   return ";
+   if (nout == 1) {
+      fGC += "tensor_" + out;
+   } else {
+      fGC += deviceReturnType + "{";
+      for (size_t i = 0; i < nout; ++i) fGC += std::string(i ? ", " : "") + "tensor_" + fOutputTensorNames[i];
+      fGC += "}";
+   }
+   fGC += ";\n}\n";
    fGC += "void sync() { Check(sofie_hip_sync(fCtx), \"sync\"); }\n";
    fGC += "};\n";
 }

@@ -379,3 +379,44 @@ def stacked_spec(name="stacked"):
 def stacked_reference():
     p = stacked_params()
     return np.matmul(np.matmul(p["x"].astype(np.float64), p["B1"].astype(np.float64)), p["B2"].astype(np.float64))
+
+
+# ------------------------------------------------------------------------------------------ several outputs
+def two_heads_spec(name="two_heads", seed=0):
+    """The MLP with its second hidden layer and its last layer both listed as outputs (one type: infer()
+    returns a vector of vectors, as the reference's does)."""
+    s, x = mlp_spec(name, seed)
+    s.lines = [ln for ln in s.lines if not ln.startswith("output ")]
+    s.output, s.outputs = None, []
+    s.set_output("h1")
+    s.set_output("y")
+    return s, x
+
+
+def two_heads_reference(oracle, seed=0):
+    Ws, Bs, x = mlp_weights(seed)
+    h = oracle.gemm_f32(x, Ws[0], Bs[0], relu=True)
+    h1 = oracle.gemm_f32(h, Ws[1], Bs[1], relu=True)
+    return h1, oracle.gemm_f32(h1, Ws[2], Bs[2])
+
+
+MIXED_SCALE, MIXED_ZP = 0.05, 3
+
+
+def mixed_outputs_spec(name="mixed_outputs", seed=0):
+    """The MLP's float result and its QuantizeLinear image as two outputs (different types: infer() returns a
+    tuple of vectors, as the reference's does)."""
+    s, x = mlp_spec(name, seed)
+    s.lines = [ln for ln in s.lines if not ln.startswith("output ")]
+    s.output, s.outputs = None, []
+    s.add_scalar("sq", MIXED_SCALE, np.float32)
+    s.add_scalar("zq", MIXED_ZP, np.int8)
+    s.quantize("y", "sq", "zq", "q")
+    s.set_output("y")
+    s.set_output("q", "INT8")
+    return s, x
+
+
+def mixed_outputs_reference(oracle, seed=0):
+    y = mlp_reference(oracle, seed)
+    return y, oracle.quantize_f32_s8(y, MIXED_SCALE, MIXED_ZP)

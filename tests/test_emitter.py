@@ -548,3 +548,27 @@ def test_every_prebuilt_session_compiles():
         for ext in (".hxx",):
             assert os.path.exists(os.path.join(emit.GEN_DIR, spec.name + ext)), spec.name
         assert os.path.exists(os.path.join(emit.GEN_DIR, "run_" + spec.name)), spec.name
+
+
+def test_several_outputs_follow_the_reference_return_convention(tmp_path):
+    """Outputs of one type come back as a vector of vectors, outputs of different types as a tuple of vectors, in
+    the order of the output list (RModel.cxx:744-801); an intermediate that is an output keeps its place in the
+    pool until the end; the generated code compiles against the runner."""
+    spec, _ = models.two_heads_spec("two_heads_probe")
+    hxx, _, _ = gen(spec, tmp_path)
+    code = open(hxx).read()
+    assert "std::vector<std::vector<float>> infer(float* tensor_x)" in code
+    assert "return std::vector<std::vector<float>>{std::move(ret_0), std::move(ret_1)};" in code
+    assert "std::tuple<const float*,const float*> infer_device(const float* tensor_x)" in code
+    off = {m.group(1): int(m.group(2)) for m in re.finditer(r"tensor_(\w+) = reinterpret_cast<float\*>\(fIntermediateMemoryPool \+ (\d+)\)", code)}
+    assert off["y"] == off["h0"]                       # the last layer reuses the dead first hidden layer ...
+    assert off["h1"] >= off["h0"] + 256 * 128 * 4       # ... and never the hidden layer that is an output
+    spec.compile_runner(str(tmp_path))
+
+    spec, _ = models.mixed_outputs_spec("mixed_probe")
+    hxx, _, _ = gen(spec, tmp_path)
+    code = open(hxx).read()
+    assert "std::tuple<std::vector<float>,std::vector<int8_t>> infer(float* tensor_x)" in code
+    assert "std::tuple<const float*,const int8_t*> infer_device(const float* tensor_x)" in code
+    assert code.index("tensor_y, ret_0.size()") < code.index("tensor_q, ret_1.size()")
+    spec.compile_runner(str(tmp_path))

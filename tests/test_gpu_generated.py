@@ -42,6 +42,21 @@ def run_session(name, x, tmp_path, out_dtype=np.float32, dat=None, iters=0):
     return (y, json.loads(res.stdout)) if iters else y
 
 
+def run_session_outputs(name, x, tmp_path, out_dtypes):
+    """Runner of a model with several outputs: one raw file per output, in the order of the output list."""
+    exe = os.path.join(emit.GEN_DIR, "run_" + name)
+    if not os.path.exists(exe):
+        raise RuntimeError("%s is missing: run python tests/build_generated.py on the build machine" % exe)
+    fin = str(tmp_path / "in.bin")
+    np.ascontiguousarray(x).tofile(fin)
+    fouts = [str(tmp_path / ("out%d.bin" % i)) for i in range(len(out_dtypes))]
+    cmd = [exe, os.path.join(emit.GEN_DIR, name + ".dat"), fin, ",".join(fouts)]
+    print("running", " ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=110)
+    assert res.returncode == 0, res.stderr
+    return [np.fromfile(f, d) for f, d in zip(fouts, out_dtypes)]
+
+
 def rel_err(a, b):
     return float(np.max(np.abs(a.astype(np.float64) - b.astype(np.float64))) / max(float(np.max(np.abs(b))), 1e-30))
 
@@ -210,3 +225,19 @@ def test_int8_cnn_batch_4096_matches_the_oracle_on_a_sample_and_is_batch_invaria
     assert np.array_equal(y[pick], ref)
     y8 = run_session("qcnn", x[:8], tmp_path).reshape(8, 5)
     assert np.array_equal(y[:8], y8)
+
+
+def test_sessions_with_several_outputs(tmp_path):
+    """Two float outputs (vector of vectors) and a float plus an int8 output (tuple): every output equals the
+    oracle's tensor, the hidden layer that is an output is intact after the layers behind it ran."""
+    _, x = models.two_heads_spec()
+    h1, y = run_session_outputs("two_heads", x, tmp_path, (np.float32, np.float32))
+    rh1, ry = models.two_heads_reference(oracle)
+    assert h1.size == rh1.size and y.size == ry.size
+    assert rel_err(h1, rh1.reshape(-1)) <= 1e-5 and rel_err(y, ry.reshape(-1)) <= 1e-5
+
+    y, q = run_session_outputs("mixed_outputs", x, tmp_path, (np.float32, np.int8))
+    ry, _ = models.mixed_outputs_reference(oracle)
+    assert rel_err(y, ry.reshape(-1)) <= 1e-5
+    # the int8 output is the quantisation of the float output the device computed, bit for bit
+    assert np.array_equal(q, oracle.quantize_f32_s8(y, models.MIXED_SCALE, models.MIXED_ZP))
