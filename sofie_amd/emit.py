@@ -47,6 +47,7 @@ class ModelSpec:
         self.outputs = []      # (name, type) of every output, in the order infer() returns them
         self.batch = None            # value of the inputs' shape parameters at generation time
         self.runtime_batch = False   # ... as a capacity: the Session also takes infer(n, ...)
+        self.no_session = False      # Options::kNoSession: free function infer, weights as literals
 
     def add_input(self, name, dtype, shape):
         t = dtype if isinstance(dtype, str) else _TYPE[np.dtype(dtype)]
@@ -123,7 +124,7 @@ class ModelSpec:
 
     # ---- generation ------------------------------------------------------------------------
     def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False, batch=None,
-                 runtime_batch=False):
+                 runtime_batch=False, no_session=False):
         """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess). `batch` gives the shape
         parameters of the inputs (dimensions written as names) their value; with `runtime_batch` it is a capacity and
         the generated Session also takes infer(n, ...) for any n up to it."""
@@ -135,6 +136,8 @@ class ModelSpec:
         spec = os.path.join(outdir, self.name + ".spec")
         with open(spec, "w") as f:
             flag = " noweightfile" if no_weight_file else (" binaryweightfile" if binary_weight_file else "")
+            if no_session or self.no_session:
+                flag = " nosession"
             batch = self.batch if batch is None else batch
             if batch is not None:
                 flag += " batch %d" % batch
@@ -160,7 +163,8 @@ class ModelSpec:
                "-DSOFIE_IN_T=%s" % _CTYPE[self.input[1]], "-DSOFIE_OUT_T=%s" % _CTYPE[self.out_type],
                "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs),
                "-DSOFIE_NUM_OUTPUTS=%d" % max(1, len(self.outputs))] + \
-              (["-DSOFIE_RUNTIME_BATCH"] if (runtime_batch or self.runtime_batch) else []) + [
+              (["-DSOFIE_RUNTIME_BATCH"] if (runtime_batch or self.runtime_batch) else []) + \
+              (["-DSOFIE_NO_SESSION"] if self.no_session else []) + [
                os.path.join(_HERE, "host", "examples", "run_session.cxx"), "-o", exe,
                "-L" + _HERE, "-lsofie_hip", "-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath," + _HERE]
         res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

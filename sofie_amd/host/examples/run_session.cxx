@@ -4,6 +4,8 @@
 // in the order of infer()'s arguments, and there is no timing).
 // For a model with several outputs add -DSOFIE_NUM_OUTPUTS=n: <output.bin> is then a comma-separated list, one file per
 // output in the order of the model's output list (infer() returns a vector of vectors or a tuple of vectors), no timing.
+// With -DSOFIE_NO_SESSION (a model generated with Options::kNoSession) the runner calls the free function infer() of the
+// model's namespace twice and writes the second result; the weight file argument is ignored.
 // With -DSOFIE_RUNTIME_BATCH (a Session generated with Options::kRuntimeBatch) the fourth argument is the batch: the
 // runner calls infer(batch, input) and writes that many rows.
 //   run_session <weights.dat> <input.bin> <output.bin> [timed iterations of infer_device | batch]
@@ -91,6 +93,14 @@ int main(int argc, char **argv)
       return 2;
    }
    try {
+#ifdef SOFIE_NO_SESSION
+      {
+         std::vector<SOFIE_IN_T> x = ReadRaw(argv[2]);
+         SOFIE_MODEL_NS::infer(x.data());
+         WriteRaw(argv[3], SOFIE_MODEL_NS::infer(x.data()));
+         return 0;
+      }
+#endif
       SOFIE_MODEL_NS::Session s(argv[1]);
 #if SOFIE_NUM_INPUTS > 1
       std::vector<std::vector<SOFIE_IN_T>> xs;

@@ -23,7 +23,7 @@ namespace SOFIE {
 
 enum class Options {
    kDefault = 0x0,
-   kNoSession = 0x1,             // not available: device memory needs an owner
+   kNoSession = 0x1,             // free function infer on one Session created at its first call; weights as literals
    kNoWeightFile = 0x2,          // weights as literals in the generated header
    kRootBinaryWeightFile = 0x4,  // not available (no ROOT)
    kGNN = 0x8,

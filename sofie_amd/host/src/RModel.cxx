@@ -950,8 +950,14 @@ void RModel::GenerateSessionCode()
 void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, long pos, bool verbose)
 {
    fVerbose = verbose;
-   if (static_cast<std::underlying_type_t<Options>>(Options::kNoSession) & options)
-      throw std::runtime_error("TMVA-SOFIE: Options::kNoSession is not available: device weights and buffers need the Session as owner");
+   // Options::kNoSession (RModel.cxx:1164-1180 of the reference: free function infer, weights as literals). Device
+   // weights and buffers still need an owner: the Session is emitted as usual, without a weight file, and the free
+   // functions behind it run on one instance created at their first call.
+   const bool noSession = (static_cast<std::underlying_type_t<Options>>(Options::kNoSession) & options) != 0;
+   if (noSession) {
+      fUseWeightFile = false;
+      fWeightFile = WeightFileType::None;
+   }
    if (static_cast<std::underlying_type_t<Options>>(Options::kRootBinaryWeightFile) & options)
       throw std::runtime_error("TMVA-SOFIE: ROOT binary weight files are not available in this build");
    if (static_cast<std::underlying_type_t<Options>>(Options::kNoWeightFile) & options) {
@@ -974,6 +980,15 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    std::string hgname;
    GenerateHeaderInfo(hgname);
    GenerateSessionCode();
+   if (noSession) {
+      fGC += "\n// Options::kNoSession: free functions on one Session that is created at the first call (not re-entrant,\n";
+      fGC += "// as the reference's free infer with its static buffers)\n";
+      fGC += "inline Session& DefaultSession() { static Session session(\"\"); return session; }\n";
+      fGC += "inline auto infer(" + GenerateInferSignature(true) + "){ return DefaultSession().infer(" + GenerateInferSignature(false) + "); }\n";
+      if (fRuntimeBatch)
+         fGC += "inline auto infer(size_t batch, " + GenerateInferSignature(true) + "){ return DefaultSession().infer(batch, " +
+                GenerateInferSignature(false) + "); }\n";
+   }
    fGC += ("} //SOFIE_" + fName + "\n");
    fGC += "\n#endif  // " + hgname + "\n";
 }

@@ -32,6 +32,7 @@ def all_specs(with_large=True):
     specs.append(models.cnn_f32_rt_spec())
     specs.append(models.two_heads_spec()[0])
     specs.append(models.mixed_outputs_spec()[0])
+    specs.append(models.mlp_nosession_spec()[0])
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs

@@ -420,3 +420,10 @@ def mixed_outputs_spec(name="mixed_outputs", seed=0):
 def mixed_outputs_reference(oracle, seed=0):
     y = mlp_reference(oracle, seed)
     return y, oracle.quantize_f32_s8(y, MIXED_SCALE, MIXED_ZP)
+
+
+def mlp_nosession_spec(name="mlp_nosession", seed=0):
+    """The MLP generated with Options::kNoSession: a free function infer, weights as literals."""
+    s, x = mlp_spec(name, seed)
+    s.no_session = True
+    return s, x

@@ -572,3 +572,16 @@ def test_several_outputs_follow_the_reference_return_convention(tmp_path):
     assert "std::tuple<const float*,const int8_t*> infer_device(const float* tensor_x)" in code
     assert code.index("tensor_y, ret_0.size()") < code.index("tensor_q, ret_1.size()")
     spec.compile_runner(str(tmp_path))
+
+
+def test_no_session_option_emits_a_free_infer_over_literal_weights(tmp_path):
+    """Options::kNoSession: no weight file is written, the weights are literals and the namespace has a free
+    function infer (the reference's no-session form); the runner compiles against it."""
+    spec, _ = models.mlp_nosession_spec("nosession_probe")
+    hxx, dat, _ = gen(spec, tmp_path)
+    assert not os.path.exists(dat)
+    code = open(hxx).read()
+    assert "static const float host[" in code
+    assert 'inline Session& DefaultSession() { static Session session(""); return session; }' in code
+    assert "inline auto infer(float* tensor_x){ return DefaultSession().infer(tensor_x); }" in code
+    spec.compile_runner(str(tmp_path))

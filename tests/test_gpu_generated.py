@@ -241,3 +241,11 @@ def test_sessions_with_several_outputs(tmp_path):
     assert rel_err(y, ry.reshape(-1)) <= 1e-5
     # the int8 output is the quantisation of the float output the device computed, bit for bit
     assert np.array_equal(q, oracle.quantize_f32_s8(y, models.MIXED_SCALE, models.MIXED_ZP))
+
+
+def test_no_session_free_function(tmp_path):
+    """A model generated with Options::kNoSession: the free function infer (called twice, on the one Session it
+    creates at its first call) gives the MLP's result."""
+    _, x = models.mlp_nosession_spec()
+    y = run_session("mlp_nosession", x, tmp_path, dat="unused")
+    assert rel_err(y, models.mlp_reference(oracle).reshape(-1)) <= 1e-5
