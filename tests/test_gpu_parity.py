@@ -773,3 +773,95 @@ def test_conv3d_f32_matches_the_column_matrix_order(ops, cfg):
         ref = oracle.conv3d_f32(x, w, bias, pads, strides, dil, groups, relu=relu)
         assert y.shape == ref.shape
         assert np.array_equal(y, ref)
+
+
+# --------------------------------------------------------------------------- the benchmark's full sizes
+def _window_sums(xs, k, p, OH, OW):
+    """S[n, c, kh, kw] = sum over the output positions of the (zero-padded) input cell that tap (kh, kw) reads."""
+    N, C, H, W = xs.shape
+    xp = np.zeros((N, C, H + 2 * p, W + 2 * p), np.int64)
+    xp[:, :, p:p + H, p:p + W] = xs
+    S = np.empty((N, C, k, k), np.int64)
+    for kh in range(k):
+        for kw in range(k):
+            S[:, :, kh, kw] = xp[:, :, kh:kh + OH, kw:kw + OW].sum(axis=(2, 3))
+    return S
+
+
+def test_qconv2d_s8_full_size_layer(ops):
+    """The benchmark's layer (batch 256, 64 -> 128 channels, 56x56, 3x3, pad 1, ReLU), int8: three images against
+    the oracle bit for bit, every image equal to the same image convolved on its own (the tiles of the batched launch
+    cross image borders), and the int32 accumulators of all 102.8 M outputs through one checksum per (image,
+    channel): sum over the pixels of acc = sum over the taps of w * (window sum of the input), exact in int64."""
+    from sofie_amd import lib as L
+    r = rng(77)
+    N, C, H, OC = 256, 64, 56, 128
+    x = r.integers(-128, 128, (N, H, H, C)).astype(np.int8)                     # channels-last, as between quantized layers
+    w = r.integers(-127, 128, (OC, 3, 3, C)).astype(np.int8)
+    scale = (r.uniform(20, 60, OC) / (73.3 * 73.3 * np.sqrt(576.0))).astype(np.float32)
+    bias = r.integers(-3000, 3000, OC).astype(np.int32)
+    y = ops.qconv2d_s8(x, w, scale, bias, (1, 1), (1, 1), 1, -128, -128, True, x_layout=L.LAYOUT_NHWC,
+                       y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+    wn = np.ascontiguousarray(w.transpose(0, 3, 1, 2))
+    for n in (0, 129, 255):
+        xn = np.ascontiguousarray(x[n:n + 1].transpose(0, 3, 1, 2))
+        ref = oracle.qconv2d_s8(xn, wn, scale, bias, (1, 1), (1, 1), 1, -128, -128, True)
+        assert np.array_equal(y[n].transpose(2, 0, 1), ref[0]), n
+    for n in (1, 77, 254):
+        alone = ops.qconv2d_s8(x[n:n + 1], w, scale, bias, (1, 1), (1, 1), 1, -128, -128, True, x_layout=L.LAYOUT_NHWC,
+                               y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+        assert np.array_equal(alone[0], y[n]), n
+    assert 0.05 < np.mean(y == -128) < 0.95 and np.mean(y == 127) < 0.2            # the scales spread the outputs
+    acc = ops.qconv2d_s8(x, w, None, None, (1, 1), (1, 1), 1, -128, x_layout=L.LAYOUT_NHWC, y_layout=L.LAYOUT_NHWC,
+                         w_layout=L.LAYOUT_NHWC, out=L.OUT_S32)
+    got = acc.sum(axis=(1, 2), dtype=np.int64)                                      # [N, OC]
+    S = _window_sums(x.transpose(0, 3, 1, 2).astype(np.int64) + 128, 3, 1, H, H)    # x - zp_x, zero outside the image
+    want = np.einsum("ockl,nckl->no", wn.astype(np.int64), S)
+    assert np.array_equal(got, want)
+
+
+def test_conv2d_f32_full_size_layer(ops):
+    """The same layer in fp32 on integer-valued data (every partial sum exact in fp32): two images against the oracle,
+    exactly, with bias and ReLU; all outputs of the batch through one checksum per (image, channel)."""
+    r = rng(78)
+    N, C, H, OC = 256, 64, 56, 128
+    x = r.integers(-3, 4, (N, C, H, H)).astype(np.float32)
+    w = r.integers(-3, 4, (OC, C, 3, 3)).astype(np.float32)
+    b = r.integers(-20, 21, OC).astype(np.float32)
+    y = ops.conv2d_f32(x, w, b, (1, 1), (1, 1), (1, 1), 1, True)
+    for n in (0, 255):
+        ref = oracle.conv2d_f32(x[n:n + 1], w, b, (1, 1), (1, 1), (1, 1), 1, True)
+        assert np.array_equal(y[n], ref[0]), n
+    del y
+    lin = ops.conv2d_f32(x, w, None, (1, 1), (1, 1), (1, 1), 1, False)
+    got = lin.sum(axis=(2, 3), dtype=np.float64)
+    S = _window_sums(x.astype(np.int64), 3, 1, H, H)
+    want = np.einsum("ockl,nckl->no", w.astype(np.int64), S)
+    assert np.array_equal(got, want.astype(np.float64))
+
+
+def test_gemm_fp8_full_size(ops):
+    """M = N = 8192, K = 4096 (the benchmark's FP8 GEMM) on small integers in e4m3, which make every sum exact: 256
+    rows against the integer product, all 67 M outputs through their row sums and column sums, and the bf16 output
+    (with the bias epilogue) equal to the rounding of the fp32 output of the same kernel."""
+    from sofie_amd import lib as L
+    r = rng(79)
+    M, N, K = 8192, 8192, 4096
+    a = r.integers(-4, 5, (M, K)).astype(np.float32)
+    b = r.integers(-4, 5, (K, N)).astype(np.float32)
+    codes = oracle.e4m3_encode(np.arange(-4, 5, dtype=np.float32))              # the nine values' codes, by table
+    A, B = codes[a.astype(np.int64) + 4], codes[b.astype(np.int64) + 4]
+    y = ops.gemm_fp8(A, B, 1.0, 1.0, None, False, out=L.OUT_F32)
+    rows = r.choice(M, 256, replace=False)
+    assert np.array_equal(y[rows], a[rows] @ b)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    assert np.array_equal(y.sum(axis=1, dtype=np.float64), a64 @ b64.sum(axis=1))
+    assert np.array_equal(y.sum(axis=0, dtype=np.float64), a64.sum(axis=0) @ b64)
+    bias = r.integers(-8, 9, N).astype(np.float32)
+    Bt = np.ascontiguousarray(B.T)
+    yf = ops.gemm_fp8(A, Bt, 0.5, 0.25, bias, True, out=L.OUT_F32)
+    assert np.array_equal(yf, y * np.float32(0.125) + bias)                     # power-of-two scales keep it exact
+    yb = ops.gemm_fp8(A, Bt, 0.5, 0.25, bias, True)
+    import torch
+    assert np.array_equal(yb, torch.from_numpy(yf).bfloat16().view(torch.int16).numpy().view(np.uint16))   # torch rounds RNE
+    assert np.array_equal(yb[rows[0]], oracle.bf16_encode(yf[rows[0]]))
