@@ -585,3 +585,26 @@ def test_no_session_option_emits_a_free_infer_over_literal_weights(tmp_path):
     assert 'inline Session& DefaultSession() { static Session session(""); return session; }' in code
     assert "inline auto infer(float* tensor_x){ return DefaultSession().infer(tensor_x); }" in code
     spec.compile_runner(str(tmp_path))
+
+
+def test_cpp_onnx_front_end_graph_with_two_outputs(tmp_path):
+    """An ONNX graph that lists a hidden Gemm result and the final result as outputs: the parser keeps both in the
+    file's order, the Gemm -> Relu pair is not fused over the tensor that is an output, and infer() returns a
+    vector of two vectors."""
+    import onnx_write as ow
+    r = np.random.default_rng(6)
+    init = {"W0": r.standard_normal((6, 4)).astype(np.float32), "B0": r.standard_normal(4).astype(np.float32),
+            "W1": r.standard_normal((4, 3)).astype(np.float32), "B1": r.standard_normal(3).astype(np.float32)}
+    nodes = [ow.node("Gemm", ["x", "W0", "B0"], ["h"]), ow.node("Relu", ["h"], ["hr"]),
+             ow.node("Gemm", ["hr", "W1", "B1"], ["y"])]
+    path = tmp_path / "two_out.onnx"
+    path.write_bytes(ow.model(nodes, init, [("x", 1, (5, 6))], [("h", 1, (5, 4)), ("y", 1, (5, 3))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode == 0, res.stderr
+    code = open(str(tmp_path / "two_out.hxx")).read()
+    assert "std::vector<std::vector<float>> infer(float* tensor_x)" in code
+    assert code.index("tensor_h, ret_0.size()") < code.index("tensor_y, ret_1.size()")
+    # the pre-activation tensor h is an output: its Gemm keeps no fused ReLU, the Relu runs as its own call
+    first = re.search(r"sofie_hip_gemm_f32\([^;]*tensor_h, 4, (SOFIE_ACT_\w+)\)", code)
+    assert first and first.group(1) == "SOFIE_ACT_NONE"
+    assert "sofie_hip_relu_f32(" in code
