@@ -271,6 +271,9 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
                      }
                   }
             }
+            // keep the order written here (reads of step s in front of the matrix instructions of step s - NBUF + 1):
+            // left alone, the scheduler sinks the reads to just before their first use
+            __builtin_amdgcn_sched_barrier(0);
          }
          return;
       }
