@@ -83,7 +83,7 @@ struct QConvTileArgs {
    int RL, RP;           // 16-byte chunks per band row; band rows fetched per pass
    int ntiles;
    unsigned fill;        // zp_x replicated into four bytes
-   FastDiv dOW, dOH, dHP, dRL, dC16;
+   FastDiv dOW, dOH, dHP, dRL, dC16, dK16;
 };
 
 // POOL: a 2x2 stride-2 max pooling is fused. A wavefront then owns 32 POOLED pixels; its MB = 4
@@ -123,13 +123,29 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
    const int mtot = a.ep.M;
 
    // ---- weights of this channel block: resident for the life of the workgroup
+   // The slice is contiguous in global memory (OCT rows of K bytes), so 16-byte chunk q of it sits at wsrc + 16 q and
+   // goes to row q / K16, column chunk q % K16 of the padded LDS rows. A thread has up to WCH loads in flight before
+   // it writes the first one: one load per store would pay the full memory latency for every chunk, with every
+   // workgroup of the launch asking for the same lines at the same time.
    {
+      constexpr int WCH = 8;
       const int K16 = a.K >> 4;
+      const int total = OCT * K16;
       const int8_t *wsrc = a.w + (size_t)ob * OCT * a.K;
-      for (int r = wave; r < OCT; r += 8)
-         for (int c = lane; c < K16; c += 64)
-            *reinterpret_cast<v4i *>(s_w + r * a.KS + c * 16) =
-               *reinterpret_cast<const v4i *>(wsrc + (size_t)r * a.K + c * 16);
+      for (int base = tid; base < total; base += 512 * WCH) {
+         v4i chunk[WCH];
+#pragma unroll
+         for (int u = 0; u < WCH; ++u) {
+            const int q = base + u * 512;
+            chunk[u] = *reinterpret_cast<const v4i *>(wsrc + (size_t)(q < total ? q : base) * 16);
+         }
+#pragma unroll
+         for (int u = 0; u < WCH; ++u) {
+            const int q = base + u * 512;
+            const int r = fdiv(q, a.dK16);
+            if (q < total) *reinterpret_cast<v4i *>(s_w + r * a.KS + (q - r * K16) * 16) = chunk[u];
+         }
+      }
    }
 
    stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
@@ -492,7 +508,7 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.ntiles = (int)((mtot + TM - 1) / TM);
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
    a.dOW = make_fastdiv(TW); a.dOH = make_fastdiv(TH); a.dHP = make_fastdiv(HP);
-   a.dRL = make_fastdiv(a.RL); a.dC16 = make_fastdiv(a.C16);
+   a.dRL = make_fastdiv(a.RL); a.dC16 = make_fastdiv(a.C16); a.dK16 = make_fastdiv(a.K / 16);
    // most rows a band can have: the convolution rows a tile touches, the image boundaries it can cross
    // (each adds the rows between the last window of one image and the first of the next) and KH - 1
    const int tile_rows = (TM - 1) / TW + 2;

@@ -251,8 +251,11 @@ __device__ __forceinline__ void stage_column_params(const GemmArgs &g, float *s_
 {
    if (tid < BN) {
       const int n = n0 + tid;
-      s_scale[tid] = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
-      s_bias[tid] = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
+      // both loads are issued before either value is stored
+      const float sc = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
+      const int bi = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
+      s_scale[tid] = sc;
+      s_bias[tid] = bi;
    }
 }
 
