@@ -61,6 +61,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-rows", type=int, default=1024)
+    ap.add_argument("--cpu-images", type=int, default=256, help="images of the CNN batch the CPU baseline leg evaluates")
     ap.add_argument("--extras", action="store_true", help="also time the FP8 GEMM, fp32 GEMM and conv layers")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch a 64 MiB copy-like kernel and the headline call three times and exit (the target of the "
@@ -145,7 +146,7 @@ def main():
         out["cpu_baseline"] = None
 
     # second half of the metric: the int8 CNN Session at batch 4096 (its own process, runs in about a second)
-    out["model_inferences"] = cnn_session_rate()
+    out["model_inferences"] = cnn_session_rate(cpu_images=0 if args.no_cpu else args.cpu_images)
     # the FP8 half of the metric's GEMM figure (e4m3 x e4m3, fp32 accumulate, bf16 out): B as it comes ([K,N])
     fp8 = fp8_gemm_rates(ctx, torch, L)["fp8_gemm_8192x8192x4096_transB0"]
     out["fp8_gemm"] = {"workload": "FP8 e4m3 GEMM M=N=8192 K=4096, B [K,N], bias, bf16 out", "ms": fp8["ms"],
@@ -241,10 +242,12 @@ def extras(ctx, torch, L, ops, rng):
     return ex
 
 
-def cnn_session_rate(iters=50):
+def cnn_session_rate(iters=50, cpu_images=0):
     """The generated Session of the int8 CNN at batch 4096 (1x40x40 input; conv 1->32, pool, conv 32->64, pool,
     conv 64->128, fc 12800->256, fc 256->5), run by its prebuilt runner as a child process: device time of
-    infer_device() on a resident input, and wall time of infer() including the PCIe copies."""
+    infer_device() on a resident input, and wall time of infer() including the PCIe copies. With cpu_images > 0 the
+    CPU restatement of the same network is timed on that many images of the batch (one thread) and the Session's
+    logits of those images are compared with it bit for bit."""
     import subprocess
     import tempfile
     gen = os.path.join(ROOT, "sofie_amd", "generated")
@@ -253,14 +256,30 @@ def cnn_session_rate(iters=50):
         return {"error": "generated Session missing: run build() first"}
     with tempfile.TemporaryDirectory() as tmp:
         xin, yout = os.path.join(tmp, "x.bin"), os.path.join(tmp, "y.bin")
-        np.random.default_rng(2).uniform(0, 1, (4096, 1, 40, 40)).astype(np.float32).tofile(xin)
+        x = np.random.default_rng(2).uniform(0, 1, (4096, 1, 40, 40)).astype(np.float32)
+        x.tofile(xin)
         res = subprocess.run([exe, dat, xin, yout, str(iters)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
                              timeout=300)
+        y = np.fromfile(yout, np.float32) if res.returncode == 0 else None
     if res.returncode != 0:
         return {"error": res.stderr.strip()[-300:]}
     t = json.loads(res.stdout.strip().splitlines()[-1])
     ops_per_image = 36968960.0
-    return {"workload": "int8 CNN classifier, batch 4096, 1x40x40 input, generated Session (infer_device on a resident input)",
+    cpu = None
+    if cpu_images > 0:
+        # checker and baseline: the oracle's network (tests/models.py builds it from the same seeded parameters)
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        import models
+        from oracle import oracle
+        models.qcnn_reference(oracle, x[:2])           # parameters and calibration are built on the first call
+        t0 = time.perf_counter()
+        ref = models.qcnn_reference(oracle, x[:cpu_images])
+        sec = time.perf_counter() - t0
+        cpu = {"value": cpu_images / sec, "unit": "inferences/s", "cores": 1, "kind": "port",
+               "sample": "oracle/sofie_oracle.c (quantize, three QLinearConv + ReLU + MaxPool, two QLinearMatMul) on the first "
+                         "%d of the 4096 images (%.2f s, gcc -O2, 1 thread)" % (cpu_images, sec),
+               "logits_bit_exact": bool(np.array_equal(y.reshape(4096, -1)[:cpu_images], ref.reshape(cpu_images, -1)))}
+    return {"cpu_baseline": cpu,"workload": "int8 CNN classifier, batch 4096, 1x40x40 input, generated Session (infer_device on a resident input)",
             "device_ms": t["device_ms"], "inferences_per_s": 4096 / (t["device_ms"] * 1e-3),
             "tops": 4096 * ops_per_image / t["device_ms"] / 1e9,
             "frac_peak": 4096 * ops_per_image / t["device_ms"] / 1e9 / PEAK_INT8_TOPS,
