@@ -266,11 +266,13 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
          for (int s = 0; s < NS + NBUF - 1; ++s) {
             if (s < NS) {
                const int kh = s / (3 * KFIX), kw = (s / KFIX) % 3, cb = s % KFIX;
+               // in the order the matrix instructions of the step need them: weights 0, every pixel tile, weights 1...
+               fb[s % NBUF][0] = *reinterpret_cast<const v4i *>(pb[0] + s * 32);
 #pragma unroll
                for (int j = 0; j < MB; ++j)
                   fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[kh][j] + (kw * CSF + cb * 32));
 #pragma unroll
-               for (int i = 0; i < NB; ++i) fb[s % NBUF][i] = *reinterpret_cast<const v4i *>(pb[i] + s * 32);
+               for (int i = 1; i < NB; ++i) fb[s % NBUF][i] = *reinterpret_cast<const v4i *>(pb[i] + s * 32);
             }
             if (s >= NBUF - 1) {
                const int d = s - (NBUF - 1), buf = d % NBUF;
@@ -287,8 +289,18 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
                      }
                   }
             }
-            // keep the order written here (reads of step s in front of the matrix instructions of step s - NBUF + 1):
-            // left alone, the scheduler sinks the reads to just before their first use
+            // Pin the order: left alone, the scheduler sinks the fragment reads of a step to just before their first use
+            // (or, in the pooled instance, behind all but one of the step's matrix instructions). One read is issued
+            // behind each of the first matrix instructions of the step, so every read has at least the rest of the step
+            // to land and the reads do not queue up in front of the matrix instructions.
+            if (s < NS && s >= NBUF - 1) {
+#pragma unroll
+               for (int gidx = 0; gidx < MB + NB; ++gidx) {
+                  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
+                  __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+               }
+               __builtin_amdgcn_sched_group_barrier(0x008, MB * NB - (MB + NB) > 0 ? MB * NB - (MB + NB) : 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
          }
          return;
