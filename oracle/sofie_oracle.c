@@ -17,9 +17,14 @@
  *                                (the reference holds no 3-D fixture); with a depth of one it
  *                                must equal or_conv2d_f32
  *   or_conv_transpose2d_f32      pinned: ConvTranspose1d/2d/Bias2d/Bias2dBatched known
- *                                answers, torch.nn.functional.conv_transpose2d on CPU
- *   or_batchnorm_f32             pinned: torch.nn.functional.batch_norm on CPU, float64
- *                                closed form (the reference holds no fixture for it)
+ *                                answers (stride 1, no pads); for strides, dilations, groups,
+ *                                begin != end pads and output padding:
+ *                                torch.nn.functional.conv_transpose2d on CPU in float64 and the
+ *                                scatter definition written out in float64
+ *                                (tests/test_oracle_math.py, the grid the GPU test uses)
+ *   or_batchnorm_f32             pinned: torch.nn.functional.batch_norm (evaluation mode) on CPU
+ *                                and the float64 closed form, with and without ReLU, two values
+ *                                of epsilon (the reference holds no fixture for it)
  *   or_einsum_f32                pinned: Einsum_matmul / _dotprod / _3 / _4 known answers of
  *                                the reference's tests, numpy.einsum in float64
  *   or_relu, or_maxpool2d        pinned: MaxPool2d known answer, torch CPU

@@ -73,6 +73,8 @@ def test_reference_known_answers_through_hip(ops, name):
     dict(N=1, C=4, H=5, W=5, OC=4, k=(2, 2), s=(1, 1), p=(2, 2, 2, 2), d=(1, 1), g=1, op=(0, 0)),       # pad beyond the kernel
     dict(N=1, C=2, H=3, W=40, OC=3, k=(1, 9), s=(1, 4), p=(0, 2, 0, 2), d=(1, 1), g=1, op=(0, 3)),
     dict(N=1, C=2, H=2, W=2, OC=2, k=(31, 31), s=(1, 1), p=(0, 0, 0, 0), d=(1, 1), g=1, op=(0, 0)),     # large kernel
+    dict(N=2, C=4, H=6, W=5, OC=6, k=(3, 4), s=(2, 3), p=(0, 2, 1, 0), d=(1, 1), g=2, op=(1, 2)),       # begin != end pads
+    dict(N=1, C=3, H=5, W=7, OC=2, k=(3, 3), s=(2, 1), p=(2, 0, 0, 1), d=(2, 2), g=1, op=(0, 0)),
 ])
 def test_conv_transpose2d_f32(ops, cfg):
     """ConvTranspose through the implicit-GEMM kernel over the zero-interleaved input against the oracle's

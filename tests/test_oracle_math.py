@@ -363,3 +363,138 @@ def test_conv3d_f32_against_torch_and_depth_one_conv2d(cfg):
     y3 = oracle.conv3d_f32(x2, w2, b, (0,) + tuple(pads[1:]), (1,) + tuple(strides[1:]), (1,) + tuple(dil[1:]), groups, relu=True)
     y2 = oracle.conv2d_f32(x2[:, :, 0], w2[:, :, 0], b, pads[1:], strides[1:], dil[1:], groups, relu=True)
     assert np.array_equal(y3[:, :, 0], y2)
+
+
+# ----------------------------------------------------------------------------- fp32 BatchNormalization
+@pytest.mark.parametrize("shape", [(3, 5, 4, 7), (6, 9), (2, 4, 11)])
+@pytest.mark.parametrize("eps", [1e-5, 1e-3])
+@pytest.mark.parametrize("relu", [False, True])
+def test_batchnorm_f32_against_torch_and_float64(shape, eps, relu):
+    """Inference BatchNormalization (the reference holds no fixture for it): torch's batch_norm in
+    evaluation mode on CPU and the float64 closed form gamma * (x - mean) / sqrt(var + eps) + beta.
+    The operands are drawn apart (mean far from 0, variance near eps in one channel, a negative gamma)
+    so that a swapped operand, a missing eps or a ReLU applied before the shift fails."""
+    r = rng(70 + len(shape))
+    C = shape[1]
+    x = (r.standard_normal(shape) * 3 + 1.5).astype(np.float32)
+    gamma = r.uniform(0.5, 2.0, C).astype(np.float32)
+    gamma[1] = -gamma[1]
+    beta = r.standard_normal(C).astype(np.float32)
+    mean = (r.standard_normal(C) * 2 + 0.7).astype(np.float32)
+    var = r.uniform(0.2, 3.0, C).astype(np.float32)
+    var[0] = 2e-4                                             # eps matters here
+    y = oracle.batchnorm_f32(x, gamma, beta, mean, var, eps, relu)
+    bshape = (1, C) + (1,) * (len(shape) - 2)
+    x64 = x.astype(np.float64)
+    t = (gamma.astype(np.float64).reshape(bshape) * (x64 - mean.astype(np.float64).reshape(bshape))
+         / np.sqrt(var.astype(np.float64).reshape(bshape) + eps) + beta.astype(np.float64).reshape(bshape))
+    tt = F.batch_norm(torch.from_numpy(x), torch.from_numpy(mean), torch.from_numpy(var), torch.from_numpy(gamma),
+                      torch.from_numpy(beta), training=False, eps=eps).numpy()
+    if relu:
+        t = np.maximum(t, 0)
+        tt = np.maximum(tt, 0)
+    assert y.shape == x.shape
+    assert np.max(np.abs(y - t)) <= 1e-5 * np.max(np.abs(t))
+    assert np.max(np.abs(y - tt)) <= 1e-5 * np.max(np.abs(tt))
+    # eps must enter under the root: with eps = 0 channel 0 differs visibly
+    t0 = gamma[0] * (x64.take(0, axis=1) - mean[0]) / np.sqrt(np.float64(var[0]))
+    got0 = y.take(0, axis=1) - beta[0]
+    if not relu:
+        assert np.max(np.abs(got0 - t0)) > 1e-3 * np.max(np.abs(t0))
+
+
+# ----------------------------------------------------------------------------- fp32 transposed convolution
+CONVT_GRID = [
+    dict(N=2, C=4, H=5, W=6, OC=6, k=(3, 3), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(0, 0)),
+    dict(N=1, C=6, H=4, W=4, OC=4, k=(2, 3), s=(3, 2), p=(0, 1, 0, 1), d=(2, 1), g=2, op=(1, 1)),
+    dict(N=2, C=3, H=7, W=5, OC=5, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(1, 0)),
+    dict(N=3, C=64, H=14, W=14, OC=96, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(0, 0)),
+    dict(N=2, C=32, H=9, W=11, OC=32, k=(3, 3), s=(1, 1), p=(1, 1, 1, 1), d=(1, 1), g=4, op=(0, 0)),
+    dict(N=1, C=8, H=6, W=6, OC=8, k=(3, 3), s=(2, 2), p=(2, 2, 2, 2), d=(1, 1), g=1, op=(1, 1)),
+    dict(N=1, C=4, H=5, W=5, OC=4, k=(2, 2), s=(1, 1), p=(2, 2, 2, 2), d=(1, 1), g=1, op=(0, 0)),
+    dict(N=1, C=2, H=3, W=40, OC=3, k=(1, 9), s=(1, 4), p=(0, 2, 0, 2), d=(1, 1), g=1, op=(0, 3)),
+    dict(N=1, C=2, H=2, W=2, OC=2, k=(31, 31), s=(1, 1), p=(0, 0, 0, 0), d=(1, 1), g=1, op=(0, 0)),
+    # begin pads that differ from the end pads (torch only knows symmetric ones: see the test)
+    dict(N=2, C=4, H=6, W=5, OC=6, k=(3, 4), s=(2, 3), p=(0, 2, 1, 0), d=(1, 1), g=2, op=(1, 2)),
+    dict(N=1, C=3, H=5, W=7, OC=2, k=(3, 3), s=(2, 1), p=(2, 0, 0, 1), d=(2, 2), g=1, op=(0, 0)),
+]
+
+
+def _convt_scatter64(x, w, bias, cfg):
+    """The definition of ONNX ConvTranspose as a scatter in float64: every input value adds
+    x * w[ic, oc, kh, kw] to y[oc, iy*stride + kh*dil - pad_begin, ...]; outputs outside [0, OH) are dropped."""
+    N, C, H, W = x.shape
+    g = cfg["g"]
+    ocg = w.shape[1]
+    kh, kw = cfg["k"]
+    sh, sw = cfg["s"]
+    dh, dw = cfg["d"]
+    pt, pl, pb, pr = cfg["p"]
+    OH = sh * (H - 1) + dh * (kh - 1) + 1 + cfg["op"][0] - pt - pb
+    OW = sw * (W - 1) + dw * (kw - 1) + 1 + cfg["op"][1] - pl - pr
+    y = np.zeros((N, ocg * g, OH, OW), np.float64)
+    cg = C // g
+    for ic in range(C):
+        grp = ic // cg
+        for a in range(kh):
+            for b in range(kw):
+                for iy in range(H):
+                    oy = iy * sh + a * dh - pt
+                    if not 0 <= oy < OH:
+                        continue
+                    for ix in range(W):
+                        ox = ix * sw + b * dw - pl
+                        if not 0 <= ox < OW:
+                            continue
+                        y[:, grp * ocg:(grp + 1) * ocg, oy, ox] += np.outer(x[:, ic, iy, ix].astype(np.float64),
+                                                                            w[ic, :, a, b].astype(np.float64))
+    if bias is not None:
+        y += bias.astype(np.float64).reshape(1, -1, 1, 1)
+    return y
+
+
+@pytest.mark.parametrize("cfg", CONVT_GRID)
+def test_conv_transpose2d_f32_against_torch_and_scatter(cfg):
+    """or_conv_transpose2d_f32 over the grid of strides, dilations, groups, pads and output paddings that
+    the GPU test compares the kernel with. Two independent answers: torch's conv_transpose2d on CPU in
+    float64 (symmetric pads only: for begin != end pads torch is run without padding and the result cropped
+    by the begin pads on the top/left and the end pads on the bottom/right, which is ONNX's definition) and
+    the scatter definition written out in float64. The reference's fixtures only cover stride 1 without
+    pads, groups, dilation or output padding."""
+    r = rng(40 + cfg["C"] + cfg["H"])
+    x = r.standard_normal((cfg["N"], cfg["C"], cfg["H"], cfg["W"])).astype(np.float32)
+    w = (r.standard_normal((cfg["C"], cfg["OC"] // cfg["g"]) + cfg["k"]) * 0.2).astype(np.float32)
+    b = r.standard_normal(cfg["OC"]).astype(np.float32)
+    pt, pl, pb, pr = cfg["p"]
+    for bias, relu in ((b, False), (None, True)):
+        y = oracle.conv_transpose2d_f32(x, w, bias, cfg["p"], cfg["s"], cfg["d"], cfg["g"], cfg["op"], relu)
+        full = F.conv_transpose2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(),
+                                  None if bias is None else torch.from_numpy(bias).double(),
+                                  stride=cfg["s"], padding=0, output_padding=0, groups=cfg["g"],
+                                  dilation=cfg["d"]).numpy()
+        # output padding appends rows/columns that receive no contribution (bias only)
+        oph, opw = cfg["op"]
+        full = np.pad(full, ((0, 0), (0, 0), (0, oph), (0, opw)))
+        if bias is not None and (oph or opw):
+            bb = bias.astype(np.float64).reshape(1, -1, 1, 1)
+            if oph:
+                full[:, :, -oph:, :] = bb
+            if opw:
+                full[:, :, :, -opw:] = bb
+        t = full[:, :, pt:full.shape[2] - pb, pl:full.shape[3] - pr]
+        s = _convt_scatter64(x, w, bias, cfg)
+        if relu:
+            t = np.maximum(t, 0)
+            s = np.maximum(s, 0)
+        assert y.shape == t.shape == s.shape
+        scale = max(np.max(np.abs(t)), 1e-30)
+        assert np.max(np.abs(s - t)) <= 1e-12 * scale            # the two truths agree
+        assert np.max(np.abs(y - t)) <= 1e-5 * scale
+        if pt == pb and pl == pr and oph < max(cfg["s"][0], cfg["d"][0]) and opw < max(cfg["s"][1], cfg["d"][1]):
+            tsym = F.conv_transpose2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(),
+                                      None if bias is None else torch.from_numpy(bias).double(),
+                                      stride=cfg["s"], padding=(pt, pl), output_padding=cfg["op"],
+                                      groups=cfg["g"], dilation=cfg["d"]).numpy()
+            if relu:
+                tsym = np.maximum(tsym, 0)
+            assert np.max(np.abs(y - tsym)) <= 1e-5 * scale
