@@ -91,8 +91,12 @@ int sofie_hip_sync(sofie_hip_ctx *ctx);
  * as a small MLP, then costs one submission instead of one per operator). The recorded calls keep their
  * pointer arguments. Nothing may allocate while recording: run the sequence once eagerly first, so that the
  * context's scratch buffer has its final size (a call that would grow it fails with a message saying so).
- * Uploads, downloads, memset and sync are not to be called between begin and end. capture_end with a NULL result
- * pointer abandons the recording. No counterpart in the reference (its generated code is a CPU call sequence). */
+ * Between begin and end sofie_hip_malloc, _free, _upload, _download, _memset, _sync, _timer_start, _timer_stop and
+ * _graph_destroy return SOFIE_HIP_EINVAL and do nothing (they would wait on, or record a memset node into, the
+ * capturing stream). capture_end with a NULL result pointer abandons the recording. A recorded graph keeps the
+ * address of the context's scratch buffer: until it is destroyed, a later call on the same context that needs a
+ * larger scratch buffer fails with SOFIE_HIP_EINVAL instead of freeing the buffer under the graph. No counterpart
+ * in the reference (its generated code is a CPU call sequence). */
 typedef struct sofie_hip_graph sofie_hip_graph;
 int sofie_hip_capture_begin(sofie_hip_ctx *ctx);
 int sofie_hip_capture_end(sofie_hip_ctx *ctx, sofie_hip_graph **graph);

@@ -16,6 +16,7 @@ struct sofie_hip_ctx {
    void *workspace = nullptr;   // scratch owned by the context (layout changes, B transposes)
    size_t workspace_bytes = 0;
    bool capturing = false;      // between sofie_hip_capture_begin and _end: nothing may allocate or synchronise
+   int live_graphs = 0;         // recorded graphs not yet destroyed: they hold the scratch buffer's address
    char err[512] = {0};
 };
 

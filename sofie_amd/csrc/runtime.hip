@@ -22,6 +22,11 @@ int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr)
       if (ctx->capturing)
          return set_error(ctx, SOFIE_HIP_EINVAL, "the scratch buffer would grow to %zu bytes while a graph is captured: "
                           "run the same calls once before capturing", bytes);
+      // a recorded graph keeps the address of the buffer it was recorded with: freeing it would leave the next
+      // replay reading and writing freed device memory
+      if (ctx->live_graphs > 0)
+         return set_error(ctx, SOFIE_HIP_EINVAL, "the scratch buffer would grow to %zu bytes while %d recorded graph(s) of "
+                          "this context still use the present one: destroy them first", bytes, ctx->live_graphs);
       // the old buffer may still be read by kernels in flight on the stream
       if (ctx->workspace) {
          SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
@@ -86,6 +91,13 @@ int sofie_hip_create(sofie_hip_ctx **out, int device, void *stream)
 int sofie_hip_destroy(sofie_hip_ctx *ctx)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   if (ctx->capturing) {   // an open recording is given up: a capturing stream cannot be waited for
+      hipGraph_t dropped = nullptr;
+      (void)hipStreamEndCapture(ctx->stream, &dropped);
+      if (dropped) (void)hipGraphDestroy(dropped);
+      (void)hipGetLastError();
+      ctx->capturing = false;
+   }
    (void)hipStreamSynchronize(ctx->stream);
    if (ctx->workspace) (void)hipFree(ctx->workspace);
    (void)hipEventDestroy(ctx->ev_start);
@@ -100,6 +112,7 @@ const char *sofie_hip_last_error(const sofie_hip_ctx *ctx) { return ctx ? ctx->e
 int sofie_hip_malloc(sofie_hip_ctx *ctx, void **dptr, size_t bytes)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    SOFIE_REQUIRE(ctx, dptr != nullptr, "null result pointer");
    *dptr = nullptr;
    if (bytes == 0) return SOFIE_HIP_OK;
@@ -113,6 +126,7 @@ int sofie_hip_malloc(sofie_hip_ctx *ctx, void **dptr, size_t bytes)
 int sofie_hip_free(sofie_hip_ctx *ctx, void *dptr)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    if (!dptr) return SOFIE_HIP_OK;
    SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
    SOFIE_HIP_CALL(ctx, hipFree(dptr));
@@ -122,6 +136,7 @@ int sofie_hip_free(sofie_hip_ctx *ctx, void *dptr)
 int sofie_hip_upload(sofie_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    if (bytes == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, dst && src, "null pointer");
    SOFIE_HIP_CALL(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, ctx->stream));
@@ -132,6 +147,7 @@ int sofie_hip_upload(sofie_hip_ctx *ctx, void *dst, const void *src, size_t byte
 int sofie_hip_download(sofie_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    if (bytes == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, dst && src, "null pointer");
    SOFIE_HIP_CALL(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, ctx->stream));
@@ -151,6 +167,7 @@ int sofie_hip_copy(sofie_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
 int sofie_hip_memset(sofie_hip_ctx *ctx, void *dptr, int value, size_t bytes)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    if (bytes == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, dptr != nullptr, "null pointer");
    SOFIE_HIP_CALL(ctx, hipMemsetAsync(dptr, value, bytes, ctx->stream));
@@ -160,6 +177,7 @@ int sofie_hip_memset(sofie_hip_ctx *ctx, void *dptr, int value, size_t bytes)
 int sofie_hip_sync(sofie_hip_ctx *ctx)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));
    return SOFIE_HIP_OK;
 }
@@ -202,6 +220,7 @@ int sofie_hip_capture_end(sofie_hip_ctx *ctx, sofie_hip_graph **out)
    g->graph = graph;
    g->exec = exec;
    *out = g;
+   ++ctx->live_graphs;
    return SOFIE_HIP_OK;
 }
 
@@ -217,17 +236,20 @@ int sofie_hip_graph_launch(sofie_hip_ctx *ctx, sofie_hip_graph *g)
 int sofie_hip_graph_destroy(sofie_hip_ctx *ctx, sofie_hip_graph *g)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    if (!g) return SOFIE_HIP_OK;
    (void)hipStreamSynchronize(ctx->stream);
    if (g->exec) (void)hipGraphExecDestroy(g->exec);
    if (g->graph) (void)hipGraphDestroy(g->graph);
    delete g;
+   if (ctx->live_graphs > 0) --ctx->live_graphs;
    return SOFIE_HIP_OK;
 }
 
 int sofie_hip_timer_start(sofie_hip_ctx *ctx)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    SOFIE_HIP_CALL(ctx, hipEventRecord(ctx->ev_start, ctx->stream));
    return SOFIE_HIP_OK;
 }
@@ -235,6 +257,7 @@ int sofie_hip_timer_start(sofie_hip_ctx *ctx)
 int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *ms)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
    SOFIE_REQUIRE(ctx, ms != nullptr, "null result pointer");
    SOFIE_HIP_CALL(ctx, hipEventRecord(ctx->ev_stop, ctx->stream));
    SOFIE_HIP_CALL(ctx, hipEventSynchronize(ctx->ev_stop));

@@ -17,10 +17,19 @@ class SofieHipError(RuntimeError):
     pass
 
 
-class Context:
-    """One sofie_hip_ctx bound to torch's current stream on `device`."""
+GUARD_BYTES = 512          # sentinel band on either side of every output buffer (a multiple of 256: keeps alignment)
+GUARD_VALUE = 0xA5
 
-    def __init__(self, device=0):
+
+class Context:
+    """One sofie_hip_ctx on `device`. The library launches on torch's current stream when that is a stream of
+    its own; with torch's default (null) stream the handle is NULL and sofie_hip_create opens a blocking stream,
+    which the null stream's implicit synchronisation orders against torch's own work (copies, fills).
+
+    Every output buffer that `empty` hands out lies between two sentinel bands that `ret` checks after the
+    call: a store outside the tensor (a ragged tile written past its edge) raises instead of going unseen."""
+
+    def __init__(self, device=0, guard=True):
         if not torch.cuda.is_available():
             raise SofieHipError("no GPU visible: the HIP library has no CPU fallback")
         self.lib = L.load()
@@ -32,6 +41,8 @@ class Context:
         if rc:
             raise SofieHipError("sofie_hip_create failed: %d" % rc)
         self.h = h
+        self.guard = guard
+        self._guarded = []
 
     def close(self):
         if self.h:
@@ -50,7 +61,9 @@ class Context:
             raise SofieHipError("%s (status %d)" % (msg, rc))
 
     def sync(self):
+        """Waits for the stream, then checks the sentinel bands of the buffers handed out since the last wait."""
         self.check(self.lib.sofie_hip_sync(self.h))
+        self._check_guards()
 
     def timer_start(self):
         self.check(self.lib.sofie_hip_timer_start(self.h))
@@ -76,7 +89,33 @@ class Context:
         return C.c_void_p(t.data_ptr()) if t is not None else None
 
     def empty(self, shape, dtype):
-        return torch.empty(shape, dtype=dtype, device=self.device)
+        if not self.guard:
+            return torch.empty(shape, dtype=dtype, device=self.device)
+        shape = tuple(int(d) for d in shape)
+        n = int(np.prod(shape, dtype=np.int64)) * torch.empty((), dtype=dtype).element_size()
+        raw = torch.empty(2 * GUARD_BYTES + n, dtype=torch.uint8, device=self.device)
+        raw[:GUARD_BYTES] = GUARD_VALUE
+        raw[GUARD_BYTES + n:] = GUARD_VALUE
+        self._guarded.append((raw, n))
+        return raw[GUARD_BYTES:GUARD_BYTES + n].view(dtype).view(shape)
+
+    def verify_guards(self):
+        if self._guarded:
+            self.sync()
+
+    def _check_guards(self):
+        pending, self._guarded = self._guarded, []
+        for raw, n in pending:
+            lo, hi = raw[:GUARD_BYTES], raw[GUARD_BYTES + n:]
+            if not (bool((lo == GUARD_VALUE).all()) and bool((hi == GUARD_VALUE).all())):
+                bad_lo = int((lo != GUARD_VALUE).sum())
+                bad_hi = int((hi != GUARD_VALUE).sum())
+                raise SofieHipError("a kernel wrote outside its output buffer of %d bytes: %d bytes changed in front of it, "
+                                    "%d behind it" % (n, bad_lo, bad_hi))
+
+    def ret(self, t, like):
+        self.verify_guards()
+        return t.cpu().numpy() if isinstance(like, np.ndarray) else t
 
 
 _default = None
@@ -87,10 +126,6 @@ def default_context():
     if _default is None:
         _default = Context(0)
     return _default
-
-
-def _ret(t, like):
-    return t.cpu().numpy() if isinstance(like, np.ndarray) else t
 
 
 # ------------------------------------------------------------------------------- fp32
@@ -113,15 +148,15 @@ def gemm_f32(A, B, bias=None, alpha=1.0, beta=1.0, transA=False, transB=False, r
     ctx.check(ctx.lib.sofie_hip_gemm_f32(ctx.h, int(transA), int(transB), M, N, K, alpha, ctx.ptr(a), a.shape[1],
                                          ctx.ptr(b), b.shape[1], beta, ctx.ptr(bt), kind, ctx.ptr(y), N,
                                          L.ACT_RELU if relu else L.ACT_NONE))
-    return _ret(y, A)
+    return ctx.ret(y, A)
 
 
 def relu_f32(x, ctx=None):
     ctx = ctx or default_context()
     xd = ctx.dev(x, torch.float32)
-    y = torch.empty_like(xd)
+    y = ctx.empty(tuple(xd.shape), torch.float32)
     ctx.check(ctx.lib.sofie_hip_relu_f32(ctx.h, ctx.ptr(xd), ctx.ptr(y), xd.numel()))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def conv_out_hw(H, W, kh, kw, ph, pw, sh, sw, dh=1, dw=1):
@@ -138,7 +173,7 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
     ctx.check(ctx.lib.sofie_hip_conv2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, H, W,
                                            OC, kh, kw, pads[0], pads[1], strides[0], strides[1], dilations[0],
                                            dilations[1], groups, L.ACT_RELU if relu else L.ACT_NONE))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def conv3d_f32(x, w, bias=None, pads=(0, 0, 0), strides=(1, 1, 1), dilations=(1, 1, 1), groups=1, relu=False, ctx=None):
@@ -151,7 +186,7 @@ def conv3d_f32(x, w, bias=None, pads=(0, 0, 0), strides=(1, 1, 1), dilations=(1,
     y = ctx.empty((N, OC, out[0], out[1], out[2]), torch.float32)
     ctx.check(ctx.lib.sofie_hip_conv3d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, D, H, W, OC, kd, kh, kw,
                                            *pads, *strides, *dilations, groups, L.ACT_RELU if relu else L.ACT_NONE))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def conv_transpose2d_f32(x, w, bias=None, pads=(0, 0, 0, 0), strides=(1, 1), dilations=(1, 1), groups=1,
@@ -169,7 +204,7 @@ def conv_transpose2d_f32(x, w, bias=None, pads=(0, 0, 0, 0), strides=(1, 1), dil
                                                      W, OC, kh, kw, pads[0], pads[1], strides[0], strides[1],
                                                      dilations[0], dilations[1], groups, OH, OW,
                                                      L.ACT_RELU if relu else L.ACT_NONE))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def batchnorm_f32(x, scale, bias, mean, var, epsilon=1e-5, relu=False, ctx=None):
@@ -185,7 +220,7 @@ def batchnorm_f32(x, scale, bias, mean, var, epsilon=1e-5, relu=False, ctx=None)
     y = ctx.empty(tuple(xd.shape), torch.float32)
     ctx.check(ctx.lib.sofie_hip_batchnorm_f32(ctx.h, ctx.ptr(xd), ctx.ptr(sd), ctx.ptr(md), ctx.ptr(bd), ctx.ptr(y), N, Cc,
                                               plane, L.ACT_RELU if relu else L.ACT_NONE))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def _matrix_product_type(ins, out, summed):
@@ -258,7 +293,7 @@ def einsum_f32(equation, operands, ctx=None):
         st = (C.c_longlong * max(1, len(strides)))(*strides)
         ctx.check(ctx.lib.sofie_hip_einsum_f32(ctx.h, len(xs), ptrs, len(labels), len(out), ext, st, ctx.ptr(y)))
     y = y.view(oshape)
-    return _ret(y, operands[0])
+    return ctx.ret(y, operands[0])
 
 
 def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0), layout=L.LAYOUT_NCHW, ctx=None):
@@ -281,7 +316,7 @@ def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0), layout=L.LAYOUT_NCHW, ctx=N
         ctx.check(ctx.lib.sofie_hip_maxpool2d_s8(ctx.h, ctx.ptr(xd), ctx.ptr(y), layout, N, Cc, H, W, kernel[0],
                                                  kernel[1], pads[0], pads[1], pads[2], pads[3], strides[0],
                                                  strides[1]))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 # ------------------------------------------------------------------------------- int8
@@ -290,7 +325,7 @@ def quantize_f32_s8(x, scale, zp=0, ctx=None):
     xd = ctx.dev(x, torch.float32)
     q = ctx.empty(xd.shape, torch.int8)
     ctx.check(ctx.lib.sofie_hip_quantize_f32_s8(ctx.h, ctx.ptr(xd), ctx.ptr(q), xd.numel(), float(scale), int(zp)))
-    return _ret(q, x)
+    return ctx.ret(q, x)
 
 
 def dequantize_s8_f32(q, scale, zp=0, ctx=None):
@@ -298,7 +333,7 @@ def dequantize_s8_f32(q, scale, zp=0, ctx=None):
     qd = ctx.dev(q, torch.int8)
     x = ctx.empty(qd.shape, torch.float32)
     ctx.check(ctx.lib.sofie_hip_dequantize_s8_f32(ctx.h, ctx.ptr(qd), ctx.ptr(x), qd.numel(), float(scale), int(zp)))
-    return _ret(x, q)
+    return ctx.ret(x, q)
 
 
 _OUT_DTYPE = {L.OUT_S8: torch.int8, L.OUT_F32: torch.float32, L.OUT_S32: torch.int32, L.OUT_BF16: torch.bfloat16}
@@ -326,7 +361,7 @@ def qgemm_s8(A, B, scale, bias=None, transB=False, zpa=0, zpy=0, relu=False, out
     ctx.check(ctx.lib.sofie_hip_qgemm_s8(ctx.h, int(transB), M, N, K, ctx.ptr(a), a.shape[1], ctx.ptr(b),
                                          b.shape[1], ctx.ptr(sd), ctx.ptr(bd), int(zpy),
                                          L.ACT_RELU if relu else L.ACT_NONE, ctx.ptr(y), N, out))
-    return _ret(y, A)
+    return ctx.ret(y, A)
 
 
 def qgemm_s8_f32out(A, B, scale, bias=None, transB=False, zpa=0, relu=False, ctx=None):
@@ -370,7 +405,7 @@ def qconv2d_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zp
                                            ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, pads[0], pads[1],
                                            strides[0], strides[1], groups, int(zpx), int(zpy),
                                            L.ACT_RELU if relu else L.ACT_NONE, out))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def qconv2d_pool_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, zpy=0, relu=False,
@@ -398,7 +433,7 @@ def qconv2d_pool_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=
                                                 pads[1], strides[0], strides[1], groups, int(zpx), int(zpy),
                                                 L.ACT_RELU if relu else L.ACT_NONE, pool[0], pool[1], pool_strides[0],
                                                 pool_strides[1]))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def quantize_qconv2d_s8(x, x_scale, zpx, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zpy=0, relu=False,
@@ -424,7 +459,7 @@ def quantize_qconv2d_s8(x, x_scale, zpx, w, scale, bias=None, pads=(0, 0), strid
                                                     pads[0], pads[1], strides[0], strides[1], groups, int(zpy),
                                                     L.ACT_RELU if relu else L.ACT_NONE, pk[0], pk[1],
                                                     pool_strides[0] if pool else 0, pool_strides[1] if pool else 0))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 def iconv2d_s8(x, w, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, ctx=None):
@@ -441,7 +476,7 @@ def relayout_s8(x, from_layout, to_layout, ctx=None):
     shape = (N, Cc, H, W) if to_layout == L.LAYOUT_NCHW else (N, H, W, Cc)
     y = ctx.empty(shape, torch.int8)
     ctx.check(ctx.lib.sofie_hip_relayout_s8(ctx.h, ctx.ptr(xd), ctx.ptr(y), N, Cc, H, W, from_layout, to_layout))
-    return _ret(y, x)
+    return ctx.ret(y, x)
 
 
 # ------------------------------------------------------------------------------- fp8
@@ -450,7 +485,7 @@ def quantize_f32_e4m3(x, inv_scale, ctx=None):
     xd = ctx.dev(x, torch.float32)
     q = ctx.empty(xd.shape, torch.uint8)
     ctx.check(ctx.lib.sofie_hip_quantize_f32_e4m3(ctx.h, ctx.ptr(xd), ctx.ptr(q), xd.numel(), float(inv_scale)))
-    return _ret(q, x)
+    return ctx.ret(q, x)
 
 
 def gemm_fp8(A, B, sa, sb, bias=None, transB=False, out=L.OUT_BF16, ctx=None):
@@ -463,6 +498,7 @@ def gemm_fp8(A, B, sa, sb, bias=None, transB=False, out=L.OUT_BF16, ctx=None):
     y = ctx.empty((M, N), _OUT_DTYPE[out])
     ctx.check(ctx.lib.sofie_hip_gemm_fp8(ctx.h, int(transB), M, N, K, ctx.ptr(a), a.shape[1], ctx.ptr(b),
                                          b.shape[1], float(sa), float(sb), ctx.ptr(bd), ctx.ptr(y), N, out))
+    ctx.verify_guards()
     if isinstance(A, np.ndarray):
         if out == L.OUT_BF16:
             return y.view(torch.int16).cpu().numpy().view(np.uint16)

@@ -867,3 +867,72 @@ def test_gemm_fp8_full_size(ops):
     import torch
     assert np.array_equal(yb, torch.from_numpy(yf).bfloat16().view(torch.int16).numpy().view(np.uint16))   # torch rounds RNE
     assert np.array_equal(yb[rows[0]], oracle.bf16_encode(yf[rows[0]]))
+
+
+# --------------------------------------------------------------------------- graph recording rules
+def test_capture_rules_are_enforced():
+    """Between capture_begin and capture_end the calls that would wait on, or record a memset node into, the
+    capturing stream return EINVAL and leave the recording intact; a recorded graph pins the context's scratch
+    buffer: a later call that would have to grow (free) it is refused until the graph is destroyed. Every kernel
+    that runs here exits normally; the refused calls never reach the device."""
+    import ctypes as C
+    from sofie_amd import lib as L
+    from sofie_amd import ops as o
+    ctx = o.Context(0, guard=False)          # a context of its own: the recorded graph pins its scratch buffer
+    lib, h, p = ctx.lib, ctx.h, ctx.ptr
+    r = rng(7)
+    M, N, K = 256, 256, 8192                 # long K, few tiles: the split-K path, partial sums in the scratch buffer
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    B = r.integers(-127, 128, (N, K)).astype(np.int8)
+    scale = (r.uniform(20, 60, N) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    dA, dB, dS = ctx.dev(A), ctx.dev(B), ctx.dev(scale)
+    y = ctx.empty((M, N), torch.int8)
+    host = np.zeros(16, np.uint8)
+
+    def call(m=M):
+        return lib.sofie_hip_qgemm_s8(h, 1, m, N, K, p(dA), K, p(dB), K, p(dS), None, 0, 0, p(y), N, L.OUT_S8)
+
+    assert call() == 0                        # eager once: the scratch buffer gets its size
+    ctx.sync()
+    want = y.cpu().numpy().copy()
+    assert np.array_equal(want, oracle.qgemm_s8(A, B, scale, transB=True))
+    assert lib.sofie_hip_capture_begin(h) == 0
+    try:
+        ms = C.c_float()
+        dp = C.c_void_p()
+        assert lib.sofie_hip_memset(h, p(y), 0, 16) == L.EINVAL
+        assert lib.sofie_hip_upload(h, p(y), host.ctypes.data_as(C.c_void_p), 16) == L.EINVAL
+        assert lib.sofie_hip_download(h, host.ctypes.data_as(C.c_void_p), p(y), 16) == L.EINVAL
+        assert lib.sofie_hip_sync(h) == L.EINVAL
+        assert lib.sofie_hip_malloc(h, C.byref(dp), 1024) == L.EINVAL and not dp.value
+        assert lib.sofie_hip_free(h, p(y)) == L.EINVAL
+        assert lib.sofie_hip_timer_start(h) == L.EINVAL
+        assert lib.sofie_hip_timer_stop(h, C.byref(ms)) == L.EINVAL
+        assert b"capture" in lib.sofie_hip_last_error(h)
+        assert call() == 0                    # recorded, not run
+    except BaseException:
+        lib.sofie_hip_capture_end(h, None)
+        raise
+    g = C.c_void_p()
+    assert lib.sofie_hip_capture_end(h, C.byref(g)) == 0 and g.value
+    for _ in range(3):                        # replays with eager work and waits in between
+        y.zero_()
+        torch.cuda.synchronize()
+        assert lib.sofie_hip_graph_launch(h, g) == 0
+        ctx.sync()
+        assert np.array_equal(y.cpu().numpy(), want)
+    # a call that needs a larger scratch buffer is refused while the graph lives ...
+    A2 = ctx.dev(np.zeros((4 * M, K), np.int8))
+    y2 = ctx.empty((4 * M, N), torch.int8)
+    big = lambda: lib.sofie_hip_qgemm_s8(h, 1, 4 * M, N, K, p(A2), K, p(dB), K, p(dS), None, 0, 0, p(y2), N, L.OUT_S8)
+    assert big() == L.EINVAL
+    assert b"graph" in lib.sofie_hip_last_error(h)
+    assert lib.sofie_hip_graph_launch(h, g) == 0          # ... and the graph still replays on the buffer it recorded
+    ctx.sync()
+    assert np.array_equal(y.cpu().numpy(), want)
+    # ... and goes through once it is destroyed
+    assert lib.sofie_hip_graph_destroy(h, g) == 0
+    assert big() == 0
+    ctx.sync()
+    assert not y2.cpu().numpy().any()
+    ctx.close()
