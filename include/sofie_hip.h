@@ -17,8 +17,9 @@
  *    sofie_hip_last_error() gives the message. Generated code turns a non-zero
  *    status into std::runtime_error, the reference's error convention
  *    (ROperator_Gemm.hxx:76,143,295,347).
- *  - The library keeps no global mutable state; one context per Session, one Session
- *    per thread slot (the reference's threading contract, SOFIEHelpers.hxx:27-48).
+ *  - The library keeps no global mutable state apart from the per-GPU scratch array of
+ *    sofie_hip_qgemm_s8_noalloc; one context per Session, one Session per thread slot
+ *    (the reference's threading contract, SOFIEHelpers.hxx:27-48).
  */
 #ifndef SOFIE_HIP_H
 #define SOFIE_HIP_H
@@ -219,6 +220,21 @@ int sofie_hip_dequantize_s8_f32(sofie_hip_ctx *ctx, const int8_t *q, float *x, s
 int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const int8_t *A,
                        int lda, const int8_t *B, int ldb, const float *scale,
                        const int32_t *bias, int zp_y, int act, void *Y, int ldy, int out_kind);
+
+/* sofie_hip_qgemm_s8 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same results bit for bit, but the call
+ * never allocates or frees. It has no counterpart in the reference. The two paths of sofie_hip_qgemm_s8 that use
+ * memory beyond the operands (the int32 partial sums of a long K cut into slices; the transposed copy of a
+ * B [K,N] whose leading dimension is not a multiple of 16) take it from a fixed array of
+ * SOFIE_HIP_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process ends; a shape
+ * that needs more returns SOFIE_HIP_EINVAL with a message and launches nothing (splits * M * round_up(N, 4) * 4
+ * bytes for the K slices, at most 16 slices; N * K bytes for the copy). All calls on one GPU share that array:
+ * two such calls that overlap in time on one GPU (two contexts, two threads) race; calls on one context's stream
+ * are ordered. Nothing in the array has to start at zero: every word whose value is used has been written by the same call. */
+#define SOFIE_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
+int sofie_hip_qgemm_s8_noalloc(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const int8_t *A,
+                               int lda, const int8_t *B, int ldb, const float *scale,
+                               const int32_t *bias, int zp_y, int act, void *Y, int ldy, int out_kind);
 
 /* int8 2-D convolution with int32 accumulation and fused requantisation.
  * x, y: int8 activations in x_layout / y_layout. w int8 (symmetric, zero-point 0):

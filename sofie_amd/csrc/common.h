@@ -16,6 +16,8 @@ struct sofie_hip_ctx {
    void *workspace = nullptr;   // scratch owned by the context (layout changes, B transposes)
    size_t workspace_bytes = 0;
    bool capturing = false;      // between sofie_hip_capture_begin and _end: nothing may allocate or synchronise
+   bool no_alloc = false;       // inside sofie_hip_qgemm_s8_noalloc: workspace() hands out the fixed array, never allocates
+   void *static_scratch = nullptr;   // this device's address of the fixed scratch array (looked up in sofie_hip_create)
    int live_graphs = 0;         // recorded graphs not yet destroyed: they hold the scratch buffer's address
    char err[512] = {0};
 };

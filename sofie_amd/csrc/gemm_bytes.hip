@@ -852,6 +852,20 @@ int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, cons
    }
 }
 
+int sofie_hip_qgemm_s8_noalloc(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const int8_t *A, int lda,
+                               const int8_t *B, int ldb, const float *scale, const int32_t *bias, int zp_y,
+                               int act, void *Y, int ldy, int out_kind)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   // Same kernels and the same choice among them as sofie_hip_qgemm_s8; the two paths that need memory beyond the
+   // operands (partial sums of a K cut into slices, the transposed copy of a B [K,N] whose rows are not 16-byte
+   // aligned) take it from the fixed array instead of the context's growable buffer.
+   ctx->no_alloc = true;
+   const int rc = sofie_hip_qgemm_s8(ctx, transB, M, N, K, A, lda, B, ldb, scale, bias, zp_y, act, Y, ldy, out_kind);
+   ctx->no_alloc = false;
+   return rc;
+}
+
 int sofie_hip_transpose_bytes(sofie_hip_ctx *ctx, const void *src, void *dst, int rows, int cols, int ld_src,
                                int ld_dst)
 {

@@ -1,7 +1,37 @@
 // Context, memory and timing entry points of libsofie_hip.so.
 #include <stdarg.h>
 
+#include <mutex>
+
 #include "common.h"
+
+// Scratch memory of the no-allocation entry point (sofie_hip_qgemm_s8_noalloc): a fixed array in the code object,
+// one copy per GPU the library is loaded on, held until the process ends. In host code the array's name is only
+// a handle for hipGetSymbolAddress: the device address is looked up once per device in sofie_hip_create and kept
+// in g_scratch_addr; kernels get that address as an ordinary argument.
+static __device__ __align__(256) unsigned char scratch[SOFIE_HIP_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_addr[kMaxDevices] = {};
+
+// With `device` current: the address of this device's copy of `scratch` (looked up at the first call).
+hipError_t scratch_address(int device, void **addr)
+{
+   *addr = nullptr;
+   if (device < 0 || device >= kMaxDevices) return hipErrorInvalidDevice;
+   std::lock_guard<std::mutex> lock(g_scratch_mutex);
+   if (!g_scratch_addr[device]) {
+      void *p = nullptr;
+      hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess) return e;
+      g_scratch_addr[device] = p;
+   }
+   *addr = g_scratch_addr[device];
+   return hipSuccess;
+}
+}  // namespace
 
 namespace sofie {
 
@@ -18,6 +48,15 @@ int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...)
 
 int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr)
 {
+   if (ctx->no_alloc) {   // inside the no-allocation entry point: the fixed array or nothing
+      if (!ctx->static_scratch)
+         return set_error(ctx, SOFIE_HIP_EHIP, "the fixed scratch array of this device could not be located when the context was created");
+      if (bytes > (size_t)SOFIE_HIP_NOALLOC_SCRATCH_BYTES)
+         return set_error(ctx, SOFIE_HIP_EINVAL, "this shape needs %zu bytes of scratch memory; the no-allocation entry "
+                          "point holds %zu: use sofie_hip_qgemm_s8", bytes, (size_t)SOFIE_HIP_NOALLOC_SCRATCH_BYTES);
+      *ptr = ctx->static_scratch;
+      return SOFIE_HIP_OK;
+   }
    if (bytes > ctx->workspace_bytes) {
       if (ctx->capturing)
          return set_error(ctx, SOFIE_HIP_EINVAL, "the scratch buffer would grow to %zu bytes while a graph is captured: "
@@ -72,6 +111,11 @@ int sofie_hip_create(sofie_hip_ctx **out, int device, void *stream)
       int cus = 0;
       if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus > 0)
          ctx->num_cus = cus;
+   }
+   if (hipError_t e = scratch_address(device, &ctx->static_scratch); e != hipSuccess) {
+      // only the no-allocation entry point needs it: that call then fails with this message
+      (void)hipGetLastError();
+      ctx->static_scratch = nullptr;
    }
    if (stream) {
       ctx->stream = static_cast<hipStream_t>(stream);
