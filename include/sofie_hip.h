@@ -125,15 +125,16 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, int M, int N,
 
 /* NCHW 2-D convolution y = conv(x, w) + bias[oc], optional ReLU.
  * x [N,C,H,W], w [OC, C/groups, KH, KW] (the ONNX layout, unpacked), bias [OC] or NULL,
- * y [N,OC,OH,OW] with OH = (H + 2*pad_h - (dil_h*(KH-1)+1)) / stride_h + 1.
+ * y [N,OC,OH,OW] with OH = (H + pad_top + pad_bottom - (dil_h*(KH-1)+1)) / stride_h + 1 (pads in ONNX order:
+ * top, left, bottom, right; begin and end pads may differ, as auto_pad SAME_UPPER / SAME_LOWER make them).
  * Replaces, per image, the emitted weight re-layout loop, UTILITY::Im2col, BLAS::sgemm_
  * and BLAS::saxpy_ of ROperator_Conv<float>::Generate (ROperator_Conv.hxx:342-518) and
  * the following ROperator_Relu loop (ROperator_Relu.hxx:54-66) with one implicit-GEMM
  * kernel over the whole batch; no im2col matrix is materialised. */
 int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w,
                          const float *bias, float *y, int N, int C, int H, int W, int OC,
-                         int KH, int KW, int pad_h, int pad_w, int stride_h, int stride_w,
-                         int dil_h, int dil_w, int groups, int act);
+                         int KH, int KW, int pad_top, int pad_left, int pad_bottom, int pad_right,
+                         int stride_h, int stride_w, int dil_h, int dil_w, int groups, int act);
 
 /* NCDHW 3-D convolution y = conv(x, w) + bias[oc], optional ReLU.
  * x [N,C,D,H,W], w [OC, C/groups, KD, KH, KW], bias [OC] or NULL, y [N,OC,OD,OH,OW] with
@@ -241,16 +242,16 @@ int sofie_hip_qgemm_s8_noalloc(sofie_hip_ctx *ctx, int transB, int M, int N, int
  * w_layout SOFIE_LAYOUT_NCHW = ONNX [OC, C/groups, KH, KW], SOFIE_LAYOUT_NHWC =
  * [OC, KH, KW, C/groups] (channels innermost, the order the matrix-core kernel reads).
  * bias [OC] int32 or NULL; scale [OC] fp32.
- * Padding cells hold zp_x (so that they contribute zero once the caller has folded
- * bias[oc] -= zp_x * sum(w[oc])). out_kind SOFIE_OUT_S8 or SOFIE_OUT_S32.
+ * Pads in ONNX order (top, left, bottom, right; begin and end pads may differ). Padding cells hold zp_x (so
+ * that they contribute zero once the caller has folded bias[oc] -= zp_x * sum(w[oc])). out_kind SOFIE_OUT_S8 or SOFIE_OUT_S32.
  * The matrix-core kernel takes groups = 1, C % 32 == 0, OC % 64 == 0 with every layout NHWC;
  * NCHW operands of such a shape are converted through the context's scratch buffer on each
  * call, every other shape runs a plain one-thread-per-output kernel. */
 int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
                          int w_layout, const int32_t *bias, const float *scale, void *y,
                          int y_layout, int N, int C, int H, int W, int OC, int KH, int KW,
-                         int pad_h, int pad_w, int stride_h, int stride_w, int groups,
-                         int zp_x, int zp_y, int act, int out_kind);
+                         int pad_top, int pad_left, int pad_bottom, int pad_right, int stride_h,
+                         int stride_w, int groups, int zp_x, int zp_y, int act, int out_kind);
 
 /* QLinearConv -> (ReLU) -> MaxPool in one call: y is the pooled int8 tensor
  * [N, OC, PH, PW] (y_layout), PH = (OH - pool_kh) / pool_stride_h + 1, no pooling pads.
@@ -263,9 +264,9 @@ int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, cons
 int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
                               int w_layout, const int32_t *bias, const float *scale, int8_t *y,
                               int y_layout, int N, int C, int H, int W, int OC, int KH, int KW,
-                              int pad_h, int pad_w, int stride_h, int stride_w, int groups,
-                              int zp_x, int zp_y, int act, int pool_kh, int pool_kw,
-                              int pool_stride_h, int pool_stride_w);
+                              int pad_top, int pad_left, int pad_bottom, int pad_right, int stride_h,
+                              int stride_w, int groups, int zp_x, int zp_y, int act, int pool_kh,
+                              int pool_kw, int pool_stride_h, int pool_stride_w);
 
 /* QuantizeLinear -> QLinearConv -> (ReLU) -> (MaxPool) in one call, for the first layer of a
  * quantized network: x is the float tensor [N, C, H, W], quantized as in
@@ -277,9 +278,9 @@ int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout,
 int sofie_hip_quantize_qconv2d_s8(sofie_hip_ctx *ctx, const float *x, float x_scale, int zp_x,
                                   const int8_t *w, int w_layout, const int32_t *bias,
                                   const float *scale, int8_t *y, int y_layout, int N, int C, int H,
-                                  int W, int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,
-                                  int stride_w, int groups, int zp_y, int act, int pool_kh,
-                                  int pool_kw, int pool_stride_h, int pool_stride_w);
+                                  int W, int OC, int KH, int KW, int pad_top, int pad_left, int pad_bottom,
+                                  int pad_right, int stride_h, int stride_w, int groups, int zp_y, int act,
+                                  int pool_kh, int pool_kw, int pool_stride_h, int pool_stride_w);
 
 /* int8 max pooling, NCHW or NHWC. */
 int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N,

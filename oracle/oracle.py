@@ -119,6 +119,20 @@ def relu_f32(x):
     return y
 
 
+def _pads_hw(x, pads, fill=0):
+    """The C restatement follows the reference's Im2col, which knows one pad per axis (SOFIE_common.hxx:485-518).
+    pads = (h, w) is handed over as it is; pads = (top, left, bottom, right) with begin != end pads, which the
+    reference cannot express (it averages them, ROperator_Conv.hxx:387-401), is ONNX's definition taken literally:
+    the padded tensor is written out (cells hold `fill`) and convolved without pads."""
+    pads = tuple(int(p) for p in pads)
+    if len(pads) == 2:
+        return x, pads
+    pt, pl, pb, pr = pads
+    if pt == pb and pl == pr:
+        return x, (pt, pl)
+    return np.pad(x, ((0, 0), (0, 0), (pt, pb), (pl, pr)), constant_values=fill), (0, 0)
+
+
 def conv_out_hw(H, W, kh, kw, ph, pw, sh, sw, dh=1, dw=1):
     return ((H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1,
             (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1)
@@ -135,6 +149,7 @@ def im2col(im, kh, kw, ph, pw, sh, sw, dh=1, dw=1):
 
 def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), groups=1,
                relu=False):
+    x, pads = _pads_hw(np.asarray(x, np.float32), pads)
     x = np.ascontiguousarray(x, np.float32)
     w = np.ascontiguousarray(w, np.float32)
     N, Cc, H, W = x.shape
@@ -300,6 +315,7 @@ def qgemm_s8_f32out(A, B, scale, bias=None, transB=False, zpa=0, relu=False):
 
 
 def iconv2d_s8(x, w, pads=(0, 0), strides=(1, 1), groups=1, zpx=0):
+    x, pads = _pads_hw(np.asarray(x, np.int8), pads, zpx)
     x = np.ascontiguousarray(x, np.int8)
     w = np.ascontiguousarray(w, np.int8)
     N, Cc, H, W = x.shape
@@ -315,6 +331,7 @@ def iconv2d_s8(x, w, pads=(0, 0), strides=(1, 1), groups=1, zpx=0):
 
 def qconv2d_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, zpy=0,
                relu=False):
+    x, pads = _pads_hw(np.asarray(x, np.int8), pads, zpx)
     x = np.ascontiguousarray(x, np.int8)
     w = np.ascontiguousarray(w, np.int8)
     N, Cc, H, W = x.shape

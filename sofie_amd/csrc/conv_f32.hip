@@ -683,25 +683,27 @@ extern "C" int sofie_hip_conv3d_f32(sofie_hip_ctx *ctx, const float *x, const fl
 }
 
 extern "C" int sofie_hip_conv2d_f32(sofie_hip_ctx *ctx, const float *x, const float *w, const float *bias, float *y,
-                                    int N, int C, int H, int W, int OC, int KH, int KW, int pad_h, int pad_w,
-                                    int stride_h, int stride_w, int dil_h, int dil_w, int groups, int act)
+                                    int N, int C, int H, int W, int OC, int KH, int KW, int pad_top, int pad_left,
+                                    int pad_bottom, int pad_right, int stride_h, int stride_w, int dil_h, int dil_w,
+                                    int groups, int act)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
    SOFIE_REQUIRE(ctx, N >= 0 && C > 0 && H > 0 && W > 0 && OC > 0 && KH > 0 && KW > 0, "non-positive dimension");
-   SOFIE_REQUIRE(ctx, pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0 && dil_h > 0 && dil_w > 0,
-                 "bad pads/strides/dilations");
+   SOFIE_REQUIRE(ctx, pad_top >= 0 && pad_left >= 0 && pad_bottom >= 0 && pad_right >= 0 && stride_h > 0 && stride_w > 0 &&
+                         dil_h > 0 && dil_w > 0, "bad pads/strides/dilations");
    SOFIE_REQUIRE(ctx, groups > 0 && C % groups == 0 && OC % groups == 0, "channels not divisible by groups");
    SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
    const int eh = dil_h * (KH - 1) + 1, ew = dil_w * (KW - 1) + 1;
-   SOFIE_REQUIRE(ctx, H + 2 * pad_h >= eh && W + 2 * pad_w >= ew, "kernel larger than padded input");
+   SOFIE_REQUIRE(ctx, H + pad_top + pad_bottom >= eh && W + pad_left + pad_right >= ew, "kernel larger than padded input");
    if (N == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, x && w && y, "null operand");
    ConvArgs g{};
    g.x = x; g.w = w; g.bias = bias; g.y = y;
    g.N = N; g.C = C; g.H = H; g.W = W; g.OC = OC; g.KH = KH; g.KW = KW;
-   g.ph = pad_h; g.pw = pad_w; g.sh = stride_h; g.sw = stride_w; g.dh = dil_h; g.dw = dil_w; g.groups = groups;
-   g.OH = (H + 2 * pad_h - eh) / stride_h + 1;
-   g.OW = (W + 2 * pad_w - ew) / stride_w + 1;
+   // the kernels place the windows by the begin pads; the end pads only decide how many windows there are
+   g.ph = pad_top; g.pw = pad_left; g.sh = stride_h; g.sw = stride_w; g.dh = dil_h; g.dw = dil_w; g.groups = groups;
+   g.OH = (H + pad_top + pad_bottom - eh) / stride_h + 1;
+   g.OW = (W + pad_left + pad_right - ew) / stride_w + 1;
    g.icg = C / groups;
    g.ocg = OC / groups;
    g.relu = act == SOFIE_ACT_RELU;

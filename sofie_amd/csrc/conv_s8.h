@@ -11,7 +11,8 @@ struct QConvArgs {
    const int32_t *bias;
    const float *scale;
    void *y;
-   int N, C, H, W, OC, KH, KW, ph, pw, sh, sw, groups;
+   int N, C, H, W, OC, KH, KW, ph, pw, sh, sw, groups;   // ph, pw: begin pads (top, left)
+   int pbh, pbw;                                         // end pads (bottom, right)
    int OH, OW, icg, ocg;
    int zpx, zpy, lo, relu;
    int x_nhwc, y_nhwc, w_ohwi;

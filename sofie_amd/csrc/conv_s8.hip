@@ -495,7 +495,7 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const int TH = pool ? g.PH : g.OH, TW = pool ? g.PW : g.OW;
    const int rpp = pool ? 2 : 1;                      // convolution rows per tile row
    const long long mtot = (long long)g.N * TH * TW;
-   const int HP = g.H + 2 * g.ph, WP = g.W + 2 * g.pw;
+   const int HP = g.H + g.ph + g.pbh, WP = g.W + g.pw + g.pbw;
    if (mtot <= 0) return SOFIE_HIP_OK;
    if (mtot >= (1ll << 31) - 1024 || (long long)g.N * HP >= (1ll << 31) - 4096) return SOFIE_HIP_OK;
    if ((size_t)g.N * g.H * g.W * g.C >= ((size_t)1 << 40)) return SOFIE_HIP_OK;
@@ -687,11 +687,12 @@ int run(sofie_hip_ctx *ctx, const QConvArgs &g)
 
 int fill_args(sofie_hip_ctx *ctx, QConvArgs &g, const int8_t *x, int x_layout, const int8_t *w, int w_layout,
               const int32_t *bias, const float *scale, void *y, int y_layout, int N, int C, int H, int W, int OC, int KH,
-              int KW, int pad_h, int pad_w, int stride_h, int stride_w, int groups, int zp_x, int zp_y, int act,
-              int out_kind)
+              int KW, int pad_top, int pad_left, int pad_bottom, int pad_right, int stride_h, int stride_w, int groups,
+              int zp_x, int zp_y, int act, int out_kind)
 {
    SOFIE_REQUIRE(ctx, N >= 0 && C > 0 && H > 0 && W > 0 && OC > 0 && KH > 0 && KW > 0, "non-positive dimension");
-   SOFIE_REQUIRE(ctx, pad_h >= 0 && pad_w >= 0 && stride_h > 0 && stride_w > 0, "bad pads/strides");
+   SOFIE_REQUIRE(ctx, pad_top >= 0 && pad_left >= 0 && pad_bottom >= 0 && pad_right >= 0 && stride_h > 0 && stride_w > 0,
+                 "bad pads/strides");
    SOFIE_REQUIRE(ctx, groups > 0 && C % groups == 0 && OC % groups == 0, "channels not divisible by groups");
    SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
    SOFIE_REQUIRE(ctx, (x_layout == SOFIE_LAYOUT_NCHW || x_layout == SOFIE_LAYOUT_NHWC) &&
@@ -699,15 +700,16 @@ int fill_args(sofie_hip_ctx *ctx, QConvArgs &g, const int8_t *x, int x_layout, c
                          (w_layout == SOFIE_LAYOUT_NCHW || w_layout == SOFIE_LAYOUT_NHWC), "unknown layout");
    SOFIE_REQUIRE(ctx, out_kind == SOFIE_OUT_S8 || out_kind == SOFIE_OUT_S32, "output kind must be S8 or S32");
    SOFIE_REQUIRE(ctx, zp_x >= -128 && zp_x <= 127 && zp_y >= -128 && zp_y <= 127, "zero-point out of int8 range");
-   SOFIE_REQUIRE(ctx, H + 2 * pad_h >= KH && W + 2 * pad_w >= KW, "kernel larger than padded input");
+   SOFIE_REQUIRE(ctx, H + pad_top + pad_bottom >= KH && W + pad_left + pad_right >= KW, "kernel larger than padded input");
    if (N == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, w && y, "null operand");
    SOFIE_REQUIRE(ctx, scale || out_kind == SOFIE_OUT_S32, "scale is required for S8 output");
    g.x = x; g.w = w; g.bias = bias; g.scale = scale; g.y = y;
    g.N = N; g.C = C; g.H = H; g.W = W; g.OC = OC; g.KH = KH; g.KW = KW;
-   g.ph = pad_h; g.pw = pad_w; g.sh = stride_h; g.sw = stride_w; g.groups = groups;
-   g.OH = (H + 2 * pad_h - KH) / stride_h + 1;
-   g.OW = (W + 2 * pad_w - KW) / stride_w + 1;
+   g.ph = pad_top; g.pw = pad_left; g.pbh = pad_bottom; g.pbw = pad_right;
+   g.sh = stride_h; g.sw = stride_w; g.groups = groups;
+   g.OH = (H + pad_top + pad_bottom - KH) / stride_h + 1;
+   g.OW = (W + pad_left + pad_right - KW) / stride_w + 1;
    g.PH = g.OH; g.PW = g.OW;
    g.icg = C / groups;
    g.ocg = OC / groups;
@@ -725,13 +727,14 @@ int fill_args(sofie_hip_ctx *ctx, QConvArgs &g, const int8_t *x, int x_layout, c
 
 extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w, int w_layout,
                                     const int32_t *bias, const float *scale, void *y, int y_layout, int N, int C,
-                                    int H, int W, int OC, int KH, int KW, int pad_h, int pad_w, int stride_h,
-                                    int stride_w, int groups, int zp_x, int zp_y, int act, int out_kind)
+                                    int H, int W, int OC, int KH, int KW, int pad_top, int pad_left, int pad_bottom,
+                                    int pad_right, int stride_h, int stride_w, int groups, int zp_x, int zp_y, int act,
+                                    int out_kind)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
    QConvArgs g{};
-   if (int rc = fill_args(ctx, g, x, x_layout, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW, pad_h, pad_w,
-                          stride_h, stride_w, groups, zp_x, zp_y, act, out_kind))
+   if (int rc = fill_args(ctx, g, x, x_layout, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW, pad_top, pad_left,
+                          pad_bottom, pad_right, stride_h, stride_w, groups, zp_x, zp_y, act, out_kind))
       return rc;
    if (N == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, x, "null operand");
@@ -741,14 +744,15 @@ extern "C" int sofie_hip_qconv2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_l
 
 extern "C" int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, const int8_t *w,
                                          int w_layout, const int32_t *bias, const float *scale, int8_t *y, int y_layout,
-                                         int N, int C, int H, int W, int OC, int KH, int KW, int pad_h, int pad_w,
-                                         int stride_h, int stride_w, int groups, int zp_x, int zp_y, int act,
+                                         int N, int C, int H, int W, int OC, int KH, int KW, int pad_top, int pad_left,
+                                         int pad_bottom, int pad_right, int stride_h, int stride_w, int groups, int zp_x,
+                                         int zp_y, int act,
                                          int pool_kh, int pool_kw, int pool_stride_h, int pool_stride_w)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
    QConvArgs g{};
-   if (int rc = fill_args(ctx, g, x, x_layout, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW, pad_h, pad_w,
-                          stride_h, stride_w, groups, zp_x, zp_y, act, SOFIE_OUT_S8))
+   if (int rc = fill_args(ctx, g, x, x_layout, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW, pad_top, pad_left,
+                          pad_bottom, pad_right, stride_h, stride_w, groups, zp_x, zp_y, act, SOFIE_OUT_S8))
       return rc;
    SOFIE_REQUIRE(ctx, pool_kh > 0 && pool_kw > 0 && pool_stride_h > 0 && pool_stride_w > 0, "bad pooling window");
    SOFIE_REQUIRE(ctx, pool_kh <= g.OH && pool_kw <= g.OW, "pooling window larger than the convolution output");
@@ -762,15 +766,16 @@ extern "C" int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, in
 
 extern "C" int sofie_hip_quantize_qconv2d_s8(sofie_hip_ctx *ctx, const float *x, float x_scale, int zp_x, const int8_t *w,
                                              int w_layout, const int32_t *bias, const float *scale, int8_t *y,
-                                             int y_layout, int N, int C, int H, int W, int OC, int KH, int KW, int pad_h,
-                                             int pad_w, int stride_h, int stride_w, int groups, int zp_y, int act,
+                                             int y_layout, int N, int C, int H, int W, int OC, int KH, int KW, int pad_top,
+                                             int pad_left, int pad_bottom, int pad_right, int stride_h, int stride_w,
+                                             int groups, int zp_y, int act,
                                              int pool_kh, int pool_kw, int pool_stride_h, int pool_stride_w)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
    SOFIE_REQUIRE(ctx, x_scale > 0.0f, "the input scale must be positive");
    QConvArgs g{};
    if (int rc = fill_args(ctx, g, nullptr, SOFIE_LAYOUT_NCHW, w, w_layout, bias, scale, y, y_layout, N, C, H, W, OC, KH, KW,
-                          pad_h, pad_w, stride_h, stride_w, groups, zp_x, zp_y, act, SOFIE_OUT_S8))
+                          pad_top, pad_left, pad_bottom, pad_right, stride_h, stride_w, groups, zp_x, zp_y, act, SOFIE_OUT_S8))
       return rc;
    if (N == 0) return SOFIE_HIP_OK;
    SOFIE_REQUIRE(ctx, x, "null operand");

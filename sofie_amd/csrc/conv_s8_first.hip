@@ -301,7 +301,8 @@ int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
 {
    *done = false;
    const bool pool = g.pool_kh != 0;
-   if (g.C != 1 || g.groups != 1 || g.KH != 3 || g.KW != 3 || g.sh != 1 || g.sw != 1 || g.ph != 1 || g.pw != 1) return SOFIE_HIP_OK;
+   if (g.C != 1 || g.groups != 1 || g.KH != 3 || g.KW != 3 || g.sh != 1 || g.sw != 1 || g.ph != 1 || g.pw != 1 ||
+       g.pbh != 1 || g.pbw != 1) return SOFIE_HIP_OK;
    if (g.OC % 16 != 0 || !g.y_nhwc || !aligned16(g.y)) return SOFIE_HIP_OK;
    if (pool && !(g.pool_kh == 2 && g.pool_kw == 2 && g.pool_sh == 2 && g.pool_sw == 2)) return SOFIE_HIP_OK;
    if (g.PH <= 0 || g.PW <= 0) return SOFIE_HIP_OK;

@@ -1,9 +1,14 @@
 // Conv emitter (1-D, 2-D and 3-D). Constructor, attribute defaults, output-shape rule and error messages follow the
 // reference's ROperator_Conv<T> (src/SOFIE_core/inc/SOFIE/ROperator_Conv.hxx:52-87,95-201,203-282):
 //   - auto_pad NOTSET with no pads attribute means 1 on every side (:136-139, not ONNX's 0);
-//   - SAME_UPPER / SAME_LOWER start from k/2 and add one at the begin / end for odd kernels (:140-158);
-//   - begin/end pads that differ are averaged with a warning (:387-401);
 //   - group == 0 means C / C_w (:110-112).
+// Two rules of the reference are NOT followed, because they make its own generated code inconsistent:
+//   - SAME_UPPER / SAME_LOWER: the reference starts from k/2 on both sides and adds one at the begin / end for odd
+//     kernels (:140-158), i.e. a total of k for a 3x3 kernel; the output shape it declares then has one row and column
+//     more than the averaged pad of its Im2col call writes. Here the pads are ONNX's: the total that makes the output
+//     ceil(in / stride), the odd unit at the end (SAME_UPPER) or at the begin (SAME_LOWER);
+//   - begin/end pads that differ: the reference averages them with a warning (:387-401) while the declared output
+//     shape uses their sum. Here the kernel library takes all four pads and the result is ONNX's.
 // Emitted code: one sofie_hip_conv2d_f32 call over the whole batch (implicit GEMM, bias and
 // optional ReLU fused) instead of the per-image weight re-layout + Im2col + sgemm_ + saxpy_. A 1-D operator
 // [N,C,W] runs as the 2-D one on [N,C,1,W] (the reference does the same inside Im2col, :424-427); a 3-D one is
@@ -49,10 +54,16 @@ struct ConvGeometry {
       if (autopad == "NOTSET" || autopad == "") {
          if (pads.empty()) pads.assign(2 * dim, 1);
       } else if (autopad == "SAME_UPPER" || autopad == "SAME_LOWER") {
+         if (strides.empty()) strides.assign(dim, 1);
+         strides.resize(dim, 1);
          pads.assign(2 * dim, 0);
          for (size_t i = 0; i < dim; ++i) {
-            pads[i] = pads[dim + i] = extent[i] / 2;
-            if (extent[i] % 2 == 1) (autopad == "SAME_UPPER") ? pads[i]++ : pads[dim + i]++;
+            const size_t in = x[i + 2], st = strides[i];
+            const size_t covered = ((in + st - 1) / st - 1) * st + extent[i];   // reach of the last of ceil(in/st) windows
+            const size_t total = covered > in ? covered - in : 0;
+            const size_t small = total / 2, large = total - small;
+            pads[i] = autopad == "SAME_UPPER" ? small : large;
+            pads[dim + i] = autopad == "SAME_UPPER" ? large : small;
          }
       } else if (autopad == "VALID") {
          pads.assign(2 * dim, 0);
@@ -66,23 +77,19 @@ struct ConvGeometry {
       for (size_t i = 0; i < dim; ++i) out.push_back((x[i + 2] + pads[i] + pads[dim + i] - extent[i]) / strides[i] + 1);
       return out;
    }
-   // begin pads handed to the kernel; begin/end pads that differ are averaged with the reference's warning (:387-411)
-   std::vector<size_t> SymmetricPads()
-   {
-      bool differ = false;
-      for (size_t i = 0; i < dim; ++i) differ = differ || pads[i] != pads[dim + i];
-      if (differ) {
-         std::cout << "TMVA SOFIE Operator Conv:  asymmetric padding not supported. Assume an average padding " << std::endl;
-         for (size_t i = 0; i < dim; ++i) pads[i] = (pads[i] + pads[dim + i]) / 2;
-      }
-      return std::vector<size_t>(pads.begin(), pads.begin() + dim);
-   }
-   void SymmetricPads(size_t &ph, size_t &pw)
+   // the four pads of a 2-D operator in ONNX order (top, left, bottom, right)
+   void Pads2D(size_t &pt, size_t &pl, size_t &pb, size_t &pr) const
    {
       if (dim != 2) throw std::runtime_error("TMVA SOFIE Conv Op: a 2-D convolution is expected here");
-      const auto p = SymmetricPads();
-      ph = p[0];
-      pw = p[1];
+      pt = pads[0]; pl = pads[1]; pb = pads[2]; pr = pads[3];
+   }
+   // 3-D operators: the kernel takes one pad per axis
+   std::vector<size_t> EqualPads() const
+   {
+      for (size_t i = 0; i < dim; ++i)
+         if (pads[i] != pads[dim + i])
+            throw std::runtime_error("TMVA SOFIE Conv Op: begin and end pads that differ are not supported for 3-D convolutions");
+      return std::vector<size_t>(pads.begin(), pads.begin() + dim);
    }
 };
 
@@ -202,7 +209,6 @@ public:
       OpName = "op_" + OpName;
       if (fShapeX.empty() || fShapeW.empty() || (fNB != "" && fShapeB.empty()) || fShapeY.empty())
          throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
-      const std::vector<size_t> p = fGeom.SymmetricPads();
       const size_t dim = fGeom.dim;
       const std::string bias = fNB.empty() ? std::string("nullptr") : "tensor_" + fNB;
       const std::string act = fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE";
@@ -214,6 +220,7 @@ public:
          for (size_t i = 1; i < 5; ++i) out << ", " << fShapeX[i];
          out << ", " << fShapeW[0];
          for (size_t i = 0; i < 3; ++i) out << ", " << fShapeW[2 + i];
+         const std::vector<size_t> p = fGeom.EqualPads();
          for (size_t i = 0; i < 3; ++i) out << ", " << p[i];
          for (size_t i = 0; i < 3; ++i) out << ", " << fGeom.strides[i];
          for (size_t i = 0; i < 3; ++i) out << ", " << fGeom.dilations[i];
@@ -224,12 +231,13 @@ public:
       const bool oneD = dim == 1;
       const size_t H = oneD ? 1 : fShapeX[2], W = fShapeX[dim + 1];
       const size_t KH = oneD ? 1 : fShapeW[2], KW = fShapeW[dim + 1];
-      const size_t ph = oneD ? 0 : p[0], pw = p[dim - 1];
+      const std::vector<size_t> &p = fGeom.pads;   // begins, then ends
+      const size_t pt = oneD ? 0 : p[0], pl = p[dim - 1], pb = oneD ? 0 : p[dim], pr = p[2 * dim - 1];
       const size_t sh = oneD ? 1 : fGeom.strides[0], sw = fGeom.strides[dim - 1];
       const size_t dh = oneD ? 1 : fGeom.dilations[0], dw = fGeom.dilations[dim - 1];
       out << SP << "Check(sofie_hip_conv2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNW << ", " << bias << ", tensor_" << fNY << ", "
-          << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << H << ", " << W << ", " << fShapeW[0] << ", " << KH << ", " << KW << ", " << ph
-          << ", " << pw << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << fGeom.group << ", " << act << "), \"Conv "
+          << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << H << ", " << W << ", " << fShapeW[0] << ", " << KH << ", " << KW << ", " << pt
+          << ", " << pl << ", " << pb << ", " << pr << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << fGeom.group << ", " << act << "), \"Conv "
           << OpName << "\");\n";
       return out.str();
    }

@@ -342,10 +342,10 @@ public:
       // the fused call exists for any shape, but only first layers (one input channel, 3x3, stride 1, pad 1,
       // OC a multiple of 16) have a kernel that never writes the int8 input: fuse only those
       if (fShapeX.empty() || !fNXFloat.empty() || fXChannelsLast) return false;
-      size_t ph, pw;
-      fGeom.SymmetricPads(ph, pw);
+      size_t pt, pl, pb, pr;
+      fGeom.Pads2D(pt, pl, pb, pr);
       if (fShapeX[1] != 1 || fGeom.group != 1 || fShapeW[2] != 3 || fShapeW[3] != 3 || fGeom.strides[0] != 1 ||
-          fGeom.strides[1] != 1 || ph != 1 || pw != 1 || fShapeW[0] % 16 != 0)
+          fGeom.strides[1] != 1 || pt != 1 || pl != 1 || pb != 1 || pr != 1 || fShapeW[0] % 16 != 0)
          return false;
       if (zeroPoint != fZpX || scale != fScaleX) return false;   // must be the quantization this operator assumes
       fNXFloat = xFloat;
@@ -444,8 +444,8 @@ public:
    std::string Generate(std::string OpName) override
    {
       if (fShapeX.empty()) throw std::runtime_error("TMVA SOFIE QLinearConv Op called to Generate without being initialized first");
-      size_t ph, pw;
-      fGeom.SymmetricPads(ph, pw);
+      size_t pt, pl, pb, pr;
+      fGeom.Pads2D(pt, pl, pb, pr);
       std::stringstream out;
       const bool pooled = !fPoolKernel.empty();
       const bool fromFloat = !fNXFloat.empty();
@@ -460,7 +460,7 @@ public:
       out << ", tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, " << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr"))
           << ", tensor_" << fNScale << ", tensor_" << (pooled ? fNYPooled : fNY) << ", SOFIE_LAYOUT_NHWC, " << BatchCount(fShapeX[0]) << ", "
           << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3] << ", " << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3]
-          << ", " << ph << ", " << pw << ", " << fGeom.strides[0] << ", " << fGeom.strides[1] << ", " << fGeom.group << ", ";
+          << ", " << pt << ", " << pl << ", " << pb << ", " << pr << ", " << fGeom.strides[0] << ", " << fGeom.strides[1] << ", " << fGeom.group << ", ";
       if (!fromFloat) out << fZpX << ", ";
       out << fZpY << ", " << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE");
       if (pooled)

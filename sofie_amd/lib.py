@@ -33,7 +33,7 @@ SIGNATURES = {
     "sofie_hip_timer_start": [_p],
     "sofie_hip_timer_stop": [_p, C.POINTER(_f)],
     "sofie_hip_gemm_f32": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i, _p, _i, _i],
-    "sofie_hip_conv2d_f32": [_p, _p, _p, _p, _p] + [_i] * 15,
+    "sofie_hip_conv2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,
     "sofie_hip_conv3d_f32": [_p, _p, _p, _p, _p] + [_i] * 20,
     "sofie_hip_conv_transpose2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,
     "sofie_hip_capture_begin": [_p],
@@ -48,9 +48,9 @@ SIGNATURES = {
     "sofie_hip_dequantize_s8_f32": [_p, _p, _p, _z, _f, _i],
     "sofie_hip_qgemm_s8": [_p, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i],
     "sofie_hip_qgemm_s8_noalloc": [_p, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i],
-    "sofie_hip_qconv2d_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 16,
-    "sofie_hip_qconv2d_pool_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 19,
-    "sofie_hip_quantize_qconv2d_s8": [_p, _p, C.c_float, _i, _p, _i, _p, _p, _p, _i] + [_i] * 18,
+    "sofie_hip_qconv2d_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 18,
+    "sofie_hip_qconv2d_pool_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 21,
+    "sofie_hip_quantize_qconv2d_s8": [_p, _p, C.c_float, _i, _p, _i, _p, _p, _p, _i] + [_i] * 20,
     "sofie_hip_maxpool2d_s8": [_p, _p, _p] + [_i] * 13,
     "sofie_hip_relayout_s8": [_p, _p, _p] + [_i] * 6,
     "sofie_hip_transpose_bytes": [_p, _p, _p, _i, _i, _i, _i],

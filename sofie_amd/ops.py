@@ -159,8 +159,15 @@ def relu_f32(x, ctx=None):
     return ctx.ret(y, x)
 
 
-def conv_out_hw(H, W, kh, kw, ph, pw, sh, sw, dh=1, dw=1):
-    return ((H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1, (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1)
+def pads4(pads):
+    """(h, w) -> (top, left, bottom, right) with equal begin and end pads; a 4-tuple is ONNX order already."""
+    pads = tuple(int(p) for p in pads)
+    return pads if len(pads) == 4 else (pads[0], pads[1], pads[0], pads[1])
+
+
+def conv_out_hw(H, W, kh, kw, pads, sh, sw, dh=1, dw=1):
+    pt, pl, pb, pr = pads4(pads)
+    return ((H + pt + pb - (dh * (kh - 1) + 1)) // sh + 1, (W + pl + pr - (dw * (kw - 1) + 1)) // sw + 1)
 
 
 def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), groups=1, relu=False, ctx=None):
@@ -168,10 +175,10 @@ def conv2d_f32(x, w, bias=None, pads=(0, 0), strides=(1, 1), dilations=(1, 1), g
     xd, wd, bd = ctx.dev(x, torch.float32), ctx.dev(w, torch.float32), ctx.dev(bias, torch.float32)
     N, Cc, H, W = xd.shape
     OC, _, kh, kw = wd.shape
-    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1], *dilations)
+    OH, OW = conv_out_hw(H, W, kh, kw, pads, strides[0], strides[1], *dilations)
     y = ctx.empty((N, OC, OH, OW), torch.float32)
     ctx.check(ctx.lib.sofie_hip_conv2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(wd), ctx.ptr(bd), ctx.ptr(y), N, Cc, H, W,
-                                           OC, kh, kw, pads[0], pads[1], strides[0], strides[1], dilations[0],
+                                           OC, kh, kw, *pads4(pads), strides[0], strides[1], dilations[0],
                                            dilations[1], groups, L.ACT_RELU if relu else L.ACT_NONE))
     return ctx.ret(y, x)
 
@@ -397,12 +404,12 @@ def qconv2d_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=1, zp
         OC, _, kh, kw = wd.shape
     else:
         OC, kh, kw, _ = wd.shape
-    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1])
+    OH, OW = conv_out_hw(H, W, kh, kw, pads, strides[0], strides[1])
     shape = (N, OC, OH, OW) if y_layout == L.LAYOUT_NCHW else (N, OH, OW, OC)
     y = ctx.empty(shape, _OUT_DTYPE[out])
     sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
     ctx.check(ctx.lib.sofie_hip_qconv2d_s8(ctx.h, ctx.ptr(xd), x_layout, ctx.ptr(wd), w_layout, ctx.ptr(bd), ctx.ptr(sd),
-                                           ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, pads[0], pads[1],
+                                           ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, *pads4(pads),
                                            strides[0], strides[1], groups, int(zpx), int(zpy),
                                            L.ACT_RELU if relu else L.ACT_NONE, out))
     return ctx.ret(y, x)
@@ -424,13 +431,13 @@ def qconv2d_pool_s8(x, w, scale, bias=None, pads=(0, 0), strides=(1, 1), groups=
         OC, _, kh, kw = wd.shape
     else:
         OC, kh, kw, _ = wd.shape
-    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1])
+    OH, OW = conv_out_hw(H, W, kh, kw, pads, strides[0], strides[1])
     PH, PW = (OH - pool[0]) // pool_strides[0] + 1, (OW - pool[1]) // pool_strides[1] + 1
     y = ctx.empty((N, OC, PH, PW) if y_layout == L.LAYOUT_NCHW else (N, PH, PW, OC), torch.int8)
     sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
     ctx.check(ctx.lib.sofie_hip_qconv2d_pool_s8(ctx.h, ctx.ptr(xd), x_layout, ctx.ptr(wd), w_layout, ctx.ptr(bd),
-                                                ctx.ptr(sd), ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, pads[0],
-                                                pads[1], strides[0], strides[1], groups, int(zpx), int(zpy),
+                                                ctx.ptr(sd), ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw, *pads4(pads),
+                                                strides[0], strides[1], groups, int(zpx), int(zpy),
                                                 L.ACT_RELU if relu else L.ACT_NONE, pool[0], pool[1], pool_strides[0],
                                                 pool_strides[1]))
     return ctx.ret(y, x)
@@ -448,7 +455,7 @@ def quantize_qconv2d_s8(x, x_scale, zpx, w, scale, bias=None, pads=(0, 0), strid
         OC, _, kh, kw = wd.shape
     else:
         OC, kh, kw, _ = wd.shape
-    OH, OW = conv_out_hw(H, W, kh, kw, pads[0], pads[1], strides[0], strides[1])
+    OH, OW = conv_out_hw(H, W, kh, kw, pads, strides[0], strides[1])
     if pool:
         OH, OW = (OH - pool[0]) // pool_strides[0] + 1, (OW - pool[1]) // pool_strides[1] + 1
     y = ctx.empty((N, OC, OH, OW) if y_layout == L.LAYOUT_NCHW else (N, OH, OW, OC), torch.int8)
@@ -456,7 +463,7 @@ def quantize_qconv2d_s8(x, x_scale, zpx, w, scale, bias=None, pads=(0, 0), strid
     pk = pool or (0, 0)
     ctx.check(ctx.lib.sofie_hip_quantize_qconv2d_s8(ctx.h, ctx.ptr(xd), float(x_scale), int(zpx), ctx.ptr(wd), w_layout,
                                                     ctx.ptr(bd), ctx.ptr(sd), ctx.ptr(y), y_layout, N, Cc, H, W, OC, kh, kw,
-                                                    pads[0], pads[1], strides[0], strides[1], groups, int(zpy),
+                                                    *pads4(pads), strides[0], strides[1], groups, int(zpy),
                                                     L.ACT_RELU if relu else L.ACT_NONE, pk[0], pk[1],
                                                     pool_strides[0] if pool else 0, pool_strides[1] if pool else 0))
     return ctx.ret(y, x)

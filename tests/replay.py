@@ -7,36 +7,32 @@ The attribute handling restates what the reference's operators do at Initialize 
 import numpy as np
 
 
-def conv_pads_like_reference(attrs, kshape):
-    """Pads (h, w) that the reference's Conv finally passes to Im2col.
+def conv_pads(attrs, kshape, in_hw, strides, dilations):
+    """Pads (top, left, bottom, right) of a Conv node as this build's emitter resolves them.
 
-    ROperator_Conv.hxx:136-158: absent pads with auto_pad NOTSET mean 1 on every side;
-    SAME_UPPER/SAME_LOWER start from k/2 and add one at the begin (UPPER) or end (LOWER)
-    for odd kernels; :387-401: asymmetric begin/end pads are averaged (integer division).
+    Absent pads with auto_pad NOTSET mean 1 on every side, the reference's rule (ROperator_Conv.hxx:136-139).
+    SAME_UPPER / SAME_LOWER are ONNX's: the total that makes the output ceil(in / stride), the odd unit at the
+    end / at the begin (the reference's own rule, :140-158, declares an output larger than its code writes).
+    Begin and end pads that differ are kept (the reference averages them, :387-401).
     """
-    kh, kw = kshape
     auto = attrs.get("auto_pad", "NOTSET")
     pads = list(attrs.get("pads", []))
     if auto == "NOTSET":
         if not pads:
             pads = [1, 1, 1, 1]
     elif auto in ("SAME_UPPER", "SAME_LOWER"):
-        pads = [kh // 2, kw // 2, kh // 2, kw // 2]
-        if kh % 2 == 1:
-            pads[0 if auto == "SAME_UPPER" else 2] += 1
-        if kw % 2 == 1:
-            pads[1 if auto == "SAME_UPPER" else 3] += 1
+        pads = [0, 0, 0, 0]
+        for i in range(2):
+            extent = dilations[i] * (kshape[i] - 1) + 1
+            covered = (-(-in_hw[i] // strides[i]) - 1) * strides[i] + extent
+            total = max(covered - in_hw[i], 0)
+            small, large = total // 2, total - total // 2
+            pads[i], pads[2 + i] = (small, large) if auto == "SAME_UPPER" else (large, small)
     elif auto == "VALID":
         pads = [0, 0, 0, 0]
     else:
         raise RuntimeError("TMVA SOFIE Conv Op invalid fAutopad")
-    out_h_pad_total = pads[0] + pads[2]
-    out_w_pad_total = pads[1] + pads[3]
-    ph, pw = pads[0], pads[1]
-    if pads[0] != pads[2] or pads[1] != pads[3]:
-        ph = (pads[0] + pads[2]) // 2
-        pw = (pads[1] + pads[3]) // 2
-    return (ph, pw), (out_h_pad_total, out_w_pad_total)
+    return tuple(pads)
 
 
 def run_graph(graph, feeds, backend):
@@ -54,10 +50,11 @@ def run_graph(graph, feeds, backend):
             y = backend.relu_f32(env[ins[0]])
         elif op == "Conv":
             w = env[ins[1]]
-            (ph, pw), _ = conv_pads_like_reference(a, w.shape[2:])
+            strides = tuple(a.get("strides", [1, 1]))
+            pads = conv_pads(a, w.shape[2:], env[ins[0]].shape[2:], strides, tuple(a.get("dilations", [1, 1])))
             bias = env[ins[2]] if len(ins) > 2 else None
-            y = backend.conv2d_f32(env[ins[0]], w, bias, pads=(ph, pw),
-                                   strides=tuple(a.get("strides", [1, 1])),
+            y = backend.conv2d_f32(env[ins[0]], w, bias, pads=pads,
+                                   strides=strides,
                                    dilations=tuple(a.get("dilations", [1, 1])),
                                    groups=a.get("group", 1))
         elif op == "ConvTranspose":

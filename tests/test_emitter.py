@@ -91,12 +91,55 @@ def test_conv_default_pads_follow_the_reference(tmp_path):
     s.conv("x", "W", None, "y", kernel=(3, 3))
     s.set_output("y")
     hxx, _, _ = gen(s, tmp_path)
-    assert re.search(r"sofie_hip_conv2d_f32\(fCtx, tensor_x, tensor_W, nullptr, tensor_y, 1, 1, 5, 5, 1, 3, 3, 1, 1, 1, 1, 1, 1, 1,", open(hxx).read())
+    assert re.search(r"sofie_hip_conv2d_f32\(fCtx, tensor_x, tensor_W, nullptr, tensor_y, 1, 1, 5, 5, 1, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1,", open(hxx).read())
     spec, _ = models.fixture_spec("ConvWithAutopadSameLower")
     hxx, _, res = gen(spec, tmp_path)
     code = open(hxx).read()
     assert "std::vector<float> ret(9);" in code
-    assert re.search(r"3, 3, 1, 1, 2, 2, 1, 1, 1, SOFIE_ACT_NONE", code)
+    assert re.search(r"3, 3, 1, 1, 1, 1, 2, 2, 1, 1, 1, SOFIE_ACT_NONE", code)
+
+
+@pytest.mark.parametrize("auto,kernel,stride,size,want_pads,want_out", [
+    ("SAME_UPPER", 3, 1, 8, (1, 1, 1, 1), 8),      # odd kernel, stride 1: one on every side, the output keeps the size
+    ("SAME_LOWER", 3, 1, 8, (1, 1, 1, 1), 8),
+    ("SAME_UPPER", 4, 1, 8, (1, 1, 2, 2), 8),      # even kernel: the odd unit at the end ...
+    ("SAME_LOWER", 4, 1, 8, (2, 2, 1, 1), 8),      # ... or at the begin
+    ("SAME_UPPER", 3, 2, 8, (0, 0, 1, 1), 4),      # stride 2 on an even size needs one cell only
+    ("SAME_LOWER", 3, 2, 8, (1, 1, 0, 0), 4),
+    ("SAME_UPPER", 5, 3, 8, (1, 1, 2, 2), 3),
+])
+def test_conv_auto_pad_same_declares_the_output_the_kernel_writes(tmp_path, auto, kernel, stride, size, want_pads, want_out):
+    """SAME_UPPER / SAME_LOWER: the declared output is ceil(in / stride) per axis and the emitted call carries the
+    four pads that produce exactly that many windows (the library derives its output size from the same four
+    numbers, so the Session's return vector and the kernel's stores agree)."""
+    s = emit.ModelSpec("same")
+    s.add_input("x", "FLOAT", (1, 1, size, size))
+    s.add_init("W", np.ones((4, 1, kernel, kernel), np.float32))
+    s.conv("x", "W", None, "y", kernel=(kernel, kernel), strides=(stride, stride), auto_pad=auto)
+    s.set_output("y")
+    hxx, _, _ = gen(s, tmp_path)
+    code = open(hxx).read()
+    assert "std::vector<float> ret(%d);" % (4 * want_out * want_out) in code
+    call = "tensor_y, 1, 1, %d, %d, 4, %d, %d, %d, %d, %d, %d, %d, %d, 1, 1, 1, SOFIE_ACT_NONE" % (
+        (size, size, kernel, kernel) + want_pads + (stride, stride))
+    assert call in code
+    pt, pl, pb, pr = want_pads
+    assert (size + pt + pb - kernel) // stride + 1 == want_out
+
+
+def test_conv_begin_and_end_pads_that_differ_are_kept(tmp_path):
+    """pads = (0, 2, 1, 0): all four reach the library (the reference averages them while declaring the output by
+    their sum); the declared output follows the sum, as the library's does."""
+    s = emit.ModelSpec("asym")
+    s.add_input("x", "FLOAT", (2, 3, 7, 6))
+    s.add_init("W", np.ones((5, 3, 3, 2), np.float32))
+    s.conv("x", "W", None, "y", kernel=(3, 2), pads=(0, 2, 1, 0))
+    s.set_output("y")
+    hxx, _, _ = gen(s, tmp_path)
+    code = open(hxx).read()
+    assert "tensor_y, 2, 3, 7, 6, 5, 3, 2, 0, 2, 1, 0, 1, 1, 1, 1, 1, SOFIE_ACT_NONE" in code
+    assert "std::vector<float> ret(%d);" % (2 * 5 * 6 * 7) in code
+    assert "average padding" not in code
 
 
 def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
@@ -114,7 +157,7 @@ def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
     # the first layer also absorbs the QuantizeLinear in front of it: it reads the float input
     assert "sofie_hip_quantize_f32_s8" not in code and "tensor_xq" not in code
     assert "sofie_hip_quantize_qconv2d_s8(fCtx, tensor_x, static_cast<float>(0.00392156886), -128, tensor_w1_ohwi" in code
-    assert "tensor_p1, SOFIE_LAYOUT_NHWC, 2, 1, 40, 40, 32, 3, 3, 1, 1, 1, 1, 1, -128, SOFIE_ACT_RELU, 2, 2, 2, 2)" in code
+    assert "tensor_p1, SOFIE_LAYOUT_NHWC, 2, 1, 40, 40, 32, 3, 3, 1, 1, 1, 1, 1, 1, 1, -128, SOFIE_ACT_RELU, 2, 2, 2, 2)" in code
     assert "SOFIE_OUT_F32" in code and "std::vector<float> infer(float* tensor_x)" in code
     q = models.qcnn_params(oracle)
     text = open(dat).read().split("\n")
@@ -471,7 +514,7 @@ def test_conv_1d_and_3d_emission(tmp_path):
     on every side of every dimension, as in the reference (ROperator_Conv.hxx:136-139)."""
     c = open(models.conv1d_spec("c1d_t").generate(str(tmp_path))[0]).read()
     # [3,4,50], kernel 5 dilated by 2 (extent 9), pads 1+1, stride 2: (50 + 2 - 9) / 2 + 1 = 22
-    assert "sofie_hip_conv2d_f32(fCtx, tensor_x, tensor_w, tensor_b, tensor_c, 3, 4, 1, 50, 6, 1, 5, 0, 1, 1, 2, 1, 2, 2, SOFIE_ACT_RELU)" in c
+    assert "sofie_hip_conv2d_f32(fCtx, tensor_x, tensor_w, tensor_b, tensor_c, 3, 4, 1, 50, 6, 1, 5, 0, 1, 0, 1, 1, 2, 1, 2, 2, SOFIE_ACT_RELU)" in c
     assert "std::vector<float> ret(396);" in c
     c = open(models.conv3d_spec("c3d_t").generate(str(tmp_path))[0]).read()
     assert ("sofie_hip_conv3d_f32(fCtx, tensor_x, tensor_w, tensor_b, tensor_y, 2, 4, 6, 9, 10, 6, 3, 2, 3, 1, 0, 2, 1, 2, 1, 1, 1, 1, 2, "

@@ -184,6 +184,13 @@ def test_gemm_f32_integer_data_is_exact(ops):
     dict(N=2, C=16, H=9, W=19, OC=96, k=(3, 3), p=(1, 1), s=(2, 2), d=(1, 1), g=2, bias=True, relu=True),
     dict(N=1, C=8, H=12, W=12, OC=130, k=(3, 3), p=(2, 2), s=(1, 1), d=(2, 2), g=1, bias=True, relu=False),
     dict(N=3, C=12, H=13, W=10, OC=64, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, bias=False, relu=True),
+    # begin pads that differ from the end pads (top, left, bottom, right), as SAME_UPPER / SAME_LOWER make them for
+    # even kernels: the oracle convolves the explicitly padded tensor
+    dict(N=2, C=3, H=8, W=8, OC=4, k=(4, 4), p=(1, 1, 2, 2), s=(1, 1), d=(1, 1), g=1, bias=True, relu=False),
+    dict(N=2, C=3, H=8, W=8, OC=4, k=(4, 4), p=(2, 2, 1, 1), s=(1, 1), d=(1, 1), g=1, bias=True, relu=True),
+    dict(N=1, C=4, H=7, W=6, OC=6, k=(3, 2), p=(0, 2, 1, 0), s=(1, 1), d=(1, 1), g=2, bias=True, relu=False),
+    dict(N=2, C=16, H=15, W=18, OC=96, k=(3, 3), p=(0, 0, 1, 1), s=(2, 2), d=(1, 1), g=1, bias=True, relu=True),
+    dict(N=1, C=8, H=12, W=12, OC=130, k=(3, 3), p=(3, 0, 1, 4), s=(1, 1), d=(2, 2), g=1, bias=False, relu=False),
 ])
 def test_conv2d_f32(ops, cfg):
     r = rng(200 + cfg["C"] + cfg["OC"])
@@ -371,6 +378,8 @@ def test_qgemm_rounding_ties_and_saturation(ops):
     dict(N=2, C=64, H=10, W=10, OC=128, k=(3, 3), p=(1, 1), s=(1, 1), g=1),
     dict(N=1, C=16, H=9, W=11, OC=24, k=(1, 1), p=(0, 0), s=(2, 2), g=1),
     dict(N=1, C=64, H=56, W=56, OC=128, k=(3, 3), p=(1, 1), s=(1, 1), g=1),
+    dict(N=2, C=6, H=7, W=6, OC=8, k=(4, 2), p=(1, 0, 2, 1), s=(1, 1), g=2),      # begin != end pads, plain kernel
+    dict(N=1, C=1, H=40, W=40, OC=32, k=(3, 3), p=(1, 1, 0, 1), s=(1, 1), g=1),   # not the first-layer kernel's shape
 ])
 def test_qconv2d_s8(ops, cfg):
     from sofie_amd import lib as L
@@ -408,6 +417,11 @@ def test_qconv2d_s8(ops, cfg):
     dict(N=3, C=32, H=11, W=8, OC=64, k=(3, 1), p=(1, 0), s=(2, 1)),
     dict(N=1, C=32, H=4, W=4, OC=64, k=(3, 3), p=(2, 2), s=(1, 1)),
     dict(N=300, C=32, H=3, W=3, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
+    # begin != end pads (top, left, bottom, right): bands of H + top + bottom rows, windows placed by the begin pads
+    dict(N=5, C=32, H=12, W=12, OC=64, k=(4, 4), p=(1, 1, 2, 2), s=(1, 1)),
+    dict(N=5, C=32, H=12, W=12, OC=64, k=(4, 4), p=(2, 2, 1, 1), s=(1, 1)),
+    dict(N=3, C=64, H=16, W=14, OC=128, k=(3, 3), p=(0, 0, 1, 1), s=(2, 2)),
+    dict(N=4, C=32, H=9, W=10, OC=64, k=(3, 3), p=(2, 0, 0, 1), s=(1, 1)),
 ])
 def test_qconv2d_s8_matrix_core_path(ops, cfg):
     """NHWC activations and [OC,KH,KW,C] weights straight into the MFMA kernel; NCHW operands of the same
@@ -550,6 +564,8 @@ def test_conv_pool_entry_point(ops, cfg):
     dict(N=2, C=32, H=17, W=9, OC=192, k=(1, 1), p=(0, 0), s=(1, 1)),
     dict(N=2, C=64, H=21, W=21, OC=64, k=(3, 3), p=(0, 0), s=(2, 2)),      # strided convolution before the pool
     dict(N=1, C=32, H=2, W=2, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),        # a single pooled pixel
+    dict(N=4, C=32, H=12, W=10, OC=64, k=(4, 4), p=(1, 1, 2, 2), s=(1, 1)),  # begin != end pads under the pooling
+    dict(N=3, C=64, H=9, W=11, OC=128, k=(3, 3), p=(2, 1, 0, 1), s=(1, 1)),
 ])
 def test_conv_pool_fused_matrix_core_kernel(ops, cfg):
     """Channels-last operands with a 2x2 stride-2 pooling: one kernel whose wavefronts pool on the accumulators.
