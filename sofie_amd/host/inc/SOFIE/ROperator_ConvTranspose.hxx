@@ -5,7 +5,8 @@
 //   - output extent = stride*(in-1) + kernel extent + output_padding - pad_begin - pad_end (:83-90), where the
 //     kernel extent counts the dilation;
 //   - an explicit output_shape attribute and auto_pad other than NOTSET are refused (:52-79,:91-97);
-//   - begin/end pads that differ are averaged with a warning at generation time (:318-346);
+//   - begin/end pads that differ: the reference averages them with a warning at generation time (:318-346) while
+//     the declared output extent uses their sum; here both reach the library and the result is ONNX's;
 //   - 3-D transposed convolutions are refused (:391).
 // Emitted code: one sofie_hip_conv_transpose2d_f32 call over the whole batch (bias and optional ReLU
 // fused) instead of the kernel re-layout loop, sgemm_ into a column matrix, col2im and saxpy_ per image.
@@ -129,14 +130,8 @@ public:
       OpName = "op_" + OpName;
       if (fShapeX.empty() || fShapeW.empty() || (fNB != "" && fShapeB.empty()) || fShapeY.empty())
          throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
-      // begin pads that differ from the end pads are averaged, as the reference does before its col2im call
-      for (size_t i = 0; i < fDim; ++i) {
-         if (fAttrPads[i] != fAttrPads[fDim + i]) {
-            std::cout << "TMVA SOFIE Operator ConvTranspose:  asymmetric padding not supported. Assume an average padding "
-                      << std::endl;
-            fAttrPads[i] = (fAttrPads[i] + fAttrPads[fDim + i]) / 2;
-         }
-      }
+      // the library places the result by the begin pads and is told the output extent (which the end pads shorten):
+      // begin and end pads that differ are exact
       const bool oneD = fDim == 1;
       const size_t H = oneD ? 1 : fShapeX[2], W = fShapeX[fDim + 1];
       const size_t KH = oneD ? 1 : fShapeW[2], KW = fShapeW[fDim + 1];

@@ -66,6 +66,8 @@ public:
       if (fAttr.kernel_shape.empty()) fAttr.kernel_shape = {input[0][2], input[0][3]};
       if (fAttr.auto_pad != "NOTSET")
          throw std::runtime_error("TMVA SOFIE" + Name() + "Op : auto_pad is not supported by the device emission");
+      if (fAttr.ceil_mode != 0)
+         throw std::runtime_error("TMVA SOFIE" + Name() + "Op : ceil_mode is not supported by the device emission");
       if (fAttr.pads.empty()) fAttr.pads = {0, 0, 0, 0};
       fAttr.pads.resize(4, 0);
       if (fAttr.strides.empty()) fAttr.strides = {1, 1};

@@ -515,7 +515,8 @@ void RModel::ReadInitializedTensorsFromFile(long /*pos*/)
       const std::string ctype = ConvertTypeToString(i.second.type());
       fGC += "   {\n";
       fGC += "      std::vector<" + ctype + "> host(" + slength + ");\n";
-      fGC += "      ReadTensor(f, binary, \"" + tensor_name + "\", " + slength + ", host.data());\n";
+      fGC += "      ReadTensor(f, binary, \"" + tensor_name + "\", " + slength + ", " +
+             std::to_string(static_cast<int>(i.second.type())) + ", host.data());\n";
       fGC += "      Check(sofie_hip_upload(fCtx, " + tensor_name + ", host.data(), " + slength + " * sizeof(" + ctype + ")), \"upload of " +
              tensor_name + "\");\n";
       fGC += "   }\n";
@@ -541,7 +542,7 @@ std::string RModel::GenerateWeightReaderHelpers()
    g += "   return false;\n";
    g += "}\n";
    g += "template <typename T>\n";
-   g += "static void ReadTensor(std::ifstream& f, bool binary, const std::string& expected, size_t expected_length, T* host) {\n";
+   g += "static void ReadTensor(std::ifstream& f, bool binary, const std::string& expected, size_t expected_length, unsigned expected_type, T* host) {\n";
    g += "   std::string tensor_name;\n";
    g += "   size_t length = 0;\n";
    g += "   if (binary) {\n";
@@ -554,6 +555,9 @@ std::string RModel::GenerateWeightReaderHelpers()
    g += "      f.read(reinterpret_cast<char*>(&type), 4);\n";
    g += "      f.read(reinterpret_cast<char*>(&count), 8);\n";
    g += "      length = count;\n";
+   g += "      // a record of the same name and count but another element type would be reinterpreted byte for byte\n";
+   g += "      if (!f.fail() && tensor_name == expected && type != expected_type)\n";
+   g += "         throw std::runtime_error(\"TMVA-SOFIE failed to read the correct tensor type for \" + expected + \"; expected type code is \" + std::to_string(expected_type) + \" , read \" + std::to_string(type));\n";
    g += "   } else {\n";
    g += "      f >> tensor_name >> length;\n";
    g += "   }\n";

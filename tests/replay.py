@@ -59,8 +59,8 @@ def run_graph(graph, feeds, backend):
                                    groups=a.get("group", 1))
         elif op == "ConvTranspose":
             # ROperator_ConvTranspose.icc:14-103: strides / dilations default to 1, pads and output_padding to 0;
-            # :318-346: begin/end pads that differ are averaged for the scatter while the output keeps the size
-            # the shape rule gave it. A 1-D operator runs as a 2-D one with a height of one.
+            # begin/end pads that differ are kept as they are (the reference averages them for the scatter, :318-346,
+            # while the output keeps the size the shape rule gave it). A 1-D operator runs as a 2-D one with a height of one.
             x, w = env[ins[0]], env[ins[1]]
             dim = x.ndim - 2
             strides = list(a.get("strides", [1] * dim))
@@ -69,7 +69,7 @@ def run_graph(graph, feeds, backend):
             opad = list(a.get("output_padding", [0] * dim))
             out = [strides[i] * (x.shape[2 + i] - 1) + dil[i] * (w.shape[2 + i] - 1) + 1 + opad[i] - pads[i] - pads[dim + i]
                    for i in range(dim)]
-            begin = [pads[i] if pads[i] == pads[dim + i] else (pads[i] + pads[dim + i]) // 2 for i in range(dim)]
+            begin = [pads[i] for i in range(dim)]
             if dim == 1:
                 x, w = x[:, :, None, :], w[:, :, None, :]
                 strides, dil, begin, out = [1] + strides, [1] + dil, [0] + begin, [1] + out

@@ -651,3 +651,27 @@ def test_cpp_onnx_front_end_graph_with_two_outputs(tmp_path):
     first = re.search(r"sofie_hip_gemm_f32\([^;]*tensor_h, 4, (SOFIE_ACT_\w+)\)", code)
     assert first and first.group(1) == "SOFIE_ACT_NONE"
     assert "sofie_hip_relu_f32(" in code
+
+
+def test_cpp_onnx_front_end_refuses_ceil_mode_pooling(tmp_path):
+    """MaxPool with ceil_mode = 1 has a different output size than the floor rule the kernels implement: refused
+    at generation time (as auto_pad and dilations of a pooling are), not silently computed with the floor rule."""
+    import onnx_write as ow
+    nodes = [ow.node("MaxPool", ["x"], ["y"], kernel_shape=[2, 2], strides=[2, 2], ceil_mode=1)]
+    path = tmp_path / "ceil.onnx"
+    path.write_bytes(ow.model(nodes, {}, [("x", 1, (1, 2, 5, 5))], [("y", 1, (1, 2, 3, 3))]))
+    res = _onnx_emit(str(path), tmp_path)
+    assert res.returncode != 0
+    assert "ceil_mode is not supported" in res.stderr + res.stdout
+
+
+def test_generated_weight_reader_checks_the_element_type(tmp_path):
+    """Every ReadTensor call of the generated constructor names the element type it expects and the binary reader
+    compares it with the record's type field."""
+    spec = models.qdq_conv_spec("qdq_type")
+    hxx, _, _ = spec.generate(str(tmp_path), binary_weight_file=True)
+    code = open(hxx).read()
+    calls = re.findall(r'ReadTensor\(f, binary, "tensor_(\w+)", (\d+), (\d+), host\.data\(\)\);', code)
+    assert calls and {int(c[2]) for c in calls} <= {1, 2, 3, 6}          # FLOAT, UINT8, INT8, INT32
+    assert any(int(c[2]) == 3 for c in calls) and any(int(c[2]) == 1 for c in calls)
+    assert "type != expected_type" in code and "failed to read the correct tensor type" in code

@@ -249,3 +249,23 @@ def test_no_session_free_function(tmp_path):
     _, x = models.mlp_nosession_spec()
     y = run_session("mlp_nosession", x, tmp_path, dat="unused")
     assert rel_err(y, models.mlp_reference(oracle).reshape(-1)) <= 1e-5
+
+
+def test_binary_weight_file_with_another_element_type_is_refused(tmp_path):
+    """A record with the right name and count but another type code would be reinterpreted byte for byte: the
+    generated constructor throws instead (the process ends with a non-zero status before any kernel runs)."""
+    import struct
+    raw = bytearray(open(os.path.join(emit.GEN_DIR, "convbn.bin"), "rb").read())
+    (nlen,) = struct.unpack_from("<I", raw, 16)
+    (type_code,) = struct.unpack_from("<I", raw, 16 + 4 + nlen)
+    assert type_code == 1
+    struct.pack_into("<I", raw, 16 + 4 + nlen, 6)          # FLOAT -> INT32: same size, another meaning
+    bad = tmp_path / "bad.bin"
+    bad.write_bytes(bytes(raw))
+    p = models.convbn_params()
+    fin, fout = str(tmp_path / "in.bin"), str(tmp_path / "out.bin")
+    np.ascontiguousarray(p["x"], np.float32).tofile(fin)
+    res = subprocess.run([os.path.join(emit.GEN_DIR, "run_convbn"), str(bad), fin, fout], stdout=subprocess.PIPE,
+                         stderr=subprocess.PIPE, text=True, timeout=110)
+    assert res.returncode != 0
+    assert "correct tensor type" in res.stderr + res.stdout
