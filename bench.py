@@ -4,17 +4,29 @@
 Headline workload (the configuration the metric is quoted on): standalone int8 GEMM with QLinearMatMul
 semantics, M=N=K=4096, A and B int8 uniform in [-127,127], per-output-channel fp32 scales
 uniform in [1e-3,1e-2], int32 accumulate, round-half-to-even requantise to int8. One "step"
-is one call of sofie_hip_qgemm_s8 on device-resident operands. Prints ONE JSON line; next to the headline value it
-carries the other two figures the metric names: `fp8_gemm` (e4m3 GEMM 8192x8192x4096, TFLOP/s and fraction of the
-FP8 MFMA peak) and `model_inferences` (the generated int8 CNN Session at batch 4096, inferences per second).
+is one call of sofie_hip_qgemm_s8 on device-resident operands (one kernel launch). Prints ONE JSON line; next to the
+headline value it carries every other configuration of the benchmark:
+  fp8_gemm          e4m3 GEMM 8192x8192x4096, bf16 out + bias, TFLOP/s and fraction of the FP8 MFMA peak
+  model_inferences  the generated int8 CNN Session at batch 4096, inferences per second
+  mlp_f32           the generated fp32 MLP Session (64 -> 128 -> 64 -> 8, batch 256)
+  conv_f32/conv_s8  the 256 x 64 -> 128 x 56 x 56 3x3 layer in fp32 and int8
+  cpu_fp32          the reference's emitted CPU call sequence for the MLP and the convolution layer
+                    (oracle/cpu_emitted_bench.c) with sgemm_ from the best BLAS found on the box, at one thread and
+                    at the box's core share
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu]
 """
 import argparse
+import glob
+import importlib.util
 import json
 import os
+import statistics
+import subprocess
 import sys
+import tempfile
 import time
+from concurrent.futures import ThreadPoolExecutor
 
 import numpy as np
 
@@ -25,33 +37,138 @@ PEAK_INT8_TOPS = 5000.0     # MI355X dense int8 MFMA, 5.0 POP/s
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_FP32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM-side bytes of one call of the headline entry point (one GEMM kernel), from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE runs scaled by the same counters on a 64 MiB copy-like kernel (FETCH_SIZE x1.999, WRITE_SIZE x1.000):
-# 96.3 MiB fetched + 16.0 MiB written. Algorithmic bytes: 50.3 MB.
+# HBM-side bytes of one call of the headline entry point (one GEMM kernel). Not measurable inside this process: the
+# figure comes from two rocprofv3 --pmc runs of `bench.py --traffic-probe` (FETCH_SIZE, then WRITE_SIZE), each scaled
+# by what the same counter reads for a 64 MiB + 64 MiB copy-like kernel in the same run; the summary is in
+# profiles/int8_gemm_4096_k_gemm_dma.md. Algorithmic bytes: 50.3 MB.
 TRAFFIC_BYTES_PER_CALL = 112.3 * 1024 * 1024
+ALGORITHMIC_BYTES_PER_CALL = 3 * 4096 * 4096 + 4 * 4096
 
 
-def cpu_baseline_int8(A, B, scale, rows):
-    """The oracle (a scalar C port of the same arithmetic) on the first `rows` rows of A."""
+def host_threads():
+    """Threads the CPU legs may use: the box's share of cores (OMP_NUM_THREADS is set to it there), at most 16."""
+    try:
+        n = int(os.environ.get("OMP_NUM_THREADS", "0"))
+    except ValueError:
+        n = 0
+    if n <= 0:
+        n = os.cpu_count() or 1
+    return max(1, min(n, 16))
+
+
+def cpu_baseline_int8(A, B, scale, rows, threads):
+    """The oracle (a scalar C port of the same arithmetic) on the first `rows` rows of A, cut into one block of rows
+    per thread (ctypes releases the interpreter lock during the call)."""
     from oracle import oracle
+    rows = min(rows, A.shape[0])
+    blocks = [(i * rows // threads, (i + 1) * rows // threads) for i in range(threads)]
     t0 = time.perf_counter()
-    y = oracle.qgemm_s8(A[:rows], B, scale)
+    with ThreadPoolExecutor(threads) as pool:
+        parts = list(pool.map(lambda b: oracle.qgemm_s8(A[b[0]:b[1]], B, scale), blocks))
     dt = time.perf_counter() - t0
     ops = 2.0 * rows * B.shape[0] * B.shape[1]
-    return y, {"value": ops / dt / 1e12, "unit": "TOPS", "cores": 1, "kind": "port",
-               "sample": "oracle/sofie_oracle.c or_qgemm_s8 on the first %d of %d rows of A against the full B "
-                         "(%.1f GOP, %.1f s, gcc -O2, 1 thread)" % (rows, A.shape[0], ops / 1e9, dt)}
+    return np.concatenate(parts), {
+        "value": ops / dt / 1e12, "unit": "TOPS", "cores": threads, "kind": "port",
+        "sample": "oracle/sofie_oracle.c or_qgemm_s8 on the first %d of %d rows of A against the full B (%.1f GOP, %.1f s, "
+                  "gcc -O2, %d threads, one block of rows each)" % (rows, A.shape[0], ops / 1e9, dt, threads)}
 
 
-def time_launches(ctx, fn, steps, warmup):
-    """HIP events on the stream the kernels run on; returns average ms per launch."""
-    for _ in range(warmup):
-        fn()
-    ctx.sync()
-    ctx.timer_start()
-    for _ in range(steps):
-        fn()
-    return ctx.timer_stop() / steps
+class LaunchTimer:
+    """Durations on the stream the kernels are launched on, from HIP events recorded into that stream between blocks
+    of back-to-back launches (no host synchronisation inside the timed region)."""
+
+    def __init__(self, torch, stream):
+        self.torch, self.stream = torch, stream
+
+    def blocks(self, fn, n_blocks, per_block, warmup):
+        torch = self.torch
+        for _ in range(warmup):
+            fn()
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n_blocks + 1)]
+        ev[0].record(self.stream)
+        for b in range(n_blocks):
+            for _ in range(per_block):
+                fn()
+            ev[b + 1].record(self.stream)
+        self.stream.synchronize()
+        return [ev[b].elapsed_time(ev[b + 1]) / per_block for b in range(n_blocks)]
+
+    def median_ms(self, fn, launches, warmup=3, per_block=None):
+        per_block = per_block or max(1, min(10, launches // 5))
+        n_blocks = max(1, launches // per_block)
+        t = self.blocks(fn, n_blocks, per_block, warmup)
+        return statistics.median(t), min(t), n_blocks * per_block
+
+
+def blas_candidates():
+    """(path, symbol prefix, name) in the order the baseline prefers them: MKL, OpenBLAS, scipy's OpenBLAS."""
+    out = []
+    for p in ("/opt/conda/lib/libmkl_rt.so.2", "/opt/conda/lib/libmkl_rt.so.1", "/opt/conda/lib/libmkl_rt.so",
+              "/usr/lib/x86_64-linux-gnu/libmkl_rt.so"):
+        if os.path.exists(p):
+            out.append((p, "", "MKL (%s)" % p))
+            break
+    for p in ("/usr/lib/x86_64-linux-gnu/libopenblas.so.0", "/opt/conda/lib/libopenblas.so.0", "/opt/conda/lib/libopenblas.so"):
+        if os.path.exists(p):
+            out.append((p, "", "OpenBLAS (%s)" % p))
+            break
+    spec = importlib.util.find_spec("scipy")
+    if spec is not None and spec.origin:
+        hits = sorted(glob.glob(os.path.join(os.path.dirname(os.path.dirname(spec.origin)), "scipy.libs",
+                                             "libscipy_openblas-*.so")))
+        if hits:
+            out.append((hits[0], "scipy_", "scipy's OpenBLAS (%s)" % os.path.basename(hits[0])))
+    return out
+
+
+def cpu_emitted(workload, threads, blas, extra=()):
+    """One run of oracle/cpu_emitted_bench as a child process with the thread count in its environment."""
+    exe = os.path.join(ROOT, "oracle", "cpu_emitted_bench")
+    if not os.path.exists(exe):
+        return None
+    env = dict(os.environ)
+    for k in ("OMP_NUM_THREADS", "MKL_NUM_THREADS", "OPENBLAS_NUM_THREADS"):
+        env[k] = str(threads)
+    env["MKL_DYNAMIC"] = "FALSE"
+    cmd = [exe, "--workload", workload] + list(extra)
+    if blas:
+        cmd += ["--blas", blas[0], "--prefix", blas[1]]
+    try:
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env, timeout=240)
+    except subprocess.TimeoutExpired:
+        return None
+    if res.returncode != 0:
+        return None
+    out = json.loads(res.stdout.strip().splitlines()[-1])
+    return out if out["selfcheck"] <= 1e-3 else None
+
+
+def cpu_fp32_baselines(threads, conv_images=64):
+    """The reference's emitted CPU sequence (bias copy + sgemm_ + ReLU; weight re-layout + Im2col + sgemm_ + saxpy_ +
+    Relu) on the host cores: first BLAS that binds and passes the self-check, at 1 thread and at `threads`."""
+    chosen = None
+    for cand in blas_candidates() + [None]:
+        probe = cpu_emitted("mlp", 1, cand, ("--calls", "20"))
+        if probe is not None:
+            chosen = cand
+            break
+    name = chosen[2] if chosen else "none found: the bundled loops of oracle/cpu_emitted_bench.c"
+    res = {"kind": "reference's emitted call sequence restated in C (oracle/cpu_emitted_bench.c), gcc -O2", "blas": name,
+           "host_cpus_visible": os.cpu_count(), "threads_used": sorted({1, threads})}
+    flops_conv = 2.0 * conv_images * 128 * 3136 * 576
+    for t in sorted({1, threads}):
+        m = cpu_emitted("mlp", t, chosen, ("--calls", "200"))
+        c = cpu_emitted("conv", t, chosen, ("--images", str(conv_images), "--calls", "3"))
+        if m:
+            res["mlp_b256_%dthr" % t] = {"median_us": m["median_ms"] * 1e3, "best_us": m["best_ms"] * 1e3,
+                                         "inferences_per_s": 256 / (m["median_ms"] * 1e-3), "cores": t, "calls": m["calls"]}
+        if c:
+            res["conv_64to128_56x56_%dthr" % t] = {
+                "median_ms": c["median_ms"], "best_ms": c["best_ms"], "gflops": flops_conv / c["median_ms"] / 1e6,
+                "cores": t, "calls": c["calls"],
+                "sample": "%d of the 256 images of the layer (per-image work is independent; %.1f GFLOP per call)"
+                          % (conv_images, flops_conv / 1e9)}
+    return res
 
 
 def main():
@@ -59,13 +176,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--cpu-rows", type=int, default=1024)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
+    ap.add_argument("--cpu-rows", type=int, default=0, help="rows of A the int8 CPU baseline evaluates (default: 256 per thread)")
     ap.add_argument("--cpu-images", type=int, default=256, help="images of the CNN batch the CPU baseline leg evaluates")
-    ap.add_argument("--extras", action="store_true", help="also time the FP8 GEMM, fp32 GEMM and conv layers")
+    ap.add_argument("--extras", action="store_true", help="accepted for compatibility: every configuration is in the default line")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch a 64 MiB copy-like kernel and the headline call three times and exit (the target of the "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
+    ap.add_argument("--kernel-probe", default="",
+                    help="launch one named workload a few times and exit (target of rocprofv3 runs): gemm_s8, gemm_s8_nk, "
+                         "gemm_fp8, gemm_fp8_nk, conv_s8, conv_f32")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collective, no sharding "
@@ -76,7 +196,12 @@ def main():
     from sofie_amd import ops
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible (the HIP library has no CPU fallback)")
-    ctx = ops.default_context()
+    # a stream of torch's (default priority) so that torch's events can be recorded into the stream the library
+    # launches on; inputs are made on torch's default stream and the device is synchronised before they are used
+    stream = torch.cuda.Stream()
+    ctx = ops.Context(0, guard=False, stream=stream)
+    timer = LaunchTimer(torch, stream)
+    threads = host_threads()
 
     n = 4096
     rng = np.random.default_rng(0)
@@ -85,6 +210,7 @@ def main():
     scale = rng.uniform(1e-3, 1e-2, n).astype(np.float32)
     dA, dB, dS = ctx.dev(A), ctx.dev(B), ctx.dev(scale)
     dY = ctx.empty((n, n), torch.int8)
+    torch.cuda.synchronize()
 
     def step():
         # B as ONNX QLinearMatMul states it: [K, N] row-major; the kernel stages rows of k in LDS and the
@@ -95,9 +221,23 @@ def main():
     if args.traffic_probe:
         X = torch.randn(16 * 1024 * 1024, device=ctx.device)      # the ReLU kernel reads 64 MiB and writes 64 MiB
         Z = torch.empty_like(X)
+        torch.cuda.synchronize()
         for _ in range(3):
             ctx.check(ctx.lib.sofie_hip_relu_f32(ctx.h, ctx.ptr(X), ctx.ptr(Z), X.numel()))
             step()
+        torch.cuda.synchronize()
+        return
+    if args.kernel_probe:
+        probes = workloads(ctx, torch, L, rng)
+        if args.kernel_probe == "gemm_s8":
+            fn = step
+        elif args.kernel_probe in probes:
+            fn = probes[args.kernel_probe][0]
+        else:
+            sys.exit("bench.py: unknown --kernel-probe %s" % args.kernel_probe)
+        torch.cuda.synchronize()
+        for _ in range(10):
+            fn()
         torch.cuda.synchronize()
         return
 
@@ -114,8 +254,9 @@ def main():
     ops_per_step = 2.0 * n * n * n
     tops = ops_per_step / (ms_per_step * 1e-3) / 1e12
 
-    # kernel duration from HIP events on the launch stream
-    kernel_ms = time_launches(ctx, step, args.steps, 2)
+    # duration of one launch: HIP events on the launch stream around blocks of 10 back-to-back launches, 25 blocks
+    # (250 launches whatever --steps says), median over the blocks
+    kernel_ms, kernel_ms_best, launches = timer.median_ms(step, 250, warmup=10, per_block=10)
     achieved = ops_per_step / (kernel_ms * 1e-3) / 1e12
 
     out = {
@@ -129,117 +270,154 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_INT8_TOPS, "traffic": TRAFFIC_BYTES_PER_CALL,
                      "kernel": "k_gemm_dma<MmaI8,128,2,S8,B_KN>",
-                     "kernel_ms": kernel_ms, "ops_per_launch": ops_per_step,
-                     "traffic_unit": "bytes per launch (profiles/int8_gemm_4096_k_gemm_dma.md)",
-                     "note": "unit counts an int8 multiply-add as 2 ops (TOP/s); one call of the entry point is one "
-                             "launch of this kernel"},
+                     "kernel_ms": kernel_ms, "kernel_ms_best_block": kernel_ms_best, "launches_timed": launches,
+                     "kernel_ms_exceeds_ms_per_step": bool(kernel_ms > ms_per_step),
+                     "ops_per_launch": ops_per_step, "algorithmic_bytes_per_launch": ALGORITHMIC_BYTES_PER_CALL,
+                     "traffic_unit": "HBM bytes per launch, from rocprofv3 --pmc runs (profiles/int8_gemm_4096_k_gemm_dma.md), "
+                                     "not measured in this process",
+                     "note": "unit counts an int8 multiply-add as 2 ops (TOP/s); one call of the entry point is one launch of "
+                             "this kernel; kernel_ms is the median over 25 blocks of 10 back-to-back launches between HIP "
+                             "events on the launch stream"},
     }
 
-    # parity spot check inside the benchmark: the timed output against the oracle on a few rows
+    # parity spot check inside the benchmark: the timed output against the oracle on a block of rows, and the same
+    # operands once more with scales that spread the outputs over the int8 range (the benchmark's scale range
+    # saturates about nine outputs in ten, which exercises the clamp but hardly the rounding)
     if not args.no_cpu:
-        y_ref, base = cpu_baseline_int8(A, B, scale, args.cpu_rows)
-        y_gpu = dY[:args.cpu_rows].cpu().numpy()
+        rows = args.cpu_rows or 256 * threads
+        y_ref, base = cpu_baseline_int8(A, B, scale, rows, threads)
+        y_gpu = dY[:rows].cpu().numpy()
         out["cpu_baseline"] = base
-        out["parity_rows_checked"] = int(args.cpu_rows)
+        out["parity_rows_checked"] = int(rows)
         out["parity_bit_exact"] = bool(np.array_equal(y_gpu, y_ref))
+        from oracle import oracle
+        spread = (np.random.default_rng(1).uniform(20, 60, n) / (73.3 * 73.3 * np.sqrt(n))).astype(np.float32)
+        dS2 = ctx.dev(spread)
+        torch.cuda.synchronize()
+        ctx.check(ctx.lib.sofie_hip_qgemm_s8(ctx.h, 0, n, n, n, ctx.ptr(dA), n, ctx.ptr(dB), n, ctx.ptr(dS2), None,
+                                             0, L.ACT_NONE, ctx.ptr(dY), n, L.OUT_S8))
+        ctx.sync()
+        y2 = dY[:128].cpu().numpy()
+        r2 = oracle.qgemm_s8(A[:128], B, spread)
+        out["parity_spread_scales"] = {"rows": 128, "bit_exact": bool(np.array_equal(y2, r2)),
+                                       "saturated_fraction": float(np.mean(np.abs(r2.astype(np.int32)) >= 127))}
     else:
         out["cpu_baseline"] = None
 
     # second half of the metric: the int8 CNN Session at batch 4096 (its own process, runs in about a second)
     out["model_inferences"] = cnn_session_rate(cpu_images=0 if args.no_cpu else args.cpu_images)
-    # the FP8 half of the metric's GEMM figure (e4m3 x e4m3, fp32 accumulate, bf16 out): B as it comes ([K,N])
-    fp8 = fp8_gemm_rates(ctx, torch, L)["fp8_gemm_8192x8192x4096_transB0"]
-    out["fp8_gemm"] = {"workload": "FP8 e4m3 GEMM M=N=8192 K=4096, B [K,N], bias, bf16 out", "ms": fp8["ms"],
-                       "tflops": fp8["tflops"], "frac_peak": fp8["frac_peak"], "peak_tflops": PEAK_FP8_TFLOPS}
-    if args.extras:
-        out["extras"] = extras(ctx, torch, L, ops, rng)
+    # every other configuration: each costs milliseconds
+    res = {}
+    for name, (fn, meta) in workloads(ctx, torch, L, rng).items():
+        torch.cuda.synchronize()
+        med, best, count = timer.median_ms(fn, meta.get("launches", 50), warmup=3)
+        entry = {"workload": meta["workload"], "ms": med, "ms_best_block": best, "launches_timed": count}
+        rate = meta["ops"] / med / 1e9
+        entry[meta["rate_unit"]] = rate
+        entry["frac_peak"] = rate / meta["peak"]
+        if "bytes" in meta:
+            entry["gbs"] = meta["bytes"] / med / 1e6
+        res[name] = entry
+    out["fp8_gemm"] = dict(res["gemm_fp8"], peak_tflops=PEAK_FP8_TFLOPS)
+    out["fp8_gemm_b_nk"] = res["gemm_fp8_nk"]
+    out["int8_gemm_b_nk"] = res["gemm_s8_nk"]
+    out["conv_f32"] = res["conv_f32"]
+    out["conv_s8"] = res["conv_s8"]
+    out["conv_transpose_f32"] = res["conv_transpose_f32"]
+    out["mlp_f32"] = mlp_session_rate()
+    if not args.no_cpu:
+        out["cpu_fp32"] = cpu_fp32_baselines(threads)
     print(json.dumps(out))
 
 
-def fp8_gemm_rates(ctx, torch, L):
-    """FP8 e4m3 GEMM 8192 x 8192 x 4096, bf16 out, fused bias, for B given [K,N] and [N,K]."""
-    res = {}
-    M, N, K = 8192, 8192, 4096
-    A8 = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=ctx.device)
-    B8 = torch.randint(0, 120, (K, N), dtype=torch.uint8, device=ctx.device)
-    bias = torch.randn(N, device=ctx.device)
-    Y16 = ctx.empty((M, N), torch.bfloat16)
-    for tb, Bm in ((0, B8), (1, B8.t().contiguous())):
-        ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_gemm_fp8(
-            ctx.h, tb, M, N, K, ctx.ptr(A8), K, ctx.ptr(Bm), Bm.shape[1], 0.01, 0.01, ctx.ptr(bias), ctx.ptr(Y16), N,
-            L.OUT_BF16)), 20, 3)
-        fl = 2.0 * M * N * K
-        res["fp8_gemm_8192x8192x4096_transB%d" % tb] = {"ms": ms, "tflops": fl / ms / 1e9,
-                                                        "frac_peak": fl / ms / 1e9 / PEAK_FP8_TFLOPS}
-    return res
-
-
-def extras(ctx, torch, L, ops, rng):
-    """Secondary figures of the other benchmark configurations (not the headline value)."""
-    ex = {}
-    # pre-transposed weights: the layout a Session keeps B in when it is an initializer
+def workloads(ctx, torch, L, rng):
+    """name -> (launcher, description): the configurations next to the headline one, on resident operands."""
+    w = {}
     n = 4096
     A = ctx.dev(rng.integers(-127, 128, (n, n)).astype(np.int8))
     Bt = ctx.dev(rng.integers(-127, 128, (n, n)).astype(np.int8))
     S = ctx.dev(rng.uniform(1e-3, 1e-2, n).astype(np.float32))
     Y = ctx.empty((n, n), torch.int8)
-    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_qgemm_s8(
-        ctx.h, 1, n, n, n, ctx.ptr(A), n, ctx.ptr(Bt), n, ctx.ptr(S), None, 0, 0, ctx.ptr(Y), n, L.OUT_S8)), 50, 5)
-    ex["int8_gemm_4096_transB"] = {"ms": ms, "tops": 2.0 * n ** 3 / ms / 1e9, "frac_peak": 2.0 * n ** 3 / ms / 1e9 / PEAK_INT8_TOPS}
-    ex.update(fp8_gemm_rates(ctx, torch, L))
+    w["gemm_s8_nk"] = (lambda: ctx.check(ctx.lib.sofie_hip_qgemm_s8(
+        ctx.h, 1, n, n, n, ctx.ptr(A), n, ctx.ptr(Bt), n, ctx.ptr(S), None, 0, 0, ctx.ptr(Y), n, L.OUT_S8)),
+        {"workload": "int8 GEMM 4096^3 with B pre-transposed to [N,K] (the layout a Session keeps an initializer in)",
+         "ops": 2.0 * n ** 3, "rate_unit": "tops", "peak": PEAK_INT8_TOPS, "launches": 100})
+    M, N, K = 8192, 8192, 4096
+    A8 = torch.randint(0, 120, (M, K), dtype=torch.uint8, device=ctx.device)
+    B8 = torch.randint(0, 120, (K, N), dtype=torch.uint8, device=ctx.device)
+    B8t = B8.t().contiguous()
+    bias = torch.randn(N, device=ctx.device)
+    Y16 = ctx.empty((M, N), torch.bfloat16)
+    for name, tb, Bm in (("gemm_fp8", 0, B8), ("gemm_fp8_nk", 1, B8t)):
+        w[name] = ((lambda tb=tb, Bm=Bm: ctx.check(ctx.lib.sofie_hip_gemm_fp8(
+            ctx.h, tb, M, N, K, ctx.ptr(A8), K, ctx.ptr(Bm), Bm.shape[1], 0.01, 0.01, ctx.ptr(bias), ctx.ptr(Y16), N,
+            L.OUT_BF16))),
+            {"workload": "FP8 e4m3 GEMM M=N=8192 K=4096, B %s, fused bias, bf16 out" % ("[N,K]" if tb else "[K,N]"),
+             "ops": 2.0 * M * N * K, "rate_unit": "tflops", "peak": PEAK_FP8_TFLOPS, "launches": 30})
     # fp32 conv layer: batch 256, 64 -> 128 channels, 56x56, 3x3, pad 1, bias + ReLU
     x = torch.rand(256, 64, 56, 56, device=ctx.device)
-    w = torch.randn(128, 64, 3, 3, device=ctx.device) * (2.0 / 576) ** 0.5
+    wt = torch.randn(128, 64, 3, 3, device=ctx.device) * (2.0 / 576) ** 0.5
     b = torch.randn(128, device=ctx.device) * 0.1
     y = ctx.empty((256, 128, 56, 56), torch.float32)
-    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_conv2d_f32(
-        ctx.h, ctx.ptr(x), ctx.ptr(w), ctx.ptr(b), ctx.ptr(y), 256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1)),
-        5, 1)
     fl = 2.0 * 256 * 128 * 3136 * 576
-    ex["conv2d_f32_b256_64to128_56x56"] = {"ms": ms, "tflops": fl / ms / 1e9, "frac_peak": fl / ms / 1e9 / PEAK_FP32_TFLOPS}
-    del x, w, y
-    # fp32 transposed conv (an upsampling layer): batch 64, 128 -> 64 channels, 28x28 -> 56x56, 4x4, stride 2, pad 1
-    x = torch.rand(64, 128, 28, 28, device=ctx.device)
-    w = torch.randn(128, 64, 4, 4, device=ctx.device) * 0.05
-    b = torch.randn(64, device=ctx.device) * 0.1
-    y = ctx.empty((64, 64, 56, 56), torch.float32)
-    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_conv_transpose2d_f32(
-        ctx.h, ctx.ptr(x), ctx.ptr(w), ctx.ptr(b), ctx.ptr(y), 64, 128, 28, 28, 64, 4, 4, 1, 1, 2, 2, 1, 1, 1, 56, 56, 0)),
-        5, 1)
-    fl = 2.0 * 64 * 128 * 64 * 16 * 784      # every input pixel meets every kernel tap once
-    ex["conv_transpose2d_f32_b64_128to64_28to56"] = {"ms": ms, "tflops": fl / ms / 1e9,
-                                                      "frac_peak": fl / ms / 1e9 / PEAK_FP32_TFLOPS}
-    # fp32 MLP batch 256: 64 -> 128 -> 64 -> 8 (three Gemm launches, ReLU fused)
-    X = torch.randn(256, 64, device=ctx.device)
-    Ws = [torch.randn(64, 128, device=ctx.device), torch.randn(128, 64, device=ctx.device),
-          torch.randn(64, 8, device=ctx.device)]
-    Bs = [torch.zeros(128, device=ctx.device), torch.zeros(64, device=ctx.device), torch.zeros(8, device=ctx.device)]
-    Hs = [ctx.empty((256, 128), torch.float32), ctx.empty((256, 64), torch.float32), ctx.empty((256, 8), torch.float32)]
-
-    def mlp():
-        cur = X
-        for i, (Wm, bm, h) in enumerate(zip(Ws, Bs, Hs)):
-            ctx.check(ctx.lib.sofie_hip_gemm_f32(ctx.h, 0, 0, 256, Wm.shape[1], Wm.shape[0], 1.0, ctx.ptr(cur),
-                                                 Wm.shape[0], ctx.ptr(Wm), Wm.shape[1], 1.0, ctx.ptr(bm), L.BIAS_ROW,
-                                                 ctx.ptr(h), Wm.shape[1], 1 if i < 2 else 0))
-            cur = h
-    ms = time_launches(ctx, mlp, 200, 10)
-    ex["mlp_f32_b256"] = {"us": ms * 1e3, "inferences_per_s": 256 / (ms * 1e-3), "gbs": 142112 / (ms * 1e-3) / 1e9}
-    del x, w, b, y
+    w["conv_f32"] = (lambda: ctx.check(ctx.lib.sofie_hip_conv2d_f32(
+        ctx.h, ctx.ptr(x), ctx.ptr(wt), ctx.ptr(b), ctx.ptr(y), 256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1)),
+        {"workload": "fp32 Conv2d NCHW batch 256, 64 -> 128 channels, 56x56, 3x3, stride 1, pad 1, bias + ReLU fused",
+         "ops": fl, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 10,
+         "bytes": 4.0 * (x.numel() + y.numel() + wt.numel() + 128)})
     # int8 conv layer of the same shape, channels-last, weights [OC][KH][KW][C], bias + ReLU + requantise fused
     xq = torch.randint(-128, 128, (256, 56, 56, 64), dtype=torch.int8, device=ctx.device)
     wq = torch.randint(-127, 128, (128, 3, 3, 64), dtype=torch.int8, device=ctx.device)
     sq = torch.full((128,), 2.0e-4, device=ctx.device)
     bq = torch.randint(-1000, 1000, (128,), dtype=torch.int32, device=ctx.device)
     yq = ctx.empty((256, 56, 56, 128), torch.int8)
-    ms = time_launches(ctx, lambda: ctx.check(ctx.lib.sofie_hip_qconv2d_s8(
+    w["conv_s8"] = (lambda: ctx.check(ctx.lib.sofie_hip_qconv2d_s8(
         ctx.h, ctx.ptr(xq), L.LAYOUT_NHWC, ctx.ptr(wq), L.LAYOUT_NHWC, ctx.ptr(bq), ctx.ptr(sq), ctx.ptr(yq), L.LAYOUT_NHWC,
-        256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, -128, -128, L.ACT_RELU, L.OUT_S8)), 20, 3)
-    fl = 2.0 * 256 * 128 * 3136 * 576
-    ex["conv2d_s8_b256_64to128_56x56"] = {"ms": ms, "tops": fl / ms / 1e9, "frac_peak": fl / ms / 1e9 / PEAK_INT8_TOPS,
-                                          "gbs": (xq.numel() + yq.numel() + wq.numel()) / ms / 1e6}
-    del xq, yq
-    return ex
+        256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, 1, 1, -128, -128, L.ACT_RELU, L.OUT_S8)),
+        {"workload": "int8 QLinearConv channels-last batch 256, 64 -> 128 channels, 56x56, 3x3, stride 1, pad 1, bias + ReLU "
+                     "+ requantise fused", "ops": fl, "rate_unit": "tops", "peak": PEAK_INT8_TOPS, "launches": 50,
+         "bytes": float(xq.numel() + yq.numel() + wq.numel() + 128 * 8)})
+    # fp32 transposed conv (an upsampling layer): batch 64, 128 -> 64 channels, 28x28 -> 56x56, 4x4, stride 2, pad 1
+    xt = torch.rand(64, 128, 28, 28, device=ctx.device)
+    wtt = torch.randn(128, 64, 4, 4, device=ctx.device) * 0.05
+    bt = torch.randn(64, device=ctx.device) * 0.1
+    yt = ctx.empty((64, 64, 56, 56), torch.float32)
+    w["conv_transpose_f32"] = (lambda: ctx.check(ctx.lib.sofie_hip_conv_transpose2d_f32(
+        ctx.h, ctx.ptr(xt), ctx.ptr(wtt), ctx.ptr(bt), ctx.ptr(yt), 64, 128, 28, 28, 64, 4, 4, 1, 1, 2, 2, 1, 1, 1, 56, 56, 0)),
+        {"workload": "fp32 ConvTranspose batch 64, 128 -> 64 channels, 28x28 -> 56x56, 4x4, stride 2, pad 1",
+         "ops": 2.0 * 64 * 128 * 64 * 16 * 784, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 10})
+    return w
+
+
+def run_generated(name, dat, x, iters):
+    """Runs sofie_amd/generated/run_<name> (a compiled generated Session) on x; returns (timings, output bytes)."""
+    gen = os.path.join(ROOT, "sofie_amd", "generated")
+    exe, datf = os.path.join(gen, "run_" + name), os.path.join(gen, dat)
+    if not (os.path.exists(exe) and os.path.exists(datf)):
+        return {"error": "generated Session %s missing: run build() first" % name}, None
+    with tempfile.TemporaryDirectory() as tmp:
+        xin, yout = os.path.join(tmp, "x.bin"), os.path.join(tmp, "y.bin")
+        x.tofile(xin)
+        res = subprocess.run([exe, datf, xin, yout, str(iters)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                             timeout=300)
+        y = np.fromfile(yout, np.float32) if res.returncode == 0 else None
+    if res.returncode != 0:
+        return {"error": res.stderr.strip()[-300:]}, None
+    return json.loads(res.stdout.strip().splitlines()[-1]), y
+
+
+def mlp_session_rate(iters=500):
+    """The generated Session of the fp32 MLP (64 -> 128 -> 64 -> 8, batch 256): three Gemm launches with fused bias and
+    ReLU. Device time of infer_device() on a resident input, replay from a HIP graph, wall time of infer()."""
+    x = np.random.default_rng(3).standard_normal((256, 64)).astype(np.float32)
+    t, _ = run_generated("mlp_c1", "mlp_c1.dat", x, iters)
+    if "error" in t:
+        return t
+    us = t["device_ms"] * 1e3
+    return {"workload": "fp32 MLP 64 -> 128 -> 64 -> 8, batch 256, generated Session (infer_device on a resident input)",
+            "us_per_batch": us, "inferences_per_s": 256 / (us * 1e-6), "gbs_algorithmic": 142112 / (us * 1e-6) / 1e9,
+            "graph_replay_us": t["graph_ms"] * 1e3, "graph_matches": t["graph_matches"],
+            "host_us_with_pcie": t["host_ms"] * 1e3, "bound": "launch latency (8.65 MFLOP, 142,112 algorithmic bytes)"}
 
 
 def cnn_session_rate(iters=50, cpu_images=0):
@@ -248,22 +426,10 @@ def cnn_session_rate(iters=50, cpu_images=0):
     infer_device() on a resident input, and wall time of infer() including the PCIe copies. With cpu_images > 0 the
     CPU restatement of the same network is timed on that many images of the batch (one thread) and the Session's
     logits of those images are compared with it bit for bit."""
-    import subprocess
-    import tempfile
-    gen = os.path.join(ROOT, "sofie_amd", "generated")
-    exe, dat = os.path.join(gen, "run_qcnn_b4096"), os.path.join(gen, "qcnn.dat")
-    if not (os.path.exists(exe) and os.path.exists(dat)):
-        return {"error": "generated Session missing: run build() first"}
-    with tempfile.TemporaryDirectory() as tmp:
-        xin, yout = os.path.join(tmp, "x.bin"), os.path.join(tmp, "y.bin")
-        x = np.random.default_rng(2).uniform(0, 1, (4096, 1, 40, 40)).astype(np.float32)
-        x.tofile(xin)
-        res = subprocess.run([exe, dat, xin, yout, str(iters)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
-                             timeout=300)
-        y = np.fromfile(yout, np.float32) if res.returncode == 0 else None
-    if res.returncode != 0:
-        return {"error": res.stderr.strip()[-300:]}
-    t = json.loads(res.stdout.strip().splitlines()[-1])
+    x = np.random.default_rng(2).uniform(0, 1, (4096, 1, 40, 40)).astype(np.float32)
+    t, y = run_generated("qcnn_b4096", "qcnn.dat", x, iters)
+    if "error" in t:
+        return t
     ops_per_image = 36968960.0
     cpu = None
     if cpu_images > 0:
@@ -279,7 +445,7 @@ def cnn_session_rate(iters=50, cpu_images=0):
                "sample": "oracle/sofie_oracle.c (quantize, three QLinearConv + ReLU + MaxPool, two QLinearMatMul) on the first "
                          "%d of the 4096 images (%.2f s, gcc -O2, 1 thread)" % (cpu_images, sec),
                "logits_bit_exact": bool(np.array_equal(y.reshape(4096, -1)[:cpu_images], ref.reshape(cpu_images, -1)))}
-    return {"cpu_baseline": cpu,"workload": "int8 CNN classifier, batch 4096, 1x40x40 input, generated Session (infer_device on a resident input)",
+    return {"cpu_baseline": cpu, "workload": "int8 CNN classifier, batch 4096, 1x40x40 input, generated Session (infer_device on a resident input)",
             "device_ms": t["device_ms"], "inferences_per_s": 4096 / (t["device_ms"] * 1e-3),
             "tops": 4096 * ops_per_image / t["device_ms"] / 1e9,
             "frac_peak": 4096 * ops_per_image / t["device_ms"] / 1e9 / PEAK_INT8_TOPS,

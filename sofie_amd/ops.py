@@ -29,13 +29,13 @@ class Context:
     Every output buffer that `empty` hands out lies between two sentinel bands that `ret` checks after the
     call: a store outside the tensor (a ragged tile written past its edge) raises instead of going unseen."""
 
-    def __init__(self, device=0, guard=True):
+    def __init__(self, device=0, guard=True, stream=None):
         if not torch.cuda.is_available():
             raise SofieHipError("no GPU visible: the HIP library has no CPU fallback")
         self.lib = L.load()
         self.device = torch.device("cuda", device)
         torch.cuda.set_device(self.device)
-        self.stream = torch.cuda.current_stream(self.device)
+        self.stream = stream if stream is not None else torch.cuda.current_stream(self.device)
         h = C.c_void_p()
         rc = self.lib.sofie_hip_create(C.byref(h), device, C.c_void_p(self.stream.cuda_stream))
         if rc:

@@ -600,7 +600,7 @@ def test_empty_and_degenerate_inputs(ops):
     assert lib.sofie_hip_qgemm_s8(h, 1, 0, 4, 16, None, 16, None, 16, None, None, 0, 0, None, 4, L.OUT_S8) == 0
     assert lib.sofie_hip_qgemm_s8(h, 1, 4, 0, 16, p(A), 16, p(A), 16, p(sc), None, 0, 0, p(y), 4, L.OUT_S8) == 0
     assert lib.sofie_hip_gemm_f32(h, 0, 0, 0, 5, 3, 1.0, None, 3, None, 5, 0.0, None, 0, None, 5, 0) == 0
-    assert lib.sofie_hip_conv2d_f32(h, None, None, None, None, 0, 3, 5, 5, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0) == 0
+    assert lib.sofie_hip_conv2d_f32(h, None, None, None, None, 0, 3, 5, 5, 4, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 0) == 0
     assert lib.sofie_hip_conv_transpose2d_f32(h, None, None, None, None, 0, 3, 5, 5, 4, 3, 3, 0, 0, 1, 1, 1, 1, 1, 7, 7, 0) == 0
     assert lib.sofie_hip_batchnorm_f32(h, None, None, None, None, None, 0, 3, 5, 0) == 0
     assert lib.sofie_hip_relu_f32(h, None, None, 0) == 0
@@ -640,18 +640,18 @@ def test_error_codes_of_the_quantized_entry_points(ops):
                  out=L.OUT_S8, ph=1)
         a.update(kw)
         return lib.sofie_hip_qconv2d_s8(h, a["x"], a["xl"], a["w"], a["wl"], None, a["s"], a["y"], L.LAYOUT_NHWC, 1, 32, 4, 4,
-                                        64, 3, 3, a["ph"], 1, 1, 1, a["groups"], a["zpx"], 0, a["act"], a["out"])
+                                        64, 3, 3, a["ph"], 1, 1, 1, 1, 1, a["groups"], a["zpx"], 0, a["act"], a["out"])
     assert conv() == 0
     for bad, text in ((dict(x=None), "null operand"), (dict(groups=3), "groups"), (dict(zpx=300), "zero-point"),
                       (dict(act=7), "activation"), (dict(xl=5), "layout"), (dict(out=L.OUT_BF16), "output kind"),
                       (dict(s=None), "scale is required"), (dict(ph=-1), "pads")):
         assert conv(**bad) == L.EINVAL, bad
         assert text in lib.sofie_hip_last_error(h).decode(), (bad, lib.sofie_hip_last_error(h))
-    assert lib.sofie_hip_qconv2d_pool_s8(h, p(x), 1, p(w), 1, None, p(sc), p(y), 1, 1, 32, 4, 4, 64, 3, 3, 1, 1, 1, 1, 1, 0, 0,
+    assert lib.sofie_hip_qconv2d_pool_s8(h, p(x), 1, p(w), 1, None, p(sc), p(y), 1, 1, 32, 4, 4, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0, 0,
                                          0, 9, 9, 1, 1) == L.EINVAL
     assert "pooling window" in lib.sofie_hip_last_error(h).decode()
     assert lib.sofie_hip_quantize_qconv2d_s8(h, p(ctx.dev(np.zeros((1, 32, 4, 4), np.float32))), -1.0, 0, p(w), 1, None, p(sc),
-                                             p(y), 1, 1, 32, 4, 4, 64, 3, 3, 1, 1, 1, 1, 1, 0, 0, 0, 0, 0, 0) == L.EINVAL
+                                             p(y), 1, 1, 32, 4, 4, 64, 3, 3, 1, 1, 1, 1, 1, 1, 1, 0, 0, 0, 0, 0, 0) == L.EINVAL
     A = ctx.dev(np.zeros((16, 16), np.int8))
     Y = ctx.empty((16, 16), torch.int8)
     assert lib.sofie_hip_qgemm_s8(h, 1, 16, 16, 16, p(A), 8, p(A), 16, p(ctx.dev(np.ones(16, np.float32))), None, 0, 0, p(Y), 16,

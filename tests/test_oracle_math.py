@@ -498,3 +498,58 @@ def test_conv_transpose2d_f32_against_torch_and_scatter(cfg):
             if relu:
                 tsym = np.maximum(tsym, 0)
             assert np.max(np.abs(y - tsym)) <= 1e-5 * scale
+
+
+# ----------------------------------------------------------------------------- the CPU baseline program
+def _cpu_emitted(args, env=None):
+    import json
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(oracle.__file__)), "cpu_emitted_bench")
+    if not os.path.exists(exe):
+        subprocess.run(["make", "-C", os.path.dirname(exe), "cpu_emitted_bench"], check=True, stdout=subprocess.DEVNULL)
+    e = dict(os.environ)
+    e.update(env or {})
+    res = subprocess.run([exe] + args, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=e, timeout=300)
+    assert res.returncode == 0, res.stderr
+    return json.loads(res.stdout.strip().splitlines()[-1])
+
+
+def _scipy_blas():
+    import glob
+    import importlib.util
+    import os
+    spec = importlib.util.find_spec("scipy")
+    if spec is None:
+        return None
+    hits = glob.glob(os.path.join(os.path.dirname(os.path.dirname(spec.origin)), "scipy.libs", "libscipy_openblas-*.so"))
+    return hits[0] if hits else None
+
+
+def test_cpu_baseline_program_computes_what_the_oracle_computes(tmp_path):
+    """oracle/cpu_emitted_bench.c (the reference's emitted call sequence for the fp32 MLP and convolution layer,
+    timed by the benchmark as the CPU baseline) against the oracle's Gemm and Conv on the inputs it dumps, with
+    its bundled loops and, where the image has one, with a BLAS bound at run time."""
+    blas = _scipy_blas()
+    variants = [[]] + ([["--blas", blas, "--prefix", "scipy_"]] if blas else [])
+    for extra in variants:
+        f = str(tmp_path / "mlp.bin")
+        out = _cpu_emitted(["--workload", "mlp", "--calls", "2", "--dump", f] + extra, {"OMP_NUM_THREADS": "2"})
+        assert out["selfcheck"] <= 1e-4
+        raw = np.fromfile(f, np.float32)
+        sizes = [256 * 64, 64 * 128, 128 * 64, 64 * 8, 256 * 8]
+        x, w0, w1, w2, y = np.split(raw, np.cumsum(sizes)[:-1])
+        h = oracle.gemm_f32(x.reshape(256, 64), w0.reshape(64, 128), np.zeros(128, np.float32), relu=True)
+        h = oracle.gemm_f32(h, w1.reshape(128, 64), np.zeros(64, np.float32), relu=True)
+        ref = oracle.gemm_f32(h, w2.reshape(64, 8), np.zeros(8, np.float32))
+        assert np.max(np.abs(y.reshape(256, 8) - ref)) <= 1e-5 * np.max(np.abs(ref))
+        # Glorot-uniform weights stay inside their limit, the input is roughly N(0,1)
+        assert np.max(np.abs(w0)) <= np.sqrt(6.0 / 192) and abs(float(x.std()) - 1.0) < 0.05
+        f = str(tmp_path / "conv.bin")
+        out = _cpu_emitted(["--workload", "conv", "--images", "2", "--calls", "1", "--dump", f] + extra,
+                           {"OMP_NUM_THREADS": "2"})
+        raw = np.fromfile(f, np.float32)
+        sizes = [2 * 64 * 56 * 56, 128 * 64 * 9, 128, 2 * 128 * 56 * 56]
+        x, w, b, y = np.split(raw, np.cumsum(sizes)[:-1])
+        ref = oracle.conv2d_f32(x.reshape(2, 64, 56, 56), w.reshape(128, 64, 3, 3), b, (1, 1), relu=True)
+        assert np.max(np.abs(y.reshape(ref.shape) - ref)) <= 1e-5 * np.max(np.abs(ref))
