@@ -228,13 +228,13 @@ def main():
         torch.cuda.synchronize()
         return
     if args.kernel_probe:
-        probes = workloads(ctx, torch, L, rng)
         if args.kernel_probe == "gemm_s8":
             fn = step
-        elif args.kernel_probe in probes:
-            fn = probes[args.kernel_probe][0]
         else:
-            sys.exit("bench.py: unknown --kernel-probe %s" % args.kernel_probe)
+            probes = workloads(ctx, torch, L, rng)
+            if args.kernel_probe not in probes:
+                sys.exit("bench.py: unknown --kernel-probe %s" % args.kernel_probe)
+            fn = probes[args.kernel_probe][0]
         torch.cuda.synchronize()
         for _ in range(10):
             fn()

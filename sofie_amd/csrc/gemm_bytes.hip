@@ -333,23 +333,34 @@ __device__ __forceinline__ void wait_vmcnt()
    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+template <int S> struct StageTag { static constexpr int value = S; };
+
+// LDS of k_gemm_dma: [A stage 0][A stage 1][B stage 0][B stage 1], BM*BK (BN*BK) bytes each. Both stages of an
+// operand lie within 64 KB of its first byte, so a fragment read is one per-lane base register plus a constant in the
+// instruction's 16-bit offset field for either stage, and the K loop (unrolled over the two stages) holds no
+// address arithmetic in the vector unit.
 template <class Mma, int BK, int NST, int OUT, bool B_KN>
 __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
 {
    static_assert(!B_KN || BK == 128, "the [K,N] operand path is laid out for 128-byte stages");
+   static_assert(NST == 2, "two stages per operand");
    constexpr int BM = 256, BN = 256;
    constexpr int TI = 4, TJ = 2;                      // wavefront tile: 128 n x 64 m
-   constexpr int STAGE = (BM + BN) * BK;              // A rows, then B^T rows
-   constexpr int DIST = NST - 1;                      // K-steps of requests in flight
+   constexpr int ABYTES = BM * BK, BBYTES = BN * BK;  // one stage of an operand
+   constexpr int BREG = NST * ABYTES;                 // first byte of the B region
    constexpr int NSUB = BK / Mma::KB;
    constexpr int CPR = BK / 16;                       // 16-byte chunks per row
    constexpr int RPB = 1024 / BK;                     // rows per 1 KB load block
    constexpr int SWS = BK == 64 ? 2 : 1;              // swizzle: chunk ^ ((row >> SWS) & (CPR-1))
    static_assert(BK == 64 || BK == 128, "stage depth");
+   static_assert(ABYTES * NST <= 65536 && BBYTES * NST <= 65536, "both stages of an operand within reach of the offset field");
    extern __shared__ __align__(16) unsigned char smem[];
    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
-   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+   const int tid = threadIdx.x, lane = tid & 63;
+   // the wavefront index is uniform: as a scalar it keeps everything derived from it (operand choice, load
+   // blocks, LDS destinations, descriptor) in scalar registers and the branches on it scalar branches
+   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
    const int wn = wave & 1, wm = wave >> 1;
    int tm, tn;
    tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
@@ -367,7 +378,7 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    // rows of k past K lie beyond the descriptor and read as zeros
    const rsrc_t rs = make_rsrc(tile_base, rows_are_k ? (unsigned)((size_t)(g.K - 1) * ld + (g.N - n0))
                                                      : (unsigned)((size_t)(rows_left - 1) * ld + g.K));
-   const int blk0 = wave * LPW;                        // first load block of this wavefront
+   const int blk0 = (wave & 3) * LPW;                  // first load block of this wavefront inside its operand's stage
    const int lrow = lane / CPR;                        // row inside a block
    // K-chunk this lane fetches in load block i: slot ^ swizzle(row); for BK = 128 the row
    // bits that enter the swizzle include the parity of the block
@@ -376,7 +387,7 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    for (int par = 0; par < 2; ++par) {
       const int row_in_tile = par * RPB + lrow;        // low bits only matter
       chunk[par] = (lane % CPR) ^ ((row_in_tile >> SWS) & (CPR - 1));
-      voff[par] = (((blk0 * RPB) & 255) + lrow) * ld + chunk[par] * 16;
+      voff[par] = (blk0 * RPB + lrow) * ld + chunk[par] * 16;
    }
    if (rows_are_k) {
       // [K,N] stage: row k holds 256 bytes of n as eight 32-byte pairs, pair p stored in slot p ^ (k & 7),
@@ -386,27 +397,31 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
          const int krow = par * 4 + (lane >> 4);
          const int slot = lane & 15;
          chunk[par] = (((slot >> 1) ^ (krow & 7)) << 1) | (slot & 1);
-         voff[par] = (((blk0 - 4 * LPW) * 4) + (lane >> 4)) * ld + chunk[par] * 16;
+         voff[par] = (blk0 * 4 + (lane >> 4)) * ld + chunk[par] * 16;
       }
    }
    const bool ktail = (g.K % BK) != 0;
    const int nk = (g.K + BK - 1) / BK;
-   auto request = [&](int t) {
-      // tile of K-step t -> stage t % NST; steps past the end repeat the last tile into a
-      // stage nobody reads any more, so the number of loads in flight never changes
+   // per-lane offsets of the last, partial K-step: chunks at or past K point beyond the descriptor and read as zeros
+   int voff_tail[2] = {voff[0], voff[1]};
+   if (ktail && !rows_are_k) {
+#pragma unroll
+      for (int par = 0; par < 2; ++par)
+         if ((nk - 1) * BK + chunk[par] * 16 >= g.K) voff_tail[par] = 0x7ffffff0;
+   }
+   const unsigned dst0 = lds0 + (uses_a ? 0 : BREG) + blk0 * 1024;   // this wavefront's first block in stage 0
+   const int row_step = rows_are_k ? 4 * ld : RPB * ld;
+   const int k_step = rows_are_k ? BK * ld : BK;
+   // tile of K-step t -> stage S of its operand; steps past the end repeat the last tile into a stage nobody reads
+   // any more, so the number of loads in flight never changes
+   auto request = [&](int t, int S) {
       const int tt = t < nk ? t : nk - 1;
-      const int k0 = tt * BK;
-      int vo[2] = {voff[0], voff[1]};
-      if (ktail && !rows_are_k) {
+      const bool tail = ktail && tt == nk - 1;
+      const int v0 = tail ? voff_tail[0] : voff[0], v1 = tail ? voff_tail[1] : voff[1];
+      const unsigned dst = dst0 + S * (uses_a ? ABYTES : BBYTES);
+      const int k_off = tt * k_step;
 #pragma unroll
-         for (int par = 0; par < 2; ++par)
-            if (k0 + chunk[par] * 16 >= g.K) vo[par] = 0x7ffffff0;   // beyond the descriptor: zeros
-      }
-      const unsigned dst = lds0 + (t % NST) * STAGE + blk0 * 1024;
-      const int row_step = rows_are_k ? 4 * ld : RPB * ld;
-      const int k_off = rows_are_k ? k0 * ld : k0;
-#pragma unroll
-      for (int i = 0; i < LPW; ++i) dma16(rs, dst + i * 1024, vo[(BK == 128) ? (i & 1) : 0], i * row_step + k_off);
+      for (int i = 0; i < LPW; ++i) dma16(rs, dst + i * 1024, (BK == 128 && (i & 1)) ? v1 : v0, i * row_step + k_off);
    };
    // --- MFMA operand addresses ---------------------------------------------------------
    const int fr = lane & 31, half = lane >> 5;
@@ -416,14 +431,24 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    // and upper half of the wavefront always read chunks that differ in bit 1 (slot ^ 2):
    // with the row swizzle this keeps the two halves of one ds_read_b128 off each other's banks.
    const int first_chunk = half * 2;
-   const int n_off = BM * BK + (wn * 128 + fr) * BK + ((first_chunk ^ sw) * 16);
+   const int n_off = BREG + (wn * 128 + fr) * BK + ((first_chunk ^ sw) * 16);
    const int m_off = (wm * 64 + fr) * BK + ((first_chunk ^ sw) * 16);
-   auto load_frag = [&](const unsigned char *stage, int off, int sub) -> typename Mma::Frag {
-      if constexpr (Mma::LANE_BYTES == 16) {      // chunk = (sub/2)*4 + half*2 + sub%2
-         return *reinterpret_cast<const v4i *>(stage + (off ^ ((sub & 1) * 16) ^ ((sub >> 1) * 64)));
-      } else {                                    // chunks sub*4 + half*2 + {0,1}
-         const v4i lo = *reinterpret_cast<const v4i *>(stage + (off ^ (sub * 64)));
-         const v4i hi = *reinterpret_cast<const v4i *>(stage + (off ^ (sub * 64) ^ 16));
+   // The chunk of sub-step `sub` is the first one XOR a constant below 128 bytes: four patterns in all
+   // (0, 16, 64, 80), one base register each per operand; tile index and stage are constants on top.
+   const unsigned char *m_base[4], *n_base[4];
+#pragma unroll
+   for (int p = 0; p < 4; ++p) {
+      const int pat = (p & 1) * 16 + (p >> 1) * 64;
+      m_base[p] = smem + (m_off ^ pat);
+      n_base[p] = smem + (n_off ^ pat);
+   }
+   // tile_off: i * 32 * BK (j * 32 * BK); stage_off: S * ABYTES (S * BBYTES)
+   auto load_frag = [&](const unsigned char *const (&base)[4], int tile_off, int stage_off, int sub) -> typename Mma::Frag {
+      if constexpr (Mma::LANE_BYTES == 16) {      // chunk = (sub/2)*4 + half*2 + sub%2: pattern index = sub
+         return *reinterpret_cast<const v4i *>(base[sub] + tile_off + stage_off);
+      } else {                                    // chunks sub*4 + half*2 + {0,1}: patterns 2*sub, 2*sub + 1
+         const v4i lo = *reinterpret_cast<const v4i *>(base[2 * sub] + tile_off + stage_off);
+         const v4i hi = *reinterpret_cast<const v4i *>(base[2 * sub + 1] + tile_off + stage_off);
          typename Mma::Frag f = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
          return f;
       }
@@ -432,14 +457,20 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    // B [K,N]: ds_read_b64_tr_b8 hands a lane eight consecutive k of its column. Of a group of 16 lanes,
    // lane s points at row (s >> 1), bytes (s & 1) * 8 .. + 7 of the group's 16 columns; lane t of the
    // group then receives column t of those eight rows. A fragment is the same K slice the A operand reads.
+   // The 32-byte pair of tile i is XORed into the address (bits 5-6): one base register per tile, with the
+   // half-wavefront's two chunks of K folded in; chunk, row group and stage are constants on top.
    const int ts = lane & 15;
-   const int kn_off = BM * BK + (ts >> 1) * 256 + ((((wn * 4) ^ (ts >> 1)) & 7) * 32) + ((lane >> 4) & 1) * 16 + (ts & 1) * 8;
-   auto load_frag_kn = [&](const unsigned char *stage, int i, int sub) -> typename Mma::Frag {
+   const int kn_off = BREG + (ts >> 1) * 256 + ((((wn * 4) ^ (ts >> 1)) & 7) * 32) + ((lane >> 4) & 1) * 16 + (ts & 1) * 8 +
+                      half * 2 * 16 * 256;
+   const unsigned char *kn_base[TI];
+#pragma unroll
+   for (int i = 0; i < TI; ++i) kn_base[i] = smem + (kn_off ^ (i * 32));
+   auto load_frag_kn = [&](int i, int stage_off, int sub) -> typename Mma::Frag {
       typedef int v2i_t __attribute__((ext_vector_type(2)));
       constexpr int NR = Mma::LANE_BYTES / 8;
-      // first 16-byte chunk of K this half of the wavefront holds in sub-step `sub` (as in load_frag)
-      const int ck = Mma::LANE_BYTES == 16 ? (sub >> 1) * 4 + half * 2 + (sub & 1) : sub * 4 + half * 2;
-      const unsigned char *p = stage + ((kn_off + ck * 16 * 256) ^ (i * 32));
+      // first 16-byte chunk of K of sub-step `sub` without the half-wavefront's share (as in load_frag)
+      const int ck = Mma::LANE_BYTES == 16 ? (sub >> 1) * 4 + (sub & 1) : sub * 4;
+      const unsigned char *p = kn_base[i] + ck * 16 * 256 + stage_off;
       typename Mma::Frag f;
 #pragma unroll
       for (int v = 0; v < NR; ++v) {
@@ -471,33 +502,33 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
       asm volatile("" ::: "memory");
    };
    if (nk > 0) {
-#pragma unroll
-      for (int t = 0; t < DIST; ++t) request(t);
-      wait_vmcnt<LPW *(DIST - 1)>();     // this wavefront's part of stage 0 has landed
+      request(0, 0);
+      wait_vmcnt<0>();                  // this wavefront's part of stage 0 has landed
    }
    barrier();
    if (group == 1) barrier();
-   for (int t = 0; t < nk; ++t) {
-      // load phase: requests for stage t+DIST (its buffer was last read one phase ago), then
-      // every operand fragment of stage t into registers
-      request(t + DIST);
-      const unsigned char *stage = smem + (t % NST) * STAGE;
+   // one K-step on the tile in stage S (a compile-time constant: the loop below is unrolled over the two stages)
+   auto kstep = [&](int t, auto tag) {
+      constexpr int S = decltype(tag)::value;
+      // load phase: requests for K-step t+1 into the other stage (last read one phase ago), then
+      // every operand fragment of stage S into registers
+      request(t + 1, 1 - S);
       typename Mma::Frag fn[NSUB][TI], fm[NSUB][TJ];
 #pragma unroll
       for (int sub = 0; sub < NSUB; ++sub) {
 #pragma unroll
          for (int i = 0; i < TI; ++i) {
-            if constexpr (B_KN) fn[sub][i] = load_frag_kn(stage, i, sub);
-            else fn[sub][i] = load_frag(stage, n_off + i * 32 * BK, sub);
+            if constexpr (B_KN) fn[sub][i] = load_frag_kn(i, S * BBYTES, sub);
+            else fn[sub][i] = load_frag(n_base, i * 32 * BK, S * BBYTES, sub);
          }
 #pragma unroll
-         for (int j = 0; j < TJ; ++j) fm[sub][j] = load_frag(stage, m_off + j * 32 * BK, sub);
+         for (int j = 0; j < TJ; ++j) fm[sub][j] = load_frag(m_base, j * 32 * BK, S * ABYTES, sub);
       }
       __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): fragments are in registers
-      // Stage t+1 is first read by group 0 right after the barrier that ends its multiply
+      // The other stage is first read by group 0 right after the barrier that ends its multiply
       // phase, which is the barrier that ends group 1's load phase: each group waits for its
-      // own part of stage t+1 just before that barrier.
-      if (group == 1) wait_vmcnt<LPW *(DIST - 1)>();
+      // own part of it just before that barrier.
+      if (group == 1) wait_vmcnt<0>();
       barrier();
       // multiply phase
 #pragma unroll
@@ -506,8 +537,12 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
          for (int i = 0; i < TI; ++i)
 #pragma unroll
             for (int j = 0; j < TJ; ++j) acc[i][j] = Mma::mma(fn[sub][i], fm[sub][j], acc[i][j]);
-      if (group == 0) wait_vmcnt<LPW *(DIST - 1)>();
+      if (group == 0) wait_vmcnt<0>();
       if (group == 0 || t + 1 < nk) barrier();
+   };
+   for (int t = 0; t < nk; t += 2) {
+      kstep(t, StageTag<0>{});
+      if (t + 1 < nk) kstep(t + 1, StageTag<1>{});
    }
    wait_vmcnt<0>();                         // the trailing dummy requests still target LDS
    __syncthreads();
