@@ -67,6 +67,15 @@ __device__ __forceinline__ unsigned f32_to_bf16(float x)
    return u >> 16;
 }
 
+// Two fp32 -> two bf16 in one dword (lo in bits 0-15), round to nearest even: v_cvt_pk_bf16_f32 of gfx950.
+__device__ __forceinline__ unsigned f32x2_to_bf16x2(float lo, float hi)
+{
+   typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+   typedef float f32x2_t __attribute__((ext_vector_type(2)));
+   const f32x2_t v = {lo, hi};
+   return __builtin_bit_cast(unsigned, __builtin_convertvector(v, bf16x2_t));
+}
+
 // Layout change of an int8 activation tensor (defined with the element-wise kernels).
 int relayout_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int N, int C, int H, int W, int from, int to);
 

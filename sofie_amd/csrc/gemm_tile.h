@@ -99,7 +99,8 @@ __device__ __forceinline__ unsigned epilogue_value(const GemmArgs &g, float sc, 
 //     wavefront's first column, filled and made visible by the caller;
 //   m_wave, n_wave: first output row and column of this wavefront.
 // ADD_BIAS false: the accumulators already include the bias.
-// PLAIN: int8 output with zero-point -128 and lower clamp -128: the byte conversion rounds half to
+// PLAIN = 2: int8 output with lower clamp -128 and any zero-point: the byte conversion's saturation at 0 is the clamp.
+// PLAIN = 1: int8 output with zero-point -128 and lower clamp -128: the byte conversion rounds half to
 // even and saturates, so it is the whole requantisation after the multiply.
 template <int TI, int OUT> struct EpilogueStaging {
    static constexpr int ESZ = OutSize<OUT>::value;
@@ -110,7 +111,7 @@ template <int TI, int OUT> struct EpilogueStaging {
 // FULLN: every 16-byte row segment lies inside the matrix and rows may be written with 16-byte
 // stores (no column checks). reg_scale: if not null, the lane's TI*4 scale vectors held in
 // registers (group gi = i*4 + q covers columns i*32 + q*8 + (lane/32)*4 .. +3); s_scale is then unused.
-template <class Mma, int TI, int TJ, int OUT, bool PLAIN, bool ADD_BIAS = true, bool FULLN = false>
+template <class Mma, int TI, int TJ, int OUT, int PLAIN, bool ADD_BIAS = true, bool FULLN = false>
 __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ],
                                                    unsigned char *stg, const float *s_scale, const int *s_bias,
                                                    int lane, int m_wave, int n_wave,
@@ -153,7 +154,8 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
             for (int t = 0; t < 4; ++t) {
                float r = __fmul_rn(__int2float_rn(acc[i][j][q * 4 + t] + (ADD_BIAS ? bi[t] : 0)), sc[t]);
                // v_cvt_pk_u8_f32 itself rounds to nearest even: with nothing to add, the product goes in as it is
-               if constexpr (!PLAIN) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
+               if constexpr (PLAIN == 0) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
+               if constexpr (PLAIN == 2) r = __fadd_rn(rintf(r), zpo);
                e[t] = r;
             }
             pk = __builtin_amdgcn_cvt_pk_u8_f32(e[0], 0, pk);
@@ -161,6 +163,16 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
             pk = __builtin_amdgcn_cvt_pk_u8_f32(e[2], 2, pk);
             pk = __builtin_amdgcn_cvt_pk_u8_f32(e[3], 3, pk);
             *reinterpret_cast<unsigned *>(dst) = pk ^ 0x80808080u;
+         } else if constexpr (!IS_INT && OUT == SOFIE_OUT_BF16) {
+            // acc * (scale_a * scale_b) [+ bias], then the hardware's packed conversion (round to nearest even)
+            float e[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+               e[t] = __fmul_rn(acc[i][j][q * 4 + t], g.s);
+               if (g.bias) e[t] = __fadd_rn(e[t], __int_as_float(bi[t]));
+            }
+            v2i p = {(int)f32x2_to_bf16x2(e[0], e[1]), (int)f32x2_to_bf16x2(e[2], e[3])};
+            *reinterpret_cast<v2i *>(dst) = p;
          } else {
             unsigned e[4];
 #pragma unroll
@@ -276,11 +288,14 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::A
    __syncthreads();
    unsigned char *stg = smem + wave * WB;
    if (OUT == SOFIE_OUT_S8 && g.zp == -128 && g.lo == -128)
-      tile_epilogue_wave<Mma, TI, TJ, OUT, true>(g, acc, stg, s_scale + wn * WN, s_bias + wn * WN, lane, m_wave,
-                                                 n0 + wn * WN);
+      tile_epilogue_wave<Mma, TI, TJ, OUT, 1>(g, acc, stg, s_scale + wn * WN, s_bias + wn * WN, lane, m_wave,
+                                              n0 + wn * WN);
+   else if (OUT == SOFIE_OUT_S8 && g.lo == -128)
+      tile_epilogue_wave<Mma, TI, TJ, OUT, 2>(g, acc, stg, s_scale + wn * WN, s_bias + wn * WN, lane, m_wave,
+                                              n0 + wn * WN);
    else
-      tile_epilogue_wave<Mma, TI, TJ, OUT, false>(g, acc, stg, s_scale + wn * WN, s_bias + wn * WN, lane, m_wave,
-                                                  n0 + wn * WN);
+      tile_epilogue_wave<Mma, TI, TJ, OUT, 0>(g, acc, stg, s_scale + wn * WN, s_bias + wn * WN, lane, m_wave,
+                                              n0 + wn * WN);
 }
 
 }  // namespace sofie
