@@ -11,7 +11,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+# SOFIE_ORACLE_LIB: another build of the same source (the sanitizer build the test suite runs in a child process)
+_LIB_PATH = os.environ.get("SOFIE_ORACLE_LIB") or os.path.join(_HERE, "liboracle.so")
 
 
 def build(force=False):

@@ -124,10 +124,11 @@ class ModelSpec:
 
     # ---- generation ------------------------------------------------------------------------
     def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False, batch=None,
-                 runtime_batch=False, no_session=False):
+                 runtime_batch=False, no_session=False, emitter=None, env=None):
         """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess). `batch` gives the shape
         parameters of the inputs (dimensions written as names) their value; with `runtime_batch` it is a capacity and
-        the generated Session also takes infer(n, ...) for any n up to it."""
+        the generated Session also takes infer(n, ...) for any n up to it. `emitter` names another build of the emit
+        program (the sanitizer build), `env` its environment."""
         os.makedirs(outdir, exist_ok=True)
         tdir = os.path.join(outdir, "tensors")
         os.makedirs(tdir, exist_ok=True)
@@ -144,9 +145,10 @@ class ModelSpec:
             if runtime_batch or self.runtime_batch:
                 flag += " runtimebatch"
             f.write("\n".join(self.lines + ["generate" + flag]) + "\n")
-        if not os.path.exists(EMIT):
+        if emitter is None and not os.path.exists(EMIT):
             build_emitter()
-        res = subprocess.run([EMIT, spec, tdir, outdir], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+        res = subprocess.run([emitter or EMIT, spec, tdir, outdir], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                             env=env)
         if check and res.returncode:
             raise RuntimeError("emitter failed: " + res.stderr)
         for fname in self.tensors:
