@@ -502,7 +502,10 @@ def cnn_session_rate(iters=50, cpu_images=0):
             "device_ms": t["device_ms"], "inferences_per_s": 4096 / (t["device_ms"] * 1e-3),
             "tops": 4096 * ops_per_image / t["device_ms"] / 1e9,
             "frac_peak": 4096 * ops_per_image / t["device_ms"] / 1e9 / PEAK_INT8_TOPS,
-            "host_ms_with_pcie": t["host_ms"], "inferences_per_s_with_pcie": 4096 / (t["host_ms"] * 1e-3)}
+            "host_ms_with_pcie": t["host_ms"], "inferences_per_s_with_pcie": 4096 / (t["host_ms"] * 1e-3),
+            "host_ms_with_pcie_pinned_input": t.get("host_pinned_ms"),
+            "inferences_per_s_with_pcie_pinned_input": 4096 / (t["host_pinned_ms"] * 1e-3) if t.get("host_pinned_ms") else None,
+            "pinned_input_same_logits": t.get("pinned_matches")}
 
 
 if __name__ == "__main__":

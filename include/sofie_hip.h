@@ -81,6 +81,12 @@ int sofie_hip_version(void);
  * members and `new char[]` pool of the generated Session (RModel.cxx:574-604). */
 int sofie_hip_malloc(sofie_hip_ctx *ctx, void **dptr, size_t bytes);
 int sofie_hip_free(sofie_hip_ctx *ctx, void *dptr);
+/* Page-locked host memory for inputs and outputs: an upload from (download into) it runs at the rate of the link,
+ * without the driver's staging copy of pageable memory. The generated Session hands such a buffer out per input
+ * (pinned_input_<name>()); infer() on that pointer is then bound by PCIe, not by the copy. No counterpart in the
+ * reference (its Session reads the caller's host pointer directly, RModel.cxx:680-801). */
+int sofie_hip_host_malloc(sofie_hip_ctx *ctx, void **hptr, size_t bytes);
+int sofie_hip_host_free(sofie_hip_ctx *ctx, void *hptr);
 int sofie_hip_upload(sofie_hip_ctx *ctx, void *dst_device, const void *src_host, size_t bytes);
 int sofie_hip_download(sofie_hip_ctx *ctx, void *dst_host, const void *src_device, size_t bytes);
 int sofie_hip_copy(sofie_hip_ctx *ctx, void *dst_device, const void *src_device, size_t bytes);
@@ -122,6 +128,18 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, int M, int N,
                        float alpha, const float *A, int lda, const float *B, int ldb,
                        float beta, const float *bias, int bias_kind, float *Y, int ldy,
                        int act);
+
+/* Stacked matrix products (numpy.matmul on operands of rank > 2) in one launch:
+ *   Y[i] = alpha * op(A[ia(i)]) * op(B[ib(i)]), optional ReLU, for every index i of the n_lead leading dimensions
+ * lead[0..n_lead) (row-major, last dimension fastest). stride_a[d] / stride_b[d] are the element strides of A / B
+ * along leading dimension d, 0 where the operand has extent 1 there and is broadcast; Y is dense: product i
+ * starts M * ldy elements after product i - 1. Replaces the loop over the stack that the reference emits around
+ * BLAS::sgemm_ (ROperator_Gemm.hxx:353-387), which hands every iteration the first matrices of A and B; here
+ * each product reads its own. No bias (the emitter refuses one on stacked operands). */
+#define SOFIE_GEMM_MAX_LEAD 6
+int sofie_hip_gemm_f32_stacked(sofie_hip_ctx *ctx, int transA, int transB, int M, int N, int K, float alpha,
+                               const float *A, int lda, const float *B, int ldb, float *Y, int ldy, int n_lead,
+                               const int *lead, const long long *stride_a, const long long *stride_b, int act);
 
 /* NCHW 2-D convolution y = conv(x, w) + bias[oc], optional ReLU.
  * x [N,C,H,W], w [OC, C/groups, KH, KW] (the ONNX layout, unpacked), bias [OC] or NULL,
@@ -196,6 +214,14 @@ int sofie_hip_relu_f32(sofie_hip_ctx *ctx, const float *x, float *y, size_t len)
 int sofie_hip_maxpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, int H,
                             int W, int kh, int kw, int pad_t, int pad_l, int pad_b,
                             int pad_r, int stride_h, int stride_w);
+
+/* NCHW average pooling over NC = N*C planes, same geometry rules as the max pooling. A window's values are summed
+ * in row-major order and divided once by the number of cells: those inside the image, or kh*kw when
+ * count_include_pad is set. GlobalAveragePool is the call with kh = H, kw = W, no pads, stride 1. Replaces the
+ * emitted loops of ROperator_Pool.hxx:371-416 in AveragePool mode (sum, nsum, `value /= float(nsum)`). */
+int sofie_hip_avgpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, int H, int W,
+                            int kh, int kw, int pad_t, int pad_l, int pad_b, int pad_r, int stride_h,
+                            int stride_w, int count_include_pad);
 
 /* ---------------------------------------------------------------- quantized operators
  * The reference has no quantized operator (its parser rejects int8 initialisers,

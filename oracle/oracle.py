@@ -66,6 +66,7 @@ _einsum = _sig("or_einsum_f32", None, [C.c_int, C.POINTER(C.c_void_p), C.c_int, 
                                      C.POINTER(C.c_longlong), _f32p])
 _bn = _sig("or_batchnorm_f32", None, [_f32p] * 5 + [C.c_float, _f32p] + [C.c_int] * 4)
 _maxpool = _sig("or_maxpool2d_f32", None, [_f32p, _f32p] + [C.c_int] * 11)
+_avgpool = _sig("or_avgpool2d_f32", None, [_f32p, _f32p] + [C.c_int] * 12)
 _maxpool_s8 = _sig("or_maxpool2d_s8", None, [_i8p, _i8p] + [C.c_int] * 11)
 _requant_one = _sig("or_requant_one", C.c_int8, [C.c_int32, C.c_float, C.c_int, C.c_int])
 _quant = _sig("or_quantize_f32_s8", None, [_f32p, _i8p, C.c_size_t, C.c_float, C.c_int])
@@ -258,6 +259,17 @@ def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0)):
     fn = _maxpool if x.dtype == np.float32 else _maxpool_s8
     fn(x, y, N * Cc, H, W, kernel[0], kernel[1], pads[0], pads[1], pads[2], pads[3],
        strides[0], strides[1])
+    return y
+
+
+def avgpool2d(x, kernel, strides, pads=(0, 0, 0, 0), count_include_pad=False):
+    """fp32 NCHW average pooling (ROperator_Pool.hxx:371-416); pads = (top, left, bottom, right)."""
+    x = np.ascontiguousarray(x, np.float32)
+    N, Cc, H, W = x.shape
+    OH, OW = _pool_out(H, W, kernel, pads, strides)
+    y = np.empty((N, Cc, OH, OW), np.float32)
+    _avgpool(x, y, N * Cc, H, W, kernel[0], kernel[1], pads[0], pads[1], pads[2], pads[3], strides[0], strides[1],
+             int(count_include_pad))
     return y
 
 

@@ -28,6 +28,8 @@
  *   or_einsum_f32                pinned: Einsum_matmul / _dotprod / _3 / _4 known answers of
  *                                the reference's tests, numpy.einsum in float64
  *   or_relu, or_maxpool2d        pinned: MaxPool2d known answer, torch CPU
+ *   or_avgpool2d_f32             pinned: torch.nn.functional.avg_pool2d on CPU (count_include_pad on and off),
+ *                                a float64 mean (the reference holds no AveragePool fixture for this path)
  *   or_broadcast_rows            pinned through the Linear_* answers (bias broadcast)
  *   or_qgemm_s8, or_qconv2d_s8,
  *   or_quantize_*, or_dequantize_*, or_gemm_fp8, or_e4m3_*, or_bf16_*
@@ -425,6 +427,44 @@ void or_einsum_f32(int n_inputs, const float *const *x, int n_labels, int n_out,
 /* skipped. Follows ROperator_Pool.hxx:371-416 (2-D branch) and the output   */
 /* size rule of :92-199. Pads are (top, left, bottom, right) = ONNX order    */
 /* pads[0], pads[1], pads[2], pads[3].                                        */
+/* ------------------------------------------------------------------------- */
+/* Average pooling as emitted by ROperator_Pool<float>::Generate in          */
+/* AveragePool mode (ROperator_Pool.hxx:371-416): per output the window's    */
+/* cells inside the image are added in row-major order into a float, nsum is */
+/* their count (or kh*kw when count_include_pad is set or there are no       */
+/* pads), then value /= float(nsum). GlobalAveragePool is the same with the  */
+/* kernel set to the image (:216-228). Pinned by: torch avg_pool2d on CPU    */
+/* (both settings of count_include_pad), a float64 mean.                     */
+/* ------------------------------------------------------------------------- */
+void or_avgpool2d_f32(const float *x, float *y, int NC, int H, int W, int kh, int kw,
+                      int pt, int pl, int pb, int pr, int sh, int sw, int include_pad)
+{
+    const int OH = (H + pt + pb - kh) / sh + 1;
+    const int OW = (W + pl + pr - kw) / sw + 1;
+    size_t o = 0;
+    for (int nc = 0; nc < NC; ++nc) {
+        const float *xi = x + (size_t)nc * H * W;
+        for (int oh = 0; oh < OH; ++oh)
+            for (int ow = 0; ow < OW; ++ow) {
+                float v = 0;
+                int nsum = 0;
+                for (int r = 0; r < kh; ++r) {
+                    const int ih = oh * sh - pt + r;
+                    if (ih < 0 || ih >= H) continue;
+                    for (int s = 0; s < kw; ++s) {
+                        const int iw = ow * sw - pl + s;
+                        if (iw < 0 || iw >= W) continue;
+                        v += xi[(size_t)ih * W + iw];
+                        nsum++;
+                    }
+                }
+                if (include_pad) nsum = kh * kw;
+                v /= (float)nsum;
+                y[o++] = v;
+            }
+    }
+}
+
 /* ------------------------------------------------------------------------- */
 void or_maxpool2d_f32(const float *x, float *y, int NC, int H, int W, int kh, int kw,
                       int pt, int pl, int pb, int pr, int sh, int sw)

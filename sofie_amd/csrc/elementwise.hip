@@ -102,6 +102,35 @@ __global__ void k_maxpool2d(const T *__restrict__ x, T *__restrict__ y, int N, i
    y[idx] = best;
 }
 
+// NCHW fp32 average pooling, one thread per output element. The window's values are added in row-major order of
+// the window (rows outside the image skipped), then divided once by the number of cells counted: the cells inside
+// the image, or the whole window when padding cells count (count_include_pad).
+__global__ void k_avgpool2d_f32(const float *__restrict__ x, float *__restrict__ y, int NC, int H, int W, int OH, int OW,
+                                int kh, int kw, int pt, int pl, int sh, int sw, int include_pad)
+{
+   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   const size_t total = (size_t)NC * OH * OW;
+   if (idx >= total) return;
+   size_t r = idx;
+   const int ow = (int)(r % OW); r /= OW;
+   const int oh = (int)(r % OH);
+   const size_t nc = r / OH;
+   const float *xi = x + nc * H * W;
+   float sum = 0.0f;
+   int count = 0;
+   for (int i = 0; i < kh; ++i) {
+      const int ih = oh * sh - pt + i;
+      if (ih < 0 || ih >= H) continue;
+      for (int j = 0; j < kw; ++j) {
+         const int iw = ow * sw - pl + j;
+         if (iw < 0 || iw >= W) continue;
+         sum = __fadd_rn(sum, xi[(size_t)ih * W + iw]);
+         ++count;
+      }
+   }
+   y[idx] = __fdiv_rn(sum, (float)(include_pad ? kh * kw : count));
+}
+
 // Channels-last int8 max pooling, 16 channels (one 16-byte vector) of one output pixel per thread.
 // Signed bytes are compared as unsigned after flipping the sign bit, four at a time.
 __device__ __forceinline__ unsigned max_u8x4(unsigned a, unsigned b)
@@ -305,6 +334,23 @@ int sofie_hip_maxpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC
    hipLaunchKernelGGL((k_maxpool2d<float, false>), dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y, 1,
                       NC, H, W, OH, OW, kh, kw, pt, pl, sh, sw);
    return check_launch(ctx, "k_maxpool2d");
+}
+
+int sofie_hip_avgpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, int H, int W, int kh, int kw,
+                            int pt, int pl, int pb, int pr, int sh, int sw, int count_include_pad)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, NC >= 0, "negative dimension");
+   if (NC == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && y, "null operand");
+   int OH, OW;
+   if (int rc = pool_dims(ctx, H, W, kh, kw, pt, pl, pb, pr, sh, sw, &OH, &OW)) return rc;
+   // a window that lies in the padding entirely would divide by zero cells
+   SOFIE_REQUIRE(ctx, count_include_pad || (pt < kh && pl < kw && pb < kh && pr < kw), "a pooling window without a cell of the image");
+   const size_t total = (size_t)NC * OH * OW;
+   hipLaunchKernelGGL(k_avgpool2d_f32, dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y, NC, H, W, OH, OW, kh, kw,
+                      pt, pl, sh, sw, count_include_pad != 0);
+   return check_launch(ctx, "k_avgpool2d_f32");
 }
 
 int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N, int C, int H, int W,

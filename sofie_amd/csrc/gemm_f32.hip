@@ -21,6 +21,12 @@ struct GemmF32Args {
    int transA, transB;
    float alpha, beta;
    int bias_kind, relu;
+   // stacked products (blockIdx.z + z0 = index of the product, row-major over the n_lead leading dimensions):
+   // element strides of A and B along each leading dimension (0 where the operand is broadcast), Y is dense
+   int n_lead, z0;
+   int lead[SOFIE_GEMM_MAX_LEAD];
+   long long sa[SOFIE_GEMM_MAX_LEAD], sb[SOFIE_GEMM_MAX_LEAD];
+   long long stride_y;
 };
 
 constexpr int BK = 16;
@@ -68,6 +74,20 @@ __global__ void __launch_bounds__(256) k_gemm_f32(GemmF32Args g)
    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
    const int wm = wave >> 1, wn = wave & 1;
    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+   if (g.n_lead > 0) {
+      // this workgroup's product of the stack: its position along every leading dimension, last dimension fastest
+      long long rem = (long long)blockIdx.z + g.z0, oa = 0, ob = 0;
+      const long long index = rem;
+      for (int d = g.n_lead - 1; d >= 0; --d) {
+         const long long pos = rem % g.lead[d];
+         rem /= g.lead[d];
+         oa += pos * g.sa[d];
+         ob += pos * g.sb[d];
+      }
+      g.A += oa;
+      g.B += ob;
+      g.Y += index * g.stride_y;
+   }
 
    float ra[BM * BK / 256], rb[BN * BK / 256];
    v16f acc[TI][TJ];
@@ -160,8 +180,11 @@ extern "C" int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, in
       bias = nullptr;
       bias_kind = SOFIE_BIAS_NONE;
    }
-   GemmF32Args g{A, B, bias, Y, M, N, K, lda, ldb, ldy, transA != 0, transB != 0, alpha, beta, bias_kind,
-                 act == SOFIE_ACT_RELU};
+   GemmF32Args g{};
+   g.A = A; g.B = B; g.bias = bias; g.Y = Y;
+   g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldy = ldy;
+   g.transA = transA != 0; g.transB = transB != 0;
+   g.alpha = alpha; g.beta = beta; g.bias_kind = bias_kind; g.relu = act == SOFIE_ACT_RELU;
    const bool small = (size_t)cdiv(M, 128) * cdiv(N, 128) < 256;
    if (small) {
       hipLaunchKernelGGL((k_gemm_f32<1, 1>), dim3(cdiv(N, 64), cdiv(M, 64)), dim3(256), 0, ctx->stream, g);
@@ -169,4 +192,41 @@ extern "C" int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, in
       hipLaunchKernelGGL((k_gemm_f32<2, 2>), dim3(cdiv(N, 128), cdiv(M, 128)), dim3(256), 0, ctx->stream, g);
    }
    return check_launch(ctx, "k_gemm_f32");
+}
+
+extern "C" int sofie_hip_gemm_f32_stacked(sofie_hip_ctx *ctx, int transA, int transB, int M, int N, int K, float alpha,
+                                          const float *A, int lda, const float *B, int ldb, float *Y, int ldy, int n_lead,
+                                          const int *lead, const long long *stride_a, const long long *stride_b, int act)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, M >= 0 && N >= 0 && K >= 0, "negative dimension");
+   SOFIE_REQUIRE(ctx, n_lead >= 1 && n_lead <= SOFIE_GEMM_MAX_LEAD && lead && stride_a && stride_b, "bad leading dimensions");
+   SOFIE_REQUIRE(ctx, act == SOFIE_ACT_NONE || act == SOFIE_ACT_RELU, "unknown activation");
+   long long stack = 1;
+   for (int d = 0; d < n_lead; ++d) {
+      SOFIE_REQUIRE(ctx, lead[d] >= 0 && stride_a[d] >= 0 && stride_b[d] >= 0, "negative extent or stride");
+      stack *= lead[d];
+      SOFIE_REQUIRE(ctx, stack < (1ll << 31), "too many stacked products");
+   }
+   if (M == 0 || N == 0 || stack == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, Y && (K == 0 || (A && B)), "null operand");
+   SOFIE_REQUIRE(ctx, lda >= (transA ? M : K) && ldb >= (transB ? K : N) && ldy >= N, "leading dimension too small");
+   GemmF32Args g{};
+   g.A = A; g.B = B; g.bias = nullptr; g.Y = Y;
+   g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldy = ldy;
+   g.transA = transA != 0; g.transB = transB != 0;
+   g.alpha = alpha; g.beta = 0.0f; g.bias_kind = SOFIE_BIAS_NONE; g.relu = act == SOFIE_ACT_RELU;
+   g.n_lead = n_lead;
+   for (int d = 0; d < n_lead; ++d) { g.lead[d] = lead[d]; g.sa[d] = stride_a[d]; g.sb[d] = stride_b[d]; }
+   g.stride_y = (long long)M * ldy;
+   // the grid's third dimension holds at most 65535 products per launch
+   for (long long z0 = 0; z0 < stack; z0 += 65535) {
+      const unsigned nz = (unsigned)((stack - z0) < 65535 ? (stack - z0) : 65535);
+      g.z0 = (int)z0;
+      const bool small = (size_t)cdiv(M, 128) * cdiv(N, 128) * nz < 256;
+      if (small) hipLaunchKernelGGL((k_gemm_f32<1, 1>), dim3(cdiv(N, 64), cdiv(M, 64), nz), dim3(256), 0, ctx->stream, g);
+      else hipLaunchKernelGGL((k_gemm_f32<2, 2>), dim3(cdiv(N, 128), cdiv(M, 128), nz), dim3(256), 0, ctx->stream, g);
+      if (int rc = check_launch(ctx, "k_gemm_f32 (stacked)")) return rc;
+   }
+   return SOFIE_HIP_OK;
 }

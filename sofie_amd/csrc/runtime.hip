@@ -177,6 +177,31 @@ int sofie_hip_free(sofie_hip_ctx *ctx, void *dptr)
    return SOFIE_HIP_OK;
 }
 
+int sofie_hip_host_malloc(sofie_hip_ctx *ctx, void **hptr, size_t bytes)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
+   SOFIE_REQUIRE(ctx, hptr != nullptr, "null result pointer");
+   *hptr = nullptr;
+   if (bytes == 0) return SOFIE_HIP_OK;
+   if (hipHostMalloc(hptr, bytes, hipHostMallocDefault) != hipSuccess) {
+      (void)hipGetLastError();
+      *hptr = nullptr;
+      return sofie::set_error(ctx, SOFIE_HIP_ENOMEM, "sofie_hip_host_malloc: %zu bytes of page-locked memory", bytes);
+   }
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_host_free(sofie_hip_ctx *ctx, void *hptr)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   if (!hptr) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
+   SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));   // a copy from or into the buffer may still run
+   SOFIE_HIP_CALL(ctx, hipHostFree(hptr));
+   return SOFIE_HIP_OK;
+}
+
 int sofie_hip_upload(sofie_hip_ctx *ctx, void *dst, const void *src, size_t bytes)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;

@@ -97,6 +97,13 @@ class ModelSpec:
     def relu(self, x, y):
         self.lines.append("op Relu %s %s" % (x, y))
 
+    def avgpool(self, x, y, kernel, pads=(0, 0, 0, 0), strides=(1, 1), count_include_pad=False):
+        self.lines.append("op %s %s %s %s %s %s" % ("AveragePoolIncludePad" if count_include_pad else "AveragePool", _lst(kernel),
+                                                    _lst(pads), _lst(strides), x, y))
+
+    def global_avgpool(self, x, y):
+        self.lines.append("op GlobalAveragePool %s %s" % (x, y))
+
     def maxpool(self, x, y, kernel, pads=(0, 0, 0, 0), strides=(1, 1)):
         self.lines.append("op MaxPool %s %s %s %s %s" % (_lst(kernel), _lst(pads), _lst(strides), x, y))
 
@@ -163,7 +170,7 @@ class ModelSpec:
         cmd = ["g++", "-std=c++17", "-O2", "-I" + os.path.join(ROOT, "include"), "-I" + outdir,
                "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % self.name, "-DSOFIE_MODEL_NS=SOFIE_%s" % self.name,
                "-DSOFIE_IN_T=%s" % _CTYPE[self.input[1]], "-DSOFIE_OUT_T=%s" % _CTYPE[self.out_type],
-               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs),
+               "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_PINNED_INPUT=pinned_input_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs),
                "-DSOFIE_NUM_OUTPUTS=%d" % max(1, len(self.outputs))] + \
               (["-DSOFIE_RUNTIME_BATCH"] if (runtime_batch or self.runtime_batch) else []) + \
               (["-DSOFIE_NO_SESSION"] if self.no_session else []) + [
@@ -236,6 +243,11 @@ def spec_from_onnx(name, graph):
             spec.batchnorm(ins[0], ins[1], ins[2], ins[3], ins[4], out, a.get("epsilon", 1e-5))
         elif op == "MaxPool":
             spec.maxpool(ins[0], out, a["kernel_shape"], a.get("pads", (0, 0, 0, 0)), a.get("strides", (1, 1)))
+        elif op == "AveragePool":
+            spec.avgpool(ins[0], out, a["kernel_shape"], a.get("pads", (0, 0, 0, 0)), a.get("strides", (1, 1)),
+                         bool(a.get("count_include_pad", 0)))
+        elif op == "GlobalAveragePool":
+            spec.global_avgpool(ins[0], out)
         elif op == "Flatten":
             spec.flatten(ins[0], out, a.get("axis", 1))
         else:

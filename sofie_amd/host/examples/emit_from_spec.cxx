@@ -16,7 +16,8 @@
 //   op ConvTranspose AUTOPAD GROUP nk k.. np p.. ns s.. nd d.. nop op.. nos os.. X W B Y
 //   op Einsum EQUATION nx X.. Y                  (the equation without blanks)
 //   op Relu X Y
-//   op MaxPool nk k.. np p.. ns s.. X Y
+//   op MaxPool|AveragePool|AveragePoolIncludePad nk k.. np p.. ns s.. X Y
+//   op GlobalAveragePool X Y
 //   op Flatten AXIS X Y
 //   op QuantizeLinear X SCALE ZP Y | op DequantizeLinear X SCALE ZP Y
 //   op QLinearMatMul A AS AZ B BS BZ YS YZ BIAS Y TRANSB
@@ -150,14 +151,19 @@ int main(int argc, char **argv)
                std::string x, y;
                in >> x >> y;
                r.reset(new ROperator_Relu<float>(x, y));
-            } else if (op == "MaxPool") {
+            } else if (op == "MaxPool" || op == "AveragePool" || op == "AveragePoolIncludePad") {
                RAttributes_Pool attr;
                attr.kernel_shape = List(in);
                attr.pads = List(in);
                attr.strides = List(in);
+               attr.count_include_pad = op == "AveragePoolIncludePad";
                std::string x, y;
                in >> x >> y;
-               r.reset(new ROperator_Pool<float>(MaxPool, attr, x, y));
+               r.reset(new ROperator_Pool<float>(op == "MaxPool" ? MaxPool : AveragePool, attr, x, y));
+            } else if (op == "GlobalAveragePool") {
+               std::string x, y;
+               in >> x >> y;
+               r.reset(new ROperator_Pool<float>(GlobalAveragePool, RAttributes_Pool(), x, y));
             } else if (op == "Flatten") {
                int axis;
                std::string x, y;

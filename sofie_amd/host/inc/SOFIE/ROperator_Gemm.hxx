@@ -36,6 +36,8 @@ private:
    size_t fStack = 1;                       // stacked products (numpy.matmul on rank > 2 operands)
    std::vector<size_t> fStackA, fStackB;    // matrix index of A and B for every stacked product
    std::vector<size_t> fLeadY;              // leading dimensions of Y
+   std::vector<size_t> fLeadStrideA, fLeadStrideB;   // element strides of A and B along them (0: broadcast)
+   static constexpr size_t SOFIE_GEMM_MAX_LEAD_DIMS = 6;   // SOFIE_GEMM_MAX_LEAD of the kernel library
 
 public:
    ROperator_Gemm() {}
@@ -122,6 +124,18 @@ public:
          fStack = 1;
          fStackA.clear();
          fStackB.clear();
+         // element strides of A and B along every leading dimension (0 where the operand is broadcast)
+         fLeadStrideA.assign(rank - 2, 0);
+         fLeadStrideB.assign(rank - 2, 0);
+         {
+            size_t sa = la[rank - 2] * la[rank - 1], sb = lb[rank - 2] * lb[rank - 1];
+            for (size_t i = rank - 2; i-- > 0;) {
+               fLeadStrideA[i] = la[i] != 1 ? sa : 0;
+               fLeadStrideB[i] = lb[i] != 1 ? sb : 0;
+               sa *= la[i];
+               sb *= lb[i];
+            }
+         }
          // offsets (in matrices) of A and B for every stacked product, row-major over the leading dimensions
          for (size_t i = 0; i + 2 < rank; ++i) fStack *= fullY[i];
          for (size_t idx = 0; idx < fStack; ++idx) {
@@ -198,29 +212,35 @@ public:
       const size_t k = fAttrTransA ? fShapeA[0] : fShapeA[1];
       std::stringstream out;
       out << "\n//--------- Gemm\n";
-      std::string offA, offB, offY, indent = SP;
+      const std::string act = fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE";
       if (fStack > 1) {
-         // one product per stacked matrix; the tables hold the matrix index of A and B (broadcast dimensions repeat)
-         const size_t lenA = fShapeA[0] * fShapeA[1], lenB = fShapeB[0] * fShapeB[1];
+         // every product of the stack in one launch: the kernel finds its matrices of A and B from the position
+         // along the leading dimensions (broadcast dimensions have stride 0)
+         if (fLeadY.size() > SOFIE_GEMM_MAX_LEAD_DIMS)
+            throw std::runtime_error("TMVA SOFIE Gemm Op " + fNY + ": more than " + std::to_string(SOFIE_GEMM_MAX_LEAD_DIMS) +
+                                     " stacked dimensions are not supported by the device emission");
          out << SP << "{\n";
-         out << SP << SP << "static const size_t " << opName << "_a[] = {";
-         for (size_t i = 0; i < fStack; ++i) out << (i ? ", " : "") << fStackA[i] * lenA;
+         out << SP << SP << "static const int " << opName << "_lead[] = {";
+         for (size_t i = 0; i < fLeadY.size(); ++i) out << (i ? ", " : "") << fLeadY[i];
          out << "};\n";
-         out << SP << SP << "static const size_t " << opName << "_b[] = {";
-         for (size_t i = 0; i < fStack; ++i) out << (i ? ", " : "") << fStackB[i] * lenB;
+         out << SP << SP << "static const long long " << opName << "_sa[] = {";
+         for (size_t i = 0; i < fLeadY.size(); ++i) out << (i ? ", " : "") << fLeadStrideA[i];
          out << "};\n";
-         out << SP << SP << "for (size_t i = 0; i < " << fStack << "; i++)\n";
-         offA = " + " + opName + "_a[i]";
-         offB = " + " + opName + "_b[i]";
-         offY = " + i * " + std::to_string(m * n);
-         indent = SP + SP + SP;
+         out << SP << SP << "static const long long " << opName << "_sb[] = {";
+         for (size_t i = 0; i < fLeadY.size(); ++i) out << (i ? ", " : "") << fLeadStrideB[i];
+         out << "};\n";
+         out << SP << SP << "Check(sofie_hip_gemm_f32_stacked(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << m
+             << ", " << n << ", " << k << ", " << FloatLiteral(fAttrAlpha) << ", tensor_" << fNA << ", " << fShapeA[1] << ", tensor_"
+             << fNB << ", " << fShapeB[1] << ", tensor_" << fNY << ", " << n << ", " << fLeadY.size() << ", " << opName << "_lead, "
+             << opName << "_sa, " << opName << "_sb, " << act << "), \"Gemm " << opName << "\");\n";
+         out << SP << "}\n";
+         return out.str();
       }
-      out << indent << "Check(sofie_hip_gemm_f32(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << BatchCount(m) << ", "
-          << n << ", " << k << ", " << FloatLiteral(fAttrAlpha) << ", tensor_" << fNA << offA << ", " << fShapeA[1] << ", tensor_" << fNB
-          << offB << ", " << fShapeB[1] << ", " << FloatLiteral(fNC.empty() ? 0.0f : fAttrBeta) << ", "
-          << (fNC.empty() ? std::string("nullptr") : "tensor_" + fNC) << ", " << fBiasKind << ", tensor_" << fNY << offY << ", " << n << ", "
-          << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << "), \"Gemm " << opName << "\");\n";
-      if (fStack > 1) out << SP << "}\n";
+      out << SP << "Check(sofie_hip_gemm_f32(fCtx, " << (fAttrTransA ? 1 : 0) << ", " << (fAttrTransB ? 1 : 0) << ", " << BatchCount(m) << ", "
+          << n << ", " << k << ", " << FloatLiteral(fAttrAlpha) << ", tensor_" << fNA << ", " << fShapeA[1] << ", tensor_" << fNB
+          << ", " << fShapeB[1] << ", " << FloatLiteral(fNC.empty() ? 0.0f : fAttrBeta) << ", "
+          << (fNC.empty() ? std::string("nullptr") : "tensor_" + fNC) << ", " << fBiasKind << ", tensor_" << fNY << ", " << n << ", "
+          << act << "), \"Gemm " << opName << "\");\n";
       return out.str();
    }
 };

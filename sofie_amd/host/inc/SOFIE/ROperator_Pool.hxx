@@ -1,6 +1,8 @@
 // Pooling emitter; interface of the reference's ROperator_Pool<T> (ROperator_Pool.hxx:17-90): a mode,
 // an attribute struct, input and output names. The device emission covers 2-D MaxPool (float NCHW and
-// int8 NCHW), with the reference's output-size rule (floor division, default pads 0, :92-199).
+// int8 in either layout), 2-D AveragePool and GlobalAveragePool (float NCHW; the latter is the average over the
+// whole image, as the reference turns it into at Initialize, :216-228), with the reference's output-size rule
+// (floor division, default pads 0, :92-199).
 #ifndef SOFIE_ROPERATOR_POOL
 #define SOFIE_ROPERATOR_POOL
 
@@ -55,7 +57,11 @@ public:
    const std::vector<size_t> &Strides() const { return fAttr.strides; }
    const std::vector<size_t> &OutputShape() const { return fShapeY; }
    ETensorType TensorType() const { return fType; }
-   std::string Name() { return fPoolMode == MaxPool ? "MaxPool" : fPoolMode == AveragePool ? "AveragePool" : "Invalid"; }
+   std::string Name()
+   {
+      return fPoolMode == MaxPool ? "MaxPool" : fPoolMode == AveragePool ? "AveragePool"
+             : fPoolMode == GlobalAveragePool ? "GlobalAveragePool" : "Invalid";
+   }
    std::vector<ETensorType> TypeInference(std::vector<ETensorType> input) override { return input; }
    std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>> input) override
    {
@@ -63,6 +69,13 @@ public:
       if (input[0].size() != 4)
          throw std::runtime_error("TMVA SOFIE" + Name() + "Op : tensors with dimension " + std::to_string(input[0].size()) +
                                   " are not yet supported");
+      if (fPoolMode == GlobalAveragePool) {
+         // a pooling whose kernel is the image (reference :216-228)
+         fAttr.kernel_shape = {input[0][2], input[0][3]};
+         fAttr.auto_pad = "NOTSET";
+         fAttr.pads = {0, 0, 0, 0};
+         fAttr.strides = {1, 1};
+      }
       if (fAttr.kernel_shape.empty()) fAttr.kernel_shape = {input[0][2], input[0][3]};
       if (fAttr.auto_pad != "NOTSET")
          throw std::runtime_error("TMVA SOFIE" + Name() + "Op : auto_pad is not supported by the device emission");
@@ -81,12 +94,14 @@ public:
    {
       if (!model.CheckIfTensorAlreadyExist(fNX))
          throw std::runtime_error("TMVA SOFIE Pool op Input Tensor " + fNX + " is not found in model");
-      if (fPoolMode != MaxPool)
+      if (fPoolMode != MaxPool && fPoolMode != AveragePool && fPoolMode != GlobalAveragePool)
          throw std::runtime_error("TMVA SOFIE Pool op " + Name() + " is not supported by the device emission");
       fShapeX = model.GetTensorShape(fNX);
       fType = model.GetTensorType(fNX);
       if (fType != ETensorType::FLOAT && fType != ETensorType::INT8)
          throw std::runtime_error("TMVA SOFIE Encountered unsupported type parsing a Pool operator");
+      if (fPoolMode != MaxPool && fType != ETensorType::FLOAT)
+         throw std::runtime_error("TMVA SOFIE Pool op " + Name() + " on a quantized tensor is not supported by the device emission");
       fShapeY = ShapeInference({fShapeX})[0];
       model.AddIntermediateTensor(fNY, fType, fShapeY);
       fChannelsLast = model.IsChannelsLast(fNX);
@@ -100,6 +115,18 @@ public:
       std::stringstream out;
       out << "\n//----  operator " << Name() << "  " << OpName << "\n";
       const auto &a = fAttr;
+      if (fPoolMode != MaxPool) {
+         // a window that lies in the padding entirely has no cell to average
+         if (!a.count_include_pad)
+            for (size_t i = 0; i < 4; ++i)
+               if (a.pads[i] >= a.kernel_shape[i % 2])
+                  throw std::runtime_error("TMVA SOFIE" + Name() + "Op : a pad as large as the kernel leaves windows without a cell of the image");
+         out << SP << "Check(sofie_hip_avgpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0] * fShapeX[1])
+             << ", " << fShapeX[2] << ", " << fShapeX[3] << ", " << a.kernel_shape[0] << ", " << a.kernel_shape[1] << ", " << a.pads[0]
+             << ", " << a.pads[1] << ", " << a.pads[2] << ", " << a.pads[3] << ", " << a.strides[0] << ", " << a.strides[1] << ", "
+             << (a.count_include_pad ? 1 : 0) << "), \"" << Name() << " " << OpName << "\");\n";
+         return out.str();
+      }
       if (fType == ETensorType::FLOAT)
          out << SP << "Check(sofie_hip_maxpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0] * fShapeX[1])
              << ", " << fShapeX[2] << ", " << fShapeX[3];

@@ -697,8 +697,10 @@ void RModel::GenerateSessionCode()
              std::to_string(ConvertShapeToLength(i.second.shape())) + " elements\n";
    }
    // inputs: device staging buffers for the host-pointer infer()
-   for (auto &n : fInputTensorNames)
+   for (auto &n : fInputTensorNames) {
       fGC += ConvertTypeToString(GetTensorType(n)) + " * fInput_" + n + " = nullptr;   // device copy of the input\n";
+      fGC += ConvertTypeToString(GetTensorType(n)) + " * fPinned_" + n + " = nullptr;   // page-locked host buffer, made on request\n";
+   }
    // intermediates: one device arena, offsets from the memory plan
    fGC += "char* fIntermediateMemoryPool = nullptr;   // device, " + std::to_string(fArenaBytes) + " bytes\n";
    for (auto &it : fIntermediateTensorInfos)
@@ -789,10 +791,22 @@ void RModel::GenerateSessionCode()
    for (auto &i : fInitializedTensors)
       if (i.second.IsWeightTensor()) fGC += "   sofie_hip_free(fCtx, tensor_" + i.first + ");\n";
    for (auto &n : fInputTensorNames) fGC += "   sofie_hip_free(fCtx, fInput_" + n + ");\n";
+   for (auto &n : fInputTensorNames) fGC += "   sofie_hip_host_free(fCtx, fPinned_" + n + ");\n";
    fGC += "   sofie_hip_free(fCtx, fIntermediateMemoryPool);\n";
    fGC += "   sofie_hip_destroy(fCtx);\n";
    fGC += "   fCtx.p = nullptr;\n";
    fGC += "}\n";
+   // page-locked host buffers of the inputs' size: a caller that fills them and passes the same pointer to infer()
+   // gets the upload at the rate of the link (pageable memory goes through the driver's staging copy first)
+   for (auto &n : fInputTensorNames) {
+      const std::string t = ConvertTypeToString(GetTensorType(n));
+      const size_t bytes = ConvertShapeToLength(GetTensorShape(n)) * GetTypeSize(GetTensorType(n));
+      fGC += t + "* pinned_input_" + n + "() {\n";
+      fGC += "   if (!fPinned_" + n + ") Check(sofie_hip_host_malloc(fCtx, reinterpret_cast<void**>(&fPinned_" + n + "), " +
+             std::to_string(bytes) + "), \"allocation of a page-locked input buffer\");\n";
+      fGC += "   return fPinned_" + n + ";\n";
+      fGC += "}\n";
+   }
    fGC += "~Session() { Release(); }\n";
    fGC += "Session(const Session&) = delete;\n";
    fGC += "Session& operator=(const Session&) = delete;\n";

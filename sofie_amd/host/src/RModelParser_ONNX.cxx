@@ -337,7 +337,7 @@ std::shared_ptr<void> TensorData(const Tensor &t, ETensorType type, size_t lengt
 
 const std::set<std::string> &Supported()
 {
-   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "BatchNormalization", "Conv", "ConvTranspose", "Einsum", "Relu", "MaxPool", "Flatten", "Reshape",
+   static const std::set<std::string> ops = {"Gemm", "MatMul", "Add", "BatchNormalization", "Conv", "ConvTranspose", "Einsum", "Relu", "MaxPool", "AveragePool", "GlobalAveragePool", "Flatten", "Reshape",
                                              "QuantizeLinear", "DequantizeLinear", "QLinearMatMul", "QLinearConv"};
    return ops;
 }
@@ -674,16 +674,19 @@ RModel RModelParser_ONNX::Parse(std::string filename, bool verbose)
          op.reset(new ROperator_Einsum<float>(equation, n.inputs, n.outputs[0]));
       } else if (t == "Relu") {
          op.reset(new ROperator_Relu<float>(n.inputs.at(0), n.outputs[0]));
-      } else if (t == "MaxPool") {
+      } else if (t == "GlobalAveragePool") {
+         op.reset(new ROperator_Pool<float>(GlobalAveragePool, RAttributes_Pool(), n.inputs.at(0), n.outputs[0]));
+      } else if (t == "MaxPool" || t == "AveragePool") {
          RAttributes_Pool attr;
          attr.auto_pad = n.String("auto_pad", "NOTSET");
          attr.ceil_mode = (int)n.Int("ceil_mode", 0);
+         attr.count_include_pad = (int)n.Int("count_include_pad", 0);
          attr.storage_order = (int)n.Int("storage_order", 0);
          attr.dilations = n.Sizes("dilations");
          attr.kernel_shape = n.Sizes("kernel_shape");
          attr.pads = n.Sizes("pads");
          attr.strides = n.Sizes("strides");
-         op.reset(new ROperator_Pool<float>(MaxPool, attr, n.inputs.at(0), n.outputs[0]));
+         op.reset(new ROperator_Pool<float>(t == "MaxPool" ? MaxPool : AveragePool, attr, n.inputs.at(0), n.outputs[0]));
       } else if (t == "Flatten") {
          op.reset(new ROperator_Reshape(Flatten, (int)n.Int("axis", 1), n.inputs.at(0), "", n.outputs[0]));
       } else if (t == "Reshape") {

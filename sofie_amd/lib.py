@@ -25,6 +25,8 @@ SIGNATURES = {
     "sofie_hip_version": [],
     "sofie_hip_malloc": [_p, C.POINTER(_p), _z],
     "sofie_hip_free": [_p, _p],
+    "sofie_hip_host_malloc": [_p, C.POINTER(_p), _z],
+    "sofie_hip_host_free": [_p, _p],
     "sofie_hip_upload": [_p, _p, _p, _z],
     "sofie_hip_download": [_p, _p, _p, _z],
     "sofie_hip_copy": [_p, _p, _p, _z],
@@ -33,6 +35,8 @@ SIGNATURES = {
     "sofie_hip_timer_start": [_p],
     "sofie_hip_timer_stop": [_p, C.POINTER(_f)],
     "sofie_hip_gemm_f32": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i, _p, _i, _i],
+    "sofie_hip_gemm_f32_stacked": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _p, _i, _i, C.POINTER(_i),
+                                   C.POINTER(C.c_longlong), C.POINTER(C.c_longlong), _i],
     "sofie_hip_conv2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,
     "sofie_hip_conv3d_f32": [_p, _p, _p, _p, _p] + [_i] * 20,
     "sofie_hip_conv_transpose2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,
@@ -44,6 +48,7 @@ SIGNATURES = {
     "sofie_hip_einsum_f32": [_p, _i, C.POINTER(_p), _i, _i, C.POINTER(_i), C.POINTER(C.c_longlong), _p],
     "sofie_hip_relu_f32": [_p, _p, _p, _z],
     "sofie_hip_maxpool2d_f32": [_p, _p, _p] + [_i] * 11,
+    "sofie_hip_avgpool2d_f32": [_p, _p, _p] + [_i] * 12,
     "sofie_hip_quantize_f32_s8": [_p, _p, _p, _z, _f, _i],
     "sofie_hip_dequantize_s8_f32": [_p, _p, _p, _z, _f, _i],
     "sofie_hip_qgemm_s8": [_p, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i],

@@ -326,6 +326,19 @@ def maxpool2d(x, kernel, strides, pads=(0, 0, 0, 0), layout=L.LAYOUT_NCHW, ctx=N
     return ctx.ret(y, x)
 
 
+def avgpool2d(x, kernel, strides, pads=(0, 0, 0, 0), count_include_pad=False, ctx=None):
+    """fp32 NCHW average pooling; pads = (top, left, bottom, right)."""
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.float32)
+    N, Cc, H, W = xd.shape
+    OH = (H + pads[0] + pads[2] - kernel[0]) // strides[0] + 1
+    OW = (W + pads[1] + pads[3] - kernel[1]) // strides[1] + 1
+    y = ctx.empty((N, Cc, OH, OW), torch.float32)
+    ctx.check(ctx.lib.sofie_hip_avgpool2d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(y), N * Cc, H, W, kernel[0], kernel[1], pads[0],
+                                              pads[1], pads[2], pads[3], strides[0], strides[1], int(count_include_pad)))
+    return ctx.ret(y, x)
+
+
 # ------------------------------------------------------------------------------- int8
 def quantize_f32_s8(x, scale, zp=0, ctx=None):
     ctx = ctx or default_context()

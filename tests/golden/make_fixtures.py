@@ -1,5 +1,5 @@
 """Collect the known-answer fixtures that the reference's own tests hold for the
-Gemm / Conv / ConvTranspose / MaxPool path into tests/golden/.
+Gemm / Conv / ConvTranspose / MaxPool / AveragePool path into tests/golden/.
 
 Run in the authoring container only (it reads /root/reference, which does not exist
 on the GPU box):   python tests/golden/make_fixtures.py
@@ -11,7 +11,7 @@ What is written:
                                      <name>.ref.hxx headers (numbers only) together with
                                      the input each test feeds (ones / iota / literal list,
                                      from TestCustomModelsFromONNX.cxx:330-349,372-391,
-                                     693-712,860-967,1023-1052,2047-2152); for the Einsum models
+                                     693-712,860-967,1023-1052,1086-1114,2047-2152); for the Einsum models
                                      the literal inputs and outputs of the tests themselves
                                      (TestCustomModelsFromONNX.cxx:3028-3103)
 """
@@ -35,6 +35,7 @@ CASES = {
     "ConvWithStridesNoPadding": ("iota", [1, 1, 7, 5], "all_ones"),
     "ConvWithAsymmetricPadding": ("iota", [1, 1, 7, 5], "all_ones"),
     "MaxPool2d": ("literal", [1, 1, 5, 10], "output"),
+    "AvgPool": ("literal", [1, 1, 5, 10], "output"),
     "ConvTranspose1d": ("iota", [1, 1, 3], "output"),
     "ConvTranspose2d": ("iota", [1, 1, 3, 3], "output"),
     "ConvTransposeBias2d": ("iota", [1, 1, 3, 3], "output"),
@@ -48,6 +49,16 @@ MAXPOOL2D_INPUT = [
     -0.3421, -1.2364, -0.5805, 0.4421, 1.2184, 0.5043, 1.6823, -1.0483, -2.2798, -1.8927,
     0.7716, 0.0405, 0.3121, -0.3011, -0.3266, -1.9660, 1.0837, 0.2317, 0.9084, -0.3285,
     -0.9398, -0.2065, -0.9499, -0.9739, -0.1288, -0.1375, -1.2612, 0.8810, 0.8506, 0.4455,
+]
+
+
+# Input of the reference's AvgPool test (TestCustomModelsFromONNX.cxx:1090-1101).
+AVGPOOL_INPUT = [
+    0.4764, -0.1976, 1.6506, -0.2421, 0.6412, 1.9985, 0.3938, 0.1347, 0.2204, -0.7503,
+    0.2139, 0.7285, -0.0210, -0.4585, -1.5333, -0.4772, 0.5560, 0.6323, -2.5372, 1.4906,
+    -1.1062, -0.9703, 0.2366, -0.9184, 0.3014, 0.7985, -0.6841, -2.2854, -2.7728, -1.2806,
+    -1.0947, -0.5990, -0.3033, -1.9042, -0.5403, 0.2332, 0.9215, -0.1549, 0.0557, -0.5567,
+    -1.4971, 0.5386, -0.2922, 0.4860, -0.3973, -0.4624, 0.4514, 0.2385, 0.3783, -1.0500,
 ]
 
 
@@ -78,7 +89,7 @@ def main():
             vals = numbers_of(f.read(), arr)
         entry = {"input_kind": kind, "input_shape": shape, "expected": vals}
         if kind == "literal":
-            entry["input"] = MAXPOOL2D_INPUT
+            entry["input"] = AVGPOOL_INPUT if name == "AvgPool" else MAXPOOL2D_INPUT
         expected[name] = entry
     for name, (inputs, answer) in EINSUM_CASES.items():
         shutil.copyfile(os.path.join(REF, name + ".onnx"), os.path.join(HERE, "onnx", name + ".onnx"))

@@ -9,7 +9,7 @@ from sofie_amd import emit, onnx_wire
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 FIXTURES = ["Linear_16", "Linear_32", "Linear_64", "ConvWithPadding", "ConvWithoutPadding",
             "ConvWithAutopadSameLower", "ConvWithStridesPadding", "ConvWithStridesNoPadding",
-            "ConvWithAsymmetricPadding", "MaxPool2d", "ConvTranspose1d", "ConvTranspose2d", "ConvTransposeBias2d",
+            "ConvWithAsymmetricPadding", "MaxPool2d", "AvgPool", "ConvTranspose1d", "ConvTranspose2d", "ConvTransposeBias2d",
             "ConvTransposeBias2dBatched", "Einsum_matmul", "Einsum_dotprod", "Einsum_3", "Einsum_4"]
 
 

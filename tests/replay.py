@@ -91,6 +91,12 @@ def run_graph(graph, feeds, backend):
             y = backend.maxpool2d(env[ins[0]], tuple(a["kernel_shape"]),
                                   tuple(a.get("strides", [1, 1])),
                                   tuple(a.get("pads", [0, 0, 0, 0])))
+        elif op == "AveragePool":
+            y = backend.avgpool2d(env[ins[0]], tuple(a["kernel_shape"]), tuple(a.get("strides", [1, 1])),
+                                  tuple(a.get("pads", [0, 0, 0, 0])), bool(a.get("count_include_pad", 0)))
+        elif op == "GlobalAveragePool":
+            x = env[ins[0]]
+            y = backend.avgpool2d(x, tuple(x.shape[2:]), (1, 1))
         elif op == "Flatten":
             x = env[ins[0]]
             y = np.ascontiguousarray(x).reshape(x.shape[0], -1)

@@ -403,14 +403,16 @@ def test_parametric_batch_dimension_is_fixed_at_generation_time(tmp_path):
 
 
 def test_stacked_matmul_shapes_and_offsets(tmp_path):
-    """Leading dimensions broadcast as in numpy.matmul; the emitted loop indexes A and B per stacked product."""
+    """Leading dimensions broadcast as in numpy.matmul; one launch per stacked operator, with the element strides of A
+    and B along every leading dimension (0 where the operand is broadcast)."""
     hxx, _, _ = models.stacked_spec("stacked_t").generate(str(tmp_path))
     code = open(hxx).read()
-    # x [2,1,4,5] @ B1 [3,5,6]: six products; A advances with the first dimension only, B with the second only
-    assert "_a[] = {0, 0, 0, 20, 20, 20};" in code and "_b[] = {0, 30, 60, 0, 30, 60};" in code
+    # x [2,1,4,5] @ B1 [3,5,6]: leading dimensions (2, 3); A advances with the first only, B with the second only
+    assert "_lead[] = {2, 3};" in code and "_sa[] = {20, 0};" in code and "_sb[] = {0, 30};" in code
     # h [2,3,4,6] @ B2 [6,2]: B is one matrix
-    assert "_a[] = {0, 24, 48, 72, 96, 120};" in code and "_b[] = {0, 0, 0, 0, 0, 0};" in code
-    assert code.count("sofie_hip_gemm_f32(") == 2
+    assert "_sa[] = {72, 24};" in code and "_sb[] = {0, 0};" in code
+    assert code.count("sofie_hip_gemm_f32_stacked(") == 2 and "sofie_hip_gemm_f32(" not in code
+    assert "tensor_x, 5, tensor_B1, 6, tensor_h, 6, 2, " in code
     bad = emit.ModelSpec("bad_stack")
     bad.add_input("x", "FLOAT", (2, 4, 5))
     bad.add_init("B", np.zeros((3, 5, 6), np.float32))

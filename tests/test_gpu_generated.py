@@ -153,6 +153,7 @@ def test_graph_replay_matches_eager(name, make_input, tmp_path):
     _, timing = run_session(name, make_input(), tmp_path, iters=5)
     assert timing["graph_matches"] is True
     assert timing["graph_ms"] > 0
+    assert timing["pinned_matches"] is True and timing["host_pinned_ms"] > 0   # infer() on the page-locked input buffer
 
 
 def test_stacked_matmul_session(tmp_path):

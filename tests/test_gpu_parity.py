@@ -58,7 +58,7 @@ def test_reference_known_answers_through_hip(ops, name):
     assert np.max(np.abs(y.reshape(-1) - want)) <= 1e-3   # the reference's own tolerance
     yo = replay.run_graph(graph, feeds, oracle)
     assert rel_err(y, yo) <= FP32_TOL
-    if name.startswith("Conv") or name.startswith("MaxPool") or name.startswith("Einsum"):
+    if name.startswith("Conv") or name.startswith("MaxPool") or name.startswith("Einsum") or name.startswith("AvgPool"):
         assert np.array_equal(y, yo)
 
 
@@ -952,3 +952,72 @@ def test_capture_rules_are_enforced():
     ctx.sync()
     assert not y2.cpu().numpy().any()
     ctx.close()
+
+
+# --------------------------------------------------------------------------- stacked matrix products
+@pytest.mark.parametrize("sa,sb,tA,tB,relu", [
+    ((2, 1, 4, 5), (3, 5, 6), 0, 0, False),          # both operands broadcast over a leading dimension
+    ((2, 3, 4, 6), (6, 2), 0, 0, True),              # one matrix against a stack
+    ((5, 7, 33), (5, 33, 70), 0, 0, False),
+    ((3, 2, 40, 17), (3, 1, 9, 40), 1, 1, False),    # both stored transposed
+    ((1, 130, 65), (4, 2, 65, 131), 0, 0, True),     # tiles of 128 x 128, ragged
+])
+def test_gemm_f32_stacked_is_numpy_matmul(sa, sb, tA, tB, relu):
+    """sofie_hip_gemm_f32_stacked against numpy.matmul in float64 (every product reads its own matrices, broadcast
+    dimensions repeat) and against the single-product entry point, which it must equal bit for bit."""
+    import ctypes as C
+    from sofie_amd import lib as L
+    from sofie_amd import ops as o
+    ctx = o.default_context()
+    r = rng(900 + sum(sa) + sum(sb))
+    A = r.standard_normal(sa).astype(np.float32)
+    B = r.standard_normal(sb).astype(np.float32)
+    a64 = np.swapaxes(A, -1, -2).astype(np.float64) if tA else A.astype(np.float64)
+    b64 = np.swapaxes(B, -1, -2).astype(np.float64) if tB else B.astype(np.float64)
+    truth = np.matmul(a64, b64)
+    if relu:
+        truth = np.maximum(truth, 0)
+    lead = truth.shape[:-2]
+    M, N = truth.shape[-2:]
+    K = a64.shape[-1]
+    la = (1,) * (len(lead) - (A.ndim - 2)) + A.shape[:-2]
+    lb = (1,) * (len(lead) - (B.ndim - 2)) + B.shape[:-2]
+
+    def strides(l, mat):
+        out, s = [0] * len(l), mat
+        for i in reversed(range(len(l))):
+            out[i] = s if l[i] != 1 else 0
+            s *= l[i]
+        return out
+    st_a, st_b = strides(la, A.shape[-2] * A.shape[-1]), strides(lb, B.shape[-2] * B.shape[-1])
+    dA, dB = ctx.dev(A), ctx.dev(B)
+    y = ctx.empty(truth.shape, torch.float32)
+    n = len(lead)
+    ctx.check(ctx.lib.sofie_hip_gemm_f32_stacked(ctx.h, tA, tB, M, N, K, 1.0, ctx.ptr(dA), A.shape[-1], ctx.ptr(dB), B.shape[-1],
+                                                 ctx.ptr(y), N, n, (C.c_int * n)(*lead), (C.c_longlong * n)(*st_a),
+                                                 (C.c_longlong * n)(*st_b), L.ACT_RELU if relu else L.ACT_NONE))
+    got = ctx.ret(y, A)
+    assert rel_err(got, truth) <= FP32_TOL
+    # the same products one at a time
+    Af = np.broadcast_to(A.reshape(la + A.shape[-2:]), lead + A.shape[-2:]).reshape((-1,) + A.shape[-2:])
+    Bf = np.broadcast_to(B.reshape(lb + B.shape[-2:]), lead + B.shape[-2:]).reshape((-1,) + B.shape[-2:])
+    for i in range(0, Af.shape[0], max(1, Af.shape[0] // 3)):
+        one = o.gemm_f32(np.ascontiguousarray(Af[i]), np.ascontiguousarray(Bf[i]), None, 1.0, 0.0, bool(tA), bool(tB), relu)
+        assert np.array_equal(one, got.reshape((-1, M, N))[i])
+
+
+# --------------------------------------------------------------------------- fp32 average pooling
+@pytest.mark.parametrize("cfg", [
+    dict(shape=(2, 3, 9, 8), k=(3, 2), s=(2, 1), p=(0, 0, 0, 0)),
+    dict(shape=(1, 4, 7, 7), k=(3, 3), s=(1, 1), p=(1, 1, 1, 1)),
+    dict(shape=(2, 2, 10, 11), k=(2, 4), s=(2, 3), p=(1, 2, 1, 0)),
+    dict(shape=(3, 130, 6, 6), k=(6, 6), s=(1, 1), p=(0, 0, 0, 0)),      # the global average of many planes
+    dict(shape=(1, 1, 40, 300), k=(5, 7), s=(3, 4), p=(2, 3, 2, 3)),
+])
+def test_avgpool2d_f32(ops, cfg):
+    """Same order of additions and one division as the oracle's restatement of the reference's loops: identical bits."""
+    r = rng(1000 + cfg["shape"][1])
+    x = r.standard_normal(cfg["shape"]).astype(np.float32)
+    for include in (False, True):
+        y = ops.avgpool2d(x, cfg["k"], cfg["s"], cfg["p"], include)
+        assert np.array_equal(y, oracle.avgpool2d(x, cfg["k"], cfg["s"], cfg["p"], include))

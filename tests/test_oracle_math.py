@@ -553,3 +553,32 @@ def test_cpu_baseline_program_computes_what_the_oracle_computes(tmp_path):
         x, w, b, y = np.split(raw, np.cumsum(sizes)[:-1])
         ref = oracle.conv2d_f32(x.reshape(2, 64, 56, 56), w.reshape(128, 64, 3, 3), b, (1, 1), relu=True)
         assert np.max(np.abs(y.reshape(ref.shape) - ref)) <= 1e-5 * np.max(np.abs(ref))
+
+
+# ----------------------------------------------------------------------------- fp32 average pooling
+@pytest.mark.parametrize("cfg", [
+    dict(shape=(2, 3, 9, 8), k=(3, 2), s=(2, 1), p=(0, 0, 0, 0)),
+    dict(shape=(1, 4, 7, 7), k=(3, 3), s=(1, 1), p=(1, 1, 1, 1)),
+    dict(shape=(2, 2, 10, 11), k=(2, 4), s=(2, 3), p=(1, 2, 1, 2)),
+    dict(shape=(3, 5, 6, 6), k=(6, 6), s=(1, 1), p=(0, 0, 0, 0)),      # the global average
+])
+def test_avgpool2d_against_torch_and_float64(cfg):
+    """or_avgpool2d_f32 against torch's avg_pool2d on CPU with count_include_pad off and on (symmetric pads, which
+    is what torch takes) and against a float64 mean of the cells inside the image."""
+    r = rng(300 + cfg["shape"][2])
+    x = r.standard_normal(cfg["shape"]).astype(np.float32)
+    pt, pl, pb, pr = cfg["p"]
+    for include in (False, True):
+        y = oracle.avgpool2d(x, cfg["k"], cfg["s"], cfg["p"], include)
+        t = F.avg_pool2d(torch.from_numpy(x).double(), cfg["k"], cfg["s"], (pt, pl), ceil_mode=False,
+                         count_include_pad=include).numpy()
+        assert y.shape == t.shape
+        assert np.max(np.abs(y - t)) <= 1e-6 * max(np.max(np.abs(t)), 1.0)
+    # brute force in float64 on one plane: mean over the cells inside the image
+    y = oracle.avgpool2d(x, cfg["k"], cfg["s"], cfg["p"], False)
+    H, W = cfg["shape"][2:]
+    for oh in range(y.shape[2]):
+        for ow in range(y.shape[3]):
+            r0, c0 = oh * cfg["s"][0] - pt, ow * cfg["s"][1] - pl
+            win = x[0, 0, max(r0, 0):min(r0 + cfg["k"][0], H), max(c0, 0):min(c0 + cfg["k"][1], W)].astype(np.float64)
+            assert abs(y[0, 0, oh, ow] - win.mean()) <= 1e-6 * max(1.0, abs(win.mean()))
