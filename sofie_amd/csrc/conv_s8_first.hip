@@ -97,7 +97,10 @@ __device__ __forceinline__ unsigned quantize4(v4f v, float scale, float inv, int
 }
 
 template <bool POOL>
-__global__ void __launch_bounds__(256, 3) k_qconv_first(FirstArgs a)
+// Four workgroups per CU (at most 128 registers): the loop is a chain of dependent vector instructions per group of
+// pixels, and a fourth wavefront per SIMD fills the gaps the other three leave (25.4 us instead of 30.8 us for 4096
+// images of 40x40 with 32 channels and pooling; five workgroups need 102 registers and lose more than they gain).
+__global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
 {
    extern __shared__ __align__(16) unsigned char smem[];
    const int OCP = a.ocb * 32;                                              // channels padded to blocks of 32
@@ -323,15 +326,15 @@ int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.drows = make_fastdiv((unsigned)a.rows);
    a.dper_image = make_fastdiv((unsigned)(g.PH * g.PW));
    a.dPW = make_fastdiv((unsigned)g.PW);
-   // Images per workgroup: three workgroups share a CU, and the kernel is as slow as the busiest CU, so the
+   // Images per workgroup: four workgroups share a CU, and the kernel is as slow as the busiest CU, so the
    // count is the one that leaves the fewest image-times on a workgroup slot (rounds of workgroups x images each);
-   // of equal ones the larger (fewer parameter loads). At most 16 images and 48 KB of them.
+   // of equal ones the larger (fewer parameter loads). At most 16 images and 36 KB of them.
    const size_t fixed = (size_t)a.ocb * 32 * 24 + 16 + 16;
-   const int slots = 3 * (ctx->num_cus > 0 ? ctx->num_cus : 256);
+   const int slots = 4 * (ctx->num_cus > 0 ? ctx->num_cus : 256);
    int best = 0;
    long best_cost = 0;
    for (int k = 1; k <= 16; ++k) {
-      if (fixed + (size_t)k * a.img_bytes > 48 * 1024) break;
+      if (fixed + (size_t)k * a.img_bytes > 36 * 1024) break;
       const long wgs = (g.N + k - 1) / k;
       const long cost = ((wgs + slots - 1) / slots) * k;
       if (best == 0 || cost <= best_cost) { best = k; best_cost = cost; }
