@@ -251,8 +251,8 @@ QGEMM_SHAPES = [
     (64, 64, 64, True), (64, 64, 64, False),
     (100, 72, 48, True), (100, 72, 48, False),          # ragged tiles, 128-tile kernel
     (300, 520, 272, True), (300, 520, 272, False),
-    (512, 2048, 512, True), (512, 2048, 512, False),    # 256-tile kernel
-    (777, 1028, 1040, True), (777, 1028, 1040, False),  # 256-tile kernel, ragged
+    (512, 2048, 512, True), (512, 2048, 512, False),    # 128 x 128 tiles (the 256 x 256 kernel starts at M * N >= 2^23:
+    (777, 1028, 1040, True), (777, 1028, 1040, False),  # test_qgemm_s8_large_b_as_k_by_n covers it), ragged
     (33, 47, 50, True), (33, 47, 50, False),            # K % 16 != 0: simple kernel
     (4096, 5, 256, True), (1, 16, 16, True),             # at most 16 columns: the dot-product kernel
     (70, 13, 1040, True), (5, 1, 32, True), (300, 9, 48, True),
