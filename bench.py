@@ -435,16 +435,20 @@ def workloads(ctx, torch, L, rng):
          "ops": fl, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 20,
          "bytes": 4.0 * (x.numel() + y.numel() + wt.numel() + 128)})
     # int8 conv layer of the same shape, channels-last, weights [OC][KH][KW][C], bias + ReLU + requantise fused
-    xq = torch.randint(-128, 128, (256, 56, 56, 64), dtype=torch.int8, device=ctx.device)
-    wq = torch.randint(-127, 128, (128, 3, 3, 64), dtype=torch.int8, device=ctx.device)
-    sq = torch.full((128,), 2.0e-4, device=ctx.device)
-    bq = torch.randint(-1000, 1000, (128,), dtype=torch.int32, device=ctx.device)
+    # activations uniform [0,1] quantised with scale 1/255 (zero-point -128); weights Kaiming-normal, symmetric int8 per
+    # output channel; the output scale puts the layer's range (about 0..4) on the 8 bits
+    xq = (torch.round(torch.rand(256, 56, 56, 64, device=ctx.device) * 255.0) - 128.0).to(torch.int8)
+    wf = torch.randn(128, 3, 3, 64, device=ctx.device) * (2.0 / 576) ** 0.5
+    sw = wf.abs().amax(dim=(1, 2, 3)) / 127.0
+    wq = torch.clamp(torch.round(wf / sw.view(-1, 1, 1, 1)), -127, 127).to(torch.int8)
+    sq = (sw * (1.0 / 255.0) / (4.0 / 255.0)).float().contiguous()
+    bq = torch.round(torch.randn(128, device=ctx.device) * 0.1 / (sw * (1.0 / 255.0))).to(torch.int32)
     yq = ctx.empty((256, 56, 56, 128), torch.int8)
     w["conv_s8"] = (lambda: ctx.check(ctx.lib.sofie_hip_qconv2d_s8(
         ctx.h, ctx.ptr(xq), L.LAYOUT_NHWC, ctx.ptr(wq), L.LAYOUT_NHWC, ctx.ptr(bq), ctx.ptr(sq), ctx.ptr(yq), L.LAYOUT_NHWC,
         256, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, 1, 1, -128, -128, L.ACT_RELU, L.OUT_S8)),
         {"workload": "int8 QLinearConv channels-last batch 256, 64 -> 128 channels, 56x56, 3x3, stride 1, pad 1, bias + ReLU "
-                     "+ requantise fused", "ops": fl, "rate_unit": "tops", "peak": PEAK_INT8_TOPS, "launches": 200,
+                     "+ requantise fused; activations U[0,1] at scale 1/255, Kaiming-normal weights symmetric int8 per channel", "ops": fl, "rate_unit": "tops", "peak": PEAK_INT8_TOPS, "launches": 200,
          "bytes": float(xq.numel() + yq.numel() + wq.numel() + 128 * 8)})
     # fp32 transposed conv (an upsampling layer): batch 64, 128 -> 64 channels, 28x28 -> 56x56, 4x4, stride 2, pad 1
     xt = torch.rand(64, 128, 28, 28, device=ctx.device)
