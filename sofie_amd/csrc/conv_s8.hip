@@ -428,10 +428,13 @@ __global__ void __launch_bounds__(512) k_qconv_mfma(QConvTileArgs a)
 
    // One tile per iteration. The two wavefronts that share a SIMD do their halves in opposite order
    // (wavefronts 0-3: matrix loop of tile t, then its epilogue; wavefronts 4-7: epilogue of their previous
-   // tile, then the matrix loop of tile t), which staggers their LDS and global-memory phases. It does not
-   // buy arithmetic overlap: on this hardware the vector instructions of one wavefront do not issue while
-   // the matrix instructions of the other wavefront of the same SIMD execute, so a tile costs the sum of
-   // both (measured with a two-wavefront microbenchmark: 129 us + 106 us apart, 231 us together).
+   // tile, then the matrix loop of tile t), which staggers their LDS and global-memory phases and lets one
+   // wavefront's requantisation run beside the other's matrix instructions. That overlap is partial: the counters of
+   // the 56x56 layer show vector instructions executing in 40 % of the matrix pipe's busy cycles, and a tile takes
+   // about 8000 cycles for 2 x 2304 cycles of matrix instructions per SIMD. A tile is one long chain of instructions
+   // per wavefront (about 810, of which 72 are matrix instructions); variants with two band buffers and one barrier
+   // per tile, with the band rows' address arithmetic on the scalar unit or in LDS tables, and with three wavefronts
+   // per SIMD were all measured and none was faster.
    const bool mma_first = wave < 4;
    int t = wg, t_prev = -1;
    Band cur = {0, 0};
