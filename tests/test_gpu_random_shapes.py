@@ -1,0 +1,225 @@
+"""Seeded sweeps over random geometries: the HIP entry points against the oracle on shapes nobody picked by hand
+(odd extents, unequal begin / end pads, strides, kernels up to 5x5, bands that cross image borders, ragged GEMM
+tiles, K tails). Every output buffer sits between sentinel bands (sofie_amd.ops.Context), so a store past the edge
+of a ragged tile fails the case that made it. Sizes are small enough for the C oracle to finish in seconds."""
+import numpy as np
+import pytest
+
+from oracle import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from sofie_amd import ops as o
+    return o
+
+
+def _conv_geometry(r, max_hw, kmax=5):
+    kh, kw = int(r.integers(1, kmax + 1)), int(r.integers(1, kmax + 1))
+    sh, sw = int(r.integers(1, 4)), int(r.integers(1, 4))
+    pads = tuple(int(v) for v in (r.integers(0, kh), r.integers(0, kw), r.integers(0, kh), r.integers(0, kw)))
+    H = int(r.integers(max(1, kh - pads[0] - pads[2]), max_hw + 1))
+    W = int(r.integers(max(1, kw - pads[1] - pads[3]), max_hw + 1))
+    return (kh, kw), (sh, sw), pads, H, W
+
+
+def _out_hw(H, W, k, s, p):
+    return (H + p[0] + p[2] - k[0]) // s[0] + 1, (W + p[1] + p[3] - k[1]) // s[1] + 1
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_qconv2d_s8_matrix_core_shapes(ops, seed):
+    """Channels-last operands with C % 32 == 0 and OC % 64 == 0: the matrix-core kernel (3x3 on 32 / 64 channels takes
+    its unrolled form), or whatever the library falls back to when a band does not fit."""
+    from sofie_amd import lib as L
+    r = np.random.default_rng(9000 + seed)
+    C = int(r.choice([32, 64, 96]))
+    OC = int(r.choice([64, 128, 192]))
+    if seed % 3 == 0:
+        k, s, p = (3, 3), (1, 1), tuple(int(v) for v in r.integers(0, 3, 4))
+        H, W = int(r.integers(3, 24)), int(r.integers(3, 24))
+    else:
+        k, s, p, H, W = _conv_geometry(r, 20)
+    OH, OW = _out_hw(H, W, k, s, p)
+    if OH < 1 or OW < 1:
+        pytest.skip("empty output")
+    N = int(r.integers(1, 9))
+    x = r.integers(-128, 128, (N, H, W, C)).astype(np.int8)
+    w = r.integers(-127, 128, (OC, C) + k).astype(np.int8)
+    Kd = C * k[0] * k[1]
+    scale = (r.uniform(20, 60, OC) / (73.3 * 73.3 * np.sqrt(Kd))).astype(np.float32)
+    if seed % 5 == 0:
+        scale[::7] *= -1.0
+    bias = r.integers(-3000, 3000, OC).astype(np.int32)
+    zpx, zpy, relu = int(r.choice([-128, 0, 5])), int(r.choice([-128, 3])), bool(r.integers(0, 2))
+    ref = oracle.qconv2d_s8(x.transpose(0, 3, 1, 2), w, scale, bias, p, s, 1, zpx, zpy, relu)
+    wh = np.ascontiguousarray(w.transpose(0, 2, 3, 1))
+    y = ops.qconv2d_s8(x, wh, scale, bias, p, s, 1, zpx, zpy, relu, x_layout=L.LAYOUT_NHWC, y_layout=L.LAYOUT_NHWC,
+                       w_layout=L.LAYOUT_NHWC)
+    assert np.array_equal(y.transpose(0, 3, 1, 2), ref), (C, OC, k, s, p, H, W, N)
+    if OH >= 2 and OW >= 2:
+        pooled = oracle.maxpool2d(ref, (2, 2), (2, 2))
+        yp = ops.qconv2d_pool_s8(x, wh, scale, bias, p, s, 1, zpx, zpy, relu, x_layout=L.LAYOUT_NHWC,
+                                 y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+        assert np.array_equal(yp.transpose(0, 3, 1, 2), pooled), (C, OC, k, s, p, H, W, N, "pooled")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_qconv2d_s8_any_shape(ops, seed):
+    """NCHW operands, any channel count and group count: the one-thread-per-output kernel and, for one input channel
+    with a 3x3 kernel and pads of one, the first-layer kernel (with and without the fused quantisation)."""
+    r = np.random.default_rng(9100 + seed)
+    first = seed % 4 == 0
+    if first:
+        g, C, OC = 1, 1, int(r.choice([16, 32, 48]))
+        k, s, p = (3, 3), (1, 1), (1, 1, 1, 1)
+        H, W = int(r.integers(4, 30)), int(r.integers(4, 30))
+    else:
+        g = int(r.choice([1, 2, 3]))
+        C, OC = g * int(r.integers(1, 6)), g * int(r.integers(1, 9))
+        k, s, p, H, W = _conv_geometry(r, 14)
+    OH, OW = _out_hw(H, W, k, s, p)
+    if OH < 1 or OW < 1:
+        pytest.skip("empty output")
+    N = int(r.integers(1, 6))
+    x = r.integers(-128, 128, (N, C, H, W)).astype(np.int8)
+    w = r.integers(-127, 128, (OC, C // g) + k).astype(np.int8)
+    Kd = C // g * k[0] * k[1]
+    scale = (r.uniform(20, 60, OC) / (73.3 * 73.3 * np.sqrt(Kd))).astype(np.float32)
+    bias = r.integers(-500, 500, OC).astype(np.int32)
+    zpx, zpy, relu = int(r.choice([-128, 0, -7])), int(r.choice([-128, 0, 9])), bool(r.integers(0, 2))
+    ref = oracle.qconv2d_s8(x, w, scale, bias, p, s, g, zpx, zpy, relu)
+    assert np.array_equal(ops.qconv2d_s8(x, w, scale, bias, p, s, g, zpx, zpy, relu), ref), (C, OC, g, k, s, p, H, W, N)
+    if first:
+        xs = np.float32(1.0 / 255.0)
+        xf = r.uniform(0.0, 1.0, (N, 1, H, W)).astype(np.float32)
+        xq = oracle.quantize_f32_s8(xf, xs, -128)
+        ref_q = oracle.qconv2d_s8(xq, w, scale, bias, p, s, 1, -128, zpy, relu)
+        got = ops.quantize_qconv2d_s8(xf, xs, -128, w, scale, bias, p, s, 1, zpy, relu)
+        assert np.array_equal(got, ref_q)
+        if OH >= 2 and OW >= 2:
+            got = ops.quantize_qconv2d_s8(xf, xs, -128, w, scale, bias, p, s, 1, zpy, relu, pool=(2, 2))
+            assert np.array_equal(got, oracle.maxpool2d(ref_q, (2, 2), (2, 2)))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_qgemm_s8_random_shapes(ops, seed):
+    r = np.random.default_rng(9200 + seed)
+    M, N = int(r.integers(1, 700)), int(r.integers(1, 700))
+    K = int(r.integers(1, 1200)) if seed % 2 else 16 * int(r.integers(1, 80))
+    if seed % 6 == 0:
+        N = int(r.integers(1, 17))                    # the dot-product kernel
+    if seed % 8 == 1:
+        M, N, K = 128 * int(r.integers(1, 4)), 128 * int(r.integers(1, 3)), 8192 + 16 * int(r.integers(0, 40))   # K slices
+    transB = bool(r.integers(0, 2))
+    A = r.integers(-128, 128, (M, K)).astype(np.int8)
+    B = r.integers(-127, 128, (N, K) if transB else (K, N)).astype(np.int8)
+    scale = (r.uniform(20, 60, N) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    bias = r.integers(-2000, 2000, N).astype(np.int32) if seed % 3 else None
+    zpa, zpy, relu = int(r.choice([0, -128, 11])), int(r.choice([0, -128, -3])), bool(r.integers(0, 2))
+    ref = oracle.qgemm_s8(A, B, scale, bias, transB, zpa, zpy, relu)
+    got = ops.qgemm_s8(A, B, scale, bias, transB, zpa, zpy, relu)
+    assert np.array_equal(got, ref), (M, N, K, transB, zpa, zpy, relu)
+    assert np.array_equal(ops.igemm_s8(A, B, transB), oracle.igemm_s8(A, B, transB))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_conv2d_f32_random_shapes(ops, seed):
+    r = np.random.default_rng(9300 + seed)
+    g = int(r.choice([1, 1, 2, 4]))
+    C, OC = g * int(r.integers(1, 9)), g * int(r.integers(1, 12))
+    k, s, p, H, W = _conv_geometry(r, 18, kmax=4)
+    d = (int(r.integers(1, 3)), int(r.integers(1, 3)))
+    ke = ((k[0] - 1) * d[0] + 1, (k[1] - 1) * d[1] + 1)
+    H, W = max(H, ke[0]), max(W, ke[1])
+    N = int(r.integers(1, 5))
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((OC, C // g) + k) / np.sqrt(C // g * k[0] * k[1])).astype(np.float32)
+    b = r.standard_normal(OC).astype(np.float32) if seed % 2 else None
+    relu = bool(r.integers(0, 2))
+    ref = oracle.conv2d_f32(x, w, b, p, s, d, g, relu)
+    got = ops.conv2d_f32(x, w, b, p, s, d, g, relu)
+    assert got.shape == ref.shape
+    assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (C, OC, g, k, s, p, d, H, W, N)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_pooling_random_shapes(ops, seed):
+    r = np.random.default_rng(9400 + seed)
+    k, s, p, H, W = _conv_geometry(r, 17, kmax=4)
+    p = tuple(min(v, (k[i % 2] - 1) // 2) for i, v in enumerate(p))      # ONNX: a pad is smaller than the kernel
+    H, W = max(H, k[0]), max(W, k[1])
+    x = r.standard_normal((int(r.integers(1, 4)), int(r.integers(1, 7)), H, W)).astype(np.float32)
+    assert np.array_equal(ops.maxpool2d(x, k, s, p), oracle.maxpool2d(x, k, s, p))
+    for cip in (False, True):
+        ref = oracle.avgpool2d(x, k, s, p, cip)
+        got = ops.avgpool2d(x, k, s, p, cip)
+        assert np.max(np.abs(got - ref)) <= 1e-6 * max(1.0, float(np.max(np.abs(ref))))
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_gemm_f32_random_shapes(ops, seed):
+    r = np.random.default_rng(9500 + seed)
+    M, N, K = int(r.integers(1, 400)), int(r.integers(1, 400)), int(r.integers(1, 500))
+    tA, tB = bool(r.integers(0, 2)), bool(r.integers(0, 2))
+    A = r.standard_normal((K, M) if tA else (M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    bias = [None, r.standard_normal(N).astype(np.float32), r.standard_normal((M, N)).astype(np.float32)][seed % 3]
+    alpha, beta, relu = float(r.choice([1.0, 0.5, -2.0])), float(r.choice([1.0, 0.25])), bool(r.integers(0, 2))
+    if bias is None:
+        beta = 0.0            # the reference refuses a non-zero beta without a bias tensor
+    ref = oracle.gemm_f32(A, B, bias, alpha, beta, tA, tB, relu)
+    got = ops.gemm_f32(A, B, bias, alpha, beta, tA, tB, relu)
+    assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (M, N, K, tA, tB)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_conv_transpose2d_f32_random_shapes(ops, seed):
+    r = np.random.default_rng(9600 + seed)
+    g = int(r.choice([1, 1, 2]))
+    C, OC = g * int(r.integers(1, 7)), g * int(r.integers(1, 7))
+    k = (int(r.integers(1, 5)), int(r.integers(1, 5)))
+    s = (int(r.integers(1, 4)), int(r.integers(1, 4)))
+    d = (int(r.integers(1, 3)), int(r.integers(1, 3)))
+    H, W = int(r.integers(1, 12)), int(r.integers(1, 12))
+    p = tuple(int(v) for v in (r.integers(0, 2), r.integers(0, 2), r.integers(0, 2), r.integers(0, 2)))
+    op = (int(r.integers(0, s[0])), int(r.integers(0, s[1])))
+    OH = s[0] * (H - 1) + d[0] * (k[0] - 1) + 1 + op[0] - p[0] - p[2]
+    OW = s[1] * (W - 1) + d[1] * (k[1] - 1) + 1 + op[1] - p[1] - p[3]
+    if OH < 1 or OW < 1:
+        pytest.skip("empty output")
+    N = int(r.integers(1, 4))
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = r.standard_normal((C, OC // g) + k).astype(np.float32)
+    b = r.standard_normal(OC).astype(np.float32) if seed % 2 else None
+    ref = oracle.conv_transpose2d_f32(x, w, b, p, s, d, g, op)
+    got = ops.conv_transpose2d_f32(x, w, b, p, s, d, g, op)
+    assert got.shape == ref.shape
+    assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (C, OC, g, k, s, d, p, op, H, W)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_gemm_fp8_random_shapes(ops, seed):
+    """The tolerance of the FP8 GEMM (one bf16 rounding of the result plus 2^-15 of the sum of magnitudes, against
+    the float64-accumulated product of the same e4m3 operands) on random shapes and both layouts of B."""
+    from sofie_amd import lib as L
+    r = np.random.default_rng(9700 + seed)
+    M, N = int(r.integers(1, 500)), 4 * int(r.integers(1, 120))
+    K = 16 * int(r.integers(1, 70))
+    transB = bool(r.integers(0, 2))
+    a = r.standard_normal((M, K)).astype(np.float32)
+    b = r.standard_normal((N, K) if transB else (K, N)).astype(np.float32)
+    sa, sb = np.float32(np.abs(a).max() / 448.0), np.float32(np.abs(b).max() / 448.0)
+    A, B = oracle.e4m3_encode(a / sa), oracle.e4m3_encode(b / sb)
+    bias = r.standard_normal(N).astype(np.float32)
+    yf = ops.gemm_fp8(A, B, sa, sb, bias, transB, out=L.OUT_F32)
+    yb = ops.gemm_fp8(A, B, sa, sb, bias, transB)
+    _, truth = oracle.gemm_fp8(A, B, sa, sb, bias, transB, acc64=True)
+    da = np.abs(oracle.e4m3_decode(A)).astype(np.float64)
+    db = np.abs(oracle.e4m3_decode(B)).astype(np.float64)
+    slack = 2.0 ** -15 * (da @ (db.T if transB else db)) * float(sa) * float(sb) + 1e-30
+    assert np.all(np.abs(yf.astype(np.float64) - truth) <= slack + 2.0 ** -22 * np.abs(truth)), (M, N, K, transB)
+    assert np.all(np.abs(oracle.bf16_decode(yb).astype(np.float64) - truth) <= 2.0 ** -8 * np.abs(truth) + slack)
+    assert np.array_equal(yb, oracle.bf16_encode(yf))
