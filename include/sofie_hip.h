@@ -129,6 +129,21 @@ int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, int M, int N,
                        float beta, const float *bias, int bias_kind, float *Y, int ldy,
                        int act);
 
+/* A chain of fully connected layers in one launch:
+ *   a_0 = x [M, dims[0]];  a_l = act_l(a_{l-1} * W_l + bias_l), l = 1..n_layers;  y = a_{n_layers} [M, dims[n_layers]]
+ * W[l-1] is [dims[l-1], dims[l]] row-major (the operand B of a Gemm with transB = 0), bias[l-1] one row of dims[l]
+ * values or NULL (bias itself may be NULL), act[l-1] SOFIE_ACT_NONE or SOFIE_ACT_RELU. Replaces n_layers times the
+ * sequence the reference emits per Gemm (ROperator_Gemm.hxx:292-390: bias copy, BLAS::sgemm_, ReLU loop) when every
+ * layer is small (widths up to SOFIE_MLP_MAX_WIDTH): the intermediate activations never leave the chip and the
+ * chain costs one launch. The emitter joins Gemm operators into such a call when each one's output feeds only the
+ * next (RModel::FuseGemmChain). Sums are fp32 fused multiply-adds over k in increasing order within a part of K;
+ * the result agrees with the separate calls to the usual 1e-5 relative tolerance, not bit for bit. */
+#define SOFIE_MLP_MAX_LAYERS 16
+#define SOFIE_MLP_MAX_WIDTH 1024
+int sofie_hip_mlp_f32(sofie_hip_ctx *ctx, int n_layers, const int *dims, const float *const *W,
+                      const float *const *bias, const int *act, const float *x, int ldx, float *y, int ldy,
+                      int M);
+
 /* Stacked matrix products (numpy.matmul on operands of rank > 2) in one launch:
  *   Y[i] = alpha * op(A[ia(i)]) * op(B[ib(i)]), optional ReLU, for every index i of the n_lead leading dimensions
  * lead[0..n_lead) (row-major, last dimension fastest). stride_a[d] / stride_b[d] are the element strides of A / B

@@ -230,3 +230,144 @@ extern "C" int sofie_hip_gemm_f32_stacked(sofie_hip_ctx *ctx, int transA, int tr
    }
    return SOFIE_HIP_OK;
 }
+
+// ------------------------------------------------------------------------------------------------------------
+// A chain of small fully connected layers in one launch: y = act_L(... act_1(x W_1 + b_1) ... W_L + b_L).
+// A multilayer perceptron on a few hundred rows is three kernel launches of a few microseconds each and nothing
+// else: the matrix cores have nothing to chew on (8.65 MFLOP for 256 rows of 64 -> 128 -> 64 -> 8) and the time
+// is the launches. Here a workgroup carries R rows through every layer with the activations in LDS; the weights
+// (W_l [K_l, N_l], row-major) come straight from L2, one coalesced row of N_l per step of k. With N_l below the
+// 256 threads of the workgroup the threads also split K: thread (o, part) sums its share of k for output o, the
+// partial sums meet in LDS. Plain fp32 fused multiply-adds in a fixed order per output; no matrix instructions.
+namespace {
+
+struct MlpArgs {
+   const float *W[SOFIE_MLP_MAX_LAYERS];
+   const float *bias[SOFIE_MLP_MAX_LAYERS];
+   int dims[SOFIE_MLP_MAX_LAYERS + 1];
+   int relu[SOFIE_MLP_MAX_LAYERS];
+   const float *x;
+   float *y;
+   int n_layers, M, ldx, ldy, maxd;
+};
+
+template <int R>
+__global__ void __launch_bounds__(256) k_mlp_f32(MlpArgs a)
+{
+   extern __shared__ __align__(16) float s_mlp[];
+   float *buf_in = s_mlp, *buf_out = s_mlp + R * a.maxd;     // activations of the rows, [R][maxd] each
+   float *part = s_mlp + 2 * R * a.maxd;                     // [256][R] partial sums
+   const int tid = threadIdx.x;
+   const int row0 = blockIdx.x * R;
+   {
+      const int K0 = a.dims[0];
+      for (int idx = tid; idx < R * K0; idx += 256) {
+         const int r = idx / K0, k = idx - r * K0;
+         buf_in[r * a.maxd + k] = row0 + r < a.M ? a.x[(size_t)(row0 + r) * a.ldx + k] : 0.0f;
+      }
+   }
+   __syncthreads();
+   for (int l = 0; l < a.n_layers; ++l) {
+      const int K = a.dims[l], N = a.dims[l + 1];
+      const float *__restrict__ W = a.W[l];
+      const bool last = l + 1 == a.n_layers;
+      // columns per pass (a power of two, at most 256) and the parts K is cut into
+      int n2 = 1;
+      while (n2 < N && n2 < 256) n2 <<= 1;
+      const int parts = 256 / n2;
+      const int kc = (K + parts - 1) / parts;
+      const int oc = tid & (n2 - 1), pt = tid / n2;
+      const int k0 = pt * kc, k1 = k0 + kc < K ? k0 + kc : K;
+      for (int o0 = 0; o0 < N; o0 += n2) {
+         const int o = o0 + oc;
+         float acc[R];
+#pragma unroll
+         for (int r = 0; r < R; ++r) acc[r] = 0.0f;
+         if (o < N) {
+            const float *w = W + (size_t)k0 * N + o;
+#pragma unroll 8
+            for (int k = k0; k < k1; ++k) {
+               const float wv = *w;
+               w += N;
+#pragma unroll
+               for (int r = 0; r < R; ++r) acc[r] = fmaf(buf_in[r * a.maxd + k], wv, acc[r]);
+            }
+         }
+         auto finish = [&](int r, int oo, float v) {
+            if (a.bias[l]) v += a.bias[l][oo];
+            if (a.relu[l]) v = fmaxf(v, 0.0f);
+            if (last) {
+               if (row0 + r < a.M) a.y[(size_t)(row0 + r) * a.ldy + oo] = v;
+            } else {
+               buf_out[r * a.maxd + oo] = v;
+            }
+         };
+         if (parts == 1) {
+            // 256 columns per pass: every thread holds the complete sums of its column
+            if (o < N) {
+#pragma unroll
+               for (int r = 0; r < R; ++r) finish(r, o, acc[r]);
+            }
+         } else {
+#pragma unroll
+            for (int r = 0; r < R; ++r) part[tid * R + r] = acc[r];
+            __syncthreads();
+            // the parts of an output are added in order by one thread per (row, output)
+            for (int idx = tid; idx < R * n2; idx += 256) {
+               const int r = idx / n2, c = idx - r * n2;
+               if (o0 + c >= N) continue;
+               float v = 0.0f;
+               for (int p = 0; p < parts; ++p) v += part[(p * n2 + c) * R + r];
+               finish(r, o0 + c, v);
+            }
+         }
+         if (parts > 1) __syncthreads();   // the partial sums are read before the next pass overwrites them
+      }
+      __syncthreads();
+      float *t = buf_in; buf_in = buf_out; buf_out = t;
+   }
+}
+
+}  // namespace
+
+extern "C" int sofie_hip_mlp_f32(sofie_hip_ctx *ctx, int n_layers, const int *dims, const float *const *W,
+                                 const float *const *bias, const int *act, const float *x, int ldx, float *y, int ldy,
+                                 int M)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, n_layers >= 1 && n_layers <= SOFIE_MLP_MAX_LAYERS && dims && W && act, "bad layer list");
+   SOFIE_REQUIRE(ctx, M >= 0, "negative dimension");
+   MlpArgs a{};
+   int maxd = 0;
+   for (int l = 0; l <= n_layers; ++l) {
+      SOFIE_REQUIRE(ctx, dims[l] >= 1 && dims[l] <= SOFIE_MLP_MAX_WIDTH, "layer width out of range");
+      a.dims[l] = dims[l];
+      if (dims[l] > maxd) maxd = dims[l];
+   }
+   for (int l = 0; l < n_layers; ++l) {
+      SOFIE_REQUIRE(ctx, W[l], "null weight matrix");
+      SOFIE_REQUIRE(ctx, act[l] == SOFIE_ACT_NONE || act[l] == SOFIE_ACT_RELU, "unknown activation");
+      a.W[l] = W[l];
+      a.bias[l] = bias ? bias[l] : nullptr;
+      a.relu[l] = act[l] == SOFIE_ACT_RELU;
+   }
+   if (M == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && y, "null operand");
+   SOFIE_REQUIRE(ctx, ldx >= dims[0] && ldy >= dims[n_layers], "leading dimension too small");
+   a.x = x; a.y = y; a.n_layers = n_layers; a.M = M; a.ldx = ldx; a.ldy = ldy;
+   a.maxd = (maxd + 3) & ~3;
+   // rows per workgroup: one while that still gives every CU a workgroup, more when there are rows to share the
+   // weight traffic between
+   const int cus = ctx->num_cus > 0 ? ctx->num_cus : 256;
+   const int R = M <= 2 * cus ? 1 : M <= 8 * cus ? 4 : 8;
+   const size_t lds = ((size_t)2 * R * a.maxd + (size_t)256 * R) * sizeof(float);
+   const dim3 grid((unsigned)cdiv(M, R)), block(256);
+   auto launch = [&](auto kern) -> int {
+      SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);
+      return SOFIE_HIP_OK;
+   };
+   if (int rc = R == 1 ? launch(k_mlp_f32<1>) : R == 4 ? launch(k_mlp_f32<4>) : launch(k_mlp_f32<8>)) return rc;
+   return check_launch(ctx, "k_mlp_f32");
+}

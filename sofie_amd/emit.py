@@ -131,7 +131,7 @@ class ModelSpec:
 
     # ---- generation ------------------------------------------------------------------------
     def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False, batch=None,
-                 runtime_batch=False, no_session=False, emitter=None, env=None):
+                 runtime_batch=False, no_session=False, emitter=None, env=None, layer_per_call=False):
         """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess). `batch` gives the shape
         parameters of the inputs (dimensions written as names) their value; with `runtime_batch` it is a capacity and
         the generated Session also takes infer(n, ...) for any n up to it. `emitter` names another build of the emit
@@ -151,6 +151,8 @@ class ModelSpec:
                 flag += " batch %d" % batch
             if runtime_batch or self.runtime_batch:
                 flag += " runtimebatch"
+            if layer_per_call:
+                flag += " layerpercall"       # Options::kLayerPerCall: no chains of fully connected layers in one launch
             f.write("\n".join(self.lines + ["generate" + flag]) + "\n")
         if emitter is None and not os.path.exists(EMIT):
             build_emitter()

@@ -30,6 +30,7 @@ enum class Options {
    kGNNComponent = 0x10,
    kBinaryWeightFile = 0x20,     // typed binary records in <name>.bin instead of the text <name>.dat (not in the reference)
    kRuntimeBatch = 0x40,         // the batch size given to Generate is a capacity: infer(n, ...) runs any n up to it
+   kLayerPerCall = 0x80,         // no chains of fully connected layers in one launch: every Gemm emits its own call
 };
 std::underlying_type_t<Options> operator|(Options opA, Options opB);
 std::underlying_type_t<Options> operator|(std::underlying_type_t<Options> opA, Options opB);
@@ -130,6 +131,7 @@ private:
       int first = 0, last = 0;
    };
    void FuseBatchNorm();
+   void FuseGemmChain();
    void FuseActivations();
    void FusePooling();
    void FuseInputQuantization();

@@ -40,6 +40,19 @@ private:
    static constexpr size_t SOFIE_GEMM_MAX_LEAD_DIMS = 6;   // SOFIE_GEMM_MAX_LEAD of the kernel library
 
 public:
+   // One layer of a chain of fully connected layers (RModel::FuseGemmChain): y = act(x W + bias), W [K, N].
+   struct ChainLayer {
+      std::string weights, bias;   // initialized tensors; bias "" if there is none
+      size_t K = 0, N = 0;
+      bool relu = false;
+   };
+   static constexpr size_t kChainMaxLayers = 16;    // SOFIE_MLP_MAX_LAYERS of the kernel library
+   static constexpr size_t kChainMaxWidth = 512;    // widths the emitter joins (the kernel takes up to SOFIE_MLP_MAX_WIDTH)
+
+private:
+   std::vector<ChainLayer> fChain;   // on the first operator of a chain: every layer, its own included
+
+public:
    ROperator_Gemm() {}
    ROperator_Gemm(float alpha, float beta, int_t transA, int_t transB, std::string nameA, std::string nameB,
                   std::string nameY, EActivationType activation = EActivationType::UNDEFINED)
@@ -194,6 +207,62 @@ public:
       model.AddNeededStdLib("algorithm");
    }
 
+   // --- chains of fully connected layers ----------------------------------------------------------------------
+   // This operator can be a layer of a chain: a plain product of a [M, K] activation with a constant [K, N] (or
+   // [N, K] with transB) matrix, alpha 1, a constant bias of one row added once (beta 1) or none, widths the
+   // one-launch kernel is meant for.
+   bool ChainCandidate(const RModel &model) const
+   {
+      if (fShapeY.empty() || fStack != 1 || fAttrTransA || fAttrAlpha != 1.0f) return false;
+      if (!model.IsInitializedTensor(fNB)) return false;
+      if (!fNC.empty() && (fBiasKind != 1 || fAttrBeta != 1.0f || !model.IsInitializedTensor(fNC))) return false;
+      const size_t k = fShapeA[1], n = fShapeY[1];
+      return k >= 1 && n >= 1 && k <= kChainMaxWidth && n <= kChainMaxWidth;
+   }
+   const std::string &NameA() const { return fNA; }
+   const std::string &NameB() const { return fNB; }
+   const std::string &NameY() const { return fNY; }
+   bool TransB() const { return fAttrTransB != 0; }
+   size_t Rows() const { return fShapeY[0]; }
+   size_t MultiplyAdds() const { return fShapeA[1] * fShapeY[1]; }
+   bool IsChainHead() const { return !fChain.empty(); }
+   // The constant matrix as [K, N]: a transposed one is rewritten once, here, at generation time.
+   void MakeWeightsKByN(RModel &model)
+   {
+      if (!fAttrTransB) return;
+      const size_t n = fShapeB[0], k = fShapeB[1];
+      const float *src = static_cast<const float *>(model.GetInitializedTensorData(fNB).get());
+      std::shared_ptr<void> dst(malloc(n * k * sizeof(float)), free);
+      float *d = static_cast<float *>(dst.get());
+      for (size_t i = 0; i < n; ++i)
+         for (size_t j = 0; j < k; ++j) d[j * n + i] = src[i * k + j];
+      model.UpdateInitializedTensor(fNB, ETensorType::FLOAT, {k, n}, dst);
+      fShapeB = {k, n};
+      fAttrTransB = 0;
+   }
+   ChainLayer AsLayer() const
+   {
+      ChainLayer l;
+      l.weights = fNB;
+      l.bias = fNC;
+      l.K = fShapeA[1];
+      l.N = fShapeY[1];
+      l.relu = fActivation == EActivationType::RELU;
+      return l;
+   }
+   // This operator becomes the first layer of a chain that ends in the tensor `last` ([M, N of the last layer]):
+   // it reads the weights and biases of every layer and writes `last` only.
+   void BecomeChainHead(const std::vector<ChainLayer> &layers, const std::string &last)
+   {
+      fChain = layers;
+      fOutputTensorNames = {last};
+      fInputTensorNames = {fNA};
+      for (auto &l : fChain) {
+         fInputTensorNames.push_back(l.weights);
+         if (!l.bias.empty()) fInputTensorNames.push_back(l.bias);
+      }
+   }
+
    // the rows of A are the batch: not with a transposed A, stacked operands or a bias of one value per row
    bool SetRuntimeBatch(const std::string &expr, size_t capacity) override
    {
@@ -211,6 +280,29 @@ public:
       const size_t m = fShapeY[0], n = fShapeY[1];
       const size_t k = fAttrTransA ? fShapeA[0] : fShapeA[1];
       std::stringstream out;
+      if (!fChain.empty()) {
+         // every layer of the chain in one launch; the activations between the layers stay on chip
+         out << "\n//--------- Gemm x " << fChain.size() << " (chain of fully connected layers)\n";
+         out << SP << "{\n";
+         out << SP << SP << "static const int " << opName << "_dims[] = {" << fChain.front().K;
+         for (auto &l : fChain) out << ", " << l.N;
+         out << "};\n";
+         out << SP << SP << "const float *" << opName << "_w[] = {";
+         for (size_t i = 0; i < fChain.size(); ++i) out << (i ? ", " : "") << "tensor_" << fChain[i].weights;
+         out << "};\n";
+         out << SP << SP << "const float *" << opName << "_b[] = {";
+         for (size_t i = 0; i < fChain.size(); ++i)
+            out << (i ? ", " : "") << (fChain[i].bias.empty() ? std::string("nullptr") : "tensor_" + fChain[i].bias);
+         out << "};\n";
+         out << SP << SP << "static const int " << opName << "_act[] = {";
+         for (size_t i = 0; i < fChain.size(); ++i) out << (i ? ", " : "") << (fChain[i].relu ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE");
+         out << "};\n";
+         out << SP << SP << "Check(sofie_hip_mlp_f32(fCtx, " << fChain.size() << ", " << opName << "_dims, " << opName << "_w, "
+             << opName << "_b, " << opName << "_act, tensor_" << fNA << ", " << fChain.front().K << ", tensor_"
+             << fOutputTensorNames[0] << ", " << fChain.back().N << ", " << BatchCount(m) << "), \"Gemm chain " << opName << "\");\n";
+         out << SP << "}\n";
+         return out.str();
+      }
       out << "\n//--------- Gemm\n";
       const std::string act = fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE";
       if (fStack > 1) {

@@ -6,6 +6,7 @@
 #include "SOFIE/RModel.hxx"
 #include "SOFIE/ROperator_BatchNormalization.hxx"
 #include "SOFIE/ROperator_Conv.hxx"
+#include "SOFIE/ROperator_Gemm.hxx"
 #include "SOFIE/ROperator_Pool.hxx"
 #include "SOFIE/ROperator_Quantized.hxx"
 
@@ -317,6 +318,74 @@ void RModel::FuseActivations()
       }
       if (other_use) continue;
       if (fOperators[i]->FuseActivation(EActivationType::RELU)) act.SetFusedAway();
+   }
+}
+
+// Gemm operators whose output feeds only the next Gemm (through a Relu that has moved into the producer's
+// epilogue, if there is one) and whose matrices are small constants: a multilayer perceptron. The first operator of
+// the chain emits one call for all layers (sofie_hip_mlp_f32), the others emit nothing, and the tensors between
+// the layers stop existing. On a few hundred rows such a chain is bound by its launches, not by arithmetic.
+void RModel::FuseGemmChain()
+{
+   auto readers_of = [&](const std::string &t) {
+      std::vector<size_t> r;
+      for (size_t k = 0; k < fOperators.size(); ++k) {
+         if (fOperators[k]->IsAbsorbed()) continue;
+         for (auto &in : fOperators[k]->GetOpInputTensors())
+            if (in == t) { r.push_back(k); break; }
+      }
+      return r;
+   };
+   auto is_output = [&](const std::string &t) {
+      return std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), t) != fOutputTensorNames.end();
+   };
+   for (size_t i = 0; i < fOperators.size(); ++i) {
+      auto *head = dynamic_cast<ROperator_Gemm<float> *>(fOperators[i].get());
+      if (!head || head->IsAbsorbed() || head->IsChainHead() || !head->ChainCandidate(*this)) continue;
+      std::vector<ROperator_Gemm<float> *> layers = {head};
+      std::vector<size_t> absorbed;            // operators that emit nothing any more
+      std::vector<std::string> gone;           // tensors between the layers
+      std::string cur = head->NameY();
+      size_t work = head->MultiplyAdds();
+      while (layers.size() < ROperator_Gemm<float>::kChainMaxLayers && !is_output(cur)) {
+         const std::vector<size_t> readers = readers_of(cur);
+         if (readers.size() != 1 || readers[0] <= i) break;
+         ROperator &next = *fOperators[readers[0]];
+         if (next.Kind() == "Relu" && next.IsFusedAway() && !next.GetOpOutputTensors().empty()) {
+            // the activation already sits in the producer: its output is the same values under another name
+            absorbed.push_back(readers[0]);
+            gone.push_back(cur);
+            cur = next.GetOpOutputTensors()[0];
+            continue;
+         }
+         auto *g = dynamic_cast<ROperator_Gemm<float> *>(&next);
+         if (!g || g->NameA() != cur || g->IsChainHead() || !g->ChainCandidate(*this)) break;
+         // a transposed matrix is rewritten as [K, N]: only if this operator is its only reader
+         if (g->TransB() && readers_of(g->NameB()).size() != 1) break;
+         layers.push_back(g);
+         absorbed.push_back(readers[0]);
+         gone.push_back(cur);
+         cur = g->NameY();
+         work += g->MultiplyAdds();
+      }
+      // a trailing activation view that was walked over without a layer behind it stays what it was
+      while (!absorbed.empty() && fOperators[absorbed.back()]->Kind() == "Relu") {
+         cur = gone.back();
+         absorbed.pop_back();
+         gone.pop_back();
+      }
+      if (layers.size() < 2) continue;
+      if (head->TransB() && readers_of(head->NameB()).size() != 1) continue;
+      // past this much arithmetic the matrix-core kernels, one launch per layer, are the faster form
+      if ((double)head->Rows() * (double)work > 536870912.0) continue;
+      std::vector<ROperator_Gemm<float>::ChainLayer> chain;
+      for (auto *g : layers) {
+         g->MakeWeightsKByN(*this);
+         chain.push_back(g->AsLayer());
+      }
+      head->BecomeChainHead(chain, cur);
+      for (size_t k : absorbed) fOperators[k]->SetAbsorbed();
+      for (auto &t : gone) fIntermediateTensorInfos.erase(t);
    }
 }
 
@@ -991,6 +1060,7 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    Initialize(batchSize, verbose);
    FuseBatchNorm();
    FuseActivations();
+   if (!(static_cast<std::underlying_type_t<Options>>(Options::kLayerPerCall) & options)) FuseGemmChain();
    FusePooling();
    FuseInputQuantization();
    PlanIntermediateMemory();

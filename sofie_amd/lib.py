@@ -35,6 +35,7 @@ SIGNATURES = {
     "sofie_hip_timer_start": [_p],
     "sofie_hip_timer_stop": [_p, C.POINTER(_f)],
     "sofie_hip_gemm_f32": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i, _p, _i, _i],
+    "sofie_hip_mlp_f32": [_p, _i, C.POINTER(_i), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(_i), _p, _i, _p, _i, _i],
     "sofie_hip_gemm_f32_stacked": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _p, _i, _i, C.POINTER(_i),
                                    C.POINTER(C.c_longlong), C.POINTER(C.c_longlong), _i],
     "sofie_hip_conv2d_f32": [_p, _p, _p, _p, _p] + [_i] * 17,

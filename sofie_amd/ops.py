@@ -151,6 +151,24 @@ def gemm_f32(A, B, bias=None, alpha=1.0, beta=1.0, transA=False, transB=False, r
     return ctx.ret(y, A)
 
 
+def mlp_f32(x, weights, biases=None, relus=None, ctx=None):
+    """y = act_L(... act_1(x W_1 + b_1) ... W_L + b_L) in one launch; W_l [K_l, N_l], b_l [N_l] or None."""
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.float32)
+    n = len(weights)
+    wd = [ctx.dev(w, torch.float32) for w in weights]
+    bd = [ctx.dev(b, torch.float32) if biases is not None and b is not None else None for b in (biases or [None] * n)]
+    dims = [xd.shape[1]] + [w.shape[1] for w in wd]
+    y = ctx.empty((xd.shape[0], dims[-1]), torch.float32)
+    c_dims = (C.c_int * (n + 1))(*dims)
+    c_w = (C.c_void_p * n)(*[w.data_ptr() for w in wd])
+    c_b = (C.c_void_p * n)(*[b.data_ptr() if b is not None else None for b in bd])
+    c_a = (C.c_int * n)(*[L.ACT_RELU if (relus and relus[i]) else L.ACT_NONE for i in range(n)])
+    ctx.check(ctx.lib.sofie_hip_mlp_f32(ctx.h, n, c_dims, c_w, c_b, c_a, ctx.ptr(xd), xd.shape[1], ctx.ptr(y), dims[-1],
+                                        xd.shape[0]))
+    return ctx.ret(y, x)
+
+
 def relu_f32(x, ctx=None):
     ctx = ctx or default_context()
     xd = ctx.dev(x, torch.float32)

@@ -72,7 +72,7 @@ def test_relu_after_gemm_and_conv_is_fused_and_flatten_is_a_view(tmp_path):
 
 def test_pool_offsets_never_overlap_while_both_tensors_are_live(tmp_path):
     spec, _ = models.mlp_spec("mlp_plan")
-    hxx, _, _ = gen(spec, tmp_path)
+    hxx, _, _ = gen(spec, tmp_path, layer_per_call=True)     # one call per Gemm: the tensors between the layers exist
     code = open(hxx).read()
     off = {m.group(1): int(m.group(2)) for m in re.finditer(r"tensor_(\w+) = reinterpret_cast<float\*>\(fIntermediateMemoryPool \+ (\d+)\)", code)}
     size = {"h0": 256 * 128 * 4, "h1": 256 * 64 * 4, "y": 256 * 8 * 4}
@@ -600,7 +600,7 @@ def test_several_outputs_follow_the_reference_return_convention(tmp_path):
     the order of the output list (RModel.cxx:744-801); an intermediate that is an output keeps its place in the
     pool until the end; the generated code compiles against the runner."""
     spec, _ = models.two_heads_spec("two_heads_probe")
-    hxx, _, _ = gen(spec, tmp_path)
+    hxx, _, _ = gen(spec, tmp_path, layer_per_call=True)   # one call per layer, so that the first hidden layer is a tensor
     code = open(hxx).read()
     assert "std::vector<std::vector<float>> infer(float* tensor_x)" in code
     assert "return std::vector<std::vector<float>>{std::move(ret_0), std::move(ret_1)};" in code
@@ -677,3 +677,49 @@ def test_generated_weight_reader_checks_the_element_type(tmp_path):
     assert calls and {int(c[2]) for c in calls} <= {1, 2, 3, 6}          # FLOAT, UINT8, INT8, INT32
     assert any(int(c[2]) == 3 for c in calls) and any(int(c[2]) == 1 for c in calls)
     assert "type != expected_type" in code and "failed to read the correct tensor type" in code
+
+
+def test_gemm_chain_becomes_one_call(tmp_path):
+    """Gemm -> Relu -> Gemm -> Relu -> Gemm on small constant matrices: one sofie_hip_mlp_f32 call, no tensor between the
+    layers, weights given [N, K] rewritten as [K, N] in the weight file; Options::kLayerPerCall keeps the three calls."""
+    spec, _ = models.mlp_spec("mlp_chain")
+    hxx, _, _ = gen(spec, tmp_path)
+    code = open(hxx).read()
+    assert code.count("sofie_hip_mlp_f32(") == 1 and "sofie_hip_gemm_f32(" not in code
+    assert re.search(r"_dims\[\] = \{64, 128, 64, 8\};", code)
+    assert re.search(r"_act\[\] = \{SOFIE_ACT_RELU, SOFIE_ACT_RELU, SOFIE_ACT_NONE\};", code)
+    assert "tensor_h0" not in code and "tensor_h1" not in code
+    hxx, _, _ = gen(spec, tmp_path, layer_per_call=True)
+    code = open(hxx).read()
+    assert code.count("sofie_hip_gemm_f32(") == 3 and "sofie_hip_mlp_f32(" not in code
+
+    # a layer whose output is also a model output ends the chain; a transposed matrix read by two layers is not rewritten
+    r = np.random.default_rng(0)
+    s2 = emit.ModelSpec("chain_breaks")
+    s2.add_input("x", "FLOAT", (4, 6))
+    s2.add_init("W", r.standard_normal((6, 6)).astype(np.float32))
+    s2.add_init("V", r.standard_normal((3, 6)).astype(np.float32))
+    s2.gemm("x", "W", None, "a", beta=0.0, transB=True)
+    s2.gemm("a", "W", None, "b", beta=0.0, transB=True)
+    s2.gemm("b", "V", None, "c", beta=0.0, transB=True)
+    s2.gemm("c", "V", None, "d", beta=0.0)
+    s2.set_output("d")
+    hxx, dat, _ = gen(s2, tmp_path)
+    code = open(hxx).read()
+    # W and V are transposed operands read by two layers each: rewriting them as [K, N] for one reader would break
+    # the other, so every layer keeps its own call
+    assert code.count("sofie_hip_gemm_f32(") == 4 and "sofie_hip_mlp_f32(" not in code
+    s3 = emit.ModelSpec("chain_to_output")
+    s3.add_input("x", "FLOAT", (4, 6))
+    for n_, shape in (("A", (6, 5)), ("B", (5, 7)), ("C", (7, 2))):
+        s3.add_init(n_, r.standard_normal(shape).astype(np.float32))
+    s3.gemm("x", "A", None, "p", beta=0.0)
+    s3.gemm("p", "B", None, "q", beta=0.0)
+    s3.gemm("q", "C", None, "t", beta=0.0)
+    s3.set_output("q")
+    s3.set_output("t")
+    hxx, _, _ = gen(s3, tmp_path)
+    code = open(hxx).read()
+    # q is a model output: the chain x -> p -> q ends there and the last layer is a call of its own
+    assert code.count("sofie_hip_mlp_f32(") == 1 and code.count("sofie_hip_gemm_f32(") == 1
+    assert re.search(r"_dims\[\] = \{6, 5, 7\};", code)

@@ -223,3 +223,26 @@ def test_gemm_fp8_random_shapes(ops, seed):
     assert np.all(np.abs(yf.astype(np.float64) - truth) <= slack + 2.0 ** -22 * np.abs(truth)), (M, N, K, transB)
     assert np.all(np.abs(oracle.bf16_decode(yb).astype(np.float64) - truth) <= 2.0 ** -8 * np.abs(truth) + slack)
     assert np.array_equal(yb, oracle.bf16_encode(yf))
+
+
+@pytest.mark.parametrize("seed", range(14))
+def test_mlp_f32_random_chains(ops, seed):
+    """The one-launch chain of fully connected layers against the oracle's Gemm applied layer by layer."""
+    r = np.random.default_rng(9800 + seed)
+    n = int(r.integers(1, 6))
+    dims = [int(r.integers(1, 300)) for _ in range(n + 1)]
+    if seed == 0:
+        n, dims = 3, [64, 128, 64, 8]                 # the benchmark's MLP
+    if seed == 1:
+        n, dims = 2, [700, 1024, 513]                 # wide layers: more than one pass of 256 columns
+    M = int(r.choice([1, 7, 256, 700, 3000])) if seed > 1 else 256
+    x = r.standard_normal((M, dims[0])).astype(np.float32)
+    Ws = [(r.standard_normal((dims[i], dims[i + 1])) / np.sqrt(dims[i])).astype(np.float32) for i in range(n)]
+    bs = [r.standard_normal(dims[i + 1]).astype(np.float32) if (seed + i) % 3 else None for i in range(n)]
+    relus = [bool((seed + i) % 2) for i in range(n)]
+    ref = x
+    for i in range(n):
+        ref = oracle.gemm_f32(ref, Ws[i], bs[i], 1.0, 1.0 if bs[i] is not None else 0.0, False, False, relus[i])
+    got = ops.mlp_f32(x, Ws, bs, relus)
+    assert got.shape == ref.shape
+    assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (dims, M)
