@@ -58,11 +58,26 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16 || NSETS > 2) ? 1 : 2) k_g
 
    int tm, tn;
    int pid = blockIdx.x;
+   bool placed = false;
    if constexpr (IS_INT && OUT == SOFIE_OUT_S32) {
       if (g.splits > 1) {
          const int tiles = g.tiles_m * g.tiles_n;
-         const int ks = pid / tiles;
-         pid -= ks * tiles;
+         int ks;
+         const int xps = 8 / g.splits;                 // XCDs per K slice
+         if (8 % g.splits == 0 && tiles % xps == 0) {
+            // Workgroup ids are dealt round-robin over the 8 XCDs. A K slice goes to 8 / splits XCDs of its own: the
+            // slice of B is then read by those XCDs only (with rows of tiles spread over all XCDs every XCD reads all
+            // of B), and the column tiles of a row panel of A sit next to each other on one XCD.
+            const int xcd = pid & 7, idx = pid >> 3;
+            ks = xcd / xps;
+            const int tile = (xcd % xps) * (tiles / xps) + idx;
+            tm = tile / g.tiles_n;
+            tn = tile - tm * g.tiles_n;
+            placed = true;
+         } else {
+            ks = pid / tiles;
+            pid -= ks * tiles;
+         }
          const int k_begin = ks * g.kslice;
          g.A += k_begin;
          g.B += B_KN ? (size_t)k_begin * g.ldb : (size_t)k_begin;
@@ -70,7 +85,7 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16 || NSETS > 2) ? 1 : 2) k_g
          g.Y = static_cast<unsigned char *>(g.Y) + (size_t)ks * g.ysplit;
       }
    }
-   tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
+   if (!placed) tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
 
    // --- global -> register staging -----------------------------------------------------
