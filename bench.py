@@ -481,7 +481,7 @@ def run_generated(name, dat, x, iters):
     return json.loads(res.stdout.strip().splitlines()[-1]), y
 
 
-def mlp_session_rate(iters=500):
+def mlp_session_rate(iters=2000):
     """The generated Session of the fp32 MLP (64 -> 128 -> 64 -> 8, batch 256): three Gemm launches with fused bias and
     ReLU. Device time of infer_device() on a resident input, replay from a HIP graph, wall time of infer()."""
     x = np.random.default_rng(3).standard_normal((256, 64)).astype(np.float32)
@@ -495,7 +495,7 @@ def mlp_session_rate(iters=500):
             "host_us_with_pcie": t["host_ms"] * 1e3, "bound": "launch latency (8.65 MFLOP, 142,112 algorithmic bytes)"}
 
 
-def cnn_session_rate(iters=50, cpu_images=0):
+def cnn_session_rate(iters=300, cpu_images=0):
     """The generated Session of the int8 CNN at batch 4096 (1x40x40 input; conv 1->32, pool, conv 32->64, pool,
     conv 64->128, fc 12800->256, fc 256->5), run by its prebuilt runner as a child process: device time of
     infer_device() on a resident input, and wall time of infer() including the PCIe copies. With cpu_images > 0 the
