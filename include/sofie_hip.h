@@ -263,6 +263,20 @@ int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, cons
                        int lda, const int8_t *B, int ldb, const float *scale,
                        const int32_t *bias, int zp_y, int act, void *Y, int ldy, int out_kind);
 
+/* Two QLinearMatMul layers, the second one narrow (a classifier's last two fully connected layers), in one call:
+ *   T = sofie_hip_qgemm_s8(transB = 1, A [M,K], B1 [N1,K], scale1, bias1, zp_mid, act1) -> int8 [M,N1]
+ *   Y = sofie_hip_qgemm_s8(transB = 1, T, B2 [N2,N1], scale2, bias2, zp_y, act2, out_kind)  (S8 or F32)
+ * with exactly those results. `mid` [M, ldmid] is a tensor the call may use for T; what it holds afterwards is
+ * unspecified. When the first layer's K is long enough to be cut into slices and N2 <= 8, the pass that adds the
+ * slices' partial sums also applies the second layer and T is never written (one kernel and one pass over memory
+ * less); otherwise the call is the two calls above through `mid`. The emitter joins two QLinearMatMul operators
+ * into this call when the first one's output feeds only the second (RModel::FuseQLinearPair). Replaces two of the
+ * reference's emitted Gemm sequences (ROperator_Gemm.hxx:292-390) on dequantised tensors. */
+int sofie_hip_qgemm_s8_pair(sofie_hip_ctx *ctx, int M, int K, const int8_t *A, int lda, int N1, const int8_t *B1,
+                            int ldb1, const float *scale1, const int32_t *bias1, int zp_mid, int act1,
+                            int8_t *mid, int ldmid, int N2, const int8_t *B2, int ldb2, const float *scale2,
+                            const int32_t *bias2, int zp_y, int act2, void *Y, int ldy, int out_kind);
+
 /* sofie_hip_qgemm_s8 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc): same arguments, same kernels, same results bit for bit, but the call
  * never allocates or frees. It has no counterpart in the reference. The two paths of sofie_hip_qgemm_s8 that use

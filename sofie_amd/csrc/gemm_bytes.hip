@@ -726,6 +726,77 @@ __global__ void __launch_bounds__(256) k_splitk_finish(GemmArgs g, const int *__
    }
 }
 
+// The second, narrow layer of a pair behind a first layer whose K was cut into slices (a classifier's last two fully
+// connected layers): the pass that adds the slices also requantises the first layer's row, multiplies it into the
+// second layer's few columns and writes those; the first layer's output is never stored. g1 describes the first
+// layer's requantisation (N = N1, scale, bias, zp, lo), g2 the second layer (B = its matrix [N2, ldb], N = N2 <= 8,
+// K = N1, scale, bias, zp, lo, relu, Y, ldy). N1 / 4 threads share a row: a power of two of at most 64, so a row's
+// threads are lanes of one wavefront and their partial dot products meet through lane shuffles.
+// Sum of a value over the 64 lanes of a wavefront, delivered in lane 63: an inclusive scan inside each row of 16 lanes
+// (row shifts by 1, 2, 4, 8), then the row totals travel to the following rows (lane 15 of a row to the next row,
+// lane 31 to the upper half). Six vector instructions, no LDS.
+__device__ __forceinline__ int wave_sum_in_lane63(int v)
+{
+   v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);
+   v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);
+   v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);
+   v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);
+   v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);
+   v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);
+   return v;
+}
+
+template <int OUT2, int QUADS>
+__global__ void __launch_bounds__(256) k_splitk_finish_pair(GemmArgs g1, const int *__restrict__ P, int splits, int ldp, GemmArgs g2)
+{
+   constexpr int quads = QUADS;
+   const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+   if (t >= (size_t)g1.M * quads) return;
+   const int m = (int)(t / quads), c = (int)(t % quads), n = c * 4;
+   const size_t plane = (size_t)g1.M * ldp;
+   v4i s = *reinterpret_cast<const v4i *>(P + (size_t)m * ldp + n);
+   for (int k = 1; k < splits; ++k) {
+      const v4i v = *reinterpret_cast<const v4i *>(P + k * plane + (size_t)m * ldp + n);
+      s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
+   }
+   unsigned packed = 0;
+#pragma unroll
+   for (int e = 0; e < 4; ++e) {
+      const unsigned r = epilogue_value<true, SOFIE_OUT_S8>(g1, g1.scale[n + e], g1.bias ? static_cast<const int *>(g1.bias)[n + e] : 0,
+                                                            s[e], 0.0f);
+      packed |= ((unsigned)((int)fminf(__uint_as_float(r), 255.0f) - 128) & 0xffu) << (8 * e);
+   }
+   int dot[8];
+#pragma unroll
+   for (int j = 0; j < 8; ++j) {
+      dot[j] = 0;
+      if (j < g2.N) {      // uniform over the launch
+         const int w = *reinterpret_cast<const int *>(g2.B + (size_t)j * g2.ldb + n);
+         dot[j] = __builtin_amdgcn_sdot4((int)packed, w, 0, false);
+         if constexpr (QUADS == 64) {
+            dot[j] = wave_sum_in_lane63(dot[j]);      // a row is a whole wavefront
+         } else {
+#pragma unroll
+            for (int d = 1; d < quads; d <<= 1) dot[j] += __shfl_xor(dot[j], d);
+         }
+      }
+   }
+   // the thread that writes output j of the row: the last lane has every sum of a whole-wavefront row, otherwise
+   // every lane of the row's group has them and lane j of the group writes
+   const bool whole_wave = QUADS == 64;
+   constexpr int ESZ = OutSize<OUT2>::value;
+#pragma unroll
+   for (int j = 0; j < 8; ++j) {
+      if ((whole_wave ? c == 63 : j == c) && j < g2.N) {
+         const unsigned r = epilogue_value<true, OUT2>(g2, g2.scale ? g2.scale[j] : 0.0f,
+                                                       g2.bias ? static_cast<const int *>(g2.bias)[j] : 0, dot[j], 0.0f);
+         unsigned char *out = static_cast<unsigned char *>(g2.Y) + ((size_t)m * g2.ldy + j) * ESZ;
+         if constexpr (ESZ == 1) *out = (unsigned char)((int)fminf(__uint_as_float(r), 255.0f) - 128);
+         else *reinterpret_cast<unsigned *>(out) = r;
+      }
+   }
+}
+
 template <class Mma, int BK, int NSETS, int TI, int TJ, int OUT, bool B_KN, bool FULL>
 int launch_tiled_impl(sofie_hip_ctx *ctx, GemmArgs &g)
 {
@@ -773,7 +844,8 @@ int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
 // K cut into `splits` slices of `kslice` bytes (a multiple of BK): partial sums into the context's scratch
 // buffer, then k_splitk_finish writes Y.
 template <class Mma, int BK, int NSETS, int OUT>
-int launch_split_k(sofie_hip_ctx *ctx, GemmArgs &g, int splits, int kslice)
+int launch_split_k(sofie_hip_ctx *ctx, GemmArgs &g, int splits, int kslice, const GemmArgs *tail = nullptr,
+                   int tail_out = SOFIE_OUT_S8)
 {
    const int ldp = cdiv(g.N, 4) * 4;
    void *part = nullptr;
@@ -790,8 +862,28 @@ int launch_split_k(sofie_hip_ctx *ctx, GemmArgs &g, int splits, int kslice)
    p.ysplit = (long long)g.M * ldp * sizeof(int);
    if (int rc = launch_tiled<Mma, BK, NSETS, 2, 2, SOFIE_OUT_S32, false>(ctx, p)) return rc;
    const size_t threads = (size_t)g.M * (ldp / 4);
-   hipLaunchKernelGGL((k_splitk_finish<OUT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, ctx->stream, g,
-                      static_cast<const int *>(part), splits, ldp);
+   const dim3 fgrid((unsigned)((threads + 255) / 256));
+   if (tail) {
+      if constexpr (OUT == SOFIE_OUT_S8) {
+         const int *pp = static_cast<const int *>(part);
+#define SOFIE_PAIR_LAUNCH(Q_)                                                                                              \
+   do {                                                                                                                     \
+      if (tail_out == SOFIE_OUT_F32)                                                                                        \
+         hipLaunchKernelGGL((k_splitk_finish_pair<SOFIE_OUT_F32, Q_>), fgrid, dim3(256), 0, ctx->stream, g, pp, splits, ldp, *tail); \
+      else                                                                                                                  \
+         hipLaunchKernelGGL((k_splitk_finish_pair<SOFIE_OUT_S8, Q_>), fgrid, dim3(256), 0, ctx->stream, g, pp, splits, ldp, *tail);  \
+   } while (0)
+         switch (ldp / 4) {
+         case 8: SOFIE_PAIR_LAUNCH(8); break;
+         case 16: SOFIE_PAIR_LAUNCH(16); break;
+         case 32: SOFIE_PAIR_LAUNCH(32); break;
+         default: SOFIE_PAIR_LAUNCH(64); break;
+         }
+#undef SOFIE_PAIR_LAUNCH
+         return check_launch(ctx, "k_splitk_finish_pair");
+      }
+   }
+   hipLaunchKernelGGL((k_splitk_finish<OUT>), fgrid, dim3(256), 0, ctx->stream, g, static_cast<const int *>(part), splits, ldp);
    return check_launch(ctx, "k_splitk_finish");
 }
 
@@ -802,6 +894,21 @@ int launch_simple(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
    hipLaunchKernelGGL((k_gemm_bytes_simple<IS_INT, OUT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
                       ctx->stream, g, transB);
    return check_launch(ctx, "k_gemm_bytes_simple");
+}
+
+// Whether an int8 product with K-contiguous operands is cut into slices of K, and how: few 128 x 128 tiles and a long
+// K (measured: pays from K = 8192 on; below that the second pass over the partial sums costs more).
+bool split_k_plan(const sofie_hip_ctx *ctx, const GemmArgs &g, int &splits, int &kslice)
+{
+   const int tiles128 = cdiv(g.M, 128) * cdiv(g.N, 128);
+   if (!(tiles128 * 2 <= ctx->num_cus && g.K >= 8192)) return false;
+   splits = ctx->num_cus / tiles128;
+   const int shortest = tiles128 * 8 <= ctx->num_cus ? 1024 : 2048;
+   if (splits > g.K / shortest) splits = g.K / shortest;
+   if (splits > 16) splits = 16;
+   kslice = cdiv(cdiv(g.K, splits), 128) * 128;
+   splits = cdiv(g.K, kslice);
+   return splits > 1;
 }
 
 template <class Mma, int OUT>
@@ -835,17 +942,8 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
       if constexpr (IS_INT) {
          // ... and a longer one is cut into slices of K: 128 x 128 tiles write int32 partial sums per slice
          // (integer sums, so the result does not depend on the cut), a second kernel adds them and converts
-         const int tiles128 = cdiv(g.M, 128) * cdiv(g.N, 128);
-         // (measured: pays from K = 8192 on; below that the second pass over the partial sums costs more)
-         if (tiles128 * 2 <= ctx->num_cus && g.K >= 8192) {
-            int splits = ctx->num_cus / tiles128;
-            const int shortest = tiles128 * 8 <= ctx->num_cus ? 1024 : 2048;
-            if (splits > g.K / shortest) splits = g.K / shortest;
-            if (splits > 16) splits = 16;
-            const int kslice = cdiv(cdiv(g.K, splits), 128) * 128;
-            splits = cdiv(g.K, kslice);
-            if (splits > 1) return launch_split_k<Mma, BK, NSETS, OUT>(ctx, g, splits, kslice);
-         }
+         int splits = 1, kslice = 0;
+         if (split_k_plan(ctx, g, splits, kslice)) return launch_split_k<Mma, BK, NSETS, OUT>(ctx, g, splits, kslice);
       }
       if (cdiv(g.M, 128) * cdiv(g.N, 128) * 2 <= ctx->num_cus && g.K >= 1024)
          return launch_tiled<Mma, BK, NSETS, 1, 1, OUT, false>(ctx, g);
@@ -904,6 +1002,59 @@ int sofie_hip_qgemm_s8(sofie_hip_ctx *ctx, int transB, int M, int N, int K, cons
    case SOFIE_OUT_F32: return dispatch<MmaI8, SOFIE_OUT_F32>(ctx, g, transB);
    default: return dispatch<MmaI8, SOFIE_OUT_S32>(ctx, g, transB);
    }
+}
+
+int sofie_hip_qgemm_s8_pair(sofie_hip_ctx *ctx, int M, int K, const int8_t *A, int lda, int N1, const int8_t *B1, int ldb1,
+                            const float *scale1, const int32_t *bias1, int zp_mid, int act1, int8_t *mid, int ldmid,
+                            int N2, const int8_t *B2, int ldb2, const float *scale2, const int32_t *bias2, int zp_y,
+                            int act2, void *Y, int ldy, int out_kind)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, M >= 0 && K >= 0 && N1 >= 0 && N2 >= 0, "negative dimension");
+   if (M == 0 || N2 == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, A && B1 && B2 && Y && scale1 && scale2 && mid, "null operand");
+   SOFIE_REQUIRE(ctx, lda >= K && ldb1 >= K && ldmid >= N1 && ldb2 >= N1 && ldy >= N2, "leading dimension too small");
+   SOFIE_REQUIRE(ctx, out_kind == SOFIE_OUT_S8 || out_kind == SOFIE_OUT_F32, "output kind must be S8 or F32");
+   SOFIE_REQUIRE(ctx, (act1 == SOFIE_ACT_NONE || act1 == SOFIE_ACT_RELU) && (act2 == SOFIE_ACT_NONE || act2 == SOFIE_ACT_RELU),
+                 "unknown activation");
+   SOFIE_REQUIRE(ctx, zp_mid >= -128 && zp_mid <= 127 && zp_y >= -128 && zp_y <= 127, "zero-point out of int8 range");
+   // One pass for both layers when the first one is cut into K slices anyway (its partial sums are added by a pass of
+   // its own, which can as well multiply the finished row into a few more columns) and a row's quads of columns
+   // are lanes of one wavefront.
+   GemmArgs g{};
+   g.A = reinterpret_cast<const uint8_t *>(A);
+   g.B = reinterpret_cast<const uint8_t *>(B1);
+   g.Y = mid;
+   g.scale = scale1;
+   g.bias = bias1;
+   g.M = M; g.N = N1; g.K = K; g.lda = lda; g.ldb = ldb1; g.ldy = ldmid;
+   g.zp = zp_mid;
+   g.relu = act1 == SOFIE_ACT_RELU;
+   g.lo = (g.relu && zp_mid > -128) ? zp_mid : -128;
+   g.s = 1.0f;
+   const int quads = N1 / 4;
+   const bool lanes_ok = N1 % 4 == 0 && quads >= 8 && quads <= 64 && (quads & (quads - 1)) == 0;
+   const bool operands_ok = K % 16 == 0 && lda % 16 == 0 && aligned16(A) && ldb1 % 16 == 0 && aligned16(B1) && ldb2 % 4 == 0 &&
+                            (reinterpret_cast<uintptr_t>(B2) & 3u) == 0;
+   int splits = 1, kslice = 0;
+   if (N2 <= 8 && lanes_ok && operands_ok && N1 > 16 && split_k_plan(ctx, g, splits, kslice) &&
+       !((size_t)M * N1 >= (size_t)256 * 256 * 128 && M >= 256 && N1 >= 256)) {
+      GemmArgs t{};
+      t.B = reinterpret_cast<const uint8_t *>(B2);
+      t.Y = Y;
+      t.scale = scale2;
+      t.bias = bias2;
+      t.M = M; t.N = N2; t.K = N1; t.ldb = ldb2; t.ldy = ldy;
+      t.zp = zp_y;
+      t.relu = act2 == SOFIE_ACT_RELU;
+      t.lo = (t.relu && zp_y > -128) ? zp_y : -128;
+      t.s = 1.0f;
+      return launch_split_k<MmaI8, 128, 2, SOFIE_OUT_S8>(ctx, g, splits, kslice, &t, out_kind);
+   }
+   // otherwise the two layers one after the other, the first one's result in the caller's scratch tensor
+   if (int rc = sofie_hip_qgemm_s8(ctx, 1, M, N1, K, A, lda, B1, ldb1, scale1, bias1, zp_mid, act1, mid, ldmid, SOFIE_OUT_S8))
+      return rc;
+   return sofie_hip_qgemm_s8(ctx, 1, M, N2, N1, mid, ldmid, B2, ldb2, scale2, bias2, zp_y, act2, Y, ldy, out_kind);
 }
 
 int sofie_hip_qgemm_s8_noalloc(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const int8_t *A, int lda,

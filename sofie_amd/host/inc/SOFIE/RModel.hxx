@@ -132,6 +132,7 @@ private:
    };
    void FuseBatchNorm();
    void FuseGemmChain();
+   void FuseQLinearPair();
    void FuseActivations();
    void FusePooling();
    void FuseInputQuantization();

@@ -185,7 +185,48 @@ class ROperator_QLinearMatMul final : public ROperator {
    int fZpY = 0;
    bool fFloatOut = false, fHasBias = false;
    EActivationType fActivation = EActivationType::UNDEFINED;
+   // the narrow layer that follows this one, emitted with it as one call (RModel::FuseQLinearPair)
+   struct Tail {
+      std::string weights, scale, bias, out;
+      size_t N = 0;
+      int zpY = 0;
+      bool relu = false, floatOut = false;
+   };
+   bool fHasTail = false;
+   Tail fTail;
 public:
+   // --- pairs of layers -------------------------------------------------------------------------------------
+   const std::string &NameA() const { return fNA; }
+   const std::string &NameY() const { return fNY; }
+   size_t Columns() const { return fN; }
+   size_t Depth() const { return fK; }
+   bool FloatOut() const { return fFloatOut; }
+   bool HasTail() const { return fHasTail; }
+   // this operator as the second layer of a pair
+   Tail AsTail() const
+   {
+      Tail t;
+      t.weights = fNBt;
+      t.scale = fNScale;
+      t.bias = fHasBias ? fNQBias : "";
+      t.out = fNY;
+      t.N = fN;
+      t.zpY = fZpY;
+      t.relu = fActivation == EActivationType::RELU;
+      t.floatOut = fFloatOut;
+      return t;
+   }
+   // This operator writes the second layer's output as well; its own output stays in the pool as the tensor the
+   // library may use between the layers.
+   void AppendTail(const Tail &t)
+   {
+      fHasTail = true;
+      fTail = t;
+      fOutputTensorNames = {fNY, t.out};
+      fInputTensorNames.push_back(t.weights);
+      fInputTensorNames.push_back(t.scale);
+      if (!t.bias.empty()) fInputTensorNames.push_back(t.bias);
+   }
    ROperator_QLinearMatMul(std::string nameA, std::string nameAScale, std::string nameAZp, std::string nameB,
                            std::string nameBScale, std::string nameBZp, std::string nameYScale, std::string nameYZp,
                            std::string nameY, std::string nameBias = "", int_t transB = 0)
@@ -295,6 +336,18 @@ public:
    {
       if (fShapeA.empty()) throw std::runtime_error("TMVA SOFIE QLinearMatMul Op called to Generate without being initialized first");
       std::stringstream out;
+      if (fHasTail) {
+         out << "\n//--------- QLinearMatMul x 2 op_" << OpName << " (the second layer in the same call)\n";
+         out << SP << "Check(sofie_hip_qgemm_s8_pair(fCtx, " << BatchCount(fM) << ", " << fK << ", tensor_" << fNA << ", " << fK << ", "
+             << fN << ", tensor_" << fNBt << ", " << fK << ", tensor_" << fNScale << ", "
+             << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", " << fZpY << ", "
+             << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << ", tensor_" << fNY << ", " << fN << ", "
+             << fTail.N << ", tensor_" << fTail.weights << ", " << fN << ", tensor_" << fTail.scale << ", "
+             << (fTail.bias.empty() ? std::string("nullptr") : "tensor_" + fTail.bias) << ", " << fTail.zpY << ", "
+             << (fTail.relu ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << ", tensor_" << fTail.out << ", " << fTail.N << ", "
+             << (fTail.floatOut ? "SOFIE_OUT_F32" : "SOFIE_OUT_S8") << "), \"QLinearMatMul pair op_" << OpName << "\");\n";
+         return out.str();
+      }
       out << "\n//--------- QLinearMatMul op_" << OpName << "\n";
       out << SP << "Check(sofie_hip_qgemm_s8(fCtx, 1, " << BatchCount(fM) << ", " << fN << ", " << fK << ", tensor_" << fNA << ", " << fK
           << ", tensor_" << fNBt << ", " << fK << ", tensor_" << fNScale << ", "

@@ -389,6 +389,48 @@ void RModel::FuseGemmChain()
    }
 }
 
+// A QLinearMatMul whose int8 output feeds only a second, narrow QLinearMatMul (at most 8 columns: the last two
+// layers of a classifier): the first operator emits one call for both (sofie_hip_qgemm_s8_pair), the second emits
+// nothing. The tensor between them keeps its place in the pool: the library may use it, or skip it when it can
+// apply the second layer in the pass that finishes the first.
+void RModel::FuseQLinearPair()
+{
+   for (size_t i = 0; i < fOperators.size(); ++i) {
+      auto *first = dynamic_cast<ROperator_QLinearMatMul *>(fOperators[i].get());
+      if (!first || first->IsAbsorbed() || first->HasTail() || first->FloatOut()) continue;
+      std::string cur = first->NameY();
+      std::vector<size_t> views;
+      ROperator_QLinearMatMul *second = nullptr;
+      size_t at = 0;
+      for (;;) {
+         if (std::find(fOutputTensorNames.begin(), fOutputTensorNames.end(), cur) != fOutputTensorNames.end()) break;
+         std::vector<size_t> readers;
+         for (size_t k = 0; k < fOperators.size(); ++k) {
+            if (fOperators[k]->IsAbsorbed()) continue;
+            for (auto &in : fOperators[k]->GetOpInputTensors())
+               if (in == cur) { readers.push_back(k); break; }
+         }
+         if (readers.size() != 1 || readers[0] <= i) break;
+         ROperator &next = *fOperators[readers[0]];
+         if (next.Kind() == "Relu" && next.IsFusedAway() && !next.GetOpOutputTensors().empty()) {
+            views.push_back(readers[0]);
+            cur = next.GetOpOutputTensors()[0];
+            continue;
+         }
+         second = dynamic_cast<ROperator_QLinearMatMul *>(&next);
+         at = readers[0];
+         if (second && (second->NameA() != cur || second->HasTail() || second->Columns() > 8 || second->Depth() != first->Columns()))
+            second = nullptr;
+         break;
+      }
+      if (!second) continue;
+      first->AppendTail(second->AsTail());
+      second->SetAbsorbed();
+      (void)at;
+      (void)views;   // the activation views between the layers stay what they are: names for the first layer's tensor
+   }
+}
+
 // QLinearConv (with its fused Relu) followed by a pad-free int8 MaxPool that is the only consumer of the
 // activation: the pooling moves into the convolution call, which then writes the pooled tensor only.
 // The unpooled tensors disappear from the model, the Relu and the MaxPool emit nothing.
@@ -1060,7 +1102,10 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    Initialize(batchSize, verbose);
    FuseBatchNorm();
    FuseActivations();
-   if (!(static_cast<std::underlying_type_t<Options>>(Options::kLayerPerCall) & options)) FuseGemmChain();
+   if (!(static_cast<std::underlying_type_t<Options>>(Options::kLayerPerCall) & options)) {
+      FuseGemmChain();
+      FuseQLinearPair();
+   }
    FusePooling();
    FuseInputQuantization();
    PlanIntermediateMemory();

@@ -53,6 +53,7 @@ SIGNATURES = {
     "sofie_hip_quantize_f32_s8": [_p, _p, _p, _z, _f, _i],
     "sofie_hip_dequantize_s8_f32": [_p, _p, _p, _z, _f, _i],
     "sofie_hip_qgemm_s8": [_p, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i],
+    "sofie_hip_qgemm_s8_pair": [_p, _i, _i, _p, _i, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i],
     "sofie_hip_qgemm_s8_noalloc": [_p, _i, _i, _i, _i, _p, _i, _p, _i, _p, _p, _i, _i, _p, _i, _i],
     "sofie_hip_qconv2d_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 18,
     "sofie_hip_qconv2d_pool_s8": [_p, _p, _i, _p, _i, _p, _p, _p, _i] + [_i] * 21,

@@ -402,6 +402,24 @@ def qgemm_s8(A, B, scale, bias=None, transB=False, zpa=0, zpy=0, relu=False, out
     return ctx.ret(y, A)
 
 
+def qgemm_s8_pair(A, B1, scale1, bias1, zp_mid, relu1, B2, scale2, bias2, zpy=0, relu2=False, out=L.OUT_S8, ctx=None):
+    """Two QLinearMatMul layers in one call; B1 [N1, K] and B2 [N2, N1] (K-contiguous), biases with the zero-points
+    of their inputs already folded in."""
+    ctx = ctx or default_context()
+    a, b1, b2 = ctx.dev(A, torch.int8), ctx.dev(B1, torch.int8), ctx.dev(B2, torch.int8)
+    M, K = a.shape
+    N1, N2 = b1.shape[0], b2.shape[0]
+    s1, s2 = ctx.dev(scale1, torch.float32), ctx.dev(scale2, torch.float32)
+    q1, q2 = ctx.dev(bias1, torch.int32), ctx.dev(bias2, torch.int32)
+    mid = ctx.empty((M, N1), torch.int8)
+    y = ctx.empty((M, N2), _OUT_DTYPE[out])
+    ctx.check(ctx.lib.sofie_hip_qgemm_s8_pair(ctx.h, M, K, ctx.ptr(a), K, N1, ctx.ptr(b1), K, ctx.ptr(s1), ctx.ptr(q1),
+                                              int(zp_mid), L.ACT_RELU if relu1 else L.ACT_NONE, ctx.ptr(mid), N1, N2,
+                                              ctx.ptr(b2), N1, ctx.ptr(s2), ctx.ptr(q2), int(zpy),
+                                              L.ACT_RELU if relu2 else L.ACT_NONE, ctx.ptr(y), N2, out))
+    return ctx.ret(y, A)
+
+
 def qgemm_s8_f32out(A, B, scale, bias=None, transB=False, zpa=0, relu=False, ctx=None):
     return qgemm_s8(A, B, scale, bias, transB, zpa, 0, relu, L.OUT_F32, ctx)
 

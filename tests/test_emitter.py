@@ -150,7 +150,13 @@ def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
     assert code.count("sofie_hip_qconv2d_pool_s8(") == 1 and code.count("sofie_hip_qconv2d_s8(") == 1
     assert code.count("sofie_hip_quantize_qconv2d_s8(") == 1
     assert "sofie_hip_maxpool2d_s8" not in code and "tensor_c1" not in code.replace("tensor_c1_q", "") and "tensor_r2" not in code
-    assert code.count("sofie_hip_qgemm_s8(") == 2
+    # the two fully connected layers are one call (the second one has five columns); one call each with kLayerPerCall
+    assert code.count("sofie_hip_qgemm_s8_pair(") == 1 and code.count("sofie_hip_qgemm_s8(") == 0
+    assert re.search(r"sofie_hip_qgemm_s8_pair\(fCtx, 2, 12800, tensor_f, 12800, 256, tensor_fc1_nk_cl, 12800, tensor_g1_qscale, "
+                     r"tensor_g1_qbias, -128, SOFIE_ACT_RELU, tensor_g1, 256, 5, tensor_fc2_nk, 256, tensor_y_qscale, tensor_y_qbias, 0, "
+                     r"SOFIE_ACT_NONE, tensor_y, 5, SOFIE_OUT_F32\)", code)
+    code_lpc = open(gen(spec, tmp_path, layer_per_call=True)[0]).read()
+    assert code_lpc.count("sofie_hip_qgemm_s8(") == 2 and "sofie_hip_qgemm_s8_pair(" not in code_lpc
     assert "int8_t * tensor_fc1_nk_cl" in code and "tensor_fc1 =" not in code   # transposed once, original dropped
     assert "tensor_w2_ohwi, SOFIE_LAYOUT_NHWC" in code and "tensor_w2 =" not in code
     # conv1 reads the one-channel quantized input as it is, everything after it is channels-last

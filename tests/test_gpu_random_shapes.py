@@ -246,3 +246,29 @@ def test_mlp_f32_random_chains(ops, seed):
     got = ops.mlp_f32(x, Ws, bs, relus)
     assert got.shape == ref.shape
     assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (dims, M)
+
+
+@pytest.mark.parametrize("M,K,N1,N2", [(4096, 12800, 256, 5), (512, 8192, 128, 8), (300, 8464, 64, 3), (1024, 16384, 32, 1),
+                                        (700, 1040, 96, 4), (256, 8192, 256, 12), (64, 512, 100, 5)])
+def test_qgemm_s8_pair(ops, M, K, N1, N2):
+    """Two QLinearMatMul layers in one call against the two separate calls of the oracle: shapes whose first layer is
+    cut into K slices (the second layer then rides on the pass that adds the slices) and shapes that take the two
+    ordinary calls; int8 and float output."""
+    from sofie_amd import lib as L
+    r = np.random.default_rng(9900 + M + N1 + N2)
+    A = r.integers(-128, 128, (M, K)).astype(np.int8)
+    B1 = r.integers(-127, 128, (N1, K)).astype(np.int8)
+    B2 = r.integers(-127, 128, (N2, N1)).astype(np.int8)
+    s1 = (r.uniform(20, 60, N1) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    s2 = (r.uniform(20, 60, N2) / (73.3 * 73.3 * np.sqrt(N1))).astype(np.float32)
+    b1 = r.integers(-2000, 2000, N1).astype(np.int32)
+    b2 = r.integers(-2000, 2000, N2).astype(np.int32)
+    for zp_mid, relu1, zpy, relu2 in ((-128, True, 3, False), (5, False, -128, True)):
+        T = oracle.qgemm_s8(A, B1, s1, b1, True, 0, zp_mid, relu1)
+        q2 = ops.fold_zero_point_gemm(B2, b2, zp_mid, True)
+        ref = oracle.qgemm_s8(T, B2, s2, q2, True, 0, zpy, relu2)
+        got = ops.qgemm_s8_pair(A, B1, s1, b1, zp_mid, relu1, B2, s2, q2, zpy, relu2)
+        assert np.array_equal(got, ref), (zp_mid, relu1, zpy, relu2)
+        reff = oracle.qgemm_s8_f32out(T, B2, s2, q2, True, 0, relu2)
+        gotf = ops.qgemm_s8_pair(A, B1, s1, b1, zp_mid, relu1, B2, s2, q2, 0, relu2, out=L.OUT_F32)
+        assert np.array_equal(gotf, reff)
