@@ -24,4 +24,8 @@ struct QConvArgs {
 // with a 2x2 stride-2 max pooling: *done tells whether the kernel took the problem.
 int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done);
 
+// 3x3 kernel, stride 1, 32 or 64 input channels, channels-last int8 in and out: the kernel that fetches the
+// input rows straight into LDS. *done tells whether the kernel took the problem.
+int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done);
+
 }  // namespace sofie

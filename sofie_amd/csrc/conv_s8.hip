@@ -491,6 +491,10 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
 {
    *done = false;
    const bool pool = g.pool_kh != 0;
+   if constexpr (OUT == SOFIE_OUT_S8) {
+      if (int rc = qconv_ring(ctx, g, done)) return rc;
+      if (*done) return SOFIE_HIP_OK;
+   }
    if (g.groups != 1 || g.C % 32 != 0 || g.OC % 64 != 0 || !g.x_nhwc || !g.y_nhwc || !g.w_ohwi) return SOFIE_HIP_OK;
    if (!aligned16(g.x) || !aligned16(g.w) || !aligned16(g.y)) return SOFIE_HIP_OK;
    if (pool && !(OUT == SOFIE_OUT_S8 && g.pool_kh == 2 && g.pool_kw == 2 && g.pool_sh == 2 && g.pool_sw == 2)) return SOFIE_HIP_OK;

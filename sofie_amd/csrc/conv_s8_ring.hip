@@ -1,0 +1,367 @@
+// int8 3x3 stride-1 convolution on the matrix cores whose input travels global memory -> LDS without registers.
+//
+// k_qconv_ring: the implicit GEMM of conv_s8.hip (NHWC activations, weights [OC][3][3][C], C = 32 or 64, the
+// workgroup's weight slice resident in LDS, 8 wavefronts of 2 x 2 accumulator tiles of 32 x 32) with another way of
+// getting the input there:
+//   * a workgroup owns a CONTIGUOUS run of pixel tiles of the linear (n, oh, ow) order, so the rows of the padded
+//     images it needs ("virtual rows": image n, padded row r -> n*HP + r) form a window that slides down; they
+//     live in a ring of R rows in LDS (row v in slot v % R). A tile only fetches the rows the previous tile did not
+//     have, and they are fetched while the previous tile is multiplied: the ring has room for the rows of two
+//     consecutive tiles.
+//   * rows are fetched with buffer_load_dwordx4 ... lds: a wavefront instruction moves 64 x 16 bytes into 1 KB of
+//     consecutive LDS, the global address is free per lane. A ring row is stored as C/16 planes
+//     [16-byte channel chunk][padded column][16 bytes]; one instruction fills one plane of one row (lane = padded
+//     column, lanes of padding columns switched off). The vector unit spends nothing on staging: no address
+//     arithmetic per 16 bytes, no registers, no LDS writes. Padding columns are written once with the input
+//     zero-point when the kernel starts, padding rows by one LDS write per plane when such a row enters the ring.
+//   * in a plane consecutive pixels are 16 bytes apart, so the 16-byte-per-lane operand read of consecutive pixels
+//     covers consecutive banks; the row pitch is padded so that this also holds across the end of an output row.
+//     The nine taps of a pixel are its base address (per kernel row and channel half) plus a constant.
+#include "common.h"
+#include "conv_s8.h"
+#include "gemm_tile.h"
+
+using namespace sofie;
+
+namespace {
+
+struct QConvRingArgs {
+   const int8_t *x;      // NHWC
+   const int8_t *w;      // [OC][3][3][C]
+   GemmArgs ep;          // Y, scale, bias, M = N*OH*OW, N = OC, ldy = OC, zp, lo, relu
+   int H, W, C, ph, pw, OH, OW, HP, WP;
+   int K, KS;            // bytes of one weight row, its LDS stride
+   int RS, PL, R;        // ring: row pitch and plane pitch in bytes, rows (a power of two)
+   int row_bytes;        // W * C: one image row in global memory
+   unsigned fill;        // zp_x replicated into four bytes
+   unsigned xbytes;
+   FastDiv dOW, dOH, dHP, dK16;
+};
+
+// C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels (tile = (8/WN)*64 pixels x WN*64 channels)
+template <int C16, int WN>
+__global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
+{
+   constexpr int MB = 2, NB = 2;
+   constexpr int WM = 8 / WN;
+   constexpr int TM = WM * MB * 32;
+   constexpr int OCT = WN * NB * 32;
+   constexpr int CB = C16 / 2;                      // 32-channel blocks
+   constexpr int NS = 9 * CB;                       // K steps of 32 bytes
+   constexpr int NRL = 8 / C16;                     // wavefronts that share the rows of one plane index
+   extern __shared__ __align__(16) unsigned char smem[];
+   unsigned char *const s_w = smem;                                        // [OCT][KS]
+   float *const s_scale = reinterpret_cast<float *>(smem + OCT * a.KS);    // [OCT]
+   int *const s_bias = reinterpret_cast<int *>(s_scale + OCT);             // [OCT]
+   unsigned char *const s_ring = reinterpret_cast<unsigned char *>(s_bias + OCT);   // [R][C16][WP][16] (+ row pad)
+   const unsigned ring0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)s_ring;
+
+   const int tid = threadIdx.x, lane = tid & 63;
+   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+   const int wn = wave % WN, wm = wave / WN;
+   const int half = lane >> 5, l32 = lane & 31;
+   const int nob = a.ep.N / OCT;
+   const int ob = blockIdx.x % nob;
+   const int wg = blockIdx.x / nob, nwg = gridDim.x / nob;
+   // The workgroup's run of pixels, dealt out in units of the 64 pixels a wavefront multiplies: its tiles start at
+   // m_begin, and of the last, partial one only the wavefronts whose pixels lie inside the run do any work.
+   constexpr int UNIT = MB * 32;
+   const int units = (a.ep.M + UNIT - 1) / UNIT;
+   const int m_begin = (int)((long long)wg * units / nwg) * UNIT;
+   const int m_stop = (int)((long long)(wg + 1) * units / nwg) * UNIT;
+   const int mtot = m_stop < a.ep.M ? m_stop : a.ep.M;       // one past the last pixel of the run
+   const int t0 = 0, t1 = (mtot - m_begin + TM - 1) / TM;
+   GemmArgs ep = a.ep;
+   ep.M = mtot;
+   const int rmask = a.R - 1;
+
+   // ---- weights of this channel block: resident for the life of the workgroup (eight loads in flight per thread)
+   {
+      constexpr int WCH = 8;
+      const int K16 = a.K >> 4;
+      const int total = OCT * K16;
+      const int8_t *wsrc = a.w + (size_t)ob * OCT * a.K;
+      for (int base = tid; base < total; base += 512 * WCH) {
+         v4i chunk[WCH];
+#pragma unroll
+         for (int u = 0; u < WCH; ++u) {
+            const int q = base + u * 512;
+            chunk[u] = *reinterpret_cast<const v4i *>(wsrc + (size_t)(q < total ? q : base) * 16);
+         }
+#pragma unroll
+         for (int u = 0; u < WCH; ++u) {
+            const int q = base + u * 512;
+            const int r = fdiv(q, a.dK16);
+            if (q < total) *reinterpret_cast<v4i *>(s_w + r * a.KS + (q - r * K16) * 16) = chunk[u];
+         }
+      }
+   }
+   stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
+   const v4i fillv = {(int)a.fill, (int)a.fill, (int)a.fill, (int)a.fill};
+   // padding columns of every ring row hold the input zero-point for the life of the kernel
+   {
+      const int npad = a.WP - a.W;
+      for (int q = tid; q < a.R * C16 * npad; q += 512) {
+         const int rc = q / npad, pc = q - rc * npad;
+         const int r = rc / C16, c = rc - r * C16;
+         const int wp = pc < a.pw ? pc : pc + a.W;
+         *reinterpret_cast<v4i *>(s_ring + r * a.RS + c * a.PL + wp * 16) = fillv;
+      }
+   }
+
+   // ---- rows of the padded images -> ring. Wavefront w fills plane w % C16 of every NRL-th row.
+   const rsrc_t rs = make_rsrc(a.x, a.xbytes);
+   const int my_plane = wave % C16, my_rl = wave / C16;
+   const int iw = lane - a.pw;
+   const bool col_data = iw >= 0 && iw < a.W;
+   const int voff = iw * a.C + my_plane * 16;
+   auto load_rows = [&](int from, int to) {
+      for (int v = from + my_rl; v <= to; v += NRL) {
+         const int n = fdiv(v, a.dHP);
+         const int ih = v - n * a.HP - a.ph;
+         const unsigned dst = (unsigned)((v & rmask) * a.RS + my_plane * a.PL);
+         if (ih >= 0 && ih < a.H) {
+            if (col_data) dma16(rs, ring0 + dst, voff, (n * a.H + ih) * a.row_bytes);
+         } else if (lane < a.WP) {
+            *reinterpret_cast<v4i *>(s_ring + dst + lane * 16) = fillv;
+         }
+      }
+   };
+   // first and last virtual row a tile reads
+   auto first_row = [&](int t) {
+      const int R0 = fdiv(m_begin + t * TM, a.dOW);
+      const int n0 = fdiv(R0, a.dOH);
+      return n0 * a.HP + (R0 - n0 * a.OH);
+   };
+   auto last_row = [&](int t) {
+      const int mlast = (m_begin + (t + 1) * TM < mtot ? m_begin + (t + 1) * TM : mtot) - 1;
+      const int R1 = fdiv(mlast, a.dOW);
+      const int n1 = fdiv(R1, a.dOH);
+      return n1 * a.HP + (R1 - n1 * a.OH) + 2;
+   };
+
+   int b_off[NB];
+#pragma unroll
+   for (int i = 0; i < NB; ++i) b_off[i] = ((wn * NB + i) * 32 + l32) * a.KS + half * 16;
+   const int nq = half * 4;
+   const float *const w_scale = s_scale + wn * NB * 32;
+   const int *const w_bias = s_bias + wn * NB * 32;
+   const bool plain = a.ep.zp == -128 && a.ep.lo == -128;
+
+   // LDS offsets of the wavefront's pixels in the ring, per kernel row and 32-channel block: the lane's half of the
+   // block is plane 2*cb + half; the column tap kw is the constant kw*16 on top
+   const unsigned char *pa[3][CB][MB];
+   const unsigned char *const lane_base = s_ring + half * a.PL;
+   auto pixel_offsets = [&](int tt) {
+#pragma unroll
+      for (int j = 0; j < MB; ++j) {
+         int m = m_begin + tt * TM + (wm * MB + j) * 32 + l32;
+         m = m < mtot ? m : mtot - 1;
+         const int R = fdiv(m, a.dOW);
+         const int ow = m - R * a.OW;
+         const int n = fdiv(R, a.dOH);
+         const int v = n * a.HP + (R - n * a.OH);
+         const unsigned char *const colb = lane_base + ow * 16;
+#pragma unroll
+         for (int kh = 0; kh < 3; ++kh) {
+            const unsigned char *const rowb = colb + ((v + kh) & rmask) * a.RS;
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) pa[kh][cb][j] = rowb + cb * 2 * a.PL;
+         }
+      }
+   };
+
+   v16i r_bias[NB];
+   v4f r_scale[NB * 4];
+   // K loop of one tile: unrolled over its 9 * CB steps; the fragment reads run two steps ahead of the matrix
+   // instructions and one read is issued behind each of a step's first matrix instructions
+   auto kloop = [&](v16i (&acc)[NB][MB]) {
+      constexpr int NBUF = 3;
+      v4i fa[NBUF][MB], fb[NBUF][NB];
+      const unsigned char *pb[NB];
+#pragma unroll
+      for (int i = 0; i < NB; ++i) pb[i] = s_w + b_off[i];
+#pragma unroll
+      for (int s = 0; s < NS + NBUF - 1; ++s) {
+         if (s < NS) {
+            const int kh = s / (3 * CB), kw = (s / CB) % 3, cb = s % CB;
+            fb[s % NBUF][0] = *reinterpret_cast<const v4i *>(pb[0] + s * 32);
+#pragma unroll
+            for (int j = 0; j < MB; ++j)
+               fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[kh][cb][j] + kw * 16);
+#pragma unroll
+            for (int i = 1; i < NB; ++i) fb[s % NBUF][i] = *reinterpret_cast<const v4i *>(pb[i] + s * 32);
+         }
+         if (s >= NBUF - 1) {
+            const int d = s - (NBUF - 1), buf = d % NBUF;
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+               for (int j = 0; j < MB; ++j) {
+                  if (d == 0) acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], r_bias[i]);
+                  else acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], acc[i][j]);
+               }
+         }
+         if (s < NS && s >= NBUF - 1) {
+#pragma unroll
+            for (int gidx = 0; gidx < MB + NB; ++gidx) {
+               __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
+               __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+            }
+         }
+         __builtin_amdgcn_sched_barrier(0);
+      }
+   };
+   auto epilogue = [&](v16i (&acc)[NB][MB], int tt) {
+      const int m_wave = m_begin + tt * TM + wm * MB * 32, n_wave = ob * OCT + wn * NB * 32;
+      if (plain) tile_epilogue_s8_direct<NB, MB, true, false>(ep, acc, w_scale, w_bias, lane, m_wave, n_wave, &r_scale);
+      else tile_epilogue_s8_direct<NB, MB, false, false>(ep, acc, w_scale, w_bias, lane, m_wave, n_wave, &r_scale);
+   };
+   // whether the wavefront has pixels in tile tt (all tiles but the last are full)
+   auto has_work = [&](int tt) { return m_begin + tt * TM + wm * MB * 32 < mtot; };
+
+   // The two wavefronts that share a SIMD do their halves in opposite order (wavefronts 0-3: matrix loop of tile t,
+   // then its epilogue; wavefronts 4-7: epilogue of their previous tile, then the matrix loop of tile t).
+   const bool mma_first = wave < 4;
+   int t = t0, t_prev = -1, hi_cur = 0;
+   if (t < t1) {
+      hi_cur = last_row(t);
+      load_rows(first_row(t), hi_cur);
+      pixel_offsets(t);
+   }
+   wait_vmcnt<0>();
+   __syncthreads();                          // weights, column parameters, padding columns and the first rows are in LDS
+#pragma unroll
+   for (int gi = 0; gi < NB * 4; ++gi) {
+      r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+      const v4i bi = *reinterpret_cast<const v4i *>(w_bias + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r_bias[gi >> 2][(gi & 3) * 4 + e] = bi[e];
+   }
+   v16i acc[NB][MB];
+   // rows tile t + 1 has and tile t does not: requested at the start of tile t into slots that tile t does not read
+   auto request_next = [&](bool more, int tn, int &hi_next) {
+      if (more) {
+         hi_next = last_row(tn);
+         load_rows(hi_cur + 1, hi_next);
+      }
+   };
+   // One loop per group, so that the accumulators of each have one home in the register file. Both run t1 - t0
+   // iterations with one workgroup barrier each: it says that the rows of the next tile are complete (every
+   // wavefront has waited for its own requests) and that every wavefront is done reading the present tile.
+   if (mma_first) {
+      while (t < t1) {
+         const int tn = t + 1;
+         const bool more = tn < t1;
+         int hi_next = hi_cur;
+         request_next(more, tn, hi_next);
+         if (has_work(t)) {
+            kloop(acc);
+            wait_vmcnt<0>();                 // before this tile's stores join the queue
+            epilogue(acc, t);
+         } else {
+            wait_vmcnt<0>();
+         }
+         if (more) pixel_offsets(tn);
+         t = tn;
+         hi_cur = hi_next;
+         __syncthreads();
+      }
+   } else {
+      while (t < t1) {
+         const int tn = t + 1;
+         const bool more = tn < t1;
+         int hi_next = hi_cur;
+         request_next(more, tn, hi_next);
+         if (t_prev >= 0) epilogue(acc, t_prev);
+         const bool work = has_work(t);
+         if (work) kloop(acc);
+         wait_vmcnt<0>();
+         if (more) pixel_offsets(tn);
+         t_prev = work ? t : -1;
+         t = tn;
+         hi_cur = hi_next;
+         __syncthreads();
+      }
+      if (t_prev >= 0) epilogue(acc, t_prev);
+   }
+}
+
+}  // namespace
+
+namespace sofie {
+
+// 3x3, stride 1, 32 or 64 input channels, channels-last int8 in and out, no fused pooling.
+int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
+{
+   *done = false;
+   if (g.pool_kh != 0 || g.xf) return SOFIE_HIP_OK;
+   if (g.groups != 1 || !(g.C == 32 || g.C == 64) || g.OC % 64 != 0 || !g.x_nhwc || !g.y_nhwc || !g.w_ohwi) return SOFIE_HIP_OK;
+   if (g.KH != 3 || g.KW != 3 || g.sh != 1 || g.sw != 1) return SOFIE_HIP_OK;
+   if (!aligned16(g.x) || !aligned16(g.w) || !aligned16(g.y)) return SOFIE_HIP_OK;
+   const long long mtot = (long long)g.N * g.OH * g.OW;
+   const int HP = g.H + g.ph + g.pbh, WP = g.W + g.pw + g.pbw;
+   if (mtot <= 0 || WP > 64) return SOFIE_HIP_OK;
+   if (mtot >= (1ll << 31) - 1024 || (long long)g.N * HP >= (1ll << 31) - 4096) return SOFIE_HIP_OK;
+   const size_t xbytes = (size_t)g.N * g.H * g.W * g.C;
+   if (xbytes >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
+   const int WN = g.OC % 128 == 0 ? 2 : 1;
+   const int OCT = WN * 64, TM = (8 / WN) * 64;   // workgroup tile: TM pixels x OCT channels
+   const int C16 = g.C / 16;
+   QConvRingArgs a{};
+   a.x = g.x; a.w = g.w;
+   a.ep.Y = g.y; a.ep.scale = g.scale; a.ep.bias = g.bias;
+   a.ep.M = (int)mtot; a.ep.N = g.OC; a.ep.ldy = g.OC;
+   a.ep.zp = g.zpy; a.ep.lo = g.lo; a.ep.relu = g.relu; a.ep.s = 1.0f;
+   a.ep.vec_store = 1;
+   a.H = g.H; a.W = g.W; a.C = g.C; a.ph = g.ph; a.pw = g.pw;
+   a.OH = g.OH; a.OW = g.OW; a.HP = HP; a.WP = WP;
+   a.K = 9 * g.C;
+   a.KS = ((a.K / 16) % 2 == 0) ? a.K + 16 : a.K;
+   a.PL = WP * 16;
+   // Row pitch: consecutive pixels of an output row are 16 bytes apart; padded so that the first pixel of the next
+   // output row continues that sequence modulo the 256 bytes the LDS banks span.
+   a.RS = C16 * a.PL;
+   a.RS += (((g.OW * 16 - a.RS) % 256) + 256) % 256;
+   a.row_bytes = g.W * g.C;
+   a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
+   a.xbytes = (unsigned)xbytes;
+   a.dOW = make_fastdiv(g.OW); a.dOH = make_fastdiv(g.OH); a.dHP = make_fastdiv(HP); a.dK16 = make_fastdiv(a.K / 16);
+   // the ring holds the rows of two consecutive tiles: the output rows 2*TM consecutive pixels can touch, the padding
+   // rows between the images they can span (HP - OH = 2 per image boundary) and the two extra rows of the last window
+   const int rows2 = (2 * TM - 1) / g.OW + 2;
+   int crossings = (rows2 - 1) / g.OH + 1;
+   if (crossings > g.N - 1) crossings = g.N - 1;
+   const int window = rows2 + 2 * crossings + 2;
+   int R = 8;
+   while (R < window) R *= 2;
+   a.R = R;
+   const size_t lds = (size_t)OCT * a.KS + (size_t)OCT * 8 + (size_t)R * a.RS;
+   if (lds > 160 * 1024) return SOFIE_HIP_OK;
+   if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
+   const int nob = g.OC / OCT;
+   int per = ctx->num_cus / nob;
+   if (per < 1) per = 1;
+   const int units = (int)((mtot + 63) / 64);
+   if (per > units) per = units;
+   const dim3 grid((unsigned)(per * nob)), block(512);
+#define SOFIE_QRING_LAUNCH(C16_, WN_)                                                                          \
+   do {                                                                                                        \
+      auto kern = k_qconv_ring<C16_, WN_>;                                                                     \
+      SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                            \
+                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));          \
+      hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                              \
+   } while (0)
+   if (C16 == 4) {
+      if (WN == 2) SOFIE_QRING_LAUNCH(4, 2);
+      else SOFIE_QRING_LAUNCH(4, 1);
+   } else {
+      if (WN == 2) SOFIE_QRING_LAUNCH(2, 2);
+      else SOFIE_QRING_LAUNCH(2, 1);
+   }
+#undef SOFIE_QRING_LAUNCH
+   *done = true;
+   return check_launch(ctx, "k_qconv_ring");
+}
+
+}  // namespace sofie

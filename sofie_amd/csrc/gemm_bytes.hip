@@ -321,36 +321,6 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16 || NSETS > 2) ? 1 : 2) k_g
 #define SOFIE_DMA_BK 128   // bytes of K per LDS stage of k_gemm_dma
 #define SOFIE_DMA_NST 2    // LDS stages
 #endif
-typedef int rsrc_t __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ rsrc_t make_rsrc(const void *base, unsigned bytes)
-{
-   // every component is wave-uniform; readfirstlane tells the compiler so (SGPR operands)
-   const unsigned long long a = reinterpret_cast<unsigned long long>(base);
-   rsrc_t r = {__builtin_amdgcn_readfirstlane((int)(unsigned)a),
-               __builtin_amdgcn_readfirstlane((int)(unsigned)((a >> 32) & 0xffffu)),
-               __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
-   return r;
-}
-
-// 16 bytes per lane from global (descriptor + per-lane offset + uniform offset) to
-// LDS address lds_base + lane*16.
-__device__ __forceinline__ void dma16(rsrc_t rs, unsigned lds_base, int voff, int soff)
-{
-   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
-                :
-                : "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "v"(voff), "s"(rs),
-                  "s"(__builtin_amdgcn_readfirstlane(soff))
-                : "memory");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-   // s_waitcnt with only the vector-memory counter constrained
-   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-}
-
 template <int S> struct StageTag { static constexpr int value = S; };
 
 // LDS of k_gemm_dma: [A stage 0][A stage 1][B stage 0][B stage 1], BM*BK (BN*BK) bytes each. Both stages of an

@@ -298,4 +298,35 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::A
                                               n0 + wn * WN);
 }
 
+// ---- global memory -> LDS without registers (buffer_load ... lds), shared by the GEMM and the convolution
+typedef int rsrc_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, unsigned bytes)
+{
+   // every component is wave-uniform; readfirstlane tells the compiler so (SGPR operands)
+   const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+   rsrc_t r = {__builtin_amdgcn_readfirstlane((int)(unsigned)a),
+               __builtin_amdgcn_readfirstlane((int)(unsigned)((a >> 32) & 0xffffu)),
+               __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000};
+   return r;
+}
+
+// 16 bytes per lane from global (descriptor + per-lane offset + uniform offset) to
+// LDS address lds_base + lane*16.
+__device__ __forceinline__ void dma16(rsrc_t rs, unsigned lds_base, int voff, int soff)
+{
+   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                :
+                : "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "v"(voff), "s"(rs),
+                  "s"(__builtin_amdgcn_readfirstlane(soff))
+                : "memory");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+   // s_waitcnt with only the vector-memory counter constrained
+   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
 }  // namespace sofie

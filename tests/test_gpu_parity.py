@@ -422,6 +422,13 @@ def test_qconv2d_s8(ops, cfg):
     dict(N=5, C=32, H=12, W=12, OC=64, k=(4, 4), p=(2, 2, 1, 1), s=(1, 1)),
     dict(N=3, C=64, H=16, W=14, OC=128, k=(3, 3), p=(0, 0, 1, 1), s=(2, 2)),
     dict(N=4, C=32, H=9, W=10, OC=64, k=(3, 3), p=(2, 0, 0, 1), s=(1, 1)),
+    # 3x3 stride 1 on 32 / 64 channels, rows fetched straight into LDS: the widest padded row it takes (64 columns) and
+    # one column more (the register-staged kernel), enough pixels for several tiles per workgroup (the window of rows
+    # slides through many images), a run of pixels per workgroup that ends inside a tile
+    dict(N=2, C=64, H=9, W=62, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=2, C=32, H=9, W=63, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=1000, C=32, H=19, W=21, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=11, C=64, H=50, W=47, OC=128, k=(3, 3), p=(0, 1, 1, 0), s=(1, 1)),
 ])
 def test_qconv2d_s8_matrix_core_path(ops, cfg):
     """NHWC activations and [OC,KH,KW,C] weights straight into the MFMA kernel; NCHW operands of the same
@@ -836,6 +843,17 @@ def test_qconv2d_s8_full_size_layer(ops):
     S = _window_sums(x.transpose(0, 3, 1, 2).astype(np.int64) + 128, 3, 1, H, H)    # x - zp_x, zero outside the image
     want = np.einsum("ockl,nckl->no", wn.astype(np.int64), S)
     assert np.array_equal(got, want)
+    # Every int8 output is the requantisation of its accumulator (the int8 launch and the accumulator launch
+    # are different kernels). The vectorised formula is tied to the oracle's on a sample first.
+    def requant_all(v):
+        q = np.rint((v + bias).astype(np.float32) * scale) - 128.0
+        return np.clip(q, -128, 127).astype(np.int8)
+    sample = acc[17, 23].reshape(-1, OC)[:40]
+    for row in sample:
+        for c in range(0, OC, 9):
+            assert requant_all(row)[c] == oracle.requant_one(int(row[c]) + int(bias[c]), float(scale[c]), -128, True)
+    for n0 in range(0, N, 32):
+        assert np.array_equal(requant_all(acc[n0:n0 + 32]), y[n0:n0 + 32]), n0
 
 
 def test_conv2d_f32_full_size_layer(ops):
