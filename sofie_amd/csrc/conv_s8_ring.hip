@@ -25,6 +25,11 @@ using namespace sofie;
 
 namespace {
 
+#ifndef SOFIE_RING_STORE
+#define SOFIE_RING_STORE(p, v) (*(p) = (v))
+#endif
+template <bool B> struct BoolTag { static constexpr bool value = B; };
+
 struct QConvRingArgs {
    const int8_t *x;      // NHWC
    const int8_t *w;      // [OC][3][3][C]
@@ -35,20 +40,24 @@ struct QConvRingArgs {
    int row_bytes;        // W * C: one image row in global memory
    unsigned fill;        // zp_x replicated into four bytes
    unsigned xbytes;
-   FastDiv dOW, dOH, dHP, dK16;
+   FastDiv dOW, dOH, dHP, dK16, dR;
 };
 
-// C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels (tile = (8/WN)*64 pixels x WN*64 channels)
+// C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels. The tile is (8/WN)*64 pixels x
+// WN*64 channels. (Twelve wavefronts per workgroup, three per SIMD, and wavefront tiles of 96 pixels were measured
+// on the 56x56 layer: the same time within 1 %.)
 template <int C16, int WN>
 __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
 {
    constexpr int MB = 2, NB = 2;
-   constexpr int WM = 8 / WN;
+   constexpr int NWAVE = 8, NT = NWAVE * 64;
+   constexpr bool REGS = true;                     // scales and bias tiles in registers
+   constexpr int WM = NWAVE / WN;
    constexpr int TM = WM * MB * 32;
    constexpr int OCT = WN * NB * 32;
    constexpr int CB = C16 / 2;                      // 32-channel blocks
    constexpr int NS = 9 * CB;                       // K steps of 32 bytes
-   constexpr int NRL = 8 / C16;                     // wavefronts that share the rows of one plane index
+   constexpr int NRL = NWAVE / C16;                 // wavefronts that share the rows of one plane index
    extern __shared__ __align__(16) unsigned char smem[];
    unsigned char *const s_w = smem;                                        // [OCT][KS]
    float *const s_scale = reinterpret_cast<float *>(smem + OCT * a.KS);    // [OCT]
@@ -73,7 +82,6 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    const int t0 = 0, t1 = (mtot - m_begin + TM - 1) / TM;
    GemmArgs ep = a.ep;
    ep.M = mtot;
-   const int rmask = a.R - 1;
 
    // ---- weights of this channel block: resident for the life of the workgroup (eight loads in flight per thread)
    {
@@ -81,16 +89,16 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       const int K16 = a.K >> 4;
       const int total = OCT * K16;
       const int8_t *wsrc = a.w + (size_t)ob * OCT * a.K;
-      for (int base = tid; base < total; base += 512 * WCH) {
+      for (int base = tid; base < total; base += NT * WCH) {
          v4i chunk[WCH];
 #pragma unroll
          for (int u = 0; u < WCH; ++u) {
-            const int q = base + u * 512;
+            const int q = base + u * NT;
             chunk[u] = *reinterpret_cast<const v4i *>(wsrc + (size_t)(q < total ? q : base) * 16);
          }
 #pragma unroll
          for (int u = 0; u < WCH; ++u) {
-            const int q = base + u * 512;
+            const int q = base + u * NT;
             const int r = fdiv(q, a.dK16);
             if (q < total) *reinterpret_cast<v4i *>(s_w + r * a.KS + (q - r * K16) * 16) = chunk[u];
          }
@@ -101,7 +109,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // padding columns of every ring row hold the input zero-point for the life of the kernel
    {
       const int npad = a.WP - a.W;
-      for (int q = tid; q < a.R * C16 * npad; q += 512) {
+      for (int q = tid; q < a.R * C16 * npad; q += NT) {
          const int rc = q / npad, pc = q - rc * npad;
          const int r = rc / C16, c = rc - r * C16;
          const int wp = pc < a.pw ? pc : pc + a.W;
@@ -115,17 +123,44 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    const int iw = lane - a.pw;
    const bool col_data = iw >= 0 && iw < a.W;
    const int voff = iw * a.C + my_plane * 16;
-   auto load_rows = [&](int from, int to) {
-      for (int v = from + my_rl; v <= to; v += NRL) {
-         const int n = fdiv(v, a.dHP);
-         const int ih = v - n * a.HP - a.ph;
-         const unsigned dst = (unsigned)((v & rmask) * a.RS + my_plane * a.PL);
-         if (ih >= 0 && ih < a.H) {
-            if (col_data) dma16(rs, ring0 + dst, voff, (n * a.H + ih) * a.row_bytes);
-         } else if (lane < a.WP) {
-            *reinterpret_cast<v4i *>(s_ring + dst + lane * 16) = fillv;
+   // A request is scalar work plus one instruction per row; it is spread over the matrix loop of the present tile
+   // (one row per call of req_step, between two K steps), where the scalar unit and the memory pipeline have nothing
+   // else to do, instead of standing in front of it. The wavefront's rows inside one image are walked as a run: one
+   // division per run, then additions only.
+   const unsigned ring_end = ring0 + (unsigned)(a.R * a.RS) + (unsigned)(my_plane * a.PL);
+   int rq_v = 0, rq_to = -1, rq_left = 0, rq_soff = 0;
+   unsigned rq_dst = 0;
+   auto req_begin = [&](int from, int to) {
+      rq_v = from + my_rl;
+      rq_to = to;
+      rq_left = 0;
+   };
+   auto req_step = [&]() {
+      if (rq_v > rq_to) return;
+      if (rq_left == 0) {
+         const int n = fdiv(rq_v, a.dHP);
+         const int ih = rq_v - n * a.HP - a.ph;
+         rq_dst = ring0 + (unsigned)((rq_v - fdiv(rq_v, a.dR) * a.R) * a.RS + my_plane * a.PL);
+         if ((unsigned)ih < (unsigned)a.H) {
+            const int in_image = (a.H - 1 - ih) / NRL, wanted = (rq_to - rq_v) / NRL;
+            rq_left = (in_image < wanted ? in_image : wanted) + 1;
+            rq_soff = (n * a.H + ih) * a.row_bytes;
+         } else {
+            // a padding row between two images (or above the first, below the last)
+            if (lane < a.WP) *reinterpret_cast<v4i *>(s_ring + (rq_dst - ring0) + lane * 16) = fillv;
+            rq_v += NRL;
+            return;
          }
       }
+      if (col_data) dma16(rs, rq_dst, voff, rq_soff);
+      rq_soff += NRL * a.row_bytes;
+      rq_dst += NRL * a.RS;
+      if (rq_dst >= ring_end) rq_dst -= a.R * a.RS;
+      rq_v += NRL;
+      --rq_left;
+   };
+   auto req_finish = [&]() {
+      while (rq_v <= rq_to) req_step();
    };
    // first and last virtual row a tile reads
    auto first_row = [&](int t) {
@@ -157,22 +192,27 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       for (int j = 0; j < MB; ++j) {
          int m = m_begin + tt * TM + (wm * MB + j) * 32 + l32;
          m = m < mtot ? m : mtot - 1;
-         const int R = fdiv(m, a.dOW);
+         // OW and OH are at least 2 (the launcher sees to it): the divisions are a multiply-high and a shift
+         const int R = (int)(__umulhi((unsigned)m, a.dOW.magic) >> a.dOW.shift);
          const int ow = m - R * a.OW;
-         const int n = fdiv(R, a.dOH);
-         const int v = n * a.HP + (R - n * a.OH);
+         const int n = (int)(__umulhi((unsigned)R, a.dOH.magic) >> a.dOH.shift);
+         const int v = R + n * 2;                       // n * HP + (R - n * OH), HP - OH = 2
          const unsigned char *const colb = lane_base + ow * 16;
+         // ring slots of the three rows: v % R, then one step at a time with the wrap
+         unsigned slot = (unsigned)v - (__umulhi((unsigned)v, a.dR.magic) >> a.dR.shift) * (unsigned)a.R;
 #pragma unroll
          for (int kh = 0; kh < 3; ++kh) {
-            const unsigned char *const rowb = colb + ((v + kh) & rmask) * a.RS;
+            const unsigned char *const rowb = colb + slot * a.RS;
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) pa[kh][cb][j] = rowb + cb * 2 * a.PL;
+            slot = slot + 1;
+            slot = slot < slot - (unsigned)a.R ? slot : slot - (unsigned)a.R;   // min(slot, slot - R): slot - R wraps below R
          }
       }
    };
 
-   v16i r_bias[NB];
-   v4f r_scale[NB * 4];
+   v16i r_bias[REGS ? NB : 1];
+   v4f r_scale[REGS ? NB * 4 : 1];
    // K loop of one tile: unrolled over its 9 * CB steps; the fragment reads run two steps ahead of the matrix
    // instructions and one read is issued behind each of a step's first matrix instructions
    auto kloop = [&](v16i (&acc)[NB][MB]) {
@@ -181,6 +221,18 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       const unsigned char *pb[NB];
 #pragma unroll
       for (int i = 0; i < NB; ++i) pb[i] = s_w + b_off[i];
+      v16i bias_tile[NB];
+      if constexpr (REGS) {
+#pragma unroll
+         for (int i = 0; i < NB; ++i) bias_tile[i] = r_bias[i];
+      } else {
+#pragma unroll
+         for (int gi = 0; gi < NB * 4; ++gi) {
+            const v4i bi = *reinterpret_cast<const v4i *>(w_bias + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bias_tile[gi >> 2][(gi & 3) * 4 + e] = bi[e];
+         }
+      }
 #pragma unroll
       for (int s = 0; s < NS + NBUF - 1; ++s) {
          if (s < NS) {
@@ -198,7 +250,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             for (int i = 0; i < NB; ++i)
 #pragma unroll
                for (int j = 0; j < MB; ++j) {
-                  if (d == 0) acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], r_bias[i]);
+                  if (d == 0) acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], bias_tile[i]);
                   else acc[i][j] = MmaI8::mma(fb[buf][i], fa[buf][j], acc[i][j]);
                }
          }
@@ -208,45 +260,88 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
             }
+            if constexpr (MB * NB > MB + NB) __builtin_amdgcn_sched_group_barrier(0x008, MB * NB - (MB + NB), 0);
          }
          __builtin_amdgcn_sched_barrier(0);
+         if (s < NS && (s & 1)) req_step();
+      }
+      req_finish();
+   };
+   // Requantisation and stores of one tile: a lane packs its four 4-channel groups of an accumulator tile into four
+   // dwords, two swaps between the halves of the wavefront turn them into 16 consecutive channels, one 16-byte store.
+   // (A store instruction so touches 32 pixels with 32 bytes each. Stores of 64 contiguous bytes per pixel, 16
+   // pixels per instruction, take 5 % off the layer when the bytes are there for free, but moving them between lanes
+   // through a private block of LDS costs what they gain.)
+   auto epilogue_as = [&](v16i (&acc)[NB][MB], int tt, auto plain_tag) {
+      constexpr bool PLAIN = decltype(plain_tag)::value;
+      const int m_wave = m_begin + tt * TM + wm * MB * 32, n_wave = ob * OCT + wn * NB * 32;
+      const float zpo = (float)(ep.zp + 128), lof = (float)(ep.lo + 128);
+#pragma unroll
+      for (int j = 0; j < MB; ++j) {
+         const int m = m_wave + j * 32 + l32;
+         int8_t *const row = static_cast<int8_t *>(ep.Y) + (size_t)(m < ep.M ? m : 0) * ep.ldy + n_wave + half * 16;
+#pragma unroll
+         for (int i = 0; i < NB; ++i) {
+            unsigned d[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+               const v4f sc = r_scale[i * 4 + q];
+               unsigned pk = 0;
+#pragma unroll
+               for (int e = 0; e < 4; ++e) {
+                  // the accumulators started from the bias; the byte conversion rounds half to even and saturates
+                  float r = __fmul_rn(__int2float_rn(acc[i][j][q * 4 + e]), sc[e]);
+                  if constexpr (!PLAIN) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
+                  pk = __builtin_amdgcn_cvt_pk_u8_f32(r, e, pk);
+               }
+               d[q] = pk ^ 0x80808080u;
+            }
+            const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+            const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+            const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+            if (m < ep.M) SOFIE_RING_STORE(reinterpret_cast<v4i *>(row + i * 32), v);
+         }
       }
    };
    auto epilogue = [&](v16i (&acc)[NB][MB], int tt) {
-      const int m_wave = m_begin + tt * TM + wm * MB * 32, n_wave = ob * OCT + wn * NB * 32;
-      if (plain) tile_epilogue_s8_direct<NB, MB, true, false>(ep, acc, w_scale, w_bias, lane, m_wave, n_wave, &r_scale);
-      else tile_epilogue_s8_direct<NB, MB, false, false>(ep, acc, w_scale, w_bias, lane, m_wave, n_wave, &r_scale);
+      if (plain) epilogue_as(acc, tt, BoolTag<true>{});
+      else epilogue_as(acc, tt, BoolTag<false>{});
    };
    // whether the wavefront has pixels in tile tt (all tiles but the last are full)
    auto has_work = [&](int tt) { return m_begin + tt * TM + wm * MB * 32 < mtot; };
 
-   // The two wavefronts that share a SIMD do their halves in opposite order (wavefronts 0-3: matrix loop of tile t,
-   // then its epilogue; wavefronts 4-7: epilogue of their previous tile, then the matrix loop of tile t).
+   // The wavefronts that share a SIMD (w, w + 4[, w + 8]) do their parts of a tile in different order, so that the
+   // matrix pipe always has a wavefront feeding it: wavefronts 0-3 multiply tile t first, then requantise it and
+   // compute the addresses of tile t + 1; the others first requantise their tile t - 1 and compute the addresses of
+   // tile t, and multiply last, up to the barrier that ends the tile.
    const bool mma_first = wave < 4;
    int t = t0, t_prev = -1, hi_cur = 0;
    if (t < t1) {
       hi_cur = last_row(t);
-      load_rows(first_row(t), hi_cur);
-      pixel_offsets(t);
+      req_begin(first_row(t), hi_cur);
+      req_finish();
+      if (mma_first) pixel_offsets(t);
    }
    wait_vmcnt<0>();
    __syncthreads();                          // weights, column parameters, padding columns and the first rows are in LDS
+   if constexpr (REGS) {
 #pragma unroll
-   for (int gi = 0; gi < NB * 4; ++gi) {
-      r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
-      const v4i bi = *reinterpret_cast<const v4i *>(w_bias + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+      for (int gi = 0; gi < NB * 4; ++gi) {
+         r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
+         const v4i bi = *reinterpret_cast<const v4i *>(w_bias + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r_bias[gi >> 2][(gi & 3) * 4 + e] = bi[e];
+         for (int e = 0; e < 4; ++e) r_bias[gi >> 2][(gi & 3) * 4 + e] = bi[e];
+      }
    }
    v16i acc[NB][MB];
-   // rows tile t + 1 has and tile t does not: requested at the start of tile t into slots that tile t does not read
+   // rows tile t + 1 has and tile t does not: requested during tile t into slots that tile t does not read
    auto request_next = [&](bool more, int tn, int &hi_next) {
       if (more) {
          hi_next = last_row(tn);
-         load_rows(hi_cur + 1, hi_next);
+         req_begin(hi_cur + 1, hi_next);
       }
    };
-   // One loop per group, so that the accumulators of each have one home in the register file. Both run t1 - t0
+   // One loop per role, so that the accumulators of each have one home in the register file. All run t1 - t0
    // iterations with one workgroup barrier each: it says that the rows of the next tile are complete (every
    // wavefront has waited for its own requests) and that every wavefront is done reading the present tile.
    if (mma_first) {
@@ -260,6 +355,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             wait_vmcnt<0>();                 // before this tile's stores join the queue
             epilogue(acc, t);
          } else {
+            req_finish();
             wait_vmcnt<0>();
          }
          if (more) pixel_offsets(tn);
@@ -275,9 +371,13 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
          request_next(more, tn, hi_next);
          if (t_prev >= 0) epilogue(acc, t_prev);
          const bool work = has_work(t);
-         if (work) kloop(acc);
+         if (work) {
+            pixel_offsets(t);
+            kloop(acc);
+         } else {
+            req_finish();
+         }
          wait_vmcnt<0>();
-         if (more) pixel_offsets(tn);
          t_prev = work ? t : -1;
          t = tn;
          hi_cur = hi_next;
@@ -301,12 +401,15 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (!aligned16(g.x) || !aligned16(g.w) || !aligned16(g.y)) return SOFIE_HIP_OK;
    const long long mtot = (long long)g.N * g.OH * g.OW;
    const int HP = g.H + g.ph + g.pbh, WP = g.W + g.pw + g.pbw;
-   if (mtot <= 0 || WP > 64) return SOFIE_HIP_OK;
+   // One instruction fetches one plane of one row, with one lane per padded column: rows wider than 64 columns do not fit
+   // it, and narrow rows waste it (a 12-column row uses 12 of the 64 lanes: the 10x10 layer of the CNN takes 39 us
+   // here against 35 us with the register-staged kernel; the 56x56 layer 55 - 57 us against 62 - 65 us).
+   if (mtot <= 0 || WP > 64 || WP < 32 || g.OW < 2 || g.OH < 2) return SOFIE_HIP_OK;
    if (mtot >= (1ll << 31) - 1024 || (long long)g.N * HP >= (1ll << 31) - 4096) return SOFIE_HIP_OK;
    const size_t xbytes = (size_t)g.N * g.H * g.W * g.C;
    if (xbytes >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
    const int WN = g.OC % 128 == 0 ? 2 : 1;
-   const int OCT = WN * 64, TM = (8 / WN) * 64;   // workgroup tile: TM pixels x OCT channels
+   const int OCT = WN * 64;
    const int C16 = g.C / 16;
    QConvRingArgs a{};
    a.x = g.x; a.w = g.w;
@@ -327,17 +430,18 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
    a.xbytes = (unsigned)xbytes;
    a.dOW = make_fastdiv(g.OW); a.dOH = make_fastdiv(g.OH); a.dHP = make_fastdiv(HP); a.dK16 = make_fastdiv(a.K / 16);
-   // the ring holds the rows of two consecutive tiles: the output rows 2*TM consecutive pixels can touch, the padding
-   // rows between the images they can span (HP - OH = 2 per image boundary) and the two extra rows of the last window
+   // The ring holds the rows of two consecutive tiles of TM pixels: the output rows 2*TM consecutive pixels can touch,
+   // the padding rows between the images they can span (HP - OH = 2 per image boundary) and the two extra rows of the
+   // last window.
+   const int TM = (8 / WN) * 64;
    const int rows2 = (2 * TM - 1) / g.OW + 2;
    int crossings = (rows2 - 1) / g.OH + 1;
    if (crossings > g.N - 1) crossings = g.N - 1;
-   const int window = rows2 + 2 * crossings + 2;
-   int R = 8;
-   while (R < window) R *= 2;
-   a.R = R;
+   const int R = rows2 + 2 * crossings + 2;
    const size_t lds = (size_t)OCT * a.KS + (size_t)OCT * 8 + (size_t)R * a.RS;
    if (lds > 160 * 1024) return SOFIE_HIP_OK;
+   a.R = R;
+   a.dR = make_fastdiv(R);
    if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
    const int nob = g.OC / OCT;
    int per = ctx->num_cus / nob;
