@@ -477,6 +477,8 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
       for (int j = 0; j < TJ; ++j)
 #pragma unroll
          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+   // scale and bias of the thread's column, in registers across the K loop
+   const ColumnParams col_params = load_column_params(g, tid, n0, BN);
 
    // --- ping-pong schedule -----------------------------------------------------------------
    // The two wavefronts of a SIMD run half a K-step apart: while one multiplies (MFMAs only,
@@ -535,7 +537,7 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    }
    wait_vmcnt<0>();                         // the trailing dummy requests still target LDS
    __syncthreads();
-   tile_epilogue<Mma, TI, TJ, OUT, 8>(g, acc, smem, tid, m0 + wm * 64, n0, wn, BN);
+   tile_epilogue<Mma, TI, TJ, OUT, 8>(g, acc, smem, tid, m0 + wm * 64, n0, wn, BN, &col_params);
 }
 
 // Byte-matrix transpose src [R, C] (ld_src) -> dst [C, R] (ld_dst), R % 16 == 0, C % 4 == 0.

@@ -275,16 +275,41 @@ __device__ __forceinline__ void stage_column_params(const GemmArgs &g, float *s_
 // wavefronts must have finished reading operand stages before the call.
 //   m_wave: first output row of this wavefront; n0: first output column of the workgroup;
 //   wn: index of the wavefront's column block; BN: columns of the workgroup tile.
+// Scale and bias bits of column n0 + tid, loaded ahead of the K loop by the kernels that can spare two registers:
+// the epilogue then starts without a round trip to memory.
+struct ColumnParams {
+   float scale;
+   int bias;
+};
+__device__ __forceinline__ ColumnParams load_column_params(const GemmArgs &g, int tid, int n0, int BN)
+{
+   ColumnParams p = {0.0f, 0};
+   if (tid < BN) {
+      const int n = n0 + tid;
+      p.scale = (g.scale && n < g.N) ? g.scale[n] : 0.0f;
+      p.bias = (g.bias && n < g.N) ? static_cast<const int *>(g.bias)[n] : 0;
+   }
+   return p;
+}
+
 template <class Mma, int TI, int TJ, int OUT, int NWAVES>
 __device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ], unsigned char *smem,
-                                              int tid, int m_wave, int n0, int wn, int BN)
+                                              int tid, int m_wave, int n0, int wn, int BN,
+                                              const ColumnParams *preloaded = nullptr)
 {
    constexpr int WB = EpilogueStaging<TI, OUT>::WAVE_BYTES;
    constexpr int WN = TI * 32;
    const int lane = tid & 63, wave = tid >> 6;
    float *s_scale = reinterpret_cast<float *>(smem + NWAVES * WB);
    int *s_bias = reinterpret_cast<int *>(s_scale + BN);
-   stage_column_params(g, s_scale, s_bias, tid, n0, BN);
+   if (preloaded) {
+      if (tid < BN) {
+         s_scale[tid] = preloaded->scale;
+         s_bias[tid] = preloaded->bias;
+      }
+   } else {
+      stage_column_params(g, s_scale, s_bias, tid, n0, BN);
+   }
    __syncthreads();
    unsigned char *stg = smem + wave * WB;
    if (OUT == SOFIE_OUT_S8 && g.zp == -128 && g.lo == -128)
