@@ -40,13 +40,15 @@ struct QConvRingArgs {
    int row_bytes;        // W * C: one image row in global memory
    unsigned fill;        // zp_x replicated into four bytes
    unsigned xbytes;
-   FastDiv dOW, dOH, dHP, dK16, dR;
+   FastDiv dOW, dOH, dHP, dK16, dR, dWP;
 };
 
 // C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels. The tile is (8/WN)*64 pixels x
 // WN*64 channels. (Twelve wavefronts per workgroup, three per SIMD, and wavefront tiles of 96 pixels were measured
 // on the 56x56 layer: the same time within 1 %.)
-template <int C16, int WN>
+// ROWDMA: a whole padded row (all planes) has at most 64 16-byte slots and is fetched by one instruction; otherwise one
+// instruction fetches one plane of a row.
+template <int C16, int WN, bool ROWDMA>
 __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
 {
    constexpr int MB = 2, NB = 2;
@@ -57,7 +59,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    constexpr int OCT = WN * NB * 32;
    constexpr int CB = C16 / 2;                      // 32-channel blocks
    constexpr int NS = 9 * CB;                       // K steps of 32 bytes
-   constexpr int NRL = NWAVE / C16;                 // wavefronts that share the rows of one plane index
+   constexpr int NRL = ROWDMA ? NWAVE : NWAVE / C16;   // wavefronts that share the rows of a request among them
    extern __shared__ __align__(16) unsigned char smem[];
    unsigned char *const s_w = smem;                                        // [OCT][KS]
    float *const s_scale = reinterpret_cast<float *>(smem + OCT * a.KS);    // [OCT]
@@ -117,12 +119,16 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       }
    }
 
-   // ---- rows of the padded images -> ring. Wavefront w fills plane w % C16 of every NRL-th row.
+   // ---- rows of the padded images -> ring. The rows of a request are cut into NRL runs of consecutive rows, one per
+   // wavefront (ROWDMA) or per group of C16 wavefronts, which take a plane each.
    const rsrc_t rs = make_rsrc(a.x, a.xbytes);
-   const int my_plane = wave % C16, my_rl = wave / C16;
-   const int iw = lane - a.pw;
-   const bool col_data = iw >= 0 && iw < a.W;
-   const int voff = iw * a.C + my_plane * 16;
+   const int my_plane = ROWDMA ? 0 : wave % C16, my_rl = ROWDMA ? wave : wave / C16;
+   const int slot_c = ROWDMA ? fdiv(lane, a.dWP) : my_plane;          // plane and padded column of the lane's 16 bytes
+   const int slot_wp = ROWDMA ? lane - slot_c * a.WP : lane;
+   const int iw = slot_wp - a.pw;
+   const bool slot_used = ROWDMA ? lane < C16 * a.WP : lane < a.WP;
+   const bool col_data = slot_used && iw >= 0 && iw < a.W;
+   const int voff = iw * a.C + slot_c * 16;
    // A request is scalar work plus one instruction per row; it is spread over the matrix loop of the present tile
    // (one row per call of req_step, between two K steps), where the scalar unit and the memory pipeline have nothing
    // else to do, instead of standing in front of it. The wavefront's rows inside one image are walked as a run: one
@@ -131,8 +137,9 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    int rq_v = 0, rq_to = -1, rq_left = 0, rq_soff = 0;
    unsigned rq_dst = 0;
    auto req_begin = [&](int from, int to) {
-      rq_v = from + my_rl;
-      rq_to = to;
+      const int per = (to - from + NRL) / NRL;          // rows per run, rounded up
+      rq_v = from + my_rl * per;
+      rq_to = rq_v + per - 1 < to ? rq_v + per - 1 : to;
       rq_left = 0;
    };
    auto req_step = [&]() {
@@ -142,21 +149,21 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
          const int ih = rq_v - n * a.HP - a.ph;
          rq_dst = ring0 + (unsigned)((rq_v - fdiv(rq_v, a.dR) * a.R) * a.RS + my_plane * a.PL);
          if ((unsigned)ih < (unsigned)a.H) {
-            const int in_image = (a.H - 1 - ih) / NRL, wanted = (rq_to - rq_v) / NRL;
+            const int in_image = a.H - 1 - ih, wanted = rq_to - rq_v;
             rq_left = (in_image < wanted ? in_image : wanted) + 1;
             rq_soff = (n * a.H + ih) * a.row_bytes;
          } else {
             // a padding row between two images (or above the first, below the last)
-            if (lane < a.WP) *reinterpret_cast<v4i *>(s_ring + (rq_dst - ring0) + lane * 16) = fillv;
-            rq_v += NRL;
+            if (slot_used) *reinterpret_cast<v4i *>(s_ring + (rq_dst - ring0) + lane * 16) = fillv;
+            rq_v += 1;
             return;
          }
       }
       if (col_data) dma16(rs, rq_dst, voff, rq_soff);
-      rq_soff += NRL * a.row_bytes;
-      rq_dst += NRL * a.RS;
+      rq_soff += a.row_bytes;
+      rq_dst += a.RS;
       if (rq_dst >= ring_end) rq_dst -= a.R * a.RS;
-      rq_v += NRL;
+      rq_v += 1;
       --rq_left;
    };
    auto req_finish = [&]() {
@@ -401,10 +408,9 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (!aligned16(g.x) || !aligned16(g.w) || !aligned16(g.y)) return SOFIE_HIP_OK;
    const long long mtot = (long long)g.N * g.OH * g.OW;
    const int HP = g.H + g.ph + g.pbh, WP = g.W + g.pw + g.pbw;
-   // One instruction fetches one plane of one row, with one lane per padded column: rows wider than 64 columns do not fit
-   // it, and narrow rows waste it (a 12-column row uses 12 of the 64 lanes: the 10x10 layer of the CNN takes 39 us
-   // here against 35 us with the register-staged kernel; the 56x56 layer 55 - 57 us against 62 - 65 us).
-   if (mtot <= 0 || WP > 64 || WP < 32 || g.OW < 2 || g.OH < 2) return SOFIE_HIP_OK;
+   // One instruction fetches a whole padded row if its C/16 planes are at most 64 16-byte slots, else one plane of a
+   // row, with one lane per padded column: rows wider than 64 columns do not fit.
+   if (mtot <= 0 || WP > 64 || g.OW < 2 || g.OH < 2) return SOFIE_HIP_OK;
    if (mtot >= (1ll << 31) - 1024 || (long long)g.N * HP >= (1ll << 31) - 4096) return SOFIE_HIP_OK;
    const size_t xbytes = (size_t)g.N * g.H * g.W * g.C;
    if (xbytes >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
@@ -442,6 +448,7 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (lds > 160 * 1024) return SOFIE_HIP_OK;
    a.R = R;
    a.dR = make_fastdiv(R);
+   a.dWP = make_fastdiv(WP);
    if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
    const int nob = g.OC / OCT;
    int per = ctx->num_cus / nob;
@@ -449,20 +456,26 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const int units = (int)((mtot + 63) / 64);
    if (per > units) per = units;
    const dim3 grid((unsigned)(per * nob)), block(512);
-#define SOFIE_QRING_LAUNCH(C16_, WN_)                                                                          \
+#define SOFIE_QRING_LAUNCH(C16_, WN_, ROW_)                                                                    \
    do {                                                                                                        \
-      auto kern = k_qconv_ring<C16_, WN_>;                                                                     \
+      auto kern = k_qconv_ring<C16_, WN_, ROW_>;                                                               \
       SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                            \
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));          \
       hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                              \
    } while (0)
+#define SOFIE_QRING_BY_ROW(C16_, WN_)                                                                          \
+   do {                                                                                                        \
+      if (C16_ * WP <= 64) SOFIE_QRING_LAUNCH(C16_, WN_, true);                                                \
+      else SOFIE_QRING_LAUNCH(C16_, WN_, false);                                                               \
+   } while (0)
    if (C16 == 4) {
-      if (WN == 2) SOFIE_QRING_LAUNCH(4, 2);
-      else SOFIE_QRING_LAUNCH(4, 1);
+      if (WN == 2) SOFIE_QRING_BY_ROW(4, 2);
+      else SOFIE_QRING_BY_ROW(4, 1);
    } else {
-      if (WN == 2) SOFIE_QRING_LAUNCH(2, 2);
-      else SOFIE_QRING_LAUNCH(2, 1);
+      if (WN == 2) SOFIE_QRING_BY_ROW(2, 2);
+      else SOFIE_QRING_BY_ROW(2, 1);
    }
+#undef SOFIE_QRING_BY_ROW
 #undef SOFIE_QRING_LAUNCH
    *done = true;
    return check_launch(ctx, "k_qconv_ring");
