@@ -38,6 +38,7 @@ struct QConvRingArgs {
    int K, KS;            // bytes of one weight row, its LDS stride
    int RS, PL, R;        // ring: row pitch and plane pitch in bytes, rows (a power of two)
    int row_bytes;        // W * C: one image row in global memory
+   int gap;              // HP - OH * (rows per pixel): padded rows between the last window row of an image and the next image
    unsigned fill;        // zp_x replicated into four bytes
    unsigned xbytes;
    FastDiv dOW, dOH, dHP, dK16, dR, dWP;
@@ -48,14 +49,21 @@ struct QConvRingArgs {
 // on the 56x56 layer: the same time within 1 %.)
 // ROWDMA: a whole padded row (all planes) has at most 64 16-byte slots and is fetched by one instruction; otherwise one
 // instruction fetches one plane of a row.
-template <int C16, int WN, bool ROWDMA>
+// POOL: a 2x2 stride-2 max pooling is fused. A wavefront then owns 32 POOLED pixels; its four accumulator tiles along m
+// are the four positions of the pooling window, the pooling is a register-wise maximum of the int32 accumulators (the
+// requantisation is monotonic; for a negative scale the minimum is taken) and a quarter of the values is converted and
+// stored. In that mode the "pixels" of tiles, runs and a.OH / a.OW / a.ep.M are pooled pixels.
+template <int C16, int WN, bool ROWDMA, bool POOL>
 __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
 {
-   constexpr int MB = 2, NB = 2;
+   constexpr int NB = 2;
+   constexpr int MB = POOL ? 4 : 2;                 // accumulator tiles along m per wavefront
+   constexpr int MBP = POOL ? 1 : 2;                // tiles of 32 (pooled) pixels per wavefront
+   constexpr int RPP = POOL ? 2 : 1;                // convolution rows (and columns) per (pooled) pixel
    constexpr int NWAVE = 8, NT = NWAVE * 64;
-   constexpr bool REGS = true;                     // scales and bias tiles in registers
+   constexpr bool REGS = !POOL;                     // scales and bias tiles in registers
    constexpr int WM = NWAVE / WN;
-   constexpr int TM = WM * MB * 32;
+   constexpr int TM = WM * MBP * 32;
    constexpr int OCT = WN * NB * 32;
    constexpr int CB = C16 / 2;                      // 32-channel blocks
    constexpr int NS = 9 * CB;                       // K steps of 32 bytes
@@ -76,7 +84,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    const int wg = blockIdx.x / nob, nwg = gridDim.x / nob;
    // The workgroup's run of pixels, dealt out in units of the 64 pixels a wavefront multiplies: its tiles start at
    // m_begin, and of the last, partial one only the wavefronts whose pixels lie inside the run do any work.
-   constexpr int UNIT = MB * 32;
+   constexpr int UNIT = MBP * 32;
    const int units = (a.ep.M + UNIT - 1) / UNIT;
    const int m_begin = (int)((long long)wg * units / nwg) * UNIT;
    const int m_stop = (int)((long long)(wg + 1) * units / nwg) * UNIT;
@@ -173,13 +181,13 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    auto first_row = [&](int t) {
       const int R0 = fdiv(m_begin + t * TM, a.dOW);
       const int n0 = fdiv(R0, a.dOH);
-      return n0 * a.HP + (R0 - n0 * a.OH);
+      return n0 * a.HP + (R0 - n0 * a.OH) * RPP;
    };
    auto last_row = [&](int t) {
       const int mlast = (m_begin + (t + 1) * TM < mtot ? m_begin + (t + 1) * TM : mtot) - 1;
       const int R1 = fdiv(mlast, a.dOW);
       const int n1 = fdiv(R1, a.dOH);
-      return n1 * a.HP + (R1 - n1 * a.OH) + 2;
+      return n1 * a.HP + (R1 - n1 * a.OH) * RPP + (RPP - 1) + 2;
    };
 
    int b_off[NB];
@@ -190,28 +198,30 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    const int *const w_bias = s_bias + wn * NB * 32;
    const bool plain = a.ep.zp == -128 && a.ep.lo == -128;
 
-   // LDS offsets of the wavefront's pixels in the ring, per kernel row and 32-channel block: the lane's half of the
-   // block is plane 2*cb + half; the column tap kw is the constant kw*16 on top
-   const unsigned char *pa[3][CB][MB];
+   // LDS addresses of the wavefront's pixels in the ring, per kernel row and 32-channel block: the lane's half of the
+   // block is plane 2*cb + half; the column tap kw is the constant kw*16 on top. With the fused pooling a lane's four
+   // window positions share their rows: four ring rows per lane (window row + kernel row), the window column is
+   // another constant.
+   const unsigned char *pa[POOL ? 4 : 3][CB][POOL ? 1 : MB];
    const unsigned char *const lane_base = s_ring + half * a.PL;
    auto pixel_offsets = [&](int tt) {
 #pragma unroll
-      for (int j = 0; j < MB; ++j) {
-         int m = m_begin + tt * TM + (wm * MB + j) * 32 + l32;
+      for (int j = 0; j < MBP; ++j) {
+         int m = m_begin + tt * TM + (wm * MBP + j) * 32 + l32;
          m = m < mtot ? m : mtot - 1;
          // OW and OH are at least 2 (the launcher sees to it): the divisions are a multiply-high and a shift
          const int R = (int)(__umulhi((unsigned)m, a.dOW.magic) >> a.dOW.shift);
          const int ow = m - R * a.OW;
          const int n = (int)(__umulhi((unsigned)R, a.dOH.magic) >> a.dOH.shift);
-         const int v = R + n * 2;                       // n * HP + (R - n * OH), HP - OH = 2
-         const unsigned char *const colb = lane_base + ow * 16;
-         // ring slots of the three rows: v % R, then one step at a time with the wrap
+         const int v = R * RPP + n * a.gap;             // n * HP + (R - n * OH) * RPP
+         const unsigned char *const colb = lane_base + ow * (RPP * 16);
+         // ring slots of the rows: v % R, then one step at a time with the wrap
          unsigned slot = (unsigned)v - (__umulhi((unsigned)v, a.dR.magic) >> a.dR.shift) * (unsigned)a.R;
 #pragma unroll
-         for (int kh = 0; kh < 3; ++kh) {
+         for (int r = 0; r < (POOL ? 4 : 3); ++r) {
             const unsigned char *const rowb = colb + slot * a.RS;
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) pa[kh][cb][j] = rowb + cb * 2 * a.PL;
+            for (int cb = 0; cb < CB; ++cb) pa[r][cb][j] = rowb + cb * 2 * a.PL;
             slot = slot + 1;
             slot = slot < slot - (unsigned)a.R ? slot : slot - (unsigned)a.R;   // min(slot, slot - R): slot - R wraps below R
          }
@@ -223,13 +233,19 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // K loop of one tile: unrolled over its 9 * CB steps; the fragment reads run two steps ahead of the matrix
    // instructions and one read is issued behind each of a step's first matrix instructions
    auto kloop = [&](v16i (&acc)[NB][MB]) {
-      constexpr int NBUF = 3;
+      constexpr int NBUF = POOL ? 2 : 3;
       v4i fa[NBUF][MB], fb[NBUF][NB];
       const unsigned char *pb[NB];
 #pragma unroll
       for (int i = 0; i < NB; ++i) pb[i] = s_w + b_off[i];
       v16i bias_tile[NB];
-      if constexpr (REGS) {
+      if constexpr (POOL) {
+         // the pooled accumulators start from zero: the bias is added to the pooled quarter (max(a + b) = max(a) + b)
+#pragma unroll
+         for (int i = 0; i < NB; ++i)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) bias_tile[i][e] = 0;
+      } else if constexpr (REGS) {
 #pragma unroll
          for (int i = 0; i < NB; ++i) bias_tile[i] = r_bias[i];
       } else {
@@ -246,8 +262,10 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             const int kh = s / (3 * CB), kw = (s / CB) % 3, cb = s % CB;
             fb[s % NBUF][0] = *reinterpret_cast<const v4i *>(pb[0] + s * 32);
 #pragma unroll
-            for (int j = 0; j < MB; ++j)
-               fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[kh][cb][j] + kw * 16);
+            for (int j = 0; j < MB; ++j) {
+               if constexpr (POOL) fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[(j >> 1) + kh][cb][0] + ((j & 1) + kw) * 16);
+               else fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[kh][cb][j] + kw * 16);
+            }
 #pragma unroll
             for (int i = 1; i < NB; ++i) fb[s % NBUF][i] = *reinterpret_cast<const v4i *>(pb[i] + s * 32);
          }
@@ -281,10 +299,10 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // through a private block of LDS costs what they gain.)
    auto epilogue_as = [&](v16i (&acc)[NB][MB], int tt, auto plain_tag) {
       constexpr bool PLAIN = decltype(plain_tag)::value;
-      const int m_wave = m_begin + tt * TM + wm * MB * 32, n_wave = ob * OCT + wn * NB * 32;
+      const int m_wave = m_begin + tt * TM + wm * MBP * 32, n_wave = ob * OCT + wn * NB * 32;
       const float zpo = (float)(ep.zp + 128), lof = (float)(ep.lo + 128);
 #pragma unroll
-      for (int j = 0; j < MB; ++j) {
+      for (int j = 0; j < MBP; ++j) {
          const int m = m_wave + j * 32 + l32;
          int8_t *const row = static_cast<int8_t *>(ep.Y) + (size_t)(m < ep.M ? m : 0) * ep.ldy + n_wave + half * 16;
 #pragma unroll
@@ -292,7 +310,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             unsigned d[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-               const v4f sc = r_scale[i * 4 + q];
+               const v4f sc = r_scale[REGS ? i * 4 + q : 0];
                unsigned pk = 0;
 #pragma unroll
                for (int e = 0; e < 4; ++e) {
@@ -310,12 +328,42 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
          }
       }
    };
+   bool any_negative = false;   // pooled variant: some scale of the workgroup's channels is negative (set below)
    auto epilogue = [&](v16i (&acc)[NB][MB], int tt) {
-      if (plain) epilogue_as(acc, tt, BoolTag<true>{});
-      else epilogue_as(acc, tt, BoolTag<false>{});
+      if constexpr (POOL) {
+         const int m_wave = m_begin + tt * TM + wm * 32, n_wave = ob * OCT + wn * NB * 32;
+         v16i pooled[NB][1];
+         if (!any_negative) {
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+               for (int e = 0; e < 16; ++e)
+                  pooled[i][0][e] = max(max(acc[i][0][e], acc[i][1][e]), max(acc[i][2][e], acc[i][3][e]));
+         } else {
+            // a negative scale turns the order around: those channels take the minimum
+#pragma unroll
+            for (int i = 0; i < NB; ++i)
+#pragma unroll
+               for (int q = 0; q < 4; ++q) {
+                  const v4f sc = *reinterpret_cast<const v4f *>(w_scale + i * 32 + q * 8 + nq);
+#pragma unroll
+                  for (int e4 = 0; e4 < 4; ++e4) {
+                     const int e = q * 4 + e4;
+                     const int hi = max(max(acc[i][0][e], acc[i][1][e]), max(acc[i][2][e], acc[i][3][e]));
+                     const int lo = min(min(acc[i][0][e], acc[i][1][e]), min(acc[i][2][e], acc[i][3][e]));
+                     pooled[i][0][e] = sc[e4] < 0.0f ? lo : hi;
+                  }
+               }
+         }
+         if (plain) tile_epilogue_s8_direct<NB, 1, true, true>(ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+         else tile_epilogue_s8_direct<NB, 1, false, true>(ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+      } else {
+         if (plain) epilogue_as(acc, tt, BoolTag<true>{});
+         else epilogue_as(acc, tt, BoolTag<false>{});
+      }
    };
    // whether the wavefront has pixels in tile tt (all tiles but the last are full)
-   auto has_work = [&](int tt) { return m_begin + tt * TM + wm * MB * 32 < mtot; };
+   auto has_work = [&](int tt) { return m_begin + tt * TM + wm * MBP * 32 < mtot; };
 
    // The wavefronts that share a SIMD (w, w + 4[, w + 8]) do their parts of a tile in different order, so that the
    // matrix pipe always has a wavefront feeding it: wavefronts 0-3 multiply tile t first, then requantise it and
@@ -331,6 +379,12 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    }
    wait_vmcnt<0>();
    __syncthreads();                          // weights, column parameters, padding columns and the first rows are in LDS
+   if constexpr (POOL) {
+      // whether any scale of the workgroup's channels is negative (uniform, so the common case pools with a maximum only)
+      int neg = 0;
+      for (int c = tid; c < OCT; c += NT) neg |= s_scale[c] < 0.0f;
+      any_negative = __syncthreads_or(neg) != 0;
+   }
    if constexpr (REGS) {
 #pragma unroll
       for (int gi = 0; gi < NB * 4; ++gi) {
@@ -398,19 +452,25 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
 
 namespace sofie {
 
-// 3x3, stride 1, 32 or 64 input channels, channels-last int8 in and out, no fused pooling.
+// 3x3, stride 1, 32 or 64 input channels, channels-last int8 in and out, rows of at most 64 padded columns; with or
+// without a fused 2x2 stride-2 max pooling.
 int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
 {
    *done = false;
-   if (g.pool_kh != 0 || g.xf) return SOFIE_HIP_OK;
+   if (g.xf) return SOFIE_HIP_OK;
+   const bool pool = g.pool_kh != 0;
+   if (pool && !(g.pool_kh == 2 && g.pool_kw == 2 && g.pool_sh == 2 && g.pool_sw == 2)) return SOFIE_HIP_OK;
    if (g.groups != 1 || !(g.C == 32 || g.C == 64) || g.OC % 64 != 0 || !g.x_nhwc || !g.y_nhwc || !g.w_ohwi) return SOFIE_HIP_OK;
    if (g.KH != 3 || g.KW != 3 || g.sh != 1 || g.sw != 1) return SOFIE_HIP_OK;
    if (!aligned16(g.x) || !aligned16(g.w) || !aligned16(g.y)) return SOFIE_HIP_OK;
-   const long long mtot = (long long)g.N * g.OH * g.OW;
+   // rows and columns the tiles count: pooled pixels when the pooling is fused
+   const int TH = pool ? g.PH : g.OH, TW = pool ? g.PW : g.OW;
+   const int rpp = pool ? 2 : 1;
+   const long long mtot = (long long)g.N * TH * TW;
    const int HP = g.H + g.ph + g.pbh, WP = g.W + g.pw + g.pbw;
    // One instruction fetches a whole padded row if its C/16 planes are at most 64 16-byte slots, else one plane of a
    // row, with one lane per padded column: rows wider than 64 columns do not fit.
-   if (mtot <= 0 || WP > 64 || g.OW < 2 || g.OH < 2) return SOFIE_HIP_OK;
+   if (mtot <= 0 || WP > 64 || TW < 2 || TH < 2) return SOFIE_HIP_OK;
    if (mtot >= (1ll << 31) - 1024 || (long long)g.N * HP >= (1ll << 31) - 4096) return SOFIE_HIP_OK;
    const size_t xbytes = (size_t)g.N * g.H * g.W * g.C;
    if (xbytes >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
@@ -424,26 +484,27 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.ep.zp = g.zpy; a.ep.lo = g.lo; a.ep.relu = g.relu; a.ep.s = 1.0f;
    a.ep.vec_store = 1;
    a.H = g.H; a.W = g.W; a.C = g.C; a.ph = g.ph; a.pw = g.pw;
-   a.OH = g.OH; a.OW = g.OW; a.HP = HP; a.WP = WP;
+   a.OH = TH; a.OW = TW; a.HP = HP; a.WP = WP;
+   a.gap = HP - TH * rpp;
    a.K = 9 * g.C;
    a.KS = ((a.K / 16) % 2 == 0) ? a.K + 16 : a.K;
    a.PL = WP * 16;
-   // Row pitch: consecutive pixels of an output row are 16 bytes apart; padded so that the first pixel of the next
-   // output row continues that sequence modulo the 256 bytes the LDS banks span.
+   // Row pitch: consecutive pixels of an output row are 16 bytes apart (32 with the pooling); padded so that the first
+   // pixel of the next output row continues that sequence modulo the 256 bytes the LDS banks span.
    a.RS = C16 * a.PL;
-   a.RS += (((g.OW * 16 - a.RS) % 256) + 256) % 256;
+   a.RS += (((TW * rpp * 16 - a.RS) % 256) + 256) % 256;
    a.row_bytes = g.W * g.C;
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
    a.xbytes = (unsigned)xbytes;
-   a.dOW = make_fastdiv(g.OW); a.dOH = make_fastdiv(g.OH); a.dHP = make_fastdiv(HP); a.dK16 = make_fastdiv(a.K / 16);
-   // The ring holds the rows of two consecutive tiles of TM pixels: the output rows 2*TM consecutive pixels can touch,
-   // the padding rows between the images they can span (HP - OH = 2 per image boundary) and the two extra rows of the
-   // last window.
-   const int TM = (8 / WN) * 64;
-   const int rows2 = (2 * TM - 1) / g.OW + 2;
-   int crossings = (rows2 - 1) / g.OH + 1;
+   a.dOW = make_fastdiv(TW); a.dOH = make_fastdiv(TH); a.dHP = make_fastdiv(HP); a.dK16 = make_fastdiv(a.K / 16);
+   // The ring holds the rows of two consecutive tiles of TM pixels: the rows 2*TM consecutive pixels can touch, the
+   // padded rows between the images they can span and the two extra rows of the last window.
+   const int unit = pool ? 32 : 64;
+   const int TM = (8 / WN) * unit;
+   const int rows2 = (2 * TM - 1) / TW + 2;
+   int crossings = (rows2 - 1) / TH + 1;
    if (crossings > g.N - 1) crossings = g.N - 1;
-   const int R = rows2 + 2 * crossings + 2;
+   const int R = rows2 * rpp + a.gap * crossings + 2;
    const size_t lds = (size_t)OCT * a.KS + (size_t)OCT * 8 + (size_t)R * a.RS;
    if (lds > 160 * 1024) return SOFIE_HIP_OK;
    a.R = R;
@@ -453,28 +514,34 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const int nob = g.OC / OCT;
    int per = ctx->num_cus / nob;
    if (per < 1) per = 1;
-   const int units = (int)((mtot + 63) / 64);
+   const int units = (int)((mtot + unit - 1) / unit);
    if (per > units) per = units;
    const dim3 grid((unsigned)(per * nob)), block(512);
-#define SOFIE_QRING_LAUNCH(C16_, WN_, ROW_)                                                                    \
+#define SOFIE_QRING_LAUNCH(C16_, WN_, ROW_, POOL_)                                                             \
    do {                                                                                                        \
-      auto kern = k_qconv_ring<C16_, WN_, ROW_>;                                                               \
+      auto kern = k_qconv_ring<C16_, WN_, ROW_, POOL_>;                                                        \
       SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                            \
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));          \
       hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                              \
    } while (0)
-#define SOFIE_QRING_BY_ROW(C16_, WN_)                                                                          \
+#define SOFIE_QRING_BY_ROW(C16_, WN_, POOL_)                                                                   \
    do {                                                                                                        \
-      if (C16_ * WP <= 64) SOFIE_QRING_LAUNCH(C16_, WN_, true);                                                \
-      else SOFIE_QRING_LAUNCH(C16_, WN_, false);                                                               \
+      if (C16_ * WP <= 64) SOFIE_QRING_LAUNCH(C16_, WN_, true, POOL_);                                         \
+      else SOFIE_QRING_LAUNCH(C16_, WN_, false, POOL_);                                                        \
+   } while (0)
+#define SOFIE_QRING_BY_POOL(C16_, WN_)                                                                         \
+   do {                                                                                                        \
+      if (pool) SOFIE_QRING_BY_ROW(C16_, WN_, true);                                                           \
+      else SOFIE_QRING_BY_ROW(C16_, WN_, false);                                                               \
    } while (0)
    if (C16 == 4) {
-      if (WN == 2) SOFIE_QRING_BY_ROW(4, 2);
-      else SOFIE_QRING_BY_ROW(4, 1);
+      if (WN == 2) SOFIE_QRING_BY_POOL(4, 2);
+      else SOFIE_QRING_BY_POOL(4, 1);
    } else {
-      if (WN == 2) SOFIE_QRING_BY_ROW(2, 2);
-      else SOFIE_QRING_BY_ROW(2, 1);
+      if (WN == 2) SOFIE_QRING_BY_POOL(2, 2);
+      else SOFIE_QRING_BY_POOL(2, 1);
    }
+#undef SOFIE_QRING_BY_POOL
 #undef SOFIE_QRING_BY_ROW
 #undef SOFIE_QRING_LAUNCH
    *done = true;

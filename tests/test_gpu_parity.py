@@ -573,6 +573,11 @@ def test_conv_pool_entry_point(ops, cfg):
     dict(N=1, C=32, H=2, W=2, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),        # a single pooled pixel
     dict(N=4, C=32, H=12, W=10, OC=64, k=(4, 4), p=(1, 1, 2, 2), s=(1, 1)),  # begin != end pads under the pooling
     dict(N=3, C=64, H=9, W=11, OC=128, k=(3, 3), p=(2, 1, 0, 1), s=(1, 1)),
+    # rows fetched straight into LDS under the pooling: the widest row, a plane per instruction (4 x 22 slots > 64),
+    # and enough images for several tiles per workgroup
+    dict(N=2, C=64, H=7, W=62, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=9, C=64, H=20, W=20, OC=128, k=(3, 3), p=(1, 1), s=(1, 1)),
+    dict(N=1200, C=32, H=20, W=20, OC=64, k=(3, 3), p=(1, 1), s=(1, 1)),
 ])
 def test_conv_pool_fused_matrix_core_kernel(ops, cfg):
     """Channels-last operands with a 2x2 stride-2 pooling: one kernel whose wavefronts pool on the accumulators.
