@@ -94,7 +94,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    ep.M = mtot;
 
    // ---- weights of this channel block: resident for the life of the workgroup (eight loads in flight per thread)
-   {
+   auto stage_weights = [&]() {
       constexpr int WCH = 8;
       const int K16 = a.K >> 4;
       const int total = OCT * K16;
@@ -113,26 +113,31 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             if (q < total) *reinterpret_cast<v4i *>(s_w + r * a.KS + (q - r * K16) * 16) = chunk[u];
          }
       }
-   }
-   stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
+      stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
+   };
+   // Slot of a padded column inside a plane. With the fused pooling the even columns come first, then the odd ones:
+   // the pixels of consecutive lanes are two columns apart, and this keeps their 16 bytes next to each other.
+   const int half_cols = (a.WP + 1) >> 1;
+   auto column_slot = [&](int wp) { return POOL ? (wp >> 1) + (wp & 1) * half_cols : wp; };
+   auto slot_column = [&](int pos) { return POOL ? (pos < half_cols ? 2 * pos : 2 * (pos - half_cols) + 1) : pos; };
    const v4i fillv = {(int)a.fill, (int)a.fill, (int)a.fill, (int)a.fill};
    // padding columns of every ring row hold the input zero-point for the life of the kernel
-   {
+   auto fill_padding_columns = [&]() {
       const int npad = a.WP - a.W;
       for (int q = tid; q < a.R * C16 * npad; q += NT) {
          const int rc = q / npad, pc = q - rc * npad;
          const int r = rc / C16, c = rc - r * C16;
          const int wp = pc < a.pw ? pc : pc + a.W;
-         *reinterpret_cast<v4i *>(s_ring + r * a.RS + c * a.PL + wp * 16) = fillv;
+         *reinterpret_cast<v4i *>(s_ring + r * a.RS + c * a.PL + column_slot(wp) * 16) = fillv;
       }
-   }
+   };
 
    // ---- rows of the padded images -> ring. The rows of a request are cut into NRL runs of consecutive rows, one per
    // wavefront (ROWDMA) or per group of C16 wavefronts, which take a plane each.
    const rsrc_t rs = make_rsrc(a.x, a.xbytes);
    const int my_plane = ROWDMA ? 0 : wave % C16, my_rl = ROWDMA ? wave : wave / C16;
    const int slot_c = ROWDMA ? fdiv(lane, a.dWP) : my_plane;          // plane and padded column of the lane's 16 bytes
-   const int slot_wp = ROWDMA ? lane - slot_c * a.WP : lane;
+   const int slot_wp = slot_column(ROWDMA ? lane - slot_c * a.WP : lane);
    const int iw = slot_wp - a.pw;
    const bool slot_used = ROWDMA ? lane < C16 * a.WP : lane < a.WP;
    const bool col_data = slot_used && iw >= 0 && iw < a.W;
@@ -202,7 +207,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // block is plane 2*cb + half; the column tap kw is the constant kw*16 on top. With the fused pooling a lane's four
    // window positions share their rows: four ring rows per lane (window row + kernel row), the window column is
    // another constant.
-   const unsigned char *pa[POOL ? 4 : 3][CB][POOL ? 1 : MB];
+   const unsigned char *pa[POOL ? 4 : 3][CB][2];   // last index: m tile, or parity of the column with the pooling
    const unsigned char *const lane_base = s_ring + half * a.PL;
    auto pixel_offsets = [&](int tt) {
 #pragma unroll
@@ -214,14 +219,21 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
          const int ow = m - R * a.OW;
          const int n = (int)(__umulhi((unsigned)R, a.dOH.magic) >> a.dOH.shift);
          const int v = R * RPP + n * a.gap;             // n * HP + (R - n * OH) * RPP
-         const unsigned char *const colb = lane_base + ow * (RPP * 16);
+         const unsigned char *const colb = lane_base + ow * 16;   // pooled: column 2*ow is slot ow of the even columns
          // ring slots of the rows: v % R, then one step at a time with the wrap
          unsigned slot = (unsigned)v - (__umulhi((unsigned)v, a.dR.magic) >> a.dR.shift) * (unsigned)a.R;
 #pragma unroll
          for (int r = 0; r < (POOL ? 4 : 3); ++r) {
             const unsigned char *const rowb = colb + slot * a.RS;
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) pa[r][cb][j] = rowb + cb * 2 * a.PL;
+            for (int cb = 0; cb < CB; ++cb) {
+               if constexpr (POOL) {
+                  pa[r][cb][0] = rowb + cb * 2 * a.PL;
+                  pa[r][cb][1] = rowb + cb * 2 * a.PL + half_cols * 16;
+               } else {
+                  pa[r][cb][j] = rowb + cb * 2 * a.PL;
+               }
+            }
             slot = slot + 1;
             slot = slot < slot - (unsigned)a.R ? slot : slot - (unsigned)a.R;   // min(slot, slot - R): slot - R wraps below R
          }
@@ -263,7 +275,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             fb[s % NBUF][0] = *reinterpret_cast<const v4i *>(pb[0] + s * 32);
 #pragma unroll
             for (int j = 0; j < MB; ++j) {
-               if constexpr (POOL) fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[(j >> 1) + kh][cb][0] + ((j & 1) + kw) * 16);
+               if constexpr (POOL) fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[(j >> 1) + kh][cb][((j & 1) + kw) & 1] + (((j & 1) + kw) >> 1) * 16);
                else fa[s % NBUF][j] = *reinterpret_cast<const v4i *>(pa[kh][cb][j] + kw * 16);
             }
 #pragma unroll
@@ -288,7 +300,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             if constexpr (MB * NB > MB + NB) __builtin_amdgcn_sched_group_barrier(0x008, MB * NB - (MB + NB), 0);
          }
          __builtin_amdgcn_sched_barrier(0);
-         if (s < NS && (s & 1)) req_step();
+         if (s < NS && (NS <= 9 || (s & 1))) req_step();   // 9 chances per tile
       }
       req_finish();
    };
@@ -377,6 +389,9 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       req_finish();
       if (mma_first) pixel_offsets(t);
    }
+   // the rows of the first tile are on their way while the weights are staged
+   stage_weights();
+   fill_padding_columns();
    wait_vmcnt<0>();
    __syncthreads();                          // weights, column parameters, padding columns and the first rows are in LDS
    if constexpr (POOL) {
@@ -489,10 +504,11 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.K = 9 * g.C;
    a.KS = ((a.K / 16) % 2 == 0) ? a.K + 16 : a.K;
    a.PL = WP * 16;
-   // Row pitch: consecutive pixels of an output row are 16 bytes apart (32 with the pooling); padded so that the first
-   // pixel of the next output row continues that sequence modulo the 256 bytes the LDS banks span.
+   // Row pitch: consecutive pixels of an output row are 16 bytes apart (with the pooling too: even and odd columns are
+   // stored apart); padded so that the first pixel of the next output row continues that sequence modulo the 256 bytes
+   // the LDS banks span.
    a.RS = C16 * a.PL;
-   a.RS += (((TW * rpp * 16 - a.RS) % 256) + 256) % 256;
+   a.RS += (((TW * 16 - a.RS) % 256) + 256) % 256;
    a.row_bytes = g.W * g.C;
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
    a.xbytes = (unsigned)xbytes;
