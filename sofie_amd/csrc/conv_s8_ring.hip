@@ -41,7 +41,7 @@ struct QConvRingArgs {
    int gap;              // HP - OH * (rows per pixel): padded rows between the last window row of an image and the next image
    unsigned fill;        // zp_x replicated into four bytes
    unsigned xbytes;
-   FastDiv dOW, dOH, dHP, dK16, dR, dWP;
+   FastDiv dOW, dOH, dHP, dKS16, dR, dWP;
 };
 
 // C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels. The tile is (8/WN)*64 pixels x
@@ -93,25 +93,18 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    GemmArgs ep = a.ep;
    ep.M = mtot;
 
-   // ---- weights of this channel block: resident for the life of the workgroup (eight loads in flight per thread)
+   // ---- weights of this channel block: resident for the life of the workgroup. They travel like the input rows, straight
+   // into LDS: an instruction fills as many padded LDS rows as fit its 64 slots (one row of 36 chunks and the pad, three
+   // rows of 18), and all of a wavefront's requests are in flight together.
    auto stage_weights = [&]() {
-      constexpr int WCH = 8;
-      const int K16 = a.K >> 4;
-      const int total = OCT * K16;
-      const int8_t *wsrc = a.w + (size_t)ob * OCT * a.K;
-      for (int base = tid; base < total; base += NT * WCH) {
-         v4i chunk[WCH];
-#pragma unroll
-         for (int u = 0; u < WCH; ++u) {
-            const int q = base + u * NT;
-            chunk[u] = *reinterpret_cast<const v4i *>(wsrc + (size_t)(q < total ? q : base) * 16);
-         }
-#pragma unroll
-         for (int u = 0; u < WCH; ++u) {
-            const int q = base + u * NT;
-            const int r = fdiv(q, a.dK16);
-            if (q < total) *reinterpret_cast<v4i *>(s_w + r * a.KS + (q - r * K16) * 16) = chunk[u];
-         }
+      const int K16 = a.K >> 4, KS16 = a.KS >> 4;
+      const int rpi = 64 / KS16;                                   // LDS rows per instruction
+      const int sub = fdiv(lane, a.dKS16), chunk = lane - sub * KS16;
+      const bool used = sub < rpi && chunk < K16;
+      const rsrc_t wrs = make_rsrc(a.w + (size_t)ob * OCT * a.K, (unsigned)(OCT * a.K));
+      const unsigned w0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)s_w;
+      for (int r0 = wave * rpi; r0 < OCT; r0 += NWAVE * rpi) {
+         if (used && r0 + sub < OCT) dma16(wrs, w0 + (unsigned)(r0 * a.KS), sub * a.K + chunk * 16, r0 * a.K);
       }
       stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
    };
@@ -512,7 +505,7 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.row_bytes = g.W * g.C;
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
    a.xbytes = (unsigned)xbytes;
-   a.dOW = make_fastdiv(TW); a.dOH = make_fastdiv(TH); a.dHP = make_fastdiv(HP); a.dK16 = make_fastdiv(a.K / 16);
+   a.dOW = make_fastdiv(TW); a.dOH = make_fastdiv(TH); a.dHP = make_fastdiv(HP); a.dKS16 = make_fastdiv(a.KS / 16);
    // The ring holds the rows of two consecutive tiles of TM pixels: the rows 2*TM consecutive pixels can touch, the
    // padded rows between the images they can span and the two extra rows of the last window.
    const int unit = pool ? 32 : 64;
