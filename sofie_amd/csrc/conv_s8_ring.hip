@@ -38,6 +38,7 @@ struct QConvRingArgs {
    int K, KS;            // bytes of one weight row, its LDS stride
    int RS, PL, R;        // ring: row pitch and plane pitch in bytes, rows (a power of two)
    int row_bytes;        // W * C: one image row in global memory
+   int units_each, units_rem;   // 64-pixel (32 pooled pixel) units per workgroup of a channel block: quotient and remainder
    int gap;              // HP - OH * (rows per pixel): padded rows between the last window row of an image and the next image
    unsigned fill;        // zp_x replicated into four bytes
    unsigned xbytes;
@@ -80,14 +81,14 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    const int wn = wave % WN, wm = wave / WN;
    const int half = lane >> 5, l32 = lane & 31;
    const int nob = a.ep.N / OCT;
-   const int ob = blockIdx.x % nob;
-   const int wg = blockIdx.x / nob, nwg = gridDim.x / nob;
+   const int ob = nob == 1 ? 0 : blockIdx.x % nob;
+   const int wg = nob == 1 ? blockIdx.x : blockIdx.x / nob;
    // The workgroup's run of pixels, dealt out in units of the 64 pixels a wavefront multiplies: its tiles start at
    // m_begin, and of the last, partial one only the wavefronts whose pixels lie inside the run do any work.
    constexpr int UNIT = MBP * 32;
-   const int units = (a.ep.M + UNIT - 1) / UNIT;
-   const int m_begin = (int)((long long)wg * units / nwg) * UNIT;
-   const int m_stop = (int)((long long)(wg + 1) * units / nwg) * UNIT;
+   // (the first units_rem workgroups of a channel block get units_each + 1 units, the others units_each: no division here)
+   const int m_begin = (wg * a.units_each + (wg < a.units_rem ? wg : a.units_rem)) * UNIT;
+   const int m_stop = m_begin + (a.units_each + (wg < a.units_rem ? 1 : 0)) * UNIT;
    const int mtot = m_stop < a.ep.M ? m_stop : a.ep.M;       // one past the last pixel of the run
    const int t0 = 0, t1 = (mtot - m_begin + TM - 1) / TM;
    GemmArgs ep = a.ep;
@@ -117,11 +118,12 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // padding columns of every ring row hold the input zero-point for the life of the kernel
    auto fill_padding_columns = [&]() {
       const int npad = a.WP - a.W;
-      for (int q = tid; q < a.R * C16 * npad; q += NT) {
-         const int rc = q / npad, pc = q - rc * npad;
-         const int r = rc / C16, c = rc - r * C16;
-         const int wp = pc < a.pw ? pc : pc + a.W;
-         *reinterpret_cast<v4i *>(s_ring + r * a.RS + c * a.PL + column_slot(wp) * 16) = fillv;
+      for (int rc = tid; rc < a.R * C16; rc += NT) {       // one plane of one ring row per thread
+         unsigned char *const plane = s_ring + (rc / C16) * a.RS + (rc % C16) * a.PL;
+         for (int pc = 0; pc < npad; ++pc) {
+            const int wp = pc < a.pw ? pc : pc + a.W;
+            *reinterpret_cast<v4i *>(plane + column_slot(wp) * 16) = fillv;
+         }
       }
    };
 
@@ -525,6 +527,8 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (per < 1) per = 1;
    const int units = (int)((mtot + unit - 1) / unit);
    if (per > units) per = units;
+   a.units_each = units / per;
+   a.units_rem = units % per;
    const dim3 grid((unsigned)(per * nob)), block(512);
 #define SOFIE_QRING_LAUNCH(C16_, WN_, ROW_, POOL_)                                                             \
    do {                                                                                                        \
