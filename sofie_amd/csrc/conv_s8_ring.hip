@@ -503,7 +503,16 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    // stored apart); padded so that the first pixel of the next output row continues that sequence modulo the 256 bytes
    // the LDS banks span.
    a.RS = C16 * a.PL;
-   a.RS += (((TW * 16 - a.RS) % 256) + 256) % 256;
+   {
+      // rpp ring rows lie between two output rows: rpp * RS = TW * 16 modulo 256, as nearly as a multiple of 16 allows
+      int best = 0, best_miss = 1 << 30;
+      for (int pad = 0; pad < 256; pad += 16) {
+         const int miss = ((rpp * (a.RS + pad) - TW * 16) % 256 + 256) % 256;
+         const int dist = miss < 256 - miss ? miss : 256 - miss;
+         if (dist < best_miss) { best_miss = dist; best = pad; }
+      }
+      a.RS += best;
+   }
    a.row_bytes = g.W * g.C;
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
    a.xbytes = (unsigned)xbytes;
