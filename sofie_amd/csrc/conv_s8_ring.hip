@@ -1,9 +1,9 @@
 // int8 3x3 stride-1 convolution on the matrix cores whose input travels global memory -> LDS without registers.
 //
 // k_qconv_ring: the implicit GEMM of conv_s8.hip (NHWC activations, weights [OC][3][3][C], C = 32 or 64, the
-// workgroup's weight slice resident in LDS, 8 wavefronts of 2 x 2 accumulator tiles of 32 x 32) with another way of
-// getting the input there:
-//   * a workgroup owns a CONTIGUOUS run of pixel tiles of the linear (n, oh, ow) order, so the rows of the padded
+// workgroup's weight slice resident in LDS, 8 wavefronts of 2 x 2 accumulator tiles of 32 x 32, optionally the fused
+// 2x2 pooling) with another way of getting the input there:
+//   * a workgroup owns a CONTIGUOUS run of pixels of the linear (n, oh, ow) order, so the rows of the padded
 //     images it needs ("virtual rows": image n, padded row r -> n*HP + r) form a window that slides down; they
 //     live in a ring of R rows in LDS (row v in slot v % R). A tile only fetches the rows the previous tile did not
 //     have, and they are fetched while the previous tile is multiplied: the ring has room for the rows of two
@@ -11,12 +11,15 @@
 //   * rows are fetched with buffer_load_dwordx4 ... lds: a wavefront instruction moves 64 x 16 bytes into 1 KB of
 //     consecutive LDS, the global address is free per lane. A ring row is stored as C/16 planes
 //     [16-byte channel chunk][padded column][16 bytes]; one instruction fills one plane of one row (lane = padded
-//     column, lanes of padding columns switched off). The vector unit spends nothing on staging: no address
-//     arithmetic per 16 bytes, no registers, no LDS writes. Padding columns are written once with the input
-//     zero-point when the kernel starts, padding rows by one LDS write per plane when such a row enters the ring.
+//     column), or the whole row where all its planes fit the 64 lanes; lanes of padding columns are switched off.
+//     The vector unit spends nothing on staging: no address arithmetic per 16 bytes, no registers, no LDS writes.
+//     Padding columns are written once with the input zero-point when the kernel starts, padding rows by one LDS
+//     write when such a row enters the ring. The weights arrive the same way.
 //   * in a plane consecutive pixels are 16 bytes apart, so the 16-byte-per-lane operand read of consecutive pixels
 //     covers consecutive banks; the row pitch is padded so that this also holds across the end of an output row.
-//     The nine taps of a pixel are its base address (per kernel row and channel half) plus a constant.
+//     The nine taps of a pixel are its base address (per kernel row and channel half) plus a constant. With the
+//     pooling, where consecutive lanes are two columns apart, a plane holds its even columns first and its odd
+//     columns behind them, to the same effect.
 #include "common.h"
 #include "conv_s8.h"
 #include "gemm_tile.h"
