@@ -66,6 +66,35 @@ def test_qconv2d_s8_matrix_core_shapes(ops, seed):
         assert np.array_equal(yp.transpose(0, 3, 1, 2), pooled), (C, OC, k, s, p, H, W, N, "pooled")
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_qconv2d_s8_many_small_images(ops, seed):
+    """3x3 stride-1 layers on thousands of small images: every workgroup of the kernel that keeps a sliding window of
+    input rows in LDS walks through several tiles and many image borders; with and without the fused pooling."""
+    from sofie_amd import lib as L
+    r = np.random.default_rng(9500 + seed)
+    C, OC = (32, 128) if seed % 2 == 0 else (64, 128)
+    H, W = int(r.integers(5, 10)), int(r.integers(5, 10))
+    p = tuple(int(v) for v in r.integers(0, 3, 4))
+    OH, OW = _out_hw(H, W, (3, 3), (1, 1), p)
+    N = int(r.integers(70000, 110000)) // (OH * OW)        # 2 - 3 tiles of 256 pixels per workgroup
+    x = r.integers(-128, 128, (N, H, W, C)).astype(np.int8)
+    w = r.integers(-127, 128, (OC, C, 3, 3)).astype(np.int8)
+    scale = (r.uniform(20, 60, OC) / (73.3 * 73.3 * np.sqrt(9.0 * C))).astype(np.float32)
+    if seed % 3 == 0:
+        scale[::7] *= -1.0
+    bias = r.integers(-3000, 3000, OC).astype(np.int32)
+    zpx, zpy, relu = int(r.choice([-128, 0, 5])), int(r.choice([-128, 3])), bool(r.integers(0, 2))
+    ref = oracle.qconv2d_s8(x.transpose(0, 3, 1, 2), w, scale, bias, p, (1, 1), 1, zpx, zpy, relu)
+    wh = np.ascontiguousarray(w.transpose(0, 2, 3, 1))
+    y = ops.qconv2d_s8(x, wh, scale, bias, p, (1, 1), 1, zpx, zpy, relu, x_layout=L.LAYOUT_NHWC, y_layout=L.LAYOUT_NHWC,
+                       w_layout=L.LAYOUT_NHWC)
+    assert np.array_equal(y.transpose(0, 3, 1, 2), ref), (C, OC, p, H, W, N)
+    pooled = oracle.maxpool2d(ref, (2, 2), (2, 2))
+    yp = ops.qconv2d_pool_s8(x, wh, scale, bias, p, (1, 1), 1, zpx, zpy, relu, x_layout=L.LAYOUT_NHWC,
+                             y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+    assert np.array_equal(yp.transpose(0, 3, 1, 2), pooled), (C, OC, p, H, W, N, "pooled")
+
+
 @pytest.mark.parametrize("seed", range(16))
 def test_qconv2d_s8_any_shape(ops, seed):
     """NCHW operands, any channel count and group count: the one-thread-per-output kernel and, for one input channel
