@@ -39,7 +39,7 @@ struct QConvRingArgs {
    GemmArgs ep;          // Y, scale, bias, M = N*OH*OW, N = OC, ldy = OC, zp, lo, relu
    int H, W, C, ph, pw, OH, OW, HP, WP;
    int K, KS;            // bytes of one weight row, its LDS stride
-   int RS, PL, R;        // ring: row pitch and plane pitch in bytes, rows (a power of two)
+   int RS, PL, R;        // ring: row pitch and plane pitch in bytes, rows
    int row_bytes;        // W * C: one image row in global memory
    int units_each, units_rem;   // 64-pixel (32 pooled pixel) units per workgroup of a channel block: quotient and remainder
    int gap;              // HP - OH * (rows per pixel): padded rows between the last window row of an image and the next image
@@ -98,17 +98,18 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    ep.M = mtot;
 
    // ---- weights of this channel block: resident for the life of the workgroup. They travel like the input rows, straight
-   // into LDS: an instruction fills as many padded LDS rows as fit its 64 slots (one row of 36 chunks and the pad, three
-   // rows of 18), and all of a wavefront's requests are in flight together.
+   // into LDS: an instruction fills 64 consecutive 16-byte slots of the padded LDS rows (a row of 36 chunks and its pad,
+   // then the start of the next row), lanes on pad slots switched off, and all of a wavefront's requests are in flight
+   // together.
    auto stage_weights = [&]() {
       const int K16 = a.K >> 4, KS16 = a.KS >> 4;
-      const int rpi = 64 / KS16;                                   // LDS rows per instruction
-      const int sub = fdiv(lane, a.dKS16), chunk = lane - sub * KS16;
-      const bool used = sub < rpi && chunk < K16;
+      const int slots = OCT * KS16;
       const rsrc_t wrs = make_rsrc(a.w + (size_t)ob * OCT * a.K, (unsigned)(OCT * a.K));
       const unsigned w0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)s_w;
-      for (int r0 = wave * rpi; r0 < OCT; r0 += NWAVE * rpi) {
-         if (used && r0 + sub < OCT) dma16(wrs, w0 + (unsigned)(r0 * a.KS), sub * a.K + chunk * 16, r0 * a.K);
+      for (int s0 = wave * 64; s0 < slots; s0 += NWAVE * 64) {
+         const int slot = s0 + lane;
+         const int row = fdiv(slot, a.dKS16), chunk = slot - row * KS16;
+         if (chunk < K16 && slot < slots) dma16(wrs, w0 + (unsigned)(s0 * 16), row * a.K + chunk * 16, 0);
       }
       stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
    };
@@ -375,7 +376,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // whether the wavefront has pixels in tile tt (all tiles but the last are full)
    auto has_work = [&](int tt) { return m_begin + tt * TM + wm * MBP * 32 < mtot; };
 
-   // The wavefronts that share a SIMD (w, w + 4[, w + 8]) do their parts of a tile in different order, so that the
+   // The two wavefronts that share a SIMD (w and w + 4) do their parts of a tile in different order, so that the
    // matrix pipe always has a wavefront feeding it: wavefronts 0-3 multiply tile t first, then requantise it and
    // compute the addresses of tile t + 1; the others first requantise their tile t - 1 and compute the addresses of
    // tile t, and multiply last, up to the barrier that ends the tile.
