@@ -26,7 +26,8 @@ namespace {
 // Geometry of one output phase of a strided transposed convolution when all phases run in one launch.
 struct PhaseArgs {
    int KH, KW, th0, tw0, ph, pw, oy0, ox0, OH, OW, rows_out, PH, PW, ICB, KC;
-   FastDiv dPW, dPH, dKC, dOW;
+   int woff;           // k_conv2d_f32_pipe: first float of the phase's sub-kernel in the gathered weights
+   FastDiv dPW, dPH, dKC, dOW, dK4;
 };
 #define SOFIE_CONV_MAX_PHASES 4
 
@@ -276,11 +277,44 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
 // per block. Blocks are small enough for a thread to carry its share: at most NP patch values and NW weights
 // (the launcher picks the channels per block accordingly and falls back to k_conv2d_f32 otherwise). Plain
 // convolutions only.
-template <int TI, int TJ>
-__global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs g)
+// PHASES: the launch holds the output phases of a strided transposed convolution (blockIdx.z = image * nphases +
+// phase). A phase is a plain unit-stride convolution of the input with its sub-kernel (g.w then holds the sub-kernels
+// gathered into the plain [OC][C][KH][KW] order, one after the other) whose outputs go to every stride-th pixel of the
+// output plane.
+template <int TI, int TJ, bool PHASES = false>
+__global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
 {
    constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
    constexpr int NP = SOFIE_CONV_PIPE_PATCH / 256, NW = SOFIE_CONV_PIPE_WEIGHTS / 256;
+   // geometry of this workgroup: the launch's own, or that of its phase (picked with static indices so that it stays
+   // in scalar registers)
+   struct Geometry {
+      const float *x, *w, *bias;
+      float *y;
+      int C, H, W, OC, KH, KW, ph, pw, sh, sw, dh, dw, OH, OW, icg, ocg, ICB, KC, PH, PW, relu;
+      FastDiv dPW, dPH, dK4;
+   } g;
+   g.x = gg.x; g.w = gg.w; g.bias = gg.bias; g.y = gg.y;
+   g.C = gg.C; g.H = gg.H; g.W = gg.W; g.OC = gg.OC; g.KH = gg.KH; g.KW = gg.KW; g.ph = gg.ph; g.pw = gg.pw;
+   g.sh = gg.sh; g.sw = gg.sw; g.dh = gg.dh; g.dw = gg.dw; g.OH = gg.OH; g.OW = gg.OW; g.icg = gg.icg; g.ocg = gg.ocg;
+   g.ICB = gg.ICB; g.KC = gg.KC; g.PH = gg.PH; g.PW = gg.PW; g.relu = gg.relu;
+   g.dPW = gg.dPW; g.dPH = gg.dPH; g.dK4 = gg.dK4;
+   int n = blockIdx.z;
+   int oy0 = 0, ox0 = 0;
+   FastDiv dOW = gg.dOW;
+   if constexpr (PHASES) {
+      const int pi = blockIdx.z % gg.nphases;
+      n = blockIdx.z / gg.nphases;
+      PhaseArgs q = gg.phase[0];
+#pragma unroll
+      for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
+         if (pi == i) q = gg.phase[i];
+      if ((int)blockIdx.x * BP >= q.OH * q.OW) return;   // the grid is as wide as the phase with most pixel tiles
+      g.KH = q.KH; g.KW = q.KW; g.ph = q.ph; g.pw = q.pw; g.OH = q.OH; g.OW = q.OW; g.ICB = q.ICB; g.KC = q.KC;
+      g.PH = q.PH; g.PW = q.PW; g.dPW = q.dPW; g.dPH = q.dPH; g.dK4 = q.dK4;
+      g.w = gg.w + q.woff;
+      oy0 = q.oy0; ox0 = q.ox0; dOW = q.dOW;
+   }
    extern __shared__ __align__(16) unsigned char smem_raw[];
    const int patch_len = g.ICB * g.PH * g.PW;
    const int buf_len = g.KC * LDW + patch_len;                       // floats of one buffer: [KC][LDW] weights, patch
@@ -293,7 +327,6 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs g)
    const int octiles = (g.ocg + BOC - 1) / BOC;
    const int grp = blockIdx.y / octiles;
    const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
-   const int n = blockIdx.z;
    const int OHW = g.OH * g.OW;
    const int p0 = blockIdx.x * BP;
    const int oh0 = p0 / g.OW;
@@ -402,13 +435,19 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs g)
       __syncthreads();
    }
 
-   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * OHW;
+   const size_t plane = PHASES ? (size_t)gg.OH0 * gg.OW0 : (size_t)OHW;
+   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane;
 #pragma unroll
    for (int i = 0; i < TI; ++i)
 #pragma unroll
       for (int j = 0; j < TJ; ++j) {
          const int p = p0 + wn * TJ * 32 + j * 32 + fr;
          if (p >= OHW) continue;
+         size_t po = (size_t)p;
+         if constexpr (PHASES) {
+            const int row = fdiv(p, dOW);
+            po = (size_t)(oy0 + row * gg.oys) * gg.OW0 + ox0 + (p - row * g.OW) * gg.oxs;
+         }
 #pragma unroll
          for (int r = 0; r < 16; ++r) {
             const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
@@ -416,9 +455,33 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs g)
             float v = acc[i][j][r];
             if (g.bias) v = __fadd_rn(v, g.bias[grp * g.ocg + oc]);
             if (g.relu) v = v > 0.0f ? v : 0.0f;
-            yn[(size_t)oc * OHW + p] = v;
+            yn[(size_t)oc * plane + po] = v;
          }
       }
+}
+
+// Sub-kernels of the output phases of a strided transposed convolution, gathered from its weights w [C, OC/groups, KH0,
+// KW0] into the order a plain convolution reads: phase after phase, each [groups][OC/groups][C/groups][KH][KW] with tap
+// (a, b) = element (th0 + a*ths, tw0 + b*tws) of the kernel. One thread per gathered value.
+__global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total)
+{
+   const int e = blockIdx.x * blockDim.x + threadIdx.x;
+   if (e >= total) return;
+   int pi = 0;
+#pragma unroll
+   for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
+      if (i < g.nphases && e >= g.phase[i].woff) pi = i;
+   PhaseArgs q = g.phase[0];
+#pragma unroll
+   for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
+      if (pi == i) q = g.phase[i];
+   int r = e - q.woff;
+   const int b = r % q.KW; r /= q.KW;
+   const int a = r % q.KH; r /= q.KH;
+   const int ic = r % g.icg; r /= g.icg;
+   const int oc = r % g.ocg;
+   const int grp = r / g.ocg;
+   dst[e] = g.w[((((size_t)grp * g.icg + ic) * g.ocg + oc) * g.KH0 + q.th0 + a * g.ths) * g.KW0 + q.tw0 + b * g.tws];
 }
 
 // One thread per output element: any kernel size, used when the staged patch of the tiled
@@ -542,6 +605,61 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    if ((size_t)g.groups * octiles > 65535 || (size_t)g.N * g.nphases > 65535) return SOFIE_HIP_OK;
    size_t lds_max = 0;
    int tiles_max = 0;
+   // First choice: the kernel that stages channel block c+1 under the matrix loop of block c, on sub-kernels gathered
+   // into the plain weight order (a small kernel in front, into the context's scratch buffer). Every phase must fit
+   // its limits (full channel blocks of K = 16 .. 80 with 16-byte weight loads, the values of a block in registers).
+   {
+      bool fits = true;
+      int woff = 0;
+      for (int i = 0; i < g.nphases && fits; ++i) {
+         PhaseArgs &p = g.phase[i];
+         const int KHW = p.KH * p.KW;
+         p.rows_out = (BP + p.OW - 2) / p.OW + 1;
+         if (p.rows_out > p.OH) p.rows_out = p.OH;
+         p.PH = (p.rows_out - 1) + (p.KH - 1) + 1;      // unit stride and dilation inside a phase
+         p.PW = (p.OW - 1) + (p.KW - 1) + 1;
+         bool found = false;
+         for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1 && !found; --icb) {
+            const int kc = icb * KHW;
+            const size_t plen = (size_t)icb * p.PH * p.PW;
+            const size_t lds = (2 * ((size_t)kc * LDW + plen) + kc) * 4;
+            if (kc < 16) break;
+            if (g.icg % icb != 0 || kc % 4 != 0 || lds > budget || (size_t)kc * BOC > SOFIE_CONV_PIPE_WEIGHTS ||
+                plen > SOFIE_CONV_PIPE_PATCH)
+               continue;
+            p.ICB = icb;
+            p.KC = kc;
+            p.dPW = make_fastdiv((unsigned)p.PW);
+            p.dPH = make_fastdiv((unsigned)p.PH);
+            p.dKC = make_fastdiv((unsigned)p.KC);
+            p.dK4 = make_fastdiv((unsigned)(p.KC / 4));
+            p.dOW = make_fastdiv((unsigned)p.OW);
+            if (lds > lds_max) lds_max = lds;
+            found = true;
+         }
+         fits = found;
+         p.woff = woff;
+         woff += g.groups * g.ocg * g.icg * KHW;         // a multiple of 4 floats: kc is, and icg is a multiple of icb
+         if (cdiv(p.OH * p.OW, BP) > tiles_max) tiles_max = cdiv(p.OH * p.OW, BP);
+      }
+      if (fits) {
+         void *ws = nullptr;
+         if (int rc = workspace(ctx, (size_t)woff * sizeof(float), &ws)) return rc;
+         hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
+                            static_cast<float *>(ws), woff);
+         if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
+         ConvArgs h = g;
+         h.w = static_cast<const float *>(ws);
+         auto kern = k_conv2d_f32_pipe<TI, TJ, true>;
+         SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+         hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
+         *done = true;
+         return check_launch(ctx, "k_conv2d_f32_pipe (phases)");
+      }
+      lds_max = 0;
+      tiles_max = 0;
+   }
    for (int i = 0; i < g.nphases; ++i) {
       PhaseArgs &p = g.phase[i];
       const int KHW = p.KH * p.KW;

@@ -68,6 +68,8 @@ def test_reference_known_answers_through_hip(ops, name):
     dict(N=1, C=6, H=4, W=4, OC=4, k=(2, 3), s=(3, 2), p=(0, 1, 0, 1), d=(2, 1), g=2, op=(1, 1)),
     dict(N=2, C=3, H=7, W=5, OC=5, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(1, 0)),
     dict(N=3, C=64, H=14, W=14, OC=96, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(0, 0)),   # 128-channel tile
+    dict(N=4, C=128, H=28, W=28, OC=64, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=1, op=(0, 0)),  # the benchmark's layer: phases on gathered sub-kernels
+    dict(N=2, C=24, H=9, W=10, OC=16, k=(4, 4), s=(2, 2), p=(1, 1, 1, 1), d=(1, 1), g=2, op=(1, 1)),     # ... with groups and output padding
     dict(N=2, C=32, H=9, W=11, OC=32, k=(3, 3), s=(1, 1), p=(1, 1, 1, 1), d=(1, 1), g=4, op=(0, 0)),    # stride 1, groups
     dict(N=1, C=8, H=6, W=6, OC=8, k=(3, 3), s=(2, 2), p=(2, 2, 2, 2), d=(1, 1), g=1, op=(1, 1)),       # pad = kernel - 1
     dict(N=1, C=4, H=5, W=5, OC=4, k=(2, 2), s=(1, 1), p=(2, 2, 2, 2), d=(1, 1), g=1, op=(0, 0)),       # pad beyond the kernel
