@@ -229,6 +229,34 @@ def test_conv_transpose2d_f32_random_shapes(ops, seed):
     assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (C, OC, g, k, s, d, p, op, H, W)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_conv_transpose2d_f32_wide_layers(ops, seed):
+    """Transposed convolutions with enough input channels that every output phase is a multiply of at least 16 taps x
+    channels: the phases then run in the pipelined convolution kernel on gathered sub-kernels (uneven phases when the
+    kernel size is not a multiple of the stride, groups, output padding, pads that differ begin to end)."""
+    r = np.random.default_rng(9700 + seed)
+    g = int(r.choice([1, 1, 2, 4]))
+    C, OC = g * int(r.choice([4, 8, 12, 16, 32])), g * int(r.integers(1, 20))
+    k = (int(r.integers(2, 6)), int(r.integers(2, 6)))
+    s = (int(r.integers(1, 4)), int(r.integers(1, 4)))
+    d = (1, 1) if seed % 4 else (int(r.integers(1, 3)), int(r.integers(1, 3)))
+    H, W = int(r.integers(2, 24)), int(r.integers(2, 24))
+    p = tuple(int(v) for v in r.integers(0, 3, 4))
+    op = (int(r.integers(0, s[0])), int(r.integers(0, s[1])))
+    OH = s[0] * (H - 1) + d[0] * (k[0] - 1) + 1 + op[0] - p[0] - p[2]
+    OW = s[1] * (W - 1) + d[1] * (k[1] - 1) + 1 + op[1] - p[1] - p[3]
+    if OH < 1 or OW < 1:
+        pytest.skip("empty output")
+    N = int(r.integers(1, 4))
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = r.standard_normal((C, OC // g) + k).astype(np.float32)
+    b = r.standard_normal(OC).astype(np.float32) if seed % 2 else None
+    ref = oracle.conv_transpose2d_f32(x, w, b, p, s, d, g, op)
+    got = ops.conv_transpose2d_f32(x, w, b, p, s, d, g, op)
+    assert got.shape == ref.shape
+    assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (C, OC, g, k, s, d, p, op, H, W, N)
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_gemm_fp8_random_shapes(ops, seed):
     """The tolerance of the FP8 GEMM (one bf16 rounding of the result plus 2^-15 of the sum of magnitudes, against
