@@ -111,8 +111,12 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
          const int row = fdiv(slot, a.dKS16), chunk = slot - row * KS16;
          if (chunk < K16 && slot < slots) dma16(wrs, w0 + (unsigned)(s0 * 16), row * a.K + chunk * 16, 0);
       }
-      stage_column_params(a.ep, s_scale, s_bias, tid, ob * OCT, OCT);
    };
+   // The weights are requested before anything else is set up and the channels' scales and biases are fetched into
+   // registers in front of them: both are on their way while the rows of the first tile are worked out and requested,
+   // and nothing in the prologue waits for memory before its last line.
+   const ColumnParams col_params = load_column_params(a.ep, tid, ob * OCT, OCT);
+   stage_weights();
    // Slot of a padded column inside a plane. With the fused pooling the even columns come first, then the odd ones:
    // the pixels of consecutive lanes are two columns apart, and this keeps their 16 bytes next to each other.
    const int half_cols = (a.WP + 1) >> 1;
@@ -388,9 +392,11 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       req_finish();
       if (mma_first) pixel_offsets(t);
    }
-   // the rows of the first tile are on their way while the weights are staged
-   stage_weights();
    fill_padding_columns();
+   if (tid < OCT) {
+      s_scale[tid] = col_params.scale;
+      s_bias[tid] = col_params.bias;
+   }
    wait_vmcnt<0>();
    __syncthreads();                          // weights, column parameters, padding columns and the first rows are in LDS
    if constexpr (POOL) {
