@@ -323,6 +323,77 @@ __device__ __forceinline__ void tile_epilogue(const GemmArgs &g, typename Mma::A
                                               n0 + wn * WN);
 }
 
+// The same epilogue for accumulators of the 16 x 16 matrix instructions (v_mfma_i32_16x16x64_i8): a wavefront owns
+// NI x MJ tiles; a lane holds output row m = lane % 16 of a tile and its columns (lane / 16) * 4 .. + 3. Two tiles
+// along m (32 rows) go through the staging block [32 m][NI*16 n] per pass, then leave as 16-byte row segments.
+// The staging block has the size of EpilogueStaging<NI / 2, OUT>.
+template <int NI, int MJ, int OUT, int PLAIN>
+__device__ __forceinline__ void tile_epilogue_wave16(const GemmArgs &g, v4i (&acc)[NI][MJ], unsigned char *stg,
+                                                     const float *s_scale, const int *s_bias, int lane, int m_wave,
+                                                     int n_wave)
+{
+   static_assert(MJ % 2 == 0, "passes of two tiles along m");
+   constexpr int ESZ = OutSize<OUT>::value;
+   static_assert(ESZ == 1 || ESZ == 4, "int8 or 32-bit outputs");
+   constexpr int WN = NI * 16;
+   constexpr int SROW = WN * ESZ + 16;
+   constexpr int CR = WN * ESZ / 16;
+   const int l16 = lane & 15;
+   const int nq = (lane >> 4) * 4;
+   const float zpo = (float)(g.zp + 128), lof = (float)(g.lo + 128);
+#pragma unroll
+   for (int jp = 0; jp < MJ; jp += 2) {
+#pragma unroll
+      for (int ni = 0; ni < NI; ++ni) {
+         const int nl = ni * 16 + nq;
+         const v4f sc = *reinterpret_cast<const v4f *>(s_scale + nl);
+         const v4i bi = *reinterpret_cast<const v4i *>(s_bias + nl);
+#pragma unroll
+         for (int jj = 0; jj < 2; ++jj) {
+            const v4i a = acc[ni][jp + jj];
+            unsigned char *dst = stg + (jj * 16 + l16) * SROW + nl * ESZ;
+            if constexpr (ESZ == 1) {
+               unsigned pk = 0;
+#pragma unroll
+               for (int t = 0; t < 4; ++t) {
+                  float r = __fmul_rn(__int2float_rn(a[t] + bi[t]), sc[t]);
+                  if constexpr (PLAIN == 0) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
+                  if constexpr (PLAIN == 2) r = __fadd_rn(rintf(r), zpo);
+                  pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);     // rounds half to even, saturates at 0 and 255
+               }
+               *reinterpret_cast<unsigned *>(dst) = pk ^ 0x80808080u;
+            } else {
+               v4i p;
+#pragma unroll
+               for (int t = 0; t < 4; ++t) p[t] = (int)epilogue_value<true, OUT>(g, sc[t], bi[t], a[t], 0.0f);
+               *reinterpret_cast<v4i *>(dst) = p;
+            }
+         }
+      }
+      __builtin_amdgcn_wave_barrier();
+      constexpr int ITERS = 32 * CR / 64;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+         const int c = it * 64 + lane;
+         const int row = c / CR, cc = c % CR;
+         const int m = m_wave + jp * 16 + row;
+         const int nfirst = n_wave + cc * (16 / ESZ);
+         if (m < g.M && nfirst < g.N) {
+            const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
+            unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
+            if (g.vec_store && nfirst + 16 / ESZ <= g.N) {
+               *reinterpret_cast<v4i *>(out) = v;
+            } else {
+               const unsigned char *src = stg + row * SROW + cc * 16;
+               const int cnt = (g.N - nfirst) < (16 / ESZ) ? (g.N - nfirst) : (16 / ESZ);
+               for (int b = 0; b < cnt * ESZ; ++b) out[b] = src[b];
+            }
+         }
+      }
+      __builtin_amdgcn_wave_barrier();
+   }
+}
+
 // ---- global memory -> LDS without registers (buffer_load ... lds), shared by the GEMM and the convolution
 typedef int rsrc_t __attribute__((ext_vector_type(4)));
 
