@@ -543,14 +543,14 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    tile_epilogue<Mma, TI, TJ, OUT, 8>(g, acc, smem, tid, m0 + wm * 64, n0, wn, BN, &col_params);
 }
 
-// k_gemm_dma16: the int8 kernel above (B^T [N,K]) on v_mfma_i32_16x16x64_i8 instead of v_mfma_i32_32x32x32_i8.
+// k_gemm_dma16: the int8 kernel above (B^T [N,K] or B [K,N]) on v_mfma_i32_16x16x64_i8 instead of v_mfma_i32_32x32x32_i8.
 // Same tile, stages, requests and two-group schedule; a wavefront's 128 x 64 part is 8 x 4 accumulator tiles of
 // 16 x 16. The instruction does the same multiply-adds per cycle, writes half as many accumulator values per
 // multiply-add and draws less power: under the device's power limit a loop of it on random operands sustains about
 // 13 % more than the 32 x 32 one (4.0 against 3.5 POP/s). A lane supplies row (lane % 16) of a tile and the 16 bytes of
 // K number lane / 16 of a 64-byte sub-step, so its LDS address is the row's base plus chunk ((lane / 16) ^ swizzle)
 // and the second sub-step of a 128-byte stage is that address XOR 64.
-template <int OUT>
+template <int OUT, bool B_KN>
 __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
 {
    constexpr int BK = 128, NST = 2;
@@ -576,7 +576,11 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
    const int rows_total = uses_a ? g.M : g.N;
    const int row0 = uses_a ? m0 : n0;
    const int rows_left = (rows_total - row0) < 256 ? (rows_total - row0) : 256;
-   const rsrc_t rs = make_rsrc((uses_a ? g.A : g.B) + (size_t)row0 * ld, (unsigned)((size_t)(rows_left - 1) * ld + g.K));
+   const bool rows_are_k = B_KN && !uses_a;            // B [K,N]: a load block is 4 rows of k x 256 bytes of n
+   const unsigned char *tile_base = rows_are_k ? g.B + n0 : (uses_a ? g.A : g.B) + (size_t)row0 * ld;
+   // rows of k past K lie beyond the descriptor and read as zeros
+   const rsrc_t rs = make_rsrc(tile_base, rows_are_k ? (unsigned)((size_t)(g.K - 1) * ld + (g.N - n0))
+                                                     : (unsigned)((size_t)(rows_left - 1) * ld + g.K));
    const int blk0 = (wave & 3) * LPW;
    const int lrow = lane / CPR;
    const bool ktail = (g.K % BK) != 0;
@@ -588,15 +592,28 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
       voff[par] = (blk0 * RPB + lrow) * ld + chunk * 16;
       voff_tail[par] = (ktail && (nk - 1) * BK + chunk * 16 >= g.K) ? 0x7ffffff0 : voff[par];
    }
+   if (rows_are_k) {
+      // [K,N] stage: row k holds 256 bytes of n as eight 32-byte pairs, pair p stored in slot p ^ (k & 7), so that
+      // the transposing LDS reads (eight rows of k, 16 bytes of n each) of a group of 16 lanes cover distinct banks
+#pragma unroll
+      for (int par = 0; par < 2; ++par) {
+         const int krow = par * 4 + (lane >> 4);
+         const int slot = lane & 15;
+         const int chunk = (((slot >> 1) ^ (krow & 7)) << 1) | (slot & 1);
+         voff[par] = (blk0 * 4 + (lane >> 4)) * ld + chunk * 16;
+         voff_tail[par] = voff[par];
+      }
+   }
    const unsigned dst0 = lds0 + (uses_a ? 0 : BREG) + blk0 * 1024;
-   const int row_step = RPB * ld;
+   const int row_step = rows_are_k ? 4 * ld : RPB * ld;
+   const int k_step = rows_are_k ? BK * ld : BK;
    auto request = [&](int t, int S) {
       const int tt = t < nk ? t : nk - 1;
-      const bool tail = ktail && tt == nk - 1;
+      const bool tail = ktail && tt == nk - 1;      // B [K,N]: both offsets are the same
       const int v0 = tail ? voff_tail[0] : voff[0], v1 = tail ? voff_tail[1] : voff[1];
       const unsigned dst = dst0 + S * (uses_a ? ABYTES : BBYTES);
 #pragma unroll
-      for (int i = 0; i < LPW; ++i) dma16(rs, dst + i * 1024, (i & 1) ? v1 : v0, i * row_step + tt * BK);
+      for (int i = 0; i < LPW; ++i) dma16(rs, dst + i * 1024, (i & 1) ? v1 : v0, i * row_step + tt * k_step);
    };
    // --- operand addresses: row lane % 16 of a tile, chunk (lane / 16) of the sub-step, swizzled by the row
    const int fr = lane & 15, kg = lane >> 4;
@@ -609,6 +626,22 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
       m_base[sub] = smem + (m_off ^ (sub * 64));
       n_base[sub] = smem + (n_off ^ (sub * 64));
    }
+   // B [K,N]: ds_read_b64_tr_b8 hands a lane eight consecutive k of its column. Of a group of 16 lanes (one 16-byte
+   // chunk of K), lane s points at row (s >> 1), bytes (s & 1) * 8 .. + 7 of the tile's 16 columns; lane t of the group
+   // then receives column t of those eight rows. Two tiles share a 32-byte pair: the pair's slot is XORed into the
+   // address, the half of the pair, the sub-step, the eight-row half and the stage are constants on top.
+   const int ts = lane & 15;
+   const int kn_off = BREG + (ts >> 1) * 256 + ((((wn * 4) ^ (ts >> 1)) & 7) * 32) + (ts & 1) * 8 + kg * 16 * 256;
+   const unsigned char *kn_base[NI / 2];
+#pragma unroll
+   for (int ip = 0; ip < NI / 2; ++ip) kn_base[ip] = smem + (kn_off ^ (ip * 32));
+   auto load_frag_kn = [&](int i, int stage_off, int sub) -> v4i {
+      typedef int v2i_t __attribute__((ext_vector_type(2)));
+      const unsigned char *p = kn_base[i >> 1] + (i & 1) * 16 + sub * 64 * 256 + stage_off;
+      const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((v2i_t __attribute__((address_space(3))) *)(p));
+      const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((v2i_t __attribute__((address_space(3))) *)(p + 8 * 256));
+      return v4i{lo[0], lo[1], hi[0], hi[1]};
+   };
    v4i acc[NI][MJ];
 #pragma unroll
    for (int i = 0; i < NI; ++i)
@@ -635,7 +668,10 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
 #pragma unroll
       for (int sub = 0; sub < NSUB; ++sub) {
 #pragma unroll
-         for (int i = 0; i < NI; ++i) fn[sub][i] = *reinterpret_cast<const v4i *>(n_base[sub] + i * 16 * BK + S * BBYTES);
+         for (int i = 0; i < NI; ++i) {
+            if constexpr (B_KN) fn[sub][i] = load_frag_kn(i, S * BBYTES, sub);
+            else fn[sub][i] = *reinterpret_cast<const v4i *>(n_base[sub] + i * 16 * BK + S * BBYTES);
+         }
 #pragma unroll
          for (int j = 0; j < MJ; ++j) fm[sub][j] = *reinterpret_cast<const v4i *>(m_base[sub] + j * 16 * BK + S * ABYTES);
       }
@@ -942,8 +978,8 @@ int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
    static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
    g.tiles_m = cdiv(g.M, 256);
    g.tiles_n = cdiv(g.N, 256);
-   if constexpr (__is_same(Mma, MmaI8) && !B_KN && BK == 128 && SOFIE_GEMM16) {
-      auto kern16 = k_gemm_dma16<OUT>;
+   if constexpr (__is_same(Mma, MmaI8) && BK == 128 && SOFIE_GEMM16) {
+      auto kern16 = k_gemm_dma16<OUT, B_KN>;
       SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern16),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
       hipLaunchKernelGGL(kern16, dim3(g.tiles_m * g.tiles_n), dim3(512), lds, ctx->stream, g);
