@@ -21,6 +21,7 @@
 //     pooling, where consecutive lanes are two columns apart, a plane holds its even columns first and its odd
 //     columns behind them, to the same effect.
 #include "common.h"
+#include <type_traits>
 #include "conv_s8.h"
 #include "gemm_tile.h"
 
@@ -66,6 +67,12 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    constexpr int RPP = POOL ? 2 : 1;                // convolution rows (and columns) per (pooled) pixel
    constexpr int NWAVE = 8, NT = NWAVE * 64;
    constexpr bool REGS = !POOL;                     // scales and bias tiles in registers
+   // 64 input channels without pooling: v_mfma_i32_16x16x64_i8 (a tap's 64 channels are one instruction's K) instead of
+   // two v_mfma_i32_32x32x32_i8. Same multiply-adds per cycle, less power, so a higher clock under the device's limit;
+   // and a lane group's four channels of four 16-channel tiles transpose into 64 contiguous bytes per pixel and store.
+   constexpr bool M16 = C16 == 4 && !POOL;
+   constexpr int NBT = M16 ? 4 : NB, MBT = M16 ? 4 : MB;   // accumulator tiles of a wavefront along channels, pixels
+   using AccT = std::conditional_t<M16, v4i, v16i>;
    constexpr int WM = NWAVE / WN;
    constexpr int TM = WM * MBP * 32;
    constexpr int OCT = WN * NB * 32;
@@ -83,6 +90,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
    const int wn = wave % WN, wm = wave / WN;
    const int half = lane >> 5, l32 = lane & 31;
+   const int kg = lane >> 4, l16 = lane & 15;           // 16 x 16 tiles: chunk of K and row / column of the lane
    const int nob = a.ep.N / OCT;
    const int ob = nob == 1 ? 0 : blockIdx.x % nob;
    const int wg = nob == 1 ? blockIdx.x : blockIdx.x / nob;
@@ -198,9 +206,10 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       return n1 * a.HP + (R1 - n1 * a.OH) * RPP + (RPP - 1) + 2;
    };
 
-   int b_off[NB];
+   int b_off[NBT];
 #pragma unroll
-   for (int i = 0; i < NB; ++i) b_off[i] = ((wn * NB + i) * 32 + l32) * a.KS + half * 16;
+   for (int i = 0; i < NBT; ++i)
+      b_off[i] = M16 ? ((wn * NB * 32 + i * 16 + l16) * a.KS + kg * 16) : (((wn * NB + i) * 32 + l32) * a.KS + half * 16);
    const int nq = half * 4;
    const float *const w_scale = s_scale + wn * NB * 32;
    const int *const w_bias = s_bias + wn * NB * 32;
@@ -212,7 +221,28 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // another constant.
    const unsigned char *pa[POOL ? 4 : 3][CB][2];   // last index: m tile, or parity of the column with the pooling
    const unsigned char *const lane_base = s_ring + half * a.PL;
+   const unsigned char *pa16[M16 ? 3 : 1][M16 ? 4 : 1];   // 16 x 16 tiles: kernel row, pixel tile; the lane's plane is kg
    auto pixel_offsets = [&](int tt) {
+      if constexpr (M16) {
+#pragma unroll
+         for (int j = 0; j < 4; ++j) {
+            int m = m_begin + tt * TM + wm * 64 + j * 16 + l16;
+            m = m < mtot ? m : mtot - 1;
+            const int R = (int)(__umulhi((unsigned)m, a.dOW.magic) >> a.dOW.shift);
+            const int ow = m - R * a.OW;
+            const int n = (int)(__umulhi((unsigned)R, a.dOH.magic) >> a.dOH.shift);
+            const int v = R + n * a.gap;
+            const unsigned char *const colb = s_ring + kg * a.PL + ow * 16;
+            unsigned slot = (unsigned)v - (__umulhi((unsigned)v, a.dR.magic) >> a.dR.shift) * (unsigned)a.R;
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+               pa16[r][j] = colb + slot * a.RS;
+               slot = slot + 1;
+               slot = slot < slot - (unsigned)a.R ? slot : slot - (unsigned)a.R;
+            }
+         }
+         return;
+      }
 #pragma unroll
       for (int j = 0; j < MBP; ++j) {
          int m = m_begin + tt * TM + (wm * MBP + j) * 32 + l32;
@@ -243,11 +273,53 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       }
    };
 
-   v16i r_bias[REGS ? NB : 1];
-   v4f r_scale[REGS ? NB * 4 : 1];
+   v16i r_bias[REGS && !M16 ? NB : 1];
+   v4f r_scale[REGS && !M16 ? NB * 4 : 1];
+   v4i r_bias16[M16 ? 4 : 1];       // 16 x 16 tiles: channels i * 16 + kg * 4 .. + 3 of tile i
+   v4f r_scale16[M16 ? 4 : 1];
    // K loop of one tile: unrolled over its 9 * CB steps; the fragment reads run two steps ahead of the matrix
    // instructions and one read is issued behind each of a step's first matrix instructions
-   auto kloop = [&](v16i (&acc)[NB][MB]) {
+   auto kloop = [&](AccT (&acc)[NBT][MBT]) {
+      if constexpr (M16) {
+         // one step per tap: four weight and four pixel fragments, 16 matrix instructions; a read of the next tap's
+         // fragments behind every second of them
+         v4i fa[2][4], fb[2][4];
+         const unsigned char *pb[4];
+#pragma unroll
+         for (int i = 0; i < 4; ++i) pb[i] = s_w + b_off[i];
+#pragma unroll
+         for (int s = 0; s < 9 + 1; ++s) {
+            if (s < 9) {
+               const int kh = s / 3, kw = s % 3;
+#pragma unroll
+               for (int i = 0; i < 4; ++i) {
+                  fb[s & 1][i] = *reinterpret_cast<const v4i *>(pb[i] + s * 64);
+                  fa[s & 1][i] = *reinterpret_cast<const v4i *>(pa16[kh][i] + kw * 16);
+               }
+            }
+            if (s >= 1) {
+               const int d = s - 1, buf = d & 1;
+#pragma unroll
+               for (int i = 0; i < 4; ++i)
+#pragma unroll
+                  for (int j = 0; j < 4; ++j)
+                     acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fb[buf][i], fa[buf][j], d == 0 ? r_bias16[i] : acc[i][j], 0, 0, 0);
+            }
+            if (s < 9 && s >= 1) {
+#pragma unroll
+               for (int gidx = 0; gidx < 8; ++gidx) {
+                  __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);   // two matrix instructions
+                  __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+               }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // four chances per tile to send a row request (measured against one behind every tap: 53.8 against
+            // 55.4 us on the 56x56 layer; the scalar bookkeeping of a request stands between two taps' instructions)
+            if (s < 9 && (s & 1)) req_step();
+         }
+         req_finish();
+         return;
+      } else {
       constexpr int NBUF = POOL ? 2 : 3;
       v4i fa[NBUF][MB], fb[NBUF][NB];
       const unsigned char *pb[NB];
@@ -306,16 +378,47 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
          if (s < NS && (NS <= 9 || (s & 1))) req_step();   // 9 chances per tile
       }
       req_finish();
+      }
    };
    // Requantisation and stores of one tile: a lane packs its four 4-channel groups of an accumulator tile into four
    // dwords, two swaps between the halves of the wavefront turn them into 16 consecutive channels, one 16-byte store.
    // (A store instruction so touches 32 pixels with 32 bytes each. Stores of 64 contiguous bytes per pixel, 16
    // pixels per instruction, take 5 % off the layer when the bytes are there for free, but moving them between lanes
    // through a private block of LDS costs what they gain.)
-   auto epilogue_as = [&](v16i (&acc)[NB][MB], int tt, auto plain_tag) {
+   auto epilogue_as = [&](AccT (&acc)[NBT][MBT], int tt, auto plain_tag) {
       constexpr bool PLAIN = decltype(plain_tag)::value;
       const int m_wave = m_begin + tt * TM + wm * MBP * 32, n_wave = ob * OCT + wn * NB * 32;
       const float zpo = (float)(ep.zp + 128), lof = (float)(ep.lo + 128);
+      if constexpr (M16) {
+         // A lane holds channels kg * 4 .. + 3 of each of the four 16-channel tiles of its pixel: packed, they are a
+         // 4 x 4 matrix of dwords over the pixel's four lanes (16 lanes apart), and two rounds of swaps (between the
+         // halves of the wavefront, then between neighbouring groups of 16 lanes) transpose it. Lane group kg then
+         // has the 16 channels of tile kg in order, and a store instruction writes 64 contiguous bytes for each of 16 pixels.
+#pragma unroll
+         for (int j = 0; j < 4; ++j) {
+            const int m = m_wave + j * 16 + l16;
+            int8_t *const row = static_cast<int8_t *>(ep.Y) + (size_t)(m < ep.M ? m : 0) * ep.ldy + n_wave + kg * 16;
+            unsigned d[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+               unsigned pk = 0;
+#pragma unroll
+               for (int e = 0; e < 4; ++e) {
+                  float r = __fmul_rn(__int2float_rn(acc[i][j][e]), r_scale16[i][e]);
+                  if constexpr (!PLAIN) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
+                  pk = __builtin_amdgcn_cvt_pk_u8_f32(r, e, pk);
+               }
+               d[i] = pk ^ 0x80808080u;
+            }
+            const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+            const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+            const auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+            const auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+            const v4i v = {(int)t01[0], (int)t01[1], (int)t23[0], (int)t23[1]};
+            if (m < ep.M) SOFIE_RING_STORE(reinterpret_cast<v4i *>(row), v);
+         }
+         return;
+      } else {
 #pragma unroll
       for (int j = 0; j < MBP; ++j) {
          const int m = m_wave + j * 32 + l32;
@@ -342,9 +445,10 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             if (m < ep.M) SOFIE_RING_STORE(reinterpret_cast<v4i *>(row + i * 32), v);
          }
       }
+      }
    };
    bool any_negative = false;   // pooled variant: some scale of the workgroup's channels is negative (set below)
-   auto epilogue = [&](v16i (&acc)[NB][MB], int tt) {
+   auto epilogue = [&](AccT (&acc)[NBT][MBT], int tt) {
       if constexpr (POOL) {
          const int m_wave = m_begin + tt * TM + wm * 32, n_wave = ob * OCT + wn * NB * 32;
          v16i pooled[NB][1];
@@ -405,7 +509,13 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       for (int c = tid; c < OCT; c += NT) neg |= s_scale[c] < 0.0f;
       any_negative = __syncthreads_or(neg) != 0;
    }
-   if constexpr (REGS) {
+   if constexpr (M16) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+         r_scale16[i] = *reinterpret_cast<const v4f *>(w_scale + i * 16 + kg * 4);
+         r_bias16[i] = *reinterpret_cast<const v4i *>(w_bias + i * 16 + kg * 4);
+      }
+   } else if constexpr (REGS) {
 #pragma unroll
       for (int gi = 0; gi < NB * 4; ++gi) {
          r_scale[gi] = *reinterpret_cast<const v4f *>(w_scale + (gi >> 2) * 32 + (gi & 3) * 8 + nq);
@@ -414,7 +524,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
          for (int e = 0; e < 4; ++e) r_bias[gi >> 2][(gi & 3) * 4 + e] = bi[e];
       }
    }
-   v16i acc[NB][MB];
+   AccT acc[NBT][MBT];
    // rows tile t + 1 has and tile t does not: requested during tile t into slots that tile t does not read
    auto request_next = [&](bool more, int tn, int &hi_next) {
       if (more) {
