@@ -313,7 +313,7 @@ def main():
                                "to int8, operands resident in HBM", "M": n, "N": n, "K": n, "seed": 0},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_INT8_TOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_INT8_TOPS, "traffic": TRAFFIC_BYTES_PER_CALL,
-                     "kernel": "k_gemm_dma<MmaI8,128,2,S8,B_KN>",
+                     "kernel": "k_gemm_dma16<S8,B_KN>",
                      "kernel_ms": kernel_ms, "kernel_ms_best_block": kernel_ms_best, "launches_timed": launches,
                      "kernel_ms_exceeds_ms_per_step": bool(kernel_ms > ms_per_step),
                      "ops_per_launch": ops_per_step, "algorithmic_bytes_per_launch": ALGORITHMIC_BYTES_PER_CALL,

@@ -46,7 +46,7 @@ struct QConvRingArgs {
    int gap;              // HP - OH * (rows per pixel): padded rows between the last window row of an image and the next image
    unsigned fill;        // zp_x replicated into four bytes
    unsigned xbytes;
-   FastDiv dOW, dOH, dHP, dKS16, dR, dWP;
+   FastDiv dOW, dOH, dHP, dKS16, dR, dPL16;   // dPL16: by the 16-byte slots of a plane
 };
 
 // C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels. The tile is (8/WN)*64 pixels x
@@ -147,10 +147,11 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    // wavefront (ROWDMA) or per group of C16 wavefronts, which take a plane each.
    const rsrc_t rs = make_rsrc(a.x, a.xbytes);
    const int my_plane = ROWDMA ? 0 : wave % C16, my_rl = ROWDMA ? wave : wave / C16;
-   const int slot_c = ROWDMA ? fdiv(lane, a.dWP) : my_plane;          // plane and padded column of the lane's 16 bytes
-   const int slot_wp = slot_column(ROWDMA ? lane - slot_c * a.WP : lane);
+   const int slot_c = ROWDMA ? fdiv(lane, a.dPL16) : my_plane;        // plane and padded column of the lane's 16 bytes
+   const int slot_pos = ROWDMA ? lane - slot_c * (a.PL >> 4) : lane;  // (a plane may be longer than the row: see the launcher)
+   const int slot_wp = slot_column(slot_pos);
    const int iw = slot_wp - a.pw;
-   const bool slot_used = ROWDMA ? lane < C16 * a.WP : lane < a.WP;
+   const bool slot_used = slot_pos < a.WP && (!ROWDMA || slot_c < C16);
    const bool col_data = slot_used && iw >= 0 && iw < a.W;
    const int voff = iw * a.C + slot_c * 16;
    // A request is scalar work plus one instruction per row; it is spread over the matrix loop of the present tile
@@ -617,22 +618,13 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    a.OH = TH; a.OW = TW; a.HP = HP; a.WP = WP;
    a.gap = HP - TH * rpp;
    a.K = 9 * g.C;
-   a.KS = ((a.K / 16) % 2 == 0) ? a.K + 16 : a.K;
-   a.PL = WP * 16;
-   // Row pitch: consecutive pixels of an output row are 16 bytes apart (with the pooling too: even and odd columns are
-   // stored apart); padded so that the first pixel of the next output row continues that sequence modulo the 256 bytes
-   // the LDS banks span.
-   a.RS = C16 * a.PL;
-   {
-      // rpp ring rows lie between two output rows: rpp * RS = TW * 16 modulo 256, as nearly as a multiple of 16 allows
-      int best = 0, best_miss = 1 << 30;
-      for (int pad = 0; pad < 256; pad += 16) {
-         const int miss = ((rpp * (a.RS + pad) - TW * 16) % 256 + 256) % 256;
-         const int dist = miss < 256 - miss ? miss : 256 - miss;
-         if (dist < best_miss) { best_miss = dist; best = pad; }
-      }
-      a.RS += best;
-   }
+   // The 64-channel layers without pooling run on 16 x 16 matrix instructions: a lane reads row (lane % 16) of a
+   // tile and chunk (lane / 16) of K. The LDS serves a 16-byte read of a wavefront in four rounds of 16 lanes
+   // (lanes 0-7 with 24-31, 8-15 with 16-23, and the same in the upper half), each free of conflicts if its lanes'
+   // 16-byte slots differ modulo 256 bytes (measured: 4.4 cycles per read against 8.1). For the pixels that asks for
+   // planes a multiple of 256 bytes apart, for the weights for a row pitch of 2, 6, 10 or 14 slots modulo 16.
+   const bool m16 = C16 == 4 && !pool;
+   a.KS = m16 ? a.K + 32 : (((a.K / 16) % 2 == 0) ? a.K + 16 : a.K);
    a.row_bytes = g.W * g.C;
    a.fill = 0x01010101u * (unsigned)(g.zpx & 0xff);
    a.xbytes = (unsigned)xbytes;
@@ -645,11 +637,28 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    int crossings = (rows2 - 1) / TH + 1;
    if (crossings > g.N - 1) crossings = g.N - 1;
    const int R = rows2 * rpp + a.gap * crossings + 2;
-   const size_t lds = (size_t)OCT * a.KS + (size_t)OCT * 8 + (size_t)R * a.RS;
+   // Plane pitch PL -> row pitch and LDS bytes. Row pitch: consecutive pixels of an output row are 16 bytes apart (with
+   // the pooling too: even and odd columns are stored apart); padded so that the first pixel of the next output row
+   // continues that sequence modulo the 256 bytes the LDS banks span.
+   auto plan = [&](int PL) {
+      a.PL = PL;
+      a.RS = C16 * PL;
+      // rpp ring rows lie between two output rows: rpp * RS = TW * 16 modulo 256, as nearly as a multiple of 16 allows
+      int best = 0, best_miss = 1 << 30;
+      for (int pad = 0; pad < 256; pad += 16) {
+         const int miss = ((rpp * (a.RS + pad) - TW * 16) % 256 + 256) % 256;
+         const int dist = miss < 256 - miss ? miss : 256 - miss;
+         if (dist < best_miss) { best_miss = dist; best = pad; }
+      }
+      a.RS += best;
+      return (size_t)OCT * a.KS + (size_t)OCT * 8 + (size_t)R * a.RS;
+   };
+   size_t lds = plan(m16 ? (WP * 16 + 255) / 256 * 256 : WP * 16);
+   if (lds > 160 * 1024 && a.PL != WP * 16) lds = plan(WP * 16);   // the longer planes do not fit: the rows as they are
    if (lds > 160 * 1024) return SOFIE_HIP_OK;
    a.R = R;
    a.dR = make_fastdiv(R);
-   a.dWP = make_fastdiv(WP);
+   a.dPL16 = make_fastdiv(a.PL / 16);
    if ((size_t)g.OC * a.K >= ((size_t)1 << 31)) return SOFIE_HIP_OK;
    const int nob = g.OC / OCT;
    int per = ctx->num_cus / nob;
@@ -668,7 +677,7 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    } while (0)
 #define SOFIE_QRING_BY_ROW(C16_, WN_, POOL_)                                                                   \
    do {                                                                                                        \
-      if (C16_ * WP <= 64) SOFIE_QRING_LAUNCH(C16_, WN_, true, POOL_);                                         \
+      if (C16_ * (a.PL / 16) <= 64) SOFIE_QRING_LAUNCH(C16_, WN_, true, POOL_);                                         \
       else SOFIE_QRING_LAUNCH(C16_, WN_, false, POOL_);                                                        \
    } while (0)
 #define SOFIE_QRING_BY_POOL(C16_, WN_)                                                                         \
