@@ -655,15 +655,17 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
    };
+   // the first two K-steps are requested together: the second one's way from memory runs under the first one's
    if (nk > 0) {
       request(0, 0);
-      wait_vmcnt<0>();
+      request(1, 1);
+      wait_vmcnt<LPW>();               // this wavefront's part of stage 0 has landed
    }
    barrier();
    if (group == 1) barrier();
    auto kstep = [&](int t, auto tag) {
       constexpr int S = decltype(tag)::value;
-      request(t + 1, 1 - S);
+      if (t > 0) request(t + 1, 1 - S);
       v4i fn[NSUB][NI], fm[NSUB][MJ];
 #pragma unroll
       for (int sub = 0; sub < NSUB; ++sub) {
