@@ -494,9 +494,11 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
       __builtin_amdgcn_s_barrier();
       asm volatile("" ::: "memory");
    };
+   // the first two K-steps are requested together: the second one's way from memory runs under the first one's
    if (nk > 0) {
       request(0, 0);
-      wait_vmcnt<0>();                  // this wavefront's part of stage 0 has landed
+      request(1, 1);
+      wait_vmcnt<LPW>();                // this wavefront's part of stage 0 has landed
    }
    barrier();
    if (group == 1) barrier();
@@ -506,7 +508,7 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
       // load phase: requests for K-step t+1 into the other stage (last read one phase ago), then
       // every operand fragment of stage S into registers. The requests go first: issued behind the fragment reads
       // they land later and the phase that waits for them grows (measured: 63.2 us instead of 59.9 us at 4096^3).
-      request(t + 1, 1 - S);
+      if (t > 0) request(t + 1, 1 - S);
       typename Mma::Frag fn[NSUB][TI], fm[NSUB][TJ];
 #pragma unroll
       for (int sub = 0; sub < NSUB; ++sub) {
