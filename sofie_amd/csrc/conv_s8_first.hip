@@ -40,23 +40,29 @@ struct FirstArgs {
    int dword_fill;        // W % 4 == 0 and x aligned: the images are filled a dword at a time
    int fast_div;          // x / xscale as a reciprocal multiply and two fused corrections (see quantize4)
    float xinv;            // 1 / xscale, correctly rounded
-   FastDiv drows, dper_image, dPW;
+   FastDiv dper_image, dPW, dHW4, dW4;
+   // how the coordinates of a work item move from one loop iteration to the next (the loops advance by a fixed
+   // number of items, so no iteration divides): a staging thread moves on by 256 groups of four pixels, a
+   // wavefront by 128 (pooled) output pixels
+   int st_im, st_row, st_col;   // 256 = st_im * (H*W/4) + st_row * (W/4) + st_col
+   int px_im, px_row, px_col;   // 128 = px_im * (PH*PW) + px_row * PW + px_col
 };
 
 
-__device__ __forceinline__ void windows(const unsigned char *row, int col, int &w0, int &w1)
+// p: the aligned dword of an LDS row that holds byte `col` of it, sh = col & 3
+__device__ __forceinline__ void windows(const unsigned char *p8, unsigned sh, int &w0, int &w1)
 {
-   // bytes col..col+3 and col+1..col+4 of an LDS row whose base is 4-byte aligned (col even)
-   const int *p = reinterpret_cast<const int *>(row + (col & ~3));
+   // bytes col..col+3 and col+1..col+4 (col even)
+   const int *p = reinterpret_cast<const int *>(p8);
    const unsigned lo = (unsigned)p[0], hi = (unsigned)p[1];
-   w0 = (int)__builtin_amdgcn_alignbyte(hi, lo, (unsigned)(col & 3));
-   w1 = (int)__builtin_amdgcn_alignbyte(hi, lo, (unsigned)(col & 3) + 1u);
+   w0 = (int)__builtin_amdgcn_alignbyte(hi, lo, sh);
+   w1 = (int)__builtin_amdgcn_alignbyte(hi, lo, sh + 1u);
 }
 
-__device__ __forceinline__ int window(const unsigned char *row, int col)
+__device__ __forceinline__ int window(const unsigned char *p8, unsigned sh)
 {
-   const int *p = reinterpret_cast<const int *>(row + (col & ~3));
-   return (int)__builtin_amdgcn_alignbyte((unsigned)p[1], (unsigned)p[0], (unsigned)(col & 3));
+   const int *p = reinterpret_cast<const int *>(p8);
+   return (int)__builtin_amdgcn_alignbyte((unsigned)p[1], (unsigned)p[0], sh);
 }
 
 __device__ __forceinline__ long pack64(int lo, int hi)
@@ -136,48 +142,55 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
    // padded images: cells outside the image hold the input zero-point; one spare row below each image is
    // read (with zero weights) by the upper half of the wavefront
    if (a.dword_fill) {
-      // LDS dword j of a row = image columns 4j-4 .. 4j-1. 16 threads per row, 16 rows per pass.
-      const int SD = a.stride >> 2, WD = a.W >> 2;
+      // Every cell first gets the zero-point (16 bytes per store), then the images' own cells are written over:
+      // a thread takes every 256th group of four pixels of the workgroup's images, which lie back to back in
+      // memory, so the loads are contiguous over the workgroup; image dword j of a row is LDS dword j + 1. The
+      // coordinates (image, row, dword) of a thread's next group follow from the present ones by additions.
       const unsigned zp4 = 0x01010101u * (unsigned)(a.zpx & 0xff);
       const float zpo = (float)(a.zpx + 128);
-      const int jj = tid & 15, rsub = tid >> 4;
-      const int total_rows = nimg * a.rows;
-      constexpr int UN = 6;   // rows per thread whose loads are in flight together
-      for (int j = jj; j < SD; j += 16) {
-         const bool col_inside = j >= 1 && j <= WD;
-         const int jsrc = col_inside ? j - 1 : 0;
-         for (int base = 0; base < total_rows; base += 16 * UN) {
-            unsigned q[UN];
-            v4f f[UN];
-            bool inside[UN];
-            unsigned *dst[UN];
+      const int bytes = nimg * a.img_bytes;                 // a multiple of 4
+      const v4i zfill = {(int)zp4, (int)zp4, (int)zp4, (int)zp4};
+      for (int i = tid; i < (bytes >> 4); i += 256) reinterpret_cast<v4i *>(s_img)[i] = zfill;
+      if (tid < ((bytes & 15) >> 2)) reinterpret_cast<unsigned *>(s_img + (bytes & ~15))[tid] = zp4;
+      __syncthreads();
+      const int HW4 = (a.H * a.W) >> 2, W4 = a.W >> 2;
+      const int total4 = nimg * HW4;
+      int im = fdiv(tid, a.dHW4);
+      int row, col;
+      {
+         const int r = tid - im * HW4;
+         row = fdiv(r, a.dW4);
+         col = r - row * W4;
+      }
+      const v4f *const srcf = reinterpret_cast<const v4f *>(a.xf + (size_t)n0 * a.H * a.W);
+      const unsigned *const srcq = reinterpret_cast<const unsigned *>(a.x + (size_t)n0 * a.H * a.W);
+      constexpr int UN = 8;   // groups per thread whose loads are in flight together
+      const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
+      for (int base = 0; base < total4; base += 256 * UN) {
+         unsigned q[UN];
+         v4f f[UN];
+         int dst[UN];
+         // a wavefront skips the groups that lie past the end for all of its lanes (the last round of a workgroup)
 #pragma unroll
-            for (int u = 0; u < UN; ++u) {
-               const int row_id = base + u * 16 + rsub;
-               const int rid = row_id < total_rows ? row_id : total_rows - 1;
-               const int im = fdiv(rid, a.drows);
-               const int lr = rid - im * a.rows;
-               const int ih = lr - 1;
-               inside[u] = col_inside && row_id < total_rows && ih >= 0 && ih < a.H;
-               const size_t src = ((size_t)(n0 + im) * a.H + (inside[u] ? ih : 0)) * a.W;
-               dst[u] = row_id < total_rows ? reinterpret_cast<unsigned *>(s_img + im * a.img_bytes + lr * a.stride) + j
-                                            : nullptr;
-               // the loads are unconditional (of the row's first cells when the cell is outside)
-               if (a.xf) f[u] = *reinterpret_cast<const v4f *>(a.xf + src + 4 * jsrc);
-               else q[u] = reinterpret_cast<const unsigned *>(a.x + src)[jsrc];
+         for (int u = 0; u < UN; ++u) {
+            const int idx = base + u * 256 + tid;
+            if (base + u * 256 + wave_first < total4) {
+               const int safe = idx < total4 ? idx : total4 - 1;   // the loads are unconditional within the wavefront
+               if (a.xf) f[u] = srcf[safe];
+               else q[u] = srcq[safe];
             }
-            if (a.xf) {
-               if (a.fast_div) {
+            dst[u] = idx < total4 ? (int)__umul24(im, a.img_bytes) + (int)__umul24(row + 1, a.stride) + 4 * col + 4 : -1;
+            col += a.st_col; row += a.st_row; im += a.st_im;
+            if (col >= W4) { col -= W4; row += 1; }
+            if (row >= a.H) { row -= a.H; im += 1; }
+         }
 #pragma unroll
-                  for (int u = 0; u < UN; ++u) q[u] = quantize4<true>(f[u], a.xscale, a.xinv, a.zpx, zpo);
-               } else {
-#pragma unroll
-                  for (int u = 0; u < UN; ++u) q[u] = quantize4<false>(f[u], a.xscale, a.xinv, a.zpx, zpo);
-               }
+         for (int u = 0; u < UN; ++u) {
+            if (base + u * 256 + wave_first < total4) {
+               if (a.xf) q[u] = a.fast_div ? quantize4<true>(f[u], a.xscale, a.xinv, a.zpx, zpo)
+                                           : quantize4<false>(f[u], a.xscale, a.xinv, a.zpx, zpo);
+               if (dst[u] >= 0) *reinterpret_cast<unsigned *>(s_img + dst[u]) = q[u];
             }
-#pragma unroll
-            for (int u = 0; u < UN; ++u)
-               if (dst[u]) *dst[u] = inside[u] ? q[u] : zp4;
          }
       }
    } else {
@@ -202,15 +215,17 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
    constexpr int NP = POOL ? 4 : 1;               // matrix instructions (window positions) per group
    // weight operand, bias and scales of a block of 32 channels: register e of a tile belongs to channel
    // (e/4)*8 + half*4 + e%4. With one block they are loaded once.
+   // The scales stay in LDS and are read where a group needs them (four 16-byte reads per group): held in
+   // registers next to the bias tile and two or three accumulator tiles they pushed the loop over the 128
+   // registers of four workgroups per CU, and a reload from scratch memory at the head of the loop waits for
+   // every earlier memory instruction of the wavefront, the stores of its previous group included.
    long wfrag = 0;
    v16i binit;
-   v4f sc[4];
    auto load_params = [&](int ob) {
       wfrag = s_wfrag[(ob * 32 + l32) * 2 + half];
 #pragma unroll
       for (int gq = 0; gq < 4; ++gq) {
          const v4i b = *reinterpret_cast<const v4i *>(s_bias + ob * 32 + gq * 8 + half * 4);
-         sc[gq] = *reinterpret_cast<const v4f *>(s_scale + ob * 32 + gq * 8 + half * 4);
 #pragma unroll
          for (int t = 0; t < 4; ++t) binit[gq * 4 + t] = b[t];
       }
@@ -222,26 +237,48 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
    auto process = [&](auto plain_c, auto negative_c) {
       constexpr bool PLAIN = decltype(plain_c)::value;
       constexpr bool NEGATIVE = decltype(negative_c)::value;
+      // The wavefront's pixels move on by 128 per iteration; image, row and column of a lane's pixel follow by
+      // additions, and the output offset is linear in the pixel's number (the images of a workgroup are stored
+      // back to back).
+      int q = wave * 32 + l32;
+      int im = fdiv(q, a.dper_image);
+      int py, px;
+      {
+         const int rem = q - im * per_image;
+         py = fdiv(rem, a.dPW);
+         px = rem - py * a.PW;
+      }
+      unsigned yoff = (unsigned)q * (unsigned)a.OC + (unsigned)half * 16u;
+      const unsigned ystep = 128u * (unsigned)a.OC;
+      int8_t *const ybase = a.y + (size_t)n0 * per_image * a.OC;
+      const int half_rows = (int)__umul24(2 * half, a.stride);
       for (int g = wave; g < groups; g += 4) {
-         const int q = g * 32 + l32;
-         const int qq = q < total ? q : total - 1;
-         const int im = fdiv(qq, a.dper_image), rem = qq - im * per_image;
-         const int py = fdiv(rem, a.dPW), px = rem - py * a.PW;
-         const int row0 = (POOL ? 2 * py : py) + 2 * half, col = (POOL ? 2 * px : px) + 2;
-         const unsigned char *base = s_img + im * a.img_bytes + row0 * a.stride;
+         const bool valid = q < total;
+         const int col = (POOL ? 2 * px : px) + 2;
+         const int cell = (int)__umul24(im, a.img_bytes) + (int)__umul24(POOL ? 2 * py : py, a.stride) + (col & ~3);
+         const unsigned char *base = s_img + half_rows + (valid ? cell : 0);   // a lane past the end reads the first pixel
+         const unsigned sh = (unsigned)(col & 3);
          long pix[NP];
          if constexpr (POOL) {
             int r[3][2];
 #pragma unroll
-            for (int k = 0; k < 3; ++k) windows(base + k * a.stride, col, r[k][0], r[k][1]);
+            for (int k = 0; k < 3; ++k) windows(base + k * a.stride, sh, r[k][0], r[k][1]);
 #pragma unroll
             for (int j = 0; j < 4; ++j) pix[j] = pack64(r[j >> 1][j & 1], r[(j >> 1) + 1][j & 1]);
          } else {
-            pix[0] = pack64(window(base, col), window(base + a.stride, col));
+            pix[0] = pack64(window(base, sh), window(base + a.stride, sh));
          }
-         int8_t *out = a.y + ((size_t)(n0 + im) * per_image + rem) * a.OC;
+         int8_t *out = ybase + yoff;
+         q += 128;
+         yoff += ystep;
+         px += a.px_col; py += a.px_row; im += a.px_im;
+         if (px >= a.PW) { px -= a.PW; py += 1; }
+         if (py >= a.PH) { py -= a.PH; im += 1; }
          for (int ob = 0; ob < a.ocb; ++ob) {
             if (!single) load_params(ob);
+            v4f sc[4];
+#pragma unroll
+            for (int gq = 0; gq < 4; ++gq) sc[gq] = *reinterpret_cast<const v4f *>(s_scale + ob * 32 + gq * 8 + half * 4);
             // one window position at a time keeps two accumulator tiles live (more wavefronts per SIMD); the
             // bias tile is the C operand of every matrix instruction (max(a + b) = max(a) + b), which costs nothing
             v16i acc = __builtin_amdgcn_mfma_i32_32x32x16_i8(wfrag, pix[0], binit, 0, 0, 0);
@@ -280,8 +317,7 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
             const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
             const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
             const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-            const int oc_first = ob * 32 + half * 16;
-            if (q < total && oc_first < a.OC) *reinterpret_cast<v4i *>(out + oc_first) = v;
+            if (valid && ob * 32 + half * 16 < a.OC) *reinterpret_cast<v4i *>(out + ob * 32) = v;
          }
       }
    };
@@ -323,7 +359,20 @@ int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
       a.fast_div = g.xf && as >= 0x1p-30f && as <= 0x1p30f;
       a.xinv = a.fast_div ? 1.0f / g.xscale : 0.0f;
    }
-   a.drows = make_fastdiv((unsigned)a.rows);
+   if (a.dword_fill) {
+      const int HW4 = g.H * g.W / 4, W4 = g.W / 4;
+      a.dHW4 = make_fastdiv((unsigned)HW4);
+      a.dW4 = make_fastdiv((unsigned)W4);
+      a.st_im = 256 / HW4;
+      a.st_row = (256 % HW4) / W4;
+      a.st_col = (256 % HW4) % W4;
+   }
+   {
+      const int per_image = g.PH * g.PW;
+      a.px_im = 128 / per_image;
+      a.px_row = (128 % per_image) / g.PW;
+      a.px_col = (128 % per_image) % g.PW;
+   }
    a.dper_image = make_fastdiv((unsigned)(g.PH * g.PW));
    a.dPW = make_fastdiv((unsigned)g.PW);
    // Images per workgroup: four workgroups share a CU, and the kernel is as slow as the busiest CU, so the
