@@ -847,6 +847,28 @@ template <class Mma, int OUT> struct IS_SPLITTABLE {
    static constexpr bool value = __is_same(typename Mma::Acc, v16i) && OUT == SOFIE_OUT_S32;
 };
 
+// Sum over the K slices of four consecutive int32 partial sums. The loads of four slices are issued together before
+// the first addition (one after the other, each waiting for the one before, they were the length of the pass).
+__device__ __forceinline__ v4i sum_slices(const int *__restrict__ p, size_t plane, int splits)
+{
+   v4i s = {0, 0, 0, 0};
+   int k = 0;
+   for (; k + 4 <= splits; k += 4) {
+      const v4i a = *reinterpret_cast<const v4i *>(p + (size_t)k * plane);
+      const v4i b = *reinterpret_cast<const v4i *>(p + (size_t)(k + 1) * plane);
+      const v4i c = *reinterpret_cast<const v4i *>(p + (size_t)(k + 2) * plane);
+      const v4i d = *reinterpret_cast<const v4i *>(p + (size_t)(k + 3) * plane);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] += (a[e] + b[e]) + (c[e] + d[e]);
+   }
+   for (; k < splits; ++k) {
+      const v4i v = *reinterpret_cast<const v4i *>(p + (size_t)k * plane);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] += v[e];
+   }
+   return s;
+}
+
 // Sum of the K slices' int32 partial tiles, then bias and the output conversion of the unsplit kernel.
 // One thread per four consecutive columns of one row; P is [splits][M][ldp], ldp a multiple of 4.
 template <int OUT>
@@ -857,11 +879,7 @@ __global__ void __launch_bounds__(256) k_splitk_finish(GemmArgs g, const int *__
    if (t >= (size_t)g.M * quads) return;
    const int m = (int)(t / quads), n = (int)(t % quads) * 4;
    const size_t plane = (size_t)g.M * ldp;
-   v4i s = *reinterpret_cast<const v4i *>(P + (size_t)m * ldp + n);
-   for (int k = 1; k < splits; ++k) {
-      const v4i v = *reinterpret_cast<const v4i *>(P + k * plane + (size_t)m * ldp + n);
-      s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
-   }
+   const v4i s = sum_slices(P + (size_t)m * ldp + n, plane, splits);
    constexpr int ESZ = OutSize<OUT>::value;
    unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + n) * ESZ;
 #pragma unroll
@@ -902,16 +920,21 @@ __global__ void __launch_bounds__(256) k_splitk_finish_pair(GemmArgs g1, const i
    if (t >= (size_t)g1.M * quads) return;
    const int m = (int)(t / quads), c = (int)(t % quads), n = c * 4;
    const size_t plane = (size_t)g1.M * ldp;
-   v4i s = *reinterpret_cast<const v4i *>(P + (size_t)m * ldp + n);
-   for (int k = 1; k < splits; ++k) {
-      const v4i v = *reinterpret_cast<const v4i *>(P + k * plane + (size_t)m * ldp + n);
-      s[0] += v[0]; s[1] += v[1]; s[2] += v[2]; s[3] += v[3];
+   // everything the thread reads is requested before the first value is used
+   float sc1[4];
+   int b1[4], w2[8];
+#pragma unroll
+   for (int e = 0; e < 4; ++e) {
+      sc1[e] = g1.scale[n + e];
+      b1[e] = g1.bias ? static_cast<const int *>(g1.bias)[n + e] : 0;
    }
+#pragma unroll
+   for (int j = 0; j < 8; ++j) w2[j] = j < g2.N ? *reinterpret_cast<const int *>(g2.B + (size_t)j * g2.ldb + n) : 0;
+   const v4i s = sum_slices(P + (size_t)m * ldp + n, plane, splits);
    unsigned packed = 0;
 #pragma unroll
    for (int e = 0; e < 4; ++e) {
-      const unsigned r = epilogue_value<true, SOFIE_OUT_S8>(g1, g1.scale[n + e], g1.bias ? static_cast<const int *>(g1.bias)[n + e] : 0,
-                                                            s[e], 0.0f);
+      const unsigned r = epilogue_value<true, SOFIE_OUT_S8>(g1, sc1[e], b1[e], s[e], 0.0f);
       packed |= ((unsigned)((int)fminf(__uint_as_float(r), 255.0f) - 128) & 0xffu) << (8 * e);
    }
    int dot[8];
@@ -919,7 +942,7 @@ __global__ void __launch_bounds__(256) k_splitk_finish_pair(GemmArgs g1, const i
    for (int j = 0; j < 8; ++j) {
       dot[j] = 0;
       if (j < g2.N) {      // uniform over the launch
-         const int w = *reinterpret_cast<const int *>(g2.B + (size_t)j * g2.ldb + n);
+         const int w = w2[j];
          dot[j] = __builtin_amdgcn_sdot4((int)packed, w, 0, false);
          if constexpr (QUADS == 64) {
             dot[j] = wave_sum_in_lane63(dot[j]);      // a row is a whole wavefront
