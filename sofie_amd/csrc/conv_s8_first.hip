@@ -317,7 +317,7 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
             const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
             const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
             const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-            if (valid && ob * 32 + half * 16 < a.OC) *reinterpret_cast<v4i *>(out + ob * 32) = v;
+            if (valid && ob * 32 + half * 16 < a.OC) store16_wt(out + ob * 32, v);   // the two halves of the wavefront write whole lines between them
          }
       }
    };

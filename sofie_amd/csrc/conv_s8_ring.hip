@@ -416,7 +416,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             const auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
             const auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
             const v4i v = {(int)t01[0], (int)t01[1], (int)t23[0], (int)t23[1]};
-            if (m < ep.M) SOFIE_RING_STORE(reinterpret_cast<v4i *>(row), v);
+            if (m < ep.M) store16_wt(row, v);
          }
          return;
       } else {

@@ -203,7 +203,7 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
             const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
             unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
             if (FULLN || (g.vec_store && nfirst + 16 / ESZ <= g.N)) {
-               *reinterpret_cast<v4i *>(out) = v;
+               store16_wt(out, v);
             } else {
                const unsigned char *src = stg + row * SROW + cc * 16;
                const int cnt = (g.N - nfirst) < (16 / ESZ) ? (g.N - nfirst) : (16 / ESZ);
@@ -382,7 +382,7 @@ __device__ __forceinline__ void tile_epilogue_wave16(const GemmArgs &g, v4i (&ac
             const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
             unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
             if (g.vec_store && nfirst + 16 / ESZ <= g.N) {
-               *reinterpret_cast<v4i *>(out) = v;
+               store16_wt(out, v);
             } else {
                const unsigned char *src = stg + row * SROW + cc * 16;
                const int cnt = (g.N - nfirst) < (16 / ESZ) ? (g.N - nfirst) : (16 / ESZ);
