@@ -382,9 +382,19 @@ def main():
     res = {}
     for name, (fn, meta) in workloads(ctx, torch, L, rng).items():
         torch.cuda.synchronize()
-        # half as many untimed launches first: a workload starts at whatever clock the one before it left
-        med, best, count = timer.median_ms(fn, meta.get("launches", 50), warmup=max(3, meta.get("launches", 50) // 2))
-        entry = {"workload": meta["workload"], "ms": med, "ms_best_block": best, "launches_timed": count}
+        # The same spin-up as in front of the headline steps: the host work between two workloads (operands drawn and
+        # uploaded) lets the device fall back to its idle clocks, and it needs tens of milliseconds of launches to
+        # leave them. The untimed phase is reported.
+        t_spin = time.perf_counter()
+        spins = 0
+        while (time.perf_counter() - t_spin) * 1e3 < args.spin_up_ms:
+            for _ in range(max(1, min(50, meta.get("launches", 50) // 4))):
+                fn()
+            torch.cuda.synchronize()
+            spins += 1
+        med, best, count = timer.median_ms(fn, meta.get("launches", 50), warmup=3)
+        entry = {"workload": meta["workload"], "ms": med, "ms_best_block": best, "launches_timed": count,
+                 "spin_up_ms": args.spin_up_ms}
         rate = meta["ops"] / med / 1e9
         entry[meta["rate_unit"]] = rate
         entry["frac_peak"] = rate / meta["peak"]
