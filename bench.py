@@ -547,7 +547,11 @@ def cnn_session_rate(iters=300, cpu_images=0):
             "host_ms_with_pcie": t["host_ms"], "inferences_per_s_with_pcie": 4096 / (t["host_ms"] * 1e-3),
             "host_ms_with_pcie_pinned_input": t.get("host_pinned_ms"),
             "inferences_per_s_with_pcie_pinned_input": 4096 / (t["host_pinned_ms"] * 1e-3) if t.get("host_pinned_ms") else None,
-            "pinned_input_same_logits": t.get("pinned_matches")}
+            "pinned_input_same_logits": t.get("pinned_matches"),
+            # two Sessions in flight on one device (two contexts and streams, a host thread each): wall time per batch
+            "two_sessions_ms_per_batch": t.get("two_sessions_ms_per_batch") or None,
+            "two_sessions_inferences_per_s": 4096 / (t["two_sessions_ms_per_batch"] * 1e-3) if t.get("two_sessions_ms_per_batch") else None,
+            "two_sessions_same_logits": t.get("two_sessions_match")}
 
 
 if __name__ == "__main__":

@@ -169,7 +169,7 @@ class ModelSpec:
         """g++ the generic runner against the generated header and libsofie_hip.so. With runtime_batch the runner's
         fourth argument is the batch it hands to infer(n, ...)."""
         exe = os.path.join(outdir, "run_" + self.name)
-        cmd = ["g++", "-std=c++17", "-O2", "-I" + os.path.join(ROOT, "include"), "-I" + outdir,
+        cmd = ["g++", "-std=c++17", "-O2", "-pthread", "-I" + os.path.join(ROOT, "include"), "-I" + outdir,
                "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % self.name, "-DSOFIE_MODEL_NS=SOFIE_%s" % self.name,
                "-DSOFIE_IN_T=%s" % _CTYPE[self.input[1]], "-DSOFIE_OUT_T=%s" % _CTYPE[self.out_type],
                "-DSOFIE_INPUT_MEMBER=fInput_%s" % self.input[0], "-DSOFIE_PINNED_INPUT=pinned_input_%s" % self.input[0], "-DSOFIE_NUM_INPUTS=%d" % len(self.inputs),

@@ -15,7 +15,9 @@
 #include <cstring>
 #include <fstream>
 #include <iostream>
+#include <memory>
 #include <string>
+#include <thread>
 #include <tuple>
 #include <utility>
 #include <vector>
@@ -178,9 +180,40 @@ int main(int argc, char **argv)
             for (int i = 0; i < iters; ++i) s.run_own_input();
             sofie_hip_timer_stop(s.fCtx, &gms);
          }
+         // Several Sessions in flight (a context and a stream each, a host thread each, as the slots of a SofieFunctor
+         // run; two unless SOFIE_RUN_SESSIONS says otherwise): the device overlaps the start of one Session's kernels with
+         // the others'. Wall time over all of them, per batch.
+         double pair_ms = 0;
+         bool pair_same = true;
+         int nsess = 2;
+         if (const char *e = std::getenv("SOFIE_RUN_SESSIONS")) nsess = std::atoi(e);
+         if (nsess >= 2 && !std::getenv("SOFIE_RUN_NO_PAIR")) {
+            s.use_graph(false);
+            std::vector<std::unique_ptr<SOFIE_MODEL_NS::Session>> others;
+            for (int k = 1; k < nsess; ++k) {
+               others.emplace_back(new SOFIE_MODEL_NS::Session(argv[1]));
+               std::vector<SOFIE_OUT_T> y2 = others.back()->infer(x.data());   // leaves the input in that Session's device buffer
+               pair_same = pair_same && y2.size() == y.size() && std::memcmp(y2.data(), y.data(), y.size() * sizeof(SOFIE_OUT_T)) == 0;
+            }
+            auto run = [iters](SOFIE_MODEL_NS::Session *sess) {
+               for (int i = 0; i < iters; ++i) sess->infer_device(sess->SOFIE_INPUT_MEMBER);
+               sess->sync();
+            };
+            auto all_at_once = [&]() {
+               std::vector<std::thread> workers;
+               for (auto &o : others) workers.emplace_back(run, o.get());
+               run(&s);
+               for (auto &w : workers) w.join();
+            };
+            all_at_once();     // untimed
+            t0 = std::chrono::steady_clock::now();
+            all_at_once();
+            pair_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / ((double)nsess * iters);
+         }
          std::printf("{\"device_ms\": %.6f, \"host_ms\": %.6f, \"host_pinned_ms\": %.6f, \"pinned_matches\": %s, \"graph_ms\": %.6f, "
-                     "\"graph_matches\": %s, \"iters\": %d}\n", ms / iters, host_ms / iters, pinned_ms / iters,
-                     pinned_same ? "true" : "false", gms / iters, same ? "true" : "false", iters);
+                     "\"graph_matches\": %s, \"sessions_in_flight\": %d, \"two_sessions_ms_per_batch\": %.6f, \"two_sessions_match\": %s, \"iters\": %d}\n",
+                     ms / iters, host_ms / iters, pinned_ms / iters, pinned_same ? "true" : "false", gms / iters,
+                     same ? "true" : "false", nsess, pair_ms, pair_same ? "true" : "false", iters);
       }
 #endif
 #endif
