@@ -29,9 +29,6 @@ using namespace sofie;
 
 namespace {
 
-#ifndef SOFIE_RING_STORE
-#define SOFIE_RING_STORE(p, v) (*(p) = (v))
-#endif
 template <bool B> struct BoolTag { static constexpr bool value = B; };
 
 struct QConvRingArgs {
@@ -49,16 +46,38 @@ struct QConvRingArgs {
    FastDiv dOW, dOH, dHP, dKS16, dR, dPL16;   // dPL16: by the 16-byte slots of a plane
 };
 
+// v[i] holds, per lane (half, l32), the 16 consecutive channels half * 16 .. + 15 of 32-channel tile i of pixel
+// m_first + l32 (what two v_permlane32_swap make of a 32 x 32 accumulator tile's packed bytes). One more swap between
+// the halves of the wavefront and one between neighbouring groups of 16 lanes sort the four 16-byte quarters of a
+// pixel's 64 channels onto the four lane groups, so that a store instruction writes the whole 64 bytes of 16 pixels
+// and can go through the L2 (store16_wt).
+__device__ __forceinline__ void store_pixels_64(const GemmArgs &g, const unsigned (&v)[2][4], int lane, int m_first, int n_wave)
+{
+   const int kg = lane >> 4, l16 = lane & 15;
+   // lane groups of 16 hold (pixels 0-15, 16-31 | quarter 0 resp. 2) in the lower half and (.. | quarter 1 resp. 3) in the
+   // upper half of v[0] resp. v[1]; after the two swaps a[] has quarter kg of pixel l16, b[] quarter kg of pixel 16 + l16
+   unsigned a[4], b[4];
+#pragma unroll
+   for (int e = 0; e < 4; ++e) {
+      const auto x = __builtin_amdgcn_permlane32_swap(v[0][e], v[1][e], false, false);
+      const auto y = __builtin_amdgcn_permlane16_swap(x[0], x[1], false, false);
+      a[e] = y[0];
+      b[e] = y[1];
+   }
+   const int ma = m_first + l16, mb = ma + 16;
+   int8_t *const col = static_cast<int8_t *>(g.Y) + n_wave + kg * 16;
+   if (ma < g.M) store16_wt(col + (size_t)ma * g.ldy, v4i{(int)a[0], (int)a[1], (int)a[2], (int)a[3]});
+   if (mb < g.M) store16_wt(col + (size_t)mb * g.ldy, v4i{(int)b[0], (int)b[1], (int)b[2], (int)b[3]});
+}
+
 // Requantisation and stores of a wavefront's 32 pooled pixels x 64 channels (two 32 x 32 accumulator tiles): as in
 // tile_epilogue_s8_direct a lane first gets the 16 consecutive channels half * 16 .. + 15 of each tile of its pixel
-// l32; one more swap between the halves of the wavefront and one between neighbouring groups of 16 lanes then sort
-// the four 16-byte quarters of a pixel onto the four lane groups, so that a store instruction writes the whole 64
-// bytes of 16 pixels and can go through the L2 (store16_wt) like the unpooled epilogue's.
+// l32, then store_pixels_64.
 template <bool PLAIN>
 __device__ __forceinline__ void pooled_epilogue_64(const GemmArgs &g, v16i (&acc)[2][1], const float *w_scale, const int *w_bias,
                                                    int lane, int m_wave, int n_wave)
 {
-   const int half = lane >> 5, nq = half * 4, kg = lane >> 4, l16 = lane & 15;
+   const int half = lane >> 5, nq = half * 4;
    const float zpo = (float)(g.zp + 128), lof = (float)(g.lo + 128);
    unsigned v[2][4];
 #pragma unroll
@@ -81,20 +100,7 @@ __device__ __forceinline__ void pooled_epilogue_64(const GemmArgs &g, v16i (&acc
       const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
       v[i][0] = s02[0]; v[i][1] = s02[1]; v[i][2] = s13[0]; v[i][3] = s13[1];
    }
-   // lane groups of 16 hold (pixels 0-15, 16-31 | quarter 0 resp. 2) in the lower half and (.. | quarter 1 resp. 3) in the
-   // upper half of v[0] resp. v[1]; after the two swaps a[] has quarter kg of pixel l16, b[] quarter kg of pixel 16 + l16
-   unsigned a[4], b[4];
-#pragma unroll
-   for (int e = 0; e < 4; ++e) {
-      const auto x = __builtin_amdgcn_permlane32_swap(v[0][e], v[1][e], false, false);
-      const auto y = __builtin_amdgcn_permlane16_swap(x[0], x[1], false, false);
-      a[e] = y[0];
-      b[e] = y[1];
-   }
-   const int ma = m_wave + l16, mb = ma + 16;
-   int8_t *const col = static_cast<int8_t *>(g.Y) + n_wave + kg * 16;
-   if (ma < g.M) store16_wt(col + (size_t)ma * g.ldy, v4i{(int)a[0], (int)a[1], (int)a[2], (int)a[3]});
-   if (mb < g.M) store16_wt(col + (size_t)mb * g.ldy, v4i{(int)b[0], (int)b[1], (int)b[2], (int)b[3]});
+   store_pixels_64(g, v, lane, m_wave, n_wave);
 }
 
 // C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels. The tile is (8/WN)*64 pixels x
@@ -430,10 +436,10 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       }
    };
    // Requantisation and stores of one tile: a lane packs its four 4-channel groups of an accumulator tile into four
-   // dwords, two swaps between the halves of the wavefront turn them into 16 consecutive channels, one 16-byte store.
-   // (A store instruction so touches 32 pixels with 32 bytes each. Stores of 64 contiguous bytes per pixel, 16
-   // pixels per instruction, take 5 % off the layer when the bytes are there for free, but moving them between lanes
-   // through a private block of LDS costs what they gain.)
+   // dwords, two swaps between the halves of the wavefront turn them into 16 consecutive channels, and two more
+   // (store_pixels_64) sort the two tiles' halves into 64 contiguous bytes per pixel, 16 pixels per store instruction.
+   // (Stored right after the first two swaps an instruction touched 32 pixels with 32 bytes each; moving the bytes
+   // between lanes through a private block of LDS instead of by swaps cost what the wider stores gained.)
    auto epilogue_as = [&](AccT (&acc)[NBT][MBT], int tt, auto plain_tag) {
       constexpr bool PLAIN = decltype(plain_tag)::value;
       const int m_wave = m_begin + tt * TM + wm * MBP * 32, n_wave = ob * OCT + wn * NB * 32;
@@ -470,8 +476,7 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
       } else {
 #pragma unroll
       for (int j = 0; j < MBP; ++j) {
-         const int m = m_wave + j * 32 + l32;
-         int8_t *const row = static_cast<int8_t *>(ep.Y) + (size_t)(m < ep.M ? m : 0) * ep.ldy + n_wave + half * 16;
+         unsigned v[2][4];
 #pragma unroll
          for (int i = 0; i < NB; ++i) {
             unsigned d[4];
@@ -490,9 +495,9 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
             }
             const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
             const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-            const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-            if (m < ep.M) SOFIE_RING_STORE(reinterpret_cast<v4i *>(row + i * 32), v);
+            v[i][0] = s02[0]; v[i][1] = s02[1]; v[i][2] = s13[0]; v[i][3] = s13[1];
          }
+         store_pixels_64(ep, v, lane, m_wave + j * 32, n_wave);
       }
       }
    };
