@@ -46,63 +46,6 @@ struct QConvRingArgs {
    FastDiv dOW, dOH, dHP, dKS16, dR, dPL16;   // dPL16: by the 16-byte slots of a plane
 };
 
-// v[i] holds, per lane (half, l32), the 16 consecutive channels half * 16 .. + 15 of 32-channel tile i of pixel
-// m_first + l32 (what two v_permlane32_swap make of a 32 x 32 accumulator tile's packed bytes). One more swap between
-// the halves of the wavefront and one between neighbouring groups of 16 lanes sort the four 16-byte quarters of a
-// pixel's 64 channels onto the four lane groups, so that a store instruction writes the whole 64 bytes of 16 pixels
-// and can go through the L2 (store16_wt).
-__device__ __forceinline__ void store_pixels_64(const GemmArgs &g, const unsigned (&v)[2][4], int lane, int m_first, int n_wave)
-{
-   const int kg = lane >> 4, l16 = lane & 15;
-   // lane groups of 16 hold (pixels 0-15, 16-31 | quarter 0 resp. 2) in the lower half and (.. | quarter 1 resp. 3) in the
-   // upper half of v[0] resp. v[1]; after the two swaps a[] has quarter kg of pixel l16, b[] quarter kg of pixel 16 + l16
-   unsigned a[4], b[4];
-#pragma unroll
-   for (int e = 0; e < 4; ++e) {
-      const auto x = __builtin_amdgcn_permlane32_swap(v[0][e], v[1][e], false, false);
-      const auto y = __builtin_amdgcn_permlane16_swap(x[0], x[1], false, false);
-      a[e] = y[0];
-      b[e] = y[1];
-   }
-   const int ma = m_first + l16, mb = ma + 16;
-   int8_t *const col = static_cast<int8_t *>(g.Y) + n_wave + kg * 16;
-   if (ma < g.M) store16_wt(col + (size_t)ma * g.ldy, v4i{(int)a[0], (int)a[1], (int)a[2], (int)a[3]});
-   if (mb < g.M) store16_wt(col + (size_t)mb * g.ldy, v4i{(int)b[0], (int)b[1], (int)b[2], (int)b[3]});
-}
-
-// Requantisation and stores of a wavefront's 32 pooled pixels x 64 channels (two 32 x 32 accumulator tiles): as in
-// tile_epilogue_s8_direct a lane first gets the 16 consecutive channels half * 16 .. + 15 of each tile of its pixel
-// l32, then store_pixels_64.
-template <bool PLAIN>
-__device__ __forceinline__ void pooled_epilogue_64(const GemmArgs &g, v16i (&acc)[2][1], const float *w_scale, const int *w_bias,
-                                                   int lane, int m_wave, int n_wave)
-{
-   const int half = lane >> 5, nq = half * 4;
-   const float zpo = (float)(g.zp + 128), lof = (float)(g.lo + 128);
-   unsigned v[2][4];
-#pragma unroll
-   for (int i = 0; i < 2; ++i) {
-      unsigned d[4];
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-         const v4f sc = *reinterpret_cast<const v4f *>(w_scale + i * 32 + q * 8 + nq);
-         const v4i bi = *reinterpret_cast<const v4i *>(w_bias + i * 32 + q * 8 + nq);
-         unsigned pk = 0;
-#pragma unroll
-         for (int t = 0; t < 4; ++t) {
-            float r = __fmul_rn(__int2float_rn(acc[i][0][q * 4 + t] + bi[t]), sc[t]);
-            if constexpr (!PLAIN) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);   // the byte conversion rounds half to even
-            pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);
-         }
-         d[q] = pk ^ 0x80808080u;
-      }
-      const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
-      const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-      v[i][0] = s02[0]; v[i][1] = s02[1]; v[i][2] = s13[0]; v[i][3] = s13[1];
-   }
-   store_pixels_64(g, v, lane, m_wave, n_wave);
-}
-
 // C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels. The tile is (8/WN)*64 pixels x
 // WN*64 channels. (Twelve wavefronts per workgroup, three per SIMD, and wavefront tiles of 96 pixels were measured
 // on the 56x56 layer: the same time within 1 %.)
@@ -528,8 +471,9 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
                   }
                }
          }
-         if (plain) pooled_epilogue_64<true>(ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
-         else pooled_epilogue_64<false>(ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+         // (two column tiles: they leave as 64 contiguous bytes per pooled pixel, written through the L2)
+         if (plain) tile_epilogue_s8_direct<NB, 1, true, true>(ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
+         else tile_epilogue_s8_direct<NB, 1, false, true>(ep, pooled, w_scale, w_bias, lane, m_wave, n_wave);
       } else {
          if (plain) epilogue_as(acc, tt, BoolTag<true>{});
          else epilogue_as(acc, tt, BoolTag<false>{});

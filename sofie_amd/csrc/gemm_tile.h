@@ -215,10 +215,35 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
    }
 }
 
+// v[i] holds, per lane (half, l32), the 16 consecutive columns half * 16 .. + 15 of 32-column tile i of row
+// m_first + l32 (what two v_permlane32_swap make of a 32 x 32 accumulator tile's packed bytes; for the convolutions a
+// row is a pixel and the columns are its channels). One more swap between the halves of the wavefront and one
+// between neighbouring groups of 16 lanes sort the four 16-byte quarters of a row's 64 columns onto the four lane
+// groups, so that a store instruction writes the whole 64 bytes of 16 rows and can go through the L2 (store16_wt).
+__device__ __forceinline__ void store_pixels_64(const GemmArgs &g, const unsigned (&v)[2][4], int lane, int m_first, int n_wave)
+{
+   const int kg = lane >> 4, l16 = lane & 15;
+   // lane groups of 16 hold (pixels 0-15, 16-31 | quarter 0 resp. 2) in the lower half and (.. | quarter 1 resp. 3) in the
+   // upper half of v[0] resp. v[1]; after the two swaps a[] has quarter kg of pixel l16, b[] quarter kg of pixel 16 + l16
+   unsigned a[4], b[4];
+#pragma unroll
+   for (int e = 0; e < 4; ++e) {
+      const auto x = __builtin_amdgcn_permlane32_swap(v[0][e], v[1][e], false, false);
+      const auto y = __builtin_amdgcn_permlane16_swap(x[0], x[1], false, false);
+      a[e] = y[0];
+      b[e] = y[1];
+   }
+   const int ma = m_first + l16, mb = ma + 16;
+   int8_t *const col = static_cast<int8_t *>(g.Y) + n_wave + kg * 16;
+   if (ma < g.M) store16_wt(col + (size_t)ma * g.ldy, v4i{(int)a[0], (int)a[1], (int)a[2], (int)a[3]});
+   if (mb < g.M) store16_wt(col + (size_t)mb * g.ldy, v4i{(int)b[0], (int)b[1], (int)b[2], (int)b[3]});
+}
+
 // int8 epilogue without LDS staging, for tiles whose columns are all inside the matrix: a lane packs its
 // four 4-column groups of a 32 x 32 accumulator tile into four dwords; two v_permlane32_swap between the
 // halves of the wavefront turn them into 16 consecutive columns per lane (lanes 0-31: columns 0-15 of
-// the tile, lanes 32-63: columns 16-31), which leave as one 16-byte store. Rows need ldy % 16 == 0 and
+// the tile, lanes 32-63: columns 16-31), which leave as one 16-byte store, or, with an even number of column tiles,
+// as 64 contiguous bytes per row of two neighbouring tiles (store_pixels_64). Rows need ldy % 16 == 0 and
 // a 16-byte aligned Y. reg_scale as in tile_epilogue_wave (may be null: scales are then read from s_scale).
 template <int TI, int TJ, bool PLAIN, bool ADD_BIAS>
 __device__ __forceinline__ void tile_epilogue_s8_direct(const GemmArgs &g, v16i (&acc)[TI][TJ], const float *s_scale,
@@ -232,6 +257,7 @@ __device__ __forceinline__ void tile_epilogue_s8_direct(const GemmArgs &g, v16i 
    for (int j = 0; j < TJ; ++j) {
       const int m = m_wave + j * 32 + l32;
       int8_t *row = static_cast<int8_t *>(g.Y) + (size_t)(m < g.M ? m : 0) * g.ldy + n_wave + half * 16;
+      unsigned pair[2][4];
 #pragma unroll
       for (int i = 0; i < TI; ++i) {
          unsigned d[4];
@@ -251,8 +277,14 @@ __device__ __forceinline__ void tile_epilogue_s8_direct(const GemmArgs &g, v16i 
          }
          const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
          const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
-         const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-         if (m < g.M) *reinterpret_cast<v4i *>(row + i * 32) = v;
+         if constexpr (TI % 2 == 0) {
+            // two neighbouring 32-column tiles leave together, as 64 contiguous bytes per row
+            pair[i & 1][0] = s02[0]; pair[i & 1][1] = s02[1]; pair[i & 1][2] = s13[0]; pair[i & 1][3] = s13[1];
+            if (i & 1) store_pixels_64(g, pair, lane, m_wave + j * 32, n_wave + (i - 1) * 32);
+         } else {
+            const v4i v = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+            if (m < g.M) *reinterpret_cast<v4i *>(row + i * 32) = v;
+         }
       }
    }
 }
