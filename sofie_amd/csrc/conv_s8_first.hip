@@ -120,6 +120,46 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
    const int n0 = blockIdx.x * a.images;
    const int nimg = (a.N - n0) < a.images ? (a.N - n0) : a.images;
 
+   // Staging of the images, in two halves: the loads of a thread's first groups of four pixels are requested here, before
+   // anything else, and used below, behind the set-up of the channels' parameters (whose own loads would otherwise
+   // be waited for first). A thread takes every 256th group of the workgroup's images, which lie back to back in
+   // memory, so the loads are contiguous over the workgroup; the coordinates (image, row, dword) of a thread's next
+   // group follow from the present ones by additions.
+   constexpr int UN = 8;   // groups per thread whose loads are in flight together
+   const int HW4 = (a.H * a.W) >> 2, W4 = a.W >> 2;
+   const int total4 = a.dword_fill ? nimg * HW4 : 0;
+   const v4f *const srcf = reinterpret_cast<const v4f *>(a.xf + (size_t)n0 * a.H * a.W);
+   const unsigned *const srcq = reinterpret_cast<const unsigned *>(a.x + (size_t)n0 * a.H * a.W);
+   const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
+   int st_im = 0, st_row = 0, st_col = 0;
+   auto request = [&](int base, unsigned (&q)[UN], v4f (&f)[UN], int (&dst)[UN]) {
+      // a wavefront skips the groups that lie past the end for all of its lanes (the last round of a workgroup)
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+         const int idx = base + u * 256 + tid;
+         if (base + u * 256 + wave_first < total4) {
+            const int safe = idx < total4 ? idx : total4 - 1;   // the loads are unconditional within the wavefront
+            if (a.xf) f[u] = srcf[safe];
+            else q[u] = srcq[safe];
+         }
+         // image dword j of a row is LDS dword j + 1
+         dst[u] = idx < total4 ? (int)__umul24(st_im, a.img_bytes) + (int)__umul24(st_row + 1, a.stride) + 4 * st_col + 4 : -1;
+         st_col += a.st_col; st_row += a.st_row; st_im += a.st_im;
+         if (st_col >= W4) { st_col -= W4; st_row += 1; }
+         if (st_row >= a.H) { st_row -= a.H; st_im += 1; }
+      }
+   };
+   unsigned q_first[UN];
+   v4f f_first[UN];
+   int dst_first[UN];
+   if (a.dword_fill) {
+      st_im = fdiv(tid, a.dHW4);
+      const int r = tid - st_im * HW4;
+      st_row = fdiv(r, a.dW4);
+      st_col = r - st_row * W4;
+      request(0, q_first, f_first, dst_first);
+   }
+
    if (tid == 0) s_flag[0] = 0;
    __syncthreads();
    for (int oc = tid; oc < OCP; oc += 256) {
@@ -142,10 +182,7 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
    // padded images: cells outside the image hold the input zero-point; one spare row below each image is
    // read (with zero weights) by the upper half of the wavefront
    if (a.dword_fill) {
-      // Every cell first gets the zero-point (16 bytes per store), then the images' own cells are written over:
-      // a thread takes every 256th group of four pixels of the workgroup's images, which lie back to back in
-      // memory, so the loads are contiguous over the workgroup; image dword j of a row is LDS dword j + 1. The
-      // coordinates (image, row, dword) of a thread's next group follow from the present ones by additions.
+      // Every cell first gets the zero-point (16 bytes per store), then the images' own cells are written over.
       const unsigned zp4 = 0x01010101u * (unsigned)(a.zpx & 0xff);
       const float zpo = (float)(a.zpx + 128);
       const int bytes = nimg * a.img_bytes;                 // a multiple of 4
@@ -153,37 +190,7 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
       for (int i = tid; i < (bytes >> 4); i += 256) reinterpret_cast<v4i *>(s_img)[i] = zfill;
       if (tid < ((bytes & 15) >> 2)) reinterpret_cast<unsigned *>(s_img + (bytes & ~15))[tid] = zp4;
       __syncthreads();
-      const int HW4 = (a.H * a.W) >> 2, W4 = a.W >> 2;
-      const int total4 = nimg * HW4;
-      int im = fdiv(tid, a.dHW4);
-      int row, col;
-      {
-         const int r = tid - im * HW4;
-         row = fdiv(r, a.dW4);
-         col = r - row * W4;
-      }
-      const v4f *const srcf = reinterpret_cast<const v4f *>(a.xf + (size_t)n0 * a.H * a.W);
-      const unsigned *const srcq = reinterpret_cast<const unsigned *>(a.x + (size_t)n0 * a.H * a.W);
-      constexpr int UN = 8;   // groups per thread whose loads are in flight together
-      const int wave_first = __builtin_amdgcn_readfirstlane(tid & ~63);
-      for (int base = 0; base < total4; base += 256 * UN) {
-         unsigned q[UN];
-         v4f f[UN];
-         int dst[UN];
-         // a wavefront skips the groups that lie past the end for all of its lanes (the last round of a workgroup)
-#pragma unroll
-         for (int u = 0; u < UN; ++u) {
-            const int idx = base + u * 256 + tid;
-            if (base + u * 256 + wave_first < total4) {
-               const int safe = idx < total4 ? idx : total4 - 1;   // the loads are unconditional within the wavefront
-               if (a.xf) f[u] = srcf[safe];
-               else q[u] = srcq[safe];
-            }
-            dst[u] = idx < total4 ? (int)__umul24(im, a.img_bytes) + (int)__umul24(row + 1, a.stride) + 4 * col + 4 : -1;
-            col += a.st_col; row += a.st_row; im += a.st_im;
-            if (col >= W4) { col -= W4; row += 1; }
-            if (row >= a.H) { row -= a.H; im += 1; }
-         }
+      auto deliver = [&](int base, unsigned (&q)[UN], v4f (&f)[UN], int (&dst)[UN]) {
 #pragma unroll
          for (int u = 0; u < UN; ++u) {
             if (base + u * 256 + wave_first < total4) {
@@ -192,6 +199,14 @@ __global__ void __launch_bounds__(256, 4) k_qconv_first(FirstArgs a)
                if (dst[u] >= 0) *reinterpret_cast<unsigned *>(s_img + dst[u]) = q[u];
             }
          }
+      };
+      deliver(0, q_first, f_first, dst_first);
+      for (int base = 256 * UN; base < total4; base += 256 * UN) {
+         unsigned q[UN];
+         v4f f[UN];
+         int dst[UN];
+         request(base, q, f, dst);
+         deliver(base, q, f, dst);
       }
    } else {
       for (int i = tid; i < nimg * a.img_bytes; i += 256) {
