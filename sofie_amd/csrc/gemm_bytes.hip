@@ -277,9 +277,10 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16 || NSETS > 2) ? 1 : 2) k_g
    Staged G[NSETS];
    if (nk > 0) {
       move_pieces(G[0], 0, 0, 0, 1, false, true);               // tile 0
-      move_pieces(G[0], 0, 0, 0, 1, true, false);               // -> stage 0
 #pragma unroll
       for (int s = 1; s < NSETS; ++s) move_pieces(G[s], 0, kclamp(s), 0, 1, false, true);   // tiles 1 .. NSETS-1
+      // (the later tiles are requested before tile 0 is waited for: their way from memory runs under its)
+      move_pieces(G[0], 0, 0, 0, 1, true, false);               // tile 0 -> stage 0
       move_pieces(G[0], 0, kclamp(NSETS), 0, 1, false, true);   // tile NSETS
       __syncthreads();
 #pragma unroll
