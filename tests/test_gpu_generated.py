@@ -154,6 +154,8 @@ def test_graph_replay_matches_eager(name, make_input, tmp_path):
     assert timing["graph_matches"] is True
     assert timing["graph_ms"] > 0
     assert timing["pinned_matches"] is True and timing["host_pinned_ms"] > 0   # infer() on the page-locked input buffer
+    # two Sessions of the model in flight at once (own contexts and streams, a host thread each) give the same bytes
+    assert timing["sessions_in_flight"] == 2 and timing["two_sessions_match"] is True and timing["two_sessions_ms_per_batch"] > 0
 
 
 def test_stacked_matmul_session(tmp_path):
