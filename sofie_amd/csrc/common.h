@@ -117,6 +117,17 @@ __device__ __forceinline__ void store16_wt(void *p, v4i v)
    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1\n\ts_nop 1" ::"v"(p), "v"(v) : "memory");
 }
 
+// Kernels that ask for more dynamic LDS than a launch may have by default need the limit raised with
+// hipFuncSetAttribute. That is a driver call, so it is made once per kernel and device when a context is created
+// (sofie_hip_create), never next to a launch and never while a stream is being captured: a launcher names its kernel
+// with SOFIE_LARGE_LDS(kern), which puts the kernel on the library's list when the library is loaded.
+void list_large_lds_kernel(const void *func);
+template <auto Kern> struct LargeLdsKernel {
+   static inline const bool listed = (list_large_lds_kernel(reinterpret_cast<const void *>(Kern)), true);
+};
+#define SOFIE_LARGE_LDS(kern) ((void)sofie::LargeLdsKernel<kern>::listed)
+constexpr int kMaxDynamicLds = 160 * 1024;   // LDS of a gfx950 compute unit
+
 inline int cdiv(int a, int b) { return (a + b - 1) / b; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

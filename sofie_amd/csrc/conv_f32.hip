@@ -554,9 +554,8 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          g.wvec = g.icg % g.ICB == 0 && g.KC == g.ICB * KHW && g.KC % 4 == 0 && (g.icg * KHW) % 4 == 0 &&
                   (reinterpret_cast<uintptr_t>(g.w) & 15u) == 0;
          if (!g.wvec) continue;
-         auto kern = k_conv2d_f32_pipe<TI, TJ>;
-         SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+         constexpr auto kern = k_conv2d_f32_pipe<TI, TJ>;
+         SOFIE_LARGE_LDS(kern);
          hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, g);
          *done = true;
          return check_launch(ctx, "k_conv2d_f32_pipe");
@@ -584,9 +583,10 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    // [OC, K] matrix 16-byte aligned
    g.wvec = !g.transposed && g.icg % g.ICB == 0 && g.KC == g.ICB * KHW && g.KC % 4 == 0 && (g.icg * KHW) % 4 == 0 &&
             (reinterpret_cast<uintptr_t>(g.w) & 15u) == 0;
-   auto kern = g.transposed ? k_conv2d_f32<TI, TJ, true> : k_conv2d_f32<TI, TJ, false>;
-   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+   constexpr auto kern_t = k_conv2d_f32<TI, TJ, true>, kern_p = k_conv2d_f32<TI, TJ, false>;
+   SOFIE_LARGE_LDS(kern_t);
+   SOFIE_LARGE_LDS(kern_p);
+   auto kern = g.transposed ? kern_t : kern_p;
    hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, g);
    *done = true;
    return check_launch(ctx, "k_conv2d_f32");
@@ -650,9 +650,8 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
          ConvArgs h = g;
          h.w = static_cast<const float *>(ws);
-         auto kern = k_conv2d_f32_pipe<TI, TJ, true>;
-         SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+         constexpr auto kern = k_conv2d_f32_pipe<TI, TJ, true>;
+         SOFIE_LARGE_LDS(kern);
          hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
          *done = true;
          return check_launch(ctx, "k_conv2d_f32_pipe (phases)");
@@ -690,9 +689,8 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    }
    g.wvec = 0;
    g.dK4 = make_fastdiv(1u);
-   auto kern = k_conv2d_f32<TI, TJ, true>;
-   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget));
+   constexpr auto kern = k_conv2d_f32<TI, TJ, true>;
+   SOFIE_LARGE_LDS(kern);
    hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, g);
    *done = true;
    return check_launch(ctx, "k_conv2d_f32 (phases)");

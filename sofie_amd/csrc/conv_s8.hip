@@ -561,9 +561,8 @@ int launch_mfma(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const dim3 grid((unsigned)(per * nob)), block(512);
 #define SOFIE_QCONV_LAUNCH_K(MB_, WN_, PF_, POOL_, KFIX_)                                                     \
    do {                                                                                                       \
-      auto kern = k_qconv_mfma<MB_, 2, WN_, PF_, OUT, POOL_, KFIX_>;                                          \
-      SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                           \
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));         \
+      constexpr auto kern = k_qconv_mfma<MB_, 2, WN_, PF_, OUT, POOL_, KFIX_>;                                \
+      SOFIE_LARGE_LDS(kern);                                                                                  \
       hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                             \
    } while (0)
 #define SOFIE_QCONV_LAUNCH(MB_, WN_, PF_, POOL_)                                                              \

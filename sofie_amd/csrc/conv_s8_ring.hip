@@ -46,6 +46,12 @@ struct QConvRingArgs {
    FastDiv dOW, dOH, dHP, dKS16, dR, dPL16;   // dPL16: by the 16-byte slots of a plane
 };
 
+// The block travels by value as the kernel's argument (and, when a call is recorded into a HIP graph, as a copy inside
+// the graph's kernel node): plain data, far below the 4 KB a launch may pass.
+static_assert(std::is_trivially_copyable<QConvRingArgs>::value && std::is_standard_layout<QConvRingArgs>::value &&
+                 sizeof(QConvRingArgs) <= 512,
+              "kernel argument block");
+
 // C16: 16-byte chunks per pixel (2 or 4); WN: wavefronts along the output channels. The tile is (8/WN)*64 pixels x
 // WN*64 channels. (Twelve wavefronts per workgroup, three per SIMD, and wavefront tiles of 96 pixels were measured
 // on the 56x56 layer: the same time within 1 %.)
@@ -667,9 +673,8 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    const dim3 grid((unsigned)(per * nob)), block(512);
 #define SOFIE_QRING_LAUNCH(C16_, WN_, ROW_, POOL_)                                                             \
    do {                                                                                                        \
-      auto kern = k_qconv_ring<C16_, WN_, ROW_, POOL_>;                                                        \
-      SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),                            \
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));          \
+      constexpr auto kern = k_qconv_ring<C16_, WN_, ROW_, POOL_>;                                              \
+      SOFIE_LARGE_LDS(kern);                                                                                   \
       hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);                                              \
    } while (0)
 #define SOFIE_QRING_BY_ROW(C16_, WN_, POOL_)                                                                   \

@@ -331,7 +331,15 @@ template <int S> struct StageTag { static constexpr int value = S; };
 // operand lie within 64 KB of its first byte, so a fragment read is one per-lane base register plus a constant in the
 // instruction's 16-bit offset field for either stage, and the K loop (unrolled over the two stages) holds no
 // address arithmetic in the vector unit.
-template <class Mma, int BK, int NST, int OUT, bool B_KN>
+// LOOP: the persistent form for launches with more tiles than compute units. A workgroup walks over the tiles
+// blockIdx.x, blockIdx.x + gridDim.x, ... (each XCD keeps its compact rectangle of tiles) and the K loop runs on
+// across the tile boundary: the last K-step of a tile requests the first K-step of the next one instead of a dummy, the
+// second follows as soon as its stage is free, and the epilogue in between works in LDS of its own (a 64-byte-wide
+// staging block per wavefront and the tile's scales and biases, behind the 128 KB of operand stages), so that the next
+// tile's operands land while the present tile is converted and stored, the stores of a tile drain under the next
+// tile's matrix instructions, and a compute unit never waits for a workgroup to end and the next one to start.
+// Needs an even number of K-steps (the stages keep their roles from tile to tile) and 1- or 2-byte outputs.
+template <class Mma, int BK, int NST, int OUT, bool B_KN, bool LOOP = false>
 __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
 {
    static_assert(!B_KN || BK == 128, "the [K,N] operand path is laid out for 128-byte stages");
@@ -354,9 +362,6 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    // blocks, LDS destinations, descriptor) in scalar registers and the branches on it scalar branches
    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
    const int wn = wave & 1, wm = wave >> 1;
-   int tm, tn;
-   tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
-   const int m0 = tm * BM, n0 = tn * BN;
 
    // --- loads: wavefronts 0-3 request the A tile, 4-7 the B^T tile -------------------------
    constexpr int LPW = (BM + BN) / RPB / 8;           // load blocks per wavefront and stage
@@ -364,12 +369,26 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    const bool rows_are_k = B_KN && !uses_a;            // B [K,N]: a load block is 4 rows of k x 256 bytes of n
    const int ld = uses_a ? g.lda : g.ldb;
    const int rows_total = uses_a ? g.M : g.N;
-   const int row0 = uses_a ? m0 : n0;
-   const int rows_left = (rows_total - row0) < 256 ? (rows_total - row0) : 256;
-   const unsigned char *tile_base = rows_are_k ? g.B + n0 : (uses_a ? g.A : g.B) + (size_t)row0 * ld;
-   // rows of k past K lie beyond the descriptor and read as zeros
-   const rsrc_t rs = make_rsrc(tile_base, rows_are_k ? (unsigned)((size_t)(g.K - 1) * ld + (g.N - n0))
-                                                     : (unsigned)((size_t)(rows_left - 1) * ld + g.K));
+   // What changes from tile to tile: the first row and column, and the descriptor of this wavefront's operand panel.
+   struct Tile {
+      rsrc_t rs;
+      int m0, n0;
+   };
+   auto describe = [&](int pid) {
+      Tile T;
+      int tm, tn;
+      tile_of_workgroup(pid, g.tiles_m, g.tiles_n, tm, tn);
+      T.m0 = tm * BM;
+      T.n0 = tn * BN;
+      const int row0 = uses_a ? T.m0 : T.n0;
+      const int rows_left = (rows_total - row0) < 256 ? (rows_total - row0) : 256;
+      const unsigned char *tile_base = rows_are_k ? g.B + T.n0 : (uses_a ? g.A : g.B) + (size_t)row0 * ld;
+      // rows of k past K lie beyond the descriptor and read as zeros
+      T.rs = make_rsrc(tile_base, rows_are_k ? (unsigned)((size_t)(g.K - 1) * ld + (g.N - T.n0))
+                                             : (unsigned)((size_t)(rows_left - 1) * ld + g.K));
+      return T;
+   };
+   Tile cur = describe(blockIdx.x);
    const int blk0 = (wave & 3) * LPW;                  // first load block of this wavefront inside its operand's stage
    const int lrow = lane / CPR;                        // row inside a block
    // K-chunk this lane fetches in load block i: slot ^ swizzle(row); for BK = 128 the row
@@ -392,7 +411,7 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
          voff[par] = (blk0 * 4 + (lane >> 4)) * ld + chunk[par] * 16;
       }
    }
-   const bool ktail = (g.K % BK) != 0;
+   const bool ktail = !LOOP && (g.K % BK) != 0;     // (the persistent form is launched on whole K-steps only)
    const int nk = (g.K + BK - 1) / BK;
    // per-lane offsets of the last, partial K-step: chunks at or past K point beyond the descriptor and read as zeros
    int voff_tail[2] = {voff[0], voff[1]};
@@ -406,7 +425,7 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    const int k_step = rows_are_k ? BK * ld : BK;
    // tile of K-step t -> stage S of its operand; steps past the end repeat the last tile into a stage nobody reads
    // any more, so the number of loads in flight never changes
-   auto request = [&](int t, int S) {
+   auto request = [&](const rsrc_t &rs, int t, int S) {
       const int tt = t < nk ? t : nk - 1;
       const bool tail = ktail && tt == nk - 1;
       const int v0 = tail ? voff_tail[0] : voff[0], v1 = tail ? voff_tail[1] : voff[1];
@@ -475,14 +494,53 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    };
 
    typename Mma::Acc acc[TI][TJ];
+   auto clear_acc = [&]() {
 #pragma unroll
-   for (int i = 0; i < TI; ++i)
+      for (int i = 0; i < TI; ++i)
 #pragma unroll
-      for (int j = 0; j < TJ; ++j)
+         for (int j = 0; j < TJ; ++j)
 #pragma unroll
-         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-   // scale and bias of the thread's column, in registers across the K loop
-   const ColumnParams col_params = load_column_params(g, tid, n0, BN);
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+   };
+   clear_acc();
+   // scale and bias of the thread's column, in registers across the K loop (the persistent form sends them to LDS
+   // per tile instead, see below)
+   ColumnParams col_params = {0.0f, 0};
+   if constexpr (!LOOP) col_params = load_column_params(g, tid, cur.n0, BN);
+
+   // --- LDS of the persistent form's epilogue, behind the operand stages: per wavefront a staging block of 32 rows x 64
+   // bytes and the scales and biases of its 128 columns. Private to the wavefront: no workgroup barrier guards it.
+   constexpr int ESZ = OutSize<OUT>::value;
+   constexpr int TP = ESZ <= 2 ? 64 / (32 * ESZ) : 1;        // 32-column tiles per epilogue pass: 64 bytes of a row
+   constexpr int WBX = EpilogueStaging<TP, OUT>::WAVE_BYTES;
+   constexpr int XREG = NST * (ABYTES + BBYTES);
+   unsigned char *const x_stg = smem + XREG + wave * WBX;
+   float *const x_scale = reinterpret_cast<float *>(smem + XREG + 8 * WBX + wave * 1024);
+   int *const x_bias = reinterpret_cast<int *>(x_scale + 128);
+   constexpr bool IS_INT = __is_same(typename Mma::Acc, v16i);
+   // stores of a full tile's epilogue and parameter loads of a tile per wavefront: the first wait of the next tile
+   // counts past them instead of waiting for them
+   constexpr int EPI_STORES = (TI / TP) * TJ * (32 * (TP * 32 * ESZ / 16) / 64);
+   const int param_loads = ((IS_INT && g.scale) ? 2 : 0) + (g.bias ? 2 : 0);
+   // The tile's per-column parameters travel straight into the wavefront's LDS block, one dword per lane and
+   // instruction; columns past N lie beyond the descriptor and read as zero.
+   // (the lane index is read off the hardware where the epilogue needs it: one register less across the K loop)
+   auto lane_now = [&]() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); };
+   auto request_params = [&](int n0) {
+      const int nw = n0 + wn * 128;
+      const int lane = lane_now();
+      const unsigned xs = lds0 + XREG + 8 * WBX + wave * 1024;
+      if (IS_INT && g.scale) {
+         const rsrc_t srs = make_rsrc(g.scale, (unsigned)g.N * 4u);
+         dma4(srs, xs, (nw + lane) * 4, 0);
+         dma4(srs, xs + 256, (nw + 64 + lane) * 4, 0);
+      }
+      if (g.bias) {
+         const rsrc_t brs = make_rsrc(g.bias, (unsigned)g.N * 4u);
+         dma4(brs, xs + 512, (nw + lane) * 4, 0);
+         dma4(brs, xs + 768, (nw + 64 + lane) * 4, 0);
+      }
+   };
 
    // --- ping-pong schedule -----------------------------------------------------------------
    // The two wavefronts of a SIMD run half a K-step apart: while one multiplies (MFMAs only,
@@ -497,53 +555,109 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
    };
    // the first two K-steps are requested together: the second one's way from memory runs under the first one's
    if (nk > 0) {
-      request(0, 0);
-      request(1, 1);
+      request(cur.rs, 0, 0);
+      request(cur.rs, 1, 1);
       wait_vmcnt<LPW>();                // this wavefront's part of stage 0 has landed
    }
+   if constexpr (LOOP) {
+      // without a bias (or scales) the block reads as zeros for the life of the kernel
+      x_scale[lane] = 0.0f; x_scale[64 + lane] = 0.0f;
+      x_bias[lane] = 0; x_bias[64 + lane] = 0;
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+   }
    barrier();
-   if (group == 1) barrier();
-   // one K-step on the tile in stage S (a compile-time constant: the loop below is unrolled over the two stages)
-   auto kstep = [&](int t, auto tag) {
-      constexpr int S = decltype(tag)::value;
-      // load phase: requests for K-step t+1 into the other stage (last read one phase ago), then
-      // every operand fragment of stage S into registers. The requests go first: issued behind the fragment reads
-      // they land later and the phase that waits for them grows (measured: 63.2 us instead of 59.9 us at 4096^3).
-      if (t > 0) request(t + 1, 1 - S);
-      typename Mma::Frag fn[NSUB][TI], fm[NSUB][TJ];
-#pragma unroll
-      for (int sub = 0; sub < NSUB; ++sub) {
-#pragma unroll
-         for (int i = 0; i < TI; ++i) {
-            if constexpr (B_KN) fn[sub][i] = load_frag_kn(i, S * BBYTES, sub);
-            else fn[sub][i] = load_frag(n_base, i * 32 * BK, S * BBYTES, sub);
+   const int tiles = g.tiles_m * g.tiles_n;
+   int pid = blockIdx.x;
+   bool stores_behind = false;          // the previous tile's epilogue left exactly EPI_STORES stores in the queue
+   for (;;) {
+      const int pid_next = pid + (int)gridDim.x;
+      const bool has_next = LOOP && pid_next < tiles;
+      Tile nxt = cur;
+      if (has_next) nxt = describe(pid_next);
+      if (group == 1) barrier();
+      if constexpr (LOOP) request_params(cur.n0);
+      // one K-step on the tile in stage S (a compile-time constant: the loop below is unrolled over the two stages)
+      auto kstep = [&](int t, auto tag) {
+         constexpr int S = decltype(tag)::value;
+         // load phase: requests for K-step t+1 into the other stage (last read one phase ago), then
+         // every operand fragment of stage S into registers. The requests go first: issued behind the fragment reads
+         // they land later and the phase that waits for them grows (measured: 63.2 us instead of 59.9 us at 4096^3).
+         if (t > 0) {
+            if (!LOOP || t + 1 < nk) request(cur.rs, t + 1, 1 - S);
+            else if (has_next) request(nxt.rs, 0, 1 - S);      // the next tile's first K-step
          }
+         typename Mma::Frag fn[NSUB][TI], fm[NSUB][TJ];
 #pragma unroll
-         for (int j = 0; j < TJ; ++j) fm[sub][j] = load_frag(m_base, j * 32 * BK, S * ABYTES, sub);
+         for (int sub = 0; sub < NSUB; ++sub) {
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+               if constexpr (B_KN) fn[sub][i] = load_frag_kn(i, S * BBYTES, sub);
+               else fn[sub][i] = load_frag(n_base, i * 32 * BK, S * BBYTES, sub);
+            }
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) fm[sub][j] = load_frag(m_base, j * 32 * BK, S * ABYTES, sub);
+         }
+         __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): fragments are in registers
+         // The other stage is first read by group 0 right after the barrier that ends its multiply
+         // phase, which is the barrier that ends group 1's load phase: each group waits for its
+         // own part of it just before that barrier. (Completion is reported in the order of issue: in the first
+         // K-step of a later tile the requests of its second K-step are followed by the previous tile's stores
+         // and this tile's parameter loads, which the wait counts past.)
+         auto wait_requests = [&]() {
+            if (LOOP && S == 0 && t == 0 && stores_behind) {
+               if (param_loads == 4) wait_vmcnt<EPI_STORES + 4>();
+               else if (param_loads == 2) wait_vmcnt<EPI_STORES + 2>();
+               else wait_vmcnt<EPI_STORES>();
+            } else {
+               wait_vmcnt<0>();
+            }
+         };
+         if (group == 1) wait_requests();
+         barrier();
+         // multiply phase
+#pragma unroll
+         for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+               for (int j = 0; j < TJ; ++j) acc[i][j] = Mma::mma(fn[sub][i], fm[sub][j], acc[i][j]);
+         if (group == 0) wait_requests();
+         if (group == 0 || t + 1 < nk) barrier();
+      };
+      for (int t = 0; t < nk; t += 2) {
+         kstep(t, StageTag<0>{});
+         if (t + 1 < nk) kstep(t + 1, StageTag<1>{});
       }
-      __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): fragments are in registers
-      // The other stage is first read by group 0 right after the barrier that ends its multiply
-      // phase, which is the barrier that ends group 1's load phase: each group waits for its
-      // own part of it just before that barrier.
-      if (group == 1) wait_vmcnt<0>();
-      barrier();
-      // multiply phase
+      if constexpr (!LOOP) break;
+      // Both groups are past the barrier behind the last load phase: stage 1 is free, the next tile's first K-step
+      // is complete in stage 0 (every wavefront waited for its part before that barrier).
+      if (has_next) request(nxt.rs, 1, 1);
+      {
+         const int m_wave = cur.m0 + wm * 64, n_wave = cur.n0 + wn * 128;
+         const bool full = g.vec_store && cur.m0 + BM <= g.M && cur.n0 + BN <= g.N;
+         const int mode = (OUT == SOFIE_OUT_S8 && g.zp == -128 && g.lo == -128) ? 1 : (OUT == SOFIE_OUT_S8 && g.lo == -128) ? 2 : 0;
+         // The epilogue's per-lane addresses are worked out afresh for every tile, from a lane index the compiler cannot
+         // trace to the one above: as loop invariants they would be kept in registers (that is, in scratch memory) across
+         // the K loop, which has none to spare.
+         const int lane_e = lane_now();
 #pragma unroll
-      for (int sub = 0; sub < NSUB; ++sub)
-#pragma unroll
-         for (int i = 0; i < TI; ++i)
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) acc[i][j] = Mma::mma(fn[sub][i], fm[sub][j], acc[i][j]);
-      if (group == 0) wait_vmcnt<0>();
-      if (group == 0 || t + 1 < nk) barrier();
-   };
-   for (int t = 0; t < nk; t += 2) {
-      kstep(t, StageTag<0>{});
-      if (t + 1 < nk) kstep(t + 1, StageTag<1>{});
+         for (int i0 = 0; i0 < TI; i0 += TP) {
+            typename Mma::Acc(&part)[TP][TJ] = reinterpret_cast<typename Mma::Acc(&)[TP][TJ]>(acc[i0]);
+            // written through on the workgroup's last tile only: nothing follows that their way out could run under
+            if (mode == 1) tile_epilogue_wave<Mma, TP, TJ, OUT, 1>(g, part, x_stg, x_scale + i0 * 32, x_bias + i0 * 32, lane_e, m_wave, n_wave + i0 * 32, nullptr, !has_next);
+            else if (mode == 2) tile_epilogue_wave<Mma, TP, TJ, OUT, 2>(g, part, x_stg, x_scale + i0 * 32, x_bias + i0 * 32, lane_e, m_wave, n_wave + i0 * 32, nullptr, !has_next);
+            else tile_epilogue_wave<Mma, TP, TJ, OUT, 0>(g, part, x_stg, x_scale + i0 * 32, x_bias + i0 * 32, lane_e, m_wave, n_wave + i0 * 32, nullptr, !has_next);
+         }
+         stores_behind = full;
+      }
+      if (!has_next) return;
+      clear_acc();
+      cur = nxt;
+      pid = pid_next;
    }
    wait_vmcnt<0>();                         // the trailing dummy requests still target LDS
    __syncthreads();
-   tile_epilogue<Mma, TI, TJ, OUT, 8>(g, acc, smem, tid, m0 + wm * 64, n0, wn, BN, &col_params);
+   tile_epilogue<Mma, TI, TJ, OUT, 8>(g, acc, smem, tid, cur.m0 + wm * 64, cur.n0, wn, BN, &col_params);
 }
 
 // k_gemm_dma16: the int8 kernel above (B^T [N,K] or B [K,N]) on v_mfma_i32_16x16x64_i8 instead of v_mfma_i32_32x32x32_i8.
@@ -980,9 +1094,8 @@ int launch_tiled_impl(sofie_hip_ctx *ctx, GemmArgs &g)
    static_assert(lds <= 160 * 1024, "tile does not fit the 160 KB LDS");
    g.tiles_m = cdiv(g.M, BM);
    g.tiles_n = cdiv(g.N, BN);
-   auto kern = k_gemm_bytes<Mma, BK, NSETS, TI, TJ, OUT, B_KN, FULL>;
-   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+   constexpr auto kern = k_gemm_bytes<Mma, BK, NSETS, TI, TJ, OUT, B_KN, FULL>;
+   SOFIE_LARGE_LDS(kern);
    const int splits = (IS_SPLITTABLE<Mma, OUT>::value && g.splits > 1) ? g.splits : 1;
    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n * splits), dim3(256), lds, ctx->stream, g);
    return check_launch(ctx, "k_gemm_bytes");
@@ -1007,15 +1120,26 @@ int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
    g.tiles_m = cdiv(g.M, 256);
    g.tiles_n = cdiv(g.N, 256);
    if constexpr (__is_same(Mma, MmaI8) && BK == 128 && SOFIE_GEMM16) {
-      auto kern16 = k_gemm_dma16<OUT, B_KN>;
-      SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern16),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      constexpr auto kern16 = k_gemm_dma16<OUT, B_KN>;
+      SOFIE_LARGE_LDS(kern16);
       hipLaunchKernelGGL(kern16, dim3(g.tiles_m * g.tiles_n), dim3(512), lds, ctx->stream, g);
       return check_launch(ctx, "k_gemm_dma16");
    }
-   auto kern = k_gemm_dma<Mma, BK, NST, OUT, B_KN>;
-   SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+   // More tiles than compute units: one workgroup per compute unit walks over its tiles (see k_gemm_dma, LOOP).
+   if constexpr (OutSize<OUT>::value <= 2) {
+      const int nk = cdiv(g.K, BK);
+      const int tiles = g.tiles_m * g.tiles_n;
+      if (tiles > ctx->num_cus && g.K % (2 * BK) == 0) {
+         constexpr size_t loop_lds = stage_bytes + (size_t)8 * EpilogueStaging<64 / (32 * OutSize<OUT>::value), OUT>::WAVE_BYTES + 8 * 1024;
+         static_assert(loop_lds <= 160 * 1024, "stages and the epilogue's own blocks do not fit the 160 KB LDS");
+         constexpr auto loop = k_gemm_dma<Mma, BK, NST, OUT, B_KN, true>;
+         SOFIE_LARGE_LDS(loop);
+         hipLaunchKernelGGL(loop, dim3(ctx->num_cus), dim3(512), loop_lds, ctx->stream, g);
+         return check_launch(ctx, "k_gemm_dma (persistent)");
+      }
+   }
+   constexpr auto kern = k_gemm_dma<Mma, BK, NST, OUT, B_KN>;
+   SOFIE_LARGE_LDS(kern);
    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(512), lds, ctx->stream, g);
    return check_launch(ctx, "k_gemm_dma");
 }

@@ -362,12 +362,12 @@ extern "C" int sofie_hip_mlp_f32(sofie_hip_ctx *ctx, int n_layers, const int *di
    const int R = M <= 2 * cus ? 1 : M <= 8 * cus ? 4 : 8;
    const size_t lds = ((size_t)2 * R * a.maxd + (size_t)256 * R) * sizeof(float);
    const dim3 grid((unsigned)cdiv(M, R)), block(256);
-   auto launch = [&](auto kern) -> int {
-      SOFIE_HIP_CALL(ctx, hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, a);
-      return SOFIE_HIP_OK;
-   };
-   if (int rc = R == 1 ? launch(k_mlp_f32<1>) : R == 4 ? launch(k_mlp_f32<4>) : launch(k_mlp_f32<8>)) return rc;
+   // (up to 72 KB of LDS at the widest layers: above the default limit of a launch)
+   SOFIE_LARGE_LDS(k_mlp_f32<1>);
+   SOFIE_LARGE_LDS(k_mlp_f32<4>);
+   SOFIE_LARGE_LDS(k_mlp_f32<8>);
+   if (R == 1) hipLaunchKernelGGL(k_mlp_f32<1>, grid, block, lds, ctx->stream, a);
+   else if (R == 4) hipLaunchKernelGGL(k_mlp_f32<4>, grid, block, lds, ctx->stream, a);
+   else hipLaunchKernelGGL(k_mlp_f32<8>, grid, block, lds, ctx->stream, a);
    return check_launch(ctx, "k_mlp_f32");
 }

@@ -115,7 +115,7 @@ template <class Mma, int TI, int TJ, int OUT, int PLAIN, bool ADD_BIAS = true, b
 __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename Mma::Acc (&acc)[TI][TJ],
                                                    unsigned char *stg, const float *s_scale, const int *s_bias,
                                                    int lane, int m_wave, int n_wave,
-                                                   const v4f (*reg_scale)[TI * 4] = nullptr)
+                                                   const v4f (*reg_scale)[TI * 4] = nullptr, bool write_through = true)
 {
    constexpr int ESZ = OutSize<OUT>::value;
    constexpr bool IS_INT = __is_same(typename Mma::Acc, v16i);
@@ -203,7 +203,8 @@ __device__ __forceinline__ void tile_epilogue_wave(const GemmArgs &g, typename M
             const v4i v = *reinterpret_cast<const v4i *>(stg + row * SROW + cc * 16);
             unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + nfirst) * ESZ;
             if (FULLN || (g.vec_store && nfirst + 16 / ESZ <= g.N)) {
-               store16_wt(out, v);
+               if (write_through) store16_wt(out, v);
+               else *reinterpret_cast<v4i *>(out) = v;
             } else {
                const unsigned char *src = stg + row * SROW + cc * 16;
                const int cnt = (g.N - nfirst) < (16 / ESZ) ? (g.N - nfirst) : (16 / ESZ);
@@ -444,6 +445,16 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void *base, unsigned bytes)
 __device__ __forceinline__ void dma16(rsrc_t rs, unsigned lds_base, int voff, int soff)
 {
    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                :
+                : "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "v"(voff), "s"(rs),
+                  "s"(__builtin_amdgcn_readfirstlane(soff))
+                : "memory");
+}
+
+// 4 bytes per lane from global to LDS address lds_base + lane*4 (per-column parameters of a tile).
+__device__ __forceinline__ void dma4(rsrc_t rs, unsigned lds_base, int voff, int soff)
+{
+   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                 :
                 : "s"(__builtin_amdgcn_readfirstlane((int)lds_base)), "v"(voff), "s"(rs),
                   "s"(__builtin_amdgcn_readfirstlane(soff))

@@ -2,6 +2,7 @@
 #include <stdarg.h>
 
 #include <mutex>
+#include <vector>
 
 #include "common.h"
 
@@ -31,9 +32,47 @@ hipError_t scratch_address(int device, void **addr)
    *addr = g_scratch_addr[device];
    return hipSuccess;
 }
+
+// Kernels listed by SOFIE_LARGE_LDS (static initialisers of the kernel translation units, so the list lives in a
+// function and exists whenever one of them runs) and the devices on which their limit has been raised.
+std::vector<const void *> &large_lds_kernels()
+{
+   static std::vector<const void *> v;
+   return v;
+}
+std::mutex g_lds_mutex;
+bool g_lds_done[kMaxDevices] = {};
+
+// With `device` current: raise the dynamic-LDS limit of every listed kernel to what the LDS holds beside the kernel's
+// own static arrays, once per device. A kernel whose limit cannot be raised is reported once on stderr and left as it
+// is: its launches with more than the default then fail with the runtime's message.
+void raise_lds_limits(int device)
+{
+   if (device < 0 || device >= kMaxDevices) return;
+   std::lock_guard<std::mutex> lock(g_lds_mutex);
+   if (g_lds_done[device]) return;
+   g_lds_done[device] = true;
+   for (const void *f : large_lds_kernels()) {
+      hipFuncAttributes attr{};
+      int limit = sofie::kMaxDynamicLds;
+      if (hipFuncGetAttributes(&attr, f) == hipSuccess) limit -= (int)attr.sharedSizeBytes;
+      else (void)hipGetLastError();
+      const hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, limit);
+      if (e != hipSuccess) {
+         (void)hipGetLastError();
+         fprintf(stderr, "libsofie_hip: dynamic LDS limit of %d bytes refused for a kernel: %s\n", limit, hipGetErrorString(e));
+      }
+   }
+}
 }  // namespace
 
 namespace sofie {
+
+void list_large_lds_kernel(const void *func)
+{
+   std::lock_guard<std::mutex> lock(g_lds_mutex);
+   large_lds_kernels().push_back(func);
+}
 
 int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...)
 {
@@ -112,6 +151,7 @@ int sofie_hip_create(sofie_hip_ctx **out, int device, void *stream)
       if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && cus > 0)
          ctx->num_cus = cus;
    }
+   raise_lds_limits(device);
    if (hipError_t e = scratch_address(device, &ctx->static_scratch); e != hipSuccess) {
       // only the no-allocation entry point needs it: that call then fails with this message
       (void)hipGetLastError();

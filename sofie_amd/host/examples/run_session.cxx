@@ -195,20 +195,28 @@ int main(int argc, char **argv)
                std::vector<SOFIE_OUT_T> y2 = others.back()->infer(x.data());   // leaves the input in that Session's device buffer
                pair_same = pair_same && y2.size() == y.size() && std::memcmp(y2.data(), y.data(), y.size() * sizeof(SOFIE_OUT_T)) == 0;
             }
-            auto run = [iters](SOFIE_MODEL_NS::Session *sess) {
-               for (int i = 0; i < iters; ++i) sess->infer_device(sess->SOFIE_INPUT_MEMBER);
+            // every Session's last result is read back after the runs in flight and compared with the serial one
+            std::vector<const SOFIE_OUT_T *> results(nsess, nullptr);
+            auto run = [iters, &results](SOFIE_MODEL_NS::Session *sess, int slot) {
+               for (int i = 0; i < iters; ++i) results[slot] = sess->infer_device(sess->SOFIE_INPUT_MEMBER);
                sess->sync();
             };
             auto all_at_once = [&]() {
                std::vector<std::thread> workers;
-               for (auto &o : others) workers.emplace_back(run, o.get());
-               run(&s);
+               for (size_t k = 0; k < others.size(); ++k) workers.emplace_back(run, others[k].get(), (int)k + 1);
+               run(&s, 0);
                for (auto &w : workers) w.join();
             };
             all_at_once();     // untimed
             t0 = std::chrono::steady_clock::now();
             all_at_once();
             pair_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count() / ((double)nsess * iters);
+            for (int k = 0; k < nsess; ++k) {
+               SOFIE_MODEL_NS::Session *sess = k == 0 ? &s : others[k - 1].get();
+               std::vector<SOFIE_OUT_T> yk(y.size());
+               const bool read = results[k] && sofie_hip_download(sess->fCtx, yk.data(), results[k], yk.size() * sizeof(SOFIE_OUT_T)) == 0;
+               pair_same = pair_same && read && std::memcmp(yk.data(), y.data(), y.size() * sizeof(SOFIE_OUT_T)) == 0;
+            }
          }
          std::printf("{\"device_ms\": %.6f, \"host_ms\": %.6f, \"host_pinned_ms\": %.6f, \"pinned_matches\": %s, \"graph_ms\": %.6f, "
                      "\"graph_matches\": %s, \"sessions_in_flight\": %d, \"two_sessions_ms_per_batch\": %.6f, \"two_sessions_match\": %s, \"iters\": %d}\n",

@@ -910,6 +910,60 @@ def test_gemm_fp8_full_size(ops):
     assert np.array_equal(yb[rows[0]], oracle.bf16_encode(yf[rows[0]]))
 
 
+@pytest.mark.parametrize("transB", [True, False])
+def test_gemm_fp8_more_tiles_than_compute_units(ops, transB):
+    """306 tiles of 256 x 256 on 256 compute units, ragged in M and N: the launch in which a workgroup walks over
+    several tiles and requests the next tile's operands before it converts the present one. Small integers and
+    power-of-two scales make every sum exact, so the bf16 output must be the rounding of the exact result."""
+    from sofie_amd import lib as L
+    r = rng(81 + int(transB))
+    M, N, K = 4100, 4356, 512
+    a = r.integers(-4, 5, (M, K)).astype(np.float32)
+    b = r.integers(-4, 5, (K, N)).astype(np.float32)
+    codes = oracle.e4m3_encode(np.arange(-4, 5, dtype=np.float32))
+    A, B = codes[a.astype(np.int64) + 4], codes[b.astype(np.int64) + 4]
+    if transB:
+        B = np.ascontiguousarray(B.T)
+    bias = r.integers(-8, 9, N).astype(np.float32)
+    exact = (a @ b) * np.float32(0.125) + bias
+    yb = ops.gemm_fp8(A, B, 0.5, 0.25, bias, transB)
+    assert np.array_equal(yb, torch.from_numpy(exact).bfloat16().view(torch.int16).numpy().view(np.uint16))
+    yn = ops.gemm_fp8(A, B, 0.5, 0.25, None, transB)      # no bias: the tile's parameter block stays zero
+    assert np.array_equal(yn, torch.from_numpy((a @ b) * np.float32(0.125)).bfloat16().view(torch.int16).numpy().view(np.uint16))
+    yf = ops.gemm_fp8(A, B, 0.5, 0.25, bias, transB, out=L.OUT_F32)
+    assert np.array_equal(yf, exact)
+
+
+@pytest.mark.parametrize("transB", [False, True])
+def test_gemm_fp8_benchmark_operands_at_full_depth(ops, transB):
+    """The benchmark's own FP8 GEMM (8192 x 8192 x 4096, N(0,1) operands cast to e4m3 at amax/448, bias, bf16 out):
+    a band of 512 rows against the fp64-accumulated product of the same e4m3 operands, with the tolerance of
+    test_gemm_fp8 (2^-8 |ref| + 2^-15 sa sb sum|a_k b_k|) at the full K = 4096; the error is printed in bf16 ulps."""
+    r = rng(83)
+    M = N = 8192
+    K = 4096
+    A, B, sa, sb = fp8_operands(r, M, N, K, transB)
+    bias = r.standard_normal(N).astype(np.float32)
+    yb = ops.gemm_fp8(A, B, sa, sb, bias, transB)
+    rows = np.sort(r.choice(M, 512, replace=False))
+    da = oracle.e4m3_decode(A[rows]).astype(np.float64)
+    db = oracle.e4m3_decode(B).astype(np.float64)
+    db = db.T if transB else db
+    truth = (da @ db) * (float(sa) * float(sb)) + bias.astype(np.float64)
+    mag = (np.abs(da) @ np.abs(db)) * (float(sa) * float(sb))
+    got = oracle.bf16_decode(yb[rows]).astype(np.float64)
+    err = np.abs(got - truth)
+    tol = 2.0 ** -8 * np.abs(truth) + 2.0 ** -15 * mag + 1e-30
+    assert np.all(err <= tol)
+    # in bf16 ulps of the true value, over the outputs that are not results of cancellation (|truth| at least a tenth
+    # of sum|a_k b_k|'s typical size would be arbitrary: the output's own root mean square is the yardstick)
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(truth), 1e-30))) - 7)
+    big = np.abs(truth) >= np.sqrt(np.mean(truth ** 2))
+    print("fp8 gemm K=4096 %s: bf16 ulp of the error max %.3f mean %.3f over the %d outputs of at least rms size; "
+          "largest error / tolerance %.3f" % ("[N,K]" if transB else "[K,N]", (err / ulp)[big].max(), (err / ulp)[big].mean(),
+                                              int(big.sum()), (err / tol).max()))
+
+
 # --------------------------------------------------------------------------- graph recording rules
 def test_capture_rules_are_enforced():
     """Between capture_begin and capture_end the calls that would wait on, or record a memset node into, the
