@@ -100,9 +100,10 @@ class LaunchTimer:
         return statistics.median(t), min(t), n_blocks * per_block
 
 
-def sclk_under_load(torch, launch, seconds=1.5):
-    """Shader clock (MHz) that rocm-smi reports while `launch` runs back to back: the median of the samples taken
-    after the first (None if the tool is not there). The matrix peaks of the data sheet assume 2400 MHz."""
+def sclk_under_load(torch, launch, stream, seconds=1.5):
+    """Shader clock (MHz) that rocm-smi reports while `launch` runs back to back, and the duration of a launch
+    measured over the same launches (HIP events on the launch stream around each block of 100): the medians of both
+    (None for the clock if the tool is not there). The matrix peaks of the data sheet assume 2400 MHz."""
     import re
     import threading
     samples, stop = [], [False]
@@ -120,13 +121,19 @@ def sclk_under_load(torch, launch, seconds=1.5):
     th = threading.Thread(target=sampler)
     th.start()
     t0 = time.perf_counter()
+    blocks = []
     while time.perf_counter() - t0 < seconds:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
         for _ in range(100):
             launch()
+        e1.record(stream)
         torch.cuda.synchronize()
+        blocks.append(e0.elapsed_time(e1) / 100)
     stop[0] = True
     th.join()
-    return statistics.median(samples[1:]) if len(samples) > 1 else None
+    ms = statistics.median(blocks[1:]) if len(blocks) > 1 else None
+    return (statistics.median(samples[1:]) if len(samples) > 1 else None), ms
 
 
 def blas_candidates():
@@ -281,9 +288,11 @@ def main():
     # the device out of its idle clocks first (reported as spin_up_ms), then the warm-up steps, then EXACTLY `steps`
     # timed steps bracketed by device synchronisation
     t_spin = time.perf_counter()
+    spin_launches = 0
     while (time.perf_counter() - t_spin) * 1e3 < args.spin_up_ms:
         for _ in range(50):
             step()
+        spin_launches += 50
         torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
@@ -305,7 +314,7 @@ def main():
     out = {
         "metric": "int8/FP8 GEMM TOPS & % MFMA peak; model inferences/sec at batch 4096",
         "value": tops, "unit": "TOPS", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "spin_up_ms": args.spin_up_ms,
+        "spin_up_ms": args.spin_up_ms, "untimed_launches_before_the_timed_steps": spin_launches + args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "int8 GEMM (QLinearMatMul) M=N=K=4096, A [M,K] and B [K,N] int8 U[-127,127], "
@@ -327,13 +336,19 @@ def main():
     # The data sheet's 5.0 POP/s is 256 CUs x 8192 ops per clock at 2400 MHz. With random int8 operands the device
     # holds a lower shader clock under this kernel (it is power-limited: the same launch on all-zero operands runs at
     # the full clock); both are reported next to the headline so that the fraction can be read against either.
-    sclk = sclk_under_load(torch, step)
-    kernel_ms2, _, _ = timer.median_ms(step, 100, warmup=5, per_block=10)
+    sclk, ms_under_sampling = sclk_under_load(torch, step, stream)
+    peak_at_clock = PEAK_INT8_TOPS * sclk / 2400.0 if sclk else None
     out["roofline"]["clock"] = {
         "sclk_mhz_under_this_kernel": sclk, "sclk_mhz_of_the_peak_figure": 2400,
-        "peak_at_measured_clock": PEAK_INT8_TOPS * sclk / 2400.0 if sclk else None,
-        "frac_at_measured_clock": (ops_per_step / (kernel_ms2 * 1e-3) / 1e12) / (PEAK_INT8_TOPS * sclk / 2400.0) if sclk else None,
-        "source": "rocm-smi --showclocks sampled while the kernel runs back to back"}
+        "peak_at_measured_clock": peak_at_clock,
+        # roofline.achieved against the peak at the clock the device holds under this kernel
+        "frac_at_measured_clock": achieved / peak_at_clock if sclk else None,
+        # the same fraction from the launches that ran while the clock was sampled
+        "kernel_ms_while_sampled": ms_under_sampling,
+        "frac_at_measured_clock_while_sampled": (ops_per_step / (ms_under_sampling * 1e-3) / 1e12) / peak_at_clock
+                                                if sclk and ms_under_sampling else None,
+        "source": "rocm-smi --showclocks sampled while the kernel runs back to back (1.5 s of launches, timed in blocks of "
+                  "100 between HIP events on the launch stream)"}
     if args.clock_probe:
         # the same launch on all-zero operands: no benchmark figure, it shows what the clock costs. Behind a flag
         # because these launches are launches of the headline kernel and would enter a profiler's average for it.
@@ -343,8 +358,7 @@ def main():
         def step_zero():
             ctx.check(ctx.lib.sofie_hip_qgemm_s8(ctx.h, 0, n, n, n, ctx.ptr(dZa), n, ctx.ptr(dZb), n, ctx.ptr(dS), None,
                                                  0, L.ACT_NONE, ctx.ptr(dY), n, L.OUT_S8))
-        sclk_zero = sclk_under_load(torch, step_zero)
-        zero_ms, _, _ = timer.median_ms(step_zero, 100, warmup=5, per_block=10)
+        sclk_zero, zero_ms = sclk_under_load(torch, step_zero, stream)
         step()                                   # dY holds the benchmark's result again
         torch.cuda.synchronize()
         out["roofline"]["clock"]["all_zero_operands"] = {
@@ -537,21 +551,65 @@ def cnn_session_rate(iters=300, cpu_images=0):
         ref = models.qcnn_reference(oracle, x[:cpu_images])
         sec = time.perf_counter() - t0
         cpu = {"value": cpu_images / sec, "unit": "inferences/s", "cores": 1, "kind": "port",
+               "role": "the checker of the Session's logits (a scalar restatement of the int8 arithmetic), not the baseline",
                "sample": "oracle/sofie_oracle.c (quantize, three QLinearConv + ReLU + MaxPool, two QLinearMatMul) on the first "
                          "%d of the 4096 images (%.2f s, gcc -O2, 1 thread)" % (cpu_images, sec),
                "logits_bit_exact": bool(np.array_equal(y.reshape(4096, -1)[:cpu_images], ref.reshape(cpu_images, -1)))}
-    return {"cpu_baseline": cpu, "workload": "int8 CNN classifier, batch 4096, 1x40x40 input, generated Session (infer_device on a resident input)",
+    # per kernel, from the runner's events behind every launch (the time of a launch runs from the end of the launch
+    # before it): operations of the layer(s) the launch computes against the int8 matrix peak
+    layer_ops = {"k_qconv_first": 2.0 * 4096 * 1600 * 32 * 9, "k_qconv_ring_pool": 2.0 * 4096 * 400 * 64 * 288,
+                 "k_qconv_ring": 2.0 * 4096 * 100 * 128 * 576, "k_gemm_bytes": 2.0 * 4096 * 256 * 12800,
+                 "k_splitk_finish_pair": 2.0 * 4096 * 5 * 256}
+    kernels = []
+    for k in t.get("kernels", []):
+        e = {"kernel": k["kernel"], "us": k["us"]}
+        if k["kernel"] in layer_ops and k["us"] > 0:
+            e["gop"] = layer_ops[k["kernel"]] / 1e9
+            e["frac_peak"] = layer_ops[k["kernel"]] / (k["us"] * 1e-6) / 1e12 / PEAK_INT8_TOPS
+        kernels.append(e)
+    return {"cpu_baseline": cnn_cpu_reference() if cpu_images > 0 else None, "int8_oracle_checker": cpu,
+            "workload": "int8 CNN classifier, batch 4096, 1x40x40 input, generated Session (infer_device on a resident input)",
             "device_ms": t["device_ms"], "inferences_per_s": 4096 / (t["device_ms"] * 1e-3),
             "tops": 4096 * ops_per_image / t["device_ms"] / 1e9,
             "frac_peak": 4096 * ops_per_image / t["device_ms"] / 1e9 / PEAK_INT8_TOPS,
+            "kernels": kernels,
+            "kernels_note": "one entry per launch of a batch, in launch order; us = time from the end of the launch before it "
+                            "to its own end (events on the Session's stream), averaged over up to 200 batches back to back",
             "host_ms_with_pcie": t["host_ms"], "inferences_per_s_with_pcie": 4096 / (t["host_ms"] * 1e-3),
             "host_ms_with_pcie_pinned_input": t.get("host_pinned_ms"),
             "inferences_per_s_with_pcie_pinned_input": 4096 / (t["host_pinned_ms"] * 1e-3) if t.get("host_pinned_ms") else None,
             "pinned_input_same_logits": t.get("pinned_matches"),
+            "graph_replay_ms": t.get("graph_ms") or None, "graph_replay_same_logits": t.get("graph_matches"),
             # two Sessions in flight on one device (two contexts and streams, a host thread each): wall time per batch
             "two_sessions_ms_per_batch": t.get("two_sessions_ms_per_batch") or None,
             "two_sessions_inferences_per_s": 4096 / (t["two_sessions_ms_per_batch"] * 1e-3) if t.get("two_sessions_ms_per_batch") else None,
             "two_sessions_same_logits": t.get("two_sessions_match")}
+
+
+def cnn_cpu_reference(images=256):
+    """The CPU baseline of the classifier: the call sequence the reference emits for the float model (Conv as weight
+    re-layout + Im2col + sgemm_ + saxpy_ per image, Relu, the MaxPool loop, Gemm as bias copy + sgemm_), restated in
+    oracle/cpu_emitted_bench.c, with sgemm_ from the best BLAS on the box, on `images` images at one thread and at the
+    box's core share. (The reference has no quantized operators: its path for this network is the fp32 one.)"""
+    threads = host_threads()
+    chosen = None
+    for cand in blas_candidates() + [None]:
+        if cpu_emitted("mlp", 1, cand, ("--calls", "20")) is not None:
+            chosen = cand
+            break
+    res = {"kind": "port", "what": "the reference's emitted fp32 call sequence for this network restated in C "
+                                   "(oracle/cpu_emitted_bench.c --workload cnn), gcc -O2",
+           "blas": chosen[2] if chosen else "none found: the bundled loops", "unit": "inferences/s"}
+    for th in sorted({1, threads}):
+        c = cpu_emitted("cnn", th, chosen, ("--images", str(images), "--calls", "3"))
+        if c:
+            res["%d_threads" % th] = {"value": images / (c["median_ms"] * 1e-3), "cores": th, "median_ms": c["median_ms"],
+                                      "sample": "%d of the 4096 images, median of %d calls" % (images, c["calls"])}
+    best = max((v["value"] for k, v in res.items() if k.endswith("_threads")), default=None)
+    res["value"] = best
+    res["sample"] = "%d of the 4096 images per call" % images
+    res["cores"] = max((v["cores"] for k, v in res.items() if k.endswith("_threads") and v["value"] == best), default=None)
+    return res
 
 
 if __name__ == "__main__":

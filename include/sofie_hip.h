@@ -114,6 +114,18 @@ int sofie_hip_graph_destroy(sofie_hip_ctx *ctx, sofie_hip_graph *graph);
 int sofie_hip_timer_start(sofie_hip_ctx *ctx);
 int sofie_hip_timer_stop(sofie_hip_ctx *ctx, float *elapsed_ms);
 
+/* Per-launch timing of whatever is enqueued on the context between the two calls: trace_begin records an event,
+ * every kernel launch of the library on this context then records one behind itself, and trace_end waits for the
+ * stream and writes one line per launch, in launch order, "<kernel> <microseconds>\n": the time from the end of the
+ * launch before it (or from trace_begin) to its own end, so the lines of a sequence add up to the sequence's time on
+ * the device, the gaps between dependent kernels included. The text is truncated to `capacity` bytes (always
+ * NUL-terminated); *launches receives the number of launches seen. Not allowed while a graph is being recorded; at
+ * most SOFIE_HIP_TRACE_MAX launches are kept, later ones are counted but not timed. No counterpart in the reference
+ * (its generated code is timed from outside); it is what the benchmark reports per-kernel figures of a Session from. */
+#define SOFIE_HIP_TRACE_MAX 4096
+int sofie_hip_trace_begin(sofie_hip_ctx *ctx);
+int sofie_hip_trace_end(sofie_hip_ctx *ctx, char *text, size_t capacity, int *launches);
+
 /* ---------------------------------------------------------------- fp32 operators */
 
 /* Y[M,N] = alpha * op(A) * op(B) + beta * bias, then optional ReLU.

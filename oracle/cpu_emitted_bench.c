@@ -10,6 +10,11 @@
  *         ROperator_Relu.hxx:54-66): inside infer the weight re-layout loop into x_f; per image Im2col
  *         (SOFIE_common.hxx:485-518), BLAS::sgemm_('N','N', m = OH*OW, n = OC, k = C*KH*KW, 1, xcol, m, x_f, k, 0,
  *         Y + off, m), BLAS::saxpy_(OC*OH*OW, 1, bias broadcast to [OC,OH,OW], 1, Y + off, 1); then the Relu loop
+ *   cnn   the classifier of the batch-4096 configuration in fp32, as the reference would emit it for the float model
+ *         (it has no quantized operators): Conv 1->32 3x3 + Relu, MaxPool 2x2, Conv 32->64 + Relu, MaxPool, Conv 64->128 +
+ *         Relu, Flatten (a view), Gemm 12800->256 + Relu, Gemm 256->5 on 1x40x40 images. Conv and Gemm as above; the
+ *         MaxPool loop of ROperator_Pool.hxx:371-416 (for every batch*channel plane, rows hmin..hmax and columns
+ *         wmin..wmax in steps of the stride, the maximum over the kh x kw window cells that lie inside the plane).
  * The FLOPs of the reference run in an external Fortran BLAS chosen when it is built (CMake find_package(BLAS));
  * here sgemm_ / saxpy_ are bound at run time with dlopen from the library named on the command line
  * (--blas PATH --prefix P: symbols P"sgemm_" and P"saxpy_"), and fall back to the loops of this file (the
@@ -157,6 +162,31 @@ static void emitted_conv_relu(int N, int C, int H, int W, int OC, int KH, int KW
     for (size_t id = 0; id < len; id++) y[id] = ((y[id] > 0) ? y[id] : 0);
 }
 
+/* ------------------------------------------------------------------ MaxPool, as ROperator_Pool emits it for 2-D inputs */
+static void emitted_maxpool(int planes, int hsize, int wsize, int kh, int kw, int pad, int sh, int sw, const float *x, float *y)
+{
+    /* hmin = -pad, hmax = hsize + pad - kh + 1 (ROperator_Pool.hxx:283-305) */
+    const int hmin = -pad, hmax = hsize + pad - kh + 1, wmin = -pad, wmax = wsize + pad - kw + 1;
+    size_t outIndex = 0;
+    for (size_t n = 0; n < (size_t)planes; n++) {
+        size_t inputOffset = n * (size_t)hsize * wsize;
+        for (int i = hmin; i < hmax; i += sh) {
+            for (int j = wmin; j < wmax; j += sw) {
+                float value = -INFINITY;
+                for (int l = i; l < i + kh; l++) {
+                    if (l < 0 || l >= hsize) continue;
+                    for (int m = j; m < j + kw; m++) {
+                        if (m < 0 || m >= wsize) continue;
+                        const float xval = x[inputOffset + (size_t)l * wsize + m];
+                        if (xval > value) value = xval;
+                    }
+                }
+                y[outIndex++] = value;
+            }
+        }
+    }
+}
+
 static float *alloc_f(size_t n)
 {
     float *p = (float *)malloc(n * sizeof(float));
@@ -194,7 +224,7 @@ int main(int argc, char **argv)
         else if (!strcmp(argv[i], "--calls") && i + 1 < argc) calls = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--images") && i + 1 < argc) images = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--dump") && i + 1 < argc) dump = argv[++i];
-        else { fprintf(stderr, "usage: %s [--workload mlp|conv] [--blas PATH --prefix P] [--calls N] [--images N] [--dump FILE]\n", argv[0]); return 2; }
+        else { fprintf(stderr, "usage: %s [--workload mlp|conv|cnn] [--blas PATH --prefix P] [--calls N] [--images N] [--dump FILE]\n", argv[0]); return 2; }
     }
     const char *bound = "bundled loops (no BLAS library)";
     if (blas) {
@@ -271,6 +301,70 @@ int main(int argc, char **argv)
             fwrite(y, sizeof(float), (size_t)N * OC * plane, f);
             fclose(f);
         }
+    } else if (!strcmp(workload, "cnn")) {
+        /* images U[0,1]; Kaiming-normal weights; small biases, broadcast at construction as the reference does */
+        const int N = images;
+        const int ch[4] = {1, 32, 64, 128}, side[4] = {40, 20, 10, 10};   /* input channels / spatial size of conv l */
+        if (calls <= 0) calls = 3;
+        float *x = alloc_f((size_t)N * 1600);
+        for (size_t i = 0; i < (size_t)N * 1600; ++i) x[i] = (float)uniform01();
+        float *cw[3], *cb[3], *cbb[3], *cxf[3], *cy[3], *pool[2];
+        size_t max_col = 0;
+        for (int l = 0; l < 3; ++l) {
+            const int C = ch[l], OC = ch[l + 1], hw = side[l] * side[l];
+            cw[l] = alloc_f((size_t)OC * C * 9);
+            cb[l] = alloc_f(OC);
+            cbb[l] = alloc_f((size_t)OC * hw);
+            cxf[l] = alloc_f((size_t)OC * C * 9);
+            cy[l] = alloc_f((size_t)N * OC * hw);
+            for (int i = 0; i < OC * C * 9; ++i) cw[l][i] = (float)(normal01() * sqrt(2.0 / (C * 9.0)));
+            for (int i = 0; i < OC; ++i) cb[l][i] = (float)(normal01() * 0.05);
+            for (int oc = 0; oc < OC; ++oc)
+                for (int p = 0; p < hw; ++p) cbb[l][(size_t)oc * hw + p] = cb[l][oc];
+            if ((size_t)C * 9 * hw > max_col) max_col = (size_t)C * 9 * hw;
+        }
+        pool[0] = alloc_f((size_t)N * 32 * 400);
+        pool[1] = alloc_f((size_t)N * 64 * 100);
+        float *xcol = alloc_f(max_col);
+        const int K1 = 12800, N1 = 256, N2 = 5;
+        float *w1 = alloc_f((size_t)K1 * N1), *w2 = alloc_f((size_t)N1 * N2), *b1 = alloc_f(N1), *b2 = alloc_f(N2);
+        float *bb1 = alloc_f((size_t)N * N1), *bb2 = alloc_f((size_t)N * N2), *g1 = alloc_f((size_t)N * N1), *g2 = alloc_f((size_t)N * N2);
+        for (size_t i = 0; i < (size_t)K1 * N1; ++i) w1[i] = (float)(normal01() * sqrt(2.0 / K1));
+        for (int i = 0; i < N1 * N2; ++i) w2[i] = (float)(normal01() * sqrt(2.0 / N1));
+        for (int i = 0; i < N1; ++i) b1[i] = (float)(normal01() * 0.05);
+        for (int i = 0; i < N2; ++i) b2[i] = (float)(normal01() * 0.05);
+        for (int r = 0; r < N; ++r) {
+            memcpy(bb1 + (size_t)r * N1, b1, N1 * sizeof(float));
+            memcpy(bb2 + (size_t)r * N2, b2, N2 * sizeof(float));
+        }
+        times = (double *)malloc(sizeof(double) * calls);
+        for (int it = -1; it < calls; ++it) {
+            const double t0 = now_ms();
+            emitted_conv_relu(N, 1, 40, 40, 32, 3, 3, 1, 1, x, cw[0], cbb[0], cxf[0], xcol, cy[0]);
+            emitted_maxpool(N * 32, 40, 40, 2, 2, 0, 2, 2, cy[0], pool[0]);
+            emitted_conv_relu(N, 32, 20, 20, 64, 3, 3, 1, 1, pool[0], cw[1], cbb[1], cxf[1], xcol, cy[1]);
+            emitted_maxpool(N * 64, 20, 20, 2, 2, 0, 2, 2, cy[1], pool[1]);
+            emitted_conv_relu(N, 64, 10, 10, 128, 3, 3, 1, 1, pool[1], cw[2], cbb[2], cxf[2], xcol, cy[2]);
+            emitted_gemm(N, N1, K1, cy[2], w1, bb1, g1, 1);          /* Flatten is a view of the convolution's output */
+            emitted_gemm(N, N2, N1, g1, w2, bb2, g2, 0);
+            if (it >= 0) times[it] = now_ms() - t0;
+        }
+        for (int i = 0; i < N * N2; ++i) checksum += g2[i];
+        if (dump) {
+            FILE *f = fopen(dump, "wb");
+            if (!f) { perror(dump); return 6; }
+            fwrite(x, sizeof(float), (size_t)N * 1600, f);
+            for (int l = 0; l < 3; ++l) {
+                fwrite(cw[l], sizeof(float), (size_t)ch[l + 1] * ch[l] * 9, f);
+                fwrite(cb[l], sizeof(float), ch[l + 1], f);
+            }
+            fwrite(w1, sizeof(float), (size_t)K1 * N1, f);
+            fwrite(b1, sizeof(float), N1, f);
+            fwrite(w2, sizeof(float), (size_t)N1 * N2, f);
+            fwrite(b2, sizeof(float), N2, f);
+            fwrite(g2, sizeof(float), (size_t)N * N2, f);
+            fclose(f);
+        }
     } else {
         fprintf(stderr, "cpu_emitted_bench: unknown workload %s\n", workload);
         return 2;
@@ -278,6 +372,6 @@ int main(int argc, char **argv)
     qsort(times, calls, sizeof(double), cmp_double);
     printf("{\"workload\": \"%s\", \"blas\": \"%s\", \"calls\": %d, \"images\": %d, \"median_ms\": %.6f, \"best_ms\": %.6f, "
            "\"checksum\": %.6e, \"selfcheck\": %.3e}\n",
-           workload, bound, calls, !strcmp(workload, "conv") ? images : 256, times[calls / 2], times[0], checksum, check);
+           workload, bound, calls, strcmp(workload, "mlp") ? images : 256, times[calls / 2], times[0], checksum, check);
     return 0;
 }

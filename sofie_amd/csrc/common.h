@@ -19,6 +19,15 @@ struct sofie_hip_ctx {
    bool no_alloc = false;       // inside sofie_hip_qgemm_s8_noalloc: workspace() hands out the fixed array, never allocates
    void *static_scratch = nullptr;   // this device's address of the fixed scratch array (looked up in sofie_hip_create)
    int live_graphs = 0;         // recorded graphs not yet destroyed: they hold the scratch buffer's address
+   // between sofie_hip_trace_begin and _end: an event behind every launch (check_launch records it), with the kernel's name
+   bool tracing = false;
+   int trace_seen = 0;
+   struct TracePoint {
+      const char *what;
+      hipEvent_t done;
+   };
+   TracePoint *trace = nullptr;   // [SOFIE_HIP_TRACE_MAX + 1], entry 0 is the start
+   int trace_len = 0;
    char err[512] = {0};
 };
 

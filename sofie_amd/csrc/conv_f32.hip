@@ -654,7 +654,7 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          SOFIE_LARGE_LDS(kern);
          hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
          *done = true;
-         return check_launch(ctx, "k_conv2d_f32_pipe (phases)");
+         return check_launch(ctx, "k_conv2d_f32_pipe_phases");
       }
       lds_max = 0;
       tiles_max = 0;
@@ -693,7 +693,7 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    SOFIE_LARGE_LDS(kern);
    hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, g);
    *done = true;
-   return check_launch(ctx, "k_conv2d_f32 (phases)");
+   return check_launch(ctx, "k_conv2d_f32_phases");
 }
 
 int run_conv(sofie_hip_ctx *ctx, ConvArgs &g)

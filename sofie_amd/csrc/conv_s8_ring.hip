@@ -698,7 +698,7 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
 #undef SOFIE_QRING_BY_ROW
 #undef SOFIE_QRING_LAUNCH
    *done = true;
-   return check_launch(ctx, "k_qconv_ring");
+   return check_launch(ctx, pool ? "k_qconv_ring_pool" : "k_qconv_ring");
 }
 
 }  // namespace sofie

@@ -1135,7 +1135,7 @@ int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
          constexpr auto loop = k_gemm_dma<Mma, BK, NST, OUT, B_KN, true>;
          SOFIE_LARGE_LDS(loop);
          hipLaunchKernelGGL(loop, dim3(ctx->num_cus), dim3(512), loop_lds, ctx->stream, g);
-         return check_launch(ctx, "k_gemm_dma (persistent)");
+         return check_launch(ctx, "k_gemm_dma_persistent");
       }
    }
    constexpr auto kern = k_gemm_dma<Mma, BK, NST, OUT, B_KN>;

@@ -226,7 +226,7 @@ extern "C" int sofie_hip_gemm_f32_stacked(sofie_hip_ctx *ctx, int transA, int tr
       const bool small = (size_t)cdiv(M, 128) * cdiv(N, 128) * nz < 256;
       if (small) hipLaunchKernelGGL((k_gemm_f32<1, 1>), dim3(cdiv(N, 64), cdiv(M, 64), nz), dim3(256), 0, ctx->stream, g);
       else hipLaunchKernelGGL((k_gemm_f32<2, 2>), dim3(cdiv(N, 128), cdiv(M, 128), nz), dim3(256), 0, ctx->stream, g);
-      if (int rc = check_launch(ctx, "k_gemm_f32 (stacked)")) return rc;
+      if (int rc = check_launch(ctx, "k_gemm_f32_stacked")) return rc;
    }
    return SOFIE_HIP_OK;
 }

@@ -128,10 +128,33 @@ int check_launch(sofie_hip_ctx *ctx, const char *what)
    hipError_t e = hipGetLastError();
    if (e != hipSuccess)
       return set_error(ctx, SOFIE_HIP_EHIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+   if (ctx->tracing) {
+      ++ctx->trace_seen;
+      if (ctx->trace_len <= SOFIE_HIP_TRACE_MAX) {
+         hipEvent_t ev = nullptr;
+         if (hipEventCreate(&ev) == hipSuccess && hipEventRecord(ev, ctx->stream) == hipSuccess) {
+            ctx->trace[ctx->trace_len].what = what;
+            ctx->trace[ctx->trace_len].done = ev;
+            ++ctx->trace_len;
+         } else {
+            (void)hipGetLastError();
+            if (ev) (void)hipEventDestroy(ev);
+         }
+      }
+   }
    return SOFIE_HIP_OK;
 }
 
 }  // namespace sofie
+
+static void drop_trace(sofie_hip_ctx *ctx)
+{
+   for (int i = 0; i < ctx->trace_len; ++i) (void)hipEventDestroy(ctx->trace[i].done);
+   delete[] ctx->trace;
+   ctx->trace = nullptr;
+   ctx->trace_len = 0;
+   ctx->tracing = false;
+}
 
 extern "C" {
 
@@ -183,6 +206,7 @@ int sofie_hip_destroy(sofie_hip_ctx *ctx)
       ctx->capturing = false;
    }
    (void)hipStreamSynchronize(ctx->stream);
+   if (ctx->trace) drop_trace(ctx);
    if (ctx->workspace) (void)hipFree(ctx->workspace);
    (void)hipEventDestroy(ctx->ev_start);
    (void)hipEventDestroy(ctx->ev_stop);
@@ -301,6 +325,7 @@ int sofie_hip_capture_begin(sofie_hip_ctx *ctx)
 {
    if (!ctx) return SOFIE_HIP_EINVAL;
    SOFIE_REQUIRE(ctx, !ctx->capturing, "a capture is already open on this context");
+   SOFIE_REQUIRE(ctx, !ctx->tracing, "a trace is open on this context: events cannot be recorded into a graph");
    SOFIE_HIP_CALL(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
    ctx->capturing = true;
    return SOFIE_HIP_OK;
@@ -352,6 +377,55 @@ int sofie_hip_graph_destroy(sofie_hip_ctx *ctx, sofie_hip_graph *g)
    if (g->graph) (void)hipGraphDestroy(g->graph);
    delete g;
    if (ctx->live_graphs > 0) --ctx->live_graphs;
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_trace_begin(sofie_hip_ctx *ctx)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
+   SOFIE_REQUIRE(ctx, !ctx->tracing, "a trace is already open on this context");
+   ctx->trace = new sofie_hip_ctx::TracePoint[SOFIE_HIP_TRACE_MAX + 1];
+   ctx->trace_len = 0;
+   ctx->trace_seen = 0;
+   hipEvent_t ev = nullptr;
+   if (hipEventCreate(&ev) != hipSuccess || hipEventRecord(ev, ctx->stream) != hipSuccess) {
+      (void)hipGetLastError();
+      if (ev) (void)hipEventDestroy(ev);
+      drop_trace(ctx);
+      return sofie::set_error(ctx, SOFIE_HIP_EHIP, "sofie_hip_trace_begin: the start event could not be recorded");
+   }
+   ctx->trace[0].what = "";
+   ctx->trace[0].done = ev;
+   ctx->trace_len = 1;
+   ctx->tracing = true;
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_trace_end(sofie_hip_ctx *ctx, char *text, size_t capacity, int *launches)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, ctx->tracing, "no trace is open on this context");
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
+   ctx->tracing = false;
+   if (launches) *launches = ctx->trace_seen;
+   if (text && capacity) text[0] = 0;
+   hipError_t e = hipStreamSynchronize(ctx->stream);
+   size_t used = 0;
+   for (int i = 1; i < ctx->trace_len && e == hipSuccess; ++i) {
+      float ms = 0.0f;
+      e = hipEventElapsedTime(&ms, ctx->trace[i - 1].done, ctx->trace[i].done);
+      if (e != hipSuccess || !text || used + 1 >= capacity) continue;
+      const int n = snprintf(text + used, capacity - used, "%s %.3f\n", ctx->trace[i].what, ms * 1e3);
+      if (n < 0 || (size_t)n >= capacity - used) {
+         text[used] = 0;       // the line does not fit: the text ends in front of it
+         used = capacity;
+      } else {
+         used += (size_t)n;
+      }
+   }
+   drop_trace(ctx);
+   if (e != hipSuccess) return sofie::set_error(ctx, SOFIE_HIP_EHIP, "sofie_hip_trace_end: %s", hipGetErrorString(e));
    return SOFIE_HIP_OK;
 }
 

@@ -16,6 +16,7 @@
 #include <fstream>
 #include <iostream>
 #include <memory>
+#include <sstream>
 #include <string>
 #include <thread>
 #include <tuple>
@@ -162,10 +163,9 @@ int main(int argc, char **argv)
          for (int i = 0; i < iters; ++i) yp = s.infer(pinned);
          const double pinned_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
          // the same sequence replayed from a HIP graph: outputs must not change, timing of back-to-back replays
-         // (SOFIE_RUN_NO_GRAPH in the environment leaves this part out, e.g. under a profiler that traces kernels only)
          bool same = true;
          float gms = 0;
-         if (!std::getenv("SOFIE_RUN_NO_GRAPH")) {
+         {
             s.use_graph(true);
             std::vector<SOFIE_OUT_T> yg = s.infer(x.data());
             same = yg.size() == y.size();
@@ -218,10 +218,45 @@ int main(int argc, char **argv)
                pair_same = pair_same && read && std::memcmp(yk.data(), y.data(), y.size() * sizeof(SOFIE_OUT_T)) == 0;
             }
          }
+         // Per launch: an event behind every kernel of the sequence (sofie_hip_trace_begin / _end), over up to 200 runs
+         // back to back; a launch's time runs from the end of the launch before it, so the entries of a run add up to
+         // the run. Averaged by position in the run.
+         std::string kernels = "[";
+         {
+            const int passes = iters < 200 ? iters : 200;
+            std::vector<char> text(1 << 20);
+            int seen = 0;
+            if (sofie_hip_trace_begin(s.fCtx) == 0) {
+               for (int i = 0; i < passes; ++i) s.infer_device(s.SOFIE_INPUT_MEMBER);
+               if (sofie_hip_trace_end(s.fCtx, text.data(), text.size(), &seen) == 0 && seen > 0 && seen % passes == 0 &&
+                   seen <= SOFIE_HIP_TRACE_MAX) {
+                  const int per = seen / passes;
+                  std::vector<std::string> names(per);
+                  std::vector<double> sum(per, 0.0);
+                  std::istringstream lines(text.data());
+                  std::string name;
+                  double us = 0;
+                  int k = 0;
+                  for (; lines >> name >> us; ++k) {
+                     names[k % per] = name;
+                     sum[k % per] += us;
+                  }
+                  if (k == seen) {
+                     for (int j = 0; j < per; ++j) {
+                        char item[256];
+                        std::snprintf(item, sizeof(item), "%s{\"kernel\": \"%s\", \"us\": %.3f}", j ? ", " : "", names[j].c_str(), sum[j] / passes);
+                        kernels += item;
+                     }
+                  }
+               }
+            }
+         }
+         kernels += "]";
          std::printf("{\"device_ms\": %.6f, \"host_ms\": %.6f, \"host_pinned_ms\": %.6f, \"pinned_matches\": %s, \"graph_ms\": %.6f, "
-                     "\"graph_matches\": %s, \"sessions_in_flight\": %d, \"two_sessions_ms_per_batch\": %.6f, \"two_sessions_match\": %s, \"iters\": %d}\n",
+                     "\"graph_matches\": %s, \"sessions_in_flight\": %d, \"two_sessions_ms_per_batch\": %.6f, \"two_sessions_match\": %s, "
+                     "\"iters\": %d, \"kernels\": %s}\n",
                      ms / iters, host_ms / iters, pinned_ms / iters, pinned_same ? "true" : "false", gms / iters,
-                     same ? "true" : "false", nsess, pair_ms, pair_same ? "true" : "false", iters);
+                     same ? "true" : "false", nsess, pair_ms, pair_same ? "true" : "false", iters, kernels.c_str());
       }
 #endif
 #endif

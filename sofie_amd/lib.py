@@ -34,6 +34,8 @@ SIGNATURES = {
     "sofie_hip_sync": [_p],
     "sofie_hip_timer_start": [_p],
     "sofie_hip_timer_stop": [_p, C.POINTER(_f)],
+    "sofie_hip_trace_begin": [_p],
+    "sofie_hip_trace_end": [_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_int)],
     "sofie_hip_gemm_f32": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _f, _p, _i, _p, _i, _i],
     "sofie_hip_mlp_f32": [_p, _i, C.POINTER(_i), C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(_i), _p, _i, _p, _i, _i],
     "sofie_hip_gemm_f32_stacked": [_p, _i, _i, _i, _i, _i, _f, _p, _i, _p, _i, _p, _i, _i, C.POINTER(_i),

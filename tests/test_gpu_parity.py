@@ -964,6 +964,44 @@ def test_gemm_fp8_benchmark_operands_at_full_depth(ops, transB):
                                               int(big.sum()), (err / tol).max()))
 
 
+def test_trace_times_every_launch(ops):
+    """sofie_hip_trace_begin / _end: one line per launch between the two calls, in launch order, with the name of the
+    kernel and a positive time; opening a second trace, ending one that is not open, or recording a graph while a trace is
+    open is refused."""
+    import ctypes as C
+    from sofie_amd import lib as L
+    ctx = ops.default_context()
+    lib = ctx.lib
+    x = ctx.dev(rng(5).standard_normal(1 << 16).astype(np.float32))
+    y = ctx.empty((1 << 16,), torch.float32)
+    a = ctx.dev(rng(6).integers(-127, 128, (64, 64)).astype(np.int8))
+    s1 = ctx.dev(np.full(64, 1e-3, np.float32))
+    yq = ctx.empty((64, 64), torch.int8)
+    buf = C.create_string_buffer(4096)
+    n = C.c_int(-1)
+    assert lib.sofie_hip_trace_end(ctx.h, buf, 4096, C.byref(n)) == L.EINVAL
+    assert lib.sofie_hip_trace_begin(ctx.h) == 0
+    assert lib.sofie_hip_trace_begin(ctx.h) == L.EINVAL
+    assert lib.sofie_hip_capture_begin(ctx.h) == L.EINVAL
+    for _ in range(3):
+        ctx.check(lib.sofie_hip_relu_f32(ctx.h, ctx.ptr(x), ctx.ptr(y), x.numel()))
+    ctx.check(lib.sofie_hip_qgemm_s8(ctx.h, 1, 64, 64, 64, ctx.ptr(a), 64, ctx.ptr(a), 64, ctx.ptr(s1), None, 0, 0, ctx.ptr(yq), 64, L.OUT_S8))
+    assert lib.sofie_hip_trace_end(ctx.h, buf, 4096, C.byref(n)) == 0
+    lines = buf.value.decode().splitlines()
+    assert n.value == 4 and len(lines) == 4
+    assert [l.split()[0] for l in lines[:3]] == ["k_relu_f32"] * 3 and lines[3].split()[0].startswith("k_")
+    assert all(float(l.split()[1]) > 0 for l in lines)
+    # a buffer too small for the text: whole lines only, NUL-terminated, the count still complete
+    assert lib.sofie_hip_trace_begin(ctx.h) == 0
+    for _ in range(3):
+        ctx.check(lib.sofie_hip_relu_f32(ctx.h, ctx.ptr(x), ctx.ptr(y), x.numel()))
+    small = C.create_string_buffer(24)
+    assert lib.sofie_hip_trace_end(ctx.h, small, 24, C.byref(n)) == 0
+    assert n.value == 3 and 1 <= len(small.value.decode().splitlines()) < 3 and small.value.decode().endswith("\n")
+    ctx.sync()
+    assert torch.equal(y, torch.relu(x))
+
+
 # --------------------------------------------------------------------------- graph recording rules
 def test_capture_rules_are_enforced():
     """Between capture_begin and capture_end the calls that would wait on, or record a memset node into, the

@@ -555,6 +555,31 @@ def test_cpu_baseline_program_computes_what_the_oracle_computes(tmp_path):
         assert np.max(np.abs(y.reshape(ref.shape) - ref)) <= 1e-5 * np.max(np.abs(ref))
 
 
+def test_cpu_baseline_cnn_computes_what_the_oracle_computes(tmp_path):
+    """The 'cnn' workload of oracle/cpu_emitted_bench.c (the reference's emitted fp32 sequence for the classifier of
+    the batch-4096 configuration: Conv + Relu, the MaxPool loop, Gemm) against the oracle's convolution, pooling and
+    Gemm on the tensors it dumps, with the bundled loops and with a BLAS bound at run time."""
+    blas = _scipy_blas()
+    variants = [[]] + ([["--blas", blas, "--prefix", "scipy_"]] if blas else [])
+    n = 3
+    for extra in variants:
+        f = str(tmp_path / "cnn.bin")
+        out = _cpu_emitted(["--workload", "cnn", "--images", str(n), "--calls", "1", "--dump", f] + extra, {"OMP_NUM_THREADS": "2"})
+        assert out["images"] == n
+        raw = np.fromfile(f, np.float32)
+        sizes = [n * 1600, 32 * 9, 32, 64 * 32 * 9, 64, 128 * 64 * 9, 128, 12800 * 256, 256, 256 * 5, 5, n * 5]
+        assert raw.size == sum(sizes)
+        x, w1, b1, w2, b2, w3, b3, f1, c1, f2, c2, y = np.split(raw, np.cumsum(sizes)[:-1])
+        h = oracle.conv2d_f32(x.reshape(n, 1, 40, 40), w1.reshape(32, 1, 3, 3), b1, (1, 1), relu=True)
+        h = oracle.maxpool2d(h, (2, 2), (2, 2))
+        h = oracle.conv2d_f32(h, w2.reshape(64, 32, 3, 3), b2, (1, 1), relu=True)
+        h = oracle.maxpool2d(h, (2, 2), (2, 2))
+        h = oracle.conv2d_f32(h, w3.reshape(128, 64, 3, 3), b3, (1, 1), relu=True)
+        g = oracle.gemm_f32(h.reshape(n, 12800), f1.reshape(12800, 256), c1, relu=True)
+        ref = oracle.gemm_f32(g, f2.reshape(256, 5), c2)
+        assert np.max(np.abs(y.reshape(n, 5) - ref)) <= 1e-5 * np.max(np.abs(ref))
+
+
 # ----------------------------------------------------------------------------- fp32 average pooling
 @pytest.mark.parametrize("cfg", [
     dict(shape=(2, 3, 9, 8), k=(3, 2), s=(2, 1), p=(0, 0, 0, 0)),
