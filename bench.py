@@ -559,6 +559,7 @@ def cnn_session_rate(iters=300, cpu_images=0):
     # before it): operations of the layer(s) the launch computes against the int8 matrix peak
     layer_ops = {"k_qconv_first": 2.0 * 4096 * 1600 * 32 * 9, "k_qconv_ring_pool": 2.0 * 4096 * 400 * 64 * 288,
                  "k_qconv_ring": 2.0 * 4096 * 100 * 128 * 576, "k_gemm_bytes": 2.0 * 4096 * 256 * 12800,
+                 "k_qconv_ring_pair": 2.0 * 4096 * 400 * 64 * 288 + 2.0 * 4096 * 100 * 128 * 576,
                  "k_splitk_finish_pair": 2.0 * 4096 * 5 * 256}
     kernels = []
     for k in t.get("kernels", []):

@@ -335,6 +335,31 @@ int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, int x_layout,
                               int stride_w, int groups, int zp_x, int zp_y, int act, int pool_kh,
                               int pool_kw, int pool_stride_h, int pool_stride_w);
 
+/* A chain of QLinearConv layers in one call: layer 0 reads x, every later layer the output of the layer before it
+ * (layers[l].y in layers[l].y_layout); each layer is what sofie_hip_qconv2d_s8 (pool_kh == 0) or
+ * sofie_hip_qconv2d_pool_s8 computes, int8 out, and the results are bit-identical to those calls made one after the
+ * other. What the call adds: two consecutive 3x3 stride-1 layers on 32 or 64 channels run as ONE kernel launch when
+ * every workgroup owns the same whole images in both (the batch a multiple of the workgroups, as at batch 4096): a
+ * workgroup then reads in the second layer only what it wrote itself in the first, so no kernel boundary is needed
+ * between them. Other shapes run layer by layer. Replaces the emitted Conv sequences of consecutive Conv (+ Relu,
+ * + MaxPool) operators (ROperator_Conv.hxx:377-522, ROperator_Pool.hxx:371-416), each of which ends with its whole
+ * output in host memory before the next begins. */
+#define SOFIE_QCONV_CHAIN_MAX 8
+typedef struct sofie_hip_qconv_layer {
+   const int8_t *w;            /* weights, layout w_layout */
+   int w_layout;
+   const int32_t *bias;        /* [OC] or NULL */
+   const float *scale;         /* [OC] */
+   int8_t *y;                  /* the layer's (pooled) output */
+   int y_layout;
+   int C, H, W, OC, KH, KW;    /* input channels and size, output channels, kernel */
+   int pad_top, pad_left, pad_bottom, pad_right, stride_h, stride_w, groups;
+   int zp_x, zp_y, act;
+   int pool_kh, pool_kw, pool_stride_h, pool_stride_w;   /* fused max pooling behind the activation; pool_kh == 0: none */
+} sofie_hip_qconv_layer;
+int sofie_hip_qconv2d_s8_chain(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, int N, int n_layers,
+                               const sofie_hip_qconv_layer *layers);
+
 /* QuantizeLinear -> QLinearConv -> (ReLU) -> (MaxPool) in one call, for the first layer of a
  * quantized network: x is the float tensor [N, C, H, W], quantized as in
  * sofie_hip_quantize_f32_s8(x, x_scale, zp_x); everything else as in

@@ -28,4 +28,8 @@ int qconv_first_layer(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done);
 // input rows straight into LDS. *done tells whether the kernel took the problem.
 int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done);
 
+// Two such layers, the second reading the first one's (pooled) output, in one launch where every workgroup owns the
+// same whole images in both. *done tells whether the launch was made (if not, nothing was launched).
+int qconv_ring_pair(sofie_hip_ctx *ctx, const QConvArgs &g1, const QConvArgs &g2, bool *done);
+
 }  // namespace sofie

@@ -770,6 +770,51 @@ extern "C" int sofie_hip_qconv2d_pool_s8(sofie_hip_ctx *ctx, const int8_t *x, in
    return run<SOFIE_OUT_S8>(ctx, g);
 }
 
+extern "C" int sofie_hip_qconv2d_s8_chain(sofie_hip_ctx *ctx, const int8_t *x, int x_layout, int N, int n_layers,
+                                          const sofie_hip_qconv_layer *layers)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, n_layers >= 1 && n_layers <= SOFIE_QCONV_CHAIN_MAX && layers, "bad layer list");
+   QConvArgs g[SOFIE_QCONV_CHAIN_MAX];
+   const int8_t *in = x;
+   int in_layout = x_layout;
+   for (int l = 0; l < n_layers; ++l) {
+      const sofie_hip_qconv_layer &q = layers[l];
+      g[l] = QConvArgs{};
+      if (int rc = fill_args(ctx, g[l], in, in_layout, q.w, q.w_layout, q.bias, q.scale, q.y, q.y_layout, N, q.C, q.H, q.W, q.OC,
+                             q.KH, q.KW, q.pad_top, q.pad_left, q.pad_bottom, q.pad_right, q.stride_h, q.stride_w, q.groups,
+                             q.zp_x, q.zp_y, q.act, SOFIE_OUT_S8))
+         return rc;
+      if (q.pool_kh != 0 || q.pool_kw != 0) {
+         SOFIE_REQUIRE(ctx, q.pool_kh > 0 && q.pool_kw > 0 && q.pool_stride_h > 0 && q.pool_stride_w > 0, "bad pooling window");
+         SOFIE_REQUIRE(ctx, q.pool_kh <= g[l].OH && q.pool_kw <= g[l].OW, "pooling window larger than the convolution output");
+         g[l].pool_kh = q.pool_kh; g[l].pool_kw = q.pool_kw; g[l].pool_sh = q.pool_stride_h; g[l].pool_sw = q.pool_stride_w;
+         g[l].PH = (g[l].OH - q.pool_kh) / q.pool_stride_h + 1;
+         g[l].PW = (g[l].OW - q.pool_kw) / q.pool_stride_w + 1;
+      }
+      if (l + 1 < n_layers)
+         SOFIE_REQUIRE(ctx, layers[l + 1].C == q.OC && layers[l + 1].H == g[l].PH && layers[l + 1].W == g[l].PW,
+                       "a layer's input shape is not the output shape of the layer before it");
+      in = q.y;
+      in_layout = q.y_layout;
+   }
+   if (N == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x, "null operand");
+   for (int l = 0; l < n_layers;) {
+      if (l + 1 < n_layers) {
+         bool done = false;
+         if (int rc = qconv_ring_pair(ctx, g[l], g[l + 1], &done)) return rc;
+         if (done) {
+            l += 2;
+            continue;
+         }
+      }
+      if (int rc = run<SOFIE_OUT_S8>(ctx, g[l])) return rc;
+      ++l;
+   }
+   return SOFIE_HIP_OK;
+}
+
 extern "C" int sofie_hip_quantize_qconv2d_s8(sofie_hip_ctx *ctx, const float *x, float x_scale, int zp_x, const int8_t *w,
                                              int w_layout, const int32_t *bias, const float *scale, int8_t *y,
                                              int y_layout, int N, int C, int H, int W, int OC, int KH, int KW, int pad_top,

@@ -62,7 +62,7 @@ static_assert(std::is_trivially_copyable<QConvRingArgs>::value && std::is_standa
 // requantisation is monotonic; for a negative scale the minimum is taken) and a quarter of the values is converted and
 // stored. In that mode the "pixels" of tiles, runs and a.OH / a.OW / a.ep.M are pooled pixels.
 template <int C16, int WN, bool ROWDMA, bool POOL>
-__global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
+__device__ __forceinline__ void qconv_ring_body(const QConvRingArgs &a, unsigned char *smem)
 {
    constexpr int NB = 2;
    constexpr int MB = POOL ? 4 : 2;                 // accumulator tiles along m per wavefront
@@ -82,7 +82,6 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    constexpr int CB = C16 / 2;                      // 32-channel blocks
    constexpr int NS = 9 * CB;                       // K steps of 32 bytes
    constexpr int NRL = ROWDMA ? NWAVE : NWAVE / C16;   // wavefronts that share the rows of a request among them
-   extern __shared__ __align__(16) unsigned char smem[];
    unsigned char *const s_w = smem;                                        // [OCT][KS]
    float *const s_scale = reinterpret_cast<float *>(smem + OCT * a.KS);    // [OCT]
    int *const s_bias = reinterpret_cast<int *>(s_scale + OCT);             // [OCT]
@@ -582,13 +581,49 @@ __global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
    }
 }
 
+template <int C16, int WN, bool ROWDMA, bool POOL>
+__global__ void __launch_bounds__(512) k_qconv_ring(QConvRingArgs a)
+{
+   extern __shared__ __align__(16) unsigned char smem[];
+   qconv_ring_body<C16, WN, ROWDMA, POOL>(a, smem);
+}
+
+// Two convolutions in one launch: layer a (64 output channels, one block of them) and layer b, which reads layer a's
+// output, for launches in which every workgroup of both layers owns the same whole images. A workgroup then reads in
+// layer b only what it wrote itself in layer a: its stores have reached the L2 once the vector-memory counter is down
+// (a compute unit's L1 is written through and holds no line of a tensor nobody has read since the kernel began), so a
+// wait and a workgroup barrier order the two layers and no kernel boundary stands between them: no wait for the
+// slowest workgroup of layer a, no write-back of the L2s, no launch latency, and layer a's result is still in the
+// workgroup's own L2 when layer b fetches it.
+template <int C16A, bool POOLA, int WNB>
+__global__ void __launch_bounds__(512) k_qconv_ring_pair(QConvRingArgs a, QConvRingArgs b)
+{
+   extern __shared__ __align__(16) unsigned char smem[];
+   qconv_ring_body<C16A, 1, true, POOLA>(a, smem);
+   wait_vmcnt<0>();
+   __syncthreads();        // every wavefront is done with layer a's LDS, every store of the workgroup is in the L2
+   qconv_ring_body<4, WNB, true, false>(b, smem);
+}
+
 }  // namespace
 
 namespace sofie {
 
 // 3x3, stride 1, 32 or 64 input channels, channels-last int8 in and out, rows of at most 64 padded columns; with or
 // without a fused 2x2 stride-2 max pooling.
-int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
+// What a launch of k_qconv_ring needs beside the argument block.
+struct RingPlan {
+   QConvRingArgs a;
+   size_t lds;
+   unsigned grid;
+   int C16, WN, nob;
+   bool row, pool;
+   long long px_per_group;   // (pooled) pixels of a workgroup's run if every run has the same length, else 0
+   int image_px;             // (pooled) pixels of one image
+};
+
+// Fills `plan` if the kernel takes the problem (*done).
+static int plan_ring(sofie_hip_ctx *ctx, const QConvArgs &g, RingPlan &out, bool *done)
 {
    *done = false;
    if (g.xf) return SOFIE_HIP_OK;
@@ -670,7 +705,28 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    if (per > units) per = units;
    a.units_each = units / per;
    a.units_rem = units % per;
-   const dim3 grid((unsigned)(per * nob)), block(512);
+   out.a = a;
+   out.lds = lds;
+   out.grid = (unsigned)(per * nob);
+   out.C16 = C16; out.WN = WN; out.nob = nob;
+   out.row = C16 * (a.PL / 16) <= 64;
+   out.pool = pool;
+   out.px_per_group = a.units_rem == 0 ? (long long)a.units_each * unit : 0;
+   out.image_px = TH * TW;
+   *done = true;
+   return SOFIE_HIP_OK;
+}
+
+int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
+{
+   RingPlan plan;
+   if (int rc = plan_ring(ctx, g, plan, done)) return rc;
+   if (!*done) return SOFIE_HIP_OK;
+   const QConvRingArgs &a = plan.a;
+   const size_t lds = plan.lds;
+   const int C16 = plan.C16, WN = plan.WN;
+   const bool pool = plan.pool;
+   const dim3 grid(plan.grid), block(512);
 #define SOFIE_QRING_LAUNCH(C16_, WN_, ROW_, POOL_)                                                             \
    do {                                                                                                        \
       constexpr auto kern = k_qconv_ring<C16_, WN_, ROW_, POOL_>;                                              \
@@ -679,7 +735,7 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
    } while (0)
 #define SOFIE_QRING_BY_ROW(C16_, WN_, POOL_)                                                                   \
    do {                                                                                                        \
-      if (C16_ * (a.PL / 16) <= 64) SOFIE_QRING_LAUNCH(C16_, WN_, true, POOL_);                                         \
+      if (plan.row) SOFIE_QRING_LAUNCH(C16_, WN_, true, POOL_);                                                \
       else SOFIE_QRING_LAUNCH(C16_, WN_, false, POOL_);                                                        \
    } while (0)
 #define SOFIE_QRING_BY_POOL(C16_, WN_)                                                                         \
@@ -697,8 +753,46 @@ int qconv_ring(sofie_hip_ctx *ctx, const QConvArgs &g, bool *done)
 #undef SOFIE_QRING_BY_POOL
 #undef SOFIE_QRING_BY_ROW
 #undef SOFIE_QRING_LAUNCH
-   *done = true;
    return check_launch(ctx, pool ? "k_qconv_ring_pool" : "k_qconv_ring");
+}
+
+// Layer g1 (its fused pooling included) and layer g2, which reads g1's output, as one launch of k_qconv_ring_pair:
+// both must be problems of k_qconv_ring with one block of output channels and a whole padded row per request, g1 with
+// the fused pooling, and every workgroup must own the same whole images in both layers. *done tells whether the launch
+// was made; if not, nothing was launched and the caller runs the layers one after the other.
+int qconv_ring_pair(sofie_hip_ctx *ctx, const QConvArgs &g1, const QConvArgs &g2, bool *done)
+{
+   *done = false;
+   if (g2.x != static_cast<const int8_t *>(g1.y) || g1.N != g2.N || g2.pool_kh != 0) return SOFIE_HIP_OK;
+   RingPlan p1, p2;
+   bool ok1 = false, ok2 = false;
+   if (int rc = plan_ring(ctx, g1, p1, &ok1)) return rc;
+   if (!ok1) return SOFIE_HIP_OK;
+   if (int rc = plan_ring(ctx, g2, p2, &ok2)) return rc;
+   if (!ok2) return SOFIE_HIP_OK;
+   if (!p1.pool || p1.WN != 1 || p1.nob != 1 || !p1.row || p2.C16 != 4 || p2.nob != 1 || !p2.row || p1.grid != p2.grid) return SOFIE_HIP_OK;
+   // the same whole images per workgroup in both layers
+   if (p1.px_per_group == 0 || p2.px_per_group == 0 || p1.px_per_group % p1.image_px != 0 || p2.px_per_group % p2.image_px != 0 ||
+       p1.px_per_group / p1.image_px != p2.px_per_group / p2.image_px)
+      return SOFIE_HIP_OK;
+   const size_t lds = p1.lds > p2.lds ? p1.lds : p2.lds;
+   const dim3 grid(p1.grid), block(512);
+#define SOFIE_QRING_PAIR(C16A_, WNB_)                                                                          \
+   do {                                                                                                        \
+      constexpr auto kern = k_qconv_ring_pair<C16A_, true, WNB_>;                                              \
+      SOFIE_LARGE_LDS(kern);                                                                                   \
+      hipLaunchKernelGGL(kern, grid, block, lds, ctx->stream, p1.a, p2.a);                                     \
+   } while (0)
+   if (p1.C16 == 2) {
+      if (p2.WN == 2) SOFIE_QRING_PAIR(2, 2);
+      else SOFIE_QRING_PAIR(2, 1);
+   } else {
+      if (p2.WN == 2) SOFIE_QRING_PAIR(4, 2);
+      else SOFIE_QRING_PAIR(4, 1);
+   }
+#undef SOFIE_QRING_PAIR
+   *done = true;
+   return check_launch(ctx, "k_qconv_ring_pair");
 }
 
 }  // namespace sofie

@@ -136,6 +136,7 @@ private:
    void FuseActivations();
    void FusePooling();
    void FuseInputQuantization();
+   void FuseQLinearConvChain();
    void PlanIntermediateMemory();
    void GenerateHeaderInfo(std::string &hgname);
    void GenerateSessionCode();

@@ -369,7 +369,40 @@ class ROperator_QLinearConv final : public ROperator {
    int fZpX = 0, fZpY = 0;
    bool fHasBias = false, fXChannelsLast = false;
    EActivationType fActivation = EActivationType::UNDEFINED;
+   // the layers that follow this one in the same library call (RModel::FuseQLinearConvChain): their descriptors, printed
+   std::vector<std::string> fChain;
 public:
+   // --- chains of layers: this operator and the QLinearConv operators that read its output, one after the other, are
+   // emitted as one sofie_hip_qconv2d_s8_chain call, which runs two of them in one launch where the batch allows it
+   const std::string &OutputName() const { return fPoolKernel.empty() ? fNY : fNYPooled; }
+   const std::string &InputName() const { return fNX; }
+   bool ChainHead() const { return fNXFloat.empty() && fXChannelsLast && !fShapeX.empty(); }
+   bool ChainLayer() const { return ChainHead() && fChain.empty(); }
+   size_t ChainLength() const { return 1 + fChain.size(); }
+   // one initializer of a sofie_hip_qconv_layer
+   std::string LayerDescriptor()
+   {
+      size_t pt, pl, pb, pr;
+      fGeom.Pads2D(pt, pl, pb, pr);
+      const bool pooled = !fPoolKernel.empty();
+      std::stringstream d;
+      d << "{tensor_" << fNWPacked << ", SOFIE_LAYOUT_NHWC, " << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", tensor_"
+        << fNScale << ", tensor_" << OutputName() << ", SOFIE_LAYOUT_NHWC, " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3]
+        << ", " << fShapeW[0] << ", " << fShapeW[2] << ", " << fShapeW[3] << ", " << pt << ", " << pl << ", " << pb << ", " << pr << ", "
+        << fGeom.strides[0] << ", " << fGeom.strides[1] << ", " << fGeom.group << ", " << fZpX << ", " << fZpY << ", "
+        << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << ", ";
+      if (pooled) d << fPoolKernel[0] << ", " << fPoolKernel[1] << ", " << fPoolStrides[0] << ", " << fPoolStrides[1];
+      else d << "0, 0, 0, 0";
+      d << "}";
+      return d.str();
+   }
+   void AppendLayer(ROperator_QLinearConv &next)
+   {
+      fChain.push_back(next.LayerDescriptor());
+      fOutputTensorNames.push_back(next.OutputName());
+      for (auto &n : next.GetOpInputTensors())
+         if (n != next.InputName()) fInputTensorNames.push_back(n);
+   }
    ROperator_QLinearConv(std::string autopad, std::vector<size_t> dilations, size_t group, std::vector<size_t> kernelShape,
                          std::vector<size_t> pads, std::vector<size_t> strides, std::string nameX, std::string nameXScale,
                          std::string nameXZp, std::string nameW, std::string nameWScale, std::string nameWZp,
@@ -502,6 +535,18 @@ public:
       std::stringstream out;
       const bool pooled = !fPoolKernel.empty();
       const bool fromFloat = !fNXFloat.empty();
+      if (!fChain.empty()) {
+         out << "\n//----  operator QLinearConv x " << ChainLength() << " op_" << OpName << " (the layers behind it in the same call)\n";
+         out << SP << "{\n";
+         out << SP << SP << "const sofie_hip_qconv_layer layers[" << ChainLength() << "] = {\n";
+         out << SP << SP << SP << LayerDescriptor();
+         for (auto &d : fChain) out << ",\n" << SP << SP << SP << d;
+         out << "};\n";
+         out << SP << SP << "Check(sofie_hip_qconv2d_s8_chain(fCtx, tensor_" << fNX << ", SOFIE_LAYOUT_NHWC, " << BatchCount(fShapeX[0])
+             << ", " << ChainLength() << ", layers), \"QLinearConv chain op_" << OpName << "\");\n";
+         out << SP << "}\n";
+         return out.str();
+      }
       out << "\n//----  operator " << (fromFloat ? "QuantizeLinear + " : "") << "QLinearConv" << (pooled ? " + MaxPool" : "") << " op_"
           << OpName << "\n";
       out << SP << "Check(";

@@ -431,6 +431,29 @@ void RModel::FuseQLinearPair()
    }
 }
 
+// Consecutive QLinearConv operators, each reading the (pooled) channels-last int8 output of the one before it, are
+// emitted as one sofie_hip_qconv2d_s8_chain call by the first of them: the library then runs two layers in one launch
+// where every workgroup owns the same images in both (no kernel boundary between them), and layer by layer otherwise,
+// with the same bytes either way. Every layer's output stays a tensor of the model (the call writes them all), so
+// other readers of them are served as before; the operators behind the first emit nothing.
+void RModel::FuseQLinearConvChain()
+{
+   for (size_t i = 0; i < fOperators.size(); ++i) {
+      auto *head = dynamic_cast<ROperator_QLinearConv *>(fOperators[i].get());
+      if (!head || head->IsAbsorbed() || !head->ChainLayer()) continue;
+      std::string cur = head->OutputName();
+      for (size_t k = i + 1; k < fOperators.size() && head->ChainLength() < 8; ++k) {
+         ROperator &op = *fOperators[k];
+         if (op.IsAbsorbed() || op.IsFusedAway()) continue;      // emits nothing: a fused Relu, an absorbed MaxPool
+         auto *next = dynamic_cast<ROperator_QLinearConv *>(&op);
+         if (!next || !next->ChainLayer() || (next->InputName() != RootOf(cur) && next->InputName() != cur)) break;
+         head->AppendLayer(*next);
+         next->SetAbsorbed();
+         cur = next->OutputName();
+      }
+   }
+}
+
 // QLinearConv (with its fused Relu) followed by a pad-free int8 MaxPool that is the only consumer of the
 // activation: the pooling moves into the convolution call, which then writes the pooled tensor only.
 // The unpooled tensors disappear from the model, the Relu and the MaxPool emit nothing.
@@ -1108,6 +1131,7 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    }
    FusePooling();
    FuseInputQuantization();
+   if (!(static_cast<std::underlying_type_t<Options>>(Options::kLayerPerCall) & options)) FuseQLinearConvChain();
    PlanIntermediateMemory();
    fGC.clear();
    std::string hgname;

@@ -68,6 +68,17 @@ SIGNATURES = {
 }
 
 
+class QConvLayer(C.Structure):
+    """sofie_hip_qconv_layer of include/sofie_hip.h."""
+    _fields_ = [("w", _p), ("w_layout", _i), ("bias", _p), ("scale", _p), ("y", _p), ("y_layout", _i)] + \
+               [(n, _i) for n in ("C", "H", "W", "OC", "KH", "KW", "pad_top", "pad_left", "pad_bottom", "pad_right", "stride_h",
+                                  "stride_w", "groups", "zp_x", "zp_y", "act", "pool_kh", "pool_kw", "pool_stride_h",
+                                  "pool_stride_w")]
+
+
+SIGNATURES["sofie_hip_qconv2d_s8_chain"] = [_p, _p, _i, _i, _i, C.POINTER(QConvLayer)]
+
+
 def build(verbose=False):
     """Compile every HIP source for gfx950 into libsofie_hip.so (hipcc cross-compiles without a GPU)."""
     cmd = ["make", "-C", os.path.join(_HERE, "csrc"), "-j8"]

@@ -518,6 +518,49 @@ def quantize_qconv2d_s8(x, x_scale, zpx, w, scale, bias=None, pads=(0, 0), strid
     return ctx.ret(y, x)
 
 
+def qconv2d_s8_chain(x, layers, x_layout=L.LAYOUT_NHWC, ctx=None):
+    """A chain of QLinearConv layers in one library call (sofie_hip_qconv2d_s8_chain). `layers` is a list of dicts with
+    the keyword arguments of qconv2d_s8 / qconv2d_pool_s8: w, scale, bias, pads, strides, groups, zpx, zpy, relu,
+    pool (None or (kh, kw)), pool_strides, y_layout, w_layout. Returns the list of every layer's output."""
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.int8)
+    if x_layout == L.LAYOUT_NCHW:
+        N, Cc, H, W = xd.shape
+    else:
+        N, H, W, Cc = xd.shape
+    descs = (L.QConvLayer * len(layers))()
+    keep, outs = [], []
+    for d, q in zip(descs, layers):
+        w, pads, strides = q["w"], q.get("pads", (0, 0)), q.get("strides", (1, 1))
+        bias = fold_zero_point_conv(w, q.get("bias"), q.get("zpx", 0)) if q.get("zpx", 0) != 0 else q.get("bias")
+        w_layout, y_layout = q.get("w_layout", L.LAYOUT_NCHW), q.get("y_layout", L.LAYOUT_NHWC)
+        wd = ctx.dev(w, torch.int8)
+        if w_layout == L.LAYOUT_NCHW:
+            OC, _, kh, kw = wd.shape
+        else:
+            OC, kh, kw, _ = wd.shape
+        OH, OW = conv_out_hw(H, W, kh, kw, pads, strides[0], strides[1])
+        pool, ps = q.get("pool"), q.get("pool_strides", (2, 2))
+        if pool:
+            OH, OW = (OH - pool[0]) // ps[0] + 1, (OW - pool[1]) // ps[1] + 1
+        y = ctx.empty((N, OC, OH, OW) if y_layout == L.LAYOUT_NCHW else (N, OH, OW, OC), torch.int8)
+        sd, bd = ctx.dev(q["scale"], torch.float32), ctx.dev(bias, torch.int32)
+        keep += [wd, sd, bd]
+        d.w, d.w_layout, d.bias, d.scale = wd.data_ptr(), w_layout, (bd.data_ptr() if bd is not None else None), sd.data_ptr()
+        d.y, d.y_layout = y.data_ptr(), y_layout
+        d.C, d.H, d.W, d.OC, d.KH, d.KW = Cc, H, W, OC, kh, kw
+        d.pad_top, d.pad_left, d.pad_bottom, d.pad_right = pads4(pads)
+        d.stride_h, d.stride_w, d.groups = strides[0], strides[1], q.get("groups", 1)
+        d.zp_x, d.zp_y, d.act = int(q.get("zpx", 0)), int(q.get("zpy", 0)), L.ACT_RELU if q.get("relu") else L.ACT_NONE
+        d.pool_kh, d.pool_kw = (pool[0], pool[1]) if pool else (0, 0)
+        d.pool_stride_h, d.pool_stride_w = (ps[0], ps[1]) if pool else (0, 0)
+        outs.append(y)
+        Cc, H, W = OC, OH, OW
+    ctx.check(ctx.lib.sofie_hip_qconv2d_s8_chain(ctx.h, ctx.ptr(xd), x_layout, N, len(layers), descs))
+    ctx.verify_guards()
+    return [o.cpu().numpy() if isinstance(x, np.ndarray) else o for o in outs]
+
+
 def iconv2d_s8(x, w, pads=(0, 0), strides=(1, 1), groups=1, zpx=0, ctx=None):
     return qconv2d_s8(x, w, None, None, pads, strides, groups, zpx, out=L.OUT_S32, ctx=ctx)
 

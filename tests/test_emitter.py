@@ -146,8 +146,14 @@ def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
     spec = models.qcnn_spec(oracle, 2, "qcnn_small")
     hxx, dat, _ = gen(spec, tmp_path)
     code = open(hxx).read()
-    # conv1 and conv2 absorb their MaxPool; the unpooled tensors no longer exist
-    assert code.count("sofie_hip_qconv2d_pool_s8(") == 1 and code.count("sofie_hip_qconv2d_s8(") == 1
+    # conv1 and conv2 absorb their MaxPool; the unpooled tensors no longer exist. conv2 (with its pooling) and conv3 are
+    # the two layers of one chain call, whose descriptors carry what the two separate calls would
+    assert code.count("sofie_hip_qconv2d_s8_chain(fCtx, tensor_p1, SOFIE_LAYOUT_NHWC, 2, 2, layers)") == 1
+    assert "sofie_hip_qconv2d_pool_s8(" not in code and "sofie_hip_qconv2d_s8(" not in code
+    assert ("{tensor_w2_ohwi, SOFIE_LAYOUT_NHWC, tensor_c2_qbias, tensor_c2_qscale, tensor_p2, SOFIE_LAYOUT_NHWC, 32, 20, 20, 64, 3, 3, "
+            "1, 1, 1, 1, 1, 1, 1, -128, -128, SOFIE_ACT_RELU, 2, 2, 2, 2}") in code
+    assert ("{tensor_w3_ohwi, SOFIE_LAYOUT_NHWC, tensor_c3_qbias, tensor_c3_qscale, tensor_c3, SOFIE_LAYOUT_NHWC, 64, 10, 10, 128, 3, 3, "
+            "1, 1, 1, 1, 1, 1, 1, -128, -128, SOFIE_ACT_RELU, 0, 0, 0, 0}") in code
     assert code.count("sofie_hip_quantize_qconv2d_s8(") == 1
     assert "sofie_hip_maxpool2d_s8" not in code and "tensor_c1" not in code.replace("tensor_c1_q", "") and "tensor_r2" not in code
     # the two fully connected layers are one call (the second one has five columns); one call each with kLayerPerCall
@@ -157,6 +163,12 @@ def test_quantized_operators_fold_scales_and_zero_points(tmp_path):
                      r"SOFIE_ACT_NONE, tensor_y, 5, SOFIE_OUT_F32\)", code)
     code_lpc = open(gen(spec, tmp_path, layer_per_call=True)[0]).read()
     assert code_lpc.count("sofie_hip_qgemm_s8(") == 2 and "sofie_hip_qgemm_s8_pair(" not in code_lpc
+    assert code_lpc.count("sofie_hip_qconv2d_pool_s8(") == 1 and code_lpc.count("sofie_hip_qconv2d_s8(") == 1 and "_chain(" not in code_lpc
+    # the chain's input and both of its outputs are alive together: none of them shares arena bytes with another
+    offs = {m.group(1): int(m.group(2)) for m in re.finditer(r"tensor_(p1|p2|c3) = reinterpret_cast<int8_t\*>\(fIntermediateMemoryPool \+ (\d+)\)", code)}
+    sizes = {"p1": 2 * 400 * 32, "p2": 2 * 100 * 64, "c3": 2 * 100 * 128}
+    spans = sorted((offs[k], offs[k] + sizes[k]) for k in ("p1", "p2", "c3"))
+    assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))
     assert "int8_t * tensor_fc1_nk_cl" in code and "tensor_fc1 =" not in code   # transposed once, original dropped
     assert "tensor_w2_ohwi, SOFIE_LAYOUT_NHWC" in code and "tensor_w2 =" not in code
     # conv1 reads the one-channel quantized input as it is, everything after it is channels-last

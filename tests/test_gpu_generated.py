@@ -160,8 +160,8 @@ def test_graph_replay_matches_eager(name, make_input, tmp_path):
     # the time of the sequence on the device (the five batches here are too few for the two to agree closely)
     assert len(timing["kernels"]) >= 1 and all(k["us"] > 0 and k["kernel"].startswith("k_") for k in timing["kernels"])
     if name == "qcnn_b4096":
-        assert [k["kernel"] for k in timing["kernels"]] == ["k_qconv_first", "k_qconv_ring_pool", "k_qconv_ring", "k_gemm_bytes",
-                                                           "k_splitk_finish_pair"]
+        # (the second and third convolution are one launch at this batch)
+        assert [k["kernel"] for k in timing["kernels"]] == ["k_qconv_first", "k_qconv_ring_pair", "k_gemm_bytes", "k_splitk_finish_pair"]
 
 
 def test_stacked_matmul_session(tmp_path):

@@ -601,6 +601,79 @@ def test_conv_pool_fused_matrix_core_kernel(ops, cfg):
         assert np.array_equal(y.transpose(0, 3, 1, 2), ref), (zpx, zpy, relu)
 
 
+def _chain_layers(r, shapes, signs=False):
+    """Random weights, scales and biases for a chain of 3x3 pad-1 layers; shapes = [(C, OC, pooled), ...]."""
+    layers, host = [], []
+    for C, OC, pooled in shapes:
+        w = r.integers(-127, 128, (OC, C, 3, 3)).astype(np.int8)
+        scale = (r.uniform(20, 60, OC) / (73.3 * 73.3 * np.sqrt(9 * C))).astype(np.float32)
+        if signs:
+            scale[2::7] *= -1
+        bias = r.integers(-3000, 3000, OC).astype(np.int32)
+        host.append((w, scale, bias, pooled))
+        layers.append(dict(w=np.ascontiguousarray(w.transpose(0, 2, 3, 1)), w_layout=1, scale=scale, bias=bias, pads=(1, 1),
+                           zpx=-128, zpy=-128, relu=True, pool=(2, 2) if pooled else None, y_layout=1))
+    return layers, host
+
+
+def _chain_reference(x_nchw, host):
+    h = x_nchw
+    outs = []
+    for w, scale, bias, pooled in host:
+        h = oracle.qconv2d_s8(h, w, scale, bias, (1, 1), (1, 1), 1, -128, -128, True)
+        if pooled:
+            h = oracle.maxpool2d(h, (2, 2), (2, 2))
+        outs.append(h)
+    return outs
+
+
+@pytest.mark.parametrize("N,H,shapes", [
+    (6, 20, [(32, 64, True), (64, 128, False)]),                   # the CNN's second and third layer, layer by layer at this batch
+    (3, 12, [(32, 64, False), (64, 64, True), (64, 128, False)]),  # three layers, the pooled one in the middle
+    (2, 9, [(16, 24, True)]),                                      # a single layer outside every matrix-core kernel
+])
+def test_qconv_chain_small(ops, N, H, shapes):
+    """sofie_hip_qconv2d_s8_chain on batches where the layers run one after the other: every layer's output equals the
+    oracle's, scales of both signs."""
+    r = rng(900 + N + H)
+    x = r.integers(-128, 128, (N, shapes[0][0], H, H)).astype(np.int8)
+    layers, host = _chain_layers(r, shapes, signs=True)
+    got = ops.qconv2d_s8_chain(np.ascontiguousarray(x.transpose(0, 2, 3, 1)), layers)
+    for y, ref in zip(got, _chain_reference(x, host)):
+        assert np.array_equal(y.transpose(0, 3, 1, 2), ref)
+
+
+def test_qconv_chain_two_layers_in_one_launch(ops):
+    """Batch 4096 of 20x20 images, conv 32 -> 64 + ReLU + 2x2 pooling, conv 64 -> 128 + ReLU: every workgroup owns 16
+    whole images in both layers, so the chain is one launch in which a workgroup reads back what it wrote. Both outputs
+    equal those of the two separate calls byte for byte, and 64 images spread over the batch equal the oracle."""
+    from sofie_amd import lib as L
+    r = rng(77)
+    N = 4096
+    x = r.integers(-128, 128, (N, 20, 20, 32)).astype(np.int8)
+    layers, host = _chain_layers(r, [(32, 64, True), (64, 128, False)])
+    ctx = ops.default_context()
+    buf = __import__("ctypes").create_string_buffer(1024)
+    n = __import__("ctypes").c_int(0)
+    assert ctx.lib.sofie_hip_trace_begin(ctx.h) == 0
+    p2, c3 = ops.qconv2d_s8_chain(x, layers)
+    assert ctx.lib.sofie_hip_trace_end(ctx.h, buf, 1024, __import__("ctypes").byref(n)) == 0
+    assert n.value == 1 and buf.value.decode().split()[0] == "k_qconv_ring_pair"       # one launch for both layers
+    a, b = layers
+    s2 = ops.qconv2d_pool_s8(x, a["w"], a["scale"], a["bias"], (1, 1), (1, 1), 1, -128, -128, True, x_layout=L.LAYOUT_NHWC,
+                             y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+    s3 = ops.qconv2d_s8(s2, b["w"], b["scale"], b["bias"], (1, 1), (1, 1), 1, -128, -128, True, x_layout=L.LAYOUT_NHWC,
+                        y_layout=L.LAYOUT_NHWC, w_layout=L.LAYOUT_NHWC)
+    assert np.array_equal(p2, s2) and np.array_equal(c3, s3)
+    pick = np.arange(0, N, 64) + (np.arange(64) % 16)            # every position inside a workgroup's 16 images
+    ref2, ref3 = _chain_reference(np.ascontiguousarray(x[pick].transpose(0, 3, 1, 2)), host)
+    assert np.array_equal(p2[pick].transpose(0, 3, 1, 2), ref2)
+    assert np.array_equal(c3[pick].transpose(0, 3, 1, 2), ref3)
+    # a second call right behind the first (the tensors of the first are rewritten): the same bytes
+    p2b, c3b = ops.qconv2d_s8_chain(x, layers)
+    assert np.array_equal(p2b, p2) and np.array_equal(c3b, c3)
+
+
 def test_empty_and_degenerate_inputs(ops):
     """Zero-sized problems return success without touching the output; K = 0 leaves the bias (the accumulators are an
     empty sum); a 1x1 image, a single row and a single column go through the general kernels."""
