@@ -325,6 +325,12 @@ __global__ void __launch_bounds__(256, (TI * TJ >= 16 || NSETS > 2) ? 1 : 2) k_g
 #ifndef SOFIE_GEMM16
 #define SOFIE_GEMM16 1
 #endif
+// Ablation builds of k_gemm_dma16 for timing only (make ABLATE=...; the results are wrong by construction): bit 0 leaves
+// out the LDS-DMA requests after the first two K-steps, bit 1 the fragment reads after the first K-step, bit 2 the matrix
+// instructions. Waits, barriers, prologue and epilogue stay. 0 in the library that is shipped.
+#ifndef SOFIE_GEMM_ABLATE
+#define SOFIE_GEMM_ABLATE 0
+#endif
 template <int S> struct StageTag { static constexpr int value = S; };
 
 // LDS of k_gemm_dma: [A stage 0][A stage 1][B stage 0][B stage 1], BM*BK (BN*BK) bytes each. Both stages of an
@@ -780,29 +786,44 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
    }
    barrier();
    if (group == 1) barrier();
+   constexpr bool NO_REQUESTS = (SOFIE_GEMM_ABLATE & 1) != 0, NO_READS = (SOFIE_GEMM_ABLATE & 2) != 0,
+                  NO_MFMA = (SOFIE_GEMM_ABLATE & 4) != 0;
+   v4i fn[NSUB][NI], fm[NSUB][MJ];          // (inside a K-step in effect: every step rewrites all of them)
    auto kstep = [&](int t, auto tag) {
       constexpr int S = decltype(tag)::value;
-      if (t > 0) request(t + 1, 1 - S);
-      v4i fn[NSUB][NI], fm[NSUB][MJ];
+      if (t > 0 && !NO_REQUESTS) request(t + 1, 1 - S);
+      if (!NO_READS || t == 0) {
 #pragma unroll
-      for (int sub = 0; sub < NSUB; ++sub) {
+         for (int sub = 0; sub < NSUB; ++sub) {
 #pragma unroll
-         for (int i = 0; i < NI; ++i) {
-            if constexpr (B_KN) fn[sub][i] = load_frag_kn(i, S * BBYTES, sub);
-            else fn[sub][i] = *reinterpret_cast<const v4i *>(n_base[sub] + i * 16 * BK + S * BBYTES);
+            for (int i = 0; i < NI; ++i) {
+               if constexpr (B_KN) fn[sub][i] = load_frag_kn(i, S * BBYTES, sub);
+               else fn[sub][i] = *reinterpret_cast<const v4i *>(n_base[sub] + i * 16 * BK + S * BBYTES);
+            }
+#pragma unroll
+            for (int j = 0; j < MJ; ++j) fm[sub][j] = *reinterpret_cast<const v4i *>(m_base[sub] + j * 16 * BK + S * ABYTES);
          }
-#pragma unroll
-         for (int j = 0; j < MJ; ++j) fm[sub][j] = *reinterpret_cast<const v4i *>(m_base[sub] + j * 16 * BK + S * ABYTES);
       }
       __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
       if (group == 1) wait_vmcnt<0>();
       barrier();
+      if constexpr (NO_MFMA) {
+         // the fragments stay "used", so that their reads are not removed with the instructions that consume them
 #pragma unroll
-      for (int sub = 0; sub < NSUB; ++sub)
+         for (int sub = 0; sub < NSUB; ++sub) {
 #pragma unroll
-         for (int i = 0; i < NI; ++i)
+            for (int i = 0; i < NI; ++i) asm volatile("" ::"v"(fn[sub][i]));
 #pragma unroll
-            for (int j = 0; j < MJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fn[sub][i], fm[sub][j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < MJ; ++j) asm volatile("" ::"v"(fm[sub][j]));
+         }
+      } else {
+#pragma unroll
+         for (int sub = 0; sub < NSUB; ++sub)
+#pragma unroll
+            for (int i = 0; i < NI; ++i)
+#pragma unroll
+               for (int j = 0; j < MJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fn[sub][i], fm[sub][j], acc[i][j], 0, 0, 0);
+      }
       if (group == 0) wait_vmcnt<0>();
       if (group == 0 || t + 1 < nk) barrier();
    };
