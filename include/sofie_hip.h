@@ -297,8 +297,11 @@ int sofie_hip_qgemm_s8_pair(sofie_hip_ctx *ctx, int M, int K, const int8_t *A, i
  * SOFIE_HIP_NOALLOC_SCRATCH_BYTES that the library holds on every GPU it runs on until the process ends; a shape
  * that needs more returns SOFIE_HIP_EINVAL with a message and launches nothing (splits * M * round_up(N, 4) * 4
  * bytes for the K slices, at most 16 slices; N * K bytes for the copy). All calls on one GPU share that array:
- * two such calls that overlap in time on one GPU (two contexts, two threads) race; calls on one context's stream
- * are ordered. Nothing in the array has to start at zero: every word whose value is used has been written by the same call. */
+ * the library lets them use it in turns (each call's kernels wait, on the device, for an event recorded behind the
+ * kernels of the call before it, whatever context, stream or thread that call came from), so calls from several
+ * contexts give the right results and run one after the other. Only calls recorded into a HIP graph are outside
+ * that order: a recorded call must not overlap with other no-allocation calls on the same GPU. Nothing in the array
+ * has to start at zero: every word whose value is used has been written by the same call. */
 #define SOFIE_HIP_NOALLOC_SCRATCH_BYTES (32u << 20)
 int sofie_hip_qgemm_s8_noalloc(sofie_hip_ctx *ctx, int transB, int M, int N, int K, const int8_t *A,
                                int lda, const int8_t *B, int ldb, const float *scale,

@@ -37,6 +37,10 @@ int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...);
 // Grow-only scratch buffer of the context. Never shrinks; freed in sofie_hip_destroy.
 int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr);
 int check_launch(sofie_hip_ctx *ctx, const char *what);
+// Bracket of a call that uses the device's fixed scratch array (sofie_hip_qgemm_s8_noalloc): orders it behind the call
+// that used the array before it, on whatever context and stream that was.
+void scratch_turn_begin(sofie_hip_ctx *ctx);
+void scratch_turn_end(sofie_hip_ctx *ctx);
 
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));

@@ -1389,9 +1389,12 @@ int sofie_hip_qgemm_s8_noalloc(sofie_hip_ctx *ctx, int transB, int M, int N, int
    // Same kernels and the same choice among them as sofie_hip_qgemm_s8; the two paths that need memory beyond the
    // operands (partial sums of a K cut into slices, the transposed copy of a B [K,N] whose rows are not 16-byte
    // aligned) take it from the fixed array instead of the context's growable buffer.
+   // Every context of a device shares the one array: the call takes its turn behind the one that used it last.
+   scratch_turn_begin(ctx);
    ctx->no_alloc = true;
    const int rc = sofie_hip_qgemm_s8(ctx, transB, M, N, K, A, lda, B, ldb, scale, bias, zp_y, act, Y, ldy, out_kind);
    ctx->no_alloc = false;
+   scratch_turn_end(ctx);
    return rc;
 }
 

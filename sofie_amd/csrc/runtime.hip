@@ -16,6 +16,10 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 void *g_scratch_addr[kMaxDevices] = {};
+// One event per device, made with the array's address (so nothing is created at call time): recorded behind the last
+// kernel of every no-allocation call and waited for in front of the first kernel of the next one, whatever context
+// and stream that call runs on. Calls from different contexts then use the array one after the other.
+hipEvent_t g_scratch_free[kMaxDevices] = {};
 
 // With `device` current: the address of this device's copy of `scratch` (looked up at the first call).
 hipError_t scratch_address(int device, void **addr)
@@ -28,6 +32,10 @@ hipError_t scratch_address(int device, void **addr)
       hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
       if (e != hipSuccess) return e;
       g_scratch_addr[device] = p;
+      if (hipEventCreateWithFlags(&g_scratch_free[device], hipEventDisableTiming) != hipSuccess) {
+         (void)hipGetLastError();
+         g_scratch_free[device] = nullptr;
+      }
    }
    *addr = g_scratch_addr[device];
    return hipSuccess;
@@ -67,6 +75,24 @@ void raise_lds_limits(int device)
 }  // namespace
 
 namespace sofie {
+
+// Around the kernels of a no-allocation call: the stream waits for the event of the call that used the array last, and
+// records it again behind its own kernels. Both under the lock, so that two threads' calls take turns in one order.
+// (Not while the stream is being captured: an event of another stream has no place in the recording; a recorded
+// no-allocation call is ordered only against the calls of its own stream.)
+void scratch_turn_begin(sofie_hip_ctx *ctx)
+{
+   g_scratch_mutex.lock();
+   hipEvent_t ev = (ctx->device >= 0 && ctx->device < kMaxDevices) ? g_scratch_free[ctx->device] : nullptr;
+   if (ev && !ctx->capturing && hipStreamWaitEvent(ctx->stream, ev, 0) != hipSuccess) (void)hipGetLastError();
+}
+
+void scratch_turn_end(sofie_hip_ctx *ctx)
+{
+   hipEvent_t ev = (ctx->device >= 0 && ctx->device < kMaxDevices) ? g_scratch_free[ctx->device] : nullptr;
+   if (ev && !ctx->capturing && hipEventRecord(ev, ctx->stream) != hipSuccess) (void)hipGetLastError();
+   g_scratch_mutex.unlock();
+}
 
 void list_large_lds_kernel(const void *func)
 {

@@ -61,6 +61,64 @@ def test_noalloc_entry_point_matches_the_allocating_one():
     ctx.close()
 
 
+def test_noalloc_first_on_a_fresh_context_allocates_nothing():
+    """On a context that has made no call yet (its own scratch buffer does not exist), the no-allocation entry point
+    runs the shapes that need scratch memory with the device's free memory unchanged across the call, and its results
+    equal the oracle's: the large B [K,N] cases on sampled rows, the K-slice case in full."""
+    from sofie_amd import lib as L
+    from sofie_amd import ops as o
+    r = np.random.default_rng(9)
+    for M, N, K, tB in ((4096, 2052, 1024, False), (2100, 4100, 528, False), (256, 256, 16384, True)):
+        print("[noalloc fresh] M=%d N=%d K=%d transB=%d" % (M, N, K, tB), flush=True)
+        ctx = o.Context(0)
+        lib, h, p = ctx.lib, ctx.h, ctx.ptr
+        A = r.integers(-127, 128, (M, K)).astype(np.int8)
+        B = r.integers(-127, 128, (N, K) if tB else (K, N)).astype(np.int8)
+        dA, dB = ctx.dev(A), ctx.dev(B)
+        y = ctx.empty((M, N), torch.int32)
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        ctx.check(lib.sofie_hip_qgemm_s8_noalloc(h, int(tB), M, N, K, p(dA), K, p(dB), B.shape[1], None, None, 0, L.ACT_NONE,
+                                                 p(y), N, L.OUT_S32))
+        ctx.sync()
+        assert torch.cuda.mem_get_info()[0] == free0
+        got = y.cpu().numpy()
+        rows = np.arange(M) if M * N * K <= 1 << 30 else np.sort(r.choice(M, 48, replace=False))
+        assert np.array_equal(got[rows], oracle.igemm_s8(A[rows], B, transB=tB))
+        # the allocating entry point on the same context afterwards: the same bytes
+        y2 = ctx.empty((M, N), torch.int32)
+        ctx.check(lib.sofie_hip_qgemm_s8(h, int(tB), M, N, K, p(dA), K, p(dB), B.shape[1], None, None, 0, L.ACT_NONE, p(y2), N, L.OUT_S32))
+        ctx.sync()
+        assert np.array_equal(y2.cpu().numpy(), got)
+        ctx.close()
+
+
+def test_noalloc_calls_from_two_contexts_take_turns():
+    """Two contexts (two streams) whose no-allocation calls both use the device's one scratch array, enqueued back to
+    back without a wait in between: the library orders them on the device, so each result equals the one the same
+    context computes alone."""
+    from sofie_amd import lib as L
+    from sofie_amd import ops as o
+    r = np.random.default_rng(10)
+    M, N, K = 256, 256, 16384                       # K cut into slices: partial sums in the array
+    ctxs = [o.Context(0, stream=torch.cuda.Stream()) for _ in range(2)]
+    ops_ = []
+    for c in ctxs:
+        A = r.integers(-127, 128, (M, K)).astype(np.int8)
+        B = r.integers(-127, 128, (N, K)).astype(np.int8)
+        ops_.append((c.dev(A), c.dev(B), c.empty((M, N), torch.int32), A, B))
+    torch.cuda.synchronize()
+    for rep in range(6):
+        for c, (dA, dB, y, _, _) in zip(ctxs, ops_):
+            c.check(c.lib.sofie_hip_qgemm_s8_noalloc(c.h, 1, M, N, K, c.ptr(dA), K, c.ptr(dB), K, None, None, 0, L.ACT_NONE,
+                                                     c.ptr(y), N, L.OUT_S32))
+    for c in ctxs:
+        c.sync()
+    for c, (dA, dB, y, A, B) in zip(ctxs, ops_):
+        assert np.array_equal(y.cpu().numpy(), oracle.igemm_s8(A, B, transB=True))
+        c.close()
+
+
 def test_noalloc_entry_point_rejects_what_does_not_fit():
     """A transposed copy of 33.7 MB does not fit the 32 MiB array: EINVAL with a message, nothing launched, nothing allocated."""
     from sofie_amd import lib as L
