@@ -427,6 +427,55 @@ __device__ __forceinline__ void tile_epilogue_wave16(const GemmArgs &g, v4i (&ac
    }
 }
 
+// The int8 epilogue of 16 x 16 accumulator tiles without LDS staging, for wavefront tiles whose columns all lie inside
+// the matrix and rows that take 16-byte stores. A lane holds columns (lane / 16) * 4 .. + 3 of each 16-column tile of
+// its row: packed, the dwords of four neighbouring tiles are a 4 x 4 matrix over the row's four lanes (16 lanes
+// apart), and two rounds of swaps (between the halves of the wavefront, then between neighbouring groups of 16 lanes)
+// transpose it. Lane group kg then has the 16 columns of tile kg in order, and a store instruction writes 64
+// contiguous bytes for each of 16 rows (written through the L2).
+template <int NI, int MJ, int PLAIN>
+__device__ __forceinline__ void tile_epilogue_wave16_direct(const GemmArgs &g, v4i (&acc)[NI][MJ], const float *s_scale,
+                                                            const int *s_bias, int lane, int m_wave, int n_wave)
+{
+   static_assert(NI % 4 == 0, "groups of four column tiles");
+   const int l16 = lane & 15, kg = lane >> 4;
+   const float zpo = (float)(g.zp + 128), lof = (float)(g.lo + 128);
+#pragma unroll
+   for (int ig = 0; ig < NI; ig += 4) {
+      v4f sc[4];
+      v4i bi[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+         sc[i] = *reinterpret_cast<const v4f *>(s_scale + (ig + i) * 16 + kg * 4);
+         bi[i] = *reinterpret_cast<const v4i *>(s_bias + (ig + i) * 16 + kg * 4);
+      }
+#pragma unroll
+      for (int j = 0; j < MJ; ++j) {
+         const int m = m_wave + j * 16 + l16;
+         int8_t *const row = static_cast<int8_t *>(g.Y) + (size_t)(m < g.M ? m : 0) * g.ldy + n_wave + ig * 16 + kg * 16;
+         unsigned d[4];
+#pragma unroll
+         for (int i = 0; i < 4; ++i) {
+            unsigned pk = 0;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+               float r = __fmul_rn(__int2float_rn(acc[ig + i][j][t] + bi[i][t]), sc[i][t]);
+               if constexpr (PLAIN == 0) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
+               if constexpr (PLAIN == 2) r = __fadd_rn(rintf(r), zpo);
+               pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);     // rounds half to even, saturates at 0 and 255
+            }
+            d[i] = pk ^ 0x80808080u;
+         }
+         const auto s02 = __builtin_amdgcn_permlane32_swap(d[0], d[2], false, false);
+         const auto s13 = __builtin_amdgcn_permlane32_swap(d[1], d[3], false, false);
+         const auto t01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+         const auto t23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+         const v4i v = {(int)t01[0], (int)t01[1], (int)t23[0], (int)t23[1]};
+         if (m < g.M) store16_wt(row, v);
+      }
+   }
+}
+
 // ---- global memory -> LDS without registers (buffer_load ... lds), shared by the GEMM and the convolution
 typedef int rsrc_t __attribute__((ext_vector_type(4)));
 
