@@ -20,7 +20,7 @@ using namespace sofie;
 namespace {
 
 // Most values of a channel block that the threads of a workgroup carry in registers in k_conv2d_f32_pipe.
-#define SOFIE_CONV_PIPE_PATCH 1536
+#define SOFIE_CONV_PIPE_PATCH 1792
 #define SOFIE_CONV_PIPE_WEIGHTS 5120
 
 // Geometry of one output phase of a strided transposed convolution when all phases run in one launch.
@@ -357,35 +357,41 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
    const float *wg = g.w + (size_t)grp * g.ocg * Kfull;
    const int K4 = g.KC >> 2;
 
-   // a thread's share of one channel block, in registers between issue() and commit()
+   // A thread's share of one channel block, in registers between issue() and commit(). Where a value comes from and
+   // where it goes does not depend on the block (every block is full: the launchers see to it), so the offsets are
+   // worked out once: pofs[u] = offset of patch cell u*256+tid inside the block's input channels (-1: padding, or past
+   // the patch), wofs[u] = offset of four consecutive k of one output channel in the block's weights (-1: past the
+   // output channels), wlds[u] = where they go in the LDS weight tile (-1: nothing to write).
    float pv[NP], wreg[NW];
-   unsigned pmask = 0, wmask = 0;
-   auto issue = [&](int ic0) {
-      const int icn = (g.icg - ic0) < g.ICB ? (g.icg - ic0) : g.ICB;
-      pmask = 0;
-      wmask = 0;
+   int pofs[NP], wofs[NW / 4], wlds[NW / 4];
 #pragma unroll
-      for (int u = 0; u < NP; ++u) {
-         const int e = u * 256 + tid;
-         const int t = fdiv(e, g.dPW), c = e - t * g.PW;
-         const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
-         const int ih = ih0 + r, iw = iw0 + c;
-         const bool inside = e < patch_len && icl < icn && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
-         // loads are unconditional (of element 0 where the cell is padding or past the block)
-         pv[u] = xg[inside ? ((size_t)(ic0 + icl) * g.H + ih) * g.W + iw : 0];
-         pmask |= inside ? (1u << u) : 0u;
-      }
-      // weights: four consecutive k of one output channel per 16-byte load (the launcher guarantees full,
-      // 16-byte aligned blocks)
+   for (int u = 0; u < NP; ++u) {
+      const int e = u * 256 + tid;
+      const int t = fdiv(e, g.dPW), c = e - t * g.PW;
+      const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
+      const int ih = ih0 + r, iw = iw0 + c;
+      const bool inside = e < patch_len && icl < g.ICB && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+      pofs[u] = inside ? (icl * g.H + ih) * g.W + iw : -1;
+   }
+#pragma unroll
+   for (int u = 0; u < NW / 4; ++u) {
+      const int e = u * 256 + tid;
+      const int ocl = fdiv(e, g.dK4), k4 = e - ocl * K4;
+      wofs[u] = (e < K4 * BOC && oc0 + ocl < g.ocg) ? (oc0 + ocl) * Kfull + 4 * k4 : -1;
+      wlds[u] = e < K4 * BOC ? 4 * k4 * LDW + ocl : -1;
+   }
+   const size_t HW = (size_t)g.H * g.W;
+   auto issue = [&](int ic0) {
+      // loads are unconditional (of the block's first element where there is nothing to load)
+      const float *const xb = xg + (size_t)ic0 * HW;
+      const float *const wb = wg + (size_t)ic0 * KHW;
+#pragma unroll
+      for (int u = 0; u < NP; ++u) pv[u] = xb[pofs[u] < 0 ? 0 : pofs[u]];
 #pragma unroll
       for (int u = 0; u < NW / 4; ++u) {
-         const int e = u * 256 + tid;
-         const int ocl = fdiv(e, g.dK4), k4 = e - ocl * K4;
-         const bool ok = e < K4 * BOC && oc0 + ocl < g.ocg;
-         const v4f v = *reinterpret_cast<const v4f *>(wg + (ok ? (size_t)(oc0 + ocl) * Kfull + (size_t)ic0 * KHW + 4 * k4 : 0));
+         const v4f v = *reinterpret_cast<const v4f *>(wb + (wofs[u] < 0 ? 0 : wofs[u]));
 #pragma unroll
          for (int q = 0; q < 4; ++q) wreg[4 * u + q] = v[q];
-         wmask |= ok ? (1u << u) : 0u;
       }
    };
    auto commit = [&](float *buf) {
@@ -393,18 +399,14 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
 #pragma unroll
       for (int u = 0; u < NP; ++u) {
          const int e = u * 256 + tid;
-         if (e < patch_len) patch[e] = ((pmask >> u) & 1u) ? pv[u] : 0.0f;
+         if (e < patch_len) patch[e] = pofs[u] < 0 ? 0.0f : pv[u];
       }
 #pragma unroll
-      for (int u = 0; u < NW / 4; ++u) {
-         const int e = u * 256 + tid;
-         const int ocl = fdiv(e, g.dK4), k4 = e - ocl * K4;
-         if (e < K4 * BOC) {
-            const bool ok = (wmask >> u) & 1u;
+      for (int u = 0; u < NW / 4; ++u)
+         if (wlds[u] >= 0) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) sW[(4 * k4 + q) * LDW + ocl] = ok ? wreg[4 * u + q] : 0.0f;
+            for (int q = 0; q < 4; ++q) sW[wlds[u] + q * LDW] = wofs[u] < 0 ? 0.0f : wreg[4 * u + q];
          }
-      }
    };
 
    const int nblocks = (g.icg + g.ICB - 1) / g.ICB;
@@ -437,6 +439,16 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
 
    const size_t plane = PHASES ? (size_t)gg.OH0 * gg.OW0 : (size_t)OHW;
    float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane;
+   // the biases of this lane's output channels, all loaded before the first store (a load behind a store that may
+   // alias it would wait for its own turn, 16 * TI * TJ times)
+   float bv[TI][16];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+         const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
+         bv[i][r] = (g.bias && oc < g.ocg) ? g.bias[grp * g.ocg + oc] : 0.0f;
+      }
 #pragma unroll
    for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -452,8 +464,7 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
          for (int r = 0; r < 16; ++r) {
             const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
             if (oc >= g.ocg) continue;
-            float v = acc[i][j][r];
-            if (g.bias) v = __fadd_rn(v, g.bias[grp * g.ocg + oc]);
+            float v = __fadd_rn(acc[i][j][r], bv[i][r]);
             if (g.relu) v = v > 0.0f ? v : 0.0f;
             yn[(size_t)oc * plane + po] = v;
          }
