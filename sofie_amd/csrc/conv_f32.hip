@@ -14,6 +14,7 @@
 #include <type_traits>
 
 #include "common.h"
+#include "gemm_tile.h"
 
 using namespace sofie;
 
@@ -22,6 +23,8 @@ namespace {
 // Most values of a channel block that the threads of a workgroup carry in registers in k_conv2d_f32_pipe.
 #define SOFIE_CONV_PIPE_PATCH 1792
 #define SOFIE_CONV_PIPE_WEIGHTS 5120
+// Most patch cells of a channel block in k_conv2d_f32_dma (a thread keeps an offset per 256 cells).
+#define SOFIE_CONV_DMA_PATCH 3584
 
 // Geometry of one output phase of a strided transposed convolution when all phases run in one launch.
 struct PhaseArgs {
@@ -356,6 +359,9 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
    const float *xg = g.x + ((size_t)n * g.C + (size_t)grp * g.icg) * g.H * g.W;
    const float *wg = g.w + (size_t)grp * g.ocg * Kfull;
    const int K4 = g.KC >> 2;
+   // a wavefront whose pixels all lie behind the end of the plane multiplies nothing (a 28x28 plane is 6 tiles of 128
+   // pixels and one of 16); it still stages its share of every block
+   const int nsteps = p0 + __builtin_amdgcn_readfirstlane(wn) * TJ * 32 < OHW ? g.KC / 2 : 0;
 
    // A thread's share of one channel block, in registers between issue() and commit(). Where a value comes from and
    // where it goes does not depend on the block (every block is full: the launchers see to it), so the offsets are
@@ -418,7 +424,7 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
       if (more) issue((c + 1) * g.ICB);
       const float *const sW = bufs + (c & 1) * buf_len, *const patch = sW + g.KC * LDW;
       const float *wrow = sW + wm * TI * 32 + fr;
-      for (int s = 0; s < g.KC / 2; ++s) {
+      for (int s = 0; s < nsteps; ++s) {
          const int kk = 2 * s + fk;
          const int ko = koff[kk];
          float fa[TI], fb[TJ];
@@ -471,10 +477,200 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
       }
 }
 
+// The same implicit GEMM with both operands of channel block c+1 travelling global memory -> LDS without registers
+// (buffer_load ... lds) under the matrix loop of block c. The weights come from a copy laid out for it, wt [group]
+// [K = input channel, tap][wstride >= OC/groups, a multiple of 4] (k_transpose_weights / k_gather_phase_weights write it
+// into the scratch buffer in front of the launch), so that a row of the LDS tile [KC][BOC] is a contiguous piece of a
+// row of wt and goes 16 bytes per lane; odd rows are rotated by 32 columns, which puts the two K halves of a fragment
+// read on different banks without padding. A patch cell is 4 bytes per lane from wherever it sits in the image;
+// padding cells ask for an offset outside the descriptor's range and receive 0. Nothing of a block depends on the
+// block but a uniform offset, so a thread keeps NP patch offsets and one weight offset for the whole kernel.
+// PHASES as in k_conv2d_f32_pipe.
+template <int TI, int TJ, bool PHASES = false>
+__global__ void __launch_bounds__(256, 3) k_conv2d_f32_dma(ConvArgs gg)
+{
+   constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32;
+   constexpr int NP = SOFIE_CONV_DMA_PATCH / 256;
+   constexpr int ROWS_PER_REQUEST = 1024 / BOC;       // weight rows one request of 256 lanes x 16 bytes covers
+   constexpr unsigned OUTSIDE = 0x40000000u;          // an offset no descriptor of this kernel reaches
+   struct Geometry {
+      const float *x, *w, *bias;
+      float *y;
+      int C, H, W, OC, KH, KW, ph, pw, sh, sw, dh, dw, OH, OW, icg, ocg, ICB, KC, PH, PW, relu;
+      FastDiv dPW, dPH;
+   } g;
+   g.x = gg.x; g.w = gg.w; g.bias = gg.bias; g.y = gg.y;
+   g.C = gg.C; g.H = gg.H; g.W = gg.W; g.OC = gg.OC; g.KH = gg.KH; g.KW = gg.KW; g.ph = gg.ph; g.pw = gg.pw;
+   g.sh = gg.sh; g.sw = gg.sw; g.dh = gg.dh; g.dw = gg.dw; g.OH = gg.OH; g.OW = gg.OW; g.icg = gg.icg; g.ocg = gg.ocg;
+   g.ICB = gg.ICB; g.KC = gg.KC; g.PH = gg.PH; g.PW = gg.PW; g.relu = gg.relu;
+   g.dPW = gg.dPW; g.dPH = gg.dPH;
+   int n = blockIdx.z;
+   int oy0 = 0, ox0 = 0;
+   FastDiv dOW = gg.dOW;
+   if constexpr (PHASES) {
+      const int pi = blockIdx.z % gg.nphases;
+      n = blockIdx.z / gg.nphases;
+      PhaseArgs q = gg.phase[0];
+#pragma unroll
+      for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
+         if (pi == i) q = gg.phase[i];
+      if ((int)blockIdx.x * BP >= q.OH * q.OW) return;   // the grid is as wide as the phase with most pixel tiles
+      g.KH = q.KH; g.KW = q.KW; g.ph = q.ph; g.pw = q.pw; g.OH = q.OH; g.OW = q.OW; g.ICB = q.ICB; g.KC = q.KC;
+      g.PH = q.PH; g.PW = q.PW; g.dPW = q.dPW; g.dPH = q.dPH;
+      g.w = gg.w + q.woff;
+      oy0 = q.oy0; ox0 = q.ox0; dOW = q.dOW;
+   }
+   extern __shared__ __align__(16) unsigned char smem_raw[];
+   const int patch_len = g.ICB * g.PH * g.PW;
+   const int patch_room = (patch_len + 255) & ~255;                  // requests write whole groups of 256 cells
+   const int buf_len = g.KC * BOC + patch_room;                      // floats of one buffer: [KC][BOC] weights, patch
+   float *const bufs = reinterpret_cast<float *>(smem_raw);
+   int *const koff = reinterpret_cast<int *>(bufs + 2 * buf_len);    // [KC]
+
+   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+   const int wm = wave >> 1, wn = wave & 1;
+   const int fr = lane & 31, fk = lane >> 5;
+   const int octiles = (g.ocg + BOC - 1) / BOC;
+   const int grp = blockIdx.y / octiles;
+   const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
+   const int OHW = g.OH * g.OW;
+   const int p0 = blockIdx.x * BP;
+   const int oh0 = p0 / g.OW;
+   const int ih0 = oh0 * g.sh - g.ph, iw0 = -g.pw;
+   const int KHW = g.KH * g.KW;
+   const int Kfull = g.icg * KHW;
+   const int wstride = (g.ocg + 3) & ~3;
+   const size_t HW = (size_t)g.H * g.W;
+
+   for (int k = tid; k < g.KC; k += 256) {
+      const int icl = k / KHW, t = k % KHW;
+      const int kh = t / g.KW, kw = t % g.KW;
+      koff[k] = (icl * g.PH + kh * g.dh) * g.PW + kw * g.dw;
+   }
+   int base[TJ];
+#pragma unroll
+   for (int j = 0; j < TJ; ++j) {
+      const int p = p0 + wn * TJ * 32 + j * 32 + fr;
+      base[j] = (p < OHW) ? ((p / g.OW - oh0) * g.sh) * g.PW + (p % g.OW) * g.sw : 0;
+   }
+   v16f acc[TI][TJ];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j)
+#pragma unroll
+         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+   // descriptors: this image's channels of the group, this group's weights (the launcher keeps both under 1 GiB)
+   const rsrc_t xrs = make_rsrc(g.x + ((size_t)n * g.C + (size_t)grp * g.icg) * HW, (unsigned)((size_t)g.icg * HW * 4));
+   const rsrc_t wrs = make_rsrc(g.w + (size_t)grp * Kfull * wstride, (unsigned)((size_t)Kfull * wstride * 4));
+   // byte offsets of this thread's patch cells inside a block's channels, and of its 16 bytes of weight row tid /
+   // (BOC/4) (the rows of its later requests are ROWS_PER_REQUEST further each: same parity, same rotation)
+   unsigned pofs[NP];
+#pragma unroll
+   for (int u = 0; u < NP; ++u) {
+      const int e = u * 256 + tid;
+      const int t = fdiv(e, g.dPW), c = e - t * g.PW;
+      const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
+      const int ih = ih0 + r, iw = iw0 + c;
+      const bool inside = e < patch_len && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+      pofs[u] = inside ? (unsigned)(((icl * g.H + ih) * g.W + iw) * 4) : OUTSIDE;
+   }
+   const int wrow0 = tid / (BOC / 4);
+   const int wcol = ((tid % (BOC / 4)) * 4 - 32 * (wrow0 & 1)) & (BOC - 1);     // column the rotated cell holds
+   const unsigned wofs = oc0 + wcol < wstride ? (unsigned)((wrow0 * wstride + oc0 + wcol) * 4) : OUTSIDE;
+   const int npatch = (patch_len + 255) >> 8;        // patch requests per thread (of NP)
+   const unsigned xblock = (unsigned)(g.ICB * HW * 4), wblock = (unsigned)(g.KC * wstride * 4);
+   const unsigned wstep = (unsigned)(ROWS_PER_REQUEST * wstride * 4);
+   const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;   // LDS byte address of the buffers
+
+   auto request = [&](int c, int buf) {
+      const unsigned sw = lds0 + (unsigned)buf * buf_len * 4, sp = sw + (unsigned)g.KC * BOC * 4;
+#pragma unroll
+      for (int u = 0; u < NP; ++u)
+         if (u < npatch) dma4(xrs, sp + (u * 256 + wave * 64) * 4, (int)pofs[u], (int)(c * xblock));
+      for (int r0 = 0; r0 < g.KC; r0 += ROWS_PER_REQUEST)
+         if (r0 + wrow0 < g.KC)
+            dma16(wrs, sw + (r0 * BOC + wave * 256) * 4, (int)wofs, (int)(c * wblock + (r0 / ROWS_PER_REQUEST) * wstep));
+   };
+
+   const int nblocks = g.icg / g.ICB;
+   const int nsteps = p0 + wn * TJ * 32 < OHW ? g.KC / 2 : 0;   // a wavefront with no pixel of the plane multiplies nothing
+   int wcolr[TI];     // this lane's column of the weight tile, rotated as the rows of its K half (odd: fk = 1) are
+#pragma unroll
+   for (int i = 0; i < TI; ++i) wcolr[i] = (wm * TI * 32 + i * 32 + fr + 32 * fk) & (BOC - 1);
+   request(0, 0);
+   wait_vmcnt<0>();
+   __syncthreads();   // block 0 and the koff table are in LDS
+   for (int c = 0; c < nblocks; ++c) {
+      if (c + 1 < nblocks) request(c + 1, (c + 1) & 1);
+      const float *const sW = bufs + (c & 1) * buf_len, *const patch = sW + g.KC * BOC;
+      for (int s = 0; s < nsteps; ++s) {
+         const int kk = 2 * s + fk;
+         const int ko = koff[kk];
+         float fa[TI], fb[TJ];
+#pragma unroll
+         for (int i = 0; i < TI; ++i) fa[i] = sW[kk * BOC + wcolr[i]];
+#pragma unroll
+         for (int j = 0; j < TJ; ++j) fb[j] = patch[base[j] + ko];
+#pragma unroll
+         for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      }
+      // the next block has landed (this wavefront's requests; the barrier makes it every wavefront's), and the
+      // buffer it replaces next was last read in this block
+      wait_vmcnt<0>();
+      __syncthreads();
+   }
+
+   const size_t plane = PHASES ? (size_t)gg.OH0 * gg.OW0 : (size_t)OHW;
+   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane;
+   float bv[TI][16];
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+         const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
+         bv[i][r] = (g.bias && oc < g.ocg) ? g.bias[grp * g.ocg + oc] : 0.0f;
+      }
+#pragma unroll
+   for (int i = 0; i < TI; ++i)
+#pragma unroll
+      for (int j = 0; j < TJ; ++j) {
+         const int p = p0 + wn * TJ * 32 + j * 32 + fr;
+         if (p >= OHW) continue;
+         size_t po = (size_t)p;
+         if constexpr (PHASES) {
+            const int row = fdiv(p, dOW);
+            po = (size_t)(oy0 + row * gg.oys) * gg.OW0 + ox0 + (p - row * g.OW) * gg.oxs;
+         }
+#pragma unroll
+         for (int r = 0; r < 16; ++r) {
+            const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
+            if (oc >= g.ocg) continue;
+            float v = __fadd_rn(acc[i][j][r], bv[i][r]);
+            if (g.relu) v = v > 0.0f ? v : 0.0f;
+            yn[(size_t)oc * plane + po] = v;
+         }
+      }
+}
+
+// Weights of a plain convolution w [OC][C/groups][KH][KW] as k_conv2d_f32_dma reads them: wt [group][K][wstride],
+// K = (input channel, tap), wstride = OC/groups rounded up to 4 (the cells behind the last channel are 0).
+__global__ void k_transpose_weights(const float *w, float *wt, int groups, int ocg, int Kfull, int wstride)
+{
+   const int e = blockIdx.x * blockDim.x + threadIdx.x;
+   if (e >= groups * Kfull * wstride) return;
+   const int oc = e % wstride, k = (e / wstride) % Kfull, grp = e / (wstride * Kfull);
+   wt[e] = oc < ocg ? w[((size_t)grp * ocg + oc) * Kfull + k] : 0.0f;
+}
+
 // Sub-kernels of the output phases of a strided transposed convolution, gathered from its weights w [C, OC/groups, KH0,
 // KW0] into the order a plain convolution reads: phase after phase, each [groups][OC/groups][C/groups][KH][KW] with tap
 // (a, b) = element (th0 + a*ths, tw0 + b*tws) of the kernel. One thread per gathered value.
-__global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total)
+__global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total, int wstride)
 {
    const int e = blockIdx.x * blockDim.x + threadIdx.x;
    if (e >= total) return;
@@ -487,6 +683,17 @@ __global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total)
    for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
       if (pi == i) q = g.phase[i];
    int r = e - q.woff;
+   if (wstride > 0) {
+      // the order k_conv2d_f32_dma reads: [groups][K = input channel, tap][wstride], zeros behind the last channel
+      const int oc = r % wstride; r /= wstride;
+      const int b = r % q.KW; r /= q.KW;
+      const int a = r % q.KH; r /= q.KH;
+      const int ic = r % g.icg;
+      const int grp = r / g.icg;
+      dst[e] = oc < g.ocg ? g.w[((((size_t)grp * g.icg + ic) * g.ocg + oc) * g.KH0 + q.th0 + a * g.ths) * g.KW0 + q.tw0 + b * g.tws]
+                          : 0.0f;
+      return;
+   }
    const int b = r % q.KW; r /= q.KW;
    const int a = r % q.KH; r /= q.KH;
    const int ic = r % g.icg; r /= g.icg;
@@ -530,6 +737,13 @@ __global__ void k_conv2d_f32_simple(ConvArgs g)
    g.y[(((size_t)n * g.OC + oc) * g.OH0 + g.oy0 + oh * g.oys) * g.OW0 + g.ox0 + ow * g.oxs] = acc;
 }
 
+// LDS of k_conv2d_f32_dma: two buffers (weight tile [kc][BOC], patch rounded up to whole requests of 256 cells) and the
+// patch offsets of the kc taps.
+inline size_t dma_lds_bytes(int kc, size_t plen, int BOC)
+{
+   return (2 * ((size_t)kc * BOC + ((plen + 255) & ~(size_t)255)) + kc) * 4;
+}
+
 template <int TI, int TJ>
 int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
 {
@@ -546,6 +760,38 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    *done = false;
    const int octiles = cdiv(g.ocg, BOC);
    if ((size_t)g.groups * octiles > 65535 || g.N > 65535) return SOFIE_HIP_OK;
+   if (!g.transposed && !getenv("SOFIE_CONV_NO_DMA")) {
+      // First choice: operands by LDS-DMA under the matrix loop (k_conv2d_f32_dma), on a copy of the weights laid out
+      // for it (a small kernel in front). The largest full channel block with an even K whose two LDS buffers fit the
+      // budget; at least nine K-steps of matrix work per block.
+      const size_t HW = (size_t)g.H * g.W;
+      const int wstride = (g.ocg + 3) & ~3;
+      const size_t wt_floats = (size_t)g.groups * g.icg * KHW * wstride;
+      if ((size_t)g.icg * HW * 4 < (1u << 30) && (size_t)g.icg * KHW * wstride * 4 < (1u << 30))
+         for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
+            const int kc = icb * KHW;
+            const size_t plen = (size_t)icb * g.PH * g.PW;
+            const size_t lds = dma_lds_bytes(kc, plen, BOC);
+            if (kc < 18) break;
+            if (g.icg % icb != 0 || kc % 2 != 0 || lds > budget || plen > SOFIE_CONV_DMA_PATCH) continue;
+            g.ICB = icb;
+            g.KC = kc;
+            g.dPW = make_fastdiv((unsigned)g.PW);
+            g.dPH = make_fastdiv((unsigned)g.PH);
+            void *ws = nullptr;
+            if (int rc = workspace(ctx, wt_floats * sizeof(float), &ws)) return rc;
+            hipLaunchKernelGGL(k_transpose_weights, dim3((unsigned)((wt_floats + 255) / 256)), dim3(256), 0, ctx->stream, g.w,
+                               static_cast<float *>(ws), g.groups, g.ocg, g.icg * KHW, wstride);
+            if (int rc = check_launch(ctx, "k_transpose_weights")) return rc;
+            ConvArgs h = g;
+            h.w = static_cast<const float *>(ws);
+            constexpr auto kern = k_conv2d_f32_dma<TI, TJ>;
+            SOFIE_LARGE_LDS(kern);
+            hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, h);
+            *done = true;
+            return check_launch(ctx, "k_conv2d_f32_dma");
+         }
+   }
    if (!g.transposed) {
       // staging under the matrix loop: the largest channel block whose two LDS buffers fit the budget and whose
       // values fit the registers the kernel sets aside; at least nine K-steps of matrix work per block
@@ -616,7 +862,58 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    if ((size_t)g.groups * octiles > 65535 || (size_t)g.N * g.nphases > 65535) return SOFIE_HIP_OK;
    size_t lds_max = 0;
    int tiles_max = 0;
-   // First choice: the kernel that stages channel block c+1 under the matrix loop of block c, on sub-kernels gathered
+   // First choice: operands by LDS-DMA under the matrix loop, on sub-kernels gathered into the [K][channel] order (a
+   // small kernel in front, into the context's scratch buffer). Every phase needs a full channel block with an even K
+   // of at least 16 that fits.
+   if (!getenv("SOFIE_CONV_NO_DMA")) {
+      const int wstride = (g.ocg + 3) & ~3;
+      bool fits = (size_t)g.icg * g.H * g.W * 4 < (1u << 30);
+      int woff = 0;
+      for (int i = 0; i < g.nphases && fits; ++i) {
+         PhaseArgs &p = g.phase[i];
+         const int KHW = p.KH * p.KW;
+         p.rows_out = (BP + p.OW - 2) / p.OW + 1;
+         if (p.rows_out > p.OH) p.rows_out = p.OH;
+         p.PH = (p.rows_out - 1) + (p.KH - 1) + 1;      // unit stride and dilation inside a phase
+         p.PW = (p.OW - 1) + (p.KW - 1) + 1;
+         bool found = false;
+         for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1 && !found; --icb) {
+            const int kc = icb * KHW;
+            const size_t plen = (size_t)icb * p.PH * p.PW;
+            const size_t lds = dma_lds_bytes(kc, plen, BOC);
+            if (kc < 16) break;
+            if (g.icg % icb != 0 || kc % 2 != 0 || lds > budget || plen > SOFIE_CONV_DMA_PATCH) continue;
+            p.ICB = icb;
+            p.KC = kc;
+            p.dPW = make_fastdiv((unsigned)p.PW);
+            p.dPH = make_fastdiv((unsigned)p.PH);
+            p.dOW = make_fastdiv((unsigned)p.OW);
+            if (lds > lds_max) lds_max = lds;
+            found = true;
+         }
+         fits = found && (size_t)g.icg * KHW * wstride * 4 < (1u << 30);
+         p.woff = woff;
+         woff += g.groups * g.icg * KHW * wstride;       // a multiple of 4 floats
+         if (cdiv(p.OH * p.OW, BP) > tiles_max) tiles_max = cdiv(p.OH * p.OW, BP);
+      }
+      if (fits) {
+         void *ws = nullptr;
+         if (int rc = workspace(ctx, (size_t)woff * sizeof(float), &ws)) return rc;
+         hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
+                            static_cast<float *>(ws), woff, wstride);
+         if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
+         ConvArgs h = g;
+         h.w = static_cast<const float *>(ws);
+         constexpr auto kern = k_conv2d_f32_dma<TI, TJ, true>;
+         SOFIE_LARGE_LDS(kern);
+         hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
+         *done = true;
+         return check_launch(ctx, "k_conv2d_f32_dma_phases");
+      }
+      lds_max = 0;
+      tiles_max = 0;
+   }
+   // Second choice: the kernel that stages channel block c+1 under the matrix loop of block c, on sub-kernels gathered
    // into the plain weight order (a small kernel in front, into the context's scratch buffer). Every phase must fit
    // its limits (full channel blocks of K = 16 .. 80 with 16-byte weight loads, the values of a block in registers).
    {
@@ -657,7 +954,7 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          void *ws = nullptr;
          if (int rc = workspace(ctx, (size_t)woff * sizeof(float), &ws)) return rc;
          hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
-                            static_cast<float *>(ws), woff);
+                            static_cast<float *>(ws), woff, 0);
          if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
          ConvArgs h = g;
          h.w = static_cast<const float *>(ws);
