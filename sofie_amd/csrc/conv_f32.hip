@@ -487,7 +487,7 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
 // block but a uniform offset, so a thread keeps NP patch offsets and one weight offset for the whole kernel.
 // PHASES as in k_conv2d_f32_pipe.
 template <int TI, int TJ, bool PHASES = false>
-__global__ void __launch_bounds__(256, 3) k_conv2d_f32_dma(ConvArgs gg)
+__global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArgs gg)
 {
    constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32;
    constexpr int NP = SOFIE_CONV_DMA_PATCH / 256;
@@ -744,6 +744,27 @@ inline size_t dma_lds_bytes(int kc, size_t plen, int BOC)
    return (2 * ((size_t)kc * BOC + ((plen + 255) & ~(size_t)255)) + kc) * 4;
 }
 
+// LDS a workgroup of k_conv2d_f32_dma may use: the CU's 160 KB over the number of workgroups it should hold. Three by
+// default (while one waits for its next channel block two keep the matrix cores busy: 2.66 ms at 64 KB, 1.99 ms at
+// 52 KB on 256x64x56x56 -> 128); more, with smaller channel blocks, when that lets a grid of few workgroups run in
+// whole rounds (the 1792 workgroups of a 64-image 28x28 -> 56x56 transposed layer: 7 per CU in one round instead of
+// 3 + 3 + 1, 145 against 162 us). max_resident: what the kernel's registers allow (7 with 32 accumulators, 3 with 128).
+inline size_t dma_lds_budget(const sofie_hip_ctx *ctx, size_t workgroups, int max_resident)
+{
+   const size_t cus = ctx->num_cus > 0 ? (size_t)ctx->num_cus : 256;
+   int best = 3;
+   double best_fill = 0.0;
+   for (int r = 3; r <= max_resident; ++r) {
+      const size_t slots = cus * r, rounds = (workgroups + slots - 1) / slots;
+      const double fill = (double)workgroups / (double)(rounds * slots);
+      if (fill > best_fill + 0.02) {
+         best = r;
+         best_fill = fill;
+      }
+   }
+   return best == 3 ? (size_t)52 * 1024 : (size_t)(160 * 1024) / best - 512;
+}
+
 template <int TI, int TJ>
 int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
 {
@@ -767,6 +788,7 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
       const size_t HW = (size_t)g.H * g.W;
       const int wstride = (g.ocg + 3) & ~3;
       const size_t wt_floats = (size_t)g.groups * g.icg * KHW * wstride;
+      const size_t budget = dma_lds_budget(ctx, (size_t)cdiv(OHW, BP) * g.groups * octiles * g.N, TI == 1 ? 7 : 3);
       if ((size_t)g.icg * HW * 4 < (1u << 30) && (size_t)g.icg * KHW * wstride * 4 < (1u << 30))
          for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
             const int kc = icb * KHW;
@@ -866,6 +888,10 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    // small kernel in front, into the context's scratch buffer). Every phase needs a full channel block with an even K
    // of at least 16 that fits.
    if (!getenv("SOFIE_CONV_NO_DMA")) {
+      size_t workgroups = 0;
+      for (int i = 0; i < g.nphases; ++i)
+         workgroups += (size_t)cdiv(g.phase[i].OH * g.phase[i].OW, BP) * g.groups * octiles * g.N;
+      const size_t budget = dma_lds_budget(ctx, workgroups, TI == 1 ? 7 : 3);
       const int wstride = (g.ocg + 3) & ~3;
       bool fits = (size_t)g.icg * g.H * g.W * 4 < (1u << 30);
       int woff = 0;
