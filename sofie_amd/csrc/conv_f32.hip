@@ -535,7 +535,7 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
    const int OHW = g.OH * g.OW;
    const int p0 = blockIdx.x * BP;
-   const int oh0 = p0 / g.OW;
+   const int oh0 = fdiv(p0, dOW);
    const int ih0 = oh0 * g.sh - g.ph, iw0 = -g.pw;
    const int KHW = g.KH * g.KW;
    const int Kfull = g.icg * KHW;
@@ -551,7 +551,8 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
 #pragma unroll
    for (int j = 0; j < TJ; ++j) {
       const int p = p0 + wn * TJ * 32 + j * 32 + fr;
-      base[j] = (p < OHW) ? ((p / g.OW - oh0) * g.sh) * g.PW + (p % g.OW) * g.sw : 0;
+      const int row = fdiv(p, dOW);
+      base[j] = (p < OHW) ? ((row - oh0) * g.sh) * g.PW + (p - row * g.OW) * g.sw : 0;
    }
    v16f acc[TI][TJ];
 #pragma unroll
@@ -566,9 +567,12 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    const rsrc_t wrs = make_rsrc(g.w + (size_t)grp * Kfull * wstride, (unsigned)((size_t)Kfull * wstride * 4));
    // byte offsets of this thread's patch cells inside a block's channels, and of its 16 bytes of weight row tid /
    // (BOC/4) (the rows of its later requests are ROWS_PER_REQUEST further each: same parity, same rotation)
+   const int npatch = (patch_len + 255) >> 8;        // patch requests per thread (of NP)
    unsigned pofs[NP];
 #pragma unroll
    for (int u = 0; u < NP; ++u) {
+      pofs[u] = OUTSIDE;
+      if (u >= npatch) continue;
       const int e = u * 256 + tid;
       const int t = fdiv(e, g.dPW), c = e - t * g.PW;
       const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
@@ -579,7 +583,6 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    const int wrow0 = tid / (BOC / 4);
    const int wcol = ((tid % (BOC / 4)) * 4 - 32 * (wrow0 & 1)) & (BOC - 1);     // column the rotated cell holds
    const unsigned wofs = oc0 + wcol < wstride ? (unsigned)((wrow0 * wstride + oc0 + wcol) * 4) : OUTSIDE;
-   const int npatch = (patch_len + 255) >> 8;        // patch requests per thread (of NP)
    const unsigned xblock = (unsigned)(g.ICB * HW * 4), wblock = (unsigned)(g.KC * wstride * 4);
    const unsigned wstep = (unsigned)(ROWS_PER_REQUEST * wstride * 4);
    const unsigned lds0 = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)smem_raw;   // LDS byte address of the buffers
@@ -625,36 +628,41 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
       __syncthreads();
    }
 
+   // Stores through a descriptor of this image's output channels of the group (the launcher keeps it under 1 GiB): a
+   // lane's offset is its pixel (and its K half's four channels), the channel of a store is a uniform offset, and what
+   // lies behind the plane's pixels or the group's channels falls outside the descriptor's range and is dropped.
    const size_t plane = PHASES ? (size_t)gg.OH0 * gg.OW0 : (size_t)OHW;
-   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane;
+   const rsrc_t yrs = make_rsrc(g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane, (unsigned)((size_t)g.ocg * plane * 4));
+   const unsigned plane4 = (unsigned)(plane * 4);
+   // biases the same way (no bias: an empty range, every load returns 0)
+   const __amdgpu_buffer_rsrc_t brs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(g.bias) + (g.bias ? grp * g.ocg : 0), 0, g.bias ? g.ocg * 4 : 0, 0x00020000);
    float bv[TI][16];
 #pragma unroll
    for (int i = 0; i < TI; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-         const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
-         bv[i][r] = (g.bias && oc < g.ocg) ? g.bias[grp * g.ocg + oc] : 0.0f;
+      for (int r = 0; r < 16; ++r)
+         bv[i][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                 brs, fk * 16, (oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + (r & 3)) * 4, 0));
+#pragma unroll
+   for (int j = 0; j < TJ; ++j) {
+      const int p = p0 + wn * TJ * 32 + j * 32 + fr;
+      unsigned po = (unsigned)p;
+      if constexpr (PHASES) {
+         const int row = fdiv(p, dOW);
+         po = (unsigned)((oy0 + row * gg.oys) * gg.OW0 + ox0 + (p - row * g.OW) * gg.oxs);
       }
+      const unsigned voff = p < OHW ? po * 4 + (unsigned)fk * 4 * plane4 : OUTSIDE;
 #pragma unroll
-   for (int i = 0; i < TI; ++i)
-#pragma unroll
-      for (int j = 0; j < TJ; ++j) {
-         const int p = p0 + wn * TJ * 32 + j * 32 + fr;
-         if (p >= OHW) continue;
-         size_t po = (size_t)p;
-         if constexpr (PHASES) {
-            const int row = fdiv(p, dOW);
-            po = (size_t)(oy0 + row * gg.oys) * gg.OW0 + ox0 + (p - row * g.OW) * gg.oxs;
-         }
+      for (int i = 0; i < TI; ++i)
 #pragma unroll
          for (int r = 0; r < 16; ++r) {
-            const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
-            if (oc >= g.ocg) continue;
+            const int oc_uniform = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + (r & 3);   // + 4 * fk in the lane's offset
             float v = __fadd_rn(acc[i][j][r], bv[i][r]);
             if (g.relu) v = v > 0.0f ? v : 0.0f;
-            yn[(size_t)oc * plane + po] = v;
+            store4_buf(yrs, v, voff, (unsigned)oc_uniform * plane4);
          }
-      }
+   }
 }
 
 // Weights of a plain convolution w [OC][C/groups][KH][KW] as k_conv2d_f32_dma reads them: wt [group][K][wstride],
@@ -789,7 +797,8 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
       const int wstride = (g.ocg + 3) & ~3;
       const size_t wt_floats = (size_t)g.groups * g.icg * KHW * wstride;
       const size_t budget = dma_lds_budget(ctx, (size_t)cdiv(OHW, BP) * g.groups * octiles * g.N, TI == 1 ? 7 : 3);
-      if ((size_t)g.icg * HW * 4 < (1u << 30) && (size_t)g.icg * KHW * wstride * 4 < (1u << 30))
+      if ((size_t)g.icg * HW * 4 < (1u << 30) && (size_t)g.icg * KHW * wstride * 4 < (1u << 30) &&
+          (size_t)g.ocg * OHW * 4 < (1u << 30))
          for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
             const int kc = icb * KHW;
             const size_t plen = (size_t)icb * g.PH * g.PW;
@@ -893,7 +902,7 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          workgroups += (size_t)cdiv(g.phase[i].OH * g.phase[i].OW, BP) * g.groups * octiles * g.N;
       const size_t budget = dma_lds_budget(ctx, workgroups, TI == 1 ? 7 : 3);
       const int wstride = (g.ocg + 3) & ~3;
-      bool fits = (size_t)g.icg * g.H * g.W * 4 < (1u << 30);
+      bool fits = (size_t)g.icg * g.H * g.W * 4 < (1u << 30) && (size_t)g.ocg * g.OH0 * g.OW0 * 4 < (1u << 30);
       int woff = 0;
       for (int i = 0; i < g.nphases && fits; ++i) {
          PhaseArgs &p = g.phase[i];

@@ -510,6 +510,16 @@ __device__ __forceinline__ void dma4(rsrc_t rs, unsigned lds_base, int voff, int
                 : "memory");
 }
 
+// 4 bytes per lane to global memory through a descriptor (per-lane offset + uniform offset): an address of a few
+// instructions less than a flat store's, and a lane whose offset lies outside the descriptor's range stores nothing.
+__device__ __forceinline__ void store4_buf(rsrc_t rs, float v, unsigned voff, unsigned soff)
+{
+   asm volatile("buffer_store_dword %0, %1, %2, %3 offen"
+                :
+                : "v"(v), "v"(voff), "s"(rs), "s"(__builtin_amdgcn_readfirstlane((int)soff))
+                : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt()
 {
