@@ -20,16 +20,13 @@ using namespace sofie;
 
 namespace {
 
-// Most values of a channel block that the threads of a workgroup carry in registers in k_conv2d_f32_pipe.
-#define SOFIE_CONV_PIPE_PATCH 1792
-#define SOFIE_CONV_PIPE_WEIGHTS 5120
 // Most patch cells of a channel block in k_conv2d_f32_dma (a thread keeps an offset per 256 cells).
 #define SOFIE_CONV_DMA_PATCH 3584
 
 // Geometry of one output phase of a strided transposed convolution when all phases run in one launch.
 struct PhaseArgs {
    int KH, KW, th0, tw0, ph, pw, oy0, ox0, OH, OW, rows_out, PH, PW, ICB, KC;
-   int woff;           // k_conv2d_f32_pipe: first float of the phase's sub-kernel in the gathered weights
+   int woff;           // k_conv2d_f32_dma: first float of the phase's sub-kernel in the gathered weights
    FastDiv dPW, dPH, dKC, dOW, dK4;
 };
 #define SOFIE_CONV_MAX_PHASES 4
@@ -275,208 +272,6 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
       }
 }
 
-// The same implicit GEMM with the staging of channel block c+1 under the matrix loop of block c: the loads of the
-// next block are issued into registers before the loop and written to the other LDS buffer after it, one barrier
-// per block. Blocks are small enough for a thread to carry its share: at most NP patch values and NW weights
-// (the launcher picks the channels per block accordingly and falls back to k_conv2d_f32 otherwise). Plain
-// convolutions only.
-// PHASES: the launch holds the output phases of a strided transposed convolution (blockIdx.z = image * nphases +
-// phase). A phase is a plain unit-stride convolution of the input with its sub-kernel (g.w then holds the sub-kernels
-// gathered into the plain [OC][C][KH][KW] order, one after the other) whose outputs go to every stride-th pixel of the
-// output plane.
-template <int TI, int TJ, bool PHASES = false>
-__global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
-{
-   constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32, LDW = BOC + 1;
-   constexpr int NP = SOFIE_CONV_PIPE_PATCH / 256, NW = SOFIE_CONV_PIPE_WEIGHTS / 256;
-   // geometry of this workgroup: the launch's own, or that of its phase (picked with static indices so that it stays
-   // in scalar registers)
-   struct Geometry {
-      const float *x, *w, *bias;
-      float *y;
-      int C, H, W, OC, KH, KW, ph, pw, sh, sw, dh, dw, OH, OW, icg, ocg, ICB, KC, PH, PW, relu;
-      FastDiv dPW, dPH, dK4;
-   } g;
-   g.x = gg.x; g.w = gg.w; g.bias = gg.bias; g.y = gg.y;
-   g.C = gg.C; g.H = gg.H; g.W = gg.W; g.OC = gg.OC; g.KH = gg.KH; g.KW = gg.KW; g.ph = gg.ph; g.pw = gg.pw;
-   g.sh = gg.sh; g.sw = gg.sw; g.dh = gg.dh; g.dw = gg.dw; g.OH = gg.OH; g.OW = gg.OW; g.icg = gg.icg; g.ocg = gg.ocg;
-   g.ICB = gg.ICB; g.KC = gg.KC; g.PH = gg.PH; g.PW = gg.PW; g.relu = gg.relu;
-   g.dPW = gg.dPW; g.dPH = gg.dPH; g.dK4 = gg.dK4;
-   int n = blockIdx.z;
-   int oy0 = 0, ox0 = 0;
-   FastDiv dOW = gg.dOW;
-   if constexpr (PHASES) {
-      const int pi = blockIdx.z % gg.nphases;
-      n = blockIdx.z / gg.nphases;
-      PhaseArgs q = gg.phase[0];
-#pragma unroll
-      for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
-         if (pi == i) q = gg.phase[i];
-      if ((int)blockIdx.x * BP >= q.OH * q.OW) return;   // the grid is as wide as the phase with most pixel tiles
-      g.KH = q.KH; g.KW = q.KW; g.ph = q.ph; g.pw = q.pw; g.OH = q.OH; g.OW = q.OW; g.ICB = q.ICB; g.KC = q.KC;
-      g.PH = q.PH; g.PW = q.PW; g.dPW = q.dPW; g.dPH = q.dPH; g.dK4 = q.dK4;
-      g.w = gg.w + q.woff;
-      oy0 = q.oy0; ox0 = q.ox0; dOW = q.dOW;
-   }
-   extern __shared__ __align__(16) unsigned char smem_raw[];
-   const int patch_len = g.ICB * g.PH * g.PW;
-   const int buf_len = g.KC * LDW + patch_len;                       // floats of one buffer: [KC][LDW] weights, patch
-   float *const bufs = reinterpret_cast<float *>(smem_raw);
-   int *const koff = reinterpret_cast<int *>(bufs + 2 * buf_len);    // [KC]
-
-   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-   const int wm = wave >> 1, wn = wave & 1;
-   const int fr = lane & 31, fk = lane >> 5;
-   const int octiles = (g.ocg + BOC - 1) / BOC;
-   const int grp = blockIdx.y / octiles;
-   const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
-   const int OHW = g.OH * g.OW;
-   const int p0 = blockIdx.x * BP;
-   const int oh0 = p0 / g.OW;
-   const int ih0 = oh0 * g.sh - g.ph, iw0 = -g.pw;
-   const int KHW = g.KH * g.KW;
-   const int Kfull = g.icg * KHW;
-
-   for (int k = tid; k < g.KC; k += 256) {
-      const int icl = k / KHW, t = k % KHW;
-      const int kh = t / g.KW, kw = t % g.KW;
-      koff[k] = (icl < g.ICB) ? (icl * g.PH + kh * g.dh) * g.PW + kw * g.dw : 0;
-   }
-   int base[TJ];
-#pragma unroll
-   for (int j = 0; j < TJ; ++j) {
-      const int p = p0 + wn * TJ * 32 + j * 32 + fr;
-      base[j] = (p < OHW) ? ((p / g.OW - oh0) * g.sh) * g.PW + (p % g.OW) * g.sw : 0;
-   }
-   v16f acc[TI][TJ];
-#pragma unroll
-   for (int i = 0; i < TI; ++i)
-#pragma unroll
-      for (int j = 0; j < TJ; ++j)
-#pragma unroll
-         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-   const float *xg = g.x + ((size_t)n * g.C + (size_t)grp * g.icg) * g.H * g.W;
-   const float *wg = g.w + (size_t)grp * g.ocg * Kfull;
-   const int K4 = g.KC >> 2;
-   // a wavefront whose pixels all lie behind the end of the plane multiplies nothing (a 28x28 plane is 6 tiles of 128
-   // pixels and one of 16); it still stages its share of every block
-   const int nsteps = p0 + __builtin_amdgcn_readfirstlane(wn) * TJ * 32 < OHW ? g.KC / 2 : 0;
-
-   // A thread's share of one channel block, in registers between issue() and commit(). Where a value comes from and
-   // where it goes does not depend on the block (every block is full: the launchers see to it), so the offsets are
-   // worked out once: pofs[u] = offset of patch cell u*256+tid inside the block's input channels (-1: padding, or past
-   // the patch), wofs[u] = offset of four consecutive k of one output channel in the block's weights (-1: past the
-   // output channels), wlds[u] = where they go in the LDS weight tile (-1: nothing to write).
-   float pv[NP], wreg[NW];
-   int pofs[NP], wofs[NW / 4], wlds[NW / 4];
-#pragma unroll
-   for (int u = 0; u < NP; ++u) {
-      const int e = u * 256 + tid;
-      const int t = fdiv(e, g.dPW), c = e - t * g.PW;
-      const int icl = fdiv(t, g.dPH), r = t - icl * g.PH;
-      const int ih = ih0 + r, iw = iw0 + c;
-      const bool inside = e < patch_len && icl < g.ICB && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
-      pofs[u] = inside ? (icl * g.H + ih) * g.W + iw : -1;
-   }
-#pragma unroll
-   for (int u = 0; u < NW / 4; ++u) {
-      const int e = u * 256 + tid;
-      const int ocl = fdiv(e, g.dK4), k4 = e - ocl * K4;
-      wofs[u] = (e < K4 * BOC && oc0 + ocl < g.ocg) ? (oc0 + ocl) * Kfull + 4 * k4 : -1;
-      wlds[u] = e < K4 * BOC ? 4 * k4 * LDW + ocl : -1;
-   }
-   const size_t HW = (size_t)g.H * g.W;
-   auto issue = [&](int ic0) {
-      // loads are unconditional (of the block's first element where there is nothing to load)
-      const float *const xb = xg + (size_t)ic0 * HW;
-      const float *const wb = wg + (size_t)ic0 * KHW;
-#pragma unroll
-      for (int u = 0; u < NP; ++u) pv[u] = xb[pofs[u] < 0 ? 0 : pofs[u]];
-#pragma unroll
-      for (int u = 0; u < NW / 4; ++u) {
-         const v4f v = *reinterpret_cast<const v4f *>(wb + (wofs[u] < 0 ? 0 : wofs[u]));
-#pragma unroll
-         for (int q = 0; q < 4; ++q) wreg[4 * u + q] = v[q];
-      }
-   };
-   auto commit = [&](float *buf) {
-      float *const sW = buf, *const patch = buf + g.KC * LDW;
-#pragma unroll
-      for (int u = 0; u < NP; ++u) {
-         const int e = u * 256 + tid;
-         if (e < patch_len) patch[e] = pofs[u] < 0 ? 0.0f : pv[u];
-      }
-#pragma unroll
-      for (int u = 0; u < NW / 4; ++u)
-         if (wlds[u] >= 0) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) sW[wlds[u] + q * LDW] = wofs[u] < 0 ? 0.0f : wreg[4 * u + q];
-         }
-   };
-
-   const int nblocks = (g.icg + g.ICB - 1) / g.ICB;
-   issue(0);
-   commit(bufs);
-   __syncthreads();   // block 0 and the koff table are in LDS
-   for (int c = 0; c < nblocks; ++c) {
-      const bool more = c + 1 < nblocks;
-      if (more) issue((c + 1) * g.ICB);
-      const float *const sW = bufs + (c & 1) * buf_len, *const patch = sW + g.KC * LDW;
-      const float *wrow = sW + wm * TI * 32 + fr;
-      for (int s = 0; s < nsteps; ++s) {
-         const int kk = 2 * s + fk;
-         const int ko = koff[kk];
-         float fa[TI], fb[TJ];
-#pragma unroll
-         for (int i = 0; i < TI; ++i) fa[i] = wrow[kk * LDW + i * 32];
-#pragma unroll
-         for (int j = 0; j < TJ; ++j) fb[j] = patch[base[j] + ko];
-#pragma unroll
-         for (int i = 0; i < TI; ++i)
-#pragma unroll
-            for (int j = 0; j < TJ; ++j)
-               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
-      }
-      // the other buffer was last read in block c-1, before the barrier that ended it
-      if (more) commit(bufs + ((c + 1) & 1) * buf_len);
-      __syncthreads();
-   }
-
-   const size_t plane = PHASES ? (size_t)gg.OH0 * gg.OW0 : (size_t)OHW;
-   float *yn = g.y + ((size_t)n * g.OC + (size_t)grp * g.ocg) * plane;
-   // the biases of this lane's output channels, all loaded before the first store (a load behind a store that may
-   // alias it would wait for its own turn, 16 * TI * TJ times)
-   float bv[TI][16];
-#pragma unroll
-   for (int i = 0; i < TI; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-         const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
-         bv[i][r] = (g.bias && oc < g.ocg) ? g.bias[grp * g.ocg + oc] : 0.0f;
-      }
-#pragma unroll
-   for (int i = 0; i < TI; ++i)
-#pragma unroll
-      for (int j = 0; j < TJ; ++j) {
-         const int p = p0 + wn * TJ * 32 + j * 32 + fr;
-         if (p >= OHW) continue;
-         size_t po = (size_t)p;
-         if constexpr (PHASES) {
-            const int row = fdiv(p, dOW);
-            po = (size_t)(oy0 + row * gg.oys) * gg.OW0 + ox0 + (p - row * g.OW) * gg.oxs;
-         }
-#pragma unroll
-         for (int r = 0; r < 16; ++r) {
-            const int oc = oc0 + wm * TI * 32 + i * 32 + (r >> 2) * 8 + fk * 4 + (r & 3);
-            if (oc >= g.ocg) continue;
-            float v = __fadd_rn(acc[i][j][r], bv[i][r]);
-            if (g.relu) v = v > 0.0f ? v : 0.0f;
-            yn[(size_t)oc * plane + po] = v;
-         }
-      }
-}
-
 // The same implicit GEMM with both operands of channel block c+1 travelling global memory -> LDS without registers
 // (buffer_load ... lds) under the matrix loop of block c. The weights come from a copy laid out for it, wt [group]
 // [K = input channel, tap][wstride >= OC/groups, a multiple of 4] (k_transpose_weights / k_gather_phase_weights write it
@@ -485,7 +280,9 @@ __global__ void __launch_bounds__(256, 3) k_conv2d_f32_pipe(ConvArgs gg)
 // read on different banks without padding. A patch cell is 4 bytes per lane from wherever it sits in the image;
 // padding cells ask for an offset outside the descriptor's range and receive 0. Nothing of a block depends on the
 // block but a uniform offset, so a thread keeps NP patch offsets and one weight offset for the whole kernel.
-// PHASES as in k_conv2d_f32_pipe.
+// PHASES: the launch holds the output phases of a strided transposed convolution (blockIdx.z = image * nphases +
+// phase). A phase is a plain unit-stride convolution of the input with its sub-kernel (g.w then holds the sub-kernels
+// in the order above, one after the other) whose outputs go to every stride-th pixel of the output plane.
 template <int TI, int TJ, bool PHASES = false>
 __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArgs gg)
 {
@@ -504,17 +301,18 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    g.sh = gg.sh; g.sw = gg.sw; g.dh = gg.dh; g.dw = gg.dw; g.OH = gg.OH; g.OW = gg.OW; g.icg = gg.icg; g.ocg = gg.ocg;
    g.ICB = gg.ICB; g.KC = gg.KC; g.PH = gg.PH; g.PW = gg.PW; g.relu = gg.relu;
    g.dPW = gg.dPW; g.dPH = gg.dPH;
-   int n = blockIdx.z;
+   const int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
+   int n = bz;
    int oy0 = 0, ox0 = 0;
    FastDiv dOW = gg.dOW;
    if constexpr (PHASES) {
-      const int pi = blockIdx.z % gg.nphases;
-      n = blockIdx.z / gg.nphases;
+      const int pi = bz % gg.nphases;
+      n = bz / gg.nphases;
       PhaseArgs q = gg.phase[0];
 #pragma unroll
       for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
          if (pi == i) q = gg.phase[i];
-      if ((int)blockIdx.x * BP >= q.OH * q.OW) return;   // the grid is as wide as the phase with most pixel tiles
+      if (bx * BP >= q.OH * q.OW) return;   // the grid is as wide as the phase with most pixel tiles
       g.KH = q.KH; g.KW = q.KW; g.ph = q.ph; g.pw = q.pw; g.OH = q.OH; g.OW = q.OW; g.ICB = q.ICB; g.KC = q.KC;
       g.PH = q.PH; g.PW = q.PW; g.dPW = q.dPW; g.dPH = q.dPH;
       g.w = gg.w + q.woff;
@@ -531,10 +329,10 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    const int wm = wave >> 1, wn = wave & 1;
    const int fr = lane & 31, fk = lane >> 5;
    const int octiles = (g.ocg + BOC - 1) / BOC;
-   const int grp = blockIdx.y / octiles;
-   const int oc0 = (blockIdx.y % octiles) * BOC;    // within the group
+   const int grp = by / octiles;
+   const int oc0 = (by % octiles) * BOC;    // within the group
    const int OHW = g.OH * g.OW;
-   const int p0 = blockIdx.x * BP;
+   const int p0 = bx * BP;
    const int oh0 = fdiv(p0, dOW);
    const int ih0 = oh0 * g.sh - g.ph, iw0 = -g.pw;
    const int KHW = g.KH * g.KW;
@@ -676,8 +474,8 @@ __global__ void k_transpose_weights(const float *w, float *wt, int groups, int o
 }
 
 // Sub-kernels of the output phases of a strided transposed convolution, gathered from its weights w [C, OC/groups, KH0,
-// KW0] into the order a plain convolution reads: phase after phase, each [groups][OC/groups][C/groups][KH][KW] with tap
-// (a, b) = element (th0 + a*ths, tw0 + b*tws) of the kernel. One thread per gathered value.
+// KW0] into the order k_conv2d_f32_dma reads: phase after phase, each [groups][K = input channel, tap][wstride] with
+// tap (a, b) = element (th0 + a*ths, tw0 + b*tws) of the kernel and zeros behind the last channel. One thread per value.
 __global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total, int wstride)
 {
    const int e = blockIdx.x * blockDim.x + threadIdx.x;
@@ -691,23 +489,13 @@ __global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total, int ws
    for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
       if (pi == i) q = g.phase[i];
    int r = e - q.woff;
-   if (wstride > 0) {
-      // the order k_conv2d_f32_dma reads: [groups][K = input channel, tap][wstride], zeros behind the last channel
-      const int oc = r % wstride; r /= wstride;
-      const int b = r % q.KW; r /= q.KW;
-      const int a = r % q.KH; r /= q.KH;
-      const int ic = r % g.icg;
-      const int grp = r / g.icg;
-      dst[e] = oc < g.ocg ? g.w[((((size_t)grp * g.icg + ic) * g.ocg + oc) * g.KH0 + q.th0 + a * g.ths) * g.KW0 + q.tw0 + b * g.tws]
-                          : 0.0f;
-      return;
-   }
+   const int oc = r % wstride; r /= wstride;
    const int b = r % q.KW; r /= q.KW;
    const int a = r % q.KH; r /= q.KH;
-   const int ic = r % g.icg; r /= g.icg;
-   const int oc = r % g.ocg;
-   const int grp = r / g.ocg;
-   dst[e] = g.w[((((size_t)grp * g.icg + ic) * g.ocg + oc) * g.KH0 + q.th0 + a * g.ths) * g.KW0 + q.tw0 + b * g.tws];
+   const int ic = r % g.icg;
+   const int grp = r / g.icg;
+   dst[e] = oc < g.ocg ? g.w[((((size_t)grp * g.icg + ic) * g.ocg + oc) * g.KH0 + q.th0 + a * g.ths) * g.KW0 + q.tw0 + b * g.tws]
+                       : 0.0f;
 }
 
 // One thread per output element: any kernel size, used when the staged patch of the tiled
@@ -789,7 +577,7 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    *done = false;
    const int octiles = cdiv(g.ocg, BOC);
    if ((size_t)g.groups * octiles > 65535 || g.N > 65535) return SOFIE_HIP_OK;
-   if (!g.transposed && !getenv("SOFIE_CONV_NO_DMA")) {
+   if (!g.transposed) {
       // First choice: operands by LDS-DMA under the matrix loop (k_conv2d_f32_dma), on a copy of the weights laid out
       // for it (a small kernel in front). The largest full channel block with an even K whose two LDS buffers fit the
       // budget; at least nine K-steps of matrix work per block.
@@ -822,32 +610,6 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             *done = true;
             return check_launch(ctx, "k_conv2d_f32_dma");
          }
-   }
-   if (!g.transposed) {
-      // staging under the matrix loop: the largest channel block whose two LDS buffers fit the budget and whose
-      // values fit the registers the kernel sets aside; at least nine K-steps of matrix work per block
-      for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
-         const int kc = (icb * KHW + 1) & ~1;
-         const size_t plen = (size_t)icb * g.PH * g.PW;
-         const size_t lds = (2 * ((size_t)kc * LDW + plen) + kc) * 4;
-         if (kc < 18) break;
-         if (lds > budget || (size_t)kc * BOC > SOFIE_CONV_PIPE_WEIGHTS || plen > SOFIE_CONV_PIPE_PATCH) continue;
-         g.ICB = icb;
-         g.KC = kc;
-         g.dPW = make_fastdiv((unsigned)g.PW);
-         g.dPH = make_fastdiv((unsigned)g.PH);
-         g.dKC = make_fastdiv((unsigned)g.KC);
-         g.dK4 = make_fastdiv((unsigned)(g.KC / 4));
-         // 16-byte weight loads only: every block full, blocks and rows of the [OC, K] matrix 16-byte aligned
-         g.wvec = g.icg % g.ICB == 0 && g.KC == g.ICB * KHW && g.KC % 4 == 0 && (g.icg * KHW) % 4 == 0 &&
-                  (reinterpret_cast<uintptr_t>(g.w) & 15u) == 0;
-         if (!g.wvec) continue;
-         constexpr auto kern = k_conv2d_f32_pipe<TI, TJ>;
-         SOFIE_LARGE_LDS(kern);
-         hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, g);
-         *done = true;
-         return check_launch(ctx, "k_conv2d_f32_pipe");
-      }
    }
    int icb = 96 / KHW;
    if (icb < 1) icb = 1;
@@ -896,7 +658,7 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
    // First choice: operands by LDS-DMA under the matrix loop, on sub-kernels gathered into the [K][channel] order (a
    // small kernel in front, into the context's scratch buffer). Every phase needs a full channel block with an even K
    // of at least 16 that fits.
-   if (!getenv("SOFIE_CONV_NO_DMA")) {
+   {
       size_t workgroups = 0;
       for (int i = 0; i < g.nphases; ++i)
          workgroups += (size_t)cdiv(g.phase[i].OH * g.phase[i].OW, BP) * g.groups * octiles * g.N;
@@ -944,60 +706,6 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
          *done = true;
          return check_launch(ctx, "k_conv2d_f32_dma_phases");
-      }
-      lds_max = 0;
-      tiles_max = 0;
-   }
-   // Second choice: the kernel that stages channel block c+1 under the matrix loop of block c, on sub-kernels gathered
-   // into the plain weight order (a small kernel in front, into the context's scratch buffer). Every phase must fit
-   // its limits (full channel blocks of K = 16 .. 80 with 16-byte weight loads, the values of a block in registers).
-   {
-      bool fits = true;
-      int woff = 0;
-      for (int i = 0; i < g.nphases && fits; ++i) {
-         PhaseArgs &p = g.phase[i];
-         const int KHW = p.KH * p.KW;
-         p.rows_out = (BP + p.OW - 2) / p.OW + 1;
-         if (p.rows_out > p.OH) p.rows_out = p.OH;
-         p.PH = (p.rows_out - 1) + (p.KH - 1) + 1;      // unit stride and dilation inside a phase
-         p.PW = (p.OW - 1) + (p.KW - 1) + 1;
-         bool found = false;
-         for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1 && !found; --icb) {
-            const int kc = icb * KHW;
-            const size_t plen = (size_t)icb * p.PH * p.PW;
-            const size_t lds = (2 * ((size_t)kc * LDW + plen) + kc) * 4;
-            if (kc < 16) break;
-            if (g.icg % icb != 0 || kc % 4 != 0 || lds > budget || (size_t)kc * BOC > SOFIE_CONV_PIPE_WEIGHTS ||
-                plen > SOFIE_CONV_PIPE_PATCH)
-               continue;
-            p.ICB = icb;
-            p.KC = kc;
-            p.dPW = make_fastdiv((unsigned)p.PW);
-            p.dPH = make_fastdiv((unsigned)p.PH);
-            p.dKC = make_fastdiv((unsigned)p.KC);
-            p.dK4 = make_fastdiv((unsigned)(p.KC / 4));
-            p.dOW = make_fastdiv((unsigned)p.OW);
-            if (lds > lds_max) lds_max = lds;
-            found = true;
-         }
-         fits = found;
-         p.woff = woff;
-         woff += g.groups * g.ocg * g.icg * KHW;         // a multiple of 4 floats: kc is, and icg is a multiple of icb
-         if (cdiv(p.OH * p.OW, BP) > tiles_max) tiles_max = cdiv(p.OH * p.OW, BP);
-      }
-      if (fits) {
-         void *ws = nullptr;
-         if (int rc = workspace(ctx, (size_t)woff * sizeof(float), &ws)) return rc;
-         hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
-                            static_cast<float *>(ws), woff, 0);
-         if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
-         ConvArgs h = g;
-         h.w = static_cast<const float *>(ws);
-         constexpr auto kern = k_conv2d_f32_pipe<TI, TJ, true>;
-         SOFIE_LARGE_LDS(kern);
-         hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
-         *done = true;
-         return check_launch(ctx, "k_conv2d_f32_pipe_phases");
       }
       lds_max = 0;
       tiles_max = 0;
