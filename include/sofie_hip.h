@@ -250,6 +250,18 @@ int sofie_hip_avgpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC
                             int kh, int kw, int pad_t, int pad_l, int pad_b, int pad_r, int stride_h,
                             int stride_w, int count_include_pad);
 
+/* Max and average pooling over three spatial axes, [NC][dims[0]][dims[1]][dims[2]] fp32: kernel[3], strides[3],
+ * pads[6] in ONNX order (the three begin pads, then the three end pads), floor output size, the window walked in
+ * row-major order with cells outside the volume skipped (for the average: summed, then divided once by the cells
+ * inside the volume, or by the whole window with count_include_pad). Replaces the emitted loops of
+ * ROperator_Pool.hxx:417-470 (the fDim == 3 branch). A pooling over one spatial axis (ROperator_Pool.hxx:329-370) is
+ * the 2-D call with H = 1 and a 1 x k kernel. */
+int sofie_hip_maxpool3d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, const int *dims,
+                            const int *kernel, const int *pads, const int *strides);
+int sofie_hip_avgpool3d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, const int *dims,
+                            const int *kernel, const int *pads, const int *strides,
+                            int count_include_pad);
+
 /* ---------------------------------------------------------------- quantized operators
  * The reference has no quantized operator (its parser rejects int8 initialisers,
  * src/SOFIE_parsers/src/RModelParser_ONNX.cxx:560-591); these follow ONNX's

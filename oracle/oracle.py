@@ -68,6 +68,7 @@ _bn = _sig("or_batchnorm_f32", None, [_f32p] * 5 + [C.c_float, _f32p] + [C.c_int
 _maxpool = _sig("or_maxpool2d_f32", None, [_f32p, _f32p] + [C.c_int] * 11)
 _avgpool = _sig("or_avgpool2d_f32", None, [_f32p, _f32p] + [C.c_int] * 12)
 _maxpool_s8 = _sig("or_maxpool2d_s8", None, [_i8p, _i8p] + [C.c_int] * 11)
+_pool3d = _sig("or_pool3d_f32", None, [_f32p, _f32p, C.c_int] + [C.POINTER(C.c_int)] * 4 + [C.c_int] * 2)
 _requant_one = _sig("or_requant_one", C.c_int8, [C.c_int32, C.c_float, C.c_int, C.c_int])
 _quant = _sig("or_quantize_f32_s8", None, [_f32p, _i8p, C.c_size_t, C.c_float, C.c_int])
 _dequant = _sig("or_dequantize_s8_f32", None, [_i8p, _f32p, C.c_size_t, C.c_float, C.c_int])
@@ -270,6 +271,18 @@ def avgpool2d(x, kernel, strides, pads=(0, 0, 0, 0), count_include_pad=False):
     y = np.empty((N, Cc, OH, OW), np.float32)
     _avgpool(x, y, N * Cc, H, W, kernel[0], kernel[1], pads[0], pads[1], pads[2], pads[3], strides[0], strides[1],
              int(count_include_pad))
+    return y
+
+
+def pool3d(x, kernel, strides, pads=(0, 0, 0, 0, 0, 0), average=False, count_include_pad=False):
+    """fp32 [N, C, D0, D1, D2] pooling (ROperator_Pool.hxx:417-470); pads = three begin pads, then three end pads."""
+    x = np.ascontiguousarray(x, np.float32)
+    N, Cc = x.shape[:2]
+    D = x.shape[2:]
+    out = tuple((D[i] + pads[i] + pads[3 + i] - kernel[i]) // strides[i] + 1 for i in range(3))
+    y = np.empty((N, Cc) + out, np.float32)
+    arr = lambda v: (C.c_int * len(v))(*[int(e) for e in v])
+    _pool3d(x, y, N * Cc, arr(D), arr(kernel), arr(pads), arr(strides), int(average), int(count_include_pad))
     return y
 
 

@@ -28,6 +28,8 @@
  *   or_einsum_f32                pinned: Einsum_matmul / _dotprod / _3 / _4 known answers of
  *                                the reference's tests, numpy.einsum in float64
  *   or_relu, or_maxpool2d        pinned: MaxPool2d known answer, torch CPU
+ *   or_pool3d_f32                pinned: torch.nn.functional.max_pool3d / avg_pool3d on CPU (both settings of
+ *                                count_include_pad), a float64 mean
  *   or_avgpool2d_f32             pinned: torch.nn.functional.avg_pool2d on CPU (count_include_pad on and off),
  *                                a float64 mean (the reference holds no AveragePool fixture for this path)
  *   or_broadcast_rows            pinned through the Linear_* answers (bias broadcast)
@@ -489,6 +491,52 @@ void or_maxpool2d_f32(const float *x, float *y, int NC, int H, int W, int kh, in
                 }
                 y[o++] = v;
             }
+    }
+}
+
+/* ------------------------------------------------------------------------- */
+/* Pooling over three spatial axes as emitted by the fDim == 3 branch of     */
+/* ROperator_Pool<float>::Generate (ROperator_Pool.hxx:417-470): per output   */
+/* the window is walked l (axis 0), m (axis 1), p (axis 2, fastest) with the  */
+/* cells outside the volume skipped; MaxPool starts from -inf, AveragePool    */
+/* sums into a float and divides once by nsum (the cells counted, or the      */
+/* whole window with count_include_pad). pads = ONNX order: three begin pads, */
+/* three end pads (the reference reads its pad vector as begin/end pairs per  */
+/* axis, :283-305, which is the same thing only when all six are equal).      */
+/* Pinned by: torch max_pool3d / avg_pool3d on CPU, a float64 mean.           */
+/* ------------------------------------------------------------------------- */
+void or_pool3d_f32(const float *x, float *y, int NC, const int *D, const int *k, const int *pads, const int *s,
+                   int average, int include_pad)
+{
+    int O[3];
+    for (int i = 0; i < 3; ++i) O[i] = (D[i] + pads[i] + pads[3 + i] - k[i]) / s[i] + 1;
+    size_t o = 0;
+    for (int nc = 0; nc < NC; ++nc) {
+        const float *xi = x + (size_t)nc * D[0] * D[1] * D[2];
+        for (int a = 0; a < O[0]; ++a)
+            for (int b = 0; b < O[1]; ++b)
+                for (int c = 0; c < O[2]; ++c) {
+                    float v = average ? 0.0f : -INFINITY;
+                    int nsum = 0;
+                    for (int l = a * s[0] - pads[0]; l < a * s[0] - pads[0] + k[0]; ++l) {
+                        if (l < 0 || l >= D[0]) continue;
+                        for (int m = b * s[1] - pads[1]; m < b * s[1] - pads[1] + k[1]; ++m) {
+                            if (m < 0 || m >= D[1]) continue;
+                            for (int p = c * s[2] - pads[2]; p < c * s[2] - pads[2] + k[2]; ++p) {
+                                if (p < 0 || p >= D[2]) continue;
+                                const float xv = xi[((size_t)l * D[1] + m) * D[2] + p];
+                                if (average) {
+                                    v += xv;
+                                    nsum++;
+                                } else if (xv > v) {
+                                    v = xv;
+                                }
+                            }
+                        }
+                    }
+                    if (average) v /= (float)(include_pad ? k[0] * k[1] * k[2] : nsum);
+                    y[o++] = v;
+                }
     }
 }
 

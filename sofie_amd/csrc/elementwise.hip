@@ -131,6 +131,49 @@ __global__ void k_avgpool2d_f32(const float *__restrict__ x, float *__restrict__
    y[idx] = __fdiv_rn(sum, (float)(include_pad ? kh * kw : count));
 }
 
+// fp32 pooling over three spatial axes [NC][D0][D1][D2], one thread per output element, the window walked in
+// row-major order (last axis fastest) with the cells outside the volume skipped: the maximum, or the sum divided once
+// by the number of cells counted (those inside the volume, or the whole window when padding cells count).
+struct Pool3dArgs {
+   int NC, D[3], O[3], k[3], pad[3], s[3];
+};
+
+template <bool AVERAGE>
+__global__ void k_pool3d_f32(const float *__restrict__ x, float *__restrict__ y, Pool3dArgs a, int include_pad)
+{
+   const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+   const size_t total = (size_t)a.NC * a.O[0] * a.O[1] * a.O[2];
+   if (idx >= total) return;
+   size_t r = idx;
+   const int o2 = (int)(r % a.O[2]); r /= a.O[2];
+   const int o1 = (int)(r % a.O[1]); r /= a.O[1];
+   const int o0 = (int)(r % a.O[0]);
+   const size_t nc = r / a.O[0];
+   const float *xi = x + nc * a.D[0] * a.D[1] * a.D[2];
+   float acc = AVERAGE ? 0.0f : -INFINITY;
+   int count = 0;
+   for (int i = 0; i < a.k[0]; ++i) {
+      const int d0 = o0 * a.s[0] - a.pad[0] + i;
+      if (d0 < 0 || d0 >= a.D[0]) continue;
+      for (int j = 0; j < a.k[1]; ++j) {
+         const int d1 = o1 * a.s[1] - a.pad[1] + j;
+         if (d1 < 0 || d1 >= a.D[1]) continue;
+         for (int l = 0; l < a.k[2]; ++l) {
+            const int d2 = o2 * a.s[2] - a.pad[2] + l;
+            if (d2 < 0 || d2 >= a.D[2]) continue;
+            const float v = xi[((size_t)d0 * a.D[1] + d1) * a.D[2] + d2];
+            if (AVERAGE) {
+               acc = __fadd_rn(acc, v);
+               ++count;
+            } else if (v > acc) {
+               acc = v;
+            }
+         }
+      }
+   }
+   y[idx] = AVERAGE ? __fdiv_rn(acc, (float)(include_pad ? a.k[0] * a.k[1] * a.k[2] : count)) : acc;
+}
+
 // Channels-last int8 max pooling, 16 channels (one 16-byte vector) of one output pixel per thread.
 // Signed bytes are compared as unsigned after flipping the sign bit, four at a time.
 __device__ __forceinline__ unsigned max_u8x4(unsigned a, unsigned b)
@@ -351,6 +394,50 @@ int sofie_hip_avgpool2d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC
    hipLaunchKernelGGL(k_avgpool2d_f32, dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y, NC, H, W, OH, OW, kh, kw,
                       pt, pl, sh, sw, count_include_pad != 0);
    return check_launch(ctx, "k_avgpool2d_f32");
+}
+
+static int pool3d(sofie_hip_ctx *ctx, bool average, const float *x, float *y, int NC, const int *dims, const int *kernel,
+                  const int *pads, const int *strides, int count_include_pad)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, NC >= 0, "negative dimension");
+   SOFIE_REQUIRE(ctx, dims && kernel && pads && strides, "null geometry");
+   Pool3dArgs a;
+   a.NC = NC;
+   size_t total = (size_t)NC;
+   for (int i = 0; i < 3; ++i) {
+      SOFIE_REQUIRE(ctx, dims[i] > 0 && kernel[i] > 0 && strides[i] > 0, "non-positive dimension");
+      SOFIE_REQUIRE(ctx, pads[i] >= 0 && pads[3 + i] >= 0, "negative padding");
+      SOFIE_REQUIRE(ctx, dims[i] + pads[i] + pads[3 + i] >= kernel[i], "kernel larger than padded input");
+      // a window that lies in the padding entirely would divide by zero cells
+      SOFIE_REQUIRE(ctx, !average || count_include_pad || (pads[i] < kernel[i] && pads[3 + i] < kernel[i]),
+                    "a pooling window without a cell of the volume");
+      a.D[i] = dims[i];
+      a.k[i] = kernel[i];
+      a.pad[i] = pads[i];
+      a.s[i] = strides[i];
+      a.O[i] = (dims[i] + pads[i] + pads[3 + i] - kernel[i]) / strides[i] + 1;
+      total *= (size_t)a.O[i];
+   }
+   if (NC == 0) return SOFIE_HIP_OK;
+   SOFIE_REQUIRE(ctx, x && y, "null operand");
+   if (average)
+      hipLaunchKernelGGL(k_pool3d_f32<true>, dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y, a, count_include_pad != 0);
+   else
+      hipLaunchKernelGGL(k_pool3d_f32<false>, dim3(blocks_for(total, 256)), dim3(256), 0, ctx->stream, x, y, a, 0);
+   return check_launch(ctx, average ? "k_avgpool3d_f32" : "k_maxpool3d_f32");
+}
+
+int sofie_hip_maxpool3d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, const int *dims, const int *kernel,
+                            const int *pads, const int *strides)
+{
+   return pool3d(ctx, false, x, y, NC, dims, kernel, pads, strides, 0);
+}
+
+int sofie_hip_avgpool3d_f32(sofie_hip_ctx *ctx, const float *x, float *y, int NC, const int *dims, const int *kernel,
+                            const int *pads, const int *strides, int count_include_pad)
+{
+   return pool3d(ctx, true, x, y, NC, dims, kernel, pads, strides, count_include_pad);
 }
 
 int sofie_hip_maxpool2d_s8(sofie_hip_ctx *ctx, const int8_t *x, int8_t *y, int layout, int N, int C, int H, int W,

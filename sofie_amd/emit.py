@@ -244,9 +244,9 @@ def spec_from_onnx(name, graph):
         elif op == "BatchNormalization":
             spec.batchnorm(ins[0], ins[1], ins[2], ins[3], ins[4], out, a.get("epsilon", 1e-5))
         elif op == "MaxPool":
-            spec.maxpool(ins[0], out, a["kernel_shape"], a.get("pads", (0, 0, 0, 0)), a.get("strides", (1, 1)))
+            spec.maxpool(ins[0], out, a["kernel_shape"], a.get("pads", ()), a.get("strides", ()))
         elif op == "AveragePool":
-            spec.avgpool(ins[0], out, a["kernel_shape"], a.get("pads", (0, 0, 0, 0)), a.get("strides", (1, 1)),
+            spec.avgpool(ins[0], out, a["kernel_shape"], a.get("pads", ()), a.get("strides", ()),
                          bool(a.get("count_include_pad", 0)))
         elif op == "GlobalAveragePool":
             spec.global_avgpool(ins[0], out)

@@ -66,29 +66,44 @@ public:
    std::vector<std::vector<size_t>> ShapeInference(std::vector<std::vector<size_t>> input) override
    {
       if (input.size() != 1) throw std::runtime_error("TMVA SOFIE" + Name() + "Op Shape inference need 1 input tensor");
-      if (input[0].size() != 4)
+      // one, two or three spatial axes behind [N, C] (reference :102-105)
+      if (input[0].size() < 3 || input[0].size() > 5)
          throw std::runtime_error("TMVA SOFIE" + Name() + "Op : tensors with dimension " + std::to_string(input[0].size()) +
                                   " are not yet supported");
+      const size_t dims = input[0].size() - 2;
+      const std::vector<size_t> spatial(input[0].begin() + 2, input[0].end());
       if (fPoolMode == GlobalAveragePool) {
          // a pooling whose kernel is the image (reference :216-228)
-         fAttr.kernel_shape = {input[0][2], input[0][3]};
+         fAttr.kernel_shape = spatial;
          fAttr.auto_pad = "NOTSET";
-         fAttr.pads = {0, 0, 0, 0};
-         fAttr.strides = {1, 1};
+         fAttr.pads.assign(2 * dims, 0);
+         fAttr.strides.assign(dims, 1);
       }
-      if (fAttr.kernel_shape.empty()) fAttr.kernel_shape = {input[0][2], input[0][3]};
+      if (fAttr.kernel_shape.empty()) fAttr.kernel_shape = spatial;
+      if (fAttr.kernel_shape.size() != dims)
+         throw std::runtime_error("TMVA SOFIE Pool Op Shape inference - invalid inputs ");
       if (fAttr.auto_pad != "NOTSET")
          throw std::runtime_error("TMVA SOFIE" + Name() + "Op : auto_pad is not supported by the device emission");
       if (fAttr.ceil_mode != 0)
          throw std::runtime_error("TMVA SOFIE" + Name() + "Op : ceil_mode is not supported by the device emission");
-      if (fAttr.pads.empty()) fAttr.pads = {0, 0, 0, 0};
-      fAttr.pads.resize(4, 0);
-      if (fAttr.strides.empty()) fAttr.strides = {1, 1};
+      // pads in ONNX order: the begin pads of the axes, then their end pads
+      if (fAttr.pads.empty()) fAttr.pads.assign(2 * dims, 0);
+      if (fAttr.pads.size() != 2 * dims)
+         throw std::runtime_error("TMVA SOFIE" + Name() + "Op : " + std::to_string(fAttr.pads.size()) + " pads for " +
+                                  std::to_string(dims) + " spatial axes");
+      if (fAttr.strides.empty()) fAttr.strides.assign(dims, 1);
+      if (fAttr.strides.size() != dims)
+         throw std::runtime_error("TMVA SOFIE" + Name() + "Op : " + std::to_string(fAttr.strides.size()) + " strides for " +
+                                  std::to_string(dims) + " spatial axes");
       for (auto d : fAttr.dilations)
          if (d != 1) throw std::runtime_error("TMVA SOFIE" + Name() + "Op : dilations are not supported by the device emission");
-      const size_t oh = (input[0][2] + fAttr.pads[0] + fAttr.pads[2] - fAttr.kernel_shape[0]) / fAttr.strides[0] + 1;
-      const size_t ow = (input[0][3] + fAttr.pads[1] + fAttr.pads[3] - fAttr.kernel_shape[1]) / fAttr.strides[1] + 1;
-      return {{input[0][0], input[0][1], oh, ow}};
+      std::vector<size_t> out = {input[0][0], input[0][1]};
+      for (size_t i = 0; i < dims; ++i) {
+         if (spatial[i] + fAttr.pads[i] + fAttr.pads[dims + i] < fAttr.kernel_shape[i] || fAttr.strides[i] == 0)
+            throw std::runtime_error("TMVA SOFIE" + Name() + "Op : kernel larger than the padded input");
+         out.push_back((spatial[i] + fAttr.pads[i] + fAttr.pads[dims + i] - fAttr.kernel_shape[i]) / fAttr.strides[i] + 1);
+      }
+      return {out};
    }
    void Initialize(RModel &model) override
    {
@@ -104,8 +119,10 @@ public:
          throw std::runtime_error("TMVA SOFIE Pool op " + Name() + " on a quantized tensor is not supported by the device emission");
       fShapeY = ShapeInference({fShapeX})[0];
       model.AddIntermediateTensor(fNY, fType, fShapeY);
-      fChannelsLast = model.IsChannelsLast(fNX);
+      fChannelsLast = fShapeX.size() == 4 && model.IsChannelsLast(fNX);
       if (fChannelsLast) model.MarkChannelsLast(fNY, fShapeY[1], fShapeY[2], fShapeY[3]);
+      if (fShapeX.size() == 5 && fType != ETensorType::FLOAT)
+         throw std::runtime_error("TMVA SOFIE Pool op " + Name() + " over three spatial axes on a quantized tensor is not supported by the device emission");
    }
    std::string Generate(std::string OpName) override
    {
@@ -114,27 +131,52 @@ public:
          throw std::runtime_error("TMVA SOFIE Pool Op called to Generate without being initialized first");
       std::stringstream out;
       out << "\n//----  operator " << Name() << "  " << OpName << "\n";
-      const auto &a = fAttr;
+      const size_t dims = fShapeX.size() - 2;
+      // a window that lies in the padding entirely has no cell to average
+      if (fPoolMode != MaxPool && !fAttr.count_include_pad)
+         for (size_t i = 0; i < 2 * dims; ++i)
+            if (fAttr.pads[i] >= fAttr.kernel_shape[i % dims])
+               throw std::runtime_error("TMVA SOFIE" + Name() + "Op : a pad as large as the kernel leaves windows without a cell of the image");
+      if (dims == 3) {
+         // three spatial axes (reference :417-470): geometry as arrays, pads in ONNX order
+         auto list = [](const std::vector<size_t> &v) {
+            std::string t = "{";
+            for (size_t i = 0; i < v.size(); ++i) t += (i ? ", " : "") + std::to_string(v[i]);
+            return t + "}";
+         };
+         out << SP << "{\n";
+         out << SP << SP << "const int dims[3] = " << list({fShapeX[2], fShapeX[3], fShapeX[4]}) << ", kernel[3] = " << list(fAttr.kernel_shape)
+             << ", pads[6] = " << list(fAttr.pads) << ", strides[3] = " << list(fAttr.strides) << ";\n";
+         out << SP << SP << "Check(sofie_hip_" << (fPoolMode == MaxPool ? "maxpool3d_f32" : "avgpool3d_f32") << "(fCtx, tensor_" << fNX << ", tensor_"
+             << fNY << ", " << BatchCount(fShapeX[0] * fShapeX[1]) << ", dims, kernel, pads, strides";
+         if (fPoolMode != MaxPool) out << ", " << (fAttr.count_include_pad ? 1 : 0);
+         out << "), \"" << Name() << " " << OpName << "\");\n";
+         out << SP << "}\n";
+         return out.str();
+      }
+      // one spatial axis (reference :329-370) is the two-axis call on [N*C, 1, W] with a 1 x k window
+      struct Geometry2d {
+         size_t H, W, kh, kw, pt, pl, pb, pr, sh, sw;
+      } a;
+      if (dims == 1)
+         a = {1, fShapeX[2], 1, fAttr.kernel_shape[0], 0, fAttr.pads[0], 0, fAttr.pads[1], 1, fAttr.strides[0]};
+      else
+         a = {fShapeX[2], fShapeX[3], fAttr.kernel_shape[0], fAttr.kernel_shape[1], fAttr.pads[0], fAttr.pads[1], fAttr.pads[2],
+              fAttr.pads[3], fAttr.strides[0], fAttr.strides[1]};
       if (fPoolMode != MaxPool) {
-         // a window that lies in the padding entirely has no cell to average
-         if (!a.count_include_pad)
-            for (size_t i = 0; i < 4; ++i)
-               if (a.pads[i] >= a.kernel_shape[i % 2])
-                  throw std::runtime_error("TMVA SOFIE" + Name() + "Op : a pad as large as the kernel leaves windows without a cell of the image");
          out << SP << "Check(sofie_hip_avgpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0] * fShapeX[1])
-             << ", " << fShapeX[2] << ", " << fShapeX[3] << ", " << a.kernel_shape[0] << ", " << a.kernel_shape[1] << ", " << a.pads[0]
-             << ", " << a.pads[1] << ", " << a.pads[2] << ", " << a.pads[3] << ", " << a.strides[0] << ", " << a.strides[1] << ", "
-             << (a.count_include_pad ? 1 : 0) << "), \"" << Name() << " " << OpName << "\");\n";
+             << ", " << a.H << ", " << a.W << ", " << a.kh << ", " << a.kw << ", " << a.pt << ", " << a.pl << ", " << a.pb << ", " << a.pr
+             << ", " << a.sh << ", " << a.sw << ", " << (fAttr.count_include_pad ? 1 : 0) << "), \"" << Name() << " " << OpName << "\");\n";
          return out.str();
       }
       if (fType == ETensorType::FLOAT)
          out << SP << "Check(sofie_hip_maxpool2d_f32(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0] * fShapeX[1])
-             << ", " << fShapeX[2] << ", " << fShapeX[3];
+             << ", " << a.H << ", " << a.W;
       else
          out << SP << "Check(sofie_hip_maxpool2d_s8(fCtx, tensor_" << fNX << ", tensor_" << fNY << ", " << (fChannelsLast ? "SOFIE_LAYOUT_NHWC" : "SOFIE_LAYOUT_NCHW") << ", "
-             << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << fShapeX[2] << ", " << fShapeX[3];
-      out << ", " << a.kernel_shape[0] << ", " << a.kernel_shape[1] << ", " << a.pads[0] << ", " << a.pads[1] << ", " << a.pads[2]
-          << ", " << a.pads[3] << ", " << a.strides[0] << ", " << a.strides[1] << "), \"" << Name() << " " << OpName << "\");\n";
+             << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << a.H << ", " << a.W;
+      out << ", " << a.kh << ", " << a.kw << ", " << a.pt << ", " << a.pl << ", " << a.pb << ", " << a.pr << ", " << a.sh << ", " << a.sw
+          << "), \"" << Name() << " " << OpName << "\");\n";
       return out.str();
    }
 };

@@ -357,6 +357,24 @@ def avgpool2d(x, kernel, strides, pads=(0, 0, 0, 0), count_include_pad=False, ct
     return ctx.ret(y, x)
 
 
+def pool3d(x, kernel, strides, pads=(0, 0, 0, 0, 0, 0), average=False, count_include_pad=False, ctx=None):
+    """fp32 [N, C, D0, D1, D2] max or average pooling; pads = the three begin pads, then the three end pads."""
+    import ctypes as C
+    ctx = ctx or default_context()
+    xd = ctx.dev(x, torch.float32)
+    N, Cc = xd.shape[:2]
+    dims = tuple(xd.shape[2:])
+    out = tuple((dims[i] + pads[i] + pads[3 + i] - kernel[i]) // strides[i] + 1 for i in range(3))
+    y = ctx.empty((N, Cc) + out, torch.float32)
+    arr = lambda v: (C.c_int * len(v))(*[int(e) for e in v])
+    d, k, p, s = arr(dims), arr(kernel), arr(pads), arr(strides)
+    if average:
+        ctx.check(ctx.lib.sofie_hip_avgpool3d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(y), N * Cc, d, k, p, s, int(count_include_pad)))
+    else:
+        ctx.check(ctx.lib.sofie_hip_maxpool3d_f32(ctx.h, ctx.ptr(xd), ctx.ptr(y), N * Cc, d, k, p, s))
+    return ctx.ret(y, x)
+
+
 # ------------------------------------------------------------------------------- int8
 def quantize_f32_s8(x, scale, zp=0, ctx=None):
     ctx = ctx or default_context()

@@ -28,6 +28,8 @@ def all_specs(with_large=True):
     specs.append(models.stacked_spec())
     specs.append(models.conv1d_spec())
     specs.append(models.conv3d_spec())
+    specs.append(models.pool1d_spec())
+    specs.append(models.pool3d_spec())
     specs.append(models.qcnn_rt_spec(oracle))
     specs.append(models.cnn_f32_rt_spec())
     specs.append(models.two_heads_spec()[0])

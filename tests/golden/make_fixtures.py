@@ -11,7 +11,7 @@ What is written:
                                      <name>.ref.hxx headers (numbers only) together with
                                      the input each test feeds (ones / iota / literal list,
                                      from TestCustomModelsFromONNX.cxx:330-349,372-391,
-                                     693-712,860-967,1023-1052,1086-1114,2047-2152); for the Einsum models
+                                     693-712,860-967,992-1085,1086-1114,2047-2152); for the Einsum models
                                      the literal inputs and outputs of the tests themselves
                                      (TestCustomModelsFromONNX.cxx:3028-3103)
 """
@@ -34,7 +34,9 @@ CASES = {
     "ConvWithStridesPadding": ("iota", [1, 1, 7, 5], "all_ones"),
     "ConvWithStridesNoPadding": ("iota", [1, 1, 7, 5], "all_ones"),
     "ConvWithAsymmetricPadding": ("iota", [1, 1, 7, 5], "all_ones"),
+    "MaxPool1d": ("literal", [1, 6, 10], "output"),
     "MaxPool2d": ("literal", [1, 1, 5, 10], "output"),
+    "MaxPool3d": ("literal", [1, 1, 3, 3, 3], "output"),
     "AvgPool": ("literal", [1, 1, 5, 10], "output"),
     "ConvTranspose1d": ("iota", [1, 1, 3], "output"),
     "ConvTranspose2d": ("iota", [1, 1, 3, 3], "output"),
@@ -49,6 +51,24 @@ MAXPOOL2D_INPUT = [
     -0.3421, -1.2364, -0.5805, 0.4421, 1.2184, 0.5043, 1.6823, -1.0483, -2.2798, -1.8927,
     0.7716, 0.0405, 0.3121, -0.3011, -0.3266, -1.9660, 1.0837, 0.2317, 0.9084, -0.3285,
     -0.9398, -0.2065, -0.9499, -0.9739, -0.1288, -0.1375, -1.2612, 0.8810, 0.8506, 0.4455,
+]
+
+
+# Input of the reference's MaxPool1d test (TestCustomModelsFromONNX.cxx:996-1007).
+MAXPOOL1D_INPUT = [
+    0.0907, 0.1029, 0.8143, 1.4497, -0.7785, 0.3825, -0.3764, 1.5785, -0.0835, 0.1622,
+    1.5867, 0.9823, -0.8821, 0.4439, -0.1378, -0.2273, -0.0198, -2.0230, 0.0905, 0.6674,
+    -1.4290, -1.3100, -0.9439, -0.0833, -0.1919, 0.6886, 0.9389, -1.2914, -1.3584, -2.0341,
+    -0.3269, 0.1704, 1.1776, 1.3972, -1.8874, -1.5334, 1.1541, 0.3011, 0.6569, -2.3504,
+    0.4033, 0.1142, 2.2846, -1.3948, -0.8573, 0.5756, -1.0864, 0.2283, 0.8947, 1.7627,
+    -0.1657, 0.0649, -1.6066, 0.4162, -1.1525, -0.8184, 1.1324, -1.1086, 0.1061, 1.0071,
+]
+
+# Input of the reference's MaxPool3d test (TestCustomModelsFromONNX.cxx:1058-1070).
+MAXPOOL3D_INPUT = [
+    -2.6496, 1.0476, -0.5153, 0.3771, 0.4129, -0.3077, -0.8717, -0.8040, -0.3525,
+    -0.1765, -0.3364, 0.8737, -0.2381, -0.8297, 0.4666, 0.6984, -0.6760, 0.6298,
+    1.3833, 0.1101, 0.2039, -0.5477, 0.2341, 0.9181, 0.3842, 0.2428, 1.7924,
 ]
 
 
@@ -89,7 +109,8 @@ def main():
             vals = numbers_of(f.read(), arr)
         entry = {"input_kind": kind, "input_shape": shape, "expected": vals}
         if kind == "literal":
-            entry["input"] = AVGPOOL_INPUT if name == "AvgPool" else MAXPOOL2D_INPUT
+            entry["input"] = {"AvgPool": AVGPOOL_INPUT, "MaxPool1d": MAXPOOL1D_INPUT, "MaxPool2d": MAXPOOL2D_INPUT,
+                              "MaxPool3d": MAXPOOL3D_INPUT}[name]
         expected[name] = entry
     for name, (inputs, answer) in EINSUM_CASES.items():
         shutil.copyfile(os.path.join(REF, name + ".onnx"), os.path.join(HERE, "onnx", name + ".onnx"))

@@ -9,7 +9,7 @@ from sofie_amd import emit, onnx_wire
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 FIXTURES = ["Linear_16", "Linear_32", "Linear_64", "ConvWithPadding", "ConvWithoutPadding",
             "ConvWithAutopadSameLower", "ConvWithStridesPadding", "ConvWithStridesNoPadding",
-            "ConvWithAsymmetricPadding", "MaxPool2d", "AvgPool", "ConvTranspose1d", "ConvTranspose2d", "ConvTransposeBias2d",
+            "ConvWithAsymmetricPadding", "MaxPool1d", "MaxPool2d", "MaxPool3d", "AvgPool", "ConvTranspose1d", "ConvTranspose2d", "ConvTransposeBias2d",
             "ConvTransposeBias2dBatched", "Einsum_matmul", "Einsum_dotprod", "Einsum_3", "Einsum_4"]
 
 
@@ -327,6 +327,46 @@ def conv3d_spec(name="conv3d"):
 def conv3d_reference(oracle):
     p = conv3d_params()
     return oracle.conv3d_f32(p["x"], p["w"], p["b"], (1, 0, 2), (1, 2, 1), (1, 1, 1), 2)
+
+
+# ------------------------------------------------------------------------------------------ pooling over one and three axes
+def pool1d_input(seed=53):
+    return np.random.default_rng(seed).standard_normal((3, 4, 50)).astype(np.float32)
+
+
+def pool1d_spec(name="pool1d"):
+    """MaxPool on [3,4,50] (window 3, pads 1 and 1, stride 2) then AveragePool (window 4, pads 2 and 1, stride 1)."""
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", pool1d_input().shape)
+    s.maxpool("x", "m", (3,), (1, 1), (2,))
+    s.avgpool("m", "y", (4,), (2, 1), (1,))
+    s.set_output("y")
+    return s
+
+
+def pool1d_reference(oracle):
+    m = oracle.maxpool2d(pool1d_input()[:, :, None, :], (1, 3), (1, 2), (0, 1, 0, 1))
+    return oracle.avgpool2d(m, (1, 4), (1, 1), (0, 2, 0, 1))[:, :, 0, :]
+
+
+def pool3d_input(seed=54):
+    return np.random.default_rng(seed).standard_normal((2, 3, 8, 9, 10)).astype(np.float32)
+
+
+def pool3d_spec(name="pool3d"):
+    """MaxPool on [2,3,8,9,10] (window 2x3x2, begin pads 1,0,1, end pads 0,1,0, strides 2,1,2) then AveragePool that
+    counts the padding cells (window 2x2x3, begin pads 0,1,1, end pads 1,0,1, strides 1,2,1)."""
+    s = emit.ModelSpec(name)
+    s.add_input("x", "FLOAT", pool3d_input().shape)
+    s.maxpool("x", "m", (2, 3, 2), (1, 0, 1, 0, 1, 0), (2, 1, 2))
+    s.avgpool("m", "y", (2, 2, 3), (0, 1, 1, 1, 0, 1), (1, 2, 1), count_include_pad=True)
+    s.set_output("y")
+    return s
+
+
+def pool3d_reference(oracle):
+    m = oracle.pool3d(pool3d_input(), (2, 3, 2), (2, 1, 2), (1, 0, 1, 0, 1, 0))
+    return oracle.pool3d(m, (2, 2, 3), (1, 2, 1), (0, 1, 1, 1, 0, 1), average=True, count_include_pad=True)
 
 
 # ------------------------------------------------------------------------------------------ four-value model for SofieFunctor

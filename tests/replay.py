@@ -1,7 +1,7 @@
 """Replay a decoded ONNX graph (Gemm / Relu / Conv / ConvTranspose / Einsum / MaxPool / Flatten) through a backend.
 
 A backend is any object with the methods gemm_f32, relu_f32, conv2d_f32, conv_transpose2d_f32, einsum_f32 and maxpool2d
-taking and returning numpy arrays: the CPU oracle module, or the HIP library wrapper.
+(pool3d for pooling over three axes) taking and returning numpy arrays: the CPU oracle module, or the HIP library wrapper.
 The attribute handling restates what the reference's operators do at Initialize time.
 """
 import numpy as np
@@ -87,13 +87,22 @@ def run_graph(graph, feeds, backend):
         elif op == "Einsum":
             eq = a["equation"]
             y = backend.einsum_f32(eq.decode() if isinstance(eq, bytes) else eq, [env[i] for i in ins])
-        elif op == "MaxPool":
-            y = backend.maxpool2d(env[ins[0]], tuple(a["kernel_shape"]),
-                                  tuple(a.get("strides", [1, 1])),
-                                  tuple(a.get("pads", [0, 0, 0, 0])))
-        elif op == "AveragePool":
-            y = backend.avgpool2d(env[ins[0]], tuple(a["kernel_shape"]), tuple(a.get("strides", [1, 1])),
-                                  tuple(a.get("pads", [0, 0, 0, 0])), bool(a.get("count_include_pad", 0)))
+        elif op in ("MaxPool", "AveragePool"):
+            # one spatial axis runs as two with a height of one, three through the backend's pool3d
+            x = env[ins[0]]
+            dim = x.ndim - 2
+            k = tuple(a["kernel_shape"])
+            st = tuple(a.get("strides", [1] * dim))
+            pads = tuple(a.get("pads", [0] * (2 * dim)))
+            include = bool(a.get("count_include_pad", 0))
+            if dim == 3:
+                y = backend.pool3d(x, k, st, pads, average=op == "AveragePool", count_include_pad=include)
+            else:
+                if dim == 1:
+                    x, k, st, pads = x[:, :, None, :], (1,) + k, (1,) + st, (0, pads[0], 0, pads[1])
+                y = backend.maxpool2d(x, k, st, pads) if op == "MaxPool" else backend.avgpool2d(x, k, st, pads, include)
+                if dim == 1:
+                    y = y[:, :, 0, :]
         elif op == "GlobalAveragePool":
             x = env[ins[0]]
             y = backend.avgpool2d(x, tuple(x.shape[2:]), (1, 1))

@@ -529,6 +529,37 @@ def test_runtime_batch_session(tmp_path):
     assert "sofie_hip_gemm_f32(fCtx, 0, 0, 6, 3, 4," in c and "fBatch" not in c
 
 
+def test_pool_1d_and_3d_emission(tmp_path):
+    """Pooling over one spatial axis (ROperator_Pool.hxx:329-370) is emitted as the two-axis call on a plane of height
+    one; over three axes (:417-470) as the calls that take the geometry as arrays, pads in ONNX order."""
+    c = open(models.pool1d_spec("p1d_t").generate(str(tmp_path))[0]).read()
+    # [3,4,50] -> (50 + 2 - 3) / 2 + 1 = 25 -> (25 + 3 - 4) + 1 = 25
+    assert "sofie_hip_maxpool2d_f32(fCtx, tensor_x, tensor_m, 12, 1, 50, 1, 3, 0, 1, 0, 1, 1, 2)" in c
+    assert "sofie_hip_avgpool2d_f32(fCtx, tensor_m, tensor_y, 12, 1, 25, 1, 4, 0, 2, 0, 1, 1, 1, 0)" in c
+    assert "std::vector<float> ret(300);" in c
+    c = open(models.pool3d_spec("p3d_t").generate(str(tmp_path))[0]).read()
+    assert "const int dims[3] = {8, 9, 10}, kernel[3] = {2, 3, 2}, pads[6] = {1, 0, 1, 0, 1, 0}, strides[3] = {2, 1, 2};" in c
+    assert "sofie_hip_maxpool3d_f32(fCtx, tensor_x, tensor_m, 6, dims, kernel, pads, strides)" in c
+    # (8 + 1 - 2) / 2 + 1 = 4, (9 + 1 - 3) + 1 = 8, (10 + 1 - 2) / 2 + 1 = 5
+    assert "const int dims[3] = {4, 8, 5}, kernel[3] = {2, 2, 3}, pads[6] = {0, 1, 1, 1, 0, 1}, strides[3] = {1, 2, 1};" in c
+    assert "sofie_hip_avgpool3d_f32(fCtx, tensor_m, tensor_y, 6, dims, kernel, pads, strides, 1)" in c
+    # (4 + 1 - 2) + 1 = 4, (8 + 1 - 2) / 2 + 1 = 4, (5 + 2 - 3) + 1 = 5
+    assert "std::vector<float> ret(%d);" % (2 * 3 * 4 * 4 * 5) in c
+    # refused at generation time: a kernel of the wrong rank, an average over inside cells with a pad as large as the window
+    s = emit.ModelSpec("p3d_bad")
+    s.add_input("x", "FLOAT", (1, 1, 4, 4, 4))
+    s.maxpool("x", "y", (2, 2), (0, 0, 0, 0), (1, 1))
+    s.set_output("y")
+    with pytest.raises(RuntimeError, match="invalid inputs"):
+        s.generate(str(tmp_path))
+    s = emit.ModelSpec("p1d_bad")
+    s.add_input("x", "FLOAT", (1, 1, 9))
+    s.avgpool("x", "y", (2,), (2, 0), (1,))
+    s.set_output("y")
+    with pytest.raises(RuntimeError, match="without a cell"):
+        s.generate(str(tmp_path))
+
+
 def test_conv_1d_and_3d_emission(tmp_path):
     """One spatial dimension runs as the 2-D call with a height of one; three as the 3-D call. Absent pads mean one
     on every side of every dimension, as in the reference (ROperator_Conv.hxx:136-139)."""

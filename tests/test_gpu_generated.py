@@ -132,6 +132,18 @@ def test_conv_1d_and_3d_sessions(tmp_path):
     assert y.size == ref.size and np.array_equal(y, ref.reshape(-1))
 
 
+def test_pooling_over_one_and_three_axes_sessions(tmp_path):
+    """MaxPool and AveragePool on [N,C,W] (the two-axis kernels with a height of one) and on [N,C,D,H,W] (kernels of
+    their own) with begin pads that differ from the end pads: the maximum is exact, the average sums in the oracle's
+    order and is exact too."""
+    y = run_session("pool1d", models.pool1d_input(), tmp_path)
+    ref = models.pool1d_reference(oracle)
+    assert y.size == ref.size and np.array_equal(y, ref.reshape(-1))
+    y = run_session("pool3d", models.pool3d_input(), tmp_path)
+    ref = models.pool3d_reference(oracle)
+    assert y.size == ref.size and np.array_equal(y, ref.reshape(-1))
+
+
 def test_conv_batchnorm_convtranspose_session(tmp_path):
     """Conv -> BatchNormalization -> Relu (folded into the convolution at generation time) -> MaxPool ->
     BatchNormalization (its own kernel) -> ConvTranspose -> Relu against the unfused oracle steps; 1e-5 relative

@@ -279,6 +279,35 @@ def test_relu_and_maxpool_f32(ops):
         assert np.array_equal(ops.maxpool2d(x, k, s, p), oracle.maxpool2d(x, k, s, p))
 
 
+@pytest.mark.parametrize("cfg", [
+    dict(shape=(2, 3, 6, 7, 8), k=(2, 3, 2), s=(2, 1, 2), p=(0, 0, 0, 0, 0, 0)),
+    dict(shape=(1, 2, 5, 5, 5), k=(3, 3, 3), s=(1, 1, 1), p=(1, 1, 1, 1, 1, 1)),
+    dict(shape=(3, 5, 9, 6, 11), k=(2, 2, 4), s=(1, 2, 3), p=(1, 0, 2, 0, 1, 3)),
+    dict(shape=(1, 1, 4, 4, 4), k=(4, 4, 4), s=(1, 1, 1), p=(0, 0, 0, 0, 0, 0)),        # the global pooling
+])
+def test_pool3d_f32(ops, cfg):
+    """Max and average pooling over three spatial axes against the oracle: the maximum exactly, the average exactly too
+    (same order of additions, one division), with padding cells counted and not."""
+    x = rng(60 + cfg["shape"][4]).standard_normal(cfg["shape"]).astype(np.float32)
+    assert np.array_equal(ops.pool3d(x, cfg["k"], cfg["s"], cfg["p"]), oracle.pool3d(x, cfg["k"], cfg["s"], cfg["p"]))
+    for include in (False, True):
+        y = ops.pool3d(x, cfg["k"], cfg["s"], cfg["p"], average=True, count_include_pad=include)
+        assert np.array_equal(y, oracle.pool3d(x, cfg["k"], cfg["s"], cfg["p"], average=True, count_include_pad=include))
+
+
+def test_pool3d_refuses_what_it_cannot_do(ops):
+    import ctypes as C
+    from sofie_amd import lib as L
+    ctx = ops.default_context()
+    x = ctx.dev(np.zeros((1, 1, 4, 4, 4), np.float32))
+    y = ctx.empty((1, 1, 4, 4, 4), torch.float32)
+    arr = lambda *v: (C.c_int * len(v))(*v)
+    # kernel larger than the padded volume; a pad as large as the window for an average over inside cells only
+    assert ctx.lib.sofie_hip_maxpool3d_f32(ctx.h, ctx.ptr(x), ctx.ptr(y), 1, arr(4, 4, 4), arr(5, 1, 1), arr(0, 0, 0, 0, 0, 0), arr(1, 1, 1)) == L.EINVAL
+    assert ctx.lib.sofie_hip_avgpool3d_f32(ctx.h, ctx.ptr(x), ctx.ptr(y), 1, arr(4, 4, 4), arr(2, 2, 2), arr(2, 0, 0, 0, 0, 0), arr(1, 1, 1), 0) == L.EINVAL
+    assert ctx.lib.sofie_hip_avgpool3d_f32(ctx.h, ctx.ptr(x), ctx.ptr(y), 1, arr(4, 4, 4), arr(2, 2, 2), arr(0, 0, 0, 0, 0, 0), arr(1, 0, 1), 0) == L.EINVAL
+
+
 # --------------------------------------------------------------------------- int8
 def test_quantize_dequantize(ops):
     r = rng(11)

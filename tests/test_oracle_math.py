@@ -607,3 +607,36 @@ def test_avgpool2d_against_torch_and_float64(cfg):
             r0, c0 = oh * cfg["s"][0] - pt, ow * cfg["s"][1] - pl
             win = x[0, 0, max(r0, 0):min(r0 + cfg["k"][0], H), max(c0, 0):min(c0 + cfg["k"][1], W)].astype(np.float64)
             assert abs(y[0, 0, oh, ow] - win.mean()) <= 1e-6 * max(1.0, abs(win.mean()))
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(shape=(2, 3, 6, 7, 8), k=(2, 3, 2), s=(2, 1, 2), p=(0, 0, 0, 0, 0, 0)),
+    dict(shape=(1, 2, 5, 5, 5), k=(3, 3, 3), s=(1, 1, 1), p=(1, 1, 1, 1, 1, 1)),
+    dict(shape=(2, 2, 7, 6, 9), k=(2, 2, 4), s=(1, 2, 3), p=(1, 0, 2, 1, 0, 2)),
+    dict(shape=(1, 3, 6, 5, 7), k=(3, 2, 2), s=(2, 2, 1), p=(2, 0, 1, 0, 1, 0)),      # begin pads differ from end pads
+])
+def test_pool3d_against_torch_and_float64(cfg):
+    """or_pool3d_f32: the maximum against torch's max_pool3d on the tensor padded with -inf by the six ONNX pads; the
+    average with count_include_pad against avg_pool3d on the tensor padded with zeros, without it against avg_pool3d
+    where the pads are symmetric (what torch takes) and against a float64 mean of the cells inside the volume."""
+    r = rng(700 + cfg["shape"][2] + cfg["k"][2])
+    x = r.standard_normal(cfg["shape"]).astype(np.float32)
+    p = cfg["p"]
+    tpad = (p[2], p[5], p[1], p[4], p[0], p[3])      # torch pads the last axis first
+    xt = torch.from_numpy(x)
+    ym = oracle.pool3d(x, cfg["k"], cfg["s"], p)
+    tm = F.max_pool3d(F.pad(xt, tpad, value=float("-inf")), cfg["k"], cfg["s"]).numpy()
+    assert ym.shape == tm.shape and np.array_equal(ym, tm)
+    ya = oracle.pool3d(x, cfg["k"], cfg["s"], p, average=True, count_include_pad=True)
+    ta = F.avg_pool3d(F.pad(xt.double(), tpad), cfg["k"], cfg["s"]).numpy()
+    assert ya.shape == ta.shape and np.max(np.abs(ya - ta)) <= 1e-6 * max(np.max(np.abs(ta)), 1.0)
+    yb = oracle.pool3d(x, cfg["k"], cfg["s"], p, average=True, count_include_pad=False)
+    if p[:3] == p[3:]:
+        tb = F.avg_pool3d(xt.double(), cfg["k"], cfg["s"], p[:3], count_include_pad=False).numpy()
+        assert np.max(np.abs(yb - tb)) <= 1e-6 * max(np.max(np.abs(tb)), 1.0)
+    D = cfg["shape"][2:]
+    for idx in np.ndindex(*yb.shape[2:]):
+        lo = [idx[i] * cfg["s"][i] - p[i] for i in range(3)]
+        win = x[0, 0, max(lo[0], 0):min(lo[0] + cfg["k"][0], D[0]), max(lo[1], 0):min(lo[1] + cfg["k"][1], D[1]),
+                max(lo[2], 0):min(lo[2] + cfg["k"][2], D[2])].astype(np.float64)
+        assert abs(yb[(0, 0) + idx] - win.mean()) <= 1e-6 * max(1.0, abs(win.mean()))
