@@ -276,14 +276,13 @@ __global__ void __launch_bounds__(256) k_conv2d_f32(ConvArgs g)
 // (buffer_load ... lds) under the matrix loop of block c. The weights come from a copy laid out for it, wt [group]
 // [K = input channel, tap][wstride >= OC/groups, a multiple of 4] (k_transpose_weights / k_gather_phase_weights write it
 // into the scratch buffer in front of the launch), so that a row of the LDS tile [KC][BOC] is a contiguous piece of a
-// row of wt and goes 16 bytes per lane; odd rows are rotated by 32 columns, which puts the two K halves of a fragment
-// read on different banks without padding. A patch cell is 4 bytes per lane from wherever it sits in the image;
+// row of wt and goes 16 bytes per lane. A patch cell is 4 bytes per lane from wherever it sits in the image;
 // padding cells ask for an offset outside the descriptor's range and receive 0. Nothing of a block depends on the
 // block but a uniform offset, so a thread keeps NP patch offsets and one weight offset for the whole kernel.
 // PHASES: the launch holds the output phases of a strided transposed convolution (blockIdx.z = image * nphases +
 // phase). A phase is a plain unit-stride convolution of the input with its sub-kernel (g.w then holds the sub-kernels
 // in the order above, one after the other) whose outputs go to every stride-th pixel of the output plane.
-template <int TI, int TJ, bool PHASES = false>
+template <int TI, int TJ, bool PHASES = false, int KWT = 0>
 __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArgs gg)
 {
    constexpr int BOC = 2 * TI * 32, BP = 2 * TJ * 32;
@@ -340,17 +339,19 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    const int wstride = (g.ocg + 3) & ~3;
    const size_t HW = (size_t)g.H * g.W;
 
-   for (int k = tid; k < g.KC; k += 256) {
-      const int icl = k / KHW, t = k % KHW;
-      const int kh = t / g.KW, kw = t % g.KW;
-      koff[k] = (icl * g.PH + kh * g.dh) * g.PW + kw * g.dw;
-   }
+   if constexpr (KWT == 0)
+      for (int k = tid; k < g.KC; k += 256) {
+         const int icl = k / KHW, t = k % KHW;
+         const int kh = t / g.KW, kw = t % g.KW;
+         koff[k] = (icl * g.PH + kh * g.dh) * g.PW + kw * g.dw;
+      }
    int base[TJ];
 #pragma unroll
    for (int j = 0; j < TJ; ++j) {
       const int p = p0 + wn * TJ * 32 + j * 32 + fr;
       const int row = fdiv(p, dOW);
       base[j] = (p < OHW) ? ((row - oh0) * g.sh) * g.PW + (p - row * g.OW) * g.sw : 0;
+      if constexpr (KWT > 0) base[j] += fk * g.PH * g.PW;
    }
    v16f acc[TI][TJ];
 #pragma unroll
@@ -379,7 +380,7 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
       pofs[u] = inside ? (unsigned)(((icl * g.H + ih) * g.W + iw) * 4) : OUTSIDE;
    }
    const int wrow0 = tid / (BOC / 4);
-   const int wcol = ((tid % (BOC / 4)) * 4 - 32 * (wrow0 & 1)) & (BOC - 1);     // column the rotated cell holds
+   const int wcol = (tid % (BOC / 4)) * 4;
    const unsigned wofs = oc0 + wcol < wstride ? (unsigned)((wrow0 * wstride + oc0 + wcol) * 4) : OUTSIDE;
    const unsigned xblock = (unsigned)(g.ICB * HW * 4), wblock = (unsigned)(g.KC * wstride * 4);
    const unsigned wstep = (unsigned)(ROWS_PER_REQUEST * wstride * 4);
@@ -397,28 +398,56 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
 
    const int nblocks = g.icg / g.ICB;
    const int nsteps = p0 + wn * TJ * 32 < OHW ? g.KC / 2 : 0;   // a wavefront with no pixel of the plane multiplies nothing
-   int wcolr[TI];     // this lane's column of the weight tile, rotated as the rows of its K half (odd: fk = 1) are
-#pragma unroll
-   for (int i = 0; i < TI; ++i) wcolr[i] = (wm * TI * 32 + i * 32 + fr + 32 * fk) & (BOC - 1);
    request(0, 0);
    wait_vmcnt<0>();
    __syncthreads();   // block 0 and the koff table are in LDS
    for (int c = 0; c < nblocks; ++c) {
       if (c + 1 < nblocks) request(c + 1, (c + 1) & 1);
       const float *const sW = bufs + (c & 1) * buf_len, *const patch = sW + g.KC * BOC;
-      for (int s = 0; s < nsteps; ++s) {
-         const int kk = 2 * s + fk;
-         const int ko = koff[kk];
-         float fa[TI], fb[TJ];
+      if constexpr (KWT > 0) {
+         // K runs (channel pair, kernel row, kernel column, channel of the pair): the two K values of a matrix
+         // instruction are the same tap of two neighbouring channels, so a lane's patch address is its own constant
+         // (pixel, channel of the pair) plus a uniform offset per kernel row, and the kernel's columns are immediate
+         // offsets: no table of offsets, three vector additions per kernel row
+         const float *wl = sW + fk * BOC + wm * TI * 32 + fr;
+         if (nsteps > 0)
+            for (int m = 0; m < g.ICB / 2; ++m)
+               for (int kh = 0; kh < g.KH; ++kh) {
+                  const int row = __builtin_amdgcn_readfirstlane((2 * m * g.PH + kh * g.dh) * g.PW);
+                  const float *pb[TJ];
 #pragma unroll
-         for (int i = 0; i < TI; ++i) fa[i] = sW[kk * BOC + wcolr[i]];
+                  for (int j = 0; j < TJ; ++j) pb[j] = patch + base[j] + row;
 #pragma unroll
-         for (int j = 0; j < TJ; ++j) fb[j] = patch[base[j] + ko];
+                  for (int kw = 0; kw < KWT; ++kw) {
+                     float fa[TI], fb[TJ];
 #pragma unroll
-         for (int i = 0; i < TI; ++i)
+                     for (int i = 0; i < TI; ++i) fa[i] = wl[kw * 2 * BOC + i * 32];
 #pragma unroll
-            for (int j = 0; j < TJ; ++j)
-               acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                     for (int j = 0; j < TJ; ++j) fb[j] = pb[j][kw];
+#pragma unroll
+                     for (int i = 0; i < TI; ++i)
+#pragma unroll
+                        for (int j = 0; j < TJ; ++j)
+                           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+                  }
+                  wl += KWT * 2 * BOC;
+               }
+      } else {
+         const float *wl = sW + wm * TI * 32 + fr;
+         for (int s = 0; s < nsteps; ++s) {
+            const int kk = 2 * s + fk;
+            const int ko = koff[kk];
+            float fa[TI], fb[TJ];
+#pragma unroll
+            for (int i = 0; i < TI; ++i) fa[i] = wl[kk * BOC + i * 32];
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) fb[j] = patch[base[j] + ko];
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+               for (int j = 0; j < TJ; ++j)
+                  acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+         }
       }
       // the next block has landed (this wavefront's requests; the barrier makes it every wavefront's), and the
       // buffer it replaces next was last read in this block
@@ -464,19 +493,23 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
 }
 
 // Weights of a plain convolution w [OC][C/groups][KH][KW] as k_conv2d_f32_dma reads them: wt [group][K][wstride],
-// K = (input channel, tap), wstride = OC/groups rounded up to 4 (the cells behind the last channel are 0).
-__global__ void k_transpose_weights(const float *w, float *wt, int groups, int ocg, int Kfull, int wstride)
+// K = (input channel, tap), or (channel pair, tap, channel of the pair) with `pairs`; wstride = OC/groups rounded up
+// to 4 (the cells behind the last channel are 0).
+__global__ void k_transpose_weights(const float *w, float *wt, int groups, int ocg, int Kfull, int wstride, int pairs, int KHW)
 {
    const int e = blockIdx.x * blockDim.x + threadIdx.x;
    if (e >= groups * Kfull * wstride) return;
-   const int oc = e % wstride, k = (e / wstride) % Kfull, grp = e / (wstride * Kfull);
+   const int oc = e % wstride, grp = e / (wstride * Kfull);
+   int k = (e / wstride) % Kfull;
+   if (pairs) k = (2 * (k / (2 * KHW)) + (k & 1)) * KHW + (k >> 1) % KHW;
    wt[e] = oc < ocg ? w[((size_t)grp * ocg + oc) * Kfull + k] : 0.0f;
 }
 
 // Sub-kernels of the output phases of a strided transposed convolution, gathered from its weights w [C, OC/groups, KH0,
-// KW0] into the order k_conv2d_f32_dma reads: phase after phase, each [groups][K = input channel, tap][wstride] with
-// tap (a, b) = element (th0 + a*ths, tw0 + b*tws) of the kernel and zeros behind the last channel. One thread per value.
-__global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total, int wstride)
+// KW0] into the order k_conv2d_f32_dma reads: phase after phase, each [groups][K = input channel, tap][wstride] (K =
+// (channel pair, tap, channel of the pair) with `pairs`) with tap (a, b) = element (th0 + a*ths, tw0 + b*tws) of the
+// kernel and zeros behind the last channel. One thread per value.
+__global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total, int wstride, int pairs)
 {
    const int e = blockIdx.x * blockDim.x + threadIdx.x;
    if (e >= total) return;
@@ -490,10 +523,20 @@ __global__ void k_gather_phase_weights(ConvArgs g, float *dst, int total, int ws
       if (pi == i) q = g.phase[i];
    int r = e - q.woff;
    const int oc = r % wstride; r /= wstride;
-   const int b = r % q.KW; r /= q.KW;
-   const int a = r % q.KH; r /= q.KH;
-   const int ic = r % g.icg;
-   const int grp = r / g.icg;
+   int a, b, ic;
+   if (pairs) {      // K = (channel pair, tap, channel of the pair)
+      const int parity = r & 1; r >>= 1;
+      b = r % q.KW; r /= q.KW;
+      a = r % q.KH; r /= q.KH;
+      ic = 2 * (r % (g.icg / 2)) + parity;
+      r /= g.icg / 2;
+   } else {
+      b = r % q.KW; r /= q.KW;
+      a = r % q.KH; r /= q.KH;
+      ic = r % g.icg;
+      r /= g.icg;
+   }
+   const int grp = r;
    dst[e] = oc < g.ocg ? g.w[((((size_t)grp * g.icg + ic) * g.ocg + oc) * g.KH0 + q.th0 + a * g.ths) * g.KW0 + q.tw0 + b * g.tws]
                        : 0.0f;
 }
@@ -586,30 +629,48 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
       const size_t wt_floats = (size_t)g.groups * g.icg * KHW * wstride;
       const size_t budget = dma_lds_budget(ctx, (size_t)cdiv(OHW, BP) * g.groups * octiles * g.N, TI == 1 ? 7 : 3);
       if ((size_t)g.icg * HW * 4 < (1u << 30) && (size_t)g.icg * KHW * wstride * 4 < (1u << 30) &&
-          (size_t)g.ocg * OHW * 4 < (1u << 30))
-         for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
-            const int kc = icb * KHW;
-            const size_t plen = (size_t)icb * g.PH * g.PW;
-            const size_t lds = dma_lds_bytes(kc, plen, BOC);
-            if (kc < 18) break;
-            if (g.icg % icb != 0 || kc % 2 != 0 || lds > budget || plen > SOFIE_CONV_DMA_PATCH) continue;
+          (size_t)g.ocg * OHW * 4 < (1u << 30)) {
+         auto pick = [&](bool even) {
+            for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
+               const int kc = icb * KHW;
+               if (kc < 18) break;
+               if (g.icg % icb != 0 || kc % 2 != 0 || (even && icb % 2 != 0) ||
+                   dma_lds_bytes(kc, (size_t)icb * g.PH * g.PW, BOC) > budget || (size_t)icb * g.PH * g.PW > SOFIE_CONV_DMA_PATCH)
+                  continue;
+               return icb;
+            }
+            return 0;
+         };
+         // kernels 2 or 3 columns wide without dilation along them run without the table of patch offsets, on even
+         // channel blocks with K ordered by channel pairs
+         const int kwt = (g.KW == 2 || g.KW == 3) && g.dw == 1 ? g.KW : 0;
+         int icb = kwt ? pick(true) : 0;
+         const bool pairs = icb > 0;
+         if (!icb) icb = pick(false);
+         if (icb) {
             g.ICB = icb;
-            g.KC = kc;
+            g.KC = icb * KHW;
             g.dPW = make_fastdiv((unsigned)g.PW);
             g.dPH = make_fastdiv((unsigned)g.PH);
             void *ws = nullptr;
             if (int rc = workspace(ctx, wt_floats * sizeof(float), &ws)) return rc;
             hipLaunchKernelGGL(k_transpose_weights, dim3((unsigned)((wt_floats + 255) / 256)), dim3(256), 0, ctx->stream, g.w,
-                               static_cast<float *>(ws), g.groups, g.ocg, g.icg * KHW, wstride);
+                               static_cast<float *>(ws), g.groups, g.ocg, g.icg * KHW, wstride, pairs ? 1 : 0, KHW);
             if (int rc = check_launch(ctx, "k_transpose_weights")) return rc;
             ConvArgs h = g;
             h.w = static_cast<const float *>(ws);
-            constexpr auto kern = k_conv2d_f32_dma<TI, TJ>;
-            SOFIE_LARGE_LDS(kern);
-            hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256), lds, ctx->stream, h);
+            constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, false, 0>, kern2 = k_conv2d_f32_dma<TI, TJ, false, 2>,
+                           kern3 = k_conv2d_f32_dma<TI, TJ, false, 3>;
+            SOFIE_LARGE_LDS(kern0);
+            SOFIE_LARGE_LDS(kern2);
+            SOFIE_LARGE_LDS(kern3);
+            const auto kern = !pairs ? kern0 : kwt == 2 ? kern2 : kern3;
+            hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256),
+                               dma_lds_bytes(g.KC, (size_t)icb * g.PH * g.PW, BOC), ctx->stream, h);
             *done = true;
-            return check_launch(ctx, "k_conv2d_f32_dma");
+            return check_launch(ctx, pairs ? "k_conv2d_f32_dma_pairs" : "k_conv2d_f32_dma");
          }
+      }
    }
    int icb = 96 / KHW;
    if (icb < 1) icb = 1;
@@ -665,47 +726,63 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
       const size_t budget = dma_lds_budget(ctx, workgroups, TI == 1 ? 7 : 3);
       const int wstride = (g.ocg + 3) & ~3;
       bool fits = (size_t)g.icg * g.H * g.W * 4 < (1u << 30) && (size_t)g.ocg * g.OH0 * g.OW0 * 4 < (1u << 30);
+      // every phase 2 (or every phase 3) columns wide: the table-free loop on even channel blocks, K by channel pairs
+      int kwt = g.phase[0].KW == 2 || g.phase[0].KW == 3 ? g.phase[0].KW : 0;
+      for (int i = 1; i < g.nphases; ++i)
+         if (g.phase[i].KW != kwt) kwt = 0;
       int woff = 0;
-      for (int i = 0; i < g.nphases && fits; ++i) {
-         PhaseArgs &p = g.phase[i];
-         const int KHW = p.KH * p.KW;
-         p.rows_out = (BP + p.OW - 2) / p.OW + 1;
-         if (p.rows_out > p.OH) p.rows_out = p.OH;
-         p.PH = (p.rows_out - 1) + (p.KH - 1) + 1;      // unit stride and dilation inside a phase
-         p.PW = (p.OW - 1) + (p.KW - 1) + 1;
-         bool found = false;
-         for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1 && !found; --icb) {
-            const int kc = icb * KHW;
-            const size_t plen = (size_t)icb * p.PH * p.PW;
-            const size_t lds = dma_lds_bytes(kc, plen, BOC);
-            if (kc < 16) break;
-            if (g.icg % icb != 0 || kc % 2 != 0 || lds > budget || plen > SOFIE_CONV_DMA_PATCH) continue;
-            p.ICB = icb;
-            p.KC = kc;
-            p.dPW = make_fastdiv((unsigned)p.PW);
-            p.dPH = make_fastdiv((unsigned)p.PH);
-            p.dOW = make_fastdiv((unsigned)p.OW);
-            if (lds > lds_max) lds_max = lds;
-            found = true;
+      auto plan = [&](bool even) {
+         bool ok = fits;
+         woff = 0;
+         lds_max = 0;
+         tiles_max = 0;
+         for (int i = 0; i < g.nphases && ok; ++i) {
+            PhaseArgs &p = g.phase[i];
+            const int KHW = p.KH * p.KW;
+            p.rows_out = (BP + p.OW - 2) / p.OW + 1;
+            if (p.rows_out > p.OH) p.rows_out = p.OH;
+            p.PH = (p.rows_out - 1) + (p.KH - 1) + 1;      // unit stride and dilation inside a phase
+            p.PW = (p.OW - 1) + (p.KW - 1) + 1;
+            bool found = false;
+            for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1 && !found; --icb) {
+               const int kc = icb * KHW;
+               const size_t plen = (size_t)icb * p.PH * p.PW;
+               const size_t lds = dma_lds_bytes(kc, plen, BOC);
+               if (kc < 16) break;
+               if (g.icg % icb != 0 || kc % 2 != 0 || (even && icb % 2 != 0) || lds > budget || plen > SOFIE_CONV_DMA_PATCH) continue;
+               p.ICB = icb;
+               p.KC = kc;
+               p.dPW = make_fastdiv((unsigned)p.PW);
+               p.dPH = make_fastdiv((unsigned)p.PH);
+               p.dOW = make_fastdiv((unsigned)p.OW);
+               if (lds > lds_max) lds_max = lds;
+               found = true;
+            }
+            ok = found && (size_t)g.icg * KHW * wstride * 4 < (1u << 30);
+            p.woff = woff;
+            woff += g.groups * g.icg * KHW * wstride;       // a multiple of 4 floats
+            if (cdiv(p.OH * p.OW, BP) > tiles_max) tiles_max = cdiv(p.OH * p.OW, BP);
          }
-         fits = found && (size_t)g.icg * KHW * wstride * 4 < (1u << 30);
-         p.woff = woff;
-         woff += g.groups * g.icg * KHW * wstride;       // a multiple of 4 floats
-         if (cdiv(p.OH * p.OW, BP) > tiles_max) tiles_max = cdiv(p.OH * p.OW, BP);
-      }
-      if (fits) {
+         return ok;
+      };
+      const bool pairs = kwt && plan(true);
+      if (pairs || plan(false)) {
          void *ws = nullptr;
          if (int rc = workspace(ctx, (size_t)woff * sizeof(float), &ws)) return rc;
          hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
-                            static_cast<float *>(ws), woff, wstride);
+                            static_cast<float *>(ws), woff, wstride, pairs ? 1 : 0);
          if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
          ConvArgs h = g;
          h.w = static_cast<const float *>(ws);
-         constexpr auto kern = k_conv2d_f32_dma<TI, TJ, true>;
-         SOFIE_LARGE_LDS(kern);
+         constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, true, 0>, kern2 = k_conv2d_f32_dma<TI, TJ, true, 2>,
+                        kern3 = k_conv2d_f32_dma<TI, TJ, true, 3>;
+         SOFIE_LARGE_LDS(kern0);
+         SOFIE_LARGE_LDS(kern2);
+         SOFIE_LARGE_LDS(kern3);
+         const auto kern = !pairs ? kern0 : kwt == 2 ? kern2 : kern3;
          hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
          *done = true;
-         return check_launch(ctx, "k_conv2d_f32_dma_phases");
+         return check_launch(ctx, pairs ? "k_conv2d_f32_dma_pairs_phases" : "k_conv2d_f32_dma_phases");
       }
       lds_max = 0;
       tiles_max = 0;

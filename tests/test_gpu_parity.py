@@ -224,16 +224,22 @@ def _kernels_of(ops, call):
     # channel counts that are no multiple of 4 (the copied weights' rows are padded), a ragged second channel tile,
     # groups, a stride and a dilation, asymmetric pads, one or several patch requests per thread, a nearly empty last
     # pixel tile, a grid small enough for more than three workgroups per compute unit
-    dict(N=3, C=16, H=20, W=20, OC=70, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1),
-    dict(N=2, C=16, H=9, W=19, OC=98, k=(3, 3), p=(1, 1), s=(2, 2), d=(1, 1), g=2),
-    dict(N=1, C=8, H=12, W=12, OC=130, k=(3, 3), p=(3, 0, 1, 4), s=(1, 1), d=(2, 2), g=1),
-    dict(N=2, C=64, H=56, W=56, OC=128, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1),
-    dict(N=5, C=24, H=17, W=33, OC=33, k=(5, 2), p=(2, 0, 2, 1), s=(1, 1), d=(1, 1), g=1),
-    dict(N=40, C=32, H=6, W=6, OC=64, k=(1, 1), p=(0, 0), s=(1, 1), d=(1, 1), g=1),
+    # ... kernels 3 and 2 columns wide take the loop without a table of offsets (K ordered by channel pairs); a dilation,
+    # a 1x1 kernel, an odd number of channels per group and a kernel 5 columns wide take the general loop
+    dict(N=3, C=16, H=20, W=20, OC=70, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, pairs=True),
+    dict(N=2, C=16, H=9, W=19, OC=98, k=(3, 3), p=(1, 1), s=(2, 2), d=(1, 1), g=2, pairs=True),
+    dict(N=1, C=8, H=12, W=12, OC=130, k=(3, 3), p=(3, 0, 1, 4), s=(1, 1), d=(2, 2), g=1, pairs=False),
+    dict(N=2, C=64, H=56, W=56, OC=128, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, pairs=True),
+    dict(N=5, C=24, H=17, W=33, OC=33, k=(5, 2), p=(2, 0, 2, 1), s=(1, 1), d=(1, 1), g=1, pairs=True),
+    dict(N=2, C=12, H=14, W=11, OC=40, k=(2, 3), p=(0, 1, 1, 1), s=(1, 2), d=(2, 1), g=2, pairs=True),
+    dict(N=40, C=32, H=6, W=6, OC=64, k=(1, 1), p=(0, 0), s=(1, 1), d=(1, 1), g=1, pairs=False),
+    dict(N=3, C=9, H=13, W=10, OC=20, k=(2, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, pairs=False),
+    dict(N=2, C=4, H=11, W=16, OC=8, k=(2, 5), p=(1, 2, 0, 2), s=(1, 1), d=(1, 1), g=1, pairs=False),
 ])
 def test_conv2d_f32_operands_by_lds_dma(ops, cfg):
     """The kernel that fetches both operands by LDS-DMA from weights copied into the [K][channel] order: the trace names
-    it, and its results are the oracle's within the fp32 tolerance (1e-5 relative), with and without bias and ReLU."""
+    it (and which of its two matrix loops ran), and its results are the oracle's within the fp32 tolerance (1e-5
+    relative), with and without bias and ReLU."""
     r = rng(230 + cfg["C"] + cfg["OC"])
     x = r.standard_normal((cfg["N"], cfg["C"], cfg["H"], cfg["W"])).astype(np.float32)
     fan = cfg["C"] // cfg["g"] * cfg["k"][0] * cfg["k"][1]
@@ -241,7 +247,7 @@ def test_conv2d_f32_operands_by_lds_dma(ops, cfg):
     b = (r.standard_normal(cfg["OC"]) * 0.1).astype(np.float32)
     for bias, relu in ((b, True), (None, False)):
         y, names = _kernels_of(ops, lambda: ops.conv2d_f32(x, w, bias, cfg["p"], cfg["s"], cfg["d"], cfg["g"], relu))
-        assert names == ["k_transpose_weights", "k_conv2d_f32_dma"], names
+        assert names == ["k_transpose_weights", "k_conv2d_f32_dma_pairs" if cfg["pairs"] else "k_conv2d_f32_dma"], names
         ref = oracle.conv2d_f32(x, w, bias, cfg["p"], cfg["s"], cfg["d"], cfg["g"], relu)
         assert y.shape == ref.shape
         assert rel_err(y, ref) <= FP32_TOL
@@ -251,12 +257,14 @@ def test_conv_transpose2d_f32_phases_by_lds_dma(ops):
     """The benchmark's upsampling layer (4x4, stride 2) runs as four phases in one launch of the LDS-DMA kernel on
     gathered sub-kernels; an odd output size gives the phases different extents."""
     r = rng(77)
-    for (N, C, H, W, OC, op) in ((3, 128, 28, 28, 64, (0, 0)), (2, 24, 9, 10, 18, (1, 1))):
+    for (N, C, H, W, OC, op, k, kern) in ((3, 128, 28, 28, 64, (0, 0), 4, "k_conv2d_f32_dma_pairs_phases"),
+                                          (2, 24, 9, 10, 18, (1, 1), 4, "k_conv2d_f32_dma_pairs_phases"),
+                                          (2, 16, 9, 10, 18, (1, 1), 3, "k_conv2d_f32_dma_phases")):   # phases 2 and 1 columns wide
         x = r.standard_normal((N, C, H, W)).astype(np.float32)
-        w = (r.standard_normal((C, OC, 4, 4)) * 0.2).astype(np.float32)
+        w = (r.standard_normal((C, OC, k, k)) * 0.2).astype(np.float32)
         b = r.standard_normal(OC).astype(np.float32)
         y, names = _kernels_of(ops, lambda: ops.conv_transpose2d_f32(x, w, b, (1, 1, 1, 1), (2, 2), (1, 1), 1, op, True))
-        assert names == ["k_gather_phase_weights", "k_conv2d_f32_dma_phases"], names
+        assert names == ["k_gather_phase_weights", kern], names
         ref = oracle.conv_transpose2d_f32(x, w, b, (1, 1, 1, 1), (2, 2), (1, 1), 1, op, True)
         assert rel_err(y, ref) <= FP32_TOL
 
