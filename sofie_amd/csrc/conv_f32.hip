@@ -641,9 +641,9 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             }
             return 0;
          };
-         // kernels 2 or 3 columns wide without dilation along them run without the table of patch offsets, on even
+         // kernels 1 to 3 columns wide without dilation along them run without the table of patch offsets, on even
          // channel blocks with K ordered by channel pairs
-         const int kwt = (g.KW == 2 || g.KW == 3) && g.dw == 1 ? g.KW : 0;
+         const int kwt = g.KW == 1 || ((g.KW == 2 || g.KW == 3) && g.dw == 1) ? g.KW : 0;
          int icb = kwt ? pick(true) : 0;
          const bool pairs = icb > 0;
          if (!icb) icb = pick(false);
@@ -659,12 +659,13 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             if (int rc = check_launch(ctx, "k_transpose_weights")) return rc;
             ConvArgs h = g;
             h.w = static_cast<const float *>(ws);
-            constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, false, 0>, kern2 = k_conv2d_f32_dma<TI, TJ, false, 2>,
-                           kern3 = k_conv2d_f32_dma<TI, TJ, false, 3>;
+            constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, false, 0>, kern1 = k_conv2d_f32_dma<TI, TJ, false, 1>,
+                           kern2 = k_conv2d_f32_dma<TI, TJ, false, 2>, kern3 = k_conv2d_f32_dma<TI, TJ, false, 3>;
             SOFIE_LARGE_LDS(kern0);
+            SOFIE_LARGE_LDS(kern1);
             SOFIE_LARGE_LDS(kern2);
             SOFIE_LARGE_LDS(kern3);
-            const auto kern = !pairs ? kern0 : kwt == 2 ? kern2 : kern3;
+            const auto kern = !pairs ? kern0 : kwt == 1 ? kern1 : kwt == 2 ? kern2 : kern3;
             hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256),
                                dma_lds_bytes(g.KC, (size_t)icb * g.PH * g.PW, BOC), ctx->stream, h);
             *done = true;
@@ -726,8 +727,8 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
       const size_t budget = dma_lds_budget(ctx, workgroups, TI == 1 ? 7 : 3);
       const int wstride = (g.ocg + 3) & ~3;
       bool fits = (size_t)g.icg * g.H * g.W * 4 < (1u << 30) && (size_t)g.ocg * g.OH0 * g.OW0 * 4 < (1u << 30);
-      // every phase 2 (or every phase 3) columns wide: the table-free loop on even channel blocks, K by channel pairs
-      int kwt = g.phase[0].KW == 2 || g.phase[0].KW == 3 ? g.phase[0].KW : 0;
+      // every phase as wide as the others, 1 to 3 columns: the table-free loop on even channel blocks, K by channel pairs
+      int kwt = g.phase[0].KW >= 1 && g.phase[0].KW <= 3 ? g.phase[0].KW : 0;
       for (int i = 1; i < g.nphases; ++i)
          if (g.phase[i].KW != kwt) kwt = 0;
       int woff = 0;
@@ -774,12 +775,13 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
          ConvArgs h = g;
          h.w = static_cast<const float *>(ws);
-         constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, true, 0>, kern2 = k_conv2d_f32_dma<TI, TJ, true, 2>,
-                        kern3 = k_conv2d_f32_dma<TI, TJ, true, 3>;
+         constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, true, 0>, kern1 = k_conv2d_f32_dma<TI, TJ, true, 1>,
+                        kern2 = k_conv2d_f32_dma<TI, TJ, true, 2>, kern3 = k_conv2d_f32_dma<TI, TJ, true, 3>;
          SOFIE_LARGE_LDS(kern0);
+         SOFIE_LARGE_LDS(kern1);
          SOFIE_LARGE_LDS(kern2);
          SOFIE_LARGE_LDS(kern3);
-         const auto kern = !pairs ? kern0 : kwt == 2 ? kern2 : kern3;
+         const auto kern = !pairs ? kern0 : kwt == 1 ? kern1 : kwt == 2 ? kern2 : kern3;
          hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
          *done = true;
          return check_launch(ctx, pairs ? "k_conv2d_f32_dma_pairs_phases" : "k_conv2d_f32_dma_phases");

@@ -224,15 +224,16 @@ def _kernels_of(ops, call):
     # channel counts that are no multiple of 4 (the copied weights' rows are padded), a ragged second channel tile,
     # groups, a stride and a dilation, asymmetric pads, one or several patch requests per thread, a nearly empty last
     # pixel tile, a grid small enough for more than three workgroups per compute unit
-    # ... kernels 3 and 2 columns wide take the loop without a table of offsets (K ordered by channel pairs); a dilation,
-    # a 1x1 kernel, an odd number of channels per group and a kernel 5 columns wide take the general loop
+    # ... kernels 1 to 3 columns wide take the loop without a table of offsets (K ordered by channel pairs); a dilation
+    # along the columns, an odd number of channels per group and a kernel 5 columns wide take the general loop
     dict(N=3, C=16, H=20, W=20, OC=70, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, pairs=True),
     dict(N=2, C=16, H=9, W=19, OC=98, k=(3, 3), p=(1, 1), s=(2, 2), d=(1, 1), g=2, pairs=True),
     dict(N=1, C=8, H=12, W=12, OC=130, k=(3, 3), p=(3, 0, 1, 4), s=(1, 1), d=(2, 2), g=1, pairs=False),
     dict(N=2, C=64, H=56, W=56, OC=128, k=(3, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, pairs=True),
     dict(N=5, C=24, H=17, W=33, OC=33, k=(5, 2), p=(2, 0, 2, 1), s=(1, 1), d=(1, 1), g=1, pairs=True),
     dict(N=2, C=12, H=14, W=11, OC=40, k=(2, 3), p=(0, 1, 1, 1), s=(1, 2), d=(2, 1), g=2, pairs=True),
-    dict(N=40, C=32, H=6, W=6, OC=64, k=(1, 1), p=(0, 0), s=(1, 1), d=(1, 1), g=1, pairs=False),
+    dict(N=40, C=32, H=6, W=6, OC=64, k=(1, 1), p=(0, 0), s=(1, 1), d=(1, 1), g=1, pairs=True),
+    dict(N=2, C=20, H=9, W=12, OC=24, k=(3, 1), p=(1, 0, 1, 0), s=(1, 1), d=(2, 3), g=1, pairs=True),
     dict(N=3, C=9, H=13, W=10, OC=20, k=(2, 3), p=(1, 1), s=(1, 1), d=(1, 1), g=1, pairs=False),
     dict(N=2, C=4, H=11, W=16, OC=8, k=(2, 5), p=(1, 2, 0, 2), s=(1, 1), d=(1, 1), g=1, pairs=False),
 ])
