@@ -153,6 +153,53 @@ def test_gemm_f32(ops, M, N, K, tA, tB, alpha, beta, relu):
     assert rel_err(y, ref) <= FP32_TOL
 
 
+@pytest.mark.parametrize("M,N,K,tB,alpha,beta,relu,kern", [
+    # the kernel that fetches its operands by LDS-DMA: ragged tiles along M and N, one K step and an odd number of them,
+    # B as [K,N] and as [N,K], with and without a bias row
+    (2100, 2052, 96, 0, 1.0, 1.0, True, "k_gemm_f32_dma"),
+    (2100, 2052, 96, 1, -0.5, 2.0, False, "k_gemm_f32_dma"),
+    (2048, 2304, 32, 1, 1.0, 0.0, False, "k_gemm_f32_dma"),
+    (2304, 2048, 64, 0, 1.0, 0.0, True, "k_gemm_f32_dma"),
+    (4096, 2048, 160, 1, 1.0, 1.0, True, "k_gemm_f32_dma"),
+    # ... and what it leaves to the register-staged kernel: K that is no multiple of 32, N that is no multiple of 4 with B [K,N]
+    (2100, 2052, 100, 1, 1.0, 1.0, True, "k_gemm_f32"),
+    (2100, 2050, 96, 0, 1.0, 1.0, True, "k_gemm_f32"),
+])
+def test_gemm_f32_large(ops, M, N, K, tB, alpha, beta, relu, kern):
+    r = rng(900 + M + N + K + tB)
+    A = r.standard_normal((M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    bias = r.standard_normal(N).astype(np.float32) if beta != 0.0 else None
+    y, names = _kernels_of(ops, lambda: ops.gemm_f32(A, B, bias, alpha, beta, False, bool(tB), relu))
+    assert names == [kern], names
+    ref = alpha * (A.astype(np.float64) @ (B.T if tB else B).astype(np.float64)) + (beta * bias if bias is not None else 0.0)
+    ref = np.maximum(ref, 0) if relu else ref
+    assert y.shape == ref.shape
+    assert rel_err(y, ref) <= FP32_TOL
+    # sampled rows against the oracle's own summation (the C restatement of the reference's sgemm_ call)
+    rows = np.concatenate([np.arange(0, 8), r.integers(0, M, 8), np.arange(M - 8, M)])
+    assert rel_err(y[rows], oracle.gemm_f32(A[rows], B, bias, alpha, beta, False, bool(tB), relu)) <= FP32_TOL
+
+
+def test_gemm_f32_large_integer_data_is_exact_with_a_column_bias(ops):
+    """Integer operands make every order of summation exact: the LDS-DMA kernel against int64 numpy, with the bias as a
+    column (one value per row of the output), through the C ABI."""
+    from sofie_amd import lib as L
+    r = rng(901)
+    M, N, K = 2200, 2048, 128
+    A = r.integers(-8, 9, (M, K)).astype(np.float32)
+    B = r.integers(-8, 9, (N, K)).astype(np.float32)
+    col = r.integers(-50, 50, M).astype(np.float32)
+    ctx = ops.default_context()
+    a, b, c = ctx.dev(A), ctx.dev(B), ctx.dev(col)
+    y = ctx.empty((M, N), torch.float32)
+    ctx.check(ctx.lib.sofie_hip_gemm_f32(ctx.h, 0, 1, M, N, K, 2.0, ctx.ptr(a), K, ctx.ptr(b), K, 3.0, ctx.ptr(c), L.BIAS_COL,
+                                         ctx.ptr(y), N, L.ACT_RELU))
+    ctx.sync()
+    ref = np.maximum(2 * (A.astype(np.int64) @ B.astype(np.int64).T) + 3 * col.astype(np.int64)[:, None], 0)
+    assert np.array_equal(y.cpu().numpy(), ref)
+
+
 def test_gemm_f32_full_bias_and_error_path(ops):
     r = rng(7)
     A = r.standard_normal((50, 20)).astype(np.float32)
