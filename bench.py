@@ -9,6 +9,7 @@ headline value it carries every other configuration of the benchmark:
   fp8_gemm          e4m3 GEMM 8192x8192x4096, bf16 out + bias, TFLOP/s and fraction of the FP8 MFMA peak
   model_inferences  the generated int8 CNN Session at batch 4096, inferences per second
   mlp_f32           the generated fp32 MLP Session (64 -> 128 -> 64 -> 8, batch 256)
+  gemm_f32          the reference's Gemm operator at 4096^3 in fp32 (bias row + ReLU), B [K,N] and [N,K]
   conv_f32/conv_s8  the 256 x 64 -> 128 x 56 x 56 3x3 layer in fp32 and int8
   cpu_fp32          the reference's emitted CPU call sequence for the MLP and the convolution layer
                     (oracle/cpu_emitted_bench.c) with sgemm_ from the best BLAS found on the box, at one thread and
@@ -195,6 +196,14 @@ def cpu_fp32_baselines(threads, conv_images=64):
     for t in sorted({1, threads}):
         m = cpu_emitted("mlp", t, chosen, ("--calls", "200"))
         c = cpu_emitted("conv", t, chosen, ("--images", str(conv_images), "--calls", "3"))
+        gemm_rows = 256 if t == 1 else 2048
+        gm = cpu_emitted("gemm", t, chosen, ("--images", str(gemm_rows), "--calls", "3"))
+        if gm:
+            res["gemm_4096_%dthr" % t] = {
+                "median_ms": gm["median_ms"], "best_ms": gm["best_ms"], "gflops": 2.0 * gemm_rows * 4096 * 4096 / gm["median_ms"] / 1e6,
+                "cores": t, "calls": gm["calls"],
+                "sample": "%d of the 4096 rows of the product (rows are independent; %.1f GFLOP per call)"
+                          % (gemm_rows, 2.0 * gemm_rows * 4096 * 4096 / 1e9)}
         if m:
             res["mlp_b256_%dthr" % t] = {"median_us": m["median_ms"] * 1e3, "best_us": m["best_ms"] * 1e3,
                                          "inferences_per_s": 256 / (m["median_ms"] * 1e-3), "cores": t, "calls": m["calls"]}
@@ -229,7 +238,7 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     ap.add_argument("--kernel-probe", default="",
                     help="launch one named workload a few times and exit (target of rocprofv3 runs): gemm_s8, gemm_s8_nk, "
-                         "gemm_fp8, gemm_fp8_nk, conv_s8, conv_f32")
+                         "gemm_fp8, gemm_fp8_nk, gemm_f32, gemm_f32_nk, conv_s8, conv_f32, conv_transpose_f32")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collective, no sharding "
@@ -418,6 +427,8 @@ def main():
     out["fp8_gemm"] = dict(res["gemm_fp8"], peak_tflops=PEAK_FP8_TFLOPS)
     out["fp8_gemm_b_nk"] = res["gemm_fp8_nk"]
     out["int8_gemm_b_nk"] = res["gemm_s8_nk"]
+    out["gemm_f32"] = res["gemm_f32"]
+    out["gemm_f32_b_nk"] = res["gemm_f32_nk"]
     out["conv_f32"] = res["conv_f32"]
     out["conv_s8"] = res["conv_s8"]
     out["conv_transpose_f32"] = res["conv_transpose_f32"]
@@ -459,6 +470,17 @@ def workloads(ctx, torch, L, rng):
             {"workload": "FP8 e4m3 GEMM M=N=8192 K=4096, A and B N(0,1) cast to e4m3 with per-tensor scales amax/448, "
                          "B %s, fused bias, bf16 out" % ("[N,K]" if tb else "[K,N]"),
              "ops": 2.0 * M * N * K, "rate_unit": "tflops", "peak": PEAK_FP8_TFLOPS, "launches": 100})
+    # fp32 Gemm as the reference's operator states it (Y = A B + bias, ReLU fused), 4096^3, B as [K,N] and as [N,K]
+    Af = torch.randn(n, n, device=ctx.device)
+    Bf = torch.randn(n, n, device=ctx.device)
+    bf = torch.randn(n, device=ctx.device)
+    Yf = ctx.empty((n, n), torch.float32)
+    for name, tb in (("gemm_f32", 0), ("gemm_f32_nk", 1)):
+        w[name] = ((lambda tb=tb: ctx.check(ctx.lib.sofie_hip_gemm_f32(
+            ctx.h, 0, tb, n, n, n, 1.0, ctx.ptr(Af), n, ctx.ptr(Bf), n, 1.0, ctx.ptr(bf), L.BIAS_ROW, ctx.ptr(Yf), n, L.ACT_RELU))),
+            {"workload": "fp32 Gemm 4096^3 (ROperator_Gemm: Y = A B + bias row, ReLU fused), A and B N(0,1), B %s"
+                         % ("[N,K] (transB = 1)" if tb else "[K,N]"),
+             "ops": 2.0 * n ** 3, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 20})
     # fp32 conv layer: batch 256, 64 -> 128 channels, 56x56, 3x3, pad 1, bias + ReLU
     x = torch.rand(256, 64, 56, 56, device=ctx.device)
     wt = torch.randn(128, 64, 3, 3, device=ctx.device) * (2.0 / 576) ** 0.5

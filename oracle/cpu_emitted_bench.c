@@ -1,11 +1,12 @@
 /*
  * cpu_emitted_bench.c -- TEST / BENCHMARK INFRASTRUCTURE, NOT PRODUCT CODE.
  *
- * The CPU call sequence that the reference's RModel::Generate emits for the two fp32 configurations of the
+ * The CPU call sequence that the reference's RModel::Generate emits for the fp32 configurations of the
  * benchmark, restated in plain C and timed on the host cores:
  *   mlp   Gemm 64->128 + ReLU, Gemm 128->64 + ReLU, Gemm 64->8 on a batch of 256
  *         per Gemm (ROperator_Gemm.hxx:360-381): std::copy(bias broadcast to [M,N] -> Y);
  *         BLAS::sgemm_(transB, transA, n, m, k, alpha, W, ldb, X, lda, beta = 1, Y, n); the ReLU loop
+ *   gemm  one large Gemm + ReLU: `--images` rows of the 4096 x 4096 x 4096 product of the benchmark (same call sequence)
  *   conv  Conv 64->128, 56x56, 3x3, stride 1, pad 1, bias, then Relu (ROperator_Conv.hxx:342-518,
  *         ROperator_Relu.hxx:54-66): inside infer the weight re-layout loop into x_f; per image Im2col
  *         (SOFIE_common.hxx:485-518), BLAS::sgemm_('N','N', m = OH*OW, n = OC, k = C*KH*KW, 1, xcol, m, x_f, k, 0,
@@ -224,7 +225,7 @@ int main(int argc, char **argv)
         else if (!strcmp(argv[i], "--calls") && i + 1 < argc) calls = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--images") && i + 1 < argc) images = atoi(argv[++i]);
         else if (!strcmp(argv[i], "--dump") && i + 1 < argc) dump = argv[++i];
-        else { fprintf(stderr, "usage: %s [--workload mlp|conv|cnn] [--blas PATH --prefix P] [--calls N] [--images N] [--dump FILE]\n", argv[0]); return 2; }
+        else { fprintf(stderr, "usage: %s [--workload mlp|gemm|conv|cnn] [--blas PATH --prefix P] [--calls N] [--images N] [--dump FILE]\n", argv[0]); return 2; }
     }
     const char *bound = "bundled loops (no BLAS library)";
     if (blas) {
@@ -271,6 +272,34 @@ int main(int argc, char **argv)
             fwrite(x, sizeof(float), (size_t)M * d[0], f);
             for (int l = 0; l < 3; ++l) fwrite(w[l], sizeof(float), (size_t)d[l] * d[l + 1], f);
             fwrite(h[2], sizeof(float), (size_t)M * d[3], f);
+            fclose(f);
+        }
+    } else if (!strcmp(workload, "gemm")) {
+        /* one large Gemm as ROperator_Gemm emits it: `images` rows of a [4096, 4096] x [4096, 4096] product (the rows of
+           the product are independent), bias broadcast to [M, N] at construction, ReLU */
+        const int M = images, N = 4096, K = 4096;
+        if (calls <= 0) calls = 3;
+        float *x = alloc_f((size_t)M * K), *w = alloc_f((size_t)K * N), *bb = alloc_f((size_t)M * N), *y = alloc_f((size_t)M * N);
+        for (size_t i = 0; i < (size_t)M * K; ++i) x[i] = (float)normal01();
+        for (size_t i = 0; i < (size_t)K * N; ++i) w[i] = (float)normal01();
+        for (int n = 0; n < N; ++n) {
+            const float b = (float)normal01();
+            for (int m = 0; m < M; ++m) bb[(size_t)m * N + n] = b;
+        }
+        times = (double *)malloc(sizeof(double) * calls);
+        for (int it = -1; it < calls; ++it) {
+            const double t0 = now_ms();
+            emitted_gemm(M, N, K, x, w, bb, y, 1);
+            if (it >= 0) times[it] = now_ms() - t0;
+        }
+        for (size_t i = 0; i < (size_t)M * N; i += 4099) checksum += y[i];
+        if (dump) {
+            FILE *f = fopen(dump, "wb");
+            if (!f) { perror(dump); return 6; }
+            fwrite(x, sizeof(float), (size_t)M * K, f);
+            fwrite(w, sizeof(float), (size_t)K * N, f);
+            fwrite(bb, sizeof(float), N, f);              /* the bias row */
+            fwrite(y, sizeof(float), (size_t)M * N, f);
             fclose(f);
         }
     } else if (!strcmp(workload, "conv")) {

@@ -188,11 +188,16 @@ __global__ void __launch_bounds__(256, 2) k_gemm_f32_dma(GemmF32Args g)
    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
    const int wm = wave >> 1, wn = wave & 1;
    const int fr = lane & 31, fk = lane >> 5;
-   // tiles in groups of 4 rows of tiles, so that the workgroups in flight share rows of A and columns of B in the L2
+   // tiles in groups of 4 rows of tiles, so that the workgroups in flight share rows of A and columns of B in an L2
    int tm, tn;
    {
       const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
-      const int pid = blockIdx.x;
+      // workgroups are dealt to the 8 XCDs in turn: renumbered so that an XCD (an L2) works on consecutive tiles
+      int pid = blockIdx.x;
+      {
+         const int tiles = tiles_m * tiles_n, xcd = pid & 7, base = tiles >> 3, rem = tiles & 7;
+         pid = (pid >> 3) + xcd * base + (xcd < rem ? xcd : rem);
+      }
       const int width = 4 * tiles_n, group = pid / width, first = group * 4;
       const int gsize = tiles_m - first < 4 ? tiles_m - first : 4;
       tm = first + (pid % width) % gsize;

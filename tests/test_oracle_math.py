@@ -553,6 +553,16 @@ def test_cpu_baseline_program_computes_what_the_oracle_computes(tmp_path):
         x, w, b, y = np.split(raw, np.cumsum(sizes)[:-1])
         ref = oracle.conv2d_f32(x.reshape(2, 64, 56, 56), w.reshape(128, 64, 3, 3), b, (1, 1), relu=True)
         assert np.max(np.abs(y.reshape(ref.shape) - ref)) <= 1e-5 * np.max(np.abs(ref))
+        # the large Gemm: a few rows of the 4096 x 4096 x 4096 product with its bias row and ReLU
+        f = str(tmp_path / "gemm.bin")
+        rows = 3
+        out = _cpu_emitted(["--workload", "gemm", "--images", str(rows), "--calls", "1", "--dump", f] + extra, {"OMP_NUM_THREADS": "2"})
+        raw = np.fromfile(f, np.float32)
+        sizes = [rows * 4096, 4096 * 4096, 4096, rows * 4096]
+        assert raw.size == sum(sizes)
+        x, w, b, y = np.split(raw, np.cumsum(sizes)[:-1])
+        ref = oracle.gemm_f32(x.reshape(rows, 4096), w.reshape(4096, 4096), b, relu=True)
+        assert np.max(np.abs(y.reshape(ref.shape) - ref)) <= 1e-5 * np.max(np.abs(ref))
 
 
 def test_cpu_baseline_cnn_computes_what_the_oracle_computes(tmp_path):
