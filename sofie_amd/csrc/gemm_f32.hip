@@ -165,21 +165,22 @@ __global__ void __launch_bounds__(256) k_gemm_f32(GemmF32Args g)
 
 // The same product for operands that allow it (A [M][K] row-major, K a multiple of 32, 16-byte aligned rows), with
 // both operand tiles travelling global memory -> LDS without registers (buffer_load_dwordx4 ... lds), two stages of
-// 32 k, under the matrix loop of the stage before. 128 x 128 tile, 4 wavefronts of 2 x 2 tiles of 32 x 32.
+// 32 k, under the matrix loop of the stage before. Tile of 64 T x 64 T (T = 2: 128 x 128, two workgroups per CU; T = 1
+// for products of few tiles: 64 x 64, four per CU), 4 wavefronts of T x T tiles of 32 x 32.
 //   * An operand whose rows run along K (A; B given [N][K]) is staged as rows of 32 floats (8 chunks of 16 bytes) with
 //     chunk c of row r in slot c ^ ((r >> 1) & 7): a lane reads 4 consecutive k of its row with one 16-byte read (lanes
 //     0-31: k = 8s .. 8s+3, lanes 32-63: k = 8s+4 .. 8s+7, which is the pairing of four matrix instructions), and the 16
 //     lanes the LDS serves together fall on 16 different slots of 256 bytes. The swizzle costs nothing: a lane of the
 //     request asks for the chunk that belongs into its slot.
-//   * B given [K][N] is staged as it is, rows of k with 128 columns, and read 4 bytes per lane.
+//   * B given [K][N] is staged as it is, rows of k with the tile's columns, and read 4 bytes per lane.
 // A lane's read addresses do not depend on the K step (the stage is an immediate offset: the loop is unrolled over the
 // two stages), so the loop holds LDS reads and matrix instructions and no vector arithmetic, which would take issue
 // cycles from the matrix instructions. Rows behind M (or N) lie outside the tile's descriptor and arrive as zeros;
 // outputs go through a descriptor too (columns behind N get an offset outside it and are dropped).
-template <bool B_KMAJOR>
-__global__ void __launch_bounds__(256, 2) k_gemm_f32_dma(GemmF32Args g)
+template <bool B_KMAJOR, int T>
+__global__ void __launch_bounds__(256, T == 2 ? 2 : 4) k_gemm_f32_dma(GemmF32Args g)
 {
-   constexpr int BM = 128, BN = 128, BKD = 32;
+   constexpr int BM = 64 * T, BN = 64 * T, BKD = 32;
    constexpr int STAGE = (BM + BN) * BKD;               // floats of one stage: the A tile, then the B tile
    constexpr unsigned OUTSIDE = 0x80000000u;            // an offset no descriptor of this kernel reaches
    extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -210,45 +211,46 @@ __global__ void __launch_bounds__(256, 2) k_gemm_f32_dma(GemmF32Args g)
                                : make_rsrc(g.B + (size_t)n0 * g.ldb, (unsigned)((size_t)rows_b * g.ldb * 4));
    // requests: 16 bytes per lane, 256 lanes per request. Row-major operand: lane -> (row tid/8 [+ 32 per request],
    // slot tid%8), it fetches chunk slot ^ swizzle(row); the swizzle is the same for every request of the lane.
+   constexpr int NRQ = 2 * T;                           // requests per operand tile and stage (4 KB each)
    const int rq_row = tid >> 3, rq_slot = tid & 7;
    const unsigned rq_a = (unsigned)((rq_row * g.lda + ((rq_slot ^ ((rq_row >> 1) & 7)) << 2)) * 4);
    unsigned rq_b;
    if constexpr (B_KMAJOR) {
-      // lane -> (k tid/32 [+ 8 per request], columns 4*(tid%32) .. +3); columns behind N ask for nothing
-      const int col = n0 + (tid & 31) * 4;
-      rq_b = col < g.N ? (unsigned)(((tid >> 5) * g.ldb + col) * 4) : OUTSIDE;
+      // lane -> (k tid/(BN/4) [+ 1024/BN per request], columns 4*(tid%(BN/4)) .. +3); columns behind N ask for nothing
+      const int col = n0 + (tid % (BN / 4)) * 4;
+      rq_b = col < g.N ? (unsigned)(((tid / (BN / 4)) * g.ldb + col) * 4) : OUTSIDE;
    } else {
       rq_b = (unsigned)((rq_row * g.ldb + ((rq_slot ^ ((rq_row >> 1) & 7)) << 2)) * 4);
    }
-   const unsigned step_a = (unsigned)(32 * g.lda * 4), step_b = (unsigned)((B_KMAJOR ? 8 : 32) * g.ldb * 4);
+   const unsigned step_a = (unsigned)(32 * g.lda * 4), step_b = (unsigned)((B_KMAJOR ? 1024 / BN : 32) * g.ldb * 4);
    auto request = [&](int kt, int stage) {
       const unsigned dst = lds0 + (unsigned)(stage * STAGE * 4) + (unsigned)(wave * 1024);
       const unsigned ka = (unsigned)(kt * BKD * 4), kb = B_KMAJOR ? (unsigned)kt * BKD * (unsigned)g.ldb * 4u : ka;
 #pragma unroll
-      for (int u = 0; u < 4; ++u) dma16(ars, dst + u * 4096, (int)rq_a, (int)(ka + u * step_a));
+      for (int u = 0; u < NRQ; ++u) dma16(ars, dst + u * 4096, (int)rq_a, (int)(ka + u * step_a));
 #pragma unroll
-      for (int u = 0; u < 4; ++u) dma16(brs, dst + BM * BKD * 4 + u * 4096, (int)rq_b, (int)(kb + u * step_b));
+      for (int u = 0; u < NRQ; ++u) dma16(brs, dst + BM * BKD * 4 + u * 4096, (int)rq_b, (int)(kb + u * step_b));
    };
    // read addresses of the lane's fragments in stage 0 (floats from the start of the LDS block)
-   int ra[2][4], rb[2][4];
+   int ra[T][4], rb[T][4];
 #pragma unroll
-   for (int i = 0; i < 2; ++i) {
-      const int row = wm * 64 + i * 32 + fr;
+   for (int i = 0; i < T; ++i) {
+      const int row = wm * 32 * T + i * 32 + fr;
 #pragma unroll
       for (int s = 0; s < 4; ++s) ra[i][s] = row * BKD + (((2 * s + fk) ^ ((row >> 1) & 7)) << 2);
    }
 #pragma unroll
-   for (int j = 0; j < 2; ++j) {
-      const int row = wn * 64 + j * 32 + fr;
+   for (int j = 0; j < T; ++j) {
+      const int row = wn * 32 * T + j * 32 + fr;
 #pragma unroll
       for (int s = 0; s < 4; ++s)
          rb[j][s] = BM * BKD + (B_KMAJOR ? (8 * s + 4 * fk) * BN + row : row * BKD + (((2 * s + fk) ^ ((row >> 1) & 7)) << 2));
    }
-   v16f acc[2][2];
+   v16f acc[T][T];
 #pragma unroll
-   for (int i = 0; i < 2; ++i)
+   for (int i = 0; i < T; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < T; ++j)
 #pragma unroll
          for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
@@ -256,11 +258,11 @@ __global__ void __launch_bounds__(256, 2) k_gemm_f32_dma(GemmF32Args g)
       constexpr int OFF = decltype(stage_c)::value * STAGE;
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-         v4f fa[2], fb[2];
+         v4f fa[T], fb[T];
 #pragma unroll
-         for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const v4f *>(lds + OFF + ra[i][s]);
+         for (int i = 0; i < T; ++i) fa[i] = *reinterpret_cast<const v4f *>(lds + OFF + ra[i][s]);
 #pragma unroll
-         for (int j = 0; j < 2; ++j) {
+         for (int j = 0; j < T; ++j) {
             if constexpr (B_KMAJOR) {
 #pragma unroll
                for (int e = 0; e < 4; ++e) fb[j][e] = lds[OFF + rb[j][s] + e * BN];
@@ -271,9 +273,9 @@ __global__ void __launch_bounds__(256, 2) k_gemm_f32_dma(GemmF32Args g)
 #pragma unroll
          for (int e = 0; e < 4; ++e)
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < T; ++i)
 #pragma unroll
-               for (int j = 0; j < 2; ++j)
+               for (int j = 0; j < T; ++j)
                   acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][e], fb[j][e], acc[i][j], 0, 0, 0);
       }
    };
@@ -299,15 +301,15 @@ __global__ void __launch_bounds__(256, 2) k_gemm_f32_dma(GemmF32Args g)
       const_cast<float *>(g.bias) + (g.bias_kind == SOFIE_BIAS_COL ? m0 : 0), 0, g.bias_kind == SOFIE_BIAS_COL ? rows_a * 4 : 0, 0x00020000);
    const unsigned ldy4 = (unsigned)g.ldy * 4u;
 #pragma unroll
-   for (int j = 0; j < 2; ++j) {
-      const int n = n0 + wn * 64 + j * 32 + fr;
+   for (int j = 0; j < T; ++j) {
+      const int n = n0 + wn * 32 * T + j * 32 + fr;
       const float brow = g.bias_kind == SOFIE_BIAS_ROW && n < g.N ? __fmul_rn(g.beta, g.bias[n]) : 0.0f;
-      const unsigned voff = n < g.N ? (unsigned)((wn * 64 + j * 32 + fr + n0) * 4) + (unsigned)fk * 4u * ldy4 : OUTSIDE;
+      const unsigned voff = n < g.N ? (unsigned)(n * 4) + (unsigned)fk * 4u * ldy4 : OUTSIDE;
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < T; ++i)
 #pragma unroll
          for (int r = 0; r < 16; ++r) {
-            const int m_uniform = wm * 64 + i * 32 + (r >> 2) * 8 + (r & 3);      // + 4 * fk in the lane's offset
+            const int m_uniform = wm * 32 * T + i * 32 + (r >> 2) * 8 + (r & 3);      // + 4 * fk in the lane's offset
             float v = __fmul_rn(g.alpha, acc[i][j][r]);
             if (g.bias_kind == SOFIE_BIAS_ROW) v = __fadd_rn(v, brow);
             else if (g.bias_kind == SOFIE_BIAS_COL)
@@ -346,18 +348,24 @@ extern "C" int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, in
    g.alpha = alpha; g.beta = beta; g.bias_kind = bias_kind; g.relu = act == SOFIE_ACT_RELU;
    const bool small = (size_t)cdiv(M, 128) * cdiv(N, 128) < 256;
    // operands by LDS-DMA: A row-major with rows of whole 16-byte chunks, K in whole stages, everything a descriptor
-   // addresses below 2 GiB, a bias that is a row, a column or absent
+   // addresses below 2 GiB, a bias that is a row, a column or absent; 64 x 64 tiles where 128 x 128 ones would leave
+   // compute units without a tile, and nothing for products of a handful of tiles
    const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; };
-   const bool dma = !small && !transA && K >= 32 && K % 32 == 0 && lda % 4 == 0 && ldb % 4 == 0 && (transB || N % 4 == 0) &&
-                    aligned16(A) && aligned16(B) && bias_kind != SOFIE_BIAS_FULL && (size_t)128 * lda * 4 < (1u << 31) &&
-                    (size_t)(transB ? 128 : K) * ldb * 4 < (1u << 31) && (size_t)128 * ldy * 4 < (1u << 31) &&
-                    (size_t)cdiv(M, 128) * cdiv(N, 128) < (1u << 30);
+   const int tile = small ? 64 : 128;
+   const bool dma = (size_t)cdiv(M, 64) * cdiv(N, 64) >= 32 && !transA && K >= 32 && K % 32 == 0 && lda % 4 == 0 && ldb % 4 == 0 &&
+                    (transB || N % 4 == 0) && aligned16(A) && aligned16(B) && bias_kind != SOFIE_BIAS_FULL &&
+                    (size_t)128 * lda * 4 < (1u << 31) && (size_t)(transB ? 128 : K) * ldb * 4 < (1u << 31) &&
+                    (size_t)128 * ldy * 4 < (1u << 31) && (size_t)cdiv(M, tile) * cdiv(N, tile) < (1u << 30);
    if (dma) {
-      constexpr auto kern_nk = k_gemm_f32_dma<false>, kern_kn = k_gemm_f32_dma<true>;
-      SOFIE_LARGE_LDS(kern_nk);
-      SOFIE_LARGE_LDS(kern_kn);
-      hipLaunchKernelGGL(transB ? kern_nk : kern_kn, dim3(cdiv(M, 128) * cdiv(N, 128)), dim3(256), 2 * (128 + 128) * 32 * 4, ctx->stream, g);
-      return check_launch(ctx, "k_gemm_f32_dma");
+      constexpr auto kern_nk2 = k_gemm_f32_dma<false, 2>, kern_kn2 = k_gemm_f32_dma<true, 2>;
+      constexpr auto kern_nk1 = k_gemm_f32_dma<false, 1>, kern_kn1 = k_gemm_f32_dma<true, 1>;
+      SOFIE_LARGE_LDS(kern_nk2);
+      SOFIE_LARGE_LDS(kern_kn2);
+      SOFIE_LARGE_LDS(kern_nk1);
+      SOFIE_LARGE_LDS(kern_kn1);
+      const auto kern = small ? (transB ? kern_nk1 : kern_kn1) : (transB ? kern_nk2 : kern_kn2);
+      hipLaunchKernelGGL(kern, dim3(cdiv(M, tile) * cdiv(N, tile)), dim3(256), 2 * (tile + tile) * 32 * 4, ctx->stream, g);
+      return check_launch(ctx, small ? "k_gemm_f32_dma64" : "k_gemm_f32_dma");
    } else if (small) {
       hipLaunchKernelGGL((k_gemm_f32<1, 1>), dim3(cdiv(N, 64), cdiv(M, 64)), dim3(256), 0, ctx->stream, g);
    } else {

@@ -161,6 +161,11 @@ def test_gemm_f32(ops, M, N, K, tA, tB, alpha, beta, relu):
     (2048, 2304, 32, 1, 1.0, 0.0, False, "k_gemm_f32_dma"),
     (2304, 2048, 64, 0, 1.0, 0.0, True, "k_gemm_f32_dma"),
     (4096, 2048, 160, 1, 1.0, 1.0, True, "k_gemm_f32_dma"),
+    # ... with 64 x 64 tiles where there are fewer than 256 tiles of 128 x 128
+    (700, 900, 256, 1, 1.0, 1.0, True, "k_gemm_f32_dma64"),
+    (700, 900, 96, 0, 0.25, -1.0, False, "k_gemm_f32_dma64"),
+    (1024, 1024, 1024, 0, 1.0, 1.0, True, "k_gemm_f32_dma64"),
+    (300, 520, 32, 1, 1.0, 0.0, False, "k_gemm_f32_dma64"),
     # ... and what it leaves to the register-staged kernel: K that is no multiple of 32, N that is no multiple of 4 with B [K,N]
     (2100, 2052, 100, 1, 1.0, 1.0, True, "k_gemm_f32"),
     (2100, 2050, 96, 0, 1.0, 1.0, True, "k_gemm_f32"),
