@@ -72,6 +72,19 @@ enum { SOFIE_LAYOUT_NCHW = 0, SOFIE_LAYOUT_NHWC = 1 };
 int sofie_hip_create(sofie_hip_ctx **ctx, int device, void *stream);
 int sofie_hip_destroy(sofie_hip_ctx *ctx);
 /* Message of the last failed call on this context ("" if none). Never NULL. */
+/* A promise of the caller: the weight tensors handed to the convolution entry points of this context from now on do
+ * not change (and their memory is not freed and reused) while the context lives or until the promise is taken back
+ * with on = 0. The library then keeps the copy of a weight tensor that it lays out for its kernels
+ * (sofie_hip_conv2d_f32: [K][channel]; sofie_hip_conv_transpose2d_f32: the gathered sub-kernels of the output phases)
+ * in a buffer of its own per tensor and geometry, made by the first call, instead of making it in front of every
+ * launch in the scratch buffer; at most SOFIE_HIP_PACKED_MAX tensors, later ones are laid out per call as before.
+ * on = 0 frees the copies. Not allowed while a graph is recorded; a new tensor met while a graph is recorded is laid
+ * out per call. A generated Session makes the promise in its constructor: its weights are uploaded once and never
+ * written again. The reference re-lays a Conv's weights inside every infer call (ROperator_Conv.hxx:342-362); no
+ * counterpart of the promise exists there. */
+#define SOFIE_HIP_PACKED_MAX 256
+int sofie_hip_constant_weights(sofie_hip_ctx *ctx, int on);
+
 const char *sofie_hip_last_error(const sofie_hip_ctx *ctx);
 /* ABI version of the library (bumped on incompatible change). */
 int sofie_hip_version(void);

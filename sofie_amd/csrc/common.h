@@ -28,6 +28,16 @@ struct sofie_hip_ctx {
    };
    TracePoint *trace = nullptr;   // [SOFIE_HIP_TRACE_MAX + 1], entry 0 is the start
    int trace_len = 0;
+   // sofie_hip_constant_weights: copies of weight tensors in the layout a kernel wants, kept per tensor and geometry
+   bool constant_weights = false;
+   struct PackedWeights {
+      const void *w;
+      unsigned long long key;
+      size_t bytes;
+      void *packed;
+   };
+   PackedWeights *packed = nullptr;   // [SOFIE_HIP_PACKED_MAX]
+   int packed_len = 0;
    char err[512] = {0};
 };
 
@@ -37,6 +47,11 @@ int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...);
 // Grow-only scratch buffer of the context. Never shrinks; freed in sofie_hip_destroy.
 int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr);
 int check_launch(sofie_hip_ctx *ctx, const char *what);
+// Where a kernel's own layout of the weight tensor `w` goes: the context's scratch buffer (*fresh = true: fill it now), or,
+// when the caller has promised that its weights do not change (sofie_hip_constant_weights), a buffer kept for this
+// tensor and `key` (a hash of everything the layout depends on), filled by the first call only.
+int packed_weights(sofie_hip_ctx *ctx, const void *w, unsigned long long key, size_t bytes, void **ptr, bool *fresh);
+unsigned long long layout_key(const int *values, int n);
 // Bracket of a call that uses the device's fixed scratch array (sofie_hip_qgemm_s8_noalloc): orders it behind the call
 // that used the array before it, on whatever context and stream that was.
 void scratch_turn_begin(sofie_hip_ctx *ctx);

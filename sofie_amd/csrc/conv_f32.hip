@@ -653,10 +653,14 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             g.dPW = make_fastdiv((unsigned)g.PW);
             g.dPH = make_fastdiv((unsigned)g.PH);
             void *ws = nullptr;
-            if (int rc = workspace(ctx, wt_floats * sizeof(float), &ws)) return rc;
-            hipLaunchKernelGGL(k_transpose_weights, dim3((unsigned)((wt_floats + 255) / 256)), dim3(256), 0, ctx->stream, g.w,
-                               static_cast<float *>(ws), g.groups, g.ocg, g.icg * KHW, wstride, pairs ? 1 : 0, KHW);
-            if (int rc = check_launch(ctx, "k_transpose_weights")) return rc;
+            bool fresh = true;
+            const int layout[] = {1, g.groups, g.ocg, g.icg, g.KH, g.KW, wstride, pairs ? 1 : 0};
+            if (int rc = packed_weights(ctx, g.w, layout_key(layout, 8), wt_floats * sizeof(float), &ws, &fresh)) return rc;
+            if (fresh) {
+               hipLaunchKernelGGL(k_transpose_weights, dim3((unsigned)((wt_floats + 255) / 256)), dim3(256), 0, ctx->stream, g.w,
+                                  static_cast<float *>(ws), g.groups, g.ocg, g.icg * KHW, wstride, pairs ? 1 : 0, KHW);
+               if (int rc = check_launch(ctx, "k_transpose_weights")) return rc;
+            }
             ConvArgs h = g;
             h.w = static_cast<const float *>(ws);
             constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, false, 0>, kern1 = k_conv2d_f32_dma<TI, TJ, false, 1>,
@@ -769,10 +773,19 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
       const bool pairs = kwt && plan(true);
       if (pairs || plan(false)) {
          void *ws = nullptr;
-         if (int rc = workspace(ctx, (size_t)woff * sizeof(float), &ws)) return rc;
-         hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
-                            static_cast<float *>(ws), woff, wstride, pairs ? 1 : 0);
-         if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
+         bool fresh = true;
+         int layout[12 + 6 * SOFIE_CONV_MAX_PHASES] = {2, g.groups, g.ocg, g.icg, g.KH0, g.KW0, g.ths, g.tws, wstride, pairs ? 1 : 0, g.nphases, woff};
+         for (int i = 0; i < g.nphases; ++i) {
+            const PhaseArgs &q = g.phase[i];
+            const int v[6] = {q.KH, q.KW, q.th0, q.tw0, q.woff, i};
+            for (int e = 0; e < 6; ++e) layout[12 + 6 * i + e] = v[e];
+         }
+         if (int rc = packed_weights(ctx, g.w, layout_key(layout, 12 + 6 * g.nphases), (size_t)woff * sizeof(float), &ws, &fresh)) return rc;
+         if (fresh) {
+            hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
+                               static_cast<float *>(ws), woff, wstride, pairs ? 1 : 0);
+            if (int rc = check_launch(ctx, "k_gather_phase_weights")) return rc;
+         }
          ConvArgs h = g;
          h.w = static_cast<const float *>(ws);
          constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, true, 0>, kern1 = k_conv2d_f32_dma<TI, TJ, true, 1>,

@@ -111,6 +111,44 @@ int set_error(sofie_hip_ctx *ctx, int code, const char *fmt, ...)
    return code;
 }
 
+unsigned long long layout_key(const int *values, int n)
+{
+   unsigned long long h = 1469598103934665603ull;      // FNV-1a over the bytes of the values
+   for (int i = 0; i < n; ++i)
+      for (int b = 0; b < 4; ++b) {
+         h ^= (unsigned long long)(((unsigned)values[i] >> (8 * b)) & 0xffu);
+         h *= 1099511628211ull;
+      }
+   return h;
+}
+
+int packed_weights(sofie_hip_ctx *ctx, const void *w, unsigned long long key, size_t bytes, void **ptr, bool *fresh)
+{
+   *fresh = true;
+   if (ctx->constant_weights && !ctx->no_alloc) {
+      for (int i = 0; i < ctx->packed_len; ++i) {
+         const sofie_hip_ctx::PackedWeights &e = ctx->packed[i];
+         if (e.w == w && e.key == key && e.bytes == bytes) {
+            *ptr = e.packed;
+            *fresh = false;
+            return SOFIE_HIP_OK;
+         }
+      }
+      // a new tensor: a buffer of its own, unless a graph is being recorded (nothing may allocate then) or the table is full
+      if (!ctx->capturing && ctx->packed_len < SOFIE_HIP_PACKED_MAX) {
+         if (!ctx->packed) ctx->packed = new sofie_hip_ctx::PackedWeights[SOFIE_HIP_PACKED_MAX];
+         void *buf = nullptr;
+         if (hipMalloc(&buf, bytes) == hipSuccess) {
+            ctx->packed[ctx->packed_len++] = {w, key, bytes, buf};
+            *ptr = buf;
+            return SOFIE_HIP_OK;
+         }
+         (void)hipGetLastError();
+      }
+   }
+   return workspace(ctx, bytes, ptr);
+}
+
 int workspace(sofie_hip_ctx *ctx, size_t bytes, void **ptr)
 {
    if (ctx->no_alloc) {   // inside the no-allocation entry point: the fixed array or nothing
@@ -234,10 +272,27 @@ int sofie_hip_destroy(sofie_hip_ctx *ctx)
    (void)hipStreamSynchronize(ctx->stream);
    if (ctx->trace) drop_trace(ctx);
    if (ctx->workspace) (void)hipFree(ctx->workspace);
+   for (int i = 0; i < ctx->packed_len; ++i) (void)hipFree(ctx->packed[i].packed);
+   delete[] ctx->packed;
    (void)hipEventDestroy(ctx->ev_start);
    (void)hipEventDestroy(ctx->ev_stop);
    if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
    delete ctx;
+   return SOFIE_HIP_OK;
+}
+
+int sofie_hip_constant_weights(sofie_hip_ctx *ctx, int on)
+{
+   if (!ctx) return SOFIE_HIP_EINVAL;
+   SOFIE_REQUIRE(ctx, !ctx->capturing, "not allowed between capture_begin and capture_end");
+   // a recorded graph may hold the address of a kept copy
+   SOFIE_REQUIRE(ctx, on || ctx->live_graphs == 0 || ctx->packed_len == 0, "recorded graphs of this context may still use the kept copies: destroy them first");
+   ctx->constant_weights = on != 0;
+   if (!on && ctx->packed_len > 0) {
+      SOFIE_HIP_CALL(ctx, hipStreamSynchronize(ctx->stream));      // kernels in flight may still read them
+      for (int i = 0; i < ctx->packed_len; ++i) (void)hipFree(ctx->packed[i].packed);
+      ctx->packed_len = 0;
+   }
    return SOFIE_HIP_OK;
 }
 

@@ -849,6 +849,8 @@ void RModel::GenerateSessionCode()
    fGC += "   { int status = sofie_hip_create(&fCtx.p, device, nullptr);\n";
    fGC += "     if (status != 0) throw std::runtime_error(\"TMVA SOFIE cannot create a device context\"); }\n";
    fGC += "   try {\n";
+   // the weights are uploaded below and never written again: the library may keep its own layouts of them
+   fGC += "   Check(sofie_hip_constant_weights(fCtx, 1), \"Session construction\");\n";
    for (auto &i : fInitializedTensors) {
       if (!i.second.IsWeightTensor()) continue;
       const size_t bytes = ConvertShapeToLength(i.second.shape()) * GetTypeSize(i.second.type());

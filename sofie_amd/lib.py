@@ -52,6 +52,7 @@ SIGNATURES = {
     "sofie_hip_relu_f32": [_p, _p, _p, _z],
     "sofie_hip_maxpool2d_f32": [_p, _p, _p] + [_i] * 11,
     "sofie_hip_avgpool2d_f32": [_p, _p, _p] + [_i] * 12,
+    "sofie_hip_constant_weights": [_p, _i],
     "sofie_hip_maxpool3d_f32": [_p, _p, _p, _i, _p, _p, _p, _p],
     "sofie_hip_avgpool3d_f32": [_p, _p, _p, _i, _p, _p, _p, _p, _i],
     "sofie_hip_quantize_f32_s8": [_p, _p, _p, _z, _f, _i],

@@ -529,6 +529,16 @@ def test_runtime_batch_session(tmp_path):
     assert "sofie_hip_gemm_f32(fCtx, 0, 0, 6, 3, 4," in c and "fBatch" not in c
 
 
+def test_session_promises_constant_weights(tmp_path):
+    """A Session's weights are uploaded in its constructor and never written again: it tells the library so, right
+    behind the creation of the context, and the library keeps its own layouts of them."""
+    c = open(models.conv1d_spec("cw_t").generate(str(tmp_path))[0]).read()
+    create = c.index("sofie_hip_create(&fCtx.p, device, nullptr)")
+    promise = c.index("Check(sofie_hip_constant_weights(fCtx, 1), \"Session construction\");")
+    upload = c.index("sofie_hip_upload(fCtx, tensor_w")
+    assert create < promise < upload
+
+
 def test_pool_1d_and_3d_emission(tmp_path):
     """Pooling over one spatial axis (ROperator_Pool.hxx:329-370) is emitted as the two-axis call on a plane of height
     one; over three axes (:417-470) as the calls that take the geometry as arrays, pads in ONNX order."""

@@ -322,6 +322,74 @@ def test_conv_transpose2d_f32_phases_by_lds_dma(ops):
         assert rel_err(y, ref) <= FP32_TOL
 
 
+def test_constant_weights_keep_the_kernels_layout_of_a_weight_tensor(ops):
+    """sofie_hip_constant_weights: with the promise made, the copy of a weight tensor in the kernel's layout is made by
+    the first call only (the trace shows the small kernel once), results stay what they were, a second geometry on
+    the same tensor gets a copy of its own, taking the promise back returns to a copy per call, and a graph recorded
+    with the promise made holds the convolution alone and replays to the same result."""
+    import ctypes as C
+    from sofie_amd import lib as L
+    r = rng(4242)
+    ctx = ops.Context(0)
+    x = r.standard_normal((3, 16, 20, 20)).astype(np.float32)
+    w = (r.standard_normal((40, 16, 3, 3)) * 0.1).astype(np.float32)
+    b = r.standard_normal(40).astype(np.float32)
+    xt = r.standard_normal((2, 24, 9, 10)).astype(np.float32)
+    wt = (r.standard_normal((24, 18, 4, 4)) * 0.2).astype(np.float32)
+    dx, dw, db, dxt, dwt = ctx.dev(x), ctx.dev(w), ctx.dev(b), ctx.dev(xt), ctx.dev(wt)
+    ctx.sync()
+
+    def traced(call):
+        buf = C.create_string_buffer(4096)
+        n = C.c_int(-1)
+        assert ctx.lib.sofie_hip_trace_begin(ctx.h) == 0
+        out = call()
+        assert ctx.lib.sofie_hip_trace_end(ctx.h, buf, 4096, C.byref(n)) == 0
+        return out, [l.split()[0] for l in buf.value.decode().splitlines()]
+
+    conv = lambda pads=(1, 1): ops.conv2d_f32(dx, dw, db, pads, (1, 1), (1, 1), 1, True, ctx=ctx)
+    convt = lambda: ops.conv_transpose2d_f32(dxt, dwt, None, (1, 1, 1, 1), (2, 2), (1, 1), 1, (0, 0), False, ctx=ctx)
+    y0, names = traced(conv)
+    assert names == ["k_transpose_weights", "k_conv2d_f32_dma_pairs"]
+    t0, names = traced(convt)
+    assert names == ["k_gather_phase_weights", "k_conv2d_f32_dma_pairs_phases"]
+    ctx.check(ctx.lib.sofie_hip_constant_weights(ctx.h, 1))
+    y1, names = traced(conv)
+    assert names == ["k_transpose_weights", "k_conv2d_f32_dma_pairs"]          # the first call with the promise lays it out
+    for _ in range(2):
+        y2, names = traced(conv)
+        assert names == ["k_conv2d_f32_dma_pairs"] and torch.equal(y2, y0)
+    t1, names = traced(convt)
+    assert names == ["k_gather_phase_weights", "k_conv2d_f32_dma_pairs_phases"]
+    t2, names = traced(convt)
+    assert names == ["k_conv2d_f32_dma_pairs_phases"] and torch.equal(t2, t0)
+    # the same tensor read as a grouped convolution's weights: another layout, another copy
+    wg_ = ctx.dev((r.standard_normal((40, 8, 3, 3)) * 0.1).astype(np.float32))
+    yg0 = ops.conv2d_f32(dx, wg_, db, (1, 1), (1, 1), (1, 1), 2, False, ctx=ctx)
+    yg1, names = traced(lambda: ops.conv2d_f32(dx, wg_, db, (1, 1), (1, 1), (1, 1), 2, False, ctx=ctx))
+    assert names == ["k_conv2d_f32_dma_pairs"] and torch.equal(yg1, yg0)
+    # recorded with the promise made: the graph holds the convolution alone
+    y3 = ctx.empty(tuple(y0.shape), torch.float32)
+    call = lambda: ctx.check(ctx.lib.sofie_hip_conv2d_f32(ctx.h, ctx.ptr(dx), ctx.ptr(dw), ctx.ptr(db), ctx.ptr(y3), 3, 16, 20, 20, 40,
+                                                          3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1))
+    ctx.check(ctx.lib.sofie_hip_capture_begin(ctx.h))
+    call()
+    graph = C.c_void_p()
+    ctx.check(ctx.lib.sofie_hip_capture_end(ctx.h, C.byref(graph)))
+    assert ctx.lib.sofie_hip_constant_weights(ctx.h, 0) == L.EINVAL          # the graph may hold a kept copy's address
+    for _ in range(2):
+        y3.zero_()
+        ctx.sync()
+        ctx.check(ctx.lib.sofie_hip_graph_launch(ctx.h, graph))
+        ctx.sync()
+        assert torch.equal(y3, y0)
+    ctx.check(ctx.lib.sofie_hip_graph_destroy(ctx.h, graph))
+    ctx.check(ctx.lib.sofie_hip_constant_weights(ctx.h, 0))
+    y4, names = traced(conv)
+    assert names == ["k_transpose_weights", "k_conv2d_f32_dma_pairs"] and torch.equal(y4, y0)
+    assert rel_err(y0.cpu().numpy(), oracle.conv2d_f32(x, w, b, (1, 1), relu=True)) <= FP32_TOL
+
+
 def test_conv2d_f32_integer_data_is_exact(ops):
     r = rng(9)
     x = r.integers(-6, 7, (2, 8, 11, 13)).astype(np.float32)
