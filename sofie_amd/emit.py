@@ -131,7 +131,7 @@ class ModelSpec:
 
     # ---- generation ------------------------------------------------------------------------
     def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False, batch=None,
-                 runtime_batch=False, no_session=False, emitter=None, env=None, layer_per_call=False):
+                 runtime_batch=False, no_session=False, emitter=None, env=None, layer_per_call=False, params=None):
         """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess). `batch` gives the shape
         parameters of the inputs (dimensions written as names) their value; with `runtime_batch` it is a capacity and
         the generated Session also takes infer(n, ...) for any n up to it. `emitter` names another build of the emit
@@ -149,6 +149,8 @@ class ModelSpec:
             batch = self.batch if batch is None else batch
             if batch is not None:
                 flag += " batch %d" % batch
+            for pname, value in (params or {}).items():      # shape parameters by name (RModel::Initialize(map))
+                flag += " param %s %d" % (pname, value)
             if runtime_batch or self.runtime_batch:
                 flag += " runtimebatch"
             if layer_per_call:

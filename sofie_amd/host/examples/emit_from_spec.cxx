@@ -23,7 +23,7 @@
 //   op QLinearMatMul A AS AZ B BS BZ YS YZ BIAS Y TRANSB
 //   op QLinearConv AUTOPAD GROUP nk k.. np p.. ns s.. X XS XZ W WS WZ YS YZ BIAS Y
 //   op GemmFP8 A AS B BS BIAS Y TRANSB
-//   generate [noweightfile | binaryweightfile | nosession] [batch N] [runtimebatch] [layerpercall]
+//   generate [noweightfile | binaryweightfile | nosession] [batch N] [param NAME VALUE]... [runtimebatch] [layerpercall]
 //                                                  batch N resolves the shape parameters; runtimebatch makes N a capacity
 #include <cctype>
 #include <fstream>
@@ -200,6 +200,7 @@ int main(int argc, char **argv)
          } else if (kw == "generate") {
             std::underlying_type_t<Options> options = static_cast<std::underlying_type_t<Options>>(Options::kDefault);
             int batch = -1;
+            std::map<std::string, size_t> params;
             for (std::string flag; in >> flag;) {
                if (flag == "noweightfile") options = options | Options::kNoWeightFile;
                else if (flag == "binaryweightfile") options = options | Options::kBinaryWeightFile;
@@ -207,7 +208,21 @@ int main(int argc, char **argv)
                else if (flag == "runtimebatch") options = options | Options::kRuntimeBatch;
                else if (flag == "layerpercall") options = options | Options::kLayerPerCall;
                else if (flag == "batch") in >> batch;
+               else if (flag == "param") {
+                  std::string pname;
+                  size_t value = 0;
+                  in >> pname >> value;
+                  params[pname] = value;
+               }
                else throw std::runtime_error("unknown generate flag " + flag);
+            }
+            // several shape parameters: the values by name, as RModel::Initialize(const std::map<...> &) takes them
+            // (the batch number still answers for "bs", "batch_size" and "input_size")
+            if (!params.empty()) {
+               if (batch > 0)
+                  for (const char *n : {"input_size", "batch_size", "bs"})
+                     if (!params.count(n)) params[n] = (size_t)batch;
+               model->Initialize(params);
             }
             model->Generate(options, batch);
             model->OutputGenerated(odir + "/" + name + ".hxx");

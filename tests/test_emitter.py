@@ -529,6 +529,25 @@ def test_runtime_batch_session(tmp_path):
     assert "sofie_hip_gemm_f32(fCtx, 0, 0, 6, 3, 4," in c and "fBatch" not in c
 
 
+def test_two_shape_parameters_get_their_values_by_name(tmp_path):
+    """An input with two named dimensions ([bs, seq, 8]): RModel::Initialize(map) gives each its value, as in the
+    reference (RModel.cxx:408-463); a MatMul of rank 3 against a [8, 4] matrix then has its sizes at generation time.
+    A parameter left without a value is an error that names the tensor."""
+    def spec(name):
+        s = emit.ModelSpec(name)
+        s.add_input("x", "FLOAT", ("bs", "seq", 8))
+        s.add_init("w", np.arange(32, dtype=np.float32).reshape(8, 4))
+        s.gemm("x", "w", None, "y", beta=0.0)
+        s.set_output("y")
+        return s
+    c = open(spec("two_params").generate(str(tmp_path), params={"bs": 3, "seq": 5})[0]).read()
+    assert "std::vector<float> ret(60);" in c            # 3 * 5 * 4
+    c = open(spec("two_params_b").generate(str(tmp_path), batch=2, params={"seq": 7})[0]).read()
+    assert "std::vector<float> ret(56);" in c            # the batch number answers for "bs"
+    with pytest.raises(RuntimeError, match="parametric shape"):
+        spec("two_params_c").generate(str(tmp_path), batch=2)
+
+
 def test_session_promises_constant_weights(tmp_path):
     """A Session's weights are uploaded in its constructor and never written again: it tells the library so, right
     behind the creation of the context, and the library keeps its own layouts of them."""
