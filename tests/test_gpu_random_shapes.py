@@ -204,6 +204,74 @@ def test_gemm_f32_random_shapes(ops, seed):
     assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (M, N, K, tA, tB)
 
 
+def _kernels_of(ops, call):
+    """Names of the kernels `call` launches on the default context (sofie_hip_trace_begin / _end)."""
+    import ctypes as C
+    ctx = ops.default_context()
+    buf = C.create_string_buffer(4096)
+    n = C.c_int(-1)
+    assert ctx.lib.sofie_hip_trace_begin(ctx.h) == 0
+    try:
+        out = call()
+    finally:
+        assert ctx.lib.sofie_hip_trace_end(ctx.h, buf, 4096, C.byref(n)) == 0
+    return out, [l.split()[0] for l in buf.value.decode().splitlines()]
+
+
+def test_gemm_f32_lds_dma_random_shapes(ops):
+    """Random products of the shapes the LDS-DMA Gemm kernels take (K in whole stages of 32, rows of whole 16-byte
+    chunks, at least 32 tiles of 64 x 64): ragged last tiles in M and N, both layouts of B, row bias or none, alpha,
+    beta, ReLU; 1e-5 relative against the oracle. The trace names the kernel, and both tile sizes occur."""
+    seen = {}
+    for seed in range(14):
+        r = np.random.default_rng(9900 + seed)
+        big = seed % 3 == 2                       # 256 tiles of 128 x 128 or more: the 128 x 128-tile form
+        M = int(r.integers(2049, 2400)) if big else int(r.integers(330, 1200))
+        N = int(r.integers(2049, 2300)) if big else int(r.integers(330, 1200))
+        K = 32 * int(r.integers(1, 5 if big else 12))
+        tB = bool(r.integers(0, 2))
+        if not tB:
+            N -= N % 4
+        A = r.standard_normal((M, K)).astype(np.float32)
+        B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+        bias = r.standard_normal(N).astype(np.float32) if seed % 2 else None
+        alpha, relu = float(r.choice([1.0, 0.5, -2.0])), bool(r.integers(0, 2))
+        beta = float(r.choice([1.0, 0.25])) if bias is not None else 0.0
+        got, names = _kernels_of(ops, lambda: ops.gemm_f32(A, B, bias, alpha, beta, False, tB, relu))
+        assert names in (["k_gemm_f32_dma"], ["k_gemm_f32_dma64"]), (names, M, N, K, tB)
+        seen[names[0]] = seen.get(names[0], 0) + 1
+        ref = oracle.gemm_f32(A, B, bias, alpha, beta, False, tB, relu)
+        assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (M, N, K, tB)
+    assert seen.get("k_gemm_f32_dma", 0) >= 3 and seen.get("k_gemm_f32_dma64", 0) >= 3, seen
+
+
+def test_conv2d_f32_lds_dma_random_shapes(ops):
+    """Random layers with channel counts the LDS-DMA convolution kernel takes (even channel blocks with at least 18
+    taps): kernels up to 4 x 4, strides, dilations, unequal pads, groups, ragged channel and pixel tiles; 1e-5 relative
+    against the oracle. Both of its matrix loops (with and without the table of patch offsets) must have run."""
+    seen = {}
+    for seed in range(24):
+        r = np.random.default_rng(9950 + seed)
+        g = int(r.choice([1, 1, 2]))
+        icg = int(r.choice([4, 6, 8, 10, 12, 16, 24, 32]))
+        C, OC = g * icg, g * int(r.integers(1, 90))
+        k, s, p, H, W = _conv_geometry(r, 26, kmax=4)
+        d = (int(r.integers(1, 3)), int(r.integers(1, 3)))
+        ke = ((k[0] - 1) * d[0] + 1, (k[1] - 1) * d[1] + 1)
+        H, W = max(H, ke[0]), max(W, ke[1])
+        N = int(r.integers(1, 4))
+        x = r.standard_normal((N, C, H, W)).astype(np.float32)
+        w = (r.standard_normal((OC, icg) + k) / np.sqrt(icg * k[0] * k[1])).astype(np.float32)
+        b = r.standard_normal(OC).astype(np.float32) if seed % 2 else None
+        relu = bool(r.integers(0, 2))
+        got, names = _kernels_of(ops, lambda: ops.conv2d_f32(x, w, b, p, s, d, g, relu))
+        seen[names[-1]] = seen.get(names[-1], 0) + 1
+        ref = oracle.conv2d_f32(x, w, b, p, s, d, g, relu)
+        assert got.shape == ref.shape
+        assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (names, C, OC, g, k, s, p, d, H, W, N)
+    assert seen.get("k_conv2d_f32_dma", 0) >= 3 and seen.get("k_conv2d_f32_dma_pairs", 0) >= 3, seen
+
+
 @pytest.mark.parametrize("seed", range(12))
 def test_conv_transpose2d_f32_random_shapes(ops, seed):
     r = np.random.default_rng(9600 + seed)
