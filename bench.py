@@ -204,6 +204,11 @@ def cpu_fp32_baselines(threads, conv_images=64):
                 "cores": t, "calls": gm["calls"],
                 "sample": "%d of the 4096 rows of the product (rows are independent; %.1f GFLOP per call)"
                           % (gemm_rows, 2.0 * gemm_rows * 4096 * 4096 / 1e9)}
+        g8 = cpu_emitted("gemm", t, chosen, ("--images", "8", "--calls", "20"))
+        if g8:
+            res["gemm_4096_batch8_%dthr" % t] = {
+                "median_ms": g8["median_ms"], "best_ms": g8["best_ms"], "gbs": 4.0 * 4096 * 4096 / g8["median_ms"] / 1e6,
+                "cores": t, "calls": g8["calls"], "sample": "the whole 8 x 4096 x 4096 product (sgemm_ on 8 rows)"}
         if m:
             res["mlp_b256_%dthr" % t] = {"median_us": m["median_ms"] * 1e3, "best_us": m["best_ms"] * 1e3,
                                          "inferences_per_s": 256 / (m["median_ms"] * 1e-3), "cores": t, "calls": m["calls"]}
@@ -238,7 +243,7 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     ap.add_argument("--kernel-probe", default="",
                     help="launch one named workload a few times and exit (target of rocprofv3 runs): gemm_s8, gemm_s8_nk, "
-                         "gemm_fp8, gemm_fp8_nk, gemm_f32, gemm_f32_nk, conv_s8, conv_f32, conv_transpose_f32")
+                         "gemm_fp8, gemm_fp8_nk, gemm_f32, gemm_f32_nk, gemm_f32_batch8, conv_s8, conv_f32, conv_transpose_f32")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collective, no sharding "
@@ -426,12 +431,16 @@ def main():
         entry["frac_peak"] = rate / meta["peak"]
         if "bytes" in meta:
             entry["gbs"] = meta["bytes"] / med / 1e6
+        if meta.get("bound") == "hbm":
+            entry["bound"] = "hbm"
+            entry["frac_hbm_peak"] = entry["gbs"] / PEAK_HBM_GBS
         res[name] = entry
     out["fp8_gemm"] = dict(res["gemm_fp8"], peak_tflops=PEAK_FP8_TFLOPS)
     out["fp8_gemm_b_nk"] = res["gemm_fp8_nk"]
     out["int8_gemm_b_nk"] = res["gemm_s8_nk"]
     out["gemm_f32"] = res["gemm_f32"]
     out["gemm_f32_b_nk"] = res["gemm_f32_nk"]
+    out["gemm_f32_batch8"] = res["gemm_f32_batch8"]
     out["conv_f32"] = res["conv_f32"]
     out["conv_s8"] = res["conv_s8"]
     out["conv_transpose_f32"] = res["conv_transpose_f32"]
@@ -484,6 +493,14 @@ def workloads(ctx, torch, L, rng):
             {"workload": "fp32 Gemm 4096^3 (ROperator_Gemm: Y = A B + bias row, ReLU fused), A and B N(0,1), B %s"
                          % ("[N,K] (transB = 1)" if tb else "[K,N]"),
              "ops": 2.0 * n ** 3, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 20})
+    # the same layer on a batch of 8 rows: a pass over the 64 MB of B, bound by memory
+    Y8 = ctx.empty((8, n), torch.float32)
+    w["gemm_f32_batch8"] = ((lambda: ctx.check(ctx.lib.sofie_hip_gemm_f32(
+        ctx.h, 0, 0, 8, n, n, 1.0, ctx.ptr(Af), n, ctx.ptr(Bf), n, 1.0, ctx.ptr(bf), L.BIAS_ROW, ctx.ptr(Y8), n, L.ACT_RELU))),
+        {"workload": "fp32 Gemm 8 x 4096 x 4096 (a 4096 -> 4096 layer on a batch of 8: Y = A B + bias row, ReLU fused), B [K,N]; "
+                     "memory-bound: gbs = algorithmic bytes (B, A, Y, bias once) per second, frac_hbm_peak against 8 TB/s",
+         "ops": 2.0 * 8 * n * n, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 200,
+         "bytes": 4.0 * (n * n + 8 * n + 8 * n + n), "bound": "hbm"})
     # fp32 conv layer: batch 256, 64 -> 128 channels, 56x56, 3x3, pad 1, bias + ReLU
     x = torch.rand(256, 64, 56, 56, device=ctx.device)
     wt = torch.randn(128, 64, 3, 3, device=ctx.device) * (2.0 / 576) ** 0.5

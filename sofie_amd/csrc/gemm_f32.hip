@@ -320,6 +320,243 @@ __global__ void __launch_bounds__(256, T == 2 ? 2 : 4) k_gemm_f32_dma(GemmF32Arg
    }
 }
 
+// Few rows of A (M <= 64: a layer on a small batch): the product is a pass over B, bound by memory, and tiles of
+// 64 x 64 outputs would leave most of the device idle. Here a wavefront owns all rows of A (MT tiles of T = 16 rows,
+// v_mfma_f32_16x16x4_f32) and 4 T = 64 columns: its accumulators are MT x 4 tiles of T x T (rows of A x columns), and B
+// goes from global memory straight into the matrix instructions' operand registers, 16 bytes per lane, with no LDS on
+// the way. With lane = (j = lane % T, kg = lane / T):
+//   * B [K][N]: a lane loads columns 4 j .. 4 j + 3 of row k0 + 4 kg + u (a wavefront's load: 4 rows of 256
+//     contiguous bytes); element e of the four feeds the tile of columns 4 j + e, so a lane ends up with 4 consecutive
+//     columns of a row.
+//   * B [N][K]: a lane loads k0 + 4 kg .. + 3 of column T q + j; element u feeds instruction u of tile q.
+// A lane's 4 consecutive k of its row of A arrive the same way (k0 + 4 kg .. + 3, one instruction per element). The
+// grid is column blocks x slices of K; the four wavefronts of a workgroup take the slice's chunks of 16 k in turn,
+// each with the loads of the next three chunks in flight while it multiplies, and add their accumulators up through
+// LDS. With more than one slice the sums go to a scratch buffer [slice][M][N] and k_gemm_f32_skinny_finish adds them
+// in slice order and applies alpha, bias and ReLU (a fixed order: the result does not depend on timing). Rows behind
+// M, columns behind N and k behind the slice get offsets outside the buffer descriptors and arrive as zeros.
+template <int T> struct SkinnyTile;
+template <> struct SkinnyTile<16> {
+   typedef v4f Acc;
+   static constexpr int NR = 4;
+   static __device__ __forceinline__ Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+   static __device__ __forceinline__ int row(int r, int kg) { return kg * 4 + r; }
+};
+
+template <bool B_NK, int T, int MT>
+__global__ void __launch_bounds__(256) k_gemm_f32_skinny(GemmF32Args g, float *partial, int kslice, int splits)
+{
+   typedef SkinnyTile<T> Tile;
+   constexpr int NR = Tile::NR;
+   constexpr int CHUNK = 256 / T;                      // k per chunk: 4 per lane, 64 / T groups of lanes
+   constexpr int COLS = 4 * T;                         // columns of a workgroup
+   constexpr unsigned OUTSIDE = 0x80000000u;
+   __shared__ float red[2 * MT * 4 * NR * 64];
+   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+   const int fr = lane % T, fk = lane / T;
+   const int c0 = blockIdx.x * COLS;
+   const int k_begin = blockIdx.y * kslice;
+   const int k_end = g.K < k_begin + kslice ? g.K : k_begin + kslice;
+   const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(g.A), 0, (int)(((size_t)(g.M - 1) * g.lda + g.K) * 4), 0x00020000);
+   const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float *>(g.B), 0, (int)((B_NK ? (size_t)(g.N - 1) * g.ldb + g.K : (size_t)(g.K - 1) * g.ldb + g.N) * 4), 0x00020000);
+   unsigned a_off[MT], b_off[B_NK ? 4 : 1];
+#pragma unroll
+   for (int t = 0; t < MT; ++t) a_off[t] = t * T + fr < g.M ? (unsigned)(((t * T + fr) * g.lda + 4 * fk) * 4) : OUTSIDE;
+   if constexpr (B_NK) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+         const int n = c0 + T * q + fr;
+         b_off[q] = n < g.N ? (unsigned)((n * g.ldb + 4 * fk) * 4) : OUTSIDE;
+      }
+   } else {
+      const int n = c0 + 4 * fr;
+      b_off[0] = n < g.N ? (unsigned)((4 * fk * g.ldb + n) * 4) : OUTSIDE;
+   }
+   struct Chunk {
+      v4f a[MT], b[4];
+   };
+   auto load = [&](Chunk &c, int k0) {
+      // a lane's four k lie inside the slice together or not at all (K and the slices are multiples of 4)
+      const bool in = k0 + 4 * fk < k_end;
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+         c.a[t] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ars, in ? a_off[t] : OUTSIDE, k0 * 4, 0));
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+         if constexpr (B_NK)
+            c.b[q] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(brs, in ? b_off[q] : OUTSIDE, k0 * 4, 0));
+         else
+            c.b[q] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(brs, in ? b_off[0] : OUTSIDE, (k0 + q) * g.ldb * 4, 0));
+      }
+   };
+   typename Tile::Acc acc[MT][4];
+#pragma unroll
+   for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+         for (int r = 0; r < NR; ++r) acc[t][q][r] = 0.0f;
+   auto multiply = [&](const Chunk &c) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+         for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+               // B [K][N]: load u is row k0 + 4 kg + u, its element q a column; B [N][K]: load q is a group of columns,
+               // its element u a k
+               const float b = B_NK ? c.b[q][u] : c.b[u][q];
+               acc[t][q] = Tile::mma(c.a[t][u], b, acc[t][q]);
+            }
+   };
+   // chunks wave, wave + 4, ... of the slice; three chunks ahead are in flight while one is multiplied (loads behind
+   // the slice's end ask for nothing)
+   constexpr int STEP = 4 * CHUNK;
+   Chunk c0_, c1_, c2_, c3_;
+   int k0 = k_begin + wave * CHUNK;
+   load(c0_, k0);
+   load(c1_, k0 + STEP);
+   load(c2_, k0 + 2 * STEP);
+   for (; k0 < k_end; k0 += STEP) {
+      load(c3_, k0 + 3 * STEP);
+      multiply(c0_);
+      c0_ = c1_;
+      c1_ = c2_;
+      c2_ = c3_;
+   }
+   // the four wavefronts' sums meet in LDS: wavefronts 2 and 3 hand theirs to 0 and 1, then 1 hands its to 0
+   // ((w0 + w2) + (w1 + w3): a fixed order)
+   auto put = [&](float *dst) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+         for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < NR; ++r) dst[((t * 4 + q) * NR + r) * 64 + lane] = acc[t][q][r];
+   };
+   auto add = [&](const float *src) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+         for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < NR; ++r) acc[t][q][r] = __fadd_rn(acc[t][q][r], src[((t * 4 + q) * NR + r) * 64 + lane]);
+   };
+   constexpr int BLOCK = MT * 4 * NR * 64;
+   if (wave >= 2) put(red + (wave - 2) * BLOCK);
+   __syncthreads();
+   if (wave < 2) add(red + wave * BLOCK);
+   __syncthreads();
+   if (wave == 1) put(red);
+   __syncthreads();
+   if (wave == 0) add(red);
+   if (wave != 0) return;
+   // tile (t, q), register r of a lane: row t * T + Tile::row(r, kg); column c0 + 4 j + q (B [K][N]) or c0 + T q + j
+   const bool last = splits == 1;
+   float *const out = last ? g.Y : partial + (size_t)blockIdx.y * g.M * g.N;
+   const int ldo = last ? g.ldy : g.N;
+   const bool vec_out = !last || (g.ldy % 4 == 0 && (reinterpret_cast<uintptr_t>(g.Y) & 15u) == 0);   // rows of whole 16-byte chunks
+   auto finish = [&](float v, int m, int n) {
+      if (!last) return v;
+      v = __fmul_rn(g.alpha, v);
+      if (g.bias_kind == SOFIE_BIAS_ROW) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[n]));
+      else if (g.bias_kind == SOFIE_BIAS_FULL) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[(size_t)m * g.ldy + n]));
+      else if (g.bias_kind == SOFIE_BIAS_COL) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[m]));
+      if (g.relu) v = v > 0.0f ? v : 0.0f;
+      return v;
+   };
+#pragma unroll
+   for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int r = 0; r < NR; ++r) {
+         const int m = t * T + Tile::row(r, fk);
+         if (m >= g.M) continue;
+         if constexpr (B_NK) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+               const int n = c0 + T * q + fr;
+               if (n < g.N) out[(size_t)m * ldo + n] = finish(acc[t][q][r], m, n);
+            }
+         } else {
+            const int n = c0 + 4 * fr;     // N is a multiple of 4 on this path: the four columns are inside together
+            if (n < g.N) {
+               float *o = out + (size_t)m * ldo + n;
+               const v4f v = {finish(acc[t][0][r], m, n), finish(acc[t][1][r], m, n + 1), finish(acc[t][2][r], m, n + 2),
+                              finish(acc[t][3][r], m, n + 3)};
+               if (vec_out) *reinterpret_cast<v4f *>(o) = v;
+               else {
+#pragma unroll
+                  for (int q = 0; q < 4; ++q) o[q] = v[q];
+               }
+            }
+         }
+      }
+}
+
+// Sum of the K slices' partial products in slice order, then alpha, bias and ReLU: one thread per output. The loads of
+// eight slices are in flight together; the additions keep the slices' order.
+__global__ void __launch_bounds__(256) k_gemm_f32_skinny_finish(GemmF32Args g, const float *__restrict__ partial, int splits)
+{
+   const int idx = blockIdx.x * 256 + threadIdx.x;
+   if (idx >= g.M * g.N) return;
+   const int m = idx / g.N, n = idx - m * g.N;
+   const size_t plane = (size_t)g.M * g.N;
+   float v = 0.0f;
+   int s = 0;
+   for (; s + 8 <= splits; s += 8) {
+      float p[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) p[i] = partial[(size_t)(s + i) * plane + idx];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v = __fadd_rn(v, p[i]);
+   }
+   for (; s < splits; ++s) v = __fadd_rn(v, partial[(size_t)s * plane + idx]);
+   v = __fmul_rn(g.alpha, v);
+   if (g.bias_kind == SOFIE_BIAS_ROW) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[n]));
+   else if (g.bias_kind == SOFIE_BIAS_FULL) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[(size_t)m * g.ldy + n]));
+   else if (g.bias_kind == SOFIE_BIAS_COL) v = __fadd_rn(v, __fmul_rn(g.beta, g.bias[m]));
+   if (g.relu) v = v > 0.0f ? v : 0.0f;
+   g.Y[(size_t)m * g.ldy + n] = v;
+}
+
+// M <= 64 rows on k_gemm_f32_skinny. Slices of K so that about eight workgroups per compute unit exist, each wavefront
+// with at least four chunks, and so that the partial sums stay below a quarter of B's bytes once they are more than a
+// few megabytes (below that the launch is latency, not traffic).
+template <bool B_NK, int T, int MT>
+int launch_skinny_as(sofie_hip_ctx *ctx, GemmF32Args &g)
+{
+   constexpr int CHUNK = 256 / T;
+   const int blocks = cdiv(g.N, 4 * T);
+   int splits = 8 * ctx->num_cus / blocks;
+   if (splits > g.K / (16 * CHUNK)) splits = g.K / (16 * CHUNK);
+   if ((size_t)splits * g.M * g.N * 4 > ((size_t)4 << 20) && splits > g.K / (4 * g.M)) splits = g.K / (4 * g.M);
+   if (splits < 1) splits = 1;
+   const int kslice = cdiv(cdiv(g.K, splits), 4 * CHUNK) * 4 * CHUNK;
+   splits = cdiv(g.K, kslice);
+   float *partial = nullptr;
+   if (splits > 1) {
+      void *ws = nullptr;
+      if (int rc = workspace(ctx, (size_t)splits * g.M * g.N * sizeof(float), &ws)) return rc;
+      partial = static_cast<float *>(ws);
+   }
+   hipLaunchKernelGGL((k_gemm_f32_skinny<B_NK, T, MT>), dim3(blocks, splits), dim3(256), 0, ctx->stream, g, partial, kslice, splits);
+   if (int rc = check_launch(ctx, "k_gemm_f32_skinny")) return rc;
+   if (splits == 1) return SOFIE_HIP_OK;
+   hipLaunchKernelGGL(k_gemm_f32_skinny_finish, dim3(cdiv(g.M * g.N, 256)), dim3(256), 0, ctx->stream, g, partial, splits);
+   return check_launch(ctx, "k_gemm_f32_skinny_finish");
+}
+
+int launch_skinny(sofie_hip_ctx *ctx, GemmF32Args &g)
+{
+   if (g.M <= 16) return g.transB ? launch_skinny_as<true, 16, 1>(ctx, g) : launch_skinny_as<false, 16, 1>(ctx, g);
+   // 17 to 64 rows as two or four tiles of 16 rows: 32 x 32 tiles (twice the columns per wavefront, twice the
+   // accumulator registers) measured 9 - 13 % slower (64 x 4096 x 4096: 42.7 against 37.7 us)
+   if (g.M <= 32) return g.transB ? launch_skinny_as<true, 16, 2>(ctx, g) : launch_skinny_as<false, 16, 2>(ctx, g);
+   return g.transB ? launch_skinny_as<true, 16, 4>(ctx, g) : launch_skinny_as<false, 16, 4>(ctx, g);
+}
+
 }  // namespace
 
 extern "C" int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, int M, int N, int K, float alpha,
@@ -356,6 +593,13 @@ extern "C" int sofie_hip_gemm_f32(sofie_hip_ctx *ctx, int transA, int transB, in
                     (transB || N % 4 == 0) && aligned16(A) && aligned16(B) && bias_kind != SOFIE_BIAS_FULL &&
                     (size_t)128 * lda * 4 < (1u << 31) && (size_t)(transB ? 128 : K) * ldb * 4 < (1u << 31) &&
                     (size_t)128 * ldy * 4 < (1u << 31) && (size_t)cdiv(M, tile) * cdiv(N, tile) < (1u << 30);
+   // a few rows of A on a B of some size: a pass over B (k_gemm_f32_skinny); needs whole 16-byte chunks per lane. With 33 to
+   // 64 rows and thousands of column tiles the 64 x 64 tiles below fill the device and reuse B from LDS.
+   const bool skinny = (M <= 32 || (M <= 64 && N < 8192)) && !transA && K >= 64 && K % 4 == 0 && (size_t)N * K >= 64 * 1024 && lda % 4 == 0 && ldb % 4 == 0 &&
+                       (transB || N % 4 == 0) && aligned16(A) && aligned16(B) &&
+                       (size_t)M * lda * 4 < (1u << 31) && (size_t)(transB ? N : K) * ldb * 4 < (1u << 31) &&
+                       (size_t)M * ldy < (1u << 31);
+   if (skinny) return launch_skinny(ctx, g);
    if (dma) {
       constexpr auto kern_nk2 = k_gemm_f32_dma<false, 2>, kern_kn2 = k_gemm_f32_dma<true, 2>;
       constexpr auto kern_nk1 = k_gemm_f32_dma<false, 1>, kern_kn1 = k_gemm_f32_dma<true, 1>;

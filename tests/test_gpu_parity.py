@@ -205,6 +205,54 @@ def test_gemm_f32_large_integer_data_is_exact_with_a_column_bias(ops):
     assert np.array_equal(y.cpu().numpy(), ref)
 
 
+@pytest.mark.parametrize("M,N,K,tB", [
+    (1, 1024, 1024, 0), (8, 4096, 2048, 0), (5, 1000, 260, 0), (32, 516, 1028, 0), (33, 768, 512, 0), (64, 2048, 4096, 0),
+    (1, 1024, 1024, 1), (7, 1003, 516, 1), (32, 130, 2048, 1), (40, 999, 1000, 1), (64, 4096, 1024, 1), (16, 256, 256, 0),
+])
+def test_gemm_f32_few_rows(ops, M, N, K, tB):
+    """A layer on a small batch (at most 64 rows of A) runs as a pass over B with K cut into slices
+    (k_gemm_f32_skinny, and k_gemm_f32_skinny_finish where there is more than one slice): both layouts of B, ragged
+    column blocks, K that is no multiple of a wavefront's chunk of 8 or of a slice, every bias kind, alpha, beta, ReLU;
+    1e-5 relative against the oracle's own summation and against float64."""
+    r = rng(930 + M + N + K + tB)
+    A = r.standard_normal((M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    for kind in range(3):
+        bias = [None, r.standard_normal(N).astype(np.float32), r.standard_normal((M, N)).astype(np.float32)][kind]
+        alpha, beta, relu = [1.0, 0.5, -2.0][kind], (0.0 if bias is None else [1.0, 0.25][kind % 2]), kind != 1
+        y, names = _kernels_of(ops, lambda: ops.gemm_f32(A, B, bias, alpha, beta, False, bool(tB), relu))
+        assert names in (["k_gemm_f32_skinny"], ["k_gemm_f32_skinny", "k_gemm_f32_skinny_finish"]), names
+        ref = alpha * (A.astype(np.float64) @ (B.T if tB else B).astype(np.float64)) + (beta * bias if bias is not None else 0.0)
+        ref = np.maximum(ref, 0) if relu else ref
+        assert y.shape == ref.shape
+        assert rel_err(y, ref) <= FP32_TOL
+        assert rel_err(y, oracle.gemm_f32(A, B, bias, alpha, beta, False, bool(tB), relu)) <= FP32_TOL
+
+
+def test_gemm_f32_few_rows_integer_data_is_exact_with_a_column_bias(ops):
+    """Integer operands make every order of summation exact: the sliced pass over B against int64 numpy, bias as a
+    column (one value per row), rows of A and Y wider than the matrices, through the C ABI."""
+    from sofie_amd import lib as L
+    r = rng(931)
+    M, N, K = 48, 1536, 2052
+    A = np.zeros((M, K + 12), dtype=np.float32)
+    A[:, :K] = r.integers(-8, 9, (M, K))
+    A[:, K:] = np.nan                                     # what lies behind K in a row must not reach the sums
+    B = r.integers(-8, 9, (K, N)).astype(np.float32)
+    col = r.integers(-50, 50, M).astype(np.float32)
+    ctx = ops.default_context()
+    a, b, c = ctx.dev(A), ctx.dev(B), ctx.dev(col)
+    y = ctx.empty((M, N + 4), torch.float32)
+    y.fill_(-7.0)
+    ctx.check(ctx.lib.sofie_hip_gemm_f32(ctx.h, 0, 0, M, N, K, 2.0, ctx.ptr(a), K + 12, ctx.ptr(b), N, 3.0, ctx.ptr(c), L.BIAS_COL,
+                                         ctx.ptr(y), N + 4, L.ACT_RELU))
+    ctx.sync()
+    ref = np.maximum(2 * (A[:, :K].astype(np.int64) @ B.astype(np.int64)) + 3 * col.astype(np.int64)[:, None], 0)
+    got = y.cpu().numpy()
+    assert np.array_equal(got[:, :N], ref)
+    assert np.all(got[:, N:] == -7.0)
+
+
 def test_gemm_f32_full_bias_and_error_path(ops):
     r = rng(7)
     A = r.standard_normal((50, 20)).astype(np.float32)

@@ -245,6 +245,34 @@ def test_gemm_f32_lds_dma_random_shapes(ops):
     assert seen.get("k_gemm_f32_dma", 0) >= 3 and seen.get("k_gemm_f32_dma64", 0) >= 3, seen
 
 
+def test_gemm_f32_few_rows_random_shapes(ops):
+    """Random layers on a small batch (1 to 64 rows of A, K a multiple of 4, B of at least 64 K elements): the sliced pass
+    over B (k_gemm_f32_skinny) against the oracle, 1e-5 relative; both layouts of B, every row-tile count, with and
+    without the second pass over the slices."""
+    seen = {}
+    for seed in range(24):
+        r = np.random.default_rng(9970 + seed)
+        M = int(r.choice([1, 2, 7, 16, 17, 31, 32, 33, 50, 64]))
+        tB = bool(r.integers(0, 2))
+        N = int(r.integers(64, 2500))
+        if not tB:
+            N -= N % 4
+        K = 4 * int(r.integers(16, 700))
+        if N * K < 65536:
+            K = 4 * (65536 // (4 * N) + 1)
+        A = r.standard_normal((M, K)).astype(np.float32)
+        B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+        bias = r.standard_normal(N).astype(np.float32) if seed % 2 else None
+        alpha, relu = float(r.choice([1.0, 0.5, -2.0])), bool(r.integers(0, 2))
+        beta = float(r.choice([1.0, 0.25])) if bias is not None else 0.0
+        got, names = _kernels_of(ops, lambda: ops.gemm_f32(A, B, bias, alpha, beta, False, tB, relu))
+        assert names[0] == "k_gemm_f32_skinny" and len(names) <= 2, (names, M, N, K, tB)
+        seen[len(names)] = seen.get(len(names), 0) + 1
+        ref = oracle.gemm_f32(A, B, bias, alpha, beta, False, tB, relu)
+        assert np.max(np.abs(got - ref)) <= 1e-5 * max(1.0, float(np.max(np.abs(ref)))), (M, N, K, tB)
+    assert seen.get(1, 0) >= 1 and seen.get(2, 0) >= 3, seen
+
+
 def test_conv2d_f32_lds_dma_random_shapes(ops):
     """Random layers with channel counts the LDS-DMA convolution kernel takes (even channel blocks with at least 18
     taps): kernels up to 4 x 4, strides, dilations, unequal pads, groups, ragged channel and pixel tiles; 1e-5 relative
