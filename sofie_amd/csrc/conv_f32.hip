@@ -53,6 +53,10 @@ struct ConvArgs {
    int wvec;           // weights are staged with 16-byte loads (see launch)
    FastDiv dPW, dPH, dKC, dK4;   // divisions by the patch extents and the K-chunk length (/4) in the staging loops
    FastDiv dUH, dUW, dOW;
+   // csplit > 1 (k_conv2d_f32_dma without phases): blockIdx.z = image * csplit + slice; a slice sums its share of the
+   // channel blocks into partial [slice][N][OC][OH*OW] without bias and ReLU, k_conv_f32_split_finish adds the slices
+   int csplit;
+   float *partial;
    // nphases > 1: blockIdx.z = image * nphases + phase, and the phase's geometry replaces the fields above
    int nphases;
    PhaseArgs phase[SOFIE_CONV_MAX_PHASES];
@@ -303,7 +307,20 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    const int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z;
    int n = bz;
    int oy0 = 0, ox0 = 0;
+   int c_begin = 0, c_end = g.icg / g.ICB;
    FastDiv dOW = gg.dOW;
+   if constexpr (!PHASES) {
+      if (gg.csplit > 1) {
+         // a slice of the channel blocks: raw sums into its plane of the scratch buffer
+         const int slice = bz % gg.csplit, per = (c_end + gg.csplit - 1) / gg.csplit;
+         n = bz / gg.csplit;
+         c_begin = slice * per;
+         c_end = c_end < c_begin + per ? c_end : c_begin + per;
+         g.y = gg.partial + (size_t)slice * gg.N * g.OC * g.OH * g.OW;
+         g.bias = nullptr;
+         g.relu = 0;
+      }
+   }
    if constexpr (PHASES) {
       const int pi = bz % gg.nphases;
       n = bz / gg.nphases;
@@ -316,6 +333,7 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
       g.PH = q.PH; g.PW = q.PW; g.dPW = q.dPW; g.dPH = q.dPH;
       g.w = gg.w + q.woff;
       oy0 = q.oy0; ox0 = q.ox0; dOW = q.dOW;
+      c_end = g.icg / g.ICB;
    }
    extern __shared__ __align__(16) unsigned char smem_raw[];
    const int patch_len = g.ICB * g.PH * g.PW;
@@ -396,14 +414,13 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
             dma16(wrs, sw + (r0 * BOC + wave * 256) * 4, (int)wofs, (int)(c * wblock + (r0 / ROWS_PER_REQUEST) * wstep));
    };
 
-   const int nblocks = g.icg / g.ICB;
    const int nsteps = p0 + wn * TJ * 32 < OHW ? g.KC / 2 : 0;   // a wavefront with no pixel of the plane multiplies nothing
-   request(0, 0);
+   request(c_begin, 0);
    wait_vmcnt<0>();
-   __syncthreads();   // block 0 and the koff table are in LDS
-   for (int c = 0; c < nblocks; ++c) {
-      if (c + 1 < nblocks) request(c + 1, (c + 1) & 1);
-      const float *const sW = bufs + (c & 1) * buf_len, *const patch = sW + g.KC * BOC;
+   __syncthreads();   // the first block and the koff table are in LDS
+   for (int c = c_begin; c < c_end; ++c) {
+      if (c + 1 < c_end) request(c + 1, (c + 1 - c_begin) & 1);
+      const float *const sW = bufs + ((c - c_begin) & 1) * buf_len, *const patch = sW + g.KC * BOC;
       if constexpr (KWT > 0) {
          // K runs (channel pair, kernel row, kernel column, channel of the pair): the two K values of a matrix
          // instruction are the same tap of two neighbouring channels, so a lane's patch address is its own constant
@@ -490,6 +507,25 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
             store4_buf(yrs, v, voff, (unsigned)oc_uniform * plane4);
          }
    }
+}
+
+// Sum of the channel slices' partial outputs in slice order, then bias and ReLU: one thread per output value.
+__global__ void __launch_bounds__(256) k_conv_f32_split_finish(const float *__restrict__ partial, float *__restrict__ y,
+                                                               const float *__restrict__ bias, int slices, size_t total,
+                                                               int plane, int OC, int relu)
+{
+   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+   if (idx >= total) return;
+   float p[8];
+#pragma unroll
+   for (int i = 0; i < 8; ++i) p[i] = i < slices ? partial[(size_t)i * total + idx] : 0.0f;
+   float v = p[0];
+#pragma unroll
+   for (int i = 1; i < 8; ++i)
+      if (i < slices) v = __fadd_rn(v, p[i]);
+   if (bias) v = __fadd_rn(v, bias[(idx / plane) % OC]);
+   if (relu) v = v > 0.0f ? v : 0.0f;
+   y[idx] = v;
 }
 
 // Weights of a plain convolution w [OC][C/groups][KH][KW] as k_conv2d_f32_dma reads them: wt [group][K][wstride],
@@ -633,7 +669,7 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          auto pick = [&](bool even) {
             for (int icb = g.icg < 96 / KHW ? g.icg : 96 / KHW; icb >= 1; --icb) {
                const int kc = icb * KHW;
-               if (kc < 18) break;
+               if (kc < 16) break;
                if (g.icg % icb != 0 || kc % 2 != 0 || (even && icb % 2 != 0) ||
                    dma_lds_bytes(kc, (size_t)icb * g.PH * g.PW, BOC) > budget || (size_t)icb * g.PH * g.PW > SOFIE_CONV_DMA_PATCH)
                   continue;
@@ -652,10 +688,32 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             g.KC = icb * KHW;
             g.dPW = make_fastdiv((unsigned)g.PW);
             g.dPH = make_fastdiv((unsigned)g.PH);
-            void *ws = nullptr;
+            // Fewer tiles than compute units (a layer on one image or a few): the channel blocks are dealt to up to 8
+            // slices, each a workgroup of its own that writes raw sums, and a second pass adds them (a fixed order)
+            const size_t tiles = (size_t)cdiv(OHW, BP) * g.groups * octiles * g.N;
+            const int nblocks = g.icg / icb;
+            int csplit = 1;
+            if (tiles < (size_t)ctx->num_cus && nblocks >= 2) {
+               int want = (int)cdiv(2 * ctx->num_cus, (int)tiles);   // more slices measured slower (one 56x56 image: 22.8 against 19.3 us)
+               if (want > 8) want = 8;
+               if (want > nblocks) want = nblocks;
+               while (want > 1 && (size_t)want * g.N * g.OC * OHW * 4 > ((size_t)32 << 20)) --want;   // partial sums of at most 32 MB
+               csplit = cdiv(nblocks, cdiv(nblocks, want));
+            }
+            const size_t out_floats = (size_t)g.N * g.OC * OHW;
+            const size_t wbytes = (wt_floats * sizeof(float) + 255) & ~(size_t)255;
+            const size_t pbytes = csplit > 1 ? (size_t)csplit * out_floats * sizeof(float) : 0;
+            void *ws = nullptr, *ps = nullptr;
             bool fresh = true;
             const int layout[] = {1, g.groups, g.ocg, g.icg, g.KH, g.KW, wstride, pairs ? 1 : 0};
             if (int rc = packed_weights(ctx, g.w, layout_key(layout, 8), wt_floats * sizeof(float), &ws, &fresh)) return rc;
+            if (pbytes) {
+               if (fresh && ws == ctx->workspace) {
+                  // the copy of the weights sits in the context's scratch buffer: the partial sums go behind it
+                  if (int rc = workspace(ctx, wbytes + pbytes, &ws)) return rc;
+                  ps = static_cast<unsigned char *>(ws) + wbytes;
+               } else if (int rc = workspace(ctx, pbytes, &ps)) return rc;
+            }
             if (fresh) {
                hipLaunchKernelGGL(k_transpose_weights, dim3((unsigned)((wt_floats + 255) / 256)), dim3(256), 0, ctx->stream, g.w,
                                   static_cast<float *>(ws), g.groups, g.ocg, g.icg * KHW, wstride, pairs ? 1 : 0, KHW);
@@ -663,6 +721,8 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             }
             ConvArgs h = g;
             h.w = static_cast<const float *>(ws);
+            h.csplit = csplit;
+            h.partial = static_cast<float *>(ps);
             constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, false, 0>, kern1 = k_conv2d_f32_dma<TI, TJ, false, 1>,
                            kern2 = k_conv2d_f32_dma<TI, TJ, false, 2>, kern3 = k_conv2d_f32_dma<TI, TJ, false, 3>;
             SOFIE_LARGE_LDS(kern0);
@@ -670,10 +730,14 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             SOFIE_LARGE_LDS(kern2);
             SOFIE_LARGE_LDS(kern3);
             const auto kern = !pairs ? kern0 : kwt == 1 ? kern1 : kwt == 2 ? kern2 : kern3;
-            hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N), dim3(256),
+            hipLaunchKernelGGL(kern, dim3(cdiv(OHW, BP), g.groups * octiles, g.N * csplit), dim3(256),
                                dma_lds_bytes(g.KC, (size_t)icb * g.PH * g.PW, BOC), ctx->stream, h);
             *done = true;
-            return check_launch(ctx, pairs ? "k_conv2d_f32_dma_pairs" : "k_conv2d_f32_dma");
+            if (int rc = check_launch(ctx, pairs ? "k_conv2d_f32_dma_pairs" : "k_conv2d_f32_dma")) return rc;
+            if (csplit == 1) return SOFIE_HIP_OK;
+            hipLaunchKernelGGL(k_conv_f32_split_finish, dim3((unsigned)((out_floats + 255) / 256)), dim3(256), 0, ctx->stream,
+                               h.partial, g.y, g.bias, csplit, out_floats, OHW, g.OC, g.relu);
+            return check_launch(ctx, "k_conv_f32_split_finish");
          }
       }
    }
@@ -852,8 +916,14 @@ int run_conv(sofie_hip_ctx *ctx, ConvArgs &g)
    g.dOW = make_fastdiv((unsigned)g.OW);
    bool done = false;
    int rc;
-   if (g.ocg > 64) rc = launch<2, 2>(ctx, g, &done);
-   else rc = launch<1, 2>(ctx, g, &done);
+   // 128 channels x 128 pixels per workgroup where that gives every compute unit a tile, else 64 x 128, else 64 x 64: a
+   // layer on one image or a few has too few of the large tiles to fill the device (one 56x56 image, 64 -> 128
+   // channels: 25 tiles of 128 x 128, 98 of 64 x 64)
+   const size_t pixels = (size_t)g.OH * g.OW;
+   auto tiles = [&](int boc, int bp) { return (size_t)cdiv((int)pixels, bp) * g.groups * cdiv(g.ocg, boc) * g.N; };
+   if (g.ocg > 64 && tiles(128, 128) >= (size_t)ctx->num_cus) rc = launch<2, 2>(ctx, g, &done);
+   else if (tiles(64, 128) >= (size_t)ctx->num_cus) rc = launch<1, 2>(ctx, g, &done);
+   else rc = launch<1, 1>(ctx, g, &done);
    if (rc || done) return rc;
    const size_t total = (size_t)g.N * g.OC * g.OH * g.OW;
    hipLaunchKernelGGL(k_conv2d_f32_simple, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, ctx->stream, g);

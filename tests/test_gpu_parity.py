@@ -348,10 +348,33 @@ def test_conv2d_f32_operands_by_lds_dma(ops, cfg):
     b = (r.standard_normal(cfg["OC"]) * 0.1).astype(np.float32)
     for bias, relu in ((b, True), (None, False)):
         y, names = _kernels_of(ops, lambda: ops.conv2d_f32(x, w, bias, cfg["p"], cfg["s"], cfg["d"], cfg["g"], relu))
-        assert names == ["k_transpose_weights", "k_conv2d_f32_dma_pairs" if cfg["pairs"] else "k_conv2d_f32_dma"], names
+        # (a layer of fewer tiles than compute units is cut into slices of channel blocks, which a second pass adds)
+        assert names[:2] == ["k_transpose_weights", "k_conv2d_f32_dma_pairs" if cfg["pairs"] else "k_conv2d_f32_dma"], names
+        assert names[2:] in ([], ["k_conv_f32_split_finish"]), names
         ref = oracle.conv2d_f32(x, w, bias, cfg["p"], cfg["s"], cfg["d"], cfg["g"], relu)
         assert y.shape == ref.shape
         assert rel_err(y, ref) <= FP32_TOL
+
+
+@pytest.mark.parametrize("N,C,H,W,OC,k,g", [(1, 64, 56, 56, 128, 3, 1), (2, 48, 20, 30, 70, 3, 1), (1, 64, 28, 28, 64, 1, 1),
+                                            (3, 32, 14, 14, 96, 3, 2), (1, 128, 9, 9, 40, 2, 1)])
+def test_conv2d_f32_on_few_images_sums_channel_slices(ops, N, C, H, W, OC, k, g):
+    """A layer with fewer tiles than the device has compute units runs on 64 x 64 tiles with its channel blocks dealt
+    to slices (k_conv2d_f32_dma writes raw sums, k_conv_f32_split_finish adds them in slice order, then bias and
+    ReLU): the trace shows the second pass, the results are the oracle's within 1e-5 relative, and a second call
+    gives the same bits (the order of the sums is fixed)."""
+    r = rng(260 + C + OC + k)
+    x = r.standard_normal((N, C, H, W)).astype(np.float32)
+    w = (r.standard_normal((OC, C // g, k, k)) * np.sqrt(2.0 / (C // g * k * k))).astype(np.float32)
+    b = (r.standard_normal(OC) * 0.1).astype(np.float32)
+    pads = (k // 2, k // 2)
+    for bias, relu in ((b, True), (None, False)):
+        y, names = _kernels_of(ops, lambda: ops.conv2d_f32(x, w, bias, pads, (1, 1), (1, 1), g, relu))
+        assert names[-1] == "k_conv_f32_split_finish" and names[-2].startswith("k_conv2d_f32_dma"), names
+        ref = oracle.conv2d_f32(x, w, bias, pads, (1, 1), (1, 1), g, relu)
+        assert y.shape == ref.shape
+        assert rel_err(y, ref) <= FP32_TOL
+        assert np.array_equal(y, ops.conv2d_f32(x, w, bias, pads, (1, 1), (1, 1), g, relu))
 
 
 def test_conv_transpose2d_f32_phases_by_lds_dma(ops):
