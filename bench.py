@@ -243,7 +243,7 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     ap.add_argument("--kernel-probe", default="",
                     help="launch one named workload a few times and exit (target of rocprofv3 runs): gemm_s8, gemm_s8_nk, "
-                         "gemm_fp8, gemm_fp8_nk, gemm_f32, gemm_f32_nk, gemm_f32_batch8, conv_s8, conv_f32, conv_transpose_f32")
+                         "gemm_fp8, gemm_fp8_nk, gemm_f32, gemm_f32_nk, gemm_f32_batch8, gemm_s8_batch8, conv_s8, conv_f32, conv_transpose_f32")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collective, no sharding "
@@ -441,6 +441,7 @@ def main():
     out["gemm_f32"] = res["gemm_f32"]
     out["gemm_f32_b_nk"] = res["gemm_f32_nk"]
     out["gemm_f32_batch8"] = res["gemm_f32_batch8"]
+    out["int8_gemm_batch8"] = res["gemm_s8_batch8"]
     out["conv_f32"] = res["conv_f32"]
     out["conv_s8"] = res["conv_s8"]
     out["conv_transpose_f32"] = res["conv_transpose_f32"]
@@ -501,6 +502,17 @@ def workloads(ctx, torch, L, rng):
                      "memory-bound: gbs = algorithmic bytes (B, A, Y, bias once) per second, frac_hbm_peak against 8 TB/s",
          "ops": 2.0 * 8 * n * n, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 200,
          "bytes": 4.0 * (n * n + 8 * n + 8 * n + n), "bound": "hbm"})
+    # the int8 layer of the headline on a batch of 8 rows, weights [N,K] as a Session keeps them: a pass over 16 MB of B
+    A8r = torch.randint(-127, 128, (8, n), dtype=torch.int8, device=ctx.device)
+    B8r = torch.randint(-127, 128, (n, n), dtype=torch.int8, device=ctx.device)
+    s8r = torch.full((n,), 2e-4, device=ctx.device)
+    Y8r = ctx.empty((8, n), torch.int8)
+    w["gemm_s8_batch8"] = ((lambda: ctx.check(ctx.lib.sofie_hip_qgemm_s8(
+        ctx.h, 1, 8, n, n, ctx.ptr(A8r), n, ctx.ptr(B8r), n, ctx.ptr(s8r), None, 0, L.ACT_NONE, ctx.ptr(Y8r), n, L.OUT_S8))),
+        {"workload": "int8 GEMM 8 x 4096 x 4096 (QLinearMatMul of a 4096 -> 4096 layer on a batch of 8), B [N,K], requantised to "
+                     "int8; memory-bound: gbs = algorithmic bytes (B, A, Y, scales once) per second, frac_hbm_peak against 8 TB/s",
+         "ops": 2.0 * 8 * n * n, "rate_unit": "tops", "peak": PEAK_INT8_TOPS, "launches": 200,
+         "bytes": 1.0 * (n * n + 8 * n + 8 * n) + 4.0 * n, "bound": "hbm"})
     # fp32 conv layer: batch 256, 64 -> 128 channels, 56x56, 3x3, pad 1, bias + ReLU
     x = torch.rand(256, 64, 56, 56, device=ctx.device)
     wt = torch.randn(128, 64, 3, 3, device=ctx.device) * (2.0 / 576) ** 0.5

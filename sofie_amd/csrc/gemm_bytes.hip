@@ -1177,6 +1177,134 @@ int launch_dma(sofie_hip_ctx *ctx, GemmArgs &g)
    return check_launch(ctx, "k_gemm_dma");
 }
 
+// Few rows of A (M <= 32: a quantised layer on a small batch) with B [N][K]: the product is a pass over B, bound by
+// memory, and 64 x 64 tiles would give a handful of compute units all the work. A wavefront owns all rows of A (MT
+// tiles of 16 rows, v_mfma_i32_16x16x64_i8) and 64 columns; B goes from global memory straight into the matrix
+// instruction's operand registers: lane (j = lane % 16, kq = lane / 16) loads bytes k0 + 16 kq .. + 15 of column 16 q + j,
+// which is its part of the operand of tile q as it stands, and the same bytes of its row of A. The grid is column
+// blocks x slices of K; a wavefront takes a quarter of the slice in chunks of 64 k (consecutive chunks: the two halves
+// of a 128-byte line are fetched one behind the other), three chunks of loads in flight while one is multiplied; the
+// four wavefronts' sums meet in LDS and go to the scratch buffer [slice][M][ldp] that k_splitk_finish adds up and
+// converts (integer sums: the result is that of the unsplit kernels bit for bit).
+template <int MT>
+__global__ void __launch_bounds__(256) k_qgemm_few_rows(GemmArgs g, int *partial, int ldp, int kslice)
+{
+   constexpr unsigned OUTSIDE = 0x80000000u;
+   __shared__ int red[2 * MT * 4 * 4 * 64];
+   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+   const int j = lane & 15, kq = lane >> 4;
+   const int c0 = blockIdx.x * 64;
+   const int k_begin = blockIdx.y * kslice + wave * (kslice >> 2);
+   int k_end = k_begin + (kslice >> 2);
+   if (k_end > g.K) k_end = g.K;
+   const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t *>(g.A), 0, (int)((size_t)(g.M - 1) * g.lda + g.K), 0x00020000);
+   const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t *>(g.B), 0, (int)((size_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
+   unsigned a_off[MT], b_off[4];
+#pragma unroll
+   for (int t = 0; t < MT; ++t) a_off[t] = t * 16 + j < g.M ? (unsigned)((t * 16 + j) * g.lda + 16 * kq) : OUTSIDE;
+#pragma unroll
+   for (int q = 0; q < 4; ++q) b_off[q] = c0 + 16 * q + j < g.N ? (unsigned)((c0 + 16 * q + j) * g.ldb + 16 * kq) : OUTSIDE;
+   struct Chunk {
+      v4i a[MT], b[4];
+   };
+   auto load = [&](Chunk &c, int k0) {
+      const bool in = k0 + 16 * kq < k_end;     // K and the wavefronts' shares are multiples of 16: a lane's bytes are in or out together
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+         c.a[t] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ars, in ? a_off[t] : OUTSIDE, k0, 0));
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+         c.b[q] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(brs, in ? b_off[q] : OUTSIDE, k0, 0));
+   };
+   v4i acc[MT][4];
+#pragma unroll
+   for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) acc[t][q] = v4i{0, 0, 0, 0};
+   Chunk c0_, c1_, c2_, c3_;
+   int k0 = k_begin;
+   load(c0_, k0);
+   load(c1_, k0 + 64);
+   load(c2_, k0 + 128);
+   for (; k0 < k_end; k0 += 64) {
+      load(c3_, k0 + 192);
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+#pragma unroll
+         for (int t = 0; t < MT; ++t) acc[t][q] = __builtin_amdgcn_mfma_i32_16x16x64_i8(c0_.a[t], c0_.b[q], acc[t][q], 0, 0, 0);
+      c0_ = c1_;
+      c1_ = c2_;
+      c2_ = c3_;
+   }
+   // wavefronts 2 and 3 hand their sums to 0 and 1, then 1 hands its to 0
+   auto put = [&](int *dst) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+         for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) dst[((t * 4 + q) * 4 + r) * 64 + lane] = acc[t][q][r];
+   };
+   auto add = [&](const int *src) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+         for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[t][q][r] += src[((t * 4 + q) * 4 + r) * 64 + lane];
+   };
+   constexpr int BLOCK = MT * 4 * 4 * 64;
+   if (wave >= 2) put(red + (wave - 2) * BLOCK);
+   __syncthreads();
+   if (wave < 2) add(red + wave * BLOCK);
+   __syncthreads();
+   if (wave == 1) put(red);
+   __syncthreads();
+   if (wave != 0) return;
+   add(red);
+   // tile (t, q), register r: row t * 16 + kq * 4 + r, column c0 + 16 q + j
+   int *const out = partial + (size_t)blockIdx.y * g.M * ldp;
+#pragma unroll
+   for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+         const int m = t * 16 + kq * 4 + r;
+         if (m >= g.M) continue;
+#pragma unroll
+         for (int q = 0; q < 4; ++q) {
+            const int n = c0 + 16 * q + j;
+            if (n < ldp) out[(size_t)m * ldp + n] = acc[t][q][r];
+         }
+      }
+}
+
+// Slices of K so that about eight workgroups per compute unit exist, every wavefront with at least two chunks, and the
+// partial sums a fraction of B's bytes.
+template <int OUT>
+int launch_few_rows(sofie_hip_ctx *ctx, GemmArgs &g)
+{
+   const int blocks = cdiv(g.N, 64);
+   int splits = 8 * ctx->num_cus / blocks;
+   if (splits > g.K / 512) splits = g.K / 512;
+   if (splits > g.K / (16 * g.M)) splits = g.K / (16 * g.M);
+   if (splits < 1) splits = 1;
+   const int kslice = cdiv(cdiv(g.K, splits), 256) * 256;
+   splits = cdiv(g.K, kslice);
+   const int ldp = cdiv(g.N, 4) * 4;
+   void *part = nullptr;
+   if (int rc = workspace(ctx, (size_t)splits * g.M * ldp * sizeof(int), &part)) return rc;
+   const dim3 grid(blocks, splits);
+   if (g.M <= 16) hipLaunchKernelGGL(k_qgemm_few_rows<1>, grid, dim3(256), 0, ctx->stream, g, static_cast<int *>(part), ldp, kslice);
+   else hipLaunchKernelGGL(k_qgemm_few_rows<2>, grid, dim3(256), 0, ctx->stream, g, static_cast<int *>(part), ldp, kslice);
+   if (int rc = check_launch(ctx, "k_qgemm_few_rows")) return rc;
+   const size_t threads = (size_t)g.M * (ldp / 4);
+   hipLaunchKernelGGL((k_splitk_finish<OUT>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, ctx->stream, g,
+                      static_cast<const int *>(part), splits, ldp);
+   return check_launch(ctx, "k_splitk_finish");
+}
+
 // K cut into `splits` slices of `kslice` bytes (a multiple of BK): partial sums into the context's scratch
 // buffer, then k_splitk_finish writes Y.
 template <class Mma, int BK, int NSETS, int OUT>
@@ -1263,6 +1391,13 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
          return launch_skinny<OUT>(ctx, g);
    }
    if (!a_ok || !(b_nk_ok || b_kn_ok)) return launch_simple<IS_INT, OUT>(ctx, g, transB);
+   if constexpr (IS_INT && OUT != SOFIE_OUT_BF16) {
+      // a small batch on a layer of 2 MB or more: a pass over B with K in slices (8 x 4096 x 4096: 9.1 against 15.1 us; a
+      // layer of 1 MB is faster on tiles in one launch: 6.0 against 7.2 us)
+      if (transB && g.M <= 32 && g.N >= 64 && g.K >= 512 && (size_t)g.N * g.K >= ((size_t)2 << 20) &&
+          (size_t)g.M * g.lda + g.K < (1u << 31) && (size_t)g.N * g.ldb + g.K < (1u << 31))
+         return launch_few_rows<OUT>(ctx, g);
+   }
    const bool big = (size_t)g.M * g.N >= (size_t)256 * 256 * 128 && g.M >= 256 && g.N >= 256;
    // 128 bytes of K per stage; int8 keeps two register sets in flight, fp8 (twice the
    // fragment registers) one.
@@ -1315,6 +1450,9 @@ int dispatch(sofie_hip_ctx *ctx, GemmArgs &g, int transB)
          if (int rc = transpose_bytes(ctx, g.B, static_cast<unsigned char *>(bt), g.K, g.N, g.ldb, g.K)) return rc;
       g.B = static_cast<const uint8_t *>(bt);
       g.ldb = g.K;
+      // a copy of its own (constant weights): every choice of the [N,K] case is open; a copy in the scratch buffer
+      // leaves the kernels that need no scratch memory themselves
+      if (bt != ctx->workspace && bt != ctx->static_scratch) return dispatch<Mma, OUT>(ctx, g, 1);
       if (cdiv(g.M, 128) * cdiv(g.N, 128) * 2 <= ctx->num_cus && g.K >= 1024)
          return launch_tiled<Mma, BK, NSETS, 1, 1, OUT, false>(ctx, g);
       return launch_tiled<Mma, BK, NSETS, 2, 2, OUT, false>(ctx, g);

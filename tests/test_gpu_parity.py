@@ -544,6 +544,9 @@ QGEMM_SHAPES = [
     (70, 13, 1040, True), (5, 1, 32, True), (300, 9, 48, True),
     (512, 256, 12800, True),                             # long K, few tiles: K cut into slices
     (300, 130, 8464, True), (129, 40, 8208, True),       # ... with ragged tiles and a last slice that is shorter
+    (1, 1024, 1024, True), (8, 4096, 2048, True),        # a small batch on a layer of some size: a pass over B [N,K] with K
+    (16, 1000, 1040, True), (17, 66, 4096, True),        # in slices (k_qgemm_few_rows): ragged columns, K no multiple of a
+    (32, 2050, 528, True), (31, 640, 8208, True),        # chunk of 64 or of a slice, one and two row tiles
 ]
 
 
@@ -575,6 +578,48 @@ def test_qgemm_s8_accumulators_and_requant(ops, M, N, K, transB):
         for i in range(flat.size):
             flat[i] = oracle.requant_one(int(az[i]), sc[i], -3, False)
         assert np.array_equal(yz, want)
+
+
+def test_qgemm_s8_few_rows_kernels_and_constant_weights(ops):
+    """Which kernels a quantised layer on a small batch runs on: B [N,K] takes the pass over B with K in slices; B [K,N]
+    is transposed into the scratch buffer first and then runs on tiles, and with the constant-weights promise the
+    transposed copy is made once and the small batch takes the pass over it. Bit-exact against the oracle each time."""
+    r = rng(612)
+    M, N, K = 8, 1536, 2048
+    A = r.integers(-127, 128, (M, K)).astype(np.int8)
+    Bnk = r.integers(-127, 128, (N, K)).astype(np.int8)
+    Bkn = np.ascontiguousarray(Bnk.T)
+    scale = (r.uniform(20.0, 60.0, N) / (73.3 * 73.3 * np.sqrt(K))).astype(np.float32)
+    bias = r.integers(-2000, 2000, N).astype(np.int32)
+    ref = oracle.qgemm_s8(A, Bnk, scale, bias, True, zpy=-128, relu=True)
+    y, names = _kernels_of(ops, lambda: ops.qgemm_s8(A, Bnk, scale, bias, True, zpy=-128, relu=True))
+    assert names == ["k_qgemm_few_rows", "k_splitk_finish"], names
+    assert np.array_equal(y, ref)
+    y, names = _kernels_of(ops, lambda: ops.qgemm_s8(A, Bkn, scale, bias, False, zpy=-128, relu=True))
+    assert names == ["k_transpose_bytes", "k_gemm_bytes"], names
+    assert np.array_equal(y, ref)
+    ctx = ops.Context(0)
+    try:
+        assert ctx.lib.sofie_hip_constant_weights(ctx.h, 1) == 0
+        a, b = ctx.dev(A, torch.int8), ctx.dev(Bkn, torch.int8)
+        sd, bd = ctx.dev(scale, torch.float32), ctx.dev(bias, torch.int32)
+        out = ctx.empty((M, N), torch.int8)
+        from sofie_amd import lib as L
+        import ctypes as C
+        seen = []
+        for _ in range(2):
+            buf = C.create_string_buffer(4096)
+            n = C.c_int(-1)
+            assert ctx.lib.sofie_hip_trace_begin(ctx.h) == 0
+            ctx.check(ctx.lib.sofie_hip_qgemm_s8(ctx.h, 0, M, N, K, ctx.ptr(a), K, ctx.ptr(b), N, ctx.ptr(sd), ctx.ptr(bd), -128,
+                                                 L.ACT_RELU, ctx.ptr(out), N, L.OUT_S8))
+            assert ctx.lib.sofie_hip_trace_end(ctx.h, buf, 4096, C.byref(n)) == 0
+            seen.append([l.split()[0] for l in buf.value.decode().splitlines()])
+            ctx.sync()
+            assert np.array_equal(out.cpu().numpy(), ref)
+        assert seen == [["k_transpose_bytes", "k_qgemm_few_rows", "k_splitk_finish"], ["k_qgemm_few_rows", "k_splitk_finish"]], seen
+    finally:
+        ctx.close()
 
 
 def test_qgemm_s8_baseline_scales_saturate_identically(ops):
