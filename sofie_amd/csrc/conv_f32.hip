@@ -53,8 +53,8 @@ struct ConvArgs {
    int wvec;           // weights are staged with 16-byte loads (see launch)
    FastDiv dPW, dPH, dKC, dK4;   // divisions by the patch extents and the K-chunk length (/4) in the staging loops
    FastDiv dUH, dUW, dOW;
-   // csplit > 1 (k_conv2d_f32_dma without phases): blockIdx.z = image * csplit + slice; a slice sums its share of the
-   // channel blocks into partial [slice][N][OC][OH*OW] without bias and ReLU, k_conv_f32_split_finish adds the slices
+   // csplit > 1 (k_conv2d_f32_dma): blockIdx.z = (image [* phases + phase]) * csplit + slice; a slice sums its share of
+   // the channel blocks into partial [slice][N][OC][output plane] without bias and ReLU, k_conv_f32_split_finish adds the slices
    int csplit;
    float *partial;
    // nphases > 1: blockIdx.z = image * nphases + phase, and the phase's geometry replaces the fields above
@@ -309,21 +309,15 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    int oy0 = 0, ox0 = 0;
    int c_begin = 0, c_end = g.icg / g.ICB;
    FastDiv dOW = gg.dOW;
-   if constexpr (!PHASES) {
-      if (gg.csplit > 1) {
-         // a slice of the channel blocks: raw sums into its plane of the scratch buffer
-         const int slice = bz % gg.csplit, per = (c_end + gg.csplit - 1) / gg.csplit;
-         n = bz / gg.csplit;
-         c_begin = slice * per;
-         c_end = c_end < c_begin + per ? c_end : c_begin + per;
-         g.y = gg.partial + (size_t)slice * gg.N * g.OC * g.OH * g.OW;
-         g.bias = nullptr;
-         g.relu = 0;
-      }
+   int slice = 0;
+   if (gg.csplit > 1) {
+      // blockIdx.z = (image [* phases + phase]) * slices + slice
+      slice = bz % gg.csplit;
+      n = bz / gg.csplit;
    }
    if constexpr (PHASES) {
-      const int pi = bz % gg.nphases;
-      n = bz / gg.nphases;
+      const int pi = n % gg.nphases;
+      n = n / gg.nphases;
       PhaseArgs q = gg.phase[0];
 #pragma unroll
       for (int i = 1; i < SOFIE_CONV_MAX_PHASES; ++i)
@@ -334,6 +328,15 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
       g.w = gg.w + q.woff;
       oy0 = q.oy0; ox0 = q.ox0; dOW = q.dOW;
       c_end = g.icg / g.ICB;
+   }
+   if (gg.csplit > 1) {
+      // a slice of the channel blocks (possibly none of them): raw sums into its copy of the output in the scratch buffer
+      const int per = (c_end + gg.csplit - 1) / gg.csplit;
+      c_begin = slice * per;
+      c_end = c_end < c_begin + per ? c_end : c_begin + per;
+      g.y = gg.partial + (size_t)slice * gg.N * g.OC * (PHASES ? gg.OH0 * gg.OW0 : g.OH * g.OW);
+      g.bias = nullptr;
+      g.relu = 0;
    }
    extern __shared__ __align__(16) unsigned char smem_raw[];
    const int patch_len = g.ICB * g.PH * g.PW;
@@ -415,7 +418,7 @@ __global__ void __launch_bounds__(256, TI == 1 ? 7 : 3) k_conv2d_f32_dma(ConvArg
    };
 
    const int nsteps = p0 + wn * TJ * 32 < OHW ? g.KC / 2 : 0;   // a wavefront with no pixel of the plane multiplies nothing
-   request(c_begin, 0);
+   if (c_begin < c_end) request(c_begin, 0);
    wait_vmcnt<0>();
    __syncthreads();   // the first block and the koff table are in LDS
    for (int c = c_begin; c < c_end; ++c) {
@@ -688,12 +691,12 @@ int launch(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             g.KC = icb * KHW;
             g.dPW = make_fastdiv((unsigned)g.PW);
             g.dPH = make_fastdiv((unsigned)g.PH);
-            // Fewer tiles than compute units (a layer on one image or a few): the channel blocks are dealt to up to 8
+            // Tiles for at most two thirds of the compute units (a layer on one image or a few): the channel blocks are dealt to up to 8
             // slices, each a workgroup of its own that writes raw sums, and a second pass adds them (a fixed order)
             const size_t tiles = (size_t)cdiv(OHW, BP) * g.groups * octiles * g.N;
             const int nblocks = g.icg / icb;
             int csplit = 1;
-            if (tiles < (size_t)ctx->num_cus && nblocks >= 2) {
+            if (tiles * 3 <= (size_t)ctx->num_cus * 2 && nblocks >= 2) {   // nearer to one tile per compute unit the second pass costs what the slices gain
                int want = (int)cdiv(2 * ctx->num_cus, (int)tiles);   // more slices measured slower (one 56x56 image: 22.8 against 19.3 us)
                if (want > 8) want = 8;
                if (want > nblocks) want = nblocks;
@@ -845,6 +848,26 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
             for (int e = 0; e < 6; ++e) layout[12 + 6 * i + e] = v[e];
          }
          if (int rc = packed_weights(ctx, g.w, layout_key(layout, 12 + 6 * g.nphases), (size_t)woff * sizeof(float), &ws, &fresh)) return rc;
+         // fewer tiles than compute units: slices of the channel blocks as in the plain convolution
+         int csplit = 1, min_blocks = g.icg;
+         for (int i = 0; i < g.nphases; ++i)
+            if (g.icg / g.phase[i].ICB < min_blocks) min_blocks = g.icg / g.phase[i].ICB;
+         const size_t out_floats = (size_t)g.N * g.OC * g.OH0 * g.OW0;
+         if (workgroups * 3 <= (size_t)ctx->num_cus * 2 && min_blocks >= 2 && (size_t)g.N * g.nphases * 8 <= 65535) {
+            int want = (int)cdiv(2 * ctx->num_cus, (int)workgroups);
+            if (want > 8) want = 8;
+            if (want > min_blocks) want = min_blocks;
+            while (want > 1 && (size_t)want * out_floats * 4 > ((size_t)32 << 20)) --want;
+            csplit = want;
+         }
+         void *ps = nullptr;
+         if (csplit > 1) {
+            const size_t wbytes = ((size_t)woff * sizeof(float) + 255) & ~(size_t)255, pbytes = (size_t)csplit * out_floats * sizeof(float);
+            if (fresh && ws == ctx->workspace) {
+               if (int rc = workspace(ctx, wbytes + pbytes, &ws)) return rc;
+               ps = static_cast<unsigned char *>(ws) + wbytes;
+            } else if (int rc = workspace(ctx, pbytes, &ps)) return rc;
+         }
          if (fresh) {
             hipLaunchKernelGGL(k_gather_phase_weights, dim3((unsigned)cdiv(woff, 256)), dim3(256), 0, ctx->stream, g,
                                static_cast<float *>(ws), woff, wstride, pairs ? 1 : 0);
@@ -852,6 +875,8 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          }
          ConvArgs h = g;
          h.w = static_cast<const float *>(ws);
+         h.csplit = csplit;
+         h.partial = static_cast<float *>(ps);
          constexpr auto kern0 = k_conv2d_f32_dma<TI, TJ, true, 0>, kern1 = k_conv2d_f32_dma<TI, TJ, true, 1>,
                         kern2 = k_conv2d_f32_dma<TI, TJ, true, 2>, kern3 = k_conv2d_f32_dma<TI, TJ, true, 3>;
          SOFIE_LARGE_LDS(kern0);
@@ -859,9 +884,13 @@ int launch_phases(sofie_hip_ctx *ctx, ConvArgs &g, bool *done)
          SOFIE_LARGE_LDS(kern2);
          SOFIE_LARGE_LDS(kern3);
          const auto kern = !pairs ? kern0 : kwt == 1 ? kern1 : kwt == 2 ? kern2 : kern3;
-         hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases), dim3(256), lds_max, ctx->stream, h);
+         hipLaunchKernelGGL(kern, dim3(tiles_max, g.groups * octiles, g.N * g.nphases * csplit), dim3(256), lds_max, ctx->stream, h);
          *done = true;
-         return check_launch(ctx, pairs ? "k_conv2d_f32_dma_pairs_phases" : "k_conv2d_f32_dma_phases");
+         if (int rc = check_launch(ctx, pairs ? "k_conv2d_f32_dma_pairs_phases" : "k_conv2d_f32_dma_phases")) return rc;
+         if (csplit == 1) return SOFIE_HIP_OK;
+         hipLaunchKernelGGL(k_conv_f32_split_finish, dim3((unsigned)((out_floats + 255) / 256)), dim3(256), 0, ctx->stream,
+                            h.partial, g.y, g.bias, csplit, out_floats, g.OH0 * g.OW0, g.OC, g.relu);
+         return check_launch(ctx, "k_conv_f32_split_finish");
       }
       lds_max = 0;
       tiles_max = 0;
@@ -1110,7 +1139,16 @@ extern "C" int sofie_hip_conv_transpose2d_f32(sofie_hip_ctx *ctx, const float *x
       if (ok && all.nphases > 1) {
          all.dUH = make_fastdiv(1u); all.dUW = make_fastdiv(1u); all.dOW = make_fastdiv(1u);
          bool done = false;
-         const int rc = all.ocg > 64 ? launch_phases<2, 2>(ctx, all, &done) : launch_phases<1, 2>(ctx, all, &done);
+         // tiles as for the plain convolution: the largest that still give every compute unit one
+         auto tiles = [&](int boc, int bp) {
+            size_t t = 0;
+            for (int i = 0; i < all.nphases; ++i) t += (size_t)cdiv(all.phase[i].OH * all.phase[i].OW, bp);
+            return t * all.groups * cdiv(all.ocg, boc) * all.N;
+         };
+         int rc;
+         if (all.ocg > 64 && tiles(128, 128) >= (size_t)ctx->num_cus) rc = launch_phases<2, 2>(ctx, all, &done);
+         else if (tiles(64, 128) >= (size_t)ctx->num_cus) rc = launch_phases<1, 2>(ctx, all, &done);
+         else rc = launch_phases<1, 1>(ctx, all, &done);
          if (rc || done) return rc;
       }
    }

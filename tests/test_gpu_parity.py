@@ -388,7 +388,9 @@ def test_conv_transpose2d_f32_phases_by_lds_dma(ops):
         w = (r.standard_normal((C, OC, k, k)) * 0.2).astype(np.float32)
         b = r.standard_normal(OC).astype(np.float32)
         y, names = _kernels_of(ops, lambda: ops.conv_transpose2d_f32(x, w, b, (1, 1, 1, 1), (2, 2), (1, 1), 1, op, True))
-        assert names == ["k_gather_phase_weights", kern], names
+        # (the small layers have fewer tiles than the device has compute units: their channel blocks are cut into
+        # slices that a second pass adds)
+        assert names[:2] == ["k_gather_phase_weights", kern] and names[2:] in ([], ["k_conv_f32_split_finish"]), names
         ref = oracle.conv_transpose2d_f32(x, w, b, (1, 1, 1, 1), (2, 2), (1, 1), 1, op, True)
         assert rel_err(y, ref) <= FP32_TOL
 
@@ -416,7 +418,8 @@ def test_constant_weights_keep_the_kernels_layout_of_a_weight_tensor(ops):
         assert ctx.lib.sofie_hip_trace_begin(ctx.h) == 0
         out = call()
         assert ctx.lib.sofie_hip_trace_end(ctx.h, buf, 4096, C.byref(n)) == 0
-        return out, [l.split()[0] for l in buf.value.decode().splitlines()]
+        # (layers this small are cut into slices of channel blocks; the pass that adds them is not what this test is about)
+        return out, [l.split()[0] for l in buf.value.decode().splitlines() if l.split()[0] != "k_conv_f32_split_finish"]
 
     conv = lambda pads=(1, 1): ops.conv2d_f32(dx, dw, db, pads, (1, 1), (1, 1), 1, True, ctx=ctx)
     convt = lambda: ops.conv_transpose2d_f32(dxt, dwt, None, (1, 1, 1, 1), (2, 2), (1, 1), 1, (0, 0), False, ctx=ctx)
