@@ -243,7 +243,7 @@ def main():
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     ap.add_argument("--kernel-probe", default="",
                     help="launch one named workload a few times and exit (target of rocprofv3 runs): gemm_s8, gemm_s8_nk, "
-                         "gemm_fp8, gemm_fp8_nk, gemm_f32, gemm_f32_nk, gemm_f32_batch8, gemm_s8_batch8, conv_s8, conv_f32, conv_transpose_f32")
+                         "gemm_fp8, gemm_fp8_nk, gemm_f32, gemm_f32_nk, gemm_f32_batch8, gemm_s8_batch8, conv_s8, conv_f32, conv_f32_batch1, conv_transpose_f32")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collective, no sharding "
@@ -443,6 +443,7 @@ def main():
     out["gemm_f32_batch8"] = res["gemm_f32_batch8"]
     out["int8_gemm_batch8"] = res["gemm_s8_batch8"]
     out["conv_f32"] = res["conv_f32"]
+    out["conv_f32_batch1"] = res["conv_f32_batch1"]
     out["conv_s8"] = res["conv_s8"]
     out["conv_transpose_f32"] = res["conv_transpose_f32"]
     out["mlp_f32"] = mlp_session_rate()
@@ -524,6 +525,12 @@ def workloads(ctx, torch, L, rng):
         {"workload": "fp32 Conv2d NCHW batch 256, 64 -> 128 channels, 56x56, 3x3, stride 1, pad 1, bias + ReLU fused; weights promised constant (laid out once, as in a Session)",
          "ops": fl, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 20,
          "bytes": 4.0 * (x.numel() + y.numel() + wt.numel() + 128)})
+    # the same layer on one image: 25 tiles of 128 x 128 would leave nine compute units in ten idle
+    w["conv_f32_batch1"] = (lambda: ctx.check(ctx.lib.sofie_hip_conv2d_f32(
+        ctx.h, ctx.ptr(x), ctx.ptr(wt), ctx.ptr(b), ctx.ptr(y), 1, 64, 56, 56, 128, 3, 3, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1)),
+        {"workload": "fp32 Conv2d NCHW, one image, 64 -> 128 channels, 56x56, 3x3, stride 1, pad 1, bias + ReLU fused (64 x 64 "
+                     "tiles, channel blocks in slices added by a second pass: two launches); weights promised constant",
+         "ops": fl / 256, "rate_unit": "tflops", "peak": PEAK_FP32_TFLOPS, "launches": 200})
     # int8 conv layer of the same shape, channels-last, weights [OC][KH][KW][C], bias + ReLU + requantise fused
     # activations uniform [0,1] quantised with scale 1/255 (zero-point -128); weights Kaiming-normal, symmetric int8 per
     # output channel; the output scale puts the layer's range (about 0..4) on the 8 bits
