@@ -229,6 +229,27 @@ def test_gemm_f32_few_rows(ops, M, N, K, tB):
         assert rel_err(y, oracle.gemm_f32(A, B, bias, alpha, beta, False, bool(tB), relu)) <= FP32_TOL
 
 
+@pytest.mark.parametrize("M,N,K,tB", [(128, 1024, 4096, 0), (200, 520, 2048, 1), (96, 2048, 1024, 0), (512, 260, 8192, 1)])
+def test_gemm_f32_few_tiles_long_k_in_slices(ops, M, N, K, tB):
+    """Products whose 64 x 64 tiles cover less than half of the compute units, with a long K: the LDS-DMA kernel runs
+    on slices of K and the pass of the few-rows kernel adds them in order (the trace shows both); every bias kind,
+    1e-5 relative against float64 and against the oracle, and the same bits on a second call."""
+    r = rng(940 + M + N + K + tB)
+    A = r.standard_normal((M, K)).astype(np.float32)
+    B = r.standard_normal((N, K) if tB else (K, N)).astype(np.float32)
+    for kind in range(3):
+        bias = [None, r.standard_normal(N).astype(np.float32), r.standard_normal((M, N)).astype(np.float32)][kind]
+        alpha, beta, relu = [1.0, 0.5, -2.0][kind], (0.0 if bias is None else [1.0, 0.25][kind % 2]), kind != 1
+        y, names = _kernels_of(ops, lambda: ops.gemm_f32(A, B, bias, alpha, beta, False, bool(tB), relu))
+        # (a bias given for every output element is not a case of the LDS-DMA kernel)
+        assert names == (["k_gemm_f32"] if kind == 2 else ["k_gemm_f32_dma64", "k_gemm_f32_skinny_finish"]), names
+        ref = alpha * (A.astype(np.float64) @ (B.T if tB else B).astype(np.float64)) + (beta * bias if bias is not None else 0.0)
+        ref = np.maximum(ref, 0) if relu else ref
+        assert rel_err(y, ref) <= FP32_TOL
+        assert rel_err(y, oracle.gemm_f32(A, B, bias, alpha, beta, False, bool(tB), relu)) <= FP32_TOL
+        assert np.array_equal(y, ops.gemm_f32(A, B, bias, alpha, beta, False, bool(tB), relu))
+
+
 def test_gemm_f32_few_rows_integer_data_is_exact_with_a_column_bias(ops):
     """Integer operands make every order of summation exact: the sliced pass over B against int64 numpy, bias as a
     column (one value per row), rows of A and Y wider than the matrices, through the C ABI."""
