@@ -180,6 +180,37 @@ def cpu_emitted(workload, threads, blas, extra=()):
     return out if out["selfcheck"] <= 1e-3 else None
 
 
+def generated_host_session(name, weights, x, threads, blas, iters):
+    """The model's Session generated as code for the host cores (Options::kHostCode: the reference's own emission, BLAS
+    calls and loops) and compiled ahead of the run (sofie_amd/generated/host/run_host_<name>), timed on `threads`
+    threads of the BLAS library: wall time of Session::infer on a host tensor, median over `iters` calls after one."""
+    exe = os.path.join(ROOT, "sofie_amd", "generated", "host", "run_host_" + name)
+    dat = os.path.join(ROOT, "sofie_amd", "generated", weights + ".dat")
+    if not os.path.exists(exe) or not os.path.exists(dat):
+        return None
+    env = dict(os.environ)
+    for k in ("OMP_NUM_THREADS", "MKL_NUM_THREADS", "OPENBLAS_NUM_THREADS"):
+        env[k] = str(threads)
+    env["MKL_DYNAMIC"] = "FALSE"
+    env.pop("SOFIE_BLAS", None)
+    env.pop("SOFIE_BLAS_PREFIX", None)
+    if blas:
+        env["SOFIE_BLAS"], env["SOFIE_BLAS_PREFIX"] = blas[0], blas[1]
+    with tempfile.TemporaryDirectory() as tmp:
+        fin, fout = os.path.join(tmp, "in.bin"), os.path.join(tmp, "out.bin")
+        np.ascontiguousarray(x, np.float32).tofile(fin)
+        try:
+            res = subprocess.run([exe, dat, fin, fout, str(iters)], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                                 env=env, timeout=240)
+        except subprocess.TimeoutExpired:
+            return None
+        if res.returncode != 0:
+            return None
+        t = json.loads(res.stdout.strip().splitlines()[-1])
+        return {"median_ms": t["host_ms"], "best_ms": t["best_ms"], "calls": iters, "cores": threads,
+                "checksum": float(np.fromfile(fout, np.float32).astype(np.float64).sum())}
+
+
 def cpu_fp32_baselines(threads, conv_images=64):
     """The reference's emitted CPU sequence (bias copy + sgemm_ + ReLU; weight re-layout + Im2col + sgemm_ + saxpy_ +
     Relu) on the host cores: first BLAS that binds and passes the self-check, at 1 thread and at `threads`."""
@@ -212,6 +243,13 @@ def cpu_fp32_baselines(threads, conv_images=64):
         if m:
             res["mlp_b256_%dthr" % t] = {"median_us": m["median_ms"] * 1e3, "best_us": m["best_ms"] * 1e3,
                                          "inferences_per_s": 256 / (m["median_ms"] * 1e-3), "cores": t, "calls": m["calls"]}
+        hs = generated_host_session("mlp_c1", "mlp_c1", np.random.default_rng(3).standard_normal((256, 64)).astype(np.float32), t, chosen, 200)
+        if hs:
+            res["mlp_b256_generated_host_session_%dthr" % t] = {
+                "median_us": hs["median_ms"] * 1e3, "best_us": hs["best_ms"] * 1e3, "inferences_per_s": 256 / (hs["median_ms"] * 1e-3),
+                "cores": t, "calls": hs["calls"],
+                "what": "the MLP's Session generated with Options::kHostCode (this build's emission of the reference's CPU "
+                        "path), g++ -O2, Session::infer on a host tensor"}
         if c:
             res["conv_64to128_56x56_%dthr" % t] = {
                 "median_ms": c["median_ms"], "best_ms": c["best_ms"], "gflops": flops_conv / c["median_ms"] / 1e6,
@@ -659,14 +697,25 @@ def cnn_cpu_reference(images=256):
         if cpu_emitted("mlp", 1, cand, ("--calls", "20")) is not None:
             chosen = cand
             break
-    res = {"kind": "port", "what": "the reference's emitted fp32 call sequence for this network restated in C "
-                                   "(oracle/cpu_emitted_bench.c --workload cnn), gcc -O2",
+    res = {"kind": "port", "what": "the reference's emitted fp32 call sequence for this network, twice: restated in C "
+                                   "(oracle/cpu_emitted_bench.c --workload cnn, gcc -O2: the N_threads entries) and as the "
+                                   "Session this build's emitter generates with Options::kHostCode (generated_host_session_*); "
+                                   "value is the best of them",
            "blas": chosen[2] if chosen else "none found: the bundled loops", "unit": "inferences/s"}
     for th in sorted({1, threads}):
         c = cpu_emitted("cnn", th, chosen, ("--images", str(images), "--calls", "3"))
         if c:
             res["%d_threads" % th] = {"value": images / (c["median_ms"] * 1e-3), "cores": th, "median_ms": c["median_ms"],
                                       "sample": "%d of the 4096 images, median of %d calls" % (images, c["calls"])}
+    x = np.random.default_rng(2).uniform(0, 1, (256, 1, 40, 40)).astype(np.float32)
+    for th in sorted({1, threads}):
+        hs = generated_host_session("cnn_f32_b256", "cnn_f32", x, th, chosen, 3)
+        if hs:
+            res["generated_host_session_%d_threads" % th] = {
+                "value": 256 / (hs["median_ms"] * 1e-3), "cores": th, "median_ms": hs["median_ms"],
+                "sample": "256 of the 4096 images, median of 3 calls of Session::infer",
+                "what": "the float model's Session generated with Options::kHostCode (this build's emission of the "
+                        "reference's CPU path: Im2col + sgemm_ + saxpy_ per image, Relu and MaxPool loops, Gemm), g++ -O2"}
     best = max((v["value"] for k, v in res.items() if k.endswith("_threads")), default=None)
     res["value"] = best
     res["sample"] = "%d of the 4096 images per call" % images

@@ -131,11 +131,13 @@ class ModelSpec:
 
     # ---- generation ------------------------------------------------------------------------
     def generate(self, outdir=GEN_DIR, no_weight_file=False, check=True, binary_weight_file=False, batch=None,
-                 runtime_batch=False, no_session=False, emitter=None, env=None, layer_per_call=False, params=None):
+                 runtime_batch=False, no_session=False, emitter=None, env=None, layer_per_call=False, params=None,
+                 host_code=False):
         """Run the C++ emitter. Returns (header path, weight file path, CompletedProcess). `batch` gives the shape
         parameters of the inputs (dimensions written as names) their value; with `runtime_batch` it is a capacity and
         the generated Session also takes infer(n, ...) for any n up to it. `emitter` names another build of the emit
-        program (the sanitizer build), `env` its environment."""
+        program (the sanitizer build), `env` its environment. `host_code` asks for Options::kHostCode: the Session for
+        the host cores (BLAS calls and loops, as the reference generates it) instead of calls into the kernel library."""
         os.makedirs(outdir, exist_ok=True)
         tdir = os.path.join(outdir, "tensors")
         os.makedirs(tdir, exist_ok=True)
@@ -155,6 +157,8 @@ class ModelSpec:
                 flag += " runtimebatch"
             if layer_per_call:
                 flag += " layerpercall"       # Options::kLayerPerCall: no chains of fully connected layers in one launch
+            if host_code:
+                flag += " hostcode"
             f.write("\n".join(self.lines + ["generate" + flag]) + "\n")
         if emitter is None and not os.path.exists(EMIT):
             build_emitter()
@@ -184,6 +188,20 @@ class ModelSpec:
         if res.returncode:
             raise RuntimeError("compiling the generated Session failed:\n" + res.stdout)
         return exe
+
+
+def compile_host_runner(model, outdir, num_inputs=1):
+    """g++ host/examples/run_host_session.cxx against a header generated with host_code=True: a program for the host
+    cores only (no kernel library, no GPU). Its sgemm_ / saxpy_ are the runner's own loops unless SOFIE_BLAS names a
+    library at run time."""
+    exe = os.path.join(outdir, "run_host_" + model)
+    cmd = ["g++", "-std=c++17", "-O2", "-I" + outdir, "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % model,
+           "-DSOFIE_MODEL_NS=SOFIE_%s" % model, "-DSOFIE_NUM_INPUTS=%d" % num_inputs,
+           os.path.join(_HERE, "host", "examples", "run_host_session.cxx"), "-o", exe, "-ldl"]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode:
+        raise RuntimeError("compiling the generated host Session failed:\n" + res.stdout)
+    return exe
 
 
 def compile_example(source, model, exe_name, outdir=GEN_DIR):

@@ -23,7 +23,7 @@
 //   op QLinearMatMul A AS AZ B BS BZ YS YZ BIAS Y TRANSB
 //   op QLinearConv AUTOPAD GROUP nk k.. np p.. ns s.. X XS XZ W WS WZ YS YZ BIAS Y
 //   op GemmFP8 A AS B BS BIAS Y TRANSB
-//   generate [noweightfile | binaryweightfile | nosession] [batch N] [param NAME VALUE]... [runtimebatch] [layerpercall]
+//   generate [noweightfile | binaryweightfile | nosession] [batch N] [param NAME VALUE]... [runtimebatch] [layerpercall] [hostcode]
 //                                                  batch N resolves the shape parameters; runtimebatch makes N a capacity
 #include <cctype>
 #include <fstream>
@@ -207,6 +207,7 @@ int main(int argc, char **argv)
                else if (flag == "nosession") options = options | Options::kNoSession;
                else if (flag == "runtimebatch") options = options | Options::kRuntimeBatch;
                else if (flag == "layerpercall") options = options | Options::kLayerPerCall;
+               else if (flag == "hostcode") options = options | Options::kHostCode;
                else if (flag == "batch") in >> batch;
                else if (flag == "param") {
                   std::string pname;

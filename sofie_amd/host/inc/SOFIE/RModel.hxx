@@ -31,6 +31,8 @@ enum class Options {
    kBinaryWeightFile = 0x20,     // typed binary records in <name>.bin instead of the text <name>.dat (not in the reference)
    kRuntimeBatch = 0x40,         // the batch size given to Generate is a capacity: infer(n, ...) runs any n up to it
    kLayerPerCall = 0x80,         // no chains of fully connected layers in one launch: every Gemm emits its own call
+   kHostCode = 0x100,            // code for the host cores, as the reference emits it (BLAS::sgemm_ / saxpy_ and loops on host
+                                 // memory) instead of calls into the kernel library: fp32 Gemm, Conv, Relu, pooling, Reshape
 };
 std::underlying_type_t<Options> operator|(Options opA, Options opB);
 std::underlying_type_t<Options> operator|(std::underlying_type_t<Options> opA, Options opB);
@@ -140,11 +142,13 @@ private:
    void PlanIntermediateMemory();
    void GenerateHeaderInfo(std::string &hgname);
    void GenerateSessionCode();
+   void GenerateHostHeaderInfo(std::string &hgname);
+   void GenerateHostSessionCode();
    std::string RootOf(const std::string &name) const;
 
    std::string fFileName, fParseTime, fName = "UnnamedModel", fGC;
    WeightFileType fWeightFile = WeightFileType::Text;
-   bool fUseWeightFile = true, fUseSession = true, fIsInitialized = false;
+   bool fUseWeightFile = true, fUseSession = true, fIsInitialized = false, fHostCode = false;
    int fVerbose = 0;
 
    std::map<std::string, TensorInfo> fReadyInputTensorInfos;

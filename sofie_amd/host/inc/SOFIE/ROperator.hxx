@@ -68,6 +68,17 @@ public:
       fBatchCapacity = capacity;
       return true;
    }
+   // --- host emission (Options::kHostCode) ----------------------------------------------------
+   // The operator as code for the host cores, in the reference's way (BLAS::sgemm_ / saxpy_ calls and plain
+   // loops on host pointers named tensor_<name>): members of the Session, statements of its constructor, and the
+   // statements of infer. An operator without a host form says so when it is asked for one.
+   virtual std::string GenerateHost(std::string /*opName*/)
+   {
+      throw std::runtime_error("TMVA SOFIE " + (Kind().empty() ? std::string("operator") : Kind()) +
+                               " Op has no host emission (Options::kHostCode)");
+   }
+   virtual std::string GenerateHostSessionMembersCode(std::string /*opName*/) { return ""; }
+   virtual std::string GenerateHostInitCode(std::string /*opName*/) { return ""; }
    // absorbed into another operator: emits nothing, and its output is written by the absorbing operator
    void SetAbsorbed() { fAbsorbed = true; }
    bool IsAbsorbed() const { return fAbsorbed; }

@@ -241,6 +241,88 @@ public:
           << OpName << "\");\n";
       return out.str();
    }
+
+   // Host form, the reference's sequence (ROperator_Conv.hxx:302-522): per image (and group) the patches are laid out
+   // as a column-major [OH*OW, C/g*KH*KW] matrix (Im2col), one BLAS::sgemm_ multiplies it with the group's filters
+   // (the [OC/g, C/g*KH*KW] rows of the weight tensor are that matrix's column-major transpose already), and the
+   // bias, broadcast to [OC,OH,OW] once in the constructor, is added with BLAS::saxpy_; then the ReLU loop. The
+   // geometry is this emitter's (ONNX pads and dilations, see the head of the file), through the same Im2col.
+   std::string GenerateHostSessionMembersCode(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShapeY.empty()) throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
+      if (fGeom.dim == 3) throw std::runtime_error("TMVA SOFIE Conv Op: three spatial dimensions have no host emission");
+      size_t spatialOut = 1, kernelCells = 1;
+      for (size_t i = 0; i < fGeom.dim; ++i) { spatialOut *= fShapeY[2 + i]; kernelCells *= fShapeW[2 + i]; }
+      std::stringstream out;
+      out << "std::vector<float> fVec_" << OpName << "_xcol = std::vector<float>(" << fShapeW[1] * kernelCells * spatialOut << ");\n";
+      if (fNB != "") out << "std::vector<float> fVec_" << OpName << "_bias = std::vector<float>(" << fShapeY[1] * spatialOut << ");\n";
+      return out.str();
+   }
+   std::string GenerateHostInitCode(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fNB == "") return "";
+      size_t spatialOut = 1;
+      for (size_t i = 0; i < fGeom.dim; ++i) spatialOut *= fShapeY[2 + i];
+      std::stringstream out;
+      out << SP << "for (size_t oc = 0; oc < " << fShapeY[1] << "; ++oc) std::fill_n(fVec_" << OpName << "_bias.data() + oc * " << spatialOut
+          << ", " << spatialOut << ", tensor_" << fNB << "[oc]);\n";
+      return out.str();
+   }
+   std::string GenerateHost(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShapeX.empty() || fShapeW.empty() || (fNB != "" && fShapeB.empty()) || fShapeY.empty())
+         throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
+      const size_t dim = fGeom.dim;
+      if (dim == 3) throw std::runtime_error("TMVA SOFIE Conv Op: three spatial dimensions have no host emission");
+      const bool oneD = dim == 1;
+      const size_t H = oneD ? 1 : fShapeX[2], W = fShapeX[dim + 1];
+      const size_t KH = oneD ? 1 : fShapeW[2], KW = fShapeW[dim + 1];
+      const size_t OH = oneD ? 1 : fShapeY[2], OW = fShapeY[dim + 1];
+      const std::vector<size_t> &p = fGeom.pads;
+      const size_t pt = oneD ? 0 : p[0], pl = p[dim - 1];
+      const size_t sh = oneD ? 1 : fGeom.strides[0], sw = fGeom.strides[dim - 1];
+      const size_t dh = oneD ? 1 : fGeom.dilations[0], dw = fGeom.dilations[dim - 1];
+      const size_t C = fShapeX[1], OC = fShapeW[0], G = fGeom.group, Cg = fShapeW[1], OCg = OC / G;
+      std::stringstream out;
+      out << "\n//----  operator Conv " << OpName << "\n";
+      out << SP << "{\n";
+      out << SP << SP << "char " << OpName << "_transA = 'N';\n";
+      out << SP << SP << "char " << OpName << "_transB = 'N';\n";
+      out << SP << SP << "int " << OpName << "_m = " << OH * OW << ";\n";
+      out << SP << SP << "int " << OpName << "_n = " << OCg << ";\n";
+      out << SP << SP << "int " << OpName << "_k = " << Cg * KH * KW << ";\n";
+      out << SP << SP << "float " << OpName << "_alpha = 1.0;\n";
+      out << SP << SP << "float " << OpName << "_beta = 0.0;\n";
+      out << SP << SP << "float * " << OpName << "_xcol = fVec_" << OpName << "_xcol.data();\n";
+      out << SP << SP << "for (size_t n = 0; n < " << BatchCount(fShapeX[0]) << "; n++) {\n";
+      out << SP << SP << SP << "for (size_t g = 0; g < " << G << "; g++) {\n";
+      out << SP << SP << SP << SP << "Im2col(tensor_" << fNX << " + (n * " << C << " + g * " << Cg << ") * " << H * W << ", " << Cg << ", " << H
+          << ", " << W << ", " << KH << ", " << KW << ", " << pt << ", " << pl << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << OH
+          << ", " << OW << ", " << OpName << "_xcol);\n";
+      out << SP << SP << SP << SP << "BLAS::sgemm_(&" << OpName << "_transA, &" << OpName << "_transB, &" << OpName << "_m, &" << OpName
+          << "_n, &" << OpName << "_k, &" << OpName << "_alpha, " << OpName << "_xcol, &" << OpName << "_m, tensor_" << fNW << " + g * "
+          << OCg * Cg * KH * KW << ", &" << OpName << "_k, &" << OpName << "_beta, tensor_" << fNY << " + (n * " << OC << " + g * " << OCg
+          << ") * " << OH * OW << ", &" << OpName << "_m);\n";
+      out << SP << SP << SP << "}\n";
+      if (fNB != "") {
+         out << SP << SP << SP << "int " << OpName << "_size = " << OC * OH * OW << ";\n";
+         out << SP << SP << SP << "float " << OpName << "_gamma = 1.0;\n";
+         out << SP << SP << SP << "int " << OpName << "_incx = 1;\n";
+         out << SP << SP << SP << "int " << OpName << "_incy = 1;\n";
+         out << SP << SP << SP << "BLAS::saxpy_(&" << OpName << "_size, &" << OpName << "_gamma, fVec_" << OpName << "_bias.data(), &" << OpName
+             << "_incx, tensor_" << fNY << " + n * " << OC * OH * OW << ", &" << OpName << "_incy);\n";
+      }
+      out << SP << SP << "}\n";
+      if (fActivation == EActivationType::RELU) {
+         out << SP << SP << "for (size_t id = 0; id < " << BatchCount(ConvertShapeToLength(fShapeY)) << "; id++)\n";
+         out << SP << SP << SP << "tensor_" << fNY << "[id] = ((tensor_" << fNY << "[id] > 0 )? tensor_" << fNY << "[id] : 0);\n";
+      }
+      out << SP << "}\n";
+      return out.str();
+   }
 };
 
 }   // namespace SOFIE

@@ -335,6 +335,69 @@ public:
           << act << "), \"Gemm " << opName << "\");\n";
       return out.str();
    }
+
+   // Host form, as the reference emits it (ROperator_Gemm.hxx:292-390): the bias broadcast to [M,N] is copied into Y,
+   // then one BLAS::sgemm_ in the column-major reading of the row-major tensors (Y^T = op(B)^T op(A)^T, so B comes
+   // first and the leading dimension of Y is N), then the ReLU loop. Stacked operands run one such product per
+   // matrix, each on its own matrices of A and B.
+   std::string GenerateHost(std::string opName) override
+   {
+      opName = "op_" + opName;
+      if (fShapeA.empty() || fShapeB.empty() || fShapeY.empty() || (fNC != "" && fShapeC.empty()))
+         throw std::runtime_error("TMVA SOFIE Gemm Op called to Generate without being initialized first");
+      if (fNC.empty() && fAttrBeta != 0)
+         throw std::runtime_error("TMVA SOFIE Gemm Op " + opName + " Bias tensor is not present but beta value in Gemm is not zero");
+      const size_t m = fShapeY[0], n = fShapeY[1];
+      const size_t k = fAttrTransA ? fShapeA[0] : fShapeA[1];
+      std::stringstream out;
+      out << "\n//--------- Gemm\n";
+      out << SP << "{\n";
+      out << SP << SP << "char " << opName << "_transA = '" << (fAttrTransA ? "t" : "n") << "';\n";
+      out << SP << SP << "char " << opName << "_transB = '" << (fAttrTransB ? "t" : "n") << "';\n";
+      out << SP << SP << "int " << opName << "_m = " << BatchCount(m) << ";\n";
+      out << SP << SP << "int " << opName << "_n = " << n << ";\n";
+      out << SP << SP << "int " << opName << "_k = " << k << ";\n";
+      out << SP << SP << "float " << opName << "_alpha = " << FloatLiteral(fAttrAlpha) << ";\n";
+      out << SP << SP << "float " << opName << "_beta = " << FloatLiteral(fNC.empty() ? 0.0f : fAttrBeta) << ";\n";
+      out << SP << SP << "int " << opName << "_lda = " << fShapeA[1] << ";\n";
+      out << SP << SP << "int " << opName << "_ldb = " << fShapeB[1] << ";\n";
+      if (!fNC.empty()) {
+         const std::string rows = opName + "_m";
+         if (fBiasKind == 2)
+            out << SP << SP << "std::copy(tensor_" << fNC << ", tensor_" << fNC << " + static_cast<size_t>(" << rows << ") * " << n
+                << ", tensor_" << fNY << ");\n";
+         else if (fBiasKind == 1)
+            out << SP << SP << "for (int row = 0; row < " << rows << "; ++row) std::copy(tensor_" << fNC << ", tensor_" << fNC << " + "
+                << n << ", tensor_" << fNY << " + static_cast<size_t>(row) * " << n << ");\n";
+         else
+            out << SP << SP << "for (int row = 0; row < " << rows << "; ++row) std::fill_n(tensor_" << fNY
+                << " + static_cast<size_t>(row) * " << n << ", " << n << ", tensor_" << fNC << "[row]);\n";
+      }
+      if (fStack > 1) {
+         const size_t sizeA = fShapeA[0] * fShapeA[1], sizeB = fShapeB[0] * fShapeB[1];
+         out << SP << SP << "static const size_t " << opName << "_offA[] = {";
+         for (size_t i = 0; i < fStack; ++i) out << (i ? ", " : "") << fStackA[i] * sizeA;
+         out << "};\n";
+         out << SP << SP << "static const size_t " << opName << "_offB[] = {";
+         for (size_t i = 0; i < fStack; ++i) out << (i ? ", " : "") << fStackB[i] * sizeB;
+         out << "};\n";
+         out << SP << SP << "for (size_t stack = 0; stack < " << fStack << "; ++stack)\n";
+         out << SP << SP << SP << "BLAS::sgemm_(&" << opName << "_transB, &" << opName << "_transA, &" << opName << "_n, &" << opName
+             << "_m, &" << opName << "_k, &" << opName << "_alpha, tensor_" << fNB << " + " << opName << "_offB[stack], &" << opName
+             << "_ldb, tensor_" << fNA << " + " << opName << "_offA[stack], &" << opName << "_lda, &" << opName << "_beta, tensor_"
+             << fNY << " + stack * " << m * n << ", &" << opName << "_n);\n";
+      } else {
+         out << SP << SP << "BLAS::sgemm_(&" << opName << "_transB, &" << opName << "_transA, &" << opName << "_n, &" << opName
+             << "_m, &" << opName << "_k, &" << opName << "_alpha, tensor_" << fNB << ", &" << opName << "_ldb, tensor_" << fNA
+             << ", &" << opName << "_lda, &" << opName << "_beta, tensor_" << fNY << ", &" << opName << "_n);\n";
+      }
+      if (fActivation == EActivationType::RELU) {
+         out << SP << SP << "for (size_t id = 0; id < static_cast<size_t>(" << opName << "_m) * " << n * fStack << "; id++)\n";
+         out << SP << SP << SP << "tensor_" << fNY << "[id] = ((tensor_" << fNY << "[id] > 0 )? tensor_" << fNY << "[id] : 0);\n";
+      }
+      out << SP << "}\n";
+      return out.str();
+   }
 };
 
 }   // namespace SOFIE

@@ -179,6 +179,39 @@ public:
           << "), \"" << Name() << " " << OpName << "\");\n";
       return out.str();
    }
+
+   // Host form: the loops of the reference's pooling (ROperator_Pool.hxx:266-476) over one, two or three spatial
+   // axes, as one helper of the generated file (Pool3d; missing leading axes have extent 1). A window takes the cells
+   // that lie inside the image; the average divides by their number, or by the kernel's size with count_include_pad.
+   std::string GenerateHost(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShapeX.empty() || fShapeY.empty())
+         throw std::runtime_error("TMVA SOFIE Pool Op called to Generate without being initialized first");
+      if (fType != ETensorType::FLOAT) throw std::runtime_error("TMVA SOFIE Pool Op " + OpName + ": the host emission takes float tensors");
+      const size_t dims = fShapeX.size() - 2;
+      if (fPoolMode != MaxPool && !fAttr.count_include_pad)
+         for (size_t i = 0; i < 2 * dims; ++i)
+            if (fAttr.pads[i] >= fAttr.kernel_shape[i % dims])
+               throw std::runtime_error("TMVA SOFIE" + Name() + "Op : a pad as large as the kernel leaves windows without a cell of the image");
+      // three axes, the given ones last
+      size_t in[3] = {1, 1, 1}, o[3] = {1, 1, 1}, k[3] = {1, 1, 1}, pb[3] = {0, 0, 0}, st[3] = {1, 1, 1};
+      for (size_t i = 0; i < dims; ++i) {
+         const size_t a = 3 - dims + i;
+         in[a] = fShapeX[2 + i]; o[a] = fShapeY[2 + i]; k[a] = fAttr.kernel_shape[i]; pb[a] = fAttr.pads[i]; st[a] = fAttr.strides[i];
+      }
+      auto list = [](const size_t (&v)[3]) { return "{" + std::to_string(v[0]) + ", " + std::to_string(v[1]) + ", " + std::to_string(v[2]) + "}"; };
+      std::stringstream out;
+      out << "\n//----  operator " << Name() << "  " << OpName << "\n";
+      out << SP << "{\n";
+      out << SP << SP << "const int " << OpName << "_in[3] = " << list(in) << ", " << OpName << "_out[3] = " << list(o) << ", " << OpName
+          << "_kernel[3] = " << list(k) << ", " << OpName << "_pads[3] = " << list(pb) << ", " << OpName << "_strides[3] = " << list(st) << ";\n";
+      out << SP << SP << "Pool3d(" << (fPoolMode == MaxPool ? "true" : "false") << ", " << (fAttr.count_include_pad ? "true" : "false") << ", tensor_"
+          << fNX << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0] * fShapeX[1]) << ", " << OpName << "_in, " << OpName << "_out, " << OpName
+          << "_kernel, " << OpName << "_pads, " << OpName << "_strides);\n";
+      out << SP << "}\n";
+      return out.str();
+   }
 };
 
 }   // namespace SOFIE

@@ -50,6 +50,19 @@ public:
           << "), \"Relu " << OpName << "\");\n";
       return out.str();
    }
+   // reference: ROperator_Relu.hxx:54-66 (one loop over the elements)
+   std::string GenerateHost(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShape.empty()) throw std::runtime_error("TMVA SOFIE Operator Relu called to Generate without being initialized first");
+      if (fType != ETensorType::FLOAT) throw std::runtime_error("TMVA SOFIE Relu Op " + OpName + ": the host emission takes float tensors");
+      std::stringstream out;
+      out << "\n//------ RELU\n";
+      out << SP << "for (size_t id = 0; id < " << BatchCount(ConvertShapeToLength(fShape)) << " ; id++){\n";
+      out << SP << SP << "tensor_" << fNY << "[id] = ((tensor_" << fNX << "[id] > 0 )? tensor_" << fNX << "[id] : 0);\n";
+      out << SP << "}\n";
+      return out.str();
+   }
 };
 
 }   // namespace SOFIE

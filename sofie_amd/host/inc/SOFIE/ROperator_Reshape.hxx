@@ -95,6 +95,15 @@ public:
              ")) Check(sofie_hip_copy(fCtx, tensor_" + fNOutput + ", tensor_" + fNData + ", " +
              BatchCount(ConvertShapeToLength(fShapeOutput)) + " * sizeof(*tensor_" + fNOutput + ")), \"Reshape\");\n";
    }
+   // the same view on host pointers; the reference copies the elements (ROperator_Reshape.hxx Generate)
+   std::string GenerateHost(std::string OpName) override
+   {
+      if (fShapeInput.empty()) throw std::runtime_error("TMVA SOFIE Reshape Op called to Generate without being initialized first");
+      return "\n//------ " + std::string(fOpMode == Flatten ? "FLATTEN" : "RESHAPE") + " op_" + OpName + "\n" + SP +
+             "if (static_cast<const void*>(tensor_" + fNOutput + ") != static_cast<const void*>(tensor_" + fNData +
+             ")) std::memcpy(tensor_" + fNOutput + ", tensor_" + fNData + ", " + BatchCount(ConvertShapeToLength(fShapeOutput)) +
+             " * sizeof(*tensor_" + fNOutput + "));\n";
+   }
 };
 
 }   // namespace SOFIE

@@ -1101,6 +1101,216 @@ void RModel::GenerateSessionCode()
    fGC += "};\n";
 }
 
+// ---- Options::kHostCode: the Session for the host cores, as the reference generates it (RModel.cxx:560-801 there):
+// weights and intermediates in host memory, operators as BLAS calls and loops, infer(float*...) returning vectors.
+void RModel::GenerateHostHeaderInfo(std::string &hgname)
+{
+   fGC += "//Code generated automatically by SOFIE (host emission) from file " + fFileName + " at [" +
+          fParseTime.substr(0, fParseTime.length() - 1) + "] \n";
+   hgname = fName;
+   std::transform(hgname.begin(), hgname.end(), hgname.begin(), [](unsigned char c) { return std::toupper(c); });
+   hgname = "SOFIE_" + hgname;
+   fGC += "\n#ifndef " + hgname + "\n";
+   fGC += "#define " + hgname + "\n\n";
+   for (auto &i : fNeededStdLib) fGC += "#include <" + i + ">\n";
+   fGC += "#include <algorithm>\n#include <cstdint>\n#include <cstring>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n"
+          "#include <tuple>\n#include <utility>\n#include <limits>\n";
+   fGC += "\nnamespace SOFIE_" + fName + "{\n";
+   // the Fortran BLAS the program is linked with, declared as the reference declares it (RModel_Base.cxx:40-58)
+   fGC += "namespace BLAS{\n";
+   fGC += "   extern \"C\" void sgemm_(const char * transa, const char * transb, const int * m, const int * n, const int * k,\n"
+          "                          const float * alpha, const float * A, const int * lda, const float * B, const int * ldb,\n"
+          "                          const float * beta, float * C, const int * ldc);\n";
+   fGC += "   extern \"C\" void saxpy_(const int * n, const float * alpha, const float * x, const int * incx, float * y, const int * incy);\n";
+   fGC += "}//BLAS\n";
+   // Patches of one image (or one group's channels of it) as a column-major [OH*OW, C*KH*KW] matrix: column
+   // (c*KH + kh)*KW + kw holds, for every output position, the input cell under kernel cell (kh, kw) of channel c,
+   // zero outside the image (the role of UTILITY::Im2col, SOFIE_common.hxx:485-518 of the reference).
+   fGC += "inline void Im2col(const float * x, int C, int H, int W, int KH, int KW, int padTop, int padLeft, int strideH, int strideW,\n"
+          "                   int dilationH, int dilationW, int OH, int OW, float * xcol) {\n"
+          "   for (int c = 0; c < C; ++c)\n"
+          "      for (int kh = 0; kh < KH; ++kh)\n"
+          "         for (int kw = 0; kw < KW; ++kw) {\n"
+          "            float * col = xcol + (static_cast<size_t>(c * KH + kh) * KW + kw) * OH * OW;\n"
+          "            for (int oh = 0; oh < OH; ++oh) {\n"
+          "               const int ih = oh * strideH - padTop + kh * dilationH;\n"
+          "               for (int ow = 0; ow < OW; ++ow) {\n"
+          "                  const int iw = ow * strideW - padLeft + kw * dilationW;\n"
+          "                  col[oh * OW + ow] = (ih >= 0 && ih < H && iw >= 0 && iw < W) ? x[(static_cast<size_t>(c) * H + ih) * W + iw] : 0.f;\n"
+          "               }\n"
+          "            }\n"
+          "         }\n"
+          "}\n";
+   // Pooling over three axes (leading axes of extent 1 for fewer): maximum, or mean, of the window's cells inside the image.
+   fGC += "inline void Pool3d(bool isMax, bool countIncludePad, const float * x, float * y, size_t planes, const int * in, const int * out,\n"
+          "                   const int * kernel, const int * pads, const int * strides) {\n"
+          "   const size_t inSize = static_cast<size_t>(in[0]) * in[1] * in[2];\n"
+          "   size_t o = 0;\n"
+          "   for (size_t p = 0; p < planes; ++p) {\n"
+          "      const float * xp = x + p * inSize;\n"
+          "      for (int od = 0; od < out[0]; ++od)\n"
+          "         for (int oh = 0; oh < out[1]; ++oh)\n"
+          "            for (int ow = 0; ow < out[2]; ++ow) {\n"
+          "               float value = isMax ? -std::numeric_limits<float>::infinity() : 0.f;\n"
+          "               int cells = 0;\n"
+          "               for (int kd = 0; kd < kernel[0]; ++kd) {\n"
+          "                  const int id = od * strides[0] - pads[0] + kd;\n"
+          "                  if (id < 0 || id >= in[0]) continue;\n"
+          "                  for (int kh = 0; kh < kernel[1]; ++kh) {\n"
+          "                     const int ih = oh * strides[1] - pads[1] + kh;\n"
+          "                     if (ih < 0 || ih >= in[1]) continue;\n"
+          "                     for (int kw = 0; kw < kernel[2]; ++kw) {\n"
+          "                        const int iw = ow * strides[2] - pads[2] + kw;\n"
+          "                        if (iw < 0 || iw >= in[2]) continue;\n"
+          "                        const float v = xp[(static_cast<size_t>(id) * in[1] + ih) * in[2] + iw];\n"
+          "                        if (isMax) { if (v > value) value = v; } else value += v;\n"
+          "                        cells++;\n"
+          "                     }\n"
+          "                  }\n"
+          "               }\n"
+          "               if (!isMax) value /= static_cast<float>(countIncludePad ? kernel[0] * kernel[1] * kernel[2] : cells);\n"
+          "               y[o++] = value;\n"
+          "            }\n"
+          "   }\n"
+          "}\n";
+}
+
+void RModel::GenerateHostSessionCode()
+{
+   fGC += "struct Session {\n";
+   if (fRuntimeBatch)
+      fGC += "size_t fBatch = " + std::to_string(fBatchCapacity) + ";   // rows of the batch the operators process, at most " +
+             std::to_string(fBatchCapacity) + "\n";
+   {
+      bool any = false;
+      for (auto &i : fInitializedTensors) any |= i.second.IsWeightTensor();
+      if (any && fUseWeightFile) fGC += GenerateWeightReaderHelpers();
+   }
+   for (auto &i : fInitializedTensors) {
+      if (!i.second.IsWeightTensor()) continue;
+      const std::string ctype = ConvertTypeToString(i.second.type());
+      const size_t length = ConvertShapeToLength(i.second.shape());
+      fGC += "std::vector<" + ctype + "> fTensor_" + i.first + " = std::vector<" + ctype + ">(" + std::to_string(length) + ");\n";
+      fGC += ctype + " * tensor_" + i.first + " = fTensor_" + i.first + ".data();\n";
+   }
+   fGC += "std::vector<char> fIntermediateMemoryPool = std::vector<char>(" + std::to_string(fArenaBytes) + ");\n";
+   for (auto &it : fIntermediateTensorInfos)
+      fGC += ConvertTypeToString(it.second.type) + " * tensor_" + it.first + " = nullptr;\n";
+   for (size_t id = 0; id < fOperators.size(); id++) fGC += fOperators[id]->GenerateHostSessionMembersCode(std::to_string(id));
+   fGC += "\n";
+   fGC += "Session(std::string filename =\"" +
+          (fUseWeightFile ? fName + (fWeightFile == WeightFileType::Binary ? ".bin" : ".dat") : std::string("")) + "\") {\n";
+   for (auto &it : fIntermediateTensorInfos) {
+      if (fViewOf.count(it.first)) continue;
+      fGC += "   tensor_" + it.first + " = reinterpret_cast<" + ConvertTypeToString(it.second.type) +
+             "*>(fIntermediateMemoryPool.data() + " + std::to_string(fPlacement[it.first].offset) + ");\n";
+   }
+   for (auto &op : fOperators)
+      for (auto &out : op->GetOpOutputTensors()) {
+         auto v = fViewOf.find(out);
+         if (v == fViewOf.end()) continue;
+         fGC += "   tensor_" + out + " = reinterpret_cast<" + ConvertTypeToString(fIntermediateTensorInfos[out].type) +
+                "*>(tensor_" + v->second + ");\n";
+      }
+   bool anyWeight = false;
+   for (auto &i : fInitializedTensors) anyWeight |= i.second.IsWeightTensor();
+   if (fUseWeightFile && anyWeight) {
+      fGC += "   std::ifstream f;\n";
+      fGC += "   f.open(filename, std::ios::binary);\n";
+      fGC += "   if (!f.is_open()) {\n";
+      fGC += "      throw std::runtime_error(\"tmva-sofie failed to open file \" + filename + \" for input weights\");\n";
+      fGC += "   }\n";
+      fGC += "   const bool binary = IsBinaryWeightFile(f);\n";
+      for (auto &i : fInitializedTensors) {
+         if (!i.second.IsWeightTensor()) continue;
+         const std::string tensor_name = "tensor_" + i.first;
+         fGC += "   ReadTensor(f, binary, \"" + tensor_name + "\", " + std::to_string(ConvertShapeToLength(i.second.shape())) + ", " +
+                std::to_string(static_cast<int>(i.second.type())) + ", " + tensor_name + ");\n";
+      }
+      fGC += "   f.close();\n";
+   } else {
+      for (auto &i : fInitializedTensors) {
+         if (!i.second.IsWeightTensor()) continue;
+         if (i.second.type() != ETensorType::FLOAT && i.second.type() != ETensorType::INT64)
+            throw std::runtime_error("tmva-sofie tensor_" + i.first + " cannot be written as a literal by the host emission");
+         const size_t length = ConvertShapeToLength(i.second.shape());
+         std::stringstream lit;
+         lit << "   { static const " << ConvertTypeToString(i.second.type()) << " host[" << (length ? length : 1) << "] = {";
+         for (size_t idx = 0; idx < length; ++idx) {
+            if (idx) lit << ", ";
+            if (i.second.type() == ETensorType::FLOAT) {
+               if (!std::isfinite(i.second.data<float>()[idx]))
+                  throw std::runtime_error("tmva-sofie tensor_" + i.first + " holds a non-finite value");
+               std::stringstream one;
+               one << std::setprecision(std::numeric_limits<float>::max_digits10) << i.second.data<float>()[idx];
+               std::string text = one.str();
+               if (text.find_first_of(".e") == std::string::npos) text += ".";
+               lit << text << "f";
+            } else {
+               lit << i.second.data<int64_t>()[idx];
+            }
+         }
+         lit << "};\n     std::copy(host, host + " << length << ", tensor_" << i.first << "); }\n";
+         fGC += lit.str();
+      }
+   }
+   for (size_t id = 0; id < fOperators.size(); id++) fGC += fOperators[id]->GenerateHostInitCode(std::to_string(id));
+   fGC += "}\n\n";
+
+   // ---- infer: the reference's signature and return convention (RModel.cxx:680-801)
+   const size_t nout = fOutputTensorNames.size();
+   if (nout == 0) throw std::runtime_error("TMVA-SOFIE: output size=0 are not supported");
+   const std::string out = fOutputTensorNames[0];
+   const std::string otype = ConvertTypeToString(GetTensorType(out));
+   bool sameOutputTypes = true;
+   for (auto &n : fOutputTensorNames) sameOutputTypes = sameOutputTypes && GetTensorType(n) == GetTensorType(out);
+   std::string inferReturnType = "std::vector<" + otype + ">";
+   if (nout > 1) {
+      if (sameOutputTypes) {
+         inferReturnType = "std::vector<std::vector<" + otype + ">>";
+      } else {
+         inferReturnType = "std::tuple<";
+         for (size_t i = 0; i < nout; ++i)
+            inferReturnType += std::string(i ? "," : "") + "std::vector<" + ConvertTypeToString(GetTensorType(fOutputTensorNames[i])) + ">";
+         inferReturnType += ">";
+      }
+   }
+   auto outputCount = [&](const std::string &n) {
+      const size_t len = ConvertShapeToLength(GetTensorShape(n));
+      return (fRuntimeBatch && fBatchTensors.count(n)) ? "fBatch * " + std::to_string(len / fBatchCapacity) : std::to_string(len);
+   };
+   auto body = [&]() {
+      for (size_t id = 0; id < fOperators.size(); id++) fGC += fOperators[id]->GenerateHost(std::to_string(id));
+      if (nout == 1) {
+         fGC += "   return std::vector<" + otype + ">(tensor_" + out + ", tensor_" + out + " + " + outputCount(out) + ");\n";
+         return;
+      }
+      fGC += "   return " + inferReturnType + "{";
+      for (size_t i = 0; i < nout; ++i) {
+         const std::string &n = fOutputTensorNames[i];
+         fGC += std::string(i ? ", " : "") + "std::vector<" + ConvertTypeToString(GetTensorType(n)) + ">(tensor_" + n + ", tensor_" + n +
+                " + " + outputCount(n) + ")";
+      }
+      fGC += "};\n";
+   };
+   if (fRuntimeBatch) {
+      fGC += inferReturnType + " infer(size_t batch, " + GenerateInferSignature(true) + "){\n";
+      fGC += "   if (batch == 0 || batch > " + std::to_string(fBatchCapacity) +
+             ") throw std::runtime_error(\"TMVA SOFIE: the batch must be between 1 and " + std::to_string(fBatchCapacity) +
+             ", the size this Session was generated for\");\n";
+      fGC += "   fBatch = batch;\n";
+      body();
+      fGC += "}\n";
+      fGC += inferReturnType + " infer(" + GenerateInferSignature(true) + "){ return infer(" + std::to_string(fBatchCapacity) + ", " +
+             GenerateInferSignature(false) + "); }\n";
+   } else {
+      fGC += inferReturnType + " infer(" + GenerateInferSignature(true) + "){\n";
+      body();
+      fGC += "}\n";
+   }
+   fGC += "};\n";
+}
+
 void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, long pos, bool verbose)
 {
    fVerbose = verbose;
@@ -1124,7 +1334,25 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    fRuntimeBatch = (static_cast<std::underlying_type_t<Options>>(Options::kRuntimeBatch) & options) != 0;
    if (fRuntimeBatch && batchSize <= 0)
       throw std::runtime_error("TMVA-SOFIE: Options::kRuntimeBatch needs the largest batch as the batch size given to Generate");
+   fHostCode = (static_cast<std::underlying_type_t<Options>>(Options::kHostCode) & options) != 0;
    Initialize(batchSize, verbose);
+   if (fHostCode) {
+      // every operator emits its own statements, as in the reference: no fusion pass runs (an activation the
+      // parser already attached to a Gemm or Conv is that operator's loop)
+      PlanIntermediateMemory();
+      fGC.clear();
+      std::string hostGuard;
+      GenerateHostHeaderInfo(hostGuard);
+      GenerateHostSessionCode();
+      if (noSession) {
+         fGC += "\n// Options::kNoSession: free function infer on one Session created at the first call\n";
+         fGC += "inline Session& DefaultSession() { static Session session(\"\"); return session; }\n";
+         fGC += "inline auto infer(" + GenerateInferSignature(true) + "){ return DefaultSession().infer(" + GenerateInferSignature(false) + "); }\n";
+      }
+      fGC += ("} //SOFIE_" + fName + "\n");
+      fGC += "\n#endif  // " + hostGuard + "\n";
+      return;
+   }
    FuseBatchNorm();
    FuseActivations();
    if (!(static_cast<std::underlying_type_t<Options>>(Options::kLayerPerCall) & options)) {

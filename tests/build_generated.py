@@ -57,6 +57,15 @@ def main():
         if spec.name in ("qcnn_b4096", "qcnn_rt", "cnn_f32_rt"):
             os.remove(dat)      # same tensors as qcnn.dat / cnn_f32.dat: the runner is pointed at that file
         print("%-28s %s" % (spec.name, res.stdout.strip().split(", ")[-1]))
+    # The fp32 networks once more as code for the host cores (Options::kHostCode), for the test that compares the two
+    # emissions on a GPU box and for the benchmark's CPU baseline: sofie_amd/generated/host/run_host_<name>. They
+    # read the weight files written above.
+    host_dir = os.path.join(emit.GEN_DIR, "host")
+    for spec in (models.mlp_spec()[0], models.cnn_f32_spec(8), models.cnn_f32_spec(256, "cnn_f32_b256")):
+        _, dat, res = spec.generate(host_dir, host_code=True)
+        emit.compile_host_runner(spec.name, host_dir)
+        os.remove(dat)
+        print("%-28s host code, %s" % (spec.name, res.stdout.strip().split(", ")[-1]))
     return 0
 
 

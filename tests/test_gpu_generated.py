@@ -89,6 +89,24 @@ def test_cnn_f32_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
+@pytest.mark.parametrize("name,weights", [("mlp_c1", "mlp_c1"), ("cnn_f32", "cnn_f32")])
+def test_host_and_device_emission_agree(name, weights, tmp_path):
+    """The same model generated twice, as calls into the kernel library and as code for the host cores
+    (Options::kHostCode: the reference's BLAS calls and loops), on the same seeded input: within 1e-5 relative."""
+    x = models.mlp_spec()[1] if name == "mlp_c1" else models.cnn_input(8)
+    y_device = run_session(name, x, tmp_path)
+    exe = os.path.join(emit.GEN_DIR, "host", "run_host_" + name)
+    if not os.path.exists(exe):
+        raise RuntimeError("%s is missing: run python tests/build_generated.py on the build machine" % exe)
+    fout = str(tmp_path / "host_out.bin")
+    res = subprocess.run([exe, os.path.join(emit.GEN_DIR, weights + ".dat"), str(tmp_path / "in.bin"), fout],
+                         stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=110)
+    assert res.returncode == 0, res.stderr
+    y_host = np.fromfile(fout, np.float32)
+    assert y_host.size == y_device.size
+    assert rel_err(y_device, y_host) <= 1e-5
+
+
 def test_runtime_batch_sessions(tmp_path):
     """Sessions generated with a batch capacity of 8 run 8, 3 and 1 images through infer(n, ...): the int8 network's
     logits are those of the oracle on the same images bit for bit, the float network's within 1e-5."""

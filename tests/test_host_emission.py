@@ -1,0 +1,100 @@
+"""Options::kHostCode: RModel::Generate emits the Session for the host cores, the way the reference does (bias
+copy + BLAS::sgemm_ for Gemm, Im2col + sgemm_ + saxpy_ per image for Conv, the Relu and pooling loops; reference
+src/SOFIE_core/inc/SOFIE/ROperator_Gemm.hxx:292-390, ROperator_Conv.hxx:302-522, ROperator_Pool.hxx:266-476,
+ROperator_Relu.hxx:54-66). The generated code is compiled with g++ and run here, without a GPU and without the kernel
+library, against the answers the reference's own tests hold for its fixtures and against the oracle."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+import models
+import replay
+from oracle import oracle
+from sofie_amd import emit
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+HOST_FIXTURES = ["Linear_16", "Linear_32", "Linear_64", "ConvWithPadding", "ConvWithoutPadding", "ConvWithAutopadSameLower",
+                 "ConvWithStridesPadding", "ConvWithStridesNoPadding", "ConvWithAsymmetricPadding", "MaxPool1d", "MaxPool2d",
+                 "MaxPool3d", "AvgPool"]
+MKL = "/opt/conda/lib/libmkl_rt.so.1"
+
+
+def run_host(spec, xs, outdir, env=None, iters=0, **generate_args):
+    """Generate the host Session of `spec` into outdir, compile its runner, run it on the inputs; returns the output."""
+    outdir = str(outdir)
+    hxx, dat, res = spec.generate(outdir, host_code=True, **generate_args)
+    text = open(hxx).read()
+    assert "sofie_hip" not in text   # host code only: no call into the kernel library
+    exe = emit.compile_host_runner(spec.name, outdir, num_inputs=len(xs))
+    names = []
+    for i, a in enumerate(xs):
+        names.append(os.path.join(outdir, "in%d.bin" % i))
+        np.ascontiguousarray(a, np.float32).tofile(names[-1])
+    fout = os.path.join(outdir, "out.bin")
+    cmd = [exe, dat, ",".join(names), fout] + ([str(iters)] if iters else [])
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300,
+                       env=dict(os.environ, **(env or {})))
+    assert r.returncode == 0, r.stderr
+    y = np.fromfile(fout, np.float32)
+    return (y, json.loads(r.stdout)) if iters else y
+
+
+def rel_err(a, b):
+    return float(np.max(np.abs(a.astype(np.float64) - b.astype(np.float64))) / max(float(np.max(np.abs(b))), 1e-30))
+
+
+@pytest.mark.parametrize("name", HOST_FIXTURES)
+def test_reference_fixture_through_host_session(name, tmp_path):
+    """The reference's fixtures through the generated host code: its expected outputs within its own tolerance, the
+    oracle's replay of the graph within 1e-5."""
+    entry = json.load(open(os.path.join(GOLD, "expected.json")))[name]
+    spec, graph = models.fixture_spec(name)
+    feeds = replay.fixture_feeds(entry, graph)
+    xs = [feeds[i[0]] for i in graph["inputs"]]
+    y = run_host(spec, xs, tmp_path)
+    want = np.array(entry["expected"], np.float32)
+    assert y.size == want.size
+    assert np.max(np.abs(y - want)) <= 1e-3
+    yo = replay.run_graph(graph, feeds, oracle)
+    assert rel_err(y, yo.reshape(-1)) <= 1e-5
+
+
+def test_mlp_and_cnn_host_sessions(tmp_path):
+    """The benchmark's fp32 networks (MLP 64-128-64-8 on 256 rows; the CNN classifier on 8 images) as host code."""
+    spec, x = models.mlp_spec()
+    y = run_host(spec, [x], tmp_path / "mlp")
+    assert rel_err(y, models.mlp_reference(oracle).reshape(-1)) <= 1e-5
+    x = models.cnn_input(8)
+    y = run_host(models.cnn_f32_spec(8), [x], tmp_path / "cnn")
+    assert rel_err(y, models.cnn_f32_stages(oracle, x)["y"].reshape(-1)) <= 1e-5
+
+
+def test_host_session_options(tmp_path):
+    """Weights as literals, a binary weight file, and a run-time batch give the same numbers as the plain host Session."""
+    spec, x = models.mlp_spec()
+    ref = models.mlp_reference(oracle).reshape(-1)
+    assert rel_err(run_host(spec, [x], tmp_path / "lit", no_weight_file=True), ref) <= 1e-5
+    assert rel_err(run_host(models.mlp_spec()[0], [x], tmp_path / "bin", binary_weight_file=True), ref) <= 1e-5
+    x8 = models.cnn_input(8)
+    y = run_host(models.cnn_f32_rt_spec(), [x8], tmp_path / "rt")      # infer(float*) runs the whole capacity
+    assert rel_err(y, models.cnn_f32_stages(oracle, x8)["y"].reshape(-1)) <= 1e-5
+
+
+def test_host_session_with_a_blas_library(tmp_path):
+    """sgemm_ / saxpy_ bound to a BLAS library at run time (SOFIE_BLAS) instead of the runner's loops."""
+    if not os.path.exists(MKL):
+        pytest.skip("no MKL in this image")
+    x = models.cnn_input(8)
+    y, timing = run_host(models.cnn_f32_spec(8), [x], tmp_path, env={"SOFIE_BLAS": MKL, "MKL_NUM_THREADS": "2"}, iters=3)
+    assert timing["blas"] == MKL and timing["host_ms"] > 0
+    assert rel_err(y, models.cnn_f32_stages(oracle, x)["y"].reshape(-1)) <= 1e-5
+
+
+@pytest.mark.parametrize("name", ["ConvTranspose2d", "Einsum_matmul"])
+def test_operators_without_a_host_form_say_so(name, tmp_path):
+    spec, _ = models.fixture_spec(name)
+    _, _, res = spec.generate(str(tmp_path), host_code=True, check=False)
+    assert res.returncode != 0 and "has no host emission" in res.stderr
