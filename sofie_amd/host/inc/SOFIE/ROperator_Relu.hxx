@@ -50,7 +50,7 @@ public:
           << "), \"Relu " << OpName << "\");\n";
       return out.str();
    }
-   // reference: ROperator_Relu.hxx:54-66 (one loop over the elements)
+   // what the loop of the reference's ROperator_Relu.hxx:54-66 computes, as one std::transform
    std::string GenerateHost(std::string OpName) override
    {
       OpName = "op_" + OpName;
@@ -58,9 +58,9 @@ public:
       if (fType != ETensorType::FLOAT) throw std::runtime_error("TMVA SOFIE Relu Op " + OpName + ": the host emission takes float tensors");
       std::stringstream out;
       out << "\n//------ RELU\n";
-      out << SP << "for (size_t id = 0; id < " << BatchCount(ConvertShapeToLength(fShape)) << " ; id++){\n";
-      out << SP << SP << "tensor_" << fNY << "[id] = ((tensor_" << fNX << "[id] > 0 )? tensor_" << fNX << "[id] : 0);\n";
-      out << SP << "}\n";
+      const std::string count = BatchCount(ConvertShapeToLength(fShape));
+      out << SP << "std::transform(tensor_" << fNX << ", tensor_" << fNX << " + " << count << ", tensor_" << fNY
+          << ", [](float v) { return v > 0 ? v : 0.0f; });\n";
       return out.str();
    }
 };
