@@ -1280,11 +1280,81 @@ __global__ void __launch_bounds__(256) k_qgemm_few_rows(GemmArgs g, int *partial
       }
 }
 
+// The same pass over B for at most 16 rows of A and enough columns to give every compute unit a workgroup without
+// cutting K across workgroups: a workgroup owns 16 columns and all of K, its eight wavefronts take an eighth of K
+// each (up to eight chunks of 64 k in flight per wavefront: with K = 4096 everything the launch reads is requested
+// before the first matrix instruction), their sums meet in LDS and the first wavefront converts and stores them. One
+// launch and no partial sums in memory; integer sums, so the result is that of every other int8 kernel bit for bit.
+template <int OUT>
+__global__ void __launch_bounds__(512) k_qgemm_few_rows_whole(GemmArgs g, int kper)
+{
+   constexpr unsigned OUTSIDE = 0x80000000u;
+   constexpr int NCH = 8;      // chunks whose loads are in flight together
+   __shared__ int red[7 * 4 * 64];
+   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+   const int j = lane & 15, kq = lane >> 4;
+   const int c0 = blockIdx.x * 16;
+   const int k_begin = wave * kper;
+   int k_end = k_begin + kper;
+   if (k_end > g.K) k_end = g.K;
+   const __amdgpu_buffer_rsrc_t ars = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t *>(g.A), 0, (int)((size_t)(g.M - 1) * g.lda + g.K), 0x00020000);
+   const __amdgpu_buffer_rsrc_t brs = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t *>(g.B), 0, (int)((size_t)(g.N - 1) * g.ldb + g.K), 0x00020000);
+   const unsigned a_off = j < g.M ? (unsigned)(j * g.lda + 16 * kq) : OUTSIDE;
+   const unsigned b_off = c0 + j < g.N ? (unsigned)((c0 + j) * g.ldb + 16 * kq) : OUTSIDE;
+   v4i acc = {0, 0, 0, 0};
+   for (int k0 = k_begin; k0 < k_end; k0 += 64 * NCH) {
+      v4i a[NCH], b[NCH];
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+         const bool in = k0 + 64 * c + 16 * kq < k_end;      // K and the wavefronts' shares are multiples of 16
+         b[c] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(brs, in ? b_off : OUTSIDE, k0 + 64 * c, 0));
+         a[c] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(ars, in ? a_off : OUTSIDE, k0 + 64 * c, 0));
+      }
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[c], b[c], acc, 0, 0, 0);
+   }
+   if (wave != 0) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[((wave - 1) * 4 + r) * 64 + lane] = acc[r];
+   }
+   __syncthreads();
+   if (wave != 0) return;
+#pragma unroll
+   for (int w = 0; w < 7; ++w)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[r] += red[(w * 4 + r) * 64 + lane];
+   // register r: row kq * 4 + r, column c0 + j
+   const int n = c0 + j;
+   if (n >= g.N) return;
+   const float sc = g.scale ? g.scale[n] : 0.0f;
+   const int bi = g.bias ? static_cast<const int *>(g.bias)[n] : 0;
+   constexpr int ESZ = OutSize<OUT>::value;
+#pragma unroll
+   for (int r = 0; r < 4; ++r) {
+      const int m = kq * 4 + r;
+      if (m >= g.M) continue;
+      const unsigned v = epilogue_value<true, OUT>(g, sc, bi, acc[r], 0.0f);
+      unsigned char *out = static_cast<unsigned char *>(g.Y) + ((size_t)m * g.ldy + n) * ESZ;
+      if constexpr (ESZ == 1) *out = (unsigned char)((int)fminf(__uint_as_float(v), 255.0f) - 128);
+      else if constexpr (ESZ == 2) *reinterpret_cast<unsigned short *>(out) = (unsigned short)v;
+      else *reinterpret_cast<unsigned *>(out) = v;
+   }
+}
+
 // Slices of K so that about eight workgroups per compute unit exist, every wavefront with at least two chunks, and the
 // partial sums a fraction of B's bytes.
 template <int OUT>
 int launch_few_rows(sofie_hip_ctx *ctx, GemmArgs &g)
 {
+   // enough columns for a workgroup of 16 columns on at least every second compute unit: one launch, K cut inside the
+   // workgroups only (8 x 4096 x 4096: see profiles/small_batch_kernels.md)
+   if (g.M <= 16 && cdiv(g.N, 16) * 2 >= ctx->num_cus) {
+      const int kper = cdiv(cdiv(g.K, 8), 64) * 64;
+      hipLaunchKernelGGL((k_qgemm_few_rows_whole<OUT>), dim3(cdiv(g.N, 16)), dim3(512), 0, ctx->stream, g, kper);
+      return check_launch(ctx, "k_qgemm_few_rows_whole");
+   }
    const int blocks = cdiv(g.N, 64);
    int splits = 8 * ctx->num_cus / blocks;
    if (splits > g.K / 512) splits = g.K / 512;

@@ -571,7 +571,9 @@ QGEMM_SHAPES = [
     (1, 1024, 1024, True), (8, 4096, 2048, True),        # a small batch on a layer of some size: a pass over B [N,K] with K
     (16, 1000, 1040, True), (17, 66, 4096, True),        # in slices (k_qgemm_few_rows): ragged columns, K no multiple of a
     (32, 2050, 528, True), (31, 640, 8208, True),        # chunk of 64 or of a slice, one and two row tiles
-]
+    (13, 2060, 1104, True), (16, 4096, 4112, True),      # ... at most 16 rows and 2048 columns or more: one launch, K cut inside
+]                                                        # the workgroups (k_qgemm_few_rows_whole): ragged columns, a last wavefront
+                                                         # with a short share of K, more than eight chunks per wavefront
 
 
 @pytest.mark.parametrize("M,N,K,transB", QGEMM_SHAPES)
@@ -619,6 +621,12 @@ def test_qgemm_s8_few_rows_kernels_and_constant_weights(ops):
     y, names = _kernels_of(ops, lambda: ops.qgemm_s8(A, Bnk, scale, bias, True, zpy=-128, relu=True))
     assert names == ["k_qgemm_few_rows", "k_splitk_finish"], names
     assert np.array_equal(y, ref)
+    # 2048 columns or more and at most 16 rows: one launch, no partial sums in memory
+    wide = r.integers(-127, 128, (4096, 1024)).astype(np.int8)
+    ws = (r.uniform(20.0, 60.0, 4096) / (73.3 * 73.3 * 32)).astype(np.float32)
+    yw, names = _kernels_of(ops, lambda: ops.qgemm_s8(A[:, :1024], wide, ws, None, True, zpy=3))
+    assert names == ["k_qgemm_few_rows_whole"], names
+    assert np.array_equal(yw, oracle.qgemm_s8(A[:, :1024], wide, ws, None, True, zpy=3))
     y, names = _kernels_of(ops, lambda: ops.qgemm_s8(A, Bkn, scale, bias, False, zpy=-128, relu=True))
     assert names == ["k_transpose_bytes", "k_gemm_bytes"], names
     assert np.array_equal(y, ref)
