@@ -98,3 +98,30 @@ def test_operators_without_a_host_form_say_so(name, tmp_path):
     spec, _ = models.fixture_spec(name)
     _, _, res = spec.generate(str(tmp_path), host_code=True, check=False)
     assert res.returncode != 0 and "has no host emission" in res.stderr
+
+
+@pytest.mark.parametrize("name", ["Linear_16", "ConvWithPadding", "MaxPool2d"])
+def test_onnx_file_to_host_session(name, tmp_path):
+    """The C++ ONNX front end with --host: the reference's fixture file straight to a host Session, same numbers as the
+    reference's expected output."""
+    emit.build_emitter()
+    entry = json.load(open(os.path.join(GOLD, "expected.json")))[name]
+    _, graph = models.fixture_spec(name)
+    feeds = replay.fixture_feeds(entry, graph)
+    xs = [feeds[i[0]] for i in graph["inputs"]]
+    out = str(tmp_path)
+    r = subprocess.run([os.path.join(emit.GEN_DIR, "emit_from_onnx"), os.path.join(GOLD, "onnx", name + ".onnx"), out, "--host"],
+                       stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    assert r.returncode == 0, r.stderr
+    assert "sofie_hip" not in open(os.path.join(out, name + ".hxx")).read()
+    exe = emit.compile_host_runner(name, out, num_inputs=len(xs))
+    names = []
+    for i, a in enumerate(xs):
+        names.append(os.path.join(out, "in%d.bin" % i))
+        np.ascontiguousarray(a, np.float32).tofile(names[-1])
+    fout = os.path.join(out, "out.bin")
+    r = subprocess.run([exe, os.path.join(out, name + ".dat"), ",".join(names), fout], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    assert r.returncode == 0, r.stderr
+    y = np.fromfile(fout, np.float32)
+    want = np.array(entry["expected"], np.float32)
+    assert y.size == want.size and np.max(np.abs(y - want)) <= 1e-3
