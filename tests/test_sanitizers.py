@@ -54,6 +54,13 @@ def test_emitters_are_clean_on_every_model(san_tools, tmp_path):
         assert res.returncode == 0, res.stderr[-2000:]
         strip = lambda path: [l for l in open(path).read().split("\n") if not l.startswith("//Code generated")]
         assert strip(hxx) == strip(hxx2)
+    # the host emission (Options::kHostCode) of the fixtures, under the sanitizers too: a model whose operators all
+    # have a host form generates, any other is refused with a message
+    for name in models.FIXTURES:
+        res = subprocess.run([onnx_exe, os.path.join(GOLD, name + ".onnx"), str(tmp_path), "--host"], stdout=subprocess.PIPE,
+                             stderr=subprocess.PIPE, text=True, env=SAN_ENV, timeout=120)
+        _clean(res)
+        assert res.returncode == 0 or "has no host emission" in res.stderr, res.stderr
 
 
 def test_onnx_parser_survives_mutated_files(san_tools, tmp_path):
