@@ -1349,7 +1349,7 @@ template <int OUT>
 int launch_few_rows(sofie_hip_ctx *ctx, GemmArgs &g)
 {
    // enough columns for a workgroup of 16 columns on at least every second compute unit: one launch, K cut inside the
-   // workgroups only (8 x 4096 x 4096: see profiles/small_batch_kernels.md)
+   // workgroups only (8 x 4096 x 4096: 5.7 against 9.3 us for the call; the second launch was a third of it)
    if (g.M <= 16 && cdiv(g.N, 16) * 2 >= ctx->num_cus) {
       const int kper = cdiv(cdiv(g.K, 8), 64) * 64;
       hipLaunchKernelGGL((k_qgemm_few_rows_whole<OUT>), dim3(cdiv(g.N, 16)), dim3(512), 0, ctx->stream, g, kper);
