@@ -716,6 +716,16 @@ def cnn_cpu_reference(images=256):
                 "sample": "256 of the 4096 images, median of 3 calls of Session::infer",
                 "what": "the float model's Session generated with Options::kHostCode (this build's emission of the "
                         "reference's CPU path: Im2col + sgemm_ + saxpy_ per image, Relu and MaxPool loops, Gemm), g++ -O2"}
+    # the int8 network itself as generated host code (the quantized operators' host form: scalar loops with int32 sums)
+    x8 = np.random.default_rng(2).uniform(0, 1, (4096, 1, 40, 40)).astype(np.float32)[:8]
+    hq = generated_host_session("qcnn", "qcnn", x8, 1, None, 3)
+    if hq:
+        res["generated_host_session_int8"] = {
+            "value": 8 / (hq["median_ms"] * 1e-3), "cores": 1, "median_ms": hq["median_ms"],
+            "sample": "the first 8 of the 4096 images, median of 3 calls of Session::infer",
+            "what": "the int8 model's Session generated with Options::kHostCode (QuantizeLinear, QLinearConv, MaxPool and "
+                    "QLinearMatMul as scalar loops), g++ -O2, one thread; its logits are the device Session's bit for bit "
+                    "(tests/test_gpu_generated.py)"}
     best = max((v["value"] for k, v in res.items() if k.endswith("_threads")), default=None)
     res["value"] = best
     res["sample"] = "%d of the 4096 images per call" % images

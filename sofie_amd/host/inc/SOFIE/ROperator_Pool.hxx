@@ -188,8 +188,18 @@ public:
       OpName = "op_" + OpName;
       if (fShapeX.empty() || fShapeY.empty())
          throw std::runtime_error("TMVA SOFIE Pool Op called to Generate without being initialized first");
-      if (fType != ETensorType::FLOAT) throw std::runtime_error("TMVA SOFIE Pool Op " + OpName + ": the host emission takes float tensors");
       const size_t dims = fShapeX.size() - 2;
+      if (fType != ETensorType::FLOAT) {
+         // int8 max pooling over two axes, on [N,C,H,W] or on the channels-last tensor of the quantized operators
+         if (fPoolMode != MaxPool || dims != 2) throw std::runtime_error("TMVA SOFIE Pool Op " + OpName + ": no host emission for this int8 pooling");
+         std::stringstream q;
+         q << "\n//----  operator MaxPool (int8)  " << OpName << "\n";
+         q << SP << "MaxPoolInt8(tensor_" << fNX << ", tensor_" << fNY << ", " << BatchCount(fShapeX[0]) << ", " << fShapeX[1] << ", " << fShapeX[2]
+           << ", " << fShapeX[3] << ", " << fAttr.kernel_shape[0] << ", " << fAttr.kernel_shape[1] << ", " << fAttr.pads[0] << ", " << fAttr.pads[1]
+           << ", " << fAttr.strides[0] << ", " << fAttr.strides[1] << ", " << fShapeY[2] << ", " << fShapeY[3] << ", "
+           << (fChannelsLast ? "true" : "false") << ");\n";
+         return q.str();
+      }
       if (fPoolMode != MaxPool && !fAttr.count_include_pad)
          for (size_t i = 0; i < 2 * dims; ++i)
             if (fAttr.pads[i] >= fAttr.kernel_shape[i % dims])

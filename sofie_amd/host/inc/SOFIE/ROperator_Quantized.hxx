@@ -115,6 +115,15 @@ public:
           << ", " << FloatLiteral(fScale) << ", " << fZp << "), \"QuantizeLinear op_" << OpName << "\");\n";
       return out.str();
    }
+   // host form: the definition, one element at a time (the division in fp32, as ONNX writes it)
+   std::string GenerateHost(std::string OpName) override
+   {
+      std::stringstream out;
+      out << "\n//------ QuantizeLinear op_" << OpName << "\n";
+      out << SP << "for (size_t id = 0; id < " << BatchCount(ConvertShapeToLength(fShape)) << "; id++)\n";
+      out << SP << SP << "tensor_" << fNY << "[id] = QuantizeOne(tensor_" << fNX << "[id], " << FloatLiteral(fScale) << ", " << fZp << ");\n";
+      return out.str();
+   }
 };
 
 // x = (q - zero_point) * scale
@@ -168,6 +177,25 @@ public:
       }
       out << SP << "Check(sofie_hip_dequantize_s8_f32(fCtx, tensor_" << src << ", tensor_" << fNY << ", " << BatchCount(ConvertShapeToLength(fShape))
           << ", " << FloatLiteral(fScale) << ", " << fZp << "), \"DequantizeLinear op_" << OpName << "\");\n";
+      return out.str();
+   }
+   // host form: a channels-last tensor is read in its own order and written as [N,C,H,W]
+   std::string GenerateHost(std::string OpName) override
+   {
+      std::stringstream out;
+      out << "\n//------ DequantizeLinear op_" << OpName << "\n";
+      if (!fNXNchw.empty()) {
+         out << SP << "for (size_t n = 0; n < " << BatchCount(fShape[0]) << "; n++)\n";
+         out << SP << SP << "for (size_t c = 0; c < " << fShape[1] << "; c++)\n";
+         out << SP << SP << SP << "for (size_t p = 0; p < " << fShape[2] * fShape[3] << "; p++)\n";
+         out << SP << SP << SP << SP << "tensor_" << fNY << "[(n * " << fShape[1] << " + c) * " << fShape[2] * fShape[3]
+             << " + p] = static_cast<float>(static_cast<int>(tensor_" << fNX << "[(n * " << fShape[2] * fShape[3] << " + p) * " << fShape[1]
+             << " + c]) - (" << fZp << ")) * " << FloatLiteral(fScale) << ";\n";
+         return out.str();
+      }
+      out << SP << "for (size_t id = 0; id < " << BatchCount(ConvertShapeToLength(fShape)) << "; id++)\n";
+      out << SP << SP << "tensor_" << fNY << "[id] = static_cast<float>(static_cast<int>(tensor_" << fNX << "[id]) - (" << fZp << ")) * "
+          << FloatLiteral(fScale) << ";\n";
       return out.str();
    }
 };
@@ -354,6 +382,33 @@ public:
           << (fHasBias ? "tensor_" + fNQBias : std::string("nullptr")) << ", " << fZpY << ", "
           << (fActivation == EActivationType::RELU ? "SOFIE_ACT_RELU" : "SOFIE_ACT_NONE") << ", tensor_" << fNY << ", " << fN << ", "
           << (fFloatOut ? "SOFIE_OUT_F32" : "SOFIE_OUT_S8") << "), \"QLinearMatMul op_" << OpName << "\");\n";
+      return out.str();
+   }
+   // host form: int32 sums over the [N,K] weights packed at generation time, then the requantisation (or, for a float
+   // output, the accumulator times the scale), one output at a time
+   std::string GenerateHost(std::string OpName) override
+   {
+      if (fShapeA.empty()) throw std::runtime_error("TMVA SOFIE QLinearMatMul Op called to Generate without being initialized first");
+      if (fHasTail) throw std::runtime_error("TMVA SOFIE QLinearMatMul Op: a pair of layers has no host emission");
+      const std::string relu = fActivation == EActivationType::RELU ? "true" : "false";
+      std::stringstream out;
+      out << "\n//--------- QLinearMatMul op_" << OpName << "\n";
+      out << SP << "for (size_t m = 0; m < " << BatchCount(fM) << "; m++) {\n";
+      out << SP << SP << "const int8_t * a = tensor_" << fNA << " + m * " << fK << ";\n";
+      out << SP << SP << "for (size_t n = 0; n < " << fN << "; n++) {\n";
+      out << SP << SP << SP << "const int8_t * b = tensor_" << fNBt << " + n * " << fK << ";\n";
+      out << SP << SP << SP << "int32_t acc = " << (fHasBias ? "tensor_" + fNQBias + "[n]" : std::string("0")) << ";\n";
+      out << SP << SP << SP << "for (size_t k = 0; k < " << fK << "; k++) acc += static_cast<int32_t>(a[k]) * static_cast<int32_t>(b[k]);\n";
+      if (fFloatOut) {
+         out << SP << SP << SP << "float v = static_cast<float>(acc) * tensor_" << fNScale << "[n];\n";
+         if (fActivation == EActivationType::RELU) out << SP << SP << SP << "if (!(v > 0)) v = 0;\n";
+         out << SP << SP << SP << "tensor_" << fNY << "[m * " << fN << " + n] = v;\n";
+      } else {
+         out << SP << SP << SP << "tensor_" << fNY << "[m * " << fN << " + n] = Requantize(acc, tensor_" << fNScale << "[n], " << fZpY << ", "
+             << relu << ");\n";
+      }
+      out << SP << SP << "}\n";
+      out << SP << "}\n";
       return out.str();
    }
 };
@@ -568,6 +623,47 @@ public:
       else
          out << ", SOFIE_OUT_S8";
       out << "), \"QLinearConv op_" << OpName << "\");\n";
+      return out.str();
+   }
+   // host form: the definition on the tensors as the generated code keeps them (input channels-last or [N,C,H,W],
+   // weights [OC][KH][KW][C/group], output channels-last): an int32 sum per output over the window, cells outside the
+   // image counting as the input zero-point (which the folded bias takes out again), then the requantisation
+   std::string GenerateHost(std::string OpName) override
+   {
+      if (fShapeX.empty()) throw std::runtime_error("TMVA SOFIE QLinearConv Op called to Generate without being initialized first");
+      if (!fChain.empty() || !fPoolKernel.empty() || !fNXFloat.empty())
+         throw std::runtime_error("TMVA SOFIE QLinearConv Op: fused layers have no host emission");
+      size_t pt, pl, pb, pr;
+      fGeom.Pads2D(pt, pl, pb, pr);
+      const size_t C = fShapeX[1], H = fShapeX[2], W = fShapeX[3], OC = fShapeW[0], Cg = fShapeW[1], KH = fShapeW[2], KW = fShapeW[3];
+      const size_t OH = fShapeY[2], OW = fShapeY[3], OCg = OC / fGeom.group;
+      std::stringstream out;
+      out << "\n//----  operator QLinearConv op_" << OpName << "\n";
+      out << SP << "for (size_t n = 0; n < " << BatchCount(fShapeX[0]) << "; n++)\n";
+      out << SP << " for (size_t oh = 0; oh < " << OH << "; oh++)\n";
+      out << SP << "  for (size_t ow = 0; ow < " << OW << "; ow++)\n";
+      out << SP << "   for (size_t oc = 0; oc < " << OC << "; oc++) {\n";
+      out << SP << SP << "const size_t c0 = (oc / " << OCg << ") * " << Cg << ";\n";
+      out << SP << SP << "int32_t acc = " << (fHasBias ? "tensor_" + fNQBias + "[oc]" : std::string("0")) << ";\n";
+      out << SP << SP << "for (size_t kh = 0; kh < " << KH << "; kh++)\n";
+      out << SP << SP << " for (size_t kw = 0; kw < " << KW << "; kw++) {\n";
+      out << SP << SP << SP << "const long ih = static_cast<long>(oh * " << fGeom.strides[0] << " + kh) - " << pt << ", iw = static_cast<long>(ow * "
+          << fGeom.strides[1] << " + kw) - " << pl << ";\n";
+      out << SP << SP << SP << "const bool inside = ih >= 0 && ih < " << H << " && iw >= 0 && iw < " << W << ";\n";
+      out << SP << SP << SP << "const int8_t * w = tensor_" << fNWPacked << " + ((oc * " << KH << " + kh) * " << KW << " + kw) * " << Cg << ";\n";
+      out << SP << SP << SP << "for (size_t ic = 0; ic < " << Cg << "; ic++) {\n";
+      if (fXChannelsLast)
+         out << SP << SP << SP << SP << "const int32_t x = inside ? tensor_" << fNX << "[((n * " << H << " + ih) * " << W << " + iw) * " << C
+             << " + c0 + ic] : " << fZpX << ";\n";
+      else
+         out << SP << SP << SP << SP << "const int32_t x = inside ? tensor_" << fNX << "[((n * " << C << " + c0 + ic) * " << H << " + ih) * " << W
+             << " + iw] : " << fZpX << ";\n";
+      out << SP << SP << SP << SP << "acc += x * static_cast<int32_t>(w[ic]);\n";
+      out << SP << SP << SP << "}\n";
+      out << SP << SP << " }\n";
+      out << SP << SP << "tensor_" << fNY << "[((n * " << OH << " + oh) * " << OW << " + ow) * " << OC << " + oc] = Requantize(acc, tensor_"
+          << fNScale << "[oc], " << fZpY << ", " << (fActivation == EActivationType::RELU ? "true" : "false") << ");\n";
+      out << SP << "   }\n";
       return out.str();
    }
 };

@@ -1113,7 +1113,7 @@ void RModel::GenerateHostHeaderInfo(std::string &hgname)
    fGC += "\n#ifndef " + hgname + "\n";
    fGC += "#define " + hgname + "\n\n";
    for (auto &i : fNeededStdLib) fGC += "#include <" + i + ">\n";
-   fGC += "#include <algorithm>\n#include <cstdint>\n#include <cstring>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n"
+   fGC += "#include <algorithm>\n#include <cmath>\n#include <cstdint>\n#include <cstring>\n#include <string>\n#include <stdexcept>\n#include <fstream>\n"
           "#include <tuple>\n#include <utility>\n#include <limits>\n";
    fGC += "\nnamespace SOFIE_" + fName + "{\n";
    // the Fortran BLAS the program is linked with, declared as the reference declares it (RModel_Base.cxx:40-58)
@@ -1140,6 +1140,44 @@ void RModel::GenerateHostHeaderInfo(std::string &hgname)
           "               }\n"
           "            }\n"
           "         }\n"
+          "}\n";
+   // The quantized operators' arithmetic, one value at a time: round half to even in fp32 (the default rounding mode),
+   // the rounded value kept inside +-1024 so that the conversion to int is defined, saturation to int8; a ReLU behind a
+   // quantized operator is a lower clamp at the output zero-point.
+   fGC += "inline int8_t Requantize(int32_t acc, float scale, int zeroPoint, bool relu) {\n"
+          "   float r = std::nearbyint(static_cast<float>(acc) * scale);\n"
+          "   r = r > 1024.f ? 1024.f : (r < -1024.f ? -1024.f : r);\n"
+          "   int q = static_cast<int>(r) + zeroPoint;\n"
+          "   const int lo = (relu && zeroPoint > -128) ? zeroPoint : -128;\n"
+          "   q = q < lo ? lo : (q > 127 ? 127 : q);\n"
+          "   return static_cast<int8_t>(q);\n"
+          "}\n";
+   fGC += "inline int8_t QuantizeOne(float x, float scale, int zeroPoint) {\n"
+          "   float r = std::nearbyint(x / scale);\n"
+          "   r = r > 1024.f ? 1024.f : (r < -1024.f ? -1024.f : r);\n"
+          "   int q = static_cast<int>(r) + zeroPoint;\n"
+          "   q = q < -128 ? -128 : (q > 127 ? 127 : q);\n"
+          "   return static_cast<int8_t>(q);\n"
+          "}\n";
+   fGC += "inline void MaxPoolInt8(const int8_t * x, int8_t * y, size_t N, size_t C, size_t H, size_t W, size_t KH, size_t KW, size_t padTop,\n"
+          "                        size_t padLeft, size_t strideH, size_t strideW, size_t OH, size_t OW, bool channelsLast) {\n"
+          "   for (size_t n = 0; n < N; ++n)\n"
+          "      for (size_t c = 0; c < C; ++c)\n"
+          "         for (size_t oh = 0; oh < OH; ++oh)\n"
+          "            for (size_t ow = 0; ow < OW; ++ow) {\n"
+          "               int best = -128;\n"
+          "               for (size_t kh = 0; kh < KH; ++kh) {\n"
+          "                  const long ih = static_cast<long>(oh * strideH + kh) - static_cast<long>(padTop);\n"
+          "                  if (ih < 0 || ih >= static_cast<long>(H)) continue;\n"
+          "                  for (size_t kw = 0; kw < KW; ++kw) {\n"
+          "                     const long iw = static_cast<long>(ow * strideW + kw) - static_cast<long>(padLeft);\n"
+          "                     if (iw < 0 || iw >= static_cast<long>(W)) continue;\n"
+          "                     const int v = channelsLast ? x[((n * H + ih) * W + iw) * C + c] : x[((n * C + c) * H + ih) * W + iw];\n"
+          "                     if (v > best) best = v;\n"
+          "                  }\n"
+          "               }\n"
+          "               y[channelsLast ? ((n * OH + oh) * OW + ow) * C + c : ((n * C + c) * OH + oh) * OW + ow] = static_cast<int8_t>(best);\n"
+          "            }\n"
           "}\n";
    // Pooling over three axes (leading axes of extent 1 for fewer): maximum, or mean, of the window's cells inside the image.
    fGC += "inline void Pool3d(bool isMax, bool countIncludePad, const float * x, float * y, size_t planes, const int * in, const int * out,\n"
@@ -1231,8 +1269,6 @@ void RModel::GenerateHostSessionCode()
    } else {
       for (auto &i : fInitializedTensors) {
          if (!i.second.IsWeightTensor()) continue;
-         if (i.second.type() != ETensorType::FLOAT && i.second.type() != ETensorType::INT64)
-            throw std::runtime_error("tmva-sofie tensor_" + i.first + " cannot be written as a literal by the host emission");
          const size_t length = ConvertShapeToLength(i.second.shape());
          std::stringstream lit;
          lit << "   { static const " << ConvertTypeToString(i.second.type()) << " host[" << (length ? length : 1) << "] = {";
@@ -1247,7 +1283,13 @@ void RModel::GenerateHostSessionCode()
                if (text.find_first_of(".e") == std::string::npos) text += ".";
                lit << text << "f";
             } else {
-               lit << i.second.data<int64_t>()[idx];
+               switch (i.second.type()) {
+               case ETensorType::INT8: lit << (int)i.second.data<int8_t>()[idx]; break;
+               case ETensorType::UINT8: lit << (int)i.second.data<uint8_t>()[idx]; break;
+               case ETensorType::INT32: lit << i.second.data<int32_t>()[idx]; break;
+               case ETensorType::INT64: lit << i.second.data<int64_t>()[idx]; break;
+               default: throw std::runtime_error("tmva-sofie tensor_" + i.first + " cannot be written as a literal");
+               }
             }
          }
          lit << "};\n     std::copy(host, host + " << length << ", tensor_" << i.first << "); }\n";
@@ -1280,7 +1322,10 @@ void RModel::GenerateHostSessionCode()
       return (fRuntimeBatch && fBatchTensors.count(n)) ? "fBatch * " + std::to_string(len / fBatchCapacity) : std::to_string(len);
    };
    auto body = [&]() {
-      for (size_t id = 0; id < fOperators.size(); id++) fGC += fOperators[id]->GenerateHost(std::to_string(id));
+      for (size_t id = 0; id < fOperators.size(); id++) {
+         if (fOperators[id]->IsFusedAway() || fOperators[id]->IsAbsorbed()) continue;
+         fGC += fOperators[id]->GenerateHost(std::to_string(id));
+      }
       if (nout == 1) {
          fGC += "   return std::vector<" + otype + ">(tensor_" + out + ", tensor_" + out + " + " + outputCount(out) + ");\n";
          return;
@@ -1337,8 +1382,10 @@ void RModel::Generate(std::underlying_type_t<Options> options, int batchSize, lo
    fHostCode = (static_cast<std::underlying_type_t<Options>>(Options::kHostCode) & options) != 0;
    Initialize(batchSize, verbose);
    if (fHostCode) {
-      // every operator emits its own statements, as in the reference: no fusion pass runs (an activation the
-      // parser already attached to a Gemm or Conv is that operator's loop)
+      // every operator emits its own statements, as in the reference. Of the fusion passes only the one that hands a
+      // Relu to the operator in front of it runs: the operator then ends in the ReLU loop (Gemm, Conv) or, for a
+      // quantized operator, clamps at its output zero-point, which a Relu operator on its own does not know
+      FuseActivations();
       PlanIntermediateMemory();
       fGC.clear();
       std::string hostGuard;

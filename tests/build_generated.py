@@ -61,7 +61,7 @@ def main():
     # emissions on a GPU box and for the benchmark's CPU baseline: sofie_amd/generated/host/run_host_<name>. They
     # read the weight files written above.
     host_dir = os.path.join(emit.GEN_DIR, "host")
-    for spec in (models.mlp_spec()[0], models.cnn_f32_spec(8), models.cnn_f32_spec(256, "cnn_f32_b256")):
+    for spec in (models.mlp_spec()[0], models.cnn_f32_spec(8), models.cnn_f32_spec(256, "cnn_f32_b256"), models.qcnn_spec(oracle, 8)):
         _, dat, res = spec.generate(host_dir, host_code=True)
         emit.compile_host_runner(spec.name, host_dir)
         os.remove(dat)

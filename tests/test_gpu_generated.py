@@ -89,10 +89,12 @@ def test_cnn_f32_session(tmp_path):
     assert rel_err(y, ref.reshape(-1)) <= 1e-5
 
 
-@pytest.mark.parametrize("name,weights", [("mlp_c1", "mlp_c1"), ("cnn_f32", "cnn_f32")])
+@pytest.mark.parametrize("name,weights", [("mlp_c1", "mlp_c1"), ("cnn_f32", "cnn_f32"), ("qcnn", "qcnn")])
 def test_host_and_device_emission_agree(name, weights, tmp_path):
     """The same model generated twice, as calls into the kernel library and as code for the host cores
-    (Options::kHostCode: the reference's BLAS calls and loops), on the same seeded input: within 1e-5 relative."""
+    (Options::kHostCode: the reference's BLAS calls and loops; for the quantized operators, which the reference does
+    not have, loops with int32 sums and the same rounding rule), on the same seeded input: within 1e-5 relative for the
+    float networks, bit for bit for the int8 network."""
     x = models.mlp_spec()[1] if name == "mlp_c1" else models.cnn_input(8)
     y_device = run_session(name, x, tmp_path)
     exe = os.path.join(emit.GEN_DIR, "host", "run_host_" + name)
@@ -104,7 +106,10 @@ def test_host_and_device_emission_agree(name, weights, tmp_path):
     assert res.returncode == 0, res.stderr
     y_host = np.fromfile(fout, np.float32)
     assert y_host.size == y_device.size
-    assert rel_err(y_device, y_host) <= 1e-5
+    if name == "qcnn":
+        assert np.array_equal(y_device, y_host)
+    else:
+        assert rel_err(y_device, y_host) <= 1e-5
 
 
 def test_runtime_batch_sessions(tmp_path):

@@ -72,6 +72,22 @@ def test_mlp_and_cnn_host_sessions(tmp_path):
     assert rel_err(y, models.cnn_f32_stages(oracle, x)["y"].reshape(-1)) <= 1e-5
 
 
+def test_quantized_models_as_host_code_are_bit_exact(tmp_path):
+    """The quantized operators have a host form as well (the reference has no quantized operators: the generated CPU
+    code of an int8 model is this emission): QuantizeLinear, QLinearConv with a ReLU behind it, int8 MaxPool, Flatten,
+    QLinearMatMul with int8 and with float output, DequantizeLinear of a channels-last tensor. Integer sums and one
+    rounding rule: the int8 CNN's logits and the dequantised convolution equal the oracle's bit for bit."""
+    x = models.cnn_input(8)
+    y = run_host(models.qcnn_spec(oracle, 8), [x], tmp_path / "qcnn")
+    assert np.array_equal(y, models.qcnn_reference(oracle, x).reshape(-1))
+    p = models.qdq_conv_params()
+    y = run_host(models.qdq_conv_spec(), [p["x"]], tmp_path / "qdq")
+    assert np.array_equal(y, models.qdq_conv_reference(oracle).reshape(-1))
+    # weights as literals (int8, int32 and float tensors in the header)
+    y = run_host(models.qdq_conv_spec(), [p["x"]], tmp_path / "qdq_lit", no_weight_file=True)
+    assert np.array_equal(y, models.qdq_conv_reference(oracle).reshape(-1))
+
+
 def test_host_session_options(tmp_path):
     """Weights as literals, a binary weight file, and a run-time batch give the same numbers as the plain host Session."""
     spec, x = models.mlp_spec()
