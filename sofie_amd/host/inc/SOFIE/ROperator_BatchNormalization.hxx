@@ -130,6 +130,30 @@ public:
           << "\");\n";
       return out.str();
    }
+
+   // host form: the loop of the reference (ROperator_BatchNormalization.hxx Generate: x - mean, times the folded scale,
+   // plus the bias, then the ReLU), one rounding per step
+   std::string GenerateHost(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShapeX.empty())
+         throw std::runtime_error("TMVA SOFIE Batch Normalization called to Generate without being initialized first");
+      size_t plane = 1;
+      for (size_t i = 2; i < fShapeX.size(); ++i) plane *= fShapeX[i];
+      std::stringstream out;
+      out << "\n\n//---- BatchNorm " << OpName << "\n";
+      out << SP << "for (size_t n = 0; n < " << BatchCount(fShapeX[0]) << "; n++)\n";
+      out << SP << SP << "for (size_t c = 0; c < " << fShapeX[1] << "; c++)\n";
+      out << SP << SP << SP << "for (size_t i = 0; i < " << plane << "; i++) {\n";
+      out << SP << SP << SP << SP << "const size_t id = (n * " << fShapeX[1] << " + c) * " << plane << " + i;\n";
+      out << SP << SP << SP << SP << "float v = tensor_" << fNX << "[id] - tensor_" << fNMean << "[c];\n";
+      out << SP << SP << SP << SP << "v = v * tensor_" << fNFolded << "[c];\n";
+      out << SP << SP << SP << SP << "v = v + tensor_" << fNB << "[c];\n";
+      if (fActivation == EActivationType::RELU) out << SP << SP << SP << SP << "v = v > 0 ? v : 0;\n";
+      out << SP << SP << SP << SP << "tensor_" << fNY << "[id] = v;\n";
+      out << SP << SP << SP << "}\n";
+      return out.str();
+   }
 };
 
 }   // namespace SOFIE

@@ -246,12 +246,12 @@ public:
    // as a column-major [OH*OW, C/g*KH*KW] matrix (Im2col), one BLAS::sgemm_ multiplies it with the group's filters
    // (the [OC/g, C/g*KH*KW] rows of the weight tensor are that matrix's column-major transpose already), and the
    // bias, broadcast to [OC,OH,OW] once in the constructor, is added with BLAS::saxpy_; then the ReLU loop. The
-   // geometry is this emitter's (ONNX pads and dilations, see the head of the file), through the same Im2col.
+   // geometry is this emitter's (ONNX pads and dilations, see the head of the file), through one Im2col for one, two
+   // or three spatial axes (the reference's Im2col and Im2col_3d).
    std::string GenerateHostSessionMembersCode(std::string OpName) override
    {
       OpName = "op_" + OpName;
       if (fShapeY.empty()) throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
-      if (fGeom.dim == 3) throw std::runtime_error("TMVA SOFIE Conv Op: three spatial dimensions have no host emission");
       size_t spatialOut = 1, kernelCells = 1;
       for (size_t i = 0; i < fGeom.dim; ++i) { spatialOut *= fShapeY[2 + i]; kernelCells *= fShapeW[2 + i]; }
       std::stringstream out;
@@ -276,44 +276,47 @@ public:
       if (fShapeX.empty() || fShapeW.empty() || (fNB != "" && fShapeB.empty()) || fShapeY.empty())
          throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
       const size_t dim = fGeom.dim;
-      if (dim == 3) throw std::runtime_error("TMVA SOFIE Conv Op: three spatial dimensions have no host emission");
-      const bool oneD = dim == 1;
-      const size_t H = oneD ? 1 : fShapeX[2], W = fShapeX[dim + 1];
-      const size_t KH = oneD ? 1 : fShapeW[2], KW = fShapeW[dim + 1];
-      const size_t OH = oneD ? 1 : fShapeY[2], OW = fShapeY[dim + 1];
-      const std::vector<size_t> &p = fGeom.pads;
-      const size_t pt = oneD ? 0 : p[0], pl = p[dim - 1];
-      const size_t sh = oneD ? 1 : fGeom.strides[0], sw = fGeom.strides[dim - 1];
-      const size_t dh = oneD ? 1 : fGeom.dilations[0], dw = fGeom.dilations[dim - 1];
+      // three spatial axes, the given ones last (missing leading axes have extent 1, no padding, unit stride)
+      size_t in[3] = {1, 1, 1}, ker[3] = {1, 1, 1}, o[3] = {1, 1, 1}, pad[3] = {0, 0, 0}, st[3] = {1, 1, 1}, dil[3] = {1, 1, 1};
+      for (size_t i = 0; i < dim; ++i) {
+         const size_t a = 3 - dim + i;
+         in[a] = fShapeX[2 + i]; ker[a] = fShapeW[2 + i]; o[a] = fShapeY[2 + i]; pad[a] = fGeom.pads[i]; st[a] = fGeom.strides[i];
+         dil[a] = fGeom.dilations[i];
+      }
+      const size_t inSize = in[0] * in[1] * in[2], kerSize = ker[0] * ker[1] * ker[2], outSize = o[0] * o[1] * o[2];
       const size_t C = fShapeX[1], OC = fShapeW[0], G = fGeom.group, Cg = fShapeW[1], OCg = OC / G;
+      auto list = [](const size_t (&v)[3]) { return "{" + std::to_string(v[0]) + ", " + std::to_string(v[1]) + ", " + std::to_string(v[2]) + "}"; };
       std::stringstream out;
       out << "\n//----  operator Conv " << OpName << "\n";
       out << SP << "{\n";
       out << SP << SP << "char " << OpName << "_transA = 'N';\n";
       out << SP << SP << "char " << OpName << "_transB = 'N';\n";
-      out << SP << SP << "int " << OpName << "_m = " << OH * OW << ";\n";
+      out << SP << SP << "int " << OpName << "_m = " << outSize << ";\n";
       out << SP << SP << "int " << OpName << "_n = " << OCg << ";\n";
-      out << SP << SP << "int " << OpName << "_k = " << Cg * KH * KW << ";\n";
+      out << SP << SP << "int " << OpName << "_k = " << Cg * kerSize << ";\n";
       out << SP << SP << "float " << OpName << "_alpha = 1.0;\n";
       out << SP << SP << "float " << OpName << "_beta = 0.0;\n";
       out << SP << SP << "float * " << OpName << "_xcol = fVec_" << OpName << "_xcol.data();\n";
+      out << SP << SP << "const int " << OpName << "_in[3] = " << list(in) << ", " << OpName << "_kernel[3] = " << list(ker) << ", " << OpName
+          << "_pads[3] = " << list(pad) << ", " << OpName << "_strides[3] = " << list(st) << ", " << OpName << "_dilations[3] = " << list(dil)
+          << ", " << OpName << "_out[3] = " << list(o) << ";\n";
       out << SP << SP << "for (size_t n = 0; n < " << BatchCount(fShapeX[0]) << "; n++) {\n";
       out << SP << SP << SP << "for (size_t g = 0; g < " << G << "; g++) {\n";
-      out << SP << SP << SP << SP << "Im2col(tensor_" << fNX << " + (n * " << C << " + g * " << Cg << ") * " << H * W << ", " << Cg << ", " << H
-          << ", " << W << ", " << KH << ", " << KW << ", " << pt << ", " << pl << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << OH
-          << ", " << OW << ", " << OpName << "_xcol);\n";
+      out << SP << SP << SP << SP << "Im2col(tensor_" << fNX << " + (n * " << C << " + g * " << Cg << ") * " << inSize << ", " << Cg << ", " << OpName
+          << "_in, " << OpName << "_kernel, " << OpName << "_pads, " << OpName << "_strides, " << OpName << "_dilations, " << OpName << "_out, "
+          << OpName << "_xcol);\n";
       out << SP << SP << SP << SP << "BLAS::sgemm_(&" << OpName << "_transA, &" << OpName << "_transB, &" << OpName << "_m, &" << OpName
           << "_n, &" << OpName << "_k, &" << OpName << "_alpha, " << OpName << "_xcol, &" << OpName << "_m, tensor_" << fNW << " + g * "
-          << OCg * Cg * KH * KW << ", &" << OpName << "_k, &" << OpName << "_beta, tensor_" << fNY << " + (n * " << OC << " + g * " << OCg
-          << ") * " << OH * OW << ", &" << OpName << "_m);\n";
+          << OCg * Cg * kerSize << ", &" << OpName << "_k, &" << OpName << "_beta, tensor_" << fNY << " + (n * " << OC << " + g * " << OCg
+          << ") * " << outSize << ", &" << OpName << "_m);\n";
       out << SP << SP << SP << "}\n";
       if (fNB != "") {
-         out << SP << SP << SP << "int " << OpName << "_size = " << OC * OH * OW << ";\n";
+         out << SP << SP << SP << "int " << OpName << "_size = " << OC * outSize << ";\n";
          out << SP << SP << SP << "float " << OpName << "_gamma = 1.0;\n";
          out << SP << SP << SP << "int " << OpName << "_incx = 1;\n";
          out << SP << SP << SP << "int " << OpName << "_incy = 1;\n";
          out << SP << SP << SP << "BLAS::saxpy_(&" << OpName << "_size, &" << OpName << "_gamma, fVec_" << OpName << "_bias.data(), &" << OpName
-             << "_incx, tensor_" << fNY << " + n * " << OC * OH * OW << ", &" << OpName << "_incy);\n";
+             << "_incx, tensor_" << fNY << " + n * " << OC * outSize << ", &" << OpName << "_incy);\n";
       }
       out << SP << SP << "}\n";
       if (fActivation == EActivationType::RELU) {

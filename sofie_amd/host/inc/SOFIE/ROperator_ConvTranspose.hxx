@@ -149,6 +149,68 @@ public:
           << "\");\n";
       return out.str();
    }
+
+   // Host form, the reference's sequence for the transposed convolution (ROperator_ConvTranspose.icc:364-474 computes
+   // it as a convolution of the zero-stuffed input with the flipped kernel; here the equivalent product-then-scatter):
+   // per image and group one BLAS::sgemm_ multiplies the [H*W, C/g] input with the group's [C/g, OC/g*KH*KW] weights,
+   // and every column of the result is added into the output at the positions its kernel cell reaches (stride,
+   // dilation, begin pads); the bias and the ReLU follow.
+   std::string GenerateHostSessionMembersCode(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShapeY.empty()) throw std::runtime_error("TMVA SOFIE ConvTranspose Op called to Generate without being initialized first");
+      size_t in = 1, cells = 1;
+      for (size_t i = 0; i < fDim; ++i) { in *= fShapeX[2 + i]; cells *= fShapeW[2 + i]; }
+      return "std::vector<float> fVec_" + OpName + "_col = std::vector<float>(" + std::to_string(fShapeW[1] * cells * in) + ");\n";
+   }
+   std::string GenerateHost(std::string OpName) override
+   {
+      OpName = "op_" + OpName;
+      if (fShapeX.empty() || fShapeW.empty() || (fNB != "" && fShapeB.empty()) || fShapeY.empty())
+         throw std::runtime_error("TMVA SOFIE Conv Op called to Generate without being initialized first");
+      const bool oneD = fDim == 1;
+      const size_t H = oneD ? 1 : fShapeX[2], W = fShapeX[fDim + 1];
+      const size_t KH = oneD ? 1 : fShapeW[2], KW = fShapeW[fDim + 1];
+      const size_t OH = oneD ? 1 : fShapeY[2], OW = fShapeY[fDim + 1];
+      const size_t ph = oneD ? 0 : fAttrPads[0], pw = fAttrPads[oneD ? 0 : 1];
+      const size_t sh = oneD ? 1 : fAttrStrides[0], sw = fAttrStrides[oneD ? 0 : 1];
+      const size_t dh = oneD ? 1 : fAttrDilations[0], dw = fAttrDilations[oneD ? 0 : 1];
+      const size_t C = fShapeX[1], OC = fShapeY[1], G = fAttrGroup, Cg = C / G, OCg = OC / G;
+      std::stringstream out;
+      out << "\n//----  operator ConvTranspose " << OpName << "\n";
+      out << SP << "{\n";
+      out << SP << SP << "char " << OpName << "_transA = 'N';\n";
+      out << SP << SP << "char " << OpName << "_transB = 'T';\n";
+      out << SP << SP << "int " << OpName << "_m = " << H * W << ";\n";
+      out << SP << SP << "int " << OpName << "_n = " << OCg * KH * KW << ";\n";
+      out << SP << SP << "int " << OpName << "_k = " << Cg << ";\n";
+      out << SP << SP << "float " << OpName << "_alpha = 1.0;\n";
+      out << SP << SP << "float " << OpName << "_beta = 0.0;\n";
+      out << SP << SP << "float * " << OpName << "_col = fVec_" << OpName << "_col.data();\n";
+      out << SP << SP << "std::fill_n(tensor_" << fNY << ", " << BatchCount(ConvertShapeToLength(fShapeY)) << ", 0.f);\n";
+      out << SP << SP << "for (size_t n = 0; n < " << BatchCount(fShapeX[0]) << "; n++) {\n";
+      out << SP << SP << SP << "for (size_t g = 0; g < " << G << "; g++) {\n";
+      out << SP << SP << SP << SP << "BLAS::sgemm_(&" << OpName << "_transA, &" << OpName << "_transB, &" << OpName << "_m, &" << OpName
+          << "_n, &" << OpName << "_k, &" << OpName << "_alpha, tensor_" << fNX << " + (n * " << C << " + g * " << Cg << ") * " << H * W << ", &"
+          << OpName << "_m, tensor_" << fNW << " + g * " << Cg * OCg * KH * KW << ", &" << OpName << "_n, &" << OpName << "_beta, " << OpName
+          << "_col, &" << OpName << "_m);\n";
+      out << SP << SP << SP << SP << "Col2im(" << OpName << "_col, " << OCg << ", " << H << ", " << W << ", " << KH << ", " << KW << ", " << ph << ", "
+          << pw << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", " << OH << ", " << OW << ", tensor_" << fNY << " + (n * " << OC
+          << " + g * " << OCg << ") * " << OH * OW << ");\n";
+      out << SP << SP << SP << "}\n";
+      out << SP << SP << "}\n";
+      if (fNB != "" || fActivation == EActivationType::RELU) {
+         out << SP << SP << "for (size_t id = 0; id < " << BatchCount(ConvertShapeToLength(fShapeY)) << "; id++) {\n";
+         out << SP << SP << SP << "float v = tensor_" << fNY << "[id]";
+         if (fNB != "") out << " + tensor_" << fNB << "[(id / " << OH * OW << ") % " << OC << "]";
+         out << ";\n";
+         if (fActivation == EActivationType::RELU) out << SP << SP << SP << "v = v > 0 ? v : 0;\n";
+         out << SP << SP << SP << "tensor_" << fNY << "[id] = v;\n";
+         out << SP << SP << "}\n";
+      }
+      out << SP << "}\n";
+      return out.str();
+   }
 };
 
 }   // namespace SOFIE

@@ -283,6 +283,83 @@ public:
       out << SP << "}\n";
       return out.str();
    }
+
+   // Host form (reference ROperator_Einsum.hxx Generate): a product of two operands whose labels make it a (stacked)
+   // matrix product is one BLAS::sgemm_ per stacked matrix; every other equation is the nest of loops over the output
+   // labels and, inside, over the summed labels, written once as a helper that walks the labels like an odometer.
+   std::string GenerateHost(std::string opName) override
+   {
+      opName = "op_" + opName;
+      if (!fInitialized || fShapeY.size() != fOutputLabels.length())
+         throw std::runtime_error("TMVA SOFIE Einsum Op called to Generate without being initialized first");
+      std::stringstream out;
+      out << "\n//-------- Einsum   \n";
+      out << SP << "{\n";
+      if (!fGemmType.empty()) {
+         const auto &sa = fShapeInputs[0], &sb = fShapeInputs[1];
+         const bool ta = fGemmType[0] == 't', tb = fGemmType[1] == 't';
+         const size_t m = ta ? sa.back() : sa[sa.size() - 2];
+         const size_t k = ta ? sa[sa.size() - 2] : sa.back();
+         const size_t n = tb ? sb[sb.size() - 2] : sb.back();
+         const std::string lead = fOutputLabels.substr(0, fOutputLabels.size() - 2);
+         const auto stA = LabelStrides(lead, fInputLabels[0].substr(0, fInputLabels[0].size() - 2),
+                                       std::vector<size_t>(sa.begin(), sa.end() - 2));
+         const auto stB = LabelStrides(lead, fInputLabels[1].substr(0, fInputLabels[1].size() - 2),
+                                       std::vector<size_t>(sb.begin(), sb.end() - 2));
+         size_t stack = 1;
+         for (size_t i = 0; i + 2 < fShapeY.size(); ++i) stack *= fShapeY[i];
+         out << SP << SP << "static const size_t " << opName << "_a[] = {";
+         for (size_t idx = 0; idx < stack; ++idx) {
+            size_t rem = idx, oa = 0;
+            for (size_t i = lead.size(); i-- > 0;) {
+               oa += (rem % fShapeY[i]) * (size_t)stA[i] * sa[sa.size() - 2] * sa.back();
+               rem /= fShapeY[i];
+            }
+            out << (idx ? ", " : "") << oa;
+         }
+         out << "};\n";
+         out << SP << SP << "static const size_t " << opName << "_b[] = {";
+         for (size_t idx = 0; idx < stack; ++idx) {
+            size_t rem = idx, ob = 0;
+            for (size_t i = lead.size(); i-- > 0;) {
+               ob += (rem % fShapeY[i]) * (size_t)stB[i] * sb[sb.size() - 2] * sb.back();
+               rem /= fShapeY[i];
+            }
+            out << (idx ? ", " : "") << ob;
+         }
+         out << "};\n";
+         out << SP << SP << "char " << opName << "_transA = '" << (ta ? "t" : "n") << "', " << opName << "_transB = '" << (tb ? "t" : "n") << "';\n";
+         out << SP << SP << "int " << opName << "_m = " << m << ", " << opName << "_n = " << n << ", " << opName << "_k = " << k << ", " << opName
+             << "_lda = " << sa.back() << ", " << opName << "_ldb = " << sb.back() << ";\n";
+         out << SP << SP << "float " << opName << "_alpha = 1.0, " << opName << "_beta = 0.0;\n";
+         out << SP << SP << "for (size_t i = 0; i < " << stack << "; i++)\n";
+         out << SP << SP << SP << "BLAS::sgemm_(&" << opName << "_transB, &" << opName << "_transA, &" << opName << "_n, &" << opName << "_m, &"
+             << opName << "_k, &" << opName << "_alpha, tensor_" << fNInputs[1] << " + " << opName << "_b[i], &" << opName << "_ldb, tensor_"
+             << fNInputs[0] << " + " << opName << "_a[i], &" << opName << "_lda, &" << opName << "_beta, tensor_" << fNY << " + i * " << m * n
+             << ", &" << opName << "_n);\n";
+         out << SP << "}\n";
+         return out.str();
+      }
+      const std::string all = fOutputLabels + fSumLabels;
+      out << SP << SP << "static const int " << opName << "_extent[] = {";
+      for (size_t l = 0; l < all.size(); ++l) out << (l ? ", " : "") << fExtent.at(all[l]);
+      out << (all.empty() ? "1" : "") << "};\n";
+      out << SP << SP << "static const long long " << opName << "_stride[] = {";
+      bool first = true;
+      for (size_t i = 0; i < fNInputs.size(); ++i)
+         for (long long s : LabelStrides(all, fInputLabels[i], fShapeInputs[i])) {
+            out << (first ? "" : ", ") << s;
+            first = false;
+         }
+      out << (first ? "0" : "") << "};\n";
+      out << SP << SP << "const float * " << opName << "_x[] = {";
+      for (size_t i = 0; i < fNInputs.size(); ++i) out << (i ? ", " : "") << "tensor_" << fNInputs[i];
+      out << "};\n";
+      out << SP << SP << "EinsumLoops(" << fNInputs.size() << ", " << opName << "_x, " << all.size() << ", " << fOutputLabels.size() << ", "
+          << opName << "_extent, " << opName << "_stride, tensor_" << fNY << ");\n";
+      out << SP << "}\n";
+      return out.str();
+   }
 };
 
 }   // namespace SOFIE

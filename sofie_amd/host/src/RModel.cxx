@@ -1123,23 +1123,74 @@ void RModel::GenerateHostHeaderInfo(std::string &hgname)
           "                          const float * beta, float * C, const int * ldc);\n";
    fGC += "   extern \"C\" void saxpy_(const int * n, const float * alpha, const float * x, const int * incx, float * y, const int * incy);\n";
    fGC += "}//BLAS\n";
-   // Patches of one image (or one group's channels of it) as a column-major [OH*OW, C*KH*KW] matrix: column
-   // (c*KH + kh)*KW + kw holds, for every output position, the input cell under kernel cell (kh, kw) of channel c,
-   // zero outside the image (the role of UTILITY::Im2col, SOFIE_common.hxx:485-518 of the reference).
-   fGC += "inline void Im2col(const float * x, int C, int H, int W, int KH, int KW, int padTop, int padLeft, int strideH, int strideW,\n"
-          "                   int dilationH, int dilationW, int OH, int OW, float * xcol) {\n"
+   // Patches of one image (or one group's channels of it) as a column-major [output positions, C * kernel cells]
+   // matrix over three spatial axes (extent 1 for missing leading ones): a column holds, for every output position,
+   // the input cell under one kernel cell of one channel, zero outside the image (the role of UTILITY::Im2col and
+   // Im2col_3d of the reference, SOFIE_common.hxx:485-518).
+   fGC += "inline void Im2col(const float * x, int C, const int * in, const int * kernel, const int * pads, const int * strides,\n"
+          "                   const int * dilations, const int * out, float * xcol) {\n"
+          "   const size_t outSize = static_cast<size_t>(out[0]) * out[1] * out[2];\n"
+          "   size_t column = 0;\n"
           "   for (int c = 0; c < C; ++c)\n"
+          "      for (int kd = 0; kd < kernel[0]; ++kd)\n"
+          "         for (int kh = 0; kh < kernel[1]; ++kh)\n"
+          "            for (int kw = 0; kw < kernel[2]; ++kw, ++column) {\n"
+          "               float * col = xcol + column * outSize;\n"
+          "               for (int od = 0; od < out[0]; ++od) {\n"
+          "                  const int id = od * strides[0] - pads[0] + kd * dilations[0];\n"
+          "                  for (int oh = 0; oh < out[1]; ++oh) {\n"
+          "                     const int ih = oh * strides[1] - pads[1] + kh * dilations[1];\n"
+          "                     for (int ow = 0; ow < out[2]; ++ow) {\n"
+          "                        const int iw = ow * strides[2] - pads[2] + kw * dilations[2];\n"
+          "                        const bool inside = id >= 0 && id < in[0] && ih >= 0 && ih < in[1] && iw >= 0 && iw < in[2];\n"
+          "                        *col++ = inside ? x[((static_cast<size_t>(c) * in[0] + id) * in[1] + ih) * in[2] + iw] : 0.f;\n"
+          "                     }\n"
+          "                  }\n"
+          "               }\n"
+          "            }\n"
+          "}\n";
+   // The other way round, for the transposed convolution: column (oc*KH + kh)*KW + kw of a column-major
+   // [H*W, OC*KH*KW] matrix is added into channel oc of the output at the positions kernel cell (kh, kw) reaches.
+   fGC += "inline void Col2im(const float * col, int OC, int H, int W, int KH, int KW, int padTop, int padLeft, int strideH, int strideW,\n"
+          "                   int dilationH, int dilationW, int OH, int OW, float * y) {\n"
+          "   for (int oc = 0; oc < OC; ++oc)\n"
           "      for (int kh = 0; kh < KH; ++kh)\n"
           "         for (int kw = 0; kw < KW; ++kw) {\n"
-          "            float * col = xcol + (static_cast<size_t>(c * KH + kh) * KW + kw) * OH * OW;\n"
-          "            for (int oh = 0; oh < OH; ++oh) {\n"
-          "               const int ih = oh * strideH - padTop + kh * dilationH;\n"
-          "               for (int ow = 0; ow < OW; ++ow) {\n"
-          "                  const int iw = ow * strideW - padLeft + kw * dilationW;\n"
-          "                  col[oh * OW + ow] = (ih >= 0 && ih < H && iw >= 0 && iw < W) ? x[(static_cast<size_t>(c) * H + ih) * W + iw] : 0.f;\n"
+          "            const float * c = col + (static_cast<size_t>(oc * KH + kh) * KW + kw) * H * W;\n"
+          "            for (int ih = 0; ih < H; ++ih) {\n"
+          "               const int oh = ih * strideH - padTop + kh * dilationH;\n"
+          "               if (oh < 0 || oh >= OH) continue;\n"
+          "               for (int iw = 0; iw < W; ++iw) {\n"
+          "                  const int ow = iw * strideW - padLeft + kw * dilationW;\n"
+          "                  if (ow >= 0 && ow < OW) y[(static_cast<size_t>(oc) * OH + oh) * OW + ow] += c[ih * W + iw];\n"
           "               }\n"
           "            }\n"
           "         }\n"
+          "}\n";
+   // Einsum as loops: labels 0 .. nOut-1 index the output (row-major), the others are summed, innermost last;
+   // stride[i*nLabels + l] is operand i's element stride along label l (0 where the operand lacks it).
+   fGC += "inline void EinsumLoops(int nInputs, const float * const * x, int nLabels, int nOut, const int * extent, const long long * stride,\n"
+          "                        float * y) {\n"
+          "   std::vector<int> pos(nLabels > 0 ? nLabels : 1, 0);\n"
+          "   size_t outputs = 1, terms = 1;\n"
+          "   for (int l = 0; l < nOut; ++l) outputs *= extent[l];\n"
+          "   for (int l = nOut; l < nLabels; ++l) terms *= extent[l];\n"
+          "   for (size_t o = 0; o < outputs; ++o) {\n"
+          "      float sum = 0.f;\n"
+          "      for (int l = nOut; l < nLabels; ++l) pos[l] = 0;\n"
+          "      for (size_t t = 0; t < terms; ++t) {\n"
+          "         float product = 1.f;\n"
+          "         for (int i = 0; i < nInputs; ++i) {\n"
+          "            long long at = 0;\n"
+          "            for (int l = 0; l < nLabels; ++l) at += pos[l] * stride[i * nLabels + l];\n"
+          "            product *= x[i][at];\n"
+          "         }\n"
+          "         sum += product;\n"
+          "         for (int l = nLabels - 1; l >= nOut; --l) { if (++pos[l] < extent[l]) break; pos[l] = 0; }\n"
+          "      }\n"
+          "      y[o] = sum;\n"
+          "      for (int l = nOut - 1; l >= 0; --l) { if (++pos[l] < extent[l]) break; pos[l] = 0; }\n"
+          "   }\n"
           "}\n";
    // The quantized operators' arithmetic, one value at a time: round half to even in fp32 (the default rounding mode),
    // the rounded value kept inside +-1024 so that the conversion to int is defined, saturation to int8; a ReLU behind a
@@ -1267,6 +1318,7 @@ void RModel::GenerateHostSessionCode()
       }
       fGC += "   f.close();\n";
    } else {
+      fGC += "   (void)filename;   // no weight file is read\n";
       for (auto &i : fInitializedTensors) {
          if (!i.second.IsWeightTensor()) continue;
          const size_t length = ConvertShapeToLength(i.second.shape());

@@ -18,7 +18,8 @@ from sofie_amd import emit
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 HOST_FIXTURES = ["Linear_16", "Linear_32", "Linear_64", "ConvWithPadding", "ConvWithoutPadding", "ConvWithAutopadSameLower",
                  "ConvWithStridesPadding", "ConvWithStridesNoPadding", "ConvWithAsymmetricPadding", "MaxPool1d", "MaxPool2d",
-                 "MaxPool3d", "AvgPool"]
+                 "MaxPool3d", "AvgPool", "ConvTranspose1d", "ConvTranspose2d", "ConvTransposeBias2d", "ConvTransposeBias2dBatched",
+                 "Einsum_matmul", "Einsum_dotprod", "Einsum_3", "Einsum_4"]
 MKL = "/opt/conda/lib/libmkl_rt.so.1"
 
 
@@ -109,11 +110,30 @@ def test_host_session_with_a_blas_library(tmp_path):
     assert rel_err(y, models.cnn_f32_stages(oracle, x)["y"].reshape(-1)) <= 1e-5
 
 
-@pytest.mark.parametrize("name", ["ConvTranspose2d", "Einsum_matmul"])
-def test_operators_without_a_host_form_say_so(name, tmp_path):
-    spec, _ = models.fixture_spec(name)
-    _, _, res = spec.generate(str(tmp_path), host_code=True, check=False)
-    assert res.returncode != 0 and "has no host emission" in res.stderr
+def test_operators_without_a_host_form_say_so(tmp_path):
+    """GemmFP8 is the one operator of the device path without a host form."""
+    s = emit.ModelSpec("fp8")
+    s.add_input("a", "FLOAT8E4M3FN", (4, 16))
+    s.add_init("b", np.zeros((16, 8), np.uint8), "FLOAT8E4M3FN")
+    s.add_scalar("sa", 1.0, np.float32)
+    s.add_scalar("sb", 1.0, np.float32)
+    s.gemm_fp8("a", "sa", "b", "sb", None, "y")
+    s.set_output("y", "BFLOAT16")
+    _, _, res = s.generate(str(tmp_path), host_code=True, check=False)
+    assert res.returncode != 0 and "no host emission" in res.stderr
+
+
+def test_batchnorm_conv_transpose_and_stacked_products_as_host_code(tmp_path):
+    """Conv + BatchNormalization + Relu (the normalisation is its own loop here: no folding pass runs), a 1-D
+    convolution, pooling over one and three axes, stacked MatMul: 1e-5 relative against the oracle's references."""
+    p = models.convbn_params()
+    assert rel_err(run_host(models.convbn_spec(), [p["x"]], tmp_path / "bn"), models.convbn_reference(oracle).reshape(-1)) <= 1e-5
+    p = models.conv1d_params()
+    assert rel_err(run_host(models.conv1d_spec(), [p["x"]], tmp_path / "c1"), models.conv1d_reference(oracle).reshape(-1)) <= 1e-5
+    p = models.conv3d_params()
+    assert rel_err(run_host(models.conv3d_spec(), [p["x"]], tmp_path / "c3"), models.conv3d_reference(oracle).reshape(-1)) <= 1e-5
+    assert rel_err(run_host(models.pool1d_spec(), [models.pool1d_input()], tmp_path / "p1"), models.pool1d_reference(oracle).reshape(-1)) <= 1e-5
+    assert rel_err(run_host(models.pool3d_spec(), [models.pool3d_input()], tmp_path / "p3"), models.pool3d_reference(oracle).reshape(-1)) <= 1e-5
 
 
 @pytest.mark.parametrize("name", ["Linear_16", "ConvWithPadding", "MaxPool2d"])
