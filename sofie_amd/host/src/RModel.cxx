@@ -1140,11 +1140,13 @@ void RModel::GenerateHostHeaderInfo(std::string &hgname)
           "                  const int id = od * strides[0] - pads[0] + kd * dilations[0];\n"
           "                  for (int oh = 0; oh < out[1]; ++oh) {\n"
           "                     const int ih = oh * strides[1] - pads[1] + kh * dilations[1];\n"
-          "                     for (int ow = 0; ow < out[2]; ++ow) {\n"
-          "                        const int iw = ow * strides[2] - pads[2] + kw * dilations[2];\n"
-          "                        const bool inside = id >= 0 && id < in[0] && ih >= 0 && ih < in[1] && iw >= 0 && iw < in[2];\n"
-          "                        *col++ = inside ? x[((static_cast<size_t>(c) * in[0] + id) * in[1] + ih) * in[2] + iw] : 0.f;\n"
+          "                     if (id < 0 || id >= in[0] || ih < 0 || ih >= in[1]) {\n"
+          "                        for (int ow = 0; ow < out[2]; ++ow) *col++ = 0.f;\n"
+          "                        continue;\n"
           "                     }\n"
+          "                     const float * row = x + ((static_cast<size_t>(c) * in[0] + id) * in[1] + ih) * in[2];\n"
+          "                     int iw = kw * dilations[2] - pads[2];\n"
+          "                     for (int ow = 0; ow < out[2]; ++ow, iw += strides[2]) *col++ = (iw >= 0 && iw < in[2]) ? row[iw] : 0.f;\n"
           "                  }\n"
           "               }\n"
           "            }\n"
