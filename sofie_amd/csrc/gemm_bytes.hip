@@ -851,6 +851,7 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
       // barrier stands between a wavefront's last matrix instruction and its epilogue: the same time within 0.4 us.)
       if (g.vec_store && n0 + BN <= g.N) {
          if (g.zp == -128 && g.lo == -128) tile_epilogue_wave16_direct<NI, MJ, 1>(g, acc, s_scale + wn * 128, s_bias + wn * 128, lane, m_wave, n_wave);
+         else if (g.lo == -128 && !g.bias) tile_epilogue_wave16_direct<NI, MJ, 2, false>(g, acc, s_scale + wn * 128, s_bias + wn * 128, lane, m_wave, n_wave);
          else if (g.lo == -128) tile_epilogue_wave16_direct<NI, MJ, 2>(g, acc, s_scale + wn * 128, s_bias + wn * 128, lane, m_wave, n_wave);
          else tile_epilogue_wave16_direct<NI, MJ, 0>(g, acc, s_scale + wn * 128, s_bias + wn * 128, lane, m_wave, n_wave);
          return;

@@ -433,7 +433,8 @@ __device__ __forceinline__ void tile_epilogue_wave16(const GemmArgs &g, v4i (&ac
 // apart), and two rounds of swaps (between the halves of the wavefront, then between neighbouring groups of 16 lanes)
 // transpose it. Lane group kg then has the 16 columns of tile kg in order, and a store instruction writes 64
 // contiguous bytes for each of 16 rows (written through the L2).
-template <int NI, int MJ, int PLAIN>
+// BIAS false: the call has no bias tensor, and the 128 additions of a zero per lane are left out.
+template <int NI, int MJ, int PLAIN, bool BIAS = true>
 __device__ __forceinline__ void tile_epilogue_wave16_direct(const GemmArgs &g, v4i (&acc)[NI][MJ], const float *s_scale,
                                                             const int *s_bias, int lane, int m_wave, int n_wave)
 {
@@ -447,7 +448,7 @@ __device__ __forceinline__ void tile_epilogue_wave16_direct(const GemmArgs &g, v
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
          sc[i] = *reinterpret_cast<const v4f *>(s_scale + (ig + i) * 16 + kg * 4);
-         bi[i] = *reinterpret_cast<const v4i *>(s_bias + (ig + i) * 16 + kg * 4);
+         if constexpr (BIAS) bi[i] = *reinterpret_cast<const v4i *>(s_bias + (ig + i) * 16 + kg * 4);
       }
 #pragma unroll
       for (int j = 0; j < MJ; ++j) {
@@ -459,7 +460,7 @@ __device__ __forceinline__ void tile_epilogue_wave16_direct(const GemmArgs &g, v
             unsigned pk = 0;
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-               float r = __fmul_rn(__int2float_rn(acc[ig + i][j][t] + bi[i][t]), sc[i][t]);
+               float r = __fmul_rn(__int2float_rn(BIAS ? acc[ig + i][j][t] + bi[i][t] : acc[ig + i][j][t]), sc[i][t]);
                if constexpr (PLAIN == 0) r = fmaxf(__fadd_rn(rintf(r), zpo), lof);
                if constexpr (PLAIN == 2) r = __fadd_rn(rintf(r), zpo);
                pk = __builtin_amdgcn_cvt_pk_u8_f32(r, t, pk);     // rounds half to even, saturates at 0 and 255
