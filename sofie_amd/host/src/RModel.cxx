@@ -846,6 +846,11 @@ void RModel::GenerateSessionCode()
    fGC += "Session(std::string filename =\"" +
           (fUseWeightFile ? fName + (fWeightFile == WeightFileType::Binary ? ".bin" : ".dat") : std::string("")) +
           "\", int device = 0) {\n";
+   {
+      bool reads_file = false;
+      for (auto &i : fInitializedTensors) reads_file = reads_file || (fUseWeightFile && i.second.IsWeightTensor());
+      if (!reads_file) fGC += "   (void)filename;   // no weight file is read\n";
+   }
    fGC += "   { int status = sofie_hip_create(&fCtx.p, device, nullptr);\n";
    fGC += "     if (status != 0) throw std::runtime_error(\"TMVA SOFIE cannot create a device context\"); }\n";
    fGC += "   try {\n";

@@ -801,3 +801,23 @@ def test_gemm_chain_becomes_one_call(tmp_path):
     # q is a model output: the chain x -> p -> q ends there and the last layer is a call of its own
     assert code.count("sofie_hip_mlp_f32(") == 1 and code.count("sofie_hip_gemm_f32(") == 1
     assert re.search(r"_dims\[\] = \{6, 5, 7\};", code)
+
+
+@pytest.mark.parametrize("host_code", [False, True])
+def test_generated_sessions_compile_without_warnings(host_code, tmp_path):
+    """What the emitter writes is code a user compiles into a program of their own: -Wall -Wextra -Wshadow -Werror on
+    the Sessions of the benchmark's networks, the quantized models, a weightless pooling graph, ConvTranspose and
+    Einsum, for the device and for the host cores."""
+    specs = [models.mlp_spec()[0], models.cnn_f32_spec(8), models.qcnn_spec(oracle, 8), models.qdq_conv_spec(),
+             models.convbn_spec(), models.conv3d_spec(), models.pool3d_spec(), models.cnn_f32_rt_spec()]
+    specs += [models.fixture_spec(n)[0] for n in ("ConvTransposeBias2d", "Einsum_3", "Einsum_4", "AvgPool", "MaxPool1d")]
+    for spec in specs:
+        d = tmp_path / (spec.name + ("_host" if host_code else "_dev"))
+        d.mkdir()
+        hxx, _, _ = spec.generate(str(d), host_code=host_code)
+        src = d / "unit.cxx"
+        src.write_text('#include "%s"\nint main() { return 0; }\n' % os.path.basename(hxx))
+        res = subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-Wshadow", "-Werror", "-fsyntax-only", "-I" + str(d),
+                              "-I" + os.path.join(emit.ROOT, "include"), "-I" + os.path.join(emit.ROOT, "sofie_amd", "host", "inc"), str(src)],
+                             stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        assert res.returncode == 0, spec.name + "\n" + res.stdout
