@@ -13,6 +13,7 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
         sys.path.insert(0, p)
 
 import models  # noqa: E402
+import random_graphs  # noqa: E402
 from oracle import oracle  # noqa: E402
 from sofie_amd import emit  # noqa: E402
 
@@ -35,6 +36,9 @@ def all_specs(with_large=True):
     specs.append(models.two_heads_spec()[0])
     specs.append(models.mixed_outputs_spec()[0])
     specs.append(models.mlp_nosession_spec()[0])
+    # graphs with seeded random attributes (tests/random_graphs.py)
+    specs += [random_graphs.float_graph(seed)[0] for seed in random_graphs.FLOAT_SEEDS]
+    specs += [random_graphs.quantized_graph(seed, oracle)[0] for seed in random_graphs.QUANT_SEEDS]
     if with_large:
         specs.append(models.qcnn_spec(oracle, 4096, "qcnn_b4096"))
     return specs

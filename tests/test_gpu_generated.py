@@ -12,6 +12,7 @@ import numpy as np
 import pytest
 
 import models
+import random_graphs
 import replay
 from oracle import oracle
 from sofie_amd import emit
@@ -73,6 +74,26 @@ def test_reference_fixture_through_generated_session(name, tmp_path):
     assert np.max(np.abs(y - want)) <= 1e-3             # the reference's own tolerance
     yo = replay.run_graph(graph, feeds, oracle)
     assert rel_err(y, yo.reshape(-1)) <= 1e-5
+
+
+@pytest.mark.parametrize("seed", random_graphs.FLOAT_SEEDS)
+def test_random_float_graph_sessions_against_torch(seed, tmp_path):
+    """Generated device Sessions of graphs with random attributes (Conv with groups, strides, dilations, four different
+    pads; Relu, MaxPool, AveragePool, Flatten + Gemm behind it) against torch's CPU operators: 1e-4 of the largest
+    output."""
+    spec, x, want = random_graphs.float_graph(seed)
+    y = run_session(spec.name, x, tmp_path)
+    assert y.size == want.size
+    assert np.max(np.abs(y - want)) <= 1e-4 * max(1.0, float(np.max(np.abs(want))))
+
+
+@pytest.mark.parametrize("seed", random_graphs.QUANT_SEEDS)
+def test_random_quantized_graph_sessions_are_bit_exact(seed, tmp_path):
+    """QuantizeLinear, QLinearConv (random channels, groups, kernel, stride, pads, zero-points, per-channel scales),
+    optional Relu and 2x2 MaxPool, DequantizeLinear as generated device Sessions: the oracle's output bit for bit."""
+    spec, x, want = random_graphs.quantized_graph(seed, oracle)
+    y = run_session(spec.name, x, tmp_path)
+    assert np.array_equal(y, want)
 
 
 def test_mlp_session(tmp_path):

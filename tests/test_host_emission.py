@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 
 import models
+import random_graphs
 import replay
 from oracle import oracle
 from sofie_amd import emit
@@ -134,6 +135,26 @@ def test_batchnorm_conv_transpose_and_stacked_products_as_host_code(tmp_path):
     assert rel_err(run_host(models.conv3d_spec(), [p["x"]], tmp_path / "c3"), models.conv3d_reference(oracle).reshape(-1)) <= 1e-5
     assert rel_err(run_host(models.pool1d_spec(), [models.pool1d_input()], tmp_path / "p1"), models.pool1d_reference(oracle).reshape(-1)) <= 1e-5
     assert rel_err(run_host(models.pool3d_spec(), [models.pool3d_input()], tmp_path / "p3"), models.pool3d_reference(oracle).reshape(-1)) <= 1e-5
+
+
+@pytest.mark.parametrize("seed", random_graphs.FLOAT_SEEDS)
+def test_random_float_graphs_against_torch(seed, tmp_path):
+    """Conv with random groups, strides, dilations and four different pads, then Relu / MaxPool / AveragePool (with and
+    without the padding cells in the count) / Flatten + Gemm: the generated host Session against torch's CPU operators,
+    which share nothing with the emitter or the oracle. 1e-4 of the largest output (torch sums in another order)."""
+    spec, x, want = random_graphs.float_graph(seed)
+    y = run_host(spec, [x], tmp_path)
+    assert y.size == want.size
+    assert np.max(np.abs(y - want)) <= 1e-4 * max(1.0, float(np.max(np.abs(want))))
+
+
+@pytest.mark.parametrize("seed", random_graphs.QUANT_SEEDS)
+def test_random_quantized_graphs_are_bit_exact(seed, tmp_path):
+    """QuantizeLinear, QLinearConv with random channels, groups, kernel, stride, pads, zero-points and per-channel
+    scales, optional Relu and 2x2 MaxPool, DequantizeLinear: the generated host Session equals the oracle bit for bit."""
+    spec, x, want = random_graphs.quantized_graph(seed, oracle)
+    y = run_host(spec, [x], tmp_path)
+    assert np.array_equal(y, want)
 
 
 @pytest.mark.parametrize("name", ["Linear_16", "ConvWithPadding", "MaxPool2d"])
