@@ -473,6 +473,9 @@ def main():
         if meta.get("bound") == "hbm":
             entry["bound"] = "hbm"
             entry["frac_hbm_peak"] = entry["gbs"] / PEAK_HBM_GBS
+        if "check" in meta:
+            torch.cuda.synchronize()
+            entry["parity"] = meta["check"]()        # outside every timed region
         res[name] = entry
     out["fp8_gemm"] = dict(res["gemm_fp8"], peak_tflops=PEAK_FP8_TFLOPS)
     out["fp8_gemm_b_nk"] = res["gemm_fp8_nk"]
@@ -489,6 +492,22 @@ def main():
     if not args.no_cpu:
         out["cpu_fp32"] = cpu_fp32_baselines(threads)
     print(json.dumps(out))
+
+
+def fp8_band_check(torch, A8, Bm, transB, sA, sB, bias, Y16, rows=64):
+    """The timed FP8 output on a band of rows against the float64 product of the same e4m3 operands (torch's own e4m3
+    type and float64 matmul: nothing of this library), with the tolerance the tests state: one bf16 rounding of the
+    result plus 7 * 2^-13 of sum|a_k b_k| (what the matrix instruction's sums of eight products may drop)."""
+    pick = torch.linspace(0, A8.shape[0] - 1, rows, device=A8.device).long()
+    a = A8[pick].view(torch.float8_e4m3fn).to(torch.float64)
+    b = Bm.view(torch.float8_e4m3fn).to(torch.float64)
+    b = b.t() if transB else b
+    truth = (a @ b) * (sA * sB) + bias.to(torch.float64)
+    mag = (a.abs() @ b.abs()) * (sA * sB)
+    err = (Y16[pick].to(torch.float64) - truth).abs()
+    tol = 2.0 ** -8 * truth.abs() + 7 * 2.0 ** -13 * mag + 1e-30
+    return {"rows": rows, "within_tolerance": bool((err <= tol).all()), "largest_error_over_tolerance": float((err / tol).max()),
+            "tolerance": "2^-8 |ref| + 7 * 2^-13 * sa sb sum|a_k b_k| against the float64 product of the same e4m3 operands"}
 
 
 def workloads(ctx, torch, L, rng):
@@ -522,7 +541,8 @@ def workloads(ctx, torch, L, rng):
             L.OUT_BF16))),
             {"workload": "FP8 e4m3 GEMM M=N=8192 K=4096, A and B N(0,1) cast to e4m3 with per-tensor scales amax/448, "
                          "B %s, fused bias, bf16 out" % ("[N,K]" if tb else "[K,N]"),
-             "ops": 2.0 * M * N * K, "rate_unit": "tflops", "peak": PEAK_FP8_TFLOPS, "launches": 100})
+             "ops": 2.0 * M * N * K, "rate_unit": "tflops", "peak": PEAK_FP8_TFLOPS, "launches": 100,
+             "check": (lambda tb=tb, Bm=Bm: fp8_band_check(torch, A8, Bm, tb, sA, sB, bias, Y16))})
     # fp32 Gemm as the reference's operator states it (Y = A B + bias, ReLU fused), 4096^3, B as [K,N] and as [N,K]
     Af = torch.randn(n, n, device=ctx.device)
     Bf = torch.randn(n, n, device=ctx.device)
