@@ -79,12 +79,12 @@ def test_reference_fixture_through_generated_session(name, tmp_path):
 @pytest.mark.parametrize("seed", random_graphs.FLOAT_SEEDS)
 def test_random_float_graph_sessions_against_torch(seed, tmp_path):
     """Generated device Sessions of graphs with random attributes (Conv with groups, strides, dilations, four different
-    pads; Relu, MaxPool, AveragePool, Flatten + Gemm behind it) against torch's CPU operators: 1e-4 of the largest
+    pads; Relu, MaxPool, AveragePool, Flatten + Gemm behind it) against torch's CPU operators: 1e-5 of the largest
     output."""
     spec, x, want = random_graphs.float_graph(seed)
     y = run_session(spec.name, x, tmp_path)
     assert y.size == want.size
-    assert np.max(np.abs(y - want)) <= 1e-4 * max(1.0, float(np.max(np.abs(want))))
+    assert np.max(np.abs(y - want)) <= 1e-5 * max(1.0, float(np.max(np.abs(want))))
 
 
 @pytest.mark.parametrize("seed", random_graphs.QUANT_SEEDS)
