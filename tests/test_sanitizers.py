@@ -1,7 +1,8 @@
 """CPU-side safety net: the host emitter, the ONNX wire parser and the oracle built with AddressSanitizer and
 UndefinedBehaviorSanitizer (`make -C sofie_amd/host SAN=1`, `make -C oracle san`), run over the fixtures, over every
 model description of the GPU tests and over mutated ONNX bytes. A parser may reject a damaged file (exit status 1
-with a message) or accept it; it may never crash, read out of bounds or overflow."""
+with a message) or accept it; it may never crash, read out of bounds or overflow. The code the emitter generates for
+the host cores is compiled with the same sanitizers and run as well."""
 import os
 import subprocess
 import sys
@@ -121,3 +122,55 @@ def test_oracle_is_clean_under_the_sanitizers():
     text = res.stdout
     assert "AddressSanitizer" not in text and "runtime error:" not in text, text[-3000:]
     assert res.returncode == 0, text[-3000:]
+
+
+def test_generated_host_sessions_run_clean(tmp_path):
+    """The code the emitter writes for the host cores, compiled with AddressSanitizer and UndefinedBehaviorSanitizer and
+    run: the fp32 CNN, the int8 CNN (QuantizeLinear, QLinearConv + pooling, QLinearMatMul), quantize -> conv ->
+    dequantize, graphs with random attributes, a transposed convolution and an Einsum. Same outputs as the ordinary
+    build checks elsewhere; here no report from either sanitizer."""
+    import random_graphs
+    import replay
+    import json
+    from oracle import oracle
+    cases = []
+    x2 = models.cnn_input(2)
+    cases.append((models.cnn_f32_spec(2, "cnn_f32_b2"), [x2], models.cnn_f32_stages(oracle, x2)["y"].reshape(-1), 1e-5))
+    cases.append((models.qcnn_spec(oracle, 2, "qcnn_b2"), [x2], models.qcnn_reference(oracle, x2).reshape(-1), 0.0))
+    cases.append((models.qdq_conv_spec(), [models.qdq_conv_params()["x"]], models.qdq_conv_reference(oracle).reshape(-1), 0.0))
+    for seed in random_graphs.FLOAT_SEEDS[:3]:
+        s, x, want = random_graphs.float_graph(seed)
+        cases.append((s, [x], want, 1e-5))
+    for seed in random_graphs.QUANT_SEEDS[1:3]:
+        s, x, want = random_graphs.quantized_graph(seed, oracle)
+        cases.append((s, [x], want, 0.0))
+    expected = json.load(open(os.path.join(ROOT, "tests", "golden", "expected.json")))
+    for name in ("ConvTransposeBias2dBatched", "Einsum_3"):
+        spec, graph = models.fixture_spec(name)
+        feeds = replay.fixture_feeds(expected[name], graph)
+        cases.append((spec, [feeds[i[0]] for i in graph["inputs"]], np.array(expected[name]["expected"], np.float32), 1e-3))
+    for spec, xs, want, tol in cases:
+        d = tmp_path / spec.name
+        d.mkdir()
+        hxx, dat, _ = spec.generate(str(d), host_code=True)
+        exe = str(d / "run")
+        cmd = ["g++", "-std=c++17", "-O1", "-g", "-fno-omit-frame-pointer", "-fsanitize=address,undefined",
+               "-fno-sanitize-recover=undefined", "-I" + str(d), "-DSOFIE_MODEL_HEADER=\"%s.hxx\"" % spec.name,
+               "-DSOFIE_MODEL_NS=SOFIE_%s" % spec.name, "-DSOFIE_NUM_INPUTS=%d" % len(xs),
+               os.path.join(ROOT, "sofie_amd", "host", "examples", "run_host_session.cxx"), "-o", exe, "-ldl"]
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        assert res.returncode == 0, res.stdout[-2000:]
+        names = []
+        for i, a in enumerate(xs):
+            names.append(str(d / ("in%d.bin" % i)))
+            np.ascontiguousarray(a, np.float32).tofile(names[-1])
+        res = subprocess.run([exe, dat, ",".join(names), str(d / "out.bin")], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                             env=SAN_ENV, timeout=300)
+        _clean(res)
+        assert res.returncode == 0, spec.name + "\n" + res.stderr[-2000:]
+        y = np.fromfile(str(d / "out.bin"), np.float32)
+        assert y.size == want.size, spec.name
+        if tol == 0.0:
+            assert np.array_equal(y, want), spec.name
+        else:
+            assert np.max(np.abs(y - want)) <= tol * max(1.0, float(np.max(np.abs(want)))), spec.name
