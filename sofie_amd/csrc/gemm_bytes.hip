@@ -23,6 +23,7 @@ namespace {
 // Workgroup id -> output tile. Ids are dealt round-robin over the 8 XCDs, each with its own
 // L2; the remap gives every XCD a contiguous run of ids and the grouped order turns that run
 // into a compact rectangle of tiles, so an XCD's L2 sees each operand panel once.
+template <int GM = 4>
 __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tiles_n, int &tm, int &tn)
 {
    const int tiles = tiles_m * tiles_n;
@@ -31,7 +32,6 @@ __device__ __forceinline__ void tile_of_workgroup(int pid, int tiles_m, int tile
       const int base = tiles >> 3, rem = tiles & 7;
       pid = local + xcd * base + (xcd < rem ? xcd : rem);
    }
-   constexpr int GM = 4;
    const int width = GM * tiles_n;
    const int group = pid / width;
    const int first = group * GM;
@@ -694,7 +694,9 @@ __global__ void __launch_bounds__(512, 2) k_gemm_dma16(GemmArgs g)
    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
    const int wn = wave & 1, wm = wave >> 1;
    int tm, tn;
-   tile_of_workgroup(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+   // an XCD's 32 tiles of a 4096^3 product: 8 m x 4 n with B [K,N] (49.4 - 50.9 against 49.7 - 51.6 us, eight of
+   // eight alternating comparisons), 4 m x 8 n with B [N,K] (no difference there; 2 x 16 and 16 x 2 cost 1.5 - 2.5 %)
+   tile_of_workgroup<B_KN ? 8 : 4>(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
    const int m0 = tm * BM, n0 = tn * BN;
 
    // --- loads: as in k_gemm_dma (wavefronts 0-3 request the A tile, 4-7 the B^T tile)
